@@ -1,0 +1,109 @@
+/* libimhip -- C ABI of the MI355X (gfx950) batched Newton linear-algebra path.
+ *
+ * Every entry point is what a binding of the reference's Python launchers for
+ * this path would call.  Citations are relative to the reference tree
+ * (Scripter36/InstantMimic).  Conventions:
+ *   - plain C types only; device buffers are caller-owned device pointers;
+ *   - every launcher takes a hipStream_t (as void*), never synchronises, never
+ *     allocates, and is safe to capture in a hipGraph;
+ *   - the return value is a status code (IM_OK == 0); nothing throws;
+ *   - planners report "ineligible" through the plan info / a status code, which
+ *     mirrors the reference returning None so that the caller keeps its fallback.
+ */
+#ifndef IMHIP_H_
+#define IMHIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define IM_OK 0
+#define IM_ERR_ARG 1         /* null pointer, negative size, bad enum */
+#define IM_ERR_STRUCTURE 2   /* CSR is not in nested-ancestor form */
+#define IM_ERR_UNSUPPORTED 3 /* shape outside what the kernels are built for */
+#define IM_ERR_HIP 4         /* a HIP runtime call failed (see im_last_hip_error) */
+#define IM_ERR_STRIDE 5      /* rows are not contiguous floats */
+
+#define IM_MAX_GROUPS 4
+
+typedef struct im_tree_plan im_tree_plan;
+
+typedef struct im_tree_plan_info {
+  int32_t nv;           /* dofs */
+  int32_t nM;           /* CSR entries of M */
+  int32_t ngroups;      /* groups in the plan (may include empty ones) */
+  int32_t ntrunk;       /* trunk dofs */
+  int32_t span;         /* critical path in update units */
+  int32_t dense_cost;   /* sum over trees of size^3 / 3 */
+  int32_t shared_bytes; /* trunk exchange footprint of the reference's CUDA kernel */
+  int32_t beats_dense;  /* 1 when the reference would use the tree solve */
+  int32_t max_depth;    /* longest ancestor chain (row length) */
+  int32_t device_ready; /* 1 when the device kernels support this shape */
+} im_tree_plan_info;
+
+/* Library / runtime ------------------------------------------------------- */
+int im_version(void);
+const char *im_status_string(int status);
+/* hipError_t of the last failing HIP call on this thread (0 if none). */
+int im_last_hip_error(void);
+
+/* Tree L'DL planning (host, integer) -------------------------------------- */
+
+/* Replaces tree_ldl_structure (src/instantmimic/utils/mjw_kernels/tree_ldl.py:66-91):
+ * IM_OK when every CSR row is "ancestors root-first, diagonal last" and each
+ * ancestor's row is a prefix of it, else IM_ERR_STRUCTURE. */
+int im_tree_structure_check(int nv, const int32_t *rowadr, const int32_t *rownnz,
+                            const int32_t *colind, int ncol);
+
+/* Replaces plan_tree_ldl (tree_ldl.py:105-170) for groups in 1..4 and
+ * best_tree_ldl_plan (tree_ldl.py:173-185) for groups == 0.  Builds the device
+ * tables on the current HIP device unless host_only != 0 (planning without a
+ * GPU).  The plan is immutable afterwards. */
+int im_tree_plan_create(int nv, const int32_t *rowadr, const int32_t *rownnz,
+                        const int32_t *colind, int ncol, int groups,
+                        int host_only, im_tree_plan **out);
+void im_tree_plan_destroy(im_tree_plan *plan);
+
+/* TreeLdlPlan fields (tree_ldl.py:47-56), tree_ldl_beats_dense (:188-193) and
+ * _shared_bytes (:98-102). */
+int im_tree_plan_get_info(const im_tree_plan *plan, im_tree_plan_info *info);
+/* group_ptr[ngroups + 1], group_dofs[nv - ntrunk] (each group descending),
+ * trunk[ntrunk] (ascending), elim_order[nv] = groups in order then the trunk
+ * descending (tree_ldl.py:256-257, 290).  Any pointer may be null. */
+int im_tree_plan_get_arrays(const im_tree_plan *plan, int32_t *group_ptr,
+                            int32_t *group_dofs, int32_t *trunk,
+                            int32_t *elim_order);
+
+/* Launchers ---------------------------------------------------------------- */
+
+/* Replaces tree_factor_solve (tree_ldl.py:419-433): x = (L'DL)^-1 y for every
+ * world, M (nworld, ldM >= nM) in the model's CSR layout, M is not modified.
+ * ld* are row strides in floats. */
+int im_tree_factor_solve(const im_tree_plan *plan, const float *M, int64_t ldM,
+                         const float *y, int64_t ldy, float *x, int64_t ldx,
+                         int nworld, void *stream);
+
+#define IM_FLAG_NEGATE 1u /* write -x (the Newton search direction) */
+
+/* The fused Newton linear step on a tree pattern: H = M + sum over rows r with
+ * state == quad and r < nefc[w] of D J'J on M's CSR entries (summation order of
+ * sparse_hessian.py:589, 622-629), tree L'DL of H and solve with grad
+ * (tree_ldl.py:215-305).  What the reference reaches through
+ * newton_fusion._update_gradient_sparse / sparse_hessian.init_factor_kernel
+ * (newton_fusion.py:480-519) and tree_ldl.tree_factor_solve.
+ *   J (nworld, njmax, nv) contiguous, D/state (nworld, njmax), nefc (nworld) or
+ *   null for njmax rows everywhere, grad (nworld, ldg), x (nworld, ldx),
+ *   Hout (nworld, nM) or null. */
+int im_assemble_tree_ldl_solve(const im_tree_plan *plan, const float *M,
+                               int64_t ldM, const float *J, int njmax,
+                               const float *D, const int32_t *state,
+                               const int32_t *nefc, int quad, const float *grad,
+                               int64_t ldg, float *x, int64_t ldx, float *Hout,
+                               int nworld, unsigned flags, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IMHIP_H_ */

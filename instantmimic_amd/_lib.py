@@ -1,0 +1,84 @@
+"""ctypes binding of ``libimhip.so`` (the C ABI declared in ``include/imhip.h``).
+
+The library must have been built (``python -m instantmimic_amd.build`` or
+``__graft_entry__.build()``); there is no fallback path when it is missing.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libimhip.so")
+
+IM_OK = 0
+IM_ERR_ARG = 1
+IM_ERR_STRUCTURE = 2
+IM_ERR_UNSUPPORTED = 3
+IM_ERR_HIP = 4
+IM_ERR_STRIDE = 5
+IM_FLAG_NEGATE = 1
+
+
+class TreePlanInfo(C.Structure):
+    _fields_ = [
+        (name, C.c_int32)
+        for name in (
+            "nv", "nM", "ngroups", "ntrunk", "span", "dense_cost", "shared_bytes", "beats_dense", "max_depth",
+            "device_ready",
+        )
+    ]  # fmt: skip
+
+
+_vp, _i, _i64, _u = C.c_void_p, C.c_int, C.c_int64, C.c_uint
+
+# name -> (restype, argtypes); the single list of symbols the header declares
+SIGNATURES = {
+    "im_version": (_i, []),
+    "im_status_string": (C.c_char_p, [_i]),
+    "im_last_hip_error": (_i, []),
+    "im_tree_structure_check": (_i, [_i, _vp, _vp, _vp, _i]),
+    "im_tree_plan_create": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, C.POINTER(_vp)]),
+    "im_tree_plan_destroy": (None, [_vp]),
+    "im_tree_plan_get_info": (_i, [_vp, C.POINTER(TreePlanInfo)]),
+    "im_tree_plan_get_arrays": (_i, [_vp, _vp, _vp, _vp, _vp]),
+    "im_tree_factor_solve": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _vp]),
+    "im_assemble_tree_ldl_solve": (
+        _i,
+        [_vp, _vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _i, _u, _vp],
+    ),
+}
+
+_lib = None
+
+
+class ImhipError(RuntimeError):
+    def __init__(self, status: int, where: str):
+        self.status = status
+        msg = lib().im_status_string(status).decode()
+        if status == IM_ERR_HIP:
+            msg += f" (hipError {lib().im_last_hip_error()})"
+        super().__init__(f"{where}: {msg}")
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m instantmimic_amd.build` "
+                "(there is no CPU fallback for the HIP kernels)"
+            )
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(status: int, where: str) -> None:
+    if status != IM_OK:
+        raise ImhipError(status, where)

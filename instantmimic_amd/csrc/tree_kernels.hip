@@ -1,0 +1,416 @@
+// Fused Hessian assembly + kinematic-tree L'DL + solve for gfx950, one wavefront
+// per world.
+//
+// What is computed (reference statements):
+//   H[e]  = M[e] + sum_r fmaf(J[r][a] * Dc[r], J[r][b], .)   rows ascending
+//           (src/instantmimic/utils/mjw_kernels/sparse_hessian.py:589, 622-629)
+//   x     = (L'DL)^-1 y on M's CSR pattern, leaves first
+//           (src/instantmimic/utils/mjw_kernels/tree_ldl.py:215-305)
+// with the plan's groups accumulating their trunk contributions from zero and
+// the trunk summing them in group order, so that every floating-point operation
+// and its order equal the reference's generated straight-line code.  Arithmetic
+// convention: t - a*b*c is fmaf(-(a*b), c, t) and s - a*b is fmaf(-a, b, s) (what
+// a contracting compiler makes of the reference's expressions); this file is
+// compiled with -ffp-contract=off and spells every fused operation.
+//
+// Mapping.  A world is served by one 64-lane wavefront (workgroup of 64).  The
+// nM entries of H live in registers, entry e in lane e % 64, register e / 64,
+// and never move: the assembly accumulates into them, eliminations update them
+// in place.  When dof k is eliminated its (final) row is published to LDS and
+// every lane whose entry belongs to an ancestor row applies its update from two
+// LDS reads.  The right-hand side rides along, one dof per lane.  Constraint
+// rows are staged through LDS in chunks, inactive rows are dropped while staging,
+// and the next chunk's global loads are in flight while the current one is summed.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+
+#include "common.h"
+
+namespace im {
+namespace {
+
+constexpr int kPF = 16;  // global-load registers per lane and chunk (1024 floats)
+
+__device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+
+template <int SPL, int NVP, bool ASM>
+__global__ __launch_bounds__(64) void tree_kernel(
+    TreeDev P, const float *__restrict__ M, int64_t ldM, const float *__restrict__ J,
+    int njmax, const float *__restrict__ D, const int32_t *__restrict__ state,
+    const int32_t *__restrict__ nefc_p, int quad, const float *__restrict__ y,
+    int64_t ldy, float *__restrict__ x, int64_t ldx, float *__restrict__ Hout,
+    int rc, float inv_nv, int njpad, unsigned flags) {
+  extern __shared__ float lds[];
+  const int lane = threadIdx.x;
+  const int w = blockIdx.x;
+  const int nv = P.nv, nM = P.nM;
+
+  float *T = lds;                      // [nM]   published rows (unscaled)
+  float *Sp = T + nM;                  // [64]   published right-hand sides
+  float *Di = Sp + 64;                 // [64]   inverse pivots
+  float *X = Di + 64;                  // [64]   solution
+  int *col = (int *)(X + 64);          // [nM]
+  float *Dc = (float *)(col + nM);     // [njpad]
+  float *Jc = Dc + njpad;              // [rc * NVP]
+  float *JDc = Jc + rc * NVP;          // [rc * NVP]
+
+  // ---- per-lane constants -------------------------------------------------
+  int se[SPL];        // CSR entry, -1 when the register is unused
+  uint32_t sd[SPL];   // a | b << 8 | p << 16 | q << 24
+  bool strunk[SPL];   // the entry's row is a trunk dof
+  float h[SPL];
+  float acc[IM_MAX_GROUPS][SPL];
+#pragma unroll
+  for (int i = 0; i < SPL; ++i) {
+    const int e = P.slot_e[i * 64 + lane];
+    const uint32_t d = P.slot_d[i * 64 + lane];
+    se[i] = e < 0 ? -1 : (e & 0xFFFF);
+    strunk[i] = e >= 0 && ((e >> 30) & 1);
+    sd[i] = d;
+    h[i] = se[i] >= 0 ? M[(int64_t)w * ldM + se[i]] : 0.0f;
+#pragma unroll
+    for (int j = 0; j < IM_MAX_GROUPS; ++j) acc[j][i] = 0.0f;
+  }
+  const int dd = P.dof_d[lane];
+  const bool isdof = dd >= 0;
+  const int drow = dd & 0xFFFF;
+  const int ddepth = isdof ? ((dd >> 16) & 0xFF) : -1;
+  const bool dtrunk = isdof && ((dd >> 24) & 1);
+  float s = isdof ? y[(int64_t)w * ldy + lane] : 0.0f;
+  float sacc[IM_MAX_GROUPS] = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int e = lane; e < nM; e += 64) col[e] = P.colind[e];
+
+  // ---- assembly -------------------------------------------------------------
+  if (ASM) {
+    int nefc = nefc_p ? nefc_p[w] : njmax;
+    nefc = nefc < njmax ? nefc : njmax;
+    nefc = __builtin_amdgcn_readfirstlane(nefc);
+    const float *Dw = D + (int64_t)w * njmax;
+    const int32_t *Sw = state + (int64_t)w * njmax;
+    for (int r = lane; r < njpad; r += 64) {
+      float dc = 0.0f;
+      if (r < nefc && Sw[r] == quad) dc = Dw[r];
+      Dc[r] = dc;
+    }
+    const float *Jw = J + (int64_t)w * njmax * nv;
+    const int nchunk = (nefc + rc - 1) / rc;
+    float cur[kPF], nxt[kPF];
+    int offa[SPL], offb[SPL];  // float offsets of a and b inside a staged row
+#pragma unroll
+    for (int i = 0; i < SPL; ++i) {
+      offa[i] = sd[i] & 0xFF;
+      offb[i] = (sd[i] >> 8) & 0xFF;
+    }
+    {
+      const int rows = nefc < rc ? nefc : rc;
+#pragma unroll
+      for (int u = 0; u < kPF; ++u) {
+        const int q = lane + 64 * u;
+        cur[u] = q < rows * nv ? Jw[q] : 0.0f;
+      }
+    }
+    __syncthreads();  // Dc visible
+    for (int c = 0; c < nchunk; ++c) {
+      {
+        const int r1 = (c + 1) * rc;
+        int rows = nefc - r1;
+        rows = rows < rc ? rows : rc;
+        const float *Jn = Jw + (int64_t)r1 * nv;
+#pragma unroll
+        for (int u = 0; u < kPF; ++u) {
+          const int q = lane + 64 * u;
+          nxt[u] = q < rows * nv ? Jn[q] : 0.0f;
+        }
+      }
+      // rows of this chunk that contribute, as a bit mask (rc <= 64)
+      const int r0 = c * rc;
+      const float mydc = lane < rc ? Dc[r0 + lane] : 0.0f;
+      const uint64_t amask = __ballot(mydc != 0.0f);
+      const int nact = __popcll(amask);
+#pragma unroll
+      for (int u = 0; u < kPF; ++u) {
+        // element -> (row, column) of the chunk
+        const int q = lane + 64 * u;
+        const int r = (int)(((float)q + 0.5f) * inv_nv);
+        if (r < rc && ((amask >> r) & 1ull)) {
+          const int dst = __popcll(amask & ((1ull << r) - 1ull)) * NVP + (q - r * nv);
+          const float dc = Dc[r0 + r];
+          Jc[dst] = cur[u];
+          JDc[dst] = cur[u] * dc;
+        }
+      }
+      __syncthreads();
+      int rl = 0;
+      for (; rl + 4 <= nact; rl += 4) {
+        const float *ja = JDc + rl * NVP;
+        const float *jb = Jc + rl * NVP;
+        float va[4][SPL], vb[4][SPL];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int i = 0; i < SPL; ++i) {
+            va[t][i] = ja[t * NVP + offa[i]];
+            vb[t][i] = jb[t * NVP + offb[i]];
+          }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int i = 0; i < SPL; ++i) h[i] = fma_(va[t][i], vb[t][i], h[i]);
+      }
+      for (; rl < nact; ++rl) {
+        const float *ja = JDc + rl * NVP;
+        const float *jb = Jc + rl * NVP;
+#pragma unroll
+        for (int i = 0; i < SPL; ++i) h[i] = fma_(ja[offa[i]], jb[offb[i]], h[i]);
+      }
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < kPF; ++u) cur[u] = nxt[u];
+    }
+    if (Hout) {
+#pragma unroll
+      for (int i = 0; i < SPL; ++i)
+        if (se[i] >= 0) Hout[(int64_t)w * nM + se[i]] = h[i];
+    }
+  }
+
+  // ---- leaves-first elimination ----------------------------------------------
+  for (int st = 0; st < P.nsteps; ++st) {
+    const int4 info = P.steps[st];
+    const int gid = info.z;
+    if (gid < 0) {
+      // trunk rows: own value plus the groups' contributions in group order
+#pragma unroll
+      for (int j = 0; j < IM_MAX_GROUPS; ++j) {
+        if (j < P.ngroups) {
+#pragma unroll
+          for (int i = 0; i < SPL; ++i) h[i] = h[i] + acc[j][i];
+          s = s + sacc[j];
+        }
+      }
+      continue;
+    }
+    const int rk = info.x, cnt = info.y, k = info.w;
+    const uint64_t anc = P.anc[st];
+#pragma unroll
+    for (int i = 0; i < SPL; ++i)
+      if (se[i] >= 0 && (int)((sd[i] >> 8) & 0xFF) == k) T[se[i]] = h[i];
+    if (lane == k) Sp[k] = s;
+    __syncthreads();
+    const float dk = 1.0f / T[rk + cnt];
+    const float sk = Sp[k];
+    if (lane == 0) Di[k] = dk;
+    const bool togroup = gid < IM_MAX_GROUPS;
+#pragma unroll
+    for (int i = 0; i < SPL; ++i) {
+      if (se[i] >= 0 && ((anc >> ((sd[i] >> 8) & 0xFF)) & 1ull)) {
+        const float v = T[rk + ((sd[i] >> 16) & 0xFF)] * T[rk + (sd[i] >> 24)];
+        if (togroup && strunk[i]) {
+          if (gid == 0) acc[0][i] = fma_(-v, dk, acc[0][i]);
+          else if (gid == 1) acc[1][i] = fma_(-v, dk, acc[1][i]);
+          else if (gid == 2) acc[2][i] = fma_(-v, dk, acc[2][i]);
+          else acc[3][i] = fma_(-v, dk, acc[3][i]);
+        } else {
+          h[i] = fma_(-v, dk, h[i]);
+        }
+      }
+    }
+    if (isdof && ((anc >> lane) & 1ull)) {
+      const float ms = T[rk + ddepth] * dk;
+      if (togroup && dtrunk) {
+        if (gid == 0) sacc[0] = fma_(-ms, sk, sacc[0]);
+        else if (gid == 1) sacc[1] = fma_(-ms, sk, sacc[1]);
+        else if (gid == 2) sacc[2] = fma_(-ms, sk, sacc[2]);
+        else sacc[3] = fma_(-ms, sk, sacc[3]);
+      } else {
+        s = fma_(-ms, sk, s);
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- back substitution, root first --------------------------------------------
+  const float di = isdof ? Di[lane] : 0.0f;
+  float xv = s * di;
+  for (int t = 0; t < P.maxdepth; ++t) {
+    if (ddepth == t) X[lane] = xv;
+    __syncthreads();
+    if (ddepth > t) {
+      const int a = col[drow + t];
+      const float ms = T[drow + t] * di;
+      xv = fma_(-ms, X[a], xv);
+    }
+  }
+  if (isdof) x[(int64_t)w * ldx + lane] = (flags & IM_FLAG_NEGATE) ? -xv : xv;
+}
+
+using KernelFn = void (*)(TreeDev, const float *, int64_t, const float *, int,
+                          const float *, const int32_t *, const int32_t *, int,
+                          const float *, int64_t, float *, int64_t, float *, int,
+                          float, int, unsigned);
+
+template <int SPL>
+KernelFn pick_nvp(int nvp) {
+  switch (nvp) {
+    case 16: if constexpr (SPL <= 4) return tree_kernel<SPL, 16, true>; else return nullptr;
+    case 32: if constexpr (SPL <= 12) return tree_kernel<SPL, 32, true>; else return nullptr;
+    case 48: return tree_kernel<SPL, 48, true>;
+    case 64: return tree_kernel<SPL, 64, true>;
+  }
+  return nullptr;
+}
+
+KernelFn pick(bool assemble, int spl, int nvp) {
+  switch (spl) {
+    case 2: return assemble ? pick_nvp<2>(nvp) : tree_kernel<2, 16, false>;
+    case 4: return assemble ? pick_nvp<4>(nvp) : tree_kernel<4, 16, false>;
+    case 6: return assemble ? pick_nvp<6>(nvp) : tree_kernel<6, 16, false>;
+    case 8: return assemble ? pick_nvp<8>(nvp) : tree_kernel<8, 16, false>;
+    case 12: return assemble ? pick_nvp<12>(nvp) : tree_kernel<12, 16, false>;
+    case 16: return assemble ? pick_nvp<16>(nvp) : tree_kernel<16, 16, false>;
+  }
+  return nullptr;
+}
+
+int round_spl(int need) {
+  for (int s : {2, 4, 6, 8, 12, 16})
+    if (need <= s) return s;
+  return 0;
+}
+
+int round_nvp(int nv) {
+  for (int s : {16, 32, 48, 64})
+    if (nv <= s) return s;
+  return 0;
+}
+
+int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
+           const float *J, int njmax, const float *D, const int32_t *state,
+           const int32_t *nefc, int quad, const float *y, int64_t ldy, float *x,
+           int64_t ldx, float *Hout, int nworld, unsigned flags, void *stream) {
+  if (!plan || !M || !y || !x || nworld < 0) return IM_ERR_ARG;
+  if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
+  if (ldM < plan->nM || ldy < plan->nv || ldx < plan->nv) return IM_ERR_STRIDE;
+  if (assemble && (!J || !D || !state || njmax < 0)) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  const int nv = plan->nv, nM = plan->nM;
+  const int nvp = round_nvp(nv);
+  int rc = 1, njpad = 0;
+  if (assemble) {
+    const int cap = std::min(64 * kPF / nv, 64);
+    while (rc * 2 <= cap) rc *= 2;
+    njpad = (njmax + 63) / 64 * 64 + 64;
+  }
+  const size_t lds_floats = (size_t)nM * 2 + 64 * 3 + (assemble ? njpad + 2 * (size_t)rc * nvp : 0);
+  const size_t lds_bytes = lds_floats * 4;
+  if (lds_bytes > 64 * 1024) return IM_ERR_UNSUPPORTED;
+  KernelFn fn = pick(assemble, plan->spl, nvp);
+  if (!fn) return IM_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(64), lds_bytes, (hipStream_t)stream, plan->dev, M,
+                     ldM, J, njmax, D, state, nefc, quad, y, ldy, x, ldx, Hout, rc,
+                     1.0f / (float)nv, njpad, flags);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+}  // namespace
+
+// Lays the plan out for the kernels: entry e of H sits in lane e % 64, register
+// e / 64; steps follow the plan's elimination order with one merge marker
+// between the groups and the trunk.
+int tree_plan_upload(im_tree_plan *pl) {
+  const int nv = pl->nv, nM = pl->nM;
+  pl->device_ready = false;
+  if (nv > 64 || nM > 65535 || pl->groups.size() > IM_MAX_GROUPS) return IM_ERR_UNSUPPORTED;
+  const int spl = round_spl((nM + 63) / 64);
+  if (!spl) return IM_ERR_UNSUPPORTED;
+  pl->spl = spl;
+  std::vector<char> in_trunk(nv, 0);
+  for (int i : pl->trunk) in_trunk[i] = 1;
+  std::vector<int32_t> slot_e(spl * 64, -1);
+  std::vector<uint32_t> slot_d(spl * 64, 0);
+  for (int b = 0; b < nv; ++b)
+    for (int q = 0; q < pl->rownnz[b]; ++q) {
+      const int e = pl->rowadr[b] + q;
+      const int a = pl->colind[e];
+      const int idx = (e / 64) * 64 + (e % 64);
+      slot_e[idx] = e | (in_trunk[b] ? (1 << 30) : 0);
+      slot_d[idx] = (uint32_t)a | ((uint32_t)b << 8) | ((uint32_t)(pl->rownnz[b] - 1) << 16) | ((uint32_t)q << 24);
+    }
+  std::vector<int4> steps;
+  std::vector<uint64_t> anc;
+  auto push = [&](int k, int gid) {
+    steps.push_back(make_int4(pl->rowadr[k], pl->rownnz[k] - 1, gid, k));
+    uint64_t m = 0;
+    for (int p = 0; p + 1 < pl->rownnz[k]; ++p) m |= 1ull << pl->colind[pl->rowadr[k] + p];
+    anc.push_back(m);
+  };
+  for (size_t j = 0; j < pl->groups.size(); ++j)
+    for (int k : pl->groups[j]) push(k, int(j));
+  if (!pl->trunk.empty()) {
+    steps.push_back(make_int4(0, 0, -1, 0));
+    anc.push_back(0);
+    for (auto it = pl->trunk.rbegin(); it != pl->trunk.rend(); ++it) push(*it, IM_MAX_GROUPS);
+  }
+  std::vector<int32_t> dof_d(64, -1);
+  for (int i = 0; i < nv; ++i)
+    dof_d[i] = pl->rowadr[i] | ((pl->rownnz[i] - 1) << 16) | (in_trunk[i] ? (1 << 24) : 0);
+
+  // one allocation, 16-byte aligned sections
+  auto align = [](size_t v) { return (v + 15) / 16 * 16; };
+  size_t off = 0;
+  const size_t o_steps = off; off = align(off + steps.size() * sizeof(int4));
+  const size_t o_anc = off;   off = align(off + anc.size() * sizeof(uint64_t));
+  const size_t o_se = off;    off = align(off + slot_e.size() * 4);
+  const size_t o_sd = off;    off = align(off + slot_d.size() * 4);
+  const size_t o_dof = off;   off = align(off + dof_d.size() * 4);
+  const size_t o_col = off;   off = align(off + (size_t)nM * 4);
+  std::vector<char> blob(off, 0);
+  std::memcpy(blob.data() + o_steps, steps.data(), steps.size() * sizeof(int4));
+  std::memcpy(blob.data() + o_anc, anc.data(), anc.size() * sizeof(uint64_t));
+  std::memcpy(blob.data() + o_se, slot_e.data(), slot_e.size() * 4);
+  std::memcpy(blob.data() + o_sd, slot_d.data(), slot_d.size() * 4);
+  std::memcpy(blob.data() + o_dof, dof_d.data(), dof_d.size() * 4);
+  std::memcpy(blob.data() + o_col, pl->colind.data(), (size_t)nM * 4);
+  IM_HIP_CHECK(hipGetDevice(&pl->device));
+  IM_HIP_CHECK(hipMalloc(&pl->dev_blob, off));
+  IM_HIP_CHECK(hipMemcpy(pl->dev_blob, blob.data(), off, hipMemcpyHostToDevice));
+  char *base = (char *)pl->dev_blob;
+  pl->dev.steps = (const int4 *)(base + o_steps);
+  pl->dev.anc = (const uint64_t *)(base + o_anc);
+  pl->dev.slot_e = (const int32_t *)(base + o_se);
+  pl->dev.slot_d = (const uint32_t *)(base + o_sd);
+  pl->dev.dof_d = (const int32_t *)(base + o_dof);
+  pl->dev.colind = (const int32_t *)(base + o_col);
+  pl->dev.nv = nv;
+  pl->dev.nM = nM;
+  pl->dev.nsteps = int(steps.size());
+  pl->dev.maxdepth = pl->maxdepth;
+  pl->dev.ngroups = int(pl->groups.size());
+  pl->device_ready = true;
+  return IM_OK;
+}
+
+}  // namespace im
+
+extern "C" {
+
+int im_tree_factor_solve(const im_tree_plan *plan, const float *M, int64_t ldM,
+                         const float *y, int64_t ldy, float *x, int64_t ldx,
+                         int nworld, void *stream) {
+  return im::launch(plan, false, M, ldM, nullptr, 0, nullptr, nullptr, nullptr, 0, y, ldy,
+                    x, ldx, nullptr, nworld, 0u, stream);
+}
+
+int im_assemble_tree_ldl_solve(const im_tree_plan *plan, const float *M, int64_t ldM,
+                               const float *J, int njmax, const float *D,
+                               const int32_t *state, const int32_t *nefc, int quad,
+                               const float *grad, int64_t ldg, float *x, int64_t ldx,
+                               float *Hout, int nworld, unsigned flags, void *stream) {
+  return im::launch(plan, true, M, ldM, J, njmax, D, state, nefc, quad, grad, ldg, x, ldx,
+                    Hout, nworld, flags, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,216 @@
+"""Seeded synthetic batches for the five benchmark shapes.
+
+There is no network and no MuJoCo in the build image, so every shape is
+generated: a dof tree (MuJoCo dof order, parent < child), a tree-sparse SPD
+``M`` in MuJoCo's CSR (row = ancestors root-first, diagonal last), constraint
+rows ``J`` supported on one root-to-leaf chain each, regularisers ``D``, a
+constraint ``state`` array (QUADRATIC = active) and a gradient.
+
+All draws use ``numpy.random.default_rng([seed, block])`` in fp64 over blocks of
+``BLOCK`` worlds and are cast to fp32, so the first ``n`` worlds of a batch do
+not depend on the batch size.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+
+QUADRATIC = 1  # mjtConstraintState.mjCNSTRSTATE_QUADRATIC
+BLOCK = 256
+
+
+def _chain(parent_of_first: int, first: int, n: int) -> list[int]:
+    return [parent_of_first] + list(range(first, first + n - 1))
+
+
+def ant_parents() -> list[int]:
+    # free joint (0..5) + four legs of two hinges hanging off dof 5
+    return [-1, 0, 1, 2, 3, 4, 5, 6, 5, 8, 5, 10, 5, 12]
+
+
+def humanoid_parents() -> list[int]:
+    # MuJoCo humanoid.xml order: root 6, abdomen z/y/x, right leg 6, left leg 6,
+    # right arm 3, left arm 3
+    return [-1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 8, 15, 16, 17, 18, 19, 5, 21, 22, 5, 24, 25]
+
+
+def g1_parents() -> list[int]:
+    p = [-1, 0, 1, 2, 3, 4]
+    p += _chain(5, 6, 6)  # left leg 6..11
+    p += _chain(5, 12, 6)  # right leg 12..17
+    p += _chain(5, 18, 3)  # waist 18..20
+    p += _chain(20, 21, 7)  # left arm 21..27
+    p += _chain(20, 28, 7)  # right arm 28..34
+    return p
+
+
+def snu_parents() -> list[int]:
+    # pelvis 6; legs (hip ball, knee, ankle ball, 3 foot hinges) 10 dofs each off
+    # dof 5; spine two balls (26..31) off dof 5; neck ball + head hinge off the
+    # spine end; arms (clavicle, shoulder balls, elbow, wrist ball) 10 each.
+    p = [-1, 0, 1, 2, 3, 4]
+    p += _chain(5, 6, 10)
+    p += _chain(5, 16, 10)
+    p += _chain(5, 26, 6)
+    p += _chain(31, 32, 4)
+    p += _chain(31, 36, 10)
+    p += _chain(31, 46, 10)
+    return p
+
+
+def stress_parents() -> list[int]:
+    # serial trunk of 64 dofs, an 8-dof side chain off trunk dofs 7, 15, ..., 63
+    p = [-1] + list(range(63))
+    first = 64
+    for t in range(7, 64, 8):
+        p += _chain(t, first, 8)
+        first += 8
+    return p
+
+
+def limbs_parents(limbs: int = 4, links: int = 6) -> list[int]:
+    """Free torso with ``limbs`` hinge chains (the reference's test model,
+    tests/test_tree_ldl.py:49-60)."""
+    p = [-1, 0, 1, 2, 3, 4]
+    for n in range(limbs):
+        p += _chain(5, 6 + n * links, links)
+    return p
+
+
+def branched_parents() -> list[int]:
+    """Free root with a hinge-hinge branch and a ball-slide branch, plus a second
+    free body (the reference's test model, tests/test_tree_ldl.py:22-36)."""
+    return [-1, 0, 1, 2, 3, 4, 5, 6, 5, 8, 9, 10, -1, 12, 13, 14, 15, 16]
+
+
+def chain_parents(hinges: int = 30) -> list[int]:
+    return [-1] + list(range(5 + hinges))
+
+
+def csr_from_parents(parent) -> tuple[np.ndarray, np.ndarray, np.ndarray]:
+    """MuJoCo's M CSR for a dof tree: ``rowadr, rownnz, colind`` (int32)."""
+    rowadr, rownnz, colind = [], [], []
+    for k in range(len(parent)):
+        chain = []
+        p = k
+        while p >= 0:
+            chain.append(p)
+            p = parent[p]
+        rowadr.append(len(colind))
+        rownnz.append(len(chain))
+        colind += chain[::-1]
+    return (np.asarray(rowadr, np.int32), np.asarray(rownnz, np.int32), np.asarray(colind, np.int32))
+
+
+@dataclass(frozen=True)
+class Shape:
+    name: str
+    parents: tuple
+    nefc: int
+    worlds: int
+    mass: tuple
+    armature: float
+    logd: tuple
+    p_active: float
+    iterations: int
+    seed: int
+    dense_rows: bool = False
+    nmuscle: int = 0
+    extra: dict = field(default_factory=dict)
+
+    @property
+    def nv(self) -> int:
+        return len(self.parents)
+
+
+SHAPES = {
+    "ant": Shape("ant", tuple(ant_parents()), 32, 64, (0.1, 2.0), 0.01, (-3.0, 3.0), 0.5, 1, 1000),
+    "humanoid": Shape("humanoid", tuple(humanoid_parents()), 64, 4096, (0.5, 8.0), 0.02, (-4.0, 4.0), 0.6, 3, 1001),
+    "g1": Shape("g1", tuple(g1_parents()), 96, 8192, (0.5, 8.0), 0.02, (-4.0, 4.0), 0.6, 1, 1002),
+    "snu": Shape("snu", tuple(snu_parents()), 128, 4096, (0.5, 8.0), 0.02, (-4.0, 4.0), 0.6, 1, 1003, nmuscle=284),
+    "stress": Shape("stress", tuple(stress_parents()), 256, 16384, (0.5, 8.0), 0.02, (-4.0, 4.0), 0.5, 3, 1004, dense_rows=True),
+}
+
+
+@dataclass
+class Batch:
+    shape: Shape
+    rowadr: np.ndarray
+    rownnz: np.ndarray
+    colind: np.ndarray
+    M: np.ndarray  # (nworld, nM) fp32, CSR values
+    J: np.ndarray  # (nworld, nefc, nv) fp32
+    D: np.ndarray  # (nworld, nefc) fp32
+    state: np.ndarray  # (iterations, nworld, nefc) int32
+    nefc: np.ndarray  # (nworld,) int32
+    grad: np.ndarray  # (nworld, nv) fp32
+
+    @property
+    def nworld(self) -> int:
+        return self.M.shape[0]
+
+
+def chain_mask(parent) -> np.ndarray:
+    """mask[k, i] = 1 when i is k or one of k's ancestors."""
+    nv = len(parent)
+    mask = np.zeros((nv, nv), dtype=bool)
+    for k in range(nv):
+        p = k
+        while p >= 0:
+            mask[k, p] = True
+            p = parent[p]
+    return mask
+
+
+def make_batch(shape: Shape | str, nworld: int | None = None, *, ragged_nefc: bool = False) -> Batch:
+    if isinstance(shape, str):
+        shape = SHAPES[shape]
+    nworld = shape.worlds if nworld is None else int(nworld)
+    nv, nefc = shape.nv, shape.nefc
+    parent = list(shape.parents)
+    rowadr, rownnz, colind = csr_from_parents(parent)
+    rowi = np.repeat(np.arange(nv), rownnz)
+    mask = chain_mask(parent)
+    nM = colind.size
+    M = np.empty((nworld, nM), np.float32)
+    J = np.empty((nworld, nefc, nv), np.float32)
+    D = np.empty((nworld, nefc), np.float32)
+    state = np.empty((shape.iterations, nworld, nefc), np.int32)
+    grad = np.empty((nworld, nv), np.float32)
+    nefc_w = np.full((nworld,), nefc, np.int32)
+    for b0 in range(0, nworld, BLOCK):
+        rng = np.random.default_rng([shape.seed, b0 // BLOCK])
+        nb = BLOCK
+        mass = rng.uniform(shape.mass[0], shape.mass[1], (nb, nv))
+        V = rng.standard_normal((nb, nv, nv)) * mask[None]
+        dense = np.einsum("wk,wki,wkj->wij", mass, V, V, optimize=True)
+        dense[:, np.arange(nv), np.arange(nv)] += shape.armature
+        body = rng.integers(0, nv, (nb, nefc))
+        rows = rng.standard_normal((nb, nefc, nv))
+        if not shape.dense_rows:
+            rows *= mask[body]
+        logd = rng.uniform(shape.logd[0], shape.logd[1], (nb, nefc))
+        act = rng.random((shape.iterations, nb, nefc)) < shape.p_active
+        g = rng.standard_normal((nb, nv))
+        ragged = rng.integers(0, nefc + 1, (nb,))
+        n = min(nb, nworld - b0)
+        M[b0 : b0 + n] = dense[:n, rowi, colind]
+        J[b0 : b0 + n] = rows[:n]
+        D[b0 : b0 + n] = 10.0 ** logd[:n]
+        state[:, b0 : b0 + n] = np.where(act[:, :n], QUADRATIC, 0)
+        grad[b0 : b0 + n] = g[:n]
+        if ragged_nefc:
+            nefc_w[b0 : b0 + n] = ragged[:n]
+    return Batch(shape, rowadr, rownnz, colind, M, J, D, state, nefc_w, grad)
+
+
+def dense_from_csr(values: np.ndarray, rowadr, rownnz, colind) -> np.ndarray:
+    """Symmetric dense (nworld, nv, nv) fp64 matrix from CSR lower-triangle values."""
+    nv = len(rowadr)
+    rowi = np.repeat(np.arange(nv), rownnz)
+    out = np.zeros((values.shape[0], nv, nv), np.float64)
+    out[:, rowi, colind] = values
+    out[:, colind, rowi] = values
+    return out

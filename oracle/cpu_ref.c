@@ -1,0 +1,262 @@
+/* CPU oracle: fp32 restatement of the reference's numeric statements for the
+ * assemble + tree L'DL + solve path.  TEST INFRASTRUCTURE ONLY -- nothing in the
+ * shipped library links or calls this file; it is the checker the HIP kernels
+ * are compared with, and the timed "cpu_baseline" of the benchmark.
+ *
+ * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off -fopenmp).  Every fused
+ * multiply-add is written as fmaf(); everything else rounds once per operator.
+ *
+ * Rounding convention of the tree L'DL.  The reference writes plain expressions
+ *     t = t - a * b * c;   s = s - a * b;
+ * (src/instantmimic/utils/mjw_kernels/tree_ldl.py:227-231, 269, 302) and leaves
+ * contraction to the compiler.  NVRTC (fmad on by default) and clang both
+ * contract the multiply that feeds the subtraction, so the statements evaluate as
+ *     t = fmaf(-(a * b), c, t);   s = fmaf(-a, b, s);
+ * which is what this file does.  Reciprocals are correctly rounded 1.0f / x.
+ */
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+int orc_max_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+void orc_set_threads(int n) {
+#ifdef _OPENMP
+  if (n > 0) omp_set_num_threads(n);
+#else
+  (void)n;
+#endif
+}
+
+/* H = M + sum over QUADRATIC rows of D * J' J on M's CSR entries.
+ * Per entry (a = column = ancestor dof, b = row dof, a <= b) the rows are summed
+ * in ascending order with v = fmaf(J[r][a] * Dc[r], J[r][b], v), Dc = D for a
+ * QUADRATIC row and 0 otherwise (sparse_hessian.py:589, 622-629). */
+static void assemble_world(int nv, int nM, const int *rowi, const int *colind,
+                           const float *M, const float *J, const float *D,
+                           const int *state, int nefc, int quad, float *H) {
+  for (int e = 0; e < nM; ++e) H[e] = M[e];
+  for (int r = 0; r < nefc; ++r) {
+    const float dc = state[r] == quad ? D[r] : 0.0f;
+    const float *Jr = J + (size_t)r * nv;
+    for (int e = 0; e < nM; ++e) {
+      const int a = colind[e], b = rowi[e];
+      H[e] = fmaf(Jr[a] * dc, Jr[b], H[e]);
+    }
+  }
+}
+
+int orc_assemble_csr(int nworld, int nv, int nM, const int *rowi,
+                     const int *colind, const float *M, const float *J,
+                     int njmax, const float *D, const int *state,
+                     const int *nefc, int quad, float *H) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    int n = nefc ? nefc[w] : njmax;
+    if (n > njmax) n = njmax;
+    assemble_world(nv, nM, rowi, colind, M + (size_t)w * nM,
+                   J + (size_t)w * njmax * nv, D + (size_t)w * njmax,
+                   state + (size_t)w * njmax, n, quad, H + (size_t)w * nM);
+  }
+  return 0;
+}
+
+/* Static description of one tree plan (tree_ldl.py:47-56 plus the CSR). */
+typedef struct {
+  int nv, nM, ngroups, ntrunk, nte; /* nte = trunk CSR entries */
+  const int *rowadr, *rownnz, *colind;
+  const int *gptr, *gdofs, *trunk;
+  int *slot;     /* CSR entry -> trunk entry slot or -1 */
+  int *dslot;    /* dof -> trunk dof slot or -1 */
+  char *touch_m; /* [ngroups][nte]  */
+  char *touch_s; /* [ngroups][ntrunk] */
+} plan_t;
+
+static void plan_init(plan_t *p) {
+  p->slot = (int *)malloc(sizeof(int) * (p->nM + 1));
+  p->dslot = (int *)malloc(sizeof(int) * (p->nv + 1));
+  for (int e = 0; e < p->nM; ++e) p->slot[e] = -1;
+  for (int i = 0; i < p->nv; ++i) p->dslot[i] = -1;
+  int n = 0;
+  for (int t = 0; t < p->ntrunk; ++t) {
+    const int i = p->trunk[t];
+    p->dslot[i] = t;
+    for (int e = p->rowadr[i]; e < p->rowadr[i] + p->rownnz[i]; ++e) p->slot[e] = n++;
+  }
+  p->nte = n;
+  p->touch_m = (char *)calloc((size_t)p->ngroups * (n + 1), 1);
+  p->touch_s = (char *)calloc((size_t)p->ngroups * (p->ntrunk + 1), 1);
+  /* tree_ldl.py:236-245 */
+  for (int j = 0; j < p->ngroups; ++j)
+    for (int g = p->gptr[j]; g < p->gptr[j + 1]; ++g) {
+      const int k = p->gdofs[g];
+      for (int q = 0; q < p->rownnz[k] - 1; ++q) {
+        const int anc = p->colind[p->rowadr[k] + q];
+        if (p->dslot[anc] < 0) continue;
+        p->touch_s[j * p->ntrunk + p->dslot[anc]] = 1;
+        for (int c = 0; c <= q; ++c) p->touch_m[j * n + p->slot[p->rowadr[anc] + c]] = 1;
+      }
+    }
+}
+
+static void plan_free(plan_t *p) {
+  free(p->slot);
+  free(p->dslot);
+  free(p->touch_m);
+  free(p->touch_s);
+}
+
+/* One world.  work holds m[nM], s[nv], d[nv], xs[nv], a[ngroups*nte],
+ * b[ngroups*ntrunk].  ld (optional) receives the factor: scaled rows of L with
+ * the unscaled pivot on the diagonal. */
+static void tree_world(const plan_t *p, const float *H, const float *y, float *x,
+                       float *work, float *ld) {
+  const int nv = p->nv, nM = p->nM, nte = p->nte, nt = p->ntrunk;
+  float *m = work, *s = m + nM, *d = s + nv, *xs = d + nv;
+  float *a = xs + nv, *b = a + (size_t)p->ngroups * nte;
+  memcpy(m, H, sizeof(float) * nM);
+  memcpy(s, y, sizeof(float) * nv);
+  for (int i = 0; i < p->ngroups * nte; ++i) a[i] = 0.0f;
+  for (int i = 0; i < p->ngroups * nt; ++i) b[i] = 0.0f;
+  /* parts, forward (tree_ldl.py:215-232, 252-259) */
+  for (int j = 0; j < p->ngroups; ++j) {
+    float *aj = a + (size_t)j * nte, *bj = b + (size_t)j * nt;
+    for (int g = p->gptr[j]; g < p->gptr[j + 1]; ++g) {
+      const int k = p->gdofs[g], start = p->rowadr[k], count = p->rownnz[k] - 1;
+      const float dk = 1.0f / m[start + count];
+      d[k] = dk;
+      for (int pp = 0; pp < count; ++pp) {
+        const int anc = p->colind[start + pp];
+        for (int q = 0; q <= pp; ++q) {
+          const int e = p->rowadr[anc] + q;
+          float *t = p->dslot[anc] >= 0 ? &aj[p->slot[e]] : &m[e];
+          *t = fmaf(-(m[start + pp] * m[start + q]), dk, *t);
+        }
+      }
+      for (int pp = 0; pp < count; ++pp) m[start + pp] = m[start + pp] * dk;
+      for (int pp = 0; pp < count; ++pp) {
+        const int anc = p->colind[start + pp];
+        float *t = p->dslot[anc] >= 0 ? &bj[p->dslot[anc]] : &s[anc];
+        *t = fmaf(-m[start + pp], s[k], *t);
+      }
+    }
+  }
+  /* trunk (tree_ldl.py:274-305) */
+  for (int t = 0; t < nt; ++t) {
+    const int i = p->trunk[t];
+    for (int e = p->rowadr[i]; e < p->rowadr[i] + p->rownnz[i]; ++e) {
+      float v = H[e];
+      for (int j = 0; j < p->ngroups; ++j)
+        if (p->touch_m[j * nte + p->slot[e]]) v = v + a[(size_t)j * nte + p->slot[e]];
+      m[e] = v;
+    }
+    float v = y[i];
+    for (int j = 0; j < p->ngroups; ++j)
+      if (p->touch_s[j * nt + t]) v = v + b[(size_t)j * nt + t];
+    s[i] = v;
+  }
+  for (int t = nt - 1; t >= 0; --t) {
+    const int k = p->trunk[t], start = p->rowadr[k], count = p->rownnz[k] - 1;
+    const float dk = 1.0f / m[start + count];
+    d[k] = dk;
+    for (int pp = 0; pp < count; ++pp) {
+      const int anc = p->colind[start + pp];
+      for (int q = 0; q <= pp; ++q) {
+        float *tt = &m[p->rowadr[anc] + q];
+        *tt = fmaf(-(m[start + pp] * m[start + q]), dk, *tt);
+      }
+    }
+    for (int pp = 0; pp < count; ++pp) m[start + pp] = m[start + pp] * dk;
+    for (int pp = 0; pp < count; ++pp) {
+      float *tt = &s[p->colind[start + pp]];
+      *tt = fmaf(-m[start + pp], s[k], *tt);
+    }
+  }
+  for (int t = 0; t < nt; ++t) {
+    const int i = p->trunk[t], start = p->rowadr[i];
+    float u = s[i] * d[i];
+    for (int pp = 0; pp < p->rownnz[i] - 1; ++pp)
+      u = fmaf(-m[start + pp], xs[p->colind[start + pp]], u);
+    xs[i] = u;
+  }
+  /* parts, backward (tree_ldl.py:262-272) */
+  for (int j = 0; j < p->ngroups; ++j)
+    for (int g = p->gptr[j + 1] - 1; g >= p->gptr[j]; --g) {
+      const int i = p->gdofs[g], start = p->rowadr[i];
+      float v = s[i] * d[i];
+      for (int pp = 0; pp < p->rownnz[i] - 1; ++pp)
+        v = fmaf(-m[start + pp], xs[p->colind[start + pp]], v);
+      xs[i] = v;
+    }
+  memcpy(x, xs, sizeof(float) * nv);
+  if (ld) memcpy(ld, m, sizeof(float) * nM);
+}
+
+static size_t work_floats(const plan_t *p) {
+  return (size_t)p->nM + 3 * (size_t)p->nv +
+         (size_t)p->ngroups * (p->nte + p->ntrunk) + 8;
+}
+
+/* x = (L'DL)^-1 y for every world; H (nworld, nM) in M's CSR layout. */
+int orc_tree_ldl_solve(int nworld, int nv, int nM, const int *rowadr,
+                       const int *rownnz, const int *colind, int ngroups,
+                       const int *gptr, const int *gdofs, int ntrunk,
+                       const int *trunk, const float *H, const float *y,
+                       float *x, float *ld) {
+  plan_t p = {nv, nM, ngroups, ntrunk, 0, rowadr, rownnz, colind, gptr, gdofs, trunk, 0, 0, 0, 0};
+  plan_init(&p);
+  const size_t wf = work_floats(&p);
+#pragma omp parallel
+  {
+    float *work = (float *)malloc(sizeof(float) * wf);
+#pragma omp for schedule(static)
+    for (int w = 0; w < nworld; ++w)
+      tree_world(&p, H + (size_t)w * nM, y + (size_t)w * nv, x + (size_t)w * nv,
+                 work, ld ? ld + (size_t)w * nM : 0);
+    free(work);
+  }
+  plan_free(&p);
+  return 0;
+}
+
+/* The fused path: assemble H on the CSR pattern, factor and solve with y = grad.
+ * Hout (optional) receives the assembled H. */
+int orc_assemble_tree_ldl_solve(int nworld, int nv, int nM, const int *rowadr,
+                                const int *rownnz, const int *colind,
+                                const int *rowi, int ngroups, const int *gptr,
+                                const int *gdofs, int ntrunk, const int *trunk,
+                                const float *M, const float *J, int njmax,
+                                const float *D, const int *state,
+                                const int *nefc, int quad, const float *grad,
+                                float *x, float *Hout) {
+  plan_t p = {nv, nM, ngroups, ntrunk, 0, rowadr, rownnz, colind, gptr, gdofs, trunk, 0, 0, 0, 0};
+  plan_init(&p);
+  const size_t wf = work_floats(&p);
+#pragma omp parallel
+  {
+    float *work = (float *)malloc(sizeof(float) * (wf + nM));
+    float *H = work + wf;
+#pragma omp for schedule(static)
+    for (int w = 0; w < nworld; ++w) {
+      int n = nefc ? nefc[w] : njmax;
+      if (n > njmax) n = njmax;
+      assemble_world(nv, nM, rowi, colind, M + (size_t)w * nM,
+                     J + (size_t)w * njmax * nv, D + (size_t)w * njmax,
+                     state + (size_t)w * njmax, n, quad, H);
+      if (Hout) memcpy(Hout + (size_t)w * nM, H, sizeof(float) * nM);
+      tree_world(&p, H, grad + (size_t)w * nv, x + (size_t)w * nv, work, 0);
+    }
+    free(work);
+  }
+  plan_free(&p);
+  return 0;
+}

@@ -1,0 +1,148 @@
+"""ctypes front end of ``cpu_ref.c`` plus fp64 NumPy references (oracle only).
+
+Pinning status
+
+* ``assemble_csr``            pinned: fp64 ``einsum`` of ``M + J' diag(D active) J``
+                              gathered on the CSR entries (tests/test_oracle.py).
+* ``tree_ldl_solve``          pinned: fp64 ``numpy.linalg.solve`` on well-conditioned
+                              matrices (the reference's own check,
+                              tests/test_tree_ldl.py:119-120), the invariant
+                              ``L' D L == H`` rebuilt from the returned factor, brute force
+                              Gaussian elimination on tiny trees, and independence of the
+                              result (to rounding) from the number of groups.
+* ``assemble_tree_ldl_solve`` composition of the two above; pinned through them.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+def build() -> str:
+    subprocess.run(["make", "-s", "-C", _HERE], check=True)
+    return os.path.join(_HERE, "_build", "liboracle.so")
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        path = os.path.join(_HERE, "_build", "liboracle.so")
+        if not os.path.exists(path):
+            build()
+        _LIB = ctypes.CDLL(path)
+    return _LIB
+
+
+def _i(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def _f(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p) if a is not None else None
+
+
+def max_threads() -> int:
+    return int(lib().orc_max_threads())
+
+
+def set_threads(n: int) -> None:
+    lib().orc_set_threads(int(n))
+
+
+def _plan_arrays(plan):
+    gptr = [0]
+    gd = []
+    for g in plan.groups:
+        gd += list(g)
+        gptr.append(len(gd))
+    return _i(gptr), _i(gd if gd else [0]), _i(plan.trunk if plan.trunk else [0])
+
+
+def rows_of(rownnz):
+    return np.repeat(np.arange(len(rownnz)), np.asarray(rownnz)).astype(np.int32)
+
+
+def assemble_csr(rowadr, rownnz, colind, M, J, D, state, nefc=None, quad=1):
+    M, J, D = _f(M), _f(J), _f(D)
+    state = _i(state)
+    nworld, nM = M.shape
+    njmax, nv = J.shape[1], J.shape[2]
+    H = np.empty_like(M)
+    ne = _i(nefc) if nefc is not None else None
+    lib().orc_assemble_csr(
+        nworld, nv, nM, _p(rows_of(rownnz)), _p(_i(colind)), _p(M), _p(J), njmax, _p(D), _p(state), _p(ne), quad, _p(H)
+    )
+    return H
+
+
+def tree_ldl_solve(rowadr, rownnz, colind, plan, H, y, want_factor=False):
+    H, y = _f(H), _f(y)
+    nworld, nM = H.shape
+    nv = y.shape[1]
+    gptr, gd, trunk = _plan_arrays(plan)
+    x = np.empty_like(y)
+    ld = np.empty_like(H) if want_factor else None
+    lib().orc_tree_ldl_solve(
+        nworld, nv, nM, _p(_i(rowadr)), _p(_i(rownnz)), _p(_i(colind)), len(plan.groups), _p(gptr), _p(gd),
+        len(plan.trunk), _p(trunk), _p(H), _p(y), _p(x), _p(ld),
+    )  # fmt: skip
+    return (x, ld) if want_factor else x
+
+
+def assemble_tree_ldl_solve(rowadr, rownnz, colind, plan, M, J, D, state, nefc, grad, quad=1, want_h=False):
+    M, J, D, grad = _f(M), _f(J), _f(D), _f(grad)
+    state = _i(state)
+    nworld, nM = M.shape
+    njmax, nv = J.shape[1], J.shape[2]
+    gptr, gd, trunk = _plan_arrays(plan)
+    x = np.empty_like(grad)
+    H = np.empty_like(M) if want_h else None
+    ne = _i(nefc) if nefc is not None else None
+    lib().orc_assemble_tree_ldl_solve(
+        nworld, nv, nM, _p(_i(rowadr)), _p(_i(rownnz)), _p(_i(colind)), _p(rows_of(rownnz)), len(plan.groups),
+        _p(gptr), _p(gd), len(plan.trunk), _p(trunk), _p(M), _p(J), njmax, _p(D), _p(state), _p(ne), quad,
+        _p(grad), _p(x), _p(H),
+    )  # fmt: skip
+    return (x, H) if want_h else x
+
+
+# ---------------------------------------------------------------- fp64 references
+
+
+def dense_from_csr(values, rowadr, rownnz, colind):
+    nv = len(rowadr)
+    rowi = rows_of(rownnz)
+    out = np.zeros((values.shape[0], nv, nv), np.float64)
+    out[:, rowi, colind] = values
+    out[:, colind, rowi] = values
+    return out
+
+
+def assemble_dense64(rowadr, rownnz, colind, M, J, D, state, nefc=None, quad=1):
+    """fp64 dense ``M + J' diag(D [state == quad]) J`` (all rows, no pattern)."""
+    J64 = np.asarray(J, np.float64)
+    w = np.where(np.asarray(state) == quad, np.asarray(D, np.float64), 0.0)
+    if nefc is not None:
+        w = w * (np.arange(J64.shape[1])[None, :] < np.asarray(nefc)[:, None])
+    return dense_from_csr(np.asarray(M, np.float64), rowadr, rownnz, colind) + np.einsum("wri,wr,wrj->wij", J64, w, J64)
+
+
+def solve64(Hd, y):
+    return np.linalg.solve(Hd, np.asarray(y, np.float64)[..., None])[..., 0]
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
