@@ -51,6 +51,7 @@ struct im_tree_plan {
   void *dev_blob = nullptr;
   im::TreeDev dev{};
   int spl = 0;  // H slots per lane
+  const void *row16 = nullptr;  // generated kernel for this structure, if one was built
 };
 
 namespace im {

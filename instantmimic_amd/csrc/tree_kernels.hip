@@ -27,9 +27,50 @@
 #include <cstring>
 
 #include "common.h"
+#include "tree_row16.h"
+#include <cstdlib>
+#include <vector>
 
 namespace im {
+namespace gen {
 namespace {
+std::vector<const Row16Entry *> &registry() {
+  static std::vector<const Row16Entry *> r;
+  return r;
+}
+}  // namespace
+Row16Register::Row16Register(const Row16Entry *e) { registry().push_back(e); }
+const Row16Entry *find_row16(uint64_t key) {
+  for (const Row16Entry *e : registry())
+    if (e->key == key) return e;
+  return nullptr;
+}
+}  // namespace gen
+
+namespace {
+
+// FNV-1a over the CSR structure and the plan; the generator computes the same key
+// (instantmimic_amd/codegen/tree_row16.py: structure_key).
+uint64_t tree_key(const im_tree_plan &pl) {
+  uint64_t h = 0xCBF29CE484222325ull;
+  auto mix = [&](uint32_t v) {
+    h ^= v;
+    h *= 0x100000001B3ull;
+  };
+  mix(pl.nv);
+  for (int v : pl.rowadr) mix(v);
+  for (int v : pl.rownnz) mix(v);
+  mix(pl.nM);
+  for (int v : pl.colind) mix(v);
+  mix((uint32_t)pl.groups.size());
+  for (const auto &g : pl.groups) {
+    mix((uint32_t)g.size());
+    for (int v : g) mix(v);
+  }
+  mix((uint32_t)pl.trunk.size());
+  for (int v : pl.trunk) mix(v);
+  return h;
+}
 
 constexpr int kPF = 16;  // global-load registers per lane and chunk (1024 floats)
 
@@ -290,11 +331,25 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
            const float *J, int njmax, const float *D, const int32_t *state,
            const int32_t *nefc, int quad, const float *y, int64_t ldy, float *x,
            int64_t ldx, float *Hout, int nworld, unsigned flags, void *stream) {
-  if (!plan || !M || !y || !x || nworld < 0) return IM_ERR_ARG;
+  if (!plan || nworld < 0) return IM_ERR_ARG;
   if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
+  if (nworld == 0) return IM_OK;
+  if (!M || !y || !x) return IM_ERR_ARG;
   if (ldM < plan->nM || ldy < plan->nv || ldx < plan->nv) return IM_ERR_STRIDE;
   if (assemble && (!J || !D || !state || njmax < 0)) return IM_ERR_ARG;
   if (nworld == 0) return IM_OK;
+  if (plan->row16) {
+    const auto *e = (const gen::Row16Entry *)plan->row16;
+    void *args[] = {&M, &ldM, &J, &njmax, &D, &state, &nefc, &quad, &y, &ldy, &x, &ldx, &Hout, &nworld, &flags};
+    // the fused kernel copies J in 16-byte pieces: every world's block must be 16-byte aligned
+    const bool aligned = !assemble || ((((size_t)njmax * plan->nv) % 4 == 0) && ((uintptr_t)J % 16 == 0));
+    if (aligned) {
+      IM_HIP_CHECK(hipLaunchKernel(assemble ? e->fused : e->solve, dim3((nworld + 3) / 4),
+                                   dim3(64), args, assemble ? e->lds_bytes : 0,
+                                   (hipStream_t)stream));
+      return IM_OK;
+    }
+  }
   const int nv = plan->nv, nM = plan->nM;
   const int nvp = round_nvp(nv);
   int rc = 1, njpad = 0;
@@ -390,6 +445,14 @@ int tree_plan_upload(im_tree_plan *pl) {
   pl->dev.maxdepth = pl->maxdepth;
   pl->dev.ngroups = int(pl->groups.size());
   pl->device_ready = true;
+  // a kernel generated for exactly this structure and plan, unless the generic one is forced
+  const char *force = std::getenv("IMHIP_TREE_KERNEL");
+  pl->row16 = (force && std::strcmp(force, "generic") == 0) ? nullptr : (const void *)gen::find_row16(tree_key(*pl));
+  if (pl->row16) {
+    const auto *e = (const gen::Row16Entry *)pl->row16;
+    if (e->lds_bytes > 64 * 1024)
+      IM_HIP_CHECK(hipFuncSetAttribute(e->fused, hipFuncAttributeMaxDynamicSharedMemorySize, e->lds_bytes));
+  }
   return IM_OK;
 }
 

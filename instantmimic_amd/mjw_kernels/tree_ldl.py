@@ -35,6 +35,10 @@ class TreeLdlPlan:
     dense_cost: int
 
 
+class UnsupportedShape(RuntimeError):
+    """The tree is valid but outside what the device kernels are built for."""
+
+
 class _PlanHandle:
     """Owns one ``im_tree_plan``."""
 
@@ -153,7 +157,7 @@ def scratch_for_plan(structure, plan: TreeLdlPlan, device: Any) -> TreeFactorSol
     if built != plan:
         raise ValueError("plan does not belong to this structure")
     if not handle.info().device_ready:
-        raise RuntimeError("shape outside the device kernels' limits (nv <= 64, nM <= 1024)")
+        raise UnsupportedShape("shape outside the device kernels' limits (nv <= 64, nM <= 1024)")
     return TreeFactorSolveScratch(kernel=handle, groups=len(plan.groups), cuda=True, plan=plan)
 
 
@@ -176,7 +180,7 @@ def create_tree_factor_solve_scratch(m: Any, device: Any = None) -> TreeFactorSo
             device = "cuda"
     try:
         return scratch_for_plan(structure, plan, device)
-    except RuntimeError:
+    except UnsupportedShape:
         return None
 
 

@@ -1,0 +1,117 @@
+"""The C ABI without a GPU: the library loads, exports what the header declares,
+and its host planner equals the oracle's restatement of the reference planner."""
+
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from instantmimic_amd import _lib, synth
+from instantmimic_amd.mjw_kernels import tree_ldl as T
+from oracle import planner as P
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    names = set()
+    inc = os.path.join(ROOT, "include")
+    for fn in os.listdir(inc):
+        if fn.endswith(".h"):
+            text = open(os.path.join(inc, fn)).read()
+            text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+            names |= set(re.findall(r"\b(im_[a-z0-9_]+)\s*\(", text))
+    return names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.lib()
+    declared = _declared_symbols()
+    assert declared, "no declarations found"
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    assert lib.im_version() >= 100
+    assert lib.im_status_string(_lib.IM_ERR_STRUCTURE)
+
+
+def _same(a, b):
+    return (a.groups, a.trunk, a.span, a.dense_cost) == (b.groups, b.trunk, b.span, b.dense_cost)
+
+
+def test_host_planner_equals_the_oracle_on_the_benchmark_trees():
+    for name, shape in synth.SHAPES.items():
+        st = T.tree_ldl_structure(*synth.csr_from_parents(shape.parents))
+        assert st == P.tree_ldl_structure(*st)
+        for g in (1, 2, 3, 4):
+            assert _same(T.plan_tree_ldl(*st, g), P.plan_tree_ldl(*st, g)), (name, g)
+        best = T.best_tree_ldl_plan(*st)
+        assert _same(best, P.best_tree_ldl_plan(*st)), name
+        assert T.tree_ldl_beats_dense(best) == P.tree_ldl_beats_dense(P.best_tree_ldl_plan(*st))
+        assert list(T.elimination_order(best)) == P.elimination_order(P.best_tree_ldl_plan(*st))
+
+
+def test_host_planner_equals_the_oracle_on_random_forests():
+    rng = np.random.default_rng(5)
+    for _ in range(200):
+        nv = int(rng.integers(1, 64))
+        parent = [-1] + [int(rng.integers(-1 if rng.random() < 0.1 else 0, k)) for k in range(1, nv)]
+        st = T.tree_ldl_structure(*synth.csr_from_parents(parent))
+        assert st is not None
+        for g in (0, 1, 2, 3, 4):
+            a = T.plan_tree_ldl(*st, g) if g else T.best_tree_ldl_plan(*st)
+            b = P.plan_tree_ldl(*st, g) if g else P.best_tree_ldl_plan(*st)
+            assert _same(a, b), (parent, g)
+
+
+def test_limbs_plan_invariants_through_the_c_abi():
+    # reference: tests/test_tree_ldl.py:123-145
+    st = T.tree_ldl_structure(*synth.csr_from_parents(synth.limbs_parents()))
+    single, split = T.plan_tree_ldl(*st, 1), T.plan_tree_ldl(*st, 4)
+    assert not single.trunk and split.trunk == tuple(range(6))
+    assert sorted(len(g) for g in split.groups) == [6, 6, 6, 6] and split.span < single.span
+    chain = T.tree_ldl_structure(*synth.csr_from_parents(synth.chain_parents(30)))
+    assert T.tree_ldl_beats_dense(T.best_tree_ldl_plan(*st))
+    assert not T.tree_ldl_beats_dense(T.best_tree_ldl_plan(*chain))
+
+
+def test_structure_check_rejects_what_the_reference_rejects():
+    # reference: tests/test_tree_ldl.py:148-161
+    rowadr, rownnz, colind = synth.csr_from_parents(synth.branched_parents())
+    assert T.tree_ldl_structure(rowadr, rownnz, colind) is not None
+    k = int(np.flatnonzero(rownnz > 2)[-1])
+    broken = colind.copy()
+    s = rowadr[k]
+    broken[s], broken[s + 1] = broken[s + 1], broken[s]
+    assert T.tree_ldl_structure(rowadr, rownnz, broken) is None
+    shifted = colind.copy()
+    shifted[rowadr[k] + rownnz[k] - 1] = 0
+    assert T.tree_ldl_structure(rowadr, rownnz, shifted) is None
+    assert T.tree_ldl_structure(rowadr, rownnz, colind[:-1]) is None
+    assert T.tree_ldl_structure([], [], []) is None
+    zero = rownnz.copy()
+    zero[3] = 0
+    assert T.tree_ldl_structure(rowadr, zero, colind) is None
+
+
+def test_status_codes():
+    lib = _lib.lib()
+    rowadr, rownnz, colind = synth.csr_from_parents(synth.ant_parents())
+    handle = C.c_void_p()
+    args = (rowadr.ctypes.data, rownnz.ctypes.data, colind.ctypes.data, int(colind.size))
+    assert lib.im_tree_plan_create(14, *args, 5, 1, C.byref(handle)) == _lib.IM_ERR_ARG
+    assert lib.im_tree_plan_create(14, None, None, None, 0, 0, 1, C.byref(handle)) == _lib.IM_ERR_ARG
+    bad = colind.copy()
+    bad[-1] = 0
+    assert lib.im_tree_plan_create(14, rowadr.ctypes.data, rownnz.ctypes.data, bad.ctypes.data, int(bad.size), 0, 1, C.byref(handle)) == _lib.IM_ERR_STRUCTURE
+    assert lib.im_tree_plan_create(14, *args, 0, 1, C.byref(handle)) == _lib.IM_OK
+    info = _lib.TreePlanInfo()
+    assert lib.im_tree_plan_get_info(handle, C.byref(info)) == _lib.IM_OK
+    assert (info.nv, info.nM, info.ngroups, info.span, info.device_ready) == (14, 81, 4, 198, 0)
+    # a host-only plan cannot launch
+    assert lib.im_tree_factor_solve(handle, 1, 81, 1, 14, 1, 14, 1, None) == _lib.IM_ERR_UNSUPPORTED
+    lib.im_tree_plan_destroy(handle)
+    with pytest.raises(_lib.ImhipError):
+        _lib.check(_lib.IM_ERR_STRIDE, "x")
