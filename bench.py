@@ -24,9 +24,12 @@ if ROOT not in sys.path:
 
 METRIC = "Hessian assemble+LDL+solve worlds/s, humanoid nv=27×4096; % HBM roofline"
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by a
-# copy kernel of known size; see profiles/.  None until measured.
-TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per launch of the fused kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain
+# 64 MiB device copy in the same run (FETCH_SIZE reads 32781 KiB for it, WRITE_SIZE 65536):
+#   (17494.05 * 65536 / 32781.22 + 448.0 * 65536 / 65536) KiB
+# Recorded in profiles/tree_row16_humanoid_pmc.txt.
+TRAFFIC_BYTES_PER_LAUNCH = int((17494.05 * 65536 / 32781.22 + 448.0) * 1024)
 
 
 def algorithmic_bytes(nv: int, nM: int, nefc: int) -> int:
@@ -74,6 +77,14 @@ def main() -> int:
     ap.add_argument("--sets", type=int, default=16, help="distinct input sets rotated over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying hipGraphs")
+    ap.add_argument(
+        "--copy-calibration",
+        type=int,
+        default=0,
+        metavar="N",
+        help="also run N plain device copies of 64 MiB (rotating buffers) so that a rocprofv3 --pmc run of this "
+        "command shows what FETCH_SIZE / WRITE_SIZE read for a kernel of known traffic",
+    )
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (worlds would shard contiguously, no exchange)", file=sys.stderr)
@@ -90,6 +101,16 @@ def main() -> int:
         return 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.copy_calibration:
+        # 8 source/destination pairs of 64 MiB: 1 GiB in rotation, nothing stays in the last-level cache
+        pairs_ = [(torch.empty(16 << 20, device=dev), torch.ones(16 << 20, device=dev)) for _ in range(8)]
+        torch.cuda.synchronize()
+        for i in range(args.copy_calibration):
+            d_, s_ = pairs_[i % 8]
+            d_.copy_(s_)
+        torch.cuda.synchronize()
+        del pairs_
 
     shape = synth.SHAPES["humanoid"]
     batch = synth.make_batch(shape)
@@ -157,11 +178,17 @@ def main() -> int:
 
     run(args.warmup)
     torch.cuda.synchronize()
+    # HIP events on the stream the kernels are launched on (torch's current stream is the
+    # one handed to the C ABI), around the timed region
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    ev0.record()
     run(args.steps)
+    ev1.record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     value = args.steps * iters * nworld / elapsed
+    region_s = ev0.elapsed_time(ev1) * 1e-3
 
     # per-launch kernel duration with HIP events on the launch stream
     nev = min(args.steps, 64)
@@ -176,7 +203,10 @@ def main() -> int:
             pairs.append((a, b))
     torch.cuda.synchronize()
     durs = np.array([a.elapsed_time(b) for a, b in pairs]) * 1e-3  # seconds
-    kernel_s = float(np.mean(durs))
+    # average launch duration over the timed region: launches run back to back, so the
+    # region divided by the launch count is the kernel's duration (it agrees with the
+    # rocprofv3 kernel trace; a lone launch bracketed by two events reads ~2 us more)
+    kernel_s = region_s / (args.steps * iters)
     B = algorithmic_bytes(nv, nM, nefc)
     achieved = B * nworld / kernel_s / 1e9
 
@@ -207,7 +237,7 @@ def main() -> int:
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": TRAFFIC_BYTES_PER_LAUNCH,
             "kernel_us": kernel_s * 1e6,
-            "kernel_us_p10_p50_p90": [float(np.percentile(durs, p)) * 1e6 for p in (10, 50, 90)],
+            "kernel_us_single_launch_p10_p50_p90": [float(np.percentile(durs, p)) * 1e6 for p in (10, 50, 90)],
             "throughput_frac": (B * value / 1e9) / HBM_PEAK_GBS,
         },
     }
