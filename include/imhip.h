@@ -103,6 +103,34 @@ int im_assemble_tree_ldl_solve(const im_tree_plan *plan, const float *M,
                                int64_t ldg, float *x, int64_t ldx, float *Hout,
                                int nworld, unsigned flags, void *stream);
 
+/* Muscle moment-arm contractions ------------------------------------------- */
+
+/* Replaces project_muscle_sparse_moment_qfrc_kernel
+ * (src/instantmimic/muscle/muscle_qfrc_projector.py:2941-2961, launched from
+ * src/instantmimic/envs/controls/fast_muscle/torque_runtime.py:895-909):
+ *   qfrc[w, root + j] = sum over s in [offsets[j], offsets[j + 1]) of
+ *                       moment[w, e] * force[w, entry_muscle[e]],  e = entry_idx[s]
+ * summed in that order.  moment (nworld, ld_moment >= nentry), force (nworld,
+ * ld_force >= nmuscle), qfrc (nworld, ld_qfrc >= root + ntorque); the three index
+ * tables are device arrays built once per model. */
+int im_muscle_project(const float *moment, int64_t ld_moment, const float *force,
+                      int64_t ld_force, const int32_t *torque_entry_offsets,
+                      const int32_t *torque_entry_idx, const int32_t *entry_muscle,
+                      int nentry, int nmuscle, int ntorque, int root_dof_count,
+                      float *qfrc, int64_t ld_qfrc, int nworld, void *stream);
+
+/* Replaces apply_muscle_implicit_qderiv_gather (muscle_qfrc_projector.py:777-809,
+ * kernel :736-774): qderiv[w, elem_ids[slot]] += timestep * sum over the slot's
+ * chunks, in order, of the chunk's 16-pair sum of
+ * (slope[w, entry_muscle[i]] * moment[w, i]) * moment[w, j], pairs packed i | j << 16
+ * at chunk_pairs[k * chunk_count + c], padding = nentry.  Deterministic (no atomics). */
+int im_muscle_implicit_gather(const float *moment, int64_t ld_moment, const float *slope,
+                              int64_t ld_slope, const int32_t *entry_muscle, int nentry,
+                              const int32_t *elem_ids, int nelem,
+                              const int32_t *chunk_offsets, const int32_t *chunk_pairs,
+                              int chunk_count, float timestep, float *qderiv,
+                              int64_t ld_qderiv, int nworld, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -48,6 +48,11 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _i, _u, _vp],
     ),
+    "im_muscle_project": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i64, _i, _vp]),
+    "im_muscle_implicit_gather": (
+        _i,
+        [_vp, _i64, _vp, _i64, _vp, _i, _vp, _i, _vp, _vp, _i, C.c_float, _vp, _i64, _i, _vp],
+    ),
 }
 
 _lib = None

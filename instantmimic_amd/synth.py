@@ -214,3 +214,74 @@ def dense_from_csr(values: np.ndarray, rowadr, rownnz, colind) -> np.ndarray:
     out[:, rowi, colind] = values
     out[:, colind, rowi] = values
     return out
+
+
+# ------------------------------------------------------------------ muscles (SNU-like shape)
+
+
+def snu_joint_chains() -> list[list[list[int]]]:
+    """Root-to-leaf joint chains of the SNU-like tree below the pelvis; a joint is the
+    list of its dofs (ball = 3 chained dofs, hinge = 1)."""
+
+    def leg(b):
+        return [[b, b + 1, b + 2], [b + 3], [b + 4, b + 5, b + 6], [b + 7], [b + 8], [b + 9]]
+
+    def arm(b):
+        return [[b, b + 1, b + 2], [b + 3, b + 4, b + 5], [b + 6], [b + 7, b + 8, b + 9]]
+
+    spine = [[26, 27, 28], [29, 30, 31]]
+    return [leg(6), leg(16), spine + [[32, 33, 34], [35]], spine + arm(36), spine + arm(46)]
+
+
+@dataclass
+class MuscleBatch:
+    nmuscle: int
+    root_dof_count: int
+    muscle_dofs: np.ndarray  # (nentry, 2) (muscle, torque dof), sorted by muscle then dof
+    moment: np.ndarray  # (nworld, nentry) fp32
+    force: np.ndarray  # (nworld, nmuscle) fp32
+    slope: np.ndarray  # (nworld, nmuscle) fp32
+    timestep: float
+
+
+def make_muscles(nworld: int, nmuscle: int = 284, seed: int = 1003) -> MuscleBatch:
+    """284 muscles, each spanning 1-3 adjacent joints of one chain; moment-arm entries
+    ~N(0, 0.05); f = a f_max l + f_passive; slope = df/dl ~ U[0, 1e3]."""
+    rng = np.random.default_rng([seed, 77])
+    chains = snu_joint_chains()
+    root = 6
+    pairs = []
+    for m in range(nmuscle):
+        chain = chains[int(rng.integers(len(chains)))]
+        span = int(rng.integers(1, 4))
+        first = int(rng.integers(0, len(chain) - span + 1))
+        for joint in chain[first : first + span]:
+            pairs += [(m, d - root) for d in joint]
+    md = np.unique(np.asarray(pairs, np.int64), axis=0)
+    nentry = md.shape[0]
+    moment = np.empty((nworld, nentry), np.float32)
+    force = np.empty((nworld, nmuscle), np.float32)
+    slope = np.empty((nworld, nmuscle), np.float32)
+    for b0 in range(0, nworld, BLOCK):
+        r = np.random.default_rng([seed, 78, b0 // BLOCK])
+        a = r.normal(0.0, 0.05, (BLOCK, nentry))
+        act = r.uniform(0, 1, (BLOCK, nmuscle))
+        fmax = r.uniform(100, 3000, (BLOCK, nmuscle))
+        lf = r.uniform(0.5, 1.0, (BLOCK, nmuscle))
+        fp = r.uniform(0, 50, (BLOCK, nmuscle))
+        sl = r.uniform(0, 1e3, (BLOCK, nmuscle))
+        n = min(BLOCK, nworld - b0)
+        moment[b0 : b0 + n] = a[:n]
+        force[b0 : b0 + n] = (act * fmax * lf + fp)[:n]
+        slope[b0 : b0 + n] = sl[:n]
+    return MuscleBatch(nmuscle, root, md, moment, force, slope, 1.0 / 480.0)
+
+
+def matrix_elemid(rowadr, rownnz, colind) -> np.ndarray:
+    """(nv, nv) table: CSR index of M's element (i, j), either order, -1 off the pattern."""
+    nv = len(rowadr)
+    out = np.full((nv, nv), -1, np.int32)
+    rowi = np.repeat(np.arange(nv), rownnz)
+    out[rowi, colind] = np.arange(len(colind))
+    out[colind, rowi] = np.arange(len(colind))
+    return out

@@ -260,3 +260,61 @@ int orc_assemble_tree_ldl_solve(int nworld, int nv, int nM, const int *rowadr,
   plan_free(&p);
   return 0;
 }
+
+/* ------------------------------------------------------------------ muscle contractions
+ * Rounding convention: the reference's kernels are Warp Python (`total += a * b`), which
+ * Warp lowers to add(total, mul(a, b)) in CUDA C++ and NVRTC contracts to one fused
+ * multiply-add; the restatement spells those fmaf()s. */
+
+/* tau[w, root + j] = sum over the entries of torque dof j, in torque-sorted order, of
+ * moment[w, e] * force[w, muscle(e)]
+ * (src/instantmimic/muscle/muscle_qfrc_projector.py:2941-2961). */
+int orc_muscle_project(int nworld, int nentry, int nmuscle, int ntorque, const float *moment,
+                       const float *force, const int *offsets, const int *entry_idx,
+                       const int *entry_muscle, int root, float *qfrc, int ldq) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    const float *m = moment + (size_t)w * nentry, *f = force + (size_t)w * nmuscle;
+    for (int j = 0; j < ntorque; ++j) {
+      float total = 0.0f;
+      for (int s = offsets[j]; s < offsets[j + 1]; ++s) {
+        const int e = entry_idx[s];
+        total = fmaf(m[e], f[entry_muscle[e]], total);
+      }
+      qfrc[(size_t)w * ldq + root + j] = total;
+    }
+  }
+  return 0;
+}
+
+/* qderiv[w, elem] += timestep * sum over the element's chunks (in order) of the chunk's
+ * 16-pair sum of (slope[w, muscle(i)] * moment[w, i]) * moment[w, j]
+ * (muscle_qfrc_projector.py:677-708 serial variant, 736-774 block variant). */
+int orc_muscle_implicit_gather(int nworld, int nentry, int nmuscle, int nelem, int chunk_count,
+                               int chunk, const float *moment, const float *slope,
+                               const int *entry_muscle, const int *elem_ids,
+                               const int *chunk_offsets, const int *chunk_pairs,
+                               float timestep, float *qderiv, int ldq) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    const float *m = moment + (size_t)w * nentry, *sl = slope + (size_t)w * nmuscle;
+    for (int slot = 0; slot < nelem; ++slot) {
+      float acc = 0.0f;
+      for (int c = chunk_offsets[slot]; c < chunk_offsets[slot + 1]; ++c) {
+        float total = 0.0f;
+        for (int k = 0; k < chunk; ++k) {
+          const int packed = chunk_pairs[(size_t)k * chunk_count + c];
+          const int i = packed & 0xFFFF, j = packed >> 16;
+          if (i < nentry) {
+            const float weighted = sl[entry_muscle[i]] * m[i];
+            total = fmaf(weighted, m[j], total);
+          }
+        }
+        acc = acc + total;
+      }
+      float *q = qderiv + (size_t)w * ldq + elem_ids[slot];
+      *q = fmaf(timestep, acc, *q);
+    }
+  }
+  return 0;
+}

@@ -146,3 +146,33 @@ def rel_l2(a, b):
     a = np.asarray(a, np.float64)
     b = np.asarray(b, np.float64)
     return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
+
+
+# ---------------------------------------------------------------- muscle contractions
+# Pinning: `muscle_project` against a dense fp64 A' f, `muscle_implicit_gather` against a
+# dense fp64 h A' diag(s) A restricted to M's pattern (tests/test_muscle.py); the index
+# tables against brute-force enumeration there as well.  The reference's own tests do not
+# cover these kernels.
+
+
+def muscle_project(moment, force, offsets, entry_idx, entry_muscle, root, nv):
+    moment, force = _f(moment), _f(force)
+    nworld, nentry = moment.shape
+    qfrc = np.zeros((nworld, nv), np.float32)
+    lib().orc_muscle_project(
+        nworld, nentry, force.shape[1], len(offsets) - 1, _p(moment), _p(force), _p(_i(offsets)), _p(_i(entry_idx)),
+        _p(_i(entry_muscle)), int(root), _p(qfrc), nv,
+    )  # fmt: skip
+    return qfrc
+
+
+def muscle_implicit_gather(moment, slope, entry_muscle, elem_ids, chunk_offsets, chunk_pairs, chunk_count, timestep, qderiv):
+    moment, slope = _f(moment), _f(slope)
+    out = np.array(qderiv, np.float32, copy=True, order="C")
+    lib().orc_muscle_implicit_gather.argtypes = None
+    lib().orc_muscle_implicit_gather(
+        moment.shape[0], moment.shape[1], slope.shape[1], len(elem_ids), int(chunk_count), 16, _p(moment), _p(slope),
+        _p(_i(entry_muscle)), _p(_i(elem_ids)), _p(_i(chunk_offsets)), _p(_i(chunk_pairs)), ctypes.c_float(timestep),
+        _p(out), out.shape[1],
+    )  # fmt: skip
+    return out
