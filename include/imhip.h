@@ -103,6 +103,32 @@ int im_assemble_tree_ldl_solve(const im_tree_plan *plan, const float *M,
                                int64_t ldg, float *x, int64_t ldx, float *Hout,
                                int nworld, unsigned flags, void *stream);
 
+/* Static-pattern sparse L'DL of H = M + J'DJ -------------------------------- */
+
+typedef struct im_sparse_plan im_sparse_plan;
+
+/* Device side of a SparseHessianPlan (src/instantmimic/utils/mjw_kernels/
+ * sparse_hessian.py:38-50, tables :360-401).  tables[16] in this order, int32 each:
+ * SH_LP, SH_LT, SH_ES, SH_EC, SH_RP, SH_RAB, SH_RKL, SH_ORIG, SH_BL, SH_BS, SH_BI, SH_BJ,
+ * SH_PM, SH_SA, SH_SB, SH_SM; block is the plan's block width (32 or 64). */
+int im_sparse_plan_create(int nv, int nv_pad, int block, int nslots, int nlevels,
+                          int ntables, const int32_t *const *tables, const int *sizes,
+                          im_sparse_plan **out);
+void im_sparse_plan_destroy(im_sparse_plan *plan);
+
+/* Replaces the launch of sparse_hessian.init_factor_kernel(plan)
+ * (sparse_hessian.py:804-846, launched from newton_fusion.py:502-519) with the same
+ * arrays: done (nworld) bytes or null, nefc (nworld), J (nworld, njmax, nv), D/state
+ * (nworld, njmax), M (nworld, ldM), grad (nworld, ldg), hfactor (nworld, nv_pad,
+ * nv_pad) used as flat scratch ([0,nfac) packed H, [nfac,2nfac) factor, then 1/D, last
+ * element = pattern-violation counter, which accumulates), search (nworld, nv),
+ * search_dot / decrement (nworld). */
+int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done,
+                          const int32_t *nefc, const float *J, int njmax, const float *D,
+                          const int32_t *state, int quad, const float *M, int ldM,
+                          const float *grad, int ldg, float *hfactor, float *search,
+                          float *search_dot, float *decrement, int nworld, void *stream);
+
 /* Muscle moment-arm contractions ------------------------------------------- */
 
 /* Replaces project_muscle_sparse_moment_qfrc_kernel

@@ -48,6 +48,12 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _i, _u, _vp],
     ),
+    "im_sparse_plan_create": (_i, [_i, _i, _i, _i, _i, _i, _vp, _vp, C.POINTER(_vp)]),
+    "im_sparse_plan_destroy": (None, [_vp]),
+    "im_sparse_init_factor": (
+        _i,
+        [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp],
+    ),
     "im_muscle_project": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i64, _i, _vp]),
     "im_muscle_implicit_gather": (
         _i,

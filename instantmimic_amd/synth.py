@@ -164,7 +164,9 @@ def chain_mask(parent) -> np.ndarray:
     return mask
 
 
-def make_batch(shape: Shape | str, nworld: int | None = None, *, ragged_nefc: bool = False) -> Batch:
+def make_batch(shape: Shape | str, nworld: int | None = None, *, ragged_nefc: bool = False, supports=None) -> Batch:
+    """``supports`` (optional, (nsup, nv) bool): the dof sets a constraint row may be
+    supported on, instead of single root-to-leaf chains."""
     if isinstance(shape, str):
         shape = SHAPES[shape]
     nworld = shape.worlds if nworld is None else int(nworld)
@@ -187,10 +189,12 @@ def make_batch(shape: Shape | str, nworld: int | None = None, *, ragged_nefc: bo
         V = rng.standard_normal((nb, nv, nv)) * mask[None]
         dense = np.einsum("wk,wki,wkj->wij", mass, V, V, optimize=True)
         dense[:, np.arange(nv), np.arange(nv)] += shape.armature
-        body = rng.integers(0, nv, (nb, nefc))
         rows = rng.standard_normal((nb, nefc, nv))
-        if not shape.dense_rows:
-            rows *= mask[body]
+        if supports is not None:
+            sup = np.asarray(supports, bool)
+            rows *= sup[rng.integers(0, sup.shape[0], (nb, nefc))]
+        elif not shape.dense_rows:
+            rows *= mask[rng.integers(0, nv, (nb, nefc))]
         logd = rng.uniform(shape.logd[0], shape.logd[1], (nb, nefc))
         act = rng.random((shape.iterations, nb, nefc)) < shape.p_active
         g = rng.standard_normal((nb, nv))
@@ -285,3 +289,65 @@ def matrix_elemid(rowadr, rownnz, colind) -> np.ndarray:
     out[rowi, colind] = np.arange(len(colind))
     out[colind, rowi] = np.arange(len(colind))
     return out
+
+
+def model_from_parents(parent, joints: list[list[int]] | None = None):
+    """A minimal model namespace (the fields the planners read) for a dof tree.  Bodies:
+    one per joint (``joints`` lists each joint's dofs; default one dof per body); body 0 is
+    the world."""
+    from types import SimpleNamespace
+
+    parent = list(parent)
+    nv = len(parent)
+    if joints is None:
+        joints = [[d] for d in range(nv)]
+    body_of_dof = {}
+    for b, dofs in enumerate(joints, start=1):
+        for d in dofs:
+            body_of_dof[d] = b
+    body_parentid, body_dofadr, body_dofnum = [0], [-1], [0]
+    for dofs in joints:
+        p = parent[dofs[0]]
+        body_parentid.append(body_of_dof[p] if p >= 0 else 0)
+        body_dofadr.append(dofs[0])
+        body_dofnum.append(len(dofs))
+    rowadr, rownnz, colind = csr_from_parents(parent)
+    return SimpleNamespace(
+        nv=nv, nv_pad=((nv + 1 + 15) // 16) * 16, dof_parentid=np.asarray(parent, np.int32),
+        body_parentid=np.asarray(body_parentid, np.int32), body_dofadr=np.asarray(body_dofadr, np.int32),
+        body_dofnum=np.asarray(body_dofnum, np.int32), M_rowadr=rowadr, M_rownnz=rownnz, M_colind=colind,
+        M_hinit_i=np.repeat(np.arange(nv), rownnz).astype(np.int32), neq=0, nflex=0, ntendon=0,
+        nxn_geom_pair_filtered=np.zeros((0, 2), np.int32), geom_bodyid=np.zeros(0, np.int32),
+    )  # fmt: skip
+
+
+def contact_model():
+    """The structure of the reference's sparse-Hessian test model
+    (tests/test_mjw_sparse_hessian.py:14-53): torso (6 dofs), two legs (ball, hinge, two
+    hinges on the foot), two arms (hinge, two hinges), two free boxes; nv = 36.  Returns the
+    model namespace and body ids by name."""
+    parent = [-1, 0, 1, 2, 3, 4]
+    joints = [[0, 1, 2, 3, 4, 5]]
+    names = ["torso"]
+
+    def add(body_name, ndof, parent_dof):
+        first = len(parent)
+        parent.extend([parent_dof] + list(range(first, first + ndof - 1)))
+        joints.append(list(range(first, first + ndof)))
+        names.append(body_name)
+        return first + ndof - 1
+
+    for s in "LR":
+        last = add("thigh" + s, 3, 5)
+        last = add("shin" + s, 1, last)
+        add("foot" + s, 2, last)
+    for s in "LR":
+        last = add("arm" + s, 1, 5)
+        add("fore" + s, 2, last)
+    for s in "AB":
+        first = len(parent)
+        parent.extend([-1] + list(range(first, first + 5)))
+        joints.append(list(range(first, first + 6)))
+        names.append("box" + s)
+    m = model_from_parents(parent, joints)
+    return m, {n: i + 1 for i, n in enumerate(names)}

@@ -318,3 +318,131 @@ int orc_muscle_implicit_gather(int nworld, int nentry, int nmuscle, int nelem, i
   }
   return 0;
 }
+
+/* ------------------------------------------------------------------ static-pattern sparse L'DL
+ * Restatement of the reference's initial assemble + factor + solve kernel
+ * (src/instantmimic/utils/mjw_kernels/sparse_hessian.py: assembly 578-630, level factor
+ * 410-452, backward solve and sums 453-479) executed lane by lane: the result depends on
+ * which lane of a team sums which terms and on the shuffle tree, so both are emulated.
+ * Plain `a - b * c` expressions of the CUDA snippet contract to fmaf(-b, c, a). */
+typedef struct {
+  int nv, nv_pad, block, nslots, nlevels;
+  const int *LP, *LT, *ES, *EC, *RP, *RAB, *RKL, *ORIG, *BL, *BS, *BI, *BJ, *PM, *SA, *SB, *SM;
+} sparse_t;
+
+static void sparse_world(const sparse_t *p, const float *J, int njmax, const float *D,
+                         const int *state, int nefc, int quad, const float *M, const float *grad,
+                         float *U, float *search, float *sdot, float *decr, float *N) {
+  const int n = p->nv, nfac = p->nslots - n, rhs = nfac, block = p->block;
+  float *iD = N + p->nslots;
+  const int words = (n + 31) / 32;
+  for (int s = 0; s < nfac; ++s) N[s] = p->SM[s] >= 0 ? M[p->SM[s]] : 0.0f;
+  if (nefc > njmax) nefc = njmax;
+  for (int k = 0; k < nefc; k += 4) {
+    float Dc[4];
+    const float *Jr[4];
+    static const float zero_row[1024] = {0};
+    for (int r = 0; r < 4; ++r) {
+      const int row = k + r;
+      Dc[r] = (row < nefc && state[row] == quad) ? D[row] : 0.0f;
+      Jr[r] = row < nefc ? J + (size_t)row * n : zero_row;
+    }
+    /* pattern check: every active row's support must lie inside the pattern */
+    for (int r = 0; r < 4; ++r) {
+      if (Dc[r] == 0.0f) continue;
+      unsigned rm[32] = {0};
+      for (int d = 0; d < n; ++d)
+        if (Jr[r][d] != 0.0f) rm[d / 32] |= 1u << (d % 32);
+      int bad = 0;
+      for (int d = 0; d < n; ++d)
+        if ((rm[d / 32] >> (d % 32)) & 1u)
+          for (int q = 0; q < words; ++q) bad |= (rm[q] & ~(unsigned)p->PM[d * words + q]) != 0u;
+      if (bad) U[p->nv_pad * p->nv_pad - 1] += 1.0f;
+    }
+    for (int s = 0; s < nfac; ++s) {
+      const int a = p->SA[s], b = p->SB[s];
+      float v = N[s];
+      for (int r = 0; r < 4; ++r) v = fmaf(Jr[r][a] * Dc[r], Jr[r][b], v);
+      N[s] = v;
+    }
+  }
+  for (int s = 0; s < nfac; ++s) U[s] = N[s];
+  for (int j = 0; j < n; ++j) N[rhs + j] = grad[p->ORIG[j]];
+  for (int l = 0; l < p->nlevels; ++l) {
+    const int T = p->LT[l];
+    for (int e = p->LP[l]; e < p->LP[l + 1]; ++e) {
+      float part[32];
+      for (int tl = 0; tl < T; ++tl) {
+        float v = 0.0f;
+        for (int r = p->RP[e]; r < p->RP[e + 1]; ++r) {
+          const unsigned ab = (unsigned)p->RAB[r], kl = (unsigned)p->RKL[r];
+          const float *pa = N + (ab & 0xFFFFu), *pb = N + (ab >> 16), *pd = iD + (kl & 0xFFFFu);
+          const int len = (int)(kl >> 16);
+          for (int t = tl; t < len; t += T) v = fmaf(pa[t] * pb[t], pd[t], v);
+        }
+        part[tl] = v;
+      }
+      for (int off = T >> 1; off > 0; off >>= 1)
+        for (int i = 0; i < off; ++i) part[i] = part[i] + part[i + off];
+      /* entries of one level never read what the level writes, so in-place is a sweep */
+      const float wv = N[p->ES[e]] - part[0];
+      N[p->ES[e]] = wv;
+      if (p->EC[e] >= 0) iD[p->EC[e]] = 1.0f / wv;
+    }
+  }
+  for (int s = 0; s < nfac; ++s) U[nfac + s] = N[s];
+  for (int j = 0; j < n; ++j) U[2 * nfac + j] = iD[j];
+  for (int l = 0; l < p->nlevels; ++l)
+    for (int q = p->BL[l]; q < p->BL[l + 1]; ++q) {
+      const int i = p->BI[q], j = p->BJ[q];
+      N[rhs + j] = fmaf(-N[p->BS[q]], N[rhs + i] * iD[i], N[rhs + j]);
+    }
+  /* per-lane sums, 32-lane shuffle tree, warps added in order */
+  float s0[64] = {0}, s1[64] = {0};
+  for (int lane = 0; lane < block; ++lane)
+    for (int j = lane; j < n; j += block) {
+      const int d = p->ORIG[j];
+      const float v = N[rhs + j] * iD[j];
+      search[d] = -v;
+      s0[lane] = fmaf(v, v, s0[lane]);
+      s1[lane] = fmaf(grad[d], v, s1[lane]);
+    }
+  float ra = 0.0f, rb = 0.0f;
+  for (int wv = 0; wv < (block + 31) / 32; ++wv) {
+    float *a = s0 + 32 * wv, *b = s1 + 32 * wv;
+    for (int off = 16; off > 0; off >>= 1)
+      for (int i = 0; i < off; ++i) {
+        a[i] = a[i] + a[i + off];
+        b[i] = b[i] + b[i + off];
+      }
+    ra = ra + a[0];
+    rb = rb + b[0];
+  }
+  *sdot = ra;
+  *decr = rb;
+}
+
+int orc_sparse_init_factor(int nv, int nv_pad, int block, int nslots, int nlevels,
+                           const int *const *tables, int nworld, const unsigned char *done,
+                           const int *nefc, const float *J, int njmax, const float *D,
+                           const int *state, int quad, const float *M, int ldM, const float *grad,
+                           int ldg, float *hfactor, float *search, float *sdot, float *decr) {
+  sparse_t p = {nv, nv_pad, block, nslots, nlevels, tables[0], tables[1], tables[2], tables[3],
+                tables[4], tables[5], tables[6], tables[7], tables[8], tables[9], tables[10],
+                tables[11], tables[12], tables[13], tables[14], tables[15]};
+  if (nv > 1024 || block > 64) return 1;
+#pragma omp parallel
+  {
+    float *N = (float *)malloc(sizeof(float) * (nslots + nv + 8));
+#pragma omp for schedule(static)
+    for (int w = 0; w < nworld; ++w) {
+      if (done && done[w]) continue;
+      sparse_world(&p, J + (size_t)w * njmax * nv, njmax, D + (size_t)w * njmax,
+                   state + (size_t)w * njmax, nefc[w], quad, M + (size_t)w * ldM,
+                   grad + (size_t)w * ldg, hfactor + (size_t)w * nv_pad * nv_pad,
+                   search + (size_t)w * nv, sdot + w, decr + w, N);
+    }
+    free(N);
+  }
+  return 0;
+}

@@ -176,3 +176,88 @@ def muscle_implicit_gather(moment, slope, entry_muscle, elem_ids, chunk_offsets,
         _p(out), out.shape[1],
     )  # fmt: skip
     return out
+
+
+# ---------------------------------------------------------------- static-pattern sparse L'DL
+# Pinning: the level/run/backward tables are executed in fp64 as parallel sweeps with a
+# race check per level (the executor the reference's own test holds,
+# tests/test_mjw_sparse_hessian.py:199-262) and must solve H x = g to 1e-10; the fp32
+# lane-by-lane C executor is then checked against that fp64 result within conditioning.
+
+TABLE_ORDER = ("SH_LP", "SH_LT", "SH_ES", "SH_EC", "SH_RP", "SH_RAB", "SH_RKL", "SH_ORIG", "SH_BL", "SH_BS", "SH_BI",
+               "SH_BJ", "SH_PM", "SH_SA", "SH_SB", "SH_SM")  # fmt: skip
+
+
+def run_tables64(T, nv, nslots, H, g):
+    """Factor and solve through the tables in fp64, each level as one parallel sweep
+    (every lane reads the level's input snapshot); asserts that no level writes what
+    another lane of it reads or writes.  Returns x = H^-1 g."""
+    nfac = nslots - nv
+    u = lambda k: T[k].astype(np.int64) & 0xFFFFFFFF  # noqa: E731
+    N, iD = np.zeros(nslots), np.zeros(nv)
+    pair = T["SH_PAIR"].reshape(nv, nv)
+    for s in range(nfac):
+        a, b = T["SH_SA"][s], T["SH_SB"][s]
+        assert pair[a, b] == s
+        N[s] = H[a, b]
+    words = (nv + 31) // 32
+    pm = u("SH_PM")
+    for a in range(nv):
+        for b in range(a, nv):
+            in_mask = (pm[a * words + b // 32] >> (b % 32)) & 1
+            assert bool(in_mask) == (pair[a, b] >= 0 or a == b)
+            assert H[a, b] == 0.0 or pair[a, b] >= 0
+    orig = T["SH_ORIG"]
+    N[nfac:] = g[orig]
+    LP, ES, EC, RP = T["SH_LP"], T["SH_ES"], T["SH_EC"], T["SH_RP"]
+    RAB, RKL = u("SH_RAB"), u("SH_RKL")
+    for lvl in range(len(LP) - 1):
+        n0, d0 = N.copy(), iD.copy()
+        written, read = set(), set()
+        for e in range(LP[lvl], LP[lvl + 1]):
+            v = 0.0
+            for r in range(RP[e], RP[e + 1]):
+                a, b, k, ln = RAB[r] & 0xFFFF, RAB[r] >> 16, RKL[r] & 0xFFFF, RKL[r] >> 16
+                v += float(np.sum(n0[a : a + ln] * n0[b : b + ln] * d0[k : k + ln]))
+                read |= {*range(a, a + ln), *range(b, b + ln), *range(-k - ln, -k)}
+            assert ES[e] not in written
+            written.add(int(ES[e]))
+            N[ES[e]] = n0[ES[e]] - v
+            if EC[e] >= 0:
+                iD[EC[e]] = 1.0 / N[ES[e]]
+                written.add(-1 - int(EC[e]))
+        assert not written & read
+    BL, BS, BI, BJ = T["SH_BL"], T["SH_BS"], T["SH_BI"], T["SH_BJ"]
+    for lvl in range(len(BL) - 1):
+        z = N[nfac:].copy()
+        src, dst = set(), set()
+        for p in range(BL[lvl], BL[lvl + 1]):
+            i, j = int(BI[p]), int(BJ[p])
+            assert j not in dst, "two pushes to one unknown in a level"
+            src.add(i)
+            dst.add(j)
+            N[nfac + j] = z[j] - N[BS[p]] * (z[i] * iD[i])
+        assert not src & dst
+    x = np.zeros(nv)
+    x[orig] = N[nfac:] * iD
+    return x
+
+
+def sparse_init_factor(plan, nefc, J, D, state, M, grad, hfactor=None, done=None, quad=1):
+    """fp32 lane-by-lane restatement of the initial assemble + factor + solve kernel."""
+    J, D, M, grad = _f(J), _f(D), _f(M), _f(grad)
+    state, nefc = _i(state), _i(nefc)
+    nworld, njmax, nv = J.shape
+    tabs = [np.ascontiguousarray(plan.tables[k], np.int32) for k in TABLE_ORDER]
+    ptrs = (ctypes.c_void_p * len(tabs))(*[t.ctypes.data for t in tabs])
+    hf = np.zeros((nworld, plan.nv_pad, plan.nv_pad), np.float32) if hfactor is None else np.array(hfactor, np.float32, order="C")
+    search = np.zeros((nworld, nv), np.float32)
+    sdot = np.zeros(nworld, np.float32)
+    decr = np.zeros(nworld, np.float32)
+    dn = None if done is None else np.ascontiguousarray(done, np.uint8)
+    status = lib().orc_sparse_init_factor(
+        plan.nv, plan.nv_pad, plan.block, plan.nslots, plan.levels, ptrs, nworld, _p(dn), _p(nefc), _p(J), njmax, _p(D),
+        _p(state), quad, _p(M), M.shape[1], _p(grad), grad.shape[1], _p(hf), _p(search), _p(sdot), _p(decr),
+    )  # fmt: skip
+    assert status == 0
+    return hf, search, sdot, decr
