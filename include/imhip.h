@@ -129,6 +129,29 @@ int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done,
                           const float *grad, int ldg, float *hfactor, float *search,
                           float *search_dot, float *decrement, int nworld, void *stream);
 
+/* Blocked dense factor + solve, dense J'DJ ----------------------------------- */
+
+/* Replaces _blocked_dense_factor_solve (src/instantmimic/utils/mjw_step_optimized.py:
+ * 958-993) and its kernel factor_solve_indexed_cholesky_kernel
+ * (src/instantmimic/utils/mjw_kernels/indexed_factor.py:176-214): upper Cholesky
+ * U'U = M by block_size x block_size tiles with indexed gather, x = M^-1 y.
+ * block_idx is the (nblk, nblk, B, B)-ordered table of element ids into M[w, :] built
+ * by create_blocked_dense_factor_solve_scratch (mjw_step_optimized.py:932-941); ids
+ * >= nM read as zero; padded diagonal entries get +1.  U (nworld, pad, pad) receives the
+ * factor (the reference's workspace) or may be null.  block_size 8 or 16. */
+int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *block_idx,
+                            int block_size, int nv, int pad, const float *y, int64_t ldy,
+                            float *U, float *x, int64_t ldx, int nworld, void *stream);
+
+/* Dense Newton Hessian on fp32 MFMA: H[w] (nv_pad, nv_pad) = Mdense[w] (nv, nv) +
+ * J[w]' diag(D [state == quad, row < nefc]) J[w].  Stands in for mujoco_warp's
+ * solver._update_gradient JTDAJ kernel, which the reference calls at
+ * src/instantmimic/utils/mjw_kernels/newton_fusion.py:470 and sizes at
+ * src/instantmimic/utils/mjw_model.py:31-35.  nv <= 128. */
+int im_jtdj_mfma(const float *Mdense, const float *J, int njmax, const float *D,
+                 const int32_t *state, const int32_t *nefc, int quad, float *H, int nv,
+                 int nv_pad, int nworld, void *stream);
+
 /* Muscle moment-arm contractions ------------------------------------------- */
 
 /* Replaces project_muscle_sparse_moment_qfrc_kernel

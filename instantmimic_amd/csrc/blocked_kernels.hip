@@ -1,0 +1,289 @@
+// Blocked dense upper Cholesky factor + solve with indexed gather of M, one workgroup
+// per world, the factor resident in LDS (the reference stores and reloads every U block
+// through global memory), plus the dense J'DJ Hessian on fp32 MFMA for large nv.
+//
+// Reference schedule: src/instantmimic/utils/mjw_kernels/indexed_factor.py:15-173
+// (left-looking by block column, forward solve fused into the factor loop, backward
+// solve), scratch layout src/instantmimic/utils/mjw_step_optimized.py:893-955.  The
+// arithmetic inside a tile operation is Warp's tile library in the reference; here it is
+// spelled out and fixed (same convention as the CPU restatement it is tested against):
+//   U_jk' U_ji updates: sum over t ascending with fma from 0, then C = C - sum;
+//   Cholesky by columns, s = fma(-l, l, s), L[i][j] = v * (1 / L[j][j]);
+//   triangular solves column oriented (j ascending forward, r descending backward).
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+
+namespace im {
+namespace {
+
+__device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+
+template <int B>
+__global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
+    const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
+    const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
+    int64_t ldx, int nv, int pad) {
+  extern __shared__ float lds[];
+  float *U = lds;             // [pad * pad]
+  float *rhs = U + pad * pad; // [pad]
+  float *A = rhs + pad;       // [(nblk) * B * B] working tiles of the current block row
+  float *L = A + (pad / B) * B * B;  // [B * B] Cholesky factor of the diagonal block (lower)
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int64_t w = blockIdx.x;
+  const int nblk = pad / B;
+  constexpr int BB = B * B;
+  const float *Mw = M + w * ldM;
+  for (int i = tid; i < pad * pad; i += nt) U[i] = 0.0f;
+  for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? y[w * ldy + i] : 0.0f;
+  __syncthreads();
+  for (int kb = 0; kb < nblk; ++kb) {
+    const int k = kb * B, end = k + B;
+    // gather the whole block row kb..nblk-1 and subtract the finished block rows above
+    const int ntile = nblk - kb;
+    for (int q = tid; q < ntile * BB; q += nt) {
+      const int tb = q / BB, e = q - tb * BB, r = e / B, c = e - r * B;
+      const int ib = kb + tb, i0 = ib * B;
+      const int idx = block_idx[(size_t)(kb * nblk + ib) * BB + e];
+      float v = idx < nM ? Mw[idx] : 0.0f;
+      if (tb == 0 && end > nv && r == c && (nblk - 1) * B + r >= nv) v = v + 1.0f;
+      for (int jb = 0; jb < kb; ++jb) {
+        const int j = jb * B;
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < B; ++t) sum = fma_(U[(j + t) * pad + k + r], U[(j + t) * pad + i0 + c], sum);
+        v = v - sum;
+      }
+      A[q] = v;
+    }
+    if (tid < B) {
+      float s = rhs[k + tid];
+      for (int jb = 0; jb < kb; ++jb) {
+        const int j = jb * B;
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < B; ++t) sum = fma_(U[(j + t) * pad + k + tid], rhs[j + t], sum);
+        s = s - sum;
+      }
+      rhs[k + tid] = s;
+    }
+    __syncthreads();
+    // Cholesky of the diagonal tile and the forward solve of the right-hand side: wave 0
+    if (tid < 64) {
+      const int i = tid;
+      for (int j = 0; j < B; ++j) {
+        float v = 0.0f;
+        if (i >= j && i < B) {
+          v = A[i * B + j];
+          for (int q = 0; q < j; ++q) v = fma_(-L[i * B + q], L[j * B + q], v);
+        }
+        if (i == j) {
+          const float d = sqrtf(v);
+          L[j * B + j] = d;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        if (i > j && i < B) L[i * B + j] = v * (1.0f / L[j * B + j]);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+      }
+      float s = i < B ? rhs[k + i] : 0.0f;
+      for (int j = 0; j < B; ++j) {
+        if (i == j) rhs[k + j] = s / L[j * B + j];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        if (i > j && i < B) s = fma_(-L[i * B + j], rhs[k + j], s);
+      }
+    }
+    __syncthreads();
+    // U_kk = L', and U_ki = L^-1 A_ki column by column
+    for (int e = tid; e < BB; e += nt) {
+      const int r = e / B, c = e - r * B;
+      if (c >= r) U[(k + r) * pad + k + c] = L[c * B + r];
+    }
+    for (int q = tid; q < (ntile - 1) * B; q += nt) {
+      const int tb = 1 + q / B, c = q - (tb - 1) * B;
+      float *At = A + tb * BB;
+      float col[B];
+#pragma unroll
+      for (int r = 0; r < B; ++r) col[r] = At[r * B + c];
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        const float z = col[j] / L[j * B + j];
+        col[j] = z;
+#pragma unroll
+        for (int i = j + 1; i < B; ++i) col[i] = fma_(-L[i * B + j], z, col[i]);
+      }
+      const int i0 = (kb + tb) * B;
+#pragma unroll
+      for (int r = 0; r < B; ++r) U[(k + r) * pad + i0 + c] = col[r];
+    }
+    __syncthreads();
+  }
+  // backward solve
+  for (int i0 = pad - B; i0 >= 0; i0 -= B) {
+    if (tid < 64) {
+      const int r = tid;
+      float s = 0.0f;
+      if (r < B) {
+        s = rhs[i0 + r];
+        for (int j = i0 + B; j < pad; j += B) {
+          float sum = 0.0f;
+#pragma unroll
+          for (int t = 0; t < B; ++t) sum = fma_(U[(i0 + r) * pad + j + t], rhs[j + t], sum);
+          s = s - sum;
+        }
+      }
+      for (int c = B - 1; c >= 0; --c) {
+        if (r == c) rhs[i0 + c] = s / U[(i0 + c) * pad + i0 + c];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        if (r < c) s = fma_(-U[(i0 + r) * pad + i0 + c], rhs[i0 + c], s);
+      }
+    }
+    __syncthreads();
+  }
+  for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
+  if (Uout)
+    for (int i = tid; i < pad * pad; i += nt) Uout[w * (int64_t)pad * pad + i] = U[i];
+}
+
+// ---------------------------------------------------------------------------- dense J'DJ
+// H[w] = M[w] + J[w]' diag(Dc[w]) J[w], H (nv_pad, nv_pad), on v_mfma_f32_32x32x2_f32.
+// One wavefront per 32x32 output tile; a workgroup of 256 threads covers a 64x64... the
+// tile grid is (ceil(nv/32))^2 per world, only tiles with column block >= row block are
+// computed and mirrored.  A = (J D)' and B = J are staged through LDS 32 rows at a time.
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void jtdj_mfma_kernel(
+    const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
+    const float *__restrict__ D, const int32_t *__restrict__ state, const int32_t *__restrict__ nefc_p,
+    int quad, float *__restrict__ H, int nv, int nv_pad) {
+  extern __shared__ float lds[];
+  const int nvr = (nv + 31) / 32 * 32;   // staged row width
+  float *Js = lds;                       // [32][nvr]   J rows
+  float *JDs = Js + 32 * nvr;            // [32][nvr]   J rows times Dc
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t w = blockIdx.x;
+  const int nb = nvr / 32;
+  // tiles (bi <= bj) distributed over the four waves; each wave keeps its tiles' accumulators
+  const int ntile = nb * (nb + 1) / 2;
+  constexpr int MAXT = 3;                // up to 10 tiles (nv <= 128) over 4 waves
+  float16v acc[MAXT];
+  int tbi[MAXT], tbj[MAXT], mine = 0;
+  {
+    int t = 0;
+#pragma unroll
+    for (int m = 0; m < MAXT; ++m) tbi[m] = tbj[m] = 0;
+    for (int bi = 0; bi < nb; ++bi)
+      for (int bj = bi; bj < nb; ++bj, ++t)
+        if (t % 4 == wave) {
+          // tile number mine of this wave (at most MAXT)
+          if (mine == 0) { tbi[0] = bi; tbj[0] = bj; }
+          else if (mine == 1) { tbi[1] = bi; tbj[1] = bj; }
+          else if (mine == 2) { tbi[2] = bi; tbj[2] = bj; }
+          ++mine;
+        }
+    mine = mine < MAXT ? mine : MAXT;
+  }
+#pragma unroll
+  for (int m = 0; m < MAXT; ++m)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[m][v] = 0.0f;
+  int nefc = nefc_p ? nefc_p[w] : njmax;
+  nefc = nefc < njmax ? nefc : njmax;
+  const float *Jw = J + w * (int64_t)njmax * nv;
+  for (int r0 = 0; r0 < nefc; r0 += 32) {
+    __syncthreads();
+    for (int q = tid; q < 32 * nvr; q += 256) {
+      const int r = q / nvr, c = q - r * nvr;
+      float v = 0.0f, dc = 0.0f;
+      if (r0 + r < nefc && c < nv) {
+        v = Jw[(int64_t)(r0 + r) * nv + c];
+        if (state[w * njmax + r0 + r] == quad) dc = D[w * njmax + r0 + r];
+      }
+      Js[q] = v;
+      JDs[q] = v * dc;
+    }
+    __syncthreads();
+    // v_mfma_f32_32x32x2_f32: lane l supplies A[i = l % 32][k = l / 32] and B[k = l / 32][j = l % 32]
+#pragma unroll
+    for (int m = 0; m < MAXT; ++m) {
+      if (m < mine) {
+        const int ci = tbi[m] * 32 + (lane & 31), cj = tbj[m] * 32 + (lane & 31);
+#pragma unroll 4
+        for (int kk = 0; kk < 32; kk += 2) {
+          const int k = kk + (lane >> 5);
+          acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(JDs[k * nvr + ci], Js[k * nvr + cj], acc[m], 0, 0, 0);
+        }
+      }
+    }
+  }
+  // accumulator layout of a 32x32 tile: lane l holds column j = l % 32 and rows
+  // i = 8 * g + 4 * (l / 32) ... for register 4 * g + v: i = 8 * g + (l / 32) * 4 + v
+  float *Hw = H + w * (int64_t)nv_pad * nv_pad;
+  const float *Mw = Mdense + w * (int64_t)nv * nv;
+#pragma unroll
+  for (int m = 0; m < MAXT; ++m) {
+    if (m >= mine) continue;
+    const int j = tbj[m] * 32 + (lane & 31);
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int i = tbi[m] * 32 + 8 * g + (lane >> 5) * 4 + v;
+        // upper triangle from the accumulators, lower triangle mirrored: H is symmetric bit for bit
+        if (i < nv && j < nv && i <= j) {
+          const float h = Mw[(int64_t)i * nv + j] + acc[m][4 * g + v];
+          Hw[(int64_t)i * nv_pad + j] = h;
+          if (i != j) Hw[(int64_t)j * nv_pad + i] = h;
+        }
+      }
+  }
+}
+
+}  // namespace
+}  // namespace im
+
+extern "C" {
+
+int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *block_idx, int block_size,
+                            int nv, int pad, const float *y, int64_t ldy, float *U, float *x, int64_t ldx,
+                            int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || pad < nv) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!M || !block_idx || !y || !x) return IM_ERR_ARG;
+  if (block_size != 8 && block_size != 16) return IM_ERR_UNSUPPORTED;
+  if (pad % block_size || pad - nv >= block_size) return IM_ERR_ARG;
+  if (ldy < nv || ldx < nv) return IM_ERR_STRIDE;
+  const int B = block_size;
+  const size_t lds_bytes = sizeof(float) * ((size_t)pad * pad + pad + (size_t)(pad / B) * B * B + B * B);
+  if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
+  auto fn = B == 8 ? im::blocked_factor_solve_kernel<8> : im::blocked_factor_solve_kernel<16>;
+  if (lds_bytes > 64 * 1024)
+    IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, M, ldM, nM, block_idx, y, ldy, U,
+                     x, ldx, nv, pad);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_jtdj_mfma(const float *Mdense, const float *J, int njmax, const float *D, const int32_t *state,
+                 const int32_t *nefc, int quad, float *H, int nv, int nv_pad, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || nv_pad < nv || njmax < 0) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!Mdense || !J || !D || !state || !H) return IM_ERR_ARG;
+  if (nv > 128) return IM_ERR_UNSUPPORTED;
+  const int nvr = (nv + 31) / 32 * 32;
+  const size_t lds_bytes = sizeof(float) * 2 * 32 * (size_t)nvr;
+  hipLaunchKernelGGL(im::jtdj_mfma_kernel, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, Mdense, J,
+                     njmax, D, state, nefc, quad, H, nv, nv_pad);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+}  // extern "C"

@@ -446,3 +446,147 @@ int orc_sparse_init_factor(int nv, int nv_pad, int block, int nslots, int nlevel
   }
   return 0;
 }
+
+/* ------------------------------------------------------------------ blocked dense Cholesky
+ * Restatement of the indexed blocked upper Cholesky factor + solve
+ * (src/instantmimic/utils/mjw_kernels/indexed_factor.py:15-173; block index layout and
+ * identity padding of src/instantmimic/utils/mjw_step_optimized.py:893-955).  The block
+ * schedule is the reference's; the arithmetic inside a tile is Warp's tile library
+ * (third party, absent), so the order INSIDE a tile operation is this file's own
+ * convention ("parity unpinned" at bit level, pinned to fp64 algebra by the tests):
+ *   matmul(A', B, C, alpha=-1):  sum = fold_t fmaf(A[t][r], B[t][c], sum) from 0; C = C - sum
+ *   cholesky (lower L, U = L'):  s = A[j][j]; s = fmaf(-L[j][k], L[j][k], s) k ascending;
+ *                                L[j][j] = sqrtf(s); inv = 1 / L[j][j];
+ *                                L[i][j] = (A[i][j] - fold_k L[i][k] L[j][k]) * inv
+ *   lower solve L z = b:         column oriented, j ascending: z[j] = s[j] / L[j][j];
+ *                                s[i] = fmaf(-L[i][j], z[j], s[i]) for i > j
+ *   upper solve U x = b:         column oriented, r descending: x[r] = s[r] / U[r][r];
+ *                                s[t] = fmaf(-U[t][r], x[r], s[t]) for t < r */
+static void blocked_world(int nv, int pad, int B, int nM, const float *M, const int *bidx,
+                          const float *y, float *U, float *x, float *rhs, float *A, float *L) {
+  const int nblk = pad / B, BB = B * B;
+  for (int i = 0; i < pad; ++i) rhs[i] = i < nv ? y[i] : 0.0f;
+  for (int i = 0; i < pad * pad; ++i) U[i] = 0.0f;
+  for (int kb = 0; kb < nblk; ++kb) {
+    const int k = kb * B, end = k + B;
+    const int *idx = bidx + (size_t)(kb * nblk + kb) * BB;
+    for (int e = 0; e < BB; ++e) {
+      float v = idx[e] < nM ? M[idx[e]] : 0.0f;
+      const int r = e / B, c = e % B;
+      if (end > nv && r == c && (nblk - 1) * B + r >= nv) v = v + 1.0f;
+      A[e] = v;
+    }
+    for (int jb = 0; jb < kb; ++jb) {
+      const int j = jb * B;
+      for (int r = 0; r < B; ++r)
+        for (int c = 0; c < B; ++c) {
+          float sum = 0.0f;
+          for (int t = 0; t < B; ++t) sum = fmaf(U[(j + t) * pad + k + r], U[(j + t) * pad + k + c], sum);
+          A[r * B + c] = A[r * B + c] - sum;
+        }
+      for (int r = 0; r < B; ++r) {
+        float sum = 0.0f;
+        for (int t = 0; t < B; ++t) sum = fmaf(U[(j + t) * pad + k + r], rhs[j + t], sum);
+        rhs[k + r] = rhs[k + r] - sum;
+      }
+    }
+    for (int j = 0; j < B; ++j) {
+      float s = A[j * B + j];
+      for (int q = 0; q < j; ++q) s = fmaf(-L[j * B + q], L[j * B + q], s);
+      const float d = sqrtf(s), inv = 1.0f / d;
+      L[j * B + j] = d;
+      for (int i = j + 1; i < B; ++i) {
+        float v = A[i * B + j];
+        for (int q = 0; q < j; ++q) v = fmaf(-L[i * B + q], L[j * B + q], v);
+        L[i * B + j] = v * inv;
+      }
+    }
+    for (int r = 0; r < B; ++r)
+      for (int c = r; c < B; ++c) U[(k + r) * pad + k + c] = L[c * B + r];
+    for (int j = 0; j < B; ++j) {
+      const float z = rhs[k + j] / L[j * B + j];
+      rhs[k + j] = z;
+      for (int i = j + 1; i < B; ++i) rhs[k + i] = fmaf(-L[i * B + j], z, rhs[k + i]);
+    }
+    for (int ib = kb + 1; ib < nblk; ++ib) {
+      const int i0 = ib * B;
+      const int *idx2 = bidx + (size_t)(kb * nblk + ib) * BB;
+      for (int e = 0; e < BB; ++e) A[e] = idx2[e] < nM ? M[idx2[e]] : 0.0f;
+      for (int jb = 0; jb < kb; ++jb) {
+        const int j = jb * B;
+        for (int r = 0; r < B; ++r)
+          for (int c = 0; c < B; ++c) {
+            float sum = 0.0f;
+            for (int t = 0; t < B; ++t) sum = fmaf(U[(j + t) * pad + k + r], U[(j + t) * pad + i0 + c], sum);
+            A[r * B + c] = A[r * B + c] - sum;
+          }
+      }
+      for (int c = 0; c < B; ++c)
+        for (int j = 0; j < B; ++j) {
+          const float z = A[j * B + c] / L[j * B + j];
+          A[j * B + c] = z;
+          for (int i = j + 1; i < B; ++i) A[i * B + c] = fmaf(-L[i * B + j], z, A[i * B + c]);
+        }
+      for (int r = 0; r < B; ++r)
+        for (int c = 0; c < B; ++c) U[(k + r) * pad + i0 + c] = A[r * B + c];
+    }
+  }
+  for (int i0 = pad - B; i0 >= 0; i0 -= B) {
+    for (int j = i0 + B; j < pad; j += B)
+      for (int r = 0; r < B; ++r) {
+        float sum = 0.0f;
+        for (int t = 0; t < B; ++t) sum = fmaf(U[(i0 + r) * pad + j + t], rhs[j + t], sum);
+        rhs[i0 + r] = rhs[i0 + r] - sum;
+      }
+    for (int r = B - 1; r >= 0; --r) {
+      const float xv = rhs[i0 + r] / U[(i0 + r) * pad + i0 + r];
+      rhs[i0 + r] = xv;
+      for (int t = 0; t < r; ++t) rhs[i0 + t] = fmaf(-U[(i0 + t) * pad + i0 + r], xv, rhs[i0 + t]);
+    }
+  }
+  for (int i = 0; i < nv; ++i) x[i] = rhs[i];
+}
+
+int orc_blocked_factor_solve(int nworld, int nv, int pad, int B, int nM, const float *M, int ldM,
+                             const int *block_idx, const float *y, float *U, float *x) {
+#pragma omp parallel
+  {
+    float *work = (float *)malloc(sizeof(float) * (pad + 2 * B * B + 8));
+    float *Ul = U ? 0 : (float *)malloc(sizeof(float) * pad * pad);
+#pragma omp for schedule(static)
+    for (int w = 0; w < nworld; ++w)
+      blocked_world(nv, pad, B, nM, M + (size_t)w * ldM, block_idx, y + (size_t)w * nv,
+                    U ? U + (size_t)w * pad * pad : Ul, x + (size_t)w * nv, work, work + pad,
+                    work + pad + B * B);
+    free(work);
+    free(Ul);
+  }
+  return 0;
+}
+
+/* Dense H = M + J' diag(D [state == quad]) J into (nv_pad, nv_pad) per world, rows summed
+ * in ascending order with fmaf(J[r][i] * Dc, J[r][j], h) starting from M (upper and lower
+ * triangle filled).  The reference takes this from mujoco_warp's solver (third party,
+ * absent); call sites src/instantmimic/utils/mjw_kernels/newton_fusion.py:470. */
+int orc_jtdj_dense(int nworld, int nv, int nv_pad, const float *Mdense, const float *J, int njmax,
+                   const float *D, const int *state, const int *nefc, int quad, float *H) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    float *h = H + (size_t)w * nv_pad * nv_pad;
+    const float *m = Mdense + (size_t)w * nv * nv;
+    int n = nefc ? nefc[w] : njmax;
+    if (n > njmax) n = njmax;
+    for (int i = 0; i < nv_pad * nv_pad; ++i) h[i] = 0.0f;
+    for (int i = 0; i < nv; ++i)
+      for (int j = 0; j < nv; ++j) {
+        float v = m[i * nv + j];
+        for (int r = 0; r < n; ++r) {
+          const float dc = state[(size_t)w * njmax + r] == quad ? D[(size_t)w * njmax + r] : 0.0f;
+          const float *Jr = J + ((size_t)w * njmax + r) * nv;
+          v = fmaf(Jr[i] * dc, Jr[j], v);
+        }
+        h[i * nv_pad + j] = v;
+      }
+  }
+  return 0;
+}

@@ -261,3 +261,29 @@ def sparse_init_factor(plan, nefc, J, D, state, M, grad, hfactor=None, done=None
     )  # fmt: skip
     assert status == 0
     return hf, search, sdot, decr
+
+
+# ---------------------------------------------------------------- blocked dense Cholesky, dense J'DJ
+# Pinning: `blocked_factor_solve` against scipy.linalg.cho_factor / cho_solve in fp64 and the
+# invariant U'U == M; the order inside a tile operation is this oracle's own convention (the
+# reference's tile arithmetic is Warp's, third party): bit-level parity with the reference is
+# UNPINNED for this function, tolerance parity is pinned.  `jtdj_dense` against fp64 einsum.
+
+
+def blocked_factor_solve(M, block_idx, nv, pad, B, y, want_factor=True):
+    M, y = _f(M), _f(y)
+    nworld, nM = M.shape
+    U = np.zeros((nworld, pad, pad), np.float32) if want_factor else None
+    x = np.zeros((nworld, nv), np.float32)
+    lib().orc_blocked_factor_solve(nworld, nv, pad, B, nM, _p(M), nM, _p(_i(block_idx)), _p(y), _p(U), _p(x))
+    return (x, U) if want_factor else x
+
+
+def jtdj_dense(Mdense, J, D, state, nefc, nv_pad, quad=1):
+    Mdense, J, D = _f(Mdense), _f(J), _f(D)
+    state = _i(state)
+    nworld, njmax, nv = J.shape
+    H = np.zeros((nworld, nv_pad, nv_pad), np.float32)
+    ne = _i(nefc) if nefc is not None else None
+    lib().orc_jtdj_dense(nworld, nv, nv_pad, _p(Mdense), _p(J), njmax, _p(D), _p(state), _p(ne), quad, _p(H))
+    return H

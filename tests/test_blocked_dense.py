@@ -1,0 +1,110 @@
+"""Blocked dense Cholesky factor + solve and the dense J'DJ Hessian."""
+
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import scipy.linalg
+
+from instantmimic_amd import synth
+from instantmimic_amd.mjw_kernels import blocked_dense as BD
+from oracle import ref as R
+
+
+def _dense_model(name, nworld, seed=0, well=False):
+    """M of a benchmark tree stored as one dense tile: values (nworld, nv * nv), elemid = identity."""
+    b = synth.make_batch(name, nworld)
+    nv = b.shape.nv
+    Md = synth.dense_from_csr(b.M.astype(np.float64), b.rowadr, b.rownnz, b.colind)
+    if well:
+        Md = Md + 5.0 * np.eye(nv)
+    return b, nv, Md
+
+
+def test_layout_matches_the_reference_scratch():
+    # reference: tests/test_blocked_dense_factor_solve.py:66-91 (nv 56: 64 * 64 indices, 8 identity pads)
+    nv = 56
+    pad, layout, identity = BD.block_index_layout(np.arange(nv * nv), nv, nv * nv, 16)
+    assert pad == 64 and layout.shape == (64 * 64,)
+    assert identity.reshape(16, 16).diagonal().sum() == 8 and identity.sum() == 8
+    assert (layout == nv * nv).sum() == 64 * 64 - nv * nv
+    # block (kb, ib) element (r, c) is M[kb * 16 + r, ib * 16 + c]
+    blk = layout.reshape(4, 4, 16, 16)
+    assert blk[1, 2, 3, 4] == (16 + 3) * nv + 32 + 4
+    # gating
+    m = SimpleNamespace(nv=20, M_tiles=[SimpleNamespace(size=20, elemid=np.arange(400))])
+    assert BD.create_blocked_dense_factor_solve_scratch(m, SimpleNamespace(nworld=1, M=None)) is None
+
+
+@pytest.mark.parametrize("name,B", [("g1", 8), ("g1", 16), ("snu", 16), ("stress", 16)])
+def test_oracle_against_scipy(name, B):
+    b, nv, Md = _dense_model(name, 6, well=True)
+    pad, layout, _ = BD.block_index_layout(np.arange(nv * nv), nv, nv * nv, B)
+    M32 = Md.reshape(6, -1).astype(np.float32)
+    x, U = R.blocked_factor_solve(M32, layout, nv, pad, B, b.grad)
+    for w in range(6):
+        A = M32[w].reshape(nv, nv).astype(np.float64)
+        c = scipy.linalg.cho_factor(A)
+        np.testing.assert_allclose(x[w], scipy.linalg.cho_solve(c, b.grad[w].astype(np.float64)), rtol=2e-4, atol=2e-5)
+        Uw = U[w].astype(np.float64)
+        assert np.abs(np.tril(Uw, -1)).max() == 0.0
+        np.testing.assert_allclose((Uw.T @ Uw)[:nv, :nv], A, rtol=1e-5, atol=1e-5)
+        # padded rows factor to the identity
+        np.testing.assert_array_equal(Uw[nv:, nv:], np.eye(pad - nv))
+        np.testing.assert_allclose(np.triu(Uw[:nv, :nv]), np.triu(scipy.linalg.cholesky(A)), rtol=2e-4, atol=2e-5)
+
+
+def test_dense_hessian_oracle_against_fp64():
+    b, nv, Md = _dense_model("g1", 5)
+    H = R.jtdj_dense(Md.reshape(5, -1), b.J, b.D, b.state[0], b.nefc, 48)
+    H64 = R.assemble_dense64(b.rowadr, b.rownnz, b.colind, b.M, b.J, b.D, b.state[0], b.nefc)
+    assert R.rel_l2(H[:, :nv, :nv], H64) < 1e-6
+    assert np.abs(H[:, nv:, :]).max() == 0 and np.abs(H[:, :, nv:]).max() == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,B,nworld", [("g1", 8, 70), ("g1", 16, 70), ("snu", 16, 33), ("stress", 16, 9)])
+def test_gpu_blocked_factor_solve_bitwise(device, name, B, nworld):
+    import torch
+
+    b, nv, Md = _dense_model(name, nworld)
+    M32 = np.ascontiguousarray(Md.reshape(nworld, -1).astype(np.float32))
+    m = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))])
+    M = torch.from_numpy(M32).to(device)
+    d = SimpleNamespace(nworld=nworld, M=M)
+    scratch = BD.create_blocked_dense_factor_solve_scratch(m, d, device, block_size=B)
+    assert scratch is not None and scratch.pad == -(-nv // B) * B
+    y = torch.from_numpy(b.grad).to(device)
+    x = torch.full_like(y, float("nan"))
+    BD._blocked_dense_factor_solve(d, M, x.reshape(nworld, nv, 1), y.reshape(nworld, nv, 1), scratch)
+    torch.cuda.synchronize()
+    x_ref, U_ref = R.blocked_factor_solve(M32, scratch.indices.cpu().numpy(), nv, scratch.pad, B, b.grad)
+    np.testing.assert_array_equal(scratch.U.cpu().numpy(), U_ref)
+    np.testing.assert_array_equal(x.cpu().numpy(), x_ref)
+    assert R.rel_l2(x.cpu().numpy(), x_ref) <= 1e-5
+    # residual of the fp32 solve against the matrix
+    res = np.einsum("wij,wj->wi", Md, x.cpu().numpy().astype(np.float64)) - b.grad
+    scale = np.linalg.norm(Md, axis=(1, 2)) * np.linalg.norm(x_ref, axis=1) + np.linalg.norm(b.grad, axis=1)
+    assert (np.linalg.norm(res, axis=1) / scale).max() < 5e-6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,nworld", [("g1", 40), ("stress", 24)])
+def test_gpu_dense_hessian_mfma(device, name, nworld):
+    import torch
+
+    b = synth.make_batch(name, nworld, ragged_nefc=True)
+    nv = b.shape.nv
+    nv_pad = ((nv + 1 + 15) // 16) * 16
+    Md = synth.dense_from_csr(b.M.astype(np.float64), b.rowadr, b.rownnz, b.colind).astype(np.float32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    H = torch.zeros((nworld, nv_pad, nv_pad), device=device)
+    BD.dense_hessian(t(Md), t(b.J), t(b.D), t(b.state[0]), t(b.nefc), H)
+    torch.cuda.synchronize()
+    Hh = H.cpu().numpy()
+    H64 = R.assemble_dense64(b.rowadr, b.rownnz, b.colind, b.M, b.J, b.D, b.state[0], b.nefc)
+    # the matrix cores sum in their own order: tolerance parity (1e-5 relative L2, fp32)
+    assert R.rel_l2(Hh[:, :nv, :nv], H64) <= 1e-5
+    assert R.rel_l2(Hh, R.jtdj_dense(Md.reshape(nworld, -1), b.J, b.D, b.state[0], b.nefc, nv_pad)) <= 1e-5
+    np.testing.assert_array_equal(Hh, Hh.transpose(0, 2, 1))
+    assert np.abs(Hh[:, nv:, :]).max() == 0
