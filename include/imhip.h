@@ -180,6 +180,106 @@ int im_muscle_implicit_gather(const float *moment, int64_t ld_moment, const floa
                               int chunk_count, float timestep, float *qderiv,
                               int64_t ld_qderiv, int nworld, void *stream);
 
+/* Muscle path geometry, activation -> torque and its gradient ------------------ */
+
+/* Curves of src/instantmimic/muscle/muscle_qfrc_projector.py:103-187.  active =
+ * (type, p1, p2): type < 0.5 gaussian with gamma = p1, else MuJoCo piecewise with
+ * (lmin, lmax) = (p1, p2).  passive = (type, p1, p2): type < 0.5 exponential with
+ * (k_pe, e_mo), else MuJoCo with (lmax, fpmax). */
+typedef struct im_muscle_force_model {
+  float force_scale;
+  float length_norm_min, length_norm_max;
+  float active[3];
+  float passive[3];
+  int32_t include_passive; /* 0 writes zeros to passive_force */
+} im_muscle_force_model;
+
+/* Per-world pose arrays, ld* = row stride in floats: waypoints (nworld, 3 nwaypoint),
+ * subtree_com (nworld, 3 nbody), cdof (nworld, 6 nv) with angular xyz then linear xyz. */
+typedef struct im_muscle_geometry {
+  const float *waypoints;
+  int64_t ld_waypoints;
+  const float *subtree_com;
+  int64_t ld_subtree_com;
+  const float *cdof;
+  int64_t ld_cdof;
+} im_muscle_geometry;
+
+/* Applied segments: waypoint ids of both ends and the tree-root body of each end's body
+ * (apply_segment_start_idx / _end_idx, segment_*_root_body_idx_i32 of the reference's
+ * MuscleDynamicsLayer, src/instantmimic/muscle/muscle_dynamics.py:1318-1341). */
+typedef struct im_muscle_segments {
+  const int32_t *start_waypoint, *end_waypoint, *start_root_body, *end_root_body;
+  int32_t nsegment;
+} im_muscle_segments;
+
+/* A CSR list of (segment, other) entries with the start/end subtree coefficients:
+ * rows = torque dofs and other = muscle (build_torque_sparse_segment_entries,
+ * muscle_qfrc_projector.py:378-456), rows = muscles and other = torque dof
+ * (build_muscle_sparse_torque_entries, :459-510), or rows = (muscle, dof) entries and
+ * other unused (MuscleDofSparseEntries, :513-533). */
+typedef struct im_muscle_entries {
+  const int32_t *offsets; /* nrow + 1 */
+  const int32_t *segment; /* nentry */
+  const int32_t *other;   /* nentry or null */
+  const float *start_coeff, *end_coeff;
+  int32_t nrow, nentry;
+} im_muscle_entries;
+
+/* Replaces _transform_waypoints_from_torch_kernel
+ * (src/instantmimic/muscle/muscle_dynamics_kernels.py:73-86): xpos (nworld, 3 nbody),
+ * xquat (nworld, 4 nbody) scalar first, normalised with the reference's 1e-8 guard. */
+int im_muscle_waypoints(const float *xpos, int64_t ld_xpos, const float *xquat,
+                        int64_t ld_xquat, const int32_t *waypoint_body,
+                        const float *waypoint_local, int nwaypoint, float *waypoints,
+                        int64_t ld_waypoints, int nworld, void *stream);
+
+/* Replaces _compute_force_magnitudes_from_waypoints_kernel
+ * (muscle_dynamics_kernels.py:644-705): polyline length over every segment of a muscle,
+ * normalised fibre length, unit (activation 1) and passive force magnitudes.
+ * muscle_params (nmuscle, ld_params >= 4) = f0, l_m0, l_t0, pennation.  passive_force may
+ * be null. */
+int im_muscle_force_magnitudes(const float *waypoints, int64_t ld_waypoints,
+                               const int32_t *all_segment_start_idx,
+                               const int32_t *all_muscle_segment_offsets,
+                               const float *muscle_params, int ld_params,
+                               const float *muscle_rest_length,
+                               const im_muscle_force_model *model, int nmuscle,
+                               float *unit_force, int64_t ld_unit, float *passive_force,
+                               int64_t ld_passive, int nworld, void *stream);
+
+/* Replaces _compute_muscle_dynamics_from_activation_sparse_kernel
+ * (muscle_dynamics_kernels.py:1707-1793), the body of the operator
+ * instantmimic_muscle::torque_forward (src/instantmimic/muscle/warp_custom_ops.py:98-114).
+ * passive_force null = the include_passive_force=False specialisation.
+ * torque (nworld, ld_torque >= torque_entries->nrow). */
+int im_muscle_torque_forward(const im_muscle_geometry *geometry,
+                             const im_muscle_segments *segments,
+                             const im_muscle_entries *torque_entries, const float *unit_force,
+                             int64_t ld_unit, const float *passive_force, int64_t ld_passive,
+                             const float *activation, int64_t ld_activation, int root_dof_count,
+                             float *torque, int64_t ld_torque, int nworld, void *stream);
+
+/* Replaces _compute_muscle_dynamics_activation_grad_sparse_kernel
+ * (muscle_dynamics_kernels.py:1796-1859), the body of instantmimic_muscle::torque_backward
+ * (warp_custom_ops.py:133-149).  Every element of grad_activation is written (zero where
+ * the unit force is zero), so the output needs no clearing. */
+int im_muscle_activation_grad(const im_muscle_geometry *geometry,
+                              const im_muscle_segments *segments,
+                              const im_muscle_entries *muscle_entries, const float *unit_force,
+                              int64_t ld_unit, const float *grad_output, int64_t ld_grad_output,
+                              int root_dof_count, float *grad_activation,
+                              int64_t ld_grad_activation, int nworld, void *stream);
+
+/* Replaces eval_muscle_sparse_moment_kernel
+ * (src/instantmimic/muscle/muscle_qfrc_projector.py:2617-2662): moment[w, e] = sum over
+ * the segments of (muscle, dof) entry e of the unit-force contribution. */
+int im_muscle_sparse_moment(const im_muscle_geometry *geometry,
+                            const im_muscle_segments *segments,
+                            const int32_t *muscle_dof_torque_idx,
+                            const im_muscle_entries *entry_segments, int root_dof_count,
+                            float *moment, int64_t ld_moment, int nworld, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

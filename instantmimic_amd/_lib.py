@@ -33,6 +33,42 @@ class TreePlanInfo(C.Structure):
 
 _vp, _i, _i64, _u = C.c_void_p, C.c_int, C.c_int64, C.c_uint
 
+
+class MuscleForceModel(C.Structure):
+    _fields_ = [
+        ("force_scale", C.c_float),
+        ("length_norm_min", C.c_float),
+        ("length_norm_max", C.c_float),
+        ("active", C.c_float * 3),
+        ("passive", C.c_float * 3),
+        ("include_passive", C.c_int32),
+    ]
+
+
+class MuscleGeometry(C.Structure):
+    _fields_ = [
+        ("waypoints", _vp), ("ld_waypoints", _i64),
+        ("subtree_com", _vp), ("ld_subtree_com", _i64),
+        ("cdof", _vp), ("ld_cdof", _i64),
+    ]  # fmt: skip
+
+
+class MuscleSegments(C.Structure):
+    _fields_ = [
+        ("start_waypoint", _vp), ("end_waypoint", _vp), ("start_root_body", _vp), ("end_root_body", _vp),
+        ("nsegment", C.c_int32),
+    ]  # fmt: skip
+
+
+class MuscleEntries(C.Structure):
+    _fields_ = [
+        ("offsets", _vp), ("segment", _vp), ("other", _vp), ("start_coeff", _vp), ("end_coeff", _vp),
+        ("nrow", C.c_int32), ("nentry", C.c_int32),
+    ]  # fmt: skip
+
+
+_pgeo, _pseg, _pent = C.POINTER(MuscleGeometry), C.POINTER(MuscleSegments), C.POINTER(MuscleEntries)
+
 # name -> (restype, argtypes); the single list of symbols the header declares
 SIGNATURES = {
     "im_version": (_i, []),
@@ -61,6 +97,17 @@ SIGNATURES = {
         _i,
         [_vp, _i64, _vp, _i64, _vp, _i, _vp, _i, _vp, _vp, _i, C.c_float, _vp, _i64, _i, _vp],
     ),
+    "im_muscle_waypoints": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _i, _vp, _i64, _i, _vp]),
+    "im_muscle_force_magnitudes": (
+        _i,
+        [_vp, _i64, _vp, _vp, _vp, _i, _vp, C.POINTER(MuscleForceModel), _i, _vp, _i64, _vp, _i64, _i, _vp],
+    ),
+    "im_muscle_torque_forward": (
+        _i,
+        [_pgeo, _pseg, _pent, _vp, _i64, _vp, _i64, _vp, _i64, _i, _vp, _i64, _i, _vp],
+    ),
+    "im_muscle_activation_grad": (_i, [_pgeo, _pseg, _pent, _vp, _i64, _vp, _i64, _i, _vp, _i64, _i, _vp]),
+    "im_muscle_sparse_moment": (_i, [_pgeo, _pseg, _vp, _pent, _i, _vp, _i64, _i, _vp]),
 }
 
 _lib = None

@@ -1,0 +1,398 @@
+// Muscle path geometry and activation <-> joint-torque contractions for gfx950.
+//
+//   waypoints[w, i]   = xpos[w, body(i)] + rot(local(i), normalize(xquat[w, body(i)]))
+//     reference: src/instantmimic/muscle/muscle_dynamics_kernels.py:73-86
+//   unit/passive force magnitudes per (world, muscle) from the polyline length
+//     reference: muscle_dynamics_kernels.py:644-705, curves muscle_qfrc_projector.py:103-277
+//   torque[w, j]      = sum over the active (segment, muscle) entries of torque dof j of
+//                       contribution(segment, dof j, unit * activation (+ passive))
+//     reference: muscle_dynamics_kernels.py:1707-1793
+//   grad_act[w, m]    = sum over muscle m's (segment, torque) entries of
+//                       grad_out[w, j] * contribution(segment, dof j, unit)
+//     reference: muscle_dynamics_kernels.py:1796-1859
+//   moment[w, e]      = sum over entry e's segments of contribution(segment, dof(e), 1)
+//     reference: muscle_qfrc_projector.py:2617-2662
+//   contribution      = dot(a (lin + ang x (p0 - c0)) - b (lin + ang x (p1 - c1)), f dir)
+//     reference: muscle_qfrc_projector.py:280-304
+//
+// All five are gathers over a world's row of poses (a few KB, L1/L2 resident after the
+// first touch) and write one float per thread; none of them reuses data across worlds, so
+// they are HBM bound on the pose rows.  Threads are laid out output-major inside a world
+// so that a wavefront's writes coalesce.  Arithmetic is written out operation by operation
+// (this file is compiled without floating-point contraction) and the CPU checker follows
+// the same order.
+#include <hip/hip_runtime.h>
+
+#include "../../include/imhip.h"
+#include "common.h"
+
+namespace im {
+namespace {
+
+struct V3 {
+  float x, y, z;
+};
+__device__ __forceinline__ V3 ld3(const float *p) { return {p[0], p[1], p[2]}; }
+__device__ __forceinline__ V3 sub(V3 a, V3 b) { return {a.x - b.x, a.y - b.y, a.z - b.z}; }
+__device__ __forceinline__ V3 add(V3 a, V3 b) { return {a.x + b.x, a.y + b.y, a.z + b.z}; }
+__device__ __forceinline__ V3 scale(float s, V3 a) { return {s * a.x, s * a.y, s * a.z}; }
+__device__ __forceinline__ float dot(V3 a, V3 b) { return a.x * b.x + a.y * b.y + a.z * b.z; }
+__device__ __forceinline__ V3 cross(V3 a, V3 b) {
+  return {a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x};
+}
+__device__ __forceinline__ float length(V3 a) { return sqrtf(dot(a, a)); }
+
+// muscle_qfrc_projector.py:280-304
+__device__ __forceinline__ float contribution(V3 lin, V3 ang, V3 p0, V3 p1, V3 c0, V3 c1, float a,
+                                              float b, float force) {
+  const V3 seg = sub(p1, p0);
+  const float len = length(seg);
+  if (len < 1.0e-8f) return 0.0f;
+  const V3 dir = {seg.x / len, seg.y / len, seg.z / len};
+  const V3 f = scale(force, dir);
+  const V3 st = add(lin, cross(ang, sub(p0, c0)));
+  const V3 en = add(lin, cross(ang, sub(p1, c1)));
+  return dot(sub(scale(a, st), scale(b, en)), f);
+}
+
+struct Geo {
+  const float *wp, *com, *cdof;
+  int64_t ldw, ldc, ldd;
+};
+struct Seg {
+  const int32_t *p0, *p1, *b0, *b1;
+};
+
+__device__ __forceinline__ float seg_term(const Geo &g, const Seg &s, int64_t w, int seg, V3 lin,
+                                          V3 ang, float a, float b, float force) {
+  const float *wp = g.wp + w * g.ldw, *com = g.com + w * g.ldc;
+  return contribution(lin, ang, ld3(wp + 3 * s.p0[seg]), ld3(wp + 3 * s.p1[seg]),
+                      ld3(com + 3 * s.b0[seg]), ld3(com + 3 * s.b1[seg]), a, b, force);
+}
+
+__global__ __launch_bounds__(256) void waypoints_kernel(
+    const float *__restrict__ xpos, int64_t ldp, const float *__restrict__ xquat, int64_t ldq,
+    const int32_t *__restrict__ wp_body, const float *__restrict__ wp_local, int nwp,
+    float *__restrict__ out, int64_t ldo, int nworld) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t w = blockIdx.y;
+  if (i >= nwp) return;
+  const int b = wp_body[i];
+  const float *q = xquat + w * ldq + 4 * b;
+  const float q0 = q[0], q1 = q[1], q2 = q[2], q3 = q[3];
+  // muscle_qfrc_projector.py:91-100
+  const float inv = 1.0f / sqrtf(q0 * q0 + q1 * q1 + q2 * q2 + q3 * q3 + 1.0e-8f);
+  const float s = q0 * inv;
+  const V3 u = {q1 * inv, q2 * inv, q3 * inv};
+  const V3 v = ld3(wp_local + 3 * i);
+  // mujoco_warp math.rot_vec_quat: 2 (u.v) u + (s s - u.u) v + 2 s (u x v)
+  V3 r = add(scale(2.0f, scale(dot(u, v), u)), scale(s * s - dot(u, u), v));
+  r = add(r, scale(2.0f * s, cross(u, v)));
+  const V3 p = add(ld3(xpos + w * ldp + 3 * b), r);
+  float *o = out + w * ldo + 3 * i;
+  o[0] = p.x;
+  o[1] = p.y;
+  o[2] = p.z;
+}
+
+// muscle_qfrc_projector.py:103-187
+__device__ __forceinline__ float active_fl(float l, const float *m) {
+  if (m[0] < 0.5f) return expf(-((l - 1.0f) * (l - 1.0f)) / m[1]);
+  const float lmin = m[1], lmax = m[2];
+  if (l < lmin || l > lmax) return 0.0f;
+  const float lo = 0.5f * (lmin + 1.0f), hi = 0.5f * (1.0f + lmax);
+  if (l <= lo) {
+    const float x = (l - lmin) / fmaxf(lo - lmin, 1.0e-8f);
+    return 0.5f * x * x;
+  }
+  if (l <= 1.0f) {
+    const float x = (1.0f - l) / fmaxf(1.0f - lo, 1.0e-8f);
+    return 1.0f - 0.5f * x * x;
+  }
+  if (l <= hi) {
+    const float x = (l - 1.0f) / fmaxf(hi - 1.0f, 1.0e-8f);
+    return 1.0f - 0.5f * x * x;
+  }
+  const float x = (lmax - l) / fmaxf(lmax - hi, 1.0e-8f);
+  return 0.5f * x * x;
+}
+__device__ __forceinline__ float passive_fl(float l, const float *m) {
+  if (m[0] < 0.5f) {
+    if (l < 1.0f) return 0.0f;
+    float x = m[1] * (l - 1.0f) / m[2];
+    x = fminf(fmaxf(x, -80.0f), 80.0f);
+    return (expf(x) - 1.0f) / (expf(m[1]) - 1.0f);
+  }
+  const float lmax = m[1], fpmax = m[2];
+  if (l <= 1.0f) return 0.0f;
+  const float mid = 0.5f * (1.0f + lmax), width = fmaxf(mid - 1.0f, 1.0e-8f);
+  if (l <= mid) {
+    const float st = (l - 1.0f) / width;
+    return 0.5f * fpmax * st * st;
+  }
+  return fpmax * (0.5f + (l - mid) / width);
+}
+
+__global__ __launch_bounds__(256) void force_kernel(
+    const float *__restrict__ wp, int64_t ldw, const int32_t *__restrict__ seg_start,
+    const int32_t *__restrict__ seg_offsets, const float *__restrict__ params, int ldpar,
+    const float *__restrict__ rest, im_muscle_force_model model, int nmuscle,
+    float *__restrict__ unit, int64_t ldu, float *__restrict__ passive, int64_t ldpa) {
+  const int m = blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t w = blockIdx.y;
+  if (m >= nmuscle) return;
+  const float *row = wp + w * ldw;
+  float len = 0.0f;  // muscle_dynamics_kernels.py:452-473
+  for (int s = seg_offsets[m]; s < seg_offsets[m + 1]; ++s) {
+    const int i = seg_start[s];
+    len = len + length(sub(ld3(row + 3 * (i + 1)), ld3(row + 3 * i)));
+  }
+  const float f0 = params[m * ldpar], lm0 = params[m * ldpar + 1], lt0 = params[m * ldpar + 2],
+              pen = params[m * ldpar + 3];
+  // muscle_qfrc_projector.py:190-205
+  const float lm = len / fmaxf(rest[m], 1.0e-6f) - lt0;
+  const float ln =
+      fminf(fmaxf(lm / fmaxf(lm0, 1.0e-6f), model.length_norm_min), model.length_norm_max);
+  const float c = cosf(pen);
+  unit[w * ldu + m] = f0 * active_fl(ln, model.active) * c * model.force_scale;
+  if (passive) {
+    float pv = 0.0f;
+    // muscle_qfrc_projector.py:249-277 with include_active 0, include_passive 1
+    if (model.include_passive)
+      pv = f0 * passive_fl(ln, model.passive) * c * model.force_scale;
+    passive[w * ldpa + m] = pv;
+  }
+}
+
+__global__ __launch_bounds__(256) void torque_forward_kernel(
+    Geo g, Seg s, const int32_t *__restrict__ offsets, const int32_t *__restrict__ e_seg,
+    const int32_t *__restrict__ e_muscle, const float *__restrict__ e_a,
+    const float *__restrict__ e_b, const float *__restrict__ unit, int64_t ldu,
+    const float *__restrict__ passive, int64_t ldpa, const float *__restrict__ act, int64_t lda,
+    int root, int ntorque, float *__restrict__ out, int64_t ldo) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t w = blockIdx.y;
+  if (j >= ntorque) return;
+  const float *cd = g.cdof + w * g.ldd + 6 * (int64_t)(j + root);
+  const V3 ang = ld3(cd), lin = ld3(cd + 3);
+  float total = 0.0f;
+  for (int e = offsets[j]; e < offsets[j + 1]; ++e) {
+    const int m = e_muscle[e];
+    float f = unit[w * ldu + m] * act[w * lda + m];
+    if (passive) f = f + passive[w * ldpa + m];
+    if (f == 0.0f) continue;
+    total = total + seg_term(g, s, w, e_seg[e], lin, ang, e_a[e], e_b[e], f);
+  }
+  out[w * ldo + j] = total;
+}
+
+__global__ __launch_bounds__(256) void activation_grad_kernel(
+    Geo g, Seg s, const int32_t *__restrict__ offsets, const int32_t *__restrict__ e_seg,
+    const int32_t *__restrict__ e_torque, const float *__restrict__ e_a,
+    const float *__restrict__ e_b, const float *__restrict__ unit, int64_t ldu,
+    const float *__restrict__ gout, int64_t ldg, int root, int nmuscle, float *__restrict__ gact,
+    int64_t lda) {
+  const int m = blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t w = blockIdx.y;
+  if (m >= nmuscle) return;
+  const float f = unit[w * ldu + m];
+  float grad = 0.0f;
+  // The reference returns before the store when f == 0 and relies on a zero-filled
+  // output (muscle_dynamics_kernels.py:1817-1819); the store of 0 here is the same value.
+  if (f != 0.0f) {
+    for (int e = offsets[m]; e < offsets[m + 1]; ++e) {
+      const int j = e_torque[e];
+      const float *cd = g.cdof + w * g.ldd + 6 * (int64_t)(j + root);
+      grad = grad + gout[w * ldg + j] *
+                        seg_term(g, s, w, e_seg[e], ld3(cd + 3), ld3(cd), e_a[e], e_b[e], f);
+    }
+  }
+  gact[w * lda + m] = grad;
+}
+
+__global__ __launch_bounds__(256) void sparse_moment_kernel(
+    Geo g, Seg s, const int32_t *__restrict__ entry_torque, const int32_t *__restrict__ offsets,
+    const int32_t *__restrict__ e_seg, const float *__restrict__ e_a,
+    const float *__restrict__ e_b, int root, int nentry, float *__restrict__ moment, int64_t ldm) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t w = blockIdx.y;
+  if (e >= nentry) return;
+  const float *cd = g.cdof + w * g.ldd + 6 * (int64_t)(entry_torque[e] + root);
+  const V3 ang = ld3(cd), lin = ld3(cd + 3);
+  float total = 0.0f;
+  for (int k = offsets[e]; k < offsets[e + 1]; ++k)
+    total = total + seg_term(g, s, w, e_seg[k], lin, ang, e_a[k], e_b[k], 1.0f);
+  moment[w * ldm + e] = total;
+}
+
+bool geo_ok(const im_muscle_geometry *g) {
+  return g && g->waypoints && g->subtree_com && g->cdof && g->ld_waypoints >= 0 &&
+         g->ld_subtree_com >= 0 && g->ld_cdof >= 0;
+}
+bool seg_ok(const im_muscle_segments *s) {
+  return s && s->start_waypoint && s->end_waypoint && s->start_root_body && s->end_root_body;
+}
+Geo geo(const im_muscle_geometry *g) {
+  return {g->waypoints, g->subtree_com, g->cdof, g->ld_waypoints, g->ld_subtree_com, g->ld_cdof};
+}
+Seg seg(const im_muscle_segments *s) {
+  return {s->start_waypoint, s->end_waypoint, s->start_root_body, s->end_root_body};
+}
+dim3 grid2(int n, int nworld) { return dim3((unsigned)((n + 255) / 256), (unsigned)nworld); }
+constexpr int kMaxGridY = 65535;
+int slab_count(int nworld, int w0) { return nworld - w0 < kMaxGridY ? nworld - w0 : kMaxGridY; }
+
+}  // namespace
+}  // namespace im
+
+using namespace im;
+
+// The y dimension of a grid carries the world; launches are split so that it stays within
+// the limit of 65535.
+#define IM_FOR_WORLD_SLABS(nworld, w0, nw)                                     \
+  for (int w0 = 0, nw = slab_count(nworld, 0); w0 < (nworld); \
+       w0 += kMaxGridY, nw = slab_count(nworld, w0))
+
+extern "C" int im_muscle_waypoints(const float *xpos, int64_t ld_xpos, const float *xquat,
+                                   int64_t ld_xquat, const int32_t *waypoint_body,
+                                   const float *waypoint_local, int nwaypoint, float *waypoints,
+                                   int64_t ld_waypoints, int nworld, void *stream) {
+  if (nworld < 0 || nwaypoint < 0) return IM_ERR_ARG;
+  if (nworld == 0 || nwaypoint == 0) return IM_OK;
+  if (!xpos || !xquat || !waypoint_body || !waypoint_local || !waypoints) return IM_ERR_ARG;
+  if (ld_waypoints < 3 * (int64_t)nwaypoint) return IM_ERR_STRIDE;
+  IM_FOR_WORLD_SLABS(nworld, w0, nw) {
+    hipLaunchKernelGGL(waypoints_kernel, grid2(nwaypoint, nw), dim3(256), 0, (hipStream_t)stream,
+                       xpos + w0 * ld_xpos, ld_xpos, xquat + w0 * ld_xquat, ld_xquat,
+                       waypoint_body, waypoint_local, nwaypoint, waypoints + w0 * ld_waypoints,
+                       ld_waypoints, nw);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_muscle_force_magnitudes(const float *waypoints, int64_t ld_waypoints,
+                                          const int32_t *all_segment_start_idx,
+                                          const int32_t *all_muscle_segment_offsets,
+                                          const float *muscle_params, int ld_params,
+                                          const float *muscle_rest_length,
+                                          const im_muscle_force_model *model, int nmuscle,
+                                          float *unit_force, int64_t ld_unit,
+                                          float *passive_force, int64_t ld_passive, int nworld,
+                                          void *stream) {
+  if (nworld < 0 || nmuscle < 0 || !model) return IM_ERR_ARG;
+  if (nworld == 0 || nmuscle == 0) return IM_OK;
+  if (!waypoints || !all_segment_start_idx || !all_muscle_segment_offsets || !muscle_params ||
+      !muscle_rest_length || !unit_force || ld_params < 4)
+    return IM_ERR_ARG;
+  if (ld_unit < nmuscle || (passive_force && ld_passive < nmuscle)) return IM_ERR_STRIDE;
+  IM_FOR_WORLD_SLABS(nworld, w0, nw) {
+    hipLaunchKernelGGL(force_kernel, grid2(nmuscle, nw), dim3(256), 0, (hipStream_t)stream,
+                       waypoints + w0 * ld_waypoints, ld_waypoints, all_segment_start_idx,
+                       all_muscle_segment_offsets, muscle_params, ld_params, muscle_rest_length,
+                       *model, nmuscle, unit_force + w0 * ld_unit, ld_unit,
+                       passive_force ? passive_force + w0 * ld_passive : nullptr, ld_passive);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+static Geo slab(const im_muscle_geometry *g, int64_t w0) {
+  Geo r = geo(g);
+  r.wp += w0 * r.ldw;
+  r.com += w0 * r.ldc;
+  r.cdof += w0 * r.ldd;
+  return r;
+}
+
+extern "C" int im_muscle_torque_forward(const im_muscle_geometry *geometry,
+                                        const im_muscle_segments *segments,
+                                        const im_muscle_entries *torque_entries,
+                                        const float *unit_force, int64_t ld_unit,
+                                        const float *passive_force, int64_t ld_passive,
+                                        const float *activation, int64_t ld_activation,
+                                        int root_dof_count, float *torque, int64_t ld_torque,
+                                        int nworld, void *stream) {
+  if (nworld < 0 || !torque_entries || torque_entries->nrow < 0 || root_dof_count < 0)
+    return IM_ERR_ARG;
+  const int nt = torque_entries->nrow;
+  if (nworld == 0 || nt == 0) return IM_OK;
+  if (!geo_ok(geometry) || !seg_ok(segments) || !torque_entries->offsets || !unit_force ||
+      !activation || !torque)
+    return IM_ERR_ARG;
+  if (torque_entries->nentry > 0 && (!torque_entries->segment || !torque_entries->other ||
+                                     !torque_entries->start_coeff || !torque_entries->end_coeff))
+    return IM_ERR_ARG;
+  if (ld_torque < nt) return IM_ERR_STRIDE;
+  IM_FOR_WORLD_SLABS(nworld, w0, nw) {
+    hipLaunchKernelGGL(torque_forward_kernel, grid2(nt, nw), dim3(256), 0, (hipStream_t)stream,
+                       slab(geometry, w0), seg(segments), torque_entries->offsets,
+                       torque_entries->segment, torque_entries->other,
+                       torque_entries->start_coeff, torque_entries->end_coeff,
+                       unit_force + w0 * ld_unit, ld_unit,
+                       passive_force ? passive_force + w0 * ld_passive : nullptr, ld_passive,
+                       activation + w0 * ld_activation, ld_activation, root_dof_count, nt,
+                       torque + w0 * ld_torque, ld_torque);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_muscle_activation_grad(const im_muscle_geometry *geometry,
+                                         const im_muscle_segments *segments,
+                                         const im_muscle_entries *muscle_entries,
+                                         const float *unit_force, int64_t ld_unit,
+                                         const float *grad_output, int64_t ld_grad_output,
+                                         int root_dof_count, float *grad_activation,
+                                         int64_t ld_grad_activation, int nworld, void *stream) {
+  if (nworld < 0 || !muscle_entries || muscle_entries->nrow < 0 || root_dof_count < 0)
+    return IM_ERR_ARG;
+  const int nm = muscle_entries->nrow;
+  if (nworld == 0 || nm == 0) return IM_OK;
+  if (!geo_ok(geometry) || !seg_ok(segments) || !muscle_entries->offsets || !unit_force ||
+      !grad_output || !grad_activation)
+    return IM_ERR_ARG;
+  if (muscle_entries->nentry > 0 && (!muscle_entries->segment || !muscle_entries->other ||
+                                     !muscle_entries->start_coeff || !muscle_entries->end_coeff))
+    return IM_ERR_ARG;
+  if (ld_grad_activation < nm || ld_unit < nm) return IM_ERR_STRIDE;
+  IM_FOR_WORLD_SLABS(nworld, w0, nw) {
+    hipLaunchKernelGGL(activation_grad_kernel, grid2(nm, nw), dim3(256), 0, (hipStream_t)stream,
+                       slab(geometry, w0), seg(segments), muscle_entries->offsets,
+                       muscle_entries->segment, muscle_entries->other,
+                       muscle_entries->start_coeff, muscle_entries->end_coeff,
+                       unit_force + w0 * ld_unit, ld_unit, grad_output + w0 * ld_grad_output,
+                       ld_grad_output, root_dof_count, nm,
+                       grad_activation + w0 * ld_grad_activation, ld_grad_activation);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_muscle_sparse_moment(const im_muscle_geometry *geometry,
+                                       const im_muscle_segments *segments,
+                                       const int32_t *muscle_dof_torque_idx,
+                                       const im_muscle_entries *entry_segments,
+                                       int root_dof_count, float *moment, int64_t ld_moment,
+                                       int nworld, void *stream) {
+  if (nworld < 0 || !entry_segments || entry_segments->nrow < 0 || root_dof_count < 0)
+    return IM_ERR_ARG;
+  const int ne = entry_segments->nrow;
+  if (nworld == 0 || ne == 0) return IM_OK;
+  if (!geo_ok(geometry) || !seg_ok(segments) || !muscle_dof_torque_idx ||
+      !entry_segments->offsets || !moment)
+    return IM_ERR_ARG;
+  if (entry_segments->nentry > 0 && (!entry_segments->segment || !entry_segments->start_coeff ||
+                                     !entry_segments->end_coeff))
+    return IM_ERR_ARG;
+  if (ld_moment < ne) return IM_ERR_STRIDE;
+  IM_FOR_WORLD_SLABS(nworld, w0, nw) {
+    hipLaunchKernelGGL(sparse_moment_kernel, grid2(ne, nw), dim3(256), 0, (hipStream_t)stream,
+                       slab(geometry, w0), seg(segments), muscle_dof_torque_idx,
+                       entry_segments->offsets, entry_segments->segment,
+                       entry_segments->start_coeff, entry_segments->end_coeff, root_dof_count, ne,
+                       moment + w0 * ld_moment, ld_moment);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}

@@ -189,12 +189,13 @@ def make_batch(shape: Shape | str, nworld: int | None = None, *, ragged_nefc: bo
         V = rng.standard_normal((nb, nv, nv)) * mask[None]
         dense = np.einsum("wk,wki,wkj->wij", mass, V, V, optimize=True)
         dense[:, np.arange(nv), np.arange(nv)] += shape.armature
+        body = rng.integers(0, nv, (nb, nefc))
         rows = rng.standard_normal((nb, nefc, nv))
         if supports is not None:
             sup = np.asarray(supports, bool)
-            rows *= sup[rng.integers(0, sup.shape[0], (nb, nefc))]
+            rows *= sup[body % sup.shape[0]]
         elif not shape.dense_rows:
-            rows *= mask[rng.integers(0, nv, (nb, nefc))]
+            rows *= mask[body]
         logd = rng.uniform(shape.logd[0], shape.logd[1], (nb, nefc))
         act = rng.random((shape.iterations, nb, nefc)) < shape.p_active
         g = rng.standard_normal((nb, nv))
@@ -351,3 +352,95 @@ def contact_model():
         names.append("box" + s)
     m = model_from_parents(parent, joints)
     return m, {n: i + 1 for i, n in enumerate(names)}
+
+
+# ------------------------------------------------------------------ muscle rig with path geometry
+
+
+@dataclass
+class MuscleRig:
+    """Waypoint muscles routed over the SNU-like tree: the arrays a MuscleDynamicsLayer is
+    built from plus the model dimensions."""
+
+    topology: object  # muscle.muscle_dynamics.MuscleTopology
+    body_count: int
+    full_torque_dim: int
+    torque_dim: int
+    muscle_count: int
+
+    def dims(self) -> dict:
+        return dict(body_count=self.body_count, full_torque_dim=self.full_torque_dim, torque_dim=self.torque_dim,
+                    muscle_count=self.muscle_count)  # fmt: skip
+
+
+def make_muscle_rig(nmuscle: int = 284, seed: int = 1003) -> MuscleRig:
+    """Each muscle runs over 1-3 adjacent joints of one chain with one or two waypoints on
+    every body it passes (local offsets ~U(-0.08, 0.08) m); the applied segments are the
+    ones whose ends sit on different bodies.  f0 ~ U[100, 3000] N, l_m0 ~ U[0.4, 0.9],
+    l_t0 ~ U[0.1, 0.5], pennation ~ U[0, 0.4] rad, rest length = 0.5 m."""
+    from .muscle.muscle_dynamics import MuscleTopology
+
+    rng = np.random.default_rng([seed, 91])
+    chains = snu_joint_chains()
+    parent = snu_parents()
+    joints = [[0, 1, 2, 3, 4, 5]]
+    for chain in chains:
+        for j in chain:
+            if j not in joints:
+                joints.append(j)
+    joints.sort(key=lambda j: j[0])
+    model = model_from_parents(parent, joints)
+    body_of_dof = {d: b for b, dofs in enumerate(joints, start=1) for d in dofs}
+    nbody = len(joints) + 1
+    wp_body, wp_local, wp_muscle = [], [], []
+    for m in range(nmuscle):
+        chain = chains[int(rng.integers(len(chains)))]
+        span = int(rng.integers(1, 4))
+        first = int(rng.integers(0, len(chain) - span + 1))
+        bodies = [int(model.body_parentid[body_of_dof[chain[first][0]]])]
+        bodies += [body_of_dof[j[0]] for j in chain[first : first + span]]
+        for b in bodies:
+            for _ in range(int(rng.integers(1, 3))):
+                wp_body.append(b)
+                wp_local.append(rng.uniform(-0.08, 0.08, 3))
+                wp_muscle.append(m)
+    wp_body, wp_muscle = np.asarray(wp_body), np.asarray(wp_muscle)
+    start = np.flatnonzero(wp_muscle[:-1] == wp_muscle[1:])
+    crossing = start[wp_body[start] != wp_body[start + 1]]
+    nv = len(parent)
+    dof_bodyid = np.asarray([body_of_dof[d] for d in range(nv)])
+    dof_bodyid[:6] = 0  # the free root's dofs move every body, as world-body dofs do
+    topo = MuscleTopology(
+        muscle_params=np.stack(
+            [rng.uniform(100, 3000, nmuscle), rng.uniform(0.4, 0.9, nmuscle), rng.uniform(0.1, 0.5, nmuscle),
+             rng.uniform(0, 0.4, nmuscle), np.ones(nmuscle)], axis=1).astype(np.float32),
+        muscle_rest_length=np.full(nmuscle, 0.5, np.float32),
+        muscle_waypoints_local=np.asarray(wp_local, np.float32),
+        muscle_waypoint_body=wp_body,
+        all_segment_muscle_idx=wp_muscle[start],
+        all_segment_start_idx=start,
+        apply_segment_muscle_idx=wp_muscle[crossing],
+        apply_segment_start_idx=crossing,
+        apply_segment_end_idx=crossing + 1,
+        apply_segment_body_start_idx=wp_body[crossing],
+        apply_segment_body_end_idx=wp_body[crossing + 1],
+        body_parentid=model.body_parentid,
+        body_rootid=np.asarray([0] + [1] * (nbody - 1)),
+        dof_bodyid=dof_bodyid,
+    )  # fmt: skip
+    return MuscleRig(topo, nbody, nv, nv - 6, nmuscle)
+
+
+def make_muscle_context(rig: MuscleRig, nworld: int, seed: int = 1003) -> np.ndarray:
+    """raw_context (nworld, 13 nbody + 6 nv) = xpos | xquat | xipos | subtree_com | cdof with
+    body positions ~N(0, 0.3) m, quaternions ~N(0, 1) (unnormalised on purpose), subtree
+    centres ~N(0, 0.2), cdof ~N(0, 1)."""
+    nb, nv = rig.body_count, rig.full_torque_dim
+    out = np.empty((nworld, 13 * nb + 6 * nv), np.float32)
+    for b0 in range(0, nworld, BLOCK):
+        r = np.random.default_rng([seed, 92, b0 // BLOCK])
+        n = min(BLOCK, nworld - b0)
+        parts = [r.normal(0, 0.3, (BLOCK, 3 * nb)), r.normal(0, 1, (BLOCK, 4 * nb)), r.normal(0, 0.3, (BLOCK, 3 * nb)),
+                 r.normal(0, 0.2, (BLOCK, 3 * nb)), r.normal(0, 1, (BLOCK, 6 * nv))]  # fmt: skip
+        out[b0 : b0 + n] = np.concatenate(parts, axis=1)[:n]
+    return out

@@ -590,3 +590,209 @@ int orc_jtdj_dense(int nworld, int nv, int nv_pad, const float *Mdense, const fl
   }
   return 0;
 }
+
+/* ---- Muscle path geometry and activation <-> torque contractions ---------------------
+ * Scalar restatement, one operation per statement in the order the formulas are written in
+ * the reference; built with -ffp-contract=off so nothing is fused.  expf/cosf come from
+ * libm, so the force magnitudes agree with a GPU evaluation only to a few ulp. */
+typedef struct {
+  float x, y, z;
+} v3;
+static v3 v_ld(const float *p) { v3 r = {p[0], p[1], p[2]}; return r; }
+static v3 v_sub(v3 a, v3 b) { v3 r = {a.x - b.x, a.y - b.y, a.z - b.z}; return r; }
+static v3 v_add(v3 a, v3 b) { v3 r = {a.x + b.x, a.y + b.y, a.z + b.z}; return r; }
+static v3 v_scale(float s, v3 a) { v3 r = {s * a.x, s * a.y, s * a.z}; return r; }
+static float v_dot(v3 a, v3 b) { return a.x * b.x + a.y * b.y + a.z * b.z; }
+static v3 v_cross(v3 a, v3 b) {
+  v3 r = {a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x};
+  return r;
+}
+static float v_len(v3 a) { return sqrtf(v_dot(a, a)); }
+
+/* segment_generalized_force_contribution_wp
+ * (src/instantmimic/muscle/muscle_qfrc_projector.py:280-304). */
+static float seg_contribution(v3 lin, v3 ang, v3 p0, v3 p1, v3 c0, v3 c1, float a, float b,
+                              float force) {
+  v3 seg = v_sub(p1, p0);
+  float len = v_len(seg);
+  if (len < 1.0e-8f) return 0.0f;
+  v3 dir = {seg.x / len, seg.y / len, seg.z / len};
+  v3 f = v_scale(force, dir);
+  v3 st = v_add(lin, v_cross(ang, v_sub(p0, c0)));
+  v3 en = v_add(lin, v_cross(ang, v_sub(p1, c1)));
+  return v_dot(v_sub(v_scale(a, st), v_scale(b, en)), f);
+}
+
+/* _transform_waypoints_from_torch_kernel (src/instantmimic/muscle/muscle_dynamics_kernels.py:
+ * 73-86), normalize_quat_wp (muscle_qfrc_projector.py:91-100) and mujoco_warp's
+ * math.rot_vec_quat (third party, absent from the tree; published form
+ * 2 (u.v) u + (s^2 - u.u) v + 2 s (u x v) for q = (s, u)). */
+int orc_muscle_waypoints(int nworld, int nbody, int nwp, const float *xpos, const float *xquat,
+                         const int *wp_body, const float *wp_local, float *out) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w)
+    for (int i = 0; i < nwp; ++i) {
+      const int b = wp_body[i];
+      const float *q = xquat + ((size_t)w * nbody + b) * 4;
+      float inv = 1.0f / sqrtf(q[0] * q[0] + q[1] * q[1] + q[2] * q[2] + q[3] * q[3] + 1.0e-8f);
+      float s = q[0] * inv;
+      v3 u = {q[1] * inv, q[2] * inv, q[3] * inv};
+      v3 v = v_ld(wp_local + 3 * i);
+      v3 r = v_add(v_scale(2.0f, v_scale(v_dot(u, v), u)), v_scale(s * s - v_dot(u, u), v));
+      r = v_add(r, v_scale(2.0f * s, v_cross(u, v)));
+      v3 p = v_add(v_ld(xpos + ((size_t)w * nbody + b) * 3), r);
+      float *o = out + ((size_t)w * nwp + i) * 3;
+      o[0] = p.x;
+      o[1] = p.y;
+      o[2] = p.z;
+    }
+  return 0;
+}
+
+/* muscle_qfrc_projector.py:103-145 */
+static float active_fl(float l, const float *m) {
+  if (m[0] < 0.5f) return expf(-((l - 1.0f) * (l - 1.0f)) / m[1]);
+  float lmin = m[1], lmax = m[2];
+  if (l < lmin || l > lmax) return 0.0f;
+  float lo = 0.5f * (lmin + 1.0f), hi = 0.5f * (1.0f + lmax), x;
+  if (l <= lo) {
+    x = (l - lmin) / fmaxf(lo - lmin, 1.0e-8f);
+    return 0.5f * x * x;
+  }
+  if (l <= 1.0f) {
+    x = (1.0f - l) / fmaxf(1.0f - lo, 1.0e-8f);
+    return 1.0f - 0.5f * x * x;
+  }
+  if (l <= hi) {
+    x = (l - 1.0f) / fmaxf(hi - 1.0f, 1.0e-8f);
+    return 1.0f - 0.5f * x * x;
+  }
+  x = (lmax - l) / fmaxf(lmax - hi, 1.0e-8f);
+  return 0.5f * x * x;
+}
+/* muscle_qfrc_projector.py:148-187 */
+static float passive_fl(float l, const float *m) {
+  if (m[0] < 0.5f) {
+    if (l < 1.0f) return 0.0f;
+    float x = m[1] * (l - 1.0f) / m[2];
+    x = fminf(fmaxf(x, -80.0f), 80.0f);
+    return (expf(x) - 1.0f) / (expf(m[1]) - 1.0f);
+  }
+  float lmax = m[1], fpmax = m[2];
+  if (l <= 1.0f) return 0.0f;
+  float mid = 0.5f * (1.0f + lmax), width = fmaxf(mid - 1.0f, 1.0e-8f);
+  if (l <= mid) {
+    float st = (l - 1.0f) / width;
+    return 0.5f * fpmax * st * st;
+  }
+  return fpmax * (0.5f + (l - mid) / width);
+}
+
+/* _compute_force_magnitudes_from_waypoints_kernel (muscle_dynamics_kernels.py:644-705);
+ * model = force_scale, lnorm_min, lnorm_max, active[3], passive[3]. */
+int orc_muscle_force_magnitudes(int nworld, int nwp, int nmuscle, const float *wp,
+                                const int *seg_start, const int *seg_offsets,
+                                const float *params, int ldpar, const float *rest,
+                                const float *model, int include_passive, float *unit,
+                                float *passive) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    const float *row = wp + (size_t)w * nwp * 3;
+    for (int m = 0; m < nmuscle; ++m) {
+      float len = 0.0f;
+      for (int s = seg_offsets[m]; s < seg_offsets[m + 1]; ++s) {
+        int i = seg_start[s];
+        len = len + v_len(v_sub(v_ld(row + 3 * (i + 1)), v_ld(row + 3 * i)));
+      }
+      const float *p = params + (size_t)m * ldpar;
+      float lm = len / fmaxf(rest[m], 1.0e-6f) - p[2];
+      float ln = fminf(fmaxf(lm / fmaxf(p[1], 1.0e-6f), model[1]), model[2]);
+      float c = cosf(p[3]);
+      unit[(size_t)w * nmuscle + m] = p[0] * active_fl(ln, model + 3) * c * model[0];
+      if (passive)
+        passive[(size_t)w * nmuscle + m] =
+            include_passive ? p[0] * passive_fl(ln, model + 6) * c * model[0] : 0.0f;
+    }
+  }
+  return 0;
+}
+
+/* rows of an entry list: offsets[nrow + 1], segment, other, start/end coefficient */
+#define ORC_GEO(w)                                                                        \
+  const float *wpw = wp + (size_t)(w) * nwp * 3, *comw = com + (size_t)(w) * nbody * 3, \
+              *cdw = cdof + (size_t)(w) * nv * 6
+#define ORC_TERM(segi, lin, ang, a, b, f)                                                  \
+  seg_contribution(lin, ang, v_ld(wpw + 3 * seg_p0[segi]), v_ld(wpw + 3 * seg_p1[segi]),  \
+                   v_ld(comw + 3 * seg_b0[segi]), v_ld(comw + 3 * seg_b1[segi]), a, b, f)
+
+/* _compute_muscle_dynamics_from_activation_sparse_kernel (muscle_dynamics_kernels.py:1707-1793) */
+int orc_muscle_torque_forward(int nworld, int nwp, int nbody, int nv, int nmuscle, int ntorque,
+                              const float *wp, const float *com, const float *cdof,
+                              const int *seg_p0, const int *seg_p1, const int *seg_b0,
+                              const int *seg_b1, const int *offsets, const int *e_seg,
+                              const int *e_muscle, const float *e_a, const float *e_b,
+                              const float *unit, const float *passive, const float *act, int root,
+                              float *out) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    ORC_GEO(w);
+    for (int j = 0; j < ntorque; ++j) {
+      v3 ang = v_ld(cdw + 6 * (j + root)), lin = v_ld(cdw + 6 * (j + root) + 3);
+      float total = 0.0f;
+      for (int e = offsets[j]; e < offsets[j + 1]; ++e) {
+        int m = e_muscle[e];
+        float f = unit[(size_t)w * nmuscle + m] * act[(size_t)w * nmuscle + m];
+        if (passive) f = f + passive[(size_t)w * nmuscle + m];
+        if (f == 0.0f) continue;
+        total = total + ORC_TERM(e_seg[e], lin, ang, e_a[e], e_b[e], f);
+      }
+      out[(size_t)w * ntorque + j] = total;
+    }
+  }
+  return 0;
+}
+
+/* _compute_muscle_dynamics_activation_grad_sparse_kernel (muscle_dynamics_kernels.py:1796-1859) */
+int orc_muscle_activation_grad(int nworld, int nwp, int nbody, int nv, int nmuscle, int ntorque,
+                               const float *wp, const float *com, const float *cdof,
+                               const int *seg_p0, const int *seg_p1, const int *seg_b0,
+                               const int *seg_b1, const int *offsets, const int *e_seg,
+                               const int *e_torque, const float *e_a, const float *e_b,
+                               const float *unit, const float *gout, int root, float *gact) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    ORC_GEO(w);
+    for (int m = 0; m < nmuscle; ++m) {
+      float f = unit[(size_t)w * nmuscle + m], grad = 0.0f;
+      if (f != 0.0f)
+        for (int e = offsets[m]; e < offsets[m + 1]; ++e) {
+          int j = e_torque[e];
+          v3 ang = v_ld(cdw + 6 * (j + root)), lin = v_ld(cdw + 6 * (j + root) + 3);
+          grad = grad + gout[(size_t)w * ntorque + j] * ORC_TERM(e_seg[e], lin, ang, e_a[e], e_b[e], f);
+        }
+      gact[(size_t)w * nmuscle + m] = grad;
+    }
+  }
+  return 0;
+}
+
+/* eval_muscle_sparse_moment_kernel (muscle_qfrc_projector.py:2617-2662) */
+int orc_muscle_sparse_moment(int nworld, int nwp, int nbody, int nv, int nentry, const float *wp,
+                             const float *com, const float *cdof, const int *seg_p0,
+                             const int *seg_p1, const int *seg_b0, const int *seg_b1,
+                             const int *entry_torque, const int *offsets, const int *e_seg,
+                             const float *e_a, const float *e_b, int root, float *moment) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    ORC_GEO(w);
+    for (int e = 0; e < nentry; ++e) {
+      int j = entry_torque[e] + root;
+      v3 ang = v_ld(cdw + 6 * j), lin = v_ld(cdw + 6 * j + 3);
+      float total = 0.0f;
+      for (int k = offsets[e]; k < offsets[e + 1]; ++k)
+        total = total + ORC_TERM(e_seg[k], lin, ang, e_a[k], e_b[k], 1.0f);
+      moment[(size_t)w * nentry + e] = total;
+    }
+  }
+  return 0;
+}

@@ -287,3 +287,91 @@ def jtdj_dense(Mdense, J, D, state, nefc, nv_pad, quad=1):
     ne = _i(nefc) if nefc is not None else None
     lib().orc_jtdj_dense(nworld, nv, nv_pad, _p(Mdense), _p(J), njmax, _p(D), _p(state), _p(ne), quad, _p(H))
     return H
+
+
+# ---------------------------------------------------------------- muscle geometry, torque ops
+# Pinning (tests/test_muscle_dynamics.py): `muscle_waypoints` against fp64 rotation matrices
+# built from the quaternions; `muscle_force_magnitudes` against an fp64 evaluation of the
+# four curves and the closed form of the reference's two-body fixture
+# (tests/muscle_warp_fixtures.py:17-180: one segment (0,1,0)->(2,1,0), gaussian gamma 0.45,
+# normalised length clamped to 1.4, unit force exp(-0.16/0.45)); `muscle_torque_forward`
+# against the same fixture's closed form (torque[1] = sum_m unit_m act_m, torque[0] = 0) and
+# a dense fp64 evaluation from the unsparsified subtree masks; `muscle_activation_grad`
+# against central finite differences of the forward in fp64 and the transpose identity
+# <g, T a> = <T' g, a>; `muscle_sparse_moment` against d torque / d force in fp64.
+# Bit-level agreement with the reference's Warp build is unpinned: Warp's lowering of the
+# vec3 expressions (operation association, contraction under NVRTC) is not visible from its
+# Python source and `rot_vec_quat` lives in mujoco_warp, which is not in the tree.
+
+
+def muscle_waypoints(xpos, xquat, wp_body, wp_local):
+    xpos, xquat, wp_local = _f(xpos), _f(xquat), _f(wp_local)
+    nworld, nbody = xpos.shape[0], xpos.shape[1]
+    out = np.zeros((nworld, len(wp_body), 3), np.float32)
+    lib().orc_muscle_waypoints(nworld, nbody, len(wp_body), _p(xpos), _p(xquat), _p(_i(wp_body)), _p(wp_local), _p(out))
+    return out
+
+
+def muscle_force_magnitudes(waypoints, seg_start, seg_offsets, params, rest, model, include_passive=True):
+    """model = (force_scale, lnorm_min, lnorm_max, active[3], passive[3]) flattened to 9 floats."""
+    waypoints, params = _f(waypoints), _f(params)
+    nworld, nwp = waypoints.shape[0], waypoints.shape[1]
+    nmuscle = len(seg_offsets) - 1
+    unit = np.zeros((nworld, nmuscle), np.float32)
+    passive = np.zeros((nworld, nmuscle), np.float32)
+    lib().orc_muscle_force_magnitudes(
+        nworld, nwp, nmuscle, _p(waypoints), _p(_i(seg_start)), _p(_i(seg_offsets)), _p(params), params.shape[1],
+        _p(_f(rest)), _p(_f(model)), int(bool(include_passive)), _p(unit), _p(passive),
+    )  # fmt: skip
+    return unit, passive
+
+
+def _geo(waypoints, com, cdof):
+    waypoints, com, cdof = _f(waypoints), _f(com), _f(cdof)
+    return waypoints, com, cdof, (waypoints.shape[0], waypoints.shape[1], com.shape[1], cdof.shape[1])
+
+
+def muscle_torque_forward(waypoints, com, cdof, seg, entries, unit, passive, act, root):
+    """seg = (p0, p1, b0, b1); entries = (offsets, segment, muscle, start_coeff, end_coeff)."""
+    waypoints, com, cdof, (nworld, nwp, nbody, nv) = _geo(waypoints, com, cdof)
+    unit, act = _f(unit), _f(act)
+    passive = None if passive is None else _f(passive)
+    off, es, em, ea, eb = entries
+    ntorque = len(off) - 1
+    out = np.zeros((nworld, ntorque), np.float32)
+    s = [_i(a) for a in seg]
+    keep = [_i(off), _i(es), _i(em), _f(ea), _f(eb)]
+    lib().orc_muscle_torque_forward(
+        nworld, nwp, nbody, nv, unit.shape[1], ntorque, _p(waypoints), _p(com), _p(cdof), *[_p(a) for a in s],
+        *[_p(a) for a in keep], _p(unit), _p(passive), _p(act), int(root), _p(out),
+    )  # fmt: skip
+    return out
+
+
+def muscle_activation_grad(waypoints, com, cdof, seg, entries, unit, gout, root):
+    """entries = (offsets, segment, torque, start_coeff, end_coeff) per muscle."""
+    waypoints, com, cdof, (nworld, nwp, nbody, nv) = _geo(waypoints, com, cdof)
+    unit, gout = _f(unit), _f(gout)
+    off, es, et, ea, eb = entries
+    nmuscle = len(off) - 1
+    out = np.zeros((nworld, nmuscle), np.float32)
+    s = [_i(a) for a in seg]
+    keep = [_i(off), _i(es), _i(et), _f(ea), _f(eb)]
+    lib().orc_muscle_activation_grad(
+        nworld, nwp, nbody, nv, nmuscle, gout.shape[1], _p(waypoints), _p(com), _p(cdof), *[_p(a) for a in s],
+        *[_p(a) for a in keep], _p(unit), _p(gout), int(root), _p(out),
+    )  # fmt: skip
+    return out
+
+
+def muscle_sparse_moment(waypoints, com, cdof, seg, entry_torque, offsets, segment, start_coeff, end_coeff, root):
+    waypoints, com, cdof, (nworld, nwp, nbody, nv) = _geo(waypoints, com, cdof)
+    nentry = len(entry_torque)
+    out = np.zeros((nworld, nentry), np.float32)
+    s = [_i(a) for a in seg]
+    keep = [_i(entry_torque), _i(offsets), _i(segment), _f(start_coeff), _f(end_coeff)]
+    lib().orc_muscle_sparse_moment(
+        nworld, nwp, nbody, nv, nentry, _p(waypoints), _p(com), _p(cdof), *[_p(a) for a in s],
+        *[_p(a) for a in keep], int(root), _p(out),
+    )  # fmt: skip
+    return out
