@@ -110,7 +110,8 @@ typedef struct im_sparse_plan im_sparse_plan;
 /* Device side of a SparseHessianPlan (src/instantmimic/utils/mjw_kernels/
  * sparse_hessian.py:38-50, tables :360-401).  tables[16] in this order, int32 each:
  * SH_LP, SH_LT, SH_ES, SH_EC, SH_RP, SH_RAB, SH_RKL, SH_ORIG, SH_BL, SH_BS, SH_BI, SH_BJ,
- * SH_PM, SH_SA, SH_SB, SH_SM; block is the plan's block width (32 or 64). */
+ * SH_PM, SH_SA, SH_SB, SH_SM; or tables[22] with the update stage's SH_PAIR, SH_FL, SH_FR,
+ * SH_RS, SH_RKP, SH_RK (:374-380) appended.  block is the plan's block width (32 or 64). */
 int im_sparse_plan_create(int nv, int nv_pad, int block, int nslots, int nlevels,
                           int ntables, const int32_t *const *tables, const int *sizes,
                           im_sparse_plan **out);
@@ -128,6 +129,42 @@ int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done,
                           const int32_t *state, int quad, const float *M, int ldM,
                           const float *grad, int ldg, float *hfactor, float *search,
                           float *search_dot, float *decrement, int nworld, void *stream);
+
+/* Replaces the factor stage of the fused Newton loop on the static pattern
+ * (newton_stages.factor_factory with a sparse plan, src/instantmimic/utils/mjw_kernels/
+ * newton_stages.py:614-742, and the native modes 0 / 1 / 2 of sparse_hessian.py:488-547).
+ * Per world, skipped when done[w] or state_changes[w] == 0:
+ *   changes[w] > 0: dof_union[w, :n] = ascending dofs the changed rows ids[w, :changes[w]]
+ *     touch, n in dof_union[w, nv]; packed H in hfactor gets, per pair of those dofs,
+ *     delta = sum over the changed rows of +-D a b (minus when the row's new state is not
+ *     quad; newton_stages.py:451-470), pairs outside the pattern count as violations; the
+ *     factor is rebuilt and stored back into hfactor;
+ *   changes[w] == 0: forward solve with the factor stored in hfactor.
+ * Then the backward solve, search = -x, search_dot, decrement.  The reference keeps the
+ * factor in a resident block's shared memory between iterations; here hfactor carries it
+ * from launch to launch.  ids (nworld, ld_ids), dof_union (nworld, nv + 1).  Needs a plan
+ * created with 22 tables. */
+int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done,
+                            const int32_t *state_changes, const int32_t *changes,
+                            const int32_t *ids, int ld_ids, const float *J, int njmax,
+                            const float *D, const int32_t *state, int quad, const float *grad,
+                            int ldg, float *hfactor, int32_t *dof_union, float *search,
+                            float *search_dot, float *decrement, int nworld, void *stream);
+
+/* The same stage on the dense Hessian (newton_stages.py:614-742 without a sparse plan):
+ * H (nworld, nv_pad, nv_pad) receives the deltas on its upper triangle
+ * (H[w, row, col] += delta, row <= col, :700-701); with changed rows the augmented blocked
+ * Cholesky of augmented_factor_solve_factory (:473-611) runs with 16 x 16 tiles: the
+ * gradient rides as column nv_pad - 1, the corner is 1e30, U (nworld, nv_pad, nv_pad)
+ * receives the factor including that column; without changed rows the stored U is solved
+ * against.  Rows and columns >= nv of H count as the identity.  nv_pad = a multiple of 16
+ * above nv (src/instantmimic/utils/mjw_model.py:30). */
+int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes,
+                           const int32_t *changes, const int32_t *ids, int ld_ids,
+                           const float *J, int njmax, const float *D, const int32_t *state,
+                           int quad, const float *grad, int64_t ldg, float *H, float *U, int nv,
+                           int nv_pad, int32_t *dof_union, float *search, int64_t ld_search,
+                           float *search_dot, float *decrement, int nworld, void *stream);
 
 /* Blocked dense factor + solve, dense J'DJ ----------------------------------- */
 

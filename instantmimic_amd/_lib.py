@@ -90,6 +90,14 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp],
     ),
+    "im_sparse_update_factor": (
+        _i,
+        [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp],
+    ),
+    "im_dense_update_factor": (
+        _i,
+        [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],
+    ),
     "im_blocked_factor_solve": (_i, [_vp, _i64, _i, _vp, _i, _i, _i, _vp, _i64, _vp, _vp, _i64, _i, _vp]),
     "im_jtdj_mfma": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
     "im_muscle_project": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i64, _i, _vp]),

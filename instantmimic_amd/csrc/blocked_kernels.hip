@@ -19,34 +19,49 @@ namespace {
 
 __device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 
+// Where a tile element comes from.  Indexed: element ids into the world's CSR values, ids
+// >= nM read as zero, padded diagonal entries get +1 (mjw_step_optimized.py:932-941).
 template <int B>
-__global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
-    const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
-    const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
-    int64_t ldx, int nv, int pad) {
-  extern __shared__ float lds[];
-  float *U = lds;             // [pad * pad]
-  float *rhs = U + pad * pad; // [pad]
-  float *A = rhs + pad;       // [(nblk) * B * B] working tiles of the current block row
-  float *L = A + (pad / B) * B * B;  // [B * B] Cholesky factor of the diagonal block (lower)
-  const int tid = threadIdx.x, nt = blockDim.x;
-  const int64_t w = blockIdx.x;
+struct IndexedSrc {
+  const float *Mw;
+  const int32_t *block_idx;
+  int nM, nv, nblk;
+  __device__ __forceinline__ float load(int kb, int ib, int e, int r, int c) const {
+    const int idx = block_idx[(size_t)(kb * nblk + ib) * (B * B) + e];
+    float v = idx < nM ? Mw[idx] : 0.0f;
+    if (ib == kb && (kb + 1) * B > nv && r == c && (nblk - 1) * B + r >= nv) v = v + 1.0f;
+    return v;
+  }
+};
+// Dense: the upper triangle of a row-major (pad, pad) matrix (the lower one is never read);
+// rows and columns >= nv are the identity whatever the buffer holds there.
+template <int B>
+struct DenseSrc {
+  const float *H;
+  int nv, pad;
+  __device__ __forceinline__ float load(int kb, int ib, int, int r, int c) const {
+    const int row = kb * B + r, col = ib * B + c;
+    // only the upper triangle is kept up to date: mirror it inside a diagonal tile
+    if (row < nv && col < nv) return row <= col ? H[(size_t)row * pad + col] : H[(size_t)col * pad + row];
+    return row == col ? 1.0f : 0.0f;
+  }
+};
+
+// Left-looking upper Cholesky by block column with the forward solve of rhs fused into the
+// loop; U (pad, pad) and rhs (pad) in LDS, U zeroed by the caller.
+template <int B, class Src>
+__device__ __forceinline__ void factor_forward(const Src &src, float *U, float *rhs, float *A, float *L, int pad,
+                                               int tid, int nt) {
   const int nblk = pad / B;
   constexpr int BB = B * B;
-  const float *Mw = M + w * ldM;
-  for (int i = tid; i < pad * pad; i += nt) U[i] = 0.0f;
-  for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? y[w * ldy + i] : 0.0f;
-  __syncthreads();
   for (int kb = 0; kb < nblk; ++kb) {
-    const int k = kb * B, end = k + B;
+    const int k = kb * B;
     // gather the whole block row kb..nblk-1 and subtract the finished block rows above
     const int ntile = nblk - kb;
     for (int q = tid; q < ntile * BB; q += nt) {
       const int tb = q / BB, e = q - tb * BB, r = e / B, c = e - r * B;
       const int ib = kb + tb, i0 = ib * B;
-      const int idx = block_idx[(size_t)(kb * nblk + ib) * BB + e];
-      float v = idx < nM ? Mw[idx] : 0.0f;
-      if (tb == 0 && end > nv && r == c && (nblk - 1) * B + r >= nv) v = v + 1.0f;
+      float v = src.load(kb, ib, e, r, c);
       for (int jb = 0; jb < kb; ++jb) {
         const int j = jb * B;
         float sum = 0.0f;
@@ -123,7 +138,11 @@ __global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
     }
     __syncthreads();
   }
-  // backward solve
+}
+
+// rhs <- U^-1 rhs, block rows from the bottom.
+template <int B>
+__device__ __forceinline__ void backward_solve(const float *U, float *rhs, int pad, int tid) {
   for (int i0 = pad - B; i0 >= 0; i0 -= B) {
     if (tid < 64) {
       const int r = tid;
@@ -147,9 +166,172 @@ __global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
     }
     __syncthreads();
   }
+}
+
+// rhs <- U'^-1 rhs with a finished factor (the forward half of a solve-only step): the
+// same operations on rhs as inside factor_forward.
+template <int B>
+__device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pad, int tid) {
+  for (int k = 0; k < pad; k += B) {
+    if (tid < B) {
+      float s = rhs[k + tid];
+      for (int j = 0; j < k; j += B) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < B; ++t) sum = fma_(U[(j + t) * pad + k + tid], rhs[j + t], sum);
+        s = s - sum;
+      }
+      rhs[k + tid] = s;
+    }
+    __syncthreads();
+    if (tid < 64) {
+      const int i = tid;
+      float s = i < B ? rhs[k + i] : 0.0f;
+      for (int j = 0; j < B; ++j) {
+        if (i == j) rhs[k + j] = s / U[(k + j) * pad + k + j];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        if (i > j && i < B) s = fma_(-U[(k + j) * pad + k + i], rhs[k + j], s);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <int B>
+__global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
+    const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
+    const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
+    int64_t ldx, int nv, int pad) {
+  extern __shared__ float lds[];
+  float *U = lds;             // [pad * pad]
+  float *rhs = U + pad * pad; // [pad]
+  float *A = rhs + pad;       // [(nblk) * B * B] working tiles of the current block row
+  float *L = A + (pad / B) * B * B;  // [B * B] Cholesky factor of the diagonal block (lower)
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int64_t w = blockIdx.x;
+  for (int i = tid; i < pad * pad; i += nt) U[i] = 0.0f;
+  for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? y[w * ldy + i] : 0.0f;
+  __syncthreads();
+  const IndexedSrc<B> src{M + w * ldM, block_idx, nM, nv, pad / B};
+  factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
+  backward_solve<B>(U, rhs, pad, tid);
   for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
   if (Uout)
     for (int i = tid; i < pad * pad; i += nt) Uout[w * (int64_t)pad * pad + i] = U[i];
+}
+
+// Per-iteration factor stage on the dense Hessian: dofs touched by the changed rows,
+// incremental update of H's upper triangle, then either the augmented blocked Cholesky
+// (the gradient rides as column pad - 1, corner 1e30) or, with no changed row, a solve with
+// the stored factor.  Reference: src/instantmimic/utils/mjw_kernels/newton_stages.py
+// :614-742 (stage), :451-470 (hessian_step), :473-611 (augmented factor).  search = -x,
+// search_dot = x.x, decrement = grad.x (strided over 64 lanes, shuffle-down tree).
+template <int B>
+__global__ __launch_bounds__(256) void dense_update_factor_kernel(
+    const uint8_t *__restrict__ done, const int32_t *__restrict__ state_changes,
+    const int32_t *__restrict__ changes, const int32_t *__restrict__ ids, int ld_ids,
+    const float *__restrict__ J, int njmax, const float *__restrict__ D, const int32_t *__restrict__ state,
+    int quad, const float *__restrict__ grad, int64_t ldg, float *H_, float *U_,
+    int32_t *__restrict__ uni_, float *__restrict__ search, int64_t lds_, float *__restrict__ search_dot,
+    float *__restrict__ decrement, int nv, int pad) {
+  extern __shared__ float lds[];
+  float *U = lds;             // [pad * pad]
+  float *rhs = U + pad * pad; // [pad]
+  float *A = rhs + pad;       // [(pad / B) * B * B]
+  float *L = A + (pad / B) * B * B;  // [B * B]
+  int *ul = (int *)(L + B * B);      // [nv] union list, [nv] = its length
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int64_t w = blockIdx.x;
+  if ((done && done[w]) || state_changes[w] == 0) return;
+  float *Hw = H_ + w * (int64_t)pad * pad, *Uw = U_ + w * (int64_t)pad * pad;
+  const float *Jw = J + w * (int64_t)njmax * nv, *Dw = D + w * njmax, *gw = grad + w * ldg;
+  const int32_t *sw = state + w * njmax, *idw = ids + w * ld_ids;
+  int count = changes[w];
+  count = count < ld_ids ? count : ld_ids;
+  for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? gw[i] : 0.0f;
+  if (count > 0) {
+    if (tid < 64) {
+      int nu = 0;
+      for (int base = 0; base < nv; base += 64) {
+        const int dof = base + tid;
+        bool hit = false;
+        if (dof < nv)
+          for (int t = 0; t < count && !hit; ++t) hit = Jw[(size_t)idw[t] * nv + dof] != 0.0f;
+        const unsigned long long mask = __ballot(hit);
+        if (hit) ul[nu + __popcll(mask & ((1ull << tid) - 1ull))] = dof;
+        nu += __popcll(mask);
+      }
+      if (tid == 0) ul[nv] = nu;
+    }
+    for (int i = tid; i < pad * pad; i += nt) U[i] = 0.0f;
+    __syncthreads();
+    const int nu = ul[nv];
+    int32_t *uni = uni_ + w * (nv + 1);
+    for (int i = tid; i < nu; i += nt) uni[i] = ul[i];
+    if (tid == 0) uni[nv] = nu;
+    const int npair = nu * (nu + 1) / 2;
+    for (int e = tid; e < npair; e += nt) {
+      int cj = (int)((sqrtf((float)(8 * e + 1)) - 1.0f) * 0.5f);
+      while ((cj + 1) * (cj + 2) / 2 <= e) ++cj;
+      while (cj * (cj + 1) / 2 > e) --cj;
+      const int row = ul[e - cj * (cj + 1) / 2], col = ul[cj];
+      float delta = 0.0f;
+      for (int t = 0; t < count; ++t) {
+        const int r = idw[t];
+        const float a = Jw[(size_t)r * nv + row], b = Jw[(size_t)r * nv + col];
+        float da = Dw[r] * a;
+        if (sw[r] != quad) da = -da;
+        if (a != 0.0f && b != 0.0f) delta = fma_(da, b, delta);
+      }
+      if (delta != 0.0f) Hw[(size_t)row * pad + col] = Hw[(size_t)row * pad + col] + delta;
+    }
+    __syncthreads();  // this workgroup's own writes to H are read back below
+    const DenseSrc<B> src{Hw, nv, pad};
+    factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
+    // stored factor: the augmented column z = U'^-1 grad above the corner sqrt(1e30 - z.z)
+    if (tid == 0) {
+      float v = 1.0e30f;
+      for (int i = 0; i < nv; ++i) v = fma_(-rhs[i], rhs[i], v);
+      L[0] = sqrtf(v);
+    }
+    __syncthreads();
+    for (int i = tid; i < pad * pad; i += nt) {
+      const int r = i / pad, c = i - r * pad;
+      float v = U[i];
+      if (c == pad - 1) v = r < nv ? rhs[r] : (r == pad - 1 ? L[0] : v);
+      Uw[i] = v;
+    }
+    __syncthreads();  // rhs is overwritten by the backward solve
+  } else {
+    for (int i = tid; i < pad * pad; i += nt) {
+      const int r = i / pad, c = i - r * pad;
+      float v = Uw[i];
+      if (c == pad - 1) v = r == pad - 1 ? 1.0f : 0.0f;  // drop the augmented column
+      U[i] = v;
+    }
+    __syncthreads();
+    forward_solve<B>(U, rhs, pad, tid);
+  }
+  backward_solve<B>(U, rhs, pad, tid);
+  if (tid < 64) {
+    float s0 = 0.0f, s1 = 0.0f;
+    for (int i = tid; i < nv; i += 64) {
+      const float v = rhs[i];
+      search[w * lds_ + i] = -v;
+      s0 = fma_(v, v, s0);
+      s1 = fma_(gw[i], v, s1);
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+      s0 = s0 + __shfl_down(s0, o, 64);
+      s1 = s1 + __shfl_down(s1, o, 64);
+    }
+    if (tid == 0) {
+      search_dot[w] = s0;
+      decrement[w] = s1;
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------- dense J'DJ
@@ -282,6 +464,32 @@ int im_jtdj_mfma(const float *Mdense, const float *J, int njmax, const float *D,
   const size_t lds_bytes = sizeof(float) * 2 * 32 * (size_t)nvr;
   hipLaunchKernelGGL(im::jtdj_mfma_kernel, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, Mdense, J,
                      njmax, D, state, nefc, quad, H, nv, nv_pad);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, const int32_t *changes,
+                           const int32_t *ids, int ld_ids, const float *J, int njmax, const float *D,
+                           const int32_t *state, int quad, const float *grad, int64_t ldg, float *H, float *U,
+                           int nv, int nv_pad, int32_t *dof_union, float *search, int64_t ld_search,
+                           float *search_dot, float *decrement, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || nv_pad <= nv || ld_ids < 0 || njmax < 0) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!state_changes || !changes || !ids || !J || !D || !state || !grad || !H || !U || !dof_union || !search ||
+      !search_dot || !decrement)
+    return IM_ERR_ARG;
+  if (nv_pad % 16) return IM_ERR_ARG;
+  if (ldg < nv || ld_search < nv) return IM_ERR_STRIDE;
+  constexpr int B = 16;
+  const size_t lds_bytes =
+      sizeof(float) * ((size_t)nv_pad * nv_pad + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + nv + 1);
+  if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
+  auto fn = im::dense_update_factor_kernel<B>;
+  if (lds_bytes > 64 * 1024)
+    IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
+                     ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, U, dof_union, search, ld_search,
+                     search_dot, decrement, nv, nv_pad);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

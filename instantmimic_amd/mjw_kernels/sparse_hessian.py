@@ -277,7 +277,8 @@ class _DevicePlan:
     """Owns the ``im_sparse_plan`` of a table set on the current device."""
 
     ORDER = ("SH_LP", "SH_LT", "SH_ES", "SH_EC", "SH_RP", "SH_RAB", "SH_RKL", "SH_ORIG", "SH_BL", "SH_BS", "SH_BI",
-             "SH_BJ", "SH_PM", "SH_SA", "SH_SB", "SH_SM")  # fmt: skip
+             "SH_BJ", "SH_PM", "SH_SA", "SH_SB", "SH_SM", "SH_PAIR", "SH_FL", "SH_FR", "SH_RS", "SH_RKP",
+             "SH_RK")  # fmt: skip
 
     def __init__(self, plan: SparseHessianPlan):
         arrays = [np.ascontiguousarray(plan.tables[k], np.int32) for k in self.ORDER]

@@ -330,10 +330,70 @@ typedef struct {
   const int *LP, *LT, *ES, *EC, *RP, *RAB, *RKL, *ORIG, *BL, *BS, *BI, *BJ, *PM, *SA, *SB, *SM;
 } sparse_t;
 
+/* level-scheduled numeric factor (sparse_hessian.py:410-452), team lanes emulated */
+static void sp_factor_levels(const sparse_t *p, float *N, float *iD) {
+  for (int l = 0; l < p->nlevels; ++l) {
+    const int T = p->LT[l];
+    for (int e = p->LP[l]; e < p->LP[l + 1]; ++e) {
+      float part[32];
+      for (int tl = 0; tl < T; ++tl) {
+        float v = 0.0f;
+        for (int r = p->RP[e]; r < p->RP[e + 1]; ++r) {
+          const unsigned ab = (unsigned)p->RAB[r], kl = (unsigned)p->RKL[r];
+          const float *pa = N + (ab & 0xFFFFu), *pb = N + (ab >> 16), *pd = iD + (kl & 0xFFFFu);
+          const int len = (int)(kl >> 16);
+          for (int t = tl; t < len; t += T) v = fmaf(pa[t] * pb[t], pd[t], v);
+        }
+        part[tl] = v;
+      }
+      for (int off = T >> 1; off > 0; off >>= 1)
+        for (int i = 0; i < off; ++i) part[i] = part[i] + part[i + off];
+      /* entries of one level never read what the level writes, so in-place is a sweep */
+      const float wv = N[p->ES[e]] - part[0];
+      N[p->ES[e]] = wv;
+      if (p->EC[e] >= 0) iD[p->EC[e]] = 1.0f / wv;
+    }
+  }
+}
+
+/* backward pushes, search = -x and the two sums (sparse_hessian.py:453-479) */
+static void sp_backward_sums(const sparse_t *p, float *N, const float *iD, const float *grad,
+                             float *search, float *sdot, float *decr) {
+  const int n = p->nv, nfac = p->nslots - n, rhs = nfac, block = p->block;
+  for (int l = 0; l < p->nlevels; ++l)
+    for (int q = p->BL[l]; q < p->BL[l + 1]; ++q) {
+      const int i = p->BI[q], j = p->BJ[q];
+      N[rhs + j] = fmaf(-N[p->BS[q]], N[rhs + i] * iD[i], N[rhs + j]);
+    }
+  /* per-lane sums, 32-lane shuffle tree, warps added in order */
+  float s0[64] = {0}, s1[64] = {0};
+  for (int lane = 0; lane < block; ++lane)
+    for (int j = lane; j < n; j += block) {
+      const int d = p->ORIG[j];
+      const float v = N[rhs + j] * iD[j];
+      search[d] = -v;
+      s0[lane] = fmaf(v, v, s0[lane]);
+      s1[lane] = fmaf(grad[d], v, s1[lane]);
+    }
+  float ra = 0.0f, rb = 0.0f;
+  for (int wv = 0; wv < (block + 31) / 32; ++wv) {
+    float *a = s0 + 32 * wv, *b = s1 + 32 * wv;
+    for (int off = 16; off > 0; off >>= 1)
+      for (int i = 0; i < off; ++i) {
+        a[i] = a[i] + a[i + off];
+        b[i] = b[i] + b[i + off];
+      }
+    ra = ra + a[0];
+    rb = rb + b[0];
+  }
+  *sdot = ra;
+  *decr = rb;
+}
+
 static void sparse_world(const sparse_t *p, const float *J, int njmax, const float *D,
                          const int *state, int nefc, int quad, const float *M, const float *grad,
                          float *U, float *search, float *sdot, float *decr, float *N) {
-  const int n = p->nv, nfac = p->nslots - n, rhs = nfac, block = p->block;
+  const int n = p->nv, nfac = p->nslots - n, rhs = nfac;
   float *iD = N + p->nslots;
   const int words = (n + 31) / 32;
   for (int s = 0; s < nfac; ++s) N[s] = p->SM[s] >= 0 ? M[p->SM[s]] : 0.0f;
@@ -368,58 +428,10 @@ static void sparse_world(const sparse_t *p, const float *J, int njmax, const flo
   }
   for (int s = 0; s < nfac; ++s) U[s] = N[s];
   for (int j = 0; j < n; ++j) N[rhs + j] = grad[p->ORIG[j]];
-  for (int l = 0; l < p->nlevels; ++l) {
-    const int T = p->LT[l];
-    for (int e = p->LP[l]; e < p->LP[l + 1]; ++e) {
-      float part[32];
-      for (int tl = 0; tl < T; ++tl) {
-        float v = 0.0f;
-        for (int r = p->RP[e]; r < p->RP[e + 1]; ++r) {
-          const unsigned ab = (unsigned)p->RAB[r], kl = (unsigned)p->RKL[r];
-          const float *pa = N + (ab & 0xFFFFu), *pb = N + (ab >> 16), *pd = iD + (kl & 0xFFFFu);
-          const int len = (int)(kl >> 16);
-          for (int t = tl; t < len; t += T) v = fmaf(pa[t] * pb[t], pd[t], v);
-        }
-        part[tl] = v;
-      }
-      for (int off = T >> 1; off > 0; off >>= 1)
-        for (int i = 0; i < off; ++i) part[i] = part[i] + part[i + off];
-      /* entries of one level never read what the level writes, so in-place is a sweep */
-      const float wv = N[p->ES[e]] - part[0];
-      N[p->ES[e]] = wv;
-      if (p->EC[e] >= 0) iD[p->EC[e]] = 1.0f / wv;
-    }
-  }
+  sp_factor_levels(p, N, iD);
   for (int s = 0; s < nfac; ++s) U[nfac + s] = N[s];
   for (int j = 0; j < n; ++j) U[2 * nfac + j] = iD[j];
-  for (int l = 0; l < p->nlevels; ++l)
-    for (int q = p->BL[l]; q < p->BL[l + 1]; ++q) {
-      const int i = p->BI[q], j = p->BJ[q];
-      N[rhs + j] = fmaf(-N[p->BS[q]], N[rhs + i] * iD[i], N[rhs + j]);
-    }
-  /* per-lane sums, 32-lane shuffle tree, warps added in order */
-  float s0[64] = {0}, s1[64] = {0};
-  for (int lane = 0; lane < block; ++lane)
-    for (int j = lane; j < n; j += block) {
-      const int d = p->ORIG[j];
-      const float v = N[rhs + j] * iD[j];
-      search[d] = -v;
-      s0[lane] = fmaf(v, v, s0[lane]);
-      s1[lane] = fmaf(grad[d], v, s1[lane]);
-    }
-  float ra = 0.0f, rb = 0.0f;
-  for (int wv = 0; wv < (block + 31) / 32; ++wv) {
-    float *a = s0 + 32 * wv, *b = s1 + 32 * wv;
-    for (int off = 16; off > 0; off >>= 1)
-      for (int i = 0; i < off; ++i) {
-        a[i] = a[i] + a[i + off];
-        b[i] = b[i] + b[i + off];
-      }
-    ra = ra + a[0];
-    rb = rb + b[0];
-  }
-  *sdot = ra;
-  *decr = rb;
+  sp_backward_sums(p, N, iD, grad, search, sdot, decr);
 }
 
 int orc_sparse_init_factor(int nv, int nv_pad, int block, int nslots, int nlevels,
@@ -447,6 +459,106 @@ int orc_sparse_init_factor(int nv, int nv_pad, int block, int nslots, int nlevel
   return 0;
 }
 
+/* Changed rows' dof union in ascending order and the incremental update of one H entry
+ * (src/instantmimic/utils/mjw_kernels/newton_stages.py:451-470, 651-701;
+ * sparse_hessian.py:505-523): delta = fold over the changed rows t, in list order, of
+ * fmaf(+-D a, b, delta), the sign negative when the row's new state is not QUADRATIC,
+ * rows that do not reach both dofs skipped. */
+static int dof_union(int n, const float *J, const int *ids, int count, int *uni) {
+  int m = 0;
+  for (int d = 0; d < n; ++d)
+    for (int t = 0; t < count; ++t)
+      if (J[(size_t)ids[t] * n + d] != 0.0f) {
+        uni[m++] = d;
+        break;
+      }
+  uni[n] = m;
+  return m;
+}
+static float pair_delta(int n, const float *J, const float *D, const int *state, int quad,
+                        const int *ids, int count, int row, int col) {
+  float delta = 0.0f;
+  for (int t = 0; t < count; ++t) {
+    const int r = ids[t];
+    const float a = J[(size_t)r * n + row], b = J[(size_t)r * n + col];
+    float da = D[r] * a;
+    if (state[r] != quad) da = -da;
+    if (a != 0.0f && b != 0.0f) delta = fmaf(da, b, delta);
+  }
+  return delta;
+}
+
+/* Per-iteration factor stage on the static pattern (sparse_hessian.py:488-547 with the
+ * factor kept in hfactor between calls instead of in a resident block's shared memory):
+ * count > 0: update packed H through SH_PAIR, refactor (mode 0); count == 0: forward solve
+ * with the stored factor (modes 2 + 1).  tables[16..21] = SH_PAIR, SH_FL, SH_FR, SH_RS,
+ * SH_RKP, SH_RK. */
+int orc_sparse_update_factor(int nv, int nv_pad, int block, int nslots, int nlevels,
+                             const int *const *tables, int nworld, const unsigned char *done,
+                             const int *state_changes, const int *changes, const int *ids,
+                             int ld_ids, const float *J, int njmax, const float *D,
+                             const int *state, int quad, const float *grad, int ldg,
+                             float *hfactor, int *uni_out, float *search, float *sdot,
+                             float *decr) {
+  sparse_t p = {nv, nv_pad, block, nslots, nlevels, tables[0], tables[1], tables[2], tables[3],
+                tables[4], tables[5], tables[6], tables[7], tables[8], tables[9], tables[10],
+                tables[11], tables[12], tables[13], tables[14], tables[15]};
+  const int *PAIR = tables[16], *FL = tables[17], *FR = tables[18], *RS = tables[19],
+            *RKP = tables[20], *RK = tables[21];
+  const int n = nv, nfac = nslots - nv, rhs = nfac;
+  if (nv > 1024 || block > 64) return 1;
+#pragma omp parallel
+  {
+    float *N = (float *)malloc(sizeof(float) * (nslots + nv + 8));
+    float *iD = N + nslots;
+#pragma omp for schedule(static)
+    for (int w = 0; w < nworld; ++w) {
+      if ((done && done[w]) || state_changes[w] == 0) continue;
+      float *U = hfactor + (size_t)w * nv_pad * nv_pad;
+      const float *Jw = J + (size_t)w * njmax * n, *Dw = D + (size_t)w * njmax;
+      const int *sw = state + (size_t)w * njmax, *idw = ids + (size_t)w * ld_ids;
+      const float *g = grad + (size_t)w * ldg;
+      int *uni = uni_out + (size_t)w * (n + 1);
+      const int count = changes[w] < ld_ids ? changes[w] : ld_ids;
+      if (count > 0) {
+        const int nu = dof_union(n, Jw, idw, count, uni);
+        for (int cj = 0; cj < nu; ++cj)
+          for (int ri = 0; ri <= cj; ++ri) {
+            const int row = uni[ri], col = uni[cj];
+            const float delta = pair_delta(n, Jw, Dw, sw, quad, idw, count, row, col);
+            if (delta != 0.0f) {
+              const int sl = PAIR[row * n + col];
+              if (sl >= 0) U[sl] = U[sl] + delta;
+              else U[nv_pad * nv_pad - 1] += 1.0f;
+            }
+          }
+        for (int s = 0; s < nfac; ++s) N[s] = U[s];
+        for (int j = 0; j < n; ++j) N[rhs + j] = g[p.ORIG[j]];
+        sp_factor_levels(&p, N, iD);
+        for (int s = 0; s < nfac; ++s) U[nfac + s] = N[s];
+        for (int j = 0; j < n; ++j) U[2 * nfac + j] = iD[j];
+      } else {
+        for (int s = 0; s < nfac; ++s) N[s] = U[nfac + s];
+        for (int j = 0; j < n; ++j) iD[j] = U[2 * nfac + j];
+        for (int l = 0; l < nlevels; ++l)
+          for (int q = FL[l]; q < FL[l + 1]; ++q) {
+            const int j = FR[q];
+            float v = g[p.ORIG[j]];
+            const float *rowp = N + RS[j];
+            for (int t = 0; t < RKP[j + 1] - RKP[j]; ++t) {
+              const int k = RK[RKP[j] + t];
+              v = fmaf(-(rowp[t] * iD[k]), N[rhs + k], v);
+            }
+            N[rhs + j] = v;
+          }
+      }
+      sp_backward_sums(&p, N, iD, g, search + (size_t)w * n, sdot + w, decr + w);
+    }
+    free(N);
+  }
+  return 0;
+}
+
 /* ------------------------------------------------------------------ blocked dense Cholesky
  * Restatement of the indexed blocked upper Cholesky factor + solve
  * (src/instantmimic/utils/mjw_kernels/indexed_factor.py:15-173; block index layout and
@@ -462,20 +574,32 @@ int orc_sparse_init_factor(int nv, int nv_pad, int block, int nslots, int nlevel
  *                                s[i] = fmaf(-L[i][j], z[j], s[i]) for i > j
  *   upper solve U x = b:         column oriented, r descending: x[r] = s[r] / U[r][r];
  *                                s[t] = fmaf(-U[t][r], x[r], s[t]) for t < r */
-static void blocked_world(int nv, int pad, int B, int nM, const float *M, const int *bidx,
-                          const float *y, float *U, float *x, float *rhs, float *A, float *L) {
+/* One tile element.  bidx != NULL: indexed gather from the CSR values with +1 on padded
+ * diagonal entries; bidx == NULL: M is a dense (pad, pad) matrix whose rows and columns
+ * >= nv count as the identity. */
+static float tile_elem(int nv, int pad, int B, int nM, const float *M, const int *bidx, int kb,
+                       int ib, int e) {
+  const int nblk = pad / B, r = e / B, c = e % B;
+  if (!bidx) {
+    const int row = kb * B + r, col = ib * B + c;
+    /* only the upper triangle is kept up to date: mirror it inside a diagonal tile */
+    if (row < nv && col < nv) return row <= col ? M[(size_t)row * pad + col] : M[(size_t)col * pad + row];
+    return row == col ? 1.0f : 0.0f;
+  }
+  const int idx = bidx[(size_t)(kb * nblk + ib) * B * B + e];
+  float v = idx < nM ? M[idx] : 0.0f;
+  if (ib == kb && (kb + 1) * B > nv && r == c && (nblk - 1) * B + r >= nv) v = v + 1.0f;
+  return v;
+}
+
+/* factor U'U = A with rhs <- U'^-1 rhs fused into the block loop */
+static void blocked_factor_forward(int nv, int pad, int B, int nM, const float *M, const int *bidx,
+                                   float *U, float *rhs, float *A, float *L) {
   const int nblk = pad / B, BB = B * B;
-  for (int i = 0; i < pad; ++i) rhs[i] = i < nv ? y[i] : 0.0f;
   for (int i = 0; i < pad * pad; ++i) U[i] = 0.0f;
   for (int kb = 0; kb < nblk; ++kb) {
-    const int k = kb * B, end = k + B;
-    const int *idx = bidx + (size_t)(kb * nblk + kb) * BB;
-    for (int e = 0; e < BB; ++e) {
-      float v = idx[e] < nM ? M[idx[e]] : 0.0f;
-      const int r = e / B, c = e % B;
-      if (end > nv && r == c && (nblk - 1) * B + r >= nv) v = v + 1.0f;
-      A[e] = v;
-    }
+    const int k = kb * B;
+    for (int e = 0; e < BB; ++e) A[e] = tile_elem(nv, pad, B, nM, M, bidx, kb, kb, e);
     for (int jb = 0; jb < kb; ++jb) {
       const int j = jb * B;
       for (int r = 0; r < B; ++r)
@@ -510,8 +634,7 @@ static void blocked_world(int nv, int pad, int B, int nM, const float *M, const 
     }
     for (int ib = kb + 1; ib < nblk; ++ib) {
       const int i0 = ib * B;
-      const int *idx2 = bidx + (size_t)(kb * nblk + ib) * BB;
-      for (int e = 0; e < BB; ++e) A[e] = idx2[e] < nM ? M[idx2[e]] : 0.0f;
+      for (int e = 0; e < BB; ++e) A[e] = tile_elem(nv, pad, B, nM, M, bidx, kb, ib, e);
       for (int jb = 0; jb < kb; ++jb) {
         const int j = jb * B;
         for (int r = 0; r < B; ++r)
@@ -531,6 +654,10 @@ static void blocked_world(int nv, int pad, int B, int nM, const float *M, const 
         for (int c = 0; c < B; ++c) U[(k + r) * pad + i0 + c] = A[r * B + c];
     }
   }
+}
+
+/* rhs <- U^-1 rhs */
+static void blocked_backward(int pad, int B, const float *U, float *rhs) {
   for (int i0 = pad - B; i0 >= 0; i0 -= B) {
     for (int j = i0 + B; j < pad; j += B)
       for (int r = 0; r < B; ++r) {
@@ -544,8 +671,33 @@ static void blocked_world(int nv, int pad, int B, int nM, const float *M, const 
       for (int t = 0; t < r; ++t) rhs[i0 + t] = fmaf(-U[(i0 + t) * pad + i0 + r], xv, rhs[i0 + t]);
     }
   }
+}
+
+/* rhs <- U'^-1 rhs with a finished factor: the operations factor_forward applies to rhs */
+static void blocked_forward(int pad, int B, const float *U, float *rhs) {
+  for (int k = 0; k < pad; k += B) {
+    for (int j = 0; j < k; j += B)
+      for (int r = 0; r < B; ++r) {
+        float sum = 0.0f;
+        for (int t = 0; t < B; ++t) sum = fmaf(U[(j + t) * pad + k + r], rhs[j + t], sum);
+        rhs[k + r] = rhs[k + r] - sum;
+      }
+    for (int j = 0; j < B; ++j) {
+      const float z = rhs[k + j] / U[(k + j) * pad + k + j];
+      rhs[k + j] = z;
+      for (int i = j + 1; i < B; ++i) rhs[k + i] = fmaf(-U[(k + j) * pad + k + i], z, rhs[k + i]);
+    }
+  }
+}
+
+static void blocked_world(int nv, int pad, int B, int nM, const float *M, const int *bidx,
+                          const float *y, float *U, float *x, float *rhs, float *A, float *L) {
+  for (int i = 0; i < pad; ++i) rhs[i] = i < nv ? y[i] : 0.0f;
+  blocked_factor_forward(nv, pad, B, nM, M, bidx, U, rhs, A, L);
+  blocked_backward(pad, B, U, rhs);
   for (int i = 0; i < nv; ++i) x[i] = rhs[i];
 }
+
 
 int orc_blocked_factor_solve(int nworld, int nv, int pad, int B, int nM, const float *M, int ldM,
                              const int *block_idx, const float *y, float *U, float *x) {
@@ -560,6 +712,74 @@ int orc_blocked_factor_solve(int nworld, int nv, int pad, int B, int nM, const f
                     work + pad + B * B);
     free(work);
     free(Ul);
+  }
+  return 0;
+}
+
+/* Per-iteration factor stage on the dense Hessian (src/instantmimic/utils/mjw_kernels/
+ * newton_stages.py:614-742): incremental update of H's upper triangle over the changed
+ * rows' dof union (:451-470, 651-701), then the augmented blocked Cholesky (:473-611; the
+ * gradient as column pad - 1, corner 1e30) or, without changed rows, a solve with the stored
+ * factor.  The tile arithmetic and the order of the two final sums are this file's
+ * conventions (the reference's come from Warp's tile library and mujoco_warp's
+ * block_cholesky, both third party): 64 lanes stride the dofs, shuffle-down tree. */
+int orc_dense_update_factor(int nworld, int nv, int pad, const unsigned char *done,
+                            const int *state_changes, const int *changes, const int *ids,
+                            int ld_ids, const float *J, int njmax, const float *D,
+                            const int *state, int quad, const float *grad, int ldg, float *H,
+                            float *Uout, int *uni_out, float *search, float *sdot, float *decr) {
+  const int B = 16;
+#pragma omp parallel
+  {
+    float *work = (float *)malloc(sizeof(float) * ((size_t)pad * pad + pad + 2 * B * B + 8));
+    float *U = work, *rhs = U + (size_t)pad * pad, *A = rhs + pad, *L = A + B * B;
+#pragma omp for schedule(static)
+    for (int w = 0; w < nworld; ++w) {
+      if ((done && done[w]) || state_changes[w] == 0) continue;
+      float *Hw = H + (size_t)w * pad * pad, *Uw = Uout + (size_t)w * pad * pad;
+      const float *Jw = J + (size_t)w * njmax * nv, *Dw = D + (size_t)w * njmax;
+      const int *sw = state + (size_t)w * njmax, *idw = ids + (size_t)w * ld_ids;
+      const float *g = grad + (size_t)w * ldg;
+      int *uni = uni_out + (size_t)w * (nv + 1);
+      const int count = changes[w] < ld_ids ? changes[w] : ld_ids;
+      for (int i = 0; i < pad; ++i) rhs[i] = i < nv ? g[i] : 0.0f;
+      if (count > 0) {
+        const int nu = dof_union(nv, Jw, idw, count, uni);
+        for (int cj = 0; cj < nu; ++cj)
+          for (int ri = 0; ri <= cj; ++ri) {
+            const int row = uni[ri], col = uni[cj];
+            const float delta = pair_delta(nv, Jw, Dw, sw, quad, idw, count, row, col);
+            if (delta != 0.0f) Hw[(size_t)row * pad + col] = Hw[(size_t)row * pad + col] + delta;
+          }
+        blocked_factor_forward(nv, pad, B, 0, Hw, 0, U, rhs, A, L);
+        float corner = 1.0e30f;
+        for (int i = 0; i < nv; ++i) corner = fmaf(-rhs[i], rhs[i], corner);
+        for (int i = 0; i < pad * pad; ++i) Uw[i] = U[i];
+        for (int i = 0; i < nv; ++i) Uw[(size_t)i * pad + pad - 1] = rhs[i];
+        Uw[(size_t)(pad - 1) * pad + pad - 1] = sqrtf(corner);
+      } else {
+        for (int i = 0; i < pad * pad; ++i) U[i] = Uw[i];
+        for (int i = 0; i < pad; ++i) U[(size_t)i * pad + pad - 1] = i == pad - 1 ? 1.0f : 0.0f;
+        blocked_forward(pad, B, U, rhs);
+      }
+      blocked_backward(pad, B, U, rhs);
+      float s0[64] = {0}, s1[64] = {0};
+      for (int lane = 0; lane < 64; ++lane)
+        for (int i = lane; i < nv; i += 64) {
+          const float v = rhs[i];
+          search[(size_t)w * nv + i] = -v;
+          s0[lane] = fmaf(v, v, s0[lane]);
+          s1[lane] = fmaf(g[i], v, s1[lane]);
+        }
+      for (int off = 32; off > 0; off >>= 1)
+        for (int i = 0; i < off; ++i) {
+          s0[i] = s0[i] + s0[i + off];
+          s1[i] = s1[i] + s1[i + off];
+        }
+      sdot[w] = s0[0];
+      decr[w] = s1[0];
+    }
+    free(work);
   }
   return 0;
 }

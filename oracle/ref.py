@@ -375,3 +375,53 @@ def muscle_sparse_moment(waypoints, com, cdof, seg, entry_torque, offsets, segme
         *[_p(a) for a in keep], int(root), _p(out),
     )  # fmt: skip
     return out
+
+
+# ---------------------------------------------------------------- per-iteration factor stage
+# Pinning (tests/test_newton_stages.py): the updated H against a fresh fp64 assembly with the
+# new states; the dof union against a NumPy any() over the changed rows; the solve against
+# fp64 `numpy.linalg.solve` within conditioning; the stored augmented factor against
+# U'U == [[H, g], [g', 1e30]] in fp64; solve-only equals refactor-with-no-change to
+# rounding.  Tile arithmetic and the order of the two sums on the dense path are this
+# oracle's own conventions (Warp tile library / mujoco_warp block_cholesky are third party):
+# bit-level parity with the reference UNPINNED there, tolerance parity pinned.
+
+UPDATE_TABLES = TABLE_ORDER + ("SH_PAIR", "SH_FL", "SH_FR", "SH_RS", "SH_RKP", "SH_RK")
+
+
+def sparse_update_factor(plan, state_changes, changes, ids, J, D, state, grad, hfactor, done=None, quad=1):
+    J, D, grad = _f(J), _f(D), _f(grad)
+    state, ids, changes, state_changes = _i(state), _i(ids), _i(changes), _i(state_changes)
+    nworld, njmax, nv = J.shape
+    tabs = [np.ascontiguousarray(plan.tables[k], np.int32) for k in UPDATE_TABLES]
+    ptrs = (ctypes.c_void_p * len(tabs))(*[t.ctypes.data for t in tabs])
+    hf = np.array(hfactor, np.float32, order="C")
+    uni = np.zeros((nworld, nv + 1), np.int32)
+    search = np.zeros((nworld, nv), np.float32)
+    sdot, decr = np.zeros(nworld, np.float32), np.zeros(nworld, np.float32)
+    dn = None if done is None else np.ascontiguousarray(done, np.uint8)
+    status = lib().orc_sparse_update_factor(
+        plan.nv, plan.nv_pad, plan.block, plan.nslots, plan.levels, ptrs, nworld, _p(dn), _p(state_changes),
+        _p(changes), _p(ids), ids.shape[1], _p(J), njmax, _p(D), _p(state), quad, _p(grad), grad.shape[1], _p(hf),
+        _p(uni), _p(search), _p(sdot), _p(decr),
+    )  # fmt: skip
+    assert status == 0
+    return hf, uni, search, sdot, decr
+
+
+def dense_update_factor(state_changes, changes, ids, J, D, state, grad, H, U, done=None, quad=1):
+    J, D, grad = _f(J), _f(D), _f(grad)
+    state, ids, changes, state_changes = _i(state), _i(ids), _i(changes), _i(state_changes)
+    nworld, njmax, nv = J.shape
+    H, U = np.array(H, np.float32, order="C"), np.array(U, np.float32, order="C")
+    pad = H.shape[1]
+    uni = np.zeros((nworld, nv + 1), np.int32)
+    search = np.zeros((nworld, nv), np.float32)
+    sdot, decr = np.zeros(nworld, np.float32), np.zeros(nworld, np.float32)
+    dn = None if done is None else np.ascontiguousarray(done, np.uint8)
+    status = lib().orc_dense_update_factor(
+        nworld, nv, pad, _p(dn), _p(state_changes), _p(changes), _p(ids), ids.shape[1], _p(J), njmax, _p(D),
+        _p(state), quad, _p(grad), grad.shape[1], _p(H), _p(U), _p(uni), _p(search), _p(sdot), _p(decr),
+    )  # fmt: skip
+    assert status == 0
+    return H, U, uni, search, sdot, decr
