@@ -308,6 +308,16 @@ int im_muscle_activation_grad(const im_muscle_geometry *geometry,
                               int root_dof_count, float *grad_activation,
                               int64_t ld_grad_activation, int nworld, void *stream);
 
+/* Replaces _compute_muscle_dynamics_sparse_bounds_kernel (muscle_dynamics_kernels.py:
+ * 1453-1528), the body of instantmimic_muscle::torque_bounds (warp_custom_ops.py:285-303):
+ * per torque dof, each muscle's unit-activation torque adds to lower when negative, else to
+ * upper.  lower / upper (nworld, ld_bounds >= torque_entries->nrow). */
+int im_muscle_torque_bounds(const im_muscle_geometry *geometry,
+                            const im_muscle_segments *segments,
+                            const im_muscle_entries *torque_entries, const float *unit_force,
+                            int64_t ld_unit, int root_dof_count, float *lower, float *upper,
+                            int64_t ld_bounds, int nworld, void *stream);
+
 /* Replaces eval_muscle_sparse_moment_kernel
  * (src/instantmimic/muscle/muscle_qfrc_projector.py:2617-2662): moment[w, e] = sum over
  * the segments of (muscle, dof) entry e of the unit-force contribution. */

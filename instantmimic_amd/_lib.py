@@ -115,6 +115,7 @@ SIGNATURES = {
         [_pgeo, _pseg, _pent, _vp, _i64, _vp, _i64, _vp, _i64, _i, _vp, _i64, _i, _vp],
     ),
     "im_muscle_activation_grad": (_i, [_pgeo, _pseg, _pent, _vp, _i64, _vp, _i64, _i, _vp, _i64, _i, _vp]),
+    "im_muscle_torque_bounds": (_i, [_pgeo, _pseg, _pent, _vp, _i64, _i, _vp, _vp, _i64, _i, _vp]),
     "im_muscle_sparse_moment": (_i, [_pgeo, _pseg, _vp, _pent, _i, _vp, _i64, _i, _vp]),
 }
 

@@ -225,6 +225,39 @@ __global__ __launch_bounds__(256) void sparse_moment_kernel(
   moment[w * ldm + e] = total;
 }
 
+// Feasible torque box over activations in [0, 1]: per torque dof the entries are grouped by
+// muscle (consecutive entries of one muscle); a muscle's total goes to the lower bound when
+// negative, else to the upper (muscle_dynamics_kernels.py:1453-1528).
+__global__ __launch_bounds__(256) void torque_bounds_kernel(
+    Geo g, Seg s, const int32_t *__restrict__ offsets, const int32_t *__restrict__ e_seg,
+    const int32_t *__restrict__ e_muscle, const float *__restrict__ e_a,
+    const float *__restrict__ e_b, const float *__restrict__ unit, int64_t ldu, int root,
+    int ntorque, float *__restrict__ lower, float *__restrict__ upper, int64_t ldo) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t w = blockIdx.y;
+  if (j >= ntorque) return;
+  const float *cd = g.cdof + w * g.ldd + 6 * (int64_t)(j + root);
+  const V3 ang = ld3(cd), lin = ld3(cd + 3);
+  int current = -1;
+  float total = 0.0f, lo = 0.0f, hi = 0.0f;
+  for (int e = offsets[j]; e < offsets[j + 1]; ++e) {
+    const int m = e_muscle[e];
+    if (current >= 0 && m != current) {
+      if (total < 0.0f) lo = lo + total;
+      else hi = hi + total;
+      total = 0.0f;
+    }
+    current = m;
+    total = total + seg_term(g, s, w, e_seg[e], lin, ang, e_a[e], e_b[e], unit[w * ldu + m]);
+  }
+  if (current >= 0) {
+    if (total < 0.0f) lo = lo + total;
+    else hi = hi + total;
+  }
+  lower[w * ldo + j] = lo;
+  upper[w * ldo + j] = hi;
+}
+
 bool geo_ok(const im_muscle_geometry *g) {
   return g && g->waypoints && g->subtree_com && g->cdof && g->ld_waypoints >= 0 &&
          g->ld_subtree_com >= 0 && g->ld_cdof >= 0;
@@ -392,6 +425,35 @@ extern "C" int im_muscle_sparse_moment(const im_muscle_geometry *geometry,
                        entry_segments->offsets, entry_segments->segment,
                        entry_segments->start_coeff, entry_segments->end_coeff, root_dof_count, ne,
                        moment + w0 * ld_moment, ld_moment);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_muscle_torque_bounds(const im_muscle_geometry *geometry,
+                                       const im_muscle_segments *segments,
+                                       const im_muscle_entries *torque_entries,
+                                       const float *unit_force, int64_t ld_unit, int root_dof_count,
+                                       float *lower, float *upper, int64_t ld_bounds, int nworld,
+                                       void *stream) {
+  if (nworld < 0 || !torque_entries || torque_entries->nrow < 0 || root_dof_count < 0)
+    return IM_ERR_ARG;
+  const int nt = torque_entries->nrow;
+  if (nworld == 0 || nt == 0) return IM_OK;
+  if (!geo_ok(geometry) || !seg_ok(segments) || !torque_entries->offsets || !unit_force || !lower ||
+      !upper)
+    return IM_ERR_ARG;
+  if (torque_entries->nentry > 0 && (!torque_entries->segment || !torque_entries->other ||
+                                     !torque_entries->start_coeff || !torque_entries->end_coeff))
+    return IM_ERR_ARG;
+  if (ld_bounds < nt) return IM_ERR_STRIDE;
+  IM_FOR_WORLD_SLABS(nworld, w0, nw) {
+    hipLaunchKernelGGL(torque_bounds_kernel, grid2(nt, nw), dim3(256), 0, (hipStream_t)stream,
+                       slab(geometry, w0), seg(segments), torque_entries->offsets,
+                       torque_entries->segment, torque_entries->other,
+                       torque_entries->start_coeff, torque_entries->end_coeff,
+                       unit_force + w0 * ld_unit, ld_unit, root_dof_count, nt,
+                       lower + w0 * ld_bounds, upper + w0 * ld_bounds, ld_bounds);
   }
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;

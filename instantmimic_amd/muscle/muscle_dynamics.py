@@ -182,6 +182,7 @@ class MuscleDynamicsLayer:
         torque_dim: int,
         muscle_count: int,
         mechanics: MuscleMechanics | None = None,
+        active_torque_indices=None,
         device="cuda",
     ):
         import torch
@@ -199,6 +200,9 @@ class MuscleDynamicsLayer:
         self.include_passive_force_in_output = self.mechanics.include_passive_force_in_output
         self.muscle_force_velocity_enabled = False
         self.device = torch.device(device)
+        # MuscleOutputSpec.active_torque_indices of the reference (runtime_specs.py:53-63)
+        self.active_torque_indices = None if active_torque_indices is None else _np(active_torque_indices)
+        self.active_output_dim = self.torque_dim if self.active_torque_indices is None else len(self.active_torque_indices)
         # raw context = xpos | xquat | xipos | subtree_com | cdof (muscle_dynamics.py:4824-4838)
         nb, nvf = self.body_count, self.full_torque_dim
         self._xpos_off, self._xquat_off = 0, 3 * nb
@@ -384,6 +388,57 @@ class MuscleDynamicsLayer:
             "im_muscle_activation_grad",
         )  # fmt: skip
         return grad
+
+    def _warp_muscle_dynamics_from_activation_forward_cached_lbs_force(
+        self, activation, raw_context, unit_force_magnitude, passive_force_magnitude, *, include_passive_force: bool
+    ):
+        """Torque from force magnitudes computed outside this call (the reference method of
+        this name behind instantmimic_muscle::torque_cached_lbs_forward)."""
+        import torch
+
+        activation, raw_context = activation.float(), raw_context.float()
+        self._need_gpu(activation, raw_context, unit_force_magnitude, passive_force_magnitude)
+        B = activation.shape[0]
+        for t in (activation, unit_force_magnitude, passive_force_magnitude):
+            if tuple(t.shape) != (B, self.muscle_count):
+                raise ValueError("activation and force magnitudes must be (batch, muscle_count)")
+        _, geo = self._prepare_waypoint_geometry(raw_context, include_passive_force_magnitude=False, compute_force_magnitudes=False)
+        mean = torch.empty((B, self.torque_dim), device=activation.device)
+        u, p = unit_force_magnitude, passive_force_magnitude
+        _lib.check(
+            _lib.lib().im_muscle_torque_forward(
+                C.byref(geo), C.byref(self._segments), C.byref(self._torque_entries), u.data_ptr(), u.stride(0),
+                p.data_ptr() if include_passive_force else None, p.stride(0), activation.data_ptr(),
+                activation.stride(0), self.root_dof_count, mean.data_ptr(), mean.stride(0), B, _stream(activation),
+            ),
+            "im_muscle_torque_forward",
+        )  # fmt: skip
+        return mean
+
+    def _compute_activation_torque_bounds_warp(self, raw_context, *, select_active: bool):
+        """(lower, upper) of the torque over activations in [0, 1] at the context's geometry
+        (reference muscle_dynamics.py:4810-4822); ``select_active`` keeps the layer's
+        active torque indices."""
+        import torch
+
+        raw_context = raw_context.float()
+        self._need_gpu(raw_context)
+        ws, geo = self._prepare_waypoint_geometry(raw_context, include_passive_force_magnitude=False)
+        B = raw_context.shape[0]
+        lower = torch.empty((B, self.torque_dim), device=raw_context.device)
+        upper = torch.empty_like(lower)
+        u = ws["unit_force_magnitude"]
+        _lib.check(
+            _lib.lib().im_muscle_torque_bounds(
+                C.byref(geo), C.byref(self._segments), C.byref(self._torque_entries), u.data_ptr(), u.stride(0),
+                self.root_dof_count, lower.data_ptr(), upper.data_ptr(), lower.stride(0), B, _stream(raw_context),
+            ),
+            "im_muscle_torque_bounds",
+        )  # fmt: skip
+        if select_active and self.active_torque_indices is not None:
+            idx = torch.from_numpy(self.active_torque_indices.astype(np.int64)).to(raw_context.device)
+            return lower.index_select(1, idx), upper.index_select(1, idx)
+        return lower, upper
 
     def eval_muscle_sparse_moment(self, raw_context, moment_out=None):
         """moment (batch, entries) of the (muscle, dof) entries in ``sparse_entries``

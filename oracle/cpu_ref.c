@@ -1016,3 +1016,38 @@ int orc_muscle_sparse_moment(int nworld, int nwp, int nbody, int nv, int nentry,
   }
   return 0;
 }
+
+/* _compute_muscle_dynamics_sparse_bounds_kernel (muscle_dynamics_kernels.py:1453-1528) */
+int orc_muscle_torque_bounds(int nworld, int nwp, int nbody, int nv, int nmuscle, int ntorque,
+                             const float *wp, const float *com, const float *cdof,
+                             const int *seg_p0, const int *seg_p1, const int *seg_b0,
+                             const int *seg_b1, const int *offsets, const int *e_seg,
+                             const int *e_muscle, const float *e_a, const float *e_b,
+                             const float *unit, int root, float *lower, float *upper) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    ORC_GEO(w);
+    for (int j = 0; j < ntorque; ++j) {
+      v3 ang = v_ld(cdw + 6 * (j + root)), lin = v_ld(cdw + 6 * (j + root) + 3);
+      int current = -1;
+      float total = 0.0f, lo = 0.0f, hi = 0.0f;
+      for (int e = offsets[j]; e < offsets[j + 1]; ++e) {
+        int m = e_muscle[e];
+        if (current >= 0 && m != current) {
+          if (total < 0.0f) lo = lo + total;
+          else hi = hi + total;
+          total = 0.0f;
+        }
+        current = m;
+        total = total + ORC_TERM(e_seg[e], lin, ang, e_a[e], e_b[e], unit[(size_t)w * nmuscle + m]);
+      }
+      if (current >= 0) {
+        if (total < 0.0f) lo = lo + total;
+        else hi = hi + total;
+      }
+      lower[(size_t)w * ntorque + j] = lo;
+      upper[(size_t)w * ntorque + j] = hi;
+    }
+  }
+  return 0;
+}

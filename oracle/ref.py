@@ -425,3 +425,21 @@ def dense_update_factor(state_changes, changes, ids, J, D, state, grad, H, U, do
     )  # fmt: skip
     assert status == 0
     return H, U, uni, search, sdot, decr
+
+
+def muscle_torque_bounds(waypoints, com, cdof, seg, entries, unit, root):
+    """Pinned by tests/test_muscle_dynamics.py: lower / upper = the negative / positive
+    parts of the dense fp64 moment matrix times the unit forces, summed over muscles."""
+    waypoints, com, cdof, (nworld, nwp, nbody, nv) = _geo(waypoints, com, cdof)
+    unit = _f(unit)
+    off, es, em, ea, eb = entries
+    ntorque = len(off) - 1
+    lower = np.zeros((nworld, ntorque), np.float32)
+    upper = np.zeros((nworld, ntorque), np.float32)
+    s = [_i(a) for a in seg]
+    keep = [_i(off), _i(es), _i(em), _f(ea), _f(eb)]
+    lib().orc_muscle_torque_bounds(
+        nworld, nwp, nbody, nv, unit.shape[1], ntorque, _p(waypoints), _p(com), _p(cdof), *[_p(a) for a in s],
+        *[_p(a) for a in keep], _p(unit), int(root), _p(lower), _p(upper),
+    )  # fmt: skip
+    return lower, upper

@@ -313,6 +313,20 @@ def test_oracle_contractions_against_dense_fp64(rig_layer):
     assert np.abs(dense - T).max() < 1e-5 * np.abs(T).max()  # nothing of T lies off the entry list
 
 
+def test_oracle_bounds_against_dense_fp64(rig_layer):
+    rig, layer = rig_layer
+    ctx = synth.make_muscle_context(rig, 8, seed=17)
+    _, wp, unit, _ = oracle_forward(layer, ctx, np.ones((8, rig.muscle_count), np.float32), False)
+    _, _, com, cdof = split_context(layer, ctx)
+    tq = layer.torque_entries_host
+    lo, hi = ref.muscle_torque_bounds(wp, com, cdof, layer.segments_host, (tq[0], tq[2], tq[3], tq[4], tq[5]), unit,
+                                      layer.root_dof_count)  # fmt: skip
+    per_muscle = moment_matrix64(layer, wp.astype(np.float64), com, cdof) * unit[:, None, :]
+    assert ref.rel_l2(lo, np.minimum(per_muscle, 0).sum(-1)) < 2e-6
+    assert ref.rel_l2(hi, np.maximum(per_muscle, 0).sum(-1)) < 2e-6
+    assert (lo <= 0).all() and (hi >= 0).all()
+
+
 def test_oracle_degenerate_segment_contributes_nothing():
     layer = fixture_layer()
     ctx = fixture_context(layer)
@@ -349,6 +363,11 @@ def test_operator_schemas_and_registry():
         c = torch.empty(5, layer.context_dim)
         assert ops.muscle_torque_forward(a, c, key, False).shape == (5, 2)
         assert ops.muscle_torque_backward(c, torch.empty(5, 2), key).shape == (5, 3)
+        u = torch.empty(5, 3)
+        assert ops.muscle_torque_cached_lbs_forward(a, c, u, u, key, True).shape == (5, 2)
+        assert ops.muscle_torque_cached_lbs_backward(c, u, torch.empty(5, 2), key).shape == (5, 3)
+        lo, hi = ops.muscle_torque_bounds(c, key, True)
+        assert lo.shape == hi.shape == (5, 2)
     del layer
     gc.collect()
     with pytest.raises(RuntimeError, match="not registered"):
@@ -461,6 +480,42 @@ def test_gpu_operator_fixture_closed_form_autograd_and_compile():
     del layer
     gc.collect()
     pending.backward()
+
+
+@pytest.mark.gpu
+def test_gpu_cached_force_ops_and_bounds():
+    rig = synth.make_muscle_rig(nmuscle=284, seed=1003)
+    active = np.arange(0, rig.torque_dim, 3)
+    layer = MuscleDynamicsLayer(rig.topology, **rig.dims(), mechanics=MuscleMechanics(), active_torque_indices=active,
+                                device="cuda")  # fmt: skip
+    nworld = 93
+    ctx = synth.make_muscle_context(rig, nworld, seed=31)
+    ctx_d = torch.from_numpy(ctx).cuda()
+    key = ops.warp_op_key(layer)
+    act = torch.rand(nworld, rig.muscle_count, device="cuda", requires_grad=True)
+    torque = ops.muscle_torque_forward(act, ctx_d, key, True)
+    ws, _ = layer._prepare_waypoint_geometry(ctx_d, include_passive_force_magnitude=True)
+    unit, pas = ws["unit_force_magnitude"], ws["passive_force_magnitude"]
+    cached = ops.muscle_torque_cached_lbs_forward(act, ctx_d, unit, pas, key, True)
+    assert torch.equal(cached, torque)
+    g = torch.randn_like(torque)
+    (g1,) = torch.autograd.grad(torque, act, g, retain_graph=True)
+    (g2,) = torch.autograd.grad(cached, act, g)
+    assert torch.equal(g1, g2) and torch.count_nonzero(g1) > 0
+    lo, hi = ops.muscle_torque_bounds(ctx_d, key, False)
+    wp = ws["transformed_waypoints"].cpu().numpy().reshape(nworld, -1, 3)
+    _, _, com, cdof = split_context(layer, ctx)
+    tq = layer.torque_entries_host
+    want_lo, want_hi = ref.muscle_torque_bounds(wp, com, cdof, layer.segments_host,
+                                                (tq[0], tq[2], tq[3], tq[4], tq[5]), unit.cpu().numpy(),
+                                                layer.root_dof_count)  # fmt: skip
+    assert np.array_equal(lo.cpu().numpy(), want_lo) and np.array_equal(hi.cpu().numpy(), want_hi)
+    # activations in [0, 1] without passive force stay inside the box
+    inside = ops.muscle_torque_forward(act.detach(), ctx_d, key, False)
+    tol = 1e-4 * hi.abs().max()
+    assert (inside >= lo - tol).all() and (inside <= hi + tol).all()
+    slo, shi = ops.muscle_torque_bounds(ctx_d, key, True)
+    assert torch.equal(slo, lo[:, active]) and torch.equal(shi, hi[:, active])
 
 
 @pytest.mark.gpu
