@@ -341,12 +341,12 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
   if (plan->row16) {
     const auto *e = (const gen::Row16Entry *)plan->row16;
     void *args[] = {&M, &ldM, &J, &njmax, &D, &state, &nefc, &quad, &y, &ldy, &x, &ldx, &Hout, &nworld, &flags};
-    // the fused kernel copies J in 16-byte pieces: every world's block must be 16-byte aligned
-    const bool aligned = !assemble || ((((size_t)njmax * plan->nv) % 4 == 0) && ((uintptr_t)J % 16 == 0));
-    if (aligned) {
+    // staged rows plus the four worlds' active-row lists (row id and D per constraint row)
+    const size_t lds = assemble ? (size_t)e->lds_bytes + 32 * (((size_t)njmax + 15) / 16 * 16) : 0;
+    if (lds <= 64 * 1024) {
+      // fused: one wavefront per world assembles, the first one factors and solves all four
       IM_HIP_CHECK(hipLaunchKernel(assemble ? e->fused : e->solve, dim3((nworld + 3) / 4),
-                                   dim3(64), args, assemble ? e->lds_bytes : 0,
-                                   (hipStream_t)stream));
+                                   dim3(assemble ? 256 : 64), args, lds, (hipStream_t)stream));
       return IM_OK;
     }
   }
@@ -450,8 +450,6 @@ int tree_plan_upload(im_tree_plan *pl) {
   pl->row16 = (force && std::strcmp(force, "generic") == 0) ? nullptr : (const void *)gen::find_row16(tree_key(*pl));
   if (pl->row16) {
     const auto *e = (const gen::Row16Entry *)pl->row16;
-    if (e->lds_bytes > 64 * 1024)
-      IM_HIP_CHECK(hipFuncSetAttribute(e->fused, hipFuncAttributeMaxDynamicSharedMemorySize, e->lds_bytes));
   }
   return IM_OK;
 }

@@ -12,6 +12,8 @@
 namespace im {
 namespace gen {
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 #define IM_ROW16_PARAMS                                                                   \
   const float *__restrict__ M, int64_t ldM, const float *__restrict__ J, int njmax,       \
       const float *__restrict__ D, const int *__restrict__ state,                         \
@@ -31,10 +33,19 @@ namespace gen {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  \
   } while (0)
 
+// orders one wavefront's LDS writes before its later reads (the workgroup is one wavefront)
+#define IM_WAVE_SYNC()                                      \
+  do {                                                      \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  \
+    __builtin_amdgcn_wave_barrier();                        \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");  \
+  } while (0)
+
 struct Row16Entry {
   uint64_t key;  // FNV-1a over the CSR structure and the plan
   int nv, nM;
-  int lds_bytes;  // dynamic LDS of the fused kernel (staged constraint rows)
+  int lds_bytes;  // dynamic LDS of the fused kernel (staged constraint rows); the launch adds
+                  // 32 bytes per constraint row (rounded up to 16 rows) for the active-row lists
   const char *name;
   const void *fused;  // assemble + factor + solve
   const void *solve;  // factor + solve
