@@ -1,44 +1,51 @@
 """Generator of plan-specialised gfx950 kernels for the fused Hessian assembly +
-tree L'DL + solve ("row16" layout).
+tree L'DL + solve.
 
-Layout.  Four worlds share a wavefront; a world owns one 16-lane DPP row.  Row b of
-H (the CSR row of dof b: its ancestors root-first, then b) lives in one VGPR per 16
-positions: lane p of register ``h{b}_{s}`` holds H[b][anc_{16 s + p}(b)].  All dofs on
-one root-to-leaf chain agree on what sits at position p, so
+Fused kernel: one workgroup of four wavefronts per four worlds.
 
-* assembling ``H[b][a] += (J[r][a] D[r]) J[r][b]`` is one ``v_fmac_f32_dpp`` per row b and
-  constraint row r: the chain-gathered J row times D in every lane, times J[r][b]
-  broadcast from b's own position with ``row_newbcast``;
-* only the rows that contribute are visited: a world's rows with ``state == quad`` below
-  ``nefc`` are compacted (ballot + prefix count, order kept) into a list in LDS, each lane
-  fetches one listed row from HBM, and the wavefront loops over the longest of its four
-  lists.  A skipped row would have added ``(J * 0) * J`` to every entry, so the sums keep
-  their values;
-* eliminating dof k updates ancestor row anc_p with
+* Assembly.  Wavefront v assembles world v on the matrix cores: H is cut into 16 x 16
+  tiles of its lower triangle and every step of four constraint rows is three (or more)
+  ``v_mfma_f32_16x16x4_f32`` with A = J and B = J * D.  The instruction accumulates its
+  four products one after the other with fused multiply-adds, which is the order and
+  rounding of ``v = fmaf(J[r][a] * D[r], J[r][b], v)`` over the rows r
+  (src/instantmimic/utils/mjw_kernels/sparse_hessian.py:622-629); the accumulators start
+  from M.  J goes from HBM straight into the operand registers (lane = (row of the step,
+  column)), never through LDS.  With at most 64 constraint rows the first 16 rows are
+  requested at once and of the others only those with ``state == quad`` below ``nefc``
+  (their ids packed in row order by a ballot and a prefix count): a row left out would
+  have added ``(J * 0) * J`` to every entry.  All loads are unconditional and counted, so
+  each step waits for exactly its own operands.
+* Hand-over.  The tiles go to a dense copy of H in LDS; from there each wavefront reads
+  the rows it factors in the "row16" layout: a world owns one 16-lane DPP row, row b of H
+  (the CSR row of dof b: its ancestors root-first, then b) lives in one VGPR per 16
+  positions, lane p of register ``h{b}_{s}`` holds H[b][anc_{16 s + p}(b)].  All dofs on one
+  root-to-leaf chain agree on what sits at position p.
+* Factor and solve (src/instantmimic/utils/mjw_kernels/tree_ldl.py:215-305).  Wavefront j
+  eliminates group j of the plan into zero-initialised trunk accumulators and publishes
+  them through LDS; wavefront 0 adds them to the trunk rows in group order, eliminates and
+  solves the trunk and publishes its solution; the groups then back-substitute.
+  Eliminating dof k updates ancestor row anc_p with
   ``h[anc_p] = fma(bcast(h[k], p) * h[k], -1/h[k][k], h[anc_p])`` (``v_mul_f32_dpp`` then a
-  plain fma) - the pivot row never leaves its registers and nothing goes through LDS;
-* right-hand side, inverse pivots and the solution are kept uniform per world; their
-  updates are single ``v_fmac_f32_dpp`` with the scaled pivot row ``T[k] = h[k] * -1/h[k][k]``
-  as the broadcast operand.
+  plain fma); right-hand side, inverse pivots and solution are uniform per world and their
+  updates are single ``v_fmac_f32_dpp`` with the scaled pivot row
+  ``T[k] = h[k] * -1/h[k][k]`` as the broadcast operand.
+
+The solve-only kernel is one wavefront per four worlds that reads M in the row16 layout
+and takes every role in turn.
 
 DPP reads of a register written by one of the two preceding VALU instructions are a
 hardware hazard that the compiler does not see inside inline assembly: every block that
-reads registers produced outside it starts with ``s_nop 1``.
-
-Lanes past a row's length hold unused values that no valid lane ever reads.  The
-order of floating-point operations per entry equals the reference's generated code
-(src/instantmimic/utils/mjw_kernels/tree_ldl.py:215-305 for the factor and solve,
-src/instantmimic/utils/mjw_kernels/sparse_hessian.py:622-629 for the assembly).
+reads registers produced outside it starts with ``s_nop 1``.  Lanes past a row's length
+hold unused values that no valid lane ever reads.
 """
 
 from __future__ import annotations
 
-import hashlib
-
-ROWS_PER_BLOCK = 16
 import os
+
+# development aid: IMHIP_EXP=timing makes the fused kernel write clock64() stamps of its phases
+# over the H output buffer instead of H
 EXP = os.environ.get("IMHIP_EXP", "")
-NOPS = True
 
 
 def structure_key(rowadr, rownnz, colind, groups, trunk) -> int:
@@ -128,7 +135,8 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     for row in idx_rows:
         emit("  {" + ",".join(str(v) for v in row) + "},")
     emit("};")
-    emit("template <bool ASM>")
+    # LONG: more constraint rows than the straight-line assembly keeps in flight (a loop instead)
+    emit("template <bool ASM, bool LONG>")
     emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? 4 : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
     emit("  const int lane = threadIdx.x & 63, p = lane & 15, wv = threadIdx.x >> 6;")
     emit("  const int w = blockIdx.x * 4 + (lane >> 4);")
@@ -188,7 +196,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     emit("    float *lds = xlds;")
     emit("    const int kq = lane >> 4;")
     emit("    const int njp = (njmax + 15) & ~15;")
-    emit(f"    float *dcl = lds + {lds_floats} + wv * njp;  // D of this world's contributing rows, 0 for the others")
+    emit(f"    float *dcl = lds + {lds_floats} + wv * (LONG ? njp : 128);  // D per row (0 where a row does not contribute)")
     emit("    const int64_t wq = blockIdx.x * 4 + wv < nworld ? blockIdx.x * 4 + wv : nworld - 1;")
     emit("    int ne = nefc_p ? nefc_p[wq] : njmax; ne = ne < njmax ? ne : njmax;")
     emit("    ne = __builtin_amdgcn_readfirstlane(ne);")
@@ -210,10 +218,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             emit(f"          g{u}_{c} = pj{c}[rowc * {nv}];")
         emit("        }")
 
-    def consume(u, step):
+    def consume(u, step, valid=None):
         # rows at or past the world's nefc may hold anything: they count as zero rows; columns
         # past nv repeat the last column, which only reaches accumulator elements outside H
-        emit(f"        {{ const int st = {step}; const float d = pd[st * 4]; const bool rv = st * 4 + kq < ne;")
+        emit(f"        {{ const int st = {step}; const float d = pd[st * 4]; const bool rv = {valid or 'st * 4 + kq < ne'};")
         for c in range(NT):
             emit(f"          const float z{c} = rv ? g{u}_{c} : 0.0f;")
         for c in range(NT):
@@ -232,21 +240,52 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             emit(f"    const int ix{n}_{v} = IDX_{name}[{n * 4 + v}][lane];")
     for i in range(MC):
         emit(f"    const float mv{i} = M[wq * ldM + min({i * 64} + lane, {nM - 1})];")
-    emit("    for (int r0 = 128; r0 < njp; r0 += 64) {  // long constraint lists: rows from 128 on, up front")
-    emit("      const int r = r0 + lane, rc = r < njmax ? r : njmax - 1;")
-    emit("      const int sv = state[wq * njmax + rc]; const float dv = D[wq * njmax + rc];")
-    emit("      if (r < njp) dcl[r] = (r < ne && sv == quad) ? dv : 0.0f;")
+    SP = 4  # steps (16 rows) requested before the row weights are known
+    emit("    int steps_s = 0, cnt = 0;  // short variant: steps and length of the compacted tail")
+    emit("    if (LONG) {")
+    emit("      for (int r0 = 128; r0 < njp; r0 += 64) {  // rows from 128 on, up front")
+    emit("        const int r = r0 + lane, rc = r < njmax ? r : njmax - 1;")
+    emit("        const int sv = state[wq * njmax + rc]; const float dv = D[wq * njmax + rc];")
+    emit("        if (r < njp) dcl[r] = (r < ne && sv == quad) ? dv : 0.0f;")
+    emit("      }")
     emit("    }")
     emit("    const int rc0 = lane < njmax ? lane : njmax - 1, rc1 = lane + 64 < njmax ? lane + 64 : njmax - 1;")
-    emit("    const int sv0 = state[wq * njmax + rc0], sv1 = state[wq * njmax + rc1];")
-    emit("    const float dv0 = D[wq * njmax + rc0], dv1 = D[wq * njmax + rc1];")
+    emit("    const int sv0 = state[wq * njmax + rc0], sv1 = LONG ? state[wq * njmax + rc1] : 0;")
+    emit("    const float dv0 = D[wq * njmax + rc0], dv1 = LONG ? D[wq * njmax + rc1] : 0.0f;")
+    emit("    if (LONG) {")
     for u in range(PD):
         load(u, str(u))
+    emit("    } else {")
+    for u in range(SP):
+        load(u, str(u))
+    emit("    }")
     emit(f"    float *mcopy = lds + wv * {W * W};  // reused for this world's dense H afterwards")
     for i in range(MC):
         emit(f"    mcopy[{i * 64} + lane] = mv{i};")
-    emit("    if (lane < njp) dcl[lane] = (lane < ne && sv0 == quad) ? dv0 : 0.0f;")
-    emit("    if (lane + 64 < njp) dcl[lane + 64] = (lane + 64 < ne && sv1 == quad) ? dv1 : 0.0f;")
+    emit("    if (LONG) {")
+    emit("      if (lane < njp) dcl[lane] = (lane < ne && sv0 == quad) ? dv0 : 0.0f;")
+    emit("      if (lane + 64 < njp) dcl[lane + 64] = (lane + 64 < ne && sv1 == quad) ? dv1 : 0.0f;")
+    emit("    } else {")
+    # Short variant (njmax <= 64, one row per lane): the first 16 rows are read as they are,
+    # with D = 0 for the ones that do not contribute; of the others only the contributing rows
+    # are read at all -- their ids and D are packed behind entry 16 in row order (ballot and
+    # prefix count), so a skipped row is one that would have added (J * 0) * J everywhere.
+    emit(f"      int *rowl = (int *)(dcl + 64);")
+    emit(f"      const bool act0 = lane < ne && sv0 == quad;")
+    emit(f"      const bool tail = act0 && lane >= {4 * SP};")
+    emit("      const unsigned long long tm = __ballot(tail);")
+    emit("      cnt = __popcll(tm);")
+    emit(f"      steps_s = ne > {4 * SP} ? {SP} + ((cnt + 3) >> 2) : ((ne + 3) >> 2);")
+    emit("      dcl[lane] = 0.0f; rowl[lane] = 0;")
+    emit(f"      if (lane < {4 * SP}) {{ dcl[lane] = act0 ? dv0 : 0.0f; rowl[lane] = lane; }}")
+    emit(f"      if (tail) {{ const int pos = {4 * SP} + __popcll(tm & ((1ull << lane) - 1ull)); dcl[pos] = dv0; rowl[pos] = lane; }}")
+    emit("      IM_WAVE_SYNC();")
+    for u in range(SP, PD):
+        emit(f"      {{ const int rowc = rowl[{4 * u} + kq];")
+        for c in range(NT):
+            emit(f"        g{u}_{c} = pj{c}[rowc * {nv}];")
+        emit("      }")
+    emit("    }")
     emit("    IM_WAVE_SYNC();")
     for n in range(len(tiles)):
         emit(f"    f32x4 acc{n};")
@@ -254,10 +293,13 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             emit(f"    {{ const float mvv = mcopy[ix{n}_{v} < 0 ? 0 : ix{n}_{v}]; acc{n}[{v}] = ix{n}_{v} >= 0 ? mvv : 0.0f; }}")
     emit("    IM_WAVE_SYNC();")
     emit("    STAMP();  // 1: row weights staged, M gathered")
-    emit(f"    if (steps <= {PD}) {{  // everything is already in flight")
+    emit("    if (!LONG) {  // every row that is needed is already in flight")
     for u in range(PD):
-        emit(f"      if ({u} < steps) {{")
-        consume(u, str(u))
+        emit(f"      if ({u} < steps_s) {{")
+        if u < SP:
+            consume(u, str(u))
+        else:
+            consume(u, str(u), valid=f"{4 * u} + kq < {4 * SP} + cnt")
         emit("      }")
     emit("    } else {")
     emit(f"    for (int s0 = 0; s0 < steps; s0 += {PD}) {{")
@@ -484,8 +526,9 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     emit("  STAMP();")
     emit("  #undef STAMP")
     emit("}")
-    emit(f"static const Row16Entry entry_{name} = {{0x{key:016x}ull, {nv}, {nM}, {lds_floats * 4}, \"{name}\",")
-    emit(f"    (const void *)tree_row16_{name}<true>, (const void *)tree_row16_{name}<false>}};")
+    emit(f"static const Row16Entry entry_{name} = {{0x{key:016x}ull, {nv}, {nM}, {lds_floats * 4}, {4 * PD}, \"{name}\",")
+    emit(f"    (const void *)tree_row16_{name}<true, false>, (const void *)tree_row16_{name}<true, true>,")
+    emit(f"    (const void *)tree_row16_{name}<false, false>}};")
     emit(f"static const Row16Register reg_{name}(&entry_{name});")
     emit("} }  // namespace im::gen")
     return "\n".join(out) + "\n"

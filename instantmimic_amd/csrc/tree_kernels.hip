@@ -342,10 +342,11 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
     const auto *e = (const gen::Row16Entry *)plan->row16;
     void *args[] = {&M, &ldM, &J, &njmax, &D, &state, &nefc, &quad, &y, &ldy, &x, &ldx, &Hout, &nworld, &flags};
     // staged rows plus the four worlds' active-row lists (row id and D per constraint row)
-    const size_t lds = assemble ? (size_t)e->lds_bytes + 32 * (((size_t)njmax + 15) / 16 * 16) : 0;
+    const size_t lds = assemble ? (size_t)e->lds_bytes + 32 * std::max<size_t>(((size_t)njmax + 15) / 16 * 16, 64) : 0;
     if (lds <= 64 * 1024) {
       // fused: one wavefront per world assembles, the first one factors and solves all four
-      IM_HIP_CHECK(hipLaunchKernel(assemble ? e->fused : e->solve, dim3((nworld + 3) / 4),
+      const void *fn = !assemble ? e->solve : (njmax <= e->short_rows ? e->fused : e->fused_long);
+      IM_HIP_CHECK(hipLaunchKernel(fn, dim3((nworld + 3) / 4),
                                    dim3(assemble ? 256 : 64), args, lds, (hipStream_t)stream));
       return IM_OK;
     }

@@ -46,9 +46,11 @@ struct Row16Entry {
   int nv, nM;
   int lds_bytes;  // dynamic LDS of the fused kernel (staged constraint rows); the launch adds
                   // 32 bytes per constraint row (rounded up to 16 rows) for the active-row lists
+  int short_rows;  // njmax up to which the straight-line fused kernel applies
   const char *name;
-  const void *fused;  // assemble + factor + solve
-  const void *solve;  // factor + solve
+  const void *fused;       // assemble + factor + solve, njmax <= short_rows
+  const void *fused_long;  // the same with a loop over the constraint rows
+  const void *solve;       // factor + solve
 };
 
 // Registers a generated kernel at load time.
