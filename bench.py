@@ -27,9 +27,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the fused kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain
 # 64 MiB device copy in the same run (FETCH_SIZE reads 32781 KiB for it, WRITE_SIZE 65536):
-#   (17494.05 * 65536 / 32781.22 + 448.0 * 65536 / 65536) KiB
+#   (15862.14 * 65536 / 32781.48 + 448.0 * 65536 / 65536) KiB
 # Recorded in profiles/tree_row16_humanoid_pmc.txt.
-TRAFFIC_BYTES_PER_LAUNCH = int((17494.05 * 65536 / 32781.22 + 448.0) * 1024)
+TRAFFIC_BYTES_PER_LAUNCH = int((15862.14 * 65536 / 32781.48 + 448.0) * 1024)
 
 
 def algorithmic_bytes(nv: int, nM: int, nefc: int) -> int:
