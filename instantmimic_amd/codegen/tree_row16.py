@@ -137,7 +137,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     emit("};")
     # LONG: more constraint rows than the straight-line assembly keeps in flight (a loop instead)
     emit("template <bool ASM, bool LONG>")
-    emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? 4 : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
+    emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? IM_OCC_{name} : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
     emit("  const int lane = threadIdx.x & 63, p = lane & 15, wv = threadIdx.x >> 6;")
     emit("  const int w = blockIdx.x * 4 + (lane >> 4);")
     emit("  const bool live = w < nworld;")
@@ -531,4 +531,9 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     emit(f"    (const void *)tree_row16_{name}<false, false>}};")
     emit(f"static const Row16Register reg_{name}(&entry_{name});")
     emit("} }  // namespace im::gen")
-    return "\n".join(out) + "\n"
+    # workgroups per CU that the fused kernel is compiled for: what the 160 KB of LDS admit (with
+    # the lists of 128 constraint rows), at most 4 -- fewer workgroups leave each wavefront more
+    # registers, which the larger trees need
+    occ = max(1, min(4, (160 * 1024) // (lds_floats * 4 + 32 * 128)))
+    text = "\n".join(out) + "\n"
+    return text.replace('#include "../tree_row16.h"', f'#include "../tree_row16.h"\n#define IM_OCC_{name} {occ}', 1)

@@ -343,7 +343,7 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
     void *args[] = {&M, &ldM, &J, &njmax, &D, &state, &nefc, &quad, &y, &ldy, &x, &ldx, &Hout, &nworld, &flags};
     // staged rows plus the four worlds' active-row lists (row id and D per constraint row)
     const size_t lds = assemble ? (size_t)e->lds_bytes + 32 * std::max<size_t>(((size_t)njmax + 15) / 16 * 16, 64) : 0;
-    if (lds <= 64 * 1024) {
+    if (lds <= 160 * 1024) {
       // fused: one wavefront per world assembles, the first one factors and solves all four
       const void *fn = !assemble ? e->solve : (njmax <= e->short_rows ? e->fused : e->fused_long);
       IM_HIP_CHECK(hipLaunchKernel(fn, dim3((nworld + 3) / 4),
@@ -450,7 +450,13 @@ int tree_plan_upload(im_tree_plan *pl) {
   const char *force = std::getenv("IMHIP_TREE_KERNEL");
   pl->row16 = (force && std::strcmp(force, "generic") == 0) ? nullptr : (const void *)gen::find_row16(tree_key(*pl));
   if (pl->row16) {
+    // the fused kernels stage four dense copies of H in LDS: large trees need more than the
+    // default 64 KB of dynamic LDS, which has to be granted before the first launch
     const auto *e = (const gen::Row16Entry *)pl->row16;
+    if (e->lds_bytes + 32 * 64 > 48 * 1024) {
+      IM_HIP_CHECK(hipFuncSetAttribute(e->fused, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+      IM_HIP_CHECK(hipFuncSetAttribute(e->fused_long, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    }
   }
   return IM_OK;
 }

@@ -1,0 +1,219 @@
+"""Per-kernel timings of the library on the configured shapes, one JSON line per kernel:
+
+    python -m instantmimic_amd.rowbench [--launches N]
+
+Every line names the kernel, the workload, the mean time of one launch (event-timed hipGraph
+replay over rotating input sets), the algorithmic bytes or flops of that launch and the
+fraction of the MI355X roofline that bounds it (HBM 8 TB/s; fp32 matrix cores 157.3 TFLOP/s).
+Algorithmic bytes count every input and output array once.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+from types import SimpleNamespace
+
+import numpy as np
+
+HBM_GBS = 8000.0
+MFMA_F32_TFLOPS = 157.3
+
+
+def _timeit(torch, fn, nsets: int, launches: int) -> float:
+    for i in range(min(nsets, 4)):
+        fn(i)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        fn(0)
+        with torch.cuda.graph(g, stream=s):
+            for i in range(launches):
+                fn(i % nsets)
+    torch.cuda.current_stream().wait_stream(s)
+    g.replay()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(5):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        best = min(best, a.elapsed_time(b) / launches * 1e-3)
+    return best
+
+
+def _line(kernel, workload, seconds, *, bytes_=None, flops=None, nworld=None):
+    out = {"kernel": kernel, "workload": workload, "us_per_launch": round(seconds * 1e6, 2)}
+    if nworld:
+        out["worlds_per_s"] = round(nworld / seconds)
+    if bytes_ is not None:
+        gbs = bytes_ / seconds / 1e9
+        out.update(bound="hbm", algorithmic_bytes=int(bytes_), achieved_GBs=round(gbs, 1), frac=round(gbs / HBM_GBS, 4))
+    if flops is not None:
+        tf = flops / seconds / 1e12
+        out.update(bound="mfma", algorithmic_flops=int(flops), achieved_TFLOPs=round(tf, 2), frac=round(tf / MFMA_F32_TFLOPS, 4))
+    print(json.dumps(out), flush=True)
+
+
+def run(launches: int = 32) -> None:
+    import torch
+
+    from . import synth
+    from .mjw_kernels import blocked_dense as BD
+    from .mjw_kernels import newton_stages as NS
+    from .mjw_kernels import sparse_hessian as SH
+    from .mjw_kernels import tree_ldl as T
+    from .muscle import muscle_qfrc_projector as Q
+    from .muscle.muscle_dynamics import MuscleDynamicsLayer
+
+    dev = torch.device("cuda:0")
+
+    def t(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    def sets_of(arrays, nsets):
+        return [[t(a) for a in arrays] for _ in range(nsets)]
+
+    # ---- fused assemble + tree L'DL + solve and solve-only on every tree shape
+    for name, nsets in (("ant", 8), ("humanoid", 16), ("g1", 8), ("snu", 8)):
+        b = synth.make_batch(name)
+        nv, nM, nefc, nworld = b.shape.nv, int(b.colind.size), b.shape.nefc, b.nworld
+        m = SimpleNamespace(nv=nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind)
+        sc = T.create_tree_factor_solve_scratch(m, dev)
+        S = sets_of((b.M, b.J, b.D, b.state[0], b.nefc, b.grad), nsets)
+        X = [torch.zeros(b.grad.shape, device=dev) for _ in range(nsets)]
+        wl = f"{name} nv={nv} nM={nM} nefc={nefc} x {nworld} worlds"
+        sec = _timeit(torch, lambda i: T.assemble_tree_factor_solve(sc, *S[i], X[i]), nsets, launches)
+        _line("im_assemble_tree_ldl_solve", wl, sec, bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv), nworld=nworld)
+        sec = _timeit(torch, lambda i: T.tree_factor_solve(sc, S[i][0], X[i], S[i][5]), nsets, launches)
+        _line("im_tree_factor_solve", wl, sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
+        if name in ("g1", "snu"):
+            # the same Hessians through the blocked dense factor and the static-pattern sparse L'DL
+            Md = synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32).reshape(nworld, -1)
+            mm = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))])
+            for B in (8, 16):
+                Mt = [t(Md) for _ in range(4)]
+                d = SimpleNamespace(nworld=nworld, M=Mt[0])
+                bs = BD.create_blocked_dense_factor_solve_scratch(mm, d, dev, block_size=B)
+                Y = t(b.grad).reshape(nworld, nv, 1)
+                Xb = torch.zeros_like(Y)
+                sec = _timeit(torch, lambda i: BD._blocked_dense_factor_solve(d, Mt[i], Xb, Y, bs), 4, launches)
+                _line(f"im_blocked_factor_solve B={B}", wl, sec, bytes_=nworld * 4 * (nv * nv + 2 * nv + bs.pad * bs.pad), nworld=nworld)
+            model = synth.model_from_parents(b.shape.parents)
+            plan, _ = SH.plan_for_model(model, None, [], SH.block_width(model.nv_pad), device=dev)
+            if plan is not None:
+                launch = SH.init_factor_kernel(plan)
+                hf = torch.zeros((nworld, plan.nv_pad, plan.nv_pad), device=dev)
+                search = torch.zeros((nworld, nv, 1), device=dev)
+                sd, de = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev)
+                G = [s[5][:, :, None].contiguous() for s in S]
+                sec = _timeit(torch, lambda i: launch(None, S[i][4], S[i][1], S[i][2], S[i][3], S[i][0], G[i], hf, search, sd, de), nsets, launches)
+                used = 2 * plan.nfac + nv
+                _line("im_sparse_init_factor", wl, sec, bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv + used + 2), nworld=nworld)
+                # per-iteration stage: a tenth of the rows change state
+                rng = np.random.default_rng(1)
+                ids = np.zeros((nworld, nefc), np.int32)
+                k = max(nefc // 10, 1)
+                for w in range(nworld):
+                    ids[w, :k] = np.sort(rng.choice(nefc, k, replace=False))
+                chg = t(np.full(nworld, k, np.int32))
+                uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=dev)
+                stage = NS.factor_factory(nv, plan.nv_pad, plan)
+                s2 = search.reshape(nworld, nv)
+                idt = t(ids)
+                sec = _timeit(torch, lambda i: stage(S[i][1], S[i][2], S[i][3], idt, chg, chg, None, S[i][5], None, hf, s2, sd, de, uni), nsets, launches)
+                _line("im_sparse_update_factor", wl + f", {k} changed rows", sec, bytes_=nworld * 4 * (k * nv + 2 * used + 2 * nv + nv + 1 + 2), nworld=nworld)
+        del S, X
+        torch.cuda.empty_cache()
+
+    # ---- stress: dense J'DJ on the matrix cores, blocked factor, dense per-iteration stage
+    b = synth.make_batch("stress", 16384)
+    nv, nefc, nworld = b.shape.nv, b.shape.nefc, b.nworld
+    pad = ((nv + 1 + 15) // 16) * 16
+    Md = t(synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32).reshape(nworld, -1))
+    J, D, st, ne, g = (t(a) for a in (b.J, b.D, b.state[0], b.nefc, b.grad))
+    H = torch.zeros((nworld, pad, pad), device=dev)
+    wl = f"stress nv={nv} nefc={nefc} x {nworld} worlds"
+    sec = _timeit(torch, lambda i: BD.dense_hessian(Md, J, D, st, ne, H), 1, 8)
+    _line("im_jtdj_mfma", wl, sec, flops=nworld * 2.0 * nv * nv * nefc, nworld=nworld)
+    _line("im_jtdj_mfma (as bytes)", wl, sec, bytes_=nworld * 4 * (nv * nv + nefc * nv + 2 * nefc + pad * pad), nworld=nworld)
+    mm = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))])
+    Hc = H[:, :nv, :nv].contiguous().reshape(nworld, -1)
+    d = SimpleNamespace(nworld=nworld, M=Hc)
+    bs = BD.create_blocked_dense_factor_solve_scratch(mm, d, dev, block_size=16)
+    Y = g.reshape(nworld, nv, 1)
+    Xb = torch.zeros_like(Y)
+    sec = _timeit(torch, lambda i: BD._blocked_dense_factor_solve(d, Hc, Xb, Y, bs), 1, 8)
+    _line("im_blocked_factor_solve B=16", wl, sec, bytes_=nworld * 4 * (nv * nv + 2 * nv + bs.pad * bs.pad), nworld=nworld)
+    rng = np.random.default_rng(2)
+    k = nefc // 10
+    ids = np.zeros((nworld, nefc), np.int32)
+    ids[:, :k] = np.sort(rng.permuted(np.tile(np.arange(nefc), (nworld, 1)), axis=1)[:, :k], axis=1)
+    chg = t(np.full(nworld, k, np.int32))
+    uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=dev)
+    U = torch.zeros((nworld, pad, pad), device=dev)
+    g3 = torch.zeros((nworld, pad, 1), device=dev)
+    g3[:, :nv, 0] = g
+    search = torch.zeros((nworld, pad, 1), device=dev)
+    sd, de = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev)
+    stage = NS.factor_factory(nv, pad)
+    idt = t(ids)
+    sec = _timeit(torch, lambda i: stage(J, D, st, idt, chg, chg, None, g3, H, U, search, sd, de, uni), 1, 8)
+    _line("im_dense_update_factor", wl + f", {k} changed rows", sec, bytes_=nworld * 4 * (k * nv + 2 * pad * pad + 2 * nv), nworld=nworld)
+    del J, H, U, Md, Hc
+    torch.cuda.empty_cache()
+
+    # ---- muscles on the SNU-like tree
+    nworld = 4096
+    mb = synth.make_muscles(nworld)
+    rowadr, rownnz, colind = synth.csr_from_parents(synth.snu_parents())
+    nv, nM = len(rowadr), int(colind.size)
+    ent = Q.entries_from_muscle_dofs(mb.muscle_dofs, mb.nmuscle)
+    ne_ = len(ent.muscle_dof_torque_idx)
+    offsets, order = Q.torque_sorted_entries(ent.muscle_dof_torque_idx, nv - mb.root_dof_count)
+    nsets = 8
+    mom = [t(mb.moment) for _ in range(nsets)]
+    frc = [t(mb.force) for _ in range(nsets)]
+    slope = [t(mb.slope) for _ in range(nsets)]
+    qfrc = torch.zeros((nworld, nv), device=dev)
+    off_d, ord_d, em_d = t(offsets), t(order), t(ent.muscle_dof_muscle_idx.astype(np.int32))
+    wl = f"snu nv={nv} muscles={mb.nmuscle} entries={ne_} x {nworld} worlds"
+    sec = _timeit(torch, lambda i: Q.project_muscle_sparse_moment_qfrc(mom[i], frc[i], off_d, ord_d, em_d, mb.root_dof_count, qfrc), nsets, launches)
+    _line("im_muscle_project", wl, sec, bytes_=nworld * 4 * (ne_ + mb.nmuscle + nv - mb.root_dof_count), nworld=nworld)
+    prepared = Q.prepare_muscle_implicit_qderiv_pairs(
+        pair_entry_i=ent.pair_entry_i, pair_entry_j=ent.pair_entry_j, pair_muscle_idx=ent.pair_muscle_idx,
+        muscle_dof_torque_idx=ent.muscle_dof_torque_idx, matrix_elemid=synth.matrix_elemid(rowadr, rownnz, colind),
+        root_dof_count=mb.root_dof_count,
+    )  # fmt: skip
+    gather = Q.build_muscle_implicit_qderiv_gather(prepared, ent.muscle_dof_muscle_idx, dev)
+    qd = torch.zeros((nworld, nM), device=dev)
+    sec = _timeit(torch, lambda i: Q.apply_muscle_implicit_qderiv_gather(gather, mom[i], slope[i], mb.timestep, qd), nsets, launches)
+    touched = int(gather.elem_ids.numel())
+    _line("im_muscle_implicit_gather", wl, sec, bytes_=nworld * 4 * (ne_ + mb.nmuscle + 2 * touched), nworld=nworld)
+    rig = synth.make_muscle_rig()
+    layer = MuscleDynamicsLayer(rig.topology, **rig.dims(), device=dev)
+    ctx = [t(synth.make_muscle_context(rig, nworld, seed=s)) for s in range(4)]
+    act = torch.rand((nworld, rig.muscle_count), device=dev)
+    gout = torch.randn((nworld, rig.torque_dim), device=dev)
+    wl = (f"snu rig: {rig.muscle_count} muscles, {layer.waypoint_count} waypoints, {len(layer.segments_host[0])} applied "
+          f"segments, {len(layer.torque_entries_host[2])} torque entries x {nworld} worlds")  # fmt: skip
+    cbytes = 4 * layer.context_dim
+    sec = _timeit(torch, lambda i: layer._warp_muscle_dynamics_from_activation_forward(act, ctx[i], include_passive_force=True), 4, launches)
+    _line("torque_forward (waypoints + force magnitudes + im_muscle_torque_forward)", wl, sec,
+          bytes_=nworld * (cbytes + 4 * (3 * layer.waypoint_count * 2 + 3 * rig.muscle_count + rig.muscle_count + rig.torque_dim)), nworld=nworld)  # fmt: skip
+    sec = _timeit(torch, lambda i: layer._warp_muscle_dynamics_from_activation_backward(ctx[i], gout), 4, launches)
+    _line("torque_backward (waypoints + force magnitudes + im_muscle_activation_grad)", wl, sec,
+          bytes_=nworld * (cbytes + 4 * (3 * layer.waypoint_count * 2 + 2 * rig.muscle_count + rig.muscle_count + rig.torque_dim)), nworld=nworld)  # fmt: skip
+    sec = _timeit(torch, lambda i: layer.eval_muscle_sparse_moment(ctx[i]), 4, launches)
+    _line("eval_muscle_sparse_moment (waypoints + im_muscle_sparse_moment)", wl, sec,
+          bytes_=nworld * (cbytes + 4 * (3 * layer.waypoint_count * 2 + len(layer.sparse_entries.muscle_dof_torque_idx))), nworld=nworld)  # fmt: skip
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--launches", type=int, default=32)
+    run(ap.parse_args().launches)
