@@ -23,6 +23,9 @@
 // the same order.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+#include <cstring>
+
 #include "../../include/imhip.h"
 #include "common.h"
 
@@ -258,6 +261,154 @@ __global__ __launch_bounds__(256) void torque_bounds_kernel(
   upper[w * ldo + j] = hi;
 }
 
+// ---- one workgroup per world --------------------------------------------------------------
+// The four contractions above visit every applied segment once per (segment, dof) entry and
+// redo its square root and three divisions each time.  Here a workgroup first leaves each
+// segment's unit direction and its two lever vectors in LDS, then every thread evaluates
+// entries (same operations, same order as contribution()), and a last pass adds each output's
+// entries in list order.  Results equal the one-thread-per-output kernels bit for bit.
+enum { MW_FORWARD, MW_GRAD, MW_BOUNDS, MW_MOMENT };
+
+struct MwArgs {
+  Geo g;
+  Seg s;
+  const int32_t *offsets, *e_seg, *e_other, *row_torque;  // row_torque: MW_MOMENT only
+  const float *e_a, *e_b;
+  const float *unit, *passive, *act, *gout;
+  int64_t ldu, ldpa, lda, ldg;
+  float *out0, *out1;
+  int64_t ldo;
+  int root, nrow, nentry, nseg;
+};
+
+// force of one muscle as the contraction sees it
+template <int MODE>
+__device__ __forceinline__ float muscle_force(const MwArgs &a, int64_t w, int muscle) {
+  if (MODE == MW_FORWARD) {
+    float f = a.unit[w * a.ldu + muscle] * a.act[w * a.lda + muscle];
+    if (a.passive) f = f + a.passive[w * a.ldpa + muscle];
+    return f;
+  }
+  return a.unit[w * a.ldu + muscle];
+}
+
+template <int MODE>
+__device__ __forceinline__ float entry_contribution(const MwArgs &a, const float *segd,
+                                                    const unsigned short *rowid, const float *cdof,
+                                                    int64_t w, int e) {
+  const int r = rowid[e];
+  int torque, muscle;
+  if (MODE == MW_GRAD) { muscle = r; torque = a.e_other[e]; }
+  else if (MODE == MW_MOMENT) { muscle = 0; torque = a.row_torque[r]; }
+  else { torque = r; muscle = a.e_other[e]; }
+  float f = 1.0f;
+  if (MODE != MW_MOMENT) f = muscle_force<MODE>(a, w, muscle);
+  const float *cd = cdof + 6 * (int64_t)(torque + a.root);
+  const V3 ang = ld3(cd), lin = ld3(cd + 3);
+  const float *sd = segd + 9 * a.e_seg[e];
+  const V3 dir = {sd[0], sd[1], sd[2]}, r0 = {sd[3], sd[4], sd[5]}, r1 = {sd[6], sd[7], sd[8]};
+  const V3 fv = scale(f, dir);
+  const V3 st = add(lin, cross(ang, r0));
+  const V3 en = add(lin, cross(ang, r1));
+  // an entry whose force is zero is skipped by the reference: it enters the sum as 0
+  return f == 0.0f ? 0.0f : dot(sub(scale(a.e_a[e], st), scale(a.e_b[e], en)), fv);
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void muscle_world_kernel(MwArgs a) {
+  extern __shared__ float lds[];
+  float *segd = lds;                           // [nseg][9]: dir (0 for a degenerate segment), p0 - c0, p1 - c1
+  float *contrib = segd + 9 * a.nseg;          // [nentry]
+  unsigned short *rowid = (unsigned short *)(contrib + a.nentry);  // [nentry]
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int64_t w = blockIdx.x;
+  const float *wp = a.g.wp + w * a.g.ldw, *com = a.g.com + w * a.g.ldc, *cdof = a.g.cdof + w * a.g.ldd;
+  for (int sg = tid; sg < a.nseg; sg += nt) {
+    const V3 p0 = ld3(wp + 3 * a.s.p0[sg]), p1 = ld3(wp + 3 * a.s.p1[sg]);
+    const V3 c0 = ld3(com + 3 * a.s.b0[sg]), c1 = ld3(com + 3 * a.s.b1[sg]);
+    const V3 seg = sub(p1, p0);
+    const float len = length(seg);
+    const bool ok = !(len < 1.0e-8f);
+    const V3 r0 = sub(p0, c0), r1 = sub(p1, c1);
+    // a degenerate segment contributes nothing: with a zero direction its entries come out as
+    // +-0, and adding +-0 to a sum that started at +0 leaves every bit of it
+    float *o = segd + 9 * sg;
+    o[0] = ok ? seg.x / len : 0.0f;
+    o[1] = ok ? seg.y / len : 0.0f;
+    o[2] = ok ? seg.z / len : 0.0f;
+    o[3] = r0.x; o[4] = r0.y; o[5] = r0.z;
+    o[6] = r1.x; o[7] = r1.y; o[8] = r1.z;
+  }
+  for (int r = tid; r < a.nrow; r += nt)
+    for (int e = a.offsets[r]; e < a.offsets[r + 1]; ++e) rowid[e] = (unsigned short)r;
+  __syncthreads();
+  // four entries per thread and trip, each read from a clamped index so that all their loads
+  // are issued before the first is needed
+  for (int e = tid; e < a.nentry; e += 4 * nt) {
+    float c[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int ee = e + k * nt < a.nentry ? e + k * nt : a.nentry - 1;
+      c[k] = entry_contribution<MODE>(a, segd, rowid, cdof, w, ee);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (e + k * nt < a.nentry) contrib[e + k * nt] = c[k];
+  }
+  __syncthreads();
+  for (int r = tid; r < a.nrow; r += nt) {
+    const int e0 = a.offsets[r], e1 = a.offsets[r + 1];
+    if (MODE == MW_FORWARD) {
+      float total = 0.0f;
+      for (int e = e0; e < e1; ++e) total = total + contrib[e];
+      a.out0[w * a.ldo + r] = total;
+    } else if (MODE == MW_GRAD) {
+      float grad = 0.0f;
+      if (a.unit[w * a.ldu + r] != 0.0f)
+        for (int e = e0; e < e1; ++e) grad = grad + a.gout[w * a.ldg + a.e_other[e]] * contrib[e];
+      a.out0[w * a.ldo + r] = grad;
+    } else if (MODE == MW_MOMENT) {
+      float total = 0.0f;
+      for (int e = e0; e < e1; ++e) total = total + contrib[e];
+      a.out0[w * a.ldo + r] = total;
+    } else {
+      int current = -1;
+      float total = 0.0f, lo = 0.0f, hi = 0.0f;
+      for (int e = e0; e < e1; ++e) {
+        const int m = a.e_other[e];
+        if (current >= 0 && m != current) {
+          if (total < 0.0f) lo = lo + total;
+          else hi = hi + total;
+          total = 0.0f;
+        }
+        current = m;
+        total = total + contrib[e];
+      }
+      if (current >= 0) {
+        if (total < 0.0f) lo = lo + total;
+        else hi = hi + total;
+      }
+      a.out0[w * a.ldo + r] = lo;
+      a.out1[w * a.ldo + r] = hi;
+    }
+  }
+}
+
+// Launches the workgroup-per-world kernel when a world's segments and entries fit in LDS;
+// returns false for the caller to use the one-thread-per-output kernel instead.
+template <int MODE>
+bool launch_world(const MwArgs &a, int nworld, hipStream_t stream) {
+  const size_t lds_bytes = 4 * ((size_t)9 * a.nseg + (size_t)a.nentry) +
+                           2 * (((size_t)a.nentry + 1) & ~(size_t)1);
+  static const bool forced_off = [] {
+    const char *e = std::getenv("IMHIP_MUSCLE_KERNEL");
+    return e && std::strcmp(e, "simple") == 0;
+  }();
+  if (forced_off || lds_bytes > 64 * 1024 || a.nentry == 0 || a.nseg == 0 || a.nrow > 65535) return false;
+  hipLaunchKernelGGL(muscle_world_kernel<MODE>, dim3((unsigned)nworld), dim3(256), lds_bytes, stream, a);
+  return true;
+}
+
 bool geo_ok(const im_muscle_geometry *g) {
   return g && g->waypoints && g->subtree_com && g->cdof && g->ld_waypoints >= 0 &&
          g->ld_subtree_com >= 0 && g->ld_cdof >= 0;
@@ -357,6 +508,17 @@ extern "C" int im_muscle_torque_forward(const im_muscle_geometry *geometry,
                                      !torque_entries->start_coeff || !torque_entries->end_coeff))
     return IM_ERR_ARG;
   if (ld_torque < nt) return IM_ERR_STRIDE;
+  {
+    MwArgs a{geo(geometry), seg(segments), torque_entries->offsets, torque_entries->segment,
+             torque_entries->other, nullptr, torque_entries->start_coeff, torque_entries->end_coeff,
+             unit_force, passive_force, activation, nullptr, ld_unit, ld_passive, ld_activation, 0,
+             torque, nullptr, ld_torque, root_dof_count, nt, torque_entries->nentry,
+             segments->nsegment};
+    if (launch_world<MW_FORWARD>(a, nworld, (hipStream_t)stream)) {
+      IM_HIP_CHECK(hipGetLastError());
+      return IM_OK;
+    }
+  }
   IM_FOR_WORLD_SLABS(nworld, w0, nw) {
     hipLaunchKernelGGL(torque_forward_kernel, grid2(nt, nw), dim3(256), 0, (hipStream_t)stream,
                        slab(geometry, w0), seg(segments), torque_entries->offsets,
@@ -389,6 +551,17 @@ extern "C" int im_muscle_activation_grad(const im_muscle_geometry *geometry,
                                      !muscle_entries->start_coeff || !muscle_entries->end_coeff))
     return IM_ERR_ARG;
   if (ld_grad_activation < nm || ld_unit < nm) return IM_ERR_STRIDE;
+  {
+    MwArgs a{geo(geometry), seg(segments), muscle_entries->offsets, muscle_entries->segment,
+             muscle_entries->other, nullptr, muscle_entries->start_coeff, muscle_entries->end_coeff,
+             unit_force, nullptr, nullptr, grad_output, ld_unit, 0, 0, ld_grad_output,
+             grad_activation, nullptr, ld_grad_activation, root_dof_count, nm, muscle_entries->nentry,
+             segments->nsegment};
+    if (launch_world<MW_GRAD>(a, nworld, (hipStream_t)stream)) {
+      IM_HIP_CHECK(hipGetLastError());
+      return IM_OK;
+    }
+  }
   IM_FOR_WORLD_SLABS(nworld, w0, nw) {
     hipLaunchKernelGGL(activation_grad_kernel, grid2(nm, nw), dim3(256), 0, (hipStream_t)stream,
                        slab(geometry, w0), seg(segments), muscle_entries->offsets,
@@ -419,6 +592,16 @@ extern "C" int im_muscle_sparse_moment(const im_muscle_geometry *geometry,
                                      !entry_segments->end_coeff))
     return IM_ERR_ARG;
   if (ld_moment < ne) return IM_ERR_STRIDE;
+  {
+    MwArgs a{geo(geometry), seg(segments), entry_segments->offsets, entry_segments->segment, nullptr,
+             muscle_dof_torque_idx, entry_segments->start_coeff, entry_segments->end_coeff, nullptr,
+             nullptr, nullptr, nullptr, 0, 0, 0, 0, moment, nullptr, ld_moment, root_dof_count, ne,
+             entry_segments->nentry, segments->nsegment};
+    if (launch_world<MW_MOMENT>(a, nworld, (hipStream_t)stream)) {
+      IM_HIP_CHECK(hipGetLastError());
+      return IM_OK;
+    }
+  }
   IM_FOR_WORLD_SLABS(nworld, w0, nw) {
     hipLaunchKernelGGL(sparse_moment_kernel, grid2(ne, nw), dim3(256), 0, (hipStream_t)stream,
                        slab(geometry, w0), seg(segments), muscle_dof_torque_idx,
@@ -447,6 +630,16 @@ extern "C" int im_muscle_torque_bounds(const im_muscle_geometry *geometry,
                                      !torque_entries->start_coeff || !torque_entries->end_coeff))
     return IM_ERR_ARG;
   if (ld_bounds < nt) return IM_ERR_STRIDE;
+  {
+    MwArgs a{geo(geometry), seg(segments), torque_entries->offsets, torque_entries->segment,
+             torque_entries->other, nullptr, torque_entries->start_coeff, torque_entries->end_coeff,
+             unit_force, nullptr, nullptr, nullptr, ld_unit, 0, 0, 0, lower, upper, ld_bounds,
+             root_dof_count, nt, torque_entries->nentry, segments->nsegment};
+    if (launch_world<MW_BOUNDS>(a, nworld, (hipStream_t)stream)) {
+      IM_HIP_CHECK(hipGetLastError());
+      return IM_OK;
+    }
+  }
   IM_FOR_WORLD_SLABS(nworld, w0, nw) {
     hipLaunchKernelGGL(torque_bounds_kernel, grid2(nt, nw), dim3(256), 0, (hipStream_t)stream,
                        slab(geometry, w0), seg(segments), torque_entries->offsets,

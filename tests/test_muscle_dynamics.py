@@ -543,3 +543,24 @@ def test_gpu_edge_cases():
         layer._warp_muscle_dynamics_from_activation_forward(
             torch.ones(5, 3, device="cuda"), wide[:, :20].contiguous(), include_passive_force=False
         )
+
+
+@pytest.mark.gpu
+def test_gpu_one_thread_per_output_kernels_agree():
+    """The contractions have two kernels each (a workgroup per world with the segments staged in
+    LDS, and one thread per output for models that do not fit): the second one is forced here
+    in a child process and must pass the same oracle comparison."""
+    import os
+    import subprocess
+    import sys
+
+    env = dict(os.environ, IMHIP_MUSCLE_KERNEL="simple")
+    code = (
+        "import sys; sys.path.insert(0, 'tests'); import test_muscle_dynamics as t;"
+        "t.test_gpu_geometry_forward_backward_match_oracle('gaussian', 'exponential', 67);"
+        "t.test_gpu_sparse_moment_matches_oracle_and_feeds_the_projection();"
+        "t.test_gpu_cached_force_ops_and_bounds(); print('simple kernels ok')"
+    )
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "simple kernels ok" in out.stdout, out.stderr[-2000:]
