@@ -13,6 +13,7 @@
 // order in which a team sums an entry's terms is the reference's.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -24,6 +25,10 @@ struct im_sparse_plan {
   int ntables = 0;
   const int32_t *t[22] = {};
   int sizes[22] = {};
+  // per lane of the lower-triangle 16 x 16 accumulator tiles: where the element comes from in a
+  // row of M and which slot it is ((M index + 1) << 16 | (slot + 1)); null when nv > 64
+  int32_t *tile_index = nullptr;
+  int nM = 0;
 };
 
 namespace im {
@@ -39,13 +44,30 @@ struct SparseDev {
 
 __device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 
-// level-scheduled numeric factor: team lanes stride an entry's terms, shuffle-down tree
+// Orders LDS writes before later reads: across the workgroup, or, when a world belongs to
+// one wavefront (WAVE), across that wavefront only.
+template <bool WAVE>
+__device__ __forceinline__ void sync_world() {
+  if (WAVE) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  } else {
+    __syncthreads();
+  }
+}
+
+// level-scheduled numeric factor: team lanes stride an entry's terms, shuffle-down tree.
+// An entry's value depends on its team width only, not on how many teams work side by side,
+// so `block` may be any multiple of the widest team.
+template <bool WAVE = false>
 __device__ __forceinline__ void factor_levels(const SparseDev &P, float *N, float *iD, int lane, int block) {
   const int32_t *LPt = P.t[LP], *LTt = P.t[LT], *ESt = P.t[ES], *ECt = P.t[EC], *RPt = P.t[RP];
   const uint32_t *RABt = (const uint32_t *)P.t[RAB], *RKLt = (const uint32_t *)P.t[RKL];
   for (int l = 0; l < P.nlevels; ++l) {
     const int e0 = LPt[l], e1 = LPt[l + 1], T = LTt[l];
-    const int tl = lane & (T - 1), team = lane / T, teams = block / T;
+    const int tshift = __builtin_ctz((unsigned)T);  // team widths are powers of two
+    const int tl = lane & (T - 1), team = lane >> tshift, teams = block >> tshift;
     for (int eb = e0; eb < e1; eb += teams) {
       const int e = eb + team;
       float v = 0.0f;
@@ -67,28 +89,31 @@ __device__ __forceinline__ void factor_levels(const SparseDev &P, float *N, floa
         if (col >= 0) iD[col] = 1.0f / wv;
       }
     }
-    __syncthreads();
+    sync_world<WAVE>();
   }
 }
 
-// backward pushes by level (root first), search = -x, (x.x, g.x) reduced warp then block
+// backward pushes by level (root first), search = -x, (x.x, g.x) reduced warp then block.
+// `nthreads` lanes work on the world; the two dot products are summed as a block of `block`
+// lanes would (the plan's width: it fixes which terms a lane adds and in which order).
+template <bool WAVE = false>
 __device__ __forceinline__ void backward_sums(const SparseDev &P, float *N, const float *iD,
                                               const float *__restrict__ gw, float *__restrict__ search,
                                               float *red, float *search_dot, float *decrement, int lane,
-                                              int block) {
+                                              int nthreads, int block) {
   const int n = P.nv, rhs = P.nslots - n, nw = (block + 31) / 32;
   const int32_t *ORIGt = P.t[ORIG];
   // backward solve, root level first
   const int32_t *BLt = P.t[BL], *BSt = P.t[BS], *BIt = P.t[BI], *BJt = P.t[BJ];
   for (int l = 0; l < P.nlevels; ++l) {
-    for (int p = BLt[l] + lane; p < BLt[l + 1]; p += block) {
+    for (int p = BLt[l] + lane; p < BLt[l + 1]; p += nthreads) {
       const int i = BIt[p], j = BJt[p];
       N[rhs + j] = fma_(-N[BSt[p]], N[rhs + i] * iD[i], N[rhs + j]);
     }
-    __syncthreads();
+    sync_world<WAVE>();
   }
   float s0 = 0.0f, s1 = 0.0f;
-  for (int j = lane; j < n; j += block) {
+  for (int j = lane; j < n && lane < block; j += block) {
     const int d = ORIGt[j];
     const float v = N[rhs + j] * iD[j];
     search[d] = -v;
@@ -99,11 +124,11 @@ __device__ __forceinline__ void backward_sums(const SparseDev &P, float *N, cons
     s0 = s0 + __shfl_down(s0, o, 32);
     s1 = s1 + __shfl_down(s1, o, 32);
   }
-  if ((lane & 31) == 0) {
+  if ((lane & 31) == 0 && lane < block) {
     red[lane >> 5] = s0;
     red[nw + (lane >> 5)] = s1;
   }
-  __syncthreads();
+  sync_world<WAVE>();
   if (lane == 0) {
     float ra = 0.0f, rb = 0.0f;
     for (int i = 0; i < nw; ++i) {
@@ -194,7 +219,192 @@ __global__ void sparse_init_kernel(SparseDev P, const uint8_t *__restrict__ done
   factor_levels(P, N, iD, lane, block);
   for (int s = lane; s < nfac; s += block) U[nfac + s] = N[s];
   for (int j = lane; j < n; j += block) U[2 * nfac + j] = iD[j];
-  backward_sums(P, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, block);
+  backward_sums(P, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, block, block);
+}
+
+// ---- initial factor, one wavefront per world --------------------------------------------
+// Four worlds per workgroup share one LDS copy of the factor and solve tables; each world
+// belongs to one wavefront, so its LDS traffic needs no workgroup barrier.  J'DJ is summed
+// on the matrix cores: v_mfma_f32_16x16x4_f32 adds its four products to the accumulator one
+// after the other with a fused multiply-add each, rows ascending, which is the order and
+// rounding of `v = fmaf(J[r][a] * Dc[r], J[r][b], v)` when one operand is the rounded
+// product J[r][a] * Dc[r]; the accumulators start from M.  The lower-triangle 16 x 16 tiles
+// hold every (a, b) pair, and the plan's slots pick theirs (pairs outside the pattern are
+// dropped, as in the reference, and their rows counted).
+constexpr int kStaged = 12;  // tables LP .. BJ, the ones the factor and the solves read
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+struct SparseWave {
+  SparseDev P;
+  int staged[kStaged];        // offsets in words from the first table (the plan stores them back to back)
+  int staged_words;           // length of that stretch, a multiple of 4
+  const int32_t *tile_index;  // [tile][4][64]: (index into M + 1) << 16 | (slot + 1), 0 = none
+  int block, nM;              // the plan's block width; length of a row of M
+};
+
+template <int NT>
+__global__ __launch_bounds__(256, NT >= 4 ? 3 : 4) void sparse_init_mfma_kernel(
+    SparseWave A, const uint8_t *__restrict__ done, const int32_t *__restrict__ nefc_p,
+    const float *__restrict__ J, int njmax, const float *__restrict__ D,
+    const int32_t *__restrict__ state, int quad, const float *__restrict__ M, int ldM,
+    const float *__restrict__ grad, int ldg, float *__restrict__ U_, float *__restrict__ search_,
+    float *__restrict__ search_dot, float *__restrict__ decrement, int nworld) {
+  constexpr int NTILE = NT * (NT + 1) / 2, PD = NT >= 4 ? 5 : NT == 3 ? 6 : 8;
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, p = lane & 15, kq = lane >> 4;
+  SparseDev Q = A.P;
+  int32_t *tab = (int32_t *)lds;
+  {
+    // one flat copy, every load issued before the first store (up to 32 KB)
+    const int4 *src = (const int4 *)A.P.t[0];
+    const int nvec = A.staged_words >> 2;
+    int4 buf[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = i * 256 + tid;
+      buf[i] = src[q < nvec ? q : nvec - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = i * 256 + tid;
+      if (q < nvec) ((int4 *)tab)[q] = buf[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kStaged; ++i) Q.t[i] = tab + A.staged[i];
+  const int off = A.staged_words;
+  __syncthreads();  // the only workgroup barrier: worlds are independent from here on
+  const int w = blockIdx.x * 4 + wv;
+  if (w >= nworld || (done && done[w])) return;
+  const int n = Q.nv, nslots = Q.nslots, nfac = nslots - n, rhs = nfac;
+  const int nw = (A.block + 31) / 32;
+  const int per_world = (nslots + n + 2 * nw + 3) & ~3;
+  float *N = lds + ((off + 3) & ~3) + wv * per_world;  // [nslots]; a row of M before the factor
+  float *iD = N + nslots;                              // [n]
+  float *red = iD + n;                                 // [2][nw]
+  float *U = U_ + (size_t)w * Q.nv_pad * Q.nv_pad;
+  const float *Mw = M + (size_t)w * ldM;
+  const float *gw = grad + (size_t)w * ldg;
+  const float *Jw = J + (size_t)w * njmax * n;
+  const float *Dw = D + (size_t)w * njmax;
+  const int32_t *sw = state + (size_t)w * njmax;
+  int ne = nefc_p[w];
+  ne = ne < njmax ? ne : njmax;
+  ne = __builtin_amdgcn_readfirstlane(ne);
+  const int steps = (ne + 3) >> 2;
+
+  // Every load below is unconditional (clamped address, value selected afterwards) and what
+  // is needed first is requested first, so that each wait counts only the loads before it.
+  int tix[NTILE][4];
+#pragma unroll
+  for (int t = 0; t < NTILE; ++t)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) tix[t][v] = A.tile_index[(t * 4 + v) * 64 + lane];
+  float mv[16];
+#pragma unroll
+  for (int c = 0; c < 16; ++c) {
+    const int e = c * 64 + lane;
+    mv[c] = Mw[e < A.nM ? e : A.nM - 1];
+  }
+  int col[NT];
+  bool colok[NT];
+  unsigned long long pm[NT];
+  const int words = (n + 31) / 32;
+  const uint32_t *PMt = (const uint32_t *)Q.t[PM];
+#pragma unroll
+  for (int c = 0; c < NT; ++c) {
+    colok[c] = 16 * c + p < n;
+    col[c] = colok[c] ? 16 * c + p : n - 1;
+    const uint32_t lo = PMt[col[c] * words], hi = PMt[col[c] * words + (words > 1 ? 1 : 0)];
+    pm[c] = (unsigned long long)lo | (words > 1 ? (unsigned long long)hi << 32 : 0ull);
+  }
+  float g[PD][NT], gd[PD];
+  int gs[PD];
+#pragma unroll
+  for (int u = 0; u < PD; ++u) {
+    const int row = 4 * u + kq, rowc = row < njmax ? row : njmax - 1;
+#pragma unroll
+    for (int c = 0; c < NT; ++c) g[u][c] = Jw[(size_t)rowc * n + col[c]];
+    gd[u] = Dw[rowc];
+    gs[u] = sw[rowc];
+  }
+#pragma unroll
+  for (int c = 0; c < 16; ++c)
+    if (c * 64 + lane < A.nM) N[c * 64 + lane] = mv[c];
+  sync_world<true>();
+  f32x4 acc[NTILE];
+#pragma unroll
+  for (int t = 0; t < NTILE; ++t)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int mi = (tix[t][v] >> 16) - 1;
+      const float m = N[mi < 0 ? 0 : mi];
+      acc[t][v] = mi >= 0 ? m : 0.0f;
+    }
+  sync_world<true>();
+  int nbad = 0;
+  for (int s0 = 0; s0 < steps; s0 += PD) {
+#pragma unroll
+    for (int u = 0; u < PD; ++u) {
+      if (s0 + u < steps) {
+        const int row = 4 * (s0 + u) + kq;
+        const bool rv = row < ne;
+        const float d = (rv && gs[u] == quad) ? gd[u] : 0.0f;
+        float z[NT], e[NT];
+#pragma unroll
+        for (int c = 0; c < NT; ++c) {
+          z[c] = rv ? g[u][c] : 0.0f;
+          e[c] = z[c] * d;
+        }
+        {
+          int t = 0;
+#pragma unroll
+          for (int ti = 0; ti < NT; ++ti)
+#pragma unroll
+            for (int tj = 0; tj <= ti; ++tj, ++t)
+              acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(z[ti], e[tj], acc[t], 0, 0, 0);
+        }
+        // an active row whose dofs do not all lie in one another's pattern row is counted
+        unsigned long long rmask = 0ull;
+#pragma unroll
+        for (int c = 0; c < NT; ++c) {
+          const unsigned long long b = __ballot(d != 0.0f && colok[c] && z[c] != 0.0f);
+          rmask |= ((b >> (16 * kq)) & 0xFFFFull) << (16 * c);
+        }
+        bool outside = false;
+#pragma unroll
+        for (int c = 0; c < NT; ++c)
+          outside = outside || (colok[c] && ((rmask >> (16 * c + p)) & 1ull) && (rmask & ~pm[c]) != 0ull);
+        const unsigned long long ob = __ballot(outside);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) nbad += ((ob >> (16 * k)) & 0xFFFFull) != 0ull;
+        // next use of this register set
+        const int nrow = 4 * (s0 + u + PD) + kq, nrowc = nrow < njmax ? nrow : njmax - 1;
+#pragma unroll
+        for (int c = 0; c < NT; ++c) g[u][c] = Jw[(size_t)nrowc * n + col[c]];
+        gd[u] = Dw[nrowc];
+        gs[u] = sw[nrowc];
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < NTILE; ++t)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int sl = (A.tile_index[(t * 4 + v) * 64 + lane] & 0xFFFF) - 1;
+      if (sl >= 0) N[sl] = acc[t][v];
+    }
+  sync_world<true>();
+  for (int s = lane; s < nfac; s += 64) U[s] = N[s];
+  const int32_t *ORIGt = Q.t[ORIG];
+  for (int j = lane; j < n; j += 64) N[rhs + j] = gw[ORIGt[j]];
+  sync_world<true>();
+  factor_levels<true>(Q, N, iD, lane, 64);
+  for (int s = lane; s < nfac; s += 64) U[nfac + s] = N[s];
+  for (int j = lane; j < n; j += 64) U[2 * nfac + j] = iD[j];
+  backward_sums<true>(Q, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, 64,
+                      A.block);
+  if (nbad && lane == 0) atomicAdd(U + Q.nv_pad * Q.nv_pad - 1, (float)nbad);
 }
 
 // Per-iteration factor stage: changed rows' dof union, incremental update of packed H,
@@ -292,7 +502,7 @@ __global__ void sparse_update_kernel(SparseDev P, const uint8_t *__restrict__ do
       __syncthreads();
     }
   }
-  backward_sums(P, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, block);
+  backward_sums(P, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, block, block);
 }
 
 }  // namespace
@@ -328,6 +538,31 @@ int im_sparse_plan_create(int nv, int nv_pad, int block, int nslots, int nlevels
     return IM_ERR_HIP;
   }
   for (int i = 0; i < ntables; ++i) pl->t[i] = (const int32_t *)((char *)pl->blob + offs[i]);
+  const int nfac = nslots - nv;
+  if (nv <= 64 && sizes[im::SA] >= nfac && sizes[im::SB] >= nfac && sizes[im::SM] >= nfac && nslots < 65535) {
+    const int32_t *sa = tables[im::SA], *sb = tables[im::SB], *sm = tables[im::SM];
+    const int nt = (nv + 15) / 16;
+    std::vector<int32_t> tix((size_t)nt * (nt + 1) / 2 * 256, 0);
+    int nM = 1;
+    bool fits = true;
+    for (int sl = 0; sl < nfac; ++sl) {
+      const int a = sa[sl], b = sb[sl], e = sm[sl];  // a <= b: tile row b, tile column a
+      if (a < 0 || b < a || b >= nv || e >= 1024) { fits = false; break; }
+      nM = e + 1 > nM ? e + 1 : nM;
+      const int ti = b / 16, tj = a / 16, i = b % 16, j = a % 16;
+      const int t = ti * (ti + 1) / 2 + tj, lane = j + 16 * (i / 4), v = i % 4;
+      tix[((size_t)t * 4 + v) * 64 + lane] = ((e + 1) << 16) | (sl + 1);
+    }
+    if (fits) {
+      if (hipMalloc((void **)&pl->tile_index, tix.size() * 4) != hipSuccess ||
+          hipMemcpy(pl->tile_index, tix.data(), tix.size() * 4, hipMemcpyHostToDevice) != hipSuccess) {
+        im::set_hip_error(hipGetLastError());
+        im_sparse_plan_destroy(pl);
+        return IM_ERR_HIP;
+      }
+      pl->nM = nM;
+    }
+  }
   *out = pl;
   return IM_OK;
 }
@@ -335,6 +570,7 @@ int im_sparse_plan_create(int nv, int nv_pad, int block, int nslots, int nlevels
 void im_sparse_plan_destroy(im_sparse_plan *plan) {
   if (!plan) return;
   if (plan->blob) (void)hipFree(plan->blob);
+  if (plan->tile_index) (void)hipFree(plan->tile_index);
   delete plan;
 }
 
@@ -350,6 +586,38 @@ int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done, const
   for (int i = 0; i < im::NTABLES; ++i) P.t[i] = plan->t[i];
   P.nv = plan->nv; P.nv_pad = plan->nv_pad; P.nslots = plan->nslots; P.nlevels = plan->nlevels;
   const int n = plan->nv, words = (n + 31) / 32, nw = (plan->block + 31) / 32;
+  static const bool simple_only = [] {
+    const char *e = std::getenv("IMHIP_SPARSE_KERNEL");
+    return e && std::strcmp(e, "simple") == 0;
+  }();
+  if (plan->tile_index && !simple_only) {
+    im::SparseWave A;
+    A.P = P;
+    for (int i = 0; i < im::kStaged; ++i) A.staged[i] = (int)(plan->t[i] - plan->t[0]);
+    const size_t staged = (size_t)(plan->t[im::kStaged] - plan->t[0]);  // tables are padded to 16 bytes
+    A.staged_words = (int)staged;
+    A.tile_index = plan->tile_index;
+    A.block = plan->block;
+    A.nM = plan->nM;
+    const size_t per_world = ((size_t)plan->nslots + n + 2 * nw + 3) & ~(size_t)3;
+    const size_t wave_lds = 4 * (((staged + 3) & ~(size_t)3) + 4 * per_world);
+    if (wave_lds <= 64 * 1024 && staged <= 8192 && ldM >= plan->nM) {
+      const dim3 grid((unsigned)((nworld + 3) / 4)), wg(256);
+      const hipStream_t st = (hipStream_t)stream;
+#define IM_SPARSE_WAVE(NT)                                                                            \
+  hipLaunchKernelGGL(im::sparse_init_mfma_kernel<NT>, grid, wg, wave_lds, st, A, done, nefc, J, njmax, D, \
+                     state, quad, M, ldM, grad, ldg, hfactor, search, search_dot, decrement, nworld)
+      switch ((n + 15) / 16) {
+        case 1: IM_SPARSE_WAVE(1); break;
+        case 2: IM_SPARSE_WAVE(2); break;
+        case 3: IM_SPARSE_WAVE(3); break;
+        default: IM_SPARSE_WAVE(4); break;
+      }
+#undef IM_SPARSE_WAVE
+      IM_HIP_CHECK(hipGetLastError());
+      return IM_OK;
+    }
+  }
   const size_t lds_bytes = 4 * ((size_t)plan->nslots + n + 2 * nw + 4 * n + 4 + 4 * words + 4);
   if (lds_bytes > 64 * 1024) return IM_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(im::sparse_init_kernel, dim3(nworld), dim3(plan->block), lds_bytes, (hipStream_t)stream, P,
