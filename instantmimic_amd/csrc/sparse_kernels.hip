@@ -243,15 +243,16 @@ struct SparseWave {
 };
 
 template <int NT>
-__global__ __launch_bounds__(256, NT >= 4 ? 3 : 4) void sparse_init_mfma_kernel(
+__global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
     SparseWave A, const uint8_t *__restrict__ done, const int32_t *__restrict__ nefc_p,
     const float *__restrict__ J, int njmax, const float *__restrict__ D,
     const int32_t *__restrict__ state, int quad, const float *__restrict__ M, int ldM,
     const float *__restrict__ grad, int ldg, float *__restrict__ U_, float *__restrict__ search_,
     float *__restrict__ search_dot, float *__restrict__ decrement, int nworld) {
-  constexpr int NTILE = NT * (NT + 1) / 2, PD = NT >= 4 ? 5 : NT == 3 ? 6 : 8;
+  constexpr int NTILE = NT * (NT + 1) / 2, PD = NT >= 4 ? 4 : NT == 3 ? 6 : 8;
   extern __shared__ float lds[];
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, p = lane & 15, kq = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63, p = lane & 15, kq = lane >> 4;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: world data is addressed from scalar registers
   SparseDev Q = A.P;
   int32_t *tab = (int32_t *)lds;
   {
@@ -308,15 +309,20 @@ __global__ __launch_bounds__(256, NT >= 4 ? 3 : 4) void sparse_init_mfma_kernel(
   }
   int col[NT];
   bool colok[NT];
-  unsigned long long pm[NT];
   const int words = (n + 31) / 32;
   const uint32_t *PMt = (const uint32_t *)Q.t[PM];
 #pragma unroll
   for (int c = 0; c < NT; ++c) {
     colok[c] = 16 * c + p < n;
     col[c] = colok[c] ? 16 * c + p : n - 1;
-    const uint32_t lo = PMt[col[c] * words], hi = PMt[col[c] * words + (words > 1 ? 1 : 0)];
-    pm[c] = (unsigned long long)lo | (words > 1 ? (unsigned long long)hi << 32 : 0ull);
+  }
+  // dofs outside the pattern row of dof `lane` (none for lanes past the last dof)
+  unsigned long long npm;
+  {
+    const int dl = lane < n ? lane : n - 1;
+    const uint32_t lo = PMt[dl * words], hi = PMt[dl * words + (words > 1 ? 1 : 0)];
+    npm = ~((unsigned long long)lo | (words > 1 ? (unsigned long long)hi << 32 : 0ull));
+    if (lane >= n) npm = 0ull;
   }
   float g[PD][NT], gd[PD];
   int gs[PD];
@@ -324,7 +330,7 @@ __global__ __launch_bounds__(256, NT >= 4 ? 3 : 4) void sparse_init_mfma_kernel(
   for (int u = 0; u < PD; ++u) {
     const int row = 4 * u + kq, rowc = row < njmax ? row : njmax - 1;
 #pragma unroll
-    for (int c = 0; c < NT; ++c) g[u][c] = Jw[(size_t)rowc * n + col[c]];
+    for (int c = 0; c < NT; ++c) g[u][c] = Jw[rowc * n + col[c]];
     gd[u] = Dw[rowc];
     gs[u] = sw[rowc];
   }
@@ -364,34 +370,39 @@ __global__ __launch_bounds__(256, NT >= 4 ? 3 : 4) void sparse_init_mfma_kernel(
             for (int tj = 0; tj <= ti; ++tj, ++t)
               acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(z[ti], e[tj], acc[t], 0, 0, 0);
         }
-        // an active row whose dofs do not all lie in one another's pattern row is counted
-        unsigned long long rmask = 0ull;
+        // An active row whose dofs do not all lie in one another's pattern row is counted.  The
+        // four rows' supports are assembled from the ballots with scalar instructions; lane d
+        // then tests dof d of each row against the dofs outside its pattern row.
+        const bool dnz = d != 0.0f;
+        unsigned long long sup[4] = {0ull, 0ull, 0ull, 0ull};
 #pragma unroll
         for (int c = 0; c < NT; ++c) {
-          const unsigned long long b = __ballot(d != 0.0f && colok[c] && z[c] != 0.0f);
-          rmask |= ((b >> (16 * kq)) & 0xFFFFull) << (16 * c);
+          const unsigned long long b = __ballot(dnz & colok[c] & (z[c] != 0.0f));
+#pragma unroll
+          for (int k = 0; k < 4; ++k) sup[k] |= ((b >> (16 * k)) & 0xFFFFull) << (16 * c);
         }
-        bool outside = false;
 #pragma unroll
-        for (int c = 0; c < NT; ++c)
-          outside = outside || (colok[c] && ((rmask >> (16 * c + p)) & 1ull) && (rmask & ~pm[c]) != 0ull);
-        const unsigned long long ob = __ballot(outside);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) nbad += ((ob >> (16 * k)) & 0xFFFFull) != 0ull;
-        // next use of this register set
-        const int nrow = 4 * (s0 + u + PD) + kq, nrowc = nrow < njmax ? nrow : njmax - 1;
-#pragma unroll
-        for (int c = 0; c < NT; ++c) g[u][c] = Jw[(size_t)nrowc * n + col[c]];
-        gd[u] = Dw[nrowc];
-        gs[u] = sw[nrowc];
+        for (int k = 0; k < 4; ++k) nbad += (__ballot((sup[k] & npm) != 0ull) & sup[k]) != 0ull;
       }
+      // Next use of this register set.  Issued whether or not the step above ran, so that the
+      // number of loads in flight at every wait is the same on every path.
+      const int nrow = 4 * (s0 + u + PD) + kq, nrowc = nrow < njmax ? nrow : njmax - 1;
+#pragma unroll
+      for (int c = 0; c < NT; ++c) g[u][c] = Jw[nrowc * n + col[c]];
+      gd[u] = Dw[nrowc];
+      gs[u] = sw[nrowc];
     }
   }
+  // the slots of this lane's accumulator elements (all requested before the first is used)
+#pragma unroll
+  for (int t = 0; t < NTILE; ++t)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) tix[t][v] = A.tile_index[(t * 4 + v) * 64 + lane];
 #pragma unroll
   for (int t = 0; t < NTILE; ++t)
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      const int sl = (A.tile_index[(t * 4 + v) * 64 + lane] & 0xFFFF) - 1;
+      const int sl = (tix[t][v] & 0xFFFF) - 1;
       if (sl >= 0) N[sl] = acc[t][v];
     }
   sync_world<true>();
