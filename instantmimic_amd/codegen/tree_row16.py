@@ -135,6 +135,56 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     for row in idx_rows:
         emit("  {" + ",".join(str(v) for v in row) + "},")
     emit("};")
+    # Right-hand side as lane vectors: lane p of register set s holds the entry of the dof at
+    # position 16 s + p of the chain being eliminated, so that one fused multiply-add per set
+    # applies a step's update to every ancestor (same operation per entry as one per ancestor).
+    # A group's lanes at trunk positions are its zero-initialised accumulators.  A group with
+    # several branches reuses the lanes past the fork: `segs[j]` lists, per run of dofs on one
+    # chain, the lanes that take new dofs (a copy of the vector keeps the finished branch).
+    tpos = {a: t.depth[a] for a in trunk}
+    assert sorted(tpos.values()) == list(range(len(trunk))), "trunk is not a chain from the root"
+    # Per group: which owner (trunk accumulator ('t', a) or group dof ('g', b)) sits in which lane
+    # while each dof is eliminated.  A new segment starts when the chain of the next dof needs a
+    # lane for another owner: the lane then takes a fresh value (the dof's right-hand side, or
+    # zero for an accumulator) or the owner's value from the segment it was last resident in.
+    segs = []      # per group: list of dict(fresh={pos: dof or -1}, restore={pos: segment})
+    seg_of = {}    # group dof -> (group, segment it is eliminated in)
+    home = []      # per group: owner -> segment whose vector holds its final value
+    for j, g in enumerate(groups):
+        lane_owner, hm_, lst = {}, {}, []
+        for k in g:
+            want = {t.depth[a]: (("t", a) if a in trunk_set else ("g", a)) for a in t.chain[k]}
+            if any(lane_owner.get(pos) != own for pos, own in want.items()):
+                seg = {"fresh": {}, "restore": {}}
+                for pos, own in want.items():
+                    if lane_owner.get(pos) == own:
+                        continue
+                    if own in hm_:
+                        seg["restore"][pos] = hm_[own]
+                    else:
+                        seg["fresh"][pos] = own[1] if own[0] == "g" else -1
+                    lane_owner[pos] = own
+                lst.append(seg)
+            for own in lane_owner.values():
+                hm_[own] = len(lst) - 1
+            seg_of[k] = (j, len(lst) - 1)
+        segs.append(lst)
+        home.append(hm_)
+    vsets = [max(t.sets(k) for k in g) for g in groups]
+    tsets = max(t.sets(k) for k in trunk) if len(trunk) else 1
+    svi_rows, svi_of = [], {}
+    for j in range(ngroups):
+        for i, take in enumerate(segs[j]):
+            for s_ in range(vsets[j]):
+                svi_of[j, i, s_] = len(svi_rows)
+                svi_rows.append([take["fresh"].get(16 * s_ + p, -1) for p in range(16)])
+    for s_ in range(tsets):
+        svi_of["T", 0, s_] = len(svi_rows)
+        svi_rows.append([trunk[16 * s_ + p] if 16 * s_ + p < len(trunk) else -1 for p in range(16)])
+    emit(f"static __device__ const signed char SVI_{name}[{len(svi_rows)}][16] = {{")
+    for row in svi_rows:
+        emit("  {" + ",".join(str(v) for v in row) + "},")
+    emit("};")
     # LONG: more constraint rows than the straight-line assembly keeps in flight (a loop instead)
     emit("template <bool ASM, bool LONG>")
     emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? IM_OCC_{name} : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
@@ -148,14 +198,28 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     # the solve-only kernel is one wavefront that takes every role in turn
     emit("  #define ROLE(j) (!ASM || wv == (j))")
     emit("  float " + ", ".join(f"S{b} = 0.0f" for b in range(nv)) + ";")
-    for j, g in enumerate(groups):
+
+    def sv(j, i, s_):
+        return f"SVT_{s_}" if j == "T" else f"SV{j}_{i}_{s_}"
+
+    def load_sv(j, i, s_, var):
+        emit(f"    {{ const int ix = SVI_{name}[{svi_of[j, i, s_]}][p]; const float yv = yw[ix < 0 ? 0 : ix];"
+             f" {var} = ix >= 0 ? yv : 0.0f; }}")
+
+    for j in range(ngroups):
+        names = [sv(j, i, s_) for i in range(len(segs[j])) for s_ in range(vsets[j])]
+        names += [f"SY{j}_{i}_{s_}" for i in range(1, len(segs[j])) for s_ in range(vsets[j])]
+        names += [f"SP{j}_{s_}" for s_ in range(vsets[j])]
+        emit("  float " + ", ".join(f"{n_} = 0.0f" for n_ in names) + ";")
         emit(f"  if (ROLE({j})) {{")
-        for b in sorted(g):
-            emit(f"    S{b} = yw[{b}];")
+        for i in range(len(segs[j])):
+            for s_ in range(vsets[j]):
+                load_sv(j, i, s_, sv(j, 0, s_) if i == 0 else f"SY{j}_{i}_{s_}")
         emit("  }")
+    emit("  float " + ", ".join(f"SVT_{s_} = 0.0f" for s_ in range(tsets)) + ";")
     emit("  if (ROLE(0)) {")
-    for b in trunk:
-        emit(f"    S{b} = yw[{b}];")
+    for s_ in range(tsets):
+        load_sv("T", 0, s_, f"SVT_{s_}")
     emit("  }")
     emit("  float " + ", ".join(f"h{b}_{s}" for b in range(nv) for s in range(t.sets(b))) + ";")
     # ---- assembly on the matrix cores: wavefront v of the workgroup assembles world v of the four
@@ -179,7 +243,9 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             for s_ in range(t.sets(a)):
                 sl[a, s_] = xoff
                 xoff += 64
-            sl[a, "S"] = xoff
+
+        for s_ in range(vsets[j]):
+            sl["S", s_] = xoff
             xoff += 64
         xslots.append(sl)
     xs_off = xoff
@@ -308,8 +374,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         # the compiler keep two copies of every accumulator
         emit(f"      if (s0 + {u} < steps) {{")
         consume(u, f"s0 + {u}")
-        load(u, f"s0 + {u + PD}")
         emit("      }")
+        # the next use of the register set is requested on every path: with the same number
+        # of loads in flight whatever steps ran, each wait counts only the loads before it
+        load(u, f"s0 + {u + PD}")
     emit("    }")
     emit("    }")
     emit("    STAMP();  // 2: assembled")
@@ -351,7 +419,6 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         for a in sorted(touched[j]):
             for s in range(t.sets(a)):
                 emit(f"  float ga{j}_{a}_{s} = 0.0f;")
-            emit(f"  float gs{j}_{a} = 0.0f;")
     for k in range(nv):
         emit(f"  float d{k} = 0.0f, nd{k} = 0.0f;")
         if t.depth[k]:
@@ -362,25 +429,41 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         c = t.depth[k]
         nset = t.sets(k)
         emit(f"    // eliminate dof {k}")
+        if j is not None and seg_of[k][1] > 0 and k == next(q for q in groups[j] if seg_of[q] == seg_of[k]):
+            # a new branch of the group: its dofs take over the lanes past the fork
+            i = seg_of[k][1]
+            for s_ in range(vsets[j]):
+                expr = sv(j, i - 1, s_)
+                for src in sorted(set(segs[j][i]["restore"].values())):
+                    mask = sum(1 << p for p in range(16) if segs[j][i]["restore"].get(16 * s_ + p) == src)
+                    if mask:
+                        expr = f"((0x{mask:x} >> p) & 1) ? {sv(j, src, s_)} : ({expr})"
+                mask = sum(1 << p for p in range(16) if 16 * s_ + p in segs[j][i]["fresh"])
+                if mask:
+                    expr = f"((0x{mask:x} >> p) & 1) ? SY{j}_{i}_{s_} : ({expr})"
+                emit(f"    {sv(j, i, s_)} = {expr};")
         emit(f"    d{k} = 1.0f / {bc(f'h{k}_{c // 16}', c % 16)};")
         emit(f"    nd{k} = -d{k};")
         if c == 0:
             return
-        # products m_kp * m_kq for every target register, then the right-hand side updates
+        vec = (lambda s_: sv(*seg_of[k], s_)) if j is not None else (lambda s_: sv("T", 0, s_))
+        # products m_kp * m_kq for every target register, then the right-hand side update
         prods = []  # (pp, s, target)
         for pp in range(c):
             a = t.anc[k][pp]
             to_acc = j is not None and a in trunk_set
             for s in range(t.sets(a)):
                 prods.append((pp, s, f"ga{j}_{a}_{s}" if to_acc else f"h{a}_{s}"))
-        rhs = []  # (pp, target)
-        for pp in range(c):
-            a = t.anc[k][pp]
-            rhs.append((pp, f"gs{j}_{a}" if (j is not None and a in trunk_set) else f"S{a}"))
+        # lanes at and past the dof's own position must not take part in the right-hand side
+        # update (they hold other dofs' entries), and there the row register holds no data
+        nsv = (c - 1) // 16 + 1
+        for s_ in range(nsv):
+            hi = c - 16 * s_
+            emit(f"    const float hm{k}_{s_} = p < {hi} ? h{k}_{s_} : 0.0f;")
         if prods:
             emit("    float " + ", ".join(f"t{k}_{pp}_{s}" for pp, s, _ in prods) + ";")
         # statement 1: T = h * nd, then as many products as fit; later statements: the rest
-        work = [("T", s) for s in range(nset)] + [("P", pp, s) for pp, s, _ in prods] + [("R", pp, tg) for pp, tg in rhs]
+        work = [("T", s) for s in range(nsv)] + [("P", pp, s) for pp, s, _ in prods] + [("R", s) for s in range(nsv)]
         pos = 0
         while pos < len(work):
             o, n_in, lines = [], [], ["s_nop 1"]
@@ -396,18 +479,18 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             while pos < len(work):
                 it = work[pos]
                 if it[0] == "T":
-                    need_i = (("h", it[1]) not in num) + ("nd" not in num)
+                    need_i = (("hm", it[1]) not in num) + ("nd" not in num)
                 elif it[0] == "P":
                     need_i = (("h", it[1] // 16) not in num) + (("h", it[2]) not in num)
                 else:
-                    need_i = (("Tin", it[1] // 16) not in num and ("T", it[1] // 16) not in num) + ("Sk" not in num)
+                    need_i = (("Tin", it[1]) not in num and ("T", it[1]) not in num) + (("V", c // 16) not in num)
                 if len(o) + 1 + len(n_in) + need_i > 28:
                     break
                 if it[0] == "T":
                     s = it[1]
                     num[("T", s)] = ("o", len(o))
                     o.append(f'"=&v"(T{k}_{s})')
-                    use_in(("h", s), f'"v"(h{k}_{s})')
+                    use_in(("hm", s), f'"v"(hm{k}_{s})')
                     use_in("nd", f'"v"(nd{k})')
                 elif it[0] == "P":
                     _, pp, s = it
@@ -416,12 +499,15 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
                     use_in(("h", pp // 16), f'"v"(h{k}_{pp // 16})')
                     use_in(("h", s), f'"v"(h{k}_{s})')
                 else:
-                    _, pp, tg = it
-                    num[("S", pp)] = ("o", len(o))
-                    o.append(f'"+v"({tg})')
-                    if ("T", pp // 16) not in num:
-                        use_in(("Tin", pp // 16), f'"v"(T{k}_{pp // 16})')
-                    use_in("Sk", f'"v"(S{k})')
+                    _, s = it
+                    if ("V", s) not in num:
+                        num[("V", s)] = ("o", len(o))
+                        o.append(f'"+v"({vec(s)})')
+                    if ("V", c // 16) not in num:
+                        num[("V", c // 16)] = ("o", len(o))
+                        o.append(f'"+v"({vec(c // 16)})')
+                    if ("T", s) not in num:
+                        use_in(("Tin", s), f'"v"(T{k}_{s})')
                 items.append(it)
                 pos += 1
 
@@ -432,32 +518,39 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             wrote_T_at = None
             for it in items:
                 if it[0] == "T":
-                    lines.append(f"v_mul_f32 {r_(('T', it[1]))}, {r_(('h', it[1]))}, {r_('nd')}")
+                    lines.append(f"v_mul_f32 {r_(('T', it[1]))}, {r_(('hm', it[1]))}, {r_('nd')}")
                     wrote_T_at = len(lines)
                 elif it[0] == "P":
                     _, pp, s = it
                     lines.append(f"v_mul_f32_dpp {r_(('t', pp, s))}, {r_(('h', pp // 16))}, {r_(('h', s))} row_newbcast:{pp % 16} {DPP}")
                 else:
-                    _, pp, tg = it
-                    tsrc = ("T", pp // 16) if ("T", pp // 16) in num else ("Tin", pp // 16)
-                    if tsrc[0] == "T" and wrote_T_at is not None and len(lines) - wrote_T_at < 2:
-                        lines.append("s_nop 1")
-                    lines.append(f"v_fmac_f32_dpp {r_(('S', pp))}, {r_(tsrc)}, {r_('Sk')} row_newbcast:{pp % 16} {DPP}")
+                    _, s = it
+                    tsrc = ("T", s) if ("T", s) in num else ("Tin", s)
+                    # entry of dof k (lane c of its set, untouched by this update) times T, added per lane
+                    lines.append(f"v_fmac_f32_dpp {r_(('V', s))}, {r_(('V', c // 16))}, {r_(tsrc)} row_newbcast:{c % 16} {DPP}")
             text = "\\n\\t".join(lines)
             emit(f'    asm("{text}" : {", ".join(o)} : {", ".join(n_in)});')
         for pp, s, tgt in prods:
             emit(f"    {tgt} = IM_FMA(t{k}_{pp}_{s}, nd{k}, {tgt});")
 
     def backsub(b):
-        # u_b = u_b d_b, then u_b += T_b[p] u_anc_p for p ascending (tree_ldl.py:298-304)
-        emit(f"    S{b} = S{b} * d{b};")
+        # u_b = u_b d_b, then u_b += T_b[p] u_anc_p for p ascending (tree_ldl.py:298-304); the
+        # entry of dof b is lane c of its chain's right-hand side vector
         c = t.depth[b]
+        src = sv(seg_of[b][0], home[seg_of[b][0]]["g", b], c // 16) if b in seg_of else sv("T", 0, c // 16)
+        if c == 0:
+            emit(f"    S{b} = {bc(src, 0)} * d{b};")
+            return
         for p0 in range(0, c, 24):
             pps = list(range(p0, min(c, p0 + 24)))
             sets_used = sorted({pp // 16 for pp in pps})
-            o = [f'"+v"(S{b})']
+            first = p0 == 0
+            o = [f'"=&v"(S{b})' if first else f'"+v"(S{b})']
             n_in = [f'"v"(T{b}_{s})' for s in sets_used] + [f'"v"(S{t.anc[b][pp]})' for pp in pps]
             lines = ["s_nop 1"]
+            if first:
+                n_in += [f'"v"({src})', f'"v"(d{b})']
+                lines.append(f"v_mul_f32_dpp %0, %{len(n_in) - 1}, %{len(n_in)} row_newbcast:{c % 16} {DPP}")
             for n, pp in enumerate(pps):
                 lines.append(f"v_fmac_f32_dpp %0, %{1 + sets_used.index(pp // 16)}, %{1 + len(sets_used) + n} row_newbcast:{pp % 16} {DPP}")
             text = "\\n\\t".join(lines)
@@ -481,9 +574,19 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         fetch_rows(sorted(g))
         for k in g:
             eliminate(k, j)
+        for s_ in range(vsets[j]):
+            expr = sv(j, len(segs[j]) - 1, s_)
+            by_src = {}
+            for a_ in touched[j]:
+                if t.depth[a_] // 16 == s_ and home[j]["t", a_] != len(segs[j]) - 1:
+                    by_src.setdefault(home[j]["t", a_], 0)
+                    by_src[home[j]["t", a_]] |= 1 << (t.depth[a_] % 16)
+            for src, mask in sorted(by_src.items()):
+                expr = f"((0x{mask:x} >> p) & 1) ? {sv(j, src, s_)} : ({expr})"
+            emit(f"    SP{j}_{s_} = {expr};")
         emit("    if (ASM) {")
         for (a, s_), off in xslots[j].items():
-            src = f"gs{j}_{a}" if s_ == "S" else f"ga{j}_{a}_{s_}"
+            src = f"SP{j}_{s_}" if a == "S" else f"ga{j}_{a}_{s_}"
             emit(f"      xlds[{off} + lane] = {src};")
         emit("    }")
         emit("  }")
@@ -498,7 +601,12 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             if a in touched[j]:
                 for s in range(t.sets(a)):
                     emit(f"    h{a}_{s} = h{a}_{s} + (ASM ? xlds[{xslots[j][a, s]} + lane] : ga{j}_{a}_{s});")
-                emit(f"    S{a} = S{a} + (ASM ? xlds[{xslots[j][a, 'S']} + lane] : gs{j}_{a});")
+    # right-hand side: the lanes a group touched take its sums, in group order
+    for j in range(ngroups):
+        for s_ in range(min(tsets, vsets[j])):
+            mask = sum(1 << p for p in range(16) if any(t.depth[a] == 16 * s_ + p for a in touched[j]))
+            if mask:
+                emit(f"    SVT_{s_} = ((0x{mask:x} >> p) & 1) ? SVT_{s_} + (ASM ? xlds[{xslots[j]['S', s_]} + lane] : SP{j}_{s_}) : SVT_{s_};")
     for k in reversed(trunk):
         eliminate(k, None)
     for b in trunk:
