@@ -238,6 +238,8 @@ struct SparseWave {
   SparseDev P;
   int staged[kStaged];        // offsets in words from the first table (the plan stores them back to back)
   int staged_words;           // length of that stretch, a multiple of 4
+  int solve[5];               // update stage only: offsets of the forward-solve tables FL .. RK from FL
+  int solve_words;            // length of that stretch, a multiple of 4 (0: not staged)
   const int32_t *tile_index;  // [tile][4][64]: (index into M + 1) << 16 | (slot + 1), 0 = none
   int block, nM;              // the plan's block width; length of a row of M
 };
@@ -416,6 +418,197 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
   backward_sums<true>(Q, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, 64,
                       A.block);
   if (nbad && lane == 0) atomicAdd(U + Q.nv_pad * Q.nv_pad - 1, (float)nbad);
+}
+
+// Per-iteration factor stage, one wavefront per world (four worlds per workgroup share the LDS
+// copy of the factor and solve tables).  Same arithmetic as sparse_update_kernel below; the
+// changed constraint rows are staged in LDS (up to kStagedRows of them, else they are read from
+// memory), packed H is updated in LDS and written back whole, and a lane keeps four pairs'
+// table look-ups in flight.
+constexpr int kStagedRows = 16;
+
+__global__ __launch_bounds__(256, 4) void sparse_update_wave_kernel(
+    SparseWave A, const uint8_t *__restrict__ done, const int32_t *__restrict__ state_changes,
+    const int32_t *__restrict__ changes, const int32_t *__restrict__ ids, int ld_ids,
+    const float *__restrict__ J, int njmax, const float *__restrict__ D,
+    const int32_t *__restrict__ state, int quad, const float *__restrict__ grad, int ldg,
+    float *__restrict__ U_, int32_t *__restrict__ uni_, float *__restrict__ search_,
+    float *__restrict__ search_dot, float *__restrict__ decrement, int nworld) {
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  SparseDev Q = A.P;
+  int32_t *tab = (int32_t *)lds;
+  {
+    const int4 *src = (const int4 *)A.P.t[0];
+    const int nvec = A.staged_words >> 2;
+    int4 buf[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = i * 256 + tid;
+      buf[i] = src[q < nvec ? q : nvec - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = i * 256 + tid;
+      if (q < nvec) ((int4 *)tab)[q] = buf[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kStaged; ++i) Q.t[i] = tab + A.staged[i];
+  {
+    // forward-solve tables (at most 16 KB), behind the first stretch
+    const int4 *src = (const int4 *)A.P.t[FL];
+    const int nvec = A.solve_words >> 2;
+    int4 buf[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = i * 256 + tid;
+      buf[i] = src[q < nvec ? q : 0];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = i * 256 + tid;
+      if (q < nvec) ((int4 *)(tab + A.staged_words))[q] = buf[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 5; ++i) Q.t[FL + i] = tab + A.staged_words + A.solve[i];
+  }
+  __syncthreads();  // the only workgroup barrier
+  const int w = blockIdx.x * 4 + wv;
+  if (w >= nworld || (done && done[w]) || state_changes[w] == 0) return;
+  const int n = Q.nv, nslots = Q.nslots, nfac = nslots - n, rhs = nfac;
+  const int nw = (A.block + 31) / 32;
+  const int per_world = (nslots + n + 2 * nw + n + kStagedRows * (n + 1) + 3) & ~3;
+  float *N = lds + A.staged_words + A.solve_words + wv * per_world;  // [nslots]
+  float *iD = N + nslots;                            // [n]
+  float *red = iD + n;                               // [2][nw]
+  int *ul = (int *)(red + 2 * nw);                   // [n] ascending dofs touched by the changed rows
+  float *jr = (float *)(ul + n);                     // [kStagedRows][n] changed rows of J
+  float *sd = jr + kStagedRows * n;                  // [kStagedRows] D of the row, negated for a row that left the quadratic state
+  float *U = U_ + (size_t)w * Q.nv_pad * Q.nv_pad;
+  const float *gw = grad + (size_t)w * ldg;
+  const float *Jw = J + (size_t)w * njmax * n;
+  const float *Dw = D + (size_t)w * njmax;
+  const int32_t *sw = state + (size_t)w * njmax, *idw = ids + (size_t)w * ld_ids;
+  const int32_t *ORIGt = Q.t[ORIG];
+  int count = changes[w];
+  count = count < ld_ids ? count : ld_ids;
+  count = __builtin_amdgcn_readfirstlane(count);
+  if (count > 0) {
+    const bool staged = count <= kStagedRows;
+    // requests first: the changed rows, their weights, packed H
+    if (staged) {
+      const int tq = lane < count ? lane : count - 1;
+      const int rq = idw[tq];
+      const float dq = Dw[rq];
+      const int sq = sw[rq];
+      float rowv[kStagedRows];
+#pragma unroll
+      for (int t = 0; t < kStagedRows; ++t) {
+        const int r = __builtin_amdgcn_readlane(rq, t < count ? t : 0);
+        rowv[t] = Jw[r * n + (lane < n ? lane : n - 1)];
+      }
+      for (int s = lane; s < nfac; s += 64) N[s] = U[s];
+      if (lane < kStagedRows) sd[lane] = sq == quad ? dq : -dq;
+#pragma unroll
+      for (int t = 0; t < kStagedRows; ++t)
+        if (t < count && lane < n) jr[t * n + lane] = rowv[t];
+    } else {
+      for (int s = lane; s < nfac; s += 64) N[s] = U[s];
+    }
+    sync_world<true>();
+    // dofs touched by the changed rows, ascending (n <= 64: one ballot)
+    bool hit = false;
+    if (lane < n) {
+      if (staged) {
+        for (int t = 0; t < count; ++t) hit = hit || jr[t * n + lane] != 0.0f;
+      } else {
+        for (int t = 0; t < count && !hit; ++t) hit = Jw[idw[t] * n + lane] != 0.0f;
+      }
+    }
+    const unsigned long long mask = __ballot(hit);
+    const int nu = __popcll(mask);
+    if (hit) ul[__popcll(mask & ((1ull << lane) - 1ull))] = lane;
+    sync_world<true>();
+    int32_t *uni = uni_ + (size_t)w * (n + 1);
+    for (int i = lane; i < nu; i += 64) uni[i] = ul[i];
+    if (lane == 0) uni[n] = nu;
+    const int32_t *PAIRt = Q.t[PAIR];
+    const int npair = nu * (nu + 1) / 2;
+    int nbad = 0;
+    for (int e0 = lane; e0 < npair; e0 += 4 * 64) {
+      int row[4], col[4], sl[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int e = e0 + 64 * k < npair ? e0 + 64 * k : npair - 1;
+        // e = cj (cj + 1) / 2 + ri with ri <= cj, found exactly
+        int cj = (int)((sqrtf((float)(8 * e + 1)) - 1.0f) * 0.5f);
+        while ((cj + 1) * (cj + 2) / 2 <= e) ++cj;
+        while (cj * (cj + 1) / 2 > e) --cj;
+        row[k] = ul[e - cj * (cj + 1) / 2];
+        col[k] = ul[cj];
+        sl[k] = PAIRt[row[k] * n + col[k]];
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float delta = 0.0f;
+        if (staged) {
+          for (int t = 0; t < count; ++t) {
+            const float a = jr[t * n + row[k]], b = jr[t * n + col[k]];
+            const float da = sd[t] * a;
+            if (a != 0.0f && b != 0.0f) delta = fma_(da, b, delta);
+          }
+        } else {
+          for (int t = 0; t < count; ++t) {
+            const int r = idw[t];
+            const float a = Jw[r * n + row[k]], b = Jw[r * n + col[k]];
+            float da = Dw[r] * a;
+            if (sw[r] != quad) da = -da;
+            if (a != 0.0f && b != 0.0f) delta = fma_(da, b, delta);
+          }
+        }
+        if (e0 + 64 * k < npair && delta != 0.0f) {
+          if (sl[k] >= 0) N[sl[k]] = N[sl[k]] + delta;  // one pair per slot: no two lanes meet
+          else ++nbad;
+        }
+      }
+    }
+    for (int o = 32; o > 0; o >>= 1) nbad += __shfl_down(nbad, o, 64);
+    if (lane == 0 && nbad) atomicAdd(U + Q.nv_pad * Q.nv_pad - 1, (float)nbad);
+    sync_world<true>();
+    for (int s = lane; s < nfac; s += 64) U[s] = N[s];
+    for (int j = lane; j < n; j += 64) N[rhs + j] = gw[ORIGt[j]];
+    sync_world<true>();
+    factor_levels<true>(Q, N, iD, lane, 64);
+    for (int s = lane; s < nfac; s += 64) U[nfac + s] = N[s];
+    for (int j = lane; j < n; j += 64) U[2 * nfac + j] = iD[j];
+  } else {
+    float *gl = (float *)ul;  // [n] right-hand side in elimination order
+    for (int s = lane; s < nfac; s += 64) N[s] = U[nfac + s];
+    for (int j = lane; j < n; j += 64) {
+      iD[j] = U[2 * nfac + j];
+      gl[j] = gw[ORIGt[j]];
+    }
+    sync_world<true>();
+    const int32_t *FLt = Q.t[FL], *FRt = Q.t[FR], *RSt = Q.t[RS], *RKPt = Q.t[RKP], *RKt = Q.t[RK];
+    for (int l = 0; l < Q.nlevels; ++l) {
+      for (int q = FLt[l] + lane; q < FLt[l + 1]; q += 64) {
+        const int j = FRt[q];
+        float v = gl[j];
+        const float *rowp = N + RSt[j];
+        const int k0 = RKPt[j], k1 = RKPt[j + 1];
+        for (int t = 0; t < k1 - k0; ++t) {
+          const int k = RKt[k0 + t];
+          v = fma_(-(rowp[t] * iD[k]), N[rhs + k], v);
+        }
+        N[rhs + j] = v;
+      }
+      sync_world<true>();
+    }
+  }
+  backward_sums<true>(Q, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, 64,
+                      A.block);
 }
 
 // Per-iteration factor stage: changed rows' dof union, incremental update of packed H,
@@ -608,6 +801,7 @@ int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done, const
     const size_t staged = (size_t)(plan->t[im::kStaged] - plan->t[0]);  // tables are padded to 16 bytes
     A.staged_words = (int)staged;
     A.tile_index = plan->tile_index;
+    A.solve_words = 0;
     A.block = plan->block;
     A.nM = plan->nM;
     const size_t per_world = ((size_t)plan->nslots + n + 2 * nw + 3) & ~(size_t)3;
@@ -653,6 +847,34 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done, con
   for (int i = 0; i < im::NTABLES; ++i) P.t[i] = plan->t[i];
   P.nv = plan->nv; P.nv_pad = plan->nv_pad; P.nslots = plan->nslots; P.nlevels = plan->nlevels;
   const int n = plan->nv, nw = (plan->block + 31) / 32;
+  static const bool simple_only = [] {
+    const char *e = std::getenv("IMHIP_SPARSE_KERNEL");
+    return e && std::strcmp(e, "simple") == 0;
+  }();
+  if (n <= 64 && !simple_only) {
+    im::SparseWave A;
+    A.P = P;
+    for (int i = 0; i < im::kStaged; ++i) A.staged[i] = (int)(plan->t[i] - plan->t[0]);
+    const size_t staged = (size_t)(plan->t[im::kStaged] - plan->t[0]);
+    A.staged_words = (int)staged;
+    A.tile_index = nullptr;
+    A.block = plan->block;
+    A.nM = 0;
+    const size_t per_world =
+        ((size_t)plan->nslots + n + 2 * nw + n + (size_t)im::kStagedRows * (n + 1) + 3) & ~(size_t)3;
+    const int32_t *solve_end = plan->t[im::RK] + ((plan->sizes[im::RK] + 3) & ~3);
+    const size_t solve_words = (size_t)(solve_end - plan->t[im::FL]);
+    for (int i = 0; i < 5; ++i) A.solve[i] = (int)(plan->t[im::FL + i] - plan->t[im::FL]);
+    A.solve_words = (int)solve_words;
+    const size_t wave_lds = 4 * (staged + solve_words + 4 * per_world);
+    if (wave_lds <= 64 * 1024 && staged <= 8192 && solve_words <= 4096) {
+      hipLaunchKernelGGL(im::sparse_update_wave_kernel, dim3((unsigned)((nworld + 3) / 4)), dim3(256), wave_lds,
+                         (hipStream_t)stream, A, done, state_changes, changes, ids, ld_ids, J, njmax, D, state,
+                         quad, grad, ldg, hfactor, dof_union, search, search_dot, decrement, nworld);
+      IM_HIP_CHECK(hipGetLastError());
+      return IM_OK;
+    }
+  }
   const size_t lds_bytes = 4 * ((size_t)plan->nslots + n + 2 * nw + n);
   if (lds_bytes > 64 * 1024) return IM_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(im::sparse_update_kernel, dim3(nworld), dim3(plan->block), lds_bytes, (hipStream_t)stream, P,
