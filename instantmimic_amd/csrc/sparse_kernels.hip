@@ -79,7 +79,19 @@ __device__ __forceinline__ void factor_levels(const SparseDev &P, float *N, floa
           const uint32_t ab = RABt[r], kl = RKLt[r];
           const float *pa = N + (ab & 0xFFFFu), *pb = N + (ab >> 16), *pd = iD + (kl & 0xFFFFu);
           const int len = (int)(kl >> 16);
-          for (int t = tl; t < len; t += T) v = fma_(pa[t] * pb[t], pd[t], v);
+          // four terms' operands are read before the first is used; the sum keeps its order
+          int t = tl;
+          for (; t + 3 * T < len; t += 4 * T) {
+            const float a0 = pa[t], b0 = pb[t], d0 = pd[t];
+            const float a1 = pa[t + T], b1 = pb[t + T], d1 = pd[t + T];
+            const float a2 = pa[t + 2 * T], b2 = pb[t + 2 * T], d2 = pd[t + 2 * T];
+            const float a3 = pa[t + 3 * T], b3 = pb[t + 3 * T], d3 = pd[t + 3 * T];
+            v = fma_(a0 * b0, d0, v);
+            v = fma_(a1 * b1, d1, v);
+            v = fma_(a2 * b2, d2, v);
+            v = fma_(a3 * b3, d3, v);
+          }
+          for (; t < len; t += T) v = fma_(pa[t] * pb[t], pd[t], v);
         }
       }
       for (int off = T >> 1; off > 0; off >>= 1) v = v + __shfl_down(v, off, T);
@@ -598,7 +610,18 @@ __global__ __launch_bounds__(256, 4) void sparse_update_wave_kernel(
         float v = gl[j];
         const float *rowp = N + RSt[j];
         const int k0 = RKPt[j], k1 = RKPt[j + 1];
-        for (int t = 0; t < k1 - k0; ++t) {
+        int t = 0;
+        for (; t + 3 < k1 - k0; t += 4) {
+          const int ka = RKt[k0 + t], kb = RKt[k0 + t + 1], kc = RKt[k0 + t + 2], kd = RKt[k0 + t + 3];
+          const float ra = rowp[t], rb = rowp[t + 1], rc = rowp[t + 2], rd = rowp[t + 3];
+          const float ia = iD[ka], ib = iD[kb], ic = iD[kc], id = iD[kd];
+          const float xa = N[rhs + ka], xb = N[rhs + kb], xc = N[rhs + kc], xd = N[rhs + kd];
+          v = fma_(-(ra * ia), xa, v);
+          v = fma_(-(rb * ib), xb, v);
+          v = fma_(-(rc * ic), xc, v);
+          v = fma_(-(rd * id), xd, v);
+        }
+        for (; t < k1 - k0; ++t) {
           const int k = RKt[k0 + t];
           v = fma_(-(rowp[t] * iD[k]), N[rhs + k], v);
         }
