@@ -18,6 +18,22 @@ namespace im {
 namespace {
 
 __device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+// value of lane n (0..15) of the caller's row of 16 lanes, in every lane of that row
+template <int N>
+__device__ __forceinline__ float row_bcast_c(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x150 + N, 0xF, 0xF, true));
+}
+// n becomes a constant once the caller's loop is unrolled; the DPP control must be one
+__device__ __forceinline__ float row_bcast(float v, int n) {
+  switch (n) {
+#define IM_BCAST_CASE(N) case N: return row_bcast_c<N>(v);
+    IM_BCAST_CASE(0) IM_BCAST_CASE(1) IM_BCAST_CASE(2) IM_BCAST_CASE(3) IM_BCAST_CASE(4) IM_BCAST_CASE(5)
+    IM_BCAST_CASE(6) IM_BCAST_CASE(7) IM_BCAST_CASE(8) IM_BCAST_CASE(9) IM_BCAST_CASE(10) IM_BCAST_CASE(11)
+    IM_BCAST_CASE(12) IM_BCAST_CASE(13) IM_BCAST_CASE(14)
+#undef IM_BCAST_CASE
+    default: return row_bcast_c<15>(v);
+  }
+}
 
 // Where a tile element comes from.  Indexed: element ids into the world's CSR values, ids
 // >= nM read as zero, padded diagonal entries get +1 (mjw_step_optimized.py:932-941).
@@ -43,6 +59,19 @@ struct DenseSrc {
     const int row = kb * B + r, col = ib * B + c;
     // only the upper triangle is kept up to date: mirror it inside a diagonal tile
     if (row < nv && col < nv) return row <= col ? H[(size_t)row * pad + col] : H[(size_t)col * pad + row];
+    return row == col ? 1.0f : 0.0f;
+  }
+};
+
+// In place: the matrix already sits in the LDS array the factor is written to (upper triangle
+// valid, everything else zero); block row kb is read before the factor overwrites it.
+template <int B>
+struct LdsSrc {
+  const float *U;
+  int nv, pad;
+  __device__ __forceinline__ float load(int kb, int ib, int, int r, int c) const {
+    const int row = kb * B + r, col = ib * B + c;
+    if (row < nv && col < nv) return row <= col ? U[row * pad + col] : U[col * pad + row];
     return row == col ? 1.0f : 0.0f;
   }
 };
@@ -83,34 +112,28 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
       rhs[k + tid] = s;
     }
     __syncthreads();
-    // Cholesky of the diagonal tile and the forward solve of the right-hand side: wave 0
+    // Cholesky of the diagonal tile and the forward solve of the right-hand side: the first B
+    // lanes of wave 0, lane i holding row i in registers.  Column j's updates are applied to
+    // the columns to its right as soon as it is final (right-looking), which gives every
+    // element the same fused multiply-adds in the same order (q ascending) as the column-wise
+    // form  v = A[i][j]; for q < j: v = fma(-L[i][q], L[j][q], v)  while the next pivot waits
+    // for one of them only.  Values of other rows come through DPP row broadcasts.
     if (tid < 64) {
       const int i = tid;
+      float a[B];
+#pragma unroll
+      for (int j = 0; j < B; ++j) a[j] = A[(i < B ? i : 0) * B + j];
+      float s = rhs[k + (i < B ? i : 0)];
+#pragma unroll
       for (int j = 0; j < B; ++j) {
-        float v = 0.0f;
-        if (i >= j && i < B) {
-          v = A[i * B + j];
-          for (int q = 0; q < j; ++q) v = fma_(-L[i * B + q], L[j * B + q], v);
-        }
-        if (i == j) {
-          const float d = sqrtf(v);
-          L[j * B + j] = d;
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        if (i > j && i < B) L[i * B + j] = v * (1.0f / L[j * B + j]);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-      }
-      float s = i < B ? rhs[k + i] : 0.0f;
-      for (int j = 0; j < B; ++j) {
-        if (i == j) rhs[k + j] = s / L[j * B + j];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        if (i > j && i < B) s = fma_(-L[i * B + j], rhs[k + j], s);
+        const float d = sqrtf(row_bcast(a[j], j));
+        const float lj = i == j ? d : a[j] * (1.0f / d);  // rows below the diagonal; unused above
+        if (i >= j && i < B) L[i * B + j] = lj;
+        const float z = row_bcast(s, j) / d;
+        if (i == j) rhs[k + j] = z;
+        s = fma_(-lj, z, s);  // meaningful for i > j
+#pragma unroll
+        for (int jj = j + 1; jj < B; ++jj) a[jj] = fma_(-lj, row_bcast(lj, jj), a[jj]);
       }
     }
     __syncthreads();
@@ -235,13 +258,14 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
     const float *__restrict__ J, int njmax, const float *__restrict__ D, const int32_t *__restrict__ state,
     int quad, const float *__restrict__ grad, int64_t ldg, float *H_, float *U_,
     int32_t *__restrict__ uni_, float *__restrict__ search, int64_t lds_, float *__restrict__ search_dot,
-    float *__restrict__ decrement, int nv, int pad) {
+    float *__restrict__ decrement, int nv, int pad, int row_cap) {
   extern __shared__ float lds[];
   float *U = lds;             // [pad * pad]
   float *rhs = U + pad * pad; // [pad]
   float *A = rhs + pad;       // [(pad / B) * B * B]
   float *L = A + (pad / B) * B * B;  // [B * B]
   int *ul = (int *)(L + B * B);      // [nv] union list, [nv] = its length
+  float *jr = (float *)(ul + nv + 1);  // [row_cap][nv] changed rows of J, then [row_cap] signed weights
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
   if ((done && done[w]) || state_changes[w] == 0) return;
@@ -252,20 +276,73 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
   count = count < ld_ids ? count : ld_ids;
   for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? gw[i] : 0.0f;
   if (count > 0) {
+    // Up to row_cap changed rows of J and their signed weights are staged in LDS, H's upper
+    // triangle is brought into the LDS array of the factor, updated there, written back, and
+    // factored in place; more changed rows than that are read from memory pair by pair.
+    const bool staged = count <= row_cap;
+    float *sd = jr + (size_t)row_cap * nv;
+    if (staged) {
+      const int total = count * nv;
+      for (int q0 = tid; q0 < total; q0 += 4 * nt) {
+        float v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int q = q0 + k * nt < total ? q0 + k * nt : total - 1;
+          const int t = q / nv;
+          v[k] = Jw[(size_t)idw[t] * nv + (q - t * nv)];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (q0 + k * nt < total) jr[q0 + k * nt] = v[k];
+      }
+      for (int t = tid; t < count; t += nt) {
+        const int r = idw[t];
+        sd[t] = sw[r] == quad ? Dw[r] : -Dw[r];
+      }
+      // 16 bytes per lane and four requests in flight: a lone workgroup per CU needs that much
+      // outstanding to stream 4 pad^2 bytes
+      const int nvec = pad * pad / 4;  // pad is a multiple of 16
+      for (int i0 = tid; i0 < nvec; i0 += 4 * nt) {
+        float4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int i = i0 + k * nt < nvec ? i0 + k * nt : nvec - 1;
+          v[k] = ((const float4 *)Hw)[i];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int i = i0 + k * nt;
+          if (i < nvec) {
+            const int r = 4 * i / pad, c = 4 * i - r * pad;
+            float4 o;
+            o.x = (r < nv && c + 0 < nv && r <= c + 0) ? v[k].x : 0.0f;
+            o.y = (r < nv && c + 1 < nv && r <= c + 1) ? v[k].y : 0.0f;
+            o.z = (r < nv && c + 2 < nv && r <= c + 2) ? v[k].z : 0.0f;
+            o.w = (r < nv && c + 3 < nv && r <= c + 3) ? v[k].w : 0.0f;
+            ((float4 *)U)[i] = o;
+          }
+        }
+      }
+      __syncthreads();
+    }
     if (tid < 64) {
       int nu = 0;
       for (int base = 0; base < nv; base += 64) {
         const int dof = base + tid;
         bool hit = false;
-        if (dof < nv)
-          for (int t = 0; t < count && !hit; ++t) hit = Jw[(size_t)idw[t] * nv + dof] != 0.0f;
+        if (dof < nv) {
+          if (staged) {
+            for (int t = 0; t < count; ++t) hit = hit || jr[t * nv + dof] != 0.0f;
+          } else {
+            for (int t = 0; t < count && !hit; ++t) hit = Jw[(size_t)idw[t] * nv + dof] != 0.0f;
+          }
+        }
         const unsigned long long mask = __ballot(hit);
         if (hit) ul[nu + __popcll(mask & ((1ull << tid) - 1ull))] = dof;
         nu += __popcll(mask);
       }
       if (tid == 0) ul[nv] = nu;
     }
-    for (int i = tid; i < pad * pad; i += nt) U[i] = 0.0f;
     __syncthreads();
     const int nu = ul[nv];
     int32_t *uni = uni_ + w * (nv + 1);
@@ -278,18 +355,53 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
       while (cj * (cj + 1) / 2 > e) --cj;
       const int row = ul[e - cj * (cj + 1) / 2], col = ul[cj];
       float delta = 0.0f;
-      for (int t = 0; t < count; ++t) {
-        const int r = idw[t];
-        const float a = Jw[(size_t)r * nv + row], b = Jw[(size_t)r * nv + col];
-        float da = Dw[r] * a;
-        if (sw[r] != quad) da = -da;
-        if (a != 0.0f && b != 0.0f) delta = fma_(da, b, delta);
+      if (staged) {
+        int t = 0;
+        for (; t + 3 < count; t += 4) {  // four rows' operands read before the first is used
+          float a[4], b[4], d[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            a[k] = jr[(t + k) * nv + row];
+            b[k] = jr[(t + k) * nv + col];
+            d[k] = sd[t + k];
+          }
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const float da = d[k] * a[k];  // -(D a) == (-D) a exactly
+            if (a[k] != 0.0f && b[k] != 0.0f) delta = fma_(da, b[k], delta);
+          }
+        }
+        for (; t < count; ++t) {
+          const float a = jr[t * nv + row], b = jr[t * nv + col];
+          const float da = sd[t] * a;
+          if (a != 0.0f && b != 0.0f) delta = fma_(da, b, delta);
+        }
+        if (delta != 0.0f) {
+          const float h = U[row * pad + col] + delta;
+          U[row * pad + col] = h;
+          Hw[(size_t)row * pad + col] = h;
+        }
+      } else {
+        for (int t = 0; t < count; ++t) {
+          const int r = idw[t];
+          const float a = Jw[(size_t)r * nv + row], b = Jw[(size_t)r * nv + col];
+          float da = Dw[r] * a;
+          if (sw[r] != quad) da = -da;
+          if (a != 0.0f && b != 0.0f) delta = fma_(da, b, delta);
+        }
+        if (delta != 0.0f) Hw[(size_t)row * pad + col] = Hw[(size_t)row * pad + col] + delta;
       }
-      if (delta != 0.0f) Hw[(size_t)row * pad + col] = Hw[(size_t)row * pad + col] + delta;
     }
-    __syncthreads();  // this workgroup's own writes to H are read back below
-    const DenseSrc<B> src{Hw, nv, pad};
-    factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
+    if (staged) {
+      __syncthreads();
+      const LdsSrc<B> src{U, nv, pad};
+      factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
+    } else {
+      for (int i = tid; i < pad * pad; i += nt) U[i] = 0.0f;
+      __syncthreads();  // this workgroup's own writes to H are read back below
+      const DenseSrc<B> src{Hw, nv, pad};
+      factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
+    }
     // stored factor: the augmented column z = U'^-1 grad above the corner sqrt(1e30 - z.z)
     if (tid == 0) {
       float v = 1.0e30f;
@@ -305,11 +417,23 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
     }
     __syncthreads();  // rhs is overwritten by the backward solve
   } else {
-    for (int i = tid; i < pad * pad; i += nt) {
-      const int r = i / pad, c = i - r * pad;
-      float v = Uw[i];
-      if (c == pad - 1) v = r == pad - 1 ? 1.0f : 0.0f;  // drop the augmented column
-      U[i] = v;
+    const int nvec = pad * pad / 4;
+    for (int i0 = tid; i0 < nvec; i0 += 4 * nt) {
+      float4 v[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int i = i0 + k * nt < nvec ? i0 + k * nt : nvec - 1;
+        v[k] = ((const float4 *)Uw)[i];
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int i = i0 + k * nt;
+        if (i < nvec) {
+          const int r = 4 * i / pad, c = 4 * i - r * pad;
+          if (c + 3 == pad - 1) v[k].w = r == pad - 1 ? 1.0f : 0.0f;  // drop the augmented column
+          ((float4 *)U)[i] = v[k];
+        }
+      }
     }
     __syncthreads();
     forward_solve<B>(U, rhs, pad, tid);
@@ -481,15 +605,19 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
   if (nv_pad % 16) return IM_ERR_ARG;
   if (ldg < nv || ld_search < nv) return IM_ERR_STRIDE;
   constexpr int B = 16;
-  const size_t lds_bytes =
+  const size_t base_bytes =
       sizeof(float) * ((size_t)nv_pad * nv_pad + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + nv + 1);
-  if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
+  if (base_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
+  // room for up to 32 changed rows of J next to the factor, as far as the 160 KB of LDS reach
+  int row_cap = ld_ids < 32 ? ld_ids : 32;
+  while (row_cap > 0 && base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1) > 160 * 1024) --row_cap;
+  const size_t lds_bytes = base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1);
   auto fn = im::dense_update_factor_kernel<B>;
   if (lds_bytes > 64 * 1024)
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
                      ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, U, dof_union, search, ld_search,
-                     search_dot, decrement, nv, nv_pad);
+                     search_dot, decrement, nv, nv_pad, row_cap);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }
