@@ -9,7 +9,8 @@
 // spelled out and fixed (same convention as the CPU restatement it is tested against):
 //   U_jk' U_ji updates: sum over t ascending with fma from 0, then C = C - sum;
 //   Cholesky by columns, s = fma(-l, l, s), L[i][j] = v * (1 / L[j][j]);
-//   triangular solves column oriented (j ascending forward, r descending backward).
+//   triangular solves column oriented (j ascending forward, r descending backward), a pivot
+//   is applied as a multiplication by 1 / diagonal (the reciprocal is an exact division).
 #include <hip/hip_runtime.h>
 
 #include "common.h"
@@ -87,18 +88,46 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
     const int k = kb * B;
     // gather the whole block row kb..nblk-1 and subtract the finished block rows above
     const int ntile = nblk - kb;
-    for (int q = tid; q < ntile * BB; q += nt) {
-      const int tb = q / BB, e = q - tb * BB, r = e / B, c = e - r * B;
-      const int ib = kb + tb, i0 = ib * B;
-      float v = src.load(kb, ib, e, r, c);
-      for (int jb = 0; jb < kb; ++jb) {
-        const int j = jb * B;
-        float sum = 0.0f;
+    if constexpr (B == 16) {
+      // One wavefront per 16 x 16 tile, the sums over a finished block row on the matrix cores:
+      // v_mfma_f32_16x16x4_f32 adds its four products to the accumulator one after the other,
+      // each with a fused multiply-add, so four of them chained from zero are the sum over
+      // t = 0..15 ascending of the scalar form.
+      typedef float f32x4 __attribute__((ext_vector_type(4)));
+      const int lane = tid & 63, p = lane & 15, kq = lane >> 4;
+      for (int tb = tid >> 6; tb < ntile; tb += nt >> 6) {
+        const int ib = kb + tb, i0 = ib * B;
+        f32x4 v;
 #pragma unroll
-        for (int t = 0; t < B; ++t) sum = fma_(U[(j + t) * pad + k + r], U[(j + t) * pad + i0 + c], sum);
-        v = v - sum;
+        for (int i = 0; i < 4; ++i) v[i] = src.load(kb, ib, (4 * kq + i) * B + p, 4 * kq + i, p);
+        for (int jb = 0; jb < kb; ++jb) {
+          const int j = jb * B;
+          f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4) {
+            const float a = U[(j + 4 * s4 + kq) * pad + k + p], b = U[(j + 4 * s4 + kq) * pad + i0 + p];
+            sum = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, sum, 0, 0, 0);
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = v[i] - sum[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) A[tb * BB + (4 * kq + i) * B + p] = v[i];
       }
-      A[q] = v;
+    } else {
+      for (int q = tid; q < ntile * BB; q += nt) {
+        const int tb = q / BB, e = q - tb * BB, r = e / B, c = e - r * B;
+        const int ib = kb + tb, i0 = ib * B;
+        float v = src.load(kb, ib, e, r, c);
+        for (int jb = 0; jb < kb; ++jb) {
+          const int j = jb * B;
+          float sum = 0.0f;
+#pragma unroll
+          for (int t = 0; t < B; ++t) sum = fma_(U[(j + t) * pad + k + r], U[(j + t) * pad + i0 + c], sum);
+          v = v - sum;
+        }
+        A[q] = v;
+      }
     }
     if (tid < B) {
       float s = rhs[k + tid];
@@ -127,10 +156,14 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
 #pragma unroll
       for (int j = 0; j < B; ++j) {
         const float d = sqrtf(row_bcast(a[j], j));
-        const float lj = i == j ? d : a[j] * (1.0f / d);  // rows below the diagonal; unused above
+        const float rinv = 1.0f / d;
+        const float lj = i == j ? d : a[j] * rinv;  // rows below the diagonal; unused above
         if (i >= j && i < B) L[i * B + j] = lj;
-        const float z = row_bcast(s, j) / d;
-        if (i == j) rhs[k + j] = z;
+        const float z = row_bcast(s, j) * rinv;
+        if (i == j) {
+          rhs[k + j] = z;
+          L[B * B + j] = rinv;  // reciprocals of the pivots, behind the tile
+        }
         s = fma_(-lj, z, s);  // meaningful for i > j
 #pragma unroll
         for (int jj = j + 1; jj < B; ++jj) a[jj] = fma_(-lj, row_bcast(lj, jj), a[jj]);
@@ -150,7 +183,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
       for (int r = 0; r < B; ++r) col[r] = At[r * B + c];
 #pragma unroll
       for (int j = 0; j < B; ++j) {
-        const float z = col[j] / L[j * B + j];
+        const float z = col[j] * L[B * B + j];
         col[j] = z;
 #pragma unroll
         for (int i = j + 1; i < B; ++i) col[i] = fma_(-L[i * B + j], z, col[i]);
@@ -163,28 +196,29 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
   }
 }
 
-// rhs <- U^-1 rhs, block rows from the bottom.
+// rhs <- U^-1 rhs, block rows from the bottom.  The first B lanes of wave 0 hold one row of the
+// diagonal tile each; the solved entries travel through DPP row broadcasts.
 template <int B>
 __device__ __forceinline__ void backward_solve(const float *U, float *rhs, int pad, int tid) {
   for (int i0 = pad - B; i0 >= 0; i0 -= B) {
     if (tid < 64) {
-      const int r = tid;
-      float s = 0.0f;
-      if (r < B) {
-        s = rhs[i0 + r];
-        for (int j = i0 + B; j < pad; j += B) {
-          float sum = 0.0f;
+      const int r = tid < B ? tid : 0;
+      float s = rhs[i0 + r];
+      float urow[B];
 #pragma unroll
-          for (int t = 0; t < B; ++t) sum = fma_(U[(i0 + r) * pad + j + t], rhs[j + t], sum);
-          s = s - sum;
-        }
+      for (int c = 0; c < B; ++c) urow[c] = U[(i0 + r) * pad + i0 + c];
+      const float rinv = 1.0f / U[(i0 + r) * pad + i0 + r];
+      for (int j = i0 + B; j < pad; j += B) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < B; ++t) sum = fma_(U[(i0 + r) * pad + j + t], rhs[j + t], sum);
+        s = s - sum;
       }
+#pragma unroll
       for (int c = B - 1; c >= 0; --c) {
-        if (r == c) rhs[i0 + c] = s / U[(i0 + c) * pad + i0 + c];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        if (r < c) s = fma_(-U[(i0 + r) * pad + i0 + c], rhs[i0 + c], s);
+        const float x = row_bcast(s * rinv, c);
+        if (tid == c) rhs[i0 + c] = x;
+        s = fma_(-urow[c], x, s);  // meaningful for rows above c
       }
     }
     __syncthreads();
@@ -196,26 +230,24 @@ __device__ __forceinline__ void backward_solve(const float *U, float *rhs, int p
 template <int B>
 __device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pad, int tid) {
   for (int k = 0; k < pad; k += B) {
-    if (tid < B) {
-      float s = rhs[k + tid];
+    if (tid < 64) {
+      const int i = tid < B ? tid : 0;
+      float s = rhs[k + i];
+      float ucol[B];
+#pragma unroll
+      for (int j = 0; j < B; ++j) ucol[j] = U[(k + j) * pad + k + i];
+      const float rinv = 1.0f / U[(k + i) * pad + k + i];
       for (int j = 0; j < k; j += B) {
         float sum = 0.0f;
 #pragma unroll
-        for (int t = 0; t < B; ++t) sum = fma_(U[(j + t) * pad + k + tid], rhs[j + t], sum);
+        for (int t = 0; t < B; ++t) sum = fma_(U[(j + t) * pad + k + i], rhs[j + t], sum);
         s = s - sum;
       }
-      rhs[k + tid] = s;
-    }
-    __syncthreads();
-    if (tid < 64) {
-      const int i = tid;
-      float s = i < B ? rhs[k + i] : 0.0f;
+#pragma unroll
       for (int j = 0; j < B; ++j) {
-        if (i == j) rhs[k + j] = s / U[(k + j) * pad + k + j];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        if (i > j && i < B) s = fma_(-U[(k + j) * pad + k + i], rhs[k + j], s);
+        const float z = row_bcast(s * rinv, j);
+        if (tid == j) rhs[k + j] = z;
+        s = fma_(-ucol[j], z, s);  // meaningful for rows below j
       }
     }
     __syncthreads();
@@ -231,7 +263,7 @@ __global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
   float *U = lds;             // [pad * pad]
   float *rhs = U + pad * pad; // [pad]
   float *A = rhs + pad;       // [(nblk) * B * B] working tiles of the current block row
-  float *L = A + (pad / B) * B * B;  // [B * B] Cholesky factor of the diagonal block (lower)
+  float *L = A + (pad / B) * B * B;  // [B * B + B] Cholesky factor of the diagonal block (lower), 1 / pivots
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
   for (int i = tid; i < pad * pad; i += nt) U[i] = 0.0f;
@@ -263,8 +295,8 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
   float *U = lds;             // [pad * pad]
   float *rhs = U + pad * pad; // [pad]
   float *A = rhs + pad;       // [(pad / B) * B * B]
-  float *L = A + (pad / B) * B * B;  // [B * B]
-  int *ul = (int *)(L + B * B);      // [nv] union list, [nv] = its length
+  float *L = A + (pad / B) * B * B;  // [B * B + B]: lower factor of the diagonal tile, 1 / pivots
+  int *ul = (int *)(L + B * B + B);  // [nv] union list, [nv] = its length
   float *jr = (float *)(ul + nv + 1);  // [row_cap][nv] changed rows of J, then [row_cap] signed weights
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
@@ -567,7 +599,7 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
   if (pad % block_size || pad - nv >= block_size) return IM_ERR_ARG;
   if (ldy < nv || ldx < nv) return IM_ERR_STRIDE;
   const int B = block_size;
-  const size_t lds_bytes = sizeof(float) * ((size_t)pad * pad + pad + (size_t)(pad / B) * B * B + B * B);
+  const size_t lds_bytes = sizeof(float) * ((size_t)pad * pad + pad + (size_t)(pad / B) * B * B + B * B + B);
   if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   auto fn = B == 8 ? im::blocked_factor_solve_kernel<8> : im::blocked_factor_solve_kernel<16>;
   if (lds_bytes > 64 * 1024)
@@ -606,7 +638,7 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
   if (ldg < nv || ld_search < nv) return IM_ERR_STRIDE;
   constexpr int B = 16;
   const size_t base_bytes =
-      sizeof(float) * ((size_t)nv_pad * nv_pad + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + nv + 1);
+      sizeof(float) * ((size_t)nv_pad * nv_pad + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + B + nv + 1);
   if (base_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   // room for up to 32 changed rows of J next to the factor, as far as the 160 KB of LDS reach
   int row_cap = ld_ids < 32 ? ld_ids : 32;

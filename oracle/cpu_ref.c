@@ -570,9 +570,9 @@ int orc_sparse_update_factor(int nv, int nv_pad, int block, int nslots, int nlev
  *   cholesky (lower L, U = L'):  s = A[j][j]; s = fmaf(-L[j][k], L[j][k], s) k ascending;
  *                                L[j][j] = sqrtf(s); inv = 1 / L[j][j];
  *                                L[i][j] = (A[i][j] - fold_k L[i][k] L[j][k]) * inv
- *   lower solve L z = b:         column oriented, j ascending: z[j] = s[j] / L[j][j];
+ *   lower solve L z = b:         column oriented, j ascending: z[j] = s[j] * (1 / L[j][j]);
  *                                s[i] = fmaf(-L[i][j], z[j], s[i]) for i > j
- *   upper solve U x = b:         column oriented, r descending: x[r] = s[r] / U[r][r];
+ *   upper solve U x = b:         column oriented, r descending: x[r] = s[r] * (1 / U[r][r]);
  *                                s[t] = fmaf(-U[t][r], x[r], s[t]) for t < r */
 /* One tile element.  bidx != NULL: indexed gather from the CSR values with +1 on padded
  * diagonal entries; bidx == NULL: M is a dense (pad, pad) matrix whose rows and columns
@@ -628,7 +628,7 @@ static void blocked_factor_forward(int nv, int pad, int B, int nM, const float *
     for (int r = 0; r < B; ++r)
       for (int c = r; c < B; ++c) U[(k + r) * pad + k + c] = L[c * B + r];
     for (int j = 0; j < B; ++j) {
-      const float z = rhs[k + j] / L[j * B + j];
+      const float z = rhs[k + j] * (1.0f / L[j * B + j]);
       rhs[k + j] = z;
       for (int i = j + 1; i < B; ++i) rhs[k + i] = fmaf(-L[i * B + j], z, rhs[k + i]);
     }
@@ -646,7 +646,7 @@ static void blocked_factor_forward(int nv, int pad, int B, int nM, const float *
       }
       for (int c = 0; c < B; ++c)
         for (int j = 0; j < B; ++j) {
-          const float z = A[j * B + c] / L[j * B + j];
+          const float z = A[j * B + c] * (1.0f / L[j * B + j]);
           A[j * B + c] = z;
           for (int i = j + 1; i < B; ++i) A[i * B + c] = fmaf(-L[i * B + j], z, A[i * B + c]);
         }
@@ -666,7 +666,7 @@ static void blocked_backward(int pad, int B, const float *U, float *rhs) {
         rhs[i0 + r] = rhs[i0 + r] - sum;
       }
     for (int r = B - 1; r >= 0; --r) {
-      const float xv = rhs[i0 + r] / U[(i0 + r) * pad + i0 + r];
+      const float xv = rhs[i0 + r] * (1.0f / U[(i0 + r) * pad + i0 + r]);
       rhs[i0 + r] = xv;
       for (int t = 0; t < r; ++t) rhs[i0 + t] = fmaf(-U[(i0 + t) * pad + i0 + r], xv, rhs[i0 + t]);
     }
@@ -683,7 +683,7 @@ static void blocked_forward(int pad, int B, const float *U, float *rhs) {
         rhs[k + r] = rhs[k + r] - sum;
       }
     for (int j = 0; j < B; ++j) {
-      const float z = rhs[k + j] / U[(k + j) * pad + k + j];
+      const float z = rhs[k + j] * (1.0f / U[(k + j) * pad + k + j]);
       rhs[k + j] = z;
       for (int i = j + 1; i < B; ++i) rhs[k + i] = fmaf(-U[(k + j) * pad + k + i], z, rhs[k + i]);
     }
