@@ -36,20 +36,7 @@ __device__ __forceinline__ float row_bcast(float v, int n) {
   }
 }
 
-// Where a tile element comes from.  Indexed: element ids into the world's CSR values, ids
-// >= nM read as zero, padded diagonal entries get +1 (mjw_step_optimized.py:932-941).
-template <int B>
-struct IndexedSrc {
-  const float *Mw;
-  const int32_t *block_idx;
-  int nM, nv, nblk;
-  __device__ __forceinline__ float load(int kb, int ib, int e, int r, int c) const {
-    const int idx = block_idx[(size_t)(kb * nblk + ib) * (B * B) + e];
-    float v = idx < nM ? Mw[idx] : 0.0f;
-    if (ib == kb && (kb + 1) * B > nv && r == c && (nblk - 1) * B + r >= nv) v = v + 1.0f;
-    return v;
-  }
-};
+// Where a tile element comes from.
 // Dense: the upper triangle of a row-major (pad, pad) matrix (the lower one is never read);
 // rows and columns >= nv are the identity whatever the buffer holds there.
 template <int B>
@@ -76,6 +63,67 @@ struct LdsSrc {
     return row == col ? 1.0f : 0.0f;
   }
 };
+
+// The tiles were gathered into the LDS array of the factor beforehand, diagonal tiles in full.
+template <int B>
+struct GatheredSrc {
+  const float *U;
+  int pad;
+  __device__ __forceinline__ float load(int kb, int ib, int, int r, int c) const {
+    return U[(kb * B + r) * pad + ib * B + c];
+  }
+};
+
+// Indexed gather of every tile on or above the diagonal into U (zeroed by the caller): ids >= nM
+// read as zero, padded diagonal entries get +1 (mjw_step_optimized.py:932-941).  A wavefront
+// takes every (number of wavefronts)-th tile and keeps eight tiles' loads in flight.
+template <int B>
+__device__ __forceinline__ void gather_tiles(const float *__restrict__ Mw, const int32_t *__restrict__ block_idx,
+                                             int nM, int nv, int pad, float *U, int tid, int nt) {
+  constexpr int BB = B * B, PER = BB / 64 > 0 ? BB / 64 : 1, G = 8;
+  const int nblk = pad / B, lane = tid & 63, nwv = nt >> 6;
+  int kb = 0, ib = 0;  // cursor over the upper tiles, row by row
+  auto advance = [&](int n) {
+    for (int s_ = 0; s_ < n && kb < nblk; ++s_)
+      if (++ib == nblk) { ++kb; ib = kb; }
+  };
+  advance(tid >> 6);
+  while (kb < nblk) {
+    int tk[G], ti[G], idx[G][PER];
+    float v[G][PER];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      tk[g] = kb < nblk ? kb : -1;
+      ti[g] = ib;
+      advance(nwv);
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const int e = u * 64 + lane;
+        const bool use = tk[g] >= 0 && e < BB;
+        idx[g][u] = block_idx[use ? (size_t)(tk[g] * nblk + ti[g]) * BB + e : 0];
+        if (!use) idx[g][u] = nM;
+      }
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int u = 0; u < PER; ++u) v[g][u] = Mw[idx[g][u] < nM ? idx[g][u] : 0];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const int e = u * 64 + lane;
+        if (tk[g] >= 0 && e < BB) {
+          const int r = e / B, c = e - r * B;
+          float x = idx[g][u] < nM ? v[g][u] : 0.0f;
+          if (ti[g] == tk[g] && (tk[g] + 1) * B > nv && r == c && (nblk - 1) * B + r >= nv) x = x + 1.0f;
+          U[(tk[g] * B + r) * pad + ti[g] * B + c] = x;
+        }
+      }
+  }
+}
 
 // Left-looking upper Cholesky by block column with the forward solve of rhs fused into the
 // loop; U (pad, pad) and rhs (pad) in LDS, U zeroed by the caller.
@@ -173,7 +221,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
     // U_kk = L', and U_ki = L^-1 A_ki column by column
     for (int e = tid; e < BB; e += nt) {
       const int r = e / B, c = e - r * B;
-      if (c >= r) U[(k + r) * pad + k + c] = L[c * B + r];
+      U[(k + r) * pad + k + c] = c >= r ? L[c * B + r] : 0.0f;  // a gathered tile may have sat there
     }
     for (int q = tid; q < (ntile - 1) * B; q += nt) {
       const int tb = 1 + q / B, c = q - (tb - 1) * B;
@@ -269,7 +317,9 @@ __global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
   for (int i = tid; i < pad * pad; i += nt) U[i] = 0.0f;
   for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? y[w * ldy + i] : 0.0f;
   __syncthreads();
-  const IndexedSrc<B> src{M + w * ldM, block_idx, nM, nv, pad / B};
+  gather_tiles<B>(M + w * ldM, block_idx, nM, nv, pad, U, tid, nt);
+  __syncthreads();
+  const GatheredSrc<B> src{U, pad};
   factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
   backward_solve<B>(U, rhs, pad, tid);
   for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
