@@ -158,7 +158,8 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done,
  * gradient rides as column nv_pad - 1, the corner is 1e30, U (nworld, nv_pad, nv_pad)
  * receives the factor including that column; without changed rows the stored U is solved
  * against.  Rows and columns >= nv of H count as the identity.  nv_pad = a multiple of 16
- * above nv (src/instantmimic/utils/mjw_model.py:30). */
+ * above nv (src/instantmimic/utils/mjw_model.py:30).  H and U must be 16-byte aligned
+ * (IM_ERR_STRIDE otherwise). */
 int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes,
                            const int32_t *changes, const int32_t *ids, int ld_ids,
                            const float *J, int njmax, const float *D, const int32_t *state,
@@ -175,7 +176,7 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes,
  * block_idx is the (nblk, nblk, B, B)-ordered table of element ids into M[w, :] built
  * by create_blocked_dense_factor_solve_scratch (mjw_step_optimized.py:932-941); ids
  * >= nM read as zero; padded diagonal entries get +1.  U (nworld, pad, pad) receives the
- * factor (the reference's workspace) or may be null.  block_size 8 or 16. */
+ * factor (the reference's workspace; 16-byte aligned) or may be null.  block_size 8 or 16. */
 int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *block_idx,
                             int block_size, int nv, int pad, const float *y, int64_t ldy,
                             float *U, float *x, int64_t ldx, int nworld, void *stream);

@@ -324,7 +324,8 @@ __global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
   backward_solve<B>(U, rhs, pad, tid);
   for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
   if (Uout)
-    for (int i = tid; i < pad * pad; i += nt) Uout[w * (int64_t)pad * pad + i] = U[i];
+    for (int i = tid; i < pad * pad / 4; i += nt)  // pad is a multiple of B >= 8
+      ((float4 *)(Uout + w * (int64_t)pad * pad))[i] = ((const float4 *)U)[i];
 }
 
 // Per-iteration factor stage on the dense Hessian: dofs touched by the changed rows,
@@ -491,11 +492,11 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
       L[0] = sqrtf(v);
     }
     __syncthreads();
-    for (int i = tid; i < pad * pad; i += nt) {
-      const int r = i / pad, c = i - r * pad;
-      float v = U[i];
-      if (c == pad - 1) v = r < nv ? rhs[r] : (r == pad - 1 ? L[0] : v);
-      Uw[i] = v;
+    for (int i = tid; i < pad * pad / 4; i += nt) {  // pad is a multiple of 16: a float4 stays in a row
+      const int r = 4 * i / pad, c = 4 * i - r * pad;
+      float4 v = ((const float4 *)U)[i];
+      if (c + 3 == pad - 1) v.w = r < nv ? rhs[r] : (r == pad - 1 ? L[0] : v.w);
+      ((float4 *)Uw)[i] = v;
     }
     __syncthreads();  // rhs is overwritten by the backward solve
   } else {
@@ -648,6 +649,7 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
   if (block_size != 8 && block_size != 16) return IM_ERR_UNSUPPORTED;
   if (pad % block_size || pad - nv >= block_size) return IM_ERR_ARG;
   if (ldy < nv || ldx < nv) return IM_ERR_STRIDE;
+  if (U && ((uintptr_t)U & 15)) return IM_ERR_STRIDE;  // written 16 bytes at a time
   const int B = block_size;
   const size_t lds_bytes = sizeof(float) * ((size_t)pad * pad + pad + (size_t)(pad / B) * B * B + B * B + B);
   if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
@@ -686,6 +688,7 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
     return IM_ERR_ARG;
   if (nv_pad % 16) return IM_ERR_ARG;
   if (ldg < nv || ld_search < nv) return IM_ERR_STRIDE;
+  if (((uintptr_t)H | (uintptr_t)U) & 15) return IM_ERR_STRIDE;  // read and written 16 bytes at a time
   constexpr int B = 16;
   const size_t base_bytes =
       sizeof(float) * ((size_t)nv_pad * nv_pad + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + B + nv + 1);
