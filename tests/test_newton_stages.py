@@ -261,3 +261,25 @@ def test_gpu_dense_stage_bitwise(device, name, nworld):
     live = _live(sc, done)
     np.testing.assert_array_equal(search.cpu().numpy()[live][:, :nv, 0], want2[3][live])
     np.testing.assert_array_equal(decr.cpu().numpy()[live], want2[5][live])
+
+
+@pytest.mark.gpu
+def test_gpu_block_per_world_sparse_kernels_agree():
+    """The sparse factor has two kernels per entry point (a wavefront per world with the tables in
+    LDS, and a workgroup of the plan's width per world for models it does not fit): the second
+    family is forced here in a child process and must pass the same bitwise comparisons."""
+    import os
+    import subprocess
+    import sys
+
+    env = dict(os.environ, IMHIP_SPARSE_KERNEL="simple")
+    code = (
+        "import sys, torch; sys.path.insert(0, 'tests');"
+        "import test_newton_stages as a, test_sparse_hessian as b; d = torch.device('cuda:0');"
+        "a.test_gpu_sparse_stage_bitwise(d, 32); a.test_gpu_sparse_stage_bitwise(d, 64);"
+        "b.test_gpu_contact_model_bitwise(d, 1, 32); b.test_gpu_benchmark_trees_bitwise(d, 'snu', 100);"
+        "b.test_gpu_done_mask_violation_counter_and_graph_replay(d); print('block-per-world kernels ok')"
+    )
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "block-per-world kernels ok" in out.stdout, out.stderr[-2000:]
