@@ -304,9 +304,14 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     for n, (ti, tj) in enumerate(tiles):
         for v in range(4):
             emit(f"    const int ix{n}_{v} = IDX_{name}[{n * 4 + v}][lane];")
+    # chain columns, needed right after the hand-over barrier: requested here, and pinned so that
+    # the load is not moved down to its use
+    for i in range(len(leaf_sets)):
+        emit(f"    int chc{i} = CH_{name}[{i}][p];")
     for i in range(MC):
         emit(f"    const float mv{i} = M[wq * ldM + min({i * 64} + lane, {nM - 1})];")
     SP = 4  # steps (16 rows) requested before the row weights are known
+    pin_ch = " ".join(f'asm volatile("" : "+v"(chc{i}));' for i in range(len(leaf_sets)))
     emit("    int steps_s = 0, cnt = 0;  // short variant: steps and length of the compacted tail")
     emit("    if (LONG) {")
     emit("      for (int r0 = 128; r0 < njp; r0 += 64) {  // rows from 128 on, up front")
@@ -358,6 +363,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         for v in range(4):
             emit(f"    {{ const float mvv = mcopy[ix{n}_{v} < 0 ? 0 : ix{n}_{v}]; acc{n}[{v}] = ix{n}_{v} >= 0 ? mvv : 0.0f; }}")
     emit("    IM_WAVE_SYNC();")
+    emit("    " + pin_ch)
     emit("    STAMP();  // 1: row weights staged, M gathered")
     emit("    if (!LONG) {  // every row that is needed is already in flight")
     for u in range(PD):
@@ -387,7 +393,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             emit(f"    lds[wv * {W * W} + ({16 * ti + v} + 4 * kq) * {W} + {16 * tj} + p] = acc{n}[{v}];")
     emit("    __syncthreads();")
     for i, (li, s) in enumerate(leaf_sets):
-        emit(f"    lh{i} = lds + kq * {W * W} + CH_{name}[{i}][p];")
+        emit(f"    lh{i} = lds + kq * {W * W} + chc{i};")
     emit("  } else {")
     emit("    const float *Mw = M + ws * ldM;")
     for b in range(nv):
