@@ -391,7 +391,9 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     for n, (ti, tj) in enumerate(tiles):
         for v in range(4):
             emit(f"    lds[wv * {W * W} + ({16 * ti + v} + 4 * kq) * {W} + {16 * tj} + p] = acc{n}[{v}];")
+    emit("    STAMP();  // tiles written")
     emit("    __syncthreads();")
+    emit("    STAMP();  // hand-over barrier passed")
     for i, (li, s) in enumerate(leaf_sets):
         emit(f"    lh{i} = lds + kq * {W * W} + chc{i};")
     emit("  } else {")
@@ -578,8 +580,12 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     for j, g in enumerate(groups):
         emit(f"  if (ROLE({j})) {{  // group {j}")
         fetch_rows(sorted(g))
+        if j == 0:
+            emit("    STAMP();  // group 0: rows fetched")
         for k in g:
             eliminate(k, j)
+        if j == 0:
+            emit("    STAMP();  // group 0: eliminated")
         for s_ in range(vsets[j]):
             expr = sv(j, len(segs[j]) - 1, s_)
             by_src = {}
@@ -613,10 +619,13 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             mask = sum(1 << p for p in range(16) if any(t.depth[a] == 16 * s_ + p for a in touched[j]))
             if mask:
                 emit(f"    SVT_{s_} = ((0x{mask:x} >> p) & 1) ? SVT_{s_} + (ASM ? xlds[{xslots[j]['S', s_]} + lane] : SP{j}_{s_}) : SVT_{s_};")
+    emit("    STAMP();  // trunk: rows fetched and merged")
     for k in reversed(trunk):
         eliminate(k, None)
+    emit("    STAMP();  // trunk: eliminated")
     for b in trunk:
         backsub(b)
+    emit("    STAMP();  // trunk: solved")
     emit("    if (ASM && p == 0) {")
     for b in trunk:
         emit(f"      xlds[{xs_off} + (lane >> 4) * {nv} + {b}] = S{b};")
