@@ -4,7 +4,8 @@
 
 * tree_plans.json   integer plans of the benchmark trees and of the reference's
                     test trees (spans per group count, chosen plan, elimination order).
-                    The values equal the hand-checked table of the survey (appendix H).
+                    The spans and chosen plans were checked by hand against the planner rule
+                    (src/instantmimic/utils/mjw_kernels/tree_ldl.py:66-193).
 * tree_small.npz    4 worlds of the ant shape: inputs, assembled H and solve result of
                     the oracle (fp32), for comparing the HIP path against stored vectors.
 """
