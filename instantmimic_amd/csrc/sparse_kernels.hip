@@ -44,6 +44,19 @@ struct SparseDev {
 
 __device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 
+// element `index` of an array whose base is the same for the whole wavefront: an unsigned
+// 32-bit offset lets the load take the base from scalar registers
+template <class T>
+__device__ __forceinline__ T ld_u32(const T *base, uint32_t index) {
+  return *(const T *)((const char *)base + (size_t)(index * (uint32_t)sizeof(T)));
+}
+
+// value of the lane N places up in the caller's row of 16 lanes (0 past the row's end)
+template <int N>
+__device__ __forceinline__ float row_shl(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x100 + N, 0xF, 0xF, true));
+}
+
 // Orders LDS writes before later reads: across the workgroup, or, when a world belongs to
 // one wavefront (WAVE), across that wavefront only.
 template <bool WAVE>
@@ -94,7 +107,14 @@ __device__ __forceinline__ void factor_levels(const SparseDev &P, float *N, floa
           for (; t < len; t += T) v = fma_(pa[t] * pb[t], pd[t], v);
         }
       }
-      for (int off = T >> 1; off > 0; off >>= 1) v = v + __shfl_down(v, off, T);
+      // shuffle-down tree of the team; inside a row of 16 lanes a DPP shift does it (what a lane
+      // past the team's end receives is never passed on to the team's first lane)
+      if (T > 32) v = v + __shfl_down(v, 32, 64);
+      if (T > 16) v = v + __shfl_down(v, 16, 64);
+      if (T > 8) v = v + row_shl<8>(v);
+      if (T > 4) v = v + row_shl<4>(v);
+      if (T > 2) v = v + row_shl<2>(v);
+      if (T > 1) v = v + row_shl<1>(v);
       if (e < e1 && tl == 0) {
         const float wv = N[sl] - v;
         N[sl] = wv;
@@ -344,9 +364,9 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
   for (int u = 0; u < PD; ++u) {
     const int row = 4 * u + kq, rowc = row < njmax ? row : njmax - 1;
 #pragma unroll
-    for (int c = 0; c < NT; ++c) g[u][c] = Jw[rowc * n + col[c]];
-    gd[u] = Dw[rowc];
-    gs[u] = sw[rowc];
+    for (int c = 0; c < NT; ++c) g[u][c] = ld_u32(Jw, (uint32_t)(rowc * n + col[c]));
+    gd[u] = ld_u32(Dw, (uint32_t)rowc);
+    gs[u] = ld_u32(sw, (uint32_t)rowc);
   }
 #pragma unroll
   for (int c = 0; c < 16; ++c)
@@ -388,23 +408,33 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
         // four rows' supports are assembled from the ballots with scalar instructions; lane d
         // then tests dof d of each row against the dofs outside its pattern row.
         const bool dnz = d != 0.0f;
-        unsigned long long sup[4] = {0ull, 0ull, 0ull, 0ull};
+        uint32_t blo[4] = {0u, 0u, 0u, 0u}, bhi[4] = {0u, 0u, 0u, 0u};  // rows 0, 1 | rows 2, 3 of a 16-dof block
 #pragma unroll
         for (int c = 0; c < NT; ++c) {
           const unsigned long long b = __ballot(dnz & colok[c] & (z[c] != 0.0f));
-#pragma unroll
-          for (int k = 0; k < 4; ++k) sup[k] |= ((b >> (16 * k)) & 0xFFFFull) << (16 * c);
+          blo[c] = (uint32_t)b;
+          bhi[c] = (uint32_t)(b >> 32);
         }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) nbad += (__ballot((sup[k] & npm) != 0ull) & sup[k]) != 0ull;
+        // 16-bit transposition: row k's support = its 16 bits of every block side by side
+        const uint32_t s0l = (blo[0] & 0xFFFFu) | (blo[1] << 16), s0h = (blo[2] & 0xFFFFu) | (blo[3] << 16);
+        const uint32_t s1l = (blo[0] >> 16) | (blo[1] & 0xFFFF0000u), s1h = (blo[2] >> 16) | (blo[3] & 0xFFFF0000u);
+        const uint32_t s2l = (bhi[0] & 0xFFFFu) | (bhi[1] << 16), s2h = (bhi[2] & 0xFFFFu) | (bhi[3] << 16);
+        const uint32_t s3l = (bhi[0] >> 16) | (bhi[1] & 0xFFFF0000u), s3h = (bhi[2] >> 16) | (bhi[3] & 0xFFFF0000u);
+        const uint32_t nl = (uint32_t)npm, nh = (uint32_t)(npm >> 32);
+        const unsigned long long sup0 = ((unsigned long long)s0h << 32) | s0l, sup1 = ((unsigned long long)s1h << 32) | s1l;
+        const unsigned long long sup2 = ((unsigned long long)s2h << 32) | s2l, sup3 = ((unsigned long long)s3h << 32) | s3l;
+        nbad += (__ballot(((s0l & nl) | (s0h & nh)) != 0u) & sup0) != 0ull;
+        nbad += (__ballot(((s1l & nl) | (s1h & nh)) != 0u) & sup1) != 0ull;
+        nbad += (__ballot(((s2l & nl) | (s2h & nh)) != 0u) & sup2) != 0ull;
+        nbad += (__ballot(((s3l & nl) | (s3h & nh)) != 0u) & sup3) != 0ull;
       }
       // Next use of this register set.  Issued whether or not the step above ran, so that the
       // number of loads in flight at every wait is the same on every path.
       const int nrow = 4 * (s0 + u + PD) + kq, nrowc = nrow < njmax ? nrow : njmax - 1;
 #pragma unroll
-      for (int c = 0; c < NT; ++c) g[u][c] = Jw[nrowc * n + col[c]];
-      gd[u] = Dw[nrowc];
-      gs[u] = sw[nrowc];
+      for (int c = 0; c < NT; ++c) g[u][c] = ld_u32(Jw, (uint32_t)(nrowc * n + col[c]));
+      gd[u] = ld_u32(Dw, (uint32_t)nrowc);
+      gs[u] = ld_u32(sw, (uint32_t)nrowc);
     }
   }
   // the slots of this lane's accumulator elements (all requested before the first is used)
