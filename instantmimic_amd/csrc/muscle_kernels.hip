@@ -19,31 +19,92 @@ namespace {
 
 __device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 
-// One wavefront per world, four worlds per workgroup.
-__global__ __launch_bounds__(256) void muscle_project_kernel(
+// One workgroup of two wavefronts per world; with 4 nentry + 2 nentry + 4 nmuscle bytes of LDS
+// sixteen and more of them fit a CU, so 4096 worlds are all resident at once.  A and the
+// muscle of every term are first brought into LDS in the order the rows consume them (every
+// lane busy, twelve terms' look-ups in flight per lane), the force row as it is; then lane j of
+// the first wavefront runs row j's chain of fused multiply-adds over consecutive LDS words.
+// Same terms, same order per row as the reference kernel.
+__global__ __launch_bounds__(128) void muscle_project_kernel(
     const float *__restrict__ moment, int64_t ldm, const float *__restrict__ force, int64_t ldf,
     const int32_t *__restrict__ offsets, const int32_t *__restrict__ entry_idx,
     const int32_t *__restrict__ entry_muscle, int nentry, int nmuscle, int ntorque, int root,
     float *__restrict__ qfrc, int64_t ldq, int nworld) {
   extern __shared__ float lds[];
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int w = blockIdx.x * 4 + wv;
-  if (w >= nworld) return;  // wave-uniform; no workgroup barrier below
-  float *prod = lds + (size_t)wv * nentry;  // A[e] and f[muscle(e)] side by side is not needed:
-  const float *mw = moment + (int64_t)w * ldm, *fw = force + (int64_t)w * ldf;
-  // stage A[w, :] (coalesced); forces are gathered straight from the row (L1 resident)
-  for (int e = lane; e < nentry; e += 64) prod[e] = mw[e];
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  for (int j = lane; j < ntorque; j += 64) {
+  constexpr int NT = 128, UN = 12;
+  const int tid = threadIdx.x;
+  const int64_t w = blockIdx.x;
+  float *av = lds;                                      // [nentry] A[entry_idx[s]]
+  float *fs = av + nentry;                              // [nmuscle] the world's forces
+  unsigned short *ms = (unsigned short *)(fs + nmuscle);  // [nentry] entry_muscle[entry_idx[s]]
+  const float *mw = moment + w * ldm, *fw = force + w * ldf;
+  // Every array is read from memory in its own order (coalesced); the permutation into the
+  // rows' order goes through LDS, in place: gather into registers, barrier, write back.
+  for (int i = tid; i < nmuscle; i += NT) fs[i] = fw[i];
+  if (nentry <= UN * NT) {
+    int e[UN], m[UN];
+    float x[UN];
+#pragma unroll
+    for (int k = 0; k < UN; ++k) {
+      const int i = tid + NT * k < nentry ? tid + NT * k : nentry - 1;
+      e[k] = entry_idx[i];
+      m[k] = entry_muscle[i];
+      x[k] = mw[i];
+    }
+#pragma unroll
+    for (int k = 0; k < UN; ++k)
+      if (tid + NT * k < nentry) {
+        av[tid + NT * k] = x[k];
+        ms[tid + NT * k] = (unsigned short)m[k];
+      }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < UN; ++k) {
+      x[k] = av[e[k]];
+      m[k] = ms[e[k]];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < UN; ++k)
+      if (tid + NT * k < nentry) {
+        av[tid + NT * k] = x[k];
+        ms[tid + NT * k] = (unsigned short)m[k];
+      }
+  } else {
+    // more entries than one trip holds: gathered from memory, twelve look-ups in flight per lane
+    for (int s0 = tid; s0 < nentry; s0 += UN * NT) {
+      int e[UN], m[UN];
+      float x[UN];
+#pragma unroll
+      for (int k = 0; k < UN; ++k) e[k] = entry_idx[s0 + NT * k < nentry ? s0 + NT * k : nentry - 1];
+#pragma unroll
+      for (int k = 0; k < UN; ++k) {
+        m[k] = entry_muscle[e[k]];
+        x[k] = mw[e[k]];
+      }
+#pragma unroll
+      for (int k = 0; k < UN; ++k)
+        if (s0 + NT * k < nentry) {
+          av[s0 + NT * k] = x[k];
+          ms[s0 + NT * k] = (unsigned short)m[k];
+        }
+    }
+  }
+  __syncthreads();
+  for (int j = tid; j < ntorque; j += NT) {
     float total = 0.0f;
     const int e1 = offsets[j + 1];
-    for (int s = offsets[j]; s < e1; ++s) {
-      const int e = entry_idx[s];
-      total = fma_(prod[e], fw[entry_muscle[e]], total);
+    int s = offsets[j];
+    for (; s + 3 < e1; s += 4) {  // four terms' operands read before the first is used
+      const float a0 = av[s], a1 = av[s + 1], a2 = av[s + 2], a3 = av[s + 3];
+      const float f0 = fs[ms[s]], f1 = fs[ms[s + 1]], f2 = fs[ms[s + 2]], f3 = fs[ms[s + 3]];
+      total = fma_(a0, f0, total);
+      total = fma_(a1, f1, total);
+      total = fma_(a2, f2, total);
+      total = fma_(a3, f3, total);
     }
-    qfrc[(int64_t)w * ldq + root + j] = total;
+    for (; s < e1; ++s) total = fma_(av[s], fs[ms[s]], total);
+    qfrc[w * ldq + root + j] = total;
   }
 }
 
@@ -59,10 +120,25 @@ __global__ __launch_bounds__(256) void muscle_gather_kernel(
   float *partial = weighted + nentry + 1;  // [chunk_count]
   const int lane = threadIdx.x, width = blockDim.x;
   const int64_t w = blockIdx.x;
-  for (int e = lane; e < nentry; e += width) {
-    const float v = moment[w * ldm + e];
-    m[e] = v;
-    weighted[e] = slope[w * lds_ + entry_muscle[e]] * v;
+  for (int e0 = lane; e0 < nentry; e0 += 8 * width) {  // eight entries' loads in flight per lane
+    float v[8], sl[8];
+    int mu[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int e = e0 + k * width < nentry ? e0 + k * width : nentry - 1;
+      v[k] = moment[w * ldm + e];
+      mu[k] = entry_muscle[e];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) sl[k] = slope[w * lds_ + mu[k]];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int e = e0 + k * width;
+      if (e < nentry) {
+        m[e] = v[k];
+        weighted[e] = sl[k] * v[k];
+      }
+    }
   }
   if (lane == 0) {
     m[nentry] = 0.0f;
@@ -82,9 +158,10 @@ __global__ __launch_bounds__(256) void muscle_gather_kernel(
   for (int slot = lane; slot < nelem; slot += width) {
     float acc = 0.0f;
     const int c1 = chunk_offsets[slot + 1];
-    for (int c = chunk_offsets[slot]; c < c1; ++c) acc = acc + partial[c];
     float *q = qderiv + w * ldq + elem_ids[slot];
-    *q = fma_(timestep, acc, *q);
+    const float q0 = *q;  // requested before the sum, used after it
+    for (int c = chunk_offsets[slot]; c < c1; ++c) acc = acc + partial[c];
+    *q = fma_(timestep, acc, q0);
   }
 }
 
@@ -101,9 +178,10 @@ int im_muscle_project(const float *moment, int64_t ld_moment, const float *force
   if (nworld == 0 || ntorque == 0) return IM_OK;
   if (!moment || !force || !torque_entry_offsets || !torque_entry_idx || !entry_muscle || !qfrc) return IM_ERR_ARG;
   if (ld_moment < nentry || ld_force < nmuscle || ld_qfrc < root_dof_count + ntorque) return IM_ERR_STRIDE;
-  const size_t lds_bytes = (size_t)4 * nentry * sizeof(float);
+  if (nmuscle > 65535) return IM_ERR_UNSUPPORTED;  // muscle ids travel as 16 bits
+  const size_t lds_bytes = sizeof(float) * ((size_t)nentry + nmuscle) + 2 * (((size_t)nentry + 1) & ~(size_t)1);
   if (lds_bytes > 64 * 1024) return IM_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(im::muscle_project_kernel, dim3((nworld + 3) / 4), dim3(256), lds_bytes, (hipStream_t)stream,
+  hipLaunchKernelGGL(im::muscle_project_kernel, dim3(nworld), dim3(128), lds_bytes, (hipStream_t)stream,
                      moment, ld_moment, force, ld_force, torque_entry_offsets, torque_entry_idx, entry_muscle,
                      nentry, nmuscle, ntorque, root_dof_count, qfrc, ld_qfrc, nworld);
   IM_HIP_CHECK(hipGetLastError());

@@ -111,3 +111,26 @@ def test_gpu_matches_oracle_bitwise(device, nworld):
     np.testing.assert_array_equal(qd.cpu().numpy(), q_ref)
     # the contract's bound as well
     assert R.rel_l2(got[:, mb.root_dof_count : nv], tau_ref[:, mb.root_dof_count :]) <= 1e-5
+
+
+@pytest.mark.gpu
+def test_gpu_projection_with_more_entries_than_one_staging_trip(device):
+    """The projection kernel permutes up to 1536 entries through LDS in one trip and gathers
+    larger sets from memory: 420 muscles give about 1900 entries."""
+    import torch
+
+    nworld = 97
+    mb = synth.make_muscles(nworld, nmuscle=420, seed=5)
+    rowadr, _, _ = synth.csr_from_parents(synth.snu_parents())
+    nv = len(rowadr)
+    ent = Q.entries_from_muscle_dofs(mb.muscle_dofs, mb.nmuscle)
+    assert len(ent.muscle_dof_torque_idx) > 1536
+    offsets, order = Q.torque_sorted_entries(ent.muscle_dof_torque_idx, nv - mb.root_dof_count)
+    t = lambda a, dt=None: torch.from_numpy(np.ascontiguousarray(a if dt is None else a.astype(dt))).to(device)  # noqa: E731
+    qfrc = torch.full((nworld, nv), 7.0, device=device)
+    Q.project_muscle_sparse_moment_qfrc(t(mb.moment), t(mb.force), t(offsets, np.int32), t(order, np.int32), t(ent.muscle_dof_muscle_idx, np.int32), mb.root_dof_count, qfrc)
+    torch.cuda.synchronize()
+    tau_ref = R.muscle_project(mb.moment, mb.force, offsets, order, ent.muscle_dof_muscle_idx, mb.root_dof_count, nv)
+    got = qfrc.cpu().numpy()
+    np.testing.assert_array_equal(got[:, mb.root_dof_count :], tau_ref[:, mb.root_dof_count :])
+    assert (got[:, : mb.root_dof_count] == 7.0).all()
