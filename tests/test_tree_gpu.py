@@ -86,6 +86,28 @@ def test_fused_full_humanoid_batch(device):
         assert (np.linalg.norm(res, axis=1) / scale).max() < 2e-6
 
 
+@pytest.mark.parametrize("name,nworld,ragged", [("humanoid", 4096, True), ("humanoid", 333, False), ("ant", 67, True), ("g1", 130, True)])
+def test_fused_without_h_output_bitwise(device, name, nworld, ragged):
+    """The fused entry without its optional H output (what the benchmark launches): x must be the
+    oracle's bit for bit, with and without the per-world row counts and with the negated result."""
+    from instantmimic_amd.mjw_kernels import tree_ldl as T
+
+    b = synth.make_batch(name, nworld, ragged_nefc=ragged)
+    scratch = T.create_tree_factor_solve_scratch(_model(b), device)
+    st = P.tree_ldl_structure(b.rowadr, b.rownnz, b.colind)
+    plan = P.best_tree_ldl_plan(*st)
+    for it in range(b.state.shape[0]):
+        x_ref = R.assemble_tree_ldl_solve(*st, plan, b.M, b.J, b.D, b.state[it], b.nefc, b.grad)
+        x, _ = _run_fused(T, scratch, b, it, device, want_h=False)
+        np.testing.assert_array_equal(x, x_ref)
+    xn, _ = _run_fused(T, scratch, b, 0, device, want_h=False, negate=True)
+    np.testing.assert_array_equal(xn, -R.assemble_tree_ldl_solve(*st, plan, b.M, b.J, b.D, b.state[0], b.nefc, b.grad))
+    full = np.full_like(b.nefc, b.J.shape[1])
+    x_all = R.assemble_tree_ldl_solve(*st, plan, b.M, b.J, b.D, b.state[0], full, b.grad)
+    xa, _ = _run_fused(T, scratch, b, 0, device, nefc=False, want_h=False)
+    np.testing.assert_array_equal(xa, x_all)
+
+
 def test_stored_vectors(device):
     from instantmimic_amd.mjw_kernels import tree_ldl as T
 
