@@ -543,24 +543,25 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
 
 // ---------------------------------------------------------------------------- dense J'DJ
 // H[w] = M[w] + J[w]' diag(Dc[w]) J[w], H (nv_pad, nv_pad), on v_mfma_f32_32x32x2_f32.
-// One wavefront per 32x32 output tile; a workgroup of 256 threads covers a 64x64... the
-// tile grid is (ceil(nv/32))^2 per world, only tiles with column block >= row block are
-// computed and mirrored.  A = (J D)' and B = J are staged through LDS 32 rows at a time.
+// One workgroup of four wavefronts per world, a wavefront per 32 x 32 output tile (the tiles
+// with column block >= row block, dealt round robin, accumulators in registers, mirrored at
+// the end).  J is staged through LDS 32 rows at a time with the row weights beside it; the
+// next 32 rows are already on their way into registers while the matrix cores work on the
+// current ones, and the weighted operand (J Dc) is formed when it is fed.
 typedef float float16v __attribute__((ext_vector_type(16)));
 
-__global__ __launch_bounds__(256) void jtdj_mfma_kernel(
+__global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
     const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
     const float *__restrict__ D, const int32_t *__restrict__ state, const int32_t *__restrict__ nefc_p,
     int quad, float *__restrict__ H, int nv, int nv_pad) {
   extern __shared__ float lds[];
   const int nvr = (nv + 31) / 32 * 32;   // staged row width
-  float *Js = lds;                       // [32][nvr]   J rows
-  float *JDs = Js + 32 * nvr;            // [32][nvr]   J rows times Dc
+  float *Js = lds;                       // [32][nvr] J rows (zero past nefc and past nv)
+  float *dcs = Js + 32 * nvr;            // [32] their weights
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t w = blockIdx.x;
   const int nb = nvr / 32;
   // tiles (bi <= bj) distributed over the four waves; each wave keeps its tiles' accumulators
-  const int ntile = nb * (nb + 1) / 2;
   constexpr int MAXT = 3;                // up to 10 tiles (nv <= 128) over 4 waves
   float16v acc[MAXT];
   int tbi[MAXT], tbj[MAXT], mine = 0;
@@ -571,7 +572,6 @@ __global__ __launch_bounds__(256) void jtdj_mfma_kernel(
     for (int bi = 0; bi < nb; ++bi)
       for (int bj = bi; bj < nb; ++bj, ++t)
         if (t % 4 == wave) {
-          // tile number mine of this wave (at most MAXT)
           if (mine == 0) { tbi[0] = bi; tbj[0] = bj; }
           else if (mine == 1) { tbi[1] = bi; tbj[1] = bj; }
           else if (mine == 2) { tbi[2] = bi; tbj[2] = bj; }
@@ -586,31 +586,58 @@ __global__ __launch_bounds__(256) void jtdj_mfma_kernel(
   int nefc = nefc_p ? nefc_p[w] : njmax;
   nefc = nefc < njmax ? nefc : njmax;
   const float *Jw = J + w * (int64_t)njmax * nv;
-  for (int r0 = 0; r0 < nefc; r0 += 32) {
-    __syncthreads();
-    for (int q = tid; q < 32 * nvr; q += 256) {
-      const int r = q / nvr, c = q - r * nvr;
-      float v = 0.0f, dc = 0.0f;
-      if (r0 + r < nefc && c < nv) {
-        v = Jw[(int64_t)(r0 + r) * nv + c];
-        if (state[w * njmax + r0 + r] == quad) dc = D[w * njmax + r0 + r];
-      }
-      Js[q] = v;
-      JDs[q] = v * dc;
+  const float *Dw = D + w * njmax;
+  const int32_t *sw = state + w * njmax;
+  // a wavefront stages 8 of a chunk's 32 rows, lanes across the columns (two per lane)
+  const int c0 = lane, c1 = lane + 64;
+  const int c0c = c0 < nv ? c0 : nv - 1, c1c = c1 < nv ? c1 : nv - 1;
+  float v0[8], v1[8], dd = 0.0f;
+  int sd = 0;
+  auto prefetch = [&](int r0) {  // every load is issued whatever the row: clamped, selected later
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = r0 + wave * 8 + i, rowc = row < njmax ? row : njmax - 1;
+      v0[i] = Jw[(int64_t)rowc * nv + c0c];
+      v1[i] = Jw[(int64_t)rowc * nv + c1c];
     }
-    __syncthreads();
+    const int row = r0 + wave * 8 + (lane & 7), rowc = row < njmax ? row : njmax - 1;
+    dd = Dw[rowc];
+    sd = sw[rowc];
+  };
+  auto stage = [&](int r0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const bool in = r0 + wave * 8 + i < nefc;
+      Js[(wave * 8 + i) * nvr + c0] = (in && c0 < nv) ? v0[i] : 0.0f;
+      if (c1 < nvr) Js[(wave * 8 + i) * nvr + c1] = (in && c1 < nv) ? v1[i] : 0.0f;
+    }
+    if (lane < 8) dcs[wave * 8 + lane] = (r0 + wave * 8 + lane < nefc && sd == quad) ? dd : 0.0f;
+  };
+  prefetch(0);
+  stage(0);
+  __syncthreads();
+  for (int r0 = 0; r0 < nefc; r0 += 32) {
+    prefetch(r0 + 32);
     // v_mfma_f32_32x32x2_f32: lane l supplies A[i = l % 32][k = l / 32] and B[k = l / 32][j = l % 32]
+    // the wavefront's tiles take turns inside the loop over the rows: independent accumulators
+    // keep the matrix core busy while one of them waits for its previous result
+    const float *pa[MAXT], *pb[MAXT];
 #pragma unroll
     for (int m = 0; m < MAXT; ++m) {
-      if (m < mine) {
-        const int ci = tbi[m] * 32 + (lane & 31), cj = tbj[m] * 32 + (lane & 31);
-#pragma unroll 4
-        for (int kk = 0; kk < 32; kk += 2) {
-          const int k = kk + (lane >> 5);
-          acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(JDs[k * nvr + ci], Js[k * nvr + cj], acc[m], 0, 0, 0);
-        }
-      }
+      pa[m] = Js + (lane >> 5) * nvr + tbi[m] * 32 + (lane & 31);
+      pb[m] = Js + (lane >> 5) * nvr + tbj[m] * 32 + (lane & 31);
     }
+#pragma unroll 4
+    for (int q = 0; q < 16; ++q) {
+      const float dk = dcs[2 * q + (lane >> 5)];
+#pragma unroll
+      for (int m = 0; m < MAXT; ++m)
+        if (m < mine)
+          acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[m][2 * q * nvr] * dk, pb[m][2 * q * nvr], acc[m], 0, 0, 0);
+    }
+    __syncthreads();  // every wavefront is done with the staged rows
+    stage(r0 + 32);
+    __syncthreads();
   }
   // accumulator layout of a 32x32 tile: lane l holds column j = l % 32 and rows
   // i = 8 * g + 4 * (l / 32) ... for register 4 * g + v: i = 8 * g + (l / 32) * 4 + v
@@ -669,7 +696,7 @@ int im_jtdj_mfma(const float *Mdense, const float *J, int njmax, const float *D,
   if (!Mdense || !J || !D || !state || !H) return IM_ERR_ARG;
   if (nv > 128) return IM_ERR_UNSUPPORTED;
   const int nvr = (nv + 31) / 32 * 32;
-  const size_t lds_bytes = sizeof(float) * 2 * 32 * (size_t)nvr;
+  const size_t lds_bytes = sizeof(float) * (32 * (size_t)nvr + 32);
   hipLaunchKernelGGL(im::jtdj_mfma_kernel, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, Mdense, J,
                      njmax, D, state, nefc, quad, H, nv, nv_pad);
   IM_HIP_CHECK(hipGetLastError());
