@@ -13,6 +13,8 @@
 //   is applied as a multiplication by 1 / diagonal (the reciprocal is an exact division).
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "common.h"
 
 namespace im {
@@ -683,8 +685,12 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
   auto fn = B == 8 ? im::blocked_factor_solve_kernel<8> : im::blocked_factor_solve_kernel<16>;
   if (lds_bytes > 64 * 1024)
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-  hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, M, ldM, nM, block_idx, y, ldy, U,
-                     x, ldx, nv, pad);
+  // The pivots of a tile are one wavefront's work whatever the workgroup size, so a small matrix
+  // takes fewer wavefronts per world and more worlds are resident per CU (measured on g1, snu and
+  // the 128-dof stress shape: 64 threads up to pad 48, 128 for 16 x 16 tiles at pad 64, else 256).
+  const int threads = pad <= 48 ? 64 : (pad <= 64 && B == 16) ? 128 : 256;
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(threads), lds_bytes, (hipStream_t)stream, M, ldM, nM, block_idx, y,
+                     ldy, U, x, ldx, nv, pad);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }
