@@ -305,7 +305,7 @@ __device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pa
 }
 
 template <int B>
-__global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
+__global__ __launch_bounds__(1024) void blocked_factor_solve_kernel(
     const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
     const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
     int64_t ldx, int nv, int pad) {
@@ -337,7 +337,7 @@ __global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
 // :614-742 (stage), :451-470 (hessian_step), :473-611 (augmented factor).  search = -x,
 // search_dot = x.x, decrement = grad.x (strided over 64 lanes, shuffle-down tree).
 template <int B>
-__global__ __launch_bounds__(256) void dense_update_factor_kernel(
+__global__ __launch_bounds__(1024) void dense_update_factor_kernel(
     const uint8_t *__restrict__ done, const int32_t *__restrict__ state_changes,
     const int32_t *__restrict__ changes, const int32_t *__restrict__ ids, int ld_ids,
     const float *__restrict__ J, int njmax, const float *__restrict__ D, const int32_t *__restrict__ state,
@@ -687,8 +687,9 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   // The pivots of a tile are one wavefront's work whatever the workgroup size, so a small matrix
   // takes fewer wavefronts per world and more worlds are resident per CU (measured on g1, snu and
-  // the 128-dof stress shape: 64 threads up to pad 48, 128 for 16 x 16 tiles at pad 64, else 256).
-  const int threads = pad <= 48 ? 64 : (pad <= 64 && B == 16) ? 128 : 256;
+  // the 128-dof stress shape: 64 threads up to pad 48, 128 for 16 x 16 tiles at pad 64, 256 up to
+  // pad 96, 512 beyond: one workgroup per CU there, the block rows' parallel parts want the lanes).
+  const int threads = pad <= 48 ? 64 : (pad <= 64 && B == 16) ? 128 : pad <= 96 ? 256 : 512;
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(threads), lds_bytes, (hipStream_t)stream, M, ldM, nM, block_idx, y,
                      ldy, U, x, ldx, nv, pad);
   IM_HIP_CHECK(hipGetLastError());
@@ -733,7 +734,8 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
   auto fn = im::dense_update_factor_kernel<B>;
   if (lds_bytes > 64 * 1024)
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-  hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
+  // a large matrix holds a CU alone: the pair sums and the copies of H and U want every lane
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(nv_pad <= 96 ? 256 : 1024), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
                      ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, U, dof_union, search, ld_search,
                      search_dot, decrement, nv, nv_pad, row_cap);
   IM_HIP_CHECK(hipGetLastError());
