@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # 64 MiB device copy in the same run (FETCH_SIZE reads 32781 KiB for it, WRITE_SIZE 65536):
 #   (15862.14 * 65536 / 32781.48 + 448.0 * 65536 / 65536) KiB
 # Recorded in profiles/tree_row16_humanoid_pmc.txt.
-TRAFFIC_BYTES_PER_LAUNCH = int((15854.98 * 65536 / 32781.60 + 448.0) * 1024)
+TRAFFIC_BYTES_PER_LAUNCH = int((15854.27 * 65536 / 32781.46 + 448.0) * 1024)
 
 
 def algorithmic_bytes(nv: int, nM: int, nefc: int) -> int:
