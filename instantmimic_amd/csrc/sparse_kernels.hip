@@ -521,12 +521,13 @@ __global__ __launch_bounds__(256, 4) void sparse_update_wave_kernel(
   if (w >= nworld || (done && done[w]) || state_changes[w] == 0) return;
   const int n = Q.nv, nslots = Q.nslots, nfac = nslots - n, rhs = nfac;
   const int nw = (A.block + 31) / 32;
-  const int per_world = (nslots + n + 2 * nw + n + kStagedRows * (n + 1) + 3) & ~3;
+  const int per_world = (nslots + n + 2 * nw + 2 * n + kStagedRows * (n + 1) + 3) & ~3;
   float *N = lds + A.staged_words + A.solve_words + wv * per_world;  // [nslots]
   float *iD = N + nslots;                            // [n]
   float *red = iD + n;                               // [2][nw]
   int *ul = (int *)(red + 2 * nw);                   // [n] ascending dofs touched by the changed rows
-  float *jr = (float *)(ul + n);                     // [kStagedRows][n] changed rows of J
+  unsigned *mkl = (unsigned *)(ul + n);              // [n] per dof: bit t set where staged row t is nonzero there
+  float *jr = (float *)(mkl + n);                    // [kStagedRows][n] changed rows of J
   float *sd = jr + kStagedRows * n;                  // [kStagedRows] D of the row, negated for a row that left the quadratic state
   float *U = U_ + (size_t)w * Q.nv_pad * Q.nv_pad;
   const float *gw = grad + (size_t)w * ldg;
@@ -564,7 +565,10 @@ __global__ __launch_bounds__(256, 4) void sparse_update_wave_kernel(
     bool hit = false;
     if (lane < n) {
       if (staged) {
-        for (int t = 0; t < count; ++t) hit = hit || jr[t * n + lane] != 0.0f;
+        unsigned mk = 0u;
+        for (int t = 0; t < count; ++t) mk |= (unsigned)(jr[t * n + lane] != 0.0f) << t;
+        mkl[lane] = mk;
+        hit = mk != 0u;
       } else {
         for (int t = 0; t < count && !hit; ++t) hit = Jw[idw[t] * n + lane] != 0.0f;
       }
@@ -596,10 +600,11 @@ __global__ __launch_bounds__(256, 4) void sparse_update_wave_kernel(
       for (int k = 0; k < 4; ++k) {
         float delta = 0.0f;
         if (staged) {
-          for (int t = 0; t < count; ++t) {
-            const float a = jr[t * n + row[k]], b = jr[t * n + col[k]];
-            const float da = sd[t] * a;
-            if (a != 0.0f && b != 0.0f) delta = fma_(da, b, delta);
+          // only the rows in which both dofs are nonzero add to the pair, ascending: most pairs
+          // of the union share no row at all
+          for (unsigned mm = mkl[row[k]] & mkl[col[k]]; mm; mm &= mm - 1u) {
+            const int t = __builtin_ctz(mm);
+            delta = fma_(sd[t] * jr[t * n + row[k]], jr[t * n + col[k]], delta);
           }
         } else {
           for (int t = 0; t < count; ++t) {
@@ -914,7 +919,7 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done, con
     A.block = plan->block;
     A.nM = 0;
     const size_t per_world =
-        ((size_t)plan->nslots + n + 2 * nw + n + (size_t)im::kStagedRows * (n + 1) + 3) & ~(size_t)3;
+        ((size_t)plan->nslots + n + 2 * nw + 2 * n + (size_t)im::kStagedRows * (n + 1) + 3) & ~(size_t)3;
     const int32_t *solve_end = plan->t[im::RK] + ((plan->sizes[im::RK] + 3) & ~3);
     const size_t solve_words = (size_t)(solve_end - plan->t[im::FL]);
     for (int i = 0; i < 5; ++i) A.solve[i] = (int)(plan->t[im::FL + i] - plan->t[im::FL]);
