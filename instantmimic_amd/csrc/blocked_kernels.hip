@@ -350,7 +350,8 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
   float *A = rhs + pad;       // [(pad / B) * B * B]
   float *L = A + (pad / B) * B * B;  // [B * B + B]: lower factor of the diagonal tile, 1 / pivots
   int *ul = (int *)(L + B * B + B);  // [nv] union list, [nv] = its length
-  float *jr = (float *)(ul + nv + 1);  // [row_cap][nv] changed rows of J, then [row_cap] signed weights
+  unsigned *mkl = (unsigned *)(ul + nv + 1);  // [nv] per dof: bit t set where staged row t is nonzero there
+  float *jr = (float *)(mkl + nv);  // [row_cap][nv] changed rows of J, then [row_cap] signed weights
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
   if ((done && done[w]) || state_changes[w] == 0) return;
@@ -417,7 +418,10 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
         bool hit = false;
         if (dof < nv) {
           if (staged) {
-            for (int t = 0; t < count; ++t) hit = hit || jr[t * nv + dof] != 0.0f;
+            unsigned mk = 0u;
+            for (int t = 0; t < count; ++t) mk |= (unsigned)(jr[t * nv + dof] != 0.0f) << t;
+            mkl[dof] = mk;
+            hit = mk != 0u;
           } else {
             for (int t = 0; t < count && !hit; ++t) hit = Jw[(size_t)idw[t] * nv + dof] != 0.0f;
           }
@@ -441,25 +445,10 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
       const int row = ul[e - cj * (cj + 1) / 2], col = ul[cj];
       float delta = 0.0f;
       if (staged) {
-        int t = 0;
-        for (; t + 3 < count; t += 4) {  // four rows' operands read before the first is used
-          float a[4], b[4], d[4];
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            a[k] = jr[(t + k) * nv + row];
-            b[k] = jr[(t + k) * nv + col];
-            d[k] = sd[t + k];
-          }
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const float da = d[k] * a[k];  // -(D a) == (-D) a exactly
-            if (a[k] != 0.0f && b[k] != 0.0f) delta = fma_(da, b[k], delta);
-          }
-        }
-        for (; t < count; ++t) {
-          const float a = jr[t * nv + row], b = jr[t * nv + col];
-          const float da = sd[t] * a;
-          if (a != 0.0f && b != 0.0f) delta = fma_(da, b, delta);
+        // only the rows in which both dofs are nonzero add to the pair, ascending
+        for (unsigned mm = mkl[row] & mkl[col]; mm; mm &= mm - 1u) {
+          const int t = __builtin_ctz(mm);
+          delta = fma_(sd[t] * jr[t * nv + row], jr[t * nv + col], delta);  // -(D a) == (-D) a exactly
         }
         if (delta != 0.0f) {
           const float h = U[row * pad + col] + delta;
@@ -725,7 +714,7 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
   if (((uintptr_t)H | (uintptr_t)U) & 15) return IM_ERR_STRIDE;  // read and written 16 bytes at a time
   constexpr int B = 16;
   const size_t base_bytes =
-      sizeof(float) * ((size_t)nv_pad * nv_pad + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + B + nv + 1);
+      sizeof(float) * ((size_t)nv_pad * nv_pad + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + B + 2 * (size_t)nv + 1);
   if (base_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   // room for up to 32 changed rows of J next to the factor, as far as the 160 KB of LDS reach
   int row_cap = ld_ids < 32 ? ld_ids : 32;
