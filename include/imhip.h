@@ -255,13 +255,18 @@ typedef struct im_muscle_segments {
  * rows = torque dofs and other = muscle (build_torque_sparse_segment_entries,
  * muscle_qfrc_projector.py:378-456), rows = muscles and other = torque dof
  * (build_muscle_sparse_torque_entries, :459-510), or rows = (muscle, dof) entries and
- * other unused (MuscleDofSparseEntries, :513-533). */
+ * other unused (MuscleDofSparseEntries, :513-533).
+ * nother bounds the column that is not the row: every `other` is in [0, nother) (the muscle
+ * count, or the torque dof count); for the third kind it is the torque dof count, which
+ * bounds muscle_dof_torque_idx.  0 = not stated: the contractions then take their
+ * one-thread-per-output kernels, which need no bound and are several times slower. */
 typedef struct im_muscle_entries {
   const int32_t *offsets; /* nrow + 1 */
   const int32_t *segment; /* nentry */
   const int32_t *other;   /* nentry or null */
   const float *start_coeff, *end_coeff;
   int32_t nrow, nentry;
+  int32_t nother;
 } im_muscle_entries;
 
 /* Replaces _transform_waypoints_from_torch_kernel

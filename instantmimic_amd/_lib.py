@@ -63,7 +63,7 @@ class MuscleSegments(C.Structure):
 class MuscleEntries(C.Structure):
     _fields_ = [
         ("offsets", _vp), ("segment", _vp), ("other", _vp), ("start_coeff", _vp), ("end_coeff", _vp),
-        ("nrow", C.c_int32), ("nentry", C.c_int32),
+        ("nrow", C.c_int32), ("nentry", C.c_int32), ("nother", C.c_int32),
     ]  # fmt: skip
 
 

@@ -265,10 +265,13 @@ __global__ __launch_bounds__(256) void torque_bounds_kernel(
 // One workgroup of 1024 threads per world (two of them share a CU; measured against 256 and
 // 512 threads, which were 20 % and 8 % slower on the 553-segment rig).
 // The four contractions above visit every applied segment once per (segment, dof) entry and
-// redo its square root and three divisions each time.  Here a workgroup first leaves each
-// segment's unit direction and its two lever vectors in LDS, then every thread evaluates
-// entries (same operations, same order as contribution()), and a last pass adds each output's
-// entries in list order.  Results equal the one-thread-per-output kernels bit for bit.
+// redo its square root and three divisions each time, and they fetch a muscle's force and a
+// dof's motion axis from memory once per entry.  Here a workgroup first leaves in LDS each
+// segment's unit direction and its two lever vectors, every muscle's force and every torque
+// dof's axis; then every thread evaluates entries (same operations, same order as
+// contribution()), and a last pass adds each output's entries in list order, reading them
+// several at a time so that only the additions wait on one another.  Results equal the
+// one-thread-per-output kernels bit for bit.
 enum { MW_FORWARD, MW_GRAD, MW_BOUNDS, MW_MOMENT };
 
 struct MwArgs {
@@ -281,47 +284,90 @@ struct MwArgs {
   float *out0, *out1;
   int64_t ldo;
   int root, nrow, nentry, nseg;
+  int ntorque, nmuscle;  // sizes of the staged axes and forces (nmuscle 0 for MW_MOMENT)
 };
 
-// force of one muscle as the contraction sees it
+constexpr int kContribPad = 4;  // floats read past the last entry by ordered_sum()
+struct MwLds {
+  float *segd;     // [nseg][9]: dir (0 for a degenerate segment), p0 - c0, p1 - c1
+  float *contrib;  // [nentry]
+  float *axis;     // [ntorque][6]: the dof's cdof
+  float *force;    // [nmuscle]: force of a muscle as the contraction sees it
+  float *gout;     // [ntorque], MW_GRAD only
+  unsigned short *rowid;  // [nentry]
+};
 template <int MODE>
-__device__ __forceinline__ float muscle_force(const MwArgs &a, int64_t w, int muscle) {
-  if (MODE == MW_FORWARD) {
-    float f = a.unit[w * a.ldu + muscle] * a.act[w * a.lda + muscle];
-    if (a.passive) f = f + a.passive[w * a.ldpa + muscle];
-    return f;
-  }
-  return a.unit[w * a.ldu + muscle];
+__host__ __device__ inline size_t mw_lds_floats(const MwArgs &a) {
+  return (size_t)9 * a.nseg + (size_t)a.nentry + kContribPad + (size_t)6 * a.ntorque + (size_t)a.nmuscle +
+         (MODE == MW_GRAD ? (size_t)a.ntorque : 0);
 }
 
 template <int MODE>
-__device__ __forceinline__ float entry_contribution(const MwArgs &a, const float *segd,
-                                                    const unsigned short *rowid, const float *cdof,
-                                                    int64_t w, int e) {
-  const int r = rowid[e];
+__device__ __forceinline__ float entry_contribution(const MwArgs &a, const MwLds &l, int e) {
+  const int r = l.rowid[e];
   int torque, muscle;
   if (MODE == MW_GRAD) { muscle = r; torque = a.e_other[e]; }
   else if (MODE == MW_MOMENT) { muscle = 0; torque = a.row_torque[r]; }
   else { torque = r; muscle = a.e_other[e]; }
   float f = 1.0f;
-  if (MODE != MW_MOMENT) f = muscle_force<MODE>(a, w, muscle);
-  const float *cd = cdof + 6 * (int64_t)(torque + a.root);
+  if (MODE != MW_MOMENT) f = l.force[muscle];
+  const float *cd = l.axis + 6 * torque;
   const V3 ang = ld3(cd), lin = ld3(cd + 3);
-  const float *sd = segd + 9 * a.e_seg[e];
+  const float *sd = l.segd + 9 * a.e_seg[e];
   const V3 dir = {sd[0], sd[1], sd[2]}, r0 = {sd[3], sd[4], sd[5]}, r1 = {sd[6], sd[7], sd[8]};
   const V3 fv = scale(f, dir);
   const V3 st = add(lin, cross(ang, r0));
   const V3 en = add(lin, cross(ang, r1));
   // an entry whose force is zero is skipped by the reference: it enters the sum as 0
-  return f == 0.0f ? 0.0f : dot(sub(scale(a.e_a[e], st), scale(a.e_b[e], en)), fv);
+  float c = f == 0.0f ? 0.0f : dot(sub(scale(a.e_a[e], st), scale(a.e_b[e], en)), fv);
+  if (MODE == MW_GRAD) c = l.gout[torque] * c;
+  return c;
+}
+
+// Sum of contrib[e0..e1) in list order from +0.  Whole groups of 16 (LONG) and of 4 entries are
+// read with one address and added without a test; the last group reads up to three floats past
+// e1 (contrib is padded for that) and enters them as +0, which leaves every bit of a sum that
+// started at +0 (such a sum is never -0).
+template <bool LONG>
+__device__ __forceinline__ float ordered_sum(const float *contrib, int e0, int e1) {
+  float total = 0.0f;
+  int e = e0;
+  if (LONG) {
+    for (; e + 16 <= e1; e += 16) {
+      float c[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) c[k] = contrib[e + k];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) total = total + c[k];
+    }
+  }
+  for (; e + 4 <= e1; e += 4) {
+    float c[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) c[k] = contrib[e + k];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) total = total + c[k];
+  }
+  if (e < e1) {
+    float c[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) c[k] = contrib[e + k];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) total = total + (e + k < e1 ? c[k] : 0.0f);
+  }
+  return total;
 }
 
 template <int MODE>
 __global__ __launch_bounds__(1024) void muscle_world_kernel(MwArgs a) {
   extern __shared__ float lds[];
-  float *segd = lds;                           // [nseg][9]: dir (0 for a degenerate segment), p0 - c0, p1 - c1
-  float *contrib = segd + 9 * a.nseg;          // [nentry]
-  unsigned short *rowid = (unsigned short *)(contrib + a.nentry);  // [nentry]
+  MwLds l;
+  l.segd = lds;
+  l.contrib = l.segd + 9 * a.nseg;
+  l.axis = l.contrib + a.nentry + kContribPad;
+  l.force = l.axis + 6 * a.ntorque;
+  l.gout = l.force + a.nmuscle;
+  l.rowid = (unsigned short *)(lds + mw_lds_floats<MODE>(a));
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
   const float *wp = a.g.wp + w * a.g.ldw, *com = a.g.com + w * a.g.ldc, *cdof = a.g.cdof + w * a.g.ldd;
@@ -334,45 +380,55 @@ __global__ __launch_bounds__(1024) void muscle_world_kernel(MwArgs a) {
     const V3 r0 = sub(p0, c0), r1 = sub(p1, c1);
     // a degenerate segment contributes nothing: with a zero direction its entries come out as
     // +-0, and adding +-0 to a sum that started at +0 leaves every bit of it
-    float *o = segd + 9 * sg;
+    float *o = l.segd + 9 * sg;
     o[0] = ok ? seg.x / len : 0.0f;
     o[1] = ok ? seg.y / len : 0.0f;
     o[2] = ok ? seg.z / len : 0.0f;
     o[3] = r0.x; o[4] = r0.y; o[5] = r0.z;
     o[6] = r1.x; o[7] = r1.y; o[8] = r1.z;
   }
-  for (int r = tid; r < a.nrow; r += nt)
-    for (int e = a.offsets[r]; e < a.offsets[r + 1]; ++e) rowid[e] = (unsigned short)r;
-  __syncthreads();
-  // four entries per thread and trip, each read from a clamped index so that all their loads
-  // are issued before the first is needed
-  for (int e = tid; e < a.nentry; e += 4 * nt) {
-    float c[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int ee = e + k * nt < a.nentry ? e + k * nt : a.nentry - 1;
-      c[k] = entry_contribution<MODE>(a, segd, rowid, cdof, w, ee);
+  for (int i = tid; i < 6 * a.ntorque; i += nt) l.axis[i] = cdof[6 * a.root + i];
+  for (int m = tid; m < a.nmuscle; m += nt) {
+    float f = a.unit[w * a.ldu + m];
+    if (MODE == MW_FORWARD) {
+      f = f * a.act[w * a.lda + m];
+      if (a.passive) f = f + a.passive[w * a.ldpa + m];
     }
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-      if (e + k * nt < a.nentry) contrib[e + k * nt] = c[k];
+    l.force[m] = f;
+  }
+  if (MODE == MW_GRAD)
+    for (int j = tid; j < a.ntorque; j += nt) l.gout[j] = a.gout[w * a.ldg + j];
+  if (a.nentry < 32 * a.nrow) {  // short rows: a thread writes its row's
+    for (int r = tid; r < a.nrow; r += nt)
+      for (int e = a.offsets[r]; e < a.offsets[r + 1]; ++e) l.rowid[e] = (unsigned short)r;
+  } else {  // long rows: a wave writes a row's
+    for (int r = tid >> 6; r < a.nrow; r += nt >> 6)
+      for (int e = a.offsets[r] + (tid & 63); e < a.offsets[r + 1]; e += 64) l.rowid[e] = (unsigned short)r;
   }
   __syncthreads();
+  // four entries per thread and trip while whole trips remain (all their loads are issued
+  // before the first is needed), then one entry per thread
+  int base = 0;
+  for (; base + 4 * nt <= a.nentry; base += 4 * nt) {
+    float c[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) c[k] = entry_contribution<MODE>(a, l, base + k * nt + tid);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) l.contrib[base + k * nt + tid] = c[k];
+  }
+  for (int e = base + tid; e < a.nentry; e += nt) l.contrib[e] = entry_contribution<MODE>(a, l, e);
+  __syncthreads();
+  const float *contrib = l.contrib;
   for (int r = tid; r < a.nrow; r += nt) {
     const int e0 = a.offsets[r], e1 = a.offsets[r + 1];
     if (MODE == MW_FORWARD) {
-      float total = 0.0f;
-      for (int e = e0; e < e1; ++e) total = total + contrib[e];
-      a.out0[w * a.ldo + r] = total;
+      a.out0[w * a.ldo + r] = ordered_sum<true>(contrib, e0, e1);
+    } else if (MODE == MW_MOMENT) {  // a (muscle, dof) pair has a few segments
+      a.out0[w * a.ldo + r] = ordered_sum<false>(contrib, e0, e1);
     } else if (MODE == MW_GRAD) {
-      float grad = 0.0f;
-      if (a.unit[w * a.ldu + r] != 0.0f)
-        for (int e = e0; e < e1; ++e) grad = grad + a.gout[w * a.ldg + a.e_other[e]] * contrib[e];
-      a.out0[w * a.ldo + r] = grad;
-    } else if (MODE == MW_MOMENT) {
-      float total = 0.0f;
-      for (int e = e0; e < e1; ++e) total = total + contrib[e];
-      a.out0[w * a.ldo + r] = total;
+      // The one-thread-per-muscle kernel leaves 0 for a muscle without force; its entries are
+      // 0 here as well (gout * 0), but an infinite gout would turn them into NaN
+      a.out0[w * a.ldo + r] = l.force[r] != 0.0f ? ordered_sum<true>(contrib, e0, e1) : 0.0f;
     } else {
       int current = -1;
       float total = 0.0f, lo = 0.0f, hi = 0.0f;
@@ -396,17 +452,19 @@ __global__ __launch_bounds__(1024) void muscle_world_kernel(MwArgs a) {
   }
 }
 
-// Launches the workgroup-per-world kernel when a world's segments and entries fit in LDS;
-// returns false for the caller to use the one-thread-per-output kernel instead.
+// Launches the workgroup-per-world kernel when a world's segments and entries fit in LDS and
+// the entry list states the range of its `other` column; returns false for the caller to use
+// the one-thread-per-output kernel instead.
 template <int MODE>
 bool launch_world(const MwArgs &a, int nworld, hipStream_t stream) {
-  const size_t lds_bytes = 4 * ((size_t)9 * a.nseg + (size_t)a.nentry) +
-                           2 * (((size_t)a.nentry + 1) & ~(size_t)1);
+  const size_t lds_bytes = 4 * mw_lds_floats<MODE>(a) + 2 * (((size_t)a.nentry + 1) & ~(size_t)1);
   static const bool forced_off = [] {
     const char *e = std::getenv("IMHIP_MUSCLE_KERNEL");
     return e && std::strcmp(e, "simple") == 0;
   }();
-  if (forced_off || lds_bytes > 64 * 1024 || a.nentry == 0 || a.nseg == 0 || a.nrow > 65535) return false;
+  if (forced_off || lds_bytes > 64 * 1024 || a.nentry == 0 || a.nseg == 0 || a.nrow > 65535 ||
+      a.ntorque <= 0 || (MODE != MW_MOMENT && a.nmuscle <= 0))
+    return false;
   hipLaunchKernelGGL(muscle_world_kernel<MODE>, dim3((unsigned)nworld), dim3(1024), lds_bytes, stream, a);
   return true;
 }
@@ -515,7 +573,7 @@ extern "C" int im_muscle_torque_forward(const im_muscle_geometry *geometry,
              torque_entries->other, nullptr, torque_entries->start_coeff, torque_entries->end_coeff,
              unit_force, passive_force, activation, nullptr, ld_unit, ld_passive, ld_activation, 0,
              torque, nullptr, ld_torque, root_dof_count, nt, torque_entries->nentry,
-             segments->nsegment};
+             segments->nsegment, nt, torque_entries->nother};
     if (launch_world<MW_FORWARD>(a, nworld, (hipStream_t)stream)) {
       IM_HIP_CHECK(hipGetLastError());
       return IM_OK;
@@ -558,7 +616,7 @@ extern "C" int im_muscle_activation_grad(const im_muscle_geometry *geometry,
              muscle_entries->other, nullptr, muscle_entries->start_coeff, muscle_entries->end_coeff,
              unit_force, nullptr, nullptr, grad_output, ld_unit, 0, 0, ld_grad_output,
              grad_activation, nullptr, ld_grad_activation, root_dof_count, nm, muscle_entries->nentry,
-             segments->nsegment};
+             segments->nsegment, muscle_entries->nother, nm};
     if (launch_world<MW_GRAD>(a, nworld, (hipStream_t)stream)) {
       IM_HIP_CHECK(hipGetLastError());
       return IM_OK;
@@ -598,7 +656,7 @@ extern "C" int im_muscle_sparse_moment(const im_muscle_geometry *geometry,
     MwArgs a{geo(geometry), seg(segments), entry_segments->offsets, entry_segments->segment, nullptr,
              muscle_dof_torque_idx, entry_segments->start_coeff, entry_segments->end_coeff, nullptr,
              nullptr, nullptr, nullptr, 0, 0, 0, 0, moment, nullptr, ld_moment, root_dof_count, ne,
-             entry_segments->nentry, segments->nsegment};
+             entry_segments->nentry, segments->nsegment, entry_segments->nother, 0};
     if (launch_world<MW_MOMENT>(a, nworld, (hipStream_t)stream)) {
       IM_HIP_CHECK(hipGetLastError());
       return IM_OK;
@@ -636,7 +694,8 @@ extern "C" int im_muscle_torque_bounds(const im_muscle_geometry *geometry,
     MwArgs a{geo(geometry), seg(segments), torque_entries->offsets, torque_entries->segment,
              torque_entries->other, nullptr, torque_entries->start_coeff, torque_entries->end_coeff,
              unit_force, nullptr, nullptr, nullptr, ld_unit, 0, 0, 0, lower, upper, ld_bounds,
-             root_dof_count, nt, torque_entries->nentry, segments->nsegment};
+             root_dof_count, nt, torque_entries->nentry, segments->nsegment, nt,
+             torque_entries->nother};
     if (launch_world<MW_BOUNDS>(a, nworld, (hipStream_t)stream)) {
       IM_HIP_CHECK(hipGetLastError());
       return IM_OK;

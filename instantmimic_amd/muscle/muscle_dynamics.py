@@ -276,16 +276,16 @@ class MuscleDynamicsLayer:
         p = [t.data_ptr() for t in d["seg"]]
         self._segments = _lib.MuscleSegments(*p, len(self.segments_host[0]))
 
-        def entries(ts, nrow, other=True):
+        def entries(ts, nrow, nother, other=True):
             off, seg = ts[0], ts[1]
             rest = ts[2:]
             o = rest[0].data_ptr() if other else None
             a, b = (rest[1], rest[2]) if other else (rest[0], rest[1])
-            return _lib.MuscleEntries(off.data_ptr(), seg.data_ptr(), o, a.data_ptr(), b.data_ptr(), nrow, seg.numel())
+            return _lib.MuscleEntries(off.data_ptr(), seg.data_ptr(), o, a.data_ptr(), b.data_ptr(), nrow, seg.numel(), nother)
 
-        self._torque_entries = entries(d["tq"], self.torque_dim)
-        self._muscle_entries = entries(d["ms"], self.muscle_count)
-        self._moment_entries = entries(d["mom"], len(e.muscle_dof_torque_idx), other=False)
+        self._torque_entries = entries(d["tq"], self.torque_dim, self.muscle_count)
+        self._muscle_entries = entries(d["ms"], self.muscle_count, self.torque_dim)
+        self._moment_entries = entries(d["mom"], len(e.muscle_dof_torque_idx), self.torque_dim, other=False)
 
     def _need_gpu(self, *tensors):
         import torch
