@@ -291,6 +291,24 @@ int im_muscle_force_magnitudes(const float *waypoints, int64_t ld_waypoints,
                                float *unit_force, int64_t ld_unit, float *passive_force,
                                int64_t ld_passive, int nworld, void *stream);
 
+/* im_muscle_waypoints followed by im_muscle_force_magnitudes in one launch, for the caller
+ * that wants both: MuscleDynamicsLayer._prepare_warp_waypoint_geometry
+ * (src/instantmimic/muscle/muscle_dynamics.py:4344-4500) launches the two kernels one after
+ * the other on the same workspace.  A workgroup keeps its world's waypoints in LDS between
+ * the two steps, so they are written once and not read back; results are those of the two
+ * calls bit for bit.  More than 5461 waypoints (64 KiB) fall back to the two launches.
+ * Arguments as in the two calls. */
+int im_muscle_waypoints_forces(const float *xpos, int64_t ld_xpos, const float *xquat,
+                               int64_t ld_xquat, const int32_t *waypoint_body,
+                               const float *waypoint_local, int nwaypoint, float *waypoints,
+                               int64_t ld_waypoints, const int32_t *all_segment_start_idx,
+                               const int32_t *all_muscle_segment_offsets,
+                               const float *muscle_params, int ld_params,
+                               const float *muscle_rest_length,
+                               const im_muscle_force_model *model, int nmuscle,
+                               float *unit_force, int64_t ld_unit, float *passive_force,
+                               int64_t ld_passive, int nworld, void *stream);
+
 /* Replaces _compute_muscle_dynamics_from_activation_sparse_kernel
  * (muscle_dynamics_kernels.py:1707-1793), the body of the operator
  * instantmimic_muscle::torque_forward (src/instantmimic/muscle/warp_custom_ops.py:98-114).

@@ -110,6 +110,11 @@ SIGNATURES = {
         _i,
         [_vp, _i64, _vp, _vp, _vp, _i, _vp, C.POINTER(MuscleForceModel), _i, _vp, _i64, _vp, _i64, _i, _vp],
     ),
+    "im_muscle_waypoints_forces": (
+        _i,
+        [_vp, _i64, _vp, _i64, _vp, _vp, _i, _vp, _i64, _vp, _vp, _vp, _i, _vp, C.POINTER(MuscleForceModel), _i,
+         _vp, _i64, _vp, _i64, _i, _vp],
+    ),  # fmt: skip
     "im_muscle_torque_forward": (
         _i,
         [_pgeo, _pseg, _pent, _vp, _i64, _vp, _i64, _vp, _i64, _i, _vp, _i64, _i, _vp],

@@ -73,15 +73,14 @@ __device__ __forceinline__ float seg_term(const Geo &g, const Seg &s, int64_t w,
                       ld3(com + 3 * s.b0[seg]), ld3(com + 3 * s.b1[seg]), a, b, force);
 }
 
-__global__ __launch_bounds__(256) void waypoints_kernel(
-    const float *__restrict__ xpos, int64_t ldp, const float *__restrict__ xquat, int64_t ldq,
-    const int32_t *__restrict__ wp_body, const float *__restrict__ wp_local, int nwp,
-    float *__restrict__ out, int64_t ldo, int nworld) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t w = blockIdx.y;
-  if (i >= nwp) return;
+// One waypoint in the world frame: the body's position plus its local offset turned by the
+// body's (renormalised) quaternion.  xpos and xquat are one world's rows.
+__device__ __forceinline__ V3 world_waypoint(const float *__restrict__ xpos,
+                                             const float *__restrict__ xquat,
+                                             const int32_t *__restrict__ wp_body,
+                                             const float *__restrict__ wp_local, int i) {
   const int b = wp_body[i];
-  const float *q = xquat + w * ldq + 4 * b;
+  const float *q = xquat + 4 * b;
   const float q0 = q[0], q1 = q[1], q2 = q[2], q3 = q[3];
   // muscle_qfrc_projector.py:91-100
   const float inv = 1.0f / sqrtf(q0 * q0 + q1 * q1 + q2 * q2 + q3 * q3 + 1.0e-8f);
@@ -91,7 +90,17 @@ __global__ __launch_bounds__(256) void waypoints_kernel(
   // mujoco_warp math.rot_vec_quat: 2 (u.v) u + (s s - u.u) v + 2 s (u x v)
   V3 r = add(scale(2.0f, scale(dot(u, v), u)), scale(s * s - dot(u, u), v));
   r = add(r, scale(2.0f * s, cross(u, v)));
-  const V3 p = add(ld3(xpos + w * ldp + 3 * b), r);
+  return add(ld3(xpos + 3 * b), r);
+}
+
+__global__ __launch_bounds__(256) void waypoints_kernel(
+    const float *__restrict__ xpos, int64_t ldp, const float *__restrict__ xquat, int64_t ldq,
+    const int32_t *__restrict__ wp_body, const float *__restrict__ wp_local, int nwp,
+    float *__restrict__ out, int64_t ldo, int nworld) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t w = blockIdx.y;
+  if (i >= nwp) return;
+  const V3 p = world_waypoint(xpos + w * ldp, xquat + w * ldq, wp_body, wp_local, i);
   float *o = out + w * ldo + 3 * i;
   o[0] = p.x;
   o[1] = p.y;
@@ -136,15 +145,12 @@ __device__ __forceinline__ float passive_fl(float l, const float *m) {
   return fpmax * (0.5f + (l - mid) / width);
 }
 
-__global__ __launch_bounds__(256) void force_kernel(
-    const float *__restrict__ wp, int64_t ldw, const int32_t *__restrict__ seg_start,
+// Length of muscle m along one world's waypoints and its force magnitudes.
+__device__ __forceinline__ void muscle_force_magnitudes(
+    const float *row, const int32_t *__restrict__ seg_start,
     const int32_t *__restrict__ seg_offsets, const float *__restrict__ params, int ldpar,
-    const float *__restrict__ rest, im_muscle_force_model model, int nmuscle,
-    float *__restrict__ unit, int64_t ldu, float *__restrict__ passive, int64_t ldpa) {
-  const int m = blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t w = blockIdx.y;
-  if (m >= nmuscle) return;
-  const float *row = wp + w * ldw;
+    const float *__restrict__ rest, const im_muscle_force_model &model, int m, float *unit,
+    float *passive) {
   float len = 0.0f;  // muscle_dynamics_kernels.py:452-473
   for (int s = seg_offsets[m]; s < seg_offsets[m + 1]; ++s) {
     const int i = seg_start[s];
@@ -157,14 +163,53 @@ __global__ __launch_bounds__(256) void force_kernel(
   const float ln =
       fminf(fmaxf(lm / fmaxf(lm0, 1.0e-6f), model.length_norm_min), model.length_norm_max);
   const float c = cosf(pen);
-  unit[w * ldu + m] = f0 * active_fl(ln, model.active) * c * model.force_scale;
+  *unit = f0 * active_fl(ln, model.active) * c * model.force_scale;
   if (passive) {
     float pv = 0.0f;
     // muscle_qfrc_projector.py:249-277 with include_active 0, include_passive 1
     if (model.include_passive)
       pv = f0 * passive_fl(ln, model.passive) * c * model.force_scale;
-    passive[w * ldpa + m] = pv;
+    *passive = pv;
   }
+}
+
+__global__ __launch_bounds__(256) void force_kernel(
+    const float *__restrict__ wp, int64_t ldw, const int32_t *__restrict__ seg_start,
+    const int32_t *__restrict__ seg_offsets, const float *__restrict__ params, int ldpar,
+    const float *__restrict__ rest, im_muscle_force_model model, int nmuscle,
+    float *__restrict__ unit, int64_t ldu, float *__restrict__ passive, int64_t ldpa) {
+  const int m = blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t w = blockIdx.y;
+  if (m >= nmuscle) return;
+  muscle_force_magnitudes(wp + w * ldw, seg_start, seg_offsets, params, ldpar, rest, model, m,
+                          unit + w * ldu + m, passive ? passive + w * ldpa + m : nullptr);
+}
+
+// Waypoints and force magnitudes of one world in one workgroup: the waypoints go to memory and
+// stay in LDS, from where the muscle lengths are taken.  Same operations as the two kernels
+// above, so the results are theirs bit for bit.
+__global__ __launch_bounds__(512) void waypoints_forces_kernel(
+    const float *__restrict__ xpos, int64_t ldp, const float *__restrict__ xquat, int64_t ldq,
+    const int32_t *__restrict__ wp_body, const float *__restrict__ wp_local, int nwp,
+    float *__restrict__ out, int64_t ldo, const int32_t *__restrict__ seg_start,
+    const int32_t *__restrict__ seg_offsets, const float *__restrict__ params, int ldpar,
+    const float *__restrict__ rest, im_muscle_force_model model, int nmuscle,
+    float *__restrict__ unit, int64_t ldu, float *__restrict__ passive, int64_t ldpa) {
+  extern __shared__ float wpl[];  // [3 * nwp]
+  const int64_t w = blockIdx.x;
+  const int tid = threadIdx.x, nt = blockDim.x;
+  for (int i = tid; i < nwp; i += nt) {
+    const V3 p = world_waypoint(xpos + w * ldp, xquat + w * ldq, wp_body, wp_local, i);
+    wpl[3 * i] = p.x;
+    wpl[3 * i + 1] = p.y;
+    wpl[3 * i + 2] = p.z;
+  }
+  __syncthreads();
+  float *o = out + w * ldo;
+  for (int k = tid; k < 3 * nwp; k += nt) o[k] = wpl[k];
+  for (int m = tid; m < nmuscle; m += nt)
+    muscle_force_magnitudes(wpl, seg_start, seg_offsets, params, ldpar, rest, model, m,
+                            unit + w * ldu + m, passive ? passive + w * ldpa + m : nullptr);
 }
 
 __global__ __launch_bounds__(256) void torque_forward_kernel(
@@ -537,6 +582,42 @@ extern "C" int im_muscle_force_magnitudes(const float *waypoints, int64_t ld_way
                        *model, nmuscle, unit_force + w0 * ld_unit, ld_unit,
                        passive_force ? passive_force + w0 * ld_passive : nullptr, ld_passive);
   }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_muscle_waypoints_forces(
+    const float *xpos, int64_t ld_xpos, const float *xquat, int64_t ld_xquat,
+    const int32_t *waypoint_body, const float *waypoint_local, int nwaypoint, float *waypoints,
+    int64_t ld_waypoints, const int32_t *all_segment_start_idx,
+    const int32_t *all_muscle_segment_offsets, const float *muscle_params, int ld_params,
+    const float *muscle_rest_length, const im_muscle_force_model *model, int nmuscle,
+    float *unit_force, int64_t ld_unit, float *passive_force, int64_t ld_passive, int nworld,
+    void *stream) {
+  const size_t lds_bytes = (size_t)12 * (nwaypoint > 0 ? nwaypoint : 0);
+  if (nworld <= 0 || nwaypoint <= 0 || nmuscle <= 0 || lds_bytes > 64 * 1024) {
+    // nothing to share between the two, or a world's waypoints do not fit in LDS
+    const int rc = im_muscle_waypoints(xpos, ld_xpos, xquat, ld_xquat, waypoint_body,
+                                       waypoint_local, nwaypoint, waypoints, ld_waypoints, nworld,
+                                       stream);
+    if (rc != IM_OK) return rc;
+    return im_muscle_force_magnitudes(waypoints, ld_waypoints, all_segment_start_idx,
+                                      all_muscle_segment_offsets, muscle_params, ld_params,
+                                      muscle_rest_length, model, nmuscle, unit_force, ld_unit,
+                                      passive_force, ld_passive, nworld, stream);
+  }
+  if (!model || !xpos || !xquat || !waypoint_body || !waypoint_local || !waypoints ||
+      !all_segment_start_idx || !all_muscle_segment_offsets || !muscle_params ||
+      !muscle_rest_length || !unit_force || ld_params < 4)
+    return IM_ERR_ARG;
+  if (ld_waypoints < 3 * (int64_t)nwaypoint || ld_unit < nmuscle ||
+      (passive_force && ld_passive < nmuscle))
+    return IM_ERR_STRIDE;
+  hipLaunchKernelGGL(waypoints_forces_kernel, dim3((unsigned)nworld), dim3(512), lds_bytes,
+                     (hipStream_t)stream, xpos, ld_xpos, xquat, ld_xquat, waypoint_body,
+                     waypoint_local, nwaypoint, waypoints, ld_waypoints, all_segment_start_idx,
+                     all_muscle_segment_offsets, muscle_params, ld_params, muscle_rest_length,
+                     *model, nmuscle, unit_force, ld_unit, passive_force, ld_passive);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

@@ -315,26 +315,26 @@ class MuscleDynamicsLayer:
         ws = {"transformed_waypoints": torch.empty((B, 3 * self.waypoint_count), device=raw_context.device)}
         wp = ws["transformed_waypoints"]
         L = _lib.lib()
-        _lib.check(
-            L.im_muscle_waypoints(
-                base + 4 * self._xpos_off, ld, base + 4 * self._xquat_off, ld, d["wp_body"].data_ptr(),
-                d["wp_local"].data_ptr(), self.waypoint_count, wp.data_ptr(), wp.stride(0), B, s,
-            ),
-            "im_muscle_waypoints",
+        wp_args = (
+            base + 4 * self._xpos_off, ld, base + 4 * self._xquat_off, ld, d["wp_body"].data_ptr(),
+            d["wp_local"].data_ptr(), self.waypoint_count, wp.data_ptr(), wp.stride(0),
         )  # fmt: skip
         if compute_force_magnitudes:
+            # both steps in one launch: a world's waypoints stay on chip between them
             ws["unit_force_magnitude"] = torch.empty((B, self.muscle_count), device=raw_context.device)
             ws["passive_force_magnitude"] = torch.empty((B, self.muscle_count), device=raw_context.device)
             self._model.include_passive = 1 if include_passive_force_magnitude else 0
             u, p = ws["unit_force_magnitude"], ws["passive_force_magnitude"]
             _lib.check(
-                L.im_muscle_force_magnitudes(
-                    wp.data_ptr(), wp.stride(0), d["all_seg_start"].data_ptr(), d["all_seg_off"].data_ptr(),
-                    d["params"].data_ptr(), self.muscle_params.shape[1], d["rest"].data_ptr(), C.byref(self._model),
-                    self.muscle_count, u.data_ptr(), u.stride(0), p.data_ptr(), p.stride(0), B, s,
+                L.im_muscle_waypoints_forces(
+                    *wp_args, d["all_seg_start"].data_ptr(), d["all_seg_off"].data_ptr(), d["params"].data_ptr(),
+                    self.muscle_params.shape[1], d["rest"].data_ptr(), C.byref(self._model), self.muscle_count,
+                    u.data_ptr(), u.stride(0), p.data_ptr(), p.stride(0), B, s,
                 ),
-                "im_muscle_force_magnitudes",
+                "im_muscle_waypoints_forces",
             )  # fmt: skip
+        else:
+            _lib.check(L.im_muscle_waypoints(*wp_args, B, s), "im_muscle_waypoints")
         geo = _lib.MuscleGeometry(
             wp.data_ptr(), wp.stride(0), base + 4 * self._com_off, ld, base + 4 * self._cdof_off, ld
         )

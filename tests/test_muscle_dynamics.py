@@ -564,3 +564,46 @@ def test_gpu_one_thread_per_output_kernels_agree():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
     assert out.returncode == 0 and "simple kernels ok" in out.stdout, out.stderr[-2000:]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nworld", [1, 333])
+def test_gpu_fused_geometry_equals_the_two_launches(nworld):
+    """im_muscle_waypoints_forces against im_muscle_waypoints followed by
+    im_muscle_force_magnitudes, through the C-ABI: the same bits, rows beyond the outputs'
+    widths untouched."""
+    import ctypes as C
+
+    from instantmimic_amd import _lib
+
+    rig = synth.make_muscle_rig(nmuscle=284, seed=1003)
+    layer = _gpu_layer(rig, active_force_type="gaussian", passive_force_type="exponential")
+    ctx_d = torch.from_numpy(synth.make_muscle_context(rig, nworld, seed=21)).cuda()
+    ws, _ = layer._prepare_waypoint_geometry(ctx_d, include_passive_force_magnitude=True)
+    d, L = layer._dev, _lib.lib()
+    base, ld = ctx_d.data_ptr(), ctx_d.stride(0)
+    pad = 5
+    wp = torch.full((nworld, 3 * layer.waypoint_count + pad), 7.0, device="cuda")
+    unit = torch.full((nworld, layer.muscle_count + pad), 7.0, device="cuda")
+    pas = torch.full((nworld, layer.muscle_count + pad), 7.0, device="cuda")
+    wp_args = (base + 4 * layer._xpos_off, ld, base + 4 * layer._xquat_off, ld, d["wp_body"].data_ptr(),
+               d["wp_local"].data_ptr(), layer.waypoint_count, wp.data_ptr(), wp.stride(0))  # fmt: skip
+    frc_args = (d["all_seg_start"].data_ptr(), d["all_seg_off"].data_ptr(), d["params"].data_ptr(),
+                layer.muscle_params.shape[1], d["rest"].data_ptr(), C.byref(layer._model), layer.muscle_count,
+                unit.data_ptr(), unit.stride(0), pas.data_ptr(), pas.stride(0), nworld, None)  # fmt: skip
+    _lib.check(L.im_muscle_waypoints(*wp_args, nworld, None), "im_muscle_waypoints")
+    _lib.check(L.im_muscle_force_magnitudes(wp.data_ptr(), wp.stride(0), *frc_args), "im_muscle_force_magnitudes")
+    torch.cuda.synchronize()
+    assert torch.equal(wp[:, :-pad], ws["transformed_waypoints"])
+    assert torch.equal(unit[:, :-pad], ws["unit_force_magnitude"])
+    assert torch.equal(pas[:, :-pad], ws["passive_force_magnitude"])
+    assert (wp[:, -pad:] == 7.0).all() and (unit[:, -pad:] == 7.0).all() and (pas[:, -pad:] == 7.0).all()
+    # the fused call with padded rows as well
+    wp2, unit2, pas2 = torch.full_like(wp, 3.0), torch.full_like(unit, 3.0), torch.full_like(pas, 3.0)
+    args2 = wp_args[:7] + (wp2.data_ptr(), wp2.stride(0)) + frc_args[:7] + (
+        unit2.data_ptr(), unit2.stride(0), pas2.data_ptr(), pas2.stride(0), nworld, None)  # fmt: skip
+    _lib.check(L.im_muscle_waypoints_forces(*args2), "im_muscle_waypoints_forces")
+    torch.cuda.synchronize()
+    assert torch.equal(wp2[:, :-pad], wp[:, :-pad]) and torch.equal(unit2[:, :-pad], unit[:, :-pad])
+    assert torch.equal(pas2[:, :-pad], pas[:, :-pad])
+    assert (wp2[:, -pad:] == 3.0).all() and (unit2[:, -pad:] == 3.0).all() and (pas2[:, -pad:] == 3.0).all()
