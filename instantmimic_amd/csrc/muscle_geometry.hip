@@ -347,24 +347,43 @@ __host__ __device__ inline size_t mw_lds_floats(const MwArgs &a) {
          (MODE == MW_GRAD ? (size_t)a.ntorque : 0);
 }
 
+// What the lists hold about one entry.
+struct MwEntry {
+  int row, other, seg;
+  float a, b;
+};
 template <int MODE>
-__device__ __forceinline__ float entry_contribution(const MwArgs &a, const MwLds &l, int e) {
-  const int r = l.rowid[e];
+__device__ __forceinline__ MwEntry load_entry(const MwArgs &a, const MwLds &l, int e) {
+  MwEntry t;
+  t.row = l.rowid[e];
+  t.other = MODE == MW_MOMENT ? 0 : a.e_other[e];
+  t.seg = a.e_seg[e];
+  t.a = a.e_a[e];
+  t.b = a.e_b[e];
+  return t;
+}
+
+template <int MODE>
+__device__ __forceinline__ float entry_contribution(const MwArgs &a, const MwLds &l, const MwEntry &t) {
   int torque, muscle;
-  if (MODE == MW_GRAD) { muscle = r; torque = a.e_other[e]; }
-  else if (MODE == MW_MOMENT) { muscle = 0; torque = a.row_torque[r]; }
-  else { torque = r; muscle = a.e_other[e]; }
+  if (MODE == MW_GRAD) { muscle = t.row; torque = t.other; }
+  else if (MODE == MW_MOMENT) { muscle = 0; torque = a.row_torque[t.row]; }
+  else { torque = t.row; muscle = t.other; }
   float f = 1.0f;
   if (MODE != MW_MOMENT) f = l.force[muscle];
   const float *cd = l.axis + 6 * torque;
   const V3 ang = ld3(cd), lin = ld3(cd + 3);
-  const float *sd = l.segd + 9 * a.e_seg[e];
+  const float *sd = l.segd + 9 * t.seg;
   const V3 dir = {sd[0], sd[1], sd[2]}, r0 = {sd[3], sd[4], sd[5]}, r1 = {sd[6], sd[7], sd[8]};
   const V3 fv = scale(f, dir);
   const V3 st = add(lin, cross(ang, r0));
   const V3 en = add(lin, cross(ang, r1));
+  float c = dot(sub(scale(t.a, st), scale(t.b, en)), fv);
+  // evaluated for every entry, without a branch around it: a thread's entries then proceed
+  // side by side instead of one after the other
+  asm volatile("" : "+v"(c));
   // an entry whose force is zero is skipped by the reference: it enters the sum as 0
-  float c = f == 0.0f ? 0.0f : dot(sub(scale(a.e_a[e], st), scale(a.e_b[e], en)), fv);
+  c = f == 0.0f ? 0.0f : c;
   if (MODE == MW_GRAD) c = l.gout[torque] * c;
   return c;
 }
@@ -455,13 +474,17 @@ __global__ __launch_bounds__(1024) void muscle_world_kernel(MwArgs a) {
   // before the first is needed), then one entry per thread
   int base = 0;
   for (; base + 4 * nt <= a.nentry; base += 4 * nt) {
+    MwEntry t[4];
     float c[4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) c[k] = entry_contribution<MODE>(a, l, base + k * nt + tid);
+    for (int k = 0; k < 4; ++k) t[k] = load_entry<MODE>(a, l, base + k * nt + tid);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) c[k] = entry_contribution<MODE>(a, l, t[k]);
 #pragma unroll
     for (int k = 0; k < 4; ++k) l.contrib[base + k * nt + tid] = c[k];
   }
-  for (int e = base + tid; e < a.nentry; e += nt) l.contrib[e] = entry_contribution<MODE>(a, l, e);
+  for (int e = base + tid; e < a.nentry; e += nt)
+    l.contrib[e] = entry_contribution<MODE>(a, l, load_entry<MODE>(a, l, e));
   __syncthreads();
   const float *contrib = l.contrib;
   for (int r = tid; r < a.nrow; r += nt) {
