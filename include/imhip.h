@@ -351,6 +351,61 @@ int im_muscle_sparse_moment(const im_muscle_geometry *geometry,
                             const im_muscle_entries *entry_segments, int root_dof_count,
                             float *moment, int64_t ld_moment, int nworld, void *stream);
 
+/* ---- steps either side of the solve that walk a world's small trees ------------------- */
+
+/* Replaces the product M v inside the fused Newton kernel
+ * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:171-176; tables m.M_mulm_rowadr /
+ * M_mulm_col / M_mulm_madr of the upstream model, :378-380): out[w, dof] = sum over
+ * k in [mulm_rowadr[dof], mulm_rowadr[dof + 1]) of M[w, mulm_madr[k]] * vec[w, mulm_col[k]],
+ * accumulated from 0 in table order with one fused multiply-add per term.
+ * M (nworld, ld_M >= nM), vec and out (nworld, ld >= nv).  skip_world (nworld bytes, may be
+ * null): worlds with a nonzero byte keep their out row (the reference's done /
+ * search-unchanged worlds). */
+int im_mul_m_sparse(const float *M, int64_t ld_M, int nM, const int32_t *mulm_rowadr,
+                    const int32_t *mulm_col, const int32_t *mulm_madr, const float *vec,
+                    int64_t ld_vec, const uint8_t *skip_world, float *out, int64_t ld_out,
+                    int nv, int nworld, void *stream);
+
+/* Replaces accumulate_body_tree_deterministic_kernel
+ * (src/instantmimic/utils/mjw_kernels/tree_fusion.py:82-113; accumulate(), :137-167), in
+ * place: for level = levels - 1 .. 1, every body of level - 1 adds the values of its
+ * children among the bodies of `level`, in the order level_bodies lists them (body 0 is
+ * never a child; with skip_root_parent the children of body 0 are not added).  The
+ * reference's default kernel (:54-80) adds the same children with atomics, that is, in no
+ * fixed order.  values (nworld, nbody, components) with ld_world floats between worlds.
+ * level_bodies / level_offsets: bodies sorted by depth and the depth offsets
+ * (create_tree_reduction_scratch, :35-51). */
+int im_tree_accumulate(const int32_t *body_parentid, const int32_t *level_bodies,
+                       const int32_t *level_offsets, int levels, int components,
+                       int skip_root_parent, float *values, int64_t ld_world, int nbody,
+                       int nworld, void *stream);
+
+/* Inputs of the body-wrench projection, all (nworld, ...) float rows with ld floats between
+ * worlds: body_force / body_torque / xipos (nbody, 3), subtree_com (nbody, 3),
+ * cdof (nvfull, 6); body_rootid (nbody). */
+typedef struct im_body_wrenches {
+  const float *body_force, *body_torque, *xipos, *subtree_com, *cdof;
+  int64_t ld_body_force, ld_body_torque, ld_xipos, ld_subtree_com, ld_cdof;
+  const int32_t *body_rootid;
+} im_body_wrenches;
+
+/* WrenchProjectionTopology (src/instantmimic/muscle/wrench_projection.py:145-155). */
+typedef struct im_wrench_topology {
+  const int32_t *dof_bodyid, *body_parentid, *level_bodies, *level_offsets;
+  int32_t levels, body_count;
+} im_wrench_topology;
+
+/* Replaces project_body_wrenches_to_dofs_kernel (wrench_projection.py:59-136): per body the
+ * force and the moment torque + (xipos - subtree_com[root]) x force, folded bottom-up along
+ * the body tree, then mean[w, j + output_dof_offset] = cdof_lin . force + cdof_ang . moment
+ * of dof j + root_dof_count's body.  The reference folds siblings with atomics (any order);
+ * here a parent adds its children in the order of level_bodies, so the result is
+ * reproducible.  Any body count that fits 64 KiB of LDS (the reference: 256 bodies). */
+int im_project_body_wrenches(const im_body_wrenches *wrenches,
+                             const im_wrench_topology *topology, int root_dof_count,
+                             int torque_dim, int output_dof_offset, float *mean,
+                             int64_t ld_mean, int nworld, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

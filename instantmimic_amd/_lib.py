@@ -67,6 +67,21 @@ class MuscleEntries(C.Structure):
     ]  # fmt: skip
 
 
+class BodyWrenches(C.Structure):
+    _fields_ = [
+        ("body_force", _vp), ("body_torque", _vp), ("xipos", _vp), ("subtree_com", _vp), ("cdof", _vp),
+        ("ld_body_force", C.c_int64), ("ld_body_torque", C.c_int64), ("ld_xipos", C.c_int64),
+        ("ld_subtree_com", C.c_int64), ("ld_cdof", C.c_int64), ("body_rootid", _vp),
+    ]  # fmt: skip
+
+
+class WrenchTopology(C.Structure):
+    _fields_ = [
+        ("dof_bodyid", _vp), ("body_parentid", _vp), ("level_bodies", _vp), ("level_offsets", _vp),
+        ("levels", C.c_int32), ("body_count", C.c_int32),
+    ]  # fmt: skip
+
+
 _pgeo, _pseg, _pent = C.POINTER(MuscleGeometry), C.POINTER(MuscleSegments), C.POINTER(MuscleEntries)
 
 # name -> (restype, argtypes); the single list of symbols the header declares
@@ -122,6 +137,12 @@ SIGNATURES = {
     "im_muscle_activation_grad": (_i, [_pgeo, _pseg, _pent, _vp, _i64, _vp, _i64, _i, _vp, _i64, _i, _vp]),
     "im_muscle_torque_bounds": (_i, [_pgeo, _pseg, _pent, _vp, _i64, _i, _vp, _vp, _i64, _i, _vp]),
     "im_muscle_sparse_moment": (_i, [_pgeo, _pseg, _vp, _pent, _i, _vp, _i64, _i, _vp]),
+    "im_mul_m_sparse": (_i, [_vp, _i64, _i, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _i, _i, _vp]),
+    "im_tree_accumulate": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _i64, _i, _i, _vp]),
+    "im_project_body_wrenches": (
+        _i,
+        [C.POINTER(BodyWrenches), C.POINTER(WrenchTopology), _i, _i, _i, _vp, _i64, _i, _vp],
+    ),
 }
 
 _lib = None

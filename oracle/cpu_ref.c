@@ -1051,3 +1051,99 @@ int orc_muscle_torque_bounds(int nworld, int nwp, int nbody, int nv, int nmuscle
   }
   return 0;
 }
+
+/* ---- steps either side of the solve that walk a world's small trees ---------------------- */
+
+/* The product M v of the fused Newton kernel
+ * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:171-176):
+ *     value = 0;  for k in row: value += M[adr[k]] * v[col[k]]
+ * with the multiply contracted into the add (one fmaf per term, as NVRTC compiles the
+ * statement).  The row tables are the upstream model's M_mulm_* arrays (mujoco_warp, absent
+ * from the tree): the order of a row's terms is theirs and is a parameter here.  Pinned by
+ * the dense fp64 product; bit-level agreement with the reference build is unpinned. */
+int orc_mul_m_sparse(int nworld, int nv, int nM, const int *rowadr, const int *col,
+                     const int *madr, const float *M, const float *vec,
+                     const unsigned char *skip, float *out) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    if (skip && skip[w]) continue;
+    const float *m = M + (size_t)w * nM, *v = vec + (size_t)w * nv;
+    for (int dof = 0; dof < nv; ++dof) {
+      float value = 0.0f;
+      for (int k = rowadr[dof]; k < rowadr[dof + 1]; ++k) value = fmaf(m[madr[k]], v[col[k]], value);
+      out[(size_t)w * nv + dof] = value;
+    }
+  }
+  return 0;
+}
+
+/* accumulate_body_tree_deterministic_kernel
+ * (src/instantmimic/utils/mjw_kernels/tree_fusion.py:82-113), in place on
+ * values (nworld, nbody, components). */
+static void orc_fold_levels(float *values, int components, const int *parent, const int *bodies,
+                            const int *offsets, int levels, int skip_root_parent) {
+  for (int level = levels - 1; level > 0; --level)
+    for (int p = offsets[level - 1]; p < offsets[level]; ++p) {
+      const int parent_id = bodies[p];
+      if (skip_root_parent && parent_id == 0) continue;
+      for (int c = 0; c < components; ++c) {
+        float value = values[parent_id * components + c];
+        for (int e = offsets[level]; e < offsets[level + 1]; ++e) {
+          const int body = bodies[e];
+          if (body != 0 && parent[body] == parent_id) value = value + values[body * components + c];
+        }
+        values[parent_id * components + c] = value;
+      }
+    }
+}
+
+int orc_tree_accumulate(int nworld, int nbody, int components, const int *parent,
+                        const int *bodies, const int *offsets, int levels,
+                        int skip_root_parent, float *values) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w)
+    orc_fold_levels(values + (size_t)w * nbody * components, components, parent, bodies, offsets,
+                    levels, skip_root_parent);
+  return 0;
+}
+
+/* project_body_wrenches_to_dofs_kernel (src/instantmimic/muscle/wrench_projection.py:59-136)
+ * with the siblings of a parent added in the order of level_bodies (the reference adds them
+ * with atomics, in no fixed order: its result is this one up to that order).  Pinned by the
+ * masked sum of the legacy kernel (muscle_dynamics_kernels.py:2906-2955) in fp64. */
+int orc_project_body_wrenches(int nworld, int nbody, int nvfull, const float *body_force,
+                              const float *body_torque, const float *xipos,
+                              const float *subtree_com, const float *cdof, const int *rootid,
+                              const int *dof_body, const int *parent, const int *bodies,
+                              const int *offsets, int levels, int root, int ntorque,
+                              int out_offset, int ld_mean, float *mean) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    float *values = (float *)malloc(sizeof(float) * 6 * (size_t)nbody);
+    for (int b = 0; b < nbody; ++b) {
+      const float *f = body_force + ((size_t)w * nbody + b) * 3;
+      const float *t = body_torque + ((size_t)w * nbody + b) * 3;
+      const float *x = xipos + ((size_t)w * nbody + b) * 3;
+      const float *c = subtree_com + ((size_t)w * nbody + rootid[b]) * 3;
+      const float rx = x[0] - c[0], ry = x[1] - c[1], rz = x[2] - c[2];
+      float *o = values + 6 * b;
+      o[0] = f[0];
+      o[1] = f[1];
+      o[2] = f[2];
+      o[3] = t[0] + (ry * f[2] - rz * f[1]);
+      o[4] = t[1] + (rz * f[0] - rx * f[2]);
+      o[5] = t[2] + (rx * f[1] - ry * f[0]);
+    }
+    orc_fold_levels(values, 6, parent, bodies, offsets, levels, 0);
+    for (int j = 0; j < ntorque; ++j) {
+      const int dof = j + root;
+      const float *v = values + 6 * dof_body[dof];
+      const float *cd = cdof + ((size_t)w * nvfull + dof) * 6;
+      const float lin = cd[3] * v[0] + cd[4] * v[1] + cd[5] * v[2];
+      const float ang = cd[0] * v[3] + cd[1] * v[4] + cd[2] * v[5];
+      mean[(size_t)w * ld_mean + j + out_offset] = lin + ang;
+    }
+    free(values);
+  }
+  return 0;
+}

@@ -443,3 +443,46 @@ def muscle_torque_bounds(waypoints, com, cdof, seg, entries, unit, root):
         *[_p(a) for a in keep], _p(unit), int(root), _p(lower), _p(upper),
     )  # fmt: skip
     return lower, upper
+
+
+# ---- steps either side of the solve that walk a world's small trees -------------------------
+# Pinning: `mul_m_sparse` against the dense fp64 product with the symmetric matrix of the CSR
+# and by linearity; `tree_accumulate` against subtree sums taken from the ancestor relation in
+# fp64 (and exactly, on integer-valued inputs, where every order of additions gives the same
+# bits); `project_body_wrenches` against the masked sum of the reference's legacy kernel
+# (muscle_dynamics_kernels.py:2906-2955) in fp64.  Bit-level agreement with the reference build
+# is unpinned for all three: the first one's term order comes from upstream tables that are not
+# in the tree, the other two add siblings with atomics in the reference's default kernels.
+
+
+def mul_m_sparse(M, vec, rowadr, col, madr, skip=None, out=None):
+    M, vec = _f(M), _f(vec)
+    nworld, nM = M.shape
+    nv = vec.shape[1]
+    out = np.zeros((nworld, nv), np.float32) if out is None else out
+    sk = None if skip is None else np.ascontiguousarray(skip, np.uint8)
+    lib().orc_mul_m_sparse(nworld, nv, nM, _p(_i(rowadr)), _p(_i(col)), _p(_i(madr)), _p(M), _p(vec),
+                           None if sk is None else _p(sk), _p(out))  # fmt: skip
+    return out
+
+
+def tree_accumulate(values, components, parent, bodies, offsets, skip_root_parent=False):
+    """Returns the accumulated copy of values (nworld, nbody, components)."""
+    out = _f(values).copy()
+    nworld, nbody = out.shape[0], out.shape[1]
+    lib().orc_tree_accumulate(nworld, nbody, components, _p(_i(parent)), _p(_i(bodies)), _p(_i(offsets)),
+                              len(offsets) - 1, int(bool(skip_root_parent)), _p(out))  # fmt: skip
+    return out
+
+
+def project_body_wrenches(body_force, body_torque, xipos, subtree_com, cdof, rootid, dof_body, parent, bodies, offsets,
+                          root, ntorque, out_offset=0, mean=None):  # fmt: skip
+    body_force, body_torque, xipos, subtree_com, cdof = (_f(a) for a in (body_force, body_torque, xipos, subtree_com, cdof))
+    nworld, nbody, nvfull = body_force.shape[0], body_force.shape[1], cdof.shape[1]
+    mean = np.zeros((nworld, ntorque + out_offset), np.float32) if mean is None else mean
+    lib().orc_project_body_wrenches(
+        nworld, nbody, nvfull, _p(body_force), _p(body_torque), _p(xipos), _p(subtree_com), _p(cdof), _p(_i(rootid)),
+        _p(_i(dof_body)), _p(_i(parent)), _p(_i(bodies)), _p(_i(offsets)), len(offsets) - 1, root, ntorque, out_offset,
+        mean.shape[1], _p(mean),
+    )  # fmt: skip
+    return mean

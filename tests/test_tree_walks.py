@@ -1,0 +1,225 @@
+"""The steps either side of the solve that walk a world's small trees: M v over the tree
+CSR, bottom-up accumulation of per-body values, body wrenches onto joint torques.  Oracle
+pinning and host tables on the CPU, bit-for-bit parity of the HIP kernels on the GPU."""
+
+import numpy as np
+import pytest
+
+from instantmimic_amd import synth
+from instantmimic_amd.mjw_kernels import newton_fusion as NF
+from instantmimic_amd.mjw_kernels import tree_fusion as TF
+from instantmimic_amd.muscle import wrench_projection as WP
+from instantmimic_amd.muscle.muscle_dynamics import build_dof_subtree_mask
+from oracle import ref as R
+
+TREES = {"ant": synth.ant_parents, "humanoid": synth.humanoid_parents, "snu": synth.snu_parents, "stress": synth.stress_parents}
+
+
+def _body_tree(nbody: int, seed: int):
+    """A random body tree with body 0 the world: parents reference earlier bodies."""
+    rng = np.random.default_rng(seed)
+    parent = np.zeros(nbody, np.int32)
+    for b in range(1, nbody):
+        parent[b] = rng.integers(max(0, b - 4), b)
+    return parent
+
+
+def _levels(parent):
+    order, offsets, _, _ = WP.tree_levels(parent)
+    return order, offsets
+
+
+def _ancestor_or_self(parent):
+    n = len(parent)
+    anc = np.zeros((n, n), bool)  # anc[b, a]: a is b or an ancestor of b
+    for b in range(n):
+        p = b
+        while True:
+            anc[b, p] = True
+            if p == 0:
+                break
+            p = int(parent[p])
+    return anc
+
+
+# ---------------------------------------------------------------- M v
+@pytest.mark.parametrize("tree", list(TREES))
+def test_mul_m_tables_and_oracle_against_dense_fp64(tree):
+    rowadr, rownnz, colind = synth.csr_from_parents(TREES[tree]())
+    nv, nM = len(rowadr), len(colind)
+    adr, col, madr = NF.mul_m_tables(rowadr, rownnz, colind)
+    # every element of the symmetric matrix exactly once, at its CSR address
+    elem = synth.matrix_elemid(rowadr, rownnz, colind)
+    assert adr[0] == 0 and adr[-1] == 2 * nM - nv
+    for i in range(nv):
+        cols = col[adr[i] : adr[i + 1]]
+        assert len(set(cols.tolist())) == len(cols)
+        assert sorted(cols.tolist()) == np.nonzero(elem[i] >= 0)[0].tolist()
+        np.testing.assert_array_equal(madr[adr[i] : adr[i + 1]], elem[i, cols])
+    rng = np.random.default_rng(5)
+    M = rng.normal(size=(9, nM)).astype(np.float32)
+    v = rng.normal(size=(9, nv)).astype(np.float32)
+    out = R.mul_m_sparse(M, v, adr, col, madr)
+    dense = synth.dense_from_csr(M.astype(np.float64), rowadr, rownnz, colind)
+    want = np.einsum("wij,wj->wi", dense, v.astype(np.float64))
+    assert R.rel_l2(out, want) < 1e-6
+    # scaling by a power of two is exact; skipped worlds keep their rows
+    np.testing.assert_array_equal(R.mul_m_sparse(M, 4 * v, adr, col, madr), 4 * out)
+    skip = np.zeros(9, np.uint8)
+    skip[[2, 7]] = 1
+    kept = R.mul_m_sparse(M, v, adr, col, madr, skip=skip, out=np.full((9, nv), 7.0, np.float32))
+    assert (kept[[2, 7]] == 7.0).all()
+    np.testing.assert_array_equal(np.delete(kept, [2, 7], 0), np.delete(out, [2, 7], 0))
+
+
+# ---------------------------------------------------------------- accumulation
+@pytest.mark.parametrize("nbody,components,skip", [(1, 3, False), (2, 3, False), (17, 3, False), (17, 10, True), (60, 6, False), (300, 10, True)])
+def test_oracle_accumulate_against_subtree_sums(nbody, components, skip):
+    parent = _body_tree(nbody, seed=nbody)
+    order, offsets = _levels(parent)
+    rng = np.random.default_rng(11)
+    vals = rng.normal(size=(5, nbody, components)).astype(np.float32)
+    got = R.tree_accumulate(vals, components, parent, order, offsets, skip)
+    anc = _ancestor_or_self(parent)
+    want = np.einsum("ba,wbc->wac", anc.astype(np.float64), vals.astype(np.float64))
+    # body 0 is never a child; with skip the children of body 0 are not added to it
+    want[:, 0] = vals[:, 0] if skip else vals[:, 0] + want[:, 1:][:, parent[1:] == 0].sum(1)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 1e-6 * scale * max(1, np.log2(nbody))
+    # integers: every order of additions gives the same bits
+    ints = rng.integers(-8, 9, size=(3, nbody, components)).astype(np.float32)
+    wi = np.einsum("ba,wbc->wac", anc.astype(np.float64), ints.astype(np.float64))
+    wi[:, 0] = ints[:, 0] if skip else ints[:, 0] + wi[:, 1:][:, parent[1:] == 0].sum(1)
+    np.testing.assert_array_equal(R.tree_accumulate(ints, components, parent, order, offsets, skip), wi.astype(np.float32))
+
+
+def test_accumulate_scratch_mirrors_the_reference_fields():
+    class M:
+        body_tree = [np.array([0]), np.array([1, 4]), np.array([2, 3, 5])]
+        body_parentid = np.array([0, 0, 1, 1, 0, 4])
+
+    class Empty:
+        body_tree = []
+        body_parentid = np.zeros(1, np.int32)
+
+    assert TF.create_tree_reduction_scratch(Empty(), device="cpu") is None
+    s = TF.create_tree_reduction_scratch(M(), deterministic=True, device="cpu")
+    assert s.levels == 3 and s.deterministic and s.cooperative and s.nbody == 6
+    assert s.bodies.tolist() == [0, 1, 4, 2, 3, 5] and s.offsets.tolist() == [0, 1, 3, 6]
+    order, offsets, child_bodies, child_offsets = WP.tree_levels(M.body_parentid)
+    assert order.tolist() == s.bodies.tolist() and offsets.tolist() == s.offsets.tolist()
+    assert child_bodies.tolist() == [1, 4, 2, 3, 5] and child_offsets.tolist() == [0, 2, 4, 4, 4, 5, 5]
+    with pytest.raises(ValueError):
+        WP.tree_levels(np.array([0, 2, 1]))
+
+
+# ---------------------------------------------------------------- wrench projection
+def _wrench_case(nworld, seed=1003):
+    rig = synth.make_muscle_rig(nmuscle=40, seed=seed)
+    topo = rig.topology
+    nb, nv = rig.body_count, rig.full_torque_dim
+    ctx = synth.make_muscle_context(rig, nworld, seed=seed + 1)
+    xipos = ctx[:, 7 * nb : 10 * nb].reshape(nworld, nb, 3)
+    com = ctx[:, 10 * nb : 13 * nb].reshape(nworld, nb, 3)
+    cdof = ctx[:, 13 * nb : 13 * nb + 6 * nv].reshape(nworld, nv, 6)
+    rng = np.random.default_rng(seed + 2)
+    force = rng.normal(0, 50, (nworld, nb, 3)).astype(np.float32)
+    torque = rng.normal(0, 5, (nworld, nb, 3)).astype(np.float32)
+    return rig, topo, force, torque, np.ascontiguousarray(xipos), np.ascontiguousarray(com), np.ascontiguousarray(cdof)
+
+
+def test_oracle_wrench_projection_against_the_masked_sum_fp64():
+    nworld = 6
+    rig, topo, force, torque, xipos, com, cdof = _wrench_case(nworld)
+    nb, root, nt = rig.body_count, rig.full_torque_dim - rig.torque_dim, rig.torque_dim
+    parent, rootid, dof_body = (np.asarray(a, np.int32) for a in (topo.body_parentid, topo.body_rootid, topo.dof_bodyid))
+    order, offsets = _levels(parent)
+    got = R.project_body_wrenches(force, torque, xipos, com, cdof, rootid, dof_body, parent, order, offsets, root, nt, out_offset=2,
+                                  mean=np.full((nworld, nt + 5), 7.0, np.float32))  # fmt: skip
+    assert (got[:, :2] == 7.0).all() and (got[:, nt + 2 :] == 7.0).all()
+    # the per-dof kernel of the reference: total += mask * (lin . f + ang . (t + (x - c_root) x f))
+    mask = build_dof_subtree_mask(parent, dof_body, nb, rig.full_torque_dim).astype(np.float64)
+    f64, t64 = force.astype(np.float64), torque.astype(np.float64)
+    arm = xipos.astype(np.float64) - com.astype(np.float64)[:, rootid]
+    moment = t64 + np.cross(arm, f64)
+    per_body = np.einsum("wdk,wbk->wdb", cdof[:, :, 3:].astype(np.float64), f64) + np.einsum(
+        "wdk,wbk->wdb", cdof[:, :, :3].astype(np.float64), moment
+    )
+    want = np.einsum("db,wdb->wd", mask, per_body)[:, root : root + nt]
+    assert R.rel_l2(got[:, 2 : nt + 2], want) < 1e-6
+
+
+# ---------------------------------------------------------------- GPU
+@pytest.mark.gpu
+@pytest.mark.parametrize("tree,nworld", [("ant", 64), ("humanoid", 4096), ("snu", 333), ("stress", 67)])
+def test_gpu_mul_m_bitwise(device, tree, nworld):
+    import torch
+
+    rowadr, rownnz, colind = synth.csr_from_parents(TREES[tree]())
+    nv, nM = len(rowadr), len(colind)
+    tables = NF.mul_m_tables(rowadr, rownnz, colind)
+    rng = np.random.default_rng(7)
+    M = rng.normal(size=(nworld, nM)).astype(np.float32)
+    v = rng.normal(size=(nworld, nv)).astype(np.float32)
+    skip = (rng.uniform(size=nworld) < 0.2).astype(np.uint8)
+    t = lambda a: torch.from_numpy(a).to(device)  # noqa: E731
+    td = [t(a) for a in tables]
+    Md = torch.zeros((nworld, nM + 3), device=device)
+    Md[:, :nM] = t(M)
+    out = torch.full((nworld, nv + 2), 7.0, device=device)
+    NF.mul_m(Md[:, :nM], t(v), out[:, :nv], *td)
+    torch.cuda.synchronize()
+    want = R.mul_m_sparse(M, v, *tables)
+    got = out.cpu().numpy()
+    np.testing.assert_array_equal(got[:, :nv], want)
+    assert (got[:, nv:] == 7.0).all()
+    out.fill_(7.0)
+    NF.mul_m(Md[:, :nM], t(v), out[:, :nv], *td, skip_world=t(skip))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert (got[skip == 1] == 7.0).all()
+    np.testing.assert_array_equal(got[skip == 0][:, :nv], want[skip == 0])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nbody,components,skip,nworld", [(2, 3, False, 5), (17, 3, False, 4096), (17, 10, True, 1000), (60, 6, False, 333), (300, 10, True, 65), (1200, 10, False, 9)])
+def test_gpu_accumulate_bitwise(device, nbody, components, skip, nworld):
+    import torch
+
+    parent = _body_tree(nbody, seed=nbody)
+    order, offsets = _levels(parent)
+
+    class M:
+        body_parentid = parent
+        body_tree = [order[offsets[i] : offsets[i + 1]] for i in range(len(offsets) - 1)]
+
+    scratch = TF.create_tree_reduction_scratch(M(), deterministic=True, device=device)
+    vals = np.random.default_rng(3).normal(size=(nworld, nbody, components)).astype(np.float32)
+    vd = torch.from_numpy(vals).to(device)
+    TF.accumulate(M(), None, vd, components, skip, scratch)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(vd.cpu().numpy(), R.tree_accumulate(vals, components, parent, order, offsets, skip))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nworld", [1, 67, 4096])
+def test_gpu_wrench_projection_bitwise(device, nworld):
+    import torch
+
+    rig, topo, force, torque, xipos, com, cdof = _wrench_case(nworld)
+    nb, root, nt = rig.body_count, rig.full_torque_dim - rig.torque_dim, rig.torque_dim
+    parent, rootid, dof_body = (np.asarray(a, np.int32) for a in (topo.body_parentid, topo.body_rootid, topo.dof_bodyid))
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    topology = WP.build_wrench_projection_topology(t(parent), t(dof_body), nb, device)
+    assert topology is not None and topology.levels == len(_levels(parent)[1]) - 1
+    mean = torch.full((nworld, nt + 5), 7.0, device=device)
+    WP.launch_project_body_wrench_to_torque(
+        topology, body_force=t(force), body_torque=t(torque), xipos=t(xipos), subtree_com=t(com), cdof=t(cdof),
+        body_rootid=t(rootid), dof_subtree_mask=None, mean=mean, body_count=nb, torque_dim=nt, root_dof_count=root,
+        output_dof_offset=2, batch_size=nworld, device=str(device),
+    )  # fmt: skip
+    torch.cuda.synchronize()
+    order, offsets = _levels(parent)
+    want = R.project_body_wrenches(force, torque, xipos, com, cdof, rootid, dof_body, parent, order, offsets, root, nt, out_offset=2,
+                                   mean=np.full((nworld, nt + 5), 7.0, np.float32))  # fmt: skip
+    np.testing.assert_array_equal(mean.cpu().numpy(), want)
