@@ -357,12 +357,13 @@ int im_muscle_sparse_moment(const im_muscle_geometry *geometry,
  * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:171-176; tables m.M_mulm_rowadr /
  * M_mulm_col / M_mulm_madr of the upstream model, :378-380): out[w, dof] = sum over
  * k in [mulm_rowadr[dof], mulm_rowadr[dof + 1]) of M[w, mulm_madr[k]] * vec[w, mulm_col[k]],
- * accumulated from 0 in table order with one fused multiply-add per term.
- * M (nworld, ld_M >= nM), vec and out (nworld, ld >= nv).  skip_world (nworld bytes, may be
+ * accumulated from 0 in table order with one fused multiply-add per term.  nterm = the
+ * length of mulm_col and mulm_madr (= mulm_rowadr[nv]; 2 nM - nv for a full symmetric table).
+ * M (nworld, ld_M >= nM), vec and out (nworld, ld >= nv); nM and nv below 65536.  skip_world (nworld bytes, may be
  * null): worlds with a nonzero byte keep their out row (the reference's done /
  * search-unchanged worlds). */
 int im_mul_m_sparse(const float *M, int64_t ld_M, int nM, const int32_t *mulm_rowadr,
-                    const int32_t *mulm_col, const int32_t *mulm_madr, const float *vec,
+                    const int32_t *mulm_col, const int32_t *mulm_madr, int nterm, const float *vec,
                     int64_t ld_vec, const uint8_t *skip_world, float *out, int64_t ld_out,
                     int nv, int nworld, void *stream);
 

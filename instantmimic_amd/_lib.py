@@ -137,7 +137,7 @@ SIGNATURES = {
     "im_muscle_activation_grad": (_i, [_pgeo, _pseg, _pent, _vp, _i64, _vp, _i64, _i, _vp, _i64, _i, _vp]),
     "im_muscle_torque_bounds": (_i, [_pgeo, _pseg, _pent, _vp, _i64, _i, _vp, _vp, _i64, _i, _vp]),
     "im_muscle_sparse_moment": (_i, [_pgeo, _pseg, _vp, _pent, _i, _vp, _i64, _i, _vp]),
-    "im_mul_m_sparse": (_i, [_vp, _i64, _i, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _i, _i, _vp]),
+    "im_mul_m_sparse": (_i, [_vp, _i64, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i64, _i, _i, _vp]),
     "im_tree_accumulate": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _i64, _i, _i, _vp]),
     "im_project_body_wrenches": (
         _i,

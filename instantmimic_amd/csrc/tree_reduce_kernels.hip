@@ -15,23 +15,49 @@ namespace {
 constexpr int kThreads = 256;
 constexpr size_t kLdsLimit = 64 * 1024;
 
+// Copies per_block worlds' rows of `stride` floats into LDS, `fetch(world, k)` giving element
+// k of a world's row.  Four elements per thread and trip, their loads issued before the first
+// store (indices past the end are clamped, their values dropped).
+template <typename Fetch>
+__device__ __forceinline__ void stage_rows(float *lds, int per_block, int stride, int64_t w0,
+                                           int nworld, Fetch fetch) {
+  const int total = per_block * stride;
+  for (int i0 = threadIdx.x; i0 < total; i0 += 4 * kThreads) {
+    float r[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * kThreads < total ? i0 + u * kThreads : total - 1;
+      const int lw = i / stride, k = i - lw * stride;
+      r[u] = fetch(w0 + lw < nworld ? w0 + lw : (int64_t)nworld - 1, k);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i0 + u * kThreads < total) lds[i0 + u * kThreads] = r[u];
+  }
+}
+
 // ---- M v -----------------------------------------------------------------------------------
 // T lanes per world (a power of two, 8..64): lane d of a world owns dofs d, d + T, ...
+// The row tables sit in LDS beside the worlds' rows, one word col | madr << 16 per term: lanes
+// of a wavefront read different rows, and such gathers cost a cache lookup per lane when they
+// go to memory.
 __global__ __launch_bounds__(kThreads) void mul_m_kernel(
     const float *__restrict__ M, int64_t ldm, int nM, const int32_t *__restrict__ rowadr,
     const int32_t *__restrict__ col, const int32_t *__restrict__ madr,
     const float *__restrict__ vec, int64_t ldv, const uint8_t *__restrict__ skip,
-    float *__restrict__ out, int64_t ldo, int nv, int nworld, int lanes) {
+    float *__restrict__ out, int64_t ldo, int nv, int nworld, int lanes, int nterm) {
   extern __shared__ float lds[];
   const int per_block = kThreads / lanes;
   const int stride = nM + nv;
   const int64_t w0 = (int64_t)blockIdx.x * per_block;
+  uint32_t *term = (uint32_t *)(lds + per_block * stride);  // [nterm]
+  int *radr = (int *)(term + nterm);                         // [nv + 1]
+  for (int k = threadIdx.x; k < nterm; k += kThreads) term[k] = (uint32_t)col[k] | (uint32_t)madr[k] << 16;
+  for (int k = threadIdx.x; k <= nv; k += kThreads) radr[k] = rowadr[k];
   // a world's M and vec rows, one world after the other, loads coalesced over the block
-  for (int i = threadIdx.x; i < per_block * stride; i += kThreads) {
-    const int lw = i / stride, k = i - lw * stride;
-    const int64_t w = w0 + lw < nworld ? w0 + lw : nworld - 1;
-    lds[i] = k < nM ? M[w * ldm + k] : vec[w * ldv + (k - nM)];
-  }
+  stage_rows(lds, per_block, stride, w0, nworld, [&](int64_t w, int k) {
+    return k < nM ? M[w * ldm + k] : vec[w * ldv + (k - nM)];
+  });
   __syncthreads();
   const int lw = threadIdx.x / lanes, lane = threadIdx.x & (lanes - 1);
   const int64_t w = w0 + lw;
@@ -39,29 +65,49 @@ __global__ __launch_bounds__(kThreads) void mul_m_kernel(
   const float *m = lds + lw * stride, *v = m + nM;
   for (int dof = lane; dof < nv; dof += lanes) {
     float value = 0.0f;
-    for (int k = rowadr[dof]; k < rowadr[dof + 1]; ++k) value = fmaf(m[madr[k]], v[col[k]], value);
+    const int end = radr[dof + 1];
+    // four terms' operands at a time; a term past the row's end repeats the last one and is
+    // dropped
+    for (int k = radr[dof]; k < end; k += 4) {
+      float a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t t = term[k + u < end ? k + u : end - 1];
+        a[u] = m[t >> 16];
+        b[u] = v[t & 0xffffu];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) value = k + u < end ? fmaf(a[u], b[u], value) : value;
+    }
     out[w * ldo + dof] = value;
   }
 }
 
 // ---- bottom-up accumulation -----------------------------------------------------------------
+// The level tables as the folds read them, in LDS: tb[c] = level_bodies[c] and
+// tb[nbody + c] = that body's parent (-1 for body 0, which is never a child).
+__device__ __forceinline__ void stage_tree(int *tb, const int32_t *__restrict__ parent,
+                                           const int32_t *__restrict__ bodies, int nbody) {
+  for (int c = threadIdx.x; c < nbody; c += kThreads) {
+    const int body = bodies[c];
+    tb[c] = body;
+    tb[nbody + c] = body != 0 ? parent[body] : -1;
+  }
+}
+
 // Folds one level's bodies into their parents: one writer per (parent, component), the
 // children added in the order the level lists them.
-__device__ __forceinline__ void fold_level(float *values, int components,
-                                           const int32_t *__restrict__ parent,
-                                           const int32_t *__restrict__ bodies, int pstart,
-                                           int start, int end, bool skip_root_parent, int lane,
-                                           int lanes) {
+__device__ __forceinline__ void fold_level(float *values, int components, const int *tb,
+                                           int nbody, int pstart, int start, int end,
+                                           bool skip_root_parent, int lane, int lanes) {
   const int pcount = start - pstart;
   for (int entry = lane; entry < pcount * components; entry += lanes) {
-    const int parent_id = bodies[pstart + entry / components];
+    const int parent_id = tb[pstart + entry / components];
     const int component = entry % components;
     if (skip_root_parent && parent_id == 0) continue;
     float value = values[parent_id * components + component];
-    for (int c = start; c < end; ++c) {
-      const int body = bodies[c];
-      if (body != 0 && parent[body] == parent_id) value = value + values[body * components + component];
-    }
+    for (int c = start; c < end; ++c)
+      if (tb[nbody + c] == parent_id) value = value + values[tb[c] * components + component];
     values[parent_id * components + component] = value;
   }
 }
@@ -74,17 +120,15 @@ __global__ __launch_bounds__(kThreads) void tree_accumulate_kernel(
   const int per_block = kThreads / lanes;
   const int stride = nbody * components;
   const int64_t w0 = (int64_t)blockIdx.x * per_block;
-  for (int i = threadIdx.x; i < per_block * stride; i += kThreads) {
-    const int lw = i / stride, k = i - lw * stride;
-    const int64_t w = w0 + lw < nworld ? w0 + lw : nworld - 1;
-    lds[i] = values[w * ldw + k];
-  }
+  int *tb = (int *)(lds + per_block * stride);
+  stage_tree(tb, parent, bodies, nbody);
+  stage_rows(lds, per_block, stride, w0, nworld, [&](int64_t w, int k) { return values[w * ldw + k]; });
   __syncthreads();
   const int lw = threadIdx.x / lanes, lane = threadIdx.x & (lanes - 1);
   float *mine = lds + lw * stride;
   // every wavefront of the block walks the same levels, so the barriers are uniform
   for (int level = levels - 1; level > 0; --level) {
-    fold_level(mine, components, parent, bodies, offsets[level - 1], offsets[level],
+    fold_level(mine, components, tb, nbody, offsets[level - 1], offsets[level],
                offsets[level + 1], skip_root_parent != 0, lane, lanes);
     __syncthreads();
   }
@@ -110,6 +154,8 @@ __global__ __launch_bounds__(kThreads) void project_wrenches_kernel(WrenchArgs a
   const int per_block = kThreads / a.lanes;
   const int stride = 6 * a.nbody;
   const int64_t w0 = (int64_t)blockIdx.x * per_block;
+  int *tb = (int *)(lds + per_block * stride);
+  stage_tree(tb, a.parent, a.bodies, a.nbody);
   // force and the moment about the root's subtree centre, per body
   for (int i = threadIdx.x; i < per_block * a.nbody; i += kThreads) {
     const int lw = i / a.nbody, body = i - lw * a.nbody;
@@ -130,7 +176,7 @@ __global__ __launch_bounds__(kThreads) void project_wrenches_kernel(WrenchArgs a
   const int lw = threadIdx.x / a.lanes, lane = threadIdx.x & (a.lanes - 1);
   float *mine = lds + lw * stride;
   for (int level = a.levels - 1; level > 0; --level) {
-    fold_level(mine, 6, a.parent, a.bodies, a.offsets[level - 1], a.offsets[level],
+    fold_level(mine, 6, tb, a.nbody, a.offsets[level - 1], a.offsets[level],
                a.offsets[level + 1], false, lane, a.lanes);
     __syncthreads();
   }
@@ -153,8 +199,9 @@ int lanes_for(int work) {
   return lanes;
 }
 // Widens the lane count until a block's worlds fit in LDS; 0 when one world alone does not.
-int fit_lanes(int lanes, size_t floats_per_world) {
-  while (lanes <= kThreads && (kThreads / lanes) * floats_per_world * 4 > kLdsLimit) lanes *= 2;
+int fit_lanes(int lanes, size_t floats_per_world, size_t shared_words = 0) {
+  while (lanes <= kThreads && ((kThreads / lanes) * floats_per_world + shared_words) * 4 > kLdsLimit)
+    lanes *= 2;
   return lanes <= kThreads ? lanes : 0;
 }
 
@@ -164,20 +211,22 @@ int fit_lanes(int lanes, size_t floats_per_world) {
 using namespace im;
 
 extern "C" int im_mul_m_sparse(const float *M, int64_t ld_M, int nM, const int32_t *mulm_rowadr,
-                               const int32_t *mulm_col, const int32_t *mulm_madr,
+                               const int32_t *mulm_col, const int32_t *mulm_madr, int nterm,
                                const float *vec, int64_t ld_vec, const uint8_t *skip_world,
                                float *out, int64_t ld_out, int nv, int nworld, void *stream) {
-  if (nworld < 0 || nv < 0 || nM < 0) return IM_ERR_ARG;
+  if (nworld < 0 || nv < 0 || nM < 0 || nterm < 0) return IM_ERR_ARG;
   if (nworld == 0 || nv == 0) return IM_OK;
   if (!M || !mulm_rowadr || !mulm_col || !mulm_madr || !vec || !out) return IM_ERR_ARG;
   if (ld_M < nM || ld_vec < nv || ld_out < nv) return IM_ERR_STRIDE;
-  const int lanes = fit_lanes(lanes_for(nv), (size_t)nM + nv);
+  const size_t shared_words = (size_t)nterm + nv + 1;
+  if (nM >= 65536 || nv >= 65536) return IM_ERR_UNSUPPORTED;  // a term is packed into 16 + 16 bits
+  const int lanes = fit_lanes(lanes_for(nv), (size_t)nM + nv, shared_words);
   if (!lanes) return IM_ERR_UNSUPPORTED;
   const int per_block = kThreads / lanes;
-  const size_t lds_bytes = (size_t)per_block * ((size_t)nM + nv) * 4;
+  const size_t lds_bytes = ((size_t)per_block * ((size_t)nM + nv) + shared_words) * 4;
   hipLaunchKernelGGL(mul_m_kernel, dim3((unsigned)((nworld + per_block - 1) / per_block)),
                      dim3(kThreads), lds_bytes, (hipStream_t)stream, M, ld_M, nM, mulm_rowadr,
-                     mulm_col, mulm_madr, vec, ld_vec, skip_world, out, ld_out, nv, nworld, lanes);
+                     mulm_col, mulm_madr, vec, ld_vec, skip_world, out, ld_out, nv, nworld, lanes, nterm);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }
@@ -190,10 +239,10 @@ extern "C" int im_tree_accumulate(const int32_t *body_parentid, const int32_t *l
   if (nworld == 0 || nbody == 0 || components == 0 || levels <= 1) return IM_OK;
   if (!body_parentid || !level_bodies || !level_offsets || !values) return IM_ERR_ARG;
   if (ld_world < (int64_t)nbody * components) return IM_ERR_STRIDE;
-  const int lanes = fit_lanes(lanes_for(nbody * components), (size_t)nbody * components);
+  const int lanes = fit_lanes(lanes_for(nbody * components), (size_t)nbody * components, 2 * (size_t)nbody);
   if (!lanes) return IM_ERR_UNSUPPORTED;
   const int per_block = kThreads / lanes;
-  const size_t lds_bytes = (size_t)per_block * nbody * components * 4;
+  const size_t lds_bytes = ((size_t)per_block * nbody * components + 2 * (size_t)nbody) * 4;
   hipLaunchKernelGGL(tree_accumulate_kernel,
                      dim3((unsigned)((nworld + per_block - 1) / per_block)), dim3(kThreads),
                      lds_bytes, (hipStream_t)stream, body_parentid, level_bodies, level_offsets,
@@ -217,7 +266,7 @@ extern "C" int im_project_body_wrenches(const im_body_wrenches *wrenches,
       !topology->level_offsets || nbody == 0)
     return IM_ERR_ARG;
   if (ld_mean < (int64_t)output_dof_offset + torque_dim) return IM_ERR_STRIDE;
-  const int lanes = fit_lanes(lanes_for(6 * nbody), (size_t)6 * nbody);
+  const int lanes = fit_lanes(lanes_for(6 * nbody), (size_t)6 * nbody, 2 * (size_t)nbody);
   if (!lanes) return IM_ERR_UNSUPPORTED;
   const int per_block = kThreads / lanes;
   WrenchArgs a{wrenches->body_force, wrenches->body_torque, wrenches->xipos,
@@ -229,7 +278,7 @@ extern "C" int im_project_body_wrenches(const im_body_wrenches *wrenches,
                ld_mean, nworld, lanes};
   hipLaunchKernelGGL(project_wrenches_kernel,
                      dim3((unsigned)((nworld + per_block - 1) / per_block)), dim3(kThreads),
-                     (size_t)per_block * 6 * nbody * 4, (hipStream_t)stream, a);
+                     ((size_t)per_block * 6 * nbody + 2 * (size_t)nbody) * 4, (hipStream_t)stream, a);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

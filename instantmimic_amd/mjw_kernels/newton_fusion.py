@@ -55,7 +55,7 @@ def mul_m(M, vec, out, mulm_rowadr, mulm_col, mulm_madr, *, skip_world: Any = No
         if t.dtype != torch.int32 or not t.is_cuda or not t.is_contiguous():
             raise TypeError("the row tables must be contiguous int32 CUDA tensors")
     nworld, nv = vec.shape
-    if out.shape != vec.shape or M.shape[0] != nworld or mulm_rowadr.numel() != nv + 1:
+    if out.shape != vec.shape or M.shape[0] != nworld or mulm_rowadr.numel() != nv + 1 or mulm_madr.numel() != mulm_col.numel():
         raise ValueError("shapes of M, vec, out and the row table disagree")
     if skip_world is not None:
         if skip_world.dtype not in (torch.bool, torch.uint8) or skip_world.numel() != nworld or not skip_world.is_contiguous():
@@ -63,7 +63,7 @@ def mul_m(M, vec, out, mulm_rowadr, mulm_col, mulm_madr, *, skip_world: Any = No
     with torch.cuda.device(M.device):
         status = _lib.lib().im_mul_m_sparse(
             M.data_ptr(), M.stride(0), int(M.shape[1]), mulm_rowadr.data_ptr(), mulm_col.data_ptr(),
-            mulm_madr.data_ptr(), vec.data_ptr(), vec.stride(0), None if skip_world is None else skip_world.data_ptr(),
+            mulm_madr.data_ptr(), int(mulm_col.numel()), vec.data_ptr(), vec.stride(0), None if skip_world is None else skip_world.data_ptr(),
             out.data_ptr(), out.stride(0), int(nv), int(nworld), int(torch.cuda.current_stream(M.device).cuda_stream),
         )  # fmt: skip
     _lib.check(status, "im_mul_m_sparse")

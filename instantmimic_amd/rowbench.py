@@ -212,6 +212,47 @@ def run(launches: int = 32) -> None:
     _line("eval_muscle_sparse_moment (waypoints + im_muscle_sparse_moment)", wl, sec,
           bytes_=nworld * (cbytes + 4 * (3 * layer.waypoint_count * 2 + len(layer.sparse_entries.muscle_dof_torque_idx))), nworld=nworld)  # fmt: skip
 
+    # ---- the tree walks either side of the solve
+    from .mjw_kernels import newton_fusion as NF
+    from .mjw_kernels import tree_fusion as TF
+    from .muscle import wrench_projection as WP
+
+    for name, nsets in (("humanoid", 16), ("snu", 8)):
+        b = synth.make_batch(name)
+        nv, nM, nworld = b.shape.nv, int(b.colind.size), b.nworld
+        tables = [t(a) for a in NF.mul_m_tables(b.rowadr, b.rownnz, b.colind)]
+        Ms, Vs = [t(b.M) for _ in range(nsets)], [t(b.grad) for _ in range(nsets)]
+        out = torch.zeros((nworld, nv), device=dev)
+        sec = _timeit(torch, lambda i: NF.mul_m(Ms[i], Vs[i], out, *tables), nsets, launches)
+        _line("im_mul_m_sparse", f"{name} nv={nv} nM={nM} x {nworld} worlds", sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
+    topo = rig.topology
+    nb, nvf = rig.body_count, rig.full_torque_dim
+    parent = np.asarray(topo.body_parentid, np.int32)
+    order, offsets, _, _ = WP.tree_levels(parent)
+    model = SimpleNamespace(body_parentid=parent, body_tree=[order[offsets[i] : offsets[i + 1]] for i in range(len(offsets) - 1)])
+    scratch = TF.create_tree_reduction_scratch(model, deterministic=True, device=dev)
+    for comp, skip, what in ((3, False, "subtree_com"), (10, True, "crb")):
+        vals = [torch.randn((nworld, nb, comp), device=dev) for _ in range(8)]
+        sec = _timeit(torch, lambda i: TF.accumulate(model, None, vals[i], comp, skip, scratch), 8, launches)
+        _line(f"im_tree_accumulate ({what}: {comp} components)", f"snu rig body tree: {nb} bodies, {len(offsets) - 1} levels x {nworld} worlds", sec,
+              bytes_=nworld * 4 * 2 * nb * comp, nworld=nworld)  # fmt: skip
+    wt = WP.build_wrench_projection_topology(t(parent), t(np.asarray(topo.dof_bodyid, np.int32)), nb, dev)
+    rootid = t(np.asarray(topo.body_rootid, np.int32))
+    ins = [[torch.randn((nworld, nb, 3), device=dev) for _ in range(4)] + [torch.randn((nworld, nvf, 6), device=dev)] for _ in range(8)]
+    mean = torch.zeros((nworld, rig.torque_dim), device=dev)
+    root = nvf - rig.torque_dim
+    sec = _timeit(
+        torch,
+        lambda i: WP.launch_project_body_wrench_to_torque(
+            wt, body_force=ins[i][0], body_torque=ins[i][1], xipos=ins[i][2], subtree_com=ins[i][3], cdof=ins[i][4],
+            body_rootid=rootid, mean=mean, body_count=nb, torque_dim=rig.torque_dim, root_dof_count=root,
+            output_dof_offset=0, batch_size=nworld,
+        ),
+        8, launches,
+    )  # fmt: skip
+    _line("im_project_body_wrenches", f"snu rig: {nb} bodies, {rig.torque_dim} torque dofs x {nworld} worlds", sec,
+          bytes_=nworld * 4 * (12 * nb + 6 * nvf + rig.torque_dim), nworld=nworld)  # fmt: skip
+
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
