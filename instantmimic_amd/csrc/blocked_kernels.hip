@@ -437,6 +437,40 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
     int32_t *uni = uni_ + w * (nv + 1);
     for (int i = tid; i < nu; i += nt) uni[i] = ul[i];
     if (tid == 0) uni[nv] = nu;
+    if (staged && B == 16) {
+      // All pair sums of a 16 x 16 tile of dofs at once on the matrix cores.  Every staged row
+      // enters every pair here, also where one of the two dofs is zero in it: such a term adds
+      // +-0 to a sum that started at +0, which leaves all its bits, so the sums equal the ones
+      // that skip those rows.  v_mfma_f32_16x16x4_f32 adds its four products one after the
+      // other with a fused multiply-add each, rows ascending.
+      typedef float f32x4 __attribute__((ext_vector_type(4)));
+      const int lane = tid & 63, p = lane & 15, kq = lane >> 4;
+      const int nb = (nv + 15) / 16, ntiles = nb * (nb + 1) / 2;
+      for (int tile = tid >> 6; tile < ntiles; tile += nt >> 6) {
+        int cb = (int)((sqrtf((float)(8 * tile + 1)) - 1.0f) * 0.5f);
+        while ((cb + 1) * (cb + 2) / 2 <= tile) ++cb;
+        while (cb * (cb + 1) / 2 > tile) --cb;
+        const int rb = tile - cb * (cb + 1) / 2;
+        const int ra = 16 * rb + p, ca = 16 * cb + p;  // the dofs this lane feeds
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int t0 = 0; t0 < count; t0 += 4) {
+          const int t = t0 + kq, tc = t < count ? t : count - 1;
+          const float wgt = t < count ? sd[tc] : 0.0f;
+          const float a = ra < nv ? wgt * jr[tc * nv + ra] : 0.0f;  // -(D a) == (-D) a exactly
+          const float b = (t < count && ca < nv) ? jr[tc * nv + ca] : 0.0f;
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int row = 16 * rb + 4 * kq + i, col = ca;
+          if (row <= col && col < nv && acc[i] != 0.0f) {
+            const float h = U[row * pad + col] + acc[i];
+            U[row * pad + col] = h;
+            Hw[(size_t)row * pad + col] = h;
+          }
+        }
+      }
+    } else {
     const int npair = nu * (nu + 1) / 2;
     for (int e = tid; e < npair; e += nt) {
       int cj = (int)((sqrtf((float)(8 * e + 1)) - 1.0f) * 0.5f);
@@ -466,6 +500,7 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
         if (delta != 0.0f) Hw[(size_t)row * pad + col] = Hw[(size_t)row * pad + col] + delta;
       }
     }
+    }
     if (staged) {
       __syncthreads();
       const LdsSrc<B> src{U, nv, pad};
@@ -477,10 +512,19 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
       factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
     }
     // stored factor: the augmented column z = U'^-1 grad above the corner sqrt(1e30 - z.z)
-    if (tid == 0) {
+    if (tid < 64) {
+      // the chain v = fma(-z_i, z_i, v) over i ascending; the z's come 64 at a time into the
+      // lanes and reach the chain through lane reads instead of one LDS round trip each
       float v = 1.0e30f;
-      for (int i = 0; i < nv; ++i) v = fma_(-rhs[i], rhs[i], v);
-      L[0] = sqrtf(v);
+      for (int base = 0; base < nv; base += 64) {
+        const float z = base + tid < nv ? rhs[base + tid] : 0.0f;
+        const int n = nv - base < 64 ? nv - base : 64;
+        for (int i = 0; i < n; ++i) {
+          const float zi = __shfl(z, i, 64);
+          v = fma_(-zi, zi, v);
+        }
+      }
+      if (tid == 0) L[0] = sqrtf(v);
     }
     __syncthreads();
     for (int i = tid; i < pad * pad / 4; i += nt) {  // pad is a multiple of 16: a float4 stays in a row
