@@ -115,3 +115,39 @@ def test_status_codes():
     lib.im_tree_plan_destroy(handle)
     with pytest.raises(_lib.ImhipError):
         _lib.check(_lib.IM_ERR_STRIDE, "x")
+
+
+def test_tree_walk_entry_points_check_their_arguments_before_any_launch():
+    """Every refusal below happens on the host, before a HIP call: negative sizes, null
+    pointers, rows shorter than their contents, worlds too large for LDS; empty batches
+    succeed."""
+    lib = _lib.lib()
+    one = 16  # any non-null address: nothing is dereferenced on these paths
+    # M v
+    assert lib.im_mul_m_sparse(one, 81, 81, one, one, one, 148, one, 14, None, one, 14, 14, -1, None) == _lib.IM_ERR_ARG
+    assert lib.im_mul_m_sparse(None, 81, 81, one, one, one, 148, one, 14, None, one, 14, 14, 3, None) == _lib.IM_ERR_ARG
+    assert lib.im_mul_m_sparse(one, 80, 81, one, one, one, 148, one, 14, None, one, 14, 14, 3, None) == _lib.IM_ERR_STRIDE
+    assert lib.im_mul_m_sparse(one, 81, 81, one, one, one, 148, one, 14, None, one, 13, 14, 3, None) == _lib.IM_ERR_STRIDE
+    assert lib.im_mul_m_sparse(one, 70000, 70000, one, one, one, 139000, one, 1000, None, one, 1000, 1000, 3, None) == _lib.IM_ERR_UNSUPPORTED
+    assert lib.im_mul_m_sparse(one, 20000, 20000, one, one, one, 39000, one, 1000, None, one, 1000, 1000, 3, None) == _lib.IM_ERR_UNSUPPORTED
+    assert lib.im_mul_m_sparse(None, 0, 0, None, None, None, 0, None, 0, None, None, 0, 0, 0, None) == _lib.IM_OK
+    # accumulation
+    assert lib.im_tree_accumulate(one, one, one, 3, 3, 0, one, 30, 10, -1, None) == _lib.IM_ERR_ARG
+    assert lib.im_tree_accumulate(one, one, one, 3, 3, 0, None, 30, 10, 4, None) == _lib.IM_ERR_ARG
+    assert lib.im_tree_accumulate(one, one, one, 3, 3, 0, one, 29, 10, 4, None) == _lib.IM_ERR_STRIDE
+    assert lib.im_tree_accumulate(one, one, one, 3, 10, 0, one, 20000, 2000, 4, None) == _lib.IM_ERR_UNSUPPORTED
+    assert lib.im_tree_accumulate(None, None, None, 1, 3, 0, None, 30, 10, 4, None) == _lib.IM_OK  # a single level: nothing to add
+    assert lib.im_tree_accumulate(None, None, None, 3, 3, 0, None, 30, 10, 0, None) == _lib.IM_OK
+    # wrench projection
+    w, t = _lib.BodyWrenches(), _lib.WrenchTopology()
+    assert lib.im_project_body_wrenches(C.byref(w), None, 6, 50, 0, one, 50, 4, None) == _lib.IM_ERR_ARG
+    t.body_count, t.levels = 26, 8
+    assert lib.im_project_body_wrenches(C.byref(w), C.byref(t), 6, 50, 0, one, 50, 4, None) == _lib.IM_ERR_ARG  # null arrays
+    assert lib.im_project_body_wrenches(C.byref(w), C.byref(t), 6, 0, 0, None, 0, 4, None) == _lib.IM_OK
+    for name in ("body_force", "body_torque", "xipos", "subtree_com", "cdof", "body_rootid"):
+        setattr(w, name, one)
+    for name in ("dof_bodyid", "body_parentid", "level_bodies", "level_offsets"):
+        setattr(t, name, one)
+    assert lib.im_project_body_wrenches(C.byref(w), C.byref(t), 6, 50, 2, one, 51, 4, None) == _lib.IM_ERR_STRIDE
+    t.body_count = 3000
+    assert lib.im_project_body_wrenches(C.byref(w), C.byref(t), 6, 50, 0, one, 50, 4, None) == _lib.IM_ERR_UNSUPPORTED
