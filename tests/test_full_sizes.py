@@ -7,6 +7,7 @@ so a world's result must not depend on where it sits in a batch -- the 16384 wor
 distinct ones drawn with repetition, every copy must equal its source bit for bit, and the 1024
 sources are checked against the oracle."""
 
+import dataclasses
 from types import SimpleNamespace
 
 import numpy as np
@@ -100,3 +101,48 @@ def test_stress_full_batch_by_world_independence(device):
     Hd = Hf[:, :nv, :nv].double()
     err = (back - Hd).flatten(1).norm(dim=1) / Hd.flatten(1).norm(dim=1)
     assert float(err.max()) < 2e-6
+
+
+@pytest.mark.parametrize("name,nworld", [("g1", 8192), ("snu", 4096)])
+def test_sparse_factor_full_batch(device, name, nworld):
+    """Static-pattern sparse L'DL at the full batch: the initial assemble + factor + solve, then
+    one per-iteration stage (changed rows, refactor or solve-only), every world bit for bit."""
+    import torch
+
+    from instantmimic_amd.mjw_kernels import newton_stages as NS
+    from instantmimic_amd.mjw_kernels import sparse_hessian as S
+    from test_newton_stages import _changes
+
+    m = synth.model_from_parents(synth.SHAPES[name].parents)
+    plan, reason = S.plan_for_model(m, None, [], S.block_width(m.nv_pad), device=device)
+    assert plan is not None, reason
+    b = synth.make_batch(dataclasses.replace(synth.SHAPES[name], iterations=2))  # a second state to move to
+    assert b.nworld == nworld
+    nv = m.nv
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    hf = torch.zeros((nworld, plan.nv_pad, plan.nv_pad), device=device)
+    search = torch.full((nworld, nv, 1), float("nan"), device=device)
+    sdot, decr = torch.zeros(nworld, device=device), torch.zeros(nworld, device=device)
+    tJ, tD = t(b.J), t(b.D)
+    S.init_factor_kernel(plan)(None, t(b.nefc), tJ, tD, t(b.state[0]), t(b.M), t(b.grad)[:, :, None].contiguous(), hf, search, sdot, decr)
+    torch.cuda.synchronize()
+    ref = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
+    n_used = 2 * plan.nfac + nv
+    np.testing.assert_array_equal(hf.cpu().numpy().reshape(nworld, -1)[:, :n_used], ref[0].reshape(nworld, -1)[:, :n_used])
+    np.testing.assert_array_equal(search.cpu().numpy()[:, :, 0], ref[1])
+    np.testing.assert_array_equal(sdot.cpu().numpy(), ref[2])
+    np.testing.assert_array_equal(decr.cpu().numpy(), ref[3])
+    assert not hf[:, -1, -1].any()  # nothing fell outside the declared pattern
+    # the per-iteration stage from there
+    new, ids, changes, sc, done, grad = _changes(b, np.random.default_rng(5))
+    want = R.sparse_update_factor(plan, sc, changes, ids, b.J, b.D, new, grad, ref[0], done=done)
+    uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=device)
+    search2 = torch.zeros((nworld, nv), device=device)
+    NS.factor_factory(nv, m.nv_pad, plan)(tJ, tD, t(new), t(ids), t(changes), t(sc), t(done), t(grad), None, hf, search2, sdot, decr, uni)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(hf.cpu().numpy().reshape(nworld, -1)[:, :n_used], want[0].reshape(nworld, -1)[:, :n_used])
+    live = (sc != 0) & (done == 0)
+    np.testing.assert_array_equal(uni.cpu().numpy()[live & (changes > 0)], want[1][live & (changes > 0)])
+    np.testing.assert_array_equal(search2.cpu().numpy()[live], want[2][live])
+    np.testing.assert_array_equal(sdot.cpu().numpy()[live], want[3][live])
+    np.testing.assert_array_equal(decr.cpu().numpy()[live], want[4][live])
