@@ -84,30 +84,50 @@ __global__ __launch_bounds__(kThreads) void mul_m_kernel(
 }
 
 // ---- bottom-up accumulation -----------------------------------------------------------------
-// The level tables as the folds read them, in LDS: tb[c] = level_bodies[c] and
-// tb[nbody + c] = that body's parent (-1 for body 0, which is never a child).
+// The level tables as the folds read them, in LDS: tb[c] = level_bodies[c],
+// tb[nbody + c] = that body's parent (-1 for body 0, which is never a child), and behind them
+// the levels + 1 level offsets.
 __device__ __forceinline__ void stage_tree(int *tb, const int32_t *__restrict__ parent,
-                                           const int32_t *__restrict__ bodies, int nbody) {
+                                           const int32_t *__restrict__ bodies,
+                                           const int32_t *__restrict__ offsets, int nbody,
+                                           int levels) {
   for (int c = threadIdx.x; c < nbody; c += kThreads) {
     const int body = bodies[c];
     tb[c] = body;
     tb[nbody + c] = body != 0 ? parent[body] : -1;
   }
+  for (int l = threadIdx.x; l <= levels; l += kThreads) tb[2 * nbody + l] = offsets[l];
+}
+__host__ __device__ inline size_t tree_words(int nbody, int levels) {
+  return 2 * (size_t)nbody + (size_t)levels + 1;
 }
 
 // Folds one level's bodies into their parents: one writer per (parent, component), the
-// children added in the order the level lists them.
-__device__ __forceinline__ void fold_level(float *values, int components, const int *tb,
-                                           int nbody, int pstart, int start, int end,
-                                           bool skip_root_parent, int lane, int lanes) {
+// children added in the order the level lists them.  Four children's parents and values are
+// read before the first is added; one that belongs to another parent is dropped.
+__device__ __forceinline__ void fold_level(float *values, int components, float inv_components,
+                                           const int *tb, int nbody, int pstart, int start,
+                                           int end, bool skip_root_parent, int lane, int lanes) {
   const int pcount = start - pstart;
   for (int entry = lane; entry < pcount * components; entry += lanes) {
-    const int parent_id = tb[pstart + entry / components];
-    const int component = entry % components;
+    // entry / components through the reciprocal: exact while entry stays below 2^20
+    const int pi = (int)(((float)entry + 0.5f) * inv_components);
+    const int parent_id = tb[pstart + pi];
+    const int component = entry - pi * components;
     if (skip_root_parent && parent_id == 0) continue;
     float value = values[parent_id * components + component];
-    for (int c = start; c < end; ++c)
-      if (tb[nbody + c] == parent_id) value = value + values[tb[c] * components + component];
+    for (int c = start; c < end; c += 4) {
+      int par[4];
+      float x[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int cc = c + u < end ? c + u : end - 1;
+        par[u] = c + u < end ? tb[nbody + cc] : -2;
+        x[u] = values[tb[cc] * components + component];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) value = par[u] == parent_id ? value + x[u] : value;
+    }
     values[parent_id * components + component] = value;
   }
 }
@@ -121,15 +141,17 @@ __global__ __launch_bounds__(kThreads) void tree_accumulate_kernel(
   const int stride = nbody * components;
   const int64_t w0 = (int64_t)blockIdx.x * per_block;
   int *tb = (int *)(lds + per_block * stride);
-  stage_tree(tb, parent, bodies, nbody);
+  stage_tree(tb, parent, bodies, offsets, nbody, levels);
   stage_rows(lds, per_block, stride, w0, nworld, [&](int64_t w, int k) { return values[w * ldw + k]; });
   __syncthreads();
   const int lw = threadIdx.x / lanes, lane = threadIdx.x & (lanes - 1);
   float *mine = lds + lw * stride;
+  const int *loff = tb + 2 * nbody;
+  const float inv_components = 1.0f / (float)components;
   // every wavefront of the block walks the same levels, so the barriers are uniform
   for (int level = levels - 1; level > 0; --level) {
-    fold_level(mine, components, tb, nbody, offsets[level - 1], offsets[level],
-               offsets[level + 1], skip_root_parent != 0, lane, lanes);
+    fold_level(mine, components, inv_components, tb, nbody, loff[level - 1], loff[level],
+               loff[level + 1], skip_root_parent != 0, lane, lanes);
     __syncthreads();
   }
   for (int i = threadIdx.x; i < per_block * stride; i += kThreads) {
@@ -155,7 +177,7 @@ __global__ __launch_bounds__(kThreads) void project_wrenches_kernel(WrenchArgs a
   const int stride = 6 * a.nbody;
   const int64_t w0 = (int64_t)blockIdx.x * per_block;
   int *tb = (int *)(lds + per_block * stride);
-  stage_tree(tb, a.parent, a.bodies, a.nbody);
+  stage_tree(tb, a.parent, a.bodies, a.offsets, a.nbody, a.levels);
   // force and the moment about the root's subtree centre, per body
   for (int i = threadIdx.x; i < per_block * a.nbody; i += kThreads) {
     const int lw = i / a.nbody, body = i - lw * a.nbody;
@@ -176,8 +198,8 @@ __global__ __launch_bounds__(kThreads) void project_wrenches_kernel(WrenchArgs a
   const int lw = threadIdx.x / a.lanes, lane = threadIdx.x & (a.lanes - 1);
   float *mine = lds + lw * stride;
   for (int level = a.levels - 1; level > 0; --level) {
-    fold_level(mine, 6, tb, a.nbody, a.offsets[level - 1], a.offsets[level],
-               a.offsets[level + 1], false, lane, a.lanes);
+    fold_level(mine, 6, 1.0f / 6.0f, tb, a.nbody, tb[2 * a.nbody + level - 1], tb[2 * a.nbody + level],
+               tb[2 * a.nbody + level + 1], false, lane, a.lanes);
     __syncthreads();
   }
   const int64_t w = w0 + lw;
@@ -235,14 +257,14 @@ extern "C" int im_tree_accumulate(const int32_t *body_parentid, const int32_t *l
                                   const int32_t *level_offsets, int levels, int components,
                                   int skip_root_parent, float *values, int64_t ld_world,
                                   int nbody, int nworld, void *stream) {
-  if (nworld < 0 || nbody < 0 || levels < 0 || components < 0) return IM_ERR_ARG;
+  if (nworld < 0 || nbody < 0 || levels < 0 || components < 0 || levels > nbody) return IM_ERR_ARG;
   if (nworld == 0 || nbody == 0 || components == 0 || levels <= 1) return IM_OK;
   if (!body_parentid || !level_bodies || !level_offsets || !values) return IM_ERR_ARG;
   if (ld_world < (int64_t)nbody * components) return IM_ERR_STRIDE;
-  const int lanes = fit_lanes(lanes_for(nbody * components), (size_t)nbody * components, 2 * (size_t)nbody);
+  const int lanes = fit_lanes(lanes_for(nbody * components), (size_t)nbody * components, tree_words(nbody, levels));
   if (!lanes) return IM_ERR_UNSUPPORTED;
   const int per_block = kThreads / lanes;
-  const size_t lds_bytes = ((size_t)per_block * nbody * components + 2 * (size_t)nbody) * 4;
+  const size_t lds_bytes = ((size_t)per_block * nbody * components + tree_words(nbody, levels)) * 4;
   hipLaunchKernelGGL(tree_accumulate_kernel,
                      dim3((unsigned)((nworld + per_block - 1) / per_block)), dim3(kThreads),
                      lds_bytes, (hipStream_t)stream, body_parentid, level_bodies, level_offsets,
@@ -256,7 +278,7 @@ extern "C" int im_project_body_wrenches(const im_body_wrenches *wrenches,
                                         int torque_dim, int output_dof_offset, float *mean,
                                         int64_t ld_mean, int nworld, void *stream) {
   if (nworld < 0 || torque_dim < 0 || root_dof_count < 0 || output_dof_offset < 0 || !topology ||
-      topology->body_count < 0 || topology->levels < 0)
+      topology->body_count < 0 || topology->levels < 0 || topology->levels > topology->body_count)
     return IM_ERR_ARG;
   if (nworld == 0 || torque_dim == 0) return IM_OK;
   const int nbody = topology->body_count;
@@ -266,7 +288,7 @@ extern "C" int im_project_body_wrenches(const im_body_wrenches *wrenches,
       !topology->level_offsets || nbody == 0)
     return IM_ERR_ARG;
   if (ld_mean < (int64_t)output_dof_offset + torque_dim) return IM_ERR_STRIDE;
-  const int lanes = fit_lanes(lanes_for(6 * nbody), (size_t)6 * nbody, 2 * (size_t)nbody);
+  const int lanes = fit_lanes(lanes_for(6 * nbody), (size_t)6 * nbody, tree_words(nbody, topology->levels));
   if (!lanes) return IM_ERR_UNSUPPORTED;
   const int per_block = kThreads / lanes;
   WrenchArgs a{wrenches->body_force, wrenches->body_torque, wrenches->xipos,
@@ -278,7 +300,7 @@ extern "C" int im_project_body_wrenches(const im_body_wrenches *wrenches,
                ld_mean, nworld, lanes};
   hipLaunchKernelGGL(project_wrenches_kernel,
                      dim3((unsigned)((nworld + per_block - 1) / per_block)), dim3(kThreads),
-                     ((size_t)per_block * 6 * nbody + 2 * (size_t)nbody) * 4, (hipStream_t)stream, a);
+                     ((size_t)per_block * 6 * nbody + tree_words(nbody, topology->levels)) * 4, (hipStream_t)stream, a);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }
