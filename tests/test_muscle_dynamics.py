@@ -607,3 +607,29 @@ def test_gpu_fused_geometry_equals_the_two_launches(nworld):
     assert torch.equal(wp2[:, :-pad], wp[:, :-pad]) and torch.equal(unit2[:, :-pad], unit[:, :-pad])
     assert torch.equal(pas2[:, :-pad], pas[:, :-pad])
     assert (wp2[:, -pad:] == 3.0).all() and (unit2[:, -pad:] == 3.0).all() and (pas2[:, -pad:] == 3.0).all()
+
+
+@pytest.mark.gpu
+def test_gpu_entry_lists_without_a_stated_range_take_the_other_kernels():
+    """An entry list whose nother field is 0 sends the contractions to the one-thread-per-output
+    kernels; results are the same bits as with the range stated."""
+    rig = synth.make_muscle_rig(nmuscle=284, seed=1003)
+    layer = _gpu_layer(rig, active_force_type="gaussian", passive_force_type="exponential")
+    nworld = 77
+    ctx_d = torch.from_numpy(synth.make_muscle_context(rig, nworld, seed=5)).cuda()
+    act = torch.rand(nworld, rig.muscle_count, device="cuda")
+    g = torch.randn(nworld, rig.torque_dim, device="cuda")
+
+    def run():
+        mean, _, unit = layer._warp_muscle_dynamics_from_activation_forward(act, ctx_d, include_passive_force=True)
+        grad = layer._warp_muscle_dynamics_from_activation_backward(ctx_d, g)
+        moment = layer.eval_muscle_sparse_moment(ctx_d)
+        torch.cuda.synchronize()
+        return mean.clone(), grad.clone(), moment.clone()
+
+    stated = run()
+    for e in (layer._torque_entries, layer._muscle_entries, layer._moment_entries):
+        assert e.nother > 0
+        e.nother = 0
+    for a, b in zip(stated, run()):
+        assert torch.equal(a, b)
