@@ -14,6 +14,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
+#include <cstring>
 
 #include "common.h"
 
@@ -328,6 +329,202 @@ __global__ __launch_bounds__(1024) void blocked_factor_solve_kernel(
   if (Uout)
     for (int i = tid; i < pad * pad / 4; i += nt)  // pad is a multiple of B >= 8
       ((float4 *)(Uout + w * (int64_t)pad * pad))[i] = ((const float4 *)U)[i];
+}
+
+// ---- 8 x 8 tiles, matrices up to 64 x 64: four worlds per wavefront -------------------------
+// With a wavefront per world most of the factor runs on 8 of 64 lanes (the pivots of a tile,
+// its triangular solves, the right-hand side), and the SIMDs spend their issue slots on idle
+// lanes.  Here a world has a DPP row of 16 lanes and a wavefront carries four worlds through
+// the same instructions; the only synchronisation is within the wavefront.  U keeps the tiles
+// on or above the diagonal only, tile (bi, bj) at 64 (bi nblk - bi (bi - 1) / 2 + bj - bi).
+// Every element sees the operations of blocked_factor_solve_kernel<8> in the same order.
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__host__ __device__ inline int quad_tiles_before(int bi, int nblk) { return bi * nblk - bi * (bi - 1) / 2; }
+// floats of LDS per world: tiles (a block row is updated in place), right-hand side, the
+// diagonal tile's lower factor and reciprocal pivots; rounded so that the four worlds start 8 banks apart
+__host__ __device__ inline int quad_world_floats(int pad) {
+  const int nblk = pad / 8;
+  const int need = 64 * quad_tiles_before(nblk, nblk) + pad + 72;
+  return (need + 31) / 32 * 32 + 8;
+}
+
+__global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
+    const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
+    const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
+    int64_t ldx, int nv, int pad, int nworld) {
+  extern __shared__ float lds[];
+  constexpr int B = 8, BB = 64;
+  const int lane = threadIdx.x, l = lane & 15, q = lane >> 4;
+  const int nblk = pad / B, ntiles = quad_tiles_before(nblk, nblk);
+  const int64_t w_raw = (int64_t)blockIdx.x * 4 + q;
+  const bool live = w_raw < nworld;
+  const int64_t w = live ? w_raw : (int64_t)nworld - 1;  // a spare row repeats the last world and stores nothing
+  float *U = lds + q * quad_world_floats(pad);
+  float *rhs = U + BB * ntiles;  // [pad]
+  float *L = rhs + pad;          // [64 + 8]
+  auto tile = [&](int bi, int bj) { return U + BB * (quad_tiles_before(bi, nblk) + bj - bi); };
+  const float *Mw = M + w * ldM;
+  {
+    // indexed gather, four tiles (16 elements per lane) in flight
+    int kb = 0, ib = 0;
+    for (int t0 = 0; t0 < ntiles; t0 += 4) {
+      int tk[4], ti[4], idx[4][4];
+      float v[4][4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        tk[g] = kb < nblk ? kb : -1;
+        ti[g] = ib;
+        if (kb < nblk && ++ib == nblk) { ++kb; ib = kb; }
+      }
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int e = l + 16 * u;
+          idx[g][u] = block_idx[tk[g] >= 0 ? (size_t)(tk[g] * nblk + ti[g]) * BB + e : 0];
+          if (tk[g] < 0) idx[g][u] = nM;
+        }
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[g][u] = Mw[idx[g][u] < nM ? idx[g][u] : 0];
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (tk[g] >= 0) {
+            const int e = l + 16 * u, r = e >> 3, c = e & 7;
+            float xv = idx[g][u] < nM ? v[g][u] : 0.0f;
+            if (ti[g] == tk[g] && (tk[g] + 1) * B > nv && r == c && (nblk - 1) * B + r >= nv) xv = xv + 1.0f;
+            U[BB * (t0 + g) + e] = xv;
+          }
+    }
+  }
+  for (int i = l; i < pad; i += 16) rhs[i] = i < nv ? y[w * ldy + i] : 0.0f;
+  wave_sync();
+  const int c = l & 7, r0 = l >> 3;  // the lane's four elements of a tile: rows r0, r0 + 2, .., column c
+  for (int kb = 0; kb < nblk; ++kb) {
+    const int k = kb * B, ntile = nblk - kb;
+    for (int tb = 0; tb < ntile; ++tb) {
+      const int ib = kb + tb;
+      float v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = tile(kb, ib)[(r0 + 2 * u) * B + c];
+      for (int jb = 0; jb < kb; ++jb) {
+        const float *Tk = tile(jb, kb), *Ti = tile(jb, ib);
+        float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int t = 0; t < B; ++t) {
+          const float b = Ti[t * B + c];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) sum[u] = fma_(Tk[t * B + r0 + 2 * u], b, sum[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = v[u] - sum[u];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) tile(kb, ib)[(r0 + 2 * u) * B + c] = v[u];  // in place: nothing else reads this tile before
+    }
+    if (l < B) {
+      float s = rhs[k + l];
+      for (int jb = 0; jb < kb; ++jb) {
+        const float *Tk = tile(jb, kb);
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < B; ++t) sum = fma_(Tk[t * B + l], rhs[jb * B + t], sum);
+        s = s - sum;
+      }
+      rhs[k + l] = s;
+    }
+    wave_sync();
+    {
+      // Cholesky of the diagonal tile and the forward solve of the right-hand side, lane i of
+      // the world's row holding row i (see blocked_factor_solve_kernel)
+      const int i = l;
+      float a[B];
+#pragma unroll
+      for (int j = 0; j < B; ++j) a[j] = tile(kb, kb)[(i < B ? i : 0) * B + j];
+      float s = rhs[k + (i < B ? i : 0)];
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        const float d = sqrtf(row_bcast(a[j], j));
+        const float rinv = 1.0f / d;
+        const float lj = i == j ? d : a[j] * rinv;
+        if (i >= j && i < B) L[i * B + j] = lj;
+        const float z = row_bcast(s, j) * rinv;
+        if (i == j) {
+          rhs[k + j] = z;
+          L[BB + j] = rinv;
+        }
+        s = fma_(-lj, z, s);
+#pragma unroll
+        for (int jj = j + 1; jj < B; ++jj) a[jj] = fma_(-lj, row_bcast(lj, jj), a[jj]);
+      }
+    }
+    wave_sync();
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int r = r0 + 2 * u;
+      tile(kb, kb)[r * B + c] = c >= r ? L[c * B + r] : 0.0f;
+    }
+    for (int qc = l; qc < (ntile - 1) * B; qc += 16) {
+      const int tb = 1 + (qc >> 3), cc = qc & 7;
+      float *Tt = tile(kb, kb + tb);
+      float col[B];
+#pragma unroll
+      for (int r = 0; r < B; ++r) col[r] = Tt[r * B + cc];
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        const float z = col[j] * L[BB + j];
+        col[j] = z;
+#pragma unroll
+        for (int i = j + 1; i < B; ++i) col[i] = fma_(-L[i * B + j], z, col[i]);
+      }
+#pragma unroll
+      for (int r = 0; r < B; ++r) Tt[r * B + cc] = col[r];
+    }
+    wave_sync();
+  }
+  // rhs <- U^-1 rhs, block rows from the bottom
+  for (int ib = nblk - 1; ib >= 0; --ib) {
+    const int i0 = ib * B, r = l < B ? l : 0;
+    const float *Td = tile(ib, ib);
+    float s = rhs[i0 + r];
+    float urow[B];
+#pragma unroll
+    for (int cc = 0; cc < B; ++cc) urow[cc] = Td[r * B + cc];
+    const float rinv = 1.0f / Td[r * B + r];
+    for (int jb = ib + 1; jb < nblk; ++jb) {
+      const float *Tj = tile(ib, jb);
+      float sum = 0.0f;
+#pragma unroll
+      for (int t = 0; t < B; ++t) sum = fma_(Tj[r * B + t], rhs[jb * B + t], sum);
+      s = s - sum;
+    }
+#pragma unroll
+    for (int cc = B - 1; cc >= 0; --cc) {
+      const float xv = row_bcast(s * rinv, cc);
+      if (l == cc) rhs[i0 + cc] = xv;
+      s = fma_(-urow[cc], xv, s);
+    }
+    wave_sync();
+  }
+  if (live) {
+    for (int i = l; i < nv; i += 16) x[w * ldx + i] = rhs[i];
+    if (Uout) {
+      float4 *dst = (float4 *)(Uout + w * (int64_t)pad * pad);
+      for (int i4 = l; i4 < pad * pad / 4; i4 += 16) {
+        const int row = 4 * i4 / pad, col = 4 * i4 - row * pad, bi = row >> 3, bj = col >> 3;
+        float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (bj >= bi) v = *(const float4 *)(tile(bi, bj) + (row & 7) * B + (col & 7));
+        dst[i4] = v;
+      }
+    }
+  }
 }
 
 // Per-iteration factor stage on the dense Hessian: dofs touched by the changed rows,
@@ -713,6 +910,18 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
   if (ldy < nv || ldx < nv) return IM_ERR_STRIDE;
   if (U && ((uintptr_t)U & 15)) return IM_ERR_STRIDE;  // written 16 bytes at a time
   const int B = block_size;
+  static const bool quad_off = [] {
+    const char *e = std::getenv("IMHIP_BLOCKED_KERNEL");
+    return e && std::strcmp(e, "simple") == 0;
+  }();
+  if (B == 8 && pad <= 64 && !quad_off) {
+    // small matrices, 8 x 8 tiles: four worlds per wavefront
+    const size_t quad_bytes = sizeof(float) * 4 * (size_t)im::quad_world_floats(pad);
+    hipLaunchKernelGGL(im::blocked_factor_solve_quad_kernel, dim3((unsigned)((nworld + 3) / 4)), dim3(64), quad_bytes,
+                       (hipStream_t)stream, M, ldM, nM, block_idx, y, ldy, U, x, ldx, nv, pad, nworld);
+    IM_HIP_CHECK(hipGetLastError());
+    return IM_OK;
+  }
   const size_t lds_bytes = sizeof(float) * ((size_t)pad * pad + pad + (size_t)(pad / B) * B * B + B * B + B);
   if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   auto fn = B == 8 ? im::blocked_factor_solve_kernel<8> : im::blocked_factor_solve_kernel<16>;

@@ -63,7 +63,7 @@ def test_dense_hessian_oracle_against_fp64():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,B,nworld", [("g1", 8, 70), ("g1", 16, 70), ("snu", 16, 33), ("stress", 16, 9)])
+@pytest.mark.parametrize("name,B,nworld", [("g1", 8, 70), ("g1", 8, 3), ("snu", 8, 33), ("g1", 16, 70), ("snu", 16, 33), ("stress", 16, 9)])
 def test_gpu_blocked_factor_solve_bitwise(device, name, B, nworld):
     import torch
 
@@ -108,3 +108,24 @@ def test_gpu_dense_hessian_mfma(device, name, nworld):
     assert R.rel_l2(Hh, R.jtdj_dense(Md.reshape(nworld, -1), b.J, b.D, b.state[0], b.nefc, nv_pad)) <= 1e-5
     np.testing.assert_array_equal(Hh, Hh.transpose(0, 2, 1))
     assert np.abs(Hh[:, nv:, :]).max() == 0
+
+
+@pytest.mark.gpu
+def test_gpu_wavefront_per_world_kernel_for_small_tiles_agrees():
+    """8 x 8 tiles on matrices up to 64 x 64 run four worlds per wavefront; the kernel with a
+    workgroup per world that serves every other shape is forced here in a child process and
+    must pass the same oracle comparison."""
+    import os
+    import subprocess
+    import sys
+
+    env = dict(os.environ, IMHIP_BLOCKED_KERNEL="simple")
+    code = (
+        "import sys, torch; sys.path.insert(0, 'tests'); import test_blocked_dense as t;"
+        "d = torch.device('cuda:0');"
+        "t.test_gpu_blocked_factor_solve_bitwise(d, 'g1', 8, 70);"
+        "t.test_gpu_blocked_factor_solve_bitwise(d, 'snu', 8, 33); print('simple kernel ok')"
+    )
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "simple kernel ok" in out.stdout, out.stderr[-2000:]
