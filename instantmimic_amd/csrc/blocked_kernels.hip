@@ -407,27 +407,30 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
   for (int i = l; i < pad; i += 16) rhs[i] = i < nv ? y[w * ldy + i] : 0.0f;
   wave_sync();
   const int c = l & 7, r0 = l >> 3;  // the lane's four elements of a tile: rows r0, r0 + 2, .., column c
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  const int m4 = l & 3, qr = l >> 3, qc = (l >> 2) & 1;  // and as a lane of quadrant (qr, qc) on the matrix cores
   for (int kb = 0; kb < nblk; ++kb) {
     const int k = kb * B, ntile = nblk - kb;
+    // The sums over a finished block row on the matrix cores: v_mfma_f32_4x4x1_16b_f32 does one
+    // fused multiply-add per element of sixteen independent 4 x 4 blocks, and a wavefront's
+    // sixteen blocks are the four quadrants of one 8 x 8 tile of each of its four worlds.  Eight
+    // of them chained from zero are the sum over t = 0..7 ascending of the scalar form.
     for (int tb = 0; tb < ntile; ++tb) {
       const int ib = kb + tb;
-      float v[4];
+      float *Tv = tile(kb, ib) + (4 * qr) * B + 4 * qc + m4;  // rows 4 qr + 0..3 of column 4 qc + m4
+      f32x4 v;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = tile(kb, ib)[(r0 + 2 * u) * B + c];
+      for (int u = 0; u < 4; ++u) v[u] = Tv[u * B];
       for (int jb = 0; jb < kb; ++jb) {
-        const float *Tk = tile(jb, kb), *Ti = tile(jb, ib);
-        float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        const float *Tk = tile(jb, kb) + 4 * qr + m4, *Ti = tile(jb, ib) + 4 * qc + m4;
+        f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int t = 0; t < B; ++t) {
-          const float b = Ti[t * B + c];
-#pragma unroll
-          for (int u = 0; u < 4; ++u) sum[u] = fma_(Tk[t * B + r0 + 2 * u], b, sum[u]);
-        }
+        for (int t = 0; t < B; ++t) sum = __builtin_amdgcn_mfma_f32_4x4x1f32(Tk[t * B], Ti[t * B], sum, 0, 0, 0);
 #pragma unroll
         for (int u = 0; u < 4; ++u) v[u] = v[u] - sum[u];
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) tile(kb, ib)[(r0 + 2 * u) * B + c] = v[u];  // in place: nothing else reads this tile before
+      for (int u = 0; u < 4; ++u) Tv[u * B] = v[u];  // in place: nothing else reads this tile before
     }
     if (l < B) {
       float s = rhs[k + l];
