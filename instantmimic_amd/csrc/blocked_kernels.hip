@@ -331,13 +331,13 @@ __global__ __launch_bounds__(1024) void blocked_factor_solve_kernel(
       ((float4 *)(Uout + w * (int64_t)pad * pad))[i] = ((const float4 *)U)[i];
 }
 
-// ---- 8 x 8 tiles, matrices up to 64 x 64: four worlds per wavefront -------------------------
-// With a wavefront per world most of the factor runs on 8 of 64 lanes (the pivots of a tile,
+// ---- matrices up to 64 x 64: four worlds per wavefront ----------------------------------------
+// With a wavefront per world most of the factor runs on 8 or 16 of 64 lanes (the pivots of a tile,
 // its triangular solves, the right-hand side), and the SIMDs spend their issue slots on idle
 // lanes.  Here a world has a DPP row of 16 lanes and a wavefront carries four worlds through
 // the same instructions; the only synchronisation is within the wavefront.  U keeps the tiles
-// on or above the diagonal only, tile (bi, bj) at 64 (bi nblk - bi (bi - 1) / 2 + bj - bi).
-// Every element sees the operations of blocked_factor_solve_kernel<8> in the same order.
+// on or above the diagonal only, tile (bi, bj) at B B (bi nblk - bi (bi - 1) / 2 + bj - bi).
+// Every element sees the operations of blocked_factor_solve_kernel<B> in the same order.
 __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -346,34 +346,36 @@ __device__ __forceinline__ void wave_sync() {
 __host__ __device__ inline int quad_tiles_before(int bi, int nblk) { return bi * nblk - bi * (bi - 1) / 2; }
 // floats of LDS per world: tiles (a block row is updated in place), right-hand side, the
 // diagonal tile's lower factor and reciprocal pivots; rounded so that the four worlds start 8 banks apart
-__host__ __device__ inline int quad_world_floats(int pad) {
-  const int nblk = pad / 8;
-  const int need = 64 * quad_tiles_before(nblk, nblk) + pad + 72;
+__host__ __device__ inline int quad_world_floats(int pad, int B) {
+  const int nblk = pad / B;
+  const int need = B * B * quad_tiles_before(nblk, nblk) + pad + B * B + B;
   return (need + 31) / 32 * 32 + 8;
 }
 
+template <int B>
 __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
     const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
     const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
     int64_t ldx, int nv, int pad, int nworld) {
   extern __shared__ float lds[];
-  constexpr int B = 8, BB = 64;
+  constexpr int BB = B * B, PER = BB / 16;  // a lane's elements of a tile: e = l + 16 u
   const int lane = threadIdx.x, l = lane & 15, q = lane >> 4;
   const int nblk = pad / B, ntiles = quad_tiles_before(nblk, nblk);
   const int64_t w_raw = (int64_t)blockIdx.x * 4 + q;
   const bool live = w_raw < nworld;
   const int64_t w = live ? w_raw : (int64_t)nworld - 1;  // a spare row repeats the last world and stores nothing
-  float *U = lds + q * quad_world_floats(pad);
+  const int world_floats = quad_world_floats(pad, B);
+  float *U = lds + q * world_floats;
   float *rhs = U + BB * ntiles;  // [pad]
-  float *L = rhs + pad;          // [64 + 8]
+  float *L = rhs + pad;          // [BB + B]
   auto tile = [&](int bi, int bj) { return U + BB * (quad_tiles_before(bi, nblk) + bj - bi); };
   const float *Mw = M + w * ldM;
   {
-    // indexed gather, four tiles (16 elements per lane) in flight
+    // indexed gather, four tiles in flight
     int kb = 0, ib = 0;
     for (int t0 = 0; t0 < ntiles; t0 += 4) {
-      int tk[4], ti[4], idx[4][4];
-      float v[4][4];
+      int tk[4], ti[4], idx[4][PER];
+      float v[4][PER];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         tk[g] = kb < nblk ? kb : -1;
@@ -383,7 +385,7 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
 #pragma unroll
       for (int g = 0; g < 4; ++g)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < PER; ++u) {
           const int e = l + 16 * u;
           idx[g][u] = block_idx[tk[g] >= 0 ? (size_t)(tk[g] * nblk + ti[g]) * BB + e : 0];
           if (tk[g] < 0) idx[g][u] = nM;
@@ -391,13 +393,13 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
 #pragma unroll
       for (int g = 0; g < 4; ++g)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[g][u] = Mw[idx[g][u] < nM ? idx[g][u] : 0];
+        for (int u = 0; u < PER; ++u) v[g][u] = Mw[idx[g][u] < nM ? idx[g][u] : 0];
 #pragma unroll
       for (int g = 0; g < 4; ++g)
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < PER; ++u)
           if (tk[g] >= 0) {
-            const int e = l + 16 * u, r = e >> 3, c = e & 7;
+            const int e = l + 16 * u, r = e / B, c = e % B;
             float xv = idx[g][u] < nM ? v[g][u] : 0.0f;
             if (ti[g] == tk[g] && (tk[g] + 1) * B > nv && r == c && (nblk - 1) * B + r >= nv) xv = xv + 1.0f;
             U[BB * (t0 + g) + e] = xv;
@@ -406,31 +408,58 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
   }
   for (int i = l; i < pad; i += 16) rhs[i] = i < nv ? y[w * ldy + i] : 0.0f;
   wave_sync();
-  const int c = l & 7, r0 = l >> 3;  // the lane's four elements of a tile: rows r0, r0 + 2, .., column c
   typedef float f32x4 __attribute__((ext_vector_type(4)));
-  const int m4 = l & 3, qr = l >> 3, qc = (l >> 2) & 1;  // and as a lane of quadrant (qr, qc) on the matrix cores
+  typedef float f32x16 __attribute__((ext_vector_type(16)));
+  const int m4 = l & 3, qr = l >> 3, qc = (l >> 2) & 1;  // B = 8: the lane within quadrant (qr, qc) of a tile
   for (int kb = 0; kb < nblk; ++kb) {
     const int k = kb * B, ntile = nblk - kb;
-    // The sums over a finished block row on the matrix cores: v_mfma_f32_4x4x1_16b_f32 does one
-    // fused multiply-add per element of sixteen independent 4 x 4 blocks, and a wavefront's
-    // sixteen blocks are the four quadrants of one 8 x 8 tile of each of its four worlds.  Eight
-    // of them chained from zero are the sum over t = 0..7 ascending of the scalar form.
+    // The sums over a finished block row on the matrix cores, with instructions that do one
+    // fused multiply-add per element and step: chained from zero over t ascending they are
+    // the scalar sums bit for bit.
     for (int tb = 0; tb < ntile; ++tb) {
       const int ib = kb + tb;
-      float *Tv = tile(kb, ib) + (4 * qr) * B + 4 * qc + m4;  // rows 4 qr + 0..3 of column 4 qc + m4
-      f32x4 v;
+      if constexpr (B == 8) {
+        // v_mfma_f32_4x4x1_16b_f32: sixteen independent 4 x 4 blocks, the four quadrants of one
+        // 8 x 8 tile of each of the four worlds
+        float *Tv = tile(kb, ib) + (4 * qr) * B + 4 * qc + m4;  // rows 4 qr + 0..3 of column 4 qc + m4
+        f32x4 v;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = Tv[u * B];
-      for (int jb = 0; jb < kb; ++jb) {
-        const float *Tk = tile(jb, kb) + 4 * qr + m4, *Ti = tile(jb, ib) + 4 * qc + m4;
-        f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int u = 0; u < 4; ++u) v[u] = Tv[u * B];
+        for (int jb = 0; jb < kb; ++jb) {
+          const float *Tk = tile(jb, kb) + 4 * qr + m4, *Ti = tile(jb, ib) + 4 * qc + m4;
+          f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int t = 0; t < B; ++t) sum = __builtin_amdgcn_mfma_f32_4x4x1f32(Tk[t * B], Ti[t * B], sum, 0, 0, 0);
+          for (int t = 0; t < B; ++t) sum = __builtin_amdgcn_mfma_f32_4x4x1f32(Tk[t * B], Ti[t * B], sum, 0, 0, 0);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = v[u] - sum[u];
+          for (int u = 0; u < 4; ++u) v[u] = v[u] - sum[u];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) Tv[u * B] = v[u];  // in place: nothing else reads this tile before
+      } else {
+        // v_mfma_f32_16x16x1_4b_f32: four independent 16 x 16 blocks, one per world.  Block b takes
+        // its operands from the lanes of world b and leaves its result in registers 4 b .. 4 b + 3
+        // of every lane: rows 4 (lane / 16) + 0..3 of column lane % 16.
+        const int toff = (int)(tile(kb, ib) - U) + (4 * q) * B + l;
+        f32x16 v;
+#pragma unroll
+        for (int wb = 0; wb < 4; ++wb)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) v[4 * wb + u] = lds[wb * world_floats + toff + u * B];
+        for (int jb = 0; jb < kb; ++jb) {
+          const float *Tk = tile(jb, kb) + l, *Ti = tile(jb, ib) + l;
+          f32x16 sum;
+#pragma unroll
+          for (int u = 0; u < 16; ++u) sum[u] = 0.0f;
+#pragma unroll
+          for (int t = 0; t < B; ++t) sum = __builtin_amdgcn_mfma_f32_16x16x1f32(Tk[t * B], Ti[t * B], sum, 0, 0, 0);
+#pragma unroll
+          for (int u = 0; u < 16; ++u) v[u] = v[u] - sum[u];
+        }
+#pragma unroll
+        for (int wb = 0; wb < 4; ++wb)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) lds[wb * world_floats + toff + u * B] = v[4 * wb + u];
       }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) Tv[u * B] = v[u];  // in place: nothing else reads this tile before
     }
     if (l < B) {
       float s = rhs[k + l];
@@ -470,12 +499,12 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
     }
     wave_sync();
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int r = r0 + 2 * u;
-      tile(kb, kb)[r * B + c] = c >= r ? L[c * B + r] : 0.0f;
+    for (int u = 0; u < PER; ++u) {
+      const int e = l + 16 * u, r = e / B, c = e % B;
+      tile(kb, kb)[e] = c >= r ? L[c * B + r] : 0.0f;
     }
-    for (int qc = l; qc < (ntile - 1) * B; qc += 16) {
-      const int tb = 1 + (qc >> 3), cc = qc & 7;
+    for (int qn = l; qn < (ntile - 1) * B; qn += 16) {
+      const int tb = 1 + qn / B, cc = qn % B;
       float *Tt = tile(kb, kb + tb);
       float col[B];
 #pragma unroll
@@ -521,9 +550,9 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
     if (Uout) {
       float4 *dst = (float4 *)(Uout + w * (int64_t)pad * pad);
       for (int i4 = l; i4 < pad * pad / 4; i4 += 16) {
-        const int row = 4 * i4 / pad, col = 4 * i4 - row * pad, bi = row >> 3, bj = col >> 3;
+        const int row = 4 * i4 / pad, col = 4 * i4 - row * pad, bi = row / B, bj = col / B;
         float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (bj >= bi) v = *(const float4 *)(tile(bi, bj) + (row & 7) * B + (col & 7));
+        if (bj >= bi) v = *(const float4 *)(tile(bi, bj) + (row % B) * B + (col % B));
         dst[i4] = v;
       }
     }
@@ -917,11 +946,13 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
     const char *e = std::getenv("IMHIP_BLOCKED_KERNEL");
     return e && std::strcmp(e, "simple") == 0;
   }();
-  if (B == 8 && pad <= 64 && !quad_off) {
-    // small matrices, 8 x 8 tiles: four worlds per wavefront
-    const size_t quad_bytes = sizeof(float) * 4 * (size_t)im::quad_world_floats(pad);
-    hipLaunchKernelGGL(im::blocked_factor_solve_quad_kernel, dim3((unsigned)((nworld + 3) / 4)), dim3(64), quad_bytes,
-                       (hipStream_t)stream, M, ldM, nM, block_idx, y, ldy, U, x, ldx, nv, pad, nworld);
+  if (pad <= (B == 8 ? 64 : 48) && !quad_off) {
+    // small matrices: four worlds per wavefront (16 x 16 tiles at pad 64 need 46 KB of LDS per
+    // wavefront, three per CU, and are no faster that way)
+    const size_t quad_bytes = sizeof(float) * 4 * (size_t)im::quad_world_floats(pad, B);
+    auto qfn = B == 8 ? im::blocked_factor_solve_quad_kernel<8> : im::blocked_factor_solve_quad_kernel<16>;
+    hipLaunchKernelGGL(qfn, dim3((unsigned)((nworld + 3) / 4)), dim3(64), quad_bytes, (hipStream_t)stream, M, ldM, nM,
+                       block_idx, y, ldy, U, x, ldx, nv, pad, nworld);
     IM_HIP_CHECK(hipGetLastError());
     return IM_OK;
   }

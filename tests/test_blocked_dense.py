@@ -63,7 +63,7 @@ def test_dense_hessian_oracle_against_fp64():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,B,nworld", [("g1", 8, 70), ("g1", 8, 3), ("snu", 8, 33), ("g1", 16, 70), ("snu", 16, 33), ("stress", 16, 9)])
+@pytest.mark.parametrize("name,B,nworld", [("g1", 8, 70), ("g1", 8, 3), ("snu", 8, 33), ("g1", 16, 70), ("g1", 16, 5), ("snu", 16, 33), ("stress", 16, 9)])
 def test_gpu_blocked_factor_solve_bitwise(device, name, B, nworld):
     import torch
 
@@ -112,7 +112,7 @@ def test_gpu_dense_hessian_mfma(device, name, nworld):
 
 @pytest.mark.gpu
 def test_gpu_wavefront_per_world_kernel_for_small_tiles_agrees():
-    """8 x 8 tiles on matrices up to 64 x 64 run four worlds per wavefront; the kernel with a
+    """Matrices up to 64 x 64 run four worlds per wavefront; the kernel with a
     workgroup per world that serves every other shape is forced here in a child process and
     must pass the same oracle comparison."""
     import os
@@ -124,7 +124,9 @@ def test_gpu_wavefront_per_world_kernel_for_small_tiles_agrees():
         "import sys, torch; sys.path.insert(0, 'tests'); import test_blocked_dense as t;"
         "d = torch.device('cuda:0');"
         "t.test_gpu_blocked_factor_solve_bitwise(d, 'g1', 8, 70);"
-        "t.test_gpu_blocked_factor_solve_bitwise(d, 'snu', 8, 33); print('simple kernel ok')"
+        "t.test_gpu_blocked_factor_solve_bitwise(d, 'snu', 8, 33);"
+        "t.test_gpu_blocked_factor_solve_bitwise(d, 'g1', 16, 70);"
+        "t.test_gpu_blocked_factor_solve_bitwise(d, 'snu', 16, 33); print('simple kernel ok')"
     )
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
