@@ -223,3 +223,54 @@ def test_gpu_wrench_projection_bitwise(device, nworld):
     want = R.project_body_wrenches(force, torque, xipos, com, cdof, rootid, dof_body, parent, order, offsets, root, nt, out_offset=2,
                                    mean=np.full((nworld, nt + 5), 7.0, np.float32))  # fmt: skip
     np.testing.assert_array_equal(mean.cpu().numpy(), want)
+
+
+@pytest.mark.gpu
+def test_gpu_tree_walks_replay_in_a_graph(device):
+    """The three launchers captured in one graph: every replay, with eager work on the same
+    buffers between the replays, gives the eager results bit for bit."""
+    import torch
+
+    nworld = 257
+    rig, topo, force, torque, xipos, com, cdof = _wrench_case(nworld)
+    nb, root, nt = rig.body_count, rig.full_torque_dim - rig.torque_dim, rig.torque_dim
+    parent, rootid, dof_body = (np.asarray(a, np.int32) for a in (topo.body_parentid, topo.body_rootid, topo.dof_bodyid))
+    order, offsets = _levels(parent)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    topology = WP.build_wrench_projection_topology(t(parent), t(dof_body), nb, device)
+    model = type("M", (), dict(body_parentid=parent, body_tree=[order[offsets[i] : offsets[i + 1]] for i in range(len(offsets) - 1)]))
+    scratch = TF.create_tree_reduction_scratch(model, deterministic=True, device=device)
+    rowadr, rownnz, colind = synth.csr_from_parents(synth.snu_parents())
+    tables = [t(a) for a in NF.mul_m_tables(rowadr, rownnz, colind)]
+    rng = np.random.default_rng(4)
+    M, v = t(rng.normal(size=(nworld, len(colind))).astype(np.float32)), t(rng.normal(size=(nworld, len(rowadr))).astype(np.float32))
+    vals0 = t(rng.normal(size=(nworld, nb, 6)).astype(np.float32))
+    ins = dict(body_force=t(force), body_torque=t(torque), xipos=t(xipos), subtree_com=t(com), cdof=t(cdof), body_rootid=t(rootid))
+    vals, mean, mv = vals0.clone(), torch.zeros((nworld, nt), device=device), torch.zeros_like(v)
+
+    def work():
+        vals.copy_(vals0)
+        TF.accumulate(model, None, vals, 6, False, scratch)
+        WP.launch_project_body_wrench_to_torque(topology, **ins, mean=mean, body_count=nb, torque_dim=nt, root_dof_count=root,
+                                                output_dof_offset=0, batch_size=nworld)  # fmt: skip
+        NF.mul_m(M, v, mv, *tables)
+
+    work()
+    torch.cuda.synchronize()
+    want = [a.clone() for a in (vals, mean, mv)]
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        work()
+    torch.cuda.current_stream().wait_stream(s)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        work()
+    for _ in range(3):
+        for a in (vals, mean, mv):
+            a.fill_(float("nan"))  # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for a, b in zip((vals, mean, mv), want):
+            assert torch.equal(a, b)
