@@ -307,8 +307,8 @@ __global__ __launch_bounds__(256) void torque_bounds_kernel(
 }
 
 // ---- one workgroup per world --------------------------------------------------------------
-// One workgroup of 1024 threads per world (two of them share a CU; measured against 256 and
-// 512 threads, which were 20 % and 8 % slower on the 553-segment rig).
+// One workgroup of 512 threads per world (three of them share a CU at the 553-segment rig's
+// 49 KB of LDS; 384, 640, 768 and 1024 threads measured 2 - 7 % slower there).
 // The four contractions above visit every applied segment once per (segment, dof) entry and
 // redo its square root and three divisions each time, and they fetch a muscle's force and a
 // dof's motion axis from memory once per entry.  Here a workgroup first leaves in LDS each
@@ -533,7 +533,7 @@ bool launch_world(const MwArgs &a, int nworld, hipStream_t stream) {
   if (forced_off || lds_bytes > 64 * 1024 || a.nentry == 0 || a.nseg == 0 || a.nrow > 65535 ||
       a.ntorque <= 0 || (MODE != MW_MOMENT && a.nmuscle <= 0))
     return false;
-  hipLaunchKernelGGL(muscle_world_kernel<MODE>, dim3((unsigned)nworld), dim3(1024), lds_bytes, stream, a);
+  hipLaunchKernelGGL(muscle_world_kernel<MODE>, dim3((unsigned)nworld), dim3(512), lds_bytes, stream, a);
   return true;
 }
 
