@@ -428,7 +428,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             for s in range(t.sets(a)):
                 emit(f"  float ga{j}_{a}_{s} = 0.0f;")
     for k in range(nv):
-        emit(f"  float d{k} = 0.0f, nd{k} = 0.0f;")
+        emit(f"  float d{k} = 0.0f;" if not t.depth[k] else f"  float d{k} = 0.0f, nd{k} = 0.0f;")
         if t.depth[k]:
             emit("  float " + ", ".join(f"T{k}_{s} = 0.0f" for s in range(t.sets(k))) + ";")
 
@@ -451,9 +451,9 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
                     expr = f"((0x{mask:x} >> p) & 1) ? SY{j}_{i}_{s_} : ({expr})"
                 emit(f"    {sv(j, i, s_)} = {expr};")
         emit(f"    d{k} = 1.0f / {bc(f'h{k}_{c // 16}', c % 16)};")
-        emit(f"    nd{k} = -d{k};")
         if c == 0:
             return
+        emit(f"    nd{k} = -d{k};")
         vec = (lambda s_: sv(*seg_of[k], s_)) if j is not None else (lambda s_: sv("T", 0, s_))
         # products m_kp * m_kq for every target register, then the right-hand side update
         prods = []  # (pp, s, target)
