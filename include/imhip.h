@@ -407,6 +407,27 @@ int im_project_body_wrenches(const im_body_wrenches *wrenches,
                              int torque_dim, int output_dof_offset, float *mean,
                              int64_t ld_mean, int nworld, void *stream);
 
+/* Replaces gradient_function of the fused Newton kernel
+ * (src/instantmimic/utils/mjw_kernels/newton_stages.py:745-798), one call for all worlds:
+ * a done world only gets search_unchanged = 1; a world whose state_changed_count is 0 gets
+ * search_unchanged = 1 and its grad_dot, newton_decrement and grad_scale rescaled by
+ * ((grad_scale - alpha) / grad_scale)^2 as there; every other world gets
+ * qfrc_constraint[w, dof] = sum over rows r < min(njmax, nefc[w]) ascending of
+ * J[w, r, dof] * efc_force[w, r] (one fused multiply-add per row),
+ * grad = efc_Ma - qfrc_smooth - qfrc_constraint, grad_dot = grad . grad summed as a block of
+ * `block` lanes (32 or 64) sums it -- lane k its dofs k, k + block, .. in order, 32 lanes in
+ * a shuffle-down tree, the trees in order (the reference leaves that order to Warp's
+ * tile_sum) --, newton_decrement = 0, grad_scale = 1, search_unchanged = 0.
+ * J (nworld, njmax, nv) contiguous; nefc and done may be null (all rows, no world done);
+ * done and search_unchanged are bytes. */
+int im_newton_gradient(const int32_t *nefc, const float *J, int njmax, const float *efc_force,
+                       int64_t ld_force, const float *qfrc_smooth, int64_t ld_smooth,
+                       const float *efc_Ma, int64_t ld_Ma, const int32_t *state_changed_count,
+                       const float *alpha, const uint8_t *done, float *qfrc_constraint,
+                       int64_t ld_constraint, float *grad, int64_t ld_grad, float *grad_dot,
+                       float *newton_decrement, float *grad_scale, uint8_t *search_unchanged,
+                       int nv, int block, int nworld, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -139,6 +139,11 @@ SIGNATURES = {
     "im_muscle_sparse_moment": (_i, [_pgeo, _pseg, _vp, _pent, _i, _vp, _i64, _i, _vp]),
     "im_mul_m_sparse": (_i, [_vp, _i64, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i64, _i, _i, _vp]),
     "im_tree_accumulate": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _i64, _i, _i, _vp]),
+    "im_newton_gradient": (
+        _i,
+        [_vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i, _i,
+         _i, _vp],
+    ),  # fmt: skip
     "im_project_body_wrenches": (
         _i,
         [C.POINTER(BodyWrenches), C.POINTER(WrenchTopology), _i, _i, _i, _vp, _i64, _i, _vp],

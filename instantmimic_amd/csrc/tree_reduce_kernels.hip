@@ -214,6 +214,97 @@ __global__ __launch_bounds__(kThreads) void project_wrenches_kernel(WrenchArgs a
   }
 }
 
+// ---- Newton gradient ---------------------------------------------------------------------------
+// qfrc_constraint = J' efc_force, grad = Ma - qfrc_smooth - qfrc_constraint, grad . grad.
+// L lanes per world (32 up to 32 dofs, else 64), a lane per dof, the rows of J streamed ROWS
+// at a time (a row of J is contiguous over the lanes); efc_force sits in LDS.
+struct GradArgs {
+  const int32_t *nefc;
+  const float *J, *force, *smooth, *Ma, *alpha;
+  const int32_t *changed;
+  const uint8_t *done;
+  float *qc, *grad, *grad_dot, *decrement, *scale;
+  uint8_t *unchanged;
+  int64_t ldf, lds_, ldm, ldq, ldg;
+  int njmax, nv, block, nworld, lanes;
+};
+
+template <int ROWS>
+__global__ __launch_bounds__(kThreads) void newton_gradient_kernel(GradArgs a) {
+  extern __shared__ float lds[];
+  const int L = a.lanes, per_block = kThreads / L;
+  const int lw = threadIdx.x / L, lane = threadIdx.x & (L - 1);
+  const int64_t w_raw = (int64_t)blockIdx.x * per_block + lw;
+  const bool live = w_raw < a.nworld;
+  const int64_t w = live ? w_raw : (int64_t)a.nworld - 1;
+  float *f = lds + lw * (a.njmax + a.nv + 64);  // [njmax] forces, then [nv] grad, then [64] lane sums
+  float *gl = f + a.njmax, *part = gl + a.nv;
+  const bool done = a.done && a.done[w] != 0;
+  const bool changed = a.changed[w] != 0;
+  int nefc = a.nefc ? a.nefc[w] : a.njmax;
+  nefc = nefc < a.njmax ? nefc : a.njmax;
+  nefc = nefc > 0 ? nefc : 0;
+  const bool work = !done && changed;
+  if (work)
+    for (int r = lane; r < nefc; r += L) f[r] = a.force[w * a.ldf + r];
+  __syncthreads();  // every thread of the block reaches the barriers: nothing above returns
+  if (work) {
+    const float *Jw = a.J + w * (int64_t)a.njmax * a.nv;
+    for (int dof = lane; dof < a.nv; dof += L) {
+      float sum = 0.0f;
+      for (int r0 = 0; r0 < nefc; r0 += ROWS) {
+        float jv[ROWS];
+#pragma unroll
+        for (int u = 0; u < ROWS; ++u) jv[u] = Jw[(int64_t)(r0 + u < nefc ? r0 + u : nefc - 1) * a.nv + dof];
+#pragma unroll
+        for (int u = 0; u < ROWS; ++u) sum = r0 + u < nefc ? fmaf(jv[u], f[r0 + u], sum) : sum;
+      }
+      const float g = a.Ma[w * a.ldm + dof] - a.smooth[w * a.lds_ + dof] - sum;
+      if (live) {
+        a.qc[w * a.ldq + dof] = sum;
+        a.grad[w * a.ldg + dof] = g;
+      }
+      gl[dof] = g;
+    }
+  }
+  __syncthreads();
+  // grad . grad as a block of `block` lanes would sum it: lane `rank` adds its dofs rank,
+  // rank + block, .. in order, 32 lanes fold in a shuffle-down tree, the folds are added in order
+  if (work) {
+    for (int rank = lane; rank < a.block; rank += L) {
+      float p = 0.0f;
+      for (int dof = rank; dof < a.nv; dof += a.block) p = fmaf(gl[dof], gl[dof], p);
+      part[rank] = p;
+    }
+  }
+  __syncthreads();
+  if (work && lane < 32) {
+    float total = 0.0f;
+    for (int wv = 0; wv < a.block / 32; ++wv) {
+      float v = part[32 * wv + lane];
+      for (int off = 16; off > 0; off >>= 1) v = v + __shfl_down(v, off, 32);
+      total = total + v;
+    }
+    if (lane == 0 && live) {
+      a.grad_dot[w] = total;
+      a.decrement[w] = 0.0f;
+      a.scale[w] = 1.0f;
+    }
+  }
+  if (lane == 0 && live) {
+    a.unchanged[w] = (done || !changed) ? 1 : 0;
+    if (!done && !changed) {
+      const float sigma = a.scale[w], new_sigma = sigma - a.alpha[w];
+      float ratio = 0.0f;
+      if (sigma != 0.0f) ratio = new_sigma / sigma;
+      const float ratio_sq = ratio * ratio;
+      a.grad_dot[w] = a.grad_dot[w] * ratio_sq;
+      a.decrement[w] = a.decrement[w] * ratio_sq;
+      a.scale[w] = new_sigma;
+    }
+  }
+}
+
 // Lanes per world: the smallest power of two in 8..64 that covers `work` items (64 beyond).
 int lanes_for(int work) {
   int lanes = 8;
@@ -301,6 +392,37 @@ extern "C" int im_project_body_wrenches(const im_body_wrenches *wrenches,
   hipLaunchKernelGGL(project_wrenches_kernel,
                      dim3((unsigned)((nworld + per_block - 1) / per_block)), dim3(kThreads),
                      ((size_t)per_block * 6 * nbody + tree_words(nbody, topology->levels)) * 4, (hipStream_t)stream, a);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_newton_gradient(const int32_t *nefc, const float *J, int njmax, const float *efc_force,
+                                  int64_t ld_force, const float *qfrc_smooth, int64_t ld_smooth,
+                                  const float *efc_Ma, int64_t ld_Ma, const int32_t *state_changed_count,
+                                  const float *alpha, const uint8_t *done, float *qfrc_constraint,
+                                  int64_t ld_constraint, float *grad, int64_t ld_grad, float *grad_dot,
+                                  float *newton_decrement, float *grad_scale, uint8_t *search_unchanged, int nv,
+                                  int block, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || njmax < 0) return IM_ERR_ARG;
+  if (block != 32 && block != 64) return IM_ERR_UNSUPPORTED;
+  if (nworld == 0) return IM_OK;
+  if (!J || !efc_force || !qfrc_smooth || !efc_Ma || !state_changed_count || !alpha || !qfrc_constraint || !grad ||
+      !grad_dot || !newton_decrement || !grad_scale || !search_unchanged)
+    return IM_ERR_ARG;
+  if (ld_force < njmax || ld_smooth < nv || ld_Ma < nv || ld_constraint < nv || ld_grad < nv) return IM_ERR_STRIDE;
+  const int lanes = nv <= 32 ? 32 : 64, per_block = kThreads / lanes;
+  const size_t lds_bytes = (size_t)per_block * ((size_t)njmax + nv + 64) * 4;
+  if (lds_bytes > kLdsLimit) return IM_ERR_UNSUPPORTED;
+  GradArgs a{nefc, J, efc_force, qfrc_smooth, efc_Ma, alpha, state_changed_count, done, qfrc_constraint, grad,
+             grad_dot, newton_decrement, grad_scale, search_unchanged, ld_force, ld_smooth, ld_Ma, ld_constraint,
+             ld_grad, njmax, nv, block, nworld, lanes};
+  // a launch of few workgroups (up to four per CU) has few wavefronts to hide the memory's latency
+  // with and asks for sixteen rows at a time; with more of them eight measured faster
+  const unsigned nblocks = (unsigned)((nworld + per_block - 1) / per_block);
+  if (nblocks <= 1024)
+    hipLaunchKernelGGL(newton_gradient_kernel<16>, dim3(nblocks), dim3(kThreads), lds_bytes, (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL(newton_gradient_kernel<8>, dim3(nblocks), dim3(kThreads), lds_bytes, (hipStream_t)stream, a);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

@@ -8,8 +8,10 @@ dof the columns of its full symmetric row and where each element sits in M's tre
 for a model that does not carry them (ancestors root first, the diagonal, then descendants
 ascending -- the upstream order is not visible from the reference's tree).
 
-The rest of that kernel (line search, gradient, convergence) is upstream mujoco_warp code and
-is not part of this module.
+:func:`gradient` is the reference's own ``gradient_function``
+(src/instantmimic/utils/mjw_kernels/newton_stages.py:745-798) for all worlds in one launch.  The
+line search and the convergence test of that kernel are upstream mujoco_warp code and are not
+part of this module.
 """
 
 from __future__ import annotations
@@ -67,3 +69,44 @@ def mul_m(M, vec, out, mulm_rowadr, mulm_col, mulm_madr, *, skip_world: Any = No
             out.data_ptr(), out.stride(0), int(nv), int(nworld), int(torch.cuda.current_stream(M.device).cuda_stream),
         )  # fmt: skip
     _lib.check(status, "im_mul_m_sparse")
+
+
+def gradient(nefc, efc_J, efc_force, qfrc_smooth, efc_Ma, state_changed_count, alpha, done, qfrc_constraint, grad,
+             grad_dot, newton_decrement, grad_scale, search_unchanged, *, block: int = 64) -> None:  # fmt: skip
+    """``qfrc_constraint = J' efc_force``, ``grad = efc_Ma - qfrc_smooth - qfrc_constraint`` and
+    ``grad . grad`` for the worlds whose states changed; the rescaling of ``grad_dot``,
+    ``newton_decrement`` and ``grad_scale`` for the others; ``search_unchanged`` for all (argument
+    names of the reference's gradient_function).  ``efc_J`` (nworld, njmax, nv) contiguous float32;
+    ``nefc`` int32 or None; ``done`` and ``search_unchanged`` bool or uint8; ``block`` = the lane
+    count whose summation order ``grad_dot`` follows (32 or 64)."""
+    import torch
+
+    if efc_J.dim() != 3 or not efc_J.is_contiguous() or efc_J.dtype != torch.float32 or not efc_J.is_cuda:
+        raise TypeError("efc_J must be a contiguous float32 CUDA tensor (nworld, njmax, nv)")
+    nworld, njmax, nv = efc_J.shape
+    rows = (efc_force, qfrc_smooth, efc_Ma, qfrc_constraint, grad)
+    for t, width in zip(rows, (njmax, nv, nv, nv, nv)):
+        if t.dtype != torch.float32 or not t.is_cuda or t.dim() != 2 or t.shape != (nworld, width) or (width > 1 and t.stride(1) != 1):
+            raise TypeError("force, smooth, Ma, constraint and grad must be float32 CUDA tensors with contiguous rows")
+    for t in (alpha, grad_dot, newton_decrement, grad_scale):
+        if t.dtype != torch.float32 or not t.is_cuda or t.numel() != nworld or not t.is_contiguous():
+            raise TypeError("the per-world scalars must be contiguous float32 CUDA tensors")
+    if state_changed_count.dtype != torch.int32 or not state_changed_count.is_contiguous() or state_changed_count.numel() != nworld:
+        raise TypeError("state_changed_count must be a contiguous int32 tensor with one element per world")
+    if nefc is not None and (nefc.dtype != torch.int32 or not nefc.is_contiguous() or nefc.numel() != nworld):
+        raise TypeError("nefc must be a contiguous int32 tensor with one element per world")
+    for t in (done, search_unchanged):
+        if t is not None and (t.dtype not in (torch.bool, torch.uint8) or not t.is_contiguous() or t.numel() != nworld):
+            raise TypeError("done and search_unchanged must be contiguous bool or uint8 tensors with one element per world")
+    if search_unchanged is None:
+        raise TypeError("search_unchanged is an output and cannot be None")
+    with torch.cuda.device(efc_J.device):
+        status = _lib.lib().im_newton_gradient(
+            None if nefc is None else nefc.data_ptr(), efc_J.data_ptr(), int(njmax), efc_force.data_ptr(),
+            efc_force.stride(0), qfrc_smooth.data_ptr(), qfrc_smooth.stride(0), efc_Ma.data_ptr(), efc_Ma.stride(0),
+            state_changed_count.data_ptr(), alpha.data_ptr(), None if done is None else done.data_ptr(),
+            qfrc_constraint.data_ptr(), qfrc_constraint.stride(0), grad.data_ptr(), grad.stride(0), grad_dot.data_ptr(),
+            newton_decrement.data_ptr(), grad_scale.data_ptr(), search_unchanged.data_ptr(), int(nv), int(block),
+            int(nworld), int(torch.cuda.current_stream(efc_J.device).cuda_stream),
+        )  # fmt: skip
+    _lib.check(status, "im_newton_gradient")

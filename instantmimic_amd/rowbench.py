@@ -225,6 +225,18 @@ def run(launches: int = 32) -> None:
         out = torch.zeros((nworld, nv), device=dev)
         sec = _timeit(torch, lambda i: NF.mul_m(Ms[i], Vs[i], out, *tables), nsets, launches)
         _line("im_mul_m_sparse", f"{name} nv={nv} nM={nM} x {nworld} worlds", sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
+    for name, nsets in (("humanoid", 16), ("g1", 8)):
+        b = synth.make_batch(name)
+        nv, nefc, nworld = b.shape.nv, b.shape.nefc, b.nworld
+        Js, Fs = [t(b.J) for _ in range(nsets)], [torch.randn((nworld, nefc), device=dev) for _ in range(nsets)]
+        ne, sm, ma = t(b.nefc), t(b.grad), torch.randn((nworld, nv), device=dev)
+        chg, al = torch.ones(nworld, dtype=torch.int32, device=dev), torch.zeros(nworld, device=dev)
+        qc, gr = torch.zeros((nworld, nv), device=dev), torch.zeros((nworld, nv), device=dev)
+        gd, de, sc = (torch.zeros(nworld, device=dev) for _ in range(3))
+        un = torch.zeros(nworld, dtype=torch.uint8, device=dev)
+        sec = _timeit(torch, lambda i: NF.gradient(ne, Js[i], Fs[i], sm, ma, chg, al, None, qc, gr, gd, de, sc, un), nsets, launches)
+        _line("im_newton_gradient", f"{name} nv={nv} nefc={nefc} x {nworld} worlds", sec,
+              bytes_=nworld * 4 * (nefc * nv + nefc + 4 * nv + 6), nworld=nworld)  # fmt: skip
     topo = rig.topology
     nb, nvf = rig.body_count, rig.full_torque_dim
     parent = np.asarray(topo.body_parentid, np.int32)

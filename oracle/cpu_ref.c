@@ -1147,3 +1147,57 @@ int orc_project_body_wrenches(int nworld, int nbody, int nvfull, const float *bo
   }
   return 0;
 }
+
+/* gradient_function of the fused Newton kernel
+ * (src/instantmimic/utils/mjw_kernels/newton_stages.py:745-798).  The sums over rows and the
+ * squares contract into fused multiply-adds; grad . grad is summed as a block of `block` lanes
+ * with a 32-lane shuffle-down tree, the convention of sp_backward_sums above (the reference
+ * leaves the order to Warp's tile_sum: bit-level agreement with it is unpinned). */
+int orc_newton_gradient(int nworld, int nv, int njmax, int block, const int *nefc, const float *J,
+                        const float *force, const float *smooth, const float *Ma,
+                        const int *changed, const float *alpha, const unsigned char *done,
+                        float *qc, float *grad, float *grad_dot, float *decrement, float *scale,
+                        unsigned char *unchanged) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    const int dn = done && done[w], ch = changed[w] != 0;
+    unchanged[w] = (dn || !ch) ? 1 : 0;
+    if (dn) continue;
+    if (!ch) {
+      const float sigma = scale[w], new_sigma = sigma - alpha[w];
+      float ratio = 0.0f;
+      if (sigma != 0.0f) ratio = new_sigma / sigma;
+      const float ratio_sq = ratio * ratio;
+      grad_dot[w] = grad_dot[w] * ratio_sq;
+      decrement[w] = decrement[w] * ratio_sq;
+      scale[w] = new_sigma;
+      continue;
+    }
+    int ne = nefc ? nefc[w] : njmax;
+    if (ne > njmax) ne = njmax;
+    const float *Jw = J + (size_t)w * njmax * nv, *f = force + (size_t)w * njmax;
+    for (int dof = 0; dof < nv; ++dof) {
+      float sum = 0.0f;
+      for (int r = 0; r < ne; ++r) sum = fmaf(Jw[(size_t)r * nv + dof], f[r], sum);
+      qc[(size_t)w * nv + dof] = sum;
+      grad[(size_t)w * nv + dof] = Ma[(size_t)w * nv + dof] - smooth[(size_t)w * nv + dof] - sum;
+    }
+    float part[64] = {0};
+    for (int lane = 0; lane < block; ++lane)
+      for (int dof = lane; dof < nv; dof += block) {
+        const float g = grad[(size_t)w * nv + dof];
+        part[lane] = fmaf(g, g, part[lane]);
+      }
+    float total = 0.0f;
+    for (int wv = 0; wv < block / 32; ++wv) {
+      float *a = part + 32 * wv;
+      for (int off = 16; off > 0; off >>= 1)
+        for (int i = 0; i < off; ++i) a[i] = a[i] + a[i + off];
+      total = total + a[0];
+    }
+    grad_dot[w] = total;
+    decrement[w] = 0.0f;
+    scale[w] = 1.0f;
+  }
+  return 0;
+}

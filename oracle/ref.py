@@ -486,3 +486,22 @@ def project_body_wrenches(body_force, body_torque, xipos, subtree_com, cdof, roo
         mean.shape[1], _p(mean),
     )  # fmt: skip
     return mean
+
+
+# `newton_gradient`: pinned by the fp64 product J' f and grad = Ma - qfrc_smooth - J' f, by
+# grad_dot against the fp64 dot product, and by the closed form of the rescaling branch; the
+# order in which a block adds its lanes' partial sums is unpinned (Warp's tile_sum).
+def newton_gradient(J, force, smooth, Ma, changed, alpha, grad_dot, decrement, scale, nefc=None, done=None, block=64):
+    """Returns (qfrc_constraint, grad, grad_dot, decrement, scale, search_unchanged); the three
+    per-world scalars start from the arrays passed in (copied)."""
+    J, force, smooth, Ma, alpha = (_f(a) for a in (J, force, smooth, Ma, alpha))
+    nworld, njmax, nv = J.shape
+    qc, grad = np.zeros((nworld, nv), np.float32), np.zeros((nworld, nv), np.float32)
+    gd, de, sc = (_f(a).copy() for a in (grad_dot, decrement, scale))
+    un = np.zeros(nworld, np.uint8)
+    dn = None if done is None else np.ascontiguousarray(done, np.uint8)
+    lib().orc_newton_gradient(
+        nworld, nv, njmax, block, None if nefc is None else _p(_i(nefc)), _p(J), _p(force), _p(smooth), _p(Ma),
+        _p(_i(changed)), _p(alpha), None if dn is None else _p(dn), _p(qc), _p(grad), _p(gd), _p(de), _p(sc), _p(un),
+    )  # fmt: skip
+    return qc, grad, gd, de, sc, un

@@ -274,3 +274,73 @@ def test_gpu_tree_walks_replay_in_a_graph(device):
         torch.cuda.synchronize()
         for a, b in zip((vals, mean, mv), want):
             assert torch.equal(a, b)
+
+
+# ---------------------------------------------------------------- Newton gradient
+def _gradient_case(name, nworld, seed=9):
+    b = synth.make_batch(name, nworld, ragged_nefc=True)
+    rng = np.random.default_rng(seed)
+    njmax, nv = b.J.shape[1], b.J.shape[2]
+    force = rng.normal(0, 3, (nworld, njmax)).astype(np.float32)
+    smooth = rng.normal(0, 1, (nworld, nv)).astype(np.float32)
+    Ma = rng.normal(0, 1, (nworld, nv)).astype(np.float32)
+    changed = rng.integers(0, 3, nworld).astype(np.int32)  # a third of the worlds keep their states
+    done = (rng.uniform(size=nworld) < 0.15).astype(np.uint8)
+    alpha = rng.uniform(0, 0.5, nworld).astype(np.float32)
+    scalars = [rng.uniform(0.5, 2, nworld).astype(np.float32) for _ in range(3)]
+    scalars[2][::11] = 0.0  # a zero scale: the ratio is defined as 0
+    return b, force, smooth, Ma, changed, alpha, done, scalars
+
+
+@pytest.mark.parametrize("name,block", [("ant", 32), ("humanoid", 64), ("snu", 32), ("stress", 64)])
+def test_oracle_newton_gradient_against_fp64(name, block):
+    nworld = 40
+    b, force, smooth, Ma, changed, alpha, done, (gd0, de0, sc0) = _gradient_case(name, nworld)
+    qc, grad, gd, de, sc, un = R.newton_gradient(b.J, force, smooth, Ma, changed, alpha, gd0, de0, sc0, nefc=b.nefc, done=done, block=block)
+    np.testing.assert_array_equal(un, ((done != 0) | (changed == 0)).astype(np.uint8))
+    work = (done == 0) & (changed != 0)
+    rows = np.arange(b.J.shape[1])[None, :] < b.nefc[:, None]
+    qc64 = np.einsum("wrd,wr->wd", b.J.astype(np.float64) * rows[:, :, None], force.astype(np.float64))
+    g64 = Ma.astype(np.float64) - smooth - qc64
+    assert R.rel_l2(qc[work], qc64[work]) < 1e-6 and R.rel_l2(grad[work], g64[work]) < 1e-6
+    np.testing.assert_allclose(gd[work], (g64[work] ** 2).sum(1), rtol=1e-5)
+    assert (de[work] == 0).all() and (sc[work] == 1).all()
+    # untouched where done; rescaled where the states did not change
+    d = done != 0
+    assert (qc[~work] == 0).all() and (grad[~work] == 0).all()
+    for got, was in ((gd, gd0), (de, de0), (sc, sc0)):
+        np.testing.assert_array_equal(got[d], was[d])
+    keep = (done == 0) & (changed == 0)
+    new_sigma = sc0 - alpha
+    ratio = np.where(sc0 != 0, new_sigma / np.where(sc0 != 0, sc0, 1), 0).astype(np.float32)
+    np.testing.assert_array_equal(sc[keep], new_sigma[keep])
+    np.testing.assert_array_equal(gd[keep], (gd0 * (ratio * ratio))[keep])
+    np.testing.assert_array_equal(de[keep], (de0 * (ratio * ratio))[keep])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,nworld,block", [("ant", 64, 32), ("humanoid", 4096, 64), ("g1", 333, 32), ("snu", 130, 64), ("stress", 37, 64)])
+def test_gpu_newton_gradient_bitwise(device, name, nworld, block):
+    import torch
+
+    b, force, smooth, Ma, changed, alpha, done, (gd0, de0, sc0) = _gradient_case(name, nworld)
+    nv = b.J.shape[2]
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    qc, grad = torch.full((nworld, nv), 7.0, device=device), torch.full((nworld, nv), 7.0, device=device)
+    gd, de, sc = t(gd0), t(de0), t(sc0)
+    un = torch.full((nworld,), 9, dtype=torch.uint8, device=device)
+    NF.gradient(t(b.nefc), t(b.J), t(force), t(smooth), t(Ma), t(changed), t(alpha), t(done), qc, grad, gd, de, sc, un, block=block)
+    torch.cuda.synchronize()
+    want = R.newton_gradient(b.J, force, smooth, Ma, changed, alpha, gd0, de0, sc0, nefc=b.nefc, done=done, block=block)
+    work = (done == 0) & (changed != 0)
+    np.testing.assert_array_equal(qc.cpu().numpy()[work], want[0][work])
+    np.testing.assert_array_equal(grad.cpu().numpy()[work], want[1][work])
+    assert (qc.cpu().numpy()[~work] == 7.0).all() and (grad.cpu().numpy()[~work] == 7.0).all()
+    for got, ref in zip((gd, de, sc, un), want[2:]):
+        np.testing.assert_array_equal(got.cpu().numpy(), ref)
+    # without the optional arrays: every row counts, no world is done
+    NF.gradient(None, t(b.J), t(force), t(smooth), t(Ma), t(changed), t(alpha), None, qc, grad, t(gd0), t(de0), t(sc0), un, block=block)
+    torch.cuda.synchronize()
+    want = R.newton_gradient(b.J, force, smooth, Ma, changed, alpha, gd0, de0, sc0, block=block)
+    np.testing.assert_array_equal(qc.cpu().numpy()[changed != 0], want[0][changed != 0])
+    np.testing.assert_array_equal(un.cpu().numpy(), want[5])
