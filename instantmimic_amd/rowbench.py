@@ -225,7 +225,7 @@ def run(launches: int = 32) -> None:
         out = torch.zeros((nworld, nv), device=dev)
         sec = _timeit(torch, lambda i: NF.mul_m(Ms[i], Vs[i], out, *tables), nsets, launches)
         _line("im_mul_m_sparse", f"{name} nv={nv} nM={nM} x {nworld} worlds", sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
-    for name, nsets in (("humanoid", 16), ("g1", 8)):
+    for name, nsets in (("humanoid", 16), ("g1", 8), ("snu", 8)):
         b = synth.make_batch(name)
         nv, nefc, nworld = b.shape.nv, b.shape.nefc, b.nworld
         Js, Fs = [t(b.J) for _ in range(nsets)], [torch.randn((nworld, nefc), device=dev) for _ in range(nsets)]
