@@ -428,6 +428,18 @@ int im_newton_gradient(const int32_t *nefc, const float *J, int njmax, const flo
                        float *newton_decrement, float *grad_scale, uint8_t *search_unchanged,
                        int nv, int block, int nworld, void *stream);
 
+/* Replaces the J v step of the fused Newton kernel's line search
+ * (src/instantmimic/utils/mjw_kernels/newton_stages.py:157-178): jv[w, r] = sum over the dofs
+ * of J[w, r, i] * search[w, i] for the rows r < min(njmax, nefc[w]); rows beyond keep their
+ * values.  Up to 50 dofs one chain of fused multiply-adds, i ascending; beyond, as the
+ * reference does to match upstream, partial sums over 20 dofs each (chains from 0) added to
+ * the total one after the other with a rounding of their own.  skip_world (bytes, may be
+ * null): worlds that are done or whose search direction did not change keep their jv.
+ * J (nworld, njmax, nv) contiguous, search (nworld, ld >= nv), jv (nworld, ld >= njmax). */
+int im_newton_jv(const float *J, int njmax, const int32_t *nefc, const float *search,
+                 int64_t ld_search, const uint8_t *skip_world, float *jv, int64_t ld_jv, int nv,
+                 int nworld, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

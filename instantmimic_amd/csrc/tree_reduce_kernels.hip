@@ -305,6 +305,75 @@ __global__ __launch_bounds__(kThreads) void newton_gradient_kernel(GradArgs a) {
   }
 }
 
+// ---- J v per constraint row ------------------------------------------------------------------
+// One wavefront takes 64 rows of one world: the rows (contiguous in memory) travel through LDS
+// with coalesced loads, sixteen in flight per lane, and a lane then walks its own row (rows sit
+// an odd number of words apart in LDS).  Up to 50 dofs the sum is one chain of fused
+// multiply-adds; beyond, partial sums over 20 dofs each are added with a rounding of their own.
+__global__ __launch_bounds__(64) void newton_jv_kernel(
+    const float *__restrict__ J, int njmax, const int32_t *__restrict__ nefc_p,
+    const float *__restrict__ search, int64_t lds_, const uint8_t *__restrict__ skip,
+    float *__restrict__ jv, int64_t ldj, int nv, int chunks) {
+  extern __shared__ float lds[];
+  const int lane = threadIdx.x;
+  const int64_t w = blockIdx.x / chunks;
+  const int r0 = (int)(blockIdx.x % chunks) * 64;
+  if (skip && skip[w]) return;  // the whole wavefront: no barrier is left behind
+  int nefc = nefc_p ? nefc_p[w] : njmax;
+  nefc = nefc < njmax ? nefc : njmax;
+  if (r0 >= nefc) return;
+  const int rows = nefc - r0 < 64 ? nefc - r0 : 64;
+  const int stride = nv | 1;
+  float *sv = lds + 64 * stride;  // [nv] the search direction
+  const float *src = J + (w * njmax + r0) * (int64_t)nv;
+  const int total = rows * nv;
+  const float inv_nv = 1.0f / (float)nv;
+  for (int i0 = lane; i0 < total; i0 += 16 * 64) {
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v[u] = src[i0 + 64 * u < total ? i0 + 64 * u : total - 1];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int i = i0 + 64 * u;
+      if (i < total) {
+        const int r = (int)(((float)i + 0.5f) * inv_nv);  // i / nv, exact while i stays below 2^20
+        lds[r * stride + (i - r * nv)] = v[u];
+      }
+    }
+  }
+  for (int i = lane; i < nv; i += 64) sv[i] = search[w * lds_ + i];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (lane < rows) {
+    const float *row = lds + lane * stride;
+    // a chain of fused multiply-adds over [i0, i1), eight operand pairs read ahead of the first
+    auto chain = [&](int i0, int i1) {
+      float p = 0.0f;
+      int i = i0;
+      for (; i + 8 <= i1; i += 8) {
+        float x[8], y[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          x[u] = row[i + u];
+          y[u] = sv[i + u];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) p = fmaf(x[u], y[u], p);
+      }
+      for (; i < i1; ++i) p = fmaf(row[i], sv[i], p);
+      return p;
+    };
+    float acc = 0.0f;
+    if (nv > 50) {
+      for (int start = 0; start < nv; start += 20) acc = acc + chain(start, start + 20 < nv ? start + 20 : nv);
+    } else {
+      acc = chain(0, nv);
+    }
+    jv[w * ldj + r0 + lane] = acc;
+  }
+}
+
 // Lanes per world: the smallest power of two in 8..64 that covers `work` items (64 beyond).
 int lanes_for(int work) {
   int lanes = 8;
@@ -423,6 +492,22 @@ extern "C" int im_newton_gradient(const int32_t *nefc, const float *J, int njmax
     hipLaunchKernelGGL(newton_gradient_kernel<16>, dim3(nblocks), dim3(kThreads), lds_bytes, (hipStream_t)stream, a);
   else
     hipLaunchKernelGGL(newton_gradient_kernel<8>, dim3(nblocks), dim3(kThreads), lds_bytes, (hipStream_t)stream, a);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_newton_jv(const float *J, int njmax, const int32_t *nefc, const float *search, int64_t ld_search,
+                            const uint8_t *skip_world, float *jv, int64_t ld_jv, int nv, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || njmax < 0) return IM_ERR_ARG;
+  if (nworld == 0 || njmax == 0) return IM_OK;
+  if (!J || !search || !jv) return IM_ERR_ARG;
+  if (ld_search < nv || ld_jv < njmax) return IM_ERR_STRIDE;
+  const size_t lds_bytes = (64 * (size_t)(nv | 1) + nv) * 4;
+  if (lds_bytes > kLdsLimit || 64 * (int64_t)nv >= (1 << 20)) return IM_ERR_UNSUPPORTED;
+  const int chunks = (njmax + 63) / 64;
+  if ((int64_t)nworld * chunks > 0x7fffffff) return IM_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(newton_jv_kernel, dim3((unsigned)((int64_t)nworld * chunks)), dim3(64), lds_bytes,
+                     (hipStream_t)stream, J, njmax, nefc, search, ld_search, skip_world, jv, ld_jv, nv, chunks);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

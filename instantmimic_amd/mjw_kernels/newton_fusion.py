@@ -9,9 +9,9 @@ for a model that does not carry them (ancestors root first, the diagonal, then d
 ascending -- the upstream order is not visible from the reference's tree).
 
 :func:`gradient` is the reference's own ``gradient_function``
-(src/instantmimic/utils/mjw_kernels/newton_stages.py:745-798) for all worlds in one launch.  The
-line search and the convergence test of that kernel are upstream mujoco_warp code and are not
-part of this module.
+(src/instantmimic/utils/mjw_kernels/newton_stages.py:745-798) and :func:`jv` the ``J v`` step at
+the head of its line search (:157-178), each for all worlds in one launch.  The scalar search
+itself and the convergence test are upstream mujoco_warp code and are not part of this module.
 """
 
 from __future__ import annotations
@@ -110,3 +110,30 @@ def gradient(nefc, efc_J, efc_force, qfrc_smooth, efc_Ma, state_changed_count, a
             int(nworld), int(torch.cuda.current_stream(efc_J.device).cuda_stream),
         )  # fmt: skip
     _lib.check(status, "im_newton_gradient")
+
+
+def jv(efc_J, search, jv_out, *, nefc=None, skip_world: Any = None) -> None:
+    """``jv_out[w, r] = J[w, r, :] . search[w]`` for the rows below ``nefc[w]``, with the
+    reference's summation rule (one chain up to 50 dofs, 20-dof partial sums beyond).  Worlds
+    whose ``skip_world`` byte is set (done, or search direction unchanged) keep their row."""
+    import torch
+
+    if efc_J.dim() != 3 or not efc_J.is_contiguous() or efc_J.dtype != torch.float32 or not efc_J.is_cuda:
+        raise TypeError("efc_J must be a contiguous float32 CUDA tensor (nworld, njmax, nv)")
+    nworld, njmax, nv = efc_J.shape
+    for t, width in ((search, nv), (jv_out, njmax)):
+        if t.dtype != torch.float32 or not t.is_cuda or t.dim() != 2 or t.shape != (nworld, width) or (width > 1 and t.stride(1) != 1):
+            raise TypeError("search (nworld, nv) and jv_out (nworld, njmax) must be float32 CUDA tensors with contiguous rows")
+    if nefc is not None and (nefc.dtype != torch.int32 or not nefc.is_contiguous() or nefc.numel() != nworld):
+        raise TypeError("nefc must be a contiguous int32 tensor with one element per world")
+    if skip_world is not None and (
+        skip_world.dtype not in (torch.bool, torch.uint8) or not skip_world.is_contiguous() or skip_world.numel() != nworld
+    ):
+        raise TypeError("skip_world must be a contiguous bool or uint8 tensor with one element per world")
+    with torch.cuda.device(efc_J.device):
+        status = _lib.lib().im_newton_jv(
+            efc_J.data_ptr(), int(njmax), None if nefc is None else nefc.data_ptr(), search.data_ptr(), search.stride(0),
+            None if skip_world is None else skip_world.data_ptr(), jv_out.data_ptr(), jv_out.stride(0), int(nv), int(nworld),
+            int(torch.cuda.current_stream(efc_J.device).cuda_stream),
+        )  # fmt: skip
+    _lib.check(status, "im_newton_jv")

@@ -237,6 +237,9 @@ def run(launches: int = 32) -> None:
         sec = _timeit(torch, lambda i: NF.gradient(ne, Js[i], Fs[i], sm, ma, chg, al, None, qc, gr, gd, de, sc, un), nsets, launches)
         _line("im_newton_gradient", f"{name} nv={nv} nefc={nefc} x {nworld} worlds", sec,
               bytes_=nworld * 4 * (nefc * nv + nefc + 4 * nv + 6), nworld=nworld)  # fmt: skip
+        jvo = torch.zeros((nworld, nefc), device=dev)
+        sec = _timeit(torch, lambda i: NF.jv(Js[i], sm, jvo, nefc=ne), nsets, launches)
+        _line("im_newton_jv", f"{name} nv={nv} nefc={nefc} x {nworld} worlds", sec, bytes_=nworld * 4 * (nefc * nv + nefc + nv), nworld=nworld)
     topo = rig.topology
     nb, nvf = rig.body_count, rig.full_torque_dim
     parent = np.asarray(topo.body_parentid, np.int32)

@@ -1201,3 +1201,33 @@ int orc_newton_gradient(int nworld, int nv, int njmax, int block, const int *nef
   }
   return 0;
 }
+
+/* The J v step of the line search (src/instantmimic/utils/mjw_kernels/newton_stages.py:157-178):
+ * one chain of fused multiply-adds up to 50 dofs; beyond, 20-dof partial sums added with their
+ * own rounding (rounded_step(jv, 1.0, partial) = jv + 1.0 * partial without contraction). */
+int orc_newton_jv(int nworld, int nv, int njmax, const int *nefc, const float *J,
+                  const float *search, const unsigned char *skip, float *jv) {
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    if (skip && skip[w]) continue;
+    int ne = nefc ? nefc[w] : njmax;
+    if (ne > njmax) ne = njmax;
+    const float *s = search + (size_t)w * nv;
+    for (int r = 0; r < ne; ++r) {
+      const float *row = J + ((size_t)w * njmax + r) * nv;
+      float acc = 0.0f;
+      if (nv > 50) {
+        for (int start = 0; start < nv; start += 20) {
+          const int end = start + 20 < nv ? start + 20 : nv;
+          float partial = 0.0f;
+          for (int i = start; i < end; ++i) partial = fmaf(row[i], s[i], partial);
+          acc = acc + partial;
+        }
+      } else {
+        for (int i = 0; i < nv; ++i) acc = fmaf(row[i], s[i], acc);
+      }
+      jv[(size_t)w * njmax + r] = acc;
+    }
+  }
+  return 0;
+}

@@ -505,3 +505,15 @@ def newton_gradient(J, force, smooth, Ma, changed, alpha, grad_dot, decrement, s
         _p(_i(changed)), _p(alpha), None if dn is None else _p(dn), _p(qc), _p(grad), _p(gd), _p(de), _p(sc), _p(un),
     )  # fmt: skip
     return qc, grad, gd, de, sc, un
+
+
+# `newton_jv`: pinned by the fp64 product J v; the chunking rule above 50 dofs is the
+# reference's own statement and is exercised on both sides of the threshold.
+def newton_jv(J, search, nefc=None, skip=None, out=None):
+    J, search = _f(J), _f(search)
+    nworld, njmax, nv = J.shape
+    out = np.zeros((nworld, njmax), np.float32) if out is None else out
+    sk = None if skip is None else np.ascontiguousarray(skip, np.uint8)
+    lib().orc_newton_jv(nworld, nv, njmax, None if nefc is None else _p(_i(nefc)), _p(J), _p(search),
+                        None if sk is None else _p(sk), _p(out))  # fmt: skip
+    return out

@@ -344,3 +344,48 @@ def test_gpu_newton_gradient_bitwise(device, name, nworld, block):
     want = R.newton_gradient(b.J, force, smooth, Ma, changed, alpha, gd0, de0, sc0, block=block)
     np.testing.assert_array_equal(qc.cpu().numpy()[changed != 0], want[0][changed != 0])
     np.testing.assert_array_equal(un.cpu().numpy(), want[5])
+
+
+# ---------------------------------------------------------------- J v of the line search
+@pytest.mark.parametrize("name", ["ant", "humanoid", "snu", "stress"])
+def test_oracle_newton_jv_against_fp64(name):
+    nworld = 24
+    b = synth.make_batch(name, nworld, ragged_nefc=True)
+    rng = np.random.default_rng(2)
+    search = rng.normal(size=(nworld, b.J.shape[2])).astype(np.float32)
+    skip = np.zeros(nworld, np.uint8)
+    skip[::5] = 1
+    got = R.newton_jv(b.J, search, nefc=b.nefc, skip=skip, out=np.full(b.J.shape[:2], 7.0, np.float32))
+    want = np.einsum("wrd,wd->wr", b.J.astype(np.float64), search.astype(np.float64))
+    rows = np.arange(b.J.shape[1])[None, :] < b.nefc[:, None]
+    live = rows & (skip == 0)[:, None]
+    assert np.abs(got[live] - want[live]).max() <= 1e-5 * np.abs(want).max()
+    assert (got[~live] == 7.0).all()
+    # one chain up to 50 dofs: the same bits as a running fused multiply-add in numpy's float32
+    if b.J.shape[2] <= 50:
+        w, r = int(np.flatnonzero(skip == 0)[0]), 0
+        acc = np.float32(0)
+        for i in range(b.J.shape[2]):
+            acc = np.float32(np.float64(b.J[w, r, i]) * np.float64(search[w, i]) + np.float64(acc))  # exact product, one rounding
+        assert got[w, r] == acc
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,nworld", [("ant", 64), ("humanoid", 4096), ("g1", 333), ("snu", 130), ("stress", 37)])
+def test_gpu_newton_jv_bitwise(device, name, nworld):
+    import torch
+
+    b = synth.make_batch(name, nworld, ragged_nefc=True)
+    njmax, nv = b.J.shape[1], b.J.shape[2]
+    rng = np.random.default_rng(2)
+    search = rng.normal(size=(nworld, nv)).astype(np.float32)
+    skip = (rng.uniform(size=nworld) < 0.2).astype(np.uint8)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    out = torch.full((nworld, njmax), 7.0, device=device)
+    NF.jv(t(b.J), t(search), out, nefc=t(b.nefc), skip_world=t(skip))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), R.newton_jv(b.J, search, nefc=b.nefc, skip=skip, out=np.full((nworld, njmax), 7.0, np.float32)))
+    out.fill_(7.0)
+    NF.jv(t(b.J), t(search), out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), R.newton_jv(b.J, search))
