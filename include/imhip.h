@@ -440,6 +440,31 @@ int im_newton_jv(const float *J, int njmax, const int32_t *nefc, const float *se
                  int64_t ld_search, const uint8_t *skip_world, float *jv, int64_t ld_jv, int nv,
                  int nworld, void *stream);
 
+/* Replaces the step along the search direction at the end of the fused Newton kernel's line
+ * search (src/instantmimic/utils/mjw_kernels/newton_stages.py:373-381): for the worlds that
+ * are not done, qacc += alpha[w] search and efc_Ma += alpha[w] mv (one fused multiply-add
+ * each), Jaref[r] = Jaref[r] + alpha[w] * jv[r] for r < min(njmax, nefc[w]) (product and sum
+ * rounded separately: the reference's rounded_step, :18-19).  All arrays (nworld, ld). */
+int im_newton_advance(const float *alpha, const float *search, int64_t ld_search, const float *mv,
+                      int64_t ld_mv, const float *jv, int64_t ld_jv, const int32_t *nefc,
+                      const uint8_t *done, float *qacc, int64_t ld_qacc, float *efc_Ma,
+                      int64_t ld_Ma, float *Jaref, int64_t ld_Jaref, int nv, int njmax, int nworld,
+                      void *stream);
+
+/* Replaces the listing of the changed rows that follows it (newton_stages.py:403-426): among
+ * the rows r < min(njmax, nefc[w]), those with (old_state == quad) != (new_state == quad) are
+ * written to quad_changed_ids[w, :] in ascending order and counted in quad_changed_count[w]
+ * (the ids and count that im_sparse_update_factor / im_dense_update_factor take), and
+ * state_changed_count[w] = the rows with old_state != new_state (the reference adds one more
+ * when its line search is exhausted: the caller's).  The reference evaluates the new states
+ * in the same loop with upstream's _eval_constraint and overwrites the old ones in place;
+ * here the two state arrays (nworld, njmax) are inputs.  Done worlds are left alone.
+ * Integer work: bit-exact. */
+int im_newton_changed_rows(const int32_t *old_state, const int32_t *new_state, int njmax,
+                           const int32_t *nefc, int quad, const uint8_t *done,
+                           int32_t *quad_changed_ids, int ld_ids, int32_t *quad_changed_count,
+                           int32_t *state_changed_count, int nworld, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -145,6 +145,11 @@ SIGNATURES = {
          _i, _vp],
     ),  # fmt: skip
     "im_newton_jv": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _vp, _i64, _i, _i, _vp]),
+    "im_newton_advance": (
+        _i,
+        [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _vp],
+    ),
+    "im_newton_changed_rows": (_i, [_vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _i, _vp]),
     "im_project_body_wrenches": (
         _i,
         [C.POINTER(BodyWrenches), C.POINTER(WrenchTopology), _i, _i, _i, _vp, _i64, _i, _vp],

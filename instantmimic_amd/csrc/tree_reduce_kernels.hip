@@ -374,6 +374,64 @@ __global__ __launch_bounds__(64) void newton_jv_kernel(
   }
 }
 
+// ---- the step along the search direction and the rows whose state changed ----------------------
+// qacc += alpha search, Ma += alpha mv (contracted), Jaref = Jaref + alpha * jv (two roundings,
+// as the reference spells it out); one thread per element, a world per blockIdx.y.
+__global__ __launch_bounds__(kThreads) void newton_advance_kernel(
+    const float *__restrict__ alpha, const float *__restrict__ search, int64_t lds_,
+    const float *__restrict__ mv, int64_t ldm, const float *__restrict__ jv, int64_t ldj,
+    const int32_t *__restrict__ nefc_p, const uint8_t *__restrict__ done, float *__restrict__ qacc, int64_t ldq,
+    float *__restrict__ Ma, int64_t lda, float *__restrict__ jaref, int64_t ldr, int nv, int njmax) {
+  const int64_t w = blockIdx.y;
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (done && done[w]) return;
+  const float a = alpha[w];
+  if (i < nv) {
+    qacc[w * ldq + i] = fmaf(a, search[w * lds_ + i], qacc[w * ldq + i]);
+    Ma[w * lda + i] = fmaf(a, mv[w * ldm + i], Ma[w * lda + i]);
+  }
+  int nefc = nefc_p ? nefc_p[w] : njmax;
+  nefc = nefc < njmax ? nefc : njmax;
+  if (i < nefc) jaref[w * ldr + i] = jaref[w * ldr + i] + a * jv[w * ldj + i];
+}
+
+// Rows whose state differs between two state arrays: the ones whose being quadratic flipped are
+// listed in ascending order (64 rows per ballot), the others only counted.  One wavefront per
+// world, four worlds per workgroup.
+__global__ __launch_bounds__(kThreads) void newton_changed_rows_kernel(
+    const int32_t *__restrict__ old_state, const int32_t *__restrict__ new_state, int njmax,
+    const int32_t *__restrict__ nefc_p, int quad, const uint8_t *__restrict__ done,
+    int32_t *__restrict__ ids, int ld_ids, int32_t *__restrict__ quad_count,
+    int32_t *__restrict__ state_count, int nworld) {
+  const int lane = threadIdx.x & 63;
+  const int64_t w = (int64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+  if (w >= nworld || (done && done[w])) return;  // a whole wavefront: no barrier follows
+  int nefc = nefc_p ? nefc_p[w] : njmax;
+  nefc = nefc < njmax ? nefc : njmax;
+  const int32_t *so = old_state + w * njmax, *sn = new_state + w * njmax;
+  int count = 0, any = 0;
+  for (int base = 0; base < nefc; base += 64) {
+    const int r = base + lane;
+    int o = 0, n = 0;
+    if (r < nefc) {
+      o = so[r];
+      n = sn[r];
+    }
+    const bool flip = r < nefc && ((o == quad) != (n == quad));
+    const unsigned long long mask = __ballot(flip);
+    if (flip) {
+      const int slot = count + __popcll(mask & ((1ull << lane) - 1ull));
+      if (slot < ld_ids) ids[w * ld_ids + slot] = r;
+    }
+    count += __popcll(mask);
+    any += __popcll(__ballot(r < nefc && o != n));
+  }
+  if (lane == 0) {
+    quad_count[w] = count;
+    state_count[w] = any;
+  }
+}
+
 // Lanes per world: the smallest power of two in 8..64 that covers `work` items (64 beyond).
 int lanes_for(int work) {
   int lanes = 8;
@@ -508,6 +566,44 @@ extern "C" int im_newton_jv(const float *J, int njmax, const int32_t *nefc, cons
   if ((int64_t)nworld * chunks > 0x7fffffff) return IM_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(newton_jv_kernel, dim3((unsigned)((int64_t)nworld * chunks)), dim3(64), lds_bytes,
                      (hipStream_t)stream, J, njmax, nefc, search, ld_search, skip_world, jv, ld_jv, nv, chunks);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_newton_advance(const float *alpha, const float *search, int64_t ld_search, const float *mv,
+                                 int64_t ld_mv, const float *jv, int64_t ld_jv, const int32_t *nefc,
+                                 const uint8_t *done, float *qacc, int64_t ld_qacc, float *efc_Ma, int64_t ld_Ma,
+                                 float *Jaref, int64_t ld_Jaref, int nv, int njmax, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || njmax < 0) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!alpha || !search || !mv || !qacc || !efc_Ma || (njmax > 0 && (!jv || !Jaref))) return IM_ERR_ARG;
+  if (ld_search < nv || ld_mv < nv || ld_qacc < nv || ld_Ma < nv || ld_jv < njmax || ld_Jaref < njmax)
+    return IM_ERR_STRIDE;
+  const int n = nv > njmax ? nv : njmax;
+  for (int w0 = 0; w0 < nworld; w0 += 65535) {  // the grid's y dimension carries the world
+    const int nw = nworld - w0 < 65535 ? nworld - w0 : 65535;
+    hipLaunchKernelGGL(newton_advance_kernel, dim3((unsigned)((n + kThreads - 1) / kThreads), (unsigned)nw),
+                       dim3(kThreads), 0, (hipStream_t)stream, alpha + w0, search + w0 * ld_search, ld_search,
+                       mv + w0 * ld_mv, ld_mv, jv ? jv + w0 * ld_jv : nullptr, ld_jv, nefc ? nefc + w0 : nullptr,
+                       done ? done + w0 : nullptr, qacc + w0 * ld_qacc, ld_qacc, efc_Ma + w0 * ld_Ma, ld_Ma,
+                       Jaref ? Jaref + w0 * ld_Jaref : nullptr, ld_Jaref, nv, njmax);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_newton_changed_rows(const int32_t *old_state, const int32_t *new_state, int njmax,
+                                      const int32_t *nefc, int quad, const uint8_t *done, int32_t *quad_changed_ids,
+                                      int ld_ids, int32_t *quad_changed_count, int32_t *state_changed_count,
+                                      int nworld, void *stream) {
+  if (nworld < 0 || njmax < 0 || ld_ids < 0) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!old_state || !new_state || !quad_changed_ids || !quad_changed_count || !state_changed_count)
+    return IM_ERR_ARG;
+  const int per_block = kThreads / 64;
+  hipLaunchKernelGGL(newton_changed_rows_kernel, dim3((unsigned)((nworld + per_block - 1) / per_block)),
+                     dim3(kThreads), 0, (hipStream_t)stream, old_state, new_state, njmax, nefc, quad, done,
+                     quad_changed_ids, ld_ids, quad_changed_count, state_changed_count, nworld);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

@@ -10,8 +10,12 @@ ascending -- the upstream order is not visible from the reference's tree).
 
 :func:`gradient` is the reference's own ``gradient_function``
 (src/instantmimic/utils/mjw_kernels/newton_stages.py:745-798) and :func:`jv` the ``J v`` step at
-the head of its line search (:157-178), each for all worlds in one launch.  The scalar search
-itself and the convergence test are upstream mujoco_warp code and are not part of this module.
+the head of its line search (:157-178); :func:`advance` is the step along the search direction
+at its end (:373-381) and :func:`changed_rows` the listing of the rows whose state changed
+(:403-426), which is what the factor stage of the next iteration takes.  Each runs for all
+worlds in one launch.  The scalar search itself, the evaluation of the constraints' new states
+and forces and the convergence test are upstream mujoco_warp code and are not part of this
+module.
 """
 
 from __future__ import annotations
@@ -137,3 +141,66 @@ def jv(efc_J, search, jv_out, *, nefc=None, skip_world: Any = None) -> None:
             int(torch.cuda.current_stream(efc_J.device).cuda_stream),
         )  # fmt: skip
     _lib.check(status, "im_newton_jv")
+
+
+def _per_world(t, nworld, dtypes, name):
+    if t.dtype not in dtypes or not t.is_cuda or not t.is_contiguous() or t.numel() != nworld:
+        raise TypeError(f"{name} must be a contiguous CUDA tensor with one element per world")
+
+
+def _rows(t, nworld, width, dtype, name):
+    if t.dtype != dtype or not t.is_cuda or t.dim() != 2 or t.shape != (nworld, width) or (width > 1 and t.stride(1) != 1):
+        raise TypeError(f"{name} must be a ({nworld}, {width}) CUDA tensor with contiguous rows")
+
+
+def advance(alpha, search, mv, jv_in, qacc, efc_Ma, Jaref, *, nefc=None, done=None) -> None:
+    """In place: ``qacc += alpha search``, ``efc_Ma += alpha mv``, ``Jaref += alpha jv`` (rows
+    below ``nefc``) for the worlds that are not done."""
+    import torch
+
+    nworld, nv = search.shape
+    njmax = jv_in.shape[1]
+    _per_world(alpha, nworld, (torch.float32,), "alpha")
+    for t, width, name in ((search, nv, "search"), (mv, nv, "mv"), (qacc, nv, "qacc"), (efc_Ma, nv, "efc_Ma"),
+                           (jv_in, njmax, "jv"), (Jaref, njmax, "Jaref")):  # fmt: skip
+        _rows(t, nworld, width, torch.float32, name)
+    if nefc is not None:
+        _per_world(nefc, nworld, (torch.int32,), "nefc")
+    if done is not None:
+        _per_world(done, nworld, (torch.bool, torch.uint8), "done")
+    with torch.cuda.device(search.device):
+        status = _lib.lib().im_newton_advance(
+            alpha.data_ptr(), search.data_ptr(), search.stride(0), mv.data_ptr(), mv.stride(0), jv_in.data_ptr(),
+            jv_in.stride(0), None if nefc is None else nefc.data_ptr(), None if done is None else done.data_ptr(),
+            qacc.data_ptr(), qacc.stride(0), efc_Ma.data_ptr(), efc_Ma.stride(0), Jaref.data_ptr(), Jaref.stride(0),
+            int(nv), int(njmax), int(nworld), int(torch.cuda.current_stream(search.device).cuda_stream),
+        )  # fmt: skip
+    _lib.check(status, "im_newton_advance")
+
+
+def changed_rows(old_state, new_state, quad_changed_ids, quad_changed_count, state_changed_count, *, nefc=None,
+                 done=None, quad: int = 1) -> None:  # fmt: skip
+    """Rows whose being quadratic flipped, ascending, into ``quad_changed_ids`` with their count,
+    and the count of rows whose state changed at all."""
+    import torch
+
+    nworld, njmax = old_state.shape
+    for t, name in ((old_state, "old_state"), (new_state, "new_state")):
+        if t.dtype != torch.int32 or not t.is_cuda or not t.is_contiguous() or t.shape != (nworld, njmax):
+            raise TypeError(f"{name} must be a contiguous int32 CUDA tensor (nworld, njmax)")
+    if quad_changed_ids.dtype != torch.int32 or not quad_changed_ids.is_contiguous() or quad_changed_ids.dim() != 2 or quad_changed_ids.shape[0] != nworld:
+        raise TypeError("quad_changed_ids must be a contiguous int32 CUDA tensor (nworld, width)")
+    _per_world(quad_changed_count, nworld, (torch.int32,), "quad_changed_count")
+    _per_world(state_changed_count, nworld, (torch.int32,), "state_changed_count")
+    if nefc is not None:
+        _per_world(nefc, nworld, (torch.int32,), "nefc")
+    if done is not None:
+        _per_world(done, nworld, (torch.bool, torch.uint8), "done")
+    with torch.cuda.device(old_state.device):
+        status = _lib.lib().im_newton_changed_rows(
+            old_state.data_ptr(), new_state.data_ptr(), int(njmax), None if nefc is None else nefc.data_ptr(), int(quad),
+            None if done is None else done.data_ptr(), quad_changed_ids.data_ptr(), int(quad_changed_ids.shape[1]),
+            quad_changed_count.data_ptr(), state_changed_count.data_ptr(), int(nworld),
+            int(torch.cuda.current_stream(old_state.device).cuda_stream),
+        )  # fmt: skip
+    _lib.check(status, "im_newton_changed_rows")

@@ -517,3 +517,38 @@ def newton_jv(J, search, nefc=None, skip=None, out=None):
     lib().orc_newton_jv(nworld, nv, njmax, None if nefc is None else _p(_i(nefc)), _p(J), _p(search),
                         None if sk is None else _p(sk), _p(out))  # fmt: skip
     return out
+
+
+# The step along the search direction and the listing of changed rows
+# (src/instantmimic/utils/mjw_kernels/newton_stages.py:373-381, 403-426), in NumPy.  `advance`
+# is pinned by its closed form in fp64 and, bit for bit, by an exact-product-one-rounding sum;
+# `changed_rows` is integer work, pinned by brute force over the rows.
+def newton_advance(alpha, search, mv, jv, qacc, Ma, jaref, nefc=None, done=None):
+    """Returns the advanced copies (qacc, Ma, jaref)."""
+    a = _f(alpha)[:, None]
+    live = np.ones(len(a), bool) if done is None else np.asarray(done) == 0
+    q64 = (np.float64(a) * _f(search).astype(np.float64) + _f(qacc)).astype(np.float32)  # one rounding: a fused multiply-add
+    m64 = (np.float64(a) * _f(mv).astype(np.float64) + _f(Ma)).astype(np.float32)
+    njmax = jv.shape[1]
+    ne = np.full(len(a), njmax) if nefc is None else np.minimum(np.asarray(nefc), njmax)
+    rows = np.arange(njmax)[None, :] < ne[:, None]
+    j2 = _f(jaref) + (a * _f(jv))  # float32 product, then float32 sum
+    sel = live[:, None]
+    return np.where(sel, q64, qacc), np.where(sel, m64, Ma), np.where(sel & rows, j2, jaref)
+
+
+def newton_changed_rows(old_state, new_state, quad=1, nefc=None, done=None, ids=None, quad_count=None, state_count=None):
+    old_state, new_state = np.asarray(old_state), np.asarray(new_state)
+    nworld, njmax = old_state.shape
+    ids = np.zeros((nworld, njmax), np.int32) if ids is None else ids.copy()
+    qc = np.zeros(nworld, np.int32) if quad_count is None else quad_count.copy()
+    sc = np.zeros(nworld, np.int32) if state_count is None else state_count.copy()
+    for w in range(nworld):
+        if done is not None and done[w]:
+            continue
+        ne = njmax if nefc is None else min(int(nefc[w]), njmax)
+        flips = [r for r in range(ne) if (old_state[w, r] == quad) != (new_state[w, r] == quad)]
+        ids[w, : len(flips)] = flips
+        qc[w] = len(flips)
+        sc[w] = int(np.count_nonzero(old_state[w, :ne] != new_state[w, :ne]))
+    return ids, qc, sc

@@ -389,3 +389,66 @@ def test_gpu_newton_jv_bitwise(device, name, nworld):
     NF.jv(t(b.J), t(search), out)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(out.cpu().numpy(), R.newton_jv(b.J, search))
+
+
+# ---------------------------------------------------------------- step and changed rows
+def _step_case(name, nworld, seed=6):
+    b = synth.make_batch(name, nworld, ragged_nefc=True)
+    rng = np.random.default_rng(seed)
+    njmax, nv = b.J.shape[1], b.J.shape[2]
+    f = lambda *shape: rng.normal(size=shape).astype(np.float32)  # noqa: E731
+    done = (rng.uniform(size=nworld) < 0.2).astype(np.uint8)
+    old = rng.integers(0, 4, (nworld, njmax)).astype(np.int32)
+    new = np.where(rng.uniform(size=old.shape) < 0.3, rng.integers(0, 4, old.shape), old).astype(np.int32)
+    return b, (f(nworld), f(nworld, nv), f(nworld, nv), f(nworld, njmax), f(nworld, nv), f(nworld, nv), f(nworld, njmax)), done, old, new
+
+
+def test_oracle_step_and_changed_rows():
+    from test_newton_stages import _changes
+
+    b, (alpha, search, mv, jv, qacc, Ma, jaref), done, old, new = _step_case("humanoid", 30)
+    q, m, j = R.newton_advance(alpha, search, mv, jv, qacc, Ma, jaref, nefc=b.nefc, done=done)
+    live = done == 0
+    want = qacc.astype(np.float64) + alpha[:, None].astype(np.float64) * search
+    assert np.abs(q[live] - want[live]).max() < 1e-6 * np.abs(want).max()
+    np.testing.assert_array_equal(q[~live], qacc[~live])
+    rows = np.arange(jv.shape[1])[None, :] < b.nefc[:, None]
+    np.testing.assert_array_equal(j[~(rows & live[:, None])], jaref[~(rows & live[:, None])])
+    assert np.abs(j - (jaref + alpha[:, None].astype(np.float64) * jv))[rows & live[:, None]].max() < 1e-6 * np.abs(jaref).max()
+    # the listing against the row lists the factor-stage tests build on their own
+    import dataclasses
+
+    b3 = synth.make_batch(dataclasses.replace(synth.SHAPES["g1"], iterations=2), 40, ragged_nefc=True)
+    new_s, ids, changes, _, _, _ = _changes(b3, np.random.default_rng(1))
+    got_ids, qc, sc = R.newton_changed_rows(b3.state[0], new_s, quad=synth.QUADRATIC, nefc=b3.nefc)
+    np.testing.assert_array_equal(qc, changes)
+    for w in range(40):
+        np.testing.assert_array_equal(got_ids[w, : qc[w]], ids[w, : changes[w]])
+    assert (sc >= qc).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,nworld", [("ant", 64), ("humanoid", 4096), ("snu", 130), ("stress", 37)])
+def test_gpu_step_and_changed_rows_bitwise(device, name, nworld):
+    import torch
+
+    b, arrays, done, old, new = _step_case(name, nworld)
+    alpha, search, mv, jv, qacc, Ma, jaref = arrays
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    qd, md, jd = t(qacc), t(Ma), t(jaref)
+    NF.advance(t(alpha), t(search), t(mv), t(jv), qd, md, jd, nefc=t(b.nefc), done=t(done))
+    torch.cuda.synchronize()
+    q, m, j = R.newton_advance(alpha, search, mv, jv, qacc, Ma, jaref, nefc=b.nefc, done=done)
+    np.testing.assert_array_equal(qd.cpu().numpy(), q)
+    np.testing.assert_array_equal(md.cpu().numpy(), m)
+    np.testing.assert_array_equal(jd.cpu().numpy(), j)
+    njmax = old.shape[1]
+    ids = torch.full((nworld, njmax), -5, dtype=torch.int32, device=device)
+    qc = torch.full((nworld,), -5, dtype=torch.int32, device=device)
+    sc = torch.full((nworld,), -5, dtype=torch.int32, device=device)
+    NF.changed_rows(t(old), t(new), ids, qc, sc, nefc=t(b.nefc), done=t(done), quad=synth.QUADRATIC)
+    torch.cuda.synchronize()
+    want = R.newton_changed_rows(old, new, quad=synth.QUADRATIC, nefc=b.nefc, done=done, ids=np.full((nworld, njmax), -5, np.int32),
+                                 quad_count=np.full(nworld, -5, np.int32), state_count=np.full(nworld, -5, np.int32))  # fmt: skip
+    for got, ref in zip((ids, qc, sc), want):
+        np.testing.assert_array_equal(got.cpu().numpy(), ref)
