@@ -283,3 +283,40 @@ def test_gpu_block_per_world_sparse_kernels_agree():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
     assert out.returncode == 0 and "block-per-world kernels ok" in out.stdout, out.stderr[-2000:]
+
+
+@pytest.mark.gpu
+def test_gpu_changed_rows_feed_the_factor_stage(device):
+    """The row lists and counts of im_newton_changed_rows, taken as they are by the sparse factor
+    stage, against the oracle run on the lists that _changes() builds on its own."""
+    import torch
+
+    from instantmimic_amd.mjw_kernels import newton_fusion as NF
+
+    m, groups, b = _contact_case(150, 23)
+    rng = np.random.default_rng(5)
+    plan = S.build_plan(m, groups, 64, device=device)
+    hf0, *_ = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
+    new, ids, changes, _, done, grad = _changes(b, rng)
+    nworld, nv, njmax = b.nworld, m.nv, b.D.shape[1]
+    ids_d = torch.zeros((nworld, njmax), dtype=torch.int32, device=device)
+    qc = torch.zeros(nworld, dtype=torch.int32, device=device)
+    sc = torch.zeros(nworld, dtype=torch.int32, device=device)
+    NF.changed_rows(_t(b.state[0], device), _t(new, device), ids_d, qc, sc, nefc=_t(b.nefc, device), quad=Q)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(qc.cpu().numpy(), changes)
+    # a world whose states did not change at all is solve-only for the stage and skipped when its count is zero:
+    # give every world at least the solve, as the reference's line search does through its own increments
+    sc_np = np.maximum(sc.cpu().numpy(), 1).astype(np.int32)
+    want = R.sparse_update_factor(plan, sc_np, changes, ids, b.J, b.D, new, grad, hf0, done=done)
+    hf = _t(hf0, device)
+    uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=device)
+    search = torch.zeros((nworld, nv), device=device)
+    sdot, decr = torch.zeros(nworld, device=device), torch.zeros(nworld, device=device)
+    stage = NS.factor_factory(nv, m.nv_pad, plan)
+    stage(_t(b.J, device), _t(b.D, device), _t(new, device), ids_d, qc, _t(sc_np, device), _t(done, device),
+          _t(grad, device), None, hf, search, sdot, decr, uni)  # fmt: skip
+    torch.cuda.synchronize()
+    n_used = 2 * plan.nfac + nv
+    np.testing.assert_array_equal(hf.cpu().numpy().reshape(nworld, -1)[:, :n_used], want[0].reshape(nworld, -1)[:, :n_used])
+    np.testing.assert_array_equal(search.cpu().numpy(), want[2])
