@@ -465,6 +465,21 @@ int im_newton_changed_rows(const int32_t *old_state, const int32_t *new_state, i
                            int32_t *quad_changed_ids, int ld_ids, int32_t *quad_changed_count,
                            int32_t *state_changed_count, int nworld, void *stream);
 
+/* Replaces the convergence test that closes an iteration of the fused Newton kernel
+ * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:265-296), for the worlds that are not
+ * done: niter += 1; scale = stat_meaninertia[w % nmeaninertia] * nv;
+ * converged = alpha == 0 || (improvement > 0 && improvement / scale < tol)
+ *          || sqrt(grad_dot) / scale < tol || 0.5 * newton_decrement / scale < tol
+ * with tol = opt_tolerance[w % ntolerance]; a world that converged or reached maxiter is
+ * marked done and taken off *nsolving (one atomic decrement each; may be null), one that
+ * reached maxiter without converging gets overflow_bit or-ed into overflow[w] (may be null;
+ * upstream's OverflowType.ITERATIONS).  done is bytes. */
+int im_newton_converged(const float *alpha, const float *improvement, const float *grad_dot,
+                        const float *newton_decrement, const float *opt_tolerance, int ntolerance,
+                        const float *stat_meaninertia, int nmeaninertia, int nv, int maxiter,
+                        int overflow_bit, int32_t *niter, int32_t *overflow, uint8_t *done,
+                        int32_t *nsolving, int nworld, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -432,6 +432,28 @@ __global__ __launch_bounds__(kThreads) void newton_changed_rows_kernel(
   }
 }
 
+// ---- convergence test of an iteration ------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void newton_converged_kernel(
+    const float *__restrict__ alpha, const float *__restrict__ improvement, const float *__restrict__ grad_dot,
+    const float *__restrict__ decrement, const float *__restrict__ tolerance, int ntol,
+    const float *__restrict__ meaninertia, int ninertia, int nv, int maxiter, int overflow_bit,
+    int32_t *__restrict__ niter, int32_t *__restrict__ overflow, uint8_t *__restrict__ done,
+    int32_t *__restrict__ nsolving, int nworld) {
+  const int w = blockIdx.x * kThreads + threadIdx.x;
+  if (w >= nworld || done[w]) return;
+  const int it = niter[w] + 1;
+  niter[w] = it;
+  const float tol = tolerance[w % ntol], scale = meaninertia[w % ninertia] * (float)nv;
+  const float imp = improvement[w];
+  const bool converged = alpha[w] == 0.0f || (imp > 0.0f && imp / scale < tol) ||
+                         sqrtf(grad_dot[w]) / scale < tol || 0.5f * decrement[w] / scale < tol;
+  if (converged || it == maxiter) {
+    if (!converged && overflow) overflow[w] = overflow[w] | overflow_bit;
+    done[w] = 1;
+    if (nsolving) atomicAdd(nsolving, -1);
+  }
+}
+
 // Lanes per world: the smallest power of two in 8..64 that covers `work` items (64 beyond).
 int lanes_for(int work) {
   int lanes = 8;
@@ -604,6 +626,24 @@ extern "C" int im_newton_changed_rows(const int32_t *old_state, const int32_t *n
   hipLaunchKernelGGL(newton_changed_rows_kernel, dim3((unsigned)((nworld + per_block - 1) / per_block)),
                      dim3(kThreads), 0, (hipStream_t)stream, old_state, new_state, njmax, nefc, quad, done,
                      quad_changed_ids, ld_ids, quad_changed_count, state_changed_count, nworld);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_newton_converged(const float *alpha, const float *improvement, const float *grad_dot,
+                                   const float *newton_decrement, const float *opt_tolerance, int ntolerance,
+                                   const float *stat_meaninertia, int nmeaninertia, int nv, int maxiter,
+                                   int overflow_bit, int32_t *niter, int32_t *overflow, uint8_t *done,
+                                   int32_t *nsolving, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || ntolerance <= 0 || nmeaninertia <= 0) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!alpha || !improvement || !grad_dot || !newton_decrement || !opt_tolerance || !stat_meaninertia || !niter ||
+      !done)
+    return IM_ERR_ARG;
+  hipLaunchKernelGGL(newton_converged_kernel, dim3((unsigned)((nworld + kThreads - 1) / kThreads)), dim3(kThreads), 0,
+                     (hipStream_t)stream, alpha, improvement, grad_dot, newton_decrement, opt_tolerance, ntolerance,
+                     stat_meaninertia, nmeaninertia, nv, maxiter, overflow_bit, niter, overflow, done, nsolving,
+                     nworld);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

@@ -12,8 +12,8 @@ ascending -- the upstream order is not visible from the reference's tree).
 (src/instantmimic/utils/mjw_kernels/newton_stages.py:745-798) and :func:`jv` the ``J v`` step at
 the head of its line search (:157-178); :func:`advance` is the step along the search direction
 at its end (:373-381) and :func:`changed_rows` the listing of the rows whose state changed
-(:403-426), which is what the factor stage of the next iteration takes.  Each runs for all
-worlds in one launch.  The scalar search itself, the evaluation of the constraints' new states
+(:403-426), which is what the factor stage of the next iteration takes; :func:`converged` is the
+test that closes an iteration (newton_fusion.py:265-296).  Each runs for all worlds in one launch.  The scalar search itself, the evaluation of the constraints' new states
 and forces and the convergence test are upstream mujoco_warp code and are not part of this
 module.
 """
@@ -204,3 +204,33 @@ def changed_rows(old_state, new_state, quad_changed_ids, quad_changed_count, sta
             int(torch.cuda.current_stream(old_state.device).cuda_stream),
         )  # fmt: skip
     _lib.check(status, "im_newton_changed_rows")
+
+
+def converged(alpha, improvement, grad_dot, newton_decrement, opt_tolerance, stat_meaninertia, nv: int, maxiter: int,
+              niter, done, *, overflow=None, overflow_bit: int = 0, nsolving=None) -> None:  # fmt: skip
+    """Counts the iteration and marks the worlds that converged (or ran out of iterations) done,
+    with the reference's four criteria; ``nsolving`` (one int32) is decremented once per such
+    world."""
+    import torch
+
+    nworld = alpha.numel()
+    for t, name in ((alpha, "alpha"), (improvement, "improvement"), (grad_dot, "grad_dot"), (newton_decrement, "newton_decrement")):
+        _per_world(t, nworld, (torch.float32,), name)
+    for t in (opt_tolerance, stat_meaninertia):
+        if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous() or t.numel() == 0:
+            raise TypeError("opt_tolerance and stat_meaninertia must be non-empty contiguous float32 CUDA tensors")
+    _per_world(niter, nworld, (torch.int32,), "niter")
+    _per_world(done, nworld, (torch.bool, torch.uint8), "done")
+    if overflow is not None:
+        _per_world(overflow, nworld, (torch.int32,), "overflow")
+    if nsolving is not None and (nsolving.dtype != torch.int32 or not nsolving.is_cuda or nsolving.numel() != 1):
+        raise TypeError("nsolving must be a one-element int32 CUDA tensor")
+    with torch.cuda.device(alpha.device):
+        status = _lib.lib().im_newton_converged(
+            alpha.data_ptr(), improvement.data_ptr(), grad_dot.data_ptr(), newton_decrement.data_ptr(),
+            opt_tolerance.data_ptr(), int(opt_tolerance.numel()), stat_meaninertia.data_ptr(), int(stat_meaninertia.numel()),
+            int(nv), int(maxiter), int(overflow_bit), niter.data_ptr(), None if overflow is None else overflow.data_ptr(),
+            done.data_ptr(), None if nsolving is None else nsolving.data_ptr(), int(nworld),
+            int(torch.cuda.current_stream(alpha.device).cuda_stream),
+        )  # fmt: skip
+    _lib.check(status, "im_newton_converged")

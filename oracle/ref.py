@@ -552,3 +552,24 @@ def newton_changed_rows(old_state, new_state, quad=1, nefc=None, done=None, ids=
         qc[w] = len(flips)
         sc[w] = int(np.count_nonzero(old_state[w, :ne] != new_state[w, :ne]))
     return ids, qc, sc
+
+
+# The convergence test of an iteration (src/instantmimic/utils/mjw_kernels/newton_fusion.py:265-296)
+# in NumPy float32; pinned by worlds built to meet exactly one criterion each.
+def newton_converged(alpha, improvement, grad_dot, decrement, tolerance, meaninertia, nv, maxiter, niter, done, overflow_bit=0):
+    """Returns (niter, done, overflow, newly_done_count)."""
+    nworld = len(alpha)
+    niter, done = np.asarray(niter, np.int32).copy(), np.asarray(done, np.uint8).copy()
+    overflow = np.zeros(nworld, np.int32)
+    w = np.arange(nworld)
+    tol = _f(tolerance)[w % len(tolerance)]
+    scale = _f(meaninertia)[w % len(meaninertia)] * np.float32(nv)
+    a, imp, gd, de = (_f(x) for x in (alpha, improvement, grad_dot, decrement))
+    with np.errstate(invalid="ignore", divide="ignore"):
+        conv = (a == 0) | ((imp > 0) & (imp / scale < tol)) | (np.sqrt(gd) / scale < tol) | (np.float32(0.5) * de / scale < tol)
+    live = done == 0
+    niter[live] += 1
+    stop = live & (conv | (niter == maxiter))
+    overflow[stop & ~conv] = overflow_bit
+    done[stop] = 1
+    return niter, done, overflow, int(stop.sum())

@@ -452,3 +452,58 @@ def test_gpu_step_and_changed_rows_bitwise(device, name, nworld):
                                  quad_count=np.full(nworld, -5, np.int32), state_count=np.full(nworld, -5, np.int32))  # fmt: skip
     for got, ref in zip((ids, qc, sc), want):
         np.testing.assert_array_equal(got.cpu().numpy(), ref)
+
+
+# ---------------------------------------------------------------- convergence test
+def _convergence_case(nworld, seed=8):
+    rng = np.random.default_rng(seed)
+    alpha = rng.uniform(0.1, 1, nworld).astype(np.float32)
+    imp = rng.uniform(1, 2, nworld).astype(np.float32)
+    gd = rng.uniform(1, 4, nworld).astype(np.float32)
+    de = rng.uniform(1, 4, nworld).astype(np.float32)
+    niter = rng.integers(0, 3, nworld).astype(np.int32)
+    done = (rng.uniform(size=nworld) < 0.1).astype(np.uint8)
+    # one criterion each for a few worlds; the others fail all four
+    kind = rng.integers(0, 6, nworld)
+    alpha[kind == 1] = 0.0
+    imp[kind == 2] = 1e-9
+    gd[kind == 3] = 1e-16
+    de[kind == 4] = 1e-9
+    imp[kind == 5] = -1.0  # a negative improvement never counts
+    return alpha, imp, gd, de, niter, done, kind
+
+
+def test_oracle_convergence_criteria():
+    nworld, nv, maxiter = 400, 27, 3
+    alpha, imp, gd, de, niter, done, kind = _convergence_case(nworld)
+    tol, inertia = np.array([1e-6, 2e-6], np.float32), np.array([0.5], np.float32)
+    it, dn, ov, count = R.newton_converged(alpha, imp, gd, de, tol, inertia, nv, maxiter, niter, done, overflow_bit=4)
+    live = done == 0
+    np.testing.assert_array_equal(it[live], niter[live] + 1)
+    np.testing.assert_array_equal(it[~live], niter[~live])
+    met = np.isin(kind, (1, 2, 3, 4))
+    out_of_iterations = (niter + 1 == maxiter) & ~met
+    np.testing.assert_array_equal(dn[live], (met | out_of_iterations)[live].astype(np.uint8))
+    assert (dn[~live] == 1).all()
+    np.testing.assert_array_equal(ov[live], np.where(out_of_iterations, 4, 0)[live])
+    assert count == int((live & (met | out_of_iterations)).sum())
+
+
+@pytest.mark.gpu
+def test_gpu_convergence_bitwise(device):
+    import torch
+
+    nworld, nv, maxiter = 5000, 27, 3
+    alpha, imp, gd, de, niter, done, _ = _convergence_case(nworld)
+    tol, inertia = np.array([1e-6, 2e-6], np.float32), np.array([0.5, 0.7, 0.9], np.float32)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    it, dn = t(niter), t(done)
+    ov = torch.zeros(nworld, dtype=torch.int32, device=device)
+    ns = torch.full((1,), int((done == 0).sum()), dtype=torch.int32, device=device)
+    NF.converged(t(alpha), t(imp), t(gd), t(de), t(tol), t(inertia), nv, maxiter, it, dn, overflow=ov, overflow_bit=4, nsolving=ns)
+    torch.cuda.synchronize()
+    want = R.newton_converged(alpha, imp, gd, de, tol, inertia, nv, maxiter, niter, done, overflow_bit=4)
+    np.testing.assert_array_equal(it.cpu().numpy(), want[0])
+    np.testing.assert_array_equal(dn.cpu().numpy(), want[1])
+    np.testing.assert_array_equal(ov.cpu().numpy(), want[2])
+    assert int(ns.item()) == int((done == 0).sum()) - want[3]
