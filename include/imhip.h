@@ -480,6 +480,22 @@ int im_newton_converged(const float *alpha, const float *improvement, const floa
                         int overflow_bit, int32_t *niter, int32_t *overflow, uint8_t *done,
                         int32_t *nsolving, int nworld, void *stream);
 
+/* Replaces _init_efc_settling_empty_worlds
+ * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:412-428): solver_niter = 0,
+ * search_dot = 0, done = (nefc == 0), and a world without constraint rows gets
+ * qacc = qacc_smooth (MuJoCo's result for nefc == 0), so it starts done. */
+int im_newton_init_empty_worlds(const int32_t *nefc, const float *qacc_smooth, int64_t ld_smooth,
+                                int32_t *solver_niter, float *search_dot, uint8_t *done,
+                                float *qacc, int64_t ld_qacc, int nv, int nworld, void *stream);
+
+/* Replaces qfrc_constraint_from_grad (newton_fusion.py:537-555):
+ * qfrc_constraint = efc_Ma - qfrc_smooth - grad_scale[w] * grad, zero for a world without
+ * constraint rows. */
+int im_qfrc_constraint_from_grad(const int32_t *nefc, const float *qfrc_smooth, int64_t ld_smooth,
+                                 const float *efc_Ma, int64_t ld_Ma, const float *grad,
+                                 int64_t ld_grad, const float *grad_scale, float *qfrc_constraint,
+                                 int64_t ld_constraint, int nv, int nworld, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -151,6 +151,8 @@ SIGNATURES = {
     ),
     "im_newton_changed_rows": (_i, [_vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _vp, _i, _vp]),
     "im_newton_converged": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
+    "im_newton_init_empty_worlds": (_i, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
+    "im_qfrc_constraint_from_grad": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64, _i, _i, _vp]),
     "im_project_body_wrenches": (
         _i,
         [C.POINTER(BodyWrenches), C.POINTER(WrenchTopology), _i, _i, _i, _vp, _i64, _i, _vp],

@@ -256,6 +256,37 @@ __global__ __launch_bounds__(kThreads) void newton_converged_kernel(
   }
 }
 
+// ---- start and finish of the fused solve ----------------------------------------------------------
+// One thread per (world, dof), a world per blockIdx.y.
+__global__ __launch_bounds__(kThreads) void newton_init_empty_kernel(
+    const int32_t *__restrict__ nefc, const float *__restrict__ qacc_smooth, int64_t lds_, int32_t *__restrict__ niter,
+    float *__restrict__ search_dot, uint8_t *__restrict__ done, float *__restrict__ qacc, int64_t ldq, int nv) {
+  const int64_t w = blockIdx.y;
+  const int dof = blockIdx.x * kThreads + threadIdx.x;
+  const bool empty = nefc[w] == 0;
+  if (dof == 0) {
+    niter[w] = 0;
+    search_dot[w] = 0.0f;
+    done[w] = empty ? 1 : 0;
+  }
+  if (empty && dof < nv) qacc[w * ldq + dof] = qacc_smooth[w * lds_ + dof];
+}
+
+__global__ __launch_bounds__(kThreads) void qfrc_from_grad_kernel(
+    const int32_t *__restrict__ nefc, const float *__restrict__ smooth, int64_t lds_, const float *__restrict__ Ma,
+    int64_t ldm, const float *__restrict__ grad, int64_t ldg, const float *__restrict__ scale,
+    float *__restrict__ out, int64_t ldo, int nv) {
+  const int64_t w = blockIdx.y;
+  const int dof = blockIdx.x * kThreads + threadIdx.x;
+  if (dof >= nv) return;
+  float v = 0.0f;
+  if (nefc[w] != 0) {
+    const float g = scale[w] * grad[w * ldg + dof];
+    v = Ma[w * ldm + dof] - smooth[w * lds_ + dof] - g;
+  }
+  out[w * ldo + dof] = v;
+}
+
 }  // namespace
 }  // namespace im
 
@@ -360,6 +391,42 @@ extern "C" int im_newton_converged(const float *alpha, const float *improvement,
                      (hipStream_t)stream, alpha, improvement, grad_dot, newton_decrement, opt_tolerance, ntolerance,
                      stat_meaninertia, nmeaninertia, nv, maxiter, overflow_bit, niter, overflow, done, nsolving,
                      nworld);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_newton_init_empty_worlds(const int32_t *nefc, const float *qacc_smooth, int64_t ld_smooth,
+                                           int32_t *solver_niter, float *search_dot, uint8_t *done, float *qacc,
+                                           int64_t ld_qacc, int nv, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!nefc || !qacc_smooth || !solver_niter || !search_dot || !done || !qacc) return IM_ERR_ARG;
+  if (ld_smooth < nv || ld_qacc < nv) return IM_ERR_STRIDE;
+  for (int w0 = 0; w0 < nworld; w0 += 65535) {
+    const int nw = nworld - w0 < 65535 ? nworld - w0 : 65535;
+    hipLaunchKernelGGL(newton_init_empty_kernel, dim3((unsigned)((nv + kThreads - 1) / kThreads), (unsigned)nw),
+                       dim3(kThreads), 0, (hipStream_t)stream, nefc + w0, qacc_smooth + w0 * ld_smooth, ld_smooth,
+                       solver_niter + w0, search_dot + w0, done + w0, qacc + w0 * ld_qacc, ld_qacc, nv);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_qfrc_constraint_from_grad(const int32_t *nefc, const float *qfrc_smooth, int64_t ld_smooth,
+                                            const float *efc_Ma, int64_t ld_Ma, const float *grad, int64_t ld_grad,
+                                            const float *grad_scale, float *qfrc_constraint, int64_t ld_constraint,
+                                            int nv, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!nefc || !qfrc_smooth || !efc_Ma || !grad || !grad_scale || !qfrc_constraint) return IM_ERR_ARG;
+  if (ld_smooth < nv || ld_Ma < nv || ld_grad < nv || ld_constraint < nv) return IM_ERR_STRIDE;
+  for (int w0 = 0; w0 < nworld; w0 += 65535) {
+    const int nw = nworld - w0 < 65535 ? nworld - w0 : 65535;
+    hipLaunchKernelGGL(qfrc_from_grad_kernel, dim3((unsigned)((nv + kThreads - 1) / kThreads), (unsigned)nw),
+                       dim3(kThreads), 0, (hipStream_t)stream, nefc + w0, qfrc_smooth + w0 * ld_smooth, ld_smooth,
+                       efc_Ma + w0 * ld_Ma, ld_Ma, grad + w0 * ld_grad, ld_grad, grad_scale + w0,
+                       qfrc_constraint + w0 * ld_constraint, ld_constraint, nv);
+  }
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

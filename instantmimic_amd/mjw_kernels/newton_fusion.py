@@ -13,7 +13,9 @@ ascending -- the upstream order is not visible from the reference's tree).
 the head of its line search (:157-178); :func:`advance` is the step along the search direction
 at its end (:373-381) and :func:`changed_rows` the listing of the rows whose state changed
 (:403-426), which is what the factor stage of the next iteration takes; :func:`converged` is the
-test that closes an iteration (newton_fusion.py:265-296).  Each runs for all worlds in one launch.  The scalar search itself, the evaluation of the constraints' new states
+test that closes an iteration (newton_fusion.py:265-296); :func:`init_empty_worlds` and
+:func:`qfrc_constraint_from_grad` are the two small kernels at the start and the end of the fused
+solve (:412-428, :537-555).  Each runs for all worlds in one launch.  The scalar search itself, the evaluation of the constraints' new states
 and forces and the convergence test are upstream mujoco_warp code and are not part of this
 module.
 """
@@ -234,3 +236,42 @@ def converged(alpha, improvement, grad_dot, newton_decrement, opt_tolerance, sta
             int(torch.cuda.current_stream(alpha.device).cuda_stream),
         )  # fmt: skip
     _lib.check(status, "im_newton_converged")
+
+
+def init_empty_worlds(nefc, qacc_smooth, solver_niter, search_dot, done, qacc) -> None:
+    """``solver_niter = 0``, ``search_dot = 0``, ``done = nefc == 0`` and ``qacc = qacc_smooth``
+    for the worlds without constraint rows."""
+    import torch
+
+    nworld, nv = qacc.shape
+    _per_world(nefc, nworld, (torch.int32,), "nefc")
+    _per_world(solver_niter, nworld, (torch.int32,), "solver_niter")
+    _per_world(search_dot, nworld, (torch.float32,), "search_dot")
+    _per_world(done, nworld, (torch.bool, torch.uint8), "done")
+    _rows(qacc_smooth, nworld, nv, torch.float32, "qacc_smooth")
+    _rows(qacc, nworld, nv, torch.float32, "qacc")
+    with torch.cuda.device(qacc.device):
+        status = _lib.lib().im_newton_init_empty_worlds(
+            nefc.data_ptr(), qacc_smooth.data_ptr(), qacc_smooth.stride(0), solver_niter.data_ptr(), search_dot.data_ptr(),
+            done.data_ptr(), qacc.data_ptr(), qacc.stride(0), int(nv), int(nworld),
+            int(torch.cuda.current_stream(qacc.device).cuda_stream),
+        )  # fmt: skip
+    _lib.check(status, "im_newton_init_empty_worlds")
+
+
+def qfrc_constraint_from_grad(nefc, qfrc_smooth, efc_Ma, grad, grad_scale, qfrc_constraint) -> None:
+    """``qfrc_constraint = efc_Ma - qfrc_smooth - grad_scale grad``; zero where ``nefc == 0``."""
+    import torch
+
+    nworld, nv = grad.shape
+    _per_world(nefc, nworld, (torch.int32,), "nefc")
+    _per_world(grad_scale, nworld, (torch.float32,), "grad_scale")
+    for t, name in ((qfrc_smooth, "qfrc_smooth"), (efc_Ma, "efc_Ma"), (grad, "grad"), (qfrc_constraint, "qfrc_constraint")):
+        _rows(t, nworld, nv, torch.float32, name)
+    with torch.cuda.device(grad.device):
+        status = _lib.lib().im_qfrc_constraint_from_grad(
+            nefc.data_ptr(), qfrc_smooth.data_ptr(), qfrc_smooth.stride(0), efc_Ma.data_ptr(), efc_Ma.stride(0),
+            grad.data_ptr(), grad.stride(0), grad_scale.data_ptr(), qfrc_constraint.data_ptr(), qfrc_constraint.stride(0),
+            int(nv), int(nworld), int(torch.cuda.current_stream(grad.device).cuda_stream),
+        )  # fmt: skip
+    _lib.check(status, "im_qfrc_constraint_from_grad")

@@ -507,3 +507,29 @@ def test_gpu_convergence_bitwise(device):
     np.testing.assert_array_equal(dn.cpu().numpy(), want[1])
     np.testing.assert_array_equal(ov.cpu().numpy(), want[2])
     assert int(ns.item()) == int((done == 0).sum()) - want[3]
+
+
+@pytest.mark.gpu
+def test_gpu_start_and_finish_of_the_fused_solve(device):
+    """_init_efc_settling_empty_worlds and qfrc_constraint_from_grad (newton_fusion.py:412-428,
+    537-555) against their statements in NumPy float32, bit for bit."""
+    import torch
+
+    nworld, nv = 777, 35
+    rng = np.random.default_rng(12)
+    nefc = rng.integers(0, 3, nworld).astype(np.int32)  # a third of the worlds have no rows
+    f = lambda *shape: rng.normal(size=shape).astype(np.float32)  # noqa: E731
+    smooth, Ma, grad, scale, qacc0 = f(nworld, nv), f(nworld, nv), f(nworld, nv), f(nworld), f(nworld, nv)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    niter = torch.full((nworld,), 9, dtype=torch.int32, device=device)
+    sdot, done, qacc = torch.full((nworld,), 9.0, device=device), torch.full((nworld,), 9, dtype=torch.uint8, device=device), t(qacc0)
+    NF.init_empty_worlds(t(nefc), t(smooth), niter, sdot, done, qacc)
+    out = torch.full((nworld, nv), 9.0, device=device)
+    NF.qfrc_constraint_from_grad(t(nefc), t(smooth), t(Ma), t(grad), t(scale), out)
+    torch.cuda.synchronize()
+    empty = nefc == 0
+    assert not niter.any() and not sdot.any()
+    np.testing.assert_array_equal(done.cpu().numpy(), empty.astype(np.uint8))
+    np.testing.assert_array_equal(qacc.cpu().numpy(), np.where(empty[:, None], smooth, qacc0))
+    want = np.where(empty[:, None], np.float32(0), (Ma - smooth) - scale[:, None] * grad)
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
