@@ -320,3 +320,66 @@ def test_gpu_changed_rows_feed_the_factor_stage(device):
     n_used = 2 * plan.nfac + nv
     np.testing.assert_array_equal(hf.cpu().numpy().reshape(nworld, -1)[:, :n_used], want[0].reshape(nworld, -1)[:, :n_used])
     np.testing.assert_array_equal(search.cpu().numpy(), want[2])
+
+
+@pytest.mark.gpu
+def test_gpu_one_iteration_chained(device):
+    """One Newton iteration with the library's pieces in the reference's order (J v, step, changed
+    rows, gradient, factor stage, convergence test) against the oracle's pieces in the same order.
+    The step length, the new states and the new forces come from outside, as they come from
+    upstream code in the reference."""
+    import torch
+
+    from instantmimic_amd.mjw_kernels import newton_fusion as NF
+
+    m, groups, b = _contact_case(150, 23)
+    rng = np.random.default_rng(15)
+    plan = S.build_plan(m, groups, 64, device=device)
+    nworld, nv, njmax = b.nworld, m.nv, b.D.shape[1]
+    hf0, search0, sdot0, decr0 = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
+    new, _, _, _, done, _ = _changes(b, rng)
+    f = lambda *shape: rng.normal(size=shape).astype(np.float32)  # noqa: E731
+    alpha = rng.uniform(0.1, 1, nworld).astype(np.float32)
+    mv, qacc, Ma, jaref, smooth, force = f(nworld, nv), f(nworld, nv), f(nworld, nv), f(nworld, njmax), f(nworld, nv), f(nworld, njmax)
+    gd0, sc0 = rng.uniform(1, 2, nworld).astype(np.float32), np.ones(nworld, np.float32)
+    imp = rng.uniform(0, 1e-3, nworld).astype(np.float32)
+    tol, inertia = np.array([1e-6], np.float32), np.array([1.0], np.float32)
+    # oracle chain
+    jv = R.newton_jv(b.J, search0, nefc=b.nefc, skip=done)
+    q1, Ma1, ja1 = R.newton_advance(alpha, search0, mv, jv, qacc, Ma, jaref, nefc=b.nefc, done=done)
+    ids, qc, sc = R.newton_changed_rows(b.state[0], new, quad=Q, nefc=b.nefc, done=done)
+    qcf, grad, gd, de, gs, un = R.newton_gradient(b.J, force, smooth, Ma1, sc, alpha, gd0, decr0, sc0, nefc=b.nefc, done=done, block=64)
+    want = R.sparse_update_factor(plan, sc, qc, ids, b.J, b.D, new, grad, hf0, done=done)
+    ran = (done == 0) & (sc != 0)  # the factor stage leaves the other worlds' decrement as the gradient step left it
+    it, dn, _, _ = R.newton_converged(alpha, imp, gd, np.where(ran, want[4], de), tol, inertia, nv, 5, np.zeros(nworld, np.int32), done)
+    # the same on the GPU
+    t = lambda a: _t(a, device)  # noqa: E731
+    J, D, nefc, dn_d, al = t(b.J), t(b.D), t(b.nefc), t(done), t(alpha)
+    search = t(search0)
+    jv_d = torch.zeros((nworld, njmax), device=device)
+    NF.jv(J, search, jv_d, nefc=nefc, skip_world=dn_d)
+    q_d, Ma_d, ja_d = t(qacc), t(Ma), t(jaref)
+    NF.advance(al, search, t(mv), jv_d, q_d, Ma_d, ja_d, nefc=nefc, done=dn_d)
+    ids_d = torch.zeros((nworld, njmax), dtype=torch.int32, device=device)
+    qc_d, sc_d = torch.zeros(nworld, dtype=torch.int32, device=device), torch.zeros(nworld, dtype=torch.int32, device=device)
+    new_d = t(new)
+    NF.changed_rows(t(b.state[0]), new_d, ids_d, qc_d, sc_d, nefc=nefc, done=dn_d, quad=Q)
+    qcf_d, grad_d = torch.zeros((nworld, nv), device=device), torch.zeros((nworld, nv), device=device)
+    gd_d, de_d, gs_d = t(gd0), t(decr0), t(sc0)
+    un_d = torch.zeros(nworld, dtype=torch.uint8, device=device)
+    NF.gradient(nefc, J, t(force), t(smooth), Ma_d, sc_d, al, dn_d, qcf_d, grad_d, gd_d, de_d, gs_d, un_d, block=64)
+    hf = t(hf0)
+    uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=device)
+    sdot_d = t(sdot0)
+    NS.factor_factory(nv, m.nv_pad, plan)(J, D, new_d, ids_d, qc_d, sc_d, dn_d, grad_d, None, hf, search, sdot_d, de_d, uni)
+    it_d = torch.zeros(nworld, dtype=torch.int32, device=device)
+    NF.converged(al, t(imp), gd_d, de_d, t(tol), t(inertia), nv, 5, it_d, dn_d)
+    torch.cuda.synchronize()
+    live = (done == 0) & (sc != 0)
+    np.testing.assert_array_equal(q_d.cpu().numpy(), q1)
+    np.testing.assert_array_equal(ja_d.cpu().numpy(), ja1)
+    np.testing.assert_array_equal(grad_d.cpu().numpy()[live], grad[live])
+    np.testing.assert_array_equal(search.cpu().numpy()[live], want[2][live])
+    np.testing.assert_array_equal(de_d.cpu().numpy()[live], want[4][live])
+    np.testing.assert_array_equal(it_d.cpu().numpy(), it)
+    np.testing.assert_array_equal(dn_d.cpu().numpy(), dn)
