@@ -151,3 +151,28 @@ def test_tree_walk_entry_points_check_their_arguments_before_any_launch():
     assert lib.im_project_body_wrenches(C.byref(w), C.byref(t), 6, 50, 2, one, 51, 4, None) == _lib.IM_ERR_STRIDE
     t.body_count = 3000
     assert lib.im_project_body_wrenches(C.byref(w), C.byref(t), 6, 50, 0, one, 50, 4, None) == _lib.IM_ERR_UNSUPPORTED
+
+
+def test_newton_entry_points_check_their_arguments_before_any_launch():
+    lib = _lib.lib()
+    one = 16  # any non-null address: nothing is dereferenced on these paths
+    g = lambda **k: lib.im_newton_gradient(  # noqa: E731
+        k.get("nefc"), k.get("J", one), 64, one, k.get("ldf", 64), one, 27, one, 27, one, one, None, one, 27, one,
+        k.get("ldg", 27), one, one, one, one, 27, k.get("block", 64), k.get("nworld", 4), None)  # fmt: skip
+    assert g(nworld=-1) == _lib.IM_ERR_ARG and g(J=None) == _lib.IM_ERR_ARG
+    assert g(block=48) == _lib.IM_ERR_UNSUPPORTED
+    assert g(ldf=63) == _lib.IM_ERR_STRIDE and g(ldg=26) == _lib.IM_ERR_STRIDE
+    assert g(nworld=0) == _lib.IM_OK
+    assert lib.im_newton_jv(one, 64, None, one, 26, None, one, 64, 27, 4, None) == _lib.IM_ERR_STRIDE
+    assert lib.im_newton_jv(one, 64, None, one, 27, None, one, 63, 27, 4, None) == _lib.IM_ERR_STRIDE
+    assert lib.im_newton_jv(None, 64, None, one, 27, None, one, 64, 27, 4, None) == _lib.IM_ERR_ARG
+    assert lib.im_newton_jv(one, 64, None, one, 400, None, one, 64, 400, 4, None) == _lib.IM_ERR_UNSUPPORTED  # 64 rows of 400 dofs exceed LDS
+    assert lib.im_newton_jv(one, 0, None, one, 27, None, one, 0, 27, 4, None) == _lib.IM_OK
+    assert lib.im_newton_advance(one, one, 27, one, 27, one, 64, None, None, one, 26, one, 27, one, 64, 27, 64, 4, None) == _lib.IM_ERR_STRIDE
+    assert lib.im_newton_advance(None, one, 27, one, 27, one, 64, None, None, one, 27, one, 27, one, 64, 27, 64, 4, None) == _lib.IM_ERR_ARG
+    assert lib.im_newton_changed_rows(one, None, 64, None, 1, None, one, 64, one, one, 4, None) == _lib.IM_ERR_ARG
+    assert lib.im_newton_changed_rows(one, one, 64, None, 1, None, one, 64, one, one, 0, None) == _lib.IM_OK
+    assert lib.im_newton_converged(one, one, one, one, one, 0, one, 1, 27, 5, 0, one, None, one, None, 4, None) == _lib.IM_ERR_ARG
+    assert lib.im_newton_converged(one, one, one, one, one, 1, one, 1, 27, 5, 0, one, None, None, None, 4, None) == _lib.IM_ERR_ARG
+    assert lib.im_newton_init_empty_worlds(one, one, 26, one, one, one, one, 27, 27, 4, None) == _lib.IM_ERR_STRIDE
+    assert lib.im_qfrc_constraint_from_grad(one, one, 27, one, 27, one, 27, None, one, 27, 27, 4, None) == _lib.IM_ERR_ARG
