@@ -240,6 +240,35 @@ def run(launches: int = 32) -> None:
         jvo = torch.zeros((nworld, nefc), device=dev)
         sec = _timeit(torch, lambda i: NF.jv(Js[i], sm, jvo, nefc=ne), nsets, launches)
         _line("im_newton_jv", f"{name} nv={nv} nefc={nefc} x {nworld} worlds", sec, bytes_=nworld * 4 * (nefc * nv + nefc + nv), nworld=nworld)
+    # ---- one Newton iteration from the library's pieces, tree path, humanoid
+    b = synth.make_batch("humanoid")
+    nv, nM, nefc, nworld = b.shape.nv, int(b.colind.size), b.shape.nefc, b.nworld
+    sc_tree = T.create_tree_factor_solve_scratch(SimpleNamespace(nv=nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind), dev)
+    nsets = 16
+    S = sets_of((b.M, b.J, b.D, b.state[0], b.state[1], b.nefc), nsets)
+    f32 = lambda *shape: torch.randn(shape, device=dev)  # noqa: E731
+    i32 = lambda: torch.zeros(nworld, dtype=torch.int32, device=dev)  # noqa: E731
+    search, mvv, qacc, Ma, smooth, force = f32(nworld, nv), f32(nworld, nv), f32(nworld, nv), f32(nworld, nv), f32(nworld, nv), f32(nworld, nefc)
+    jvv, jaref, alpha = torch.zeros((nworld, nefc), device=dev), f32(nworld, nefc), torch.rand(nworld, device=dev)
+    ids, qcnt, scnt, nit = torch.zeros((nworld, nefc), dtype=torch.int32, device=dev), i32(), i32(), i32()
+    qc, gr = torch.zeros((nworld, nv), device=dev), torch.zeros((nworld, nv), device=dev)
+    gd, de, gs, imp = (torch.ones(nworld, device=dev) for _ in range(4))
+    un, dn = torch.zeros(nworld, dtype=torch.uint8, device=dev), torch.zeros(nworld, dtype=torch.uint8, device=dev)
+    tol, inertia = torch.full((1,), 1e-30, device=dev), torch.ones(1, device=dev)
+
+    def iteration(i):
+        M_, J_, D_, s0, s1, ne_ = S[i]
+        NF.jv(J_, search, jvv, nefc=ne_, skip_world=dn)
+        NF.advance(alpha, search, mvv, jvv, qacc, Ma, jaref, nefc=ne_, done=dn)
+        NF.changed_rows(s0, s1, ids, qcnt, scnt, nefc=ne_, done=dn)
+        NF.gradient(ne_, J_, force, smooth, Ma, scnt, alpha, dn, qc, gr, gd, de, gs, un)
+        T.assemble_tree_factor_solve(sc_tree, M_, J_, D_, s1, ne_, gr, search, negate=True)
+        NF.converged(alpha, imp, gd, de, tol, inertia, nv, 1 << 30, nit, dn)
+
+    sec = _timeit(torch, iteration, nsets, launches)
+    _line("one Newton iteration: jv, step, changed rows, gradient, fused tree solve, convergence test (six launches)",
+          f"humanoid nv={nv} nefc={nefc} x {nworld} worlds", sec,
+          bytes_=nworld * 4 * (3 * nefc * nv + nM + 8 * nefc + 12 * nv + 10), nworld=nworld)  # fmt: skip
     topo = rig.topology
     nb, nvf = rig.body_count, rig.full_torque_dim
     parent = np.asarray(topo.body_parentid, np.int32)
