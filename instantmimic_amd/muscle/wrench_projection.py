@@ -44,20 +44,29 @@ def body_cap_for(body_count: int):
 
 
 def tree_levels(body_parentid):
-    """Depth-sorted bodies, depth offsets, and a child list (wrench_projection.py:166-184)."""
-    parents = np.asarray(body_parentid, dtype=np.int32)
-    depth = np.zeros(parents.shape[0], dtype=np.int32)
-    for body in range(1, parents.shape[0]):
-        parent = int(parents[body])
-        if parent >= body:
+    """``(level_bodies, level_offsets, child_bodies, child_offsets)`` of a body tree whose
+    parents precede their children: the bodies grouped by depth (ascending id inside a depth)
+    with the depths' start offsets, and every body's children (ascending) behind one another
+    with per-body offsets -- the four arrays of the reference's function of this name
+    (wrench_projection.py:166-184)."""
+    parent = [int(p) for p in np.asarray(body_parentid).reshape(-1)]
+    nbody = len(parent)
+    depth = [0] * nbody
+    children: list[list[int]] = [[] for _ in range(nbody)]
+    for body in range(1, nbody):
+        if parent[body] >= body:
             raise ValueError("body_parentid must reference an earlier body")
-        depth[body] = depth[parent] + 1
-    order = np.argsort(depth, kind="stable").astype(np.int32)
-    counts = np.bincount(depth, minlength=int(depth.max()) + 1 if depth.size else 1)
-    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
-    child_bodies = np.arange(1, parents.shape[0], dtype=np.int32)[np.argsort(parents[1:], kind="stable")]
-    child_offsets = np.concatenate([[0], np.cumsum(np.bincount(parents[1:], minlength=parents.shape[0]))]).astype(np.int32)
-    return order, offsets, child_bodies, child_offsets
+        depth[body] = depth[parent[body]] + 1
+        children[parent[body]].append(body)
+    by_depth: list[list[int]] = [[] for _ in range(max(depth, default=0) + 1)]
+    for body in range(nbody):
+        by_depth[depth[body]].append(body)
+    i32 = lambda values: np.asarray(values, dtype=np.int32)  # noqa: E731
+    level_bodies = i32([body for level in by_depth for body in level])
+    level_offsets = i32(np.cumsum([0] + [len(level) for level in by_depth]))
+    child_bodies = i32([c for kids in children for c in kids])
+    child_offsets = i32(np.cumsum([0] + [len(kids) for kids in children]))
+    return level_bodies, level_offsets, child_bodies, child_offsets
 
 
 def build_wrench_projection_topology(body_parentid, dof_bodyid, body_count: int, device):
