@@ -15,7 +15,8 @@ Fused kernel: one workgroup of four wavefronts per four worlds.
   (their ids packed in row order by a ballot and a prefix count): a row left out would
   have added ``(J * 0) * J`` to every entry.  All loads are unconditional and counted, so
   each step waits for exactly its own operands.
-* Hand-over.  The tiles go to a dense copy of H in LDS; from there each wavefront reads
+* Hand-over.  The tiles go to a copy of H's lower triangle in LDS (a row as long as its
+  tile row reaches); from there each wavefront reads
   the rows it factors in the "row16" layout: a world owns one 16-lane DPP row, row b of H
   (the CSR row of dof b: its ancestors root-first, then b) lives in one VGPR per 16
   positions, lane p of register ``h{b}_{s}`` holds H[b][anc_{16 s + p}(b)].  All dofs on one
@@ -225,7 +226,19 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     # ---- assembly on the matrix cores: wavefront v of the workgroup assembles world v of the four
     NT = -(-nv // 16)  # 16-wide blocks of dofs
     tiles = [(ti, tj) for ti in range(NT) for tj in range(ti + 1)]  # lower triangle
-    W = NT * 16  # row length of the dense staging copy of H
+    # Staging copy of H's lower triangle in LDS, per world: the rows of tile row ti are 16 (ti + 1)
+    # words long and follow one another, the last tile row stops at the last dof (rounded up to
+    # the four rows a lane group stores), and worlds lie 16 words off a multiple of the banks so
+    # that two worlds' lanes of one request fall on different banks.
+    last_rows = 4 * -(-(nv - 16 * (NT - 1)) // 4)
+    tile_rows = [16] * (NT - 1) + [last_rows]
+    row_len = [16 * (ti + 1) for ti in range(NT)]
+    band_off = [sum(tile_rows[i] * row_len[i] for i in range(ti)) for ti in range(NT + 1)]
+    TW = band_off[NT] + 16  # words per world
+
+    def h_off(b):
+        return band_off[b // 16] + (b % 16) * row_len[b // 16]
+
     PD = max(2, min(16, 48 // NT))  # steps of 4 constraint rows in flight
     touched = [set() for _ in range(ngroups)]
     for j, g in enumerate(groups):
@@ -236,7 +249,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     # exchange through LDS: every group's trunk accumulators (one 64-lane vector per register)
     # and the trunk's solution per world
     xslots = []
-    xoff = 4 * W * W
+    xoff = 4 * TW
     for j in range(ngroups):
         sl = {}
         for a in sorted(touched[j]):
@@ -300,7 +313,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     # accumulator index table, M (as a flat copy that is then gathered from LDS, so that the
     # table and M travel together instead of one after the other), the row weights; then J.
     MC = -(-nM // 64)
-    assert MC * 64 <= W * W
+    assert MC * 64 <= TW
     for n, (ti, tj) in enumerate(tiles):
         for v in range(4):
             emit(f"    const int ix{n}_{v} = IDX_{name}[{n * 4 + v}][lane];")
@@ -330,7 +343,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     for u in range(SP):
         load(u, str(u))
     emit("    }")
-    emit(f"    float *mcopy = lds + wv * {W * W};  // reused for this world's dense H afterwards")
+    emit(f"    float *mcopy = lds + wv * {TW};  // reused for this world's copy of H afterwards")
     for i in range(MC):
         emit(f"    mcopy[{i * 64} + lane] = mv{i};")
     emit("    if (LONG) {")
@@ -387,15 +400,16 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     emit("    }")
     emit("    }")
     emit("    STAMP();  // 2: assembled")
-    # accumulators -> dense copy of H in LDS -> (wavefront 0) one register per row, lane = position on the chain
+    # accumulators -> lower triangle of H in LDS -> (wavefront 0) one register per row, lane = position on the chain
     for n, (ti, tj) in enumerate(tiles):
+        guard = f"if (kq < {tile_rows[ti] // 4}) " if tile_rows[ti] < 16 else ""
         for v in range(4):
-            emit(f"    lds[wv * {W * W} + ({16 * ti + v} + 4 * kq) * {W} + {16 * tj} + p] = acc{n}[{v}];")
+            emit(f"    {guard}lds[wv * {TW} + {band_off[ti]} + ({v} + 4 * kq) * {row_len[ti]} + {16 * tj} + p] = acc{n}[{v}];")
     emit("    STAMP();  // tiles written")
     emit("    __syncthreads();")
     emit("    STAMP();  // hand-over barrier passed")
     for i, (li, s) in enumerate(leaf_sets):
-        emit(f"    lh{i} = lds + kq * {W * W} + chc{i};")
+        emit(f"    lh{i} = lds + kq * {TW} + chc{i};")
     emit("  } else {")
     emit("    const float *Mw = M + ws * ldM;")
     for b in range(nv):
@@ -408,12 +422,12 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         return f"IM_BC({expr}, {pos})"
 
     def fetch_rows(dofs):
-        """rows of H into registers (fused kernel: from the dense copy in LDS), optional H output"""
+        """rows of H into registers (fused kernel: from the copy in LDS), optional H output"""
         emit("    if (ASM) {")
         for b in dofs:
             for s in range(t.sets(b)):
                 i = leaf_sets.index((t.leaf_of[b], s))
-                emit(f"      h{b}_{s} = lh{i}[{b * W}];")
+                emit(f"      h{b}_{s} = lh{i}[{h_off(b)}];")
         emit("      if (Hout && live && %d) {" % (0 if EXP == "timing" else 1))
         for b in dofs:
             for s in range(t.sets(b)):
