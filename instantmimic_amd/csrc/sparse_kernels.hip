@@ -462,14 +462,15 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
   if (nbad && lane == 0) atomicAdd(U + Q.nv_pad * Q.nv_pad - 1, (float)nbad);
 }
 
-// Per-iteration factor stage, one wavefront per world (four worlds per workgroup share the LDS
-// copy of the factor and solve tables).  Same arithmetic as sparse_update_kernel below; the
-// changed constraint rows are staged in LDS (up to kStagedRows of them, else they are read from
-// memory), packed H is updated in LDS and written back whole, and a lane keeps four pairs'
-// table look-ups in flight.
+// Per-iteration factor stage, one wavefront per world (WAVES worlds per workgroup share the LDS
+// copy of the factor and solve tables: four, eight or sixteen, chosen by the launcher).  Same arithmetic as
+// sparse_update_kernel below; the changed constraint rows are staged in LDS (up to kStagedRows
+// of them, else they are read from memory), packed H is updated in LDS and written back whole,
+// and a lane keeps four pairs' table look-ups in flight.
 constexpr int kStagedRows = 16;
 
-__global__ __launch_bounds__(256, 4) void sparse_update_wave_kernel(
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void sparse_update_wave_kernel(
     SparseWave A, const uint8_t *__restrict__ done, const int32_t *__restrict__ state_changes,
     const int32_t *__restrict__ changes, const int32_t *__restrict__ ids, int ld_ids,
     const float *__restrict__ J, int njmax, const float *__restrict__ D,
@@ -484,15 +485,16 @@ __global__ __launch_bounds__(256, 4) void sparse_update_wave_kernel(
   {
     const int4 *src = (const int4 *)A.P.t[0];
     const int nvec = A.staged_words >> 2;
-    int4 buf[8];
+    constexpr int T = 64 * WAVES, NB = 2048 / T;  // the host admits at most 8192 words
+    int4 buf[NB];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int q = i * 256 + tid;
+    for (int i = 0; i < NB; ++i) {
+      const int q = i * T + tid;
       buf[i] = src[q < nvec ? q : nvec - 1];
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int q = i * 256 + tid;
+    for (int i = 0; i < NB; ++i) {
+      const int q = i * T + tid;
       if (q < nvec) ((int4 *)tab)[q] = buf[i];
     }
   }
@@ -502,22 +504,23 @@ __global__ __launch_bounds__(256, 4) void sparse_update_wave_kernel(
     // forward-solve tables (at most 16 KB), behind the first stretch
     const int4 *src = (const int4 *)A.P.t[FL];
     const int nvec = A.solve_words >> 2;
-    int4 buf[4];
+    constexpr int T = 64 * WAVES, NB = 1024 / T;  // at most 4096 words
+    int4 buf[NB];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int q = i * 256 + tid;
+    for (int i = 0; i < NB; ++i) {
+      const int q = i * T + tid;
       buf[i] = src[q < nvec ? q : 0];
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int q = i * 256 + tid;
+    for (int i = 0; i < NB; ++i) {
+      const int q = i * T + tid;
       if (q < nvec) ((int4 *)(tab + A.staged_words))[q] = buf[i];
     }
 #pragma unroll
     for (int i = 0; i < 5; ++i) Q.t[FL + i] = tab + A.staged_words + A.solve[i];
   }
   __syncthreads();  // the only workgroup barrier
-  const int w = blockIdx.x * 4 + wv;
+  const int w = blockIdx.x * WAVES + wv;
   if (w >= nworld || (done && done[w]) || state_changes[w] == 0) return;
   const int n = Q.nv, nslots = Q.nslots, nfac = nslots - n, rhs = nfac;
   const int nw = (A.block + 31) / 32;
@@ -926,9 +929,34 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done, con
     A.solve_words = (int)solve_words;
     const size_t wave_lds = 4 * (staged + solve_words + 4 * per_world);
     if (wave_lds <= 64 * 1024 && staged <= 8192 && solve_words <= 4096) {
-      hipLaunchKernelGGL(im::sparse_update_wave_kernel, dim3((unsigned)((nworld + 3) / 4)), dim3(256), wave_lds,
-                         (hipStream_t)stream, A, done, state_changes, changes, ids, ld_ids, J, njmax, D, state,
-                         quad, grad, ldg, hfactor, dof_union, search, search_dot, decrement, nworld);
+      // Worlds per workgroup: every workgroup stages the tables for itself, so larger workgroups
+      // leave more of a CU's 160 KB to the worlds.  The count that keeps the most worlds on a CU
+      // (at most 32 wavefronts of 57 registers) is taken, the smallest on a tie and where four
+      // per workgroup already hold the whole batch.
+      constexpr size_t kCuLds = 160 * 1024;
+      int waves = 4;
+      int64_t best = 0;
+      for (int cand = 4; cand <= 16; cand *= 2) {
+        const size_t bytes = 4 * (staged + solve_words + (size_t)cand * per_world);
+        int64_t held = (int64_t)(kCuLds / bytes) * cand;
+        held = held < 32 ? held : 32;
+        if (held > best && (cand == 4 || (int64_t)nworld > best * 256)) best = held, waves = cand;
+      }
+      const size_t lds_bytes = 4 * (staged + solve_words + (size_t)waves * per_world);
+      const dim3 grid((unsigned)((nworld + waves - 1) / waves)), wg(64 * waves);
+#define IM_UPDATE_WAVE(W)                                                                                     \
+  do {                                                                                                        \
+    if (lds_bytes > 64 * 1024)                                                                                \
+      IM_HIP_CHECK(hipFuncSetAttribute((const void *)im::sparse_update_wave_kernel<W>,                        \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));          \
+    hipLaunchKernelGGL(im::sparse_update_wave_kernel<W>, grid, wg, lds_bytes, (hipStream_t)stream, A, done,   \
+                       state_changes, changes, ids, ld_ids, J, njmax, D, state, quad, grad, ldg, hfactor,     \
+                       dof_union, search, search_dot, decrement, nworld);                                     \
+  } while (0)
+      if (waves == 16) IM_UPDATE_WAVE(16);
+      else if (waves == 8) IM_UPDATE_WAVE(8);
+      else IM_UPDATE_WAVE(4);
+#undef IM_UPDATE_WAVE
       IM_HIP_CHECK(hipGetLastError());
       return IM_OK;
     }
