@@ -109,9 +109,11 @@ __global__ __launch_bounds__(kThreads) void newton_gradient_kernel(GradArgs a) {
 
 // ---- J v per constraint row ------------------------------------------------------------------
 // One wavefront takes 64 rows of one world: the rows (contiguous in memory) travel through LDS
-// with coalesced loads, sixteen in flight per lane, and a lane then walks its own row (rows sit
+// with coalesced loads, U in flight per lane (the launcher picks U so that one batch covers the
+// 64 rows: a wavefront then waits for memory once), and a lane then walks its own row (rows sit
 // an odd number of words apart in LDS).  Up to 50 dofs the sum is one chain of fused
 // multiply-adds; beyond, partial sums over 20 dofs each are added with a rounding of their own.
+template <int U>
 __global__ __launch_bounds__(64) void newton_jv_kernel(
     const float *__restrict__ J, int njmax, const int32_t *__restrict__ nefc_p,
     const float *__restrict__ search, int64_t lds_, const uint8_t *__restrict__ skip,
@@ -130,12 +132,12 @@ __global__ __launch_bounds__(64) void newton_jv_kernel(
   const float *src = J + (w * njmax + r0) * (int64_t)nv;
   const int total = rows * nv;
   const float inv_nv = 1.0f / (float)nv;
-  for (int i0 = lane; i0 < total; i0 += 16 * 64) {
-    float v[16];
+  for (int i0 = lane; i0 < total; i0 += U * 64) {
+    float v[U];
 #pragma unroll
-    for (int u = 0; u < 16; ++u) v[u] = src[i0 + 64 * u < total ? i0 + 64 * u : total - 1];
+    for (int u = 0; u < U; ++u) v[u] = src[i0 + 64 * u < total ? i0 + 64 * u : total - 1];
 #pragma unroll
-    for (int u = 0; u < 16; ++u) {
+    for (int u = 0; u < U; ++u) {
       const int i = i0 + 64 * u;
       if (i < total) {
         const int r = (int)(((float)i + 0.5f) * inv_nv);  // i / nv, exact while i stays below 2^20
@@ -333,8 +335,16 @@ extern "C" int im_newton_jv(const float *J, int njmax, const int32_t *nefc, cons
   if (lds_bytes > kLdsLimit || 64 * (int64_t)nv >= (1 << 20)) return IM_ERR_UNSUPPORTED;
   const int chunks = (njmax + 63) / 64;
   if ((int64_t)nworld * chunks > 0x7fffffff) return IM_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(newton_jv_kernel, dim3((unsigned)((int64_t)nworld * chunks)), dim3(64), lds_bytes,
-                     (hipStream_t)stream, J, njmax, nefc, search, ld_search, skip_world, jv, ld_jv, nv, chunks);
+  const dim3 grid((unsigned)((int64_t)nworld * chunks));
+#define IM_JV(U)                                                                                          \
+  hipLaunchKernelGGL(newton_jv_kernel<U>, grid, dim3(64), lds_bytes, (hipStream_t)stream, J, njmax, nefc, \
+                     search, ld_search, skip_world, jv, ld_jv, nv, chunks)
+  // 64 rows of nv words are nv words per lane
+  if (nv <= 16) IM_JV(16);
+  else if (nv <= 32) IM_JV(32);
+  else if (nv <= 48) IM_JV(48);
+  else IM_JV(64);
+#undef IM_JV
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }
