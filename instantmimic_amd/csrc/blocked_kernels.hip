@@ -39,6 +39,20 @@ __device__ __forceinline__ float row_bcast(float v, int n) {
   }
 }
 
+// The factor's LDS array: U is upper triangular, so the rows of block row t keep the columns from
+// t * B on and follow one another (a staircase by tiles: 46 KB at pad 144 where the square takes
+// 83 KB, which is what lets two workgroups share a CU there).  Diagonal tiles are held in full.
+template <int B>
+struct Stair {
+  int pad;
+  // words in front of block row t
+  __device__ __host__ __forceinline__ int band(int t) const { return B * t * pad - (B * B / 2) * t * (t - 1); }
+  // row r of block row t, column col >= t * B
+  __device__ __forceinline__ int in_band(int t, int r, int col) const { return band(t) + r * (pad - t * B) + col - t * B; }
+  __device__ __forceinline__ int at(int row, int col) const { return in_band(row / B, row % B, col); }
+  __device__ __host__ __forceinline__ int words() const { return band(pad / B); }
+};
+
 // Where a tile element comes from.
 // Dense: the upper triangle of a row-major (pad, pad) matrix (the lower one is never read);
 // rows and columns >= nv are the identity whatever the buffer holds there.
@@ -62,7 +76,8 @@ struct LdsSrc {
   int nv, pad;
   __device__ __forceinline__ float load(int kb, int ib, int, int r, int c) const {
     const int row = kb * B + r, col = ib * B + c;
-    if (row < nv && col < nv) return row <= col ? U[row * pad + col] : U[col * pad + row];
+    const Stair<B> S{pad};
+    if (row < nv && col < nv) return row <= col ? U[S.at(row, col)] : U[S.at(col, row)];
     return row == col ? 1.0f : 0.0f;
   }
 };
@@ -73,7 +88,7 @@ struct GatheredSrc {
   const float *U;
   int pad;
   __device__ __forceinline__ float load(int kb, int ib, int, int r, int c) const {
-    return U[(kb * B + r) * pad + ib * B + c];
+    return U[Stair<B>{pad}.in_band(kb, r, ib * B + c)];
   }
 };
 
@@ -122,19 +137,20 @@ __device__ __forceinline__ void gather_tiles(const float *__restrict__ Mw, const
           const int r = e / B, c = e - r * B;
           float x = idx[g][u] < nM ? v[g][u] : 0.0f;
           if (ti[g] == tk[g] && (tk[g] + 1) * B > nv && r == c && (nblk - 1) * B + r >= nv) x = x + 1.0f;
-          U[(tk[g] * B + r) * pad + ti[g] * B + c] = x;
+          U[Stair<B>{pad}.in_band(tk[g], r, ti[g] * B + c)] = x;
         }
       }
   }
 }
 
 // Left-looking upper Cholesky by block column with the forward solve of rhs fused into the
-// loop; U (pad, pad) and rhs (pad) in LDS, U zeroed by the caller.
+// loop; U (the staircase of pad) and rhs (pad) in LDS, U zeroed by the caller.
 template <int B, class Src>
 __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *rhs, float *A, float *L, int pad,
                                                int tid, int nt) {
   const int nblk = pad / B;
   constexpr int BB = B * B;
+  const Stair<B> S{pad};
   for (int kb = 0; kb < nblk; ++kb) {
     const int k = kb * B;
     // gather the whole block row kb..nblk-1 and subtract the finished block rows above
@@ -156,7 +172,8 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
           f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
           for (int s4 = 0; s4 < 4; ++s4) {
-            const float a = U[(j + 4 * s4 + kq) * pad + k + p], b = U[(j + 4 * s4 + kq) * pad + i0 + p];
+            const int at = S.in_band(jb, 4 * s4 + kq, p);
+            const float a = U[at + k], b = U[at + i0];
             sum = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, sum, 0, 0, 0);
           }
 #pragma unroll
@@ -174,7 +191,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
           const int j = jb * B;
           float sum = 0.0f;
 #pragma unroll
-          for (int t = 0; t < B; ++t) sum = fma_(U[(j + t) * pad + k + r], U[(j + t) * pad + i0 + c], sum);
+          for (int t = 0; t < B; ++t) sum = fma_(U[S.in_band(jb, t, k + r)], U[S.in_band(jb, t, i0 + c)], sum);
           v = v - sum;
         }
         A[q] = v;
@@ -186,7 +203,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
         const int j = jb * B;
         float sum = 0.0f;
 #pragma unroll
-        for (int t = 0; t < B; ++t) sum = fma_(U[(j + t) * pad + k + tid], rhs[j + t], sum);
+        for (int t = 0; t < B; ++t) sum = fma_(U[S.in_band(jb, t, k + tid)], rhs[j + t], sum);
         s = s - sum;
       }
       rhs[k + tid] = s;
@@ -224,7 +241,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
     // U_kk = L', and U_ki = L^-1 A_ki column by column
     for (int e = tid; e < BB; e += nt) {
       const int r = e / B, c = e - r * B;
-      U[(k + r) * pad + k + c] = c >= r ? L[c * B + r] : 0.0f;  // a gathered tile may have sat there
+      U[S.in_band(kb, r, k + c)] = c >= r ? L[c * B + r] : 0.0f;  // a gathered tile may have sat there
     }
     for (int q = tid; q < (ntile - 1) * B; q += nt) {
       const int tb = 1 + q / B, c = q - (tb - 1) * B;
@@ -241,7 +258,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
       }
       const int i0 = (kb + tb) * B;
 #pragma unroll
-      for (int r = 0; r < B; ++r) U[(k + r) * pad + i0 + c] = col[r];
+      for (int r = 0; r < B; ++r) U[S.in_band(kb, r, i0 + c)] = col[r];
     }
     __syncthreads();
   }
@@ -251,18 +268,20 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
 // diagonal tile each; the solved entries travel through DPP row broadcasts.
 template <int B>
 __device__ __forceinline__ void backward_solve(const float *U, float *rhs, int pad, int tid) {
+  const Stair<B> S{pad};
   for (int i0 = pad - B; i0 >= 0; i0 -= B) {
     if (tid < 64) {
       const int r = tid < B ? tid : 0;
       float s = rhs[i0 + r];
       float urow[B];
+      const float *Ur = U + S.in_band(i0 / B, r, 0);  // row i0 + r, indexed by column
 #pragma unroll
-      for (int c = 0; c < B; ++c) urow[c] = U[(i0 + r) * pad + i0 + c];
-      const float rinv = 1.0f / U[(i0 + r) * pad + i0 + r];
+      for (int c = 0; c < B; ++c) urow[c] = Ur[i0 + c];
+      const float rinv = 1.0f / Ur[i0 + r];
       for (int j = i0 + B; j < pad; j += B) {
         float sum = 0.0f;
 #pragma unroll
-        for (int t = 0; t < B; ++t) sum = fma_(U[(i0 + r) * pad + j + t], rhs[j + t], sum);
+        for (int t = 0; t < B; ++t) sum = fma_(Ur[j + t], rhs[j + t], sum);
         s = s - sum;
       }
 #pragma unroll
@@ -280,18 +299,19 @@ __device__ __forceinline__ void backward_solve(const float *U, float *rhs, int p
 // same operations on rhs as inside factor_forward.
 template <int B>
 __device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pad, int tid) {
+  const Stair<B> S{pad};
   for (int k = 0; k < pad; k += B) {
     if (tid < 64) {
       const int i = tid < B ? tid : 0;
       float s = rhs[k + i];
       float ucol[B];
 #pragma unroll
-      for (int j = 0; j < B; ++j) ucol[j] = U[(k + j) * pad + k + i];
-      const float rinv = 1.0f / U[(k + i) * pad + k + i];
+      for (int j = 0; j < B; ++j) ucol[j] = U[S.in_band(k / B, j, k + i)];
+      const float rinv = 1.0f / U[S.in_band(k / B, i, k + i)];
       for (int j = 0; j < k; j += B) {
         float sum = 0.0f;
 #pragma unroll
-        for (int t = 0; t < B; ++t) sum = fma_(U[(j + t) * pad + k + i], rhs[j + t], sum);
+        for (int t = 0; t < B; ++t) sum = fma_(U[S.in_band(j / B, t, k + i)], rhs[j + t], sum);
         s = s - sum;
       }
 #pragma unroll
@@ -311,13 +331,15 @@ __global__ __launch_bounds__(1024) void blocked_factor_solve_kernel(
     const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
     int64_t ldx, int nv, int pad) {
   extern __shared__ float lds[];
-  float *U = lds;             // [pad * pad]
-  float *rhs = U + pad * pad; // [pad]
+  const Stair<B> S{pad};
+  const int nU = S.words();
+  float *U = lds;             // [nU] the factor, block row by block row
+  float *rhs = U + nU;        // [pad]
   float *A = rhs + pad;       // [(nblk) * B * B] working tiles of the current block row
   float *L = A + (pad / B) * B * B;  // [B * B + B] Cholesky factor of the diagonal block (lower), 1 / pivots
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
-  for (int i = tid; i < pad * pad; i += nt) U[i] = 0.0f;
+  for (int i = tid; i < nU; i += nt) U[i] = 0.0f;
   for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? y[w * ldy + i] : 0.0f;
   __syncthreads();
   gather_tiles<B>(M + w * ldM, block_idx, nM, nv, pad, U, tid, nt);
@@ -327,8 +349,12 @@ __global__ __launch_bounds__(1024) void blocked_factor_solve_kernel(
   backward_solve<B>(U, rhs, pad, tid);
   for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
   if (Uout)
-    for (int i = tid; i < pad * pad / 4; i += nt)  // pad is a multiple of B >= 8
-      ((float4 *)(Uout + w * (int64_t)pad * pad))[i] = ((const float4 *)U)[i];
+    for (int i = tid; i < pad * pad / 4; i += nt) {  // pad is a multiple of B >= 8: a float4 stays in a tile
+      const int r = 4 * i / pad, c = 4 * i - r * pad;
+      float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (c >= r / B * B) v = *(const float4 *)(U + S.at(r, c));
+      ((float4 *)(Uout + w * (int64_t)pad * pad))[i] = v;
+    }
 }
 
 // ---- matrices up to 64 x 64: four worlds per wavefront ----------------------------------------
@@ -574,8 +600,10 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
     int32_t *__restrict__ uni_, float *__restrict__ search, int64_t lds_, float *__restrict__ search_dot,
     float *__restrict__ decrement, int nv, int pad, int row_cap) {
   extern __shared__ float lds[];
-  float *U = lds;             // [pad * pad]
-  float *rhs = U + pad * pad; // [pad]
+  const Stair<B> S{pad};
+  const int nU = S.words();
+  float *U = lds;             // [nU] the factor, block row by block row
+  float *rhs = U + nU;        // [pad]
   float *A = rhs + pad;       // [(pad / B) * B * B]
   float *L = A + (pad / B) * B * B;  // [B * B + B]: lower factor of the diagonal tile, 1 / pivots
   int *ul = (int *)(L + B * B + B);  // [nv] union list, [nv] = its length
@@ -614,27 +642,29 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
         const int r = idw[t];
         sd[t] = sw[r] == quad ? Dw[r] : -Dw[r];
       }
-      // 16 bytes per lane and four requests in flight: a lone workgroup per CU needs that much
-      // outstanding to stream 4 pad^2 bytes
+      // 16 bytes per lane and four requests in flight; the tiles below the diagonal are not read
       const int nvec = pad * pad / 4;  // pad is a multiple of 16
       for (int i0 = tid; i0 < nvec; i0 += 4 * nt) {
         float4 v[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           const int i = i0 + k * nt < nvec ? i0 + k * nt : nvec - 1;
-          v[k] = ((const float4 *)Hw)[i];
+          const int r = 4 * i / pad, c = 4 * i - r * pad;
+          v[k] = ((const float4 *)Hw)[c >= r / B * B ? i : nvec - 1];
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           const int i = i0 + k * nt;
           if (i < nvec) {
             const int r = 4 * i / pad, c = 4 * i - r * pad;
-            float4 o;
-            o.x = (r < nv && c + 0 < nv && r <= c + 0) ? v[k].x : 0.0f;
-            o.y = (r < nv && c + 1 < nv && r <= c + 1) ? v[k].y : 0.0f;
-            o.z = (r < nv && c + 2 < nv && r <= c + 2) ? v[k].z : 0.0f;
-            o.w = (r < nv && c + 3 < nv && r <= c + 3) ? v[k].w : 0.0f;
-            ((float4 *)U)[i] = o;
+            if (c >= r / B * B) {
+              float4 o;
+              o.x = (r < nv && c + 0 < nv && r <= c + 0) ? v[k].x : 0.0f;
+              o.y = (r < nv && c + 1 < nv && r <= c + 1) ? v[k].y : 0.0f;
+              o.z = (r < nv && c + 2 < nv && r <= c + 2) ? v[k].z : 0.0f;
+              o.w = (r < nv && c + 3 < nv && r <= c + 3) ? v[k].w : 0.0f;
+              *(float4 *)(U + S.at(r, c)) = o;
+            }
           }
         }
       }
@@ -693,8 +723,8 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
         for (int i = 0; i < 4; ++i) {
           const int row = 16 * rb + 4 * kq + i, col = ca;
           if (row <= col && col < nv && acc[i] != 0.0f) {
-            const float h = U[row * pad + col] + acc[i];
-            U[row * pad + col] = h;
+            const float h = U[S.at(row, col)] + acc[i];
+            U[S.at(row, col)] = h;
             Hw[(size_t)row * pad + col] = h;
           }
         }
@@ -714,8 +744,8 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
           delta = fma_(sd[t] * jr[t * nv + row], jr[t * nv + col], delta);  // -(D a) == (-D) a exactly
         }
         if (delta != 0.0f) {
-          const float h = U[row * pad + col] + delta;
-          U[row * pad + col] = h;
+          const float h = U[S.at(row, col)] + delta;
+          U[S.at(row, col)] = h;
           Hw[(size_t)row * pad + col] = h;
         }
       } else {
@@ -735,7 +765,7 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
       const LdsSrc<B> src{U, nv, pad};
       factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
     } else {
-      for (int i = tid; i < pad * pad; i += nt) U[i] = 0.0f;
+      for (int i = tid; i < nU; i += nt) U[i] = 0.0f;
       __syncthreads();  // this workgroup's own writes to H are read back below
       const DenseSrc<B> src{Hw, nv, pad};
       factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
@@ -758,7 +788,8 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
     __syncthreads();
     for (int i = tid; i < pad * pad / 4; i += nt) {  // pad is a multiple of 16: a float4 stays in a row
       const int r = 4 * i / pad, c = 4 * i - r * pad;
-      float4 v = ((const float4 *)U)[i];
+      float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (c >= r / B * B) v = *(const float4 *)(U + S.at(r, c));
       if (c + 3 == pad - 1) v.w = r < nv ? rhs[r] : (r == pad - 1 ? L[0] : v.w);
       ((float4 *)Uw)[i] = v;
     }
@@ -770,7 +801,8 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const int i = i0 + k * nt < nvec ? i0 + k * nt : nvec - 1;
-        v[k] = ((const float4 *)Uw)[i];
+        const int r = 4 * i / pad, c = 4 * i - r * pad;
+        v[k] = ((const float4 *)Uw)[c >= r / B * B ? i : nvec - 1];
       }
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
@@ -778,7 +810,7 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
         if (i < nvec) {
           const int r = 4 * i / pad, c = 4 * i - r * pad;
           if (c + 3 == pad - 1) v[k].w = r == pad - 1 ? 1.0f : 0.0f;  // drop the augmented column
-          ((float4 *)U)[i] = v[k];
+          if (c >= r / B * B) *(float4 *)(U + S.at(r, c)) = v[k];
         }
       }
     }
@@ -956,7 +988,8 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
     IM_HIP_CHECK(hipGetLastError());
     return IM_OK;
   }
-  const size_t lds_bytes = sizeof(float) * ((size_t)pad * pad + pad + (size_t)(pad / B) * B * B + B * B + B);
+  const size_t u_words = B == 8 ? im::Stair<8>{pad}.words() : im::Stair<16>{pad}.words();
+  const size_t lds_bytes = sizeof(float) * (u_words + pad + (size_t)(pad / B) * B * B + B * B + B);
   if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   auto fn = B == 8 ? im::blocked_factor_solve_kernel<8> : im::blocked_factor_solve_kernel<16>;
   if (lds_bytes > 64 * 1024)
@@ -964,7 +997,7 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
   // The pivots of a tile are one wavefront's work whatever the workgroup size, so a small matrix
   // takes fewer wavefronts per world and more worlds are resident per CU (measured on g1, snu and
   // the 128-dof stress shape: 64 threads up to pad 48, 128 for 16 x 16 tiles at pad 64, 256 up to
-  // pad 96, 512 beyond: one workgroup per CU there, the block rows' parallel parts want the lanes).
+  // pad 96, 512 beyond: two workgroups per CU there, the block rows' parallel parts want the lanes).
   const int threads = pad <= 48 ? 64 : (pad <= 64 && B == 16) ? 128 : pad <= 96 ? 256 : 512;
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(threads), lds_bytes, (hipStream_t)stream, M, ldM, nM, block_idx, y,
                      ldy, U, x, ldx, nv, pad);
@@ -1001,7 +1034,8 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
   if (((uintptr_t)H | (uintptr_t)U) & 15) return IM_ERR_STRIDE;  // read and written 16 bytes at a time
   constexpr int B = 16;
   const size_t base_bytes =
-      sizeof(float) * ((size_t)nv_pad * nv_pad + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + B + 2 * (size_t)nv + 1);
+      sizeof(float) * ((size_t)im::Stair<B>{nv_pad}.words() + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + B +
+                       2 * (size_t)nv + 1);
   if (base_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   // room for up to 32 changed rows of J next to the factor, as far as the 160 KB of LDS reach
   int row_cap = ld_ids < 32 ? ld_ids : 32;
@@ -1010,8 +1044,14 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
   auto fn = im::dense_update_factor_kernel<B>;
   if (lds_bytes > 64 * 1024)
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-  // a large matrix holds a CU alone: the pair sums and the copies of H and U want every lane
-  hipLaunchKernelGGL(fn, dim3(nworld), dim3(nv_pad <= 96 ? 256 : 1024), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
+  // 512 threads for a large matrix: two such workgroups share a CU (75 KB of LDS each at nv 128)
+  // and one's single-wavefront parts (pivots, union, corner chain) run beside the other's wide ones
+  static const int wide_threads = [] {
+    const char *e = std::getenv("IMHIP_DENSE_THREADS");
+    const int v = e ? std::atoi(e) : 0;
+    return (v == 256 || v == 512 || v == 1024) ? v : 512;
+  }();
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(nv_pad <= 96 ? 256 : wide_threads), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
                      ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, U, dof_union, search, ld_search,
                      search_dot, decrement, nv, nv_pad, row_cap);
   IM_HIP_CHECK(hipGetLastError());
