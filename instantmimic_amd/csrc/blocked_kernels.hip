@@ -325,8 +325,11 @@ __device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pa
   }
 }
 
-template <int B>
-__global__ __launch_bounds__(1024) void blocked_factor_solve_kernel(
+// LEAN: compiled for six wavefronts per SIMD (80 registers a lane), so that a third workgroup of
+// 512 starts on a CU where the LDS admits it (nv 128: 47 KB each); the few spills that costs are
+// in the gather.  Smaller matrices run fewer wavefronts per workgroup and keep the full budget.
+template <int B, bool LEAN>
+__global__ __launch_bounds__(512, LEAN ? 6 : 2) void blocked_factor_solve_kernel(
     const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
     const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
     int64_t ldx, int nv, int pad) {
@@ -991,7 +994,9 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
   const size_t u_words = B == 8 ? im::Stair<8>{pad}.words() : im::Stair<16>{pad}.words();
   const size_t lds_bytes = sizeof(float) * (u_words + pad + (size_t)(pad / B) * B * B + B * B + B);
   if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
-  auto fn = B == 8 ? im::blocked_factor_solve_kernel<8> : im::blocked_factor_solve_kernel<16>;
+  const bool lean = pad > 96;
+  auto fn = B == 8 ? (lean ? im::blocked_factor_solve_kernel<8, true> : im::blocked_factor_solve_kernel<8, false>)
+                   : (lean ? im::blocked_factor_solve_kernel<16, true> : im::blocked_factor_solve_kernel<16, false>);
   if (lds_bytes > 64 * 1024)
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   // The pivots of a tile are one wavefront's work whatever the workgroup size, so a small matrix
