@@ -1051,12 +1051,7 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   // 512 threads for a large matrix: two such workgroups share a CU (75 KB of LDS each at nv 128)
   // and one's single-wavefront parts (pivots, union, corner chain) run beside the other's wide ones
-  static const int wide_threads = [] {
-    const char *e = std::getenv("IMHIP_DENSE_THREADS");
-    const int v = e ? std::atoi(e) : 0;
-    return (v == 256 || v == 512 || v == 1024) ? v : 512;
-  }();
-  hipLaunchKernelGGL(fn, dim3(nworld), dim3(nv_pad <= 96 ? 256 : wide_threads), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(nv_pad <= 96 ? 256 : 512), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
                      ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, U, dof_union, search, ld_search,
                      search_dot, decrement, nv, nv_pad, row_cap);
   IM_HIP_CHECK(hipGetLastError());
