@@ -103,19 +103,80 @@ int im_assemble_tree_ldl_solve(const im_tree_plan *plan, const float *M,
                                int64_t ldg, float *x, int64_t ldx, float *Hout,
                                int nworld, unsigned flags, void *stream);
 
+/* Coupling pattern of a model's dofs: which pairs (a, b) may be nonzero in H.  Replaces
+ * hessian_pattern (src/instantmimic/utils/mjw_kernels/sparse_hessian.py:62-118) as a builder:
+ * creation couples every dof with its tree ancestors (:70-75; dof_parentid[d] < d), and the
+ * caller adds one clique per source of constraint rows.  body_parentid / body_dofadr /
+ * body_dofnum (nbody each, body 0 = world) are the model's. */
+typedef struct im_dof_pattern im_dof_pattern;
+int im_dof_pattern_create(int nv, const int32_t *dof_parentid, int nbody,
+                          const int32_t *body_parentid, const int32_t *body_dofadr,
+                          const int32_t *body_dofnum, im_dof_pattern **out);
+void im_dof_pattern_destroy(im_dof_pattern *pattern);
+/* All dofs on the chains from the listed bodies to the world couple pairwise: a declared body
+ * group, the two bodies of a connect / weld equality or of a collision pair, a flex element
+ * (`clique` of the reference, :77-86). */
+int im_dof_pattern_couple_bodies(im_dof_pattern *pattern, const int32_t *bodies, int n);
+/* The listed dofs couple pairwise (a joint equality, :104-107). */
+int im_dof_pattern_couple_dofs(im_dof_pattern *pattern, const int32_t *dofs, int n);
+/* adjacency (nv, nv) bytes, 1 where dofs a != b couple; symmetric, zero diagonal. */
+int im_dof_pattern_get(const im_dof_pattern *pattern, uint8_t *adjacency);
+
 /* Static-pattern sparse L'DL of H = M + J'DJ -------------------------------- */
 
 typedef struct im_sparse_plan im_sparse_plan;
 
-/* Device side of a SparseHessianPlan (src/instantmimic/utils/mjw_kernels/
- * sparse_hessian.py:38-50, tables :360-401).  tables[16] in this order, int32 each:
- * SH_LP, SH_LT, SH_ES, SH_EC, SH_RP, SH_RAB, SH_RKL, SH_ORIG, SH_BL, SH_BS, SH_BI, SH_BJ,
- * SH_PM, SH_SA, SH_SB, SH_SM; or tables[22] with the update stage's SH_PAIR, SH_FL, SH_FR,
- * SH_RS, SH_RKP, SH_RK (:374-380) appended.  block is the plan's block width (32 or 64). */
-int im_sparse_plan_create(int nv, int nv_pad, int block, int nslots, int nlevels,
-                          int ntables, const int32_t *const *tables, const int *sizes,
-                          im_sparse_plan **out);
+#define IM_SPARSE_FUSED 0    /* path "fused": the persistent Newton's layout of hfactor */
+#define IM_SPARSE_NONFUSED 1 /* path "nonfused": factor gathered from the dense H */
+
+/* Why a plan was refused (the reference raises ValueError with these meanings,
+ * sparse_hessian.py:249-250, 337-338, 680-684). */
+#define IM_SPARSE_ACCEPTED 0
+#define IM_SPARSE_REFUSED_LAYOUT 1  /* nslots >= 65536 or nfac + nv > nv_pad^2 */
+#define IM_SPARSE_REFUSED_INDEX16 2 /* a table value does not fit 16 bits */
+#define IM_SPARSE_REFUSED_HFACTOR 3 /* 2 nfac + nv >= nv_pad^2 - 1 */
+#define IM_SPARSE_REFUSED_SHARED 4  /* factor larger than the reference's 46 KB of shared memory */
+
+/* Table ids for im_sparse_plan_get_table, the reference's SH_* arrays (:360-401, SH_GAT :291-297). */
+enum {
+  IM_SH_LP, IM_SH_LT, IM_SH_ES, IM_SH_EC, IM_SH_RP, IM_SH_RAB, IM_SH_RKL, IM_SH_ORIG, IM_SH_BL,
+  IM_SH_BS, IM_SH_BI, IM_SH_BJ, IM_SH_PM, IM_SH_SA, IM_SH_SB, IM_SH_SM, IM_SH_PAIR, IM_SH_FL,
+  IM_SH_FR, IM_SH_RS, IM_SH_RKP, IM_SH_RK, IM_SH_GAT, IM_SH_COUNT
+};
+
+/* SparseHessianPlan (sparse_hessian.py:38-50). */
+typedef struct im_sparse_plan_info {
+  int32_t nv, nv_pad, block, path;
+  int32_t nslots;  /* factor slots + nv right-hand-side slots */
+  int32_t nfac;    /* factor slots: entries of L incl. the diagonal */
+  int32_t nterms;  /* multiply-adds of one numeric factor */
+  int32_t nlevels; /* elimination-tree levels */
+  int32_t device_ready;
+  double density;  /* nfac over the dense triangle */
+} im_sparse_plan_info;
+
+/* Replaces build_plan (sparse_hessian.py:229-401, 680-702): symbolic factor in elimination
+ * order e = nv - 1 - dof (:192-212, 235-237), row-major slots (:239-248), per level the
+ * entries with their runs of contiguous slots sorted by falling term count and the team width
+ * (:263-290, 215-221), the solve, pair, assembly, gather and pattern-mask tables (:291-401).
+ * M_rowi / M_colind (nM): row and column dof of every CSR element of M (m.M_hinit_i,
+ * m.M_colind).  block: the workgroup width the team widths are computed for.  A pattern the
+ * reference refuses yields IM_OK, *out = NULL and *refused != 0 (the caller keeps its dense
+ * factor, as for None).  The device tables go to the current HIP device unless host_only. */
+int im_sparse_plan_build(const im_dof_pattern *pattern, int nv_pad, int block, int path,
+                         const int32_t *M_rowi, const int32_t *M_colind, int nM, int host_only,
+                         int *refused, im_sparse_plan **out);
 void im_sparse_plan_destroy(im_sparse_plan *plan);
+int im_sparse_plan_get_info(const im_sparse_plan *plan, im_sparse_plan_info *info);
+/* Number of int32 values of a table, -1 for a bad id; an empty table holds one 0. */
+int im_sparse_plan_table_size(const im_sparse_plan *plan, int table);
+int im_sparse_plan_get_table(const im_sparse_plan *plan, int table, int32_t *out, int capacity);
+/* The fill pattern and elimination levels for a bit-exact comparison: column k of the factor
+ * (elimination index) has the later rows col_idx[col_ptr[k] .. col_ptr[k + 1]) ascending
+ * (col_ptr nv + 1 values, col_idx nfac - nv) and sits on level col_level[k].  Any pointer may
+ * be null. */
+int im_sparse_plan_get_structure(const im_sparse_plan *plan, int32_t *col_ptr, int32_t *col_idx,
+                                 int32_t *col_level);
 
 /* Replaces the launch of sparse_hessian.init_factor_kernel(plan)
  * (sparse_hessian.py:804-846, launched from newton_fusion.py:502-519) with the same

@@ -34,6 +34,20 @@ class TreePlanInfo(C.Structure):
 _vp, _i, _i64, _u = C.c_void_p, C.c_int, C.c_int64, C.c_uint
 
 
+class SparsePlanInfo(C.Structure):
+    _fields_ = [
+        ("nv", C.c_int32), ("nv_pad", C.c_int32), ("block", C.c_int32), ("path", C.c_int32),
+        ("nslots", C.c_int32), ("nfac", C.c_int32), ("nterms", C.c_int32), ("nlevels", C.c_int32),
+        ("device_ready", C.c_int32), ("density", C.c_double),
+    ]  # fmt: skip
+
+
+# order of the IM_SH_* table ids of imhip.h
+SPARSE_TABLES = ("SH_LP", "SH_LT", "SH_ES", "SH_EC", "SH_RP", "SH_RAB", "SH_RKL", "SH_ORIG", "SH_BL", "SH_BS",
+                 "SH_BI", "SH_BJ", "SH_PM", "SH_SA", "SH_SB", "SH_SM", "SH_PAIR", "SH_FL", "SH_FR", "SH_RS",
+                 "SH_RKP", "SH_RK", "SH_GAT")  # fmt: skip
+
+
 class MuscleForceModel(C.Structure):
     _fields_ = [
         ("force_scale", C.c_float),
@@ -99,7 +113,16 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _i, _u, _vp],
     ),
-    "im_sparse_plan_create": (_i, [_i, _i, _i, _i, _i, _i, _vp, _vp, C.POINTER(_vp)]),
+    "im_dof_pattern_create": (_i, [_i, _vp, _i, _vp, _vp, _vp, C.POINTER(_vp)]),
+    "im_dof_pattern_destroy": (None, [_vp]),
+    "im_dof_pattern_couple_bodies": (_i, [_vp, _vp, _i]),
+    "im_dof_pattern_couple_dofs": (_i, [_vp, _vp, _i]),
+    "im_dof_pattern_get": (_i, [_vp, _vp]),
+    "im_sparse_plan_build": (_i, [_vp, _i, _i, _i, _vp, _vp, _i, _i, C.POINTER(_i), C.POINTER(_vp)]),
+    "im_sparse_plan_get_info": (_i, [_vp, C.POINTER(SparsePlanInfo)]),
+    "im_sparse_plan_table_size": (_i, [_vp, _i]),
+    "im_sparse_plan_get_table": (_i, [_vp, _i, _vp, _i]),
+    "im_sparse_plan_get_structure": (_i, [_vp, _vp, _vp, _vp]),
     "im_sparse_plan_destroy": (None, [_vp]),
     "im_sparse_init_factor": (
         _i,

@@ -18,7 +18,7 @@ GEN = os.path.join(CSRC, "gen")
 OBJ = os.path.join(HERE, "_obj")
 LIB = os.path.join(HERE, "libimhip.so")
 
-SOURCES = ["tree_plan.cpp", "tree_kernels.hip", "muscle_kernels.hip", "muscle_geometry.hip", "sparse_kernels.hip", "blocked_kernels.hip", "tree_reduce_kernels.hip", "newton_kernels.hip"]
+SOURCES = ["tree_plan.cpp", "sparse_plan.cpp", "tree_kernels.hip", "muscle_kernels.hip", "muscle_geometry.hip", "sparse_kernels.hip", "blocked_kernels.hip", "tree_reduce_kernels.hip", "newton_kernels.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950",
@@ -37,12 +37,50 @@ FLAGS = [
 ]  # fmt: skip
 
 
-def _python_planner(parents):
-    """The reference planner's result for a tree, through the library's host planner
-    when it is already built, else through a local restatement (bootstrap)."""
-    from .codegen import plan_bootstrap
+PLANNER_LIB = os.path.join(OBJ, "libimplan_host.so")
 
-    return plan_bootstrap.best_plan(parents)
+
+def _host_planner():
+    """The library's own host planner (csrc/tree_plan.cpp), built alone ahead of everything
+    else: the kernel generator needs each known tree's plan before ``libimhip.so`` exists."""
+    import ctypes as C
+
+    src = os.path.join(CSRC, "tree_plan.cpp")
+    os.makedirs(OBJ, exist_ok=True)
+    stale = not os.path.exists(PLANNER_LIB) or os.path.getmtime(PLANNER_LIB) < max(
+        os.path.getmtime(p) for p in (src, os.path.join(CSRC, "common.h"), os.path.join(HERE, "..", "include", "imhip.h"))
+    )
+    if stale or os.environ.get("IMHIP_REBUILD"):
+        cmd = ["hipcc", "--offload-arch=gfx950", "-O1", "-std=c++17", "-fPIC", "-shared", "-DIM_PLANNER_ONLY",
+               "-Wno-unused-command-line-argument", "-x", "hip", src, "-o", PLANNER_LIB]  # fmt: skip
+        subprocess.run(cmd, check=True)
+    return C.CDLL(PLANNER_LIB)
+
+
+def _plan_of_tree(parents):
+    """((rowadr, rownnz, colind), groups, trunk, eligible) of a dof tree from the host planner."""
+    import ctypes as C
+
+    from . import _lib, synth
+
+    rowadr, rownnz, colind = synth.csr_from_parents(parents)
+    lib = _host_planner()
+    handle = C.c_void_p()
+    vp = lambda a: C.c_void_p(a.ctypes.data)  # noqa: E731
+    status = lib.im_tree_plan_create(len(parents), vp(rowadr), vp(rownnz), vp(colind), int(colind.size), 0, 1, C.byref(handle))
+    if status != 0:
+        raise RuntimeError(f"host planner refused the tree (status {status})")
+    info = _lib.TreePlanInfo()
+    lib.im_tree_plan_get_info(handle, C.byref(info))
+    import numpy as np
+
+    gptr, gdofs, trunk = np.zeros(info.ngroups + 1, np.int32), np.zeros(max(info.nv - info.ntrunk, 1), np.int32), np.zeros(max(info.ntrunk, 1), np.int32)
+    lib.im_tree_plan_get_arrays(handle, vp(gptr), vp(gdofs), vp(trunk), None)
+    lib.im_tree_plan_destroy.argtypes = [C.c_void_p]
+    lib.im_tree_plan_destroy(handle)
+    groups = tuple(tuple(int(d) for d in gdofs[gptr[j] : gptr[j + 1]]) for j in range(info.ngroups))
+    st = tuple(tuple(int(v) for v in a) for a in (rowadr, rownnz, colind))
+    return st, groups, tuple(int(d) for d in trunk[: info.ntrunk]), bool(info.beats_dense)
 
 
 def generate_sources() -> list[str]:
@@ -55,7 +93,7 @@ def generate_sources() -> list[str]:
     for name, shape in synth.SHAPES.items():
         if only and name not in only.split(","):
             continue
-        st, groups, trunk, eligible = _python_planner(list(shape.parents))
+        st, groups, trunk, eligible = _plan_of_tree(list(shape.parents))
         if not eligible or len(st[0]) > 64:
             continue
         src = tree_row16.generate(name, *st, groups, trunk)

@@ -907,7 +907,7 @@ __global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const bool in = r0 + wave * 8 + i < nefc;
-      Js[(wave * 8 + i) * nvr + c0] = (in && c0 < nv) ? v0[i] : 0.0f;
+      if (c0 < nvr) Js[(wave * 8 + i) * nvr + c0] = (in && c0 < nv) ? v0[i] : 0.0f;  // nvr is 32 for nv <= 32
       if (c1 < nvr) Js[(wave * 8 + i) * nvr + c1] = (in && c1 < nv) ? v1[i] : 0.0f;
     }
     if (lane < 8) dcs[wave * 8 + lane] = (r0 + wave * 8 + lane < nefc && sd == quad) ? dd : 0.0f;
@@ -1012,7 +1012,7 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
 
 int im_jtdj_mfma(const float *Mdense, const float *J, int njmax, const float *D, const int32_t *state,
                  const int32_t *nefc, int quad, float *H, int nv, int nv_pad, int nworld, void *stream) {
-  if (nworld < 0 || nv <= 0 || nv_pad < nv || njmax < 0) return IM_ERR_ARG;
+  if (nworld < 0 || nv <= 0 || nv_pad < nv || njmax <= 0) return IM_ERR_ARG;  // rows are clamped to njmax - 1
   if (nworld == 0) return IM_OK;
   if (!Mdense || !J || !D || !state || !H) return IM_ERR_ARG;
   if (nv > 128) return IM_ERR_UNSUPPORTED;
@@ -1029,7 +1029,7 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
                            const int32_t *state, int quad, const float *grad, int64_t ldg, float *H, float *U,
                            int nv, int nv_pad, int32_t *dof_union, float *search, int64_t ld_search,
                            float *search_dot, float *decrement, int nworld, void *stream) {
-  if (nworld < 0 || nv <= 0 || nv_pad <= nv || ld_ids < 0 || njmax < 0) return IM_ERR_ARG;
+  if (nworld < 0 || nv <= 0 || nv_pad <= nv || ld_ids < 0 || njmax <= 0) return IM_ERR_ARG;
   if (nworld == 0) return IM_OK;
   if (!state_changes || !changes || !ids || !J || !D || !state || !grad || !H || !U || !dof_union || !search ||
       !search_dot || !decrement)

@@ -176,6 +176,7 @@ int im_muscle_project(const float *moment, int64_t ld_moment, const float *force
                       int root_dof_count, float *qfrc, int64_t ld_qfrc, int nworld, void *stream) {
   if (nworld < 0 || nentry < 0 || ntorque < 0) return IM_ERR_ARG;
   if (nworld == 0 || ntorque == 0) return IM_OK;
+  if (nentry == 0) return IM_ERR_ARG;  // entry indices are clamped to nentry - 1
   if (!moment || !force || !torque_entry_offsets || !torque_entry_idx || !entry_muscle || !qfrc) return IM_ERR_ARG;
   if (ld_moment < nentry || ld_force < nmuscle || ld_qfrc < root_dof_count + ntorque) return IM_ERR_STRIDE;
   if (nmuscle > 65535) return IM_ERR_UNSUPPORTED;  // muscle ids travel as 16 bits

@@ -8,8 +8,7 @@
 //   backward pushes per level, search = -x, (x.x, g.x) reduced warp then block      :453-479
 //   hfactor layout: [0,nfac) packed H, [nfac,2nfac) N = L D, [2nfac,2nfac+n) 1/D,
 //   last element = pattern-violation counter                                        :488-489, 634-635
-// The tables come from the host planner (instantmimic_amd/mjw_kernels/sparse_hessian.py)
-// instead of generated source; team widths and block width are the plan's, so the
+// The tables come from the host planner (sparse_plan.cpp) instead of generated source; team widths and block width are the plan's, so the
 // order in which a team sums an entry's terms is the reference's.
 #include <hip/hip_runtime.h>
 
@@ -18,24 +17,10 @@
 #include <vector>
 
 #include "common.h"
-
-struct im_sparse_plan {
-  int nv, nv_pad, block, nslots, nlevels;
-  void *blob = nullptr;
-  int ntables = 0;
-  const int32_t *t[22] = {};
-  int sizes[22] = {};
-  // per lane of the lower-triangle 16 x 16 accumulator tiles: where the element comes from in a
-  // row of M and which slot it is ((M index + 1) << 16 | (slot + 1)); null when nv > 64
-  int32_t *tile_index = nullptr;
-  int nM = 0;
-};
+#include "sparse_plan.h"
 
 namespace im {
 namespace {
-
-enum { LP, LT, ES, EC, RP, RAB, RKL, ORIG, BL, BS, BI, BJ, PM, SA, SB, SM, NINIT,
-       PAIR = NINIT, FL, FR, RS, RKP, RK, NTABLES };
 
 struct SparseDev {
   const int32_t *t[NTABLES];
@@ -775,62 +760,53 @@ __global__ void sparse_update_kernel(SparseDev P, const uint8_t *__restrict__ do
 
 extern "C" {
 
-int im_sparse_plan_create(int nv, int nv_pad, int block, int nslots, int nlevels, int ntables,
-                          const int32_t *const *tables, const int *sizes, im_sparse_plan **out) {
-  if (!out) return IM_ERR_ARG;
-  *out = nullptr;
-  if (!tables || !sizes || (ntables != im::NINIT && ntables != im::NTABLES) || nv <= 0 || nslots <= nv)
-    return IM_ERR_ARG;
-  if (block != 32 && block != 64) return IM_ERR_UNSUPPORTED;
-  auto *pl = new im_sparse_plan;
-  pl->nv = nv; pl->nv_pad = nv_pad; pl->block = block; pl->nslots = nslots; pl->nlevels = nlevels;
-  pl->ntables = ntables;
+}  // extern "C"
+
+namespace im {
+
+int sparse_plan_upload(im_sparse_plan *pl) {
+  pl->device_ready = false;
+  if (pl->block != 32 && pl->block != 64) return IM_ERR_UNSUPPORTED;  // the kernels' workgroup widths
+  const int nv = pl->nv, nfac = pl->nfac;
   size_t total = 0;
-  for (int i = 0; i < ntables; ++i) total += ((size_t)sizes[i] * 4 + 15) / 16 * 16;
+  size_t offs[NTABLES];
+  for (int i = 0; i < NTABLES; ++i) {
+    offs[i] = total;
+    pl->sizes[i] = (int)pl->table[i].size();
+    total += (pl->table[i].size() * 4 + 15) / 16 * 16;
+  }
   std::vector<char> host(total, 0);
-  size_t off = 0;
-  std::vector<size_t> offs(ntables);
-  for (int i = 0; i < ntables; ++i) {
-    offs[i] = off;
-    memcpy(host.data() + off, tables[i], (size_t)sizes[i] * 4);
-    off += ((size_t)sizes[i] * 4 + 15) / 16 * 16;
-    pl->sizes[i] = sizes[i];
-  }
-  if (hipMalloc(&pl->blob, total) != hipSuccess || hipMemcpy(pl->blob, host.data(), total, hipMemcpyHostToDevice) != hipSuccess) {
-    im::set_hip_error(hipGetLastError());
-    if (pl->blob) (void)hipFree(pl->blob);
-    delete pl;
-    return IM_ERR_HIP;
-  }
-  for (int i = 0; i < ntables; ++i) pl->t[i] = (const int32_t *)((char *)pl->blob + offs[i]);
-  const int nfac = nslots - nv;
-  if (nv <= 64 && sizes[im::SA] >= nfac && sizes[im::SB] >= nfac && sizes[im::SM] >= nfac && nslots < 65535) {
-    const int32_t *sa = tables[im::SA], *sb = tables[im::SB], *sm = tables[im::SM];
+  for (int i = 0; i < NTABLES; ++i) memcpy(host.data() + offs[i], pl->table[i].data(), pl->table[i].size() * 4);
+  IM_HIP_CHECK(hipMalloc(&pl->blob, total));
+  IM_HIP_CHECK(hipMemcpy(pl->blob, host.data(), total, hipMemcpyHostToDevice));
+  for (int i = 0; i < NTABLES; ++i) pl->t[i] = (const int32_t *)((char *)pl->blob + offs[i]);
+  if (nv <= 64 && pl->nslots < 65535) {
+    const int32_t *sa = pl->table[SA].data(), *sb = pl->table[SB].data(), *sm = pl->table[SM].data();
     const int nt = (nv + 15) / 16;
     std::vector<int32_t> tix((size_t)nt * (nt + 1) / 2 * 256, 0);
     int nM = 1;
     bool fits = true;
     for (int sl = 0; sl < nfac; ++sl) {
       const int a = sa[sl], b = sb[sl], e = sm[sl];  // a <= b: tile row b, tile column a
-      if (a < 0 || b < a || b >= nv || e >= 1024) { fits = false; break; }
+      if (e >= 1024) { fits = false; break; }
       nM = e + 1 > nM ? e + 1 : nM;
       const int ti = b / 16, tj = a / 16, i = b % 16, j = a % 16;
       const int t = ti * (ti + 1) / 2 + tj, lane = j + 16 * (i / 4), v = i % 4;
       tix[((size_t)t * 4 + v) * 64 + lane] = ((e + 1) << 16) | (sl + 1);
     }
     if (fits) {
-      if (hipMalloc((void **)&pl->tile_index, tix.size() * 4) != hipSuccess ||
-          hipMemcpy(pl->tile_index, tix.data(), tix.size() * 4, hipMemcpyHostToDevice) != hipSuccess) {
-        im::set_hip_error(hipGetLastError());
-        im_sparse_plan_destroy(pl);
-        return IM_ERR_HIP;
-      }
+      IM_HIP_CHECK(hipMalloc((void **)&pl->tile_index, tix.size() * 4));
+      IM_HIP_CHECK(hipMemcpy(pl->tile_index, tix.data(), tix.size() * 4, hipMemcpyHostToDevice));
       pl->nM = nM;
     }
   }
-  *out = pl;
+  pl->device_ready = true;
   return IM_OK;
 }
+
+}  // namespace im
+
+extern "C" {
 
 void im_sparse_plan_destroy(im_sparse_plan *plan) {
   if (!plan) return;
@@ -843,7 +819,8 @@ int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done, const
                           const float *J, int njmax, const float *D, const int32_t *state, int quad,
                           const float *M, int ldM, const float *grad, int ldg, float *hfactor,
                           float *search, float *search_dot, float *decrement, int nworld, void *stream) {
-  if (!plan || nworld < 0) return IM_ERR_ARG;
+  if (!plan || nworld < 0 || njmax <= 0) return IM_ERR_ARG;  // rows are clamped to njmax - 1
+  if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
   if (nworld == 0) return IM_OK;
   if (!nefc || !J || !D || !state || !M || !grad || !hfactor || !search || !search_dot || !decrement) return IM_ERR_ARG;
   if (ldg < plan->nv) return IM_ERR_STRIDE;
@@ -897,8 +874,8 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done, con
                             const float *D, const int32_t *state, int quad, const float *grad, int ldg,
                             float *hfactor, int32_t *dof_union, float *search, float *search_dot,
                             float *decrement, int nworld, void *stream) {
-  if (!plan || nworld < 0 || ld_ids < 0) return IM_ERR_ARG;
-  if (plan->ntables != im::NTABLES) return IM_ERR_UNSUPPORTED;  // built without the update tables
+  if (!plan || nworld < 0 || ld_ids < 0 || njmax <= 0) return IM_ERR_ARG;
+  if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
   if (nworld == 0) return IM_OK;
   if (!state_changes || !changes || !ids || !J || !D || !state || !grad || !hfactor || !dof_union || !search ||
       !search_dot || !decrement)

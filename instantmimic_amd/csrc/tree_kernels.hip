@@ -336,8 +336,8 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
   if (nworld == 0) return IM_OK;
   if (!M || !y || !x) return IM_ERR_ARG;
   if (ldM < plan->nM || ldy < plan->nv || ldx < plan->nv) return IM_ERR_STRIDE;
-  if (assemble && (!J || !D || !state || njmax < 0)) return IM_ERR_ARG;
-  if (nworld == 0) return IM_OK;
+  // njmax >= 1: the kernels clamp row indices to njmax - 1
+  if (assemble && (!J || !D || !state || njmax <= 0)) return IM_ERR_ARG;
   if (plan->row16) {
     const auto *e = (const gen::Row16Entry *)plan->row16;
     void *args[] = {&M, &ldM, &J, &njmax, &D, &state, &nefc, &quad, &y, &ldy, &x, &ldx, &Hout, &nworld, &flags};

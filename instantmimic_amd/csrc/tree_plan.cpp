@@ -154,6 +154,10 @@ int exchange_bytes(const im_tree_plan &pl, int groups) {
 
 namespace im {
 void set_hip_error(hipError_t e) { g_last_hip_error = int(e); }
+#ifdef IM_PLANNER_ONLY
+// this file alone as a host-only planner (used while the library itself is being built)
+int tree_plan_upload(im_tree_plan *) { return IM_ERR_UNSUPPORTED; }
+#endif
 }  // namespace im
 
 extern "C" {

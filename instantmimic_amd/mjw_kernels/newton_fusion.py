@@ -29,6 +29,91 @@ import numpy as np
 from .. import _lib
 
 
+# mujoco_warp's enums are not importable here; members are matched by name when the model
+# carries enum objects and by MuJoCo's published integer values otherwise (mjtSolver: NEWTON = 2;
+# mjtCone: PYRAMIDAL = 0; the DISCRETE integrator is an addition of the reference's mujoco_warp
+# build and is matched by name only).
+SOLVER_NEWTON = 2
+CONE_PYRAMIDAL = 0
+
+
+def _is_member(value, name: str, number) -> bool:
+    label = getattr(value, "name", None)
+    if label is not None:
+        return str(label).upper() == name
+    return number is not None and value is not None and int(value) == number
+
+
+def _sparse_compact(ctx) -> bool:
+    return bool(getattr(ctx, "sparse_compact", False)) if ctx is not None else False
+
+
+def _option_gates(m) -> bool:
+    """Newton solver with a positive iteration budget, pyramidal cone, not the DISCRETE
+    integrator; a model without ``opt`` does not qualify."""
+    opt = getattr(m, "opt", None)
+    if opt is None:
+        return False
+    return (
+        _is_member(getattr(opt, "solver", None), "NEWTON", SOLVER_NEWTON)
+        and _is_member(getattr(opt, "cone", None), "PYRAMIDAL", CONE_PYRAMIDAL)
+        and not _is_member(getattr(opt, "integrator", None), "DISCRETE", None)
+        and int(getattr(opt, "iterations", 0)) > 0
+    )
+
+
+def eligible(m, ctx, *, compact: bool = False, device="cuda") -> bool:
+    """Whether the fused Newton takes the model: ``eligible`` of the reference
+    (src/instantmimic/utils/mjw_kernels/newton_fusion.py:307-322).  Fields the reference reads
+    from the uploaded model are read from ``m`` and a missing one disqualifies.  Upstream's
+    ``_use_incremental`` is taken as "Newton solver" (the gate the reference itself mirrors in
+    src/instantmimic/utils/mjw_model.py:95-102) unless the model states ``use_incremental``;
+    ``_sparse_compact`` is read from ``ctx.sparse_compact``.  ``device=None`` stands for
+    planning on the host for a GPU run."""
+    arr = getattr(m, "body_parentid", None)
+    where = None if isinstance(arr, np.ndarray) else getattr(arr, "device", None)  # NumPy copies say nothing
+    if where is not None:
+        on_gpu = bool(getattr(where, "is_cuda", False) or getattr(where, "type", "") == "cuda")
+    else:
+        on_gpu = device is None or str(device).startswith("cuda")
+    nv, nv_pad = int(m.nv), int(getattr(m, "nv_pad", 0))
+    incremental = getattr(m, "use_incremental", None)
+    if incremental is None:
+        incremental = _is_member(getattr(getattr(m, "opt", None), "solver", None), "NEWTON", SOLVER_NEWTON)
+    width = getattr(getattr(m, "block_dim", None), "linesearch_iterative", None)
+    return bool(
+        not compact
+        and on_gpu
+        and 0 < nv <= 79
+        and nv_pad % 16 == 0
+        and 0 < nv_pad <= 80
+        and incremental
+        and _option_gates(m)
+        and getattr(m, "is_sparse", None) is False
+        and not _sparse_compact(ctx)
+        and width == 32
+    )
+
+
+def upstream_newton_structure(m, ctx, *, compact: bool = False) -> bool:
+    """The gate of the upstream (non-fused) iteration with the sparse factor substituted
+    (src/instantmimic/utils/mjw_kernels/sparse_hessian.py:738-746)."""
+    hfactor = getattr(ctx, "hfactor", None) if ctx is not None else None
+    return bool(
+        _option_gates(m)
+        and not compact
+        and not _sparse_compact(ctx)
+        and hfactor is not None
+        and len(hfactor.shape) > 1
+        and int(hfactor.shape[1]) == int(getattr(m, "nv_pad", -1))
+    )
+
+
+def newton_block_dim(m) -> int:
+    """Physical Newton block width (newton_fusion.py:325-327)."""
+    return 64 if int(m.nv_pad) >= 64 else int(m.block_dim.linesearch_iterative)
+
+
 def mul_m_tables(rowadr, rownnz, colind):
     """(mulm_rowadr[nv + 1], mulm_col, mulm_madr) int32 for M's CSR (row = ancestors root
     first, diagonal last)."""

@@ -64,7 +64,7 @@ def factor_factory(nv: int, pad: int, sparse_plan: SparseHessianPlan | None = No
                 if lds != nv:
                     raise ValueError("search must be (nworld, nv) on the sparse path")
                 status = L.im_sparse_update_factor(
-                    sparse_plan.handle.ptr, done_ptr, state_changes.data_ptr(), changes.data_ptr(), ids.data_ptr(),
+                    sparse_plan.ptr, done_ptr, state_changes.data_ptr(), changes.data_ptr(), ids.data_ptr(),
                     int(ids.shape[1]), J.data_ptr(), int(njmax), D.data_ptr(), state.data_ptr(), int(quad),
                     grad.data_ptr(), int(ldg), U.data_ptr(), dof_union.data_ptr(), search.data_ptr(),
                     search_dot.data_ptr(), decrement.data_ptr(), int(nworld), stream,

@@ -1,23 +1,21 @@
 """Static-pattern sparse L'DL of the Newton Hessian ``H = M + J'DJ`` on MI355X.
 
 Drop-in for the reference module ``instantmimic.utils.mjw_kernels.sparse_hessian``
-(src/instantmimic/utils/mjw_kernels/sparse_hessian.py): the coupling pattern of the
-model (:62-118), its symbolic factor and elimination levels (:192-212), the level /
-run / backward tables of the numeric factor (:229-401) and the launcher of the initial
-assemble + factor + solve (:804-846).  Here the tables are NumPy arrays handed to
-``libimhip`` (the reference bakes them into generated CUDA source); the numeric kernel
-is ``csrc/sparse_kernels.hip``.
+(src/instantmimic/utils/mjw_kernels/sparse_hessian.py).  This module only marshals: it reads
+the model's arrays, names the sources of constraint rows to the library's pattern builder
+(:62-171), asks the library for the plan (symbolic factor, levels, tables: :192-401) and
+launches the numeric kernels (:804-894).  The planning itself is ``csrc/sparse_plan.cpp``, the
+kernels ``csrc/sparse_kernels.hip``; the reference bakes its tables into generated CUDA
+source, here they are device arrays owned by the plan handle.
 
 Entries hold ``N = L D``; slots are row-major in elimination order (leaves first:
-elimination index ``e = nv - 1 - dof``) so an entry's terms are runs of contiguous
-slots; the right-hand side rides as an augmented last row.
+elimination index ``e = nv - 1 - dof``); the right-hand side rides as an augmented last row.
 """
 
 from __future__ import annotations
 
 import ctypes as C
-from dataclasses import dataclass, field
-from typing import Any, Sequence
+from typing import Any, Iterable, Iterator, Sequence
 
 import numpy as np
 
@@ -26,270 +24,179 @@ from .. import _lib
 EQ_CONNECT, EQ_WELD, EQ_JOINT = 0, 1, 2
 EQ_FLEX, EQ_FLEXVERT, EQ_FLEXSTRAIN = 4, 5, 6
 OBJ_SITE = 6
-MAX_SHARED_BYTES = 46 * 1024
-MAX_DENSITY = 0.6
-MIN_NV = 33
-NONFUSED_MIN_NV = 80
+MAX_DENSITY = 0.6  # sparse_hessian.py:183
+MIN_NV = 33  # :184
+NONFUSED_MIN_NV = 80  # :189
 QUADRATIC = 1  # mjtConstraintState.mjCNSTRSTATE_QUADRATIC
-ROWS_PER_TILE = 4  # constraint rows per staged tile of the initial assembly
+PATHS = {"fused": 0, "nonfused": 1}
+REFUSALS = {
+    1: "sparse Hessian factor does not fit the packed layout",
+    2: "sparse Hessian tables exceed 16-bit indices",
+    3: "packed H and factor do not fit hfactor",
+    4: "the factor does not fit the block's shared memory",
+}
 
 
-def _arr(a) -> np.ndarray:
+def _host(a, dtype=np.int32) -> np.ndarray:
+    """A model array (NumPy, torch or anything with ``numpy()``) as a contiguous host array."""
     if a is None:
-        return np.zeros(0, np.int64)
+        return np.zeros(0, dtype)
     if hasattr(a, "detach"):
         a = a.detach().cpu()
     if hasattr(a, "numpy"):
         a = a.numpy()
-    return np.asarray(a)
+    return np.ascontiguousarray(np.asarray(a), dtype)
 
 
-def _chain(body, body_parentid, body_dofadr, body_dofnum) -> list[int]:
-    out, b = [], int(body)
-    while b > 0:
-        out += range(int(body_dofadr[b]), int(body_dofadr[b]) + int(body_dofnum[b]))
-        b = int(body_parentid[b])
-    return out
+class DofPattern:
+    """Owns an ``im_dof_pattern``; reads like the reference's ``list[set[int]]`` adjacency
+    (``len(p)``, ``p[dof]`` = set of coupled dofs)."""
 
-
-def hessian_pattern(m: Any, body_groups: Sequence[Sequence[int]]) -> list[set[int]]:
-    """Upper bound of H's off-diagonal pattern as dof adjacency (MuJoCo dof order):
-    tree ancestry, cliques over the dof chains of every declared body group, equality
-    constraints and native collision candidates."""
-    nv = int(m.nv)
-    dof_parentid = _arr(m.dof_parentid)
-    body_parentid, body_dofadr, body_dofnum = _arr(m.body_parentid), _arr(m.body_dofadr), _arr(m.body_dofnum)
-    adj = [set() for _ in range(nv)]
-    for d in range(nv):
-        p = int(dof_parentid[d])
-        while p >= 0:
-            adj[d].add(p)
-            adj[p].add(d)
-            p = int(dof_parentid[p])
-
-    def clique(bodies):
-        dofs = sorted({d for b in bodies for d in _chain(b, body_parentid, body_dofadr, body_dofnum)})
-        for a in dofs:
-            adj[a].update(x for x in dofs if x != a)
-
-    for group in body_groups:
-        clique(group)
-    if int(getattr(m, "neq", 0)):
-        eq_type, obj1, obj2 = _arr(m.eq_type), _arr(m.eq_obj1id), _arr(m.eq_obj2id)
-        objtype, site_bodyid, jnt_dofadr = _arr(m.eq_objtype), _arr(m.site_bodyid), _arr(m.jnt_dofadr)
-        for t, a, b, ot in zip(eq_type, obj1, obj2, objtype, strict=True):
-            if t in (EQ_CONNECT, EQ_WELD):
-                if ot == OBJ_SITE:
-                    a, b = site_bodyid[a], site_bodyid[b]
-                clique((a, max(int(b), 0)))
-            elif t in (EQ_FLEX, EQ_FLEXVERT, EQ_FLEXSTRAIN):
-                continue
-            elif t == EQ_JOINT:
-                dofs = [int(jnt_dofadr[a])] + ([int(jnt_dofadr[b])] if b >= 0 else [])
-                for x in dofs:
-                    adj[x].update(y for y in dofs if y != x)
-            else:
-                raise ValueError(f"equality type {int(t)} is not supported")
-    if int(getattr(m, "nflex", 0)):
-        raise ValueError("flex objects are not supported by this build")
-    pairs = _arr(getattr(m, "nxn_geom_pair_filtered", None))
-    if pairs.size:
-        geom_bodyid = _arr(m.geom_bodyid)
-        for g1, g2 in pairs.reshape(-1, 2):
-            clique((geom_bodyid[g1], geom_bodyid[g2]))
-    return adj
-
-
-def _symbolic(adj_e: list[set[int]]):
-    """Fill pattern and elimination levels of an L'DL in index order.  Returns
-    ``rowstruct`` (earlier columns of each row), ``colstruct`` (later rows of each
-    column) and ``levels`` (columns grouped by longest path in the elimination tree)."""
-    n = len(adj_e)
-    upper = [set(a for a in adj_e[k] if a > k) for k in range(n)]
-    for k in range(n):
-        nb = sorted(upper[k])
-        for i, a in enumerate(nb):
-            upper[a].update(nb[i + 1 :])
-    colstruct = [sorted(upper[k]) for k in range(n)]
-    rowstruct = [[] for _ in range(n)]
-    for k in range(n):
-        for i in colstruct[k]:
-            rowstruct[i].append(k)
-    parent = [c[0] if c else -1 for c in colstruct]
-    level = [0] * n
-    for k in range(n):
-        if parent[k] >= 0:
-            level[parent[k]] = max(level[parent[k]], level[k] + 1)
-    levels = [[] for _ in range(max(level) + 1)]
-    for k in range(n):
-        levels[level[k]].append(k)
-    return rowstruct, colstruct, levels
-
-
-def _team(nentries: int, maxterms: int, lanes: int) -> int:
-    """Lanes per entry of a level: the width minimising sweeps x (terms per lane +
-    reduction steps)."""
-    best, cost = 1, None
-    for T in (1, 2, 4, 8, 16, 32):
-        c = -(-nentries // (lanes // T)) * (-(-maxterms // T) + 2 * int(np.log2(T)))
-        if cost is None or c < cost:
-            best, cost = T, c
-    return best
-
-
-@dataclass
-class SparseHessianPlan:
-    nv: int
-    nv_pad: int
-    block: int
-    nslots: int
-    nterms: int
-    levels: int
-    density: float
-    path: str
-    tables: dict = field(repr=False, default_factory=dict)
-    colstruct: list = field(repr=False, default_factory=list)
-    level_cols: list = field(repr=False, default_factory=list)
-    handle: Any = field(repr=False, default=None)
-
-    @property
-    def nfac(self) -> int:
-        return self.nslots - self.nv
-
-
-def build_tables(nv: int, nv_pad: int, adj: list[set[int]], M_rowi, M_colind, block: int, path: str = "fused") -> SparseHessianPlan:
-    """The plan (tables only, no device state) of a dof adjacency."""
-    orig = [nv - 1 - e for e in range(nv)]
-    adj_e = [set(nv - 1 - a for a in adj[orig[e]]) for e in range(nv)]
-    rowstruct, colstruct, levels = _symbolic(adj_e)
-    n = nv
-    slot = {}
-    for i in range(n):
-        for k in rowstruct[i]:
-            slot[i, k] = len(slot)
-        slot[i, i] = len(slot)
-    nfac = len(slot)
-    for k in range(n):
-        slot[n, k] = len(slot)
-    nslots = len(slot)
-    if nslots >= 65536 or nfac + n > nv_pad * nv_pad:
-        raise ValueError("sparse Hessian factor does not fit the packed layout")
-    rs = [set(r) for r in rowstruct]
-    lvl_ptr, lvl_team, ent_slot, ent_col, run_ptr, run_ab, run_kl = [0], [], [], [], [0], [], []
-    nterms = 0
-    for cols in levels:
-        entries = []
-        for j in cols:
-            for i in [j, *colstruct[j], n]:
-                ks = sorted(rs[j]) if i in (j, n) else sorted(rs[j] & rs[i])
-                runs = []
-                for k in ks:
-                    last = runs[-1] if runs else None
-                    if last and k == last[2] + last[3] and slot[i, k] == last[0] + last[3] and slot[j, k] == last[1] + last[3]:
-                        last[3] += 1
-                    else:
-                        runs.append([slot[i, k], slot[j, k], k, 1])
-                entries.append((slot[i, j], j if i == j else -1, runs, len(ks)))
-        entries.sort(key=lambda e: -e[3])  # stable: longest entries first
-        for s, c, runs, nt in entries:
-            ent_slot.append(s)
-            ent_col.append(c)
-            for a, b, k, ln in runs:
-                run_ab.append(a | (b << 16))
-                run_kl.append(k | (ln << 16))
-            run_ptr.append(len(run_ab))
-            nterms += nt
-        lvl_ptr.append(len(ent_slot))
-        lvl_team.append(_team(len(entries), max(e[3] for e in entries), block))
-    by_slot = sorted(((s, ij) for ij, s in slot.items() if s < nfac))
-    gat = [min(orig[i], orig[j]) * nv_pad + max(orig[i], orig[j]) for _, (i, j) in by_slot]
-    f_lvl, f_row = [0], []
-    for cols in levels:
-        f_row += cols
-        f_lvl.append(len(f_row))
-    row_start = [slot[j, rowstruct[j][0]] if rowstruct[j] else slot[j, j] for j in range(n)]
-    rk_ptr, rk = [0], []
-    for j in range(n):
-        rk += rowstruct[j]
-        rk_ptr.append(len(rk))
-    b_lvl, b_slot, b_src, b_dst = [0], [], [], []
-    for cols in reversed(levels):
-        for i in cols:
-            for j in rowstruct[i]:
-                b_slot.append(slot[i, j])
-                b_src.append(i)
-                b_dst.append(j)
-        b_lvl.append(len(b_slot))
-    for a in (lvl_ptr, ent_slot, run_ptr, f_lvl, f_row, row_start, rk_ptr, rk, b_lvl, b_slot, b_src, b_dst):
-        if max(a, default=0) >= 65536:
-            raise ValueError("sparse Hessian tables exceed 16-bit indices")
-    pair = [-1] * (nv * nv)
-    for a in range(nv):
-        for b in range(a, nv):
-            i, j = nv - 1 - a, nv - 1 - b
-            if (i, j) in slot and slot[i, j] < nfac:
-                pair[a * nv + b] = slot[i, j]
-    csr = {}
-    for e, (r, c) in enumerate(zip(_arr(M_rowi), _arr(M_colind), strict=True)):
-        csr[min(int(r), int(c)), max(int(r), int(c))] = e
-    s_a, s_b, s_m = [], [], []
-    for _, (i, j) in by_slot:
-        a, b = sorted((orig[i], orig[j]))
-        s_a.append(a)
-        s_b.append(b)
-        s_m.append(csr.get((a, b), -1))
-    words = (nv + 31) // 32
-    pmask = []
-    for a in range(nv):
-        bits = [0] * words
-        for b in range(nv):
-            if b == a or pair[min(a, b) * nv + max(a, b)] >= 0:
-                bits[b // 32] |= 1 << (b % 32)
-        pmask += bits
-    if 2 * nfac + n >= nv_pad * nv_pad - 1:
-        raise ValueError("packed H and factor do not fit hfactor")
-    nw = max(block // 32, 1)
-    init_tile = ROWS_PER_TILE * nv + ROWS_PER_TILE if path == "fused" else 0
-    if 4 * (nslots + n + 2 * nw + init_tile) > MAX_SHARED_BYTES:
-        raise ValueError("the factor does not fit the block's shared memory")
-    i32 = lambda v: np.asarray(v if len(v) else [0], np.int32)  # noqa: E731
-    tables = {
-        "SH_LP": i32(lvl_ptr), "SH_LT": i32(lvl_team), "SH_ES": i32(ent_slot), "SH_EC": i32(ent_col),
-        "SH_RP": i32(run_ptr), "SH_RAB": np.asarray(run_ab if run_ab else [0], np.uint32).view(np.int32),
-        "SH_RKL": np.asarray(run_kl if run_kl else [0], np.uint32).view(np.int32), "SH_ORIG": i32(orig),
-        "SH_BL": i32(b_lvl), "SH_BS": i32(b_slot), "SH_BI": i32(b_src), "SH_BJ": i32(b_dst), "SH_PAIR": i32(pair),
-        "SH_FL": i32(f_lvl), "SH_FR": i32(f_row), "SH_RS": i32(row_start), "SH_RKP": i32(rk_ptr), "SH_RK": i32(rk),
-        "SH_PM": np.asarray(pmask, np.uint32).view(np.int32), "SH_SA": i32(s_a), "SH_SB": i32(s_b), "SH_SM": i32(s_m),
-        "SH_GAT": i32(gat),
-    }  # fmt: skip
-    return SparseHessianPlan(
-        nv, nv_pad, block, nslots, nterms, len(levels), nfac / (nv * (nv + 1) / 2), path, tables, colstruct, levels
-    )
-
-
-def _rowi(m) -> np.ndarray:
-    if getattr(m, "M_hinit_i", None) is not None:
-        return _arr(m.M_hinit_i)
-    return np.repeat(np.arange(int(m.nv)), _arr(m.M_rownnz))
-
-
-class _DevicePlan:
-    """Owns the ``im_sparse_plan`` of a table set on the current device."""
-
-    ORDER = ("SH_LP", "SH_LT", "SH_ES", "SH_EC", "SH_RP", "SH_RAB", "SH_RKL", "SH_ORIG", "SH_BL", "SH_BS", "SH_BI",
-             "SH_BJ", "SH_PM", "SH_SA", "SH_SB", "SH_SM", "SH_PAIR", "SH_FL", "SH_FR", "SH_RS", "SH_RKP",
-             "SH_RK")  # fmt: skip
-
-    def __init__(self, plan: SparseHessianPlan):
-        arrays = [np.ascontiguousarray(plan.tables[k], np.int32) for k in self.ORDER]
-        ptrs = (C.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
-        sizes = (C.c_int * len(arrays))(*[a.size for a in arrays])
+    def __init__(self, m: Any):
+        self.nv = int(m.nv)
         handle = C.c_void_p()
-        status = _lib.lib().im_sparse_plan_create(
-            plan.nv, plan.nv_pad, plan.block, plan.nslots, plan.levels, len(arrays), ptrs, sizes, C.byref(handle)
+        arrays = [_host(getattr(m, k)) for k in ("dof_parentid", "body_parentid", "body_dofadr", "body_dofnum")]
+        status = _lib.lib().im_dof_pattern_create(
+            self.nv, arrays[0].ctypes.data, int(arrays[1].size), *[a.ctypes.data for a in arrays[1:]], C.byref(handle)
         )
-        _lib.check(status, "im_sparse_plan_create")
+        _lib.check(status, "im_dof_pattern_create")
         self.ptr = handle
+        self._dense = None
+
+    def __del__(self):
+        ptr, self.ptr = getattr(self, "ptr", None), None
+        if ptr:
+            try:
+                _lib.lib().im_dof_pattern_destroy(ptr)
+            except Exception:
+                pass
+
+    def couple_bodies(self, bodies: Iterable[int]) -> None:
+        ids = np.fromiter((int(b) for b in bodies), np.int32)
+        self._dense = None
+        _lib.check(_lib.lib().im_dof_pattern_couple_bodies(self.ptr, ids.ctypes.data, int(ids.size)), "im_dof_pattern_couple_bodies")
+
+    def couple_dofs(self, dofs: Iterable[int]) -> None:
+        ids = np.fromiter((int(d) for d in dofs), np.int32)
+        self._dense = None
+        _lib.check(_lib.lib().im_dof_pattern_couple_dofs(self.ptr, ids.ctypes.data, int(ids.size)), "im_dof_pattern_couple_dofs")
+
+    def dense(self) -> np.ndarray:
+        """(nv, nv) bool, True where two different dofs couple."""
+        if self._dense is None:
+            out = np.zeros((self.nv, self.nv), np.uint8)
+            _lib.check(_lib.lib().im_dof_pattern_get(self.ptr, out.ctypes.data), "im_dof_pattern_get")
+            self._dense = out.astype(bool)
+        return self._dense
+
+    def __len__(self) -> int:
+        return self.nv
+
+    def __getitem__(self, dof: int) -> set[int]:
+        return set(np.flatnonzero(self.dense()[dof]).tolist())
+
+    def __iter__(self) -> Iterator[set[int]]:
+        return (self[d] for d in range(self.nv))
+
+
+def _equality_sources(m: Any):
+    """(kind, ids) per equality constraint: the two bodies a connect / weld ties together (a
+    missing second object is the world), or the dofs a joint equality ties (:90-109)."""
+    kinds = _host(m.eq_type)
+    first, second, objtype = _host(m.eq_obj1id), _host(m.eq_obj2id), _host(m.eq_objtype)
+    site_body, joint_dof = _host(getattr(m, "site_bodyid", None)), _host(getattr(m, "jnt_dofadr", None))
+    if not (kinds.size == first.size == second.size == objtype.size):
+        raise ValueError("equality arrays differ in length")
+    for q in range(kinds.size):
+        kind, a, b = int(kinds[q]), int(first[q]), int(second[q])
+        if kind in (EQ_FLEX, EQ_FLEXVERT, EQ_FLEXSTRAIN):
+            continue  # these rows stay inside the flex couplings
+        if kind == EQ_JOINT:
+            yield "dofs", [int(joint_dof[a])] + ([int(joint_dof[b])] if b >= 0 else [])
+        elif kind in (EQ_CONNECT, EQ_WELD):
+            if int(objtype[q]) == OBJ_SITE:
+                a, b = int(site_body[a]), int(site_body[b])
+            yield "bodies", (a, max(b, 0))
+        else:
+            raise ValueError(f"equality type {kind} is not supported")
+
+
+def _flex_sources(m: Any):
+    """Body sets one flex row can couple (:121-170): the vertex bodies of an element (or all
+    nodes of an interpolated flex), an element together with the body of a geom it may touch,
+    and two flexes that may collide (a flex with itself when it self-collides) as a whole."""
+    nflex = int(m.nflex)
+    vert_body, node_body = _host(m.flex_vertbodyid), _host(getattr(m, "flex_nodebodyid", None))
+    vertadr, vertnum = _host(m.flex_vertadr), _host(m.flex_vertnum)
+    elemnum, dataadr, dim = _host(m.flex_elemnum), _host(m.flex_elemdataadr), _host(m.flex_dim)
+    elem, interp = _host(m.flex_elem), _host(m.flex_interp)
+    nodeadr, nodenum = _host(getattr(m, "flex_nodeadr", None)), _host(getattr(m, "flex_nodenum", None))
+    whole: list[tuple[int, ...]] = []  # every body of flex f
+    pieces: list[list[tuple[int, ...]]] = []  # distinct element body sets of flex f
+    for f in range(nflex):
+        if interp[f]:
+            nodes = tuple(int(b) for b in node_body[nodeadr[f] : nodeadr[f] + nodenum[f]])
+            whole.append(nodes)
+            pieces.append([nodes] if elemnum[f] else [])
+            yield nodes
+            continue
+        mine = vert_body[vertadr[f] : vertadr[f] + vertnum[f]]
+        whole.append(tuple(int(b) for b in mine))
+        corners = elem[dataadr[f] : dataadr[f] + int(elemnum[f]) * (int(dim[f]) + 1)].reshape(int(elemnum[f]), int(dim[f]) + 1)
+        distinct = list(dict.fromkeys(tuple(int(b) for b in mine[row]) for row in corners))
+        pieces.append(distinct)
+        yield from distinct
+    contype, conaff = _host(m.flex_contype), _host(m.flex_conaffinity)
+    gtype, gaff, geom_body = _host(m.geom_contype), _host(m.geom_conaffinity), _host(m.geom_bodyid)
+    for f in range(nflex):
+        touching = np.flatnonzero((contype[f] & gaff[: int(m.ngeom)]) | (gtype[: int(m.ngeom)] & conaff[f]))
+        for body in dict.fromkeys(int(geom_body[g]) for g in touching):
+            for piece in pieces[f]:
+                yield (*piece, body)
+    selfcollide = _host(m.flex_selfcollide)
+    for f in range(nflex):
+        for h in range(f, nflex):
+            if ((contype[f] & conaff[h]) or (contype[h] & conaff[f])) and (f != h or selfcollide[f]):
+                yield whole[f] + whole[h]
+
+
+def hessian_pattern(m: Any, body_groups: Sequence[Sequence[int]]) -> DofPattern:
+    """Upper bound of H's off-diagonal pattern (dof adjacency, MuJoCo dof order): tree
+    ancestry, then one clique per declared body group, equality constraint, flex coupling and
+    native collision candidate (:62-118)."""
+    pattern = DofPattern(m)
+    for group in body_groups:
+        pattern.couple_bodies(group)
+    if int(getattr(m, "neq", 0)):
+        for kind, ids in _equality_sources(m):
+            (pattern.couple_dofs if kind == "dofs" else pattern.couple_bodies)(ids)
+    if int(getattr(m, "nflex", 0)):
+        for bodies in _flex_sources(m):
+            pattern.couple_bodies(bodies)
+    pairs = _host(getattr(m, "nxn_geom_pair_filtered", None)).reshape(-1, 2)
+    if pairs.size:
+        geom_body = _host(m.geom_bodyid)
+        for b1, b2 in dict.fromkeys(map(tuple, geom_body[pairs].tolist())):
+            pattern.couple_bodies((b1, b2))
+    return pattern
+
+
+class SparseHessianPlan:
+    """The reference's ``SparseHessianPlan`` (:38-50) over an ``im_sparse_plan`` handle; the
+    generated-source fields are replaced by the handle, ``tables`` reads the SH_* arrays back."""
+
+    def __init__(self, ptr, on_device: bool):
+        self.ptr = ptr
+        info = _lib.SparsePlanInfo()
+        _lib.check(_lib.lib().im_sparse_plan_get_info(ptr, C.byref(info)), "im_sparse_plan_get_info")
+        self.nv, self.nv_pad, self.block = int(info.nv), int(info.nv_pad), int(info.block)
+        self.nslots, self.nterms, self.levels = int(info.nslots), int(info.nterms), int(info.nlevels)
+        self.nfac = int(info.nfac)
+        self.density = float(info.density)
+        self.path = "fused" if info.path == PATHS["fused"] else "nonfused"
+        self.device_ready = bool(info.device_ready)
+        self.handle = self if (on_device and self.device_ready) else None
+        self._tables = None
 
     def __del__(self):
         ptr, self.ptr = getattr(self, "ptr", None), None
@@ -299,16 +206,74 @@ class _DevicePlan:
             except Exception:
                 pass
 
+    def __repr__(self) -> str:
+        return (f"SparseHessianPlan(nv={self.nv}, nv_pad={self.nv_pad}, block={self.block}, nslots={self.nslots}, "
+                f"nterms={self.nterms}, levels={self.levels}, density={self.density:.3f}, path={self.path!r})")  # fmt: skip
 
-def build_plan(m: Any, body_groups: Sequence[Sequence[int]], block: int, path: str = "fused", *, device=None) -> SparseHessianPlan:
-    """Tables of the model's pattern; with ``device`` also the device-side plan."""
-    plan = build_tables(int(m.nv), int(m.nv_pad), hessian_pattern(m, body_groups), _rowi(m), m.M_colind, block, path)
-    if device is not None:
+    @property
+    def tables(self) -> dict[str, np.ndarray]:
+        if self._tables is None:
+            lib, out = _lib.lib(), {}
+            for tid, name in enumerate(_lib.SPARSE_TABLES):
+                arr = np.zeros(lib.im_sparse_plan_table_size(self.ptr, tid), np.int32)
+                _lib.check(lib.im_sparse_plan_get_table(self.ptr, tid, arr.ctypes.data, int(arr.size)), "im_sparse_plan_get_table")
+                out[name] = arr
+            self._tables = out
+        return self._tables
+
+    def _structure(self):
+        ptr, idx, lvl = np.zeros(self.nv + 1, np.int32), np.zeros(max(self.nfac - self.nv, 1), np.int32), np.zeros(self.nv, np.int32)
+        _lib.check(_lib.lib().im_sparse_plan_get_structure(self.ptr, ptr.ctypes.data, idx.ctypes.data, lvl.ctypes.data), "im_sparse_plan_get_structure")
+        return ptr, idx, lvl
+
+    @property
+    def colstruct(self) -> list[list[int]]:
+        """Fill pattern: the later rows of every column of the factor, elimination indices."""
+        ptr, idx, _ = self._structure()
+        return [idx[ptr[k] : ptr[k + 1]].tolist() for k in range(self.nv)]
+
+    @property
+    def level_cols(self) -> list[list[int]]:
+        _, _, lvl = self._structure()
+        return [np.flatnonzero(lvl == q).tolist() for q in range(self.levels)]
+
+
+def _rowi(m) -> np.ndarray:
+    if getattr(m, "M_hinit_i", None) is not None:
+        return _host(m.M_hinit_i)
+    return np.repeat(np.arange(int(m.nv), dtype=np.int32), _host(m.M_rownnz))
+
+
+def plan_from_pattern(pattern: DofPattern, nv_pad: int, M_rowi, M_colind, block: int, path: str = "fused", *, device=None) -> SparseHessianPlan:
+    """The plan of a dof pattern; ``device=None`` plans on the host only (no GPU needed).
+    Raises ``ValueError`` with the reference's messages when the factor exceeds its limits."""
+    rowi, colind = _host(M_rowi), _host(M_colind)
+    if rowi.size != colind.size:
+        raise ValueError("M_rowi and M_colind differ in length")
+    handle, refused = C.c_void_p(), C.c_int(0)
+
+    def call():
+        return _lib.lib().im_sparse_plan_build(
+            pattern.ptr, int(nv_pad), int(block), PATHS[path], rowi.ctypes.data, colind.ctypes.data, int(rowi.size),
+            int(device is None), C.byref(refused), C.byref(handle),
+        )  # fmt: skip
+
+    if device is None:
+        status = call()
+    else:
         import torch
 
         with torch.cuda.device(torch.device(device)):
-            plan.handle = _DevicePlan(plan)
-    return plan
+            status = call()
+    _lib.check(status, "im_sparse_plan_build")
+    if not handle:
+        raise ValueError(REFUSALS[refused.value])
+    return SparseHessianPlan(handle, device is not None)
+
+
+def build_plan(m: Any, body_groups: Sequence[Sequence[int]], block: int, path: str = "fused", *, device=None) -> SparseHessianPlan:
+    """``build_plan`` of the reference (:229-702) for a model."""
+    return plan_from_pattern(hessian_pattern(m, body_groups), int(m.nv_pad), _rowi(m), m.M_colind, block, path, device=device)
 
 
 def block_width(nv_pad: int) -> int:
@@ -316,24 +281,43 @@ def block_width(nv_pad: int) -> int:
     return 64 if nv_pad >= 64 else 32
 
 
+def _on_gpu(m: Any, device) -> bool:
+    arr = getattr(m, "body_parentid", None)
+    dev = None if isinstance(arr, np.ndarray) else getattr(arr, "device", None)  # host-side NumPy copies say nothing
+    if dev is not None:
+        return bool(getattr(dev, "is_cuda", False) or getattr(dev, "type", "") == "cuda")
+    return True if device is None else str(device).startswith("cuda")
+
+
 def plan_for_model(m: Any, ctx: Any, body_groups, block: int, *, compact: bool = False, fused_runtime: bool = True, device="cuda"):
-    """The plan when the model qualifies, else ``None`` and the reason (same order of
-    checks and same messages as the reference, sparse_hessian.py:705-758).  Only the
-    fused path exists in this build."""
+    """The plan when the model qualifies, else ``None`` and the reason: the reference's checks in
+    the reference's order with its messages (:705-758).  ``device=None`` plans on the host and
+    skips nothing but the upload; a model whose arrays say where they live is judged by that."""
+    from . import newton_fusion
+
+    nv = int(m.nv)
     if body_groups is None:
         return None, "a custom contact producer did not declare its body groups"
-    if int(m.nv) < MIN_NV:
-        return None, f"nv {int(m.nv)} < {MIN_NV}"
+    if not _on_gpu(m, device):
+        return None, "fused Newton not eligible (CPU)"
+    if nv < MIN_NV:
+        return None, f"nv {nv} < {MIN_NV}"
     if int(getattr(m, "ntendon", 0)) and (
-        int(_arr(getattr(m, "tendon_limited_adr", None)).shape[0]) or bool((_arr(m.tendon_frictionloss) > 0).any())
+        int(_host(getattr(m, "tendon_limited_adr", None)).shape[0]) or bool((_host(m.tendon_frictionloss, np.float32) > 0).any())
     ):
         return None, "tendon limit or frictionloss rows"
-    if not fused_runtime or compact or int(m.nv) > 79:
+    if fused_runtime and newton_fusion.eligible(m, ctx, compact=compact, device=device):
+        if int(getattr(m, "nflex", 0)):
+            return None, "flex objects on the fused path"
+        path, width = "fused", block
+    elif newton_fusion.upstream_newton_structure(m, ctx, compact=compact):
+        if nv < NONFUSED_MIN_NV:
+            return None, f"upstream iteration with nv {nv} < {NONFUSED_MIN_NV}"
+        path, width = "nonfused", 64 if nv <= 96 else 128
+    else:
         return None, "Newton solver structure not supported"
-    if int(getattr(m, "nflex", 0)):
-        return None, "flex objects on the fused path"
     try:
-        plan = build_plan(m, body_groups, block, "fused", device=device)
+        plan = build_plan(m, body_groups, width, path, device=device)
     except ValueError as exc:
         return None, str(exc)
     if plan.density > MAX_DENSITY:
@@ -341,26 +325,33 @@ def plan_for_model(m: Any, ctx: Any, body_groups, block: int, *, compact: bool =
     return plan, "enabled"
 
 
-def violation_counter(hfactor, plan: SparseHessianPlan):
+def violation_counter(hfactor, plan):
     """Per-world view of the pattern-violation counter, the last element of each world's
-    ``hfactor``; accumulates until it is zeroed."""
+    ``hfactor``; accumulates until it is zeroed (:786-796)."""
     if plan.path != "fused":
         raise ValueError("the violation counter exists on the fused path only")
     last = plan.nv_pad - 1
     return hfactor[:, last, last]
 
 
-def violations(hfactor, plan: SparseHessianPlan) -> np.ndarray:
+def violations(hfactor, plan) -> np.ndarray:
     return violation_counter(hfactor, plan).cpu().numpy()
+
+
+def _device_plan(plan: SparseHessianPlan):
+    if plan.handle is None:
+        raise RuntimeError("the plan has no device state (build it with device=...)")
+    return plan.ptr
 
 
 def init_factor_kernel(plan: SparseHessianPlan):
     """Launcher of the initial ``H = M + J'DJ`` on the pattern, factor and solve; fills
     ``hfactor``, ``search = -H^-1 grad``, ``search_dot`` and ``decrement``.  Called with
     the reference kernel's arguments
-    ``(done, nefc, J, D, state, M, grad3, hfactor, search3, search_dot, decrement)``."""
-    if plan.handle is None:
-        raise RuntimeError("the plan has no device state (build it with device=...)")
+    ``(done, nefc, J, D, state, M, grad3, hfactor, search3, search_dot, decrement)`` (:804-846)."""
+    ptr = _device_plan(plan)
+    if plan.path != "fused":
+        raise ValueError("the initial assemble + factor exists on the fused path only")
 
     def launch(done, nefc, J, D, state, M, grad, hfactor, search, search_dot, decrement, *, quad: int = QUADRATIC):
         import torch
@@ -368,18 +359,22 @@ def init_factor_kernel(plan: SparseHessianPlan):
         nworld, njmax, nv = J.shape
         if nv != plan.nv or tuple(hfactor.shape) != (nworld, plan.nv_pad, plan.nv_pad):
             raise ValueError("array shapes do not match the plan")
+        if tuple(D.shape) != (nworld, njmax) or tuple(state.shape) != (nworld, njmax) or nefc.numel() != nworld:
+            raise ValueError("D, state and nefc do not match J")
+        if M.shape[0] != nworld or grad.shape[0] != nworld or grad[0].numel() < nv or search[0].numel() != nv:
+            raise ValueError("M, grad and search do not match J")
         for t in (J, D, state, M, grad, hfactor, search, search_dot, decrement, nefc):
-            if not t.is_cuda or not t.is_contiguous():
-                raise ValueError("arrays must be contiguous CUDA tensors")
+            if not t.is_cuda or not t.is_contiguous() or t.device != J.device:
+                raise ValueError("arrays must be contiguous CUDA tensors on one device")
         done_ptr = None
         if done is not None:
-            if done.dtype not in (torch.bool, torch.uint8):
-                raise TypeError("done must be a bool tensor")
+            if done.dtype not in (torch.bool, torch.uint8) or done.numel() != nworld:
+                raise TypeError("done must be a bool tensor with one element per world")
             done_ptr = done.data_ptr()
         with torch.cuda.device(J.device):
             status = _lib.lib().im_sparse_init_factor(
-                plan.handle.ptr, done_ptr, nefc.data_ptr(), J.data_ptr(), int(njmax), D.data_ptr(), state.data_ptr(),
-                int(quad), M.data_ptr(), int(M.shape[1]), grad.data_ptr(), int(grad.shape[1]), hfactor.data_ptr(),
+                ptr, done_ptr, nefc.data_ptr(), J.data_ptr(), int(njmax), D.data_ptr(), state.data_ptr(),
+                int(quad), M.data_ptr(), int(M.shape[1]), grad.data_ptr(), int(grad[0].numel()), hfactor.data_ptr(),
                 search.data_ptr(), search_dot.data_ptr(), decrement.data_ptr(), int(nworld),
                 int(torch.cuda.current_stream(J.device).cuda_stream),
             )  # fmt: skip
@@ -388,13 +383,16 @@ def init_factor_kernel(plan: SparseHessianPlan):
     return launch
 
 
-def pattern_misses(h: np.ndarray, plan_adj: list[set[int]], tol: float = 0.0) -> int:
+def pattern_misses(h: np.ndarray, plan_adj, tol: float = 0.0) -> int:
     """Nonzero upper-triangle entries of dense Hessians ``h`` (nworld, nv_pad, nv_pad)
-    outside a dof adjacency."""
-    nv = len(plan_adj)
-    mask = np.eye(nv, dtype=bool)
-    for a in range(nv):
-        for b in plan_adj[a]:
-            mask[a, b] = True
-    off = np.triu(np.ones((nv, nv), bool)) & ~mask
-    return int((np.abs(h[:, :nv, :nv][:, off]) > tol).sum())
+    outside a dof adjacency (:946-957)."""
+    if isinstance(plan_adj, DofPattern):
+        allowed = plan_adj.dense().copy()
+    else:
+        allowed = np.zeros((len(plan_adj), len(plan_adj)), bool)
+        for a, neighbours in enumerate(plan_adj):
+            allowed[a, list(neighbours)] = True
+    nv = allowed.shape[0]
+    np.fill_diagonal(allowed, True)
+    outside = np.triu(~allowed)
+    return int((np.abs(h[:, :nv, :nv][:, outside]) > tol).sum())

@@ -197,6 +197,22 @@ def _check_rows(*tensors) -> None:
             raise ValueError("tree_factor_solve needs rows of contiguous floats")
 
 
+def _check_against_plan(scratch, M, x, y, others=()) -> int:
+    """Every array against the plan's sizes and against each other before a pointer leaves
+    Python: the C ABI sees addresses and strides only.  Returns the world count."""
+    info = scratch.kernel.info()
+    nworld = int(M.shape[0])
+    if M.shape[1] < info.nM or x.shape[1] < info.nv or y.shape[1] < info.nv:
+        raise ValueError(f"rows shorter than the plan's sizes (nM {info.nM}, nv {info.nv})")
+    for t in (x, y, *others):
+        if t is not None and t.shape[0] != nworld:
+            raise ValueError(f"{t.shape[0]} worlds where M has {nworld}")
+    for t in (x, y, *others):
+        if t is not None and t.device != M.device:
+            raise ValueError("all arrays must live on one device")
+    return nworld
+
+
 def tree_factor_solve(scratch: TreeFactorSolveScratch, M, x, y) -> None:
     """x = M^-1 y for an M in the model's CSR layout (argument order of the
     reference: scratch, M, x, y)."""
@@ -206,7 +222,7 @@ def tree_factor_solve(scratch: TreeFactorSolveScratch, M, x, y) -> None:
     for t in (M, x, y):
         if t.dtype != torch.float32 or not t.is_cuda:
             raise TypeError("tree_factor_solve needs float32 CUDA tensors")
-    nworld = M.shape[0]
+    nworld = _check_against_plan(scratch, M, x, y)
     with torch.cuda.device(M.device):
         status = _lib.lib().im_tree_factor_solve(
             scratch.kernel.ptr, M.data_ptr(), M.stride(0), y.data_ptr(), y.stride(0), x.data_ptr(), x.stride(0),
@@ -235,7 +251,12 @@ def assemble_tree_factor_solve(
     for t in (M, J, D, grad, x):
         if t.dtype != torch.float32 or not t.is_cuda:
             raise TypeError("assemble_tree_factor_solve needs float32 CUDA tensors")
-    nworld, njmax, nv = J.shape
+    njmax, nv = int(J.shape[1]), int(J.shape[2])
+    nworld = _check_against_plan(scratch, M, x, grad, (J, D, state, nefc, H_out))
+    if nv != scratch.kernel.info().nv or njmax < 1:
+        raise ValueError("J must be (nworld, njmax >= 1, nv) with the plan's nv")
+    if tuple(D.shape) != (nworld, njmax) or tuple(state.shape) != (nworld, njmax) or (nefc is not None and nefc.numel() != nworld):
+        raise ValueError("D and state must be (nworld, njmax), nefc (nworld,)")
     if H_out is not None and (not H_out.is_contiguous() or H_out.shape != (nworld, scratch.kernel.info().nM)):
         raise ValueError("H_out must be a contiguous (nworld, nM) tensor")
     with torch.cuda.device(M.device):

@@ -319,6 +319,10 @@ def model_from_parents(parent, joints: list[list[int]] | None = None):
         body_dofnum=np.asarray(body_dofnum, np.int32), M_rowadr=rowadr, M_rownnz=rownnz, M_colind=colind,
         M_hinit_i=np.repeat(np.arange(nv), rownnz).astype(np.int32), neq=0, nflex=0, ntendon=0,
         nxn_geom_pair_filtered=np.zeros((0, 2), np.int32), geom_bodyid=np.zeros(0, np.int32),
+        # what the fused Newton's eligibility test reads: Newton solver (mjSOL_NEWTON = 2), pyramidal cone
+        # (mjCONE_PYRAMIDAL = 0), implicitfast integrator (3), dense Jacobian, 32-lane line search
+        opt=SimpleNamespace(solver=2, cone=0, integrator=3, iterations=100), is_sparse=False,
+        block_dim=SimpleNamespace(linesearch_iterative=32),
     )  # fmt: skip
 
 

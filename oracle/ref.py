@@ -243,6 +243,14 @@ def run_tables64(T, nv, nslots, H, g):
     return x
 
 
+def sparse_plan(m, body_groups, block, path="fused"):
+    """The oracle's own plan of a model (planner.sparse_pattern + planner.sparse_tables): what
+    ``sparse_init_factor`` / ``sparse_update_factor`` execute, independent of the product's planner."""
+    from . import planner
+
+    return planner.sparse_tables(int(m.nv), int(m.nv_pad), planner.sparse_pattern(m, body_groups), m.M_hinit_i, m.M_colind, block, path)
+
+
 def sparse_init_factor(plan, nefc, J, D, state, M, grad, hfactor=None, done=None, quad=1):
     """fp32 lane-by-lane restatement of the initial assemble + factor + solve kernel."""
     J, D, M, grad = _f(J), _f(D), _f(M), _f(grad)

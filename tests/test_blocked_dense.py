@@ -89,7 +89,7 @@ def test_gpu_blocked_factor_solve_bitwise(device, name, B, nworld):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,nworld", [("g1", 40), ("stress", 24)])
+@pytest.mark.parametrize("name,nworld", [("ant", 50), ("humanoid", 50), ("g1", 40), ("snu", 30), ("stress", 24)])
 def test_gpu_dense_hessian_mfma(device, name, nworld):
     import torch
 
@@ -131,3 +131,20 @@ def test_gpu_wavefront_per_world_kernel_for_small_tiles_agrees():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
     assert out.returncode == 0 and "simple kernel ok" in out.stdout, out.stderr[-2000:]
+
+
+def test_dense_hessian_staging_indices_stay_inside_a_row():
+    """The staging step of the dense J'DJ kernel writes row r of a 32-row chunk at
+    Js[r * nvr + c] for the columns c = lane and lane + 64 that lie below nvr = the dofs rounded
+    up to 32 (csrc/blocked_kernels.hip, stage()): replayed here for every supported width, every
+    element of the chunk is written exactly once and nothing outside it."""
+    for nv in (1, 14, 27, 32, 33, 35, 56, 64, 65, 96, 128):
+        nvr = (nv + 31) // 32 * 32
+        hits = np.zeros(32 * nvr + 32, int)
+        for wave in range(4):
+            for lane in range(64):
+                for i in range(8):
+                    for c in (lane, lane + 64):
+                        if c < nvr:
+                            hits[(wave * 8 + i) * nvr + c] += 1
+        assert (hits[: 32 * nvr] == 1).all() and (hits[32 * nvr :] == 0).all(), nv

@@ -176,3 +176,15 @@ def test_newton_entry_points_check_their_arguments_before_any_launch():
     assert lib.im_newton_converged(one, one, one, one, one, 1, one, 1, 27, 5, 0, one, None, None, None, 4, None) == _lib.IM_ERR_ARG
     assert lib.im_newton_init_empty_worlds(one, one, 26, one, one, one, one, 27, 27, 4, None) == _lib.IM_ERR_STRIDE
     assert lib.im_qfrc_constraint_from_grad(one, one, 27, one, 27, one, 27, None, one, 27, 27, 4, None) == _lib.IM_ERR_ARG
+
+
+def test_entry_points_that_clamp_rows_refuse_an_empty_row_range():
+    """The assembly kernels clamp a row index to njmax - 1 (every load is issued, the value
+    selected afterwards), so njmax = 0 is refused on the host instead of reading before the
+    arrays; likewise an empty entry list of the torque projection."""
+    lib = _lib.lib()
+    one = 16
+    assert lib.im_jtdj_mfma(one, one, 0, one, one, None, 1, one, 27, 32, 4, None) == _lib.IM_ERR_ARG
+    assert lib.im_muscle_project(one, 0, one, 4, one, one, one, 0, 4, 3, 0, one, 3, 2, None) == _lib.IM_ERR_ARG
+    assert lib.im_muscle_project(one, 0, one, 4, one, one, one, 0, 4, 0, 0, one, 3, 2, None) == _lib.IM_OK
+    assert lib.im_dense_update_factor(None, one, one, one, 8, one, 0, one, one, 1, one, 27, 32, 32, 27, 32, one, one, 27, one, one, 4, None) == _lib.IM_ERR_ARG

@@ -116,6 +116,7 @@ def test_sparse_factor_full_batch(device, name, nworld):
     m = synth.model_from_parents(synth.SHAPES[name].parents)
     plan, reason = S.plan_for_model(m, None, [], S.block_width(m.nv_pad), device=device)
     assert plan is not None, reason
+    oplan = R.sparse_plan(m, [], plan.block)
     b = synth.make_batch(dataclasses.replace(synth.SHAPES[name], iterations=2))  # a second state to move to
     assert b.nworld == nworld
     nv = m.nv
@@ -126,7 +127,7 @@ def test_sparse_factor_full_batch(device, name, nworld):
     tJ, tD = t(b.J), t(b.D)
     S.init_factor_kernel(plan)(None, t(b.nefc), tJ, tD, t(b.state[0]), t(b.M), t(b.grad)[:, :, None].contiguous(), hf, search, sdot, decr)
     torch.cuda.synchronize()
-    ref = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
+    ref = R.sparse_init_factor(oplan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
     n_used = 2 * plan.nfac + nv
     np.testing.assert_array_equal(hf.cpu().numpy().reshape(nworld, -1)[:, :n_used], ref[0].reshape(nworld, -1)[:, :n_used])
     np.testing.assert_array_equal(search.cpu().numpy()[:, :, 0], ref[1])
@@ -135,7 +136,7 @@ def test_sparse_factor_full_batch(device, name, nworld):
     assert not hf[:, -1, -1].any()  # nothing fell outside the declared pattern
     # the per-iteration stage from there
     new, ids, changes, sc, done, grad = _changes(b, np.random.default_rng(5))
-    want = R.sparse_update_factor(plan, sc, changes, ids, b.J, b.D, new, grad, ref[0], done=done)
+    want = R.sparse_update_factor(oplan, sc, changes, ids, b.J, b.D, new, grad, ref[0], done=done)
     uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=device)
     search2 = torch.zeros((nworld, nv), device=device)
     NS.factor_factory(nv, m.nv_pad, plan)(tJ, tD, t(new), t(ids), t(changes), t(sc), t(done), t(grad), None, hf, search2, sdot, decr, uni)

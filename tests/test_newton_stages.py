@@ -8,6 +8,7 @@ import pytest
 from instantmimic_amd import synth
 from instantmimic_amd.mjw_kernels import newton_stages as NS
 from instantmimic_amd.mjw_kernels import sparse_hessian as S
+from oracle import planner as P
 from oracle import ref as R
 
 Q = synth.QUADRATIC
@@ -21,7 +22,7 @@ def _contact_case(nworld, seed):
     for g in groups:
         mask = np.zeros(nv, bool)
         for b in g:
-            mask[S._chain(b, m.body_parentid, m.body_dofadr, m.body_dofnum)] = True
+            mask[P.body_chain(b, m.body_parentid, m.body_dofadr, m.body_dofnum)] = True
         sup += [mask] * 6
     shape = synth.Shape("contact", tuple(int(p) for p in m.dof_parentid), 40, nworld, (0.5, 8.0), 0.02, (-4.0, 4.0),
                         0.6, 2, seed)  # fmt: skip
@@ -65,7 +66,7 @@ def test_oracle_sparse_stage_against_fp64():
     m, groups, b = _contact_case(36, 21)
     rng = np.random.default_rng(4)
     for block in (32, 64):
-        plan = S.build_tables(m.nv, m.nv_pad, S.hessian_pattern(m, groups), m.M_hinit_i, m.M_colind, block)
+        plan = R.sparse_plan(m, groups, block)
         hf0, *_ = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
         new, ids, changes, sc, done, grad = _changes(b, rng)
         hf, uni, search, sdot, decr = R.sparse_update_factor(plan, sc, changes, ids, b.J, b.D, new, grad, hf0, done=done)
@@ -189,14 +190,15 @@ def test_gpu_sparse_stage_bitwise(device, block):
     m, groups, b = _contact_case(150, 23)
     rng = np.random.default_rng(5)
     plan = S.build_plan(m, groups, block, device=device)
-    hf0, *_ = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
+    oplan = R.sparse_plan(m, groups, block)
+    hf0, *_ = R.sparse_init_factor(oplan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
     new, ids, changes, sc, done, grad = _changes(b, rng)
     # one update outside the declared pattern: a changed row coupling the two arms
     w_bad = int(np.flatnonzero(_live(sc, done) & (changes > 0))[0])
     r_bad = ids[w_bad, 0]
     b.J[w_bad, r_bad, :] = 0.0
     b.J[w_bad, r_bad, [18, 21]] = 1.0
-    want = R.sparse_update_factor(plan, sc, changes, ids, b.J, b.D, new, grad, hf0, done=done)
+    want = R.sparse_update_factor(oplan, sc, changes, ids, b.J, b.D, new, grad, hf0, done=done)
     nworld, nv = b.nworld, m.nv
     hf = _t(hf0, device)
     uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=device)
@@ -296,7 +298,8 @@ def test_gpu_changed_rows_feed_the_factor_stage(device):
     m, groups, b = _contact_case(150, 23)
     rng = np.random.default_rng(5)
     plan = S.build_plan(m, groups, 64, device=device)
-    hf0, *_ = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
+    oplan = R.sparse_plan(m, groups, 64)
+    hf0, *_ = R.sparse_init_factor(oplan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
     new, ids, changes, _, done, grad = _changes(b, rng)
     nworld, nv, njmax = b.nworld, m.nv, b.D.shape[1]
     ids_d = torch.zeros((nworld, njmax), dtype=torch.int32, device=device)
@@ -308,7 +311,7 @@ def test_gpu_changed_rows_feed_the_factor_stage(device):
     # a world whose states did not change at all is solve-only for the stage and skipped when its count is zero:
     # give every world at least the solve, as the reference's line search does through its own increments
     sc_np = np.maximum(sc.cpu().numpy(), 1).astype(np.int32)
-    want = R.sparse_update_factor(plan, sc_np, changes, ids, b.J, b.D, new, grad, hf0, done=done)
+    want = R.sparse_update_factor(oplan, sc_np, changes, ids, b.J, b.D, new, grad, hf0, done=done)
     hf = _t(hf0, device)
     uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=device)
     search = torch.zeros((nworld, nv), device=device)
@@ -335,8 +338,9 @@ def test_gpu_one_iteration_chained(device):
     m, groups, b = _contact_case(150, 23)
     rng = np.random.default_rng(15)
     plan = S.build_plan(m, groups, 64, device=device)
+    oplan = R.sparse_plan(m, groups, 64)
     nworld, nv, njmax = b.nworld, m.nv, b.D.shape[1]
-    hf0, search0, sdot0, decr0 = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
+    hf0, search0, sdot0, decr0 = R.sparse_init_factor(oplan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
     new, _, _, _, done, _ = _changes(b, rng)
     f = lambda *shape: rng.normal(size=shape).astype(np.float32)  # noqa: E731
     alpha = rng.uniform(0.1, 1, nworld).astype(np.float32)
@@ -349,7 +353,7 @@ def test_gpu_one_iteration_chained(device):
     q1, Ma1, ja1 = R.newton_advance(alpha, search0, mv, jv, qacc, Ma, jaref, nefc=b.nefc, done=done)
     ids, qc, sc = R.newton_changed_rows(b.state[0], new, quad=Q, nefc=b.nefc, done=done)
     qcf, grad, gd, de, gs, un = R.newton_gradient(b.J, force, smooth, Ma1, sc, alpha, gd0, decr0, sc0, nefc=b.nefc, done=done, block=64)
-    want = R.sparse_update_factor(plan, sc, qc, ids, b.J, b.D, new, grad, hf0, done=done)
+    want = R.sparse_update_factor(oplan, sc, qc, ids, b.J, b.D, new, grad, hf0, done=done)
     ran = (done == 0) & (sc != 0)  # the factor stage leaves the other worlds' decrement as the gradient step left it
     it, dn, _, _ = R.newton_converged(alpha, imp, gd, np.where(ran, want[4], de), tol, inertia, nv, 5, np.zeros(nworld, np.int32), done)
     # the same on the GPU

@@ -4,14 +4,43 @@ numeric kernel against the lane-by-lane oracle."""
 import numpy as np
 import pytest
 
+from types import SimpleNamespace
+
 from instantmimic_amd import synth
 from instantmimic_amd.mjw_kernels import sparse_hessian as S
+from oracle import planner as P
 from oracle import ref as R
 
 
-def _tables_plan(m, groups, block=None):
+def _tables_plan(m, groups, block=None, path="fused"):
+    """The product's plan (C++ planner through the C ABI), host only."""
     block = block or S.block_width(m.nv_pad)
-    return S.build_tables(m.nv, m.nv_pad, S.hessian_pattern(m, groups), m.M_hinit_i, m.M_colind, block)
+    return S.plan_from_pattern(S.hessian_pattern(m, groups), m.nv_pad, m.M_hinit_i, m.M_colind, block, path)
+
+
+def _oracle_plan(m, groups, block=None, path="fused"):
+    """The same plan from the oracle's restatement of the reference planner."""
+    block = block or S.block_width(m.nv_pad)
+    return P.sparse_tables(m.nv, m.nv_pad, P.sparse_pattern(m, groups), m.M_hinit_i, m.M_colind, block, path)
+
+
+def _assert_same_plan(got, exp, what=""):
+    assert (got.nslots, got.nfac, got.nterms, got.levels, got.path, got.block) == (exp.nslots, exp.nfac, exp.nterms, exp.levels, exp.path, exp.block), what
+    assert got.density == exp.density
+    assert got.colstruct == exp.colstruct and got.level_cols == exp.level_cols, what
+    assert set(got.tables) == set(exp.tables)
+    for name, table in exp.tables.items():
+        np.testing.assert_array_equal(got.tables[name], table, err_msg=f"{what} {name}")
+
+
+def _pattern_of_edges(n, edges):
+    """A pattern over n unrelated dofs (every dof a root) with the given couplings."""
+    m = SimpleNamespace(nv=n, dof_parentid=np.full(n, -1, np.int32), body_parentid=np.zeros(1, np.int32),
+                        body_dofadr=np.full(1, -1, np.int32), body_dofnum=np.zeros(1, np.int32))  # fmt: skip
+    pat = S.DofPattern(m)
+    for a, b in edges:
+        pat.couple_dofs((a, b))
+    return pat
 
 
 def test_symbolic_fill_contains_the_numeric_factor():
@@ -25,7 +54,12 @@ def test_symbolic_fill_contains_the_numeric_factor():
             if a != b:
                 adj[a].add(int(b))
                 adj[b].add(int(a))
-        rowstruct, colstruct, levels = S._symbolic(adj)
+        rowstruct, colstruct, levels = P.sparse_symbolic(adj)
+        # the product's symbolic factor of the same graph (adjacency given in elimination order:
+        # dof d = n - 1 - e), through the C ABI
+        pat = _pattern_of_edges(n, [(n - 1 - a, n - 1 - b) for a in range(n) for b in adj[a] if a < b])
+        plan = S.plan_from_pattern(pat, 64, [], [], 32)
+        assert plan.colstruct == colstruct and plan.level_cols == levels
         H = np.eye(n) * n
         for a in range(n):
             for b in adj[a]:
@@ -88,8 +122,9 @@ def test_tables_solve_h_without_a_race_inside_any_level():
                     H[a, b] = H[b, a] = rng.normal()
         H += np.diag(np.abs(H).sum(1) + 1.0 + rng.random(nv))
         g = rng.normal(size=nv)
-        plan = _tables_plan(m, groups, 64)
+        plan = _oracle_plan(m, groups, 64)
         x = R.run_tables64(plan.tables, nv, plan.nslots, H, g)
+        _assert_same_plan(_tables_plan(m, groups, 64), plan)
         assert plan.levels > 1
         np.testing.assert_allclose(x, np.linalg.solve(H, g), rtol=1e-10, atol=1e-12)
 
@@ -120,11 +155,133 @@ def test_expected_plans_of_the_benchmark_trees():
             assert col == sorted(anc)
 
 
+
+def _random_model(rng, nv):
+    """A random forest of joints (1-3 dofs each, 10 % roots) with bodies, plus the M CSR."""
+    parent, joints, d = [], [], 0
+    while d < nv:
+        k = min(int(rng.integers(1, 4)), nv - d)
+        p = -1 if (d == 0 or rng.random() < 0.1) else int(rng.integers(0, d))
+        parent += [p] + list(range(d, d + k - 1))
+        joints.append(list(range(d, d + k)))
+        d += k
+    return synth.model_from_parents(parent, joints)
+
+
+def test_planner_equals_the_oracle_table_for_table():
+    """The C++ bit-row planner against the oracle's set-based restatement of the reference
+    planner: every SH_* table, the fill pattern and the levels, on the benchmark trees, the
+    contact model's cases and 120 random models with random groups, equalities and pairs."""
+    for name, shape in synth.SHAPES.items():
+        m = synth.model_from_parents(shape.parents)
+        for path in ("fused", "nonfused"):
+            try:
+                exp = _oracle_plan(m, [], path=path)
+            except ValueError as exc:
+                with pytest.raises(ValueError, match=str(exc)):
+                    _tables_plan(m, [], path=path)
+                continue
+            _assert_same_plan(_tables_plan(m, [], path=path), exp, f"{name} {path}")
+    m, cases = _cases()
+    for groups in cases:
+        for block in (32, 64, 128):
+            for path in ("fused", "nonfused"):
+                _assert_same_plan(_tables_plan(m, groups, block, path), _oracle_plan(m, groups, block, path), f"contact {block} {path}")
+    rng = np.random.default_rng(17)
+    refused = 0
+    for trial in range(120):
+        nv = int(rng.integers(2, 90))
+        m = _random_model(rng, nv)
+        nbody = m.body_parentid.size
+        groups = [list(rng.integers(1, nbody, int(rng.integers(1, 4)))) for _ in range(int(rng.integers(0, 4)))]
+        if trial % 3 == 0 and nbody > 2:
+            m.neq = 3
+            m.eq_type = np.array([S.EQ_CONNECT, S.EQ_JOINT, S.EQ_WELD])
+            m.eq_obj1id = np.array([rng.integers(1, nbody), rng.integers(0, nbody - 1), rng.integers(0, 2)])
+            m.eq_obj2id = np.array([rng.integers(-1, nbody), rng.integers(-1, nbody - 1), rng.integers(0, 2)])
+            m.eq_objtype = np.array([1, 3, S.OBJ_SITE])
+            m.site_bodyid = rng.integers(0, nbody, 2)
+            m.jnt_dofadr = m.body_dofadr[1:]
+        if trial % 4 == 0:
+            m.geom_bodyid = rng.integers(0, nbody, 6).astype(np.int32)
+            m.nxn_geom_pair_filtered = rng.integers(0, 6, (3, 2)).astype(np.int32)
+        if trial % 5 == 0:  # M elements in a shuffled order with a duplicate: the last one listed wins
+            order = rng.permutation(m.M_colind.size)
+            m.M_hinit_i, m.M_colind = np.append(m.M_hinit_i[order], m.M_hinit_i[order[0]]), np.append(m.M_colind[order], m.M_colind[order[0]])
+        np.testing.assert_array_equal(S.hessian_pattern(m, groups).dense(), _dense(P.sparse_pattern(m, groups)))
+        block, path = int(rng.choice([32, 64, 128])), str(rng.choice(["fused", "nonfused"]))
+        nv_pad = m.nv_pad if trial % 7 else max(16, m.nv_pad - 16 * int(rng.integers(1, 4)))  # some too small
+        m.nv_pad = nv_pad
+        try:
+            exp = _oracle_plan(m, groups, block, path)
+        except ValueError as exc:
+            refused += 1
+            with pytest.raises(ValueError, match=str(exc)):
+                _tables_plan(m, groups, block, path)
+            continue
+        _assert_same_plan(_tables_plan(m, groups, block, path), exp, f"trial {trial}")
+    assert 0 < refused < 40
+
+
+def _dense(adj):
+    out = np.zeros((len(adj), len(adj)), bool)
+    for a, nb in enumerate(adj):
+        out[a, list(nb)] = True
+    return out
+
+
+def test_refusals_carry_the_reference_messages():
+    # sparse_hessian.py:249-250, 680-684
+    m = synth.model_from_parents(synth.chain_parents(160))  # 12880 factor slots: 51 KB
+    with pytest.raises(ValueError, match="does not fit the block's shared memory"):
+        S.plan_from_pattern(S.hessian_pattern(m, []), m.nv_pad, m.M_hinit_i, m.M_colind, 64, "fused")
+    g1 = synth.model_from_parents(synth.SHAPES["g1"].parents)
+    with pytest.raises(ValueError, match="does not fit the packed layout"):
+        S.plan_from_pattern(S.hessian_pattern(g1, []), 16, g1.M_hinit_i, g1.M_colind, 32)
+    with pytest.raises(ValueError, match="packed H and factor do not fit hfactor"):
+        S.plan_from_pattern(S.hessian_pattern(g1, []), 24, g1.M_hinit_i, g1.M_colind, 32)
+
+
+def test_flex_couplings():
+    """sparse_hessian.py:121-170 on a hand-made model: a 2-triangle cloth over four vertex
+    bodies plus a geom it may touch couples each triangle's bodies with the geom's body, and a
+    self-colliding flex couples all its bodies."""
+    # bodies 1..4 = cloth vertices (3 dofs each, roots), body 5 = a free box (6 dofs)
+    parent, joints = [], []
+    for b in range(4):
+        parent += [-1, 3 * b, 3 * b + 1]
+        joints.append([3 * b, 3 * b + 1, 3 * b + 2])
+    parent += [-1, 12, 13, 14, 15, 16]
+    joints.append(list(range(12, 18)))
+    m = synth.model_from_parents(parent, joints)
+    m.nflex, m.ngeom = 1, 1
+    m.flex_vertadr, m.flex_vertnum, m.flex_vertbodyid = np.array([0]), np.array([4]), np.array([1, 2, 3, 4])
+    m.flex_elemadr, m.flex_elemnum, m.flex_elemdataadr, m.flex_dim = np.array([0]), np.array([2]), np.array([0]), np.array([2])
+    m.flex_elem = np.array([0, 1, 2, 1, 2, 3])
+    m.flex_interp, m.flex_nodeadr, m.flex_nodenum, m.flex_nodebodyid = np.array([0]), np.array([0]), np.array([0]), np.zeros(0, int)
+    m.flex_contype, m.flex_conaffinity, m.flex_selfcollide = np.array([1]), np.array([1]), np.array([0])
+    m.geom_contype, m.geom_conaffinity, m.geom_bodyid = np.array([0]), np.array([0]), np.array([5])
+    dofs = lambda b: set(range(3 * (b - 1), 3 * b)) if b < 5 else set(range(12, 18))  # noqa: E731
+    adj = S.hessian_pattern(m, [])
+    assert dofs(2) | dofs(3) <= adj[0] and not (dofs(4) & adj[0])  # vertex 1 shares no triangle with vertex 4
+    assert dofs(1) | dofs(3) | dofs(4) <= adj[3] | {3} and not (dofs(5) & adj[0])
+    m.geom_conaffinity = np.array([1])  # the box may touch the cloth: triangle by triangle
+    adj = S.hessian_pattern(m, [])
+    assert dofs(5) <= adj[0] and dofs(1) <= adj[12] and not (dofs(4) & adj[0])
+    m.flex_selfcollide = np.array([1])
+    assert dofs(4) <= S.hessian_pattern(m, [])[0]
+    m.flex_interp, m.flex_nodenum, m.flex_nodebodyid = np.array([1]), np.array([2]), np.array([1, 4])
+    m.flex_selfcollide, m.geom_conaffinity = np.array([0]), np.array([0])
+    adj = S.hessian_pattern(m, [])
+    assert dofs(4) <= adj[0] and not (dofs(2) & adj[0])  # an interpolated flex couples its nodes only
+
 def test_plan_gating():
-    # reference: sparse_hessian.py:705-758, tests/test_mjw_sparse_hessian.py:294-300
+    # reference: sparse_hessian.py:705-758, newton_fusion.py:307-322, tests/test_mjw_sparse_hessian.py:294-300
     m, cases = _cases()
     plan, reason = S.plan_for_model(m, None, None, 64, device=None)
     assert plan is None and "declare" in reason
+    plan, reason = S.plan_for_model(m, None, cases[1], 32, device="cpu")
+    assert plan is None and reason == "fused Newton not eligible (CPU)"
     small = synth.model_from_parents(synth.humanoid_parents())
     plan, reason = S.plan_for_model(small, None, [], 32, device=None)
     assert plan is None and reason == "nv 27 < 33"
@@ -134,6 +291,36 @@ def test_plan_gating():
     assert plan is not None and reason == "enabled" and plan.path == "fused"
     with pytest.raises(ValueError):
         S.violation_counter(np.zeros((1, 48, 48)), type("p", (), dict(path="nonfused", nv_pad=48)))
+    # every gate of the fused Newton's eligibility test refuses on its own
+    for field, value in (("opt.cone", 1), ("opt.solver", 1), ("opt.iterations", 0), ("is_sparse", True),
+                         ("block_dim.linesearch_iterative", 64), ("nv_pad", 40), ("use_incremental", False)):  # fmt: skip
+        bad, _ = synth.contact_model()
+        target, leaf = (bad, field) if "." not in field else (getattr(bad, field.split(".")[0]), field.split(".")[1])
+        setattr(target, leaf, value)
+        plan, reason = S.plan_for_model(bad, None, cases[1], 32, device=None)
+        assert plan is None and reason == "Newton solver structure not supported", field
+    named, _ = synth.contact_model()
+    named.opt.integrator = type("E", (), dict(name="DISCRETE"))()
+    assert S.plan_for_model(named, None, cases[1], 32, device=None)[0] is None
+    bare, _ = synth.contact_model()
+    del bare.opt
+    assert S.plan_for_model(bare, None, cases[1], 32, device=None) == (None, "Newton solver structure not supported")
+    for kw in (dict(compact=True), dict(fused_runtime=False)):
+        assert S.plan_for_model(m, None, cases[1], 32, device=None, **kw)[0] is None
+    assert S.plan_for_model(m, type("c", (), dict(sparse_compact=True))(), cases[1], 32, device=None)[0] is None
+    tendon, _ = synth.contact_model()
+    tendon.ntendon, tendon.tendon_limited_adr, tendon.tendon_frictionloss = 1, np.zeros(0, int), np.array([0.5])
+    assert S.plan_for_model(tendon, None, cases[1], 32, device=None) == (None, "tendon limit or frictionloss rows")
+    # the upstream (non-fused) iteration: models the fused Newton does not take, from 80 dofs on
+    big = synth.model_from_parents(synth.SHAPES["stress"].parents)
+    ctx = type("c", (), dict(hfactor=np.zeros((2, big.nv_pad, big.nv_pad), np.float32)))()
+    plan, reason = S.plan_for_model(big, ctx, [], 64, device=None)
+    assert reason == "enabled" and plan.path == "nonfused" and plan.block == 128
+    assert S.plan_for_model(big, None, [], 64, device=None) == (None, "Newton solver structure not supported")
+    mid, _ = synth.contact_model()
+    mid.is_sparse = True
+    ctx = type("c", (), dict(hfactor=np.zeros((2, mid.nv_pad, mid.nv_pad), np.float32)))()
+    assert S.plan_for_model(mid, ctx, cases[1], 32, device=None) == (None, "upstream iteration with nv 36 < 80")
 
 
 def _batch(m, groups, nworld, nefc, seed, ragged=True):
@@ -143,7 +330,7 @@ def _batch(m, groups, nworld, nefc, seed, ragged=True):
     for g in groups:
         mask = np.zeros(nv, bool)
         for b in g:
-            mask[S._chain(b, m.body_parentid, m.body_dofadr, m.body_dofnum)] = True
+            mask[P.body_chain(b, m.body_parentid, m.body_dofadr, m.body_dofnum)] = True
         sup += [mask] * 6
     shape = synth.Shape("contact", tuple(int(p) for p in m.dof_parentid), nefc, nworld, (0.5, 8.0), 0.02, (-4.0, 4.0), 0.6, 1, seed)
     return synth.make_batch(shape, nworld, ragged_nefc=ragged, supports=np.array(sup))
@@ -153,7 +340,7 @@ def test_oracle_executor_against_fp64():
     m, cases = _cases()
     for groups in cases:
         for block in (32, 64):
-            plan = _tables_plan(m, groups, block)
+            plan = _oracle_plan(m, groups, block)
             b = _batch(m, groups, 12, 40, 7)
             hf, search, sdot, decr = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
             st = (b.rowadr, b.rownnz, b.colind)
@@ -200,7 +387,7 @@ def test_gpu_contact_model_bitwise(device, case, block):
     m, cases = _cases()
     plan = S.build_plan(m, cases[case], block, device=device)
     b = _batch(m, cases[case], 137, 40, 11)
-    ref = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
+    ref = R.sparse_init_factor(_oracle_plan(m, cases[case], block), b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
     got = _run_gpu(plan, b, device)
     n_used = 2 * plan.nfac + plan.nv
     np.testing.assert_array_equal(got[0].reshape(137, -1)[:, :n_used], ref[0].reshape(137, -1)[:, :n_used])
@@ -218,7 +405,7 @@ def test_gpu_benchmark_trees_bitwise(device, name, nworld):
     plan, reason = S.plan_for_model(m, None, [], S.block_width(m.nv_pad), device=device)
     assert plan is not None, reason
     b = synth.make_batch(name, nworld, ragged_nefc=True)
-    ref = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
+    ref = R.sparse_init_factor(_oracle_plan(m, []), b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
     got = _run_gpu(plan, b, device)
     for g, r in zip(got[1:4], ref[1:]):
         np.testing.assert_array_equal(g, r)
@@ -242,7 +429,7 @@ def test_gpu_done_mask_violation_counter_and_graph_replay(device):
     done[7] = 1
     hf0 = np.zeros((64, plan.nv_pad, plan.nv_pad), np.float32)
     hf0[:, -1, -1] = 2.0  # the counter accumulates
-    ref = R.sparse_init_factor(plan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad, hfactor=hf0, done=done)
+    ref = R.sparse_init_factor(_oracle_plan(m, cases[1], 64), b.nefc, b.J, b.D, b.state[0], b.M, b.grad, hfactor=hf0, done=done)
     got = _run_gpu(plan, b, device, hfactor0=hf0, done=done)
     cnt = got[0][:, -1, -1]
     assert cnt[5] == 3.0 and (np.delete(cnt, 5) == 2.0).all()
