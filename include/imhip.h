@@ -242,6 +242,38 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
                             int block_size, int nv, int pad, const float *y, int64_t ldy,
                             float *U, float *x, int64_t ldx, int nworld, void *stream);
 
+/* The index table of create_blocked_dense_factor_solve_scratch
+ * (src/instantmimic/utils/mjw_step_optimized.py:932-946), on the host: elemid (nv, nv) = element
+ * of M[w, :] behind every entry of the dense tile (the model's M_tiles[0].elemid); layout
+ * receives pad * pad ids in (nblk, nblk, B, B) order with pad = nv rounded up to block_size and
+ * nM on the padding; identity (B * B floats, may be null) is 1 on the padded diagonal entries of
+ * the last block. */
+int im_blocked_index_layout(const int32_t *elemid, int nv, int nM, int block_size,
+                            int32_t *layout, float *identity);
+
+/* Replaces make_indexed_cholesky_multi_solve_kernel (indexed_factor.py:394-493): x = M^-1 y for
+ * rhs_count right-hand sides from a stored factor U (nworld, pad, pad) (upper triangle read), y and
+ * x (nworld, nv, rhs_count) contiguous.  Worlds with active[w] == 0 are left alone (active may be
+ * null: all worlds).  A column sees the operations of im_blocked_factor_solve's own forward and
+ * backward substitution in the same order. */
+int im_blocked_multi_solve(const float *U, int block_size, int nv, int pad, const float *y,
+                           int rhs_count, const int32_t *active, float *x, int nworld, void *stream);
+
+/* Replaces make_indexed_cholesky_factor_multi_solve_kernel (indexed_factor.py:217-391): the
+ * factor of im_blocked_factor_solve into the workspace U (nworld, pad, pad; required, 16-byte
+ * aligned), then im_blocked_multi_solve from it -- two launches, so the result equals a later
+ * im_blocked_multi_solve on the same U bit for bit.  Inactive worlds: neither U nor x is touched. */
+int im_blocked_factor_multi_solve(const float *M, int64_t ldM, int nM, const int32_t *block_idx,
+                                  int block_size, int nv, int pad, const float *y, int rhs_count,
+                                  const int32_t *active, float *U, float *x, int nworld,
+                                  void *stream);
+
+/* Replaces _copy_dense_factor_kernel (src/instantmimic/utils/mjw_step_optimized.py:875-886):
+ * L_out[w, block_adr[0] + row * nv + col] = U[w, row, col] for row, col < nv; block_adr is the
+ * device array m.qLD_block_adr, L_out (nworld, ld_out) the caller's d.qLD. */
+int im_copy_dense_factor(const float *U, int pad, const int32_t *block_adr, int nv, float *L_out,
+                         int64_t ld_out, int nworld, void *stream);
+
 /* Dense Newton Hessian on fp32 MFMA: H[w] (nv_pad, nv_pad) = Mdense[w] (nv, nv) +
  * J[w]' diag(D [state == quad, row < nefc]) J[w].  Stands in for mujoco_warp's
  * solver._update_gradient JTDAJ kernel, which the reference calls at

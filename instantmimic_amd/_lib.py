@@ -137,6 +137,10 @@ SIGNATURES = {
         [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],
     ),
     "im_blocked_factor_solve": (_i, [_vp, _i64, _i, _vp, _i, _i, _i, _vp, _i64, _vp, _vp, _i64, _i, _vp]),
+    "im_blocked_index_layout": (_i, [_vp, _i, _i, _i, _vp, _vp]),
+    "im_blocked_multi_solve": (_i, [_vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _vp]),
+    "im_blocked_factor_multi_solve": (_i, [_vp, _i64, _i, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _vp]),
+    "im_copy_dense_factor": (_i, [_vp, _i, _vp, _i, _vp, _i64, _i, _vp]),
     "im_jtdj_mfma": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
     "im_muscle_project": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i64, _i, _vp]),
     "im_muscle_implicit_gather": (

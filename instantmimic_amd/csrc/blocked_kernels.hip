@@ -332,8 +332,9 @@ template <int B, bool LEAN>
 __global__ __launch_bounds__(512, LEAN ? 6 : 2) void blocked_factor_solve_kernel(
     const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
     const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
-    int64_t ldx, int nv, int pad) {
+    int64_t ldx, int nv, int pad, const int32_t *__restrict__ active) {
   extern __shared__ float lds[];
+  if (active && active[blockIdx.x] == 0) return;  // the whole workgroup: nothing of this world is touched
   const Stair<B> S{pad};
   const int nU = S.words();
   float *U = lds;             // [nU] the factor, block row by block row
@@ -343,14 +344,15 @@ __global__ __launch_bounds__(512, LEAN ? 6 : 2) void blocked_factor_solve_kernel
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
   for (int i = tid; i < nU; i += nt) U[i] = 0.0f;
-  for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? y[w * ldy + i] : 0.0f;
+  for (int i = tid; i < pad; i += nt) rhs[i] = (y && i < nv) ? y[w * ldy + i] : 0.0f;  // factor only: no y, no x
   __syncthreads();
   gather_tiles<B>(M + w * ldM, block_idx, nM, nv, pad, U, tid, nt);
   __syncthreads();
   const GatheredSrc<B> src{U, pad};
   factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
   backward_solve<B>(U, rhs, pad, tid);
-  for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
+  if (x)
+    for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
   if (Uout)
     for (int i = tid; i < pad * pad / 4; i += nt) {  // pad is a multiple of B >= 8: a float4 stays in a tile
       const int r = 4 * i / pad, c = 4 * i - r * pad;
@@ -385,14 +387,15 @@ template <int B>
 __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
     const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
     const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
-    int64_t ldx, int nv, int pad, int nworld) {
+    int64_t ldx, int nv, int pad, int nworld, const int32_t *__restrict__ active) {
   extern __shared__ float lds[];
   constexpr int BB = B * B, PER = BB / 16;  // a lane's elements of a tile: e = l + 16 u
   const int lane = threadIdx.x, l = lane & 15, q = lane >> 4;
   const int nblk = pad / B, ntiles = quad_tiles_before(nblk, nblk);
   const int64_t w_raw = (int64_t)blockIdx.x * 4 + q;
-  const bool live = w_raw < nworld;
-  const int64_t w = live ? w_raw : (int64_t)nworld - 1;  // a spare row repeats the last world and stores nothing
+  // an inactive world rides along like a spare row: computed, nothing stored
+  const bool live = w_raw < nworld && (!active || active[w_raw] != 0);
+  const int64_t w = w_raw < nworld ? w_raw : (int64_t)nworld - 1;  // a spare row repeats the last world and stores nothing
   const int world_floats = quad_world_floats(pad, B);
   float *U = lds + q * world_floats;
   float *rhs = U + BB * ntiles;  // [pad]
@@ -435,7 +438,7 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
           }
     }
   }
-  for (int i = l; i < pad; i += 16) rhs[i] = i < nv ? y[w * ldy + i] : 0.0f;
+  for (int i = l; i < pad; i += 16) rhs[i] = (y && i < nv) ? y[w * ldy + i] : 0.0f;
   wave_sync();
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -575,7 +578,8 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
     wave_sync();
   }
   if (live) {
-    for (int i = l; i < nv; i += 16) x[w * ldx + i] = rhs[i];
+    if (x)
+      for (int i = l; i < nv; i += 16) x[w * ldx + i] = rhs[i];
     if (Uout) {
       float4 *dst = (float4 *)(Uout + w * (int64_t)pad * pad);
       for (int i4 = l; i4 < pad * pad / 4; i4 += 16) {
@@ -840,6 +844,96 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------- stored factor, several right-hand sides
+// x = (U'U)^-1 y for `nrhs` columns with a factor computed earlier: forward substitution with U',
+// backward with U, block by block as the fused kernels do for their single right-hand side, so a
+// column here sees the operations of blocked_factor_solve_kernel in the same order.
+// Reference: multi_solve_indexed_cholesky_kernel and the solve half of
+// factor_multi_solve_indexed_cholesky_kernel
+// (src/instantmimic/utils/mjw_kernels/indexed_factor.py:394-493, 217-391).
+// One wavefront per world: the upper triangle of U packed row by row in LDS, the right-hand
+// sides beside it; lane (r, c) = row r of the current block, column c of a group of 64 / B columns.
+__host__ __device__ inline int packed_upper_at(int r, int c, int pad) { return r * pad - r * (r - 1) / 2 + (c - r); }
+
+template <int B>
+__global__ __launch_bounds__(64) void blocked_multi_solve_kernel(
+    const float *__restrict__ Uin, const float *__restrict__ y, const int32_t *__restrict__ active,
+    float *__restrict__ x, int nv, int pad, int nrhs) {
+  extern __shared__ float lds[];
+  const int64_t w = blockIdx.x;
+  if (active && active[w] == 0) return;
+  float *U = lds;                          // [pad (pad + 1) / 2]
+  float *rhs = U + pad * (pad + 1) / 2;    // [pad][nrhs]
+  const int lane = threadIdx.x, r = lane % B, cg = lane / B;
+  constexpr int CPL = 64 / B;              // columns per pass
+  const float *Uw = Uin + w * (int64_t)pad * pad;
+  for (int i = lane; i < pad * pad; i += 64) {
+    const int row = i / pad, col = i - row * pad;
+    if (col >= row) U[packed_upper_at(row, col, pad)] = Uw[i];
+  }
+  for (int i = lane; i < pad * nrhs; i += 64) rhs[i] = i < nv * nrhs ? y[w * (int64_t)nv * nrhs + i] : 0.0f;
+  wave_sync();
+  for (int c0 = 0; c0 < nrhs; c0 += CPL) {
+    const int col = c0 + cg < nrhs ? c0 + cg : nrhs - 1;  // spare lanes repeat the last column
+    const bool mine = c0 + cg < nrhs;
+    const int base = cg * B;                              // first lane of this column's group
+    // forward: z = U'^-1 y
+    for (int k = 0; k < pad; k += B) {
+      float s = rhs[(k + r) * nrhs + col];
+      for (int j = 0; j < k; j += B) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < B; ++t) sum = fma_(U[packed_upper_at(j + t, k + r, pad)], rhs[(j + t) * nrhs + col], sum);
+        s = s - sum;
+      }
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        const float inv = 1.0f / U[packed_upper_at(k + j, k + j, pad)];
+        const float z = __shfl(s * inv, base + j);
+        if (r == j) s = z;
+        if (r > j) s = fma_(-U[packed_upper_at(k + j, k + r, pad)], z, s);
+      }
+      wave_sync();  // every lane has read this block's old values
+      if (mine) rhs[(k + r) * nrhs + col] = s;
+      wave_sync();
+    }
+    // backward: x = U^-1 z
+    for (int i0 = pad - B; i0 >= 0; i0 -= B) {
+      float s = rhs[(i0 + r) * nrhs + col];
+      for (int j = i0 + B; j < pad; j += B) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < B; ++t) sum = fma_(U[packed_upper_at(i0 + r, j + t, pad)], rhs[(j + t) * nrhs + col], sum);
+        s = s - sum;
+      }
+#pragma unroll
+      for (int rr = B - 1; rr >= 0; --rr) {
+        const float inv = 1.0f / U[packed_upper_at(i0 + rr, i0 + rr, pad)];
+        const float xv = __shfl(s * inv, base + rr);
+        if (r == rr) s = xv;
+        if (r < rr) s = fma_(-U[packed_upper_at(i0 + r, i0 + rr, pad)], xv, s);
+      }
+      wave_sync();
+      if (mine) rhs[(i0 + r) * nrhs + col] = s;
+      wave_sync();
+    }
+  }
+  for (int i = lane; i < nv * nrhs; i += 64) x[w * (int64_t)nv * nrhs + i] = rhs[i];
+}
+
+// L_out[w, adr[0] + row * nv + col] = U[w, row, col] over the nv x nv corner: the blocked upper
+// factor in the dense-block layout of the caller's factor array
+// (_copy_dense_factor_kernel, src/instantmimic/utils/mjw_step_optimized.py:875-886).
+__global__ __launch_bounds__(256) void copy_dense_factor_kernel(const float *__restrict__ U, int pad,
+                                                                const int32_t *__restrict__ block_adr, int nv,
+                                                                float *__restrict__ L_out, int64_t ld_out) {
+  const int64_t w = blockIdx.y;
+  const int slot = blockIdx.x * 256 + threadIdx.x;
+  if (slot >= nv * nv) return;
+  const int row = slot / nv, col = slot - row * nv;
+  L_out[w * ld_out + block_adr[0] + slot] = U[(w * pad + row) * (int64_t)pad + col];
+}
+
 // ---------------------------------------------------------------------------- dense J'DJ
 // H[w] = M[w] + J[w]' diag(Dc[w]) J[w], H (nv_pad, nv_pad), on v_mfma_f32_32x32x2_f32.
 // One workgroup of four wavefronts per world, a wavefront per 32 x 32 output tile (the tiles
@@ -966,16 +1060,11 @@ __global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
 
 extern "C" {
 
-int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *block_idx, int block_size,
-                            int nv, int pad, const float *y, int64_t ldy, float *U, float *x, int64_t ldx,
-                            int nworld, void *stream) {
-  if (nworld < 0 || nv <= 0 || pad < nv) return IM_ERR_ARG;
-  if (nworld == 0) return IM_OK;
-  if (!M || !block_idx || !y || !x) return IM_ERR_ARG;
-  if (block_size != 8 && block_size != 16) return IM_ERR_UNSUPPORTED;
-  if (pad % block_size || pad - nv >= block_size) return IM_ERR_ARG;
-  if (ldy < nv || ldx < nv) return IM_ERR_STRIDE;
-  if (U && ((uintptr_t)U & 15)) return IM_ERR_STRIDE;  // written 16 bytes at a time
+// factor (+ forward / backward solve when y and x are given) for every world whose `active`
+// entry is nonzero (all when null)
+static int launch_blocked_factor(const float *M, int64_t ldM, int nM, const int32_t *block_idx, int block_size,
+                                 int nv, int pad, const float *y, int64_t ldy, float *U, float *x, int64_t ldx,
+                                 const int32_t *active, int nworld, void *stream) {
   const int B = block_size;
   static const bool quad_off = [] {
     const char *e = std::getenv("IMHIP_BLOCKED_KERNEL");
@@ -987,7 +1076,7 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
     const size_t quad_bytes = sizeof(float) * 4 * (size_t)im::quad_world_floats(pad, B);
     auto qfn = B == 8 ? im::blocked_factor_solve_quad_kernel<8> : im::blocked_factor_solve_quad_kernel<16>;
     hipLaunchKernelGGL(qfn, dim3((unsigned)((nworld + 3) / 4)), dim3(64), quad_bytes, (hipStream_t)stream, M, ldM, nM,
-                       block_idx, y, ldy, U, x, ldx, nv, pad, nworld);
+                       block_idx, y, ldy, U, x, ldx, nv, pad, nworld, active);
     IM_HIP_CHECK(hipGetLastError());
     return IM_OK;
   }
@@ -1005,7 +1094,91 @@ int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *
   // pad 96, 512 beyond: two workgroups per CU there, the block rows' parallel parts want the lanes).
   const int threads = pad <= 48 ? 64 : (pad <= 64 && B == 16) ? 128 : pad <= 96 ? 256 : 512;
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(threads), lds_bytes, (hipStream_t)stream, M, ldM, nM, block_idx, y,
-                     ldy, U, x, ldx, nv, pad);
+                     ldy, U, x, ldx, nv, pad, active);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+static int check_blocked_shape(int block_size, int nv, int pad) {
+  if (nv <= 0 || pad < nv) return IM_ERR_ARG;
+  if (block_size != 8 && block_size != 16) return IM_ERR_UNSUPPORTED;
+  if (pad % block_size || pad - nv >= block_size) return IM_ERR_ARG;
+  return IM_OK;
+}
+
+static int launch_multi_solve(const float *U, int block_size, int nv, int pad, const float *y, int nrhs,
+                              const int32_t *active, float *x, int nworld, void *stream) {
+  const size_t lds_bytes = sizeof(float) * ((size_t)pad * (pad + 1) / 2 + (size_t)pad * nrhs);
+  if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
+  auto fn = block_size == 8 ? im::blocked_multi_solve_kernel<8> : im::blocked_multi_solve_kernel<16>;
+  if (lds_bytes > 64 * 1024)
+    IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(64), lds_bytes, (hipStream_t)stream, U, y, active, x, nv, pad, nrhs);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *block_idx, int block_size,
+                            int nv, int pad, const float *y, int64_t ldy, float *U, float *x, int64_t ldx,
+                            int nworld, void *stream) {
+  if (nworld < 0) return IM_ERR_ARG;
+  if (const int st = check_blocked_shape(block_size, nv, pad)) return st;
+  if (nworld == 0) return IM_OK;
+  if (!M || !block_idx || !y || !x) return IM_ERR_ARG;
+  if (ldy < nv || ldx < nv) return IM_ERR_STRIDE;
+  if (U && ((uintptr_t)U & 15)) return IM_ERR_STRIDE;  // written 16 bytes at a time
+  return launch_blocked_factor(M, ldM, nM, block_idx, block_size, nv, pad, y, ldy, U, x, ldx, nullptr, nworld, stream);
+}
+
+int im_blocked_multi_solve(const float *U, int block_size, int nv, int pad, const float *y, int rhs_count,
+                           const int32_t *active, float *x, int nworld, void *stream) {
+  if (nworld < 0 || rhs_count <= 0) return IM_ERR_ARG;
+  if (const int st = check_blocked_shape(block_size, nv, pad)) return st;
+  if (nworld == 0) return IM_OK;
+  if (!U || !y || !x) return IM_ERR_ARG;
+  return launch_multi_solve(U, block_size, nv, pad, y, rhs_count, active, x, nworld, stream);
+}
+
+int im_blocked_factor_multi_solve(const float *M, int64_t ldM, int nM, const int32_t *block_idx, int block_size,
+                                  int nv, int pad, const float *y, int rhs_count, const int32_t *active, float *U,
+                                  float *x, int nworld, void *stream) {
+  if (nworld < 0 || rhs_count <= 0) return IM_ERR_ARG;
+  if (const int st = check_blocked_shape(block_size, nv, pad)) return st;
+  if (nworld == 0) return IM_OK;
+  if (!M || !block_idx || !y || !x || !U) return IM_ERR_ARG;
+  if ((uintptr_t)U & 15) return IM_ERR_STRIDE;
+  const int st = launch_blocked_factor(M, ldM, nM, block_idx, block_size, nv, pad, nullptr, 0, U, nullptr, 0, active,
+                                       nworld, stream);
+  if (st != IM_OK) return st;
+  return launch_multi_solve(U, block_size, nv, pad, y, rhs_count, active, x, nworld, stream);
+}
+
+int im_blocked_index_layout(const int32_t *elemid, int nv, int nM, int block_size, int32_t *layout,
+                            float *identity) {
+  if (!elemid || !layout || nv <= 0 || nM < 0 || block_size <= 0) return IM_ERR_ARG;
+  const int B = block_size, nblk = (nv + B - 1) / B;
+  int32_t *out = layout;
+  for (int kb = 0; kb < nblk; ++kb)
+    for (int ib = 0; ib < nblk; ++ib)
+      for (int r = 0; r < B; ++r)
+        for (int c = 0; c < B; ++c) {
+          const int row = kb * B + r, col = ib * B + c;
+          *out++ = (row < nv && col < nv) ? elemid[(size_t)row * nv + col] : nM;  // nM: out of range, reads as zero
+        }
+  if (identity)
+    for (int r = 0; r < B; ++r)
+      for (int c = 0; c < B; ++c) identity[r * B + c] = (r == c && (nblk - 1) * B + r >= nv) ? 1.0f : 0.0f;
+  return IM_OK;
+}
+
+int im_copy_dense_factor(const float *U, int pad, const int32_t *block_adr, int nv, float *L_out, int64_t ld_out,
+                         int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || pad < nv) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!U || !block_adr || !L_out) return IM_ERR_ARG;
+  if (ld_out < (int64_t)nv * nv) return IM_ERR_STRIDE;
+  hipLaunchKernelGGL(im::copy_dense_factor_kernel, dim3((unsigned)((nv * nv + 255) / 256), (unsigned)nworld), dim3(256),
+                     0, (hipStream_t)stream, U, pad, block_adr, nv, L_out, ld_out);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

@@ -716,6 +716,31 @@ int orc_blocked_factor_solve(int nworld, int nv, int pad, int B, int nM, const f
   return 0;
 }
 
+/* x = (U'U)^-1 y for nrhs columns from a stored factor: per column the forward and backward
+ * substitution blocked_world applies to its single right-hand side
+ * (src/instantmimic/utils/mjw_kernels/indexed_factor.py:394-493); y and x (nworld, nv, nrhs),
+ * worlds with active[w] == 0 are left alone. */
+int orc_blocked_multi_solve(int nworld, int nv, int pad, int B, const float *U, const float *y,
+                            int nrhs, const int *active, float *x) {
+#pragma omp parallel
+  {
+    float *rhs = (float *)malloc(sizeof(float) * pad);
+#pragma omp for schedule(static)
+    for (int w = 0; w < nworld; ++w) {
+      if (active && active[w] == 0) continue;
+      const float *Uw = U + (size_t)w * pad * pad;
+      for (int c = 0; c < nrhs; ++c) {
+        for (int i = 0; i < pad; ++i) rhs[i] = i < nv ? y[((size_t)w * nv + i) * nrhs + c] : 0.0f;
+        blocked_forward(pad, B, Uw, rhs);
+        blocked_backward(pad, B, Uw, rhs);
+        for (int i = 0; i < nv; ++i) x[((size_t)w * nv + i) * nrhs + c] = rhs[i];
+      }
+    }
+    free(rhs);
+  }
+  return 0;
+}
+
 /* Per-iteration factor stage on the dense Hessian (src/instantmimic/utils/mjw_kernels/
  * newton_stages.py:614-742): incremental update of H's upper triangle over the changed
  * rows' dof union (:451-470, 651-701), then the augmented blocked Cholesky (:473-611; the

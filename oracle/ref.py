@@ -34,7 +34,8 @@ def lib():
     global _LIB
     if _LIB is None:
         path = os.path.join(_HERE, "_build", "liboracle.so")
-        if not os.path.exists(path):
+        src = os.path.join(_HERE, "cpu_ref.c")
+        if not os.path.exists(path) or os.path.getmtime(path) < os.path.getmtime(src):
             build()
         _LIB = ctypes.CDLL(path)
     return _LIB
@@ -285,6 +286,18 @@ def blocked_factor_solve(M, block_idx, nv, pad, B, y, want_factor=True):
     x = np.zeros((nworld, nv), np.float32)
     lib().orc_blocked_factor_solve(nworld, nv, pad, B, nM, _p(M), nM, _p(_i(block_idx)), _p(y), _p(U), _p(x))
     return (x, U) if want_factor else x
+
+
+def blocked_multi_solve(U, nv, B, y, active=None, x=None):
+    """Solve with stored factors U (nworld, pad, pad) for y (nworld, nv, nrhs); inactive worlds
+    keep ``x`` (zeros when not given)."""
+    U, y = _f(U), _f(y)
+    nworld, pad, _ = U.shape
+    nrhs = y.shape[2]
+    x = np.zeros_like(y) if x is None else _f(x).copy()
+    act = _i(active) if active is not None else None
+    lib().orc_blocked_multi_solve(nworld, nv, pad, B, _p(U), _p(y), nrhs, _p(act), _p(x))
+    return x
 
 
 def jtdj_dense(Mdense, J, D, state, nefc, nv_pad, quad=1):

@@ -148,3 +148,99 @@ def test_dense_hessian_staging_indices_stay_inside_a_row():
                         if c < nvr:
                             hits[(wave * 8 + i) * nvr + c] += 1
         assert (hits[: 32 * nvr] == 1).all() and (hits[32 * nvr :] == 0).all(), nv
+
+
+def test_multi_solve_oracle_against_the_single_solve_and_fp64():
+    """The stored-factor solve, column by column, is the single-right-hand-side solve bit for bit
+    (same substitution steps), and solves M x = y; inactive worlds keep their x."""
+    b, nv, Md = _dense_model("snu", 5, well=True)
+    pad, layout, _ = BD.block_index_layout(np.arange(nv * nv), nv, nv * nv, 16)
+    M32 = Md.reshape(5, -1).astype(np.float32)
+    rng = np.random.default_rng(2)
+    y = rng.normal(size=(5, nv, 3)).astype(np.float32)
+    _, U = R.blocked_factor_solve(M32, layout, nv, pad, 16, y[:, :, 0])
+    active = np.array([1, 0, 1, 1, 0], np.int32)
+    x = R.blocked_multi_solve(U, nv, 16, y, active)
+    assert np.abs(x[active == 0]).max() == 0.0
+    for c in range(3):
+        single = R.blocked_factor_solve(M32, layout, nv, pad, 16, np.ascontiguousarray(y[:, :, c]), want_factor=False)
+        np.testing.assert_array_equal(x[active == 1, :, c], single[active == 1])
+    for w in np.flatnonzero(active):
+        want = np.linalg.solve(M32[w].reshape(nv, nv).astype(np.float64), y[w].astype(np.float64))
+        np.testing.assert_allclose(x[w], want, rtol=2e-4, atol=2e-5)
+
+
+def test_factor_solve_dispatcher_precedence_and_errors():
+    # reference: src/instantmimic/utils/mjw_step_optimized.py:1030-1070, 984-986
+    with pytest.raises(RuntimeError, match="requires the blocked dense path"):
+        BD._factor_solve_i_dense(None, None, None, None, None, None, factor_workspace=object())
+    with pytest.raises(NotImplementedError):
+        BD._factor_solve_i_dense(None, None, None, None, None, None)
+    seen = []
+    BD._factor_solve_i_dense(None, None, None, None, None, None, retain_factor=True, upstream=seen.append)
+    assert seen == [True]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,B,nworld,nrhs", [("snu", 16, 3, 5), ("g1", 8, 37, 3), ("g1", 16, 37, 1), ("stress", 16, 6, 9), ("snu", 8, 20, 17)])
+def test_gpu_blocked_multi_solve(device, name, B, nworld, nrhs):
+    """reference: tests/test_blocked_dense_factor_solve.py:528-626 -- several right-hand sides with
+    an active mask; the reuse kernel on a factor stored by the single-solve path equals the
+    fused kernel bit for bit; inactive worlds are untouched; everything equals the oracle."""
+    import torch
+
+    b, nv, Md = _dense_model(name, nworld, well=True)
+    M32 = np.ascontiguousarray(Md.reshape(nworld, -1).astype(np.float32))
+    m = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))])
+    M = torch.from_numpy(M32).to(device)
+    d = SimpleNamespace(nworld=nworld, M=M)
+    scratch = BD.create_blocked_dense_factor_solve_scratch(m, d, device, block_size=B)
+    rng = np.random.default_rng(31)
+    rhs = rng.normal(size=(nworld, nv, nrhs)).astype(np.float32)
+    act = (rng.random(nworld) < 0.7).astype(np.int32)
+    act[0], act[1] = 1, 0
+    y, active = torch.from_numpy(rhs).to(device), torch.from_numpy(act).to(device)
+    factor = torch.full((nworld, scratch.pad, scratch.pad), 7.0, device=device)
+    solution = torch.zeros_like(y)
+    BD.blocked_factor_multi_solve(M, scratch, y, active, factor, solution)
+    # the single-solve path stores its factor in a second workspace; solve again from it
+    reused_factor = torch.zeros_like(factor)
+    single_x = torch.zeros((nworld, nv), device=device)
+    BD._factor_solve_i_dense(m, d, M, single_x, y[:, :, 0].contiguous(), scratch, factor_workspace=reused_factor)
+    reused = torch.zeros_like(y)
+    BD.blocked_multi_solve(reused_factor, scratch, y, active, reused)
+    torch.cuda.synchronize()
+    got = solution.cpu().numpy()
+    np.testing.assert_array_equal(reused.cpu().numpy(), got)
+    np.testing.assert_array_equal(got[act == 0], 0.0)
+    assert (factor.cpu().numpy()[act == 0] == 7.0).all()  # an inactive world's factor is not written either
+    np.testing.assert_array_equal(factor.cpu().numpy()[act == 1], reused_factor.cpu().numpy()[act == 1])
+    _, U_ref = R.blocked_factor_solve(M32, scratch.indices.cpu().numpy(), nv, scratch.pad, B, rhs[:, :, 0])
+    np.testing.assert_array_equal(got, R.blocked_multi_solve(U_ref, nv, B, rhs, act))
+    np.testing.assert_array_equal(single_x.cpu().numpy()[act == 1], got[act == 1, :, 0])
+    for w in np.flatnonzero(act)[:4]:
+        want = np.linalg.solve(M32[w].reshape(nv, nv).astype(np.float64), rhs[w].astype(np.float64))
+        assert np.abs(got[w] - want).max() / max(np.abs(want).max(), 1e-6) < 2e-3
+
+
+@pytest.mark.gpu
+def test_gpu_retained_factor_goes_to_the_dense_block_layout(device):
+    # reference: src/instantmimic/utils/mjw_step_optimized.py:875-886, 984-993
+    import torch
+
+    nworld = 11
+    b, nv, Md = _dense_model("g1", nworld, well=True)
+    M = torch.from_numpy(np.ascontiguousarray(Md.reshape(nworld, -1).astype(np.float32))).to(device)
+    m = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))],
+                        qLD_block_adr=torch.tensor([13], dtype=torch.int32, device=device))  # fmt: skip
+    d = SimpleNamespace(nworld=nworld, M=M, qLD=torch.full((nworld, 13 + nv * nv + 5), -3.0, device=device))
+    scratch = BD.create_blocked_dense_factor_solve_scratch(m, d, device)
+    y = torch.from_numpy(b.grad).to(device)
+    x = torch.zeros_like(y)
+    BD._factor_solve_i_dense(m, d, M, x, y, scratch, retain_factor=True)
+    torch.cuda.synchronize()
+    qLD, U = d.qLD.cpu().numpy(), scratch.U.cpu().numpy()
+    np.testing.assert_array_equal(qLD[:, 13 : 13 + nv * nv].reshape(nworld, nv, nv), U[:, :nv, :nv])
+    assert (qLD[:, :13] == -3.0).all() and (qLD[:, 13 + nv * nv :] == -3.0).all()
+    with pytest.raises(RuntimeError, match="requires qLD block offsets"):
+        BD._blocked_dense_factor_solve(d, M, x, y, scratch, factor_out=d.qLD)
