@@ -25,6 +25,7 @@ extern "C" {
 #define IM_ERR_UNSUPPORTED 3 /* shape outside what the kernels are built for */
 #define IM_ERR_HIP 4         /* a HIP runtime call failed (see im_last_hip_error) */
 #define IM_ERR_STRIDE 5      /* rows are not contiguous floats */
+#define IM_ERR_SCRATCH 6     /* the batch needs more than IM_STATIC_SCRATCH_BYTES of the static scratch */
 
 #define IM_MAX_GROUPS 4
 
@@ -267,6 +268,20 @@ int im_blocked_factor_multi_solve(const float *M, int64_t ldM, int nM, const int
                                   int block_size, int nv, int pad, const float *y, int rhs_count,
                                   const int32_t *active, float *U, float *x, int nworld,
                                   void *stream);
+
+/* im_blocked_factor_multi_solve for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.  The
+ * factor workspace U is a static device array of IM_STATIC_SCRATCH_BYTES inside the library, one
+ * per GPU, held until the process ends; the call allocates nothing.  nworld * pad * pad * 4 bytes
+ * beyond that size are refused with IM_ERR_SCRATCH.  Results equal im_blocked_factor_multi_solve
+ * bit for bit.  All calls on one GPU share the array: calls that overlap there (two streams, two
+ * threads) race, and the factor of one call is gone after the next.  The first call on a device
+ * looks the array's address up and must not be made under stream capture. */
+#define IM_STATIC_SCRATCH_BYTES (32u << 20)
+int im_blocked_factor_multi_solve_static(const float *M, int64_t ldM, int nM,
+                                         const int32_t *block_idx, int block_size, int nv, int pad,
+                                         const float *y, int rhs_count, const int32_t *active,
+                                         float *x, int nworld, void *stream);
 
 /* Replaces _copy_dense_factor_kernel (src/instantmimic/utils/mjw_step_optimized.py:875-886):
  * L_out[w, block_adr[0] + row * nv + col] = U[w, row, col] for row, col < nv; block_adr is the

@@ -18,6 +18,7 @@ IM_ERR_STRUCTURE = 2
 IM_ERR_UNSUPPORTED = 3
 IM_ERR_HIP = 4
 IM_ERR_STRIDE = 5
+IM_ERR_SCRATCH = 6
 IM_FLAG_NEGATE = 1
 
 
@@ -140,6 +141,7 @@ SIGNATURES = {
     "im_blocked_index_layout": (_i, [_vp, _i, _i, _i, _vp, _vp]),
     "im_blocked_multi_solve": (_i, [_vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _vp]),
     "im_blocked_factor_multi_solve": (_i, [_vp, _i64, _i, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _vp]),
+    "im_blocked_factor_multi_solve_static": (_i, [_vp, _i64, _i, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _vp]),
     "im_copy_dense_factor": (_i, [_vp, _i, _vp, _i, _vp, _i64, _i, _vp]),
     "im_jtdj_mfma": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
     "im_muscle_project": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i64, _i, _vp]),

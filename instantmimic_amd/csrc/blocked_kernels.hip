@@ -14,6 +14,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
+#include <mutex>
 #include <cstring>
 
 #include "common.h"
@@ -1060,6 +1061,29 @@ __global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
 
 extern "C" {
 
+// Factor store of im_blocked_factor_multi_solve_static: one array per GPU, held from the moment
+// the library is loaded on it until the process ends.  In host code the name below is only a
+// handle for hipGetSymbolAddress; kernels get the address that call returns.
+static __device__ __align__(256) float scratch[IM_STATIC_SCRATCH_BYTES / sizeof(float)];
+
+// Address of `scratch` on the current device, looked up once per device.
+static int static_scratch(float **out) {
+  constexpr int kMaxDevices = 64;
+  static float *ptr[kMaxDevices] = {};
+  static std::mutex guard;
+  int dev = -1;
+  IM_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return IM_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(guard);
+  if (!ptr[dev]) {
+    float *p = nullptr;
+    IM_HIP_CHECK(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+    ptr[dev] = p;
+  }
+  *out = ptr[dev];
+  return IM_OK;
+}
+
 // factor (+ forward / backward solve when y and x are given) for every world whose `active`
 // entry is nonzero (all when null)
 static int launch_blocked_factor(const float *M, int64_t ldM, int nM, const int32_t *block_idx, int block_size,
@@ -1147,6 +1171,24 @@ int im_blocked_factor_multi_solve(const float *M, int64_t ldM, int nM, const int
   if (nworld == 0) return IM_OK;
   if (!M || !block_idx || !y || !x || !U) return IM_ERR_ARG;
   if ((uintptr_t)U & 15) return IM_ERR_STRIDE;
+  const int st = launch_blocked_factor(M, ldM, nM, block_idx, block_size, nv, pad, nullptr, 0, U, nullptr, 0, active,
+                                       nworld, stream);
+  if (st != IM_OK) return st;
+  return launch_multi_solve(U, block_size, nv, pad, y, rhs_count, active, x, nworld, stream);
+}
+
+int im_blocked_factor_multi_solve_static(const float *M, int64_t ldM, int nM, const int32_t *block_idx,
+                                         int block_size, int nv, int pad, const float *y, int rhs_count,
+                                         const int32_t *active, float *x, int nworld, void *stream) {
+  if (nworld < 0 || rhs_count <= 0) return IM_ERR_ARG;
+  if (const int st = check_blocked_shape(block_size, nv, pad)) return st;
+  if ((uint64_t)nworld * pad * pad * sizeof(float) > IM_STATIC_SCRATCH_BYTES) return IM_ERR_SCRATCH;
+  if (nworld == 0) return IM_OK;
+  if (!M || !block_idx || !y || !x) return IM_ERR_ARG;
+  float *U = nullptr;
+  if (const int st = static_scratch(&U)) return st;
+  // every active world's (pad, pad) slice is written whole by the factor kernel before the
+  // solve reads it, and the solve skips the inactive ones: nothing has to start at zero
   const int st = launch_blocked_factor(M, ldM, nM, block_idx, block_size, nv, pad, nullptr, 0, U, nullptr, 0, active,
                                        nworld, stream);
   if (st != IM_OK) return st;

@@ -174,6 +174,7 @@ const char *im_status_string(int status) {
     case IM_ERR_UNSUPPORTED: return "shape not supported by the device kernels";
     case IM_ERR_HIP: return "HIP runtime error";
     case IM_ERR_STRIDE: return "rows must be contiguous floats";
+    case IM_ERR_SCRATCH: return "the batch exceeds the library's static scratch (IM_STATIC_SCRATCH_BYTES)";
     default: return "unknown status";
   }
 }
