@@ -104,6 +104,33 @@ int im_assemble_tree_ldl_solve(const im_tree_plan *plan, const float *M,
                                int64_t ldg, float *x, int64_t ldx, float *Hout,
                                int nworld, unsigned flags, void *stream);
 
+/* im_assemble_tree_ldl_solve for `niter` Newton iterations that share M, J and D and differ in
+ * the constraint states (and optionally the gradient): what a step of the reference's Newton
+ * loop does with a world kept resident in one block across its iterations
+ * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:57-298).  Iteration i reads
+ * state + i * state_iter_stride (ints) and grad + i * grad_iter_stride (floats; 0 = one gradient
+ * for all) and writes x + i * x_iter_stride.  Every iteration assembles H afresh from M, so the
+ * results are those of niter calls of im_assemble_tree_ldl_solve bit for bit; where a generated
+ * kernel exists for the tree the whole sequence is one launch whose grid covers (worlds,
+ * iteration) with the iterations of a world scheduled next to one L2, so M and J come from
+ * memory once and one iteration's factor phase overlaps another's reads. */
+int im_assemble_tree_ldl_solve_iters(const im_tree_plan *plan, const float *M, int64_t ldM,
+                                     const float *J, int njmax, const float *D,
+                                     const int32_t *state, int64_t state_iter_stride,
+                                     const int32_t *nefc, int quad, const float *grad, int64_t ldg,
+                                     int64_t grad_iter_stride, float *x, int64_t ldx,
+                                     int64_t x_iter_stride, int nworld, int niter, unsigned flags,
+                                     void *stream);
+
+/* Self-check of an arithmetic shortcut (no counterpart in the reference): the generated tree
+ * kernels take a pivot's reciprocal as the hardware estimate plus one exact-residual correction
+ * instead of the full division whenever 2^-101 <= |pivot| < 2^102.  This launch compares the two
+ * for every float whose bit pattern lies in [first_bits, last_bits] and that is in that range,
+ * and adds the number of differing results to *mismatches (a device counter the caller zeroes).
+ * It must stay 0: the kernels' bit-for-bit agreement with the reference's 1.0f / x rests on it. */
+int im_check_reciprocal(uint32_t first_bits, uint32_t last_bits, unsigned long long *mismatches,
+                        void *stream);
+
 /* Coupling pattern of a model's dofs: which pairs (a, b) may be nonzero in H.  Replaces
  * hessian_pattern (src/instantmimic/utils/mjw_kernels/sparse_hessian.py:62-118) as a builder:
  * creation couples every dof with its tree ancestors (:70-75; dof_parentid[d] < d), and the

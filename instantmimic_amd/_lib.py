@@ -114,6 +114,11 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _i, _u, _vp],
     ),
+    "im_assemble_tree_ldl_solve_iters": (
+        _i,
+        [_vp, _vp, _i64, _vp, _i, _vp, _vp, _i64, _vp, _i, _vp, _i64, _i64, _vp, _i64, _i64, _i, _i, _u, _vp],
+    ),
+    "im_check_reciprocal": (_i, [C.c_uint32, C.c_uint32, _vp, _vp]),
     "im_dof_pattern_create": (_i, [_i, _vp, _i, _vp, _vp, _vp, C.POINTER(_vp)]),
     "im_dof_pattern_destroy": (None, [_vp]),
     "im_dof_pattern_couple_bodies": (_i, [_vp, _vp, _i]),

@@ -131,7 +131,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     for ti in range(NT_):
         for tj in range(ti + 1):
             for v in range(4):
-                idx_rows.append([pos_of.get((16 * ti + 4 * (l // 16) + v, 16 * tj + l % 16), -1) for l in range(64)])
+                idx_rows.append([4 * pos_of.get((16 * ti + 4 * (l // 16) + v, 16 * tj + l % 16), nM) for l in range(64)])
     emit(f"static __device__ const short IDX_{name}[{len(idx_rows)}][64] = {{")
     for row in idx_rows:
         emit("  {" + ",".join(str(v) for v in row) + "},")
@@ -190,7 +190,18 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     emit("template <bool ASM, bool LONG>")
     emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? IM_OCC_{name} : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
     emit("  const int lane = threadIdx.x & 63, p = lane & 15, wv = threadIdx.x >> 6;")
-    emit("  const int w = blockIdx.x * 4 + (lane >> 4);")
+    # Several iterations in one launch (fused kernels only): the grid covers (four worlds, iteration)
+    # pairs.  Workgroups go to the chip's eight XCDs in turn, each with an L2 of its own, so the
+    # iterations of one group of worlds take consecutive workgroups of one XCD: they run at about
+    # the same time next to the same L2 and M and J come from memory once.
+    emit("  int bid = blockIdx.x;")
+    emit("  if (ASM && niter > 1) {")
+    emit("    const int slot = bid >> 3, it = slot % niter;")
+    emit("    bid = (slot / niter) * 8 + (bid & 7);")
+    emit("    if (bid * 4 >= nworld) return;  // the grid is rounded up to whole rounds of the XCDs")
+    emit("    state += it * state_it; y += it * y_it; x += it * x_it;")
+    emit("  }")
+    emit("  const int w = bid * 4 + (lane >> 4);")
     emit("  const bool live = w < nworld;")
     emit("  const int64_t ws = live ? w : nworld - 1;")
     # ---- right-hand side, uniform per world (wavefront 0 factors and solves)
@@ -207,18 +218,50 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         emit(f"    {{ const int ix = SVI_{name}[{svi_of[j, i, s_]}][p]; const float yv = yw[ix < 0 ? 0 : ix];"
              f" {var} = ix >= 0 ? yv : 0.0f; }}")
 
+    # The fused kernels read the right-hand side through the chain tables they hold anyway (lane p
+    # of a chain's vector = the dof at position p), every wavefront all vectors, right behind
+    # the requests for J and without a branch: a load under a role's branch is waited for inside
+    # the branch, ahead of everything that follows.  rhs_src[j, i, s_] = (index of the chain
+    # table row, lanes that take a right-hand side entry).
+    rhs_src = {}
+    for j, g in enumerate(groups):
+        for i, take in enumerate(segs[j]):
+            k_first = next(q for q in g if seg_of[q] == (j, i))
+            for s_ in range(vsets[j]):
+                mask = sum(1 << p for p in range(16) if take["fresh"].get(16 * s_ + p, -1) >= 0)
+                ci = leaf_sets.index((t.leaf_of[k_first], s_)) if (t.leaf_of[k_first], s_) in leaf_sets else None
+                if mask:
+                    assert ci is not None and all(tab[ci][p] == take["fresh"][16 * s_ + p] for p in range(16) if (mask >> p) & 1)
+                rhs_src[j, i, s_] = (ci, mask)
+    if len(trunk):
+        below = next(li for li, leaf in enumerate(t.leaves) if trunk[-1] in t.chain[leaf])
+        for s_ in range(tsets):
+            mask = sum(1 << p for p in range(16) if 16 * s_ + p < len(trunk))
+            ci = leaf_sets.index((below, s_))
+            assert all(tab[ci][p] == trunk[16 * s_ + p] for p in range(16) if (mask >> p) & 1)
+            rhs_src["T", 0, s_] = (ci, mask)
+    else:
+        for s_ in range(tsets):
+            rhs_src["T", 0, s_] = (None, 0)
+    rhs_tables = sorted({ci for ci, mask in rhs_src.values() if mask})
+    emit("  float " + ", ".join(f"yv{ci} = 0.0f" for ci in rhs_tables) + ";")
+
+    def take_rhs(j, i, s_, var):
+        ci, mask = rhs_src[j, i, s_]
+        emit(f"      {var} = " + (f"im_lane_select(yv{ci}, IM_ROW_MASK(0x{mask:x}));" if mask else "0.0f;"))
+
     for j in range(ngroups):
         names = [sv(j, i, s_) for i in range(len(segs[j])) for s_ in range(vsets[j])]
         names += [f"SY{j}_{i}_{s_}" for i in range(1, len(segs[j])) for s_ in range(vsets[j])]
         names += [f"SP{j}_{s_}" for s_ in range(vsets[j])]
         emit("  float " + ", ".join(f"{n_} = 0.0f" for n_ in names) + ";")
-        emit(f"  if (ROLE({j})) {{")
+        emit(f"  if (!ASM) {{")
         for i in range(len(segs[j])):
             for s_ in range(vsets[j]):
                 load_sv(j, i, s_, sv(j, 0, s_) if i == 0 else f"SY{j}_{i}_{s_}")
         emit("  }")
     emit("  float " + ", ".join(f"SVT_{s_} = 0.0f" for s_ in range(tsets)) + ";")
-    emit("  if (ROLE(0)) {")
+    emit("  if (!ASM) {")
     for s_ in range(tsets):
         load_sv("T", 0, s_, f"SVT_{s_}")
     emit("  }")
@@ -264,7 +307,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     xs_off = xoff
     lds_floats = xs_off + 4 * nv
     if EXP == "timing":
-        emit("  unsigned long long *tdbg = (unsigned long long *)Hout + (size_t)blockIdx.x * 16; int tn = 0;")
+        emit("  unsigned long long *tdbg = (unsigned long long *)Hout + (size_t)bid * 16; int tn = 0;")
         emit("  #define STAMP() do { if (threadIdx.x == 0) tdbg[tn] = clock64(); ++tn; } while (0)")
         emit("  STAMP();")
     else:
@@ -276,15 +319,21 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     emit("    const int kq = lane >> 4;")
     emit("    const int njp = (njmax + 15) & ~15;")
     emit(f"    float *dcl = lds + {lds_floats} + wv * (LONG ? njp : 128);  // D per row (0 where a row does not contribute)")
-    emit("    const int64_t wq = blockIdx.x * 4 + wv < nworld ? blockIdx.x * 4 + wv : nworld - 1;")
+    emit("    const int64_t wq = bid * 4 + wv < nworld ? bid * 4 + wv : nworld - 1;")
     emit("    int ne = nefc_p ? nefc_p[wq] : njmax; ne = ne < njmax ? ne : njmax;")
     emit("    ne = __builtin_amdgcn_readfirstlane(ne);")
     emit("    const int steps = (ne + 3) >> 2;")
     # every load below is unconditional (clamped address, value selected afterwards): a load
     # under a lane mask turns into a branch and a wait in the instruction stream
+    # J through a buffer descriptor over the world's njmax x nv block: the address of a load is a
+    # scalar base, one 32-bit lane offset and an immediate (no 64-bit arithmetic per load), and a
+    # row at or past njmax reads as zero without a clamp
+    emit("    const int wqs = __builtin_amdgcn_readfirstlane((int)wq);")
+    emit(f"    const __amdgpu_buffer_rsrc_t jrs = __builtin_amdgcn_make_buffer_rsrc((void *)(J + (int64_t)wqs * njmax * {nv}), (short)0, njmax * {4 * nv}, 0x00020000);")
     for c in range(NT):
         col = f"p + {16 * c}" if 16 * c + 16 <= nv else f"min(p + {16 * c}, {nv - 1})"
-        emit(f"    const float *pj{c} = J + wq * (int64_t)njmax * {nv} + {col};")
+        emit(f"    const int vc{c} = ({col}) * 4;            // byte offset of the lane's column")
+        emit(f"    const int vo{c} = kq * {4 * nv} + vc{c};  // ... within the step's four rows")
     emit("    const float *pd = dcl + kq;")
     for u in range(PD):
         emit("    float " + ", ".join(f"g{u}_{c}" for c in range(NT)) + ";")
@@ -292,17 +341,17 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     def load(u, step):
         # always issued, from a clamped row, so that the number of loads in flight is known at
         # compile time (a load under a condition makes every later wait a wait for all loads)
-        emit(f"        {{ const int row = ({step}) * 4 + kq; const int rowc = row < njmax ? row : njmax - 1;")
         for c in range(NT):
-            emit(f"          g{u}_{c} = pj{c}[rowc * {nv}];")
-        emit("        }")
+            emit(f"        g{u}_{c} = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(jrs, vo{c}, ({step}) * {16 * nv}, 0));")
 
-    def consume(u, step, valid=None):
+    def consume(u, step, listed=False):
         # rows at or past the world's nefc may hold anything: they count as zero rows; columns
-        # past nv repeat the last column, which only reaches accumulator elements outside H
-        emit(f"        {{ const int st = {step}; const float d = pd[st * 4]; const bool rv = {valid or 'st * 4 + kq < ne'};")
+        # past nv repeat the last column, which only reaches accumulator elements outside H.
+        # listed: the step's rows come from the list of contributing rows, whose spare entries
+        # name row 0 with weight 0 -- a row below nefc whenever a listed step runs at all
+        emit(f"        {{ const int st = {step}; const float d = pd[st * 4];" + ("" if listed else " const bool rv = st * 4 + kq < ne;"))
         for c in range(NT):
-            emit(f"          const float z{c} = rv ? g{u}_{c} : 0.0f;")
+            emit(f"          const float z{c} = " + (f"g{u}_{c};" if listed else f"rv ? g{u}_{c} : 0.0f;"))
         for c in range(NT):
             emit(f"          const float e{c} = d * z{c};")
         for n, (ti, tj) in enumerate(tiles):
@@ -313,10 +362,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     # accumulator index table, M (as a flat copy that is then gathered from LDS, so that the
     # table and M travel together instead of one after the other), the row weights; then J.
     MC = -(-nM // 64)
-    assert MC * 64 <= TW
+    assert MC * 64 <= TW and nM < TW and 4 * nM < 32768
     for n, (ti, tj) in enumerate(tiles):
         for v in range(4):
-            emit(f"    const int ix{n}_{v} = IDX_{name}[{n * 4 + v}][lane];")
+            emit(f"    const int ix{n}_{v} = IDX_{name}[{n * 4 + v}][lane];  // byte offset into the copy of M")
     # chain columns, needed right after the hand-over barrier: requested here, and pinned so that
     # the load is not moved down to its use
     for i in range(len(leaf_sets)):
@@ -343,9 +392,12 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     for u in range(SP):
         load(u, str(u))
     emit("    }")
+    for ci in rhs_tables:
+        emit(f"    yv{ci} = yw[chc{ci}];")
     emit(f"    float *mcopy = lds + wv * {TW};  // reused for this world's copy of H afterwards")
     for i in range(MC):
         emit(f"    mcopy[{i * 64} + lane] = mv{i};")
+    emit(f"    mcopy[{nM}] = 0.0f;  // where the table sends accumulator elements outside the pattern")
     emit("    if (LONG) {")
     emit("      if (lane < njp) dcl[lane] = (lane < ne && sv0 == quad) ? dv0 : 0.0f;")
     emit("      if (lane + 64 < njp) dcl[lane + 64] = (lane + 64 < ne && sv1 == quad) ? dv1 : 0.0f;")
@@ -365,16 +417,16 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     emit(f"      if (tail) {{ const int pos = {4 * SP} + __popcll(tm & ((1ull << lane) - 1ull)); dcl[pos] = dv0; rowl[pos] = lane; }}")
     emit("      IM_WAVE_SYNC();")
     for u in range(SP, PD):
-        emit(f"      {{ const int rowc = rowl[{4 * u} + kq];")
+        emit(f"      {{ const int rowb = rowl[{4 * u} + kq] * {4 * nv};")
         for c in range(NT):
-            emit(f"        g{u}_{c} = pj{c}[rowc * {nv}];")
+            emit(f"        g{u}_{c} = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(jrs, rowb + vc{c}, 0, 0));")
         emit("      }")
     emit("    }")
     emit("    IM_WAVE_SYNC();")
     for n in range(len(tiles)):
         emit(f"    f32x4 acc{n};")
         for v in range(4):
-            emit(f"    {{ const float mvv = mcopy[ix{n}_{v} < 0 ? 0 : ix{n}_{v}]; acc{n}[{v}] = ix{n}_{v} >= 0 ? mvv : 0.0f; }}")
+            emit(f"    acc{n}[{v}] = *(const float *)((const char *)mcopy + ix{n}_{v});")
     emit("    IM_WAVE_SYNC();")
     emit("    " + pin_ch)
     emit("    STAMP();  // 1: row weights staged, M gathered")
@@ -384,7 +436,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         if u < SP:
             consume(u, str(u))
         else:
-            consume(u, str(u), valid=f"{4 * u} + kq < {4 * SP} + cnt")
+            consume(u, str(u), listed=True)
         emit("      }")
     emit("    } else {")
     emit(f"    for (int s0 = 0; s0 < steps; s0 += {PD}) {{")
@@ -459,19 +511,21 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
                 for src in sorted(set(segs[j][i]["restore"].values())):
                     mask = sum(1 << p for p in range(16) if segs[j][i]["restore"].get(16 * s_ + p) == src)
                     if mask:
-                        expr = f"((0x{mask:x} >> p) & 1) ? {sv(j, src, s_)} : ({expr})"
+                        expr = f"im_lane_select2({sv(j, src, s_)}, {expr}, IM_ROW_MASK(0x{mask:x}))"
                 mask = sum(1 << p for p in range(16) if 16 * s_ + p in segs[j][i]["fresh"])
                 if mask:
-                    expr = f"((0x{mask:x} >> p) & 1) ? SY{j}_{i}_{s_} : ({expr})"
+                    expr = f"im_lane_select2(SY{j}_{i}_{s_}, {expr}, IM_ROW_MASK(0x{mask:x}))"
                 emit(f"    {sv(j, i, s_)} = {expr};")
-        emit(f"    d{k} = 1.0f / {bc(f'h{k}_{c // 16}', c % 16)};")
+        # the pivot's reciprocal is the head of the dependent chain from one pivot to the next: its
+        # operand is fetched first, the products below (which need the row only) fill its latency
+        emit(f"    const float piv{k} = {bc(f'h{k}_{c // 16}', c % 16)};")
         if c == 0:
+            emit(f"    d{k} = im_reciprocal(piv{k});")
             return
-        emit(f"    nd{k} = -d{k};")
         vec = (lambda s_: sv(*seg_of[k], s_)) if j is not None else (lambda s_: sv("T", 0, s_))
-        # products m_kp * m_kq for every target register, then the right-hand side update
+        # products m_kp * m_kq for every target register, the row eliminated next (the parent) first
         prods = []  # (pp, s, target)
-        for pp in range(c):
+        for pp in reversed(range(c)):
             a = t.anc[k][pp]
             to_acc = j is not None and a in trunk_set
             for s in range(t.sets(a)):
@@ -481,102 +535,193 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         nsv = (c - 1) // 16 + 1
         for s_ in range(nsv):
             hi = c - 16 * s_
-            emit(f"    const float hm{k}_{s_} = p < {hi} ? h{k}_{s_} : 0.0f;")
+            emit(f"    const float hm{k}_{s_} = " + (f"im_lane_select(h{k}_{s_}, IM_ROW_MASK(0x{(1 << hi) - 1:x}));" if hi < 16 else f"h{k}_{s_};"))
         if prods:
             emit("    float " + ", ".join(f"t{k}_{pp}_{s}" for pp, s, _ in prods) + ";")
-        # statement 1: T = h * nd, then as many products as fit; later statements: the rest
-        work = [("T", s) for s in range(nsv)] + [("P", pp, s) for pp, s, _ in prods] + [("R", s) for s in range(nsv)]
-        pos = 0
-        while pos < len(work):
-            o, n_in, lines = [], [], ["s_nop 1"]
-            num = {}
 
-            def use_in(tag, text):
-                if tag not in num:
-                    num[tag] = ("i", len(n_in))
-                    n_in.append(text)
-                return tag
-
-            items = []
+        def pack(work, weave_reciprocal=False):
+            """inline-assembly statements of at most 28 operands each for the listed items; with
+            weave_reciprocal the first statement also starts the pivot's reciprocal (hardware
+            estimate, residual, correction: im_reciprocal_fast) with the products in its latency"""
+            pos = 0
+            first = True
             while pos < len(work):
-                it = work[pos]
-                if it[0] == "T":
-                    need_i = (("hm", it[1]) not in num) + ("nd" not in num)
-                elif it[0] == "P":
-                    need_i = (("h", it[1] // 16) not in num) + (("h", it[2]) not in num)
-                else:
-                    need_i = (("Tin", it[1]) not in num and ("T", it[1]) not in num) + (("V", c // 16) not in num)
-                if len(o) + 1 + len(n_in) + need_i > 28:
-                    break
-                if it[0] == "T":
-                    s = it[1]
-                    num[("T", s)] = ("o", len(o))
-                    o.append(f'"=&v"(T{k}_{s})')
-                    use_in(("hm", s), f'"v"(hm{k}_{s})')
-                    use_in("nd", f'"v"(nd{k})')
-                elif it[0] == "P":
-                    _, pp, s = it
-                    num[("t", pp, s)] = ("o", len(o))
-                    o.append(f'"=&v"(t{k}_{pp}_{s})')
-                    use_in(("h", pp // 16), f'"v"(h{k}_{pp // 16})')
-                    use_in(("h", s), f'"v"(h{k}_{s})')
-                else:
-                    _, s = it
-                    if ("V", s) not in num:
-                        num[("V", s)] = ("o", len(o))
-                        o.append(f'"+v"({vec(s)})')
-                    if ("V", c // 16) not in num:
-                        num[("V", c // 16)] = ("o", len(o))
-                        o.append(f'"+v"({vec(c // 16)})')
-                    if ("T", s) not in num:
-                        use_in(("Tin", s), f'"v"(T{k}_{s})')
-                items.append(it)
-                pos += 1
+                # No wait states in front of these statements: a register they read through DPP was
+                # written at least two instructions earlier -- the pivot row by the update before the
+                # compiler's own DPP read of its diagonal, the right-hand side vector before the
+                # statement with the products
+                o, n_in, lines = [], [], []
+                num = {}
+                weave = weave_reciprocal and first
+                first = False
+                if weave:
+                    o += [f'"=&v"(df{k})', f'"=&v"(de{k})']
+                    num["df"], num["de"] = ("o", 0), ("o", 1)
+                    num["piv"] = ("i", 0)
+                    n_in.append(f'"v"(piv{k})')
 
-            def r_(tag):
-                kind, n = num[tag]
-                return f"%{n}" if kind == "o" else f"%{len(o) + n}"
+                def use_in(tag, text):
+                    if tag not in num:
+                        num[tag] = ("i", len(n_in))
+                        n_in.append(text)
+                    return tag
 
-            wrote_T_at = None
-            for it in items:
-                if it[0] == "T":
-                    lines.append(f"v_mul_f32 {r_(('T', it[1]))}, {r_(('hm', it[1]))}, {r_('nd')}")
-                    wrote_T_at = len(lines)
-                elif it[0] == "P":
-                    _, pp, s = it
-                    lines.append(f"v_mul_f32_dpp {r_(('t', pp, s))}, {r_(('h', pp // 16))}, {r_(('h', s))} row_newbcast:{pp % 16} {DPP}")
-                else:
-                    _, s = it
-                    tsrc = ("T", s) if ("T", s) in num else ("Tin", s)
-                    # entry of dof k (lane c of its set, untouched by this update) times T, added per lane
-                    lines.append(f"v_fmac_f32_dpp {r_(('V', s))}, {r_(('V', c // 16))}, {r_(tsrc)} row_newbcast:{c % 16} {DPP}")
-            text = "\\n\\t".join(lines)
-            emit(f'    asm("{text}" : {", ".join(o)} : {", ".join(n_in)});')
+                items = []
+                while pos < len(work):
+                    it = work[pos]
+                    if it[0] == "T":
+                        need_i = (("hm", it[1]) not in num) + ("nd" not in num)
+                    elif it[0] == "P":
+                        need_i = (("h", it[1] // 16) not in num) + (("h", it[2]) not in num)
+                    else:
+                        need_i = (("Tin", it[1]) not in num and ("T", it[1]) not in num) + (("V", c // 16) not in num)
+                    if len(o) + 1 + len(n_in) + need_i > 28:
+                        break
+                    if it[0] == "T":
+                        s = it[1]
+                        num[("T", s)] = ("o", len(o))
+                        o.append(f'"=&v"(T{k}_{s})')
+                        use_in(("hm", s), f'"v"(hm{k}_{s})')
+                        use_in("nd", f'"v"(nd{k})')
+                    elif it[0] == "P":
+                        _, pp, s = it
+                        num[("t", pp, s)] = ("o", len(o))
+                        o.append(f'"=&v"(t{k}_{pp}_{s})')
+                        use_in(("h", pp // 16), f'"v"(h{k}_{pp // 16})')
+                        use_in(("h", s), f'"v"(h{k}_{s})')
+                    else:
+                        _, s = it
+                        if ("V", s) not in num:
+                            num[("V", s)] = ("o", len(o))
+                            o.append(f'"+v"({vec(s)})')
+                        if ("V", c // 16) not in num:
+                            num[("V", c // 16)] = ("o", len(o))
+                            o.append(f'"+v"({vec(c // 16)})')
+                        if ("T", s) not in num:
+                            use_in(("Tin", s), f'"v"(T{k}_{s})')
+                    items.append(it)
+                    pos += 1
+
+                def r_(tag):
+                    kind, n = num[tag]
+                    return f"%{n}" if kind == "o" else f"%{len(o) + n}"
+
+                body = []
+                for it in items:
+                    if it[0] == "T":
+                        body.append(f"v_mul_f32 {r_(('T', it[1]))}, {r_(('hm', it[1]))}, {r_('nd')}")
+                    elif it[0] == "P":
+                        _, pp, s = it
+                        body.append(f"v_mul_f32_dpp {r_(('t', pp, s))}, {r_(('h', pp // 16))}, {r_(('h', s))} row_newbcast:{pp % 16} {DPP}")
+                    else:
+                        _, s = it
+                        tsrc = ("T", s) if ("T", s) in num else ("Tin", s)
+                        # entry of dof k (lane c of its set, untouched by this update) times T, added per lane
+                        body.append(f"v_fmac_f32_dpp {r_(('V', s))}, {r_(('V', c // 16))}, {r_(tsrc)} row_newbcast:{c % 16} {DPP}")
+                if weave:
+                    # estimate first, the residual after four products, the correction after two more;
+                    # a transcendental's result needs two instructions' distance before its first use
+                    n_e, n_r = min(4, len(body)), min(6, len(body))
+                    # of the negated pivot: -1 / pivot is what the updates multiply with
+                    body[n_r:n_r] = [f"v_fma_f32 {r_('df')}, {r_('de')}, {r_('df')}, {r_('df')}"]
+                    body[n_e:n_e] = (["s_nop 1"] if n_e < 2 else []) + [f"v_fma_f32 {r_('de')}, {r_('piv')}, {r_('df')}, 1.0"]
+                    body.insert(0, f"v_rcp_f32_e64 {r_('df')}, -{r_('piv')}")
+                lines += body
+                text = "\\n\\t".join(lines)
+                emit(f'    asm("{text}" : {", ".join(o)} : {", ".join(n_in)});')
+
+        emit(f"    float df{k}, de{k};")
+        pack([("P", pp, s) for pp, s, _ in prods], weave_reciprocal=True)
+        emit(f"    nd{k} = im_negative_reciprocal_checked(piv{k}, df{k});")
+        emit(f"    d{k} = -nd{k};")
         for pp, s, tgt in prods:
             emit(f"    {tgt} = IM_FMA(t{k}_{pp}_{s}, nd{k}, {tgt});")
+        # T = h * nd and the right-hand side update
+        pack([("T", s) for s in range(nsv)] + [("R", s) for s in range(nsv)])
 
-    def backsub(b):
-        # u_b = u_b d_b, then u_b += T_b[p] u_anc_p for p ascending (tree_ldl.py:298-304); the
-        # entry of dof b is lane c of its chain's right-hand side vector
-        c = t.depth[b]
-        src = sv(seg_of[b][0], home[seg_of[b][0]]["g", b], c // 16) if b in seg_of else sv("T", 0, c // 16)
-        if c == 0:
-            emit(f"    S{b} = {bc(src, 0)} * d{b};")
-            return
-        for p0 in range(0, c, 24):
-            pps = list(range(p0, min(c, p0 + 24)))
-            sets_used = sorted({pp // 16 for pp in pps})
-            first = p0 == 0
-            o = [f'"=&v"(S{b})' if first else f'"+v"(S{b})']
-            n_in = [f'"v"(T{b}_{s})' for s in sets_used] + [f'"v"(S{t.anc[b][pp]})' for pp in pps]
-            lines = ["s_nop 1"]
-            if first:
-                n_in += [f'"v"({src})', f'"v"(d{b})']
-                lines.append(f"v_mul_f32_dpp %0, %{len(n_in) - 1}, %{len(n_in)} row_newbcast:{c % 16} {DPP}")
-            for n, pp in enumerate(pps):
-                lines.append(f"v_fmac_f32_dpp %0, %{1 + sets_used.index(pp // 16)}, %{1 + len(sets_used) + n} row_newbcast:{pp % 16} {DPP}")
-            text = "\\n\\t".join(lines)
-            emit(f'    asm("{text}" : {", ".join(o)} : {", ".join(n_in)});')
+    def backsub_many(dofs):
+        """Solutions of `dofs` (ancestors first): u_b = u_b d_b, then u_b += T_b[p] u_anc_p for p
+        ascending (tree_ldl.py:298-304); the entry of dof b is lane c of its chain's right-hand side
+        vector.  A dof's sum is a chain of dependent instructions, so the chains of all dofs are
+        emitted interleaved, a term as soon as the ancestor it needs is complete: the order of
+        each dof's own terms is untouched."""
+        dofs = list(dofs)
+        inset = set(dofs)
+        emitted = {b: -1 for b in dofs}  # -1: the product with d_b is still to come
+        complete, seq = set(), []
+        while len(complete) < len(dofs):
+            newly = []
+            for b in dofs:
+                if b in complete or b in newly:
+                    continue
+                if emitted[b] == -1:
+                    seq.append((b, None))
+                    emitted[b] = 0
+                else:
+                    a_ = t.anc[b][emitted[b]]
+                    if a_ in inset and a_ not in complete:
+                        continue
+                    seq.append((b, emitted[b]))
+                    emitted[b] += 1
+                if emitted[b] == t.depth[b]:
+                    newly.append(b)
+            assert newly or any(True for _ in seq)
+            complete.update(newly)
+
+        def src_of(b_):
+            c_ = t.depth[b_]
+            return sv(seg_of[b_][0], home[seg_of[b_][0]]["g", b_], c_ // 16) if b_ in seg_of else sv("T", 0, c_ // 16)
+
+        pos, first_stmt = 0, True
+        while pos < len(seq):
+            outs, ins, lines = {}, {}, (["s_nop 1"] if first_stmt else [])
+            first_stmt = False
+
+            def need(b_, pp):
+                names = [("o", f"S{b_}")]
+                if pp is None:
+                    names += [("i", src_of(b_)), ("i", f"d{b_}")]
+                else:
+                    names += [("i", f"T{b_}_{pp // 16}"), ("oi", f"S{t.anc[b_][pp]}")]
+                return names
+
+            while pos < len(seq):
+                b_, pp = seq[pos]
+                extra = 0
+                for kind, nm in need(b_, pp):
+                    if nm in outs or nm in ins:
+                        continue
+                    extra += 1
+                if len(outs) + len(ins) + extra > 26 and (outs or ins):
+                    break
+                for kind, nm in need(b_, pp):
+                    if nm in outs or nm in ins:
+                        continue
+                    if kind == "o":
+                        outs[nm] = None
+                    else:
+                        ins[nm] = None
+                pos += 1
+                lines.append((b_, pp))
+            # an S read before this statement writes it is an input-output as well: "+v" covers both
+            olist = list(outs)
+            ilist = [nm for nm in ins if nm not in outs]
+            ref = {nm: f"%{n}" for n, nm in enumerate(olist)}
+            ref.update({nm: f"%{len(olist) + n}" for n, nm in enumerate(ilist)})
+            text = []
+            for item in lines:
+                if isinstance(item, str):
+                    text.append(item)
+                    continue
+                b_, pp = item
+                if pp is None:
+                    text.append(f"v_mul_f32_dpp {ref[f'S{b_}']}, {ref[src_of(b_)]}, {ref[f'd{b_}']} row_newbcast:{t.depth[b_] % 16} {DPP}")
+                else:
+                    text.append(f"v_fmac_f32_dpp {ref[f'S{b_}']}, {ref[f'T{b_}_{pp // 16}']}, {ref[f'S{t.anc[b_][pp]}']} row_newbcast:{pp % 16} {DPP}")
+            joined = "\\n\\t".join(text)
+            o_txt = ", ".join('"+v"(%s)' % nm for nm in olist)
+            i_txt = ", ".join('"v"(%s)' % nm for nm in ilist)
+            emit(f'    asm("{joined}" : {o_txt} : {i_txt});')
 
     def store_x(dofs):
         emit("    if (live && p == 0) {")
@@ -593,6 +738,11 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     # ---- phase 1: the groups, each into its own zero-initialised trunk accumulators
     for j, g in enumerate(groups):
         emit(f"  if (ROLE({j})) {{  // group {j}")
+        emit("    if (ASM) {")
+        for i in range(len(segs[j])):
+            for s_ in range(vsets[j]):
+                take_rhs(j, i, s_, sv(j, 0, s_) if i == 0 else f"SY{j}_{i}_{s_}")
+        emit("    }")
         fetch_rows(sorted(g))
         if j == 0:
             emit("    STAMP();  // group 0: rows fetched")
@@ -608,7 +758,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
                     by_src.setdefault(home[j]["t", a_], 0)
                     by_src[home[j]["t", a_]] |= 1 << (t.depth[a_] % 16)
             for src, mask in sorted(by_src.items()):
-                expr = f"((0x{mask:x} >> p) & 1) ? {sv(j, src, s_)} : ({expr})"
+                expr = f"im_lane_select2({sv(j, src, s_)}, {expr}, IM_ROW_MASK(0x{mask:x}))"
             emit(f"    SP{j}_{s_} = {expr};")
         emit("    if (ASM) {")
         for (a, s_), off in xslots[j].items():
@@ -621,6 +771,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     # ---- phase 2: trunk rows = own value plus the groups' contributions in group order
     # (tree_ldl.py:274-289), eliminated in reverse, then solved root first
     emit("  if (ROLE(0)) {  // trunk")
+    emit("    if (ASM) {")
+    for s_ in range(tsets):
+        take_rhs("T", 0, s_, f"SVT_{s_}")
+    emit("    }")
     fetch_rows(list(trunk))
     for a in trunk:
         for j in range(ngroups):
@@ -632,13 +786,12 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         for s_ in range(min(tsets, vsets[j])):
             mask = sum(1 << p for p in range(16) if any(t.depth[a] == 16 * s_ + p for a in touched[j]))
             if mask:
-                emit(f"    SVT_{s_} = ((0x{mask:x} >> p) & 1) ? SVT_{s_} + (ASM ? xlds[{xslots[j]['S', s_]} + lane] : SP{j}_{s_}) : SVT_{s_};")
+                emit(f"    SVT_{s_} = im_lane_select2(SVT_{s_} + (ASM ? xlds[{xslots[j]['S', s_]} + lane] : SP{j}_{s_}), SVT_{s_}, IM_ROW_MASK(0x{mask:x}));")
     emit("    STAMP();  // trunk: rows fetched and merged")
     for k in reversed(trunk):
         eliminate(k, None)
     emit("    STAMP();  // trunk: eliminated")
-    for b in trunk:
-        backsub(b)
+    backsub_many(trunk)
     emit("    STAMP();  // trunk: solved")
     emit("    if (ASM && p == 0) {")
     for b in trunk:
@@ -656,8 +809,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             for a in sorted(touched[j]):
                 emit(f"      S{a} = xlds[{xs_off} + (lane >> 4) * {nv} + {a}];")
             emit("    }")
-        for b in reversed(g):
-            backsub(b)
+        backsub_many(list(reversed(g)))
         store_x(sorted(g))
         emit("  }")
     emit("  STAMP();")

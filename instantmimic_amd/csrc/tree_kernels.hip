@@ -327,10 +327,32 @@ int round_nvp(int nv) {
   return 0;
 }
 
+// Every float whose bit pattern lies in [first, last]: does the short reciprocal of the pivot
+// chain (tree_row16.h) give the bits of the division?  In-range values must, the others are
+// counted only when they claim to be in range.
+__global__ void check_reciprocal_kernel(uint32_t first, uint32_t last, unsigned long long *mismatches) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  unsigned long long bad = 0;
+  for (uint64_t u = (uint64_t)first + blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; u <= last; u += stride) {
+    const float x = __builtin_bit_cast(float, (uint32_t)u);
+    if (!gen::im_reciprocal_in_range(x)) continue;
+    bad += __builtin_bit_cast(uint32_t, gen::im_reciprocal_fast(x)) != __builtin_bit_cast(uint32_t, 1.0f / x);
+  }
+  if (bad) atomicAdd(mismatches, bad);
+}
+
+// One launch of the generated kernels for `niter` iterations (see the kernels' prologue); the
+// table-driven kernel takes one iteration at a time.
+struct Iterations {
+  int niter = 1;
+  int64_t state_it = 0, y_it = 0, x_it = 0;
+};
+
 int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
            const float *J, int njmax, const float *D, const int32_t *state,
            const int32_t *nefc, int quad, const float *y, int64_t ldy, float *x,
-           int64_t ldx, float *Hout, int nworld, unsigned flags, void *stream) {
+           int64_t ldx, float *Hout, int nworld, unsigned flags, void *stream,
+           Iterations its = Iterations()) {
   if (!plan || nworld < 0) return IM_ERR_ARG;
   if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
   if (nworld == 0) return IM_OK;
@@ -340,16 +362,28 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
   if (assemble && (!J || !D || !state || njmax <= 0)) return IM_ERR_ARG;
   if (plan->row16) {
     const auto *e = (const gen::Row16Entry *)plan->row16;
-    void *args[] = {&M, &ldM, &J, &njmax, &D, &state, &nefc, &quad, &y, &ldy, &x, &ldx, &Hout, &nworld, &flags};
+    void *args[] = {&M,     &ldM,      &J,         &njmax,        &D,        &state,   &nefc,
+                    &quad,  &y,        &ldy,       &x,            &ldx,      &Hout,    &nworld,
+                    &flags, &its.niter, &its.state_it, &its.y_it, &its.x_it};
     // staged rows plus the four worlds' active-row lists (row id and D per constraint row)
     const size_t lds = assemble ? (size_t)e->lds_bytes + 32 * std::max<size_t>(((size_t)njmax + 15) / 16 * 16, 64) : 0;
     if (lds <= 160 * 1024) {
       // fused: one wavefront per world assembles, the first one factors and solves all four
       const void *fn = !assemble ? e->solve : (njmax <= e->short_rows ? e->fused : e->fused_long);
-      IM_HIP_CHECK(hipLaunchKernel(fn, dim3((nworld + 3) / 4),
-                                   dim3(assemble ? 256 : 64), args, lds, (hipStream_t)stream));
+      // several iterations: whole rounds of the eight XCDs per iteration (spare workgroups exit)
+      const unsigned quads = (unsigned)((nworld + 3) / 4);
+      const unsigned grid = its.niter > 1 ? (quads + 7) / 8 * 8 * (unsigned)its.niter : quads;
+      IM_HIP_CHECK(hipLaunchKernel(fn, dim3(grid), dim3(assemble ? 256 : 64), args, lds, (hipStream_t)stream));
       return IM_OK;
     }
+  }
+  if (its.niter > 1) {  // the table-driven kernel: one launch per iteration
+    for (int it = 0; it < its.niter; ++it) {
+      const int st = launch(plan, assemble, M, ldM, J, njmax, D, state + it * its.state_it, nefc, quad,
+                            y + it * its.y_it, ldy, x + it * its.x_it, ldx, nullptr, nworld, flags, stream);
+      if (st != IM_OK) return st;
+    }
+    return IM_OK;
   }
   const int nv = plan->nv, nM = plan->nM;
   const int nvp = round_nvp(nv);
@@ -470,6 +504,36 @@ int im_tree_factor_solve(const im_tree_plan *plan, const float *M, int64_t ldM,
                          int nworld, void *stream) {
   return im::launch(plan, false, M, ldM, nullptr, 0, nullptr, nullptr, nullptr, 0, y, ldy,
                     x, ldx, nullptr, nworld, 0u, stream);
+}
+
+int im_check_reciprocal(uint32_t first_bits, uint32_t last_bits, unsigned long long *mismatches, void *stream) {
+  if (!mismatches || last_bits < first_bits) return IM_ERR_ARG;
+  hipLaunchKernelGGL(im::check_reciprocal_kernel, dim3(4096), dim3(256), 0, (hipStream_t)stream, first_bits, last_bits,
+                     mismatches);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_assemble_tree_ldl_solve_iters(const im_tree_plan *plan, const float *M, int64_t ldM, const float *J,
+                                     int njmax, const float *D, const int32_t *state, int64_t state_iter_stride,
+                                     const int32_t *nefc, int quad, const float *grad, int64_t ldg,
+                                     int64_t grad_iter_stride, float *x, int64_t ldx, int64_t x_iter_stride,
+                                     int nworld, int niter, unsigned flags, void *stream) {
+  if (!plan || nworld < 0 || niter < 0 || state_iter_stride < 0 || grad_iter_stride < 0 || x_iter_stride < 0)
+    return IM_ERR_ARG;
+  if (niter > 1 && (state_iter_stride < (int64_t)nworld * njmax || x_iter_stride < (int64_t)(nworld - 1) * ldx + plan->nv))
+    return IM_ERR_STRIDE;  // iterations must not overlap
+  if (niter == 0 || nworld == 0) return IM_OK;
+  if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
+  if (!M || !grad || !x || !J || !D || !state || njmax <= 0) return IM_ERR_ARG;
+  if (ldM < plan->nM || ldg < plan->nv || ldx < plan->nv) return IM_ERR_STRIDE;
+  im::Iterations its;
+  its.niter = niter;
+  its.state_it = state_iter_stride;
+  its.y_it = grad_iter_stride;
+  its.x_it = x_iter_stride;
+  return im::launch(plan, true, M, ldM, J, njmax, D, state, nefc, quad, grad, ldg, x, ldx, nullptr, nworld, flags,
+                    stream, its);
 }
 
 int im_assemble_tree_ldl_solve(const im_tree_plan *plan, const float *M, int64_t ldM,

@@ -267,3 +267,44 @@ def assemble_tree_factor_solve(
             _lib.IM_FLAG_NEGATE if negate else 0, _stream_ptr(M),
         )  # fmt: skip
     _lib.check(status, "im_assemble_tree_ldl_solve")
+
+
+def assemble_tree_factor_solve_iters(
+    scratch: TreeFactorSolveScratch, M, J, D, states, nefc, grad, x, *, negate: bool = False, quad: int = QUADRATIC
+) -> None:
+    """``niter`` Newton linear steps that share ``M``, ``J`` and ``D``: ``states`` (niter, nworld,
+    njmax) int32, ``x`` (niter, nworld, nv); ``grad`` is (nworld, nv) for one gradient or (niter,
+    nworld, nv).  Same results as ``niter`` calls of :func:`assemble_tree_factor_solve``; one
+    launch that reads ``M`` and ``J`` once where the library has a generated kernel for the tree."""
+    import torch
+
+    if states.dim() != 3 or x.dim() != 3 or states.shape[0] != x.shape[0]:
+        raise ValueError("states must be (niter, nworld, njmax) and x (niter, nworld, nv)")
+    niter = int(states.shape[0])
+    grad0 = grad[0] if grad.dim() == 3 else grad
+    if grad.dim() == 3 and grad.shape[0] != niter:
+        raise ValueError("grad must be (nworld, nv) or (niter, nworld, nv)")
+    _check_rows(M, x[0], grad0)
+    if J.dim() != 3 or not J.is_contiguous() or not D.is_contiguous() or not states.is_contiguous():
+        raise ValueError("J, D and states must be contiguous")
+    if states.dtype != torch.int32 or (nefc is not None and nefc.dtype != torch.int32):
+        raise TypeError("states and nefc must be int32")
+    for t in (M, J, D, grad, x):
+        if t.dtype != torch.float32 or not t.is_cuda:
+            raise TypeError("assemble_tree_factor_solve_iters needs float32 CUDA tensors")
+    njmax, nv = int(J.shape[1]), int(J.shape[2])
+    nworld = _check_against_plan(scratch, M, x[0], grad0, (J, D, states[0], nefc))
+    if nv != scratch.kernel.info().nv or njmax < 1:
+        raise ValueError("J must be (nworld, njmax >= 1, nv) with the plan's nv")
+    if tuple(D.shape) != (nworld, njmax) or tuple(states.shape[1:]) != (nworld, njmax) or (nefc is not None and nefc.numel() != nworld):
+        raise ValueError("D must be (nworld, njmax), states (niter, nworld, njmax), nefc (nworld,)")
+    if x.stride(2) != 1 or (grad.dim() == 3 and grad.stride(2) != 1):
+        raise ValueError("rows of x and grad must be contiguous floats")
+    with torch.cuda.device(M.device):
+        status = _lib.lib().im_assemble_tree_ldl_solve_iters(
+            scratch.kernel.ptr, M.data_ptr(), M.stride(0), J.data_ptr(), njmax, D.data_ptr(), states.data_ptr(),
+            states.stride(0), nefc.data_ptr() if nefc is not None else None, int(quad), grad.data_ptr(),
+            grad0.stride(0), grad.stride(0) if grad.dim() == 3 else 0, x.data_ptr(), x.stride(1), x.stride(0),
+            int(nworld), niter, _lib.IM_FLAG_NEGATE if negate else 0, _stream_ptr(M),
+        )  # fmt: skip
+    _lib.check(status, "im_assemble_tree_ldl_solve_iters")

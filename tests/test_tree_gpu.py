@@ -199,3 +199,47 @@ def test_ineligible_models_return_none(device):
     m = type("m", (), dict(nv=len(rowadr), M_rowadr=rowadr, M_rownnz=rownnz, M_colind=colind))
     assert T.create_tree_factor_solve_scratch(m, device) is None
     assert T.create_tree_factor_solve_scratch(type("m", (), dict(nv=0)), device) is None
+
+
+@pytest.mark.parametrize("name,nworld,niter,ragged,per_iter_grad", [
+    ("humanoid", 4096, 3, False, False), ("humanoid", 333, 5, True, True), ("ant", 65, 3, True, False),
+    ("g1", 257, 3, True, True), ("snu", 130, 2, True, False), ("humanoid", 7, 1, True, False),
+])  # fmt: skip
+def test_iterations_in_one_call_match_the_oracle_bitwise(device, name, nworld, niter, ragged, per_iter_grad):
+    """im_assemble_tree_ldl_solve_iters: the iterations of a step share M, J and D; every iteration
+    assembles afresh, so each equals the single call (and the oracle) bit for bit -- on the
+    kernel that keeps J in registers (humanoid, ant: up to 64 rows) and on the launch-per-iteration
+    path behind the same entry point (g1: 96 rows, snu: 128 rows, niter = 1)."""
+    import torch
+
+    from instantmimic_amd.mjw_kernels import tree_ldl as T
+
+    b = synth.make_batch(name, nworld, ragged_nefc=ragged)
+    rng = np.random.default_rng(3)
+    states = np.stack([np.where(rng.random(b.state[0].shape) < 0.6, synth.QUADRATIC, 0).astype(np.int32) for _ in range(niter)])
+    grads = rng.normal(size=(niter, nworld, b.shape.nv)).astype(np.float32) if per_iter_grad else b.grad
+    scratch = T.create_tree_factor_solve_scratch(_model(b), device)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    x = torch.full((niter, nworld, b.shape.nv), float("nan"), device=device)
+    T.assemble_tree_factor_solve_iters(scratch, t(b.M), t(b.J), t(b.D), t(states), t(b.nefc), t(grads), x, negate=True)
+    torch.cuda.synchronize()
+    st = P.tree_ldl_structure(b.rowadr, b.rownnz, b.colind)
+    plan = P.best_tree_ldl_plan(*st)
+    for it in range(niter):
+        g = grads[it] if per_iter_grad else grads
+        x_ref = R.assemble_tree_ldl_solve(*st, plan, b.M, b.J, b.D, states[it], b.nefc, g)
+        np.testing.assert_array_equal(x[it].cpu().numpy(), -x_ref, err_msg=f"iteration {it}")
+
+
+def test_short_reciprocal_equals_the_division_for_every_float_in_its_range(device):
+    """The pivot chain of the generated kernels replaces 1.0f / x by the hardware estimate and one
+    exact-residual correction inside 2^-101 <= |x| < 2^102: all 3.4e9 such floats, both signs."""
+    import torch
+
+    from instantmimic_amd import _lib
+
+    count = torch.zeros(1, dtype=torch.int64, device=device)
+    stream = int(torch.cuda.current_stream(device).cuda_stream)
+    assert _lib.lib().im_check_reciprocal(0, 0xFFFFFFFF, count.data_ptr(), stream) == _lib.IM_OK
+    torch.cuda.synchronize()
+    assert int(count.item()) == 0
