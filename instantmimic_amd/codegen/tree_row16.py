@@ -494,7 +494,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             for s in range(t.sets(a)):
                 emit(f"  float ga{j}_{a}_{s} = 0.0f;")
     for k in range(nv):
-        emit(f"  float d{k} = 0.0f;" if not t.depth[k] else f"  float d{k} = 0.0f, nd{k} = 0.0f;")
+        emit(f"  float nd{k} = 0.0f;  // -1 / pivot")
         if t.depth[k]:
             emit("  float " + ", ".join(f"T{k}_{s} = 0.0f" for s in range(t.sets(k))) + ";")
 
@@ -520,7 +520,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         # operand is fetched first, the products below (which need the row only) fill its latency
         emit(f"    const float piv{k} = {bc(f'h{k}_{c // 16}', c % 16)};")
         if c == 0:
-            emit(f"    d{k} = im_reciprocal(piv{k});")
+            emit(f"    nd{k} = im_negative_reciprocal_checked(piv{k}, im_reciprocal_fast(-piv{k}));")
             return
         vec = (lambda s_: sv(*seg_of[k], s_)) if j is not None else (lambda s_: sv("T", 0, s_))
         # products m_kp * m_kq for every target register, the row eliminated next (the parent) first
@@ -631,11 +631,17 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
                 emit(f'    asm("{text}" : {", ".join(o)} : {", ".join(n_in)});')
 
         emit(f"    float df{k}, de{k};")
-        pack([("P", pp, s) for pp, s, _ in prods], weave_reciprocal=True)
+        # eight products at a time, each batch followed by its updates: the temporaries of a deep
+        # row would otherwise all be live at once
+        BATCH = 8
+        pack([("P", pp, s) for pp, s, _ in prods[:BATCH]], weave_reciprocal=True)
         emit(f"    nd{k} = im_negative_reciprocal_checked(piv{k}, df{k});")
-        emit(f"    d{k} = -nd{k};")
-        for pp, s, tgt in prods:
+        for pp, s, tgt in prods[:BATCH]:
             emit(f"    {tgt} = IM_FMA(t{k}_{pp}_{s}, nd{k}, {tgt});")
+        for b0 in range(BATCH, len(prods), BATCH):
+            pack([("P", pp, s) for pp, s, _ in prods[b0 : b0 + BATCH]])
+            for pp, s, tgt in prods[b0 : b0 + BATCH]:
+                emit(f"    {tgt} = IM_FMA(t{k}_{pp}_{s}, nd{k}, {tgt});")
         # T = h * nd and the right-hand side update
         pack([("T", s) for s in range(nsv)] + [("R", s) for s in range(nsv)])
 
@@ -680,7 +686,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             def need(b_, pp):
                 names = [("o", f"S{b_}")]
                 if pp is None:
-                    names += [("i", src_of(b_)), ("i", f"d{b_}")]
+                    names += [("i", src_of(b_)), ("i", f"nd{b_}")]
                 else:
                     names += [("i", f"T{b_}_{pp // 16}"), ("oi", f"S{t.anc[b_][pp]}")]
                 return names
@@ -715,7 +721,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
                     continue
                 b_, pp = item
                 if pp is None:
-                    text.append(f"v_mul_f32_dpp {ref[f'S{b_}']}, {ref[src_of(b_)]}, {ref[f'd{b_}']} row_newbcast:{t.depth[b_] % 16} {DPP}")
+                    text.append(f"v_mul_f32_dpp {ref[f'S{b_}']}, {ref[src_of(b_)]}, -{ref[f'nd{b_}']} row_newbcast:{t.depth[b_] % 16} {DPP}")
                 else:
                     text.append(f"v_fmac_f32_dpp {ref[f'S{b_}']}, {ref[f'T{b_}_{pp // 16}']}, {ref[f'S{t.anc[b_][pp]}']} row_newbcast:{pp % 16} {DPP}")
             joined = "\\n\\t".join(text)
@@ -736,8 +742,12 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         emit("    }")
 
     # ---- phase 1: the groups, each into its own zero-initialised trunk accumulators
+    # Each role's work is a lambda per phase, called from one branch per wavefront below: a
+    # wavefront's path through the kernel then holds its own role's values only (with the roles
+    # as guarded blocks one after the other, every role's values stay allocated across the others' code).
+    LAMBDA = "[&]() __attribute__((always_inline))"
     for j, g in enumerate(groups):
-        emit(f"  if (ROLE({j})) {{  // group {j}")
+        emit(f"  auto phase1_{j} = {LAMBDA} {{  // group {j}")
         emit("    if (ASM) {")
         for i in range(len(segs[j])):
             for s_ in range(vsets[j]):
@@ -765,12 +775,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             src = f"SP{j}_{s_}" if a == "S" else f"ga{j}_{a}_{s_}"
             emit(f"      xlds[{off} + lane] = {src};")
         emit("    }")
-        emit("  }")
-    emit("  if (ASM) __syncthreads();")
-    emit("  STAMP();  // groups eliminated")
+        emit("  };")
     # ---- phase 2: trunk rows = own value plus the groups' contributions in group order
     # (tree_ldl.py:274-289), eliminated in reverse, then solved root first
-    emit("  if (ROLE(0)) {  // trunk")
+    emit(f"  auto phase2 = {LAMBDA} {{  // trunk")
     emit("    if (ASM) {")
     for s_ in range(tsets):
         take_rhs("T", 0, s_, f"SVT_{s_}")
@@ -798,12 +806,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         emit(f"      xlds[{xs_off} + (lane >> 4) * {nv} + {b}] = S{b};")
     emit("    }")
     store_x(list(trunk))
-    emit("  }")
-    emit("  if (ASM) __syncthreads();")
-    emit("  STAMP();  // trunk solved")
+    emit("  };")
     # ---- phase 3: the groups' solutions, ancestors first
     for j, g in enumerate(groups):
-        emit(f"  if (ROLE({j})) {{")
+        emit(f"  auto phase3_{j} = {LAMBDA} {{")
         if j != 0:
             emit("    if (ASM) {")
             for a in sorted(touched[j]):
@@ -811,7 +817,32 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
             emit("    }")
         backsub_many(list(reversed(g)))
         store_x(sorted(g))
-        emit("  }")
+        emit("  };")
+    emit("  if (ASM) {")
+    for j in range(max(ngroups, 1)):
+        emit(("    if" if j == 0 else "    } else if") + f" (wv == {j}) {{")
+        if j < ngroups:
+            emit(f"      phase1_{j}();")
+        emit("      IM_BLOCK_SYNC();")
+        if j == 0:
+            emit("      STAMP();  // groups eliminated")
+            emit("      phase2();")
+        emit("      IM_BLOCK_SYNC();")
+        if j == 0:
+            emit("      STAMP();  // trunk solved")
+        if j < ngroups:
+            emit(f"      phase3_{j}();")
+    emit("    } else {  // a wavefront without a group only keeps the barriers' count")
+    emit("      IM_BLOCK_SYNC();")
+    emit("      IM_BLOCK_SYNC();")
+    emit("    }")
+    emit("  } else {")
+    for j in range(ngroups):
+        emit(f"    phase1_{j}();")
+    emit("    phase2();")
+    for j in range(ngroups):
+        emit(f"    phase3_{j}();")
+    emit("  }")
     emit("  STAMP();")
     emit("  #undef STAMP")
     emit("}")
@@ -823,6 +854,6 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     # workgroups per CU that the fused kernel is compiled for: what the 160 KB of LDS admit (with
     # the lists of 128 constraint rows), at most 4 -- fewer workgroups leave each wavefront more
     # registers, which the larger trees need
-    occ = max(1, min(4, (160 * 1024) // (lds_floats * 4 + 32 * 128)))
+    occ = max(1, min(int(os.environ.get("IMHIP_OCC", "4")), (160 * 1024) // (lds_floats * 4 + 32 * 128)))
     text = "\n".join(out) + "\n"
     return text.replace('#include "../tree_row16.h"', f'#include "../tree_row16.h"\n#define IM_OCC_{name} {occ}', 1)
