@@ -3,11 +3,13 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A step is one pass of the hot path over one synthetic batch of the headline
-shape: humanoid, nv = 27, nefc = 64, 4096 worlds, three Newton iterations (three
-launches, each with its own active mask).  Inputs are resident in HBM before the
-timed region; the steps rotate over enough distinct input sets (> 512 MB) that
-reads cannot be served by the 256 MB last-level cache.  Prints one JSON line.
+A step is one pass of the hot path over one synthetic batch of the headline shape: humanoid,
+nv = 27, nefc = 64, 4096 worlds, three Newton iterations with a fresh active mask each -- one
+call of im_assemble_tree_ldl_solve_iters (one launch whose grid covers worlds x iterations).
+Inputs are resident in HBM before the timed region; every step takes the next of 16 distinct
+input sets (> 560 MB in rotation), so no launch finds its M or J in the 256 MB memory-side cache.
+Beside the headline the same batch is timed as three launches of im_assemble_tree_ldl_solve per
+step, each launch on an input set of its own (`single_launch`).  Prints one JSON line.
 """
 
 from __future__ import annotations
@@ -24,12 +26,12 @@ if ROOT not in sys.path:
 
 METRIC = "Hessian assemble+LDL+solve worlds/s, humanoid nv=27×4096; % HBM roofline"
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-# HBM bytes per launch of the fused kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then
-# WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for a plain
-# 64 MiB device copy in the same run (FETCH_SIZE reads 32781 KiB for it, WRITE_SIZE 65536):
-#   (15862.14 * 65536 / 32781.48 + 448.0 * 65536 / 65536) KiB
-# Recorded in profiles/tree_row16_humanoid_pmc.txt.
-TRAFFIC_BYTES_PER_LAUNCH = int((15854.27 * 65536 / 32781.46 + 448.0) * 1024)
+# HBM bytes per launch of the iterations kernel (3 solves x 4096 worlds) from two rocprofv3 --pmc
+# runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads
+# for a plain 64 MiB device copy in the same run; recorded in
+# profiles/tree_row16_humanoid_iters_pmc.txt.
+TRAFFIC_BYTES_PER_LAUNCH = None
+MIN_TIMED_LAUNCHES = 256  # the kernel duration is averaged over at least this many launches
 
 
 def algorithmic_bytes(nv: int, nM: int, nefc: int) -> int:
@@ -37,9 +39,14 @@ def algorithmic_bytes(nv: int, nM: int, nefc: int) -> int:
     return 4 * (nM + nefc * nv + nefc + nefc + nv) + 4 * nv
 
 
-def cpu_baseline(batch, plan_struct, seconds: float = 12.0):
-    """The CPU oracle (a C restatement of the reference path, OpenMP over worlds) timed
-    on this host's cores on the same workload; used as the checker elsewhere."""
+def algorithmic_bytes_fused(nv: int, nM: int, nefc: int, iters: int) -> int:
+    """Bytes of one world over `iters` fused solves when M and J are counted once per launch."""
+    return 4 * (nM + nefc * nv) + iters * 4 * (2 * nefc + 2 * nv)
+
+
+def cpu_baseline(batch, plan_struct, seconds: float = 10.0):
+    """The CPU oracle (a C restatement of the reference path, OpenMP over worlds) timed on this
+    host's cores on the same workload: all threads, then one thread."""
     from oracle import planner as P
     from oracle import ref as R
 
@@ -48,24 +55,36 @@ def cpu_baseline(batch, plan_struct, seconds: float = 12.0):
     threads = R.max_threads()
     iters = batch.state.shape[0]
 
-    def one_pass():
-        for it in range(iters):
-            R.assemble_tree_ldl_solve(*st, plan, batch.M, batch.J, batch.D, batch.state[it], batch.nefc, batch.grad)
+    def timed(nworld: int, budget: float):
+        M, J, D, ne, g = batch.M[:nworld], batch.J[:nworld], batch.D[:nworld], batch.nefc[:nworld], batch.grad[:nworld]
 
-    one_pass()
-    t0 = time.perf_counter()
-    reps = 0
-    while time.perf_counter() - t0 < seconds or reps < 3:
+        def one_pass():
+            for it in range(iters):
+                R.assemble_tree_ldl_solve(*st, plan, M, J, D, batch.state[it][:nworld], ne, g)
+
         one_pass()
-        reps += 1
-    dt = time.perf_counter() - t0
-    solves = reps * iters * batch.nworld
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < budget or reps < 2:
+            one_pass()
+            reps += 1
+        dt = time.perf_counter() - t0
+        return reps * iters * nworld / dt, reps, dt
+
+    rate_all, reps_all, dt_all = timed(batch.nworld, seconds)
+    R.set_threads(1)
+    try:
+        rate_one, reps_one, dt_one = timed(min(batch.nworld, 512), seconds / 2)
+    finally:
+        R.set_threads(threads)
     return {
-        "value": solves / dt,
+        "value": rate_all,
         "unit": "world*solves/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"{reps} passes of the same {batch.nworld}-world x {iters}-iteration batch ({dt:.1f} s), all {threads} OpenMP threads",
+        "sample": f"{reps_all} passes of the same {batch.nworld}-world x {iters}-iteration batch ({dt_all:.1f} s), all {threads} OpenMP threads",
+        "single_core_value": rate_one,
+        "single_core_sample": f"{reps_one} passes over the first {min(batch.nworld, 512)} worlds ({dt_one:.1f} s), 1 thread",
     }
 
 
@@ -77,6 +96,7 @@ def main() -> int:
     ap.add_argument("--sets", type=int, default=16, help="distinct input sets rotated over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying hipGraphs")
+    ap.add_argument("--single-only", action="store_true", help="time the three-launch form only (for profiles of the single launch)")
     ap.add_argument(
         "--copy-calibration",
         type=int,
@@ -130,85 +150,117 @@ def main() -> int:
         sh = (s * 257) % nworld
         M, J, D, ne, g = (torch.roll(t, sh, 0).contiguous() for t in base)
         st = torch.roll(base_state, sh, 1).contiguous()
-        sets.append((M, J, D, st, ne, g, torch.zeros_like(g)))
+        sets.append((M, J, D, st, ne, g, torch.zeros((iters, nworld, nv), device=dev)))
     torch.cuda.synchronize()
 
     def step(s: int) -> None:
         M, J, D, st, ne, g, x = sets[s % nsets]
-        for it in range(iters):
-            T.assemble_tree_factor_solve(scratch, M, J, D, st[it], ne, g, x)
+        T.assemble_tree_factor_solve_iters(scratch, M, J, D, st, ne, g, x)
 
-    # correctness guard on the data actually benchmarked (cheap fp64 residual on a few worlds)
+    def step_single(s: int) -> None:
+        # the same work as one launch per iteration, every launch on another input set
+        for it in range(iters):
+            M, J, D, st, ne, g, x = sets[(s * iters + it) % nsets]
+            T.assemble_tree_factor_solve(scratch, M, J, D, st[it], ne, g, x[it])
+
+    # correctness guard on the data benchmarked: set 0 (the batch as generated) against the CPU
+    # oracle, bit for bit, on the first 64 worlds of every iteration
     step(0)
     torch.cuda.synchronize()
+    from oracle import planner as P
+    from oracle import ref as R
+
+    stc = P.tree_ldl_structure(batch.rowadr, batch.rownnz, batch.colind)
+    planc = P.best_tree_ldl_plan(*stc)
+    for it in range(iters):
+        want = R.assemble_tree_ldl_solve(*stc, planc, batch.M[:64], batch.J[:64], batch.D[:64], batch.state[it][:64], batch.nefc[:64], batch.grad[:64])
+        if not np.array_equal(sets[0][6][it, :64].cpu().numpy(), want):
+            raise RuntimeError(f"the benchmarked kernel disagrees with the oracle in iteration {it}")
 
     use_graph = not args.no_graph
-    single, multi = [], None
-    if use_graph:
+
+    def build(fn):
+        """Replays of `fn` over the rotation: one graph per set and one over all sets."""
+        if not use_graph:
+            return None, None
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             for s in range(nsets):
-                step(s)
+                fn(s)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
+        single = []
         for s in range(nsets):
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
-                step(s)
+                fn(s)
             single.append(g)
         multi = torch.cuda.CUDAGraph()
         with torch.cuda.graph(multi):
             for s in range(nsets):
-                step(s)
+                fn(s)
+        return single, multi
 
-    def run(nsteps: int, first: int = 0) -> None:
-        i = 0
-        if use_graph:
-            while first % nsets == 0 and nsteps - i >= nsets:
-                multi.replay()
-                i += nsets
-            while i < nsteps:
-                single[(first + i) % nsets].replay()
-                i += 1
-        else:
-            while i < nsteps:
-                step(first + i)
-                i += 1
+    def runner(fn):
+        single, multi = build(fn)
 
-    run(args.warmup)
-    torch.cuda.synchronize()
-    # HIP events on the stream the kernels are launched on (torch's current stream is the
-    # one handed to the C ABI), around the timed region
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    ev0.record()
-    run(args.steps)
-    ev1.record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    value = args.steps * iters * nworld / elapsed
-    region_s = ev0.elapsed_time(ev1) * 1e-3
+        def run(nsteps: int) -> None:
+            i = 0
+            if use_graph:
+                while nsteps - i >= nsets:
+                    multi.replay()
+                    i += nsets
+                while i < nsteps:
+                    single[i % nsets].replay()
+                    i += 1
+            else:
+                while i < nsteps:
+                    fn(i)
+                    i += 1
 
-    # per-launch kernel duration with HIP events on the launch stream
-    nev = min(args.steps, 64)
-    pairs = []
-    for i in range(nev):
-        M, J, D, st, ne, g, x = sets[i % nsets]
-        for it in range(iters):
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            T.assemble_tree_factor_solve(scratch, M, J, D, st[it], ne, g, x)
-            b.record()
-            pairs.append((a, b))
-    torch.cuda.synchronize()
-    durs = np.array([a.elapsed_time(b) for a, b in pairs]) * 1e-3  # seconds
-    # average launch duration over the timed region: launches run back to back, so the
-    # region divided by the launch count is the kernel's duration (it agrees with the
-    # rocprofv3 kernel trace; a lone launch bracketed by two events reads ~2 us more)
-    kernel_s = region_s / (args.steps * iters)
+        return run
+
+    def region(run, nsteps: int):
+        """Wall time and HIP-event time (on the stream the kernels are launched on: torch's
+        current stream is the one handed to the C ABI) of `nsteps` steps."""
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev0.record()
+        run(nsteps)
+        ev1.record()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, ev0.elapsed_time(ev1) * 1e-3
+
     B = algorithmic_bytes(nv, nM, nefc)
-    achieved = B * nworld / kernel_s / 1e9
+    B3 = algorithmic_bytes_fused(nv, nM, nefc, iters)
+    run_single = runner(step_single)
+    run_single(max(args.warmup, nsets))
+    n_single = max(args.steps, -(-MIN_TIMED_LAUNCHES // iters))
+    _, ev_single = region(run_single, n_single)
+    single_us = ev_single / (n_single * iters) * 1e6
+    single = {
+        "kernel_us": single_us,
+        "launches_timed": n_single * iters,
+        "achieved": B * nworld / (single_us * 1e-6) / 1e9,
+        "frac": B * nworld / (single_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+        "note": "one launch per solve (im_assemble_tree_ldl_solve), every launch on an input set of its own",
+    }
+
+    if args.single_only:
+        print(json.dumps({"single_launch": single}))
+        return 0
+
+    run = runner(step)
+    run(args.warmup)
+    elapsed, _ = region(run, args.steps)
+    value = args.steps * iters * nworld / elapsed
+    # the kernel's duration from a region of its own whose length does not depend on --steps
+    n_kernel = max(args.steps, MIN_TIMED_LAUNCHES)
+    _, ev_kernel = region(run, n_kernel)
+    kernel_s = ev_kernel / n_kernel  # one launch = one step = `iters` solves of every world
+    achieved = B * iters * nworld / kernel_s / 1e9
 
     out = {
         "metric": METRIC,
@@ -224,10 +276,11 @@ def main() -> int:
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": f"humanoid nv={nv} nM={nM} nefc={nefc} x {nworld} worlds, {iters} Newton iterations (launches) per step, fresh active mask each",
+            "workload": f"humanoid nv={nv} nM={nM} nefc={nefc} x {nworld} worlds, {iters} Newton iterations per step with a fresh active mask each, one launch per step (im_assemble_tree_ldl_solve_iters)",
             "input_sets": nsets,
             "launch": "hipGraph replay" if use_graph else "eager",
             "bytes_per_world_solve": B,
+            "bytes_per_world_step_fused": B3,
         },
         "roofline": {
             "bound": "hbm",
@@ -237,13 +290,18 @@ def main() -> int:
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": TRAFFIC_BYTES_PER_LAUNCH,
             "kernel_us": kernel_s * 1e6,
-            "kernel_us_single_launch_p10_p50_p90": [float(np.percentile(durs, p)) * 1e6 for p in (10, 50, 90)],
+            "launches_timed": n_kernel,
+            "solves_per_launch": iters,
+            "us_per_solve": kernel_s * 1e6 / iters,
+            "bytes_definition": f"per-solve B = {B} bytes x {iters} solves x {nworld} worlds per launch (every solve counted as if it read M and J itself)",
+            "frac_fused_bytes": B3 * nworld / kernel_s / 1e9 / HBM_PEAK_GBS,
+            "frac_fused_bytes_definition": f"B3 = {B3} bytes per world and launch: M and J once, state / D / gradient / x per iteration",
             "throughput_frac": (B * value / 1e9) / HBM_PEAK_GBS,
+            "single_launch": single,
         },
     }
     if not args.no_cpu:
-        st = T.tree_ldl_structure(batch.rowadr, batch.rownnz, batch.colind)
-        out["cpu_baseline"] = cpu_baseline(batch, st)
+        out["cpu_baseline"] = cpu_baseline(batch, T.tree_ldl_structure(batch.rowadr, batch.rownnz, batch.colind))
     print(json.dumps(out))
     return 0
 
