@@ -372,7 +372,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
         emit(f"    int chc{i} = CH_{name}[{i}][p];")
     for i in range(MC):
         emit(f"    const float mv{i} = M[wq * ldM + min({i * 64} + lane, {nM - 1})];")
-    SP = 4  # steps (16 rows) requested before the row weights are known
+    SP = min(PD, int(os.environ.get("IMHIP_SP", "2")))  # steps (4 rows each) requested before the row weights are known
     pin_ch = " ".join(f'asm volatile("" : "+v"(chc{i}));' for i in range(len(leaf_sets)))
     emit("    int steps_s = 0, cnt = 0;  // short variant: steps and length of the compacted tail")
     emit("    if (LONG) {")
