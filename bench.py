@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the iterations kernel (3 solves x 4096 worlds) from two rocprofv3 --pmc
 # runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads
 # for a plain 64 MiB device copy in the same run; recorded in
-# profiles/tree_row16_humanoid_iters_pmc.txt.
-TRAFFIC_BYTES_PER_LAUNCH = None
+# profiles/tree_row16_humanoid_pmc.txt:  (18292.13 * 65536 / 32783.90 + 1344.0) KiB
+TRAFFIC_BYTES_PER_LAUNCH = int((18292.13 * 65536 / 32783.90 + 1344.0) * 1024)
 MIN_TIMED_LAUNCHES = 256  # the kernel duration is averaged over at least this many launches
 
 
