@@ -173,6 +173,66 @@ __device__ __forceinline__ void muscle_force_magnitudes(
   }
 }
 
+// MuJoCo's force-velocity multiplier and its derivative in the normalised velocity
+// (muscle_qfrc_projector.py:2505-2524)
+__device__ __forceinline__ void force_velocity_curve(float v, float fvmax, float *mult, float *slope) {
+  const float y = fvmax - 1.0f;
+  if (v <= -1.0f) {
+    *mult = 0.0f;
+    *slope = 0.0f;
+  } else if (v <= 0.0f) {
+    const float shifted = v + 1.0f;
+    *mult = shifted * shifted;
+    *slope = 2.0f * shifted;
+  } else if (v <= y) {
+    const float remaining = y - v;
+    *mult = fvmax - remaining * remaining / y;
+    *slope = 2.0f * remaining / y;
+  } else {
+    *mult = fvmax;
+    *slope = 0.0f;
+  }
+}
+
+// eval_muscle_force_velocity_state_kernel (muscle_qfrc_projector.py:2816-2884): one muscle of
+// one world -- its length over consecutive waypoints, its lengthening velocity -sum moment qvel
+// over its (muscle, dof) entries, and the force-velocity response (:2528-2570).
+__global__ __launch_bounds__(256) void force_velocity_state_kernel(
+    const float *__restrict__ wp, int64_t ldw, const int32_t *__restrict__ waypoint_start,
+    const float *__restrict__ params, int ldpar, const float *__restrict__ rest,
+    const float *__restrict__ length_scale, const float *__restrict__ activation, int64_t lda,
+    const float *__restrict__ qvel, int64_t ldq, const float *__restrict__ moment, int64_t ldm,
+    const int32_t *__restrict__ dof_offsets, const int32_t *__restrict__ dof_torque_idx, int root,
+    im_muscle_force_model model, im_muscle_force_velocity_model fv, int nmuscle, float *__restrict__ out_length,
+    float *__restrict__ out_activation, float *__restrict__ out_velocity, float *__restrict__ out_multiplier,
+    float *__restrict__ out_slope, int64_t ldo) {
+  const int m = blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t w = blockIdx.y;
+  if (m >= nmuscle) return;
+  const float *row = wp + w * ldw;
+  float len = 0.0f;
+  for (int i = waypoint_start[m]; i < waypoint_start[m + 1] - 1; ++i)
+    len = len + length(sub(ld3(row + 3 * (i + 1)), ld3(row + 3 * i)));
+  float velocity = 0.0f;
+  for (int e = dof_offsets[m]; e < dof_offsets[m + 1]; ++e)
+    velocity = __builtin_fmaf(-moment[w * ldm + e], qvel[w * ldq + dof_torque_idx[e] + root], velocity);
+  const float f0 = params[m * ldpar], lm0 = params[m * ldpar + 1], lt0 = params[m * ldpar + 2],
+              pen = params[m * ldpar + 3];
+  const float velocity_scale = fmaxf(length_scale[m] * fv.vmax, 1.0e-6f);
+  float mult, dmult;
+  force_velocity_curve(velocity / velocity_scale, fv.fvmax, &mult, &dmult);
+  float active = activation[w * lda + m];
+  if (fv.clamp_activation != 0.0f) active = fminf(fmaxf(active, 0.0f), 1.0f);
+  const float lm = len / fmaxf(rest[m], 1.0e-6f) - lt0;
+  const float ln = fminf(fmaxf(lm / fmaxf(lm0, 1.0e-6f), model.length_norm_min), model.length_norm_max);
+  const float unit = f0 * active_fl(ln, model.active) * cosf(pen) * model.force_scale;
+  out_length[w * ldo + m] = len;
+  out_activation[w * ldo + m] = active * mult;
+  out_velocity[w * ldo + m] = velocity;
+  out_multiplier[w * ldo + m] = mult;
+  out_slope[w * ldo + m] = fv.include_active * active * unit * dmult / velocity_scale;
+}
+
 __global__ __launch_bounds__(256) void force_kernel(
     const float *__restrict__ wp, int64_t ldw, const int32_t *__restrict__ seg_start,
     const int32_t *__restrict__ seg_offsets, const float *__restrict__ params, int ldpar,
@@ -604,6 +664,36 @@ extern "C" int im_muscle_force_magnitudes(const float *waypoints, int64_t ld_way
                        all_muscle_segment_offsets, muscle_params, ld_params, muscle_rest_length,
                        *model, nmuscle, unit_force + w0 * ld_unit, ld_unit,
                        passive_force ? passive_force + w0 * ld_passive : nullptr, ld_passive);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_muscle_force_velocity_state(
+    const float *waypoints, int64_t ld_waypoints, const int32_t *muscle_waypoint_start,
+    const float *muscle_params, int ld_params, const float *muscle_rest_length,
+    const float *force_velocity_length_scale, const float *activation, int64_t ld_activation,
+    const float *qvel, int64_t ld_qvel, const float *moment, int64_t ld_moment,
+    const int32_t *muscle_dof_offsets, const int32_t *muscle_dof_torque_idx, int root_dof_count,
+    const im_muscle_force_model *model, const im_muscle_force_velocity_model *fv, int nmuscle,
+    float *muscle_length, float *effective_activation, float *length_velocity,
+    float *force_velocity_multiplier, float *force_velocity_slope, int64_t ld_out, int nworld, void *stream) {
+  if (nworld < 0 || nmuscle < 0 || root_dof_count < 0) return IM_ERR_ARG;
+  if (nworld == 0 || nmuscle == 0) return IM_OK;
+  if (!waypoints || !muscle_waypoint_start || !muscle_params || !muscle_rest_length ||
+      !force_velocity_length_scale || !activation || !qvel || !moment || !muscle_dof_offsets ||
+      !muscle_dof_torque_idx || !model || !fv || !muscle_length || !effective_activation || !length_velocity ||
+      !force_velocity_multiplier || !force_velocity_slope || ld_params < 4)
+    return IM_ERR_ARG;
+  if (ld_out < nmuscle || ld_activation < nmuscle) return IM_ERR_STRIDE;
+  IM_FOR_WORLD_SLABS(nworld, w0, nw) {
+    hipLaunchKernelGGL(force_velocity_state_kernel, grid2(nmuscle, nw), dim3(256), 0, (hipStream_t)stream,
+                       waypoints + w0 * ld_waypoints, ld_waypoints, muscle_waypoint_start, muscle_params, ld_params,
+                       muscle_rest_length, force_velocity_length_scale, activation + w0 * ld_activation,
+                       ld_activation, qvel + w0 * ld_qvel, ld_qvel, moment + w0 * ld_moment, ld_moment,
+                       muscle_dof_offsets, muscle_dof_torque_idx, root_dof_count, *model, *fv, nmuscle,
+                       muscle_length + w0 * ld_out, effective_activation + w0 * ld_out, length_velocity + w0 * ld_out,
+                       force_velocity_multiplier + w0 * ld_out, force_velocity_slope + w0 * ld_out, ld_out);
   }
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;

@@ -12,6 +12,9 @@
 // reference (Warp lowers `total += a * b` to one fma under NVRTC's default contraction).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <vector>
+
 #include "common.h"
 
 namespace im {
@@ -186,6 +189,47 @@ int im_muscle_project(const float *moment, int64_t ld_moment, const float *force
                      moment, ld_moment, force, ld_force, torque_entry_offsets, torque_entry_idx, entry_muscle,
                      nentry, nmuscle, ntorque, root_dof_count, qfrc, ld_qfrc, nworld);
   IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_muscle_gather_tables(const int32_t *pair_elem_id, const int32_t *pair_entry_i, const int32_t *pair_entry_j,
+                            int npair, int nentry, int32_t *elem_ids, int32_t *chunk_offsets, int32_t *chunk_pairs,
+                            int *nelem, int *chunk_count) {
+  if (npair < 0 || nentry < 0 || !nelem || !chunk_count || (npair > 0 && !pair_elem_id)) return IM_ERR_ARG;
+  if (nentry >= 0x7FFF) return IM_ERR_UNSUPPORTED;  // two entry indices share one int32
+  // pairs in the order of their M element, ties in list order
+  std::vector<int> order(npair);
+  for (int q = 0; q < npair; ++q) order[q] = q;
+  std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return pair_elem_id[a] < pair_elem_id[b]; });
+  // first pass: elements and their chunks of 16 pairs
+  int elems = 0, chunks = 0;
+  for (int q = 0; q < npair;) {
+    int end = q;
+    while (end < npair && pair_elem_id[order[end]] == pair_elem_id[order[q]]) ++end;
+    if (elem_ids) elem_ids[elems] = pair_elem_id[order[q]];
+    if (chunk_offsets) chunk_offsets[elems] = chunks;
+    chunks += (end - q + 15) / 16;
+    ++elems;
+    q = end;
+  }
+  if (chunk_offsets) chunk_offsets[elems] = chunks;
+  *nelem = elems;
+  *chunk_count = chunks;
+  if (!chunk_pairs) return IM_OK;
+  if (!pair_entry_i || !pair_entry_j || !chunk_offsets) return IM_ERR_ARG;
+  // second pass: pair k of chunk c at k * chunk_count + c, the padding names entry `nentry` twice
+  for (size_t v = 0; v < (size_t)16 * chunks; ++v) chunk_pairs[v] = nentry | (nentry << 16);
+  int slot = 0, rank = 0;
+  for (int q = 0; q < npair; ++q) {
+    if (q > 0 && pair_elem_id[order[q]] != pair_elem_id[order[q - 1]]) {
+      ++slot;
+      rank = 0;
+    }
+    const int i = pair_entry_i[order[q]], j = pair_entry_j[order[q]];
+    if (i < 0 || j < 0 || i >= nentry || j >= nentry) return IM_ERR_ARG;
+    chunk_pairs[(size_t)(rank % 16) * chunks + chunk_offsets[slot] + rank / 16] = i | (j << 16);
+    ++rank;
+  }
   return IM_OK;
 }
 

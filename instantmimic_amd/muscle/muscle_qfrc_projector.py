@@ -165,33 +165,30 @@ class MuscleImplicitQderivGather:
 
 
 def gather_tables(prepared: PreparedMuscleImplicitQderivPairs, entry_muscle_idx):
-    """Host tables of the deterministic gather (NumPy): elem_ids, chunk_offsets,
-    chunk_pairs; ``None`` when there is nothing to gather or the index limit is hit."""
-    elem = _np(prepared.pair_elem_id)
+    """Host tables of the deterministic gather: (elem_ids, chunk_offsets, chunk_pairs, entry_count,
+    chunk_count) from ``im_muscle_gather_tables``; ``None`` when there is nothing to gather or the
+    index limit is hit."""
+    import ctypes as C
+
+    elem = np.ascontiguousarray(_np(prepared.pair_elem_id), np.int32)
     entry_muscle = _np(entry_muscle_idx)
     entry_count = int(entry_muscle.size)
     if elem.size == 0 or entry_count >= _QDERIV_GATHER_MAX_ENTRIES:
         return None
-    pi, pj, pm = _np(prepared.pair_entry_i), _np(prepared.pair_entry_j), _np(prepared.pair_muscle_idx)
+    pi, pj, pm = (np.ascontiguousarray(_np(a), np.int32) for a in (prepared.pair_entry_i, prepared.pair_entry_j, prepared.pair_muscle_idx))
     if not (np.array_equal(entry_muscle[pi], pm) and np.array_equal(entry_muscle[pj], pm)):
         raise ValueError("every implicit qDeriv pair must join entries of its muscle")
-    order = np.argsort(elem, kind="stable")
-    elem, pi, pj = elem[order], pi[order], pj[order]
-    elem_ids, counts = np.unique(elem, return_counts=True)
-    chunk = _QDERIV_GATHER_CHUNK
-    chunks = (counts + chunk - 1) // chunk
-    chunk_offsets = np.zeros(chunks.size + 1, np.int64)
-    chunk_offsets[1:] = np.cumsum(chunks)
-    chunk_count = int(chunk_offsets[-1])
-    starts = np.cumsum(counts) - counts
-    rank = np.arange(elem.size) - np.repeat(starts, counts)
-    row = np.repeat(chunk_offsets[:-1], counts) + rank // chunk
-    packed = np.full((chunk_count, chunk), entry_count | entry_count << 16, np.int64)
-    packed[row, rank % chunk] = pi | pj << 16
-    return (
-        elem_ids.astype(np.int32), chunk_offsets.astype(np.int32),
-        np.ascontiguousarray(packed.T).reshape(-1).astype(np.int32), entry_count, chunk_count,
+    nelem, nchunk = C.c_int(0), C.c_int(0)
+    lib = _lib.lib()
+    _lib.check(lib.im_muscle_gather_tables(elem.ctypes.data, None, None, int(elem.size), entry_count, None, None, None, C.byref(nelem), C.byref(nchunk)), "im_muscle_gather_tables")
+    elem_ids, chunk_offsets = np.zeros(nelem.value, np.int32), np.zeros(nelem.value + 1, np.int32)
+    chunk_pairs = np.zeros(_QDERIV_GATHER_CHUNK * nchunk.value, np.int32)
+    _lib.check(
+        lib.im_muscle_gather_tables(elem.ctypes.data, pi.ctypes.data, pj.ctypes.data, int(elem.size), entry_count, elem_ids.ctypes.data,
+                                    chunk_offsets.ctypes.data, chunk_pairs.ctypes.data, C.byref(nelem), C.byref(nchunk)),
+        "im_muscle_gather_tables",
     )  # fmt: skip
+    return elem_ids, chunk_offsets, chunk_pairs, entry_count, int(nchunk.value)
 
 
 def build_muscle_implicit_qderiv_gather(prepared, entry_muscle_idx, device) -> MuscleImplicitQderivGather | None:
@@ -268,3 +265,52 @@ def project_muscle_sparse_moment_qfrc(
             qfrc_applied.data_ptr(), qfrc_applied.stride(0), int(moment.shape[0]), _stream(moment),
         )  # fmt: skip
     _lib.check(status, "im_muscle_project")
+
+
+def eval_muscle_force_velocity_state(
+    transformed_waypoints, muscle_waypoint_start, muscle_params, muscle_rest_length, force_velocity_length_scale,
+    activation, qvel, moment, muscle_dof_offsets, muscle_dof_torque_idx, root_dof_count: int, *,
+    muscle_force_scale: float, muscle_length_norm_min: float, muscle_length_norm_max: float, vmax: float,
+    fvmax: float, clamp_activation: bool, include_active: bool, active_force_model_params,
+    muscle_length, effective_activation, length_velocity, force_velocity_multiplier, force_velocity_slope,
+) -> None:  # fmt: skip
+    """Launch of ``eval_muscle_force_velocity_state_kernel`` with the reference's arrays
+    (src/instantmimic/muscle/muscle_qfrc_projector.py:2816-2884): waypoints (nworld, nwaypoint, 3),
+    activation and the five outputs (nworld, nmuscle), qvel (nworld, nv), moment (nworld, nentry);
+    the index tables int32 tensors on the same GPU.  ``force_velocity_slope`` is what
+    :func:`apply_muscle_implicit_qderiv_gather` takes."""
+    import torch
+
+    nworld, nmuscle = int(activation.shape[0]), int(activation.shape[1])
+    outs = (muscle_length, effective_activation, length_velocity, force_velocity_multiplier, force_velocity_slope)
+    wp2 = transformed_waypoints.reshape(nworld, -1)
+    _f32_rows(wp2, activation, qvel, moment, muscle_params, *outs)
+    for t in outs:
+        if tuple(t.shape) != (nworld, nmuscle) or t.stride(0) != outs[0].stride(0):
+            raise ValueError("the five outputs must be (nworld, nmuscle) with one row stride")
+    for t in (muscle_waypoint_start, muscle_dof_offsets, muscle_dof_torque_idx):
+        if t.dtype != torch.int32 or not t.is_cuda or not t.is_contiguous():
+            raise TypeError("index tables must be contiguous int32 CUDA tensors")
+    if muscle_waypoint_start.numel() != nmuscle + 1 or muscle_dof_offsets.numel() != nmuscle + 1:
+        raise ValueError("muscle_waypoint_start and muscle_dof_offsets need nmuscle + 1 entries")
+    if qvel.shape[0] != nworld or moment.shape[0] != nworld or moment.shape[1] < muscle_dof_torque_idx.numel():
+        raise ValueError("qvel and moment do not match the batch or the entry table")
+    if muscle_rest_length.numel() != nmuscle or force_velocity_length_scale.numel() != nmuscle or muscle_params.shape[0] != nmuscle:
+        raise ValueError("per-muscle arrays need nmuscle rows")
+    model = _lib.MuscleForceModel()
+    model.force_scale, model.length_norm_min, model.length_norm_max = muscle_force_scale, muscle_length_norm_min, muscle_length_norm_max
+    for k, v in enumerate(active_force_model_params):
+        model.active[k] = float(v)
+    fv = _lib.MuscleForceVelocityModel(float(vmax), float(fvmax), float(bool(clamp_activation)), float(bool(include_active)))
+    import ctypes as C
+
+    with torch.cuda.device(activation.device):
+        status = _lib.lib().im_muscle_force_velocity_state(
+            wp2.data_ptr(), wp2.stride(0), muscle_waypoint_start.data_ptr(), muscle_params.data_ptr(),
+            muscle_params.stride(0), muscle_rest_length.data_ptr(), force_velocity_length_scale.data_ptr(),
+            activation.data_ptr(), activation.stride(0), qvel.data_ptr(), qvel.stride(0), moment.data_ptr(),
+            moment.stride(0), muscle_dof_offsets.data_ptr(), muscle_dof_torque_idx.data_ptr(), int(root_dof_count),
+            C.byref(model), C.byref(fv), nmuscle, *[t.data_ptr() for t in outs], outs[0].stride(0), nworld,
+            _stream(activation),
+        )  # fmt: skip
+    _lib.check(status, "im_muscle_force_velocity_state")

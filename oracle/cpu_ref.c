@@ -962,6 +962,52 @@ int orc_muscle_force_magnitudes(int nworld, int nwp, int nmuscle, const float *w
   return 0;
 }
 
+/* eval_muscle_force_velocity_state_kernel (src/instantmimic/muscle/muscle_qfrc_projector.py:
+ * 2816-2884) with muscle_force_velocity_curve_wp (:2505-2524) and
+ * muscle_force_velocity_response_wp (:2528-2570); model as in orc_muscle_force_magnitudes,
+ * fv = vmax, fvmax, clamp_activation, include_active; out = five (nworld, nmuscle) arrays one
+ * after the other: length, effective activation, velocity, multiplier, slope. */
+int orc_muscle_force_velocity_state(int nworld, int nwp, int nmuscle, int nentry, int nvfull,
+                                    const float *wp, const int *wp_start, const float *params,
+                                    int ldpar, const float *rest, const float *length_scale,
+                                    const float *act, const float *qvel, const float *moment,
+                                    const int *dof_offsets, const int *dof_torque, int root,
+                                    const float *model, const float *fv, float *out) {
+  const size_t plane = (size_t)nworld * nmuscle;
+#pragma omp parallel for schedule(static)
+  for (int w = 0; w < nworld; ++w) {
+    const float *row = wp + (size_t)w * nwp * 3;
+    for (int m = 0; m < nmuscle; ++m) {
+      float len = 0.0f;
+      for (int i = wp_start[m]; i < wp_start[m + 1] - 1; ++i)
+        len = len + v_len(v_sub(v_ld(row + 3 * (i + 1)), v_ld(row + 3 * i)));
+      float vel = 0.0f;
+      for (int e = dof_offsets[m]; e < dof_offsets[m + 1]; ++e)
+        vel = fmaf(-moment[(size_t)w * nentry + e], qvel[(size_t)w * nvfull + dof_torque[e] + root], vel);
+      const float *p = params + (size_t)m * ldpar;
+      const float vscale = fmaxf(length_scale[m] * fv[0], 1.0e-6f);
+      const float v = vel / vscale, fvmax = fv[1], y = fvmax - 1.0f;
+      float mult, slope;
+      if (v <= -1.0f) { mult = 0.0f; slope = 0.0f; }
+      else if (v <= 0.0f) { const float sh = v + 1.0f; mult = sh * sh; slope = 2.0f * sh; }
+      else if (v <= y) { const float rem = y - v; mult = fvmax - rem * rem / y; slope = 2.0f * rem / y; }
+      else { mult = fvmax; slope = 0.0f; }
+      float a = act[(size_t)w * nmuscle + m];
+      if (fv[2] != 0.0f) a = fminf(fmaxf(a, 0.0f), 1.0f);
+      const float lm = len / fmaxf(rest[m], 1.0e-6f) - p[2];
+      const float ln = fminf(fmaxf(lm / fmaxf(p[1], 1.0e-6f), model[1]), model[2]);
+      const float unit = p[0] * active_fl(ln, model + 3) * cosf(p[3]) * model[0];
+      const size_t o = (size_t)w * nmuscle + m;
+      out[o] = len;
+      out[plane + o] = a * mult;
+      out[2 * plane + o] = vel;
+      out[3 * plane + o] = mult;
+      out[4 * plane + o] = fv[3] * a * unit * slope / vscale;
+    }
+  }
+  return 0;
+}
+
 /* rows of an entry list: offsets[nrow + 1], segment, other, start/end coefficient */
 #define ORC_GEO(w)                                                                        \
   const float *wpw = wp + (size_t)(w) * nwp * 3, *comw = com + (size_t)(w) * nbody * 3, \

@@ -347,6 +347,22 @@ def muscle_force_magnitudes(waypoints, seg_start, seg_offsets, params, rest, mod
     return unit, passive
 
 
+def muscle_force_velocity_state(waypoints, wp_start, params, rest, length_scale, act, qvel, moment, dof_offsets,
+                                dof_torque, root, model, fv):
+    """model = the 9 floats of muscle_force_magnitudes; fv = (vmax, fvmax, clamp_activation,
+    include_active).  Returns (length, effective_activation, velocity, multiplier, slope)."""
+    waypoints, params, act, qvel, moment = _f(waypoints), _f(params), _f(act), _f(qvel), _f(moment)
+    nworld, nwp = waypoints.shape[0], waypoints.shape[1]
+    nmuscle = len(wp_start) - 1
+    out = np.zeros((5, nworld, nmuscle), np.float32)
+    lib().orc_muscle_force_velocity_state(
+        nworld, nwp, nmuscle, moment.shape[1], qvel.shape[1], _p(waypoints), _p(_i(wp_start)), _p(params),
+        params.shape[1], _p(_f(rest)), _p(_f(length_scale)), _p(act), _p(qvel), _p(moment), _p(_i(dof_offsets)),
+        _p(_i(dof_torque)), int(root), _p(_f(model)), _p(_f(fv)), _p(out),
+    )  # fmt: skip
+    return tuple(out)
+
+
 def _geo(waypoints, com, cdof):
     waypoints, com, cdof = _f(waypoints), _f(com), _f(cdof)
     return waypoints, com, cdof, (waypoints.shape[0], waypoints.shape[1], com.shape[1], cdof.shape[1])

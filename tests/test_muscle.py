@@ -134,3 +134,93 @@ def test_gpu_projection_with_more_entries_than_one_staging_trip(device):
     got = qfrc.cpu().numpy()
     np.testing.assert_array_equal(got[:, mb.root_dof_count :], tau_ref[:, mb.root_dof_count :])
     assert (got[:, : mb.root_dof_count] == 7.0).all()
+
+
+def _fv_case(nworld, seed=4, active_type=1.0):
+    """Random muscles over random waypoints: every branch of the force-velocity curve is hit."""
+    rng = np.random.default_rng(seed)
+    nmuscle, nv, root = 37, 30, 6
+    counts = rng.integers(2, 6, nmuscle)
+    wp_start = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    nwp = int(wp_start[-1])
+    waypoints = rng.normal(size=(nworld, nwp, 3)).astype(np.float32)
+    ndof = rng.integers(1, 4, nmuscle)
+    dof_offsets = np.concatenate([[0], np.cumsum(ndof)]).astype(np.int32)
+    dof_torque = np.concatenate([np.sort(rng.choice(nv - root, n, replace=False)) for n in ndof]).astype(np.int32)
+    params = np.stack([rng.uniform(100, 3000, nmuscle), rng.uniform(0.5, 1.5, nmuscle), rng.uniform(0.0, 0.5, nmuscle), rng.uniform(0, 0.5, nmuscle)], 1).astype(np.float32)
+    rest = rng.uniform(2.0, 6.0, nmuscle).astype(np.float32)
+    scale = rng.uniform(0.1, 0.5, nmuscle).astype(np.float32)
+    act = rng.uniform(-0.2, 1.3, (nworld, nmuscle)).astype(np.float32)
+    qvel = rng.normal(scale=3.0, size=(nworld, nv)).astype(np.float32)
+    moment = rng.normal(scale=0.2, size=(nworld, int(dof_offsets[-1]))).astype(np.float32)
+    model = np.array([1.2, 0.4, 1.6, active_type, 0.5 if active_type else 0.45, 1.6, 0, 0, 0], np.float32)
+    fv = np.array([1.5, 1.4, 1.0, 1.0], np.float32)
+    return dict(waypoints=waypoints, wp_start=wp_start, params=params, rest=rest, length_scale=scale, act=act, qvel=qvel,
+                moment=moment, dof_offsets=dof_offsets, dof_torque=dof_torque, root=root, model=model, fv=fv)  # fmt: skip
+
+
+def _fv64(c):
+    """The same state in fp64 NumPy, written from the formulas (muscle_qfrc_projector.py:2505-2570)."""
+    wp = c["waypoints"].astype(np.float64)
+    nworld, nmuscle = wp.shape[0], len(c["wp_start"]) - 1
+    seg = np.linalg.norm(np.diff(wp, axis=1), axis=2)
+    out = np.zeros((5, nworld, nmuscle))
+    vmax, fvmax, clamp, inc = (float(v) for v in c["fv"])
+    for m in range(nmuscle):
+        a, b = c["wp_start"][m], c["wp_start"][m + 1]
+        length = seg[:, a : b - 1].sum(1)
+        e0, e1 = c["dof_offsets"][m], c["dof_offsets"][m + 1]
+        vel = -(c["moment"][:, e0:e1].astype(np.float64) * c["qvel"][:, c["dof_torque"][e0:e1] + c["root"]]).sum(1)
+        vs = max(float(c["length_scale"][m]) * vmax, 1e-6)
+        v, y = vel / vs, fvmax - 1.0
+        mult = np.where(v <= -1, 0.0, np.where(v <= 0, (v + 1) ** 2, np.where(v <= y, fvmax - (y - v) ** 2 / y, fvmax)))
+        slope = np.where(v <= -1, 0.0, np.where(v <= 0, 2 * (v + 1), np.where(v <= y, 2 * (y - v) / y, 0.0)))
+        act = np.clip(c["act"][:, m].astype(np.float64), 0, 1) if clamp else c["act"][:, m]
+        f0, lm0, lt0, pen = (float(x) for x in c["params"][m])
+        ln = np.clip((length / max(float(c["rest"][m]), 1e-6) - lt0) / max(lm0, 1e-6), float(c["model"][1]), float(c["model"][2]))
+        lmin, lmax = float(c["model"][4]), float(c["model"][5])  # MuJoCo piecewise-quadratic active curve
+        lo, hi = 0.5 * (lmin + 1), 0.5 * (1 + lmax)
+        fl = np.where((ln < lmin) | (ln > lmax), 0.0, np.where(ln <= lo, 0.5 * ((ln - lmin) / (lo - lmin)) ** 2, np.where(
+            ln <= 1, 1 - 0.5 * ((1 - ln) / (1 - lo)) ** 2, np.where(ln <= hi, 1 - 0.5 * ((ln - 1) / (hi - 1)) ** 2, 0.5 * ((lmax - ln) / (lmax - hi)) ** 2))))  # fmt: skip
+        unit = f0 * fl * np.cos(pen) * float(c["model"][0])
+        out[:, :, m] = length, act * mult, vel, mult, inc * act * unit * slope / vs
+    return out
+
+
+def test_force_velocity_state_oracle_against_fp64():
+    c = _fv_case(50)
+    got = np.stack(R.muscle_force_velocity_state(**c))
+    want = _fv64(c)
+    for k, name in enumerate(("length", "effective activation", "velocity", "multiplier", "slope")):
+        np.testing.assert_allclose(got[k], want[k], rtol=3e-5, atol=3e-5 * max(1.0, np.abs(want[k]).max()), err_msg=name)
+    v = want[2] / np.maximum(c["length_scale"] * 1.5, 1e-6)
+    assert (v <= -1).any() and ((v > -1) & (v <= 0)).any() and ((v > 0) & (v <= 0.4)).any() and (v > 0.4).any()
+    assert (c["act"] < 0).any() and (got[1] >= 0).all()  # clamped activation
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("active_type", [1.0, 0.0])
+def test_gpu_force_velocity_state(device, active_type):
+    """im_muscle_force_velocity_state against the oracle: length, velocity, multiplier and effective
+    activation bit for bit; the slope carries cosf (and expf with the gaussian active curve), which
+    differ by a few ulp between libm and the GPU, and is held to 2e-6."""
+    import torch
+
+    c = _fv_case(130, active_type=active_type)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    outs = [torch.full((130, 37), float("nan"), device=device) for _ in range(5)]
+    Q.eval_muscle_force_velocity_state(
+        t(c["waypoints"]), t(c["wp_start"]), t(c["params"]), t(c["rest"]), t(c["length_scale"]), t(c["act"]), t(c["qvel"]),
+        t(c["moment"]), t(c["dof_offsets"]), t(c["dof_torque"]), c["root"], muscle_force_scale=float(c["model"][0]),
+        muscle_length_norm_min=float(c["model"][1]), muscle_length_norm_max=float(c["model"][2]), vmax=1.5, fvmax=1.4,
+        clamp_activation=True, include_active=True, active_force_model_params=c["model"][3:6],
+        muscle_length=outs[0], effective_activation=outs[1], length_velocity=outs[2], force_velocity_multiplier=outs[3],
+        force_velocity_slope=outs[4],
+    )  # fmt: skip
+    torch.cuda.synchronize()
+    want = R.muscle_force_velocity_state(**c)
+    for k in range(4):
+        np.testing.assert_array_equal(outs[k].cpu().numpy(), want[k])
+    np.testing.assert_allclose(outs[4].cpu().numpy(), want[4], rtol=2e-6, atol=1e-6 * np.abs(want[4]).max())
+    assert (want[4] == 0).any() and (want[4] != 0).any()
+    np.testing.assert_array_equal(outs[4].cpu().numpy() == 0, want[4] == 0)  # the curve's flat parts are exact
