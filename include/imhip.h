@@ -96,13 +96,28 @@ int im_tree_factor_solve(const im_tree_plan *plan, const float *M, int64_t ldM,
  * (newton_fusion.py:480-519) and tree_ldl.tree_factor_solve.
  *   J (nworld, njmax, nv) contiguous, D/state (nworld, njmax), nefc (nworld) or
  *   null for njmax rows everywhere, grad (nworld, ldg), x (nworld, ldx),
- *   Hout (nworld, nM) or null. */
+ *   Hout (nworld, nM) or null.
+ * Products of a row outside M's pattern (a row over two branches) are dropped:
+ * im_tree_pattern_violations counts such rows. */
 int im_assemble_tree_ldl_solve(const im_tree_plan *plan, const float *M,
                                int64_t ldM, const float *J, int njmax,
                                const float *D, const int32_t *state,
                                const int32_t *nefc, int quad, const float *grad,
                                int64_t ldg, float *x, int64_t ldx, float *Hout,
                                int nworld, unsigned flags, void *stream);
+
+/* The guard of the tree pattern.  im_assemble_tree_ldl_solve holds H on M's CSR entries, that is
+ * on pairs (dof, ancestor): a constraint row whose nonzero dofs do not all lie on one
+ * root-to-leaf chain has products outside that pattern, which are dropped without a trace.
+ * This launch counts such rows per world -- rows r < nefc[w] with state == quad and D != 0, as
+ * the reference's sparse assembly counts rows outside its declared pattern
+ * (src/instantmimic/utils/mjw_kernels/sparse_hessian.py:605-621, read back through
+ * violation_counter, :786-796) -- and adds the count to violations[w] (float, accumulates until
+ * the caller zeroes it: a periodic check sees every violation).  Costs one pass over J; run it
+ * when a row producer changes, or every so many steps. */
+int im_tree_pattern_violations(const im_tree_plan *plan, const float *J, int njmax, const float *D,
+                               const int32_t *state, const int32_t *nefc, int quad,
+                               float *violations, int nworld, void *stream);
 
 /* im_assemble_tree_ldl_solve for `niter` Newton iterations that share M, J and D and differ in
  * the constraint states (and optionally the gradient): what a step of the reference's Newton
@@ -341,6 +356,18 @@ int im_muscle_project(const float *moment, int64_t ld_moment, const float *force
                       int nentry, int nmuscle, int ntorque, int root_dof_count,
                       float *qfrc, int64_t ld_qfrc, int nworld, void *stream);
 
+/* The tables of build_muscle_implicit_qderiv_gather
+ * (src/instantmimic/muscle/muscle_qfrc_projector.py:614-669), on the host: the pairs
+ * (pair_entry_i, pair_entry_j) grouped by their M element pair_elem_id (ties in list order), every
+ * element's pairs cut into chunks of 16, packed i | j << 16 chunk-interleaved (pair k of chunk c
+ * at chunk_pairs[k * chunk_count + c]) and padded with nentry | nentry << 16.  Call once with
+ * the three output arrays null to learn *nelem and *chunk_count, then with elem_ids (nelem),
+ * chunk_offsets (nelem + 1) and chunk_pairs (16 * chunk_count). */
+int im_muscle_gather_tables(const int32_t *pair_elem_id, const int32_t *pair_entry_i,
+                            const int32_t *pair_entry_j, int npair, int nentry, int32_t *elem_ids,
+                            int32_t *chunk_offsets, int32_t *chunk_pairs, int *nelem,
+                            int *chunk_count);
+
 /* Replaces apply_muscle_implicit_qderiv_gather (muscle_qfrc_projector.py:777-809,
  * kernel :736-774): qderiv[w, elem_ids[slot]] += timestep * sum over the slot's
  * chunks, in order, of the chunk's 16-pair sum of
@@ -425,6 +452,35 @@ int im_muscle_force_magnitudes(const float *waypoints, int64_t ld_waypoints,
                                const im_muscle_force_model *model, int nmuscle,
                                float *unit_force, int64_t ld_unit, float *passive_force,
                                int64_t ld_passive, int nworld, void *stream);
+
+/* MuJoCo's force-velocity curve parameters and the two switches of
+ * muscle_force_velocity_response_wp (muscle_qfrc_projector.py:2528-2570). */
+typedef struct im_muscle_force_velocity_model {
+  float vmax, fvmax;
+  float clamp_activation; /* nonzero: activation clamped to [0, 1] */
+  float include_active;   /* factor of the slope (0 switches the implicit term off) */
+} im_muscle_force_velocity_model;
+
+/* Replaces eval_muscle_force_velocity_state_kernel
+ * (src/instantmimic/muscle/muscle_qfrc_projector.py:2816-2884), the producer of the slope that
+ * im_muscle_implicit_gather takes: per world and muscle the length over its consecutive
+ * waypoints [muscle_waypoint_start[m], muscle_waypoint_start[m + 1]), the lengthening velocity
+ * -sum over its entries e in [muscle_dof_offsets[m], muscle_dof_offsets[m + 1]) of
+ * moment[w, e] * qvel[w, muscle_dof_torque_idx[e] + root_dof_count] (one fused multiply-add per
+ * entry, in order), and from them effective_activation = a * fv, length_velocity,
+ * force_velocity_multiplier = fv and force_velocity_slope = include_active * a * unit_force *
+ * fv' / velocity_scale, velocity_scale = max(length_scale[m] * vmax, 1e-6).  The five outputs are
+ * (nworld, ld_out >= nmuscle).  Only the active curve of `model` is read. */
+int im_muscle_force_velocity_state(
+    const float *waypoints, int64_t ld_waypoints, const int32_t *muscle_waypoint_start,
+    const float *muscle_params, int ld_params, const float *muscle_rest_length,
+    const float *force_velocity_length_scale, const float *activation, int64_t ld_activation,
+    const float *qvel, int64_t ld_qvel, const float *moment, int64_t ld_moment,
+    const int32_t *muscle_dof_offsets, const int32_t *muscle_dof_torque_idx, int root_dof_count,
+    const im_muscle_force_model *model, const im_muscle_force_velocity_model *fv, int nmuscle,
+    float *muscle_length, float *effective_activation, float *length_velocity,
+    float *force_velocity_multiplier, float *force_velocity_slope, int64_t ld_out, int nworld,
+    void *stream);
 
 /* im_muscle_waypoints followed by im_muscle_force_magnitudes in one launch, for the caller
  * that wants both: MuscleDynamicsLayer._prepare_warp_waypoint_geometry

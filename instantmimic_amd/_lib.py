@@ -60,6 +60,10 @@ class MuscleForceModel(C.Structure):
     ]
 
 
+class MuscleForceVelocityModel(C.Structure):
+    _fields_ = [("vmax", C.c_float), ("fvmax", C.c_float), ("clamp_activation", C.c_float), ("include_active", C.c_float)]
+
+
 class MuscleGeometry(C.Structure):
     _fields_ = [
         ("waypoints", _vp), ("ld_waypoints", _i64),
@@ -118,6 +122,7 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _i64, _vp, _i, _vp, _vp, _i64, _vp, _i, _vp, _i64, _i64, _vp, _i64, _i64, _i, _i, _u, _vp],
     ),
+    "im_tree_pattern_violations": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp]),
     "im_check_reciprocal": (_i, [C.c_uint32, C.c_uint32, _vp, _vp]),
     "im_dof_pattern_create": (_i, [_i, _vp, _i, _vp, _vp, _vp, C.POINTER(_vp)]),
     "im_dof_pattern_destroy": (None, [_vp]),
@@ -150,6 +155,7 @@ SIGNATURES = {
     "im_copy_dense_factor": (_i, [_vp, _i, _vp, _i, _vp, _i64, _i, _vp]),
     "im_jtdj_mfma": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
     "im_muscle_project": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i64, _i, _vp]),
+    "im_muscle_gather_tables": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "im_muscle_implicit_gather": (
         _i,
         [_vp, _i64, _vp, _i64, _vp, _i, _vp, _i, _vp, _vp, _i, C.c_float, _vp, _i64, _i, _vp],
@@ -159,6 +165,11 @@ SIGNATURES = {
         _i,
         [_vp, _i64, _vp, _vp, _vp, _i, _vp, C.POINTER(MuscleForceModel), _i, _vp, _i64, _vp, _i64, _i, _vp],
     ),
+    "im_muscle_force_velocity_state": (
+        _i,
+        [_vp, _i64, _vp, _vp, _i, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i, C.POINTER(MuscleForceModel),
+         C.POINTER(MuscleForceVelocityModel), _i, _vp, _vp, _vp, _vp, _vp, _i64, _i, _vp],
+    ),  # fmt: skip
     "im_muscle_waypoints_forces": (
         _i,
         [_vp, _i64, _vp, _i64, _vp, _vp, _i, _vp, _i64, _vp, _vp, _vp, _i, _vp, C.POINTER(MuscleForceModel), _i,

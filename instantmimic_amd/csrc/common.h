@@ -32,6 +32,7 @@ struct TreeDev {
   const uint64_t *anc;      // [nsteps]    bit i set when dof i is a strict ancestor of k
   const int32_t *dof_d;     // [64]        rowadr | depth << 16 | trunk << 24, -1 past nv
   const int32_t *colind;    // [nM]
+  const uint64_t *related;  // [64]        bit i set when dof i is dof k itself, an ancestor or a descendant of it
   int32_t nv, nM, nsteps, maxdepth, ngroups;
 };
 

@@ -341,6 +341,44 @@ __global__ void check_reciprocal_kernel(uint32_t first, uint32_t last, unsigned 
   if (bad) atomicAdd(mismatches, bad);
 }
 
+// Constraint rows whose dofs do not all lie on one root-to-leaf chain: such a row has products
+// outside M's pattern, which the fused kernels cannot hold (they are dropped).  One wavefront per
+// world, a lane per dof; a row counts when its weight is not zero and some dof with a nonzero
+// entry is unrelated to another one.  The check of the reference's sparse assembly
+// (src/instantmimic/utils/mjw_kernels/sparse_hessian.py:605-621) on the tree pattern.
+__global__ __launch_bounds__(64) void tree_violation_kernel(const uint64_t *__restrict__ related, int nv,
+                                                            const float *__restrict__ J, int njmax,
+                                                            const float *__restrict__ D,
+                                                            const int32_t *__restrict__ state,
+                                                            const int32_t *__restrict__ nefc_p, int quad,
+                                                            float *__restrict__ violations) {
+  const int64_t w = blockIdx.x;
+  const int lane = threadIdx.x;
+  int ne = nefc_p ? nefc_p[w] : njmax;
+  ne = ne < njmax ? ne : njmax;
+  const uint64_t mine = lane < nv ? related[lane] : ~0ull;
+  const float *Jw = J + w * (int64_t)njmax * nv;
+  int bad_rows = 0;
+  for (int r0 = 0; r0 < ne; r0 += 4) {
+    float v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {  // four rows' entries in flight
+      const int r = r0 + u < ne ? r0 + u : ne - 1;
+      v[u] = lane < nv ? Jw[(int64_t)r * nv + lane] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int r = r0 + u;
+      if (r >= ne) break;
+      const bool counted = state[w * njmax + r] == quad && D[w * njmax + r] != 0.0f;
+      const uint64_t row = __ballot(v[u] != 0.0f);
+      const bool off_pattern = v[u] != 0.0f && (row & ~mine) != 0;
+      if (counted && __any(off_pattern)) ++bad_rows;
+    }
+  }
+  if (lane == 0 && bad_rows) violations[w] = violations[w] + (float)bad_rows;
+}
+
 // One launch of the generated kernels for `niter` iterations (see the kernels' prologue); the
 // table-driven kernel takes one iteration at a time.
 struct Iterations {
@@ -457,6 +495,15 @@ int tree_plan_upload(im_tree_plan *pl) {
   const size_t o_sd = off;    off = align(off + slot_d.size() * 4);
   const size_t o_dof = off;   off = align(off + dof_d.size() * 4);
   const size_t o_col = off;   off = align(off + (size_t)nM * 4);
+  const size_t o_rel = off;   off = align(off + 64 * sizeof(uint64_t));
+  // M's pattern row of every dof: itself, its ancestors, its descendants
+  std::vector<uint64_t> related(64, 0);
+  for (int b = 0; b < nv; ++b)
+    for (int q = 0; q < pl->rownnz[b]; ++q) {
+      const int a = pl->colind[pl->rowadr[b] + q];
+      related[b] |= 1ull << a;
+      related[a] |= 1ull << b;
+    }
   std::vector<char> blob(off, 0);
   std::memcpy(blob.data() + o_steps, steps.data(), steps.size() * sizeof(int4));
   std::memcpy(blob.data() + o_anc, anc.data(), anc.size() * sizeof(uint64_t));
@@ -464,6 +511,7 @@ int tree_plan_upload(im_tree_plan *pl) {
   std::memcpy(blob.data() + o_sd, slot_d.data(), slot_d.size() * 4);
   std::memcpy(blob.data() + o_dof, dof_d.data(), dof_d.size() * 4);
   std::memcpy(blob.data() + o_col, pl->colind.data(), (size_t)nM * 4);
+  std::memcpy(blob.data() + o_rel, related.data(), 64 * sizeof(uint64_t));
   IM_HIP_CHECK(hipGetDevice(&pl->device));
   IM_HIP_CHECK(hipMalloc(&pl->dev_blob, off));
   IM_HIP_CHECK(hipMemcpy(pl->dev_blob, blob.data(), off, hipMemcpyHostToDevice));
@@ -474,6 +522,7 @@ int tree_plan_upload(im_tree_plan *pl) {
   pl->dev.slot_d = (const uint32_t *)(base + o_sd);
   pl->dev.dof_d = (const int32_t *)(base + o_dof);
   pl->dev.colind = (const int32_t *)(base + o_col);
+  pl->dev.related = (const uint64_t *)(base + o_rel);
   pl->dev.nv = nv;
   pl->dev.nM = nM;
   pl->dev.nsteps = int(steps.size());
@@ -504,6 +553,19 @@ int im_tree_factor_solve(const im_tree_plan *plan, const float *M, int64_t ldM,
                          int nworld, void *stream) {
   return im::launch(plan, false, M, ldM, nullptr, 0, nullptr, nullptr, nullptr, 0, y, ldy,
                     x, ldx, nullptr, nworld, 0u, stream);
+}
+
+int im_tree_pattern_violations(const im_tree_plan *plan, const float *J, int njmax, const float *D,
+                               const int32_t *state, const int32_t *nefc, int quad, float *violations, int nworld,
+                               void *stream) {
+  if (!plan || nworld < 0 || njmax < 0) return IM_ERR_ARG;
+  if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
+  if (nworld == 0 || njmax == 0) return IM_OK;
+  if (!J || !D || !state || !violations) return IM_ERR_ARG;
+  hipLaunchKernelGGL(im::tree_violation_kernel, dim3(nworld), dim3(64), 0, (hipStream_t)stream, plan->dev.related,
+                     plan->nv, J, njmax, D, state, nefc, quad, violations);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
 }
 
 int im_check_reciprocal(uint32_t first_bits, uint32_t last_bits, unsigned long long *mismatches, void *stream) {

@@ -83,16 +83,3 @@ def factor_factory(nv: int, pad: int, sparse_plan: SparseHessianPlan | None = No
                 _lib.check(status, "im_dense_update_factor")
 
     return kernel
-
-
-def hessian_step(J, D, state, w: int, r: int, row: int, col: int, delta: float, quad: int = QUADRATIC) -> Any:
-    """Host statement of one term of the incremental update, for callers that need the
-    rule itself (reference newton_stages.py:451-470): delta + (+-D a b), unchanged when the
-    row does not reach both dofs.  Not used by the launchers."""
-    a, b = float(J[w, r, row]), float(J[w, r, col])
-    if a == 0.0 or b == 0.0:
-        return delta
-    da = float(D[w, r]) * a
-    if int(state[w, r]) != quad:
-        da = -da
-    return delta + da * b

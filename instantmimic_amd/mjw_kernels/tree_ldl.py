@@ -308,3 +308,27 @@ def assemble_tree_factor_solve_iters(
             int(nworld), niter, _lib.IM_FLAG_NEGATE if negate else 0, _stream_ptr(M),
         )  # fmt: skip
     _lib.check(status, "im_assemble_tree_ldl_solve_iters")
+
+
+def pattern_violations(scratch: TreeFactorSolveScratch, J, D, state, nefc, violations, *, quad: int = QUADRATIC) -> None:
+    """Adds to ``violations`` (nworld,) float32 the number of active constraint rows of every world
+    whose dofs do not lie on one root-to-leaf chain: rows the fused tree solve cannot represent
+    (their products outside M's pattern are dropped).  The counter accumulates, like the
+    reference's ``violation_counter`` (sparse_hessian.py:786-796); zero it after a nonzero read."""
+    import torch
+
+    if J.dim() != 3 or not J.is_contiguous() or not D.is_contiguous() or not state.is_contiguous():
+        raise ValueError("J, D and state must be contiguous")
+    nworld, njmax, nv = (int(v) for v in J.shape)
+    if nv != scratch.kernel.info().nv or tuple(D.shape) != (nworld, njmax) or tuple(state.shape) != (nworld, njmax):
+        raise ValueError("J, D and state do not match the plan or each other")
+    if violations.dtype != torch.float32 or violations.numel() != nworld or not violations.is_contiguous():
+        raise TypeError("violations must be a contiguous float32 tensor with one element per world")
+    if state.dtype != torch.int32 or (nefc is not None and (nefc.dtype != torch.int32 or nefc.numel() != nworld)):
+        raise TypeError("state and nefc must be int32, nefc one element per world")
+    with torch.cuda.device(J.device):
+        status = _lib.lib().im_tree_pattern_violations(
+            scratch.kernel.ptr, J.data_ptr(), njmax, D.data_ptr(), state.data_ptr(),
+            nefc.data_ptr() if nefc is not None else None, int(quad), violations.data_ptr(), nworld, _stream_ptr(J),
+        )  # fmt: skip
+    _lib.check(status, "im_tree_pattern_violations")

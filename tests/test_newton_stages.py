@@ -165,14 +165,6 @@ def test_oracle_dense_stage_against_fp64(name, nworld):
     assert (err / (cond * 6e-8))[refactored].max() < 4.0
 
 
-def test_hessian_step_rule():
-    J = np.array([[[2.0, 0.0, 3.0]]])
-    D = np.array([[5.0]])
-    assert NS.hessian_step(J, D, np.array([[Q]]), 0, 0, 0, 2, 1.0) == 1.0 + 5 * 2 * 3
-    assert NS.hessian_step(J, D, np.array([[0]]), 0, 0, 0, 2, 1.0) == 1.0 - 5 * 2 * 3
-    assert NS.hessian_step(J, D, np.array([[Q]]), 0, 0, 0, 1, 1.0) == 1.0
-
-
 # ---------------------------------------------------------------- GPU parity
 
 
