@@ -255,6 +255,23 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done,
                             int ldg, float *hfactor, int32_t *dof_union, float *search,
                             float *search_dot, float *decrement, int nworld, void *stream);
 
+/* Replaces the factor step of the upstream (non-fused) Newton iteration on the static pattern
+ * (nonfused_kernel, src/instantmimic/utils/mjw_kernels/sparse_hessian.py:849-894, native modes 4
+ * and 5 of :639-679).  Needs a plan built with IM_SPARSE_NONFUSED.  Per world, skipped when
+ * done[w], or when skip_noflip and state_changed[w] == 0:
+ *   refactor (always, unless skip_unchanged and quad_changed[w] == 0): the slots of the factor
+ *     are gathered from the dense Hessian H[w] (nv_pad x nv_pad, world stride ldH) through SH_GAT,
+ *     factored level by level with grad as the augmented row, and hfactor[w] receives
+ *     [0, nfac) N = L D and [nfac, nfac + nv) 1 / D;
+ *   otherwise the factor stored in hfactor[w] solves the new gradient.
+ * Then the backward solve, search = -x, search_dot, decrement.  done, quad_changed,
+ * state_changed may be null where the flags do not ask for them. */
+int im_sparse_dense_factor(const im_sparse_plan *plan, const uint8_t *done, const float *grad, int ldg,
+                           const float *H, int64_t ldH, const int32_t *quad_changed,
+                           const int32_t *state_changed, int skip_unchanged, int skip_noflip,
+                           float *hfactor, float *search, int ld_search, float *search_dot,
+                           float *decrement, int nworld, void *stream);
+
 /* The same stage on the dense Hessian (newton_stages.py:614-742 without a sparse plan):
  * H (nworld, nv_pad, nv_pad) receives the deltas on its upper triangle
  * (H[w, row, col] += delta, row <= col, :700-701); with changed rows the augmented blocked

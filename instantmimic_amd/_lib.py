@@ -143,6 +143,7 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp],
     ),
+    "im_sparse_dense_factor": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i, _vp, _vp, _i, _vp]),
     "im_dense_update_factor": (
         _i,
         [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],

@@ -615,8 +615,8 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
   float *A = rhs + pad;       // [(pad / B) * B * B]
   float *L = A + (pad / B) * B * B;  // [B * B + B]: lower factor of the diagonal tile, 1 / pivots
   int *ul = (int *)(L + B * B + B);  // [nv] union list, [nv] = its length
-  unsigned *mkl = (unsigned *)(ul + nv + 1);  // [nv] per dof: bit t set where staged row t is nonzero there
-  float *jr = (float *)(mkl + nv);  // [row_cap][nv] changed rows of J, then [row_cap] signed weights
+  unsigned *mkl = (unsigned *)(ul + nv + 1);  // [nv] per dof: nonzero when a changed row reaches it
+  float *jr = (float *)(mkl + nv);  // [row_cap][nv] a batch of changed rows of J, then [row_cap] signed weights
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
   if ((done && done[w]) || state_changes[w] == 0) return;
@@ -627,29 +627,13 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
   count = count < ld_ids ? count : ld_ids;
   for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? gw[i] : 0.0f;
   if (count > 0) {
-    // Up to row_cap changed rows of J and their signed weights are staged in LDS, H's upper
-    // triangle is brought into the LDS array of the factor, updated there, written back, and
-    // factored in place; more changed rows than that are read from memory pair by pair.
-    const bool staged = count <= row_cap;
+    // H's upper triangle is brought into the LDS array of the factor, updated there, written back,
+    // and factored in place.  The changed rows of J and their signed weights pass through LDS
+    // row_cap at a time, the pair sums staying in the matrix cores' accumulators from one batch to
+    // the next; without room for a batch of four rows they are read from memory pair by pair.
+    const bool staged = row_cap >= 4;
     float *sd = jr + (size_t)row_cap * nv;
     if (staged) {
-      const int total = count * nv;
-      for (int q0 = tid; q0 < total; q0 += 4 * nt) {
-        float v[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const int q = q0 + k * nt < total ? q0 + k * nt : total - 1;
-          const int t = q / nv;
-          v[k] = Jw[(size_t)idw[t] * nv + (q - t * nv)];
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if (q0 + k * nt < total) jr[q0 + k * nt] = v[k];
-      }
-      for (int t = tid; t < count; t += nt) {
-        const int r = idw[t];
-        sd[t] = sw[r] == quad ? Dw[r] : -Dw[r];
-      }
       // 16 bytes per lane and four requests in flight; the tiles below the diagonal are not read
       const int nvec = pad * pad / 4;  // pad is a multiple of 16
       for (int i0 = tid; i0 < nvec; i0 += 4 * nt) {
@@ -676,6 +660,84 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
           }
         }
       }
+      for (int dof = tid; dof < nv; dof += nt) mkl[dof] = 0u;
+      // All pair sums of a 16 x 16 tile of dofs at once on the matrix cores.  Every changed row
+      // enters every pair here, also where one of the two dofs is zero in it: such a term adds
+      // +-0 to a sum that started at +0, which leaves all its bits, so the sums equal the ones
+      // that skip those rows.  v_mfma_f32_16x16x4_f32 adds its four products one after the
+      // other with a fused multiply-add each, rows ascending; a batch holds a multiple of four
+      // rows, so the chain of a pair runs through the batches as through one list.
+      typedef float f32x4 __attribute__((ext_vector_type(4)));
+      constexpr int HELD = 5;  // tiles a wavefront keeps sums for at a time (36 tiles over 8 wavefronts at nv 128)
+      const int lane = tid & 63, p = lane & 15, kq = lane >> 4, wv = tid >> 6, nwv = nt >> 6;
+      const int nb = (nv + 15) / 16, ntiles = nb * (nb + 1) / 2;
+      for (int tile0 = 0; tile0 < ntiles; tile0 += HELD * nwv) {
+        f32x4 acc[HELD];
+        int ra[HELD], ca[HELD];
+#pragma unroll
+        for (int h = 0; h < HELD; ++h) {
+          acc[h] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+          const int tile = tile0 + wv + h * nwv;
+          int cb = (int)((sqrtf((float)(8 * tile + 1)) - 1.0f) * 0.5f);
+          while ((cb + 1) * (cb + 2) / 2 <= tile) ++cb;
+          while (cb * (cb + 1) / 2 > tile) --cb;
+          const int rb = tile - cb * (cb + 1) / 2;
+          ra[h] = tile < ntiles ? 16 * rb + p : -1;  // the dofs this lane feeds; -1: no such tile
+          ca[h] = 16 * cb + p;
+        }
+        for (int c0 = 0; c0 < count; c0 += row_cap) {
+          const int nrow = count - c0 < row_cap ? count - c0 : row_cap;
+          __syncthreads();  // the batch before this one has been read by everyone
+          const int total = nrow * nv;
+          for (int q0 = tid; q0 < total; q0 += 4 * nt) {
+            float v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int q = q0 + k * nt < total ? q0 + k * nt : total - 1;
+              const int t = q / nv;
+              v[k] = Jw[(size_t)idw[c0 + t] * nv + (q - t * nv)];
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+              if (q0 + k * nt < total) jr[q0 + k * nt] = v[k];
+          }
+          for (int t = tid; t < nrow; t += nt) {
+            const int r = idw[c0 + t];
+            sd[t] = sw[r] == quad ? Dw[r] : -Dw[r];
+          }
+          __syncthreads();
+          if (tile0 == 0)  // dofs some changed row reaches
+            for (int dof = tid; dof < nv; dof += nt) {
+              unsigned hit = mkl[dof];
+              for (int t = 0; t < nrow && !hit; ++t) hit = jr[t * nv + dof] != 0.0f;
+              mkl[dof] = hit;
+            }
+#pragma unroll
+          for (int h = 0; h < HELD; ++h) {
+            if (ra[h] < 0) continue;  // the same for the whole wavefront
+            for (int t0 = 0; t0 < nrow; t0 += 4) {
+              const int t = t0 + kq, tc = t < nrow ? t : nrow - 1;
+              const float wgt = t < nrow ? sd[tc] : 0.0f;
+              const float a = ra[h] < nv ? wgt * jr[tc * nv + ra[h]] : 0.0f;  // -(D a) == (-D) a exactly
+              const float b = (t < nrow && ca[h] < nv) ? jr[tc * nv + ca[h]] : 0.0f;
+              acc[h] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[h], 0, 0, 0);
+            }
+          }
+        }
+#pragma unroll
+        for (int h = 0; h < HELD; ++h) {
+          if (ra[h] < 0) continue;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int row = ra[h] - p + 4 * kq + i, col = ca[h];
+            if (row <= col && col < nv && acc[h][i] != 0.0f) {
+              const float hv = U[S.at(row, col)] + acc[h][i];
+              U[S.at(row, col)] = hv;
+              Hw[(size_t)row * pad + col] = hv;
+            }
+          }
+        }
+      }
       __syncthreads();
     }
     if (tid < 64) {
@@ -685,10 +747,7 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
         bool hit = false;
         if (dof < nv) {
           if (staged) {
-            unsigned mk = 0u;
-            for (int t = 0; t < count; ++t) mk |= (unsigned)(jr[t * nv + dof] != 0.0f) << t;
-            mkl[dof] = mk;
-            hit = mk != 0u;
+            hit = mkl[dof] != 0u;
           } else {
             for (int t = 0; t < count && !hit; ++t) hit = Jw[(size_t)idw[t] * nv + dof] != 0.0f;
           }
@@ -704,59 +763,14 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
     int32_t *uni = uni_ + w * (nv + 1);
     for (int i = tid; i < nu; i += nt) uni[i] = ul[i];
     if (tid == 0) uni[nv] = nu;
-    if (staged && B == 16) {
-      // All pair sums of a 16 x 16 tile of dofs at once on the matrix cores.  Every staged row
-      // enters every pair here, also where one of the two dofs is zero in it: such a term adds
-      // +-0 to a sum that started at +0, which leaves all its bits, so the sums equal the ones
-      // that skip those rows.  v_mfma_f32_16x16x4_f32 adds its four products one after the
-      // other with a fused multiply-add each, rows ascending.
-      typedef float f32x4 __attribute__((ext_vector_type(4)));
-      const int lane = tid & 63, p = lane & 15, kq = lane >> 4;
-      const int nb = (nv + 15) / 16, ntiles = nb * (nb + 1) / 2;
-      for (int tile = tid >> 6; tile < ntiles; tile += nt >> 6) {
-        int cb = (int)((sqrtf((float)(8 * tile + 1)) - 1.0f) * 0.5f);
-        while ((cb + 1) * (cb + 2) / 2 <= tile) ++cb;
-        while (cb * (cb + 1) / 2 > tile) --cb;
-        const int rb = tile - cb * (cb + 1) / 2;
-        const int ra = 16 * rb + p, ca = 16 * cb + p;  // the dofs this lane feeds
-        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (int t0 = 0; t0 < count; t0 += 4) {
-          const int t = t0 + kq, tc = t < count ? t : count - 1;
-          const float wgt = t < count ? sd[tc] : 0.0f;
-          const float a = ra < nv ? wgt * jr[tc * nv + ra] : 0.0f;  // -(D a) == (-D) a exactly
-          const float b = (t < count && ca < nv) ? jr[tc * nv + ca] : 0.0f;
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc, 0, 0, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int row = 16 * rb + 4 * kq + i, col = ca;
-          if (row <= col && col < nv && acc[i] != 0.0f) {
-            const float h = U[S.at(row, col)] + acc[i];
-            U[S.at(row, col)] = h;
-            Hw[(size_t)row * pad + col] = h;
-          }
-        }
-      }
-    } else {
-    const int npair = nu * (nu + 1) / 2;
-    for (int e = tid; e < npair; e += nt) {
-      int cj = (int)((sqrtf((float)(8 * e + 1)) - 1.0f) * 0.5f);
-      while ((cj + 1) * (cj + 2) / 2 <= e) ++cj;
-      while (cj * (cj + 1) / 2 > e) --cj;
-      const int row = ul[e - cj * (cj + 1) / 2], col = ul[cj];
-      float delta = 0.0f;
-      if (staged) {
-        // only the rows in which both dofs are nonzero add to the pair, ascending
-        for (unsigned mm = mkl[row] & mkl[col]; mm; mm &= mm - 1u) {
-          const int t = __builtin_ctz(mm);
-          delta = fma_(sd[t] * jr[t * nv + row], jr[t * nv + col], delta);  // -(D a) == (-D) a exactly
-        }
-        if (delta != 0.0f) {
-          const float h = U[S.at(row, col)] + delta;
-          U[S.at(row, col)] = h;
-          Hw[(size_t)row * pad + col] = h;
-        }
-      } else {
+    if (!staged) {
+      const int npair = nu * (nu + 1) / 2;
+      for (int e = tid; e < npair; e += nt) {
+        int cj = (int)((sqrtf((float)(8 * e + 1)) - 1.0f) * 0.5f);
+        while ((cj + 1) * (cj + 2) / 2 <= e) ++cj;
+        while (cj * (cj + 1) / 2 > e) --cj;
+        const int row = ul[e - cj * (cj + 1) / 2], col = ul[cj];
+        float delta = 0.0f;
         for (int t = 0; t < count; ++t) {
           const int r = idw[t];
           const float a = Jw[(size_t)r * nv + row], b = Jw[(size_t)r * nv + col];
@@ -766,7 +780,6 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
         }
         if (delta != 0.0f) Hw[(size_t)row * pad + col] = Hw[(size_t)row * pad + col] + delta;
       }
-    }
     }
     if (staged) {
       __syncthreads();
@@ -1257,9 +1270,10 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
       sizeof(float) * ((size_t)im::Stair<B>{nv_pad}.words() + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + B +
                        2 * (size_t)nv + 1);
   if (base_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
-  // room for up to 32 changed rows of J next to the factor, as far as the 160 KB of LDS reach
-  int row_cap = ld_ids < 32 ? ld_ids : 32;
-  while (row_cap > 0 && base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1) > 160 * 1024) --row_cap;
+  // room for a batch of up to 32 changed rows of J next to the factor (a multiple of four rows), as
+  // far as the 160 KB of LDS reach
+  int row_cap = 32;
+  while (row_cap > 0 && base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1) > 160 * 1024) row_cap -= 4;
   const size_t lds_bytes = base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1);
   auto fn = im::dense_update_factor_kernel<B>;
   if (lds_bytes > 64 * 1024)

@@ -23,7 +23,7 @@ namespace im {
 namespace {
 
 struct SparseDev {
-  const int32_t *t[NTABLES];
+  const int32_t *t[NHOST];
   int nv, nv_pad, nslots, nlevels;
 };
 
@@ -755,6 +755,64 @@ __global__ void sparse_update_kernel(SparseDev P, const uint8_t *__restrict__ do
   backward_sums(P, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, block, block);
 }
 
+// Upstream (non-fused) iteration: the dense Hessian that the upstream assembly and incremental
+// update maintain is read through SH_GAT into the factor's slots and factored on the pattern, or,
+// for a world whose QUADRATIC rows did not change, the stored factor solves the new gradient.
+// hfactor holds [0, nfac) N = L D and [nfac, nfac + n) 1 / D.  Reference: sparse_hessian.py:639-679
+// (modes 4 and 5) inside nonfused_kernel (:849-894).
+__global__ void sparse_dense_factor_kernel(SparseDev P, const uint8_t *__restrict__ done,
+                                           const float *__restrict__ grad, int ldg,
+                                           const float *__restrict__ H, int64_t ldH,
+                                           const int32_t *__restrict__ quad_changed,
+                                           const int32_t *__restrict__ state_changed, int skip_unchanged,
+                                           int skip_noflip, float *__restrict__ U_, float *__restrict__ search_,
+                                           int ld_search, float *__restrict__ search_dot,
+                                           float *__restrict__ decrement) {
+  extern __shared__ float lds[];
+  const int w = blockIdx.x, lane = threadIdx.x, block = blockDim.x;
+  if (done && done[w]) return;
+  if (skip_noflip && state_changed[w] == 0) return;
+  const bool refactor = !(skip_unchanged && quad_changed[w] == 0);
+  const int n = P.nv, nslots = P.nslots, nfac = nslots - n, rhs = nfac;
+  const int nw = (block + 31) / 32;
+  float *N = lds;          // [nslots]
+  float *iD = N + nslots;  // [n]
+  float *red = iD + n;     // [2][nw]
+  float *U = U_ + (size_t)w * P.nv_pad * P.nv_pad;
+  const float *gw = grad + (size_t)w * ldg;
+  const int32_t *ORIGt = P.t[ORIG];
+  if (refactor) {
+    const float *Hw = H + (size_t)w * ldH;
+    const uint32_t *GATt = (const uint32_t *)P.t[GAT];
+    for (int s = lane; s < nfac; s += block) N[s] = Hw[GATt[s]];
+    for (int j = lane; j < n; j += block) N[rhs + j] = gw[ORIGt[j]];
+    __syncthreads();
+    factor_levels(P, N, iD, lane, block);
+    for (int s = lane; s < nfac; s += block) U[s] = N[s];
+    for (int j = lane; j < n; j += block) U[nfac + j] = iD[j];
+  } else {
+    for (int s = lane; s < nfac; s += block) N[s] = U[s];
+    for (int j = lane; j < n; j += block) iD[j] = U[nfac + j];
+    __syncthreads();
+    const int32_t *FLt = P.t[FL], *FRt = P.t[FR], *RSt = P.t[RS], *RKPt = P.t[RKP], *RKt = P.t[RK];
+    for (int l = 0; l < P.nlevels; ++l) {
+      for (int q = FLt[l] + lane; q < FLt[l + 1]; q += block) {
+        const int j = FRt[q];
+        float v = gw[ORIGt[j]];
+        const float *rowp = N + RSt[j];
+        const int k0 = RKPt[j], k1 = RKPt[j + 1];
+        for (int t = 0; t < k1 - k0; ++t) {
+          const int k = RKt[k0 + t];
+          v = fma_(-(rowp[t] * iD[k]), N[rhs + k], v);
+        }
+        N[rhs + j] = v;
+      }
+      __syncthreads();
+    }
+  }
+  backward_sums(P, N, iD, gw, search_ + (size_t)w * ld_search, red, search_dot + w, decrement + w, lane, block, block);
+}
+
 }  // namespace
 }  // namespace im
 
@@ -766,21 +824,22 @@ namespace im {
 
 int sparse_plan_upload(im_sparse_plan *pl) {
   pl->device_ready = false;
-  if (pl->block != 32 && pl->block != 64) return IM_ERR_UNSUPPORTED;  // the kernels' workgroup widths
+  // the kernels' workgroup widths; 128 lanes only in the upstream-iteration kernel
+  if (pl->block != 32 && pl->block != 64 && !(pl->path == IM_SPARSE_NONFUSED && pl->block == 128)) return IM_ERR_UNSUPPORTED;
   const int nv = pl->nv, nfac = pl->nfac;
   size_t total = 0;
-  size_t offs[NTABLES];
-  for (int i = 0; i < NTABLES; ++i) {
+  size_t offs[NHOST];
+  for (int i = 0; i < NHOST; ++i) {
     offs[i] = total;
     pl->sizes[i] = (int)pl->table[i].size();
     total += (pl->table[i].size() * 4 + 15) / 16 * 16;
   }
   std::vector<char> host(total, 0);
-  for (int i = 0; i < NTABLES; ++i) memcpy(host.data() + offs[i], pl->table[i].data(), pl->table[i].size() * 4);
+  for (int i = 0; i < NHOST; ++i) memcpy(host.data() + offs[i], pl->table[i].data(), pl->table[i].size() * 4);
   IM_HIP_CHECK(hipMalloc(&pl->blob, total));
   IM_HIP_CHECK(hipMemcpy(pl->blob, host.data(), total, hipMemcpyHostToDevice));
-  for (int i = 0; i < NTABLES; ++i) pl->t[i] = (const int32_t *)((char *)pl->blob + offs[i]);
-  if (nv <= 64 && pl->nslots < 65535) {
+  for (int i = 0; i < NHOST; ++i) pl->t[i] = (const int32_t *)((char *)pl->blob + offs[i]);
+  if (nv <= 64 && pl->nslots < 65535 && !pl->table[SA].empty()) {
     const int32_t *sa = pl->table[SA].data(), *sb = pl->table[SB].data(), *sm = pl->table[SM].data();
     const int nt = (nv + 15) / 16;
     std::vector<int32_t> tix((size_t)nt * (nt + 1) / 2 * 256, 0);
@@ -820,12 +879,12 @@ int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done, const
                           const float *M, int ldM, const float *grad, int ldg, float *hfactor,
                           float *search, float *search_dot, float *decrement, int nworld, void *stream) {
   if (!plan || nworld < 0 || njmax <= 0) return IM_ERR_ARG;  // rows are clamped to njmax - 1
-  if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
+  if (!plan->device_ready || plan->path != IM_SPARSE_FUSED) return IM_ERR_UNSUPPORTED;
   if (nworld == 0) return IM_OK;
   if (!nefc || !J || !D || !state || !M || !grad || !hfactor || !search || !search_dot || !decrement) return IM_ERR_ARG;
   if (ldg < plan->nv) return IM_ERR_STRIDE;
   im::SparseDev P;
-  for (int i = 0; i < im::NTABLES; ++i) P.t[i] = plan->t[i];
+  for (int i = 0; i < im::NHOST; ++i) P.t[i] = plan->t[i];
   P.nv = plan->nv; P.nv_pad = plan->nv_pad; P.nslots = plan->nslots; P.nlevels = plan->nlevels;
   const int n = plan->nv, words = (n + 31) / 32, nw = (plan->block + 31) / 32;
   static const bool simple_only = [] {
@@ -875,14 +934,14 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done, con
                             float *hfactor, int32_t *dof_union, float *search, float *search_dot,
                             float *decrement, int nworld, void *stream) {
   if (!plan || nworld < 0 || ld_ids < 0 || njmax <= 0) return IM_ERR_ARG;
-  if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
+  if (!plan->device_ready || plan->path != IM_SPARSE_FUSED) return IM_ERR_UNSUPPORTED;
   if (nworld == 0) return IM_OK;
   if (!state_changes || !changes || !ids || !J || !D || !state || !grad || !hfactor || !dof_union || !search ||
       !search_dot || !decrement)
     return IM_ERR_ARG;
   if (ldg < plan->nv) return IM_ERR_STRIDE;
   im::SparseDev P;
-  for (int i = 0; i < im::NTABLES; ++i) P.t[i] = plan->t[i];
+  for (int i = 0; i < im::NHOST; ++i) P.t[i] = plan->t[i];
   P.nv = plan->nv; P.nv_pad = plan->nv_pad; P.nslots = plan->nslots; P.nlevels = plan->nlevels;
   const int n = plan->nv, nw = (plan->block + 31) / 32;
   static const bool simple_only = [] {
@@ -943,6 +1002,30 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done, con
   hipLaunchKernelGGL(im::sparse_update_kernel, dim3(nworld), dim3(plan->block), lds_bytes, (hipStream_t)stream, P,
                      done, state_changes, changes, ids, ld_ids, J, njmax, D, state, quad, grad, ldg, hfactor,
                      dof_union, search, search_dot, decrement);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_sparse_dense_factor(const im_sparse_plan *plan, const uint8_t *done, const float *grad, int ldg,
+                           const float *H, int64_t ldH, const int32_t *quad_changed,
+                           const int32_t *state_changed, int skip_unchanged, int skip_noflip, float *hfactor,
+                           float *search, int ld_search, float *search_dot, float *decrement, int nworld,
+                           void *stream) {
+  if (!plan || nworld < 0) return IM_ERR_ARG;
+  if (!plan->device_ready || plan->sizes[im::GAT] == 0) return IM_ERR_UNSUPPORTED;  // a plan of the fused path
+  if (nworld == 0) return IM_OK;
+  if (!grad || !H || !hfactor || !search || !search_dot || !decrement) return IM_ERR_ARG;
+  if ((skip_unchanged && !quad_changed) || (skip_noflip && !state_changed)) return IM_ERR_ARG;
+  if (ldg < plan->nv || ld_search < plan->nv || ldH < (int64_t)plan->nv_pad * plan->nv_pad) return IM_ERR_STRIDE;
+  im::SparseDev P;
+  for (int i = 0; i < im::NHOST; ++i) P.t[i] = plan->t[i];
+  P.nv = plan->nv; P.nv_pad = plan->nv_pad; P.nslots = plan->nslots; P.nlevels = plan->nlevels;
+  const int nw = (plan->block + 31) / 32;
+  const size_t lds_bytes = 4 * ((size_t)plan->nslots + plan->nv + 2 * nw);
+  if (lds_bytes > 64 * 1024) return IM_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(im::sparse_dense_factor_kernel, dim3(nworld), dim3(plan->block), lds_bytes, (hipStream_t)stream,
+                     P, done, grad, ldg, H, ldH, quad_changed, state_changed, skip_unchanged, skip_noflip, hfactor,
+                     search, ld_search, search_dot, decrement);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

@@ -30,8 +30,8 @@ struct im_sparse_plan {
   // device side (sparse_kernels.hip)
   bool device_ready = false;
   void *blob = nullptr;
-  const int32_t *t[im::NTABLES] = {};
-  int sizes[im::NTABLES] = {};
+  const int32_t *t[im::NHOST] = {};
+  int sizes[im::NHOST] = {};
   // per lane of the lower-triangle 16 x 16 accumulator tiles: where the element comes from in a
   // row of M and which slot it is ((M index + 1) << 16 | (slot + 1)); null when nv > 64
   int32_t *tile_index = nullptr;

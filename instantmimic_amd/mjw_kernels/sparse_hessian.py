@@ -383,6 +383,73 @@ def init_factor_kernel(plan: SparseHessianPlan):
     return launch
 
 
+def nonfused_kernel(plan: SparseHessianPlan, skip_unchanged: bool, skip_noflip: bool):
+    """Launcher of the upstream iteration's factor step with the sparse factor: refactor from the
+    dense Hessian when rows changed QUADRATIC state (always without ``skip_unchanged``), else
+    solve with the stored factor; ``skip_noflip`` leaves worlds without state changes alone.
+    Called with the reference kernel's arguments
+    ``(done, grad3, H, quad_changed, state_changed, hfactor, search3, search_dot, decrement)`` (:849-894)."""
+    ptr = _device_plan(plan)
+    if plan.path != "nonfused":
+        raise ValueError("the upstream-iteration factor needs a plan of the nonfused path")
+    skip_unchanged, skip_noflip = bool(skip_unchanged), bool(skip_noflip)
+
+    def launch(done, grad, H, quad_changed, state_changed, hfactor, search, search_dot, decrement):
+        import torch
+
+        nworld = int(H.shape[0])
+        if tuple(H.shape) != (nworld, plan.nv_pad, plan.nv_pad) or tuple(hfactor.shape) != tuple(H.shape):
+            raise ValueError("H and hfactor must be (nworld, nv_pad, nv_pad)")
+        if grad.shape[0] != nworld or grad[0].numel() < plan.nv or search.shape[0] != nworld or search[0].numel() < plan.nv:
+            raise ValueError("grad and search do not match the plan")
+        for t in (grad, H, hfactor, search, search_dot, decrement):
+            if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous() or t.device != H.device:
+                raise ValueError("arrays must be contiguous float32 CUDA tensors on one device")
+        ptrs = []
+        for t, name, dtypes, needed in ((done, "done", (torch.bool, torch.uint8), False),
+                                        (quad_changed, "quad_changed", (torch.int32,), skip_unchanged),
+                                        (state_changed, "state_changed", (torch.int32,), skip_noflip)):  # fmt: skip
+            if t is None:
+                if needed:
+                    raise ValueError(f"{name} is needed with this kernel's skip flags")
+                ptrs.append(None)
+                continue
+            if t.dtype not in dtypes or t.numel() != nworld or not t.is_cuda or not t.is_contiguous():
+                raise TypeError(f"{name} must be a contiguous CUDA tensor with one element per world")
+            ptrs.append(t.data_ptr())
+        with torch.cuda.device(H.device):
+            status = _lib.lib().im_sparse_dense_factor(
+                ptr, ptrs[0], grad.data_ptr(), int(grad[0].numel()), H.data_ptr(), int(H.stride(0)), ptrs[1], ptrs[2],
+                int(skip_unchanged), int(skip_noflip), hfactor.data_ptr(), search.data_ptr(), int(search[0].numel()),
+                search_dot.data_ptr(), decrement.data_ptr(), nworld, int(torch.cuda.current_stream(H.device).cuda_stream),
+            )  # fmt: skip
+        _lib.check(status, "im_sparse_dense_factor")
+
+    return launch
+
+
+def nonfused_solver_functions(plan: SparseHessianPlan):
+    """``cholesky_factorize_solve(m, d, ctx, skip_unchanged=False, skip_noflip=False)``: the
+    function the reference substitutes for upstream's ``_cholesky_factorize_solve`` (:909-942),
+    reading ``ctx.done, grad, h, quad_changed_count, state_changed_count, hfactor, search,
+    search_dot, newton_decrement``.  Upstream's ``_update_gradient`` / ``_solver_iteration``,
+    which the reference rebinds around it, are third-party code and stay the caller's."""
+    kernels = {}
+
+    def cholesky_factorize_solve(m, d, ctx, skip_unchanged=False, skip_noflip=False):
+        key = (bool(skip_unchanged), bool(skip_noflip))
+        if key not in kernels:
+            kernels[key] = nonfused_kernel(plan, *key)
+        state = ctx.state_changed_count if skip_noflip else ctx.quad_changed_count
+        nworld = int(d.nworld)
+        kernels[key](
+            ctx.done, ctx.grad.reshape(nworld, ctx.grad.shape[1], 1), ctx.h, ctx.quad_changed_count, state, ctx.hfactor,
+            ctx.search.reshape(nworld, int(m.nv), 1), ctx.search_dot, ctx.newton_decrement,
+        )  # fmt: skip
+
+    return cholesky_factorize_solve
+
+
 def pattern_misses(h: np.ndarray, plan_adj, tol: float = 0.0) -> int:
     """Nonzero upper-triangle entries of dense Hessians ``h`` (nworld, nv_pad, nv_pad)
     outside a dof adjacency (:946-957)."""

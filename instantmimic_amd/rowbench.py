@@ -1,6 +1,6 @@
 """Per-kernel timings of the library on the configured shapes, one JSON line per kernel:
 
-    python -m instantmimic_amd.rowbench [--launches N]
+    python -m instantmimic_amd.rowbench [--launches N] [--only trees,stress,muscles,walks,iteration,bodies] [--no-graph]
 
 Every line names the kernel, the workload, the mean time of one launch (event-timed hipGraph
 replay over rotating input sets), the algorithmic bytes or flops of that launch and the
@@ -20,10 +20,21 @@ HBM_GBS = 8000.0
 MFMA_F32_TFLOPS = 157.3
 
 
+GRAPH = True  # False (--no-graph): plain launches, which is what a counter run of rocprofv3 sees per dispatch
+
+
 def _timeit(torch, fn, nsets: int, launches: int) -> float:
     for i in range(min(nsets, 4)):
         fn(i)
     torch.cuda.synchronize()
+    if not GRAPH:
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(launches):
+            fn(i % nsets)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / launches * 1e-3
     g = torch.cuda.CUDAGraph()
     s = torch.cuda.Stream()
     s.wait_stream(torch.cuda.current_stream())
@@ -59,15 +70,19 @@ def _line(kernel, workload, seconds, *, bytes_=None, flops=None, nworld=None):
     print(json.dumps(out), flush=True)
 
 
-def run(launches: int = 32) -> None:
+def run(launches: int = 32, only: str | None = None) -> None:
+    """``only``: comma-separated section names out of trees, stress, muscles, walks, iteration, bodies."""
     import torch
 
     from . import synth
     from .mjw_kernels import blocked_dense as BD
+    from .mjw_kernels import newton_fusion as NF
     from .mjw_kernels import newton_stages as NS
     from .mjw_kernels import sparse_hessian as SH
+    from .mjw_kernels import tree_fusion as TF
     from .mjw_kernels import tree_ldl as T
     from .muscle import muscle_qfrc_projector as Q
+    from .muscle import wrench_projection as WP
     from .muscle.muscle_dynamics import MuscleDynamicsLayer
 
     dev = torch.device("cuda:0")
@@ -78,227 +93,305 @@ def run(launches: int = 32) -> None:
     def sets_of(arrays, nsets):
         return [[t(a) for a in arrays] for _ in range(nsets)]
 
+    wanted = None if only is None else {w.strip() for w in only.split(",")}
+
+    def section(name):
+        return wanted is None or name in wanted
+
+    # ---- a 64 MiB device copy, for scaling the FETCH_SIZE / WRITE_SIZE counters of a profiler run (only when asked for)
+    if wanted is not None and "calibration" in wanted:
+        src, dst = torch.ones(16 << 20, device=dev), torch.zeros(16 << 20, device=dev)
+        sec = _timeit(torch, lambda i: dst.copy_(src), 1, 8)
+        _line("64 MiB device copy", "16 Mi floats", sec, bytes_=2 * (64 << 20))
+        del src, dst
+
     # ---- fused assemble + tree L'DL + solve and solve-only on every tree shape
-    for name, nsets in (("ant", 8), ("humanoid", 16), ("g1", 8), ("snu", 8)):
-        b = synth.make_batch(name)
-        nv, nM, nefc, nworld = b.shape.nv, int(b.colind.size), b.shape.nefc, b.nworld
-        m = SimpleNamespace(nv=nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind)
-        sc = T.create_tree_factor_solve_scratch(m, dev)
-        S = sets_of((b.M, b.J, b.D, b.state[0], b.nefc, b.grad), nsets)
-        X = [torch.zeros(b.grad.shape, device=dev) for _ in range(nsets)]
-        wl = f"{name} nv={nv} nM={nM} nefc={nefc} x {nworld} worlds"
-        sec = _timeit(torch, lambda i: T.assemble_tree_factor_solve(sc, *S[i], X[i]), nsets, launches)
-        _line("im_assemble_tree_ldl_solve", wl, sec, bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv), nworld=nworld)
-        sec = _timeit(torch, lambda i: T.tree_factor_solve(sc, S[i][0], X[i], S[i][5]), nsets, launches)
-        _line("im_tree_factor_solve", wl, sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
-        if name in ("g1", "snu"):
-            # the same Hessians through the blocked dense factor and the static-pattern sparse L'DL
-            Md = synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32).reshape(nworld, -1)
-            mm = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))])
-            for B in (8, 16):
-                Mt = [t(Md) for _ in range(4)]
-                d = SimpleNamespace(nworld=nworld, M=Mt[0])
-                bs = BD.create_blocked_dense_factor_solve_scratch(mm, d, dev, block_size=B)
-                Y = t(b.grad).reshape(nworld, nv, 1)
-                Xb = torch.zeros_like(Y)
-                sec = _timeit(torch, lambda i: BD._blocked_dense_factor_solve(d, Mt[i], Xb, Y, bs), 4, launches)
-                _line(f"im_blocked_factor_solve B={B}", wl, sec, bytes_=nworld * 4 * (nv * nv + 2 * nv + bs.pad * bs.pad), nworld=nworld)
-            model = synth.model_from_parents(b.shape.parents)
-            plan, _ = SH.plan_for_model(model, None, [], SH.block_width(model.nv_pad), device=dev)
-            if plan is not None:
-                launch = SH.init_factor_kernel(plan)
-                hf = torch.zeros((nworld, plan.nv_pad, plan.nv_pad), device=dev)
-                search = torch.zeros((nworld, nv, 1), device=dev)
-                sd, de = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev)
-                G = [s[5][:, :, None].contiguous() for s in S]
-                sec = _timeit(torch, lambda i: launch(None, S[i][4], S[i][1], S[i][2], S[i][3], S[i][0], G[i], hf, search, sd, de), nsets, launches)
-                used = 2 * plan.nfac + nv
-                _line("im_sparse_init_factor", wl, sec, bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv + used + 2), nworld=nworld)
-                # per-iteration stage: a tenth of the rows change state
-                rng = np.random.default_rng(1)
-                ids = np.zeros((nworld, nefc), np.int32)
-                k = max(nefc // 10, 1)
-                for w in range(nworld):
-                    ids[w, :k] = np.sort(rng.choice(nefc, k, replace=False))
-                chg = t(np.full(nworld, k, np.int32))
-                uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=dev)
-                stage = NS.factor_factory(nv, plan.nv_pad, plan)
-                s2 = search.reshape(nworld, nv)
-                idt = t(ids)
-                sec = _timeit(torch, lambda i: stage(S[i][1], S[i][2], S[i][3], idt, chg, chg, None, S[i][5], None, hf, s2, sd, de, uni), nsets, launches)
-                _line("im_sparse_update_factor", wl + f", {k} changed rows", sec, bytes_=nworld * 4 * (k * nv + 2 * used + 2 * nv + nv + 1 + 2), nworld=nworld)
-        del S, X
-        torch.cuda.empty_cache()
+    if section("trees"):
+        for name, nsets in (("ant", 8), ("humanoid", 16), ("g1", 8), ("snu", 8)):
+            b = synth.make_batch(name)
+            nv, nM, nefc, nworld = b.shape.nv, int(b.colind.size), b.shape.nefc, b.nworld
+            m = SimpleNamespace(nv=nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind)
+            sc = T.create_tree_factor_solve_scratch(m, dev)
+            S = sets_of((b.M, b.J, b.D, b.state[0], b.nefc, b.grad), nsets)
+            X = [torch.zeros(b.grad.shape, device=dev) for _ in range(nsets)]
+            wl = f"{name} nv={nv} nM={nM} nefc={nefc} x {nworld} worlds"
+            sec = _timeit(torch, lambda i: T.assemble_tree_factor_solve(sc, *S[i], X[i]), nsets, launches)
+            _line("im_assemble_tree_ldl_solve", wl, sec, bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv), nworld=nworld)
+            if name != "ant":
+                # a step's three Newton iterations in one launch: M and J once, states / gradients / x per iteration
+                St = [torch.stack([s[3], 1 - s[3], s[3]]).contiguous() for s in S]
+                G3 = [torch.stack([s[5], -s[5], 2 * s[5]]).contiguous() for s in S]
+                X3 = [torch.zeros((3,) + tuple(b.grad.shape), device=dev) for _ in range(nsets)]
+                sec = _timeit(torch, lambda i: T.assemble_tree_factor_solve_iters(sc, S[i][0], S[i][1], S[i][2], St[i], S[i][4], G3[i], X3[i]), nsets, launches)
+                _line("im_assemble_tree_ldl_solve_iters (3 iterations, bytes of three separate solves)", wl, sec,
+                      bytes_=3 * nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv), nworld=3 * nworld)  # fmt: skip
+                del St, G3, X3
+            sec = _timeit(torch, lambda i: T.tree_factor_solve(sc, S[i][0], X[i], S[i][5]), nsets, launches)
+            _line("im_tree_factor_solve", wl, sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
+            if name in ("g1", "snu"):
+                # the same Hessians through the blocked dense factor and the static-pattern sparse L'DL
+                Md = synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32).reshape(nworld, -1)
+                mm = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))])
+                for B in (8, 16):
+                    Mt = [t(Md) for _ in range(4)]
+                    d = SimpleNamespace(nworld=nworld, M=Mt[0])
+                    bs = BD.create_blocked_dense_factor_solve_scratch(mm, d, dev, block_size=B)
+                    Y = t(b.grad).reshape(nworld, nv, 1)
+                    Xb = torch.zeros_like(Y)
+                    sec = _timeit(torch, lambda i: BD._blocked_dense_factor_solve(d, Mt[i], Xb, Y, bs), 4, launches)
+                    _line(f"im_blocked_factor_solve B={B}", wl, sec, bytes_=nworld * 4 * (nv * nv + 2 * nv + bs.pad * bs.pad), nworld=nworld)
+                model = synth.model_from_parents(b.shape.parents)
+                plan, _ = SH.plan_for_model(model, None, [], SH.block_width(model.nv_pad), device=dev)
+                if plan is not None:
+                    launch = SH.init_factor_kernel(plan)
+                    hf = torch.zeros((nworld, plan.nv_pad, plan.nv_pad), device=dev)
+                    search = torch.zeros((nworld, nv, 1), device=dev)
+                    sd, de = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev)
+                    G = [s[5][:, :, None].contiguous() for s in S]
+                    sec = _timeit(torch, lambda i: launch(None, S[i][4], S[i][1], S[i][2], S[i][3], S[i][0], G[i], hf, search, sd, de), nsets, launches)
+                    used = 2 * plan.nfac + nv
+                    _line("im_sparse_init_factor", wl, sec, bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv + used + 2), nworld=nworld)
+                    # per-iteration stage: a tenth of the rows change state
+                    rng = np.random.default_rng(1)
+                    ids = np.zeros((nworld, nefc), np.int32)
+                    k = max(nefc // 10, 1)
+                    for w in range(nworld):
+                        ids[w, :k] = np.sort(rng.choice(nefc, k, replace=False))
+                    chg = t(np.full(nworld, k, np.int32))
+                    uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=dev)
+                    stage = NS.factor_factory(nv, plan.nv_pad, plan)
+                    s2 = search.reshape(nworld, nv)
+                    idt = t(ids)
+                    sec = _timeit(torch, lambda i: stage(S[i][1], S[i][2], S[i][3], idt, chg, chg, None, S[i][5], None, hf, s2, sd, de, uni), nsets, launches)
+                    _line("im_sparse_update_factor", wl + f", {k} changed rows", sec, bytes_=nworld * 4 * (k * nv + 2 * used + 2 * nv + nv + 1 + 2), nworld=nworld)
+            del S, X
+            torch.cuda.empty_cache()
 
     # ---- stress: dense J'DJ on the matrix cores, blocked factor, dense per-iteration stage
-    b = synth.make_batch("stress", 16384)
-    nv, nefc, nworld = b.shape.nv, b.shape.nefc, b.nworld
-    pad = ((nv + 1 + 15) // 16) * 16
-    Md = t(synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32).reshape(nworld, -1))
-    J, D, st, ne, g = (t(a) for a in (b.J, b.D, b.state[0], b.nefc, b.grad))
-    H = torch.zeros((nworld, pad, pad), device=dev)
-    wl = f"stress nv={nv} nefc={nefc} x {nworld} worlds"
-    sec = _timeit(torch, lambda i: BD.dense_hessian(Md, J, D, st, ne, H), 1, 8)
-    _line("im_jtdj_mfma", wl, sec, flops=nworld * 2.0 * nv * nv * nefc, nworld=nworld)
-    _line("im_jtdj_mfma (as bytes)", wl, sec, bytes_=nworld * 4 * (nv * nv + nefc * nv + 2 * nefc + pad * pad), nworld=nworld)
-    mm = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))])
-    Hc = H[:, :nv, :nv].contiguous().reshape(nworld, -1)
-    d = SimpleNamespace(nworld=nworld, M=Hc)
-    bs = BD.create_blocked_dense_factor_solve_scratch(mm, d, dev, block_size=16)
-    Y = g.reshape(nworld, nv, 1)
-    Xb = torch.zeros_like(Y)
-    sec = _timeit(torch, lambda i: BD._blocked_dense_factor_solve(d, Hc, Xb, Y, bs), 1, 8)
-    _line("im_blocked_factor_solve B=16", wl, sec, bytes_=nworld * 4 * (nv * nv + 2 * nv + bs.pad * bs.pad), nworld=nworld)
-    rng = np.random.default_rng(2)
-    k = nefc // 10
-    ids = np.zeros((nworld, nefc), np.int32)
-    ids[:, :k] = np.sort(rng.permuted(np.tile(np.arange(nefc), (nworld, 1)), axis=1)[:, :k], axis=1)
-    chg = t(np.full(nworld, k, np.int32))
-    uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=dev)
-    U = torch.zeros((nworld, pad, pad), device=dev)
-    g3 = torch.zeros((nworld, pad, 1), device=dev)
-    g3[:, :nv, 0] = g
-    search = torch.zeros((nworld, pad, 1), device=dev)
-    sd, de = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev)
-    stage = NS.factor_factory(nv, pad)
-    idt = t(ids)
-    sec = _timeit(torch, lambda i: stage(J, D, st, idt, chg, chg, None, g3, H, U, search, sd, de, uni), 1, 8)
-    _line("im_dense_update_factor", wl + f", {k} changed rows", sec, bytes_=nworld * 4 * (k * nv + 2 * pad * pad + 2 * nv), nworld=nworld)
-    del J, H, U, Md, Hc
-    torch.cuda.empty_cache()
+    if section("stress"):
+        b = synth.make_batch("stress", 16384)
+        nv, nefc, nworld = b.shape.nv, b.shape.nefc, b.nworld
+        pad = ((nv + 1 + 15) // 16) * 16
+        Md = t(synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32).reshape(nworld, -1))
+        J, D, st, ne, g = (t(a) for a in (b.J, b.D, b.state[0], b.nefc, b.grad))
+        H = torch.zeros((nworld, pad, pad), device=dev)
+        wl = f"stress nv={nv} nefc={nefc} x {nworld} worlds"
+        sec = _timeit(torch, lambda i: BD.dense_hessian(Md, J, D, st, ne, H), 1, 8)
+        _line("im_jtdj_mfma", wl, sec, flops=nworld * 2.0 * nv * nv * nefc, nworld=nworld)
+        _line("im_jtdj_mfma (as bytes)", wl, sec, bytes_=nworld * 4 * (nv * nv + nefc * nv + 2 * nefc + pad * pad), nworld=nworld)
+        mm = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))])
+        Hc = H[:, :nv, :nv].contiguous().reshape(nworld, -1)
+        d = SimpleNamespace(nworld=nworld, M=Hc)
+        bs = BD.create_blocked_dense_factor_solve_scratch(mm, d, dev, block_size=16)
+        Y = g.reshape(nworld, nv, 1)
+        Xb = torch.zeros_like(Y)
+        sec = _timeit(torch, lambda i: BD._blocked_dense_factor_solve(d, Hc, Xb, Y, bs), 1, 8)
+        _line("im_blocked_factor_solve B=16", wl, sec, bytes_=nworld * 4 * (nv * nv + 2 * nv + bs.pad * bs.pad), nworld=nworld)
+        rng = np.random.default_rng(2)
+        k = nefc // 10
+        ids = np.zeros((nworld, nefc), np.int32)
+        ids[:, :k] = np.sort(rng.permuted(np.tile(np.arange(nefc), (nworld, 1)), axis=1)[:, :k], axis=1)
+        chg = t(np.full(nworld, k, np.int32))
+        uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=dev)
+        U = torch.zeros((nworld, pad, pad), device=dev)
+        g3 = torch.zeros((nworld, pad, 1), device=dev)
+        g3[:, :nv, 0] = g
+        search = torch.zeros((nworld, pad, 1), device=dev)
+        sd, de = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev)
+        stage = NS.factor_factory(nv, pad)
+        idt = t(ids)
+        sec = _timeit(torch, lambda i: stage(J, D, st, idt, chg, chg, None, g3, H, U, search, sd, de, uni), 1, 8)
+        _line("im_dense_update_factor", wl + f", {k} changed rows", sec, bytes_=nworld * 4 * (k * nv + 2 * pad * pad + 2 * nv), nworld=nworld)
+        k = nefc // 2
+        ids[:, :k] = np.sort(rng.permuted(np.tile(np.arange(nefc), (nworld, 1)), axis=1)[:, :k], axis=1)
+        idt, chg = t(ids), t(np.full(nworld, k, np.int32))
+        sec = _timeit(torch, lambda i: stage(J, D, st, idt, chg, chg, None, g3, H, U, search, sd, de, uni), 1, 8)
+        _line("im_dense_update_factor", wl + f", {k} changed rows (a fresh active mask)", sec, bytes_=nworld * 4 * (k * nv + 2 * pad * pad + 2 * nv), nworld=nworld)
+        del J, H, U, Md, Hc
+        torch.cuda.empty_cache()
 
     # ---- muscles on the SNU-like tree
-    nworld = 4096
-    mb = synth.make_muscles(nworld)
-    rowadr, rownnz, colind = synth.csr_from_parents(synth.snu_parents())
-    nv, nM = len(rowadr), int(colind.size)
-    ent = Q.entries_from_muscle_dofs(mb.muscle_dofs, mb.nmuscle)
-    ne_ = len(ent.muscle_dof_torque_idx)
-    offsets, order = Q.torque_sorted_entries(ent.muscle_dof_torque_idx, nv - mb.root_dof_count)
-    nsets = 8
-    mom = [t(mb.moment) for _ in range(nsets)]
-    frc = [t(mb.force) for _ in range(nsets)]
-    slope = [t(mb.slope) for _ in range(nsets)]
-    qfrc = torch.zeros((nworld, nv), device=dev)
-    off_d, ord_d, em_d = t(offsets), t(order), t(ent.muscle_dof_muscle_idx.astype(np.int32))
-    wl = f"snu nv={nv} muscles={mb.nmuscle} entries={ne_} x {nworld} worlds"
-    sec = _timeit(torch, lambda i: Q.project_muscle_sparse_moment_qfrc(mom[i], frc[i], off_d, ord_d, em_d, mb.root_dof_count, qfrc), nsets, launches)
-    _line("im_muscle_project", wl, sec, bytes_=nworld * 4 * (ne_ + mb.nmuscle + nv - mb.root_dof_count), nworld=nworld)
-    prepared = Q.prepare_muscle_implicit_qderiv_pairs(
-        pair_entry_i=ent.pair_entry_i, pair_entry_j=ent.pair_entry_j, pair_muscle_idx=ent.pair_muscle_idx,
-        muscle_dof_torque_idx=ent.muscle_dof_torque_idx, matrix_elemid=synth.matrix_elemid(rowadr, rownnz, colind),
-        root_dof_count=mb.root_dof_count,
-    )  # fmt: skip
-    gather = Q.build_muscle_implicit_qderiv_gather(prepared, ent.muscle_dof_muscle_idx, dev)
-    qd = torch.zeros((nworld, nM), device=dev)
-    sec = _timeit(torch, lambda i: Q.apply_muscle_implicit_qderiv_gather(gather, mom[i], slope[i], mb.timestep, qd), nsets, launches)
-    touched = int(gather.elem_ids.numel())
-    _line("im_muscle_implicit_gather", wl, sec, bytes_=nworld * 4 * (ne_ + mb.nmuscle + 2 * touched), nworld=nworld)
-    rig = synth.make_muscle_rig()
-    layer = MuscleDynamicsLayer(rig.topology, **rig.dims(), device=dev)
-    ctx = [t(synth.make_muscle_context(rig, nworld, seed=s)) for s in range(4)]
-    act = torch.rand((nworld, rig.muscle_count), device=dev)
-    gout = torch.randn((nworld, rig.torque_dim), device=dev)
-    wl = (f"snu rig: {rig.muscle_count} muscles, {layer.waypoint_count} waypoints, {len(layer.segments_host[0])} applied "
-          f"segments, {len(layer.torque_entries_host[2])} torque entries x {nworld} worlds")  # fmt: skip
-    cbytes = 4 * layer.context_dim
-    sec = _timeit(torch, lambda i: layer._warp_muscle_dynamics_from_activation_forward(act, ctx[i], include_passive_force=True), 4, launches)
-    _line("torque_forward (waypoints + force magnitudes + im_muscle_torque_forward)", wl, sec,
-          bytes_=nworld * (cbytes + 4 * (3 * layer.waypoint_count * 2 + 3 * rig.muscle_count + rig.muscle_count + rig.torque_dim)), nworld=nworld)  # fmt: skip
-    sec = _timeit(torch, lambda i: layer._warp_muscle_dynamics_from_activation_backward(ctx[i], gout), 4, launches)
-    _line("torque_backward (waypoints + force magnitudes + im_muscle_activation_grad)", wl, sec,
-          bytes_=nworld * (cbytes + 4 * (3 * layer.waypoint_count * 2 + 2 * rig.muscle_count + rig.muscle_count + rig.torque_dim)), nworld=nworld)  # fmt: skip
-    sec = _timeit(torch, lambda i: layer.eval_muscle_sparse_moment(ctx[i]), 4, launches)
-    _line("eval_muscle_sparse_moment (waypoints + im_muscle_sparse_moment)", wl, sec,
-          bytes_=nworld * (cbytes + 4 * (3 * layer.waypoint_count * 2 + len(layer.sparse_entries.muscle_dof_torque_idx))), nworld=nworld)  # fmt: skip
+    if section("muscles"):
+        nworld = 4096
+        mb = synth.make_muscles(nworld)
+        rowadr, rownnz, colind = synth.csr_from_parents(synth.snu_parents())
+        nv, nM = len(rowadr), int(colind.size)
+        ent = Q.entries_from_muscle_dofs(mb.muscle_dofs, mb.nmuscle)
+        ne_ = len(ent.muscle_dof_torque_idx)
+        offsets, order = Q.torque_sorted_entries(ent.muscle_dof_torque_idx, nv - mb.root_dof_count)
+        nsets = 8
+        mom = [t(mb.moment) for _ in range(nsets)]
+        frc = [t(mb.force) for _ in range(nsets)]
+        slope = [t(mb.slope) for _ in range(nsets)]
+        qfrc = torch.zeros((nworld, nv), device=dev)
+        off_d, ord_d, em_d = t(offsets), t(order), t(ent.muscle_dof_muscle_idx.astype(np.int32))
+        wl = f"snu nv={nv} muscles={mb.nmuscle} entries={ne_} x {nworld} worlds"
+        sec = _timeit(torch, lambda i: Q.project_muscle_sparse_moment_qfrc(mom[i], frc[i], off_d, ord_d, em_d, mb.root_dof_count, qfrc), nsets, launches)
+        _line("im_muscle_project", wl, sec, bytes_=nworld * 4 * (ne_ + mb.nmuscle + nv - mb.root_dof_count), nworld=nworld)
+        prepared = Q.prepare_muscle_implicit_qderiv_pairs(
+            pair_entry_i=ent.pair_entry_i, pair_entry_j=ent.pair_entry_j, pair_muscle_idx=ent.pair_muscle_idx,
+            muscle_dof_torque_idx=ent.muscle_dof_torque_idx, matrix_elemid=synth.matrix_elemid(rowadr, rownnz, colind),
+            root_dof_count=mb.root_dof_count,
+        )  # fmt: skip
+        gather = Q.build_muscle_implicit_qderiv_gather(prepared, ent.muscle_dof_muscle_idx, dev)
+        qd = torch.zeros((nworld, nM), device=dev)
+        sec = _timeit(torch, lambda i: Q.apply_muscle_implicit_qderiv_gather(gather, mom[i], slope[i], mb.timestep, qd), nsets, launches)
+        touched = int(gather.elem_ids.numel())
+        _line("im_muscle_implicit_gather", wl, sec, bytes_=nworld * 4 * (ne_ + mb.nmuscle + 2 * touched), nworld=nworld)
+        # the muscle terms into the fused solve: h A'sA into M, tau = A'f out of the right-hand side, solve
+        b = synth.make_batch("snu")
+        sc = T.create_tree_factor_solve_scratch(SimpleNamespace(nv=nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind), dev)
+        S = sets_of((b.M, b.J, b.D, b.state[0], b.nefc, b.grad), nsets)
+        Mq = [torch.empty_like(s[0]) for s in S]
+        rhs, xs = torch.zeros((nworld, nv), device=dev), torch.zeros((nworld, nv), device=dev)
+        nefc = b.shape.nefc
+
+        def chain(i):
+            Mq[i].copy_(S[i][0])
+            Q.apply_muscle_implicit_qderiv_gather(gather, mom[i], slope[i], mb.timestep, Mq[i])
+            Q.project_muscle_sparse_moment_qfrc(mom[i], frc[i], off_d, ord_d, em_d, mb.root_dof_count, qfrc)
+            torch.sub(S[i][5], qfrc, out=rhs)
+            T.assemble_tree_factor_solve(sc, Mq[i], S[i][1], S[i][2], S[i][3], S[i][4], rhs, xs)
+
+        sec = _timeit(torch, chain, nsets, launches)
+        _line("muscle terms + fused solve: copy M, im_muscle_implicit_gather, im_muscle_project, subtract, im_assemble_tree_ldl_solve (five launches)",
+              wl + f" nefc={nefc}", sec, bytes_=nworld * 4 * (2 * ne_ + 2 * mb.nmuscle + nM + nefc * nv + 2 * nefc + 2 * nv), nworld=nworld)  # fmt: skip
+        # the slope's producer
+        ws = np.concatenate([[0], np.cumsum(np.full(mb.nmuscle, 4))]).astype(np.int32)
+        rngm = np.random.default_rng(4)
+        wps = [torch.randn((nworld, int(ws[-1]), 3), device=dev) for _ in range(4)]
+        par = t(np.stack([rngm.uniform(100, 3000, mb.nmuscle), rngm.uniform(0.5, 1.5, mb.nmuscle), rngm.uniform(0, 0.5, mb.nmuscle), rngm.uniform(0, 0.5, mb.nmuscle)], 1).astype(np.float32))
+        rest, scale = t(rngm.uniform(2, 6, mb.nmuscle).astype(np.float32)), t(rngm.uniform(0.1, 0.5, mb.nmuscle).astype(np.float32))
+        actv, qv = torch.rand((nworld, mb.nmuscle), device=dev), torch.randn((nworld, nv), device=dev)
+        outs = [torch.zeros((nworld, mb.nmuscle), device=dev) for _ in range(5)]
+        ws_d = t(ws)
+        dof_off, dof_tq = t(ent.muscle_dof_offsets.astype(np.int32)), t(ent.muscle_dof_torque_idx.astype(np.int32))
+        sec = _timeit(
+            torch,
+            lambda i: Q.eval_muscle_force_velocity_state(
+                wps[i], ws_d, par, rest, scale, actv, qv, mom[i], dof_off, dof_tq, mb.root_dof_count,
+                muscle_force_scale=1.0, muscle_length_norm_min=0.4, muscle_length_norm_max=1.6, vmax=1.5, fvmax=1.4,
+                clamp_activation=True, include_active=True, active_force_model_params=np.array([1.0, 0.5, 1.6], np.float32),
+                muscle_length=outs[0], effective_activation=outs[1], length_velocity=outs[2],
+                force_velocity_multiplier=outs[3], force_velocity_slope=outs[4],
+            ),
+            4, launches,
+        )  # fmt: skip
+        _line("im_muscle_force_velocity_state", wl + f", {int(ws[-1])} waypoints", sec,
+              bytes_=nworld * 4 * (3 * int(ws[-1]) + ne_ + nv + mb.nmuscle + 5 * mb.nmuscle), nworld=nworld)  # fmt: skip
+        del S, Mq
+        rig = synth.make_muscle_rig()
+        layer = MuscleDynamicsLayer(rig.topology, **rig.dims(), device=dev)
+        ctx = [t(synth.make_muscle_context(rig, nworld, seed=s)) for s in range(4)]
+        act = torch.rand((nworld, rig.muscle_count), device=dev)
+        gout = torch.randn((nworld, rig.torque_dim), device=dev)
+        wl = (f"snu rig: {rig.muscle_count} muscles, {layer.waypoint_count} waypoints, {len(layer.segments_host[0])} applied "
+              f"segments, {len(layer.torque_entries_host[2])} torque entries x {nworld} worlds")  # fmt: skip
+        cbytes = 4 * layer.context_dim
+        sec = _timeit(torch, lambda i: layer._warp_muscle_dynamics_from_activation_forward(act, ctx[i], include_passive_force=True), 4, launches)
+        _line("torque_forward (waypoints + force magnitudes + im_muscle_torque_forward)", wl, sec,
+              bytes_=nworld * (cbytes + 4 * (3 * layer.waypoint_count * 2 + 3 * rig.muscle_count + rig.muscle_count + rig.torque_dim)), nworld=nworld)  # fmt: skip
+        sec = _timeit(torch, lambda i: layer._warp_muscle_dynamics_from_activation_backward(ctx[i], gout), 4, launches)
+        _line("torque_backward (waypoints + force magnitudes + im_muscle_activation_grad)", wl, sec,
+              bytes_=nworld * (cbytes + 4 * (3 * layer.waypoint_count * 2 + 2 * rig.muscle_count + rig.muscle_count + rig.torque_dim)), nworld=nworld)  # fmt: skip
+        sec = _timeit(torch, lambda i: layer.eval_muscle_sparse_moment(ctx[i]), 4, launches)
+        _line("eval_muscle_sparse_moment (waypoints + im_muscle_sparse_moment)", wl, sec,
+              bytes_=nworld * (cbytes + 4 * (3 * layer.waypoint_count * 2 + len(layer.sparse_entries.muscle_dof_torque_idx))), nworld=nworld)  # fmt: skip
 
     # ---- the tree walks either side of the solve
-    from .mjw_kernels import newton_fusion as NF
-    from .mjw_kernels import tree_fusion as TF
-    from .muscle import wrench_projection as WP
+    if section("walks"):
+        for name, nsets in (("humanoid", 16), ("snu", 8)):
+            b = synth.make_batch(name)
+            nv, nM, nworld = b.shape.nv, int(b.colind.size), b.nworld
+            tables = [t(a) for a in NF.mul_m_tables(b.rowadr, b.rownnz, b.colind)]
+            Ms, Vs = [t(b.M) for _ in range(nsets)], [t(b.grad) for _ in range(nsets)]
+            out = torch.zeros((nworld, nv), device=dev)
+            sec = _timeit(torch, lambda i: NF.mul_m(Ms[i], Vs[i], out, *tables), nsets, launches)
+            _line("im_mul_m_sparse", f"{name} nv={nv} nM={nM} x {nworld} worlds", sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
+        for name, nsets in (("humanoid", 16), ("g1", 8), ("snu", 8)):
+            b = synth.make_batch(name)
+            nv, nefc, nworld = b.shape.nv, b.shape.nefc, b.nworld
+            Js, Fs = [t(b.J) for _ in range(nsets)], [torch.randn((nworld, nefc), device=dev) for _ in range(nsets)]
+            ne, sm, ma = t(b.nefc), t(b.grad), torch.randn((nworld, nv), device=dev)
+            chg, al = torch.ones(nworld, dtype=torch.int32, device=dev), torch.zeros(nworld, device=dev)
+            qc, gr = torch.zeros((nworld, nv), device=dev), torch.zeros((nworld, nv), device=dev)
+            gd, de, sc = (torch.zeros(nworld, device=dev) for _ in range(3))
+            un = torch.zeros(nworld, dtype=torch.uint8, device=dev)
+            sec = _timeit(torch, lambda i: NF.gradient(ne, Js[i], Fs[i], sm, ma, chg, al, None, qc, gr, gd, de, sc, un), nsets, launches)
+            _line("im_newton_gradient", f"{name} nv={nv} nefc={nefc} x {nworld} worlds", sec,
+                  bytes_=nworld * 4 * (nefc * nv + nefc + 4 * nv + 6), nworld=nworld)  # fmt: skip
+            jvo = torch.zeros((nworld, nefc), device=dev)
+            sec = _timeit(torch, lambda i: NF.jv(Js[i], sm, jvo, nefc=ne), nsets, launches)
+            _line("im_newton_jv", f"{name} nv={nv} nefc={nefc} x {nworld} worlds", sec, bytes_=nworld * 4 * (nefc * nv + nefc + nv), nworld=nworld)
 
-    for name, nsets in (("humanoid", 16), ("snu", 8)):
-        b = synth.make_batch(name)
-        nv, nM, nworld = b.shape.nv, int(b.colind.size), b.nworld
-        tables = [t(a) for a in NF.mul_m_tables(b.rowadr, b.rownnz, b.colind)]
-        Ms, Vs = [t(b.M) for _ in range(nsets)], [t(b.grad) for _ in range(nsets)]
-        out = torch.zeros((nworld, nv), device=dev)
-        sec = _timeit(torch, lambda i: NF.mul_m(Ms[i], Vs[i], out, *tables), nsets, launches)
-        _line("im_mul_m_sparse", f"{name} nv={nv} nM={nM} x {nworld} worlds", sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
-    for name, nsets in (("humanoid", 16), ("g1", 8), ("snu", 8)):
-        b = synth.make_batch(name)
-        nv, nefc, nworld = b.shape.nv, b.shape.nefc, b.nworld
-        Js, Fs = [t(b.J) for _ in range(nsets)], [torch.randn((nworld, nefc), device=dev) for _ in range(nsets)]
-        ne, sm, ma = t(b.nefc), t(b.grad), torch.randn((nworld, nv), device=dev)
-        chg, al = torch.ones(nworld, dtype=torch.int32, device=dev), torch.zeros(nworld, device=dev)
-        qc, gr = torch.zeros((nworld, nv), device=dev), torch.zeros((nworld, nv), device=dev)
-        gd, de, sc = (torch.zeros(nworld, device=dev) for _ in range(3))
-        un = torch.zeros(nworld, dtype=torch.uint8, device=dev)
-        sec = _timeit(torch, lambda i: NF.gradient(ne, Js[i], Fs[i], sm, ma, chg, al, None, qc, gr, gd, de, sc, un), nsets, launches)
-        _line("im_newton_gradient", f"{name} nv={nv} nefc={nefc} x {nworld} worlds", sec,
-              bytes_=nworld * 4 * (nefc * nv + nefc + 4 * nv + 6), nworld=nworld)  # fmt: skip
-        jvo = torch.zeros((nworld, nefc), device=dev)
-        sec = _timeit(torch, lambda i: NF.jv(Js[i], sm, jvo, nefc=ne), nsets, launches)
-        _line("im_newton_jv", f"{name} nv={nv} nefc={nefc} x {nworld} worlds", sec, bytes_=nworld * 4 * (nefc * nv + nefc + nv), nworld=nworld)
     # ---- one Newton iteration from the library's pieces, tree path, humanoid
-    b = synth.make_batch("humanoid")
-    nv, nM, nefc, nworld = b.shape.nv, int(b.colind.size), b.shape.nefc, b.nworld
-    sc_tree = T.create_tree_factor_solve_scratch(SimpleNamespace(nv=nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind), dev)
-    nsets = 16
-    S = sets_of((b.M, b.J, b.D, b.state[0], b.state[1], b.nefc), nsets)
-    f32 = lambda *shape: torch.randn(shape, device=dev)  # noqa: E731
-    i32 = lambda: torch.zeros(nworld, dtype=torch.int32, device=dev)  # noqa: E731
-    search, mvv, qacc, Ma, smooth, force = f32(nworld, nv), f32(nworld, nv), f32(nworld, nv), f32(nworld, nv), f32(nworld, nv), f32(nworld, nefc)
-    jvv, jaref, alpha = torch.zeros((nworld, nefc), device=dev), f32(nworld, nefc), torch.rand(nworld, device=dev)
-    ids, qcnt, scnt, nit = torch.zeros((nworld, nefc), dtype=torch.int32, device=dev), i32(), i32(), i32()
-    qc, gr = torch.zeros((nworld, nv), device=dev), torch.zeros((nworld, nv), device=dev)
-    gd, de, gs, imp = (torch.ones(nworld, device=dev) for _ in range(4))
-    un, dn = torch.zeros(nworld, dtype=torch.uint8, device=dev), torch.zeros(nworld, dtype=torch.uint8, device=dev)
-    tol, inertia = torch.full((1,), 1e-30, device=dev), torch.ones(1, device=dev)
+    if section("iteration"):
+        b = synth.make_batch("humanoid")
+        nv, nM, nefc, nworld = b.shape.nv, int(b.colind.size), b.shape.nefc, b.nworld
+        sc_tree = T.create_tree_factor_solve_scratch(SimpleNamespace(nv=nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind), dev)
+        nsets = 16
+        S = sets_of((b.M, b.J, b.D, b.state[0], b.state[1], b.nefc), nsets)
+        f32 = lambda *shape: torch.randn(shape, device=dev)  # noqa: E731
+        i32 = lambda: torch.zeros(nworld, dtype=torch.int32, device=dev)  # noqa: E731
+        search, mvv, qacc, Ma, smooth, force = f32(nworld, nv), f32(nworld, nv), f32(nworld, nv), f32(nworld, nv), f32(nworld, nv), f32(nworld, nefc)
+        jvv, jaref, alpha = torch.zeros((nworld, nefc), device=dev), f32(nworld, nefc), torch.rand(nworld, device=dev)
+        ids, qcnt, scnt, nit = torch.zeros((nworld, nefc), dtype=torch.int32, device=dev), i32(), i32(), i32()
+        qc, gr = torch.zeros((nworld, nv), device=dev), torch.zeros((nworld, nv), device=dev)
+        gd, de, gs, imp = (torch.ones(nworld, device=dev) for _ in range(4))
+        un, dn = torch.zeros(nworld, dtype=torch.uint8, device=dev), torch.zeros(nworld, dtype=torch.uint8, device=dev)
+        tol, inertia = torch.full((1,), 1e-30, device=dev), torch.ones(1, device=dev)
 
-    def iteration(i):
-        M_, J_, D_, s0, s1, ne_ = S[i]
-        NF.jv(J_, search, jvv, nefc=ne_, skip_world=dn)
-        NF.advance(alpha, search, mvv, jvv, qacc, Ma, jaref, nefc=ne_, done=dn)
-        NF.changed_rows(s0, s1, ids, qcnt, scnt, nefc=ne_, done=dn)
-        NF.gradient(ne_, J_, force, smooth, Ma, scnt, alpha, dn, qc, gr, gd, de, gs, un)
-        T.assemble_tree_factor_solve(sc_tree, M_, J_, D_, s1, ne_, gr, search, negate=True)
-        NF.converged(alpha, imp, gd, de, tol, inertia, nv, 1 << 30, nit, dn)
+        def iteration(i):
+            M_, J_, D_, s0, s1, ne_ = S[i]
+            NF.jv(J_, search, jvv, nefc=ne_, skip_world=dn)
+            NF.advance(alpha, search, mvv, jvv, qacc, Ma, jaref, nefc=ne_, done=dn)
+            NF.changed_rows(s0, s1, ids, qcnt, scnt, nefc=ne_, done=dn)
+            NF.gradient(ne_, J_, force, smooth, Ma, scnt, alpha, dn, qc, gr, gd, de, gs, un)
+            T.assemble_tree_factor_solve(sc_tree, M_, J_, D_, s1, ne_, gr, search, negate=True)
+            NF.converged(alpha, imp, gd, de, tol, inertia, nv, 1 << 30, nit, dn)
 
-    sec = _timeit(torch, iteration, nsets, launches)
-    _line("one Newton iteration: jv, step, changed rows, gradient, fused tree solve, convergence test (six launches)",
-          f"humanoid nv={nv} nefc={nefc} x {nworld} worlds", sec,
-          bytes_=nworld * 4 * (3 * nefc * nv + nM + 8 * nefc + 12 * nv + 10), nworld=nworld)  # fmt: skip
-    topo = rig.topology
-    nb, nvf = rig.body_count, rig.full_torque_dim
-    parent = np.asarray(topo.body_parentid, np.int32)
-    order, offsets, _, _ = WP.tree_levels(parent)
-    model = SimpleNamespace(body_parentid=parent, body_tree=[order[offsets[i] : offsets[i + 1]] for i in range(len(offsets) - 1)])
-    scratch = TF.create_tree_reduction_scratch(model, deterministic=True, device=dev)
-    for comp, skip, what in ((3, False, "subtree_com"), (10, True, "crb")):
-        vals = [torch.randn((nworld, nb, comp), device=dev) for _ in range(8)]
-        sec = _timeit(torch, lambda i: TF.accumulate(model, None, vals[i], comp, skip, scratch), 8, launches)
-        _line(f"im_tree_accumulate ({what}: {comp} components)", f"snu rig body tree: {nb} bodies, {len(offsets) - 1} levels x {nworld} worlds", sec,
-              bytes_=nworld * 4 * 2 * nb * comp, nworld=nworld)  # fmt: skip
-    wt = WP.build_wrench_projection_topology(t(parent), t(np.asarray(topo.dof_bodyid, np.int32)), nb, dev)
-    rootid = t(np.asarray(topo.body_rootid, np.int32))
-    ins = [[torch.randn((nworld, nb, 3), device=dev) for _ in range(4)] + [torch.randn((nworld, nvf, 6), device=dev)] for _ in range(8)]
-    mean = torch.zeros((nworld, rig.torque_dim), device=dev)
-    root = nvf - rig.torque_dim
-    sec = _timeit(
-        torch,
-        lambda i: WP.launch_project_body_wrench_to_torque(
-            wt, body_force=ins[i][0], body_torque=ins[i][1], xipos=ins[i][2], subtree_com=ins[i][3], cdof=ins[i][4],
-            body_rootid=rootid, mean=mean, body_count=nb, torque_dim=rig.torque_dim, root_dof_count=root,
-            output_dof_offset=0, batch_size=nworld,
-        ),
-        8, launches,
-    )  # fmt: skip
-    _line("im_project_body_wrenches", f"snu rig: {nb} bodies, {rig.torque_dim} torque dofs x {nworld} worlds", sec,
-          bytes_=nworld * 4 * (12 * nb + 6 * nvf + rig.torque_dim), nworld=nworld)  # fmt: skip
+        sec = _timeit(torch, iteration, nsets, launches)
+        _line("one Newton iteration: jv, step, changed rows, gradient, fused tree solve, convergence test (six launches)",
+              f"humanoid nv={nv} nefc={nefc} x {nworld} worlds", sec,
+              bytes_=nworld * 4 * (3 * nefc * nv + nM + 8 * nefc + 12 * nv + 10), nworld=nworld)  # fmt: skip
+
+    # ---- body-tree accumulations and the wrench projection
+    if section("bodies"):
+        rig = synth.make_muscle_rig()
+        topo = rig.topology
+        nb, nvf = rig.body_count, rig.full_torque_dim
+        parent = np.asarray(topo.body_parentid, np.int32)
+        order, offsets, _, _ = WP.tree_levels(parent)
+        model = SimpleNamespace(body_parentid=parent, body_tree=[order[offsets[i] : offsets[i + 1]] for i in range(len(offsets) - 1)])
+        scratch = TF.create_tree_reduction_scratch(model, deterministic=True, device=dev)
+        for comp, skip, what in ((3, False, "subtree_com"), (10, True, "crb")):
+            vals = [torch.randn((nworld, nb, comp), device=dev) for _ in range(8)]
+            sec = _timeit(torch, lambda i: TF.accumulate(model, None, vals[i], comp, skip, scratch), 8, launches)
+            _line(f"im_tree_accumulate ({what}: {comp} components)", f"snu rig body tree: {nb} bodies, {len(offsets) - 1} levels x {nworld} worlds", sec,
+                  bytes_=nworld * 4 * 2 * nb * comp, nworld=nworld)  # fmt: skip
+        wt = WP.build_wrench_projection_topology(t(parent), t(np.asarray(topo.dof_bodyid, np.int32)), nb, dev)
+        rootid = t(np.asarray(topo.body_rootid, np.int32))
+        ins = [[torch.randn((nworld, nb, 3), device=dev) for _ in range(4)] + [torch.randn((nworld, nvf, 6), device=dev)] for _ in range(8)]
+        mean = torch.zeros((nworld, rig.torque_dim), device=dev)
+        root = nvf - rig.torque_dim
+        sec = _timeit(
+            torch,
+            lambda i: WP.launch_project_body_wrench_to_torque(
+                wt, body_force=ins[i][0], body_torque=ins[i][1], xipos=ins[i][2], subtree_com=ins[i][3], cdof=ins[i][4],
+                body_rootid=rootid, mean=mean, body_count=nb, torque_dim=rig.torque_dim, root_dof_count=root,
+                output_dof_offset=0, batch_size=nworld,
+            ),
+            8, launches,
+        )  # fmt: skip
+        _line("im_project_body_wrenches", f"snu rig: {nb} bodies, {rig.torque_dim} torque dofs x {nworld} worlds", sec,
+              bytes_=nworld * 4 * (12 * nb + 6 * nvf + rig.torque_dim), nworld=nworld)  # fmt: skip
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--launches", type=int, default=32)
-    run(ap.parse_args().launches)
+    ap.add_argument("--only", default=None, help="comma-separated sections: trees, stress, muscles, walks, iteration, bodies")
+    ap.add_argument("--no-graph", action="store_true", help="plain launches instead of a hipGraph replay")
+    args = ap.parse_args()
+    GRAPH = not args.no_graph
+    run(args.launches, args.only)

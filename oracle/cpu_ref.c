@@ -366,7 +366,7 @@ static void sp_backward_sums(const sparse_t *p, float *N, const float *iD, const
       N[rhs + j] = fmaf(-N[p->BS[q]], N[rhs + i] * iD[i], N[rhs + j]);
     }
   /* per-lane sums, 32-lane shuffle tree, warps added in order */
-  float s0[64] = {0}, s1[64] = {0};
+  float s0[128] = {0}, s1[128] = {0};
   for (int lane = 0; lane < block; ++lane)
     for (int j = lane; j < n; j += block) {
       const int d = p->ORIG[j];
@@ -540,6 +540,60 @@ int orc_sparse_update_factor(int nv, int nv_pad, int block, int nslots, int nlev
       } else {
         for (int s = 0; s < nfac; ++s) N[s] = U[nfac + s];
         for (int j = 0; j < n; ++j) iD[j] = U[2 * nfac + j];
+        for (int l = 0; l < nlevels; ++l)
+          for (int q = FL[l]; q < FL[l + 1]; ++q) {
+            const int j = FR[q];
+            float v = g[p.ORIG[j]];
+            const float *rowp = N + RS[j];
+            for (int t = 0; t < RKP[j + 1] - RKP[j]; ++t) {
+              const int k = RK[RKP[j] + t];
+              v = fmaf(-(rowp[t] * iD[k]), N[rhs + k], v);
+            }
+            N[rhs + j] = v;
+          }
+      }
+      sp_backward_sums(&p, N, iD, g, search + (size_t)w * n, sdot + w, decr + w);
+    }
+    free(N);
+  }
+  return 0;
+}
+
+/* Factor step of the upstream (non-fused) iteration (sparse_hessian.py:639-679, modes 4 / 5,
+ * dispatched as in nonfused_kernel :849-894): refactor from the dense H through SH_GAT, or solve
+ * with the stored factor; hfactor = [0, nfac) N, [nfac, nfac + n) 1 / D.  tables[16..21] as in
+ * orc_sparse_update_factor, tables[22] = SH_GAT. */
+int orc_sparse_dense_factor(int nv, int nv_pad, int block, int nslots, int nlevels,
+                            const int *const *tables, int nworld, const unsigned char *done,
+                            const float *grad, int ldg, const float *H, const int *quad_changed,
+                            const int *state_changed, int skip_unchanged, int skip_noflip,
+                            float *hfactor, float *search, float *sdot, float *decr) {
+  sparse_t p = {nv, nv_pad, block, nslots, nlevels, tables[0], tables[1], tables[2], tables[3],
+                tables[4], tables[5], tables[6], tables[7], tables[8], tables[9], tables[10],
+                tables[11], tables[12], tables[13], tables[14], tables[15]};
+  const int *FL = tables[17], *FR = tables[18], *RS = tables[19], *RKP = tables[20],
+            *RK = tables[21], *GAT = tables[22];
+  const int n = nv, nfac = nslots - nv, rhs = nfac;
+  if (nv > 1024 || block > 128) return 1;
+#pragma omp parallel
+  {
+    float *N = (float *)malloc(sizeof(float) * (nslots + nv + 8));
+    float *iD = N + nslots;
+#pragma omp for schedule(static)
+    for (int w = 0; w < nworld; ++w) {
+      if (done && done[w]) continue;
+      if (skip_noflip && state_changed[w] == 0) continue;
+      float *U = hfactor + (size_t)w * nv_pad * nv_pad;
+      const float *Hw = H + (size_t)w * nv_pad * nv_pad, *g = grad + (size_t)w * ldg;
+      if (!(skip_unchanged && quad_changed[w] == 0)) {
+        for (int s = 0; s < nfac; ++s) N[s] = Hw[GAT[s]];
+        for (int j = 0; j < n; ++j) N[rhs + j] = g[p.ORIG[j]];
+        sp_factor_levels(&p, N, iD);
+        for (int s = 0; s < nfac; ++s) U[s] = N[s];
+        for (int j = 0; j < n; ++j) U[nfac + j] = iD[j];
+      } else {
+        for (int s = 0; s < nfac; ++s) N[s] = U[s];
+        for (int j = 0; j < n; ++j) iD[j] = U[nfac + j];
         for (int l = 0; l < nlevels; ++l)
           for (int q = FL[l]; q < FL[l + 1]; ++q) {
             const int j = FR[q];
@@ -788,7 +842,7 @@ int orc_dense_update_factor(int nworld, int nv, int pad, const unsigned char *do
         blocked_forward(pad, B, U, rhs);
       }
       blocked_backward(pad, B, U, rhs);
-      float s0[64] = {0}, s1[64] = {0};
+      float s0[128] = {0}, s1[128] = {0};
       for (int lane = 0; lane < 64; ++lane)
         for (int i = lane; i < nv; i += 64) {
           const float v = rhs[i];

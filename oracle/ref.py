@@ -446,6 +446,29 @@ def sparse_update_factor(plan, state_changes, changes, ids, J, D, state, grad, h
     return hf, uni, search, sdot, decr
 
 
+def sparse_dense_factor(plan, grad, H, hfactor, quad_changed=None, state_changed=None, skip_unchanged=False,
+                        skip_noflip=False, done=None):
+    """Factor step of the upstream iteration on a plan of path "nonfused": lane-by-lane fp32
+    restatement of sparse_hessian.py:639-679 (modes 4 / 5) under the dispatch of :849-894."""
+    grad, H = _f(grad), _f(H)
+    nworld, nv = grad.shape[0], plan.nv
+    tabs = [np.ascontiguousarray(plan.tables[k], np.int32) for k in UPDATE_TABLES + ("SH_GAT",)]
+    ptrs = (ctypes.c_void_p * len(tabs))(*[t.ctypes.data for t in tabs])
+    hf = np.array(hfactor, np.float32, order="C")
+    assert H.shape == (nworld, plan.nv_pad, plan.nv_pad) and hf.shape == H.shape
+    search = np.zeros((nworld, nv), np.float32)
+    sdot, decr = np.zeros(nworld, np.float32), np.zeros(nworld, np.float32)
+    dn = None if done is None else np.ascontiguousarray(done, np.uint8)
+    qc = None if quad_changed is None else _i(quad_changed)
+    sc = None if state_changed is None else _i(state_changed)
+    status = lib().orc_sparse_dense_factor(
+        plan.nv, plan.nv_pad, plan.block, plan.nslots, plan.levels, ptrs, nworld, _p(dn), _p(grad), grad.shape[1], _p(H),
+        _p(qc), _p(sc), int(skip_unchanged), int(skip_noflip), _p(hf), _p(search), _p(sdot), _p(decr),
+    )  # fmt: skip
+    assert status == 0
+    return hf, search, sdot, decr
+
+
 def dense_update_factor(state_changes, changes, ids, J, D, state, grad, H, U, done=None, quad=1):
     J, D, grad = _f(J), _f(D), _f(grad)
     state, ids, changes, state_changes = _i(state), _i(ids), _i(changes), _i(state_changes)
