@@ -648,6 +648,35 @@ int im_newton_jv(const float *J, int njmax, const int32_t *nefc, const float *se
                  int64_t ld_search, const uint8_t *skip_world, float *jv, int64_t ld_jv, int nv,
                  int nworld, void *stream);
 
+/* ---- implicit-fast integrator matrix ---------------------------------------------------------
+ * qH = M - h dF/dv on M's CSR pattern, the matrix that implicit_factor_optimized
+ * (src/instantmimic/utils/mjw_step_optimized.py:4936-4968) hands to _factor_solve_i_dense.
+ * The reference assembles it with upstream kernels that are not part of its tree
+ * (derivative._qderiv_*, forward._implicit_free_body_reset_m, called from deriv_smooth_vel
+ * :3803-3900 and _prepare_implicit_qh :3734-3745); the arithmetic here is MuJoCo's published
+ * mjd_smooth_vel for this integrator.
+ *
+ * im_implicit_qh_base: qH[w, e] = M[w, e] + timestep * dof_damping[elem_dof[e]] where
+ * elem_dof[e] >= 0 (the diagonal element of a damped dof outside every free body), M[w, e]
+ * elsewhere (elem_dof[e] = -1: off-diagonal elements, rows of free bodies, which
+ * _prepare_implicit_qh resets to M).  dof_damping (nv) shared by the worlds with
+ * ld_damping = 0, or one row per world.  The actuator term -h moment' diag(gain) moment, the
+ * tendon-damping term +h J' diag(b) J and the muscle term +h A' diag(s) A are pair sums over
+ * sparse rows: im_muscle_implicit_gather adds each of them on top, with pairs in free-body rows
+ * left out of its tables. */
+int im_implicit_qh_base(const float *M, int64_t ldM, int nM, const int32_t *elem_dof, const float *dof_damping,
+                        int64_t ld_damping, float timestep, float *qH, int64_t ld_qH, int nworld, void *stream);
+
+/* Velocity gain of actuators with affine gain / bias (what derivative._qderiv_actuator_passive_vel
+ * produces for them, mjw_step_optimized.py:3818-3846): gain[w, a] = biasprm[a, 2] (biastype 1)
+ * + gainprm[a, 2] * input[w, a] (gaintype 1), zero when forcelimited[a] and force[w, a] is at or
+ * beyond forcerange[a].  input is ctrl, or the activation for stateful actuators.  forcelimited
+ * and force may be null. */
+int im_actuator_velocity_gain(const int32_t *gaintype, const int32_t *biastype, const float *gainprm,
+                              const float *biasprm, int ld_prm, const uint8_t *forcelimited,
+                              const float *forcerange, const float *input, int64_t ld_input, const float *force,
+                              int64_t ld_force, float *gain, int64_t ld_gain, int nu, int nworld, void *stream);
+
 /* Replaces the step along the search direction at the end of the fused Newton kernel's line
  * search (src/instantmimic/utils/mjw_kernels/newton_stages.py:373-381): for the worlds that
  * are not done, qacc += alpha[w] search and efc_Ma += alpha[w] mv (one fused multiply-add

@@ -613,6 +613,40 @@ int orc_sparse_dense_factor(int nv, int nv_pad, int block, int nslots, int nleve
   return 0;
 }
 
+/* ------------------------------------------------------------------ implicit-fast integrator matrix
+ * qH = M + h damping on the diagonal elements of damped dofs outside free bodies (elem_dof >= 0),
+ * M elsewhere; and the velocity gain of affine actuators.  MuJoCo's published mjd_smooth_vel
+ * (the reference calls upstream kernels that are not in its tree:
+ * src/instantmimic/utils/mjw_step_optimized.py:3803-3900, 3734-3745). */
+int orc_implicit_qh_base(int nworld, int nM, const float *M, int ldM, const int *elem_dof,
+                         const float *damping, int ld_damping, float timestep, float *out, int ldo) {
+  for (int w = 0; w < nworld; ++w)
+    for (int e = 0; e < nM; ++e) {
+      const float v = M[(size_t)w * ldM + e];
+      out[(size_t)w * ldo + e] =
+          elem_dof[e] >= 0 ? fmaf(timestep, damping[(size_t)w * ld_damping + elem_dof[e]], v) : v;
+    }
+  return 0;
+}
+
+int orc_actuator_velocity_gain(int nworld, int nu, const int *gaintype, const int *biastype,
+                               const float *gainprm, const float *biasprm, int ldprm,
+                               const unsigned char *forcelimited, const float *forcerange,
+                               const float *input, const float *force, float *gain) {
+  for (int w = 0; w < nworld; ++w)
+    for (int a = 0; a < nu; ++a) {
+      float v = 0.0f;
+      if (biastype[a] == 1) v = biasprm[a * ldprm + 2];
+      if (gaintype[a] == 1) v = fmaf(gainprm[a * ldprm + 2], input[(size_t)w * nu + a], v);
+      if (forcelimited && forcelimited[a] && force) {
+        const float f = force[(size_t)w * nu + a];
+        if (f <= forcerange[2 * a] || f >= forcerange[2 * a + 1]) v = 0.0f;
+      }
+      gain[(size_t)w * nu + a] = v;
+    }
+  return 0;
+}
+
 /* ------------------------------------------------------------------ blocked dense Cholesky
  * Restatement of the indexed blocked upper Cholesky factor + solve
  * (src/instantmimic/utils/mjw_kernels/indexed_factor.py:15-173; block index layout and

@@ -633,3 +633,32 @@ def newton_converged(alpha, improvement, grad_dot, decrement, tolerance, meanine
     overflow[stop & ~conv] = overflow_bit
     done[stop] = 1
     return niter, done, overflow, int(stop.sum())
+
+
+# ---------------------------------------------------------------- implicit-fast integrator matrix
+# Pinned by tests/test_implicit_qh.py against the dense fp64 statement
+# qH = M + h diag(b) - h A' diag(g) A + h Jt' diag(bt) Jt on M's pattern with free-body rows reset to M.
+# Upstream's kernels are absent from the reference tree: bit-level parity with them is UNPINNED.
+
+
+def implicit_qh_base(M, elem_dof, damping, timestep):
+    M, damping = _f(M), _f(damping)
+    elem_dof = _i(elem_dof)
+    nworld, nM = M.shape
+    out = np.zeros_like(M)
+    ld = 0 if damping.ndim == 1 else damping.shape[1]
+    assert lib().orc_implicit_qh_base(nworld, nM, _p(M), nM, _p(elem_dof), _p(damping), ld, ctypes.c_float(timestep), _p(out), nM) == 0
+    return out
+
+
+def actuator_velocity_gain(gaintype, biastype, gainprm, biasprm, inp, forcelimited=None, forcerange=None, force=None):
+    gainprm, biasprm, inp = _f(gainprm), _f(biasprm), _f(inp)
+    gaintype, biastype = _i(gaintype), _i(biastype)
+    nworld, nu = inp.shape
+    out = np.zeros_like(inp)
+    fl = None if forcelimited is None else np.ascontiguousarray(forcelimited, np.uint8)
+    fr = None if forcerange is None else _f(forcerange)
+    fo = None if force is None else _f(force)
+    assert lib().orc_actuator_velocity_gain(nworld, nu, _p(gaintype), _p(biastype), _p(gainprm), _p(biasprm), gainprm.shape[1],
+                                            _p(fl), _p(fr), _p(inp), _p(fo), _p(out)) == 0  # fmt: skip
+    return out
