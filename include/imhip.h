@@ -688,6 +688,44 @@ int im_newton_advance(const float *alpha, const float *search, int64_t ld_search
                       int64_t ld_Ma, float *Jaref, int64_t ld_Jaref, int nv, int njmax, int nworld,
                       void *stream);
 
+/* Replaces the scalar search of the fused Newton kernel's line-search stage
+ * (src/instantmimic/utils/mjw_kernels/newton_stages.py:179-372) for the worlds that are not done:
+ * the step length alpha[w] along search that minimises the constraint-solver cost, the cost
+ * decrease improvement[w], and ls_exhausted[w] = |alpha| below the noise floor of the line's
+ * slope.  The stage's flow is the reference's: Gauss term and equality rows as one quadratic,
+ * Newton step from alpha 0, then up to ls_iterations rounds of three candidates (Newton steps from
+ * the bracket's ends and its midpoint) with its acceptance tests; sums over 32 lanes by a
+ * shuffle-down tree.  The per-row cost model is upstream's (solver._compute_efc_eval_pt_*_pyramidal,
+ * not in the reference tree), restated from MuJoCo's primal line search: rows [0, ne) equality,
+ * [ne, ne + nf) friction loss, the rest one-sided.  jv and mv are the products J search and
+ * M search (im_newton_jv, im_mul_m_sparse).  overflow[w] |= overflow_bit when the rounds run out;
+ * tolerance arrays are indexed by w modulo their length.  ne, nf, nefc, done, overflow,
+ * efc_frictionloss (with nf) may be null. */
+int im_newton_linesearch(const float *opt_tolerance, int ntolerance, const float *opt_ls_tolerance,
+                         int nls_tolerance, const float *stat_meaninertia, int nmeaninertia, const int32_t *ne,
+                         const int32_t *nf, const int32_t *nefc, int njmax, const float *qfrc_smooth,
+                         int64_t ld_smooth, const float *efc_D, int64_t ld_D, const float *efc_frictionloss,
+                         int64_t ld_frictionloss, const float *Jaref, int64_t ld_Jaref, const float *search,
+                         int64_t ld_search, const float *search_dot, const float *mv, int64_t ld_mv,
+                         const float *jv, int64_t ld_jv, const float *efc_Ma, int64_t ld_Ma, const uint8_t *done,
+                         int ls_iterations, int overflow_bit, float *alpha, float *improvement,
+                         uint8_t *ls_exhausted, int32_t *overflow, int nv, int nworld, void *stream);
+
+/* Replaces the re-evaluation of the constraints that closes the line-search stage
+ * (newton_stages.py:385-444, upstream's _eval_constraint for pyramidal cones): from the Jaref
+ * that im_newton_advance has moved, efc_force and efc_state of every row below nefc[w] (state 0
+ * satisfied, 1 quadratic, 2 / 3 linear negative / positive for friction loss), in place; the rows
+ * whose being quadratic flipped, ascending, in quad_changed_ids[w, :] with their count; and
+ * state_changed_count[w] = the rows whose state changed, plus one when ls_exhausted[w].  Both
+ * counts are zeroed for done worlds, which are otherwise left alone. */
+int im_newton_eval_constraints(const float *Jaref, int64_t ld_Jaref, const float *efc_D, int64_t ld_D,
+                               const float *efc_frictionloss, int64_t ld_frictionloss, const int32_t *ne,
+                               const int32_t *nf, const int32_t *nefc, int njmax, const uint8_t *done,
+                               const uint8_t *ls_exhausted, float *efc_force, int64_t ld_force,
+                               int32_t *efc_state, int64_t ld_state, int32_t *quad_changed_ids, int ld_ids,
+                               int32_t *quad_changed_count, int32_t *state_changed_count, int nworld,
+                               void *stream);
+
 /* Replaces the listing of the changed rows that follows it (newton_stages.py:403-426): among
  * the rows r < min(njmax, nefc[w]), those with (old_state == quad) != (new_state == quad) are
  * written to quad_changed_ids[w, :] in ascending order and counted in quad_changed_count[w]

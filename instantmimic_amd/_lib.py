@@ -146,6 +146,15 @@ SIGNATURES = {
     "im_sparse_dense_factor": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i, _vp, _vp, _i, _vp]),
     "im_implicit_qh_base": (_i, [_vp, _i64, _i, _vp, _vp, _i64, C.c_float, _vp, _i64, _i, _vp]),
     "im_actuator_velocity_gain": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _vp]),
+    "im_newton_linesearch": (
+        _i,
+        [_vp, _i, _vp, _i, _vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64,
+         _vp, _i64, _vp, _i64, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _vp],
+    ),  # fmt: skip
+    "im_newton_eval_constraints": (
+        _i,
+        [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i, _vp, _vp, _i, _vp],
+    ),
     "im_dense_update_factor": (
         _i,
         [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],

@@ -360,3 +360,130 @@ def qfrc_constraint_from_grad(nefc, qfrc_smooth, efc_Ma, grad, grad_scale, qfrc_
             int(nv), int(nworld), int(torch.cuda.current_stream(grad.device).cuda_stream),
         )  # fmt: skip
     _lib.check(status, "im_qfrc_constraint_from_grad")
+
+
+def linesearch(opt_tolerance, opt_ls_tolerance, stat_meaninertia, ne, nf, nefc, qfrc_smooth, efc_D, efc_frictionloss, Jaref,
+               search, search_dot, mv, jv_in, efc_Ma, done, alpha, improvement, ls_exhausted, *, ls_iterations: int,
+               overflow=None, overflow_bit: int = 0) -> None:  # fmt: skip
+    """The scalar search of the line-search stage (newton_stages.py:179-372): ``alpha``,
+    ``improvement`` and ``ls_exhausted`` per world from ``Jaref``, ``jv = J search``,
+    ``mv = M search`` and the rows' weights.  ``ne`` / ``nf`` / ``nefc`` int32 per world or None."""
+    import torch
+
+    nworld, nv = search.shape
+    njmax = efc_D.shape[1]
+    for t, width, name in ((qfrc_smooth, nv, "qfrc_smooth"), (search, nv, "search"), (mv, nv, "mv"), (efc_Ma, nv, "efc_Ma"),
+                           (efc_D, njmax, "efc_D"), (Jaref, njmax, "Jaref"), (jv_in, njmax, "jv")):  # fmt: skip
+        _rows(t, nworld, width, torch.float32, name)
+    if efc_frictionloss is not None:
+        _rows(efc_frictionloss, nworld, njmax, torch.float32, "efc_frictionloss")
+    for t, name in ((search_dot, "search_dot"), (alpha, "alpha"), (improvement, "improvement")):
+        _per_world(t, nworld, (torch.float32,), name)
+    _per_world(ls_exhausted, nworld, (torch.bool, torch.uint8), "ls_exhausted")
+    for t, name in ((ne, "ne"), (nf, "nf"), (nefc, "nefc"), (overflow, "overflow")):
+        if t is not None:
+            _per_world(t, nworld, (torch.int32,), name)
+    if done is not None:
+        _per_world(done, nworld, (torch.bool, torch.uint8), "done")
+    for t in (opt_tolerance, opt_ls_tolerance, stat_meaninertia):
+        if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous() or t.numel() < 1:
+            raise TypeError("tolerances and meaninertia must be contiguous float32 CUDA tensors")
+    ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
+    with torch.cuda.device(search.device):
+        status = _lib.lib().im_newton_linesearch(
+            opt_tolerance.data_ptr(), int(opt_tolerance.numel()), opt_ls_tolerance.data_ptr(), int(opt_ls_tolerance.numel()),
+            stat_meaninertia.data_ptr(), int(stat_meaninertia.numel()), ptr(ne), ptr(nf), ptr(nefc), int(njmax),
+            qfrc_smooth.data_ptr(), qfrc_smooth.stride(0), efc_D.data_ptr(), efc_D.stride(0), ptr(efc_frictionloss),
+            0 if efc_frictionloss is None else efc_frictionloss.stride(0), Jaref.data_ptr(), Jaref.stride(0),
+            search.data_ptr(), search.stride(0), search_dot.data_ptr(), mv.data_ptr(), mv.stride(0), jv_in.data_ptr(),
+            jv_in.stride(0), efc_Ma.data_ptr(), efc_Ma.stride(0), ptr(done), int(ls_iterations), int(overflow_bit),
+            alpha.data_ptr(), improvement.data_ptr(), ls_exhausted.data_ptr(), ptr(overflow), int(nv), int(nworld),
+            int(torch.cuda.current_stream(search.device).cuda_stream),
+        )  # fmt: skip
+    _lib.check(status, "im_newton_linesearch")
+
+
+def eval_constraints(Jaref, efc_D, efc_frictionloss, ne, nf, nefc, done, ls_exhausted, efc_force, efc_state, quad_changed_ids,
+                     quad_changed_count, state_changed_count) -> None:  # fmt: skip
+    """Force and state of every row from the advanced ``Jaref`` (in place), the ascending list of
+    the rows whose being QUADRATIC flipped and the two counts (newton_stages.py:385-444)."""
+    import torch
+
+    nworld, njmax = efc_D.shape
+    for t, name in ((Jaref, "Jaref"), (efc_D, "efc_D"), (efc_force, "efc_force")):
+        _rows(t, nworld, njmax, torch.float32, name)
+    if efc_frictionloss is not None:
+        _rows(efc_frictionloss, nworld, njmax, torch.float32, "efc_frictionloss")
+    _rows(efc_state, nworld, njmax, torch.int32, "efc_state")
+    if quad_changed_ids.dtype != torch.int32 or not quad_changed_ids.is_contiguous() or quad_changed_ids.dim() != 2 or quad_changed_ids.shape[0] != nworld:
+        raise TypeError("quad_changed_ids must be a contiguous int32 CUDA tensor (nworld, width)")
+    for t, name in ((ne, "ne"), (nf, "nf"), (nefc, "nefc")):
+        if t is not None:
+            _per_world(t, nworld, (torch.int32,), name)
+    _per_world(quad_changed_count, nworld, (torch.int32,), "quad_changed_count")
+    _per_world(state_changed_count, nworld, (torch.int32,), "state_changed_count")
+    for t, name in ((done, "done"), (ls_exhausted, "ls_exhausted")):
+        if t is not None:
+            _per_world(t, nworld, (torch.bool, torch.uint8), name)
+    ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
+    with torch.cuda.device(efc_D.device):
+        status = _lib.lib().im_newton_eval_constraints(
+            Jaref.data_ptr(), Jaref.stride(0), efc_D.data_ptr(), efc_D.stride(0), ptr(efc_frictionloss),
+            0 if efc_frictionloss is None else efc_frictionloss.stride(0), ptr(ne), ptr(nf), ptr(nefc), int(njmax),
+            ptr(done), ptr(ls_exhausted), efc_force.data_ptr(), efc_force.stride(0), efc_state.data_ptr(),
+            efc_state.stride(0), quad_changed_ids.data_ptr(), int(quad_changed_ids.shape[1]), quad_changed_count.data_ptr(),
+            state_changed_count.data_ptr(), int(nworld), int(torch.cuda.current_stream(efc_D.device).cuda_stream),
+        )  # fmt: skip
+    _lib.check(status, "im_newton_eval_constraints")
+
+
+OVERFLOW_LS_ITERATIONS = 4  # bits of d.overflow: the caller's OverflowType where it differs
+OVERFLOW_ITERATIONS = 8
+
+
+def iteration(m, d, ctx, nsolving=None, *, stage=None) -> None:
+    """One iteration of the fused Newton loop for every world that is not done, as seven launches in
+    the reference kernel's order (newton_fusion.py:151-296): M search, J search, the scalar search,
+    the step, the constraints' new forces and states, the gradient, the factor stage, the
+    convergence test."""
+    from . import newton_stages
+
+    nworld, nv = int(d.nworld), int(m.nv)
+    if stage is None:
+        stage = newton_stages.factor_factory(nv, int(m.nv_pad), getattr(ctx, "sparse_hessian_plan", None))
+    mul_m(d.M, ctx.search, ctx.mv, m.M_mulm_rowadr, m.M_mulm_col, m.M_mulm_madr, skip_world=ctx.search_unchanged)
+    jv(d.efc.J, ctx.search, ctx.jv, nefc=d.nefc, skip_world=ctx.search_unchanged)
+    linesearch(m.opt.tolerance, m.opt.ls_tolerance, m.stat.meaninertia, d.ne, d.nf, d.nefc, d.qfrc_smooth, d.efc.D,
+               d.efc.frictionloss, ctx.Jaref, ctx.search, ctx.search_dot, ctx.mv, ctx.jv, d.efc.Ma, ctx.done, ctx.alpha,
+               ctx.improvement, ctx.ls_exhausted, ls_iterations=int(m.opt.ls_iterations), overflow=d.overflow,
+               overflow_bit=OVERFLOW_LS_ITERATIONS)  # fmt: skip
+    advance(ctx.alpha, ctx.search, ctx.mv, ctx.jv, d.qacc, d.efc.Ma, ctx.Jaref, nefc=d.nefc, done=ctx.done)
+    eval_constraints(ctx.Jaref, d.efc.D, d.efc.frictionloss, d.ne, d.nf, d.nefc, ctx.done, ctx.ls_exhausted, d.efc.force,
+                     d.efc.state, ctx.quad_changed_ids, ctx.quad_changed_count, ctx.state_changed_count)  # fmt: skip
+    gradient(d.nefc, d.efc.J, d.efc.force, d.qfrc_smooth, d.efc.Ma, ctx.state_changed_count, ctx.alpha, ctx.done,
+             d.qfrc_constraint, ctx.grad[:, :nv], ctx.grad_dot, ctx.newton_decrement, ctx.grad_scale, ctx.search_unchanged,
+             block=newton_block_dim(m))  # fmt: skip
+    sparse = getattr(ctx, "sparse_hessian_plan", None) is not None
+    stage(d.efc.J, d.efc.D, d.efc.state, ctx.quad_changed_ids, ctx.quad_changed_count, ctx.state_changed_count, ctx.done,
+          ctx.grad, None if sparse else ctx.h, ctx.hfactor, ctx.search, ctx.search_dot, ctx.newton_decrement, ctx.newton_dof_union)  # fmt: skip
+    converged(ctx.alpha, ctx.improvement, ctx.grad_dot, ctx.newton_decrement, m.opt.tolerance, m.stat.meaninertia, nv,
+              int(m.opt.iterations), d.solver_niter, ctx.done, overflow=d.overflow, overflow_bit=OVERFLOW_ITERATIONS,
+              nsolving=nsolving)  # fmt: skip
+
+
+def run(m, d, ctx, nsolving, *, check_every: int = 4) -> int:
+    """The fused Newton solve with the reference's signature (newton_fusion.py:330-409): iterates
+    until every world is done or ``m.opt.iterations`` is reached.  The reference keeps a world in
+    one resident block for the whole loop; here an iteration is seven launches over all worlds
+    (finished worlds drop out of each through ``ctx.done``), and the host reads ``nsolving`` every
+    ``check_every`` iterations to stop early.  Returns the number of iterations launched."""
+    from . import newton_stages
+
+    stage = newton_stages.factor_factory(int(m.nv), int(m.nv_pad), getattr(ctx, "sparse_hessian_plan", None))
+    launched = 0
+    for it in range(int(m.opt.iterations)):
+        iteration(m, d, ctx, nsolving, stage=stage)
+        launched += 1
+        if check_every > 0 and (it + 1) % check_every == 0 and int(nsolving.item()) <= 0:
+            break
+    return launched

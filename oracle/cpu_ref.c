@@ -613,6 +613,225 @@ int orc_sparse_dense_factor(int nv, int nv_pad, int block, int nslots, int nleve
   return 0;
 }
 
+/* ------------------------------------------------------------------ Newton line search
+ * Lane-by-lane restatement of the reference's line-search stage
+ * (src/instantmimic/utils/mjw_kernels/newton_stages.py:79-444): 32 lanes stride the dofs and the
+ * rows, sums go through a shuffle-down tree whose lane 0 is broadcast.  The per-row cost model
+ * (solver._compute_efc_eval_pt_*_pyramidal, _eval_pt, _in_bracket, _eval_constraint, safe_div,
+ * _ALPHA_NOISE_EPS) is upstream mujoco_warp code absent from the reference tree: it is restated
+ * from MuJoCo's published primal line search, so bit-level parity with upstream is UNPINNED; the
+ * tests pin it to the exact minimiser of the line's cost in fp64. */
+typedef struct {
+  float c, g, h;
+} pt3;
+static pt3 pt_add(pt3 a, pt3 b) { pt3 r = {a.c + b.c, a.g + b.g, a.h + b.h}; return r; }
+static float ls_safe_div(float x, float y) { return x / (y != 0.0f ? y : 1.0e-15f); }
+static pt3 ls_eval_pt(pt3 q, float a) {
+  pt3 r = {a * a * q.h + a * q.g + q.c, 2.0f * a * q.h + q.g, 2.0f * q.h};
+  return r;
+}
+static int ls_in_bracket(pt3 x, pt3 y) { return (x.g < y.g && y.g < 0.0f) || (x.g > y.g && y.g > 0.0f); }
+static pt3 ls_row_quad(int friction, float D, float f, float jaref, float jv, float x) {
+  pt3 quad = {0.5f * jaref * jaref * D, jv * jaref * D, 0.5f * jv * jv * D};
+  pt3 zero = {0.0f, 0.0f, 0.0f};
+  if (friction) {
+    const float rf = ls_safe_div(f, D);
+    if (x <= -rf) { pt3 r = {f * (-0.5f * rf - jaref), -f * jv, 0.0f}; return r; }
+    if (x >= rf) { pt3 r = {f * (-0.5f * rf + jaref), f * jv, 0.0f}; return r; }
+    return quad;
+  }
+  return x < 0.0f ? quad : zero;
+}
+static pt3 ls_row_point(int friction, float D, float f, float jaref, float jv, float alpha) {
+  pt3 p = ls_eval_pt(ls_row_quad(friction, D, f, jaref, jv, jaref + alpha * jv), alpha);
+  p.c = p.c - ls_row_quad(friction, D, f, jaref, jv, jaref).c;
+  return p;
+}
+static float ls_tree(float *a) {
+  for (int off = 16; off > 0; off >>= 1)
+    for (int i = 0; i < off; ++i) a[i] = a[i] + a[i + off];
+  return a[0] + 0.0f;
+}
+typedef struct {
+  int ne, nf, nefc;
+  const float *D, *fl, *Jaref, *jv;
+} ls_rows;
+/* sum over the rows [ne, nefc) of the row points at alpha (zero != 0: the absolute point at alpha 0) */
+static pt3 ls_rows_at(const ls_rows *R, float alpha, int zero) {
+  float c[32] = {0}, g[32] = {0}, h[32] = {0};
+  for (int lane = 0; lane < 32; ++lane)
+    for (int r = R->ne + lane; r < R->nefc; r += 32) {
+      const int fr = r < R->ne + R->nf;
+      const float f = R->fl ? R->fl[r] : 0.0f;
+      pt3 p;
+      if (zero) {
+        const pt3 q = ls_row_quad(fr, R->D[r], f, R->Jaref[r], R->jv[r], R->Jaref[r]);
+        p.c = q.c, p.g = q.g, p.h = 2.0f * q.h;
+      } else {
+        p = ls_row_point(fr, R->D[r], f, R->Jaref[r], R->jv[r], alpha);
+      }
+      c[lane] = c[lane] + p.c, g[lane] = g[lane] + p.g, h[lane] = h[lane] + p.h;
+    }
+  pt3 out = {ls_tree(c), ls_tree(g), ls_tree(h)};
+  return out;
+}
+
+int orc_newton_linesearch(int nworld, int nv, int njmax, const float *tolerance, int ntol,
+                          const float *ls_tolerance, int nls, const float *meaninertia, int nmi,
+                          const int *ne_, const int *nf_, const int *nefc_, const float *smooth,
+                          const float *D, const float *frictionloss, const float *Jaref,
+                          const float *search, const float *search_dot, const float *mv,
+                          const float *jv, const float *Ma, const unsigned char *done,
+                          int ls_iterations, int overflow_bit, float *alpha_out, float *improvement_out,
+                          unsigned char *exhausted, int *overflow) {
+  const float noise = 0x1p-20f;
+  for (int w = 0; w < nworld; ++w) {
+    if (done && done[w]) continue;
+    ls_rows R = {ne_ ? ne_[w] : 0, nf_ ? nf_[w] : 0, 0, D + (size_t)w * njmax,
+                 frictionloss ? frictionloss + (size_t)w * njmax : NULL, Jaref + (size_t)w * njmax,
+                 jv + (size_t)w * njmax};
+    R.nefc = nefc_ ? nefc_[w] : njmax;
+    if (R.nefc > njmax) R.nefc = njmax;
+    const float snorm = sqrtf(search_dot[w]);
+    const float scale = meaninertia[w % nmi] * (float)nv;
+    const float gtol = fmaxf(tolerance[w % ntol] * ls_tolerance[w % nls] * snorm * scale, 1.0e-6f);
+    float a1[32] = {0}, a2[32] = {0};
+    for (int lane = 0; lane < 32; ++lane) {
+      for (int dof = lane; dof < nv; dof += 32) {
+        const float sv = search[(size_t)w * nv + dof];
+        a1[lane] = a1[lane] + sv * (Ma[(size_t)w * nv + dof] - smooth[(size_t)w * nv + dof]);
+        a2[lane] = a2[lane] + 0.5f * sv * mv[(size_t)w * nv + dof];
+      }
+      for (int r = lane; r < R.ne; r += 32) {
+        const float jvD = R.jv[r] * R.D[r];
+        a1[lane] = a1[lane] + jvD * R.Jaref[r];
+        a2[lane] = a2[lane] + 0.5f * R.jv[r] * jvD;
+      }
+    }
+    pt3 gauss = {0.0f, 0.0f, 0.0f};
+    gauss.g = ls_tree(a1);
+    gauss.h = ls_tree(a2);
+    const pt3 rows0 = ls_rows_at(&R, 0.0f, 1);
+    const pt3 p0 = {gauss.c + rows0.c, gauss.g + rows0.g, 2.0f * gauss.h + rows0.h};
+    const pt3 p0_delta = {0.0f, p0.g, p0.h};
+    const float q1_abs = sqrtf(2.0f * fmaxf(rows0.c, 0.0f) * fmaxf(rows0.h, 0.0f)) + fabsf(gauss.g);
+    const float gtol_accept = fmaxf(gtol, noise * q1_abs);
+    const float noise_floor = noise * fmaxf(1.0f, ls_safe_div(q1_abs, p0.h));
+    float alpha = 0.0f, improvement = 0.0f;
+    int converged = fabsf(p0.g) < noise * q1_abs;
+    const float lo_alpha_in = -ls_safe_div(p0.g, p0.h);
+    pt3 lo_in = {0.0f, 0.0f, 0.0f};
+    if (!converged) {
+      lo_in = pt_add(ls_eval_pt(gauss, lo_alpha_in), ls_rows_at(&R, lo_alpha_in, 0));
+      if (fabsf(lo_in.g) < gtol_accept && lo_in.c < 0.0f) {
+        converged = 1;
+        alpha = lo_alpha_in;
+        improvement = -lo_in.c;
+      }
+    }
+    if (!converged) {
+      const int lo_less = lo_in.g < p0.g;
+      pt3 lo = lo_less ? lo_in : p0_delta, hi = lo_less ? p0_delta : lo_in;
+      float lo_alpha = lo_less ? lo_alpha_in : 0.0f, hi_alpha = lo_less ? 0.0f : lo_alpha_in;
+      for (int it = 0; it < ls_iterations; ++it) {
+        const float lo_next_alpha = lo_alpha - ls_safe_div(lo.g, lo.h);
+        const float hi_next_alpha = hi_alpha - ls_safe_div(hi.g, hi.h);
+        const float mid_alpha = 0.5f * (lo_alpha + hi_alpha);
+        const pt3 lo_next = pt_add(ls_eval_pt(gauss, lo_next_alpha), ls_rows_at(&R, lo_next_alpha, 0));
+        const pt3 hi_next = pt_add(ls_eval_pt(gauss, hi_next_alpha), ls_rows_at(&R, hi_next_alpha, 0));
+        const pt3 mid = pt_add(ls_eval_pt(gauss, mid_alpha), ls_rows_at(&R, mid_alpha, 0));
+        const int conv_lo = fabsf(lo_next.g) < gtol_accept && lo_next.c < 0.0f;
+        const int conv_hi = fabsf(hi_next.g) < gtol_accept && hi_next.c < 0.0f;
+        const int conv_mid = fabsf(mid.g) < gtol_accept && mid.c < 0.0f;
+        const int conv = conv_lo || conv_hi || conv_mid;
+        int swap_lo = 0, swap_hi = 0;
+        if (conv) {
+          pt3 best = {1.0e10f, 0.0f, 0.0f};
+          float best_alpha = 0.0f;
+          if (conv_lo && lo_next.c < best.c) best = lo_next, best_alpha = lo_next_alpha;
+          if (conv_hi && hi_next.c < best.c) best = hi_next, best_alpha = hi_next_alpha;
+          if (conv_mid && mid.c < best.c) best = mid, best_alpha = mid_alpha;
+          lo = hi = best;
+          lo_alpha = hi_alpha = best_alpha;
+        } else {
+          const int s1 = ls_in_bracket(lo, lo_next);
+          if (s1) lo = lo_next, lo_alpha = lo_next_alpha;
+          const int s2 = ls_in_bracket(lo, mid);
+          if (s2) lo = mid, lo_alpha = mid_alpha;
+          const int s3 = ls_in_bracket(lo, hi_next);
+          if (s3) lo = hi_next, lo_alpha = hi_next_alpha;
+          swap_lo = s1 || s2 || s3;
+          const int t1 = ls_in_bracket(hi, hi_next) || (hi.g < 0.0f && hi_next.g > 0.0f);
+          if (t1) hi = hi_next, hi_alpha = hi_next_alpha;
+          const int t2 = ls_in_bracket(hi, mid);
+          if (t2) hi = mid, hi_alpha = mid_alpha;
+          const int t3 = ls_in_bracket(hi, lo_next);
+          if (t3) hi = lo_next, hi_alpha = lo_next_alpha;
+          swap_hi = t1 || t2 || t3;
+        }
+        const int ls_done = conv || (!swap_lo && !swap_hi) || (lo.c < 0.0f && lo.g < 0.0f && lo.g > -gtol) ||
+                            (hi.c < 0.0f && hi.g > 0.0f && hi.g < gtol);
+        if (lo.c < 0.0f || hi.c < 0.0f) {
+          const int lo_better = lo.c < hi.c;
+          alpha = lo_better ? lo_alpha : hi_alpha;
+          improvement = -(lo_better ? lo.c : hi.c);
+        }
+        if (ls_done) {
+          converged = 1;
+          break;
+        }
+      }
+    }
+    alpha_out[w] = alpha;
+    improvement_out[w] = improvement;
+    exhausted[w] = fabsf(alpha) < noise_floor;
+    if (!converged && overflow) overflow[w] |= overflow_bit;
+  }
+  return 0;
+}
+
+/* force and state of every row from the new Jaref, ascending list of the rows whose being
+ * QUADRATIC flipped, counts (newton_stages.py:385-444; upstream's _eval_constraint restated) */
+int orc_newton_eval_constraints(int nworld, int njmax, const float *Jaref, const float *D,
+                                const float *frictionloss, const int *ne_, const int *nf_,
+                                const int *nefc_, const unsigned char *done,
+                                const unsigned char *exhausted, float *force, int *state, int *ids,
+                                int ld_ids, int *quad_count, int *state_count) {
+  for (int w = 0; w < nworld; ++w) {
+    quad_count[w] = 0;
+    state_count[w] = 0;
+    if (done && done[w]) continue;
+    const int ne = ne_ ? ne_[w] : 0, nf = nf_ ? nf_[w] : 0;
+    int nefc = nefc_ ? nefc_[w] : njmax;
+    if (nefc > njmax) nefc = njmax;
+    int nq = 0, ns = 0;
+    for (int r = 0; r < nefc; ++r) {
+      const size_t k = (size_t)w * njmax + r;
+      const float x = Jaref[k], d = D[k];
+      float f = -d * x;
+      int s = 1;
+      if (r >= ne && r < ne + nf) {
+        const float fr = frictionloss[k], rf = ls_safe_div(fr, d);
+        if (x <= -rf) f = fr, s = 2;
+        else if (x >= rf) f = -fr, s = 3;
+      } else if (r >= ne && x >= 0.0f) {
+        f = 0.0f, s = 0;
+      }
+      const int old = state[k];
+      force[k] = f;
+      state[k] = s;
+      if ((old == 1) != (s == 1)) {
+        if (nq < ld_ids) ids[(size_t)w * ld_ids + nq] = r;
+        ++nq;
+      }
+      ns += old != s;
+    }
+    quad_count[w] = nq;
+    state_count[w] = ns + (exhausted && exhausted[w] ? 1 : 0);
+  }
+  return 0;
+}
+
 /* ------------------------------------------------------------------ implicit-fast integrator matrix
  * qH = M + h damping on the diagonal elements of damped dofs outside free bodies (elem_dof >= 0),
  * M elsewhere; and the velocity gain of affine actuators.  MuJoCo's published mjd_smooth_vel

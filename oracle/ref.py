@@ -635,6 +635,52 @@ def newton_converged(alpha, improvement, grad_dot, decrement, tolerance, meanine
     return niter, done, overflow, int(stop.sum())
 
 
+# The scalar line search and the constraint re-evaluation of the line-search stage
+# (newton_stages.py:179-444).  The stage's flow is the reference's; the per-row cost model is
+# upstream's and restated from MuJoCo's primal line search: parity with upstream's bits is
+# UNPINNED.  Pinned by tests/test_newton_linesearch.py: against the exact minimiser of the line's
+# cost in fp64 (slope at alpha within the stage's tolerance, cost decrease equal to the reported
+# improvement), by the closed form without one-sided rows (alpha = -p'(0) / p''(0)), and the
+# states / forces by brute force from their definitions.
+def newton_linesearch(tolerance, ls_tolerance, meaninertia, ne, nf, nefc, smooth, D, frictionloss, Jaref, search, search_dot,
+                      mv, jv, Ma, done=None, ls_iterations=50, overflow_bit=4):  # fmt: skip
+    """Returns (alpha, improvement, ls_exhausted, overflow)."""
+    smooth, D, Jaref, search, search_dot, mv, jv, Ma = (_f(a) for a in (smooth, D, Jaref, search, search_dot, mv, jv, Ma))
+    nworld, nv = search.shape
+    njmax = D.shape[1]
+    alpha, imp = np.zeros(nworld, np.float32), np.zeros(nworld, np.float32)
+    ex, ov = np.zeros(nworld, np.uint8), np.zeros(nworld, np.int32)
+    tol, lst, mi = _f(tolerance), _f(ls_tolerance), _f(meaninertia)
+    fl = None if frictionloss is None else _f(frictionloss)
+    dn = None if done is None else np.ascontiguousarray(done, np.uint8)
+    opt = lambda a: None if a is None else _p(_i(a))  # noqa: E731
+    status = lib().orc_newton_linesearch(
+        nworld, nv, njmax, _p(tol), len(tol), _p(lst), len(lst), _p(mi), len(mi), opt(ne), opt(nf), opt(nefc), _p(smooth), _p(D),
+        _p(fl), _p(Jaref), _p(search), _p(search_dot), _p(mv), _p(jv), _p(Ma), _p(dn), int(ls_iterations), int(overflow_bit),
+        _p(alpha), _p(imp), _p(ex), _p(ov),
+    )  # fmt: skip
+    assert status == 0
+    return alpha, imp, ex, ov
+
+
+def newton_eval_constraints(Jaref, D, frictionloss, ne, nf, nefc, state, done=None, exhausted=None):
+    """Returns (force, new state, ids, quad_changed_count, state_changed_count)."""
+    Jaref, D = _f(Jaref), _f(D)
+    nworld, njmax = D.shape
+    force = np.zeros((nworld, njmax), np.float32)
+    st = np.array(state, np.int32, order="C")
+    ids = np.zeros((nworld, njmax), np.int32)
+    qc, sc = np.zeros(nworld, np.int32), np.zeros(nworld, np.int32)
+    fl = None if frictionloss is None else _f(frictionloss)
+    dn = None if done is None else np.ascontiguousarray(done, np.uint8)
+    ex = None if exhausted is None else np.ascontiguousarray(exhausted, np.uint8)
+    opt = lambda a: None if a is None else _p(_i(a))  # noqa: E731
+    status = lib().orc_newton_eval_constraints(nworld, njmax, _p(Jaref), _p(D), _p(fl), opt(ne), opt(nf), opt(nefc), _p(dn), _p(ex),
+                                               _p(force), _p(st), _p(ids), njmax, _p(qc), _p(sc))  # fmt: skip
+    assert status == 0
+    return force, st, ids, qc, sc
+
+
 # ---------------------------------------------------------------- implicit-fast integrator matrix
 # Pinned by tests/test_implicit_qh.py against the dense fp64 statement
 # qH = M + h diag(b) - h A' diag(g) A + h Jt' diag(bt) Jt on M's pattern with free-body rows reset to M.

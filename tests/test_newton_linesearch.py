@@ -1,0 +1,343 @@
+"""The scalar line search, the constraints' re-evaluation and the Newton loop built from the
+library's pieces (reference: src/instantmimic/utils/mjw_kernels/newton_stages.py:179-444,
+newton_fusion.py:57-298, 330-409).  The per-row cost model is upstream mujoco_warp code that the
+reference tree does not hold; it is restated from MuJoCo's primal line search, so parity with
+upstream's bits is unpinned.  Pinned here: the step against the exact minimiser of the line's cost
+in fp64, the closed form without one-sided rows, states and forces by their definitions, a
+monotone cost, and the converged solution against an fp64 Newton solve."""
+
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+
+from instantmimic_amd import synth
+from oracle import ref as R
+
+NOISE = 2.0**-20
+
+
+def _line_case(nworld, nv, njmax, seed, one_sided=True):
+    rng = np.random.default_rng(seed)
+    f = lambda *s: rng.normal(size=s).astype(np.float32)  # noqa: E731
+    ne = rng.integers(0, 4, nworld).astype(np.int32)
+    nf = rng.integers(0, 5, nworld).astype(np.int32)
+    nefc = rng.integers(8, njmax + 1, nworld).astype(np.int32)
+    if not one_sided:
+        nf[:] = 0
+        nefc = ne.copy()
+    c = SimpleNamespace(ne=ne, nf=nf, nefc=nefc, D=(10.0 ** rng.uniform(-1, 3, (nworld, njmax))).astype(np.float32),
+                        frictionloss=rng.uniform(0.05, 2.0, (nworld, njmax)).astype(np.float32), Jaref=f(nworld, njmax),
+                        jv=f(nworld, njmax), search=f(nworld, nv), smooth=f(nworld, nv), Ma=f(nworld, nv))  # fmt: skip
+    # mv = M search with M positive definite: search . mv > 0
+    A = rng.normal(size=(nworld, nv, nv))
+    Mm = np.einsum("wik,wjk->wij", A, A) + 0.1 * np.eye(nv)
+    c.mv = np.einsum("wij,wj->wi", Mm, c.search).astype(np.float32)
+    # a descent direction: the slope at alpha 0 is negative
+    c.search_dot = (c.search.astype(np.float64) ** 2).sum(1).astype(np.float32)
+    c.tol, c.ls_tol, c.mi = np.array([1e-8], np.float32), np.array([0.01], np.float32), np.array([1.0], np.float32)
+    return c
+
+
+def _row_cost64(c, w, x):
+    """Cost of the rows [ne, nefc) of world w at positions x (fp64), and its slope in x."""
+    ne, nf, nefc = int(c.ne[w]), int(c.nf[w]), int(c.nefc[w])
+    D, f = c.D[w].astype(np.float64), c.frictionloss[w].astype(np.float64)
+    cost, slope = np.zeros_like(x), np.zeros_like(x)
+    r = np.arange(len(x))
+    fr = (r >= ne) & (r < ne + nf)
+    one = (r >= ne + nf) & (r < nefc)
+    rf = f / D
+    quad = 0.5 * D * x * x
+    cost[fr] = np.where(np.abs(x) < rf, quad, f * (np.abs(x) - 0.5 * rf))[fr]
+    slope[fr] = np.where(np.abs(x) < rf, D * x, f * np.sign(x))[fr]
+    cost[one] = np.where(x < 0, quad, 0.0)[one]
+    slope[one] = np.where(x < 0, D * x, 0.0)[one]
+    return cost, slope
+
+
+def _line64(c, w, alpha):
+    """Cost along the line relative to alpha 0 and its derivative, fp64."""
+    ne = int(c.ne[w])
+    s, mv = c.search[w].astype(np.float64), c.mv[w].astype(np.float64)
+    ja, jv, D = c.Jaref[w].astype(np.float64), c.jv[w].astype(np.float64), c.D[w].astype(np.float64)
+    g1 = s @ (c.Ma[w].astype(np.float64) - c.smooth[w]) + (jv[:ne] * D[:ne] * ja[:ne]).sum()
+    g2 = 0.5 * s @ mv + 0.5 * (jv[:ne] ** 2 * D[:ne]).sum()
+    c0, _ = _row_cost64(c, w, ja)
+    ca, sl = _row_cost64(c, w, ja + alpha * jv)
+    return alpha * g1 + alpha * alpha * g2 + ca.sum() - c0.sum(), g1 + 2 * alpha * g2 + (sl * jv).sum()
+
+
+def _exact_alpha(c, w):
+    lo, hi = -1e3, 1e3
+    for _ in range(200):
+        mid = 0.5 * (lo + hi)
+        if _line64(c, w, mid)[1] < 0:
+            lo = mid
+        else:
+            hi = mid
+    return 0.5 * (lo + hi)
+
+
+def _search(c, done=None, its=50):
+    return R.newton_linesearch(c.tol, c.ls_tol, c.mi, c.ne, c.nf, c.nefc, c.smooth, c.D, c.frictionloss, c.Jaref, c.search,
+                               c.search_dot, c.mv, c.jv, c.Ma, done=done, ls_iterations=its)  # fmt: skip
+
+
+def test_oracle_step_against_the_exact_minimiser():
+    nworld, nv = 120, 27
+    c = _line_case(nworld, nv, 64, 5)
+    alpha, imp, ex, ov = _search(c)
+    assert (ov == 0).all()
+    worse = 0
+    for w in range(nworld):
+        a_star = _exact_alpha(c, w)
+        cost_star, _ = _line64(c, w, a_star)
+        cost, slope = _line64(c, w, float(alpha[w]))
+        curv = abs(_line64(c, w, a_star + 1e-3)[1] - _line64(c, w, a_star - 1e-3)[1]) / 2e-3
+        assert cost <= 1e-6 * abs(cost_star), w  # never uphill
+        # the slope left over is within what the stage accepts, or the step is within the noise floor
+        scale = np.sqrt(float(c.search_dot[w])) * nv
+        gtol = max(float(c.tol[0] * c.ls_tol[0]) * scale, 1e-6)
+        q1 = abs(_line64(c, w, 0.0)[1]) + 1.0
+        assert abs(slope) < max(10 * gtol, 64 * NOISE * q1 * 40, 1e-4 * curv * abs(a_star)) or ex[w], (w, slope, a_star, alpha[w])
+        # the reported decrease is a difference of fp32 sums of the rows' costs: absolute error against their size
+        size = _row_cost64(c, w, c.Jaref[w].astype(np.float64))[0].sum() + _row_cost64(c, w, c.Jaref[w] + float(alpha[w]) * c.jv[w].astype(np.float64))[0].sum()
+        np.testing.assert_allclose(imp[w], -cost, rtol=2e-3, atol=2e-6 * size + 1e-6)
+        worse += cost > cost_star * (1 - 1e-3)
+    assert worse <= nworld // 20  # nearly all steps reach the minimum's cost to 0.1 %
+
+
+def test_oracle_closed_form_without_one_sided_rows():
+    c = _line_case(60, 35, 24, 7, one_sided=False)
+    alpha, imp, ex, ov = _search(c)
+    for w in range(60):
+        _, s0 = _line64(c, w, 0.0)
+        _, s1 = _line64(c, w, 1.0)
+        a_star = -s0 / (s1 - s0)  # the line is one parabola
+        np.testing.assert_allclose(alpha[w], a_star, rtol=2e-5)
+        np.testing.assert_allclose(imp[w], -_line64(c, w, a_star)[0], rtol=1e-4)
+    # the budget of rounds is reported when it runs out: one round is too few for a kinked line
+    k = _line_case(60, 27, 64, 5)
+    _, _, _, ov1 = _search(k, its=0)
+    assert (ov1 == 4).any() and set(np.unique(ov1)) <= {0, 4}
+    # done worlds are left alone
+    done = np.zeros(60, np.uint8)
+    done[::3] = 1
+    a2, *_ = _search(k, done=done)
+    assert (a2[::3] == 0).all() and (a2[1::3] != 0).any()
+
+
+def test_oracle_constraint_states_by_definition():
+    c = _line_case(80, 20, 48, 9)
+    old = np.random.default_rng(1).integers(0, 4, (80, 48)).astype(np.int32)
+    ex = (np.arange(80) % 5 == 0).astype(np.uint8)
+    done = (np.arange(80) % 11 == 0).astype(np.uint8)
+    force, st, ids, qc, sc = R.newton_eval_constraints(c.Jaref, c.D, c.frictionloss, c.ne, c.nf, c.nefc, old, done=done, exhausted=ex)
+    for w in range(80):
+        if done[w]:
+            assert qc[w] == 0 and sc[w] == 0 and np.array_equal(st[w], old[w])
+            continue
+        ne, nf, nefc = int(c.ne[w]), int(c.nf[w]), int(c.nefc[w])
+        x, D, f = c.Jaref[w], c.D[w], c.frictionloss[w]
+        want_s = np.ones(48, np.int32)
+        want_f = -D * x
+        r = np.arange(48)
+        fr = (r >= ne) & (r < ne + nf)
+        lo, hi = fr & (x <= -f / D), fr & (x >= f / D)
+        want_s[lo], want_f[lo] = 2, f[lo]
+        want_s[hi], want_f[hi] = 3, -f[hi]
+        sat = (r >= ne + nf) & (x >= 0)
+        want_s[sat], want_f[sat] = 0, 0.0
+        np.testing.assert_array_equal(st[w, :nefc], want_s[:nefc])
+        np.testing.assert_array_equal(st[w, nefc:], old[w, nefc:])
+        np.testing.assert_array_equal(force[w, :nefc], want_f[:nefc])
+        flips = np.flatnonzero((old[w, :nefc] == 1) != (want_s[:nefc] == 1))
+        assert qc[w] == len(flips) and np.array_equal(ids[w, : len(flips)], flips)
+        assert sc[w] == (old[w, :nefc] != want_s[:nefc]).sum() + ex[w]
+
+
+# ---------------------------------------------------------------- a whole Newton solve
+
+
+def _problem(nworld, seed=21):
+    """Humanoid tree, 64 rows: 2 equality, 3 friction loss, the rest one-sided; the solver's state
+    after upstream's initialisation, built with the oracle's pieces from qacc = qacc_smooth."""
+    b = synth.make_batch("humanoid", nworld, ragged_nefc=True)
+    rng = np.random.default_rng(seed)
+    nv, njmax = b.shape.nv, b.shape.nefc
+    pad = 32
+    p = SimpleNamespace(b=b, nv=nv, njmax=njmax, pad=pad, nworld=nworld)
+    p.nefc = np.maximum(b.nefc, 8).astype(np.int32)
+    p.ne, p.nf = np.full(nworld, 2, np.int32), np.full(nworld, 3, np.int32)
+    p.J = b.J
+    p.D = (10.0 ** rng.uniform(0, 3, (nworld, njmax))).astype(np.float32)
+    p.frictionloss = rng.uniform(0.1, 1.0, (nworld, njmax)).astype(np.float32)
+    p.aref = rng.normal(scale=2.0, size=(nworld, njmax)).astype(np.float32)
+    p.qacc_smooth = rng.normal(size=(nworld, nv)).astype(np.float32)
+    p.tables = [np.asarray(a) for a in __import__("instantmimic_amd.mjw_kernels.newton_fusion", fromlist=["x"]).mul_m_tables(b.rowadr, b.rownnz, b.colind)]
+    p.smooth = R.mul_m_sparse(b.M, p.qacc_smooth, *p.tables)
+    p.tol, p.ls_tol, p.mi = np.array([1e-7], np.float32), np.array([0.01], np.float32), np.array([1.0], np.float32)
+    p.maxiter, p.ls_iterations = 30, 50
+    # state after the initialisation
+    s = SimpleNamespace()
+    s.qacc = p.qacc_smooth.copy()
+    s.Ma = p.smooth.copy()
+    s.Jaref = (np.einsum("wrj,wj->wr", p.J.astype(np.float64), s.qacc) - p.aref).astype(np.float32)
+    s.done = np.zeros(nworld, np.uint8)
+    s.niter = np.zeros(nworld, np.int32)
+    s.force, s.state, s.ids, s.qc, s.sc = R.newton_eval_constraints(s.Jaref, p.D, p.frictionloss, p.ne, p.nf, p.nefc, np.zeros((nworld, njmax), np.int32))
+    s.alpha, s.improvement = np.ones(nworld, np.float32), np.zeros(nworld, np.float32)
+    one = np.ones(nworld, np.float32)
+    _, s.grad, s.grad_dot, s.decrement, s.grad_scale, s.unchanged = R.newton_gradient(p.J, s.force, p.smooth, s.Ma, s.sc, s.alpha, one, one, one, nefc=p.nefc, done=s.done, block=32)
+    Md = synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32)
+    H0 = R.jtdj_dense(Md.reshape(nworld, -1), p.J, p.D, np.zeros((nworld, njmax), np.int32), p.nefc, pad)  # M alone
+    s.H, s.U, s.uni, s.search, s.search_dot, s.decrement = R.dense_update_factor(s.sc, s.qc, s.ids, p.J, p.D, s.state, s.grad, H0, np.zeros_like(H0), done=s.done)
+    s.mv, s.jv = np.zeros((nworld, nv), np.float32), np.zeros((nworld, njmax), np.float32)
+    s.exhausted, s.overflow = np.zeros(nworld, np.uint8), np.zeros(nworld, np.int32)
+    return p, s
+
+
+def _oracle_iteration(p, s):
+    b = p.b
+    live = s.done == 0
+    s.mv = np.where((s.unchanged != 0)[:, None], s.mv, R.mul_m_sparse(b.M, s.search, *p.tables))
+    s.jv = R.newton_jv(p.J, s.search, nefc=p.nefc, skip=s.unchanged, out=s.jv.copy())
+    a, imp, ex, ov = R.newton_linesearch(p.tol, p.ls_tol, p.mi, p.ne, p.nf, p.nefc, p.smooth, p.D, p.frictionloss, s.Jaref, s.search,
+                                         s.search_dot, s.mv, s.jv, s.Ma, done=s.done, ls_iterations=p.ls_iterations)  # fmt: skip
+    s.alpha, s.improvement, s.exhausted = np.where(live, a, s.alpha), np.where(live, imp, s.improvement), np.where(live, ex, s.exhausted)
+    s.overflow |= ov
+    s.qacc, s.Ma, s.Jaref = R.newton_advance(s.alpha, s.search, s.mv, s.jv, s.qacc, s.Ma, s.Jaref, nefc=p.nefc, done=s.done)
+    force, state, ids, s.qc, s.sc = R.newton_eval_constraints(s.Jaref, p.D, p.frictionloss, p.ne, p.nf, p.nefc, s.state, done=s.done, exhausted=s.exhausted)
+    s.force, s.state = np.where(live[:, None], force, s.force), state
+    s.ids = np.where(live[:, None], ids, s.ids)
+    _, grad, s.grad_dot, s.decrement, s.grad_scale, s.unchanged = R.newton_gradient(p.J, s.force, p.smooth, s.Ma, s.sc, s.alpha, s.grad_dot, s.decrement, s.grad_scale, nefc=p.nefc, done=s.done, block=32)
+    ran = live & (s.sc != 0)
+    s.grad = np.where(ran[:, None], grad, s.grad)
+    H, U, _, search, sdot, decr = R.dense_update_factor(s.sc, s.qc, s.ids, p.J, p.D, s.state, s.grad, s.H, s.U, done=s.done)
+    s.H, s.U = H, U
+    s.search = np.where(ran[:, None], search, s.search)
+    s.search_dot, s.decrement = np.where(ran, sdot, s.search_dot), np.where(ran, decr, s.decrement)
+    s.niter, s.done, ov2, _ = R.newton_converged(s.alpha, s.improvement, s.grad_dot, s.decrement, p.tol, p.mi, p.nv, p.maxiter, s.niter, s.done, overflow_bit=8)
+    s.overflow |= ov2
+
+
+def _cost64(p, qacc):
+    """The constraint solver's cost at qacc, fp64, per world."""
+    b = p.b
+    M64 = synth.dense_from_csr(b.M.astype(np.float64), b.rowadr, b.rownnz, b.colind)
+    dq = qacc.astype(np.float64) - p.qacc_smooth
+    gauss = 0.5 * np.einsum("wi,wij,wj->w", dq, M64, dq)
+    x = np.einsum("wrj,wj->wr", p.J.astype(np.float64), qacc.astype(np.float64)) - p.aref
+    out = gauss.copy()
+    for w in range(p.nworld):
+        c = SimpleNamespace(ne=p.ne, nf=p.nf, nefc=p.nefc, D=p.D, frictionloss=p.frictionloss)
+        rows, _ = _row_cost64(c, w, x[w])
+        ne = int(p.ne[w])
+        out[w] += rows.sum() + 0.5 * (p.D[w, :ne].astype(np.float64) * x[w, :ne] ** 2).sum()
+    return out
+
+
+def test_oracle_newton_loop_converges_with_a_monotone_cost():
+    p, s = _problem(40)
+    costs = [_cost64(p, s.qacc)]
+    for _ in range(p.maxiter):
+        _oracle_iteration(p, s)
+        costs.append(_cost64(p, s.qacc))
+        if s.done.all():
+            break
+    costs = np.array(costs)
+    assert s.done.all() and (s.overflow & 8 == 0).all() and s.niter.max() < 20
+    assert (np.diff(costs, axis=0) <= 1e-5 * np.abs(costs[:-1]) + 1e-6).all()
+    # at the solution the gradient of the fp64 cost vanishes against the problem's scale
+    b = p.b
+    M64 = synth.dense_from_csr(b.M.astype(np.float64), b.rowadr, b.rownnz, b.colind)
+    x = np.einsum("wrj,wj->wr", p.J.astype(np.float64), s.qacc.astype(np.float64)) - p.aref
+    g = np.einsum("wij,wj->wi", M64, s.qacc.astype(np.float64) - p.qacc_smooth)
+    for w in range(p.nworld):
+        c = SimpleNamespace(ne=p.ne, nf=p.nf, nefc=p.nefc, D=p.D, frictionloss=p.frictionloss)
+        _, slope = _row_cost64(c, w, x[w])
+        ne = int(p.ne[w])
+        slope[:ne] = p.D[w, :ne] * x[w, :ne]
+        g[w] += slope @ p.J[w].astype(np.float64)
+    g0 = np.linalg.norm(np.einsum("wrj,wr->wj", p.J.astype(np.float64), p.D * np.abs(p.aref)), axis=1)
+    assert (np.linalg.norm(g, axis=1) / g0).max() < 1e-4
+
+
+@pytest.mark.gpu
+def test_gpu_linesearch_and_constraints_bitwise(device):
+    import torch
+
+    from instantmimic_amd.mjw_kernels import newton_fusion as NF
+
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    for nworld, nv, njmax, seed in ((333, 27, 64, 5), (100, 56, 128, 6), (64, 14, 32, 8)):
+        c = _line_case(nworld, nv, njmax, seed)
+        done = (np.arange(nworld) % 7 == 3).astype(np.uint8)
+        want = _search(c, done=done, its=6)
+        alpha, imp = torch.full((nworld,), 9.0, device=device), torch.full((nworld,), 9.0, device=device)
+        ex, ov = torch.zeros(nworld, dtype=torch.uint8, device=device), torch.zeros(nworld, dtype=torch.int32, device=device)
+        NF.linesearch(t(c.tol), t(c.ls_tol), t(c.mi), t(c.ne), t(c.nf), t(c.nefc), t(c.smooth), t(c.D), t(c.frictionloss), t(c.Jaref),
+                      t(c.search), t(c.search_dot), t(c.mv), t(c.jv), t(c.Ma), t(done), alpha, imp, ex, ls_iterations=6, overflow=ov,
+                      overflow_bit=4)  # fmt: skip
+        torch.cuda.synchronize()
+        live = done == 0
+        np.testing.assert_array_equal(alpha.cpu().numpy()[live], want[0][live])
+        np.testing.assert_array_equal(imp.cpu().numpy()[live], want[1][live])
+        np.testing.assert_array_equal(ex.cpu().numpy()[live], want[2][live])
+        np.testing.assert_array_equal(ov.cpu().numpy(), want[3])
+        assert (alpha.cpu().numpy()[~live] == 9.0).all()
+        old = np.random.default_rng(seed).integers(0, 4, (nworld, njmax)).astype(np.int32)
+        wf, ws, wi, wq, wc = R.newton_eval_constraints(c.Jaref, c.D, c.frictionloss, c.ne, c.nf, c.nefc, old, done=done, exhausted=want[2])
+        force, state = torch.zeros((nworld, njmax), device=device), t(old)
+        ids = torch.zeros((nworld, njmax), dtype=torch.int32, device=device)
+        qc, sc = torch.full((nworld,), 5, dtype=torch.int32, device=device), torch.full((nworld,), 5, dtype=torch.int32, device=device)
+        NF.eval_constraints(t(c.Jaref), t(c.D), t(c.frictionloss), t(c.ne), t(c.nf), t(c.nefc), t(done), t(want[2]), force, state, ids, qc, sc)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(force.cpu().numpy(), wf)
+        np.testing.assert_array_equal(state.cpu().numpy(), ws)
+        np.testing.assert_array_equal(qc.cpu().numpy(), wq)
+        np.testing.assert_array_equal(sc.cpu().numpy(), wc)
+        for w in range(nworld):
+            np.testing.assert_array_equal(ids.cpu().numpy()[w, : wq[w]], wi[w, : wq[w]])
+
+
+@pytest.mark.gpu
+def test_gpu_newton_run_against_the_oracle_chain(device):
+    """newton_fusion.run on 500 worlds against the oracle's pieces chained in the same order:
+    the same number of iterations per world and the same qacc, bit for bit."""
+    import torch
+
+    from instantmimic_amd.mjw_kernels import newton_fusion as NF
+
+    nworld = 500
+    p, s = _problem(nworld)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    b = p.b
+    m = SimpleNamespace(nv=p.nv, nv_pad=p.pad, M_mulm_rowadr=t(p.tables[0]), M_mulm_col=t(p.tables[1]), M_mulm_madr=t(p.tables[2]),
+                        opt=SimpleNamespace(tolerance=t(p.tol), ls_tolerance=t(p.ls_tol), iterations=p.maxiter, ls_iterations=p.ls_iterations),
+                        stat=SimpleNamespace(meaninertia=t(p.mi)), block_dim=SimpleNamespace(linesearch_iterative=32))  # fmt: skip
+    grad = torch.zeros((nworld, p.pad), device=device)
+    grad[:, : p.nv] = t(s.grad)
+    d = SimpleNamespace(nworld=nworld, M=t(b.M), ne=t(p.ne), nf=t(p.nf), nefc=t(p.nefc), qfrc_smooth=t(p.smooth), qacc=t(s.qacc),
+                        efc=SimpleNamespace(J=t(p.J), D=t(p.D), frictionloss=t(p.frictionloss), Ma=t(s.Ma), force=t(s.force), state=t(s.state)),
+                        qfrc_constraint=torch.zeros((nworld, p.nv), device=device), solver_niter=t(s.niter), overflow=t(s.overflow))  # fmt: skip
+    ctx = SimpleNamespace(search=t(s.search), search_dot=t(s.search_dot), mv=t(s.mv), jv=t(s.jv), Jaref=t(s.Jaref), done=t(s.done),
+                          alpha=t(s.alpha), improvement=t(s.improvement), ls_exhausted=t(s.exhausted), quad_changed_ids=t(s.ids),
+                          quad_changed_count=t(s.qc), state_changed_count=t(s.sc), search_unchanged=t(s.unchanged), grad=grad,
+                          grad_dot=t(s.grad_dot), grad_scale=t(s.grad_scale), newton_decrement=t(s.decrement), h=t(s.H), hfactor=t(s.U),
+                          newton_dof_union=torch.zeros((nworld, p.nv + 1), dtype=torch.int32, device=device))  # fmt: skip
+    nsolving = torch.full((1,), nworld, dtype=torch.int32, device=device)
+    start = _cost64(p, s.qacc)
+    launched = NF.run(m, d, ctx, nsolving)
+    torch.cuda.synchronize()
+    for _ in range(launched):
+        _oracle_iteration(p, s)
+    assert int(nsolving.item()) == 0 and s.done.all() and launched < p.maxiter
+    np.testing.assert_array_equal(d.solver_niter.cpu().numpy(), s.niter)
+    np.testing.assert_array_equal(ctx.done.cpu().numpy(), s.done)
+    np.testing.assert_array_equal(d.qacc.cpu().numpy(), s.qacc)
+    np.testing.assert_array_equal(d.efc.state.cpu().numpy(), s.state)
+    np.testing.assert_array_equal(d.efc.force.cpu().numpy(), s.force)
+    np.testing.assert_array_equal(d.overflow.cpu().numpy(), s.overflow)
+    assert (_cost64(p, d.qacc.cpu().numpy()) < start).all()
