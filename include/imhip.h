@@ -137,6 +137,19 @@ int im_assemble_tree_ldl_solve_iters(const im_tree_plan *plan, const float *M, i
                                      int64_t x_iter_stride, int nworld, int niter, unsigned flags,
                                      void *stream);
 
+/* Kernels generated for one structure and plan, loaded at run time.  The reference emits
+ * straight-line code for any model when its scratch is created
+ * (src/instantmimic/utils/mjw_kernels/tree_ldl.py:196-359, 393-416); here the library carries such
+ * kernels for a few known trees and takes the others as a gfx950 code object that the host side
+ * builds from the generator's source (instantmimic_amd/codegen/tree_row16.py, module form).
+ * im_tree_plan_kernel_key: the 64-bit key of the plan's structure and elimination plan, and whether
+ * the plan already has generated kernels.  im_tree_plan_attach_kernels: loads the code object
+ * (kept by the plan until it is destroyed) after checking that it was generated for this key;
+ * IM_ERR_STRUCTURE otherwise.  The plan's launches then use it.  Once per plan, on the plan's
+ * device, not while the plan is in use by another thread. */
+int im_tree_plan_kernel_key(const im_tree_plan *plan, unsigned long long *key, int *has_kernel);
+int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object);
+
 /* Self-check of an arithmetic shortcut (no counterpart in the reference): the generated tree
  * kernels take a pivot's reciprocal as the hardware estimate plus one exact-residual correction
  * instead of the full division whenever 2^-101 <= |pivot| < 2^102.  This launch compares the two

@@ -57,7 +57,7 @@ def _host_planner():
     return C.CDLL(PLANNER_LIB)
 
 
-def _plan_of_tree(parents):
+def _plan_of_tree(parents, groups: int = 0):
     """((rowadr, rownnz, colind), groups, trunk, eligible) of a dof tree from the host planner."""
     import ctypes as C
 
@@ -67,7 +67,7 @@ def _plan_of_tree(parents):
     lib = _host_planner()
     handle = C.c_void_p()
     vp = lambda a: C.c_void_p(a.ctypes.data)  # noqa: E731
-    status = lib.im_tree_plan_create(len(parents), vp(rowadr), vp(rownnz), vp(colind), int(colind.size), 0, 1, C.byref(handle))
+    status = lib.im_tree_plan_create(len(parents), vp(rowadr), vp(rownnz), vp(colind), int(colind.size), int(groups), 1, C.byref(handle))
     if status != 0:
         raise RuntimeError(f"host planner refused the tree (status {status})")
     info = _lib.TreePlanInfo()
@@ -103,6 +103,23 @@ def generate_sources() -> list[str]:
                 f.write(src)
         out.append(path)
     return out
+
+
+def prebuild_kernels(trees, group_counts=(0,)) -> list[str]:
+    """Code objects of the generated kernels for the given dof trees (parent lists) and group
+    counts (0 = the best plan), into the kernel cache beside the library: what plan creation would
+    otherwise compile on first use."""
+    from .codegen import jit, tree_row16
+
+    keys = set()
+    for parents in trees:
+        for count in group_counts:
+            st, groups, trunk, _ = _plan_of_tree(list(parents), count)
+            if len(st[0]) > 64:
+                continue
+            if jit.code_object(st, groups, trunk) is not None:
+                keys.add(f"{tree_row16.structure_key(*st, groups, trunk):016x}")
+    return sorted(keys)
 
 
 def _compile(src: str) -> str:

@@ -96,7 +96,11 @@ class _Tree:
         return self.depth[k] // 16 + 1
 
 
-def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
+def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = False) -> str:
+    """HIP source of the kernels for one (structure, plan).  ``module``: a stand-alone code object
+    (kernels ``im_row16_fused``, ``im_row16_fused_long``, ``im_row16_solve`` with C names and the
+    constants ``im_row16_key`` / ``im_row16_info`` that describe them) for loading at run time;
+    otherwise a source file of the library that registers its kernels when the library loads."""
     t = _Tree(rowadr, rownnz, colind)
     nv, nM = t.nv, t.nM
     trunk_set = set(trunk)
@@ -188,7 +192,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     emit("};")
     # LONG: more constraint rows than the straight-line assembly keeps in flight (a loop instead)
     emit("template <bool ASM, bool LONG>")
-    emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? IM_OCC_{name} : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
+    if module:  # the body as a function: the kernels with C names at the end of the file call it
+        emit(f"__device__ __forceinline__ void tree_row16_{name}(IM_ROW16_PARAMS) {{")
+    else:
+        emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? IM_OCC_{name} : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
     emit("  const int lane = threadIdx.x & 63, p = lane & 15, wv = threadIdx.x >> 6;")
     # Several iterations in one launch (fused kernels only): the grid covers (four worlds, iteration)
     # pairs.  Workgroups go to the chip's eight XCDs in turn, each with an L2 of its own, so the
@@ -846,14 +853,26 @@ def generate(name, rowadr, rownnz, colind, groups, trunk) -> str:
     emit("  STAMP();")
     emit("  #undef STAMP")
     emit("}")
-    emit(f"static const Row16Entry entry_{name} = {{0x{key:016x}ull, {nv}, {nM}, {lds_floats * 4}, {4 * PD}, \"{name}\",")
-    emit(f"    (const void *)tree_row16_{name}<true, false>, (const void *)tree_row16_{name}<true, true>,")
-    emit(f"    (const void *)tree_row16_{name}<false, false>}};")
-    emit(f"static const Row16Register reg_{name}(&entry_{name});")
-    emit("} }  // namespace im::gen")
+    if module:
+        args = "M, ldM, J, njmax, D, state, nefc_p, quad, y, ldy, x, ldx, Hout, nworld, flags, niter, state_it, y_it, x_it"
+        emit("} }  // namespace im::gen")
+        for kernel, asm_, long_, bounds in (("fused", "true", "false", f"256, IM_OCC_{name}"), ("fused_long", "true", "true", f"256, IM_OCC_{name}"),
+                                            ("solve", "false", "false", "64, 1")):  # fmt: skip
+            emit(f'extern "C" __global__ __launch_bounds__({bounds}) void im_row16_{kernel}(IM_ROW16_PARAMS) {{')
+            emit(f"  im::gen::tree_row16_{name}<{asm_}, {long_}>({args});")
+            emit("}")
+        emit(f'extern "C" __device__ const unsigned long long im_row16_key = 0x{key:016x}ull;')
+        emit(f'extern "C" __device__ const int im_row16_info[4] = {{{nv}, {nM}, {lds_floats * 4}, {4 * PD}}};  // nv, nM, LDS bytes, short rows')
+    else:
+        emit(f"static const Row16Entry entry_{name} = {{0x{key:016x}ull, {nv}, {nM}, {lds_floats * 4}, {4 * PD}, \"{name}\",")
+        emit(f"    (const void *)tree_row16_{name}<true, false>, (const void *)tree_row16_{name}<true, true>,")
+        emit(f"    (const void *)tree_row16_{name}<false, false>}};")
+        emit(f"static const Row16Register reg_{name}(&entry_{name});")
+        emit("} }  // namespace im::gen")
     # workgroups per CU that the fused kernel is compiled for: what the 160 KB of LDS admit (with
     # the lists of 128 constraint rows), at most 4 -- fewer workgroups leave each wavefront more
     # registers, which the larger trees need
-    occ = max(1, min(int(os.environ.get("IMHIP_OCC", "4")), (160 * 1024) // (lds_floats * 4 + 32 * 128)))
+    occ = max(1, min(int(os.environ.get("IMHIP_OCC", "4")), 4, (160 * 1024) // (lds_floats * 4 + 32 * 128)))
     text = "\n".join(out) + "\n"
-    return text.replace('#include "../tree_row16.h"', f'#include "../tree_row16.h"\n#define IM_OCC_{name} {occ}', 1)
+    header = '#include "tree_row16.h"' if module else '#include "../tree_row16.h"'  # a module is built with -I csrc
+    return text.replace('#include "../tree_row16.h"', f'{header}\n#define IM_OCC_{name} {occ}', 1)

@@ -53,6 +53,10 @@ struct im_tree_plan {
   im::TreeDev dev{};
   int spl = 0;  // H slots per lane
   const void *row16 = nullptr;  // generated kernel for this structure, if one was built
+  // kernels loaded at run time from a code object (im_tree_plan_attach_kernels): row16 then points
+  // at row16_own, whose kernel fields hold hipFunction_t handles of `module`
+  void *module = nullptr;
+  void *row16_own = nullptr;
 };
 
 namespace im {

@@ -411,7 +411,11 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
       // several iterations: whole rounds of the eight XCDs per iteration (spare workgroups exit)
       const unsigned quads = (unsigned)((nworld + 3) / 4);
       const unsigned grid = its.niter > 1 ? (quads + 7) / 8 * 8 * (unsigned)its.niter : quads;
-      IM_HIP_CHECK(hipLaunchKernel(fn, dim3(grid), dim3(assemble ? 256 : 64), args, lds, (hipStream_t)stream));
+      if (plan->module)
+        IM_HIP_CHECK(hipModuleLaunchKernel((hipFunction_t)fn, grid, 1, 1, assemble ? 256 : 64, 1, 1, (unsigned)lds,
+                                           (hipStream_t)stream, args, nullptr));
+      else
+        IM_HIP_CHECK(hipLaunchKernel(fn, dim3(grid), dim3(assemble ? 256 : 64), args, lds, (hipStream_t)stream));
       return IM_OK;
     }
   }
@@ -565,6 +569,53 @@ int im_tree_pattern_violations(const im_tree_plan *plan, const float *J, int njm
   hipLaunchKernelGGL(im::tree_violation_kernel, dim3(nworld), dim3(64), 0, (hipStream_t)stream, plan->dev.related,
                      plan->nv, J, njmax, D, state, nefc, quad, violations);
   IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_tree_plan_kernel_key(const im_tree_plan *plan, unsigned long long *key, int *has_kernel) {
+  if (!plan || !key) return IM_ERR_ARG;
+  *key = im::tree_key(*plan);
+  if (has_kernel) *has_kernel = plan->row16 != nullptr;
+  return IM_OK;
+}
+
+int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object) {
+  if (!plan || !code_object) return IM_ERR_ARG;
+  if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
+  if (plan->module) return IM_ERR_ARG;  // once per plan
+  hipModule_t mod = nullptr;
+  IM_HIP_CHECK(hipModuleLoadData(&mod, code_object));
+  auto fail = [&](int code) {
+    (void)hipModuleUnload(mod);
+    return code;
+  };
+  unsigned long long key = 0;
+  int info[4] = {0, 0, 0, 0};
+  hipDeviceptr_t sym = nullptr;
+  size_t bytes = 0;
+  if (hipModuleGetGlobal(&sym, &bytes, mod, "im_row16_key") != hipSuccess || bytes != sizeof(key) ||
+      hipMemcpyDtoH(&key, sym, sizeof(key)) != hipSuccess)
+    return fail(IM_ERR_STRUCTURE);
+  if (hipModuleGetGlobal(&sym, &bytes, mod, "im_row16_info") != hipSuccess || bytes != sizeof(info) ||
+      hipMemcpyDtoH(info, sym, sizeof(info)) != hipSuccess)
+    return fail(IM_ERR_STRUCTURE);
+  // the kernels are straight-line code for one structure and plan: anything else would read and
+  // write out of place
+  if (key != im::tree_key(*plan) || info[0] != plan->nv || info[1] != plan->nM) return fail(IM_ERR_STRUCTURE);
+  if (info[2] <= 0 || info[2] + 32 * 64 > 64 * 1024 || info[3] <= 0) return fail(IM_ERR_UNSUPPORTED);
+  hipFunction_t fused = nullptr, fused_long = nullptr, solve = nullptr;
+  if (hipModuleGetFunction(&fused, mod, "im_row16_fused") != hipSuccess ||
+      hipModuleGetFunction(&fused_long, mod, "im_row16_fused_long") != hipSuccess ||
+      hipModuleGetFunction(&solve, mod, "im_row16_solve") != hipSuccess)
+    return fail(IM_ERR_STRUCTURE);
+  // plain data, released with free() when the plan goes
+  auto *e = (im::gen::Row16Entry *)std::malloc(sizeof(im::gen::Row16Entry));
+  if (!e) return fail(IM_ERR_ARG);
+  *e = im::gen::Row16Entry{key, info[0], info[1], info[2], info[3], "module", (const void *)fused,
+                           (const void *)fused_long, (const void *)solve};
+  plan->module = mod;
+  plan->row16_own = e;
+  plan->row16 = e;
   return IM_OK;
 }
 

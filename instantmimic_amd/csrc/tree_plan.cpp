@@ -7,6 +7,7 @@
 //   tree_ldl_structure :66-91, _shared_bytes :98-102, plan_tree_ldl :105-170,
 //   best_tree_ldl_plan :173-185, tree_ldl_beats_dense :188-193.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <numeric>
 
@@ -245,6 +246,8 @@ int im_tree_plan_create(int nv, const int32_t *rowadr, const int32_t *rownnz,
 void im_tree_plan_destroy(im_tree_plan *plan) {
   if (!plan) return;
   if (plan->dev_blob) (void)hipFree(plan->dev_blob);
+  if (plan->module) (void)hipModuleUnload((hipModule_t)plan->module);
+  std::free(plan->row16_own);
   delete plan;
 }
 

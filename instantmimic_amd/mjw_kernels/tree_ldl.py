@@ -158,6 +158,11 @@ def scratch_for_plan(structure, plan: TreeLdlPlan, device: Any) -> TreeFactorSol
         raise ValueError("plan does not belong to this structure")
     if not handle.info().device_ready:
         raise UnsupportedShape("shape outside the device kernels' limits (nv <= 64, nM <= 1024)")
+    # straight-line kernels for this model, generated and compiled now unless the library has them
+    from ..codegen import jit
+
+    with torch.cuda.device(dev):
+        jit.attach(handle.ptr, handle.structure, plan.groups, plan.trunk)
     return TreeFactorSolveScratch(kernel=handle, groups=len(plan.groups), cuda=True, plan=plan)
 
 

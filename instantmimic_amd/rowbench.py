@@ -1,6 +1,6 @@
 """Per-kernel timings of the library on the configured shapes, one JSON line per kernel:
 
-    python -m instantmimic_amd.rowbench [--launches N] [--only trees,stress,muscles,walks,iteration,bodies] [--no-graph]
+    python -m instantmimic_amd.rowbench [--launches N] [--only trees,generated,stress,muscles,walks,iteration,bodies] [--no-graph]
 
 Every line names the kernel, the workload, the mean time of one launch (event-timed hipGraph
 replay over rotating input sets), the algorithmic bytes or flops of that launch and the
@@ -71,7 +71,7 @@ def _line(kernel, workload, seconds, *, bytes_=None, flops=None, nworld=None):
 
 
 def run(launches: int = 32, only: str | None = None) -> None:
-    """``only``: comma-separated section names out of trees, stress, muscles, walks, iteration, bodies."""
+    """``only``: comma-separated section names out of trees, generated, stress, muscles, walks, iteration, bodies."""
     import torch
 
     from . import synth
@@ -164,6 +164,32 @@ def run(launches: int = 32, only: str | None = None) -> None:
                     idt = t(ids)
                     sec = _timeit(torch, lambda i: stage(S[i][1], S[i][2], S[i][3], idt, chg, chg, None, S[i][5], None, hf, s2, sd, de, uni), nsets, launches)
                     _line("im_sparse_update_factor", wl + f", {k} changed rows", sec, bytes_=nworld * 4 * (k * nv + 2 * used + 2 * nv + nv + 1 + 2), nworld=nworld)
+            del S, X
+            torch.cuda.empty_cache()
+
+    # ---- trees beside the benchmark shapes: kernels generated and compiled when the plan is created
+    if section("generated"):
+        import os
+
+        for name, parents in synth.extra_trees().items():
+            if name not in ("limbs", "branched", "limbs62"):
+                continue
+            shape = synth.Shape(name, tuple(parents), 64, 4096, (0.5, 8.0), 0.02, (-4.0, 4.0), 0.6, 3, 1001)
+            b = synth.make_batch(shape)
+            nv, nM, nefc, nworld = b.shape.nv, int(b.colind.size), b.shape.nefc, b.nworld
+            m = SimpleNamespace(nv=nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind)
+            S = sets_of((b.M, b.J, b.D, b.state[0], b.nefc, b.grad), 8)
+            X = [torch.zeros(b.grad.shape, device=dev) for _ in range(8)]
+            wl = f"{name} nv={nv} nM={nM} nefc={nefc} x {nworld} worlds"
+            for kind in ("generated", "table-driven"):
+                if kind == "table-driven":
+                    os.environ["IMHIP_TREE_KERNEL"] = "generic"
+                try:
+                    sc = T.create_tree_factor_solve_scratch(m, dev)
+                finally:
+                    os.environ.pop("IMHIP_TREE_KERNEL", None)
+                sec = _timeit(torch, lambda i: T.assemble_tree_factor_solve(sc, *S[i], X[i]), 8, launches)
+                _line(f"im_assemble_tree_ldl_solve ({kind} kernel)", wl, sec, bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv), nworld=nworld)
             del S, X
             torch.cuda.empty_cache()
 
@@ -390,7 +416,7 @@ def run(launches: int = 32, only: str | None = None) -> None:
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--launches", type=int, default=32)
-    ap.add_argument("--only", default=None, help="comma-separated sections: trees, stress, muscles, walks, iteration, bodies")
+    ap.add_argument("--only", default=None, help="comma-separated sections: trees, generated, stress, muscles, walks, iteration, bodies")
     ap.add_argument("--no-graph", action="store_true", help="plain launches instead of a hipGraph replay")
     args = ap.parse_args()
     GRAPH = not args.no_graph

@@ -89,6 +89,19 @@ def chain_parents(hinges: int = 30) -> list[int]:
     return [-1] + list(range(5 + hinges))
 
 
+def extra_trees() -> dict[str, list[int]]:
+    """Dof trees beside the five benchmark shapes that the tests and the per-kernel timings run the
+    generated kernels on: the reference's test models, a 62-dof torso with eight limbs, the contact
+    model's tree and the SNU-like tree with a second free body."""
+    snu_free = snu_parents()
+    n0 = len(snu_free)
+    snu_free += [-1] + list(range(n0, n0 + 5))
+    return {
+        "limbs": limbs_parents(), "branched": branched_parents(), "limbs62": limbs_parents(8, 7),
+        "contact": [int(p) for p in contact_model()[0].dof_parentid], "snu_free": snu_free,
+    }  # fmt: skip
+
+
 def csr_from_parents(parent) -> tuple[np.ndarray, np.ndarray, np.ndarray]:
     """MuJoCo's M CSR for a dof tree: ``rowadr, rownnz, colind`` (int32)."""
     rowadr, rownnz, colind = [], [], []

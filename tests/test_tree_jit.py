@@ -1,0 +1,115 @@
+"""Kernels generated for a model at plan creation (the reference emits straight-line code for any
+model: src/instantmimic/utils/mjw_kernels/tree_ldl.py:196-359, 393-416; its test models:
+tests/test_tree_ldl.py:22-60, 99-236): source from the generator, a gfx950 code object, loaded
+into the plan through the C ABI."""
+
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from instantmimic_amd import _lib, build, synth
+from instantmimic_amd.codegen import jit, tree_row16
+from oracle import planner as P
+from oracle import ref as R
+
+TREES = synth.extra_trees()
+
+
+def test_code_objects_and_keys():
+    for name in ("limbs", "branched"):
+        st, groups, trunk, _ = build._plan_of_tree(TREES[name])
+        blob = jit.code_object(st, groups, trunk)
+        assert blob is not None and len(blob) > 10000 and blob == jit.code_object(st, groups, trunk)
+        for symbol in (b"im_row16_fused", b"im_row16_fused_long", b"im_row16_solve", b"im_row16_key", b"im_row16_info"):
+            assert symbol in blob
+        # the library's key of the same plan (host-only plan: no GPU needed)
+        rowadr, rownnz, colind = (np.asarray(a, np.int32) for a in st)
+        handle = C.c_void_p()
+        assert _lib.lib().im_tree_plan_create(len(rowadr), rowadr.ctypes.data, rownnz.ctypes.data, colind.ctypes.data, len(colind), 0, 1, C.byref(handle)) == 0
+        key, has = C.c_ulonglong(0), C.c_int(7)
+        assert _lib.lib().im_tree_plan_kernel_key(handle, C.byref(key), C.byref(has)) == 0
+        assert key.value == tree_row16.structure_key(*st, groups, trunk) and has.value == 0
+        # a host-only plan takes no kernels
+        buf = C.create_string_buffer(blob, len(blob))
+        assert _lib.lib().im_tree_plan_attach_kernels(handle, buf) == _lib.IM_ERR_UNSUPPORTED
+        assert _lib.lib().im_tree_plan_attach_kernels(handle, None) == _lib.IM_ERR_ARG
+        _lib.lib().im_tree_plan_destroy(handle)
+    # the module form differs from the library form in its kernel heads and tail only
+    st, groups, trunk, _ = build._plan_of_tree(TREES["limbs"])
+    a, b = tree_row16.generate("t", *st, groups, trunk), tree_row16.generate("t", *st, groups, trunk, module=True)
+    la, lb = a.splitlines(), b.splitlines()
+    assert sum(x != y for x, y in zip(la, lb)) <= 12 and abs(len(la) - len(lb)) < 20 and len(la) > 500
+
+
+def _has_kernel(scratch) -> bool:
+    key, has = C.c_ulonglong(0), C.c_int(0)
+    assert _lib.lib().im_tree_plan_kernel_key(scratch.kernel.ptr, C.byref(key), C.byref(has)) == 0
+    return bool(has.value)
+
+
+def _batch(name, nworld, nefc=48):
+    parents = TREES[name]
+    shape = synth.Shape(name, tuple(parents), nefc, nworld, (0.5, 8.0), 0.02, (-4.0, 4.0), 0.6, 3, 31)
+    return synth.make_batch(shape, nworld, ragged_nefc=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,nworld", [("limbs", 203), ("branched", 64), ("limbs62", 130), ("contact", 99), ("snu_free", 77)])
+def test_gpu_generated_kernels_match_the_oracle_bitwise(device, monkeypatch, name, nworld):
+    import torch
+
+    from instantmimic_amd.mjw_kernels import tree_ldl as T
+
+    b = _batch(name, nworld)
+    m = type("m", (), dict(nv=b.shape.nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind))
+    scratch = T.create_tree_factor_solve_scratch(m, device)
+    assert scratch is not None and _has_kernel(scratch)
+    monkeypatch.setenv("IMHIP_TREE_KERNEL", "generic")
+    table_driven = T.create_tree_factor_solve_scratch(m, device)
+    monkeypatch.delenv("IMHIP_TREE_KERNEL")
+    assert not _has_kernel(table_driven)
+    st = (b.rowadr, b.rownnz, b.colind)
+    oplan = P.best_tree_ldl_plan(*st)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    M, J, D, N, G = t(b.M), t(b.J), t(b.D), t(b.nefc), t(b.grad)
+    for sc in (scratch, table_driven):
+        x, H = torch.full_like(G, float("nan")), torch.full_like(M, float("nan"))
+        T.assemble_tree_factor_solve(sc, M, J, D, t(b.state[0]), N, G, x, H_out=H)
+        torch.cuda.synchronize()
+        x_ref, H_ref = R.assemble_tree_ldl_solve(*st, oplan, b.M, b.J, b.D, b.state[0], b.nefc, b.grad, want_h=True)
+        np.testing.assert_array_equal(H.cpu().numpy(), H_ref)
+        np.testing.assert_array_equal(x.cpu().numpy(), x_ref)
+        assert R.rel_l2(x.cpu().numpy(), x_ref) <= 1e-5
+    # factor + solve alone and a step's three iterations in one launch, on the generated kernels
+    x = torch.full_like(G, float("nan"))
+    T.tree_factor_solve(scratch, M, x, G)
+    x3 = torch.full((3,) + tuple(G.shape), float("nan"), device=device)
+    T.assemble_tree_factor_solve_iters(scratch, M, J, D, t(b.state), N, G, x3)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(x.cpu().numpy(), R.tree_ldl_solve(*st, oplan, b.M, b.grad))
+    for it in range(3):
+        np.testing.assert_array_equal(x3[it].cpu().numpy(), R.assemble_tree_ldl_solve(*st, oplan, b.M, b.J, b.D, b.state[it], b.nefc, b.grad))
+
+
+@pytest.mark.gpu
+def test_gpu_attach_checks_the_structure(device):
+    import torch
+
+    from instantmimic_amd.mjw_kernels import tree_ldl as T
+
+    st, groups, trunk, _ = build._plan_of_tree(TREES["limbs"])
+    other = jit.code_object(st, groups, trunk)
+    b = _batch("branched", 8)
+    st_b = T.tree_ldl_structure(b.rowadr, b.rownnz, b.colind)
+    with torch.cuda.device(device):
+        handle = T._PlanHandle(st_b, 0, host_only=False)
+        buf = C.create_string_buffer(other, len(other))
+        assert _lib.lib().im_tree_plan_attach_kernels(handle.ptr, buf) == _lib.IM_ERR_STRUCTURE  # generated for another tree
+        assert jit.attach(handle.ptr, handle.structure, handle.plan().groups, handle.plan().trunk)
+        mine = jit.code_object(handle.structure, handle.plan().groups, handle.plan().trunk)
+        assert _lib.lib().im_tree_plan_attach_kernels(handle.ptr, C.create_string_buffer(mine, len(mine))) == _lib.IM_ERR_ARG  # once per plan
+    # a benchmark tree has its kernels in the library: nothing to attach
+    h = synth.make_batch("humanoid", 4)
+    scratch = T.create_tree_factor_solve_scratch(type("m", (), dict(nv=27, M_rowadr=h.rowadr, M_rownnz=h.rownnz, M_colind=h.colind)), device)
+    assert _has_kernel(scratch)
