@@ -147,14 +147,16 @@ __device__ __forceinline__ void gather_tiles(const float *__restrict__ Mw, const
 // Left-looking upper Cholesky by block column with the forward solve of rhs fused into the
 // loop; U (the staircase of pad) and rhs (pad) in LDS, U zeroed by the caller.
 template <int B, class Src>
-__device__ __forceinline__ void factor_forward(const Src &src, float *U, float *rhs, float *A, float *L, int pad,
-                                               int tid, int nt) {
+__device__ __forceinline__ void factor_forward(const Src &src, float *U, float *rhs, float *L, int pad, int tid,
+                                               int nt) {
   const int nblk = pad / B;
   constexpr int BB = B * B;
   const Stair<B> S{pad};
   for (int kb = 0; kb < nblk; ++kb) {
     const int k = kb * B;
-    // gather the whole block row kb..nblk-1 and subtract the finished block rows above
+    // the whole block row kb..nblk-1 minus the finished block rows above, in place: a tile's
+    // elements are read (from U itself or from the source) before the same wavefront or thread
+    // writes them, and the block rows above are final
     const int ntile = nblk - kb;
     if constexpr (B == 16) {
       // One wavefront per 16 x 16 tile, the sums over a finished block row on the matrix cores:
@@ -181,7 +183,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
           for (int i = 0; i < 4; ++i) v[i] = v[i] - sum[i];
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) A[tb * BB + (4 * kq + i) * B + p] = v[i];
+        for (int i = 0; i < 4; ++i) U[S.in_band(kb, 4 * kq + i, i0 + p)] = v[i];
       }
     } else {
       for (int q = tid; q < ntile * BB; q += nt) {
@@ -195,7 +197,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
           for (int t = 0; t < B; ++t) sum = fma_(U[S.in_band(jb, t, k + r)], U[S.in_band(jb, t, i0 + c)], sum);
           v = v - sum;
         }
-        A[q] = v;
+        U[S.in_band(kb, r, i0 + c)] = v;
       }
     }
     if (tid < B) {
@@ -220,7 +222,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
       const int i = tid;
       float a[B];
 #pragma unroll
-      for (int j = 0; j < B; ++j) a[j] = A[(i < B ? i : 0) * B + j];
+      for (int j = 0; j < B; ++j) a[j] = U[S.in_band(kb, i < B ? i : 0, k + j)];
       float s = rhs[k + (i < B ? i : 0)];
 #pragma unroll
       for (int j = 0; j < B; ++j) {
@@ -246,10 +248,10 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
     }
     for (int q = tid; q < (ntile - 1) * B; q += nt) {
       const int tb = 1 + q / B, c = q - (tb - 1) * B;
-      float *At = A + tb * BB;
+      const int i0 = (kb + tb) * B;
       float col[B];
 #pragma unroll
-      for (int r = 0; r < B; ++r) col[r] = At[r * B + c];
+      for (int r = 0; r < B; ++r) col[r] = U[S.in_band(kb, r, i0 + c)];
 #pragma unroll
       for (int j = 0; j < B; ++j) {
         const float z = col[j] * L[B * B + j];
@@ -257,7 +259,6 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
 #pragma unroll
         for (int i = j + 1; i < B; ++i) col[i] = fma_(-L[i * B + j], z, col[i]);
       }
-      const int i0 = (kb + tb) * B;
 #pragma unroll
       for (int r = 0; r < B; ++r) U[S.in_band(kb, r, i0 + c)] = col[r];
     }
@@ -340,8 +341,7 @@ __global__ __launch_bounds__(512, LEAN ? 6 : 2) void blocked_factor_solve_kernel
   const int nU = S.words();
   float *U = lds;             // [nU] the factor, block row by block row
   float *rhs = U + nU;        // [pad]
-  float *A = rhs + pad;       // [(nblk) * B * B] working tiles of the current block row
-  float *L = A + (pad / B) * B * B;  // [B * B + B] Cholesky factor of the diagonal block (lower), 1 / pivots
+  float *L = rhs + pad;       // [B * B + B] Cholesky factor of the diagonal block (lower), 1 / pivots
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
   for (int i = tid; i < nU; i += nt) U[i] = 0.0f;
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(512, LEAN ? 6 : 2) void blocked_factor_solve_kernel
   gather_tiles<B>(M + w * ldM, block_idx, nM, nv, pad, U, tid, nt);
   __syncthreads();
   const GatheredSrc<B> src{U, pad};
-  factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
+  factor_forward<B>(src, U, rhs, L, pad, tid, nt);
   backward_solve<B>(U, rhs, pad, tid);
   if (x)
     for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
@@ -612,8 +612,7 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
   const int nU = S.words();
   float *U = lds;             // [nU] the factor, block row by block row
   float *rhs = U + nU;        // [pad]
-  float *A = rhs + pad;       // [(pad / B) * B * B]
-  float *L = A + (pad / B) * B * B;  // [B * B + B]: lower factor of the diagonal tile, 1 / pivots
+  float *L = rhs + pad;       // [B * B + B]: lower factor of the diagonal tile, 1 / pivots
   int *ul = (int *)(L + B * B + B);  // [nv] union list, [nv] = its length
   unsigned *mkl = (unsigned *)(ul + nv + 1);  // [nv] per dof: nonzero when a changed row reaches it
   float *jr = (float *)(mkl + nv);  // [row_cap][nv] a batch of changed rows of J, then [row_cap] signed weights
@@ -784,12 +783,12 @@ __global__ __launch_bounds__(1024) void dense_update_factor_kernel(
     if (staged) {
       __syncthreads();
       const LdsSrc<B> src{U, nv, pad};
-      factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
+      factor_forward<B>(src, U, rhs, L, pad, tid, nt);
     } else {
       for (int i = tid; i < nU; i += nt) U[i] = 0.0f;
       __syncthreads();  // this workgroup's own writes to H are read back below
       const DenseSrc<B> src{Hw, nv, pad};
-      factor_forward<B>(src, U, rhs, A, L, pad, tid, nt);
+      factor_forward<B>(src, U, rhs, L, pad, tid, nt);
     }
     // stored factor: the augmented column z = U'^-1 grad above the corner sqrt(1e30 - z.z)
     if (tid < 64) {
@@ -952,17 +951,23 @@ __global__ __launch_bounds__(256) void copy_dense_factor_kernel(const float *__r
 // H[w] = M[w] + J[w]' diag(Dc[w]) J[w], H (nv_pad, nv_pad), on v_mfma_f32_32x32x2_f32.
 // One workgroup of four wavefronts per world, a wavefront per 32 x 32 output tile (the tiles
 // with column block >= row block, dealt round robin, accumulators in registers, mirrored at
-// the end).  J is staged through LDS 32 rows at a time with the row weights beside it; the
-// next 32 rows are already on their way into registers while the matrix cores work on the
-// current ones, and the weighted operand (J Dc) is formed when it is fed.
+// the end).  J is staged through LDS 32 rows at a time with the row weights beside it, in two
+// copies used in turn; the next 32 rows are already on their way into registers while the matrix
+// cores work on the current ones, and the weighted operand (J Dc) is formed when it is fed.
 typedef float float16v __attribute__((ext_vector_type(16)));
 
+// NVR: the staged row width when it is known at compile time (operand addresses then differ by
+// constants that the LDS instructions carry themselves), 0 for any width.
+template <int NVR>
 __global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
     const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
     const float *__restrict__ D, const int32_t *__restrict__ state, const int32_t *__restrict__ nefc_p,
     int quad, float *__restrict__ H, int nv, int nv_pad) {
   extern __shared__ float lds[];
-  const int nvr = (nv + 31) / 32 * 32;   // staged row width
+  const int nvr = NVR ? NVR : (nv + 31) / 32 * 32;   // staged row width
+  // two copies of the staging area: the rows of the next chunk are written while wavefronts that
+  // are behind still read the current one, which leaves one barrier per chunk
+  const int stage_words = 32 * nvr + 32;
   float *Js = lds;                       // [32][nvr] J rows (zero past nefc and past nv)
   float *dcs = Js + 32 * nvr;            // [32] their weights
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1011,39 +1016,41 @@ __global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
     dd = Dw[rowc];
     sd = sw[rowc];
   };
-  auto stage = [&](int r0) {
+  auto stage = [&](int r0, int buf) {
+    float *Jb = Js + buf * stage_words, *db = dcs + buf * stage_words;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const bool in = r0 + wave * 8 + i < nefc;
-      if (c0 < nvr) Js[(wave * 8 + i) * nvr + c0] = (in && c0 < nv) ? v0[i] : 0.0f;  // nvr is 32 for nv <= 32
-      if (c1 < nvr) Js[(wave * 8 + i) * nvr + c1] = (in && c1 < nv) ? v1[i] : 0.0f;
+      if (c0 < nvr) Jb[(wave * 8 + i) * nvr + c0] = (in && c0 < nv) ? v0[i] : 0.0f;  // nvr is 32 for nv <= 32
+      if (c1 < nvr) Jb[(wave * 8 + i) * nvr + c1] = (in && c1 < nv) ? v1[i] : 0.0f;
     }
-    if (lane < 8) dcs[wave * 8 + lane] = (r0 + wave * 8 + lane < nefc && sd == quad) ? dd : 0.0f;
+    if (lane < 8) db[wave * 8 + lane] = (r0 + wave * 8 + lane < nefc && sd == quad) ? dd : 0.0f;
   };
   prefetch(0);
-  stage(0);
+  stage(0, 0);
   __syncthreads();
-  for (int r0 = 0; r0 < nefc; r0 += 32) {
+  for (int r0 = 0, buf = 0; r0 < nefc; r0 += 32, buf ^= 1) {
     prefetch(r0 + 32);
     // v_mfma_f32_32x32x2_f32: lane l supplies A[i = l % 32][k = l / 32] and B[k = l / 32][j = l % 32]
     // the wavefront's tiles take turns inside the loop over the rows: independent accumulators
     // keep the matrix core busy while one of them waits for its previous result
     const float *pa[MAXT], *pb[MAXT];
+    const float *Jc = Js + buf * stage_words, *dc = dcs + buf * stage_words;
 #pragma unroll
     for (int m = 0; m < MAXT; ++m) {
-      pa[m] = Js + (lane >> 5) * nvr + tbi[m] * 32 + (lane & 31);
-      pb[m] = Js + (lane >> 5) * nvr + tbj[m] * 32 + (lane & 31);
+      pa[m] = Jc + (lane >> 5) * nvr + tbi[m] * 32 + (lane & 31);
+      pb[m] = Jc + (lane >> 5) * nvr + tbj[m] * 32 + (lane & 31);
     }
-#pragma unroll 4
+#pragma unroll
     for (int q = 0; q < 16; ++q) {
-      const float dk = dcs[2 * q + (lane >> 5)];
+      const float dk = dc[2 * q + (lane >> 5)];
 #pragma unroll
       for (int m = 0; m < MAXT; ++m)
         if (m < mine)
           acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[m][2 * q * nvr] * dk, pb[m][2 * q * nvr], acc[m], 0, 0, 0);
     }
-    __syncthreads();  // every wavefront is done with the staged rows
-    stage(r0 + 32);
+    // the other copy was last read one chunk ago, before the barrier that every wavefront has passed since
+    stage(r0 + 32, buf ^ 1);
     __syncthreads();
   }
   // accumulator layout of a 32x32 tile: lane l holds column j = l % 32 and rows
@@ -1118,7 +1125,7 @@ static int launch_blocked_factor(const float *M, int64_t ldM, int nM, const int3
     return IM_OK;
   }
   const size_t u_words = B == 8 ? im::Stair<8>{pad}.words() : im::Stair<16>{pad}.words();
-  const size_t lds_bytes = sizeof(float) * (u_words + pad + (size_t)(pad / B) * B * B + B * B + B);
+  const size_t lds_bytes = sizeof(float) * (u_words + pad + B * B + B);
   if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   const bool lean = pad > 96;
   auto fn = B == 8 ? (lean ? im::blocked_factor_solve_kernel<8, true> : im::blocked_factor_solve_kernel<8, false>)
@@ -1245,9 +1252,10 @@ int im_jtdj_mfma(const float *Mdense, const float *J, int njmax, const float *D,
   if (!Mdense || !J || !D || !state || !H) return IM_ERR_ARG;
   if (nv > 128) return IM_ERR_UNSUPPORTED;
   const int nvr = (nv + 31) / 32 * 32;
-  const size_t lds_bytes = sizeof(float) * (32 * (size_t)nvr + 32);
-  hipLaunchKernelGGL(im::jtdj_mfma_kernel, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, Mdense, J,
-                     njmax, D, state, nefc, quad, H, nv, nv_pad);
+  const size_t lds_bytes = sizeof(float) * 2 * (32 * (size_t)nvr + 32);  // two copies of the staged rows
+  auto fn = nvr == 128 ? im::jtdj_mfma_kernel<128> : im::jtdj_mfma_kernel<0>;
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, Mdense, J, njmax, D, state, nefc,
+                     quad, H, nv, nv_pad);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }
@@ -1267,13 +1275,14 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
   if (((uintptr_t)H | (uintptr_t)U) & 15) return IM_ERR_STRIDE;  // read and written 16 bytes at a time
   constexpr int B = 16;
   const size_t base_bytes =
-      sizeof(float) * ((size_t)im::Stair<B>{nv_pad}.words() + nv_pad + (size_t)(nv_pad / B) * B * B + B * B + B +
+      sizeof(float) * ((size_t)im::Stair<B>{nv_pad}.words() + nv_pad + B * B + B +
                        2 * (size_t)nv + 1);
   if (base_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   // room for a batch of up to 32 changed rows of J next to the factor (a multiple of four rows), as
   // far as the 160 KB of LDS reach
   int row_cap = 32;
-  while (row_cap > 0 && base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1) > 160 * 1024) row_cap -= 4;
+  const size_t budget = 160 * 1024;
+  while (row_cap > 0 && base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1) > budget) row_cap -= 4;
   const size_t lds_bytes = base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1);
   auto fn = im::dense_update_factor_kernel<B>;
   if (lds_bytes > 64 * 1024)

@@ -244,3 +244,4 @@ def test_gpu_retained_factor_goes_to_the_dense_block_layout(device):
     assert (qLD[:, :13] == -3.0).all() and (qLD[:, 13 + nv * nv :] == -3.0).all()
     with pytest.raises(RuntimeError, match="requires qLD block offsets"):
         BD._blocked_dense_factor_solve(d, M, x, y, scratch, factor_out=d.qLD)
+
