@@ -115,7 +115,7 @@ def prebuild_kernels(trees, group_counts=(0,)) -> list[str]:
     for parents in trees:
         for count in group_counts:
             st, groups, trunk, _ = _plan_of_tree(list(parents), count)
-            if len(st[0]) > 64:
+            if len(st[0]) > 96:
                 continue
             if jit.code_object(st, groups, trunk) is not None:
                 keys.add(f"{tree_row16.structure_key(*st, groups, trunk):016x}")

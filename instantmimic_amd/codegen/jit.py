@@ -93,7 +93,7 @@ def attach(plan_ptr, structure, groups, trunk) -> bool:
     _lib.check(_lib.lib().im_tree_plan_kernel_key(plan_ptr, C.byref(key), C.byref(has)), "im_tree_plan_kernel_key")
     if has.value:
         return True
-    if not enabled() or len(structure[0]) > 64:
+    if not enabled() or len(structure[0]) > 96:
         return False
     if key.value != tree_row16.structure_key(*structure, groups, trunk):
         raise RuntimeError("the generator's structure key differs from the library's")

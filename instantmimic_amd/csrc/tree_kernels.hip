@@ -419,6 +419,7 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
       return IM_OK;
     }
   }
+  if (!plan->table_driven) return IM_ERR_UNSUPPORTED;  // no generated kernels attached (or they need too much LDS)
   if (its.niter > 1) {  // the table-driven kernel: one launch per iteration
     for (int it = 0; it < its.niter; ++it) {
       const int st = launch(plan, assemble, M, ldM, J, njmax, D, state + it * its.state_it, nefc, quad,
@@ -455,6 +456,15 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
 int tree_plan_upload(im_tree_plan *pl) {
   const int nv = pl->nv, nM = pl->nM;
   pl->device_ready = false;
+  if (nv > 64 && nv <= 96 && nM <= 1024 && pl->groups.size() <= IM_MAX_GROUPS) {
+    // the reference's 68- to 79-dof models: generated kernels only (their lanes follow the chains,
+    // not the dofs), attached by the caller; no tables of the table-driven kernel
+    pl->table_driven = false;
+    pl->row16 = nullptr;
+    IM_HIP_CHECK(hipGetDevice(&pl->device));
+    pl->device_ready = true;
+    return IM_OK;
+  }
   if (nv > 64 || nM > 65535 || pl->groups.size() > IM_MAX_GROUPS) return IM_ERR_UNSUPPORTED;
   const int spl = round_spl((nM + 63) / 64);
   if (!spl) return IM_ERR_UNSUPPORTED;
@@ -564,6 +574,7 @@ int im_tree_pattern_violations(const im_tree_plan *plan, const float *J, int njm
                                void *stream) {
   if (!plan || nworld < 0 || njmax < 0) return IM_ERR_ARG;
   if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
+  if (!plan->table_driven) return IM_ERR_UNSUPPORTED;  // the relation masks hold 64 dofs
   if (nworld == 0 || njmax == 0) return IM_OK;
   if (!J || !D || !state || !violations) return IM_ERR_ARG;
   hipLaunchKernelGGL(im::tree_violation_kernel, dim3(nworld), dim3(64), 0, (hipStream_t)stream, plan->dev.related,
@@ -602,12 +613,19 @@ int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object) {
   // the kernels are straight-line code for one structure and plan: anything else would read and
   // write out of place
   if (key != im::tree_key(*plan) || info[0] != plan->nv || info[1] != plan->nM) return fail(IM_ERR_STRUCTURE);
-  if (info[2] <= 0 || info[2] + 32 * 64 > 64 * 1024 || info[3] <= 0) return fail(IM_ERR_UNSUPPORTED);
+  if (info[2] <= 0 || info[2] + 32 * 64 > 160 * 1024 || info[3] <= 0) return fail(IM_ERR_UNSUPPORTED);
   hipFunction_t fused = nullptr, fused_long = nullptr, solve = nullptr;
   if (hipModuleGetFunction(&fused, mod, "im_row16_fused") != hipSuccess ||
       hipModuleGetFunction(&fused_long, mod, "im_row16_fused_long") != hipSuccess ||
       hipModuleGetFunction(&solve, mod, "im_row16_solve") != hipSuccess)
     return fail(IM_ERR_STRUCTURE);
+  if (info[2] + 32 * 64 > 48 * 1024) {
+    // more than the default dynamic LDS: asked for here; a runtime that refuses the request for a
+    // module's function reports it at the launch
+    (void)hipFuncSetAttribute((const void *)fused, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipFuncSetAttribute((const void *)fused_long, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipGetLastError();
+  }
   // plain data, released with free() when the plan goes
   auto *e = (im::gen::Row16Entry *)std::malloc(sizeof(im::gen::Row16Entry));
   if (!e) return fail(IM_ERR_ARG);

@@ -157,12 +157,14 @@ def scratch_for_plan(structure, plan: TreeLdlPlan, device: Any) -> TreeFactorSol
     if built != plan:
         raise ValueError("plan does not belong to this structure")
     if not handle.info().device_ready:
-        raise UnsupportedShape("shape outside the device kernels' limits (nv <= 64, nM <= 1024)")
+        raise UnsupportedShape("shape outside the device kernels' limits (nv <= 96, nM <= 1024)")
     # straight-line kernels for this model, generated and compiled now unless the library has them
     from ..codegen import jit
 
     with torch.cuda.device(dev):
-        jit.attach(handle.ptr, handle.structure, plan.groups, plan.trunk)
+        attached = jit.attach(handle.ptr, handle.structure, plan.groups, plan.trunk)
+    if not attached and handle.info().nv > 64:
+        raise UnsupportedShape("more than 64 dofs run on generated kernels only, and none could be built")
     return TreeFactorSolveScratch(kernel=handle, groups=len(plan.groups), cuda=True, plan=plan)
 
 

@@ -172,7 +172,7 @@ def run(launches: int = 32, only: str | None = None) -> None:
         import os
 
         for name, parents in synth.extra_trees().items():
-            if name not in ("limbs", "branched", "limbs62"):
+            if name not in ("limbs", "branched", "limbs62", "limbs70", "limbs78"):
                 continue
             shape = synth.Shape(name, tuple(parents), 64, 4096, (0.5, 8.0), 0.02, (-4.0, 4.0), 0.6, 3, 1001)
             b = synth.make_batch(shape)
@@ -181,7 +181,7 @@ def run(launches: int = 32, only: str | None = None) -> None:
             S = sets_of((b.M, b.J, b.D, b.state[0], b.nefc, b.grad), 8)
             X = [torch.zeros(b.grad.shape, device=dev) for _ in range(8)]
             wl = f"{name} nv={nv} nM={nM} nefc={nefc} x {nworld} worlds"
-            for kind in ("generated", "table-driven"):
+            for kind in ("generated", "table-driven") if nv <= 64 else ("generated",):  # beyond 64 dofs: generated kernels only
                 if kind == "table-driven":
                     os.environ["IMHIP_TREE_KERNEL"] = "generic"
                 try:

@@ -91,13 +91,14 @@ def chain_parents(hinges: int = 30) -> list[int]:
 
 def extra_trees() -> dict[str, list[int]]:
     """Dof trees beside the five benchmark shapes that the tests and the per-kernel timings run the
-    generated kernels on: the reference's test models, a 62-dof torso with eight limbs, the contact
+    generated kernels on: the reference's test models, torsos with limbs of 62, 70 and 78 dofs, the contact
     model's tree and the SNU-like tree with a second free body."""
     snu_free = snu_parents()
     n0 = len(snu_free)
     snu_free += [-1] + list(range(n0, n0 + 5))
     return {
         "limbs": limbs_parents(), "branched": branched_parents(), "limbs62": limbs_parents(8, 7),
+        "limbs70": limbs_parents(8, 8), "limbs78": limbs_parents(6, 12),
         "contact": [int(p) for p in contact_model()[0].dof_parentid], "snu_free": snu_free,
     }  # fmt: skip
 

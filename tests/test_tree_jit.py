@@ -57,6 +57,24 @@ def _batch(name, nworld, nefc=48):
 @pytest.mark.gpu
 @pytest.mark.parametrize("name,nworld", [("limbs", 203), ("branched", 64), ("limbs62", 130), ("contact", 99), ("snu_free", 77)])
 def test_gpu_generated_kernels_match_the_oracle_bitwise(device, monkeypatch, name, nworld):
+    _generated_against_oracle(device, monkeypatch, name, nworld, table_driven_too=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,nworld", [("limbs70", 101), ("limbs78", 67)])
+def test_gpu_more_than_64_dofs_run_on_generated_kernels(device, monkeypatch, name, nworld):
+    """The reference's fused Newton takes up to 79 dofs (its test models have 68, 70 and 78:
+    tests/test_tree_ldl.py:178-236); beyond 64 the table-driven kernel does not apply."""
+    from instantmimic_amd.mjw_kernels import tree_ldl as T
+
+    _generated_against_oracle(device, monkeypatch, name, nworld, table_driven_too=False)
+    b = _batch(name, 4)
+    m = type("m", (), dict(nv=b.shape.nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind))
+    monkeypatch.setenv("IMHIP_TREE_JIT", "0")
+    assert T.create_tree_factor_solve_scratch(m, device) is None  # nothing to run it on without generated kernels
+
+
+def _generated_against_oracle(device, monkeypatch, name, nworld, table_driven_too):
     import torch
 
     from instantmimic_amd.mjw_kernels import tree_ldl as T
@@ -65,15 +83,17 @@ def test_gpu_generated_kernels_match_the_oracle_bitwise(device, monkeypatch, nam
     m = type("m", (), dict(nv=b.shape.nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind))
     scratch = T.create_tree_factor_solve_scratch(m, device)
     assert scratch is not None and _has_kernel(scratch)
-    monkeypatch.setenv("IMHIP_TREE_KERNEL", "generic")
-    table_driven = T.create_tree_factor_solve_scratch(m, device)
-    monkeypatch.delenv("IMHIP_TREE_KERNEL")
-    assert not _has_kernel(table_driven)
+    kernels = [scratch]
+    if table_driven_too:
+        monkeypatch.setenv("IMHIP_TREE_KERNEL", "generic")
+        kernels.append(T.create_tree_factor_solve_scratch(m, device))
+        monkeypatch.delenv("IMHIP_TREE_KERNEL")
+        assert not _has_kernel(kernels[1])
     st = (b.rowadr, b.rownnz, b.colind)
     oplan = P.best_tree_ldl_plan(*st)
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
     M, J, D, N, G = t(b.M), t(b.J), t(b.D), t(b.nefc), t(b.grad)
-    for sc in (scratch, table_driven):
+    for sc in kernels:
         x, H = torch.full_like(G, float("nan")), torch.full_like(M, float("nan"))
         T.assemble_tree_factor_solve(sc, M, J, D, t(b.state[0]), N, G, x, H_out=H)
         torch.cuda.synchronize()
