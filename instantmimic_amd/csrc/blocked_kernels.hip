@@ -327,11 +327,8 @@ __device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pa
   }
 }
 
-// LEAN: compiled for six wavefronts per SIMD (80 registers a lane), so that a third workgroup of
-// 512 starts on a CU where the LDS admits it (nv 128: 47 KB each); the few spills that costs are
-// in the gather.  Smaller matrices run fewer wavefronts per workgroup and keep the full budget.
-template <int B, bool LEAN>
-__global__ __launch_bounds__(512, LEAN ? 6 : 2) void blocked_factor_solve_kernel(
+template <int B>
+__global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
     const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
     const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
     int64_t ldx, int nv, int pad, const int32_t *__restrict__ active) {
@@ -600,7 +597,7 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
 // :614-742 (stage), :451-470 (hessian_step), :473-611 (augmented factor).  search = -x,
 // search_dot = x.x, decrement = grad.x (strided over 64 lanes, shuffle-down tree).
 template <int B>
-__global__ __launch_bounds__(1024) void dense_update_factor_kernel(
+__global__ __launch_bounds__(256) void dense_update_factor_kernel(
     const uint8_t *__restrict__ done, const int32_t *__restrict__ state_changes,
     const int32_t *__restrict__ changes, const int32_t *__restrict__ ids, int ld_ids,
     const float *__restrict__ J, int njmax, const float *__restrict__ D, const int32_t *__restrict__ state,
@@ -1127,16 +1124,16 @@ static int launch_blocked_factor(const float *M, int64_t ldM, int nM, const int3
   const size_t u_words = B == 8 ? im::Stair<8>{pad}.words() : im::Stair<16>{pad}.words();
   const size_t lds_bytes = sizeof(float) * (u_words + pad + B * B + B);
   if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
-  const bool lean = pad > 96;
-  auto fn = B == 8 ? (lean ? im::blocked_factor_solve_kernel<8, true> : im::blocked_factor_solve_kernel<8, false>)
-                   : (lean ? im::blocked_factor_solve_kernel<16, true> : im::blocked_factor_solve_kernel<16, false>);
+  auto fn = B == 8 ? im::blocked_factor_solve_kernel<8> : im::blocked_factor_solve_kernel<16>;
   if (lds_bytes > 64 * 1024)
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-  // The pivots of a tile are one wavefront's work whatever the workgroup size, so a small matrix
-  // takes fewer wavefronts per world and more worlds are resident per CU (measured on g1, snu and
-  // the 128-dof stress shape: 64 threads up to pad 48, 128 for 16 x 16 tiles at pad 64, 256 up to
-  // pad 96, 512 beyond: two workgroups per CU there, the block rows' parallel parts want the lanes).
-  const int threads = pad <= 48 ? 64 : (pad <= 64 && B == 16) ? 128 : pad <= 96 ? 256 : 512;
+  // The pivots of a tile, the triangular solves and the right-hand side are one wavefront's work
+  // whatever the workgroup size, and the other wavefronts wait at the barriers meanwhile: what
+  // counts is how many worlds are resident on a CU.  Small workgroups leave the registers for more
+  // of them (measured on g1, snu and the 128-dof stress shape: 64 threads up to pad 48, 128 for
+  // 16 x 16 tiles at pad 64, 256 beyond; at pad 128 four workgroups of 38 KB share a CU and the
+  // launch takes 1.30 ms for 16384 worlds where two of 512 threads took 1.90).
+  const int threads = pad <= 48 ? 64 : (pad <= 64 && B == 16) ? 128 : 256;
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(threads), lds_bytes, (hipStream_t)stream, M, ldM, nM, block_idx, y,
                      ldy, U, x, ldx, nv, pad, active);
   IM_HIP_CHECK(hipGetLastError());
@@ -1281,15 +1278,17 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
   // room for a batch of up to 32 changed rows of J next to the factor (a multiple of four rows), as
   // far as the 160 KB of LDS reach
   int row_cap = 32;
-  const size_t budget = 160 * 1024;
+  // a batch of eight rows where that lets a third workgroup share the CU (nv 128): with few
+  // changed rows, the usual case after the first iterations, the stage is bound by its
+  // single-wavefront parts, which more resident worlds hide (2.83 ms against 3.24 for 25 changed
+  // rows of 256 at 16384 worlds; 4.64 against 4.28 when half of the rows change)
+  const size_t budget = base_bytes + sizeof(float) * 8 * (size_t)(nv + 1) <= 160 * 1024 / 3 ? 160 * 1024 / 3 : 160 * 1024;
   while (row_cap > 0 && base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1) > budget) row_cap -= 4;
   const size_t lds_bytes = base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1);
   auto fn = im::dense_update_factor_kernel<B>;
   if (lds_bytes > 64 * 1024)
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-  // 512 threads for a large matrix: two such workgroups share a CU (75 KB of LDS each at nv 128)
-  // and one's single-wavefront parts (pivots, union, corner chain) run beside the other's wide ones
-  hipLaunchKernelGGL(fn, dim3(nworld), dim3(nv_pad <= 96 ? 256 : 512), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
                      ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, U, dof_union, search, ld_search,
                      search_dot, decrement, nv, nv_pad, row_cap);
   IM_HIP_CHECK(hipGetLastError());
