@@ -159,6 +159,11 @@ int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object);
 int im_check_reciprocal(uint32_t first_bits, uint32_t last_bits, unsigned long long *mismatches,
                         void *stream);
 
+/* The same for the blocked Cholesky's pivots: counts the floats with bit patterns in
+ * [first_bits, last_bits] and value in [2^-96, inf) for which the kernels' short square root or
+ * the short reciprocal of the root differ from sqrtf(x) or 1.0f / sqrtf(x).  Expected: 0. */
+int im_check_pivot_sqrt(uint32_t first_bits, uint32_t last_bits, unsigned long long *mismatches, void *stream);
+
 /* Coupling pattern of a model's dofs: which pairs (a, b) may be nonzero in H.  Replaces
  * hessian_pattern (src/instantmimic/utils/mjw_kernels/sparse_hessian.py:62-118) as a builder:
  * creation couples every dof with its tree ancestors (:70-75; dof_parentid[d] < d), and the

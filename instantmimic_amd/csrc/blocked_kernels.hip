@@ -40,6 +40,36 @@ __device__ __forceinline__ float row_bcast(float v, int n) {
   }
 }
 
+// Square root of a pivot and its reciprocal, IEEE-rounded, without what the compiler adds for
+// tiny, huge and special inputs: v_sqrt_f32 is one ulp off at most and the neighbour test picks
+// the rounded root; the reciprocal is the estimate plus one correction.  Both equal sqrtf(x) and
+// 1.0f / sqrtf(x) bit for bit for every x in [2^-96, inf) (checked over all such floats by
+// im_check_pivot_sqrt); other inputs take the library forms.  The chain from one pivot to the
+// next is less than half as long this way, and that chain bounds the factor.
+__device__ __forceinline__ bool pivot_in_range(float x) { return x >= 0x1p-96f && x < __builtin_inff(); }
+__device__ __forceinline__ float pivot_sqrt_fast(float x) {
+  const float s = __builtin_amdgcn_sqrtf(x);
+  const float below = __builtin_bit_cast(float, __builtin_bit_cast(int, s) - 1);
+  const float above = __builtin_bit_cast(float, __builtin_bit_cast(int, s) + 1);
+  const float eb = fma_(-below, s, x), ea = fma_(-above, s, x);
+  float r = eb <= 0.0f ? below : s;
+  r = ea > 0.0f ? above : r;
+  return r;
+}
+__device__ __forceinline__ float pivot_rcp_fast(float d) {
+  const float r = __builtin_amdgcn_rcpf(d);
+  return fma_(fma_(-d, r, 1.0f), r, r);
+}
+// d = sqrtf(x), rinv = 1.0f / d; `checked`: the lanes whose x is a pivot (the others may hold anything)
+__device__ __forceinline__ void pivot_sqrt_rcp(float x, bool checked, float &d, float &rinv) {
+  d = pivot_sqrt_fast(x);
+  rinv = pivot_rcp_fast(d);
+  if (__builtin_expect(__any(checked && !pivot_in_range(x)), 0)) {
+    d = sqrtf(x);
+    rinv = 1.0f / d;
+  }
+}
+
 // The factor's LDS array: U is upper triangular, so the rows of block row t keep the columns from
 // t * B on and follow one another (a staircase by tiles: 46 KB at pad 144 where the square takes
 // 83 KB, which is what lets two workgroups share a CU there).  Diagonal tiles are held in full.
@@ -224,20 +254,28 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
 #pragma unroll
       for (int j = 0; j < B; ++j) a[j] = U[S.in_band(kb, i < B ? i : 0, k + j)];
       float s = rhs[k + (i < B ? i : 0)];
+      float my_z = 0.0f, my_rinv = 0.0f;
+      // nothing is stored inside the loop: a store's wait and the branch around it would sit in
+      // the chain from one pivot to the next.  Column j of the factor replaces a[j], lane j keeps
+      // the solved right-hand side entry and the pivot's reciprocal.
 #pragma unroll
       for (int j = 0; j < B; ++j) {
-        const float d = sqrtf(row_bcast(a[j], j));
-        const float rinv = 1.0f / d;
+        float d, rinv;
+        pivot_sqrt_rcp(row_bcast(a[j], j), i < B, d, rinv);
         const float lj = i == j ? d : a[j] * rinv;  // rows below the diagonal; unused above
-        if (i >= j && i < B) L[i * B + j] = lj;
         const float z = row_bcast(s, j) * rinv;
-        if (i == j) {
-          rhs[k + j] = z;
-          L[B * B + j] = rinv;  // reciprocals of the pivots, behind the tile
-        }
+        my_z = i == j ? z : my_z;
+        my_rinv = i == j ? rinv : my_rinv;
         s = fma_(-lj, z, s);  // meaningful for i > j
 #pragma unroll
         for (int jj = j + 1; jj < B; ++jj) a[jj] = fma_(-lj, row_bcast(lj, jj), a[jj]);
+        a[j] = lj;
+      }
+      if (i < B) {
+#pragma unroll
+        for (int j = 0; j < B; ++j) L[i * B + j] = a[j];  // entries above the diagonal are never read
+        rhs[k + i] = my_z;
+        L[B * B + i] = my_rinv;  // reciprocals of the pivots, behind the tile
       }
     }
     __syncthreads();
@@ -286,12 +324,14 @@ __device__ __forceinline__ void backward_solve(const float *U, float *rhs, int p
         for (int t = 0; t < B; ++t) sum = fma_(Ur[j + t], rhs[j + t], sum);
         s = s - sum;
       }
+      float my_x = 0.0f;
 #pragma unroll
       for (int c = B - 1; c >= 0; --c) {
         const float x = row_bcast(s * rinv, c);
-        if (tid == c) rhs[i0 + c] = x;
+        my_x = tid == c ? x : my_x;
         s = fma_(-urow[c], x, s);  // meaningful for rows above c
       }
+      if (tid < B) rhs[i0 + tid] = my_x;
     }
     __syncthreads();
   }
@@ -316,12 +356,14 @@ __device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pa
         for (int t = 0; t < B; ++t) sum = fma_(U[S.in_band(j / B, t, k + i)], rhs[j + t], sum);
         s = s - sum;
       }
+      float my_z = 0.0f;
 #pragma unroll
       for (int j = 0; j < B; ++j) {
         const float z = row_bcast(s * rinv, j);
-        if (tid == j) rhs[k + j] = z;
+        my_z = tid == j ? z : my_z;
         s = fma_(-ucol[j], z, s);  // meaningful for rows below j
       }
+      if (tid < B) rhs[k + tid] = my_z;
     }
     __syncthreads();
   }
@@ -513,8 +555,8 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
       float s = rhs[k + (i < B ? i : 0)];
 #pragma unroll
       for (int j = 0; j < B; ++j) {
-        const float d = sqrtf(row_bcast(a[j], j));
-        const float rinv = 1.0f / d;
+        float d, rinv;
+        pivot_sqrt_rcp(row_bcast(a[j], j), true, d, rinv);
         const float lj = i == j ? d : a[j] * rinv;
         if (i >= j && i < B) L[i * B + j] = lj;
         const float z = row_bcast(s, j) * rinv;
@@ -612,7 +654,7 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
   float *L = rhs + pad;       // [B * B + B]: lower factor of the diagonal tile, 1 / pivots
   int *ul = (int *)(L + B * B + B);  // [nv] union list, [nv] = its length
   unsigned *mkl = (unsigned *)(ul + nv + 1);  // [nv] per dof: nonzero when a changed row reaches it
-  float *jr = (float *)(mkl + nv);  // [row_cap][nv] a batch of changed rows of J, then [row_cap] signed weights
+  float *jr = (float *)(mkl + nv);  // [row_cap] signed weights of a batch of changed rows, [row_cap] their numbers
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
   if ((done && done[w]) || state_changes[w] == 0) return;
@@ -623,13 +665,108 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
   count = count < ld_ids ? count : ld_ids;
   for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? gw[i] : 0.0f;
   if (count > 0) {
-    // H's upper triangle is brought into the LDS array of the factor, updated there, written back,
-    // and factored in place.  The changed rows of J and their signed weights pass through LDS
-    // row_cap at a time, the pair sums staying in the matrix cores' accumulators from one batch to
-    // the next; without room for a batch of four rows they are read from memory pair by pair.
+    // The changed rows of J and their signed weights pass through LDS in batches that use the
+    // factor's array while it is still free (up to 64 rows each), the pair sums staying in the
+    // matrix cores' accumulators from one batch to the next; the sums go to H in memory, and H's
+    // upper triangle is then brought into the array and factored in place.  Without room for a
+    // batch of four rows the pairs are read from memory one by one.
     const bool staged = row_cap >= 4;
-    float *sd = jr + (size_t)row_cap * nv;
+    float *sd = jr;  // [row_cap] signed weights of a batch
     if (staged) {
+      float *jb = U;  // [row_cap][nv] a batch of changed rows
+      for (int dof = tid; dof < nv; dof += nt) mkl[dof] = 0u;
+      // All pair sums of a 16 x 16 tile of dofs at once on the matrix cores.  Every changed row
+      // enters every pair here, also where one of the two dofs is zero in it: such a term adds
+      // +-0 to a sum that started at +0, which leaves all its bits, so the sums equal the ones
+      // that skip those rows.  v_mfma_f32_16x16x4_f32 adds its four products one after the
+      // other with a fused multiply-add each, rows ascending; a batch holds a multiple of four
+      // rows, so the chain of a pair runs through the batches as through one list.
+      typedef float f32x4 __attribute__((ext_vector_type(4)));
+      constexpr int HELD = 5;  // tiles a wavefront keeps sums for at a time; more tiles (36 over 4 wavefronts at nv 128) take another pass over the rows
+      const int lane = tid & 63, p = lane & 15, kq = lane >> 4, wv = tid >> 6, nwv = nt >> 6;
+      const int nb = (nv + 15) / 16, ntiles = nb * (nb + 1) / 2;
+      for (int tile0 = 0; tile0 < ntiles; tile0 += HELD * nwv) {
+        f32x4 acc[HELD];
+        int ra[HELD], ca[HELD];
+#pragma unroll
+        for (int h = 0; h < HELD; ++h) {
+          acc[h] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+          const int tile = tile0 + wv + h * nwv;
+          int cb = (int)((sqrtf((float)(8 * tile + 1)) - 1.0f) * 0.5f);
+          while ((cb + 1) * (cb + 2) / 2 <= tile) ++cb;
+          while (cb * (cb + 1) / 2 > tile) --cb;
+          const int rb = tile - cb * (cb + 1) / 2;
+          ra[h] = tile < ntiles ? 16 * rb + p : -1;  // the dofs this lane feeds; -1: no such tile
+          ca[h] = 16 * cb + p;
+        }
+        for (int c0 = 0; c0 < count; c0 += row_cap) {
+          const int nrow = count - c0 < row_cap ? count - c0 : row_cap;
+          __syncthreads();  // the batch before this one has been read by everyone
+          // the batch's row numbers first, then every element of its rows is requested before the
+          // first one is stored: one trip to memory for the numbers and one for the rows
+          int *rowid = (int *)(sd + row_cap);
+          for (int t = tid; t < nrow; t += nt) {
+            const int r = idw[c0 + t];
+            rowid[t] = r;
+            sd[t] = sw[r] == quad ? Dw[r] : -Dw[r];
+          }
+          __syncthreads();
+          const int total = nrow * nv;
+          constexpr int INFLIGHT = 16;
+          for (int q0 = tid; q0 < total; q0 += INFLIGHT * nt) {
+            float v[INFLIGHT];
+#pragma unroll
+            for (int k = 0; k < INFLIGHT; ++k) {
+              const int q = q0 + k * nt < total ? q0 + k * nt : total - 1;
+              const int t = q / nv;
+              v[k] = Jw[(size_t)rowid[t] * nv + (q - t * nv)];
+            }
+#pragma unroll
+            for (int k = 0; k < INFLIGHT; ++k)
+              if (q0 + k * nt < total) jb[q0 + k * nt] = v[k];
+          }
+          __syncthreads();
+          if (tile0 == 0)  // dofs some changed row reaches
+            for (int dof = tid; dof < nv; dof += nt) {
+              unsigned hit = mkl[dof];
+              for (int t = 0; t < nrow && !hit; ++t) hit = jb[t * nv + dof] != 0.0f;
+              mkl[dof] = hit;
+            }
+          // four rows at a time for all the held tiles: their sums are independent, so the matrix
+          // cores work on one while the operands of the next arrive
+          for (int t0 = 0; t0 < nrow; t0 += 4) {
+            const int t = t0 + kq, tc = t < nrow ? t : nrow - 1;
+            const float wgt = t < nrow ? sd[tc] : 0.0f;
+            const float *row = jb + tc * nv;
+#pragma unroll
+            for (int h = 0; h < HELD; ++h) {
+              if (ra[h] >= 0) {  // the same for the whole wavefront
+                const float a = ra[h] < nv ? wgt * row[ra[h]] : 0.0f;  // -(D a) == (-D) a exactly
+                const float b = (t < nrow && ca[h] < nv) ? row[ca[h]] : 0.0f;
+                acc[h] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[h], 0, 0, 0);
+              }
+            }
+          }
+        }
+        // H's elements of all the held tiles are requested before the first sum is added
+        float hv[HELD][4];
+#pragma unroll
+        for (int h = 0; h < HELD; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int row = ra[h] - p + 4 * kq + i, col = ca[h];
+            const bool mine = ra[h] >= 0 && row <= col && col < nv && acc[h][i] != 0.0f;
+            hv[h][i] = mine ? Hw[(size_t)row * pad + col] : 0.0f;
+          }
+#pragma unroll
+        for (int h = 0; h < HELD; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int row = ra[h] - p + 4 * kq + i, col = ca[h];
+            if (ra[h] >= 0 && row <= col && col < nv && acc[h][i] != 0.0f) Hw[(size_t)row * pad + col] = hv[h][i] + acc[h][i];
+          }
+      }
+      __syncthreads();  // the rows are done with the array; this workgroup's writes to H are read back below
       // 16 bytes per lane and four requests in flight; the tiles below the diagonal are not read
       const int nvec = pad * pad / 4;  // pad is a multiple of 16
       for (int i0 = tid; i0 < nvec; i0 += 4 * nt) {
@@ -652,84 +789,6 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
               o.z = (r < nv && c + 2 < nv && r <= c + 2) ? v[k].z : 0.0f;
               o.w = (r < nv && c + 3 < nv && r <= c + 3) ? v[k].w : 0.0f;
               *(float4 *)(U + S.at(r, c)) = o;
-            }
-          }
-        }
-      }
-      for (int dof = tid; dof < nv; dof += nt) mkl[dof] = 0u;
-      // All pair sums of a 16 x 16 tile of dofs at once on the matrix cores.  Every changed row
-      // enters every pair here, also where one of the two dofs is zero in it: such a term adds
-      // +-0 to a sum that started at +0, which leaves all its bits, so the sums equal the ones
-      // that skip those rows.  v_mfma_f32_16x16x4_f32 adds its four products one after the
-      // other with a fused multiply-add each, rows ascending; a batch holds a multiple of four
-      // rows, so the chain of a pair runs through the batches as through one list.
-      typedef float f32x4 __attribute__((ext_vector_type(4)));
-      constexpr int HELD = 5;  // tiles a wavefront keeps sums for at a time (36 tiles over 8 wavefronts at nv 128)
-      const int lane = tid & 63, p = lane & 15, kq = lane >> 4, wv = tid >> 6, nwv = nt >> 6;
-      const int nb = (nv + 15) / 16, ntiles = nb * (nb + 1) / 2;
-      for (int tile0 = 0; tile0 < ntiles; tile0 += HELD * nwv) {
-        f32x4 acc[HELD];
-        int ra[HELD], ca[HELD];
-#pragma unroll
-        for (int h = 0; h < HELD; ++h) {
-          acc[h] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-          const int tile = tile0 + wv + h * nwv;
-          int cb = (int)((sqrtf((float)(8 * tile + 1)) - 1.0f) * 0.5f);
-          while ((cb + 1) * (cb + 2) / 2 <= tile) ++cb;
-          while (cb * (cb + 1) / 2 > tile) --cb;
-          const int rb = tile - cb * (cb + 1) / 2;
-          ra[h] = tile < ntiles ? 16 * rb + p : -1;  // the dofs this lane feeds; -1: no such tile
-          ca[h] = 16 * cb + p;
-        }
-        for (int c0 = 0; c0 < count; c0 += row_cap) {
-          const int nrow = count - c0 < row_cap ? count - c0 : row_cap;
-          __syncthreads();  // the batch before this one has been read by everyone
-          const int total = nrow * nv;
-          for (int q0 = tid; q0 < total; q0 += 4 * nt) {
-            float v[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-              const int q = q0 + k * nt < total ? q0 + k * nt : total - 1;
-              const int t = q / nv;
-              v[k] = Jw[(size_t)idw[c0 + t] * nv + (q - t * nv)];
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-              if (q0 + k * nt < total) jr[q0 + k * nt] = v[k];
-          }
-          for (int t = tid; t < nrow; t += nt) {
-            const int r = idw[c0 + t];
-            sd[t] = sw[r] == quad ? Dw[r] : -Dw[r];
-          }
-          __syncthreads();
-          if (tile0 == 0)  // dofs some changed row reaches
-            for (int dof = tid; dof < nv; dof += nt) {
-              unsigned hit = mkl[dof];
-              for (int t = 0; t < nrow && !hit; ++t) hit = jr[t * nv + dof] != 0.0f;
-              mkl[dof] = hit;
-            }
-#pragma unroll
-          for (int h = 0; h < HELD; ++h) {
-            if (ra[h] < 0) continue;  // the same for the whole wavefront
-            for (int t0 = 0; t0 < nrow; t0 += 4) {
-              const int t = t0 + kq, tc = t < nrow ? t : nrow - 1;
-              const float wgt = t < nrow ? sd[tc] : 0.0f;
-              const float a = ra[h] < nv ? wgt * jr[tc * nv + ra[h]] : 0.0f;  // -(D a) == (-D) a exactly
-              const float b = (t < nrow && ca[h] < nv) ? jr[tc * nv + ca[h]] : 0.0f;
-              acc[h] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[h], 0, 0, 0);
-            }
-          }
-        }
-#pragma unroll
-        for (int h = 0; h < HELD; ++h) {
-          if (ra[h] < 0) continue;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int row = ra[h] - p + 4 * kq + i, col = ca[h];
-            if (row <= col && col < nv && acc[h][i] != 0.0f) {
-              const float hv = U[S.at(row, col)] + acc[h][i];
-              U[S.at(row, col)] = hv;
-              Hw[(size_t)row * pad + col] = hv;
             }
           }
         }
@@ -1073,6 +1132,21 @@ __global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
   }
 }
 
+// Every float whose bit pattern lies in [first, last] and that is in the pivots' range: do the
+// short forms give the bits of sqrtf and of 1.0f / sqrtf?
+__global__ void check_pivot_sqrt_kernel(uint32_t first, uint32_t last, unsigned long long *mismatches) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  unsigned long long bad = 0;
+  for (uint64_t u = (uint64_t)first + blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; u <= last; u += stride) {
+    const float x = __builtin_bit_cast(float, (uint32_t)u);
+    if (!pivot_in_range(x)) continue;
+    const float d = pivot_sqrt_fast(x), want = sqrtf(x);
+    bad += __builtin_bit_cast(uint32_t, d) != __builtin_bit_cast(uint32_t, want);
+    bad += __builtin_bit_cast(uint32_t, pivot_rcp_fast(want)) != __builtin_bit_cast(uint32_t, 1.0f / want);
+  }
+  if (bad) atomicAdd(mismatches, bad);
+}
+
 }  // namespace
 }  // namespace im
 
@@ -1275,22 +1349,24 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
       sizeof(float) * ((size_t)im::Stair<B>{nv_pad}.words() + nv_pad + B * B + B +
                        2 * (size_t)nv + 1);
   if (base_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
-  // room for a batch of up to 32 changed rows of J next to the factor (a multiple of four rows), as
-  // far as the 160 KB of LDS reach
-  int row_cap = 32;
-  // a batch of eight rows where that lets a third workgroup share the CU (nv 128): with few
-  // changed rows, the usual case after the first iterations, the stage is bound by its
-  // single-wavefront parts, which more resident worlds hide (2.83 ms against 3.24 for 25 changed
-  // rows of 256 at 16384 worlds; 4.64 against 4.28 when half of the rows change)
-  const size_t budget = base_bytes + sizeof(float) * 8 * (size_t)(nv + 1) <= 160 * 1024 / 3 ? 160 * 1024 / 3 : 160 * 1024;
-  while (row_cap > 0 && base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1) > budget) row_cap -= 4;
-  const size_t lds_bytes = base_bytes + sizeof(float) * (size_t)row_cap * (nv + 1);
+  // a batch of changed rows uses the factor's array: up to 64 rows, a multiple of four
+  int row_cap = (int)(im::Stair<B>{nv_pad}.words() / (size_t)nv) & ~3;
+  row_cap = row_cap < 64 ? row_cap : 64;
+  const size_t lds_bytes = base_bytes + sizeof(float) * 128;  // the batch's weights and row numbers behind the tables
   auto fn = im::dense_update_factor_kernel<B>;
   if (lds_bytes > 64 * 1024)
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, done, state_changes, changes,
                      ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, U, dof_union, search, ld_search,
                      search_dot, decrement, nv, nv_pad, row_cap);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_check_pivot_sqrt(uint32_t first_bits, uint32_t last_bits, unsigned long long *mismatches, void *stream) {
+  if (!mismatches || last_bits < first_bits) return IM_ERR_ARG;
+  hipLaunchKernelGGL(im::check_pivot_sqrt_kernel, dim3(4096), dim3(256), 0, (hipStream_t)stream, first_bits, last_bits,
+                     mismatches);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

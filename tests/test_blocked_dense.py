@@ -245,3 +245,18 @@ def test_gpu_retained_factor_goes_to_the_dense_block_layout(device):
     with pytest.raises(RuntimeError, match="requires qLD block offsets"):
         BD._blocked_dense_factor_solve(d, M, x, y, scratch, factor_out=d.qLD)
 
+
+@pytest.mark.gpu
+def test_gpu_short_pivot_forms_equal_sqrtf_and_the_division(device):
+    """The blocked Cholesky takes the square root of a pivot as the hardware's estimate plus a
+    neighbour test and its reciprocal as the estimate plus one correction: both must be the IEEE
+    results for every float in [2^-96, inf), all 1.9e9 of them."""
+    import torch
+
+    from instantmimic_amd import _lib
+
+    count = torch.zeros(1, dtype=torch.int64, device=device)
+    stream = int(torch.cuda.current_stream(device).cuda_stream)
+    assert _lib.lib().im_check_pivot_sqrt(0, 0x7F800000, count.data_ptr(), stream) == _lib.IM_OK
+    torch.cuda.synchronize()
+    assert int(count.item()) == 0
