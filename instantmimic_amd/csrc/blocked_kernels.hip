@@ -200,8 +200,22 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
         f32x4 v;
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = src.load(kb, ib, (4 * kq + i) * B + p, 4 * kq + i, p);
-        for (int jb = 0; jb < kb; ++jb) {
-          const int j = jb * B;
+        // two finished block rows at a time: their sums are independent chains on the matrix
+        // cores; they are subtracted in the block rows' order
+        int jb = 0;
+        for (; jb + 1 < kb; jb += 2) {
+          f32x4 sum0 = {0.0f, 0.0f, 0.0f, 0.0f}, sum1 = sum0;
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4) {
+            const int at0 = S.in_band(jb, 4 * s4 + kq, p), at1 = S.in_band(jb + 1, 4 * s4 + kq, p);
+            const float a0 = U[at0 + k], b0 = U[at0 + i0], a1 = U[at1 + k], b1 = U[at1 + i0];
+            sum0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0, sum0, 0, 0, 0);
+            sum1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1, sum1, 0, 0, 0);
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = (v[i] - sum0[i]) - sum1[i];
+        }
+        if (jb < kb) {
           f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
           for (int s4 = 0; s4 < 4; ++s4) {
@@ -230,16 +244,19 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
         U[S.in_band(kb, r, i0 + c)] = v;
       }
     }
-    if (tid < B) {
-      float s = rhs[k + tid];
+    // the right-hand side's share of the block row: the first B lanes of the last wavefront, which
+    // has the fewest tiles to update
+    const int lr = tid - (nt - 64);
+    if (lr >= 0 && lr < B) {
+      float s = rhs[k + lr];
       for (int jb = 0; jb < kb; ++jb) {
         const int j = jb * B;
         float sum = 0.0f;
 #pragma unroll
-        for (int t = 0; t < B; ++t) sum = fma_(U[S.in_band(jb, t, k + tid)], rhs[j + t], sum);
+        for (int t = 0; t < B; ++t) sum = fma_(U[S.in_band(jb, t, k + lr)], rhs[j + t], sum);
         s = s - sum;
       }
-      rhs[k + tid] = s;
+      rhs[k + lr] = s;
     }
     __syncthreads();
     // Cholesky of the diagonal tile and the forward solve of the right-hand side: the first B
@@ -273,7 +290,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
       }
       if (i < B) {
 #pragma unroll
-        for (int j = 0; j < B; ++j) L[i * B + j] = a[j];  // entries above the diagonal are never read
+        for (int j = 0; j < B; ++j) L[j * B + i] = a[j];  // column j of the factor in a row of L; entries above the diagonal are never read
         rhs[k + i] = my_z;
         L[B * B + i] = my_rinv;  // reciprocals of the pivots, behind the tile
       }
@@ -282,7 +299,7 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
     // U_kk = L', and U_ki = L^-1 A_ki column by column
     for (int e = tid; e < BB; e += nt) {
       const int r = e / B, c = e - r * B;
-      U[S.in_band(kb, r, k + c)] = c >= r ? L[c * B + r] : 0.0f;  // a gathered tile may have sat there
+      U[S.in_band(kb, r, k + c)] = c >= r ? L[r * B + c] : 0.0f;  // a gathered tile may have sat there
     }
     for (int q = tid; q < (ntile - 1) * B; q += nt) {
       const int tb = 1 + q / B, c = q - (tb - 1) * B;
@@ -290,12 +307,26 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
       float col[B];
 #pragma unroll
       for (int r = 0; r < B; ++r) col[r] = U[S.in_band(kb, r, i0 + c)];
+      // column j of the factor is a row of L here: 16 bytes at a time (the same words for every lane)
+      const float4 *L4 = (const float4 *)L;
+      float rinv[B];
+#pragma unroll
+      for (int q4 = 0; q4 < B / 4; ++q4) {
+        const float4 t4 = L4[B * B / 4 + q4];
+        rinv[4 * q4] = t4.x, rinv[4 * q4 + 1] = t4.y, rinv[4 * q4 + 2] = t4.z, rinv[4 * q4 + 3] = t4.w;
+      }
 #pragma unroll
       for (int j = 0; j < B; ++j) {
-        const float z = col[j] * L[B * B + j];
+        const float z = col[j] * rinv[j];
         col[j] = z;
+        float lt[B];
 #pragma unroll
-        for (int i = j + 1; i < B; ++i) col[i] = fma_(-L[i * B + j], z, col[i]);
+        for (int q4 = (j + 1) / 4; q4 < B / 4; ++q4) {
+          const float4 t4 = L4[j * (B / 4) + q4];
+          lt[4 * q4] = t4.x, lt[4 * q4 + 1] = t4.y, lt[4 * q4 + 2] = t4.z, lt[4 * q4 + 3] = t4.w;
+        }
+#pragma unroll
+        for (int i = j + 1; i < B; ++i) col[i] = fma_(-lt[i], z, col[i]);
       }
 #pragma unroll
       for (int r = 0; r < B; ++r) U[S.in_band(kb, r, i0 + c)] = col[r];
@@ -369,8 +400,10 @@ __device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pa
   }
 }
 
+// Compiled for four wavefronts per SIMD (128 registers a lane): four workgroups of 256 share a CU
+// at pad 128, where the LDS admits them.
 template <int B>
-__global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
+__global__ __launch_bounds__(256, 4) void blocked_factor_solve_kernel(
     const float *__restrict__ M, int64_t ldM, int nM, const int32_t *__restrict__ block_idx,
     const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x,
     int64_t ldx, int nv, int pad, const int32_t *__restrict__ active) {
@@ -380,7 +413,7 @@ __global__ __launch_bounds__(256) void blocked_factor_solve_kernel(
   const int nU = S.words();
   float *U = lds;             // [nU] the factor, block row by block row
   float *rhs = U + nU;        // [pad]
-  float *L = rhs + pad;       // [B * B + B] Cholesky factor of the diagonal block (lower), 1 / pivots
+  float *L = rhs + pad;       // [B * B + B] Cholesky factor of the diagonal block (column j in row j), 1 / pivots
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
   for (int i = tid; i < nU; i += nt) U[i] = 0.0f;
@@ -651,7 +684,7 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
   const int nU = S.words();
   float *U = lds;             // [nU] the factor, block row by block row
   float *rhs = U + nU;        // [pad]
-  float *L = rhs + pad;       // [B * B + B]: lower factor of the diagonal tile, 1 / pivots
+  float *L = rhs + pad;       // [B * B + B]: factor of the diagonal tile (column j in row j), 1 / pivots
   int *ul = (int *)(L + B * B + B);  // [nv] union list, [nv] = its length
   unsigned *mkl = (unsigned *)(ul + nv + 1);  // [nv] per dof: nonzero when a changed row reaches it
   float *jr = (float *)(mkl + nv);  // [row_cap] signed weights of a batch of changed rows, [row_cap] their numbers
