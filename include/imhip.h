@@ -252,6 +252,17 @@ int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done,
                           const float *grad, int ldg, float *hfactor, float *search,
                           float *search_dot, float *decrement, int nworld, void *stream);
 
+/* im_jtdj_mfma followed by im_blocked_factor_solve (block size 16, the whole H as one dense tile)
+ * in one launch: a Newton iteration's dense Hessian, its upper Cholesky factor and the solve
+ * (the reference runs the upstream assembly and its blocked factor as separate kernels around
+ * src/instantmimic/utils/mjw_kernels/newton_stages.py:614-742).  H (nworld, nv_pad, nv_pad) is
+ * written when not null (the per-iteration stage updates it later), U (nworld, pad, pad) when not
+ * null, x = H^-1 y when x and y are given.  pad = nv rounded up to 16.  Results equal those of
+ * the two entry points called one after the other, bit for bit.  nv <= 128. */
+int im_jtdj_factor_solve(const float *Mdense, const float *J, int njmax, const float *D, const int32_t *state,
+                         const int32_t *nefc, int quad, float *H, int nv, int nv_pad, const float *y, int64_t ldy,
+                         float *U, int pad, float *x, int64_t ldx, int nworld, void *stream);
+
 /* Replaces the factor stage of the fused Newton loop on the static pattern
  * (newton_stages.factor_factory with a sparse plan, src/instantmimic/utils/mjw_kernels/
  * newton_stages.py:614-742, and the native modes 0 / 1 / 2 of sparse_hessian.py:488-547).

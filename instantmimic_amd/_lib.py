@@ -156,6 +156,7 @@ SIGNATURES = {
         [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i, _vp, _vp, _i, _vp],
     ),
     "im_check_pivot_sqrt": (_i, [_u, _u, _vp, _vp]),
+    "im_jtdj_factor_solve": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _i, _vp, _i64, _vp, _i, _vp, _i64, _i, _vp]),
     "im_tree_plan_kernel_key": (_i, [_vp, _vp, _vp]),
     "im_tree_plan_attach_kernels": (_i, [_vp, _vp]),
     "im_dense_update_factor": (

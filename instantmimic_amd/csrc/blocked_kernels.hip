@@ -1047,12 +1047,12 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 
 // NVR: the staged row width when it is known at compile time (operand addresses then differ by
 // constants that the LDS instructions carry themselves), 0 for any width.
-template <int NVR>
-__global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
-    const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
-    const float *__restrict__ D, const int32_t *__restrict__ state, const int32_t *__restrict__ nefc_p,
-    int quad, float *__restrict__ H, int nv, int nv_pad) {
-  extern __shared__ float lds[];
+// `out(i, j, h)` receives every element i <= j < nv of H once, from the lane that holds it.
+template <int NVR, class Out>
+__device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
+                                           const float *__restrict__ D, const int32_t *__restrict__ state,
+                                           const int32_t *__restrict__ nefc_p, int quad, int nv, float *lds,
+                                           const Out &out) {
   const int nvr = NVR ? NVR : (nv + 31) / 32 * 32;   // staged row width
   // two copies of the staging area: the rows of the next chunk are written while wavefronts that
   // are behind still read the current one, which leaves one barrier per chunk
@@ -1144,7 +1144,6 @@ __global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
   }
   // accumulator layout of a 32x32 tile: lane l holds column j = l % 32 and rows
   // i = 8 * g + 4 * (l / 32) ... for register 4 * g + v: i = 8 * g + (l / 32) * 4 + v
-  float *Hw = H + w * (int64_t)nv_pad * nv_pad;
   const float *Mw = Mdense + w * (int64_t)nv * nv;
 #pragma unroll
   for (int m = 0; m < MAXT; ++m) {
@@ -1155,14 +1154,73 @@ __global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int i = tbi[m] * 32 + 8 * g + (lane >> 5) * 4 + v;
-        // upper triangle from the accumulators, lower triangle mirrored: H is symmetric bit for bit
-        if (i < nv && j < nv && i <= j) {
-          const float h = Mw[(int64_t)i * nv + j] + acc[m][4 * g + v];
-          Hw[(int64_t)i * nv_pad + j] = h;
-          if (i != j) Hw[(int64_t)j * nv_pad + i] = h;
-        }
+        if (i < nv && j < nv && i <= j) out(i, j, Mw[(int64_t)i * nv + j] + acc[m][4 * g + v]);
       }
   }
+}
+
+template <int NVR>
+__global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
+    const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
+    const float *__restrict__ D, const int32_t *__restrict__ state, const int32_t *__restrict__ nefc_p,
+    int quad, float *__restrict__ H, int nv, int nv_pad) {
+  extern __shared__ float lds[];
+  float *Hw = H + blockIdx.x * (int64_t)nv_pad * nv_pad;
+  // upper triangle from the accumulators, lower triangle mirrored: H is symmetric bit for bit
+  jtdj_tiles<NVR>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, [&](int i, int j, float h) {
+    Hw[(int64_t)i * nv_pad + j] = h;
+    if (i != j) Hw[(int64_t)j * nv_pad + i] = h;
+  });
+}
+
+// The same assembly followed, in the same workgroup, by the blocked Cholesky of H and the solve:
+// H goes to memory (the per-iteration stage keeps updating it there) and into the factor's LDS
+// array at once, so the factor neither gathers it from memory nor waits for another launch, and
+// on a CU the matrix-core phase of one world runs beside the pivot chains of the others.  The rows
+// of J are staged in the factor's array, which is free until H is complete.  Results are those of
+// im_jtdj_mfma followed by im_blocked_factor_solve (B = 16) bit for bit.
+template <int NVR>
+__global__ __launch_bounds__(256, 4) void jtdj_factor_solve_kernel(
+    const float *__restrict__ Mdense, const float *__restrict__ J, int njmax, const float *__restrict__ D,
+    const int32_t *__restrict__ state, const int32_t *__restrict__ nefc_p, int quad, float *__restrict__ H, int nv,
+    int nv_pad, const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x, int64_t ldx,
+    int pad) {
+  constexpr int B = 16;
+  extern __shared__ float lds[];
+  const Stair<B> S{pad};
+  const int nU = S.words();
+  const int nvr = NVR ? NVR : (nv + 31) / 32 * 32, stage_words = 2 * (32 * nvr + 32);
+  float *U = lds;       // first the staged rows of J (two copies), then [nU] H, then the factor
+  float *rhs = lds + (nU > stage_words ? nU : stage_words);  // [pad]
+  float *L = rhs + pad;  // [B * B + B]
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int64_t w = blockIdx.x;
+  for (int i = tid; i < pad; i += nt) rhs[i] = (y && i < nv) ? y[w * ldy + i] : 0.0f;
+  float *Hw = H ? H + w * (int64_t)nv_pad * nv_pad : nullptr;
+  // the assembly's last barrier is behind every wavefront when the elements come out, so they can
+  // go where the rows were staged.  The factor reads the upper triangle below nv only (the rest
+  // of a diagonal tile by symmetry, the padding as the identity) and writes every entry of a block
+  // row before anything reads it, so the array needs no clearing.
+  jtdj_tiles<NVR>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, [&](int i, int j, float h) {
+    if (Hw) {
+      Hw[(int64_t)i * nv_pad + j] = h;
+      if (i != j) Hw[(int64_t)j * nv_pad + i] = h;
+    }
+    U[S.at(i, j)] = h;
+  });
+  __syncthreads();
+  const LdsSrc<B> src{U, nv, pad};
+  factor_forward<B>(src, U, rhs, L, pad, tid, nt);
+  backward_solve<B>(U, rhs, pad, tid);
+  if (x)
+    for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
+  if (Uout)
+    for (int i = tid; i < pad * pad / 4; i += nt) {
+      const int r = 4 * i / pad, c = 4 * i - r * pad;
+      float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (c >= r / B * B) v = *(const float4 *)(U + S.at(r, c));
+      ((float4 *)(Uout + w * (int64_t)pad * pad))[i] = v;
+    }
 }
 
 // Every float whose bit pattern lies in [first, last] and that is in the pivots' range: do the
@@ -1360,6 +1418,29 @@ int im_jtdj_mfma(const float *Mdense, const float *J, int njmax, const float *D,
   auto fn = nvr == 128 ? im::jtdj_mfma_kernel<128> : im::jtdj_mfma_kernel<0>;
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, Mdense, J, njmax, D, state, nefc,
                      quad, H, nv, nv_pad);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_jtdj_factor_solve(const float *Mdense, const float *J, int njmax, const float *D, const int32_t *state,
+                         const int32_t *nefc, int quad, float *H, int nv, int nv_pad, const float *y, int64_t ldy,
+                         float *U, int pad, float *x, int64_t ldx, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || njmax <= 0 || (H && nv_pad < nv)) return IM_ERR_ARG;
+  if (check_blocked_shape(16, nv, pad) != IM_OK) return check_blocked_shape(16, nv, pad);
+  if (nworld == 0) return IM_OK;
+  if (!Mdense || !J || !D || !state || (x && !y)) return IM_ERR_ARG;
+  if (nv > 128) return IM_ERR_UNSUPPORTED;
+  if ((y && ldy < nv) || (x && ldx < nv)) return IM_ERR_STRIDE;
+  if (U && ((uintptr_t)U & 15)) return IM_ERR_STRIDE;
+  const int nvr = (nv + 31) / 32 * 32;
+  const size_t stage_words = 2 * (32 * (size_t)nvr + 32), u_words = im::Stair<16>{pad}.words();
+  const size_t lds_bytes = sizeof(float) * ((u_words > stage_words ? u_words : stage_words) + pad + 16 * 16 + 16);
+  if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
+  auto fn = nvr == 128 ? im::jtdj_factor_solve_kernel<128> : im::jtdj_factor_solve_kernel<0>;
+  if (lds_bytes > 64 * 1024)
+    IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, Mdense, J, njmax, D, state, nefc, quad,
+                     H, nv, nv_pad, y, ldy, U, x, ldx, pad);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

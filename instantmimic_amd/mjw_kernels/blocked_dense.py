@@ -229,3 +229,37 @@ def dense_hessian(M_dense, J, D, state, nefc, H, *, quad: int = QUADRATIC) -> No
             int(nworld), int(torch.cuda.current_stream(J.device).cuda_stream),
         )  # fmt: skip
     _lib.check(status, "im_jtdj_mfma")
+
+
+def dense_hessian_factor_solve(M_dense, J, D, state, nefc, H, y, x, *, factor=None, quad: int = QUADRATIC) -> None:
+    """:func:`dense_hessian` and the blocked Cholesky (16 x 16 tiles) with its solve in one launch:
+    ``H`` (nworld, nv_pad, nv_pad) or None, ``x = H^-1 y`` (nworld, nv), ``factor`` (nworld, pad,
+    pad) with ``pad`` = nv rounded up to 16, or None.  Bit for bit what :func:`dense_hessian`
+    followed by :func:`_blocked_dense_factor_solve` on the whole H gives."""
+    import torch
+
+    nworld, njmax, nv = J.shape
+    pad = -(-nv // 16) * 16
+    for t in (M_dense, J, D, state, y, x):
+        if not t.is_cuda or t.device != J.device:
+            raise ValueError("dense_hessian_factor_solve needs CUDA tensors on one device")
+    for t in (M_dense, J, D, state):
+        if not t.is_contiguous():
+            raise ValueError("M_dense, J, D and state must be contiguous")
+    if njmax < 1 or tuple(D.shape) != (nworld, njmax) or tuple(state.shape) != (nworld, njmax) or M_dense.numel() != nworld * nv * nv:
+        raise ValueError("D and state must be (nworld, njmax >= 1) and M_dense (nworld, nv, nv)")
+    if H is not None and (not H.is_contiguous() or H.dim() != 3 or H.shape[0] != nworld or H.shape[1] != H.shape[2] or H.shape[1] < nv):
+        raise ValueError("H must be a contiguous (nworld, nv_pad, nv_pad) tensor")
+    y2, x2 = y.reshape(nworld, -1), x.reshape(nworld, -1)
+    if y2.shape[1] < nv or x2.shape[1] < nv or y2.stride(1) != 1 or x2.stride(1) != 1 or y.dtype != torch.float32 or x.dtype != torch.float32:
+        raise ValueError("y and x must be float32 (nworld, >= nv) tensors with contiguous rows")
+    if factor is not None and (not factor.is_contiguous() or tuple(factor.shape) != (nworld, pad, pad) or factor.dtype != torch.float32):
+        raise ValueError(f"factor must be a contiguous float32 (nworld, {pad}, {pad}) tensor")
+    with torch.cuda.device(J.device):
+        status = _lib.lib().im_jtdj_factor_solve(
+            M_dense.data_ptr(), J.data_ptr(), int(njmax), D.data_ptr(), state.data_ptr(),
+            nefc.data_ptr() if nefc is not None else None, int(quad), None if H is None else H.data_ptr(), int(nv),
+            0 if H is None else int(H.shape[1]), y2.data_ptr(), y2.stride(0), None if factor is None else factor.data_ptr(),
+            pad, x2.data_ptr(), x2.stride(0), int(nworld), _stream(J),
+        )  # fmt: skip
+    _lib.check(status, "im_jtdj_factor_solve")

@@ -213,6 +213,10 @@ def run(launches: int = 32, only: str | None = None) -> None:
         Xb = torch.zeros_like(Y)
         sec = _timeit(torch, lambda i: BD._blocked_dense_factor_solve(d, Hc, Xb, Y, bs), 1, 8)
         _line("im_blocked_factor_solve B=16", wl, sec, bytes_=nworld * 4 * (nv * nv + 2 * nv + bs.pad * bs.pad), nworld=nworld)
+        Uf, xf = torch.zeros((nworld, bs.pad, bs.pad), device=dev), torch.zeros((nworld, nv), device=dev)
+        sec = _timeit(torch, lambda i: BD.dense_hessian_factor_solve(Md, J, D, st, ne, H, g, xf, factor=Uf), 1, 8)
+        _line("im_jtdj_factor_solve (J'DJ + blocked factor + solve in one launch)", wl, sec,
+              bytes_=nworld * 4 * (nv * nv + nefc * nv + 2 * nefc + pad * pad + bs.pad * bs.pad + 2 * nv), nworld=nworld)  # fmt: skip
         rng = np.random.default_rng(2)
         k = nefc // 10
         ids = np.zeros((nworld, nefc), np.int32)

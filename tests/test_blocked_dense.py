@@ -260,3 +260,39 @@ def test_gpu_short_pivot_forms_equal_sqrtf_and_the_division(device):
     assert _lib.lib().im_check_pivot_sqrt(0, 0x7F800000, count.data_ptr(), stream) == _lib.IM_OK
     torch.cuda.synchronize()
     assert int(count.item()) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,nworld", [("stress", 40), ("g1", 70), ("humanoid", 50), ("snu", 33), ("ant", 9)])
+def test_gpu_hessian_factor_solve_in_one_launch(device, name, nworld):
+    """im_jtdj_factor_solve against im_jtdj_mfma followed by im_blocked_factor_solve: H, the factor
+    and x bit for bit; x against the fp64 solve within what cond(H) allows."""
+    import torch
+
+    b, nv, Md = _dense_model(name, nworld)
+    pad16 = -(-nv // 16) * 16
+    nv_pad = ((nv + 1 + 15) // 16) * 16
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    M32, J, D, S, N, g = t(Md.reshape(nworld, -1).astype(np.float32)), t(b.J), t(b.D), t(b.state[0]), t(b.nefc), t(b.grad)
+    H1 = torch.zeros((nworld, nv_pad, nv_pad), device=device)
+    BD.dense_hessian(M32, J, D, S, N, H1)
+    Hc = H1[:, :nv, :nv].contiguous().reshape(nworld, -1)
+    m = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))])
+    d = SimpleNamespace(nworld=nworld, M=Hc)
+    scratch = BD.create_blocked_dense_factor_solve_scratch(m, d, device, block_size=16, minimum_nv=1)
+    x1 = torch.zeros((nworld, nv), device=device)
+    BD._blocked_dense_factor_solve(d, Hc, x1, g, scratch)
+    H2 = torch.full_like(H1, 0.0)
+    U2 = torch.full((nworld, pad16, pad16), float("nan"), device=device)
+    x2 = torch.full((nworld, nv), float("nan"), device=device)
+    BD.dense_hessian_factor_solve(M32, J, D, S, N, H2, g, x2, factor=U2)
+    x3 = torch.full((nworld, nv), float("nan"), device=device)
+    BD.dense_hessian_factor_solve(M32, J, D, S, N, None, g, x3)  # neither H nor the factor kept
+    torch.cuda.synchronize()
+    assert torch.equal(H1, H2)
+    assert torch.equal(scratch.U, U2)
+    assert torch.equal(x1, x2) and torch.equal(x1, x3)
+    H64 = H1[:, :nv, :nv].double().cpu().numpy()
+    x64 = np.linalg.solve(H64, b.grad.astype(np.float64)[:, :, None])[:, :, 0]
+    err = np.linalg.norm(x2.cpu().numpy() - x64, axis=1) / np.linalg.norm(x64, axis=1)
+    assert (err / (np.linalg.cond(H64) * 6e-8)).max() < 2.0
