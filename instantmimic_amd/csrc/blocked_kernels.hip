@@ -70,6 +70,130 @@ __device__ __forceinline__ void pivot_sqrt_rcp(float x, bool checked, float &d, 
   }
 }
 
+// a[jj] = fma(-lj, lj of lane jj, a[jj]) for the columns jj right of pivot column j, as v_fmac_f32 with the
+// broadcast on its first operand (one instruction per column; the compiler forms a move and a
+// fused multiply-add).  A DPP operand must not be read within two cycles of the vector instruction
+// that wrote it, and the compiler does not look inside these blocks: each waits on entry (lj was
+// just computed) and on exit (the next pivot is read from a[j + 1] through DPP).  The first column
+// has a block of its own so that the rest can be scheduled into the pivot's square root.
+#define IM_TR(jj) "v_fmac_f32_dpp %[a" #jj "], %[lj], %[nl] row_newbcast:" #jj " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+#define IM_TO(jj) [a##jj] "+v"(a[jj])
+__device__ __forceinline__ void trailing_update16(float (&a)[16], float lj, int j) {
+  const float nl = -lj;
+  switch (j) {
+    case 0:
+      asm("s_nop 1\n\t" IM_TR(1) "s_nop 1" : IM_TO(1) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(2) IM_TR(3) IM_TR(4) IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) "s_nop 1" : IM_TO(2), IM_TO(3), IM_TO(4), IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 1:
+      asm("s_nop 1\n\t" IM_TR(2) "s_nop 1" : IM_TO(2) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(3) IM_TR(4) IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) "s_nop 1" : IM_TO(3), IM_TO(4), IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 2:
+      asm("s_nop 1\n\t" IM_TR(3) "s_nop 1" : IM_TO(3) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(4) IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) "s_nop 1" : IM_TO(4), IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 3:
+      asm("s_nop 1\n\t" IM_TR(4) "s_nop 1" : IM_TO(4) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) "s_nop 1" : IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(15) "s_nop 1" : IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 4:
+      asm("s_nop 1\n\t" IM_TR(5) "s_nop 1" : IM_TO(5) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 5:
+      asm("s_nop 1\n\t" IM_TR(6) "s_nop 1" : IM_TO(6) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 6:
+      asm("s_nop 1\n\t" IM_TR(7) "s_nop 1" : IM_TO(7) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 7:
+      asm("s_nop 1\n\t" IM_TR(8) "s_nop 1" : IM_TO(8) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 8:
+      asm("s_nop 1\n\t" IM_TR(9) "s_nop 1" : IM_TO(9) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 9:
+      asm("s_nop 1\n\t" IM_TR(10) "s_nop 1" : IM_TO(10) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 10:
+      asm("s_nop 1\n\t" IM_TR(11) "s_nop 1" : IM_TO(11) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 11:
+      asm("s_nop 1\n\t" IM_TR(12) "s_nop 1" : IM_TO(12) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 12:
+      asm("s_nop 1\n\t" IM_TR(13) "s_nop 1" : IM_TO(13) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 13:
+      asm("s_nop 1\n\t" IM_TR(14) "s_nop 1" : IM_TO(14) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(15) "s_nop 1" : IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    case 14:
+      asm("s_nop 1\n\t" IM_TR(15) "s_nop 1" : IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      break;
+    default: break;
+  }
+}
+#undef IM_TR
+#undef IM_TO
+
+// Cholesky of a B x B diagonal tile with the forward solve of the right-hand side riding along:
+// lane i of a row of DPP lanes holds row i of the tile in a[] and the row's right-hand side in s.
+// Column j's updates are applied to the columns to its right as soon as it is final
+// (right-looking), which gives every element the same fused multiply-adds in the same order
+// (q ascending) as the column-wise form  v = A[i][j]; for q < j: v = fma(-L[i][q], L[j][q], v)
+// while the next pivot waits for one of them only.  Nothing is stored inside the loop: column j of
+// the factor replaces a[j], lane j keeps the solved right-hand side entry and the pivot's
+// reciprocal.  FAST: the short forms of the square root and the reciprocal; lo / hi receive the
+// smallest and largest bit pattern among the pivots, for the caller to check against the range
+// the short forms are exact in (the check is off the chain from one pivot to the next that way).
+template <int B, bool FAST>
+__device__ __forceinline__ void diag_tile(float (&a)[B], float &s, int i, float &my_z, float &my_rinv, uint32_t &lo,
+                                          uint32_t &hi) {
+#pragma unroll
+  for (int j = 0; j < B; ++j) {
+    const float x = row_bcast(a[j], j);
+    float d, rinv;
+    if constexpr (FAST) {
+      const uint32_t bits = __builtin_bit_cast(uint32_t, x);
+      lo = bits < lo ? bits : lo;
+      hi = bits > hi ? bits : hi;
+      d = pivot_sqrt_fast(x);
+      rinv = pivot_rcp_fast(d);
+    } else {
+      d = sqrtf(x);
+      rinv = 1.0f / d;
+    }
+    const float lj = i == j ? d : a[j] * rinv;  // rows below the diagonal; unused above
+    const float z = row_bcast(s, j) * rinv;
+    my_z = i == j ? z : my_z;
+    my_rinv = i == j ? rinv : my_rinv;
+    s = fma_(-lj, z, s);  // meaningful for i > j
+    if constexpr (FAST && B == 16) {
+      trailing_update16(a, lj, j);
+    } else {
+#pragma unroll
+      for (int jj = j + 1; jj < B; ++jj) a[jj] = fma_(-lj, row_bcast(lj, jj), a[jj]);
+    }
+    a[j] = lj;
+  }
+}
+constexpr uint32_t kPivotBitsLo = 0x0F800000u;  // 2^-96
+constexpr uint32_t kPivotBitsHi = 0x7F800000u;  // +inf: negative numbers and NaNs lie above as unsigned patterns
+
 // The factor's LDS array: U is upper triangular, so the rows of block row t keep the columns from
 // t * B on and follow one another (a staircase by tiles: 46 KB at pad 144 where the square takes
 // 83 KB, which is what lets two workgroups share a CU there).  Diagonal tiles are held in full.
@@ -123,13 +247,14 @@ struct GatheredSrc {
   }
 };
 
-// Indexed gather of every tile on or above the diagonal into U (zeroed by the caller): ids >= nM
+// Indexed gather of every tile on or above the diagonal into U: ids >= nM
 // read as zero, padded diagonal entries get +1 (mjw_step_optimized.py:932-941).  A wavefront
-// takes every (number of wavefronts)-th tile and keeps eight tiles' loads in flight.
+// takes every (number of wavefronts)-th tile and keeps eight or nine tiles' loads in flight.
+// Every word of the staircase belongs to one of these tiles, so U needs no clearing first.
 template <int B>
 __device__ __forceinline__ void gather_tiles(const float *__restrict__ Mw, const int32_t *__restrict__ block_idx,
                                              int nM, int nv, int pad, float *U, int tid, int nt) {
-  constexpr int BB = B * B, PER = BB / 64 > 0 ? BB / 64 : 1, G = 8;
+  constexpr int BB = B * B, PER = BB / 64 > 0 ? BB / 64 : 1, G = B == 16 ? 9 : 8;  // 36 tiles at pad 128: one round for four wavefronts
   const int nblk = pad / B, lane = tid & 63, nwv = nt >> 6;
   int kb = 0, ib = 0;  // cursor over the upper tiles, row by row
   auto advance = [&](int n) {
@@ -175,7 +300,7 @@ __device__ __forceinline__ void gather_tiles(const float *__restrict__ Mw, const
 }
 
 // Left-looking upper Cholesky by block column with the forward solve of rhs fused into the
-// loop; U (the staircase of pad) and rhs (pad) in LDS, U zeroed by the caller.
+// loop; U (the staircase of pad) and rhs (pad) in LDS.
 template <int B, class Src>
 __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *rhs, float *L, int pad, int tid,
                                                int nt) {
@@ -244,27 +369,21 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
         U[S.in_band(kb, r, i0 + c)] = v;
       }
     }
-    // the right-hand side's share of the block row: the first B lanes of the last wavefront, which
-    // has the fewest tiles to update
-    const int lr = tid - (nt - 64);
-    if (lr >= 0 && lr < B) {
-      float s = rhs[k + lr];
-      for (int jb = 0; jb < kb; ++jb) {
-        const int j = jb * B;
+    // the right-hand side: every row below the block row that was finished last subtracts that
+    // block row's sum (a chain of B terms from zero); a row has seen the block rows above it in
+    // ascending order when its own turn comes
+    if (kb > 0)
+      for (int r = k + tid; r < pad; r += nt) {
         float sum = 0.0f;
 #pragma unroll
-        for (int t = 0; t < B; ++t) sum = fma_(U[S.in_band(jb, t, k + lr)], rhs[j + t], sum);
-        s = s - sum;
+        for (int t = 0; t < B; ++t) sum = fma_(U[S.in_band(kb - 1, t, r)], rhs[k - B + t], sum);
+        rhs[r] = rhs[r] - sum;
       }
-      rhs[k + lr] = s;
-    }
     __syncthreads();
     // Cholesky of the diagonal tile and the forward solve of the right-hand side: the first B
-    // lanes of wave 0, lane i holding row i in registers.  Column j's updates are applied to
-    // the columns to its right as soon as it is final (right-looking), which gives every
-    // element the same fused multiply-adds in the same order (q ascending) as the column-wise
-    // form  v = A[i][j]; for q < j: v = fma(-L[i][q], L[j][q], v)  while the next pivot waits
-    // for one of them only.  Values of other rows come through DPP row broadcasts.
+    // lanes of wave 0, lane i holding row i in registers; values of other rows come through DPP
+    // row broadcasts.  The short forms first; a pivot outside their range (not seen with a positive
+    // definite matrix of ordinary scale) repeats the tile with the library forms.
     if (tid < 64) {
       const int i = tid;
       float a[B];
@@ -272,21 +391,13 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
       for (int j = 0; j < B; ++j) a[j] = U[S.in_band(kb, i < B ? i : 0, k + j)];
       float s = rhs[k + (i < B ? i : 0)];
       float my_z = 0.0f, my_rinv = 0.0f;
-      // nothing is stored inside the loop: a store's wait and the branch around it would sit in
-      // the chain from one pivot to the next.  Column j of the factor replaces a[j], lane j keeps
-      // the solved right-hand side entry and the pivot's reciprocal.
+      uint32_t lo = kPivotBitsLo, hi = kPivotBitsLo;
+      diag_tile<B, true>(a, s, i, my_z, my_rinv, lo, hi);
+      if (__builtin_expect(__any(i < B && (lo < kPivotBitsLo || hi >= kPivotBitsHi)), 0)) {
 #pragma unroll
-      for (int j = 0; j < B; ++j) {
-        float d, rinv;
-        pivot_sqrt_rcp(row_bcast(a[j], j), i < B, d, rinv);
-        const float lj = i == j ? d : a[j] * rinv;  // rows below the diagonal; unused above
-        const float z = row_bcast(s, j) * rinv;
-        my_z = i == j ? z : my_z;
-        my_rinv = i == j ? rinv : my_rinv;
-        s = fma_(-lj, z, s);  // meaningful for i > j
-#pragma unroll
-        for (int jj = j + 1; jj < B; ++jj) a[jj] = fma_(-lj, row_bcast(lj, jj), a[jj]);
-        a[j] = lj;
+        for (int j = 0; j < B; ++j) a[j] = U[S.in_band(kb, i < B ? i : 0, k + j)];
+        s = rhs[k + (i < B ? i : 0)];
+        diag_tile<B, false>(a, s, i, my_z, my_rinv, lo, hi);
       }
       if (i < B) {
 #pragma unroll
@@ -335,10 +446,18 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
   }
 }
 
-// rhs <- U^-1 rhs, block rows from the bottom.  The first B lanes of wave 0 hold one row of the
-// diagonal tile each; the solved entries travel through DPP row broadcasts.
+// rhs <- U^-1 rhs, block rows from the bottom.  Row r's value before its block's substitution is
+//   s = rhs[r]; for j = r's block + 1 .. last block: s = s - sum_j,  sum_j = U[r][block j] . x[block j]
+// with each sum_j a chain of B fused multiply-adds from zero.  The sums do not depend on s, so thread r
+// forms sum_j as soon as block j is solved (every row above it at once) and keeps it in a register; when
+// its own block's turn comes the subtractions run in ascending j as written above and the block's B lanes
+// (one row of 16 DPP lanes, or half of one) substitute with row broadcasts.  One dependent chain of B
+// terms per block row instead of one over all the columns to the right.
+// Needs a thread per row and at most kBackBlocks block rows; backward_solve_serial covers the rest.
+constexpr int kBackBlocks = 16;
+
 template <int B>
-__device__ __forceinline__ void backward_solve(const float *U, float *rhs, int pad, int tid) {
+__device__ __forceinline__ void backward_solve_serial(const float *U, float *rhs, int pad, int tid) {
   const Stair<B> S{pad};
   for (int i0 = pad - B; i0 >= 0; i0 -= B) {
     if (tid < 64) {
@@ -368,10 +487,58 @@ __device__ __forceinline__ void backward_solve(const float *U, float *rhs, int p
   }
 }
 
-// rhs <- U'^-1 rhs with a finished factor (the forward half of a solve-only step): the
-// same operations on rhs as inside factor_forward.
 template <int B>
-__device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pad, int tid) {
+__device__ __forceinline__ void backward_solve(const float *U, float *rhs, int pad, int tid, int nt) {
+  const int nblk = pad / B;
+  if (nblk > kBackBlocks || pad > nt) {  // uniform
+    backward_solve_serial<B>(U, rhs, pad, tid);
+    return;
+  }
+  const Stair<B> S{pad};
+  const bool has_row = tid < pad;
+  const int r = has_row ? tid : 0, b = r / B, ri = r - b * B;
+  const float *Ur = U + S.in_band(b, ri, 0);  // row r, indexed by column
+  float urow[B];
+#pragma unroll
+  for (int c = 0; c < B; ++c) urow[c] = Ur[b * B + c];
+  const float rinv = 1.0f / Ur[r];
+  float part[kBackBlocks];
+#pragma unroll
+  for (int jb = kBackBlocks - 1; jb >= 0; --jb) {
+    if (jb < nblk) {  // uniform
+      if (has_row && b == jb) {
+        float s = rhs[r];
+#pragma unroll
+        for (int j = jb + 1; j < kBackBlocks; ++j)
+          if (j < nblk) s = s - part[j];
+        constexpr int kRow = 16 / B;            // blocks per row of 16 DPP lanes
+        const int off = (jb % kRow) * B;        // where this block's lanes start in their DPP row
+        float my_x = 0.0f;
+#pragma unroll
+        for (int c = B - 1; c >= 0; --c) {
+          const float x = row_bcast(s * rinv, off + c);
+          my_x = ri == c ? x : my_x;
+          s = fma_(-urow[c], x, s);  // meaningful for rows above c
+        }
+        rhs[r] = my_x;
+      }
+      __syncthreads();
+      float sum = 0.0f;
+      if (has_row && b < jb) {
+#pragma unroll
+        for (int t = 0; t < B; ++t) sum = fma_(Ur[jb * B + t], rhs[jb * B + t], sum);
+      }
+      part[jb] = sum;
+    }
+  }
+}
+
+// rhs <- U'^-1 rhs with a finished factor (the forward half of a solve-only step): the same
+// operations on rhs as inside factor_forward.  Thread r keeps row r's value in a register; once a
+// block is solved every row below it subtracts that block's sum (a chain of B terms from zero),
+// blocks ascending.
+template <int B>
+__device__ __forceinline__ void forward_solve_serial(const float *U, float *rhs, int pad, int tid) {
   const Stair<B> S{pad};
   for (int k = 0; k < pad; k += B) {
     if (tid < 64) {
@@ -400,6 +567,53 @@ __device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pa
   }
 }
 
+template <int B>
+__device__ __forceinline__ void forward_solve(const float *U, float *rhs, int pad, int tid, int nt) {
+  if (pad > nt) {  // uniform
+    forward_solve_serial<B>(U, rhs, pad, tid);
+    return;
+  }
+  const Stair<B> S{pad};
+  const int nblk = pad / B;
+  const bool has_row = tid < pad;
+  const int r = has_row ? tid : 0, b = r / B, ri = r - b * B;
+  float ucol[B];
+#pragma unroll
+  for (int j = 0; j < B; ++j) ucol[j] = U[S.in_band(b, j, r)];
+  const float rinv = 1.0f / U[S.in_band(b, ri, r)];
+  float s = rhs[r];
+  for (int kb = 0; kb < nblk; ++kb) {
+    if (has_row && b == kb) {
+      constexpr int kRow = 16 / B;
+      const int off = (kb % kRow) * B;
+      float my_z = 0.0f;
+      if (off == 0) {
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+          const float z = row_bcast(s * rinv, j);
+          my_z = ri == j ? z : my_z;
+          s = fma_(-ucol[j], z, s);  // meaningful for rows below j
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+          const float z = row_bcast(s * rinv, (16 - B) % 16 + j);
+          my_z = ri == j ? z : my_z;
+          s = fma_(-ucol[j], z, s);
+        }
+      }
+      rhs[r] = my_z;
+    }
+    __syncthreads();
+    if (has_row && b > kb) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int t = 0; t < B; ++t) sum = fma_(U[S.in_band(kb, t, r)], rhs[kb * B + t], sum);
+      s = s - sum;
+    }
+  }
+}
+
 // Compiled for four wavefronts per SIMD (128 registers a lane): four workgroups of 256 share a CU
 // at pad 128, where the LDS admits them.
 template <int B>
@@ -416,14 +630,12 @@ __global__ __launch_bounds__(256, 4) void blocked_factor_solve_kernel(
   float *L = rhs + pad;       // [B * B + B] Cholesky factor of the diagonal block (column j in row j), 1 / pivots
   const int tid = threadIdx.x, nt = blockDim.x;
   const int64_t w = blockIdx.x;
-  for (int i = tid; i < nU; i += nt) U[i] = 0.0f;
   for (int i = tid; i < pad; i += nt) rhs[i] = (y && i < nv) ? y[w * ldy + i] : 0.0f;  // factor only: no y, no x
-  __syncthreads();
   gather_tiles<B>(M + w * ldM, block_idx, nM, nv, pad, U, tid, nt);
   __syncthreads();
   const GatheredSrc<B> src{U, pad};
   factor_forward<B>(src, U, rhs, L, pad, tid, nt);
-  backward_solve<B>(U, rhs, pad, tid);
+  backward_solve<B>(U, rhs, pad, tid, nt);
   if (x)
     for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
   if (Uout)
@@ -924,9 +1136,9 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
       }
     }
     __syncthreads();
-    forward_solve<B>(U, rhs, pad, tid);
+    forward_solve<B>(U, rhs, pad, tid, nt);
   }
-  backward_solve<B>(U, rhs, pad, tid);
+  backward_solve<B>(U, rhs, pad, tid, nt);
   if (tid < 64) {
     float s0 = 0.0f, s1 = 0.0f;
     for (int i = tid; i < nv; i += 64) {
@@ -1211,7 +1423,7 @@ __global__ __launch_bounds__(256, 4) void jtdj_factor_solve_kernel(
   __syncthreads();
   const LdsSrc<B> src{U, nv, pad};
   factor_forward<B>(src, U, rhs, L, pad, tid, nt);
-  backward_solve<B>(U, rhs, pad, tid);
+  backward_solve<B>(U, rhs, pad, tid, nt);
   if (x)
     for (int i = tid; i < nv; i += nt) x[w * ldx + i] = rhs[i];
   if (Uout)
