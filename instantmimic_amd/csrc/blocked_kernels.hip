@@ -40,30 +40,25 @@ __device__ __forceinline__ float row_bcast(float v, int n) {
   }
 }
 
-// Square root of a pivot and its reciprocal, IEEE-rounded, without what the compiler adds for
-// tiny, huge and special inputs: v_sqrt_f32 is one ulp off at most and the neighbour test picks
-// the rounded root; the reciprocal is the estimate plus one correction.  Both equal sqrtf(x) and
+// Square root of a pivot and the reciprocal of that root, IEEE-rounded, without what the compiler
+// adds for tiny, huge and special inputs, and in few dependent steps: the chain from one pivot to
+// the next bounds the factor.  With s = v_sqrt_f32(x) and y = v_rsq_f32(x) (both within an ulp),
+// d = fma(fma(-s, s, x), y / 2, s) is the rounded root (the exact residual times the root's
+// derivative); rinv is v_rcp_f32(d) plus one Newton step.  Both equal sqrtf(x) and
 // 1.0f / sqrtf(x) bit for bit for every x in [2^-96, inf) (checked over all such floats by
-// im_check_pivot_sqrt); other inputs take the library forms.  The chain from one pivot to the
-// next is less than half as long this way, and that chain bounds the factor.
+// im_check_pivot_sqrt; a reciprocal seeded from y or from 1 / s instead is one ulp off for a
+// few hundred of them); other inputs take the library forms.
 __device__ __forceinline__ bool pivot_in_range(float x) { return x >= 0x1p-96f && x < __builtin_inff(); }
-__device__ __forceinline__ float pivot_sqrt_fast(float x) {
+__device__ __forceinline__ void pivot_sqrt_rcp_fast(float x, float &d, float &rinv) {
   const float s = __builtin_amdgcn_sqrtf(x);
-  const float below = __builtin_bit_cast(float, __builtin_bit_cast(int, s) - 1);
-  const float above = __builtin_bit_cast(float, __builtin_bit_cast(int, s) + 1);
-  const float eb = fma_(-below, s, x), ea = fma_(-above, s, x);
-  float r = eb <= 0.0f ? below : s;
-  r = ea > 0.0f ? above : r;
-  return r;
-}
-__device__ __forceinline__ float pivot_rcp_fast(float d) {
+  const float y = __builtin_amdgcn_rsqf(x);
+  d = fma_(fma_(-s, s, x), 0.5f * y, s);
   const float r = __builtin_amdgcn_rcpf(d);
-  return fma_(fma_(-d, r, 1.0f), r, r);
+  rinv = fma_(fma_(-d, r, 1.0f), r, r);
 }
 // d = sqrtf(x), rinv = 1.0f / d; `checked`: the lanes whose x is a pivot (the others may hold anything)
 __device__ __forceinline__ void pivot_sqrt_rcp(float x, bool checked, float &d, float &rinv) {
-  d = pivot_sqrt_fast(x);
-  rinv = pivot_rcp_fast(d);
+  pivot_sqrt_rcp_fast(x, d, rinv);
   if (__builtin_expect(__any(checked && !pivot_in_range(x)), 0)) {
     d = sqrtf(x);
     rinv = 1.0f / d;
@@ -71,78 +66,77 @@ __device__ __forceinline__ void pivot_sqrt_rcp(float x, bool checked, float &d, 
 }
 
 // a[jj] = fma(-lj, lj of lane jj, a[jj]) for the columns jj right of pivot column j, as v_fmac_f32 with the
-// broadcast on its first operand (one instruction per column; the compiler forms a move and a
+// broadcast on its first operand and the sign on its second (one instruction per column; the compiler forms a move and a
 // fused multiply-add).  A DPP operand must not be read within two cycles of the vector instruction
 // that wrote it, and the compiler does not look inside these blocks: each waits on entry (lj was
 // just computed) and on exit (the next pivot is read from a[j + 1] through DPP).  The first column
 // has a block of its own so that the rest can be scheduled into the pivot's square root.
-#define IM_TR(jj) "v_fmac_f32_dpp %[a" #jj "], %[lj], %[nl] row_newbcast:" #jj " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+#define IM_TR(jj) "v_fmac_f32_dpp %[a" #jj "], %[lj], -%[lj] row_newbcast:" #jj " row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
 #define IM_TO(jj) [a##jj] "+v"(a[jj])
 __device__ __forceinline__ void trailing_update16(float (&a)[16], float lj, int j) {
-  const float nl = -lj;
   switch (j) {
     case 0:
-      asm("s_nop 1\n\t" IM_TR(1) "s_nop 1" : IM_TO(1) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(2) IM_TR(3) IM_TR(4) IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) "s_nop 1" : IM_TO(2), IM_TO(3), IM_TO(4), IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(1) "s_nop 1" : IM_TO(1) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(2) IM_TR(3) IM_TR(4) IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) "s_nop 1" : IM_TO(2), IM_TO(3), IM_TO(4), IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 1:
-      asm("s_nop 1\n\t" IM_TR(2) "s_nop 1" : IM_TO(2) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(3) IM_TR(4) IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) "s_nop 1" : IM_TO(3), IM_TO(4), IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(2) "s_nop 1" : IM_TO(2) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(3) IM_TR(4) IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) "s_nop 1" : IM_TO(3), IM_TO(4), IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 2:
-      asm("s_nop 1\n\t" IM_TR(3) "s_nop 1" : IM_TO(3) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(4) IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) "s_nop 1" : IM_TO(4), IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(3) "s_nop 1" : IM_TO(3) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(4) IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) "s_nop 1" : IM_TO(4), IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 3:
-      asm("s_nop 1\n\t" IM_TR(4) "s_nop 1" : IM_TO(4) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) "s_nop 1" : IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(15) "s_nop 1" : IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(4) "s_nop 1" : IM_TO(4) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(5) IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) "s_nop 1" : IM_TO(5), IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(15) "s_nop 1" : IM_TO(15) : [lj] "v"(lj));
       break;
     case 4:
-      asm("s_nop 1\n\t" IM_TR(5) "s_nop 1" : IM_TO(5) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(5) "s_nop 1" : IM_TO(5) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(6) IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(6), IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 5:
-      asm("s_nop 1\n\t" IM_TR(6) "s_nop 1" : IM_TO(6) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(6) "s_nop 1" : IM_TO(6) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(7) IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(7), IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 6:
-      asm("s_nop 1\n\t" IM_TR(7) "s_nop 1" : IM_TO(7) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(7) "s_nop 1" : IM_TO(7) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(8) IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(8), IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 7:
-      asm("s_nop 1\n\t" IM_TR(8) "s_nop 1" : IM_TO(8) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(8) "s_nop 1" : IM_TO(8) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(9) IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(9), IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 8:
-      asm("s_nop 1\n\t" IM_TR(9) "s_nop 1" : IM_TO(9) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(9) "s_nop 1" : IM_TO(9) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(10) IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(10), IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 9:
-      asm("s_nop 1\n\t" IM_TR(10) "s_nop 1" : IM_TO(10) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(10) "s_nop 1" : IM_TO(10) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(11) IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(11), IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 10:
-      asm("s_nop 1\n\t" IM_TR(11) "s_nop 1" : IM_TO(11) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(11) "s_nop 1" : IM_TO(11) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(12) IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(12), IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 11:
-      asm("s_nop 1\n\t" IM_TR(12) "s_nop 1" : IM_TO(12) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(12) "s_nop 1" : IM_TO(12) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(13) IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(13), IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 12:
-      asm("s_nop 1\n\t" IM_TR(13) "s_nop 1" : IM_TO(13) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(14), IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(13) "s_nop 1" : IM_TO(13) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(14) IM_TR(15) "s_nop 1" : IM_TO(14), IM_TO(15) : [lj] "v"(lj));
       break;
     case 13:
-      asm("s_nop 1\n\t" IM_TR(14) "s_nop 1" : IM_TO(14) : [lj] "v"(lj), [nl] "v"(nl));
-      asm("s_nop 1\n\t" IM_TR(15) "s_nop 1" : IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(14) "s_nop 1" : IM_TO(14) : [lj] "v"(lj));
+      asm("s_nop 1\n\t" IM_TR(15) "s_nop 1" : IM_TO(15) : [lj] "v"(lj));
       break;
     case 14:
-      asm("s_nop 1\n\t" IM_TR(15) "s_nop 1" : IM_TO(15) : [lj] "v"(lj), [nl] "v"(nl));
+      asm("s_nop 1\n\t" IM_TR(15) "s_nop 1" : IM_TO(15) : [lj] "v"(lj));
       break;
     default: break;
   }
@@ -171,13 +165,14 @@ __device__ __forceinline__ void diag_tile(float (&a)[B], float &s, int i, float 
       const uint32_t bits = __builtin_bit_cast(uint32_t, x);
       lo = bits < lo ? bits : lo;
       hi = bits > hi ? bits : hi;
-      d = pivot_sqrt_fast(x);
-      rinv = pivot_rcp_fast(d);
+      pivot_sqrt_rcp_fast(x, d, rinv);
     } else {
       d = sqrtf(x);
       rinv = 1.0f / d;
     }
-    const float lj = i == j ? d : a[j] * rinv;  // rows below the diagonal; unused above
+    // rows below the diagonal; the pivot's own lane gets d further down, and what it and the lanes
+    // above it compute in the meantime is never read
+    const float lj = a[j] * rinv;
     const float z = row_bcast(s, j) * rinv;
     my_z = i == j ? z : my_z;
     my_rinv = i == j ? rinv : my_rinv;
@@ -188,7 +183,7 @@ __device__ __forceinline__ void diag_tile(float (&a)[B], float &s, int i, float 
 #pragma unroll
       for (int jj = j + 1; jj < B; ++jj) a[jj] = fma_(-lj, row_bcast(lj, jj), a[jj]);
     }
-    a[j] = lj;
+    a[j] = i == j ? d : lj;
   }
 }
 constexpr uint32_t kPivotBitsLo = 0x0F800000u;  // 2^-96
@@ -325,9 +320,30 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
         f32x4 v;
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = src.load(kb, ib, (4 * kq + i) * B + p, 4 * kq + i, p);
-        // two finished block rows at a time: their sums are independent chains on the matrix
-        // cores; they are subtracted in the block rows' order
+        // four (then two) finished block rows at a time: their sums are independent chains on the
+        // matrix cores, fed by loads that are all in flight at once; they are subtracted in the
+        // block rows' order
         int jb = 0;
+        for (; jb + 3 < kb; jb += 4) {
+          f32x4 sum[4];
+          float a[4][4], b[4][4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            sum[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4) {
+              const int at = S.in_band(jb + u, 4 * s4 + kq, p);
+              a[u][s4] = U[at + k];
+              b[u][s4] = U[at + i0];
+            }
+          }
+#pragma unroll
+          for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) sum[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u][s4], b[u][s4], sum[u], 0, 0, 0);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = (((v[i] - sum[0][i]) - sum[1][i]) - sum[2][i]) - sum[3][i];
+        }
         for (; jb + 1 < kb; jb += 2) {
           f32x4 sum0 = {0.0f, 0.0f, 0.0f, 0.0f}, sum1 = sum0;
 #pragma unroll
@@ -892,11 +908,16 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
     int32_t *__restrict__ uni_, float *__restrict__ search, int64_t lds_, float *__restrict__ search_dot,
     float *__restrict__ decrement, int nv, int pad, int row_cap) {
   extern __shared__ float lds[];
-  const Stair<B> S{pad};
+  // The factor proper covers the dofs rounded up to whole tiles (pf); the rows and columns from
+  // there to pad are the identity with the augmented column and the corner in the last place,
+  // which are written out directly: at nv = 128 the array in LDS is that of eight block rows, not
+  // nine, and four worlds share a CU.
+  const int pf = (nv + B - 1) / B * B;
+  const Stair<B> S{pf};
   const int nU = S.words();
   float *U = lds;             // [nU] the factor, block row by block row
-  float *rhs = U + nU;        // [pad]
-  float *L = rhs + pad;       // [B * B + B]: factor of the diagonal tile (column j in row j), 1 / pivots
+  float *rhs = U + nU;        // [pf]
+  float *L = rhs + pf;        // [B * B + B]: factor of the diagonal tile (column j in row j), 1 / pivots
   int *ul = (int *)(L + B * B + B);  // [nv] union list, [nv] = its length
   unsigned *mkl = (unsigned *)(ul + nv + 1);  // [nv] per dof: nonzero when a changed row reaches it
   float *jr = (float *)(mkl + nv);  // [row_cap] signed weights of a batch of changed rows, [row_cap] their numbers
@@ -908,7 +929,7 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
   const int32_t *sw = state + w * njmax, *idw = ids + w * ld_ids;
   int count = changes[w];
   count = count < ld_ids ? count : ld_ids;
-  for (int i = tid; i < pad; i += nt) rhs[i] = i < nv ? gw[i] : 0.0f;
+  for (int i = tid; i < pf; i += nt) rhs[i] = i < nv ? gw[i] : 0.0f;
   if (count > 0) {
     // The changed rows of J and their signed weights pass through LDS in batches that use the
     // factor's array while it is still free (up to 64 rows each), the pair sums staying in the
@@ -1013,20 +1034,20 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
       }
       __syncthreads();  // the rows are done with the array; this workgroup's writes to H are read back below
       // 16 bytes per lane and four requests in flight; the tiles below the diagonal are not read
-      const int nvec = pad * pad / 4;  // pad is a multiple of 16
+      const int nvec = pf * pf / 4, last = (pf - 1) * (pad / 4) + pf / 4 - 1;  // pf is a multiple of 16
       for (int i0 = tid; i0 < nvec; i0 += 4 * nt) {
         float4 v[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           const int i = i0 + k * nt < nvec ? i0 + k * nt : nvec - 1;
-          const int r = 4 * i / pad, c = 4 * i - r * pad;
-          v[k] = ((const float4 *)Hw)[c >= r / B * B ? i : nvec - 1];
+          const int r = 4 * i / pf, c = 4 * i - r * pf;
+          v[k] = ((const float4 *)Hw)[c >= r / B * B ? r * (pad / 4) + c / 4 : last];
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           const int i = i0 + k * nt;
           if (i < nvec) {
-            const int r = 4 * i / pad, c = 4 * i - r * pad;
+            const int r = 4 * i / pf, c = 4 * i - r * pf;
             if (c >= r / B * B) {
               float4 o;
               o.x = (r < nv && c + 0 < nv && r <= c + 0) ? v[k].x : 0.0f;
@@ -1083,13 +1104,13 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
     }
     if (staged) {
       __syncthreads();
-      const LdsSrc<B> src{U, nv, pad};
-      factor_forward<B>(src, U, rhs, L, pad, tid, nt);
+      const LdsSrc<B> src{U, nv, pf};
+      factor_forward<B>(src, U, rhs, L, pf, tid, nt);
     } else {
       for (int i = tid; i < nU; i += nt) U[i] = 0.0f;
       __syncthreads();  // this workgroup's own writes to H are read back below
-      const DenseSrc<B> src{Hw, nv, pad};
-      factor_forward<B>(src, U, rhs, L, pad, tid, nt);
+      const DenseSrc<B> src{Hw, nv, pad};  // pad: the row stride of H in memory
+      factor_forward<B>(src, U, rhs, L, pf, tid, nt);
     }
     // stored factor: the augmented column z = U'^-1 grad above the corner sqrt(1e30 - z.z)
     if (tid < 64) {
@@ -1110,35 +1131,39 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
     for (int i = tid; i < pad * pad / 4; i += nt) {  // pad is a multiple of 16: a float4 stays in a row
       const int r = 4 * i / pad, c = 4 * i - r * pad;
       float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (c >= r / B * B) v = *(const float4 *)(U + S.at(r, c));
+      if (r < pf && c < pf) {
+        if (c >= r / B * B) v = *(const float4 *)(U + S.at(r, c));
+      } else if (r >= pf && r - c >= 0 && r - c < 4) {  // the identity below and right of the factor
+        v.x = r == c ? 1.0f : 0.0f, v.y = r == c + 1 ? 1.0f : 0.0f, v.z = r == c + 2 ? 1.0f : 0.0f, v.w = r == c + 3 ? 1.0f : 0.0f;
+      }
       if (c + 3 == pad - 1) v.w = r < nv ? rhs[r] : (r == pad - 1 ? L[0] : v.w);
       ((float4 *)Uw)[i] = v;
     }
     __syncthreads();  // rhs is overwritten by the backward solve
   } else {
-    const int nvec = pad * pad / 4;
+    const int nvec = pf * pf / 4, last = (pf - 1) * (pad / 4) + pf / 4 - 1;
     for (int i0 = tid; i0 < nvec; i0 += 4 * nt) {
       float4 v[4];
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const int i = i0 + k * nt < nvec ? i0 + k * nt : nvec - 1;
-        const int r = 4 * i / pad, c = 4 * i - r * pad;
-        v[k] = ((const float4 *)Uw)[c >= r / B * B ? i : nvec - 1];
+        const int r = 4 * i / pf, c = 4 * i - r * pf;
+        v[k] = ((const float4 *)Uw)[c >= r / B * B ? r * (pad / 4) + c / 4 : last];
       }
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const int i = i0 + k * nt;
         if (i < nvec) {
-          const int r = 4 * i / pad, c = 4 * i - r * pad;
+          const int r = 4 * i / pf, c = 4 * i - r * pf;
           if (c + 3 == pad - 1) v[k].w = r == pad - 1 ? 1.0f : 0.0f;  // drop the augmented column
           if (c >= r / B * B) *(float4 *)(U + S.at(r, c)) = v[k];
         }
       }
     }
     __syncthreads();
-    forward_solve<B>(U, rhs, pad, tid, nt);
+    forward_solve<B>(U, rhs, pf, tid, nt);
   }
-  backward_solve<B>(U, rhs, pad, tid, nt);
+  backward_solve<B>(U, rhs, pf, tid, nt);
   if (tid < 64) {
     float s0 = 0.0f, s1 = 0.0f;
     for (int i = tid; i < nv; i += 64) {
@@ -1443,9 +1468,11 @@ __global__ void check_pivot_sqrt_kernel(uint32_t first, uint32_t last, unsigned 
   for (uint64_t u = (uint64_t)first + blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; u <= last; u += stride) {
     const float x = __builtin_bit_cast(float, (uint32_t)u);
     if (!pivot_in_range(x)) continue;
-    const float d = pivot_sqrt_fast(x), want = sqrtf(x);
+    float d, rinv;
+    pivot_sqrt_rcp_fast(x, d, rinv);
+    const float want = sqrtf(x);
     bad += __builtin_bit_cast(uint32_t, d) != __builtin_bit_cast(uint32_t, want);
-    bad += __builtin_bit_cast(uint32_t, pivot_rcp_fast(want)) != __builtin_bit_cast(uint32_t, 1.0f / want);
+    bad += __builtin_bit_cast(uint32_t, rinv) != __builtin_bit_cast(uint32_t, 1.0f / want);
   }
   if (bad) atomicAdd(mismatches, bad);
 }
@@ -1671,12 +1698,12 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
   if (ldg < nv || ld_search < nv) return IM_ERR_STRIDE;
   if (((uintptr_t)H | (uintptr_t)U) & 15) return IM_ERR_STRIDE;  // read and written 16 bytes at a time
   constexpr int B = 16;
+  const int pf = (nv + B - 1) / B * B;  // the factor in LDS covers the dofs; the kernel writes the identity beyond them itself
   const size_t base_bytes =
-      sizeof(float) * ((size_t)im::Stair<B>{nv_pad}.words() + nv_pad + B * B + B +
-                       2 * (size_t)nv + 1);
+      sizeof(float) * ((size_t)im::Stair<B>{pf}.words() + pf + B * B + B + 2 * (size_t)nv + 1);
   if (base_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   // a batch of changed rows uses the factor's array: up to 64 rows, a multiple of four
-  int row_cap = (int)(im::Stair<B>{nv_pad}.words() / (size_t)nv) & ~3;
+  int row_cap = (int)(im::Stair<B>{pf}.words() / (size_t)nv) & ~3;
   row_cap = row_cap < 64 ? row_cap : 64;
   const size_t lds_bytes = base_bytes + sizeof(float) * 128;  // the batch's weights and row numbers behind the tables
   auto fn = im::dense_update_factor_kernel<B>;
