@@ -257,7 +257,8 @@ int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done,
  * (the reference runs the upstream assembly and its blocked factor as separate kernels around
  * src/instantmimic/utils/mjw_kernels/newton_stages.py:614-742).  H (nworld, nv_pad, nv_pad) is
  * written when not null (the per-iteration stage updates it later), U (nworld, pad, pad) when not
- * null, x = H^-1 y when x and y are given.  pad = nv rounded up to 16.  Results equal those of
+ * null (tiles on and right of the block diagonal, as im_blocked_factor_solve), x = H^-1 y when x
+ * and y are given.  pad = nv rounded up to 16.  Results equal those of
  * the two entry points called one after the other, bit for bit.  nv <= 128. */
 int im_jtdj_factor_solve(const float *Mdense, const float *J, int njmax, const float *D, const int32_t *state,
                          const int32_t *nefc, int quad, float *H, int nv, int nv_pad, const float *y, int64_t ldy,
@@ -306,7 +307,8 @@ int im_sparse_dense_factor(const im_sparse_plan *plan, const uint8_t *done, cons
  * (H[w, row, col] += delta, row <= col, :700-701); with changed rows the augmented blocked
  * Cholesky of augmented_factor_solve_factory (:473-611) runs with 16 x 16 tiles: the
  * gradient rides as column nv_pad - 1, the corner is 1e30, U (nworld, nv_pad, nv_pad)
- * receives the factor including that column; without changed rows the stored U is solved
+ * receives the factor including that column (the 16 x 16 tiles on and right of the block diagonal;
+ * those below it are never written or read); without changed rows the stored U is solved
  * against.  Rows and columns >= nv of H count as the identity.  nv_pad = a multiple of 16
  * above nv (src/instantmimic/utils/mjw_model.py:30).  H and U must be 16-byte aligned
  * (IM_ERR_STRIDE otherwise). */
@@ -326,7 +328,10 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes,
  * block_idx is the (nblk, nblk, B, B)-ordered table of element ids into M[w, :] built
  * by create_blocked_dense_factor_solve_scratch (mjw_step_optimized.py:932-941); ids
  * >= nM read as zero; padded diagonal entries get +1.  U (nworld, pad, pad) receives the
- * factor (the reference's workspace; 16-byte aligned) or may be null.  block_size 8 or 16. */
+ * factor (the reference's workspace; 16-byte aligned) or may be null: the tiles on and right of
+ * the block diagonal are written, as by the reference's kernel (indexed_factor.py:115, 141); the
+ * tiles below it keep what the caller's buffer holds (zeros in the reference's scratch) and no
+ * entry point reads them.  block_size 8 or 16. */
 int im_blocked_factor_solve(const float *M, int64_t ldM, int nM, const int32_t *block_idx,
                             int block_size, int nv, int pad, const float *y, int64_t ldy,
                             float *U, float *x, int64_t ldx, int nworld, void *stream);

@@ -657,9 +657,9 @@ __global__ __launch_bounds__(256, 4) void blocked_factor_solve_kernel(
   if (Uout)
     for (int i = tid; i < pad * pad / 4; i += nt) {  // pad is a multiple of B >= 8: a float4 stays in a tile
       const int r = 4 * i / pad, c = 4 * i - r * pad;
-      float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (c >= r / B * B) v = *(const float4 *)(U + S.at(r, c));
-      ((float4 *)(Uout + w * (int64_t)pad * pad))[i] = v;
+      // the tiles below the block diagonal are left as the caller has them (the reference's kernel
+      // stores the tiles on and right of the diagonal only, indexed_factor.py:115, 141)
+      if (c >= r / B * B) ((float4 *)(Uout + w * (int64_t)pad * pad))[i] = *(const float4 *)(U + S.at(r, c));
     }
 }
 
@@ -885,9 +885,7 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
       float4 *dst = (float4 *)(Uout + w * (int64_t)pad * pad);
       for (int i4 = l; i4 < pad * pad / 4; i4 += 16) {
         const int row = 4 * i4 / pad, col = 4 * i4 - row * pad, bi = row / B, bj = col / B;
-        float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (bj >= bi) v = *(const float4 *)(tile(bi, bj) + (row % B) * B + (col % B));
-        dst[i4] = v;
+        if (bj >= bi) dst[i4] = *(const float4 *)(tile(bi, bj) + (row % B) * B + (col % B));  // lower tiles: not written
       }
     }
   }
@@ -1137,7 +1135,7 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
         v.x = r == c ? 1.0f : 0.0f, v.y = r == c + 1 ? 1.0f : 0.0f, v.z = r == c + 2 ? 1.0f : 0.0f, v.w = r == c + 3 ? 1.0f : 0.0f;
       }
       if (c + 3 == pad - 1) v.w = r < nv ? rhs[r] : (r == pad - 1 ? L[0] : v.w);
-      ((float4 *)Uw)[i] = v;
+      if (c >= r / B * B) ((float4 *)Uw)[i] = v;  // the tiles below the block diagonal are not written
     }
     __syncthreads();  // rhs is overwritten by the backward solve
   } else {
@@ -1317,10 +1315,24 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
         }
     mine = mine < MAXT ? mine : MAXT;
   }
+  // The accumulators start from M (accumulator layout of a 32x32 tile: lane l holds column
+  // j = l % 32 and, in register 4 * g + v, row i = 8 * g + 4 * (l / 32) + v): every lane asks for
+  // all its elements at once, with clamped indices so that no load hangs on a condition, and the
+  // answers arrive while the first rows of J are staged.  Read at the end instead, behind the
+  // conditions of the stores, the same loads ran one after the other and took as long as the
+  // matrix-core loops.
+  const float *Mw = Mdense + w * (int64_t)nv * nv;
 #pragma unroll
-  for (int m = 0; m < MAXT; ++m)
+  for (int m = 0; m < MAXT; ++m) {
+    const int j = tbj[m] * 32 + (lane & 31), jc = j < nv ? j : nv - 1;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[m][v] = 0.0f;
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int i = tbi[m] * 32 + 8 * g + (lane >> 5) * 4 + v, ic = i < nv ? i : nv - 1;
+        acc[m][4 * g + v] = Mw[(int64_t)ic * nv + jc];
+      }
+  }
   int nefc = nefc_p ? nefc_p[w] : njmax;
   nefc = nefc < njmax ? nefc : njmax;
   const float *Jw = J + w * (int64_t)njmax * nv;
@@ -1379,9 +1391,6 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
     stage(r0 + 32, buf ^ 1);
     __syncthreads();
   }
-  // accumulator layout of a 32x32 tile: lane l holds column j = l % 32 and rows
-  // i = 8 * g + 4 * (l / 32) ... for register 4 * g + v: i = 8 * g + (l / 32) * 4 + v
-  const float *Mw = Mdense + w * (int64_t)nv * nv;
 #pragma unroll
   for (int m = 0; m < MAXT; ++m) {
     if (m >= mine) continue;
@@ -1391,7 +1400,7 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int i = tbi[m] * 32 + 8 * g + (lane >> 5) * 4 + v;
-        if (i < nv && j < nv && i <= j) out(i, j, Mw[(int64_t)i * nv + j] + acc[m][4 * g + v]);
+        if (i < nv && j < nv && i <= j) out(i, j, acc[m][4 * g + v]);
       }
   }
 }
@@ -1454,9 +1463,9 @@ __global__ __launch_bounds__(256, 4) void jtdj_factor_solve_kernel(
   if (Uout)
     for (int i = tid; i < pad * pad / 4; i += nt) {
       const int r = 4 * i / pad, c = 4 * i - r * pad;
-      float4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (c >= r / B * B) v = *(const float4 *)(U + S.at(r, c));
-      ((float4 *)(Uout + w * (int64_t)pad * pad))[i] = v;
+      // the tiles below the block diagonal are left as the caller has them (the reference's kernel
+      // stores the tiles on and right of the diagonal only, indexed_factor.py:115, 141)
+      if (c >= r / B * B) ((float4 *)(Uout + w * (int64_t)pad * pad))[i] = *(const float4 *)(U + S.at(r, c));
     }
 }
 

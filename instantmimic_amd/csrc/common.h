@@ -44,7 +44,8 @@ struct im_tree_plan {
   std::vector<std::vector<int>> groups;  // dofs descending
   std::vector<int> trunk;                // ascending
   std::vector<int> elim;
-  int span = 0, dense_cost = 0, shared_bytes = 0, maxdepth = 0;
+  int span = 0, shared_bytes = 0, maxdepth = 0;
+  int64_t dense_cost = 0;  // size^3 / 3 summed over the trees: beyond 32 bits from 1861 dofs in one tree
   bool beats_dense = false;
   // device side
   bool device_ready = false;

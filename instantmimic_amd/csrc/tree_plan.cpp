@@ -141,7 +141,7 @@ void plan_for_groups(im_tree_plan *pl, const Tree &t, int groups) {
     pl->groups.push_back(nodes);
   }
   pl->dense_cost = 0;
-  for (int r : t.roots) pl->dense_cost += (t.size[r] * t.size[r] * t.size[r]) / 3;
+  for (int r : t.roots) pl->dense_cost += ((int64_t)t.size[r] * t.size[r] * t.size[r]) / 3;
 }
 
 int exchange_bytes(const im_tree_plan &pl, int groups) {
@@ -258,7 +258,7 @@ int im_tree_plan_get_info(const im_tree_plan *plan, im_tree_plan_info *info) {
   info->ngroups = int(plan->groups.size());
   info->ntrunk = int(plan->trunk.size());
   info->span = plan->span;
-  info->dense_cost = plan->dense_cost;
+  info->dense_cost = (int32_t)std::min<int64_t>(plan->dense_cost, INT32_MAX);  // saturates; beats_dense is decided on the full value
   info->shared_bytes = plan->shared_bytes;
   info->beats_dense = plan->beats_dense ? 1 : 0;
   info->max_depth = plan->maxdepth + 1;

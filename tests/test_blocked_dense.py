@@ -214,7 +214,13 @@ def test_gpu_blocked_multi_solve(device, name, B, nworld, nrhs):
     np.testing.assert_array_equal(reused.cpu().numpy(), got)
     np.testing.assert_array_equal(got[act == 0], 0.0)
     assert (factor.cpu().numpy()[act == 0] == 7.0).all()  # an inactive world's factor is not written either
-    np.testing.assert_array_equal(factor.cpu().numpy()[act == 1], reused_factor.cpu().numpy()[act == 1])
+    # the factor: the tiles on and right of the block diagonal; those below it keep the caller's values,
+    # as in the reference, whose kernel stores U_kk and U_ki for i > k only (indexed_factor.py:322, 360)
+    blk = np.arange(scratch.pad) // B
+    upper = blk[:, None] <= blk[None, :]
+    f, fr = factor.cpu().numpy()[act == 1], reused_factor.cpu().numpy()[act == 1]
+    np.testing.assert_array_equal(f[:, upper], fr[:, upper])
+    assert (f[:, ~upper] == 7.0).all() and (fr[:, ~upper] == 0.0).all()
     _, U_ref = R.blocked_factor_solve(M32, scratch.indices.cpu().numpy(), nv, scratch.pad, B, rhs[:, :, 0])
     np.testing.assert_array_equal(got, R.blocked_multi_solve(U_ref, nv, B, rhs, act))
     np.testing.assert_array_equal(single_x.cpu().numpy()[act == 1], got[act == 1, :, 0])
@@ -290,7 +296,10 @@ def test_gpu_hessian_factor_solve_in_one_launch(device, name, nworld):
     BD.dense_hessian_factor_solve(M32, J, D, S, N, None, g, x3)  # neither H nor the factor kept
     torch.cuda.synchronize()
     assert torch.equal(H1, H2)
-    assert torch.equal(scratch.U, U2)
+    # the factor's tiles on and right of the block diagonal; the others are not written
+    blk = torch.arange(pad16, device=device) // 16
+    upper = blk[:, None] <= blk[None, :]
+    assert torch.equal(scratch.U[:, upper], U2[:, upper]) and bool(torch.isnan(U2[:, ~upper]).all())
     assert torch.equal(x1, x2) and torch.equal(x1, x3)
     H64 = H1[:, :nv, :nv].double().cpu().numpy()
     x64 = np.linalg.solve(H64, b.grad.astype(np.float64)[:, :, None])[:, :, 0]
