@@ -471,18 +471,34 @@ def iteration(m, d, ctx, nsolving=None, *, stage=None) -> None:
               nsolving=nsolving)  # fmt: skip
 
 
-def run(m, d, ctx, nsolving, *, check_every: int = 4) -> int:
+def run(m, d, ctx, nsolving, *, check_every: int = 4, graph: bool = False) -> int:
     """The fused Newton solve with the reference's signature (newton_fusion.py:330-409): iterates
     until every world is done or ``m.opt.iterations`` is reached.  The reference keeps a world in
     one resident block for the whole loop; here an iteration is seven launches over all worlds
     (finished worlds drop out of each through ``ctx.done``), and the host reads ``nsolving`` every
-    ``check_every`` iterations to stop early.  Returns the number of iterations launched."""
+    ``check_every`` iterations to stop early.  ``graph``: the first iteration runs as plain
+    launches, the second is captured in a graph that the later ones replay (the arrays of ``d`` and
+    ``ctx`` must then stay where they are for the whole solve; they do when the caller does not
+    reallocate them), which takes the seven launches' host cost out of every iteration.  Returns the
+    number of iterations launched."""
+    import torch
+
     from . import newton_stages
 
     stage = newton_stages.factor_factory(int(m.nv), int(m.nv_pad), getattr(ctx, "sparse_hessian_plan", None))
+    limit = int(m.opt.iterations)
+    captured = None
     launched = 0
-    for it in range(int(m.opt.iterations)):
-        iteration(m, d, ctx, nsolving, stage=stage)
+    for it in range(limit):
+        if not graph or it == 0:
+            iteration(m, d, ctx, nsolving, stage=stage)
+        elif captured is None:
+            captured = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(captured):
+                iteration(m, d, ctx, nsolving, stage=stage)
+            captured.replay()  # capturing records the launches without running them
+        else:
+            captured.replay()
         launched += 1
         if check_every > 0 and (it + 1) % check_every == 0 and int(nsolving.item()) <= 0:
             break

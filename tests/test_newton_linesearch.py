@@ -303,9 +303,11 @@ def test_gpu_linesearch_and_constraints_bitwise(device):
 
 
 @pytest.mark.gpu
-def test_gpu_newton_run_against_the_oracle_chain(device):
+@pytest.mark.parametrize("graph", [False, True])
+def test_gpu_newton_run_against_the_oracle_chain(device, graph):
     """newton_fusion.run on 500 worlds against the oracle's pieces chained in the same order:
-    the same number of iterations per world and the same qacc, bit for bit."""
+    the same number of iterations per world and the same qacc, bit for bit; with plain launches
+    and with the iteration captured in a graph that is replayed between the host's checks."""
     import torch
 
     from instantmimic_amd.mjw_kernels import newton_fusion as NF
@@ -329,7 +331,8 @@ def test_gpu_newton_run_against_the_oracle_chain(device):
                           newton_dof_union=torch.zeros((nworld, p.nv + 1), dtype=torch.int32, device=device))  # fmt: skip
     nsolving = torch.full((1,), nworld, dtype=torch.int32, device=device)
     start = _cost64(p, s.qacc)
-    launched = NF.run(m, d, ctx, nsolving)
+    launched = NF.run(m, d, ctx, nsolving, graph=graph)
+    assert launched > 4  # the graph has been replayed, with the host's check in between
     torch.cuda.synchronize()
     for _ in range(launched):
         _oracle_iteration(p, s)
