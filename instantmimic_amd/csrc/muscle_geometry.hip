@@ -233,6 +233,55 @@ __global__ __launch_bounds__(256) void force_velocity_state_kernel(
   out_slope[w * ldo + m] = fv.include_active * active * unit * dmult / velocity_scale;
 }
 
+// The same per world in one workgroup: the world's waypoints, moment entries and velocities come
+// into LDS with coalesced loads (a lane of the kernel above walks a few 12-byte waypoints and a
+// few scattered entries of its own, a cache line per request), then every muscle reads LDS.  Same
+// operations in the same order, so the same bits.  nwords_wp / nentry: what is staged (the
+// arrays' row lengths).
+__global__ __launch_bounds__(256) void force_velocity_state_world_kernel(
+    const float *__restrict__ wp, int64_t ldw, int nwords_wp, const int32_t *__restrict__ waypoint_start,
+    const float *__restrict__ params, int ldpar, const float *__restrict__ rest,
+    const float *__restrict__ length_scale, const float *__restrict__ activation, int64_t lda,
+    const float *__restrict__ qvel, int64_t ldq, int nqvel, const float *__restrict__ moment, int64_t ldm, int nentry,
+    const int32_t *__restrict__ dof_offsets, const int32_t *__restrict__ dof_torque_idx, int root,
+    im_muscle_force_model model, im_muscle_force_velocity_model fv, int nmuscle, float *__restrict__ out_length,
+    float *__restrict__ out_activation, float *__restrict__ out_velocity, float *__restrict__ out_multiplier,
+    float *__restrict__ out_slope, int64_t ldo) {
+  extern __shared__ float fv_lds[];
+  float *row = fv_lds;            // [nwords_wp]
+  float *mom = row + nwords_wp;   // [nentry]
+  float *qv = mom + nentry;       // [nqvel]
+  const int64_t w = blockIdx.x;
+  const int tid = threadIdx.x, nt = blockDim.x;
+  for (int i = tid; i < nwords_wp; i += nt) row[i] = wp[w * ldw + i];
+  for (int i = tid; i < nentry; i += nt) mom[i] = moment[w * ldm + i];
+  for (int i = tid; i < nqvel; i += nt) qv[i] = qvel[w * ldq + i];
+  __syncthreads();
+  for (int m = tid; m < nmuscle; m += nt) {
+    float len = 0.0f;
+    for (int i = waypoint_start[m]; i < waypoint_start[m + 1] - 1; ++i)
+      len = len + length(sub(ld3(row + 3 * (i + 1)), ld3(row + 3 * i)));
+    float velocity = 0.0f;
+    for (int e = dof_offsets[m]; e < dof_offsets[m + 1]; ++e)
+      velocity = __builtin_fmaf(-mom[e], qv[dof_torque_idx[e] + root], velocity);
+    const float f0 = params[m * ldpar], lm0 = params[m * ldpar + 1], lt0 = params[m * ldpar + 2],
+                pen = params[m * ldpar + 3];
+    const float velocity_scale = fmaxf(length_scale[m] * fv.vmax, 1.0e-6f);
+    float mult, dmult;
+    force_velocity_curve(velocity / velocity_scale, fv.fvmax, &mult, &dmult);
+    float active = activation[w * lda + m];
+    if (fv.clamp_activation != 0.0f) active = fminf(fmaxf(active, 0.0f), 1.0f);
+    const float lm = len / fmaxf(rest[m], 1.0e-6f) - lt0;
+    const float ln = fminf(fmaxf(lm / fmaxf(lm0, 1.0e-6f), model.length_norm_min), model.length_norm_max);
+    const float unit = f0 * active_fl(ln, model.active) * cosf(pen) * model.force_scale;
+    out_length[w * ldo + m] = len;
+    out_activation[w * ldo + m] = active * mult;
+    out_velocity[w * ldo + m] = velocity;
+    out_multiplier[w * ldo + m] = mult;
+    out_slope[w * ldo + m] = fv.include_active * active * unit * dmult / velocity_scale;
+  }
+}
+
 __global__ __launch_bounds__(256) void force_kernel(
     const float *__restrict__ wp, int64_t ldw, const int32_t *__restrict__ seg_start,
     const int32_t *__restrict__ seg_offsets, const float *__restrict__ params, int ldpar,
@@ -686,6 +735,24 @@ extern "C" int im_muscle_force_velocity_state(
       !force_velocity_multiplier || !force_velocity_slope || ld_params < 4)
     return IM_ERR_ARG;
   if (ld_out < nmuscle || ld_activation < nmuscle) return IM_ERR_STRIDE;
+  // a world's rows of waypoints, moments and velocities staged in LDS when they fit (the rows'
+  // strides bound what the tables can address); IMHIP_MUSCLE_KERNEL=simple keeps the lane-per-muscle kernel
+  static const bool forced_off = [] {
+    const char *e = std::getenv("IMHIP_MUSCLE_KERNEL");
+    return e && std::strcmp(e, "simple") == 0;
+  }();
+  const int64_t staged_words = ld_waypoints + ld_moment + ld_qvel;
+  if (!forced_off && ld_waypoints > 0 && ld_moment > 0 && ld_qvel > 0 && staged_words * 4 <= 64 * 1024) {
+    const int threads = 256;  // measured at 284 muscles: 45 us; 192 threads (two even passes) 49 us, 320 (one pass) 52 us
+    hipLaunchKernelGGL(force_velocity_state_world_kernel, dim3((unsigned)nworld), dim3(threads), (size_t)staged_words * 4,
+                       (hipStream_t)stream, waypoints, ld_waypoints, (int)ld_waypoints, muscle_waypoint_start,
+                       muscle_params, ld_params, muscle_rest_length, force_velocity_length_scale, activation,
+                       ld_activation, qvel, ld_qvel, (int)ld_qvel, moment, ld_moment, (int)ld_moment, muscle_dof_offsets,
+                       muscle_dof_torque_idx, root_dof_count, *model, *fv, nmuscle, muscle_length, effective_activation,
+                       length_velocity, force_velocity_multiplier, force_velocity_slope, ld_out);
+    IM_HIP_CHECK(hipGetLastError());
+    return IM_OK;
+  }
   IM_FOR_WORLD_SLABS(nworld, w0, nw) {
     hipLaunchKernelGGL(force_velocity_state_kernel, grid2(nmuscle, nw), dim3(256), 0, (hipStream_t)stream,
                        waypoints + w0 * ld_waypoints, ld_waypoints, muscle_waypoint_start, muscle_params, ld_params,
