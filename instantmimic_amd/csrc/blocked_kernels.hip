@@ -320,30 +320,9 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
         f32x4 v;
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = src.load(kb, ib, (4 * kq + i) * B + p, 4 * kq + i, p);
-        // four (then two) finished block rows at a time: their sums are independent chains on the
-        // matrix cores, fed by loads that are all in flight at once; they are subtracted in the
-        // block rows' order
+        // two finished block rows at a time: their sums are independent chains on the matrix
+        // cores; they are subtracted in the block rows' order (four at a time measured the same)
         int jb = 0;
-        for (; jb + 3 < kb; jb += 4) {
-          f32x4 sum[4];
-          float a[4][4], b[4][4];
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            sum[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-            for (int s4 = 0; s4 < 4; ++s4) {
-              const int at = S.in_band(jb + u, 4 * s4 + kq, p);
-              a[u][s4] = U[at + k];
-              b[u][s4] = U[at + i0];
-            }
-          }
-#pragma unroll
-          for (int s4 = 0; s4 < 4; ++s4)
-#pragma unroll
-            for (int u = 0; u < 4; ++u) sum[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u][s4], b[u][s4], sum[u], 0, 0, 0);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) v[i] = (((v[i] - sum[0][i]) - sum[1][i]) - sum[2][i]) - sum[3][i];
-        }
         for (; jb + 1 < kb; jb += 2) {
           f32x4 sum0 = {0.0f, 0.0f, 0.0f, 0.0f}, sum1 = sum0;
 #pragma unroll
