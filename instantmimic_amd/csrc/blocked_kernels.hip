@@ -877,7 +877,7 @@ __global__ __launch_bounds__(64) void blocked_factor_solve_quad_kernel(
 // :614-742 (stage), :451-470 (hessian_step), :473-611 (augmented factor).  search = -x,
 // search_dot = x.x, decrement = grad.x (strided over 64 lanes, shuffle-down tree).
 template <int B>
-__global__ __launch_bounds__(256) void dense_update_factor_kernel(
+__global__ __launch_bounds__(256, 4) void dense_update_factor_kernel(
     const uint8_t *__restrict__ done, const int32_t *__restrict__ state_changes,
     const int32_t *__restrict__ changes, const int32_t *__restrict__ ids, int ld_ids,
     const float *__restrict__ J, int njmax, const float *__restrict__ D, const int32_t *__restrict__ state,
@@ -925,7 +925,7 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
       // other with a fused multiply-add each, rows ascending; a batch holds a multiple of four
       // rows, so the chain of a pair runs through the batches as through one list.
       typedef float f32x4 __attribute__((ext_vector_type(4)));
-      constexpr int HELD = 5;  // tiles a wavefront keeps sums for at a time; more tiles (36 over 4 wavefronts at nv 128) take another pass over the rows
+      constexpr int HELD = 9;  // tiles a wavefront keeps sums for at a time (36 over 4 wavefronts at nv 128: one pass over the rows); more tiles take another pass
       const int lane = tid & 63, p = lane & 15, kq = lane >> 4, wv = tid >> 6, nwv = nt >> 6;
       const int nb = (nv + 15) / 16, ntiles = nb * (nb + 1) / 2;
       for (int tile0 = 0; tile0 < ntiles; tile0 += HELD * nwv) {
@@ -991,23 +991,28 @@ __global__ __launch_bounds__(256) void dense_update_factor_kernel(
             }
           }
         }
-        // H's elements of all the held tiles are requested before the first sum is added
-        float hv[HELD][4];
+        // H's elements of up to five held tiles are requested before the first of their sums is added
+        // (all nine at once would take the registers that let four worlds share a CU)
+        constexpr int APPLY = 5;
 #pragma unroll
-        for (int h = 0; h < HELD; ++h)
+        for (int h0 = 0; h0 < HELD; h0 += APPLY) {
+          float hv[APPLY][4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int row = ra[h] - p + 4 * kq + i, col = ca[h];
-            const bool mine = ra[h] >= 0 && row <= col && col < nv && acc[h][i] != 0.0f;
-            hv[h][i] = mine ? Hw[(size_t)row * pad + col] : 0.0f;
-          }
+          for (int h = h0; h < h0 + APPLY && h < HELD; ++h)
 #pragma unroll
-        for (int h = 0; h < HELD; ++h)
+            for (int i = 0; i < 4; ++i) {
+              const int row = ra[h] - p + 4 * kq + i, col = ca[h];
+              const bool mine = ra[h] >= 0 && row <= col && col < nv && acc[h][i] != 0.0f;
+              hv[h - h0][i] = mine ? Hw[(size_t)row * pad + col] : 0.0f;
+            }
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int row = ra[h] - p + 4 * kq + i, col = ca[h];
-            if (ra[h] >= 0 && row <= col && col < nv && acc[h][i] != 0.0f) Hw[(size_t)row * pad + col] = hv[h][i] + acc[h][i];
-          }
+          for (int h = h0; h < h0 + APPLY && h < HELD; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int row = ra[h] - p + 4 * kq + i, col = ca[h];
+              if (ra[h] >= 0 && row <= col && col < nv && acc[h][i] != 0.0f) Hw[(size_t)row * pad + col] = hv[h - h0][i] + acc[h][i];
+            }
+        }
       }
       __syncthreads();  // the rows are done with the array; this workgroup's writes to H are read back below
       // 16 bytes per lane and four requests in flight; the tiles below the diagonal are not read
