@@ -928,6 +928,15 @@ __global__ __launch_bounds__(256, 4) void dense_update_factor_kernel(
       constexpr int HELD = 9;  // tiles a wavefront keeps sums for at a time (36 over 4 wavefronts at nv 128: one pass over the rows); more tiles take another pass
       const int lane = tid & 63, p = lane & 15, kq = lane >> 4, wv = tid >> 6, nwv = nt >> 6;
       const int nb = (nv + 15) / 16, ntiles = nb * (nb + 1) / 2;
+      // thread t asks for the number and the signed weight of changed row t once, at the start: a
+      // batch then finds them in registers instead of making two trips to memory of its own
+      const bool ids_held = count <= nt;
+      int my_row = 0;
+      float my_sd = 0.0f;
+      if (ids_held && tid < count) {
+        my_row = idw[tid];
+        my_sd = sw[my_row] == quad ? Dw[my_row] : -Dw[my_row];
+      }
       for (int tile0 = 0; tile0 < ntiles; tile0 += HELD * nwv) {
         f32x4 acc[HELD];
         int ra[HELD], ca[HELD];
@@ -946,12 +955,19 @@ __global__ __launch_bounds__(256, 4) void dense_update_factor_kernel(
           const int nrow = count - c0 < row_cap ? count - c0 : row_cap;
           __syncthreads();  // the batch before this one has been read by everyone
           // the batch's row numbers first, then every element of its rows is requested before the
-          // first one is stored: one trip to memory for the numbers and one for the rows
+          // first one is stored
           int *rowid = (int *)(sd + row_cap);
-          for (int t = tid; t < nrow; t += nt) {
-            const int r = idw[c0 + t];
-            rowid[t] = r;
-            sd[t] = sw[r] == quad ? Dw[r] : -Dw[r];
+          if (ids_held) {
+            if (tid >= c0 && tid < c0 + nrow) {
+              rowid[tid - c0] = my_row;
+              sd[tid - c0] = my_sd;
+            }
+          } else {
+            for (int t = tid; t < nrow; t += nt) {
+              const int r = idw[c0 + t];
+              rowid[t] = r;
+              sd[t] = sw[r] == quad ? Dw[r] : -Dw[r];
+            }
           }
           __syncthreads();
           const int total = nrow * nv;
