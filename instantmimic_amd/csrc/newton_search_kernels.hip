@@ -45,10 +45,10 @@ __device__ __forceinline__ Pt row_quad(bool friction, float D, float f, float ja
   if (x < 0.0f) return quad;
   return {0.0f, 0.0f, 0.0f};
 }
-// point of a row at alpha, cost relative to alpha 0
-__device__ __forceinline__ Pt row_point(bool friction, float D, float f, float jaref, float jv, float alpha) {
+// point of a row at alpha, cost relative to alpha 0, with the row's cost at alpha 0 computed beforehand (row_quad(..., jaref).c)
+__device__ __forceinline__ Pt row_point_from(bool friction, float D, float f, float jaref, float jv, float c0, float alpha) {
   Pt p = eval_pt(row_quad(friction, D, f, jaref, jv, jaref + alpha * jv), alpha);
-  p.c = p.c - row_quad(friction, D, f, jaref, jv, jaref).c;
+  p.c = p.c - c0;
   return p;
 }
 // point of a row at alpha 0 with its cost itself
@@ -58,10 +58,30 @@ __device__ __forceinline__ Pt row_point_zero(bool friction, float D, float f, fl
 }
 
 // sum over the 32 lanes of a world: shuffle-down tree, lane 0's value to all, then the +0 of the
-// later warps' empty partials (newton_stages.py:36-52)
+// later warps' empty partials (newton_stages.py:36-52).  The tree's first step crosses the two
+// rows of 16 lanes of a world (v_permlane16_swap_b32 hands every even row the odd row behind it),
+// the others stay inside a row (DPP shifts); what a lane receives from beyond its row or world
+// never reaches lane 0, whose sum has the association of the 32-lane shuffle-down tree.  Lane 0's
+// (lane 32's) value then goes to its world through a lane read.  A world's 32 lanes are active or
+// inactive together.
+template <int N>
+__device__ __forceinline__ float row_shl(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x100 + N, 0xF, 0xF, true));
+}
 __device__ __forceinline__ float lanes_sum(float s) {
-  for (int o = 16; o > 0; o >>= 1) s = s + __shfl_down(s, o, 32);
-  s = __shfl(s, 0, 32);
+  // v_permlane16_swap_b32 a, b: the odd rows of a change places with the even rows of b.  Written
+  // out, with its wait states: the compiler's builtin returns the first result twice when both
+  // operands hold the same value.
+  unsigned upper = __builtin_bit_cast(unsigned, s), lower = upper;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lower), "+v"(upper));
+  s = s + __builtin_bit_cast(float, upper);  // lane i of an even row: lane i + 16
+  s = s + row_shl<8>(s);
+  s = s + row_shl<4>(s);
+  s = s + row_shl<2>(s);
+  s = s + row_shl<1>(s);
+  const float first = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s), 0));
+  const float second = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s), 32));
+  s = (threadIdx.x & 32) ? second : first;
   return s + 0.0f;
 }
 __device__ __forceinline__ Pt lanes_sum(Pt p) { return {lanes_sum(p.c), lanes_sum(p.g), lanes_sum(p.h)}; }
@@ -79,7 +99,11 @@ struct SearchArgs {
   int overflow_bit, nv, njmax, ls_iterations, nworld;
 };
 
-// Two worlds per wavefront, 32 lanes each (the reference's reduction width).
+// Two worlds per wavefront, 32 lanes each (the reference's reduction width).  HELD: rows of the
+// world a lane keeps in registers (weight, friction loss, Jaref, jv and the cost at alpha 0) --
+// every candidate step evaluates every row, three candidates per round; 0: more rows than that,
+// read from memory at every evaluation.
+template <int HELD>
 __global__ __launch_bounds__(64) void newton_linesearch_kernel(SearchArgs a) {
   const int lane = threadIdx.x & 31;
   const int64_t w = (int64_t)blockIdx.x * 2 + (threadIdx.x >> 5);
@@ -108,13 +132,44 @@ __global__ __launch_bounds__(64) void newton_linesearch_kernel(SearchArgs a) {
     g2 = g2 + 0.5f * jv[r] * jvD;
   }
   const Pt gauss = {0.0f, lanes_sum(g1), lanes_sum(g2)};
+  // this lane's rows ne + lane, ne + lane + 32, ...
+  constexpr int NH = HELD > 0 ? HELD : 1;
+  float hd[NH], hf[NH], hja[NH], hv[NH], hc0[NH];
+  if constexpr (HELD > 0) {
+#pragma unroll
+    for (int k = 0; k < HELD; ++k) {
+      const int r = ne + lane + 32 * k, rc = r < nefc ? r : (nefc > 0 ? nefc - 1 : 0);
+      const bool in = r < nefc;
+      hd[k] = in ? D[rc] : 0.0f;
+      hf[k] = (in && fl) ? fl[rc] : 0.0f;
+      hja[k] = in ? Jaref[rc] : 0.0f;
+      hv[k] = in ? jv[rc] : 0.0f;
+      hc0[k] = row_quad(r < ne + nf, hd[k], hf[k], hja[k], hv[k], hja[k]).c;
+    }
+  }
+  // sum over this lane's rows of the rows' points at one or three step lengths
+  auto rows_sum = [&](auto point) {
+    if constexpr (HELD > 0) {
+#pragma unroll
+      for (int k = 0; k < HELD; ++k) {
+        const int r = ne + lane + 32 * k;
+        if (r < nefc) point(r < ne + nf, hd[k], hf[k], hja[k], hv[k], hc0[k]);
+      }
+    } else {
+      for (int r = ne + lane; r < nefc; r += 32) {
+        const bool fr = r < ne + nf;
+        const float d = D[r], f = fl ? fl[r] : 0.0f, ja = Jaref[r], v = jv[r];
+        point(fr, d, f, ja, v, row_quad(fr, d, f, ja, v, ja).c);
+      }
+    }
+  };
   auto rows_at = [&](float alpha) {
     Pt s = {0.0f, 0.0f, 0.0f};
-    for (int r = ne + lane; r < nefc; r += 32) s = s + row_point(r < ne + nf, D[r], fl ? fl[r] : 0.0f, Jaref[r], jv[r], alpha);
+    rows_sum([&](bool fr, float d, float f, float ja, float v, float c0) { s = s + row_point_from(fr, d, f, ja, v, c0, alpha); });
     return lanes_sum(s);
   };
   Pt z = {0.0f, 0.0f, 0.0f};
-  for (int r = ne + lane; r < nefc; r += 32) z = z + row_point_zero(r < ne + nf, D[r], fl ? fl[r] : 0.0f, Jaref[r], jv[r]);
+  rows_sum([&](bool fr, float d, float f, float ja, float v, float) { z = z + row_point_zero(fr, d, f, ja, v); });
   const Pt rows0 = lanes_sum(z);
   const Pt p0 = {gauss.c + rows0.c, gauss.g + rows0.g, 2.0f * gauss.h + rows0.h};
   const Pt p0_delta = {0.0f, p0.g, p0.h};
@@ -142,13 +197,11 @@ __global__ __launch_bounds__(64) void newton_linesearch_kernel(SearchArgs a) {
       const float hi_next_alpha = hi_alpha - safe_div(hi.g, hi.h);
       const float mid_alpha = 0.5f * (lo_alpha + hi_alpha);
       Pt s_lo = {0.0f, 0.0f, 0.0f}, s_hi = s_lo, s_mid = s_lo;
-      for (int r = ne + lane; r < nefc; r += 32) {
-        const bool fr = r < ne + nf;
-        const float d = D[r], f = fl ? fl[r] : 0.0f, ja = Jaref[r], v = jv[r];
-        s_lo = s_lo + row_point(fr, d, f, ja, v, lo_next_alpha);
-        s_hi = s_hi + row_point(fr, d, f, ja, v, hi_next_alpha);
-        s_mid = s_mid + row_point(fr, d, f, ja, v, mid_alpha);
-      }
+      rows_sum([&](bool fr, float d, float f, float ja, float v, float c0) {
+        s_lo = s_lo + row_point_from(fr, d, f, ja, v, c0, lo_next_alpha);
+        s_hi = s_hi + row_point_from(fr, d, f, ja, v, c0, hi_next_alpha);
+        s_mid = s_mid + row_point_from(fr, d, f, ja, v, c0, mid_alpha);
+      });
       const Pt lo_next = eval_pt(gauss, lo_next_alpha) + lanes_sum(s_lo);
       const Pt hi_next = eval_pt(gauss, hi_next_alpha) + lanes_sum(s_hi);
       const Pt mid = eval_pt(gauss, mid_alpha) + lanes_sum(s_mid);
@@ -290,7 +343,10 @@ extern "C" int im_newton_linesearch(const float *opt_tolerance, int ntolerance, 
                nefc, qfrc_smooth, efc_D, efc_frictionloss, Jaref, search, search_dot, mv, jv, efc_Ma, ld_smooth, ld_D,
                ld_frictionloss, ld_Jaref, ld_search, ld_mv, ld_jv, ld_Ma, done, alpha, improvement, ls_exhausted,
                overflow, overflow_bit, nv, njmax, ls_iterations, nworld};
-  hipLaunchKernelGGL(newton_linesearch_kernel, dim3((unsigned)((nworld + 1) / 2)), dim3(64), 0, (hipStream_t)stream, a);
+  // rows per lane: two up to 64 rows, four up to 128, eight up to 256
+  auto fn = njmax <= 64 ? newton_linesearch_kernel<2> : njmax <= 128 ? newton_linesearch_kernel<4>
+            : njmax <= 256 ? newton_linesearch_kernel<8> : newton_linesearch_kernel<0>;
+  hipLaunchKernelGGL(fn, dim3((unsigned)((nworld + 1) / 2)), dim3(64), 0, (hipStream_t)stream, a);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

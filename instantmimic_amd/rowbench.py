@@ -71,7 +71,7 @@ def _line(kernel, workload, seconds, *, bytes_=None, flops=None, nworld=None):
 
 
 def run(launches: int = 32, only: str | None = None) -> None:
-    """``only``: comma-separated section names out of trees, generated, stress, muscles, walks, iteration, bodies."""
+    """``only``: comma-separated section names out of trees, generated, stress, muscles, walks, iteration, implicit, bodies."""
     import torch
 
     from . import synth
@@ -385,6 +385,104 @@ def run(launches: int = 32, only: str | None = None) -> None:
               f"humanoid nv={nv} nefc={nefc} x {nworld} worlds", sec,
               bytes_=nworld * 4 * (3 * nefc * nv + nM + 8 * nefc + 12 * nv + 10), nworld=nworld)  # fmt: skip
 
+        # the line search on a consistent problem: search = -H^-1 grad of the first iteration, mv = M search and
+        # jv = J search from the library's own kernels, one-sided rows only; then the whole iteration of
+        # newton_fusion.iteration (eight launches: M search, J search, scalar search, step, constraints, gradient,
+        # fused tree solve, convergence test)
+        tables = [t(a) for a in NF.mul_m_tables(b.rowadr, b.rownnz, b.colind)]
+        M0, J0, D0, st0, _, ne0 = S[0]
+        qacc0 = 0.1 * f32(nworld, nv)
+        Ma0, jar0, sr0 = torch.zeros((nworld, nv), device=dev), torch.zeros((nworld, nefc), device=dev), torch.zeros((nworld, nv), device=dev)
+        NF.mul_m(M0, qacc0, Ma0, *tables)
+        NF.jv(J0, qacc0, jar0, nefc=ne0)
+        jar0 += 0.3 * f32(nworld, nefc)  # J qacc - aref
+        grad0 = t(b.grad)
+        T.assemble_tree_factor_solve(sc_tree, M0, J0, D0, st0, ne0, grad0, sr0, negate=True)
+        sdot0 = (sr0 * sr0).sum(1)
+        mv0, jv0 = torch.zeros((nworld, nv), device=dev), torch.zeros((nworld, nefc), device=dev)
+        NF.mul_m(M0, sr0, mv0, *tables)
+        NF.jv(J0, sr0, jv0, nefc=ne0)
+        smooth0 = Ma0 - grad0  # so that the unconstrained gradient is the batch's
+        ls_tol, tol8 = torch.full((1,), 0.01, device=dev), torch.full((1,), 1e-8, device=dev)
+        al, im_, ex = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev), torch.zeros(nworld, dtype=torch.uint8, device=dev)
+        ovf = torch.zeros(nworld, dtype=torch.int32, device=dev)
+        sec = _timeit(torch, lambda i: NF.linesearch(tol8, ls_tol, inertia, None, None, ne0, smooth0, D0, None, jar0, sr0, sdot0, mv0, jv0, Ma0, None,
+                                                     al, im_, ex, ls_iterations=50, overflow=ovf, overflow_bit=4), 1, launches)  # fmt: skip
+        _line("im_newton_linesearch (up to 50 rounds of three candidates)", f"humanoid nv={nv} nefc={nefc} x {nworld} worlds", sec,
+              bytes_=nworld * 4 * (4 * nefc + 5 * nv + 6), nworld=nworld)  # fmt: skip
+        frc, est = torch.zeros((nworld, nefc), device=dev), torch.zeros((nworld, nefc), dtype=torch.int32, device=dev)
+        sec = _timeit(torch, lambda i: NF.eval_constraints(jar0, D0, None, None, None, ne0, None, ex, frc, est, ids, qcnt, scnt), 1, launches)
+        _line("im_newton_eval_constraints", f"humanoid nv={nv} nefc={nefc} x {nworld} worlds", sec,
+              bytes_=nworld * 4 * (5 * nefc + 3), nworld=nworld)  # fmt: skip
+        mm = SimpleNamespace(nv=nv, nv_pad=(nv + 1 + 15) // 16 * 16, M_mulm_rowadr=tables[0], M_mulm_col=tables[1], M_mulm_madr=tables[2],
+                             opt=SimpleNamespace(tolerance=tol8, ls_tolerance=ls_tol, iterations=1 << 30, ls_iterations=50),
+                             stat=SimpleNamespace(meaninertia=inertia), block_dim=SimpleNamespace(linesearch_iterative=32))  # fmt: skip
+
+        def tree_stage(J_, D_, state_, ids_, qcnt_, scnt_, done_, grad_, h_, hfactor_, search_, sdot_, decr_, union_):
+            T.assemble_tree_factor_solve(sc_tree, M0, J_, D_, state_, ne0, grad_[:, :nv], search_, negate=True)
+
+        def whole(i):
+            M_, J_, D_, s0, _, ne_ = S[i]
+            dd = SimpleNamespace(nworld=nworld, M=M_, ne=None, nf=None, nefc=ne_, qfrc_smooth=smooth0, qacc=qacc0,
+                                 efc=SimpleNamespace(J=J_, D=D_, frictionloss=None, Ma=Ma0, force=frc, state=est),
+                                 qfrc_constraint=qc, solver_niter=nit, overflow=ovf)  # fmt: skip
+            cx = SimpleNamespace(search=sr0, search_dot=sdot0, mv=mv0, jv=jv0, Jaref=jar0, done=dn, alpha=al, improvement=im_,
+                                 ls_exhausted=ex, quad_changed_ids=ids, quad_changed_count=qcnt, state_changed_count=scnt,
+                                 search_unchanged=un, grad=gr, grad_dot=gd, grad_scale=gs, newton_decrement=de, h=None, hfactor=None,
+                                 newton_dof_union=None)  # fmt: skip
+            NF.iteration(mm, dd, cx, None, stage=tree_stage)
+
+        sec = _timeit(torch, whole, nsets, launches)
+        _line("newton_fusion.iteration: M search, J search, line search, step, constraints, gradient, fused tree solve, convergence test (eight launches)",
+              f"humanoid nv={nv} nefc={nefc} x {nworld} worlds", sec,
+              bytes_=nworld * 4 * (3 * nefc * nv + 2 * nM + 14 * nefc + 20 * nv + 16), nworld=nworld)  # fmt: skip
+
+    # ---- implicit-fast integrator matrix and its solve; the upstream-iteration sparse factor from the dense Hessian
+    if section("implicit"):
+        from .mjw_kernels import implicit_qh as IQ
+
+        nworld = 4096
+        m, d, st, _ = synth.make_implicit_case(nworld)
+        dd = SimpleNamespace(nworld=nworld, M=t(d.M), moment_rownnz=d.moment_rownnz, moment_rowadr=d.moment_rowadr, moment_colind=d.moment_colind,
+                             actuator_moment=t(d.actuator_moment), ten_J=t(d.ten_J), ctrl=t(d.ctrl), actuator_force=t(d.actuator_force),
+                             efc=SimpleNamespace(Ma=t(d.efc.Ma)))  # fmt: skip
+        scratch = IQ.create_implicit_qh_scratch(m, dd, dev)
+        nM, nmom, nten, nu = int(st[2].size), int(d.moment_colind.size), int(m.ten_J_colind.size), int(m.nactuator)
+        wl = f"snu + a free body nv={m.nv} nM={nM}, {nu} actuators ({nmom} moment entries), {m.ntendon} tendons ({nten} entries) x {nworld} worlds"
+        sec = _timeit(torch, lambda i: IQ.deriv_smooth_vel(m, dd, scratch.implicit_qderiv, scratch), 1, launches)
+        _line("qH = M - h dF/dv: im_implicit_qh_base, im_actuator_velocity_gain, two pair-sum gathers", wl, sec,
+              bytes_=nworld * 4 * (2 * nM + nmom + nten + 3 * nu), nworld=nworld)  # fmt: skip
+        scratch.tree_factor_solve = T.create_tree_factor_solve_scratch(m, dev)
+        sec = _timeit(torch, lambda i: IQ.implicit_factor_optimized(m, dd, scratch), 1, launches)
+        _line("implicit_factor_optimized: qH and the tree L'DL solve on it", wl, sec,
+              bytes_=nworld * 4 * (2 * nM + nmom + nten + 3 * nu + nM + 2 * m.nv), nworld=nworld)  # fmt: skip
+        del dd, scratch
+        torch.cuda.empty_cache()
+        # non-fused sparse factor on a model the fused loop does not take (84 dofs), H = M + J'DJ from the dense assembly
+        parents = tuple(synth.limbs_parents(6, 13))
+        model = synth.model_from_parents(parents)
+        b = synth.make_batch(synth.Shape("limbs84", parents, 48, nworld, (0.5, 8.0), 0.02, (-3.0, 3.0), 0.6, 2, 11), nworld)
+        nv = model.nv
+        plan, reason = SH.plan_for_model(model, SimpleNamespace(hfactor=np.zeros((1, model.nv_pad, model.nv_pad), np.float32)), [], 64, device=dev)
+        if plan is not None and plan.path == "nonfused":
+            Md = t(synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32).reshape(nworld, -1))
+            H = torch.zeros((nworld, model.nv_pad, model.nv_pad), device=dev)
+            BD.dense_hessian(Md, t(b.J), t(b.D), t(b.state[0]), t(b.nefc), H)
+            hf = torch.zeros_like(H)
+            g3, s3 = t(b.grad).reshape(nworld, nv, 1), torch.zeros((nworld, nv, 1), device=dev)
+            sd, de = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev)
+            refactor = SH.nonfused_kernel(plan, False, False)
+            sec = _timeit(torch, lambda i: refactor(None, g3, H, None, None, hf, s3, sd, de), 1, launches)
+            used = plan.nfac + nv
+            _line("im_sparse_dense_factor (refactor from the dense H)", f"limbs84 nv={nv} nfac={plan.nfac} x {nworld} worlds", sec,
+                  bytes_=nworld * 4 * (2 * used + 2 * nv + 2), nworld=nworld)  # fmt: skip
+            zero = torch.zeros(nworld, dtype=torch.int32, device=dev)
+            one = torch.ones(nworld, dtype=torch.int32, device=dev)
+            solve_only = SH.nonfused_kernel(plan, True, True)
+            sec = _timeit(torch, lambda i: solve_only(None, g3, H, zero, one, hf, s3, sd, de), 1, launches)
+            _line("im_sparse_dense_factor (solve with the stored factor)", f"limbs84 nv={nv} nfac={plan.nfac} x {nworld} worlds", sec,
+                  bytes_=nworld * 4 * (used + 2 * nv + 2), nworld=nworld)  # fmt: skip
+
     # ---- body-tree accumulations and the wrench projection
     if section("bodies"):
         rig = synth.make_muscle_rig()
@@ -420,7 +518,7 @@ def run(launches: int = 32, only: str | None = None) -> None:
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--launches", type=int, default=32)
-    ap.add_argument("--only", default=None, help="comma-separated sections: trees, generated, stress, muscles, walks, iteration, bodies")
+    ap.add_argument("--only", default=None, help="comma-separated sections: trees, generated, stress, muscles, walks, iteration, implicit, bodies")
     ap.add_argument("--no-graph", action="store_true", help="plain launches instead of a hipGraph replay")
     args = ap.parse_args()
     GRAPH = not args.no_graph

@@ -14,6 +14,7 @@ not depend on the batch size.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from types import SimpleNamespace
 
 import numpy as np
 
@@ -373,6 +374,62 @@ def contact_model():
 
 
 # ------------------------------------------------------------------ muscle rig with path geometry
+
+
+def make_implicit_case(nworld: int, timestep: float = 0.004, seed: int = 3):
+    """A model and data for the implicit-fast integrator matrix: the SNU-like tree with a second,
+    free-floating body of six dofs appended, 40 affine actuators over one to three dofs of a chain,
+    12 damped tendons.  Returns (m, d, (rowadr, rownnz, colind), dofs of the first tree); arrays are NumPy."""
+    rng = np.random.default_rng(seed)
+    parents = list(snu_parents())
+    nv0 = len(parents)
+    parents += [-1, nv0, nv0 + 1, nv0 + 2, nv0 + 3, nv0 + 4]  # a free body: rows reset to M
+    nv = len(parents)
+    m = model_from_parents(parents)
+    rowadr, rownnz, colind = csr_from_parents(parents)
+    # bodies: model_from_parents makes one body per dof; body k + 1 holds dof k
+    m.body_freeadr = np.array([nv0 + 1], np.int32)
+    m.body_dofadr[nv0 + 1] = nv0
+    m.dof_damping = rng.uniform(0.0, 2.0, nv).astype(np.float32)
+    m.dof_damping[::7] = 0.0
+    m.opt.timestep = timestep
+    m.opt.disableflags = 0
+    chain = chain_mask(parents)
+
+    def rows(n, kmax):
+        nnz, adr, col = [], [], []
+        for _ in range(n):
+            leaf = int(rng.integers(6, nv))
+            support = np.flatnonzero(chain[leaf])
+            k = int(rng.integers(1, kmax + 1))
+            dofs = np.sort(rng.choice(support, min(k, len(support)), replace=False))
+            adr.append(len(col))
+            nnz.append(len(dofs))
+            col += dofs.tolist()
+        return np.array(nnz, np.int32), np.array(adr, np.int32), np.array(col, np.int32)
+
+    nu, nt = 40, 12
+    m.nactuator = nu
+    m.actuator_gaintype = rng.integers(0, 2, nu).astype(np.int32)
+    m.actuator_biastype = rng.integers(0, 2, nu).astype(np.int32)
+    m.actuator_gainprm = rng.normal(size=(nu, 10)).astype(np.float32)
+    m.actuator_biasprm = rng.normal(size=(nu, 10)).astype(np.float32) * 5
+    m.actuator_forcelimited = (rng.random(nu) < 0.3).astype(np.uint8)
+    m.actuator_forcerange = np.stack([-np.ones(nu), np.ones(nu)], 1).astype(np.float32)
+    m.ntendon = nt
+    m.ten_J_rownnz, m.ten_J_rowadr, m.ten_J_colind = rows(nt, 4)
+    m.tendon_damping = rng.uniform(0.0, 3.0, nt).astype(np.float32)
+    mom = rows(nu, 3)
+    b = make_batch(Shape("snu+free", tuple(parents), 8, nworld, (0.5, 8.0), 0.02, (-3.0, 3.0), 0.6, 1, seed), nworld)
+    d = SimpleNamespace(
+        nworld=nworld, M=b.M, moment_rownnz=mom[0], moment_rowadr=mom[1], moment_colind=mom[2],
+        actuator_moment=rng.normal(scale=0.3, size=(nworld, len(mom[2]))).astype(np.float32),
+        ten_J=rng.normal(scale=0.5, size=(nworld, len(m.ten_J_colind))).astype(np.float32),
+        ctrl=rng.uniform(-1, 1, (nworld, nu)).astype(np.float32),
+        actuator_force=rng.uniform(-1.5, 1.5, (nworld, nu)).astype(np.float32),
+        efc=SimpleNamespace(Ma=b.grad),
+    )  # fmt: skip
+    return m, d, (rowadr, rownnz, colind), nv0
 
 
 @dataclass
