@@ -178,46 +178,47 @@ def main() -> int:
 
     use_graph = not args.no_graph
 
-    def build(fn):
-        """Replays of `fn` over the rotation: one graph per set and one over all sets."""
-        if not use_graph:
-            return None, None
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for s in range(nsets):
-                fn(s)
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        single = []
-        for s in range(nsets):
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                fn(s)
-            single.append(g)
-        multi = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(multi):
-            for s in range(nsets):
-                fn(s)
-        return single, multi
+    MAX_GRAPH_STEPS = 1024  # steps recorded in one graph; longer runs replay it several times
 
     def runner(fn):
-        single, multi = build(fn)
+        """`run(n)`: n steps over the rotation of input sets.  With graphs, the steps of a run are
+        one graph (recorded and replayed once when `prepare(n)` is called, outside any timed
+        region), so that a timed region is one graph launch whatever its length."""
+        graphs = {}
+        if use_graph:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for s in range(nsets):
+                    fn(s)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+
+        def prepare(nsteps: int) -> None:
+            n = min(nsteps, MAX_GRAPH_STEPS)
+            if not use_graph or n <= 0 or n in graphs:
+                return
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for s in range(n):
+                    fn(s)
+            g.replay()  # the first replay of a graph also uploads it
+            torch.cuda.synchronize()
+            graphs[n] = g
 
         def run(nsteps: int) -> None:
-            i = 0
-            if use_graph:
-                while nsteps - i >= nsets:
-                    multi.replay()
-                    i += nsets
-                while i < nsteps:
-                    single[i % nsets].replay()
-                    i += 1
-            else:
-                while i < nsteps:
+            if not use_graph:
+                for i in range(nsteps):
                     fn(i)
-                    i += 1
+                return
+            left = nsteps
+            while left > 0:
+                n = min(left, MAX_GRAPH_STEPS)
+                prepare(n)
+                graphs[n].replay()
+                left -= n
 
+        run.prepare = prepare
         return run
 
     def region(run, nsteps: int):
@@ -235,8 +236,9 @@ def main() -> int:
     B = algorithmic_bytes(nv, nM, nefc)
     B3 = algorithmic_bytes_fused(nv, nM, nefc, iters)
     run_single = runner(step_single)
-    run_single(max(args.warmup, nsets))
     n_single = max(args.steps, -(-MIN_TIMED_LAUNCHES // iters))
+    run_single.prepare(n_single)
+    run_single(max(args.warmup, nsets))
     _, ev_single = region(run_single, n_single)
     single_us = ev_single / (n_single * iters) * 1e6
     single = {
@@ -252,11 +254,13 @@ def main() -> int:
         return 0
 
     run = runner(step)
+    n_kernel = max(args.steps, MIN_TIMED_LAUNCHES)
+    for n in (args.warmup, args.steps, n_kernel):
+        run.prepare(n)
     run(args.warmup)
     elapsed, _ = region(run, args.steps)
     value = args.steps * iters * nworld / elapsed
     # the kernel's duration from a region of its own whose length does not depend on --steps
-    n_kernel = max(args.steps, MIN_TIMED_LAUNCHES)
     _, ev_kernel = region(run, n_kernel)
     kernel_s = ev_kernel / n_kernel  # one launch = one step = `iters` solves of every world
     achieved = B * iters * nworld / kernel_s / 1e9
