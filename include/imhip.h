@@ -701,6 +701,41 @@ int im_newton_jv(const float *J, int njmax, const int32_t *nefc, const float *se
 int im_implicit_qh_base(const float *M, int64_t ldM, int nM, const int32_t *elem_dof, const float *dof_damping,
                         int64_t ld_damping, float timestep, float *qH, int64_t ld_qH, int nworld, void *stream);
 
+/* One term of qH's derivative part: scale * sum over sparse rows r of weight[w, r] row_r' row_r on M's
+ * pattern (actuator moments with the gains as weights and scale -h, tendon Jacobians with the tendon
+ * damping and scale +h).  values (nworld, ld_values): the rows' entries as the caller holds them;
+ * entry e of the sorted entry list reads values[w, entry_source[e]] (entry_source null: e itself) and
+ * belongs to row entry_row[e]; elem_ids / chunk_offsets / chunk_pairs / chunk_count are the gather
+ * tables of im_muscle_gather_tables for that entry list.  weight null: the actuator gains computed
+ * in the same call. */
+typedef struct im_row_pair_term {
+  const float *values;
+  int64_t ld_values;
+  const int32_t *entry_source;
+  const int32_t *entry_row;
+  int32_t nentry;
+  const int32_t *elem_ids;
+  int32_t nelem;
+  const int32_t *chunk_offsets;
+  const int32_t *chunk_pairs;
+  int32_t chunk_count;
+  const float *weight;
+  int64_t ld_weight;
+  float scale;
+} im_row_pair_term;
+
+/* deriv_smooth_vel (src/instantmimic/utils/mjw_step_optimized.py:3803-3900) in one launch:
+ * im_implicit_qh_base, im_actuator_velocity_gain (gain (nworld, ld_gain) is written when not null)
+ * and one pair-sum term each for the actuators and the tendons (either may be null), in that order;
+ * qH equals the separate calls bit for bit.  A world's row of qH, the gains and the larger term's
+ * entries must fit 64 KB of LDS (IM_ERR_UNSUPPORTED otherwise: use the separate calls). */
+int im_implicit_qh(const float *M, int64_t ldM, int nM, const int32_t *elem_dof, const float *dof_damping,
+                   int64_t ld_damping, float timestep, const int32_t *gaintype, const int32_t *biastype,
+                   const float *gainprm, const float *biasprm, int ld_prm, const uint8_t *forcelimited,
+                   const float *forcerange, const float *input, int64_t ld_input, const float *force, int64_t ld_force,
+                   float *gain, int64_t ld_gain, int nu, const im_row_pair_term *actuators,
+                   const im_row_pair_term *tendons, float *qH, int64_t ld_qH, int nworld, void *stream);
+
 /* Velocity gain of actuators with affine gain / bias (what derivative._qderiv_actuator_passive_vel
  * produces for them, mjw_step_optimized.py:3818-3846): gain[w, a] = biasprm[a, 2] (biastype 1)
  * + gainprm[a, 2] * input[w, a] (gaintype 1), zero when forcelimited[a] and force[w, a] is at or

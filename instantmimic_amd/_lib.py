@@ -64,6 +64,17 @@ class MuscleForceVelocityModel(C.Structure):
     _fields_ = [("vmax", C.c_float), ("fvmax", C.c_float), ("clamp_activation", C.c_float), ("include_active", C.c_float)]
 
 
+class RowPairTerm(C.Structure):
+    """im_row_pair_term"""
+
+    _fields_ = [
+        ("values", C.c_void_p), ("ld_values", C.c_int64), ("entry_source", C.c_void_p), ("entry_row", C.c_void_p),
+        ("nentry", C.c_int32), ("elem_ids", C.c_void_p), ("nelem", C.c_int32), ("chunk_offsets", C.c_void_p),
+        ("chunk_pairs", C.c_void_p), ("chunk_count", C.c_int32), ("weight", C.c_void_p), ("ld_weight", C.c_int64),
+        ("scale", C.c_float),
+    ]  # fmt: skip
+
+
 class MuscleGeometry(C.Structure):
     _fields_ = [
         ("waypoints", _vp), ("ld_waypoints", _i64),
@@ -146,6 +157,11 @@ SIGNATURES = {
     "im_sparse_dense_factor": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i, _vp, _vp, _i, _vp]),
     "im_implicit_qh_base": (_i, [_vp, _i64, _i, _vp, _vp, _i64, C.c_float, _vp, _i64, _i, _vp]),
     "im_actuator_velocity_gain": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _vp]),
+    "im_implicit_qh": (
+        _i,
+        [_vp, _i64, _i, _vp, _vp, _i64, C.c_float, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i,
+         C.POINTER(RowPairTerm), C.POINTER(RowPairTerm), _vp, _i64, _i, _vp],
+    ),  # fmt: skip
     "im_newton_linesearch": (
         _i,
         [_vp, _i, _vp, _i, _vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i64,

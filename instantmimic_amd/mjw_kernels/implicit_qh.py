@@ -192,6 +192,24 @@ def actuator_velocity_gain(m: Any, d: Any, scratch: ImplicitQhScratch) -> None:
     """``scratch.actuator_gain[w, a]``: d force / d velocity of every actuator."""
     import torch
 
+    t, inp, force = _actuator_inputs(m, d, scratch)
+    gain, nu = scratch.actuator_gain, scratch.actuator_gain.shape[1]
+    with torch.cuda.device(gain.device):
+        status = _lib.lib().im_actuator_velocity_gain(
+            t["gaintype"].data_ptr(), t["biastype"].data_ptr(), t["gainprm"].data_ptr(), t["biasprm"].data_ptr(),
+            int(t["gainprm"].shape[1]), None if t["forcelimited"] is None else t["forcelimited"].data_ptr(),
+            None if t["forcerange"] is None else t["forcerange"].data_ptr(), inp.data_ptr(), inp.stride(0),
+            None if force is None else force.data_ptr(), 0 if force is None else force.stride(0), gain.data_ptr(),
+            gain.stride(0), int(nu), int(gain.shape[0]), _stream(gain),
+        )  # fmt: skip
+    _lib.check(status, "im_actuator_velocity_gain")
+
+
+def _actuator_inputs(m: Any, d: Any, scratch: ImplicitQhScratch):
+    """The actuators' parameter tables on the device (made once), what drives each gain, and the
+    forces that the force range is tested against (or None)."""
+    import torch
+
     dev = scratch.actuator_gain.device
     t = scratch.tables
     if "gaintype" not in t:
@@ -213,23 +231,79 @@ def actuator_velocity_gain(m: Any, d: Any, scratch: ImplicitQhScratch) -> None:
     if t["act_index"] is not None:
         inp = d.ctrl.clone()
         inp[:, t["act_index"][0]] = d.act[:, t["act_index"][1]]
-    gain, nu = scratch.actuator_gain, scratch.actuator_gain.shape[1]
     force = getattr(d, "actuator_force", None) if t["forcelimited"] is not None else None
-    if inp.dtype != torch.float32 or inp.stride(1) != 1 or inp.shape != gain.shape:
+    if inp.dtype != torch.float32 or inp.stride(1) != 1 or inp.shape != scratch.actuator_gain.shape:
         raise TypeError("ctrl must be a float32 (nworld, nactuator) tensor with contiguous rows")
-    with torch.cuda.device(dev):
-        status = _lib.lib().im_actuator_velocity_gain(
-            t["gaintype"].data_ptr(), t["biastype"].data_ptr(), t["gainprm"].data_ptr(), t["biasprm"].data_ptr(),
-            int(t["gainprm"].shape[1]), None if t["forcelimited"] is None else t["forcelimited"].data_ptr(),
-            None if t["forcerange"] is None else t["forcerange"].data_ptr(), inp.data_ptr(), inp.stride(0),
-            None if force is None else force.data_ptr(), 0 if force is None else force.stride(0), gain.data_ptr(),
-            gain.stride(0), int(nu), int(gain.shape[0]), _stream(gain),
+    return t, inp, force
+
+
+def _pair_term(rows: RowPairGather, values, weight, scale: float):
+    """im_row_pair_term of a row set: the caller's values are read through ``entry_source``."""
+    g = rows.gather
+    if g is None:
+        return None
+    if "source32" not in rows.__dict__:
+        import torch
+
+        rows.source32 = rows.entry_source.to(dtype=torch.int32)
+    term = _lib.RowPairTerm()
+    term.values, term.ld_values = values.data_ptr(), values.stride(0)
+    term.entry_source, term.entry_row, term.nentry = rows.source32.data_ptr(), g.entry_muscle.data_ptr(), int(g.entry_count)
+    term.elem_ids, term.nelem = g.elem_ids.data_ptr(), int(g.elem_ids.numel())
+    term.chunk_offsets, term.chunk_pairs, term.chunk_count = g.chunk_offsets.data_ptr(), g.chunk_pairs.data_ptr(), int(g.chunk_count)
+    term.weight, term.ld_weight = (None, 0) if weight is None else (weight.data_ptr(), weight.stride(0))
+    term.scale = float(scale)
+    return term
+
+
+def _deriv_smooth_vel_fused(m, d, out, scratch: ImplicitQhScratch, damping, nworld: int, nM: int) -> bool:
+    """The whole of ``deriv_smooth_vel`` through im_implicit_qh; False when a world's rows do not
+    fit the kernel's LDS (the caller then makes the separate calls)."""
+    import ctypes as C
+
+    import torch
+
+    acts = scratch.actuators is not None and scratch.actuators.gather is not None
+    tens = scratch.tendons is not None and scratch.tendons.gather is not None
+    if scratch.actuators is not None:
+        t, inp, force = _actuator_inputs(m, d, scratch)
+        gain = scratch.actuator_gain
+        gain_args = [t["gaintype"].data_ptr(), t["biastype"].data_ptr(), t["gainprm"].data_ptr(), t["biasprm"].data_ptr(),
+                     int(t["gainprm"].shape[1]), None if t["forcelimited"] is None else t["forcelimited"].data_ptr(),
+                     None if t["forcerange"] is None else t["forcerange"].data_ptr(), inp.data_ptr(), inp.stride(0),
+                     None if force is None else force.data_ptr(), 0 if force is None else force.stride(0), gain.data_ptr(),
+                     gain.stride(0), int(gain.shape[1])]  # fmt: skip
+    else:
+        gain_args = [None, None, None, None, 0, None, None, None, 0, None, 0, None, 0, 0]
+    ta = tt = None
+    if acts:
+        values = d.actuator_moment.reshape(nworld, -1)
+        if values.dtype != torch.float32 or values.stride(1) != 1:
+            return False
+        ta = _pair_term(scratch.actuators, values, None, -scratch.timestep)
+    if tens:
+        values = d.ten_J.reshape(nworld, -1)
+        if values.dtype != torch.float32 or values.stride(1) != 1:
+            return False
+        tt = _pair_term(scratch.tendons, values, scratch.tendon_damping, scratch.timestep)
+    with torch.cuda.device(out.device):
+        status = _lib.lib().im_implicit_qh(
+            d.M.data_ptr(), d.M.stride(0), nM, scratch.elem_dof.data_ptr(), damping.data_ptr(),
+            damping.stride(0) if damping.shape[0] > 1 else 0, scratch.timestep, *gain_args,
+            None if ta is None else C.byref(ta), None if tt is None else C.byref(tt), out.data_ptr(), out.stride(0), nworld,
+            _stream(out),
         )  # fmt: skip
-    _lib.check(status, "im_actuator_velocity_gain")
+    if status == _lib.IM_ERR_UNSUPPORTED:
+        return False
+    _lib.check(status, "im_implicit_qh")
+    return True
 
 
-def deriv_smooth_vel(m: Any, d: Any, out, scratch: ImplicitQhScratch) -> None:
-    """``out = M - h qDeriv`` on M's pattern (:3803-3900): damping, actuators, tendon damping."""
+def deriv_smooth_vel(m: Any, d: Any, out, scratch: ImplicitQhScratch, *, fused: bool = True) -> None:
+    """``out = M - h qDeriv`` on M's pattern (:3803-3900): damping, actuators, tendon damping.
+    ``fused``: one launch (im_implicit_qh) where a world's rows fit its LDS; otherwise, and with
+    ``fused=False``, the base, the gains and one gather per term as separate launches.  The two
+    forms give the same bits."""
     import torch
 
     M = d.M
@@ -239,6 +313,8 @@ def deriv_smooth_vel(m: Any, d: Any, out, scratch: ImplicitQhScratch) -> None:
     if M.dtype != torch.float32 or out.dtype != torch.float32 or M.stride(1) != 1 or out.stride(1) != 1 or M.shape != out.shape:
         raise TypeError("M and out must be float32 (nworld, nM) tensors with contiguous rows")
     nworld, nM = int(M.shape[0]), int(scratch.elem_dof.numel())
+    if fused and _deriv_smooth_vel_fused(m, d, out, scratch, damping, nworld, nM):
+        return
     with torch.cuda.device(out.device):
         status = _lib.lib().im_implicit_qh_base(
             M.data_ptr(), M.stride(0), nM, scratch.elem_dof.data_ptr(), damping.data_ptr(),

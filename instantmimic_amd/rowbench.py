@@ -450,7 +450,10 @@ def run(launches: int = 32, only: str | None = None) -> None:
         nM, nmom, nten, nu = int(st[2].size), int(d.moment_colind.size), int(m.ten_J_colind.size), int(m.nactuator)
         wl = f"snu + a free body nv={m.nv} nM={nM}, {nu} actuators ({nmom} moment entries), {m.ntendon} tendons ({nten} entries) x {nworld} worlds"
         sec = _timeit(torch, lambda i: IQ.deriv_smooth_vel(m, dd, scratch.implicit_qderiv, scratch), 1, launches)
-        _line("qH = M - h dF/dv: im_implicit_qh_base, im_actuator_velocity_gain, two pair-sum gathers", wl, sec,
+        _line("im_implicit_qh: qH = M - h dF/dv in one launch (damping, actuator gains and pair sums, tendon pair sums)", wl, sec,
+              bytes_=nworld * 4 * (2 * nM + nmom + nten + 3 * nu), nworld=nworld)  # fmt: skip
+        sec = _timeit(torch, lambda i: IQ.deriv_smooth_vel(m, dd, scratch.implicit_qderiv, scratch, fused=False), 1, launches)
+        _line("the same as separate launches: im_implicit_qh_base, im_actuator_velocity_gain, two entry permutations, two gathers", wl, sec,
               bytes_=nworld * 4 * (2 * nM + nmom + nten + 3 * nu), nworld=nworld)  # fmt: skip
         scratch.tree_factor_solve = T.create_tree_factor_solve_scratch(m, dev)
         sec = _timeit(torch, lambda i: IQ.implicit_factor_optimized(m, dd, scratch), 1, launches)

@@ -113,10 +113,14 @@ def test_gpu_qh_and_solve(device):
                          efc=SimpleNamespace(Ma=t(d.efc.Ma)))  # fmt: skip
     scratch = Q.create_implicit_qh_scratch(m, dd, device)
     assert scratch.actuators.dropped_pair_count > 0  # pairs on the free body's rows: those rows keep M
-    Q.deriv_smooth_vel(m, dd, scratch.implicit_qderiv, scratch)
-    torch.cuda.synchronize()
-    np.testing.assert_array_equal(scratch.actuator_gain.cpu().numpy(), want_gain)
-    np.testing.assert_array_equal(scratch.implicit_qderiv.cpu().numpy(), want_qh)
+    # one launch (im_implicit_qh), then the separate launches: base, gains, one gather per term
+    for fused in (True, False):
+        scratch.implicit_qderiv.fill_(float("nan"))
+        scratch.actuator_gain.fill_(float("nan"))
+        Q.deriv_smooth_vel(m, dd, scratch.implicit_qderiv, scratch, fused=fused)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(scratch.actuator_gain.cpu().numpy(), want_gain)
+        np.testing.assert_array_equal(scratch.implicit_qderiv.cpu().numpy(), want_qh)
     # the whole step: qH, then the tree L'DL (the model is a forest: 56 + 6 dofs)
     scratch.tree_factor_solve = T.create_tree_factor_solve_scratch(m, device)
     assert scratch.tree_factor_solve is not None
