@@ -178,6 +178,31 @@ def test_newton_entry_points_check_their_arguments_before_any_launch():
     assert lib.im_qfrc_constraint_from_grad(one, one, 27, one, 27, one, 27, None, one, 27, 27, 4, None) == _lib.IM_ERR_ARG
 
 
+def test_implicit_matrix_entry_points_check_their_arguments_before_any_launch():
+    lib = _lib.lib()
+    one = 16
+    q = lambda **k: lib.im_implicit_qh(  # noqa: E731
+        k.get("M", one), k.get("ldM", 737), 737, one, one, 0, 0.004, one, one, one, one, k.get("ldprm", 10), None, None, one,
+        k.get("ld_input", 40), None, 0, one, 40, k.get("nu", 40), k.get("ta"), k.get("tt"), one, k.get("ldq", 737),
+        k.get("nworld", 4), None)  # fmt: skip
+    assert q(nworld=-1) == _lib.IM_ERR_ARG and q(M=None) == _lib.IM_ERR_ARG and q(ldprm=2) == _lib.IM_ERR_ARG
+    assert q(ldM=700) == _lib.IM_ERR_STRIDE and q(ldq=700) == _lib.IM_ERR_STRIDE and q(ld_input=39) == _lib.IM_ERR_ARG
+    assert q(nworld=0) == _lib.IM_OK
+    term = _lib.RowPairTerm()
+    term.nentry, term.nelem, term.chunk_count = 80, 60, 30  # tables missing
+    assert q(ta=C.byref(term)) == _lib.IM_ERR_ARG
+    for name in ("values", "entry_row", "elem_ids", "chunk_offsets", "chunk_pairs"):
+        setattr(term, name, one)
+    assert q(tt=C.byref(term)) == _lib.IM_ERR_ARG  # the tendon term needs its weights
+    assert q(ta=C.byref(term), nu=0) == _lib.IM_ERR_ARG  # the actuator term's weights are the gains
+    term.nentry = 40000
+    assert q(ta=C.byref(term)) == _lib.IM_ERR_UNSUPPORTED  # entry indices travel as 15 bits
+    term.nentry, term.chunk_count = 9000, 9000
+    assert q(ta=C.byref(term)) == _lib.IM_ERR_UNSUPPORTED  # a world's rows exceed 64 KB of LDS
+    assert lib.im_implicit_qh_base(one, 700, 737, one, one, 0, 0.004, one, 737, 4, None) == _lib.IM_ERR_STRIDE
+    assert lib.im_actuator_velocity_gain(one, one, one, one, 2, None, None, one, 40, None, 0, one, 40, 40, 4, None) == _lib.IM_ERR_ARG
+
+
 def test_entry_points_that_clamp_rows_refuse_an_empty_row_range():
     """The assembly kernels clamp a row index to njmax - 1 (every load is issued, the value
     selected afterwards), so njmax = 0 is refused on the host instead of reading before the
