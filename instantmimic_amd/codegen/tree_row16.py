@@ -325,11 +325,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("    float *lds = xlds;")
     emit("    const int kq = lane >> 4;")
     emit("    const int njp = (njmax + 15) & ~15;")
-    emit(f"    float *dcl = lds + {lds_floats} + wv * (LONG ? njp : 128);  // D per row (0 where a row does not contribute)")
+    emit(f"    float *dcl = lds + {lds_floats} + wv * (LONG ? 2 * njp : 128);  // D per listed row, and the list of rows behind it")
     emit("    const int64_t wq = bid * 4 + wv < nworld ? bid * 4 + wv : nworld - 1;")
     emit("    int ne = nefc_p ? nefc_p[wq] : njmax; ne = ne < njmax ? ne : njmax;")
     emit("    ne = __builtin_amdgcn_readfirstlane(ne);")
-    emit("    const int steps = (ne + 3) >> 2;")
     # every load below is unconditional (clamped address, value selected afterwards): a load
     # under a lane mask turns into a branch and a wait in the instruction stream
     # J through a buffer descriptor over the world's njmax x nv block: the address of a load is a
@@ -345,18 +344,28 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     for u in range(PD):
         emit("    float " + ", ".join(f"g{u}_{c}" for c in range(NT)) + ";")
 
-    def load(u, step):
+    def load(u, step, listed=False):
         # always issued, from a clamped row, so that the number of loads in flight is known at
-        # compile time (a load under a condition makes every later wait a wait for all loads)
+        # compile time (a load under a condition makes every later wait a wait for all loads).
+        # listed: the step's rows are entries 4 step .. 4 step + 3 of the list of contributing rows
+        # (long variant; a step past the list reads its last entry and is never used)
+        if listed:
+            emit(f"        {{ const int li = 4 * ({step}) + kq; const int rowb = rowl[li < njp ? li : njp - 1] * {4 * nv};")
+            for c in range(NT):
+                emit(f"          g{u}_{c} = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(jrs, rowb + vc{c}, 0, 0));")
+            emit("        }")
+            return
         for c in range(NT):
             emit(f"        g{u}_{c} = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(jrs, vo{c}, ({step}) * {16 * nv}, 0));")
 
-    def consume(u, step, listed=False):
+    def consume(u, step, listed=False, mixed=False):
         # rows at or past the world's nefc may hold anything: they count as zero rows; columns
         # past nv repeat the last column, which only reaches accumulator elements outside H.
         # listed: the step's rows come from the list of contributing rows, whose spare entries
         # name row 0 with weight 0 -- a row below nefc whenever a listed step runs at all
-        emit(f"        {{ const int st = {step}; const float d = pd[st * 4];" + ("" if listed else " const bool rv = st * 4 + kq < ne;"))
+        # mixed (long variant): steps below SP are rows 4 st .. 4 st + 3 as they are, later ones are listed
+        emit(f"        {{ const int st = {step}; const float d = pd[st * 4];" + ("" if listed else
+             (f" const bool rv = st >= {SP} || st * 4 + kq < ne;" if mixed else " const bool rv = st * 4 + kq < ne;")))
         for c in range(NT):
             emit(f"          const float z{c} = " + (f"g{u}_{c};" if listed else f"rv ? g{u}_{c} : 0.0f;"))
         for c in range(NT):
@@ -381,54 +390,55 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
         emit(f"    const float mv{i} = M[wq * ldM + min({i * 64} + lane, {nM - 1})];")
     SP = min(PD, int(os.environ.get("IMHIP_SP", "2")))  # steps (4 rows each) requested before the row weights are known
     pin_ch = " ".join(f'asm volatile("" : "+v"(chc{i}));' for i in range(len(leaf_sets)))
-    emit("    int steps_s = 0, cnt = 0;  // short variant: steps and length of the compacted tail")
-    emit("    if (LONG) {")
-    emit("      for (int r0 = 128; r0 < njp; r0 += 64) {  // rows from 128 on, up front")
-    emit("        const int r = r0 + lane, rc = r < njmax ? r : njmax - 1;")
-    emit("        const int sv = state[wq * njmax + rc]; const float dv = D[wq * njmax + rc];")
-    emit("        if (r < njp) dcl[r] = (r < ne && sv == quad) ? dv : 0.0f;")
-    emit("      }")
-    emit("    }")
+    # Of the rows beyond the first 4 SP only the contributing ones are read: their numbers and
+    # weights are packed behind entry 4 SP of a list, in row order (ballot and prefix count), so a
+    # skipped row is one that would have added (J * 0) * J everywhere.  The first 4 SP rows are
+    # requested before the weights are known and enter as they are, with weight 0 where they do
+    # not contribute.  Short variant (njmax <= 64): one row per lane, every listed step in flight
+    # at once.  Long variant: rows 64 lanes at a time, PD steps in flight in a loop.
+    emit("    int steps = 0, cnt = 0;  // steps of four rows to run; length of the list behind the first rows")
     emit("    const int rc0 = lane < njmax ? lane : njmax - 1, rc1 = lane + 64 < njmax ? lane + 64 : njmax - 1;")
     emit("    const int sv0 = state[wq * njmax + rc0], sv1 = LONG ? state[wq * njmax + rc1] : 0;")
     emit("    const float dv0 = D[wq * njmax + rc0], dv1 = LONG ? D[wq * njmax + rc1] : 0.0f;")
-    emit("    if (LONG) {")
-    for u in range(PD):
-        load(u, str(u))
-    emit("    } else {")
     for u in range(SP):
         load(u, str(u))
-    emit("    }")
     for ci in rhs_tables:
         emit(f"    yv{ci} = yw[chc{ci}];")
     emit(f"    float *mcopy = lds + wv * {TW};  // reused for this world's copy of H afterwards")
     for i in range(MC):
         emit(f"    mcopy[{i * 64} + lane] = mv{i};")
     emit(f"    mcopy[{nM}] = 0.0f;  // where the table sends accumulator elements outside the pattern")
-    emit("    if (LONG) {")
-    emit("      if (lane < njp) dcl[lane] = (lane < ne && sv0 == quad) ? dv0 : 0.0f;")
-    emit("      if (lane + 64 < njp) dcl[lane + 64] = (lane + 64 < ne && sv1 == quad) ? dv1 : 0.0f;")
-    emit("    } else {")
-    # Short variant (njmax <= 64, one row per lane): the first 16 rows are read as they are,
-    # with D = 0 for the ones that do not contribute; of the others only the contributing rows
-    # are read at all -- their ids and D are packed behind entry 16 in row order (ballot and
-    # prefix count), so a skipped row is one that would have added (J * 0) * J everywhere.
-    emit(f"      int *rowl = (int *)(dcl + 64);")
-    emit(f"      const bool act0 = lane < ne && sv0 == quad;")
+    emit("    int *rowl = (int *)(dcl + (LONG ? njp : 64));")
+    emit("    {")
+    emit("      const unsigned long long below = (1ull << lane) - 1ull;")
+    emit("      const bool act0 = lane < ne && sv0 == quad;")
     emit(f"      const bool tail = act0 && lane >= {4 * SP};")
     emit("      const unsigned long long tm = __ballot(tail);")
     emit("      cnt = __popcll(tm);")
-    emit(f"      steps_s = ne > {4 * SP} ? {SP} + ((cnt + 3) >> 2) : ((ne + 3) >> 2);")
-    emit("      dcl[lane] = 0.0f; rowl[lane] = 0;")
+    emit("      if (!LONG) { dcl[lane] = 0.0f; rowl[lane] = 0; }")
     emit(f"      if (lane < {4 * SP}) {{ dcl[lane] = act0 ? dv0 : 0.0f; rowl[lane] = lane; }}")
-    emit(f"      if (tail) {{ const int pos = {4 * SP} + __popcll(tm & ((1ull << lane) - 1ull)); dcl[pos] = dv0; rowl[pos] = lane; }}")
-    emit("      IM_WAVE_SYNC();")
-    for u in range(SP, PD):
-        emit(f"      {{ const int rowb = rowl[{4 * u} + kq] * {4 * nv};")
-        for c in range(NT):
-            emit(f"        g{u}_{c} = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(jrs, rowb + vc{c}, 0, 0));")
-        emit("      }")
+    emit(f"      if (tail) {{ const int pos = {4 * SP} + __popcll(tm & below); dcl[pos] = dv0; rowl[pos] = lane; }}")
+    emit("      if (LONG) {")
+    emit("        const bool act1 = lane + 64 < ne && sv1 == quad;")
+    emit("        const unsigned long long tm1 = __ballot(act1);")
+    emit(f"        if (act1) {{ const int pos = {4 * SP} + cnt + __popcll(tm1 & below); dcl[pos] = dv1; rowl[pos] = lane + 64; }}")
+    emit("        cnt += __popcll(tm1);")
+    emit("        for (int r0 = 128; r0 < njp; r0 += 64) {  // more than 128 rows")
+    emit("          const int r = r0 + lane, rc = r < njmax ? r : njmax - 1;")
+    emit("          const int sv = state[wq * njmax + rc]; const float dv = D[wq * njmax + rc];")
+    emit("          const bool act = r < ne && sv == quad;")
+    emit("          const unsigned long long tmr = __ballot(act);")
+    emit(f"          if (act) {{ const int pos = {4 * SP} + cnt + __popcll(tmr & below); dcl[pos] = dv; rowl[pos] = r; }}")
+    emit("          cnt += __popcll(tmr);")
+    emit("        }")
+    emit("        // the spare entries of the last step: row 0 with weight 0")
+    emit(f"        if (lane < 3 && {4 * SP} + cnt + lane < njp) {{ dcl[{4 * SP} + cnt + lane] = 0.0f; rowl[{4 * SP} + cnt + lane] = 0; }}")
+    emit("      }")
+    emit(f"      steps = ne > {4 * SP} ? {SP} + ((cnt + 3) >> 2) : ((ne + 3) >> 2);")
     emit("    }")
+    emit("    IM_WAVE_SYNC();")
+    for u in range(SP, PD):
+        load(u, str(u), listed=True)
     emit("    IM_WAVE_SYNC();")
     for n in range(len(tiles)):
         emit(f"    f32x4 acc{n};")
@@ -439,7 +449,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("    STAMP();  // 1: row weights staged, M gathered")
     emit("    if (!LONG) {  // every row that is needed is already in flight")
     for u in range(PD):
-        emit(f"      if ({u} < steps_s) {{")
+        emit(f"      if ({u} < steps) {{")
         if u < SP:
             consume(u, str(u))
         else:
@@ -451,11 +461,11 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
         # guards instead of early exits: an exit from the middle of the unrolled body makes
         # the compiler keep two copies of every accumulator
         emit(f"      if (s0 + {u} < steps) {{")
-        consume(u, f"s0 + {u}")
+        consume(u, f"s0 + {u}", mixed=True)
         emit("      }")
         # the next use of the register set is requested on every path: with the same number
         # of loads in flight whatever steps ran, each wait counts only the loads before it
-        load(u, f"s0 + {u + PD}")
+        load(u, f"s0 + {u + PD}", listed=True)
     emit("    }")
     emit("    }")
     emit("    STAMP();  // 2: assembled")
