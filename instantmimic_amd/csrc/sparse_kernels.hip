@@ -298,10 +298,13 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
   if (w >= nworld || (done && done[w])) return;
   const int n = Q.nv, nslots = Q.nslots, nfac = nslots - n, rhs = nfac;
   const int nw = (A.block + 31) / 32;
-  const int per_world = (nslots + n + 2 * nw + 3) & ~3;
+  const int njp = (njmax + 3) & ~3, factor_words = (nslots + n + 2 * nw + 3) & ~3;
+  const int per_world = factor_words + 2 * njp;
   float *N = lds + ((off + 3) & ~3) + wv * per_world;  // [nslots]; a row of M before the factor
   float *iD = N + nslots;                              // [n]
   float *red = iD + n;                                 // [2][nw]
+  float *dl = N + factor_words;                        // [njp] weights of the listed constraint rows
+  int *rowl = (int *)(dl + njp);                       // [njp] their numbers
   float *U = U_ + (size_t)w * Q.nv_pad * Q.nv_pad;
   const float *Mw = M + (size_t)w * ldM;
   const float *gw = grad + (size_t)w * ldg;
@@ -311,7 +314,6 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
   int ne = nefc_p[w];
   ne = ne < njmax ? ne : njmax;
   ne = __builtin_amdgcn_readfirstlane(ne);
-  const int steps = (ne + 3) >> 2;
 
   // Every load below is unconditional (clamped address, value selected afterwards) and what
   // is needed first is requested first, so that each wait counts only the loads before it.
@@ -343,8 +345,13 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
     npm = ~((unsigned long long)lo | (words > 1 ? (unsigned long long)hi << 32 : 0ull));
     if (lane >= n) npm = 0ull;
   }
+  // The first 4 PD rows are requested as they are, before anything is known of them; of the rows
+  // behind them only the contributing ones are read at all: their numbers and weights go into a
+  // list in row order (ballot and prefix count, 64 rows at a time), so a skipped row is one
+  // that would have added (J * 0) * J everywhere.
   float g[PD][NT], gd[PD];
   int gs[PD];
+  bool gv[PD];  // the register set holds a row below nefc
 #pragma unroll
   for (int u = 0; u < PD; ++u) {
     const int row = 4 * u + kq, rowc = row < njmax ? row : njmax - 1;
@@ -352,7 +359,23 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
     for (int c = 0; c < NT; ++c) g[u][c] = ld_u32(Jw, (uint32_t)(rowc * n + col[c]));
     gd[u] = ld_u32(Dw, (uint32_t)rowc);
     gs[u] = ld_u32(sw, (uint32_t)rowc);
+    gv[u] = row < ne;
   }
+  int cnt = 0;
+  for (int r0 = 4 * PD; r0 < ne; r0 += 64) {  // the same trips for every lane
+    const int r = r0 + lane, rc = r < njmax ? r : njmax - 1;
+    const int sv = sw[rc];
+    const float dv = Dw[rc];
+    const bool act = r < ne && sv == quad;
+    const unsigned long long tm = __ballot(act);
+    if (act) {
+      const int pos = cnt + __popcll(tm & ((1ull << lane) - 1ull));
+      dl[pos] = dv;
+      rowl[pos] = r;
+    }
+    cnt += __popcll(tm);
+  }
+  const int steps = ne > 4 * PD ? PD + ((cnt + 3) >> 2) : (ne + 3) >> 2;
 #pragma unroll
   for (int c = 0; c < 16; ++c)
     if (c * 64 + lane < A.nM) N[c * 64 + lane] = mv[c];
@@ -372,8 +395,7 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
 #pragma unroll
     for (int u = 0; u < PD; ++u) {
       if (s0 + u < steps) {
-        const int row = 4 * (s0 + u) + kq;
-        const bool rv = row < ne;
+        const bool rv = gv[u];
         const float d = (rv && gs[u] == quad) ? gd[u] : 0.0f;
         float z[NT], e[NT];
 #pragma unroll
@@ -415,11 +437,15 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
       }
       // Next use of this register set.  Issued whether or not the step above ran, so that the
       // number of loads in flight at every wait is the same on every path.
-      const int nrow = 4 * (s0 + u + PD) + kq, nrowc = nrow < njmax ? nrow : njmax - 1;
+      // (step s0 + u + PD: entries 4 (s0 + u) .. + 3 of the list; past its end row 0 with weight 0)
+      const int li = 4 * (s0 + u) + kq;
+      const bool lv = li < cnt;
+      const int nrowc = lv ? rowl[li] : 0;
 #pragma unroll
       for (int c = 0; c < NT; ++c) g[u][c] = ld_u32(Jw, (uint32_t)(nrowc * n + col[c]));
-      gd[u] = ld_u32(Dw, (uint32_t)nrowc);
-      gs[u] = ld_u32(sw, (uint32_t)nrowc);
+      gd[u] = lv ? dl[li] : 0.0f;
+      gs[u] = quad;
+      gv[u] = lv;
     }
   }
   // the slots of this lane's accumulator elements (all requested before the first is used)
@@ -901,7 +927,8 @@ int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done, const
     A.solve_words = 0;
     A.block = plan->block;
     A.nM = plan->nM;
-    const size_t per_world = ((size_t)plan->nslots + n + 2 * nw + 3) & ~(size_t)3;
+    // per world: the factor's arrays and the list of contributing constraint rows (weight and number)
+    const size_t per_world = (((size_t)plan->nslots + n + 2 * nw + 3) & ~(size_t)3) + 2 * (((size_t)njmax + 3) & ~(size_t)3);
     const size_t wave_lds = 4 * (((staged + 3) & ~(size_t)3) + 4 * per_world);
     if (wave_lds <= 64 * 1024 && staged <= 8192 && ldM >= plan->nM) {
       const dim3 grid((unsigned)((nworld + 3) / 4)), wg(256);
