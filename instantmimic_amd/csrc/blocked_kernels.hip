@@ -1343,32 +1343,72 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
   const int c0c = c0 < nv ? c0 : nv - 1, c1c = c1 < nv ? c1 : nv - 1;
   float v0[8], v1[8], dd = 0.0f;
   int sd = 0;
-  auto prefetch = [&](int r0) {  // every load is issued whatever the row: clamped, selected later
+  // The first 32 rows are read as they lie.  Of the rows behind them only those that contribute
+  // (inside nefc, state `quad`) are read at all: every wavefront counts them by ballot, 256 rows
+  // per round with the loads of a round issued together, and the wavefronts share out the writing
+  // of the list of their numbers and weights, which the barrier behind the first chunk publishes.
+  int *rowl = (int *)(lds + 2 * stage_words);  // [njmax rounded up to 4]
+  float *dl = (float *)(rowl + ((njmax + 3) & ~3));
+  {  // every load is issued whatever the row: clamped, selected later
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int row = r0 + wave * 8 + i, rowc = row < njmax ? row : njmax - 1;
+      const int row = wave * 8 + i, rowc = row < njmax ? row : njmax - 1;
       v0[i] = Jw[(int64_t)rowc * nv + c0c];
       v1[i] = Jw[(int64_t)rowc * nv + c1c];
     }
-    const int row = r0 + wave * 8 + (lane & 7), rowc = row < njmax ? row : njmax - 1;
+    const int row = wave * 8 + (lane & 7), rowc = row < njmax ? row : njmax - 1;
     dd = Dw[rowc];
     sd = sw[rowc];
+  }
+  int cnt = 0;
+  for (int r = 32; r < njmax; r += 256) {
+    int st[4];
+    float dv[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int row = r + 64 * q + lane, rowc = row < njmax ? row : njmax - 1;
+      st[q] = sw[rowc];
+      dv[q] = Dw[rowc];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int row = r + 64 * q + lane;
+      const bool act = row < nefc && st[q] == quad;
+      const uint64_t mask = __ballot(act);
+      if (q == wave && act) {
+        const int pos = cnt + __popcll(mask & ((1ull << lane) - 1));
+        rowl[pos] = row;
+        dl[pos] = dv[q];
+      }
+      cnt += __popcll(mask);
+    }
+  }
+  auto prefetch = [&](int p0) {  // list positions p0 .. p0 + 31
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int pos = p0 + wave * 8 + i, row = pos < cnt ? rowl[pos] : 0;
+      v0[i] = Jw[(int64_t)row * nv + c0c];
+      v1[i] = Jw[(int64_t)row * nv + c1c];
+    }
   };
-  auto stage = [&](int r0, int buf) {
+  auto stage = [&](int p0, int buf, bool listed) {
     float *Jb = Js + buf * stage_words, *db = dcs + buf * stage_words;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const bool in = r0 + wave * 8 + i < nefc;
+      const bool in = p0 + wave * 8 + i < (listed ? cnt : nefc);
       if (c0 < nvr) Jb[(wave * 8 + i) * nvr + c0] = (in && c0 < nv) ? v0[i] : 0.0f;  // nvr is 32 for nv <= 32
       if (c1 < nvr) Jb[(wave * 8 + i) * nvr + c1] = (in && c1 < nv) ? v1[i] : 0.0f;
     }
-    if (lane < 8) db[wave * 8 + lane] = (r0 + wave * 8 + lane < nefc && sd == quad) ? dd : 0.0f;
+    if (lane < 8) {
+      const int pos = p0 + wave * 8 + lane;
+      db[wave * 8 + lane] = listed ? (pos < cnt ? dl[pos] : 0.0f) : ((pos < nefc && sd == quad) ? dd : 0.0f);
+    }
   };
-  prefetch(0);
-  stage(0, 0);
+  stage(0, 0, false);
   __syncthreads();
-  for (int r0 = 0, buf = 0; r0 < nefc; r0 += 32, buf ^= 1) {
-    prefetch(r0 + 32);
+  const int nchunk = nefc > 0 ? 1 + (cnt + 31) / 32 : 0;
+  for (int c = 0, buf = 0; c < nchunk; ++c, buf ^= 1) {
+    prefetch(32 * c);
     // v_mfma_f32_32x32x2_f32: lane l supplies A[i = l % 32][k = l / 32] and B[k = l / 32][j = l % 32]
     // the wavefront's tiles take turns inside the loop over the rows: independent accumulators
     // keep the matrix core busy while one of them waits for its previous result
@@ -1388,7 +1428,7 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
           acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[m][2 * q * nvr] * dk, pb[m][2 * q * nvr], acc[m], 0, 0, 0);
     }
     // the other copy was last read one chunk ago, before the barrier that every wavefront has passed since
-    stage(r0 + 32, buf ^ 1);
+    stage(32 * c, buf ^ 1, true);
     __syncthreads();
   }
 #pragma unroll
@@ -1435,8 +1475,8 @@ __global__ __launch_bounds__(256, 4) void jtdj_factor_solve_kernel(
   extern __shared__ float lds[];
   const Stair<B> S{pad};
   const int nU = S.words();
-  const int nvr = NVR ? NVR : (nv + 31) / 32 * 32, stage_words = 2 * (32 * nvr + 32);
-  float *U = lds;       // first the staged rows of J (two copies), then [nU] H, then the factor
+  const int nvr = NVR ? NVR : (nv + 31) / 32 * 32, stage_words = 2 * (32 * nvr + 32) + 2 * ((njmax + 3) & ~3);
+  float *U = lds;       // first the staged rows of J (two copies) and the list of contributing rows, then [nU] H, then the factor
   float *rhs = lds + (nU > stage_words ? nU : stage_words);  // [pad]
   float *L = rhs + pad;  // [B * B + B]
   const int tid = threadIdx.x, nt = blockDim.x;
@@ -1662,8 +1702,12 @@ int im_jtdj_mfma(const float *Mdense, const float *J, int njmax, const float *D,
   if (!Mdense || !J || !D || !state || !H) return IM_ERR_ARG;
   if (nv > 128) return IM_ERR_UNSUPPORTED;
   const int nvr = (nv + 31) / 32 * 32;
-  const size_t lds_bytes = sizeof(float) * 2 * (32 * (size_t)nvr + 32);  // two copies of the staged rows
+  // two copies of the staged rows, the list of contributing rows with their weights
+  const size_t lds_bytes = sizeof(float) * (2 * (32 * (size_t)nvr + 32) + 2 * (size_t)((njmax + 3) & ~3));
+  if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   auto fn = nvr == 128 ? im::jtdj_mfma_kernel<128> : im::jtdj_mfma_kernel<0>;
+  if (lds_bytes > 64 * 1024)
+    IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, Mdense, J, njmax, D, state, nefc,
                      quad, H, nv, nv_pad);
   IM_HIP_CHECK(hipGetLastError());
@@ -1681,7 +1725,7 @@ int im_jtdj_factor_solve(const float *Mdense, const float *J, int njmax, const f
   if ((y && ldy < nv) || (x && ldx < nv)) return IM_ERR_STRIDE;
   if (U && ((uintptr_t)U & 15)) return IM_ERR_STRIDE;
   const int nvr = (nv + 31) / 32 * 32;
-  const size_t stage_words = 2 * (32 * (size_t)nvr + 32), u_words = im::Stair<16>{pad}.words();
+  const size_t stage_words = 2 * (32 * (size_t)nvr + 32) + 2 * (size_t)((njmax + 3) & ~3), u_words = im::Stair<16>{pad}.words();
   const size_t lds_bytes = sizeof(float) * ((u_words > stage_words ? u_words : stage_words) + pad + 16 * 16 + 16);
   if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
   auto fn = nvr == 128 ? im::jtdj_factor_solve_kernel<128> : im::jtdj_factor_solve_kernel<0>;
