@@ -19,7 +19,8 @@ constexpr size_t kLdsLimit = 64 * 1024;
 // ---- Newton gradient ---------------------------------------------------------------------------
 // qfrc_constraint = J' efc_force, grad = Ma - qfrc_smooth - qfrc_constraint, grad . grad.
 // L lanes per world (32 up to 32 dofs, else 64), a lane per dof, the rows of J streamed ROWS
-// at a time (a row of J is contiguous over the lanes); efc_force sits in LDS.
+// at a time (a row of J is contiguous over the lanes); the nonzero entries of efc_force sit in
+// LDS with their row numbers, and only those rows of J are read.
 struct GradArgs {
   const int32_t *nefc;
   const float *J, *force, *smooth, *Ma, *alpha;
@@ -39,29 +40,48 @@ __global__ __launch_bounds__(kThreads) void newton_gradient_kernel(GradArgs a) {
   const int64_t w_raw = (int64_t)blockIdx.x * per_block + lw;
   const bool live = w_raw < a.nworld;
   const int64_t w = live ? w_raw : (int64_t)a.nworld - 1;
-  float *f = lds + lw * (a.njmax + a.nv + 64);  // [njmax] forces, then [nv] grad, then [64] lane sums
-  float *gl = f + a.njmax, *part = gl + a.nv;
+  // [njmax] the nonzero forces, [njmax] their rows, then [nv] grad, then [64] lane sums
+  float *f = lds + lw * (2 * a.njmax + a.nv + 64);
+  int *rowl = (int *)(f + a.njmax);
+  float *gl = f + 2 * a.njmax, *part = gl + a.nv;
   const bool done = a.done && a.done[w] != 0;
   const bool changed = a.changed[w] != 0;
   int nefc = a.nefc ? a.nefc[w] : a.njmax;
   nefc = nefc < a.njmax ? nefc : a.njmax;
   nefc = nefc > 0 ? nefc : 0;
   const bool work = !done && changed;
-  if (work)
-    for (int r = lane; r < nefc; r += L) f[r] = a.force[w * a.ldf + r];
+  // A row whose force is zero (every satisfied constraint) adds nothing to J' f and is not read:
+  // the world's lanes list the other rows in order, by ballot.
+  int cnt = 0;
+  if (work) {
+    const int shift = (threadIdx.x & 63) & ~(L - 1);  // where the world's lanes start in the wavefront
+    const uint64_t group = L == 64 ? ~0ull : 0xFFFFFFFFull;
+    for (int r0 = 0; r0 < nefc; r0 += L) {
+      const int r = r0 + lane;
+      const float v = r < nefc ? a.force[w * a.ldf + r] : 0.0f;
+      const uint64_t mask = (__ballot(v != 0.0f) >> shift) & group;
+      if (v != 0.0f) {
+        const int pos = cnt + __popcll(mask & ((1ull << lane) - 1));
+        f[pos] = v;
+        rowl[pos] = r;
+      }
+      cnt += __popcll(mask);
+    }
+  }
   __syncthreads();  // every thread of the block reaches the barriers: nothing above returns
   if (work) {
     const float *Jw = a.J + w * (int64_t)a.njmax * a.nv;
     for (int dof = lane; dof < a.nv; dof += L) {
+      const float ma = a.Ma[w * a.ldm + dof], sm = a.smooth[w * a.lds_ + dof];  // on their way beside the rows of J
       float sum = 0.0f;
-      for (int r0 = 0; r0 < nefc; r0 += ROWS) {
+      for (int p0 = 0; p0 < cnt; p0 += ROWS) {
         float jv[ROWS];
 #pragma unroll
-        for (int u = 0; u < ROWS; ++u) jv[u] = Jw[(int64_t)(r0 + u < nefc ? r0 + u : nefc - 1) * a.nv + dof];
+        for (int u = 0; u < ROWS; ++u) jv[u] = Jw[(int64_t)rowl[p0 + u < cnt ? p0 + u : cnt - 1] * a.nv + dof];
 #pragma unroll
-        for (int u = 0; u < ROWS; ++u) sum = r0 + u < nefc ? fmaf(jv[u], f[r0 + u], sum) : sum;
+        for (int u = 0; u < ROWS; ++u) sum = p0 + u < cnt ? fmaf(jv[u], f[p0 + u], sum) : sum;
       }
-      const float g = a.Ma[w * a.ldm + dof] - a.smooth[w * a.lds_ + dof] - sum;
+      const float g = ma - sm - sum;
       if (live) {
         a.qc[w * a.ldq + dof] = sum;
         a.grad[w * a.ldg + dof] = g;
@@ -309,7 +329,7 @@ extern "C" int im_newton_gradient(const int32_t *nefc, const float *J, int njmax
     return IM_ERR_ARG;
   if (ld_force < njmax || ld_smooth < nv || ld_Ma < nv || ld_constraint < nv || ld_grad < nv) return IM_ERR_STRIDE;
   const int lanes = nv <= 32 ? 32 : 64, per_block = kThreads / lanes;
-  const size_t lds_bytes = (size_t)per_block * ((size_t)njmax + nv + 64) * 4;
+  const size_t lds_bytes = (size_t)per_block * (2 * (size_t)njmax + nv + 64) * 4;
   if (lds_bytes > kLdsLimit) return IM_ERR_UNSUPPORTED;
   GradArgs a{nefc, J, efc_force, qfrc_smooth, efc_Ma, alpha, state_changed_count, done, qfrc_constraint, grad,
              grad_dot, newton_decrement, grad_scale, search_unchanged, ld_force, ld_smooth, ld_Ma, ld_constraint,

@@ -341,7 +341,9 @@ def run(launches: int = 32, only: str | None = None) -> None:
         for name, nsets in (("humanoid", 16), ("g1", 8), ("snu", 8)):
             b = synth.make_batch(name)
             nv, nefc, nworld = b.shape.nv, b.shape.nefc, b.nworld
-            Js, Fs = [t(b.J) for _ in range(nsets)], [torch.randn((nworld, nefc), device=dev) for _ in range(nsets)]
+            # a constraint's force is zero unless its state is quadratic, as after the reference's update of the constraints
+            quad_rows = t(b.state[0] == synth.QUADRATIC)
+            Js, Fs = [t(b.J) for _ in range(nsets)], [torch.randn((nworld, nefc), device=dev) * quad_rows for _ in range(nsets)]
             ne, sm, ma = t(b.nefc), t(b.grad), torch.randn((nworld, nv), device=dev)
             chg, al = torch.ones(nworld, dtype=torch.int32, device=dev), torch.zeros(nworld, device=dev)
             qc, gr = torch.zeros((nworld, nv), device=dev), torch.zeros((nworld, nv), device=dev)
