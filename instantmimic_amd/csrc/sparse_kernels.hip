@@ -117,17 +117,29 @@ template <bool WAVE = false>
 __device__ __forceinline__ void backward_sums(const SparseDev &P, float *N, const float *iD,
                                               const float *__restrict__ gw, float *__restrict__ search,
                                               float *red, float *search_dot, float *decrement, int lane,
-                                              int nthreads, int block) {
+                                              int nthreads, int block, const uint32_t *staged = nullptr) {
   const int n = P.nv, rhs = P.nslots - n, nw = (block + 31) / 32;
   const int32_t *ORIGt = P.t[ORIG];
   // backward solve, root level first
   const int32_t *BLt = P.t[BL], *BSt = P.t[BS], *BIt = P.t[BI], *BJt = P.t[BJ];
-  for (int l = 0; l < P.nlevels; ++l) {
-    for (int p = BLt[l] + lane; p < BLt[l + 1]; p += nthreads) {
-      const int i = BIt[p], j = BJt[p];
-      N[rhs + j] = fma_(-N[BSt[p]], N[rhs + i] * iD[i], N[rhs + j]);
+  if (staged) {  // the tables from LDS (stage_backward_tables): no level waits for memory
+    const uint32_t *lev = staged, *push = staged + P.nlevels + 1;
+    for (int l = 0; l < P.nlevels; ++l) {
+      for (int p = lev[l] + lane; p < (int)lev[l + 1]; p += nthreads) {
+        const uint32_t u = push[p];
+        const int i = (u >> 16) & 0xFF, j = u >> 24;
+        N[rhs + j] = fma_(-N[u & 0xFFFFu], N[rhs + i] * iD[i], N[rhs + j]);
+      }
+      sync_world<WAVE>();
     }
-    sync_world<WAVE>();
+  } else {
+    for (int l = 0; l < P.nlevels; ++l) {
+      for (int p = BLt[l] + lane; p < BLt[l + 1]; p += nthreads) {
+        const int i = BIt[p], j = BJt[p];
+        N[rhs + j] = fma_(-N[BSt[p]], N[rhs + i] * iD[i], N[rhs + j]);
+      }
+      sync_world<WAVE>();
+    }
   }
   float s0 = 0.0f, s1 = 0.0f;
   for (int j = lane; j < n && lane < block; j += block) {
@@ -154,6 +166,102 @@ __device__ __forceinline__ void backward_sums(const SparseDev &P, float *N, cons
     }
     *search_dot = ra;
     *decrement = rb;
+  }
+}
+
+// dst[i] = f(i) for i < count, a lane's next eight values asked for before the first is stored: a
+// plain loop waits for every load in turn, and a world's lanes are few.
+template <class F>
+__device__ __forceinline__ void fill_lds(float *dst, int count, int lane, int block, const F &f) {
+  for (int i0 = lane; i0 < count; i0 += 8 * block) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * block;
+      v[u] = f(i < count ? i : count - 1);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * block;
+      if (i < count) dst[i] = v[u];
+    }
+  }
+}
+
+// The backward solve's tables in LDS for backward_sums: [nlevels + 1] first push of each level, then a
+// word per push (slot of the factor entry | row << 16 | column << 24).  For up to 256 dofs and
+// 65535 slots; a barrier must follow before backward_sums reads them.  nlevels + 1 + pushes words.
+__device__ __forceinline__ void stage_backward_tables(const SparseDev &P, uint32_t *staged, int lane, int block) {
+  const int32_t *BLt = P.t[BL], *BSt = P.t[BS], *BIt = P.t[BI], *BJt = P.t[BJ];
+  for (int l = lane; l <= P.nlevels; l += block) staged[l] = (uint32_t)BLt[l];
+  uint32_t *push = staged + P.nlevels + 1;
+  fill_lds((float *)push, BLt[P.nlevels], lane, block, [&](int p) {
+    return __builtin_bit_cast(float, (uint32_t)BSt[p] | ((uint32_t)BIt[p] << 16) | ((uint32_t)BJt[p] << 24));
+  });
+}
+
+// Forward substitution with a stored factor: N[rhs + j] = g[j] - sum_k (N[j,k] / D[k]) N[rhs + k],
+// a lane per row of a level, the row's terms in order.  The rows' tables (row, slot of its first
+// term, place and count of its columns) and the gradient come into LDS first, all rows at once:
+// read level by level from memory, each level waited for three memory round trips in a row.
+// The column numbers of every term come in as 16-bit words: a row's chain of up to n terms runs on
+// one lane, and a trip to memory per handful of terms was most of the kernel.
+// `meta` holds 4 n + 2 + (nfac + 1) / 2 words.
+__device__ __forceinline__ void forward_rhs_levels(const SparseDev &P, float *N, const float *iD,
+                                                   const float *__restrict__ gw, int rhs, int *meta, int lane,
+                                                   int block) {
+  const int n = P.nv;
+  const int32_t *ORIGt = P.t[ORIG];
+  const int32_t *FLt = P.t[FL], *FRt = P.t[FR], *RSt = P.t[RS], *RKPt = P.t[RKP], *RKt = P.t[RK];
+  int *row = meta, *first = meta + n, *cols = meta + 2 * n, *level = meta + 3 * n;  // level: [nlevels + 1]
+  for (int q = lane; q < n; q += block) {
+    const int j = FRt[q], k0 = RKPt[j];
+    row[q] = j | ((RKPt[j + 1] - k0) << 16);
+    first[q] = RSt[j];
+    cols[q] = k0;
+    N[rhs + q] = gw[ORIGt[q]];
+  }
+  for (int l = lane; l <= P.nlevels; l += block) level[l] = FLt[l];
+  unsigned short *rk = (unsigned short *)(meta + 4 * n + 2);  // [nfac] columns of the terms, row after row
+  for (int e0 = lane, nrk = RKPt[n]; e0 < nrk; e0 += 8 * block) {  // nrk <= nfac
+    int kk[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) kk[u] = RKt[e0 + u * block < nrk ? e0 + u * block : nrk - 1];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (e0 + u * block < nrk) rk[e0 + u * block] = (unsigned short)kk[u];
+  }
+  __syncthreads();
+  for (int l = 0; l < P.nlevels; ++l) {
+    for (int q = level[l] + lane; q < level[l + 1]; q += block) {
+      const int j = row[q] & 0xFFFF, len = row[q] >> 16, k0 = cols[q];
+      float v = N[rhs + j];
+      const float *rowp = N + first[q];
+      // whole batches of eight terms without a condition (operand addresses differ by constants
+      // that the LDS instructions carry), then the rest one by one
+      const unsigned short *kp = rk + k0;
+      const float *xs = N + rhs;
+      int t = 0;
+      for (; t + 8 <= len; t += 8) {
+        int k[8];
+        float c[8], xk[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) k[u] = kp[t + u];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          c[u] = -(rowp[t + u] * iD[k[u]]);
+          xk[u] = xs[k[u]];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v = fma_(c[u], xk[u], v);
+      }
+      for (; t < len; ++t) {
+        const int k = kp[t];
+        v = fma_(-(rowp[t] * iD[k]), xs[k], v);
+      }
+      N[rhs + j] = v;
+    }
+    __syncthreads();
   }
 }
 
@@ -761,22 +869,7 @@ __global__ void sparse_update_kernel(SparseDev P, const uint8_t *__restrict__ do
   } else {
     for (int s = lane; s < nfac; s += block) N[s] = U[nfac + s];
     for (int j = lane; j < n; j += block) iD[j] = U[2 * nfac + j];
-    __syncthreads();
-    const int32_t *FLt = P.t[FL], *FRt = P.t[FR], *RSt = P.t[RS], *RKPt = P.t[RKP], *RKt = P.t[RK];
-    for (int l = 0; l < P.nlevels; ++l) {
-      for (int q = FLt[l] + lane; q < FLt[l + 1]; q += block) {
-        const int j = FRt[q];
-        float v = gw[ORIGt[j]];
-        const float *rowp = N + RSt[j];
-        const int k0 = RKPt[j], k1 = RKPt[j + 1];
-        for (int t = 0; t < k1 - k0; ++t) {
-          const int k = RKt[k0 + t];
-          v = fma_(-(rowp[t] * iD[k]), N[rhs + k], v);
-        }
-        N[rhs + j] = v;
-      }
-      __syncthreads();
-    }
+    forward_rhs_levels(P, N, iD, gw, rhs, ul + n, lane, block);
   }
   backward_sums(P, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, block, block);
 }
@@ -807,36 +900,31 @@ __global__ void sparse_dense_factor_kernel(SparseDev P, const uint8_t *__restric
   float *U = U_ + (size_t)w * P.nv_pad * P.nv_pad;
   const float *gw = grad + (size_t)w * ldg;
   const int32_t *ORIGt = P.t[ORIG];
+  // The solves' tables come into LDS, the forward solve's and then the backward solve's in the same
+  // words: a world's share of LDS decides how many worlds a CU holds at once, and with every world
+  // of a batch resident a launch lasts as long as one world's chain.
+  int *meta = (int *)(red + 2 * nw);
+  uint32_t *back = (n <= 256 && nslots <= 65535) ? (uint32_t *)meta : nullptr;
   if (refactor) {
+    if (back) stage_backward_tables(P, back, lane, block);  // every use has a barrier before it
     const float *Hw = H + (size_t)w * ldH;
     const uint32_t *GATt = (const uint32_t *)P.t[GAT];
-    for (int s = lane; s < nfac; s += block) N[s] = Hw[GATt[s]];
-    for (int j = lane; j < n; j += block) N[rhs + j] = gw[ORIGt[j]];
+    fill_lds(N, nfac, lane, block, [&](int s) { return Hw[GATt[s]]; });
+    fill_lds(N + rhs, n, lane, block, [&](int j) { return gw[ORIGt[j]]; });
     __syncthreads();
     factor_levels(P, N, iD, lane, block);
     for (int s = lane; s < nfac; s += block) U[s] = N[s];
     for (int j = lane; j < n; j += block) U[nfac + j] = iD[j];
   } else {
-    for (int s = lane; s < nfac; s += block) N[s] = U[s];
-    for (int j = lane; j < n; j += block) iD[j] = U[nfac + j];
-    __syncthreads();
-    const int32_t *FLt = P.t[FL], *FRt = P.t[FR], *RSt = P.t[RS], *RKPt = P.t[RKP], *RKt = P.t[RK];
-    for (int l = 0; l < P.nlevels; ++l) {
-      for (int q = FLt[l] + lane; q < FLt[l + 1]; q += block) {
-        const int j = FRt[q];
-        float v = gw[ORIGt[j]];
-        const float *rowp = N + RSt[j];
-        const int k0 = RKPt[j], k1 = RKPt[j + 1];
-        for (int t = 0; t < k1 - k0; ++t) {
-          const int k = RKt[k0 + t];
-          v = fma_(-(rowp[t] * iD[k]), N[rhs + k], v);
-        }
-        N[rhs + j] = v;
-      }
+    fill_lds(N, nfac, lane, block, [&](int s) { return U[s]; });
+    fill_lds(iD, n, lane, block, [&](int j) { return U[nfac + j]; });
+    forward_rhs_levels(P, N, iD, gw, rhs, meta, lane, block);  // ends with a barrier
+    if (back) {
+      stage_backward_tables(P, back, lane, block);
       __syncthreads();
     }
   }
-  backward_sums(P, N, iD, gw, search_ + (size_t)w * ld_search, red, search_dot + w, decrement + w, lane, block, block);
+  backward_sums(P, N, iD, gw, search_ + (size_t)w * ld_search, red, search_dot + w, decrement + w, lane, block, block, back);
 }
 
 }  // namespace
@@ -1024,7 +1112,7 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done, con
       return IM_OK;
     }
   }
-  const size_t lds_bytes = 4 * ((size_t)plan->nslots + n + 2 * nw + n);
+  const size_t lds_bytes = 4 * ((size_t)plan->nslots + n + 2 * nw + n + 4 * n + 2 + ((size_t)plan->nfac + 1) / 2);
   if (lds_bytes > 64 * 1024) return IM_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(im::sparse_update_kernel, dim3(nworld), dim3(plan->block), lds_bytes, (hipStream_t)stream, P,
                      done, state_changes, changes, ids, ld_ids, J, njmax, D, state, quad, grad, ldg, hfactor,
@@ -1048,7 +1136,9 @@ int im_sparse_dense_factor(const im_sparse_plan *plan, const uint8_t *done, cons
   for (int i = 0; i < im::NHOST; ++i) P.t[i] = plan->t[i];
   P.nv = plan->nv; P.nv_pad = plan->nv_pad; P.nslots = plan->nslots; P.nlevels = plan->nlevels;
   const int nw = (plan->block + 31) / 32;
-  const size_t lds_bytes = 4 * ((size_t)plan->nslots + plan->nv + 2 * nw);
+  // the forward solve's tables, or the backward solve's (its pushes <= nfac) in the same words
+  const size_t fwd_words = 4 * (size_t)plan->nv + 2 + ((size_t)plan->nfac + 1) / 2, bwd_words = (size_t)plan->nlevels + 1 + plan->nfac;
+  const size_t lds_bytes = 4 * ((size_t)plan->nslots + plan->nv + 2 * nw + (fwd_words > bwd_words ? fwd_words : bwd_words));
   if (lds_bytes > 64 * 1024) return IM_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(im::sparse_dense_factor_kernel, dim3(nworld), dim3(plan->block), lds_bytes, (hipStream_t)stream,
                      P, done, grad, ldg, H, ldH, quad_changed, state_changed, skip_unchanged, skip_noflip, hfactor,
