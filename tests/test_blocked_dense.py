@@ -111,6 +111,43 @@ def test_gpu_dense_hessian_mfma(device, name, nworld):
 
 
 @pytest.mark.gpu
+def test_gpu_dense_hessian_row_counts_and_masks(device):
+    """The dense J'DJ kernel stages rows 0..31 as they lie and, behind them, only the rows that
+    contribute (inside nefc, QUADRATIC).  Row counts on both sides of 32 and of a chunk of 32
+    listed rows, no active row at all, every row active, njmax that is no multiple of 4, and
+    non-finite values in rows that must not be read (inactive, or past nefc)."""
+    import torch
+
+    rng = np.random.default_rng(21)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    for nv, njmax in ((27, 70), (35, 33), (128, 131), (56, 300)):
+        counts = [0, 1, 31, 32, 33, 63, 64, 65, njmax - 1, njmax]
+        nworld = 3 * len(counts)
+        nefc = np.array(counts * 3, np.int32)
+        J = rng.normal(size=(nworld, njmax, nv)).astype(np.float32)
+        D = rng.uniform(0.5, 4.0, (nworld, njmax)).astype(np.float32)
+        state = np.where(rng.uniform(size=(nworld, njmax)) < 0.5, synth.QUADRATIC, 0).astype(np.int32)
+        state[: len(counts)] = 0  # no active row
+        state[len(counts) : 2 * len(counts)] = synth.QUADRATIC  # every row active
+        A = rng.normal(size=(nworld, nv, nv))
+        Md = (A @ A.transpose(0, 2, 1) / nv + np.eye(nv)).astype(np.float32)
+        Jdirty = J.copy()
+        for w in range(nworld):
+            Jdirty[w, nefc[w] :] = np.nan
+            idle = np.flatnonzero(state[w, 32:] != synth.QUADRATIC) + 32  # behind the first chunk
+            Jdirty[w, idle] = np.inf
+        nv_pad = ((nv + 1 + 15) // 16) * 16
+        H = torch.full((nworld, nv_pad, nv_pad), 7.0, device=device)
+        BD.dense_hessian(t(Md), t(Jdirty), t(D), t(state), t(nefc), H)
+        torch.cuda.synchronize()
+        Hh = H.cpu().numpy()[:, :nv, :nv]
+        want = R.jtdj_dense(Md.reshape(nworld, -1), J, D, state, nefc, nv_pad)[:, :nv, :nv]
+        assert np.isfinite(Hh).all(), (nv, njmax)
+        assert R.rel_l2(Hh, want) <= 1e-5, (nv, njmax)
+        np.testing.assert_array_equal(Hh[: len(counts)], Md[: len(counts)])  # M + nothing
+
+
+@pytest.mark.gpu
 def test_gpu_wavefront_per_world_kernel_for_small_tiles_agrees():
     """Matrices up to 64 x 64 run four worlds per wavefront; the kernel with a
     workgroup per world that serves every other shape is forced here in a child process and

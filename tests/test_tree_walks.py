@@ -286,6 +286,7 @@ def _gradient_case(name, nworld, seed=9):
     idle = rng.uniform(size=force.shape)
     force[idle < 0.4] = 0.0
     force[idle < 0.05] = -0.0
+    force[0] = 0.0  # a world without any force
     smooth = rng.normal(0, 1, (nworld, nv)).astype(np.float32)
     Ma = rng.normal(0, 1, (nworld, nv)).astype(np.float32)
     changed = rng.integers(0, 3, nworld).astype(np.int32)  # a third of the worlds keep their states
