@@ -58,53 +58,70 @@ __device__ __forceinline__ void sync_world() {
 // level-scheduled numeric factor: team lanes stride an entry's terms, shuffle-down tree.
 // An entry's value depends on its team width only, not on how many teams work side by side,
 // so `block` may be any multiple of the widest team.
+// One level with the team width T as a compile-time constant: the operands of a lane's next four
+// terms then lie at constant distances, which the LDS instructions carry themselves.
+template <bool WAVE, int T>
+__device__ __forceinline__ void factor_level(const SparseDev &P, float *N, float *iD, int lane, int block, int e0,
+                                             int e1) {
+  const int32_t *ESt = P.t[ES], *ECt = P.t[EC], *RPt = P.t[RP];
+  const uint32_t *RABt = (const uint32_t *)P.t[RAB], *RKLt = (const uint32_t *)P.t[RKL];
+  constexpr int tshift = __builtin_ctz((unsigned)T);
+  const int tl = lane & (T - 1), team = lane >> tshift, teams = block >> tshift;
+  for (int eb = e0; eb < e1; eb += teams) {
+    const int e = eb + team;
+    float v = 0.0f;
+    int sl = 0, col = -1;
+    if (e < e1) {
+      sl = ESt[e];
+      col = ECt[e];
+      for (int r = RPt[e]; r < RPt[e + 1]; ++r) {
+        const uint32_t ab = RABt[r], kl = RKLt[r];
+        const float *pa = N + (ab & 0xFFFFu) + tl, *pb = N + (ab >> 16) + tl, *pd = iD + (kl & 0xFFFFu) + tl;
+        const int len = (int)(kl >> 16) - tl;  // terms from this lane's first on
+        // four terms' operands are read before the first is used; the sum keeps its order
+        int t = 0;
+        for (; t + 3 * T < len; t += 4 * T) {
+          const float a0 = pa[t], b0 = pb[t], d0 = pd[t];
+          const float a1 = pa[t + T], b1 = pb[t + T], d1 = pd[t + T];
+          const float a2 = pa[t + 2 * T], b2 = pb[t + 2 * T], d2 = pd[t + 2 * T];
+          const float a3 = pa[t + 3 * T], b3 = pb[t + 3 * T], d3 = pd[t + 3 * T];
+          v = fma_(a0 * b0, d0, v);
+          v = fma_(a1 * b1, d1, v);
+          v = fma_(a2 * b2, d2, v);
+          v = fma_(a3 * b3, d3, v);
+        }
+        for (; t < len; t += T) v = fma_(pa[t] * pb[t], pd[t], v);
+      }
+    }
+    // shuffle-down tree of the team; inside a row of 16 lanes a DPP shift does it (what a lane
+    // past the team's end receives is never passed on to the team's first lane)
+    if (T > 32) v = v + __shfl_down(v, 32, 64);
+    if (T > 16) v = v + __shfl_down(v, 16, 64);
+    if (T > 8) v = v + row_shl<8>(v);
+    if (T > 4) v = v + row_shl<4>(v);
+    if (T > 2) v = v + row_shl<2>(v);
+    if (T > 1) v = v + row_shl<1>(v);
+    if (e < e1 && tl == 0) {
+      const float wv = N[sl] - v;
+      N[sl] = wv;
+      if (col >= 0) iD[col] = 1.0f / wv;
+    }
+  }
+}
+
 template <bool WAVE = false>
 __device__ __forceinline__ void factor_levels(const SparseDev &P, float *N, float *iD, int lane, int block) {
-  const int32_t *LPt = P.t[LP], *LTt = P.t[LT], *ESt = P.t[ES], *ECt = P.t[EC], *RPt = P.t[RP];
-  const uint32_t *RABt = (const uint32_t *)P.t[RAB], *RKLt = (const uint32_t *)P.t[RKL];
+  const int32_t *LPt = P.t[LP], *LTt = P.t[LT];
   for (int l = 0; l < P.nlevels; ++l) {
-    const int e0 = LPt[l], e1 = LPt[l + 1], T = LTt[l];
-    const int tshift = __builtin_ctz((unsigned)T);  // team widths are powers of two
-    const int tl = lane & (T - 1), team = lane >> tshift, teams = block >> tshift;
-    for (int eb = e0; eb < e1; eb += teams) {
-      const int e = eb + team;
-      float v = 0.0f;
-      int sl = 0, col = -1;
-      if (e < e1) {
-        sl = ESt[e];
-        col = ECt[e];
-        for (int r = RPt[e]; r < RPt[e + 1]; ++r) {
-          const uint32_t ab = RABt[r], kl = RKLt[r];
-          const float *pa = N + (ab & 0xFFFFu), *pb = N + (ab >> 16), *pd = iD + (kl & 0xFFFFu);
-          const int len = (int)(kl >> 16);
-          // four terms' operands are read before the first is used; the sum keeps its order
-          int t = tl;
-          for (; t + 3 * T < len; t += 4 * T) {
-            const float a0 = pa[t], b0 = pb[t], d0 = pd[t];
-            const float a1 = pa[t + T], b1 = pb[t + T], d1 = pd[t + T];
-            const float a2 = pa[t + 2 * T], b2 = pb[t + 2 * T], d2 = pd[t + 2 * T];
-            const float a3 = pa[t + 3 * T], b3 = pb[t + 3 * T], d3 = pd[t + 3 * T];
-            v = fma_(a0 * b0, d0, v);
-            v = fma_(a1 * b1, d1, v);
-            v = fma_(a2 * b2, d2, v);
-            v = fma_(a3 * b3, d3, v);
-          }
-          for (; t < len; t += T) v = fma_(pa[t] * pb[t], pd[t], v);
-        }
-      }
-      // shuffle-down tree of the team; inside a row of 16 lanes a DPP shift does it (what a lane
-      // past the team's end receives is never passed on to the team's first lane)
-      if (T > 32) v = v + __shfl_down(v, 32, 64);
-      if (T > 16) v = v + __shfl_down(v, 16, 64);
-      if (T > 8) v = v + row_shl<8>(v);
-      if (T > 4) v = v + row_shl<4>(v);
-      if (T > 2) v = v + row_shl<2>(v);
-      if (T > 1) v = v + row_shl<1>(v);
-      if (e < e1 && tl == 0) {
-        const float wv = N[sl] - v;
-        N[sl] = wv;
-        if (col >= 0) iD[col] = 1.0f / wv;
-      }
+    const int e0 = LPt[l], e1 = LPt[l + 1];
+    switch (LTt[l]) {  // team widths are powers of two
+      case 1: factor_level<WAVE, 1>(P, N, iD, lane, block, e0, e1); break;
+      case 2: factor_level<WAVE, 2>(P, N, iD, lane, block, e0, e1); break;
+      case 4: factor_level<WAVE, 4>(P, N, iD, lane, block, e0, e1); break;
+      case 8: factor_level<WAVE, 8>(P, N, iD, lane, block, e0, e1); break;
+      case 16: factor_level<WAVE, 16>(P, N, iD, lane, block, e0, e1); break;
+      case 32: factor_level<WAVE, 32>(P, N, iD, lane, block, e0, e1); break;
+      default: factor_level<WAVE, 64>(P, N, iD, lane, block, e0, e1); break;
     }
     sync_world<WAVE>();
   }
