@@ -1272,19 +1272,45 @@ __global__ __launch_bounds__(256) void copy_dense_factor_kernel(const float *__r
 }
 
 // ---------------------------------------------------------------------------- dense J'DJ
-// H[w] = M[w] + J[w]' diag(Dc[w]) J[w], H (nv_pad, nv_pad), on v_mfma_f32_32x32x2_f32.
-// One workgroup of four wavefronts per world, a wavefront per 32 x 32 output tile (the tiles
-// with column block >= row block, dealt round robin, accumulators in registers, mirrored at
-// the end).  J is staged through LDS 32 rows at a time with the row weights beside it, in two
+// H[w] = M[w] + J[w]' diag(Dc[w]) J[w], H (nv_pad, nv_pad), on v_mfma_f32_16x16x4_f32.
+// One workgroup of four wavefronts per world.  The 16 x 16 output tiles on and right of the block
+// diagonal are dealt to the wavefronts round robin (36 tiles at 128 dofs: nine each, where 32 x 32
+// tiles left two wavefronts with two tiles against three), accumulators in registers, mirrored at
+// the end.  J is staged through LDS 32 rows at a time with the row weights beside it, in two
 // copies used in turn; the next 32 rows are already on their way into registers while the matrix
 // cores work on the current ones, and the weighted operand (J Dc) is formed when it is fed.
-typedef float float16v __attribute__((ext_vector_type(16)));
+// An element's sum is the chain fma(J[r][i] * Dc[r], J[r][j], .) over the rows in order, from M.
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+// The 36 tiles of a matrix of eight 16-column blocks, nine per wavefront, chosen so that a
+// wavefront's tiles share operands: wavefronts 0 and 1 take the triangles of blocks 0-3 and 4-7
+// (four blocks read per step of four rows, each also in its weighted form), wavefronts 2 and 3
+// the rectangle of rows 0-1 / 2-3 against columns 4-7 (six blocks read) and, to even the count,
+// one diagonal tile of a block they hold anyway.  {row block, column block}.
+__device__ constexpr signed char kJtdjTile[4][9][2] = {
+    {{0, 1}, {0, 2}, {0, 3}, {1, 1}, {1, 2}, {1, 3}, {2, 2}, {2, 3}, {3, 3}},
+    {{4, 4}, {4, 5}, {4, 6}, {4, 7}, {5, 5}, {5, 6}, {5, 7}, {6, 6}, {6, 7}},
+    {{0, 4}, {0, 5}, {0, 6}, {0, 7}, {1, 4}, {1, 5}, {1, 6}, {1, 7}, {0, 0}},
+    {{2, 4}, {2, 5}, {2, 6}, {2, 7}, {3, 4}, {3, 5}, {3, 6}, {3, 7}, {7, 7}},
+};
+constexpr bool jtdj_role_reads(int role, int b) {  // does a wavefront of this role use block b at all
+  for (int m = 0; m < 9; ++m)
+    if (kJtdjTile[role][m][0] == b || kJtdjTile[role][m][1] == b) return true;
+  return false;
+}
+constexpr bool jtdj_role_weights(int role, int b) {  // ... and in its weighted form (as a tile's row block)
+  for (int m = 0; m < 9; ++m)
+    if (kJtdjTile[role][m][0] == b) return true;
+  return false;
+}
 
 // NVR: the staged row width when it is known at compile time (operand addresses then differ by
 // constants that the LDS instructions carry themselves), 0 for any width.
+// ROLE: 0..3 = this wavefront's row of kJtdjTile (eight blocks, NVR 128), -1 = tiles dealt round
+// robin at run time, each with operand reads of its own.
 // `out(i, j, h)` receives every element i <= j < nv of H once, from the lane that holds it.
-template <int NVR, class Out>
-__device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
+template <int NVR, int ROLE, class Out>
+__device__ __forceinline__ void jtdj_tiles_as(const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
                                            const float *__restrict__ D, const int32_t *__restrict__ state,
                                            const int32_t *__restrict__ nefc_p, int quad, int nv, float *lds,
                                            const Out &out) {
@@ -1296,42 +1322,51 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
   float *dcs = Js + 32 * nvr;            // [32] their weights
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t w = blockIdx.x;
-  const int nb = nvr / 32;
+  const int nb = (nv + 15) / 16;
+  // A matrix-core operand is 16 columns of four consecutive rows, which lie a whole number of
+  // bank rounds apart: the 16-column groups of a row are stored exchanged by the row's number
+  // (all four ways where the width is a multiple of 64, two ways otherwise), so the four rows of
+  // a request fall on different banks.
+  const int swz = nvr % 64 == 0 ? 3 : 1;
+  const int kq = lane >> 4, kqs = kq & swz;
   // tiles (bi <= bj) distributed over the four waves; each wave keeps its tiles' accumulators
-  constexpr int MAXT = 3;                // up to 10 tiles (nv <= 128) over 4 waves
-  float16v acc[MAXT];
+  constexpr int MAXT = 9;                // up to 36 tiles (nv <= 128) over 4 waves
+  float4v acc[MAXT];
   int tbi[MAXT], tbj[MAXT], mine = 0;
-  {
+  if (ROLE >= 0) {
+#pragma unroll
+    for (int m = 0; m < MAXT; ++m) {
+      tbi[m] = kJtdjTile[ROLE < 0 ? 0 : ROLE][m][0];
+      tbj[m] = kJtdjTile[ROLE < 0 ? 0 : ROLE][m][1];
+    }
+    mine = MAXT;
+  } else {
     int t = 0;
 #pragma unroll
     for (int m = 0; m < MAXT; ++m) tbi[m] = tbj[m] = 0;
     for (int bi = 0; bi < nb; ++bi)
       for (int bj = bi; bj < nb; ++bj, ++t)
-        if (t % 4 == wave) {
-          if (mine == 0) { tbi[0] = bi; tbj[0] = bj; }
-          else if (mine == 1) { tbi[1] = bi; tbj[1] = bj; }
-          else if (mine == 2) { tbi[2] = bi; tbj[2] = bj; }
+        if ((t & 3) == wave) {
+#pragma unroll
+          for (int m = 0; m < MAXT; ++m)
+            if (mine == m) { tbi[m] = bi; tbj[m] = bj; }
           ++mine;
         }
     mine = mine < MAXT ? mine : MAXT;
   }
-  // The accumulators start from M (accumulator layout of a 32x32 tile: lane l holds column
-  // j = l % 32 and, in register 4 * g + v, row i = 8 * g + 4 * (l / 32) + v): every lane asks for
-  // all its elements at once, with clamped indices so that no load hangs on a condition, and the
-  // answers arrive while the first rows of J are staged.  Read at the end instead, behind the
-  // conditions of the stores, the same loads ran one after the other and took as long as the
-  // matrix-core loops.
+  // The accumulators start from M (accumulator layout of a 16x16 tile: lane l holds column
+  // j = l % 16 and, in register v, row i = 4 * (l / 16) + v): every lane asks for all its elements
+  // at once, with clamped indices so that no load hangs on a condition, and the answers arrive
+  // while the first rows of J are staged.
   const float *Mw = Mdense + w * (int64_t)nv * nv;
 #pragma unroll
   for (int m = 0; m < MAXT; ++m) {
-    const int j = tbj[m] * 32 + (lane & 31), jc = j < nv ? j : nv - 1;
+    const int j = tbj[m] * 16 + (lane & 15), jc = j < nv ? j : nv - 1;
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int i = tbi[m] * 32 + 8 * g + (lane >> 5) * 4 + v, ic = i < nv ? i : nv - 1;
-        acc[m][4 * g + v] = Mw[(int64_t)ic * nv + jc];
-      }
+    for (int v = 0; v < 4; ++v) {
+      const int i = tbi[m] * 16 + 4 * kq + v, ic = i < nv ? i : nv - 1;
+      acc[m][v] = Mw[(int64_t)ic * nv + jc];
+    }
   }
   int nefc = nefc_p ? nefc_p[w] : njmax;
   nefc = nefc < njmax ? nefc : njmax;
@@ -1396,8 +1431,9 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const bool in = p0 + wave * 8 + i < (listed ? cnt : nefc);
-      if (c0 < nvr) Jb[(wave * 8 + i) * nvr + c0] = (in && c0 < nv) ? v0[i] : 0.0f;  // nvr is 32 for nv <= 32
-      if (c1 < nvr) Jb[(wave * 8 + i) * nvr + c1] = (in && c1 < nv) ? v1[i] : 0.0f;
+      const int x = 16 * ((wave * 8 + i) & swz);  // the row's exchange of its 16-column groups
+      if (c0 < nvr) Jb[(wave * 8 + i) * nvr + (c0 ^ x)] = (in && c0 < nv) ? v0[i] : 0.0f;  // nvr is 32 for nv <= 32
+      if (c1 < nvr) Jb[(wave * 8 + i) * nvr + (c1 ^ x)] = (in && c1 < nv) ? v1[i] : 0.0f;
     }
     if (lane < 8) {
       const int pos = p0 + wave * 8 + lane;
@@ -1409,23 +1445,42 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
   const int nchunk = nefc > 0 ? 1 + (cnt + 31) / 32 : 0;
   for (int c = 0, buf = 0; c < nchunk; ++c, buf ^= 1) {
     prefetch(32 * c);
-    // v_mfma_f32_32x32x2_f32: lane l supplies A[i = l % 32][k = l / 32] and B[k = l / 32][j = l % 32]
+    // v_mfma_f32_16x16x4_f32: lane l supplies A[i = l % 16][k = l / 16] and B[k = l / 16][j = l % 16]
     // the wavefront's tiles take turns inside the loop over the rows: independent accumulators
     // keep the matrix core busy while one of them waits for its previous result
-    const float *pa[MAXT], *pb[MAXT];
     const float *Jc = Js + buf * stage_words, *dc = dcs + buf * stage_words;
+    if (ROLE >= 0) {
+      constexpr int R = ROLE < 0 ? 0 : ROLE;
+      const float *pblk[8];
 #pragma unroll
-    for (int m = 0; m < MAXT; ++m) {
-      pa[m] = Jc + (lane >> 5) * nvr + tbi[m] * 32 + (lane & 31);
-      pb[m] = Jc + (lane >> 5) * nvr + tbj[m] * 32 + (lane & 31);
-    }
+      for (int b = 0; b < 8; ++b) pblk[b] = Jc + kq * nvr + (b ^ kqs) * 16 + (lane & 15);
 #pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      const float dk = dc[2 * q + (lane >> 5)];
+      for (int q = 0; q < 8; ++q) {
+        const float dk = dc[4 * q + kq];
+        float u[8], wt[8];
 #pragma unroll
-      for (int m = 0; m < MAXT; ++m)
-        if (m < mine)
-          acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[m][2 * q * nvr] * dk, pb[m][2 * q * nvr], acc[m], 0, 0, 0);
+        for (int b = 0; b < 8; ++b) u[b] = jtdj_role_reads(R, b) ? pblk[b][4 * q * nvr] : 0.0f;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) wt[b] = jtdj_role_weights(R, b) ? u[b] * dk : 0.0f;
+#pragma unroll
+        for (int m = 0; m < MAXT; ++m)
+          acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(wt[kJtdjTile[R][m][0]], u[kJtdjTile[R][m][1]], acc[m], 0, 0, 0);
+      }
+    } else {
+      const float *pa[MAXT], *pb[MAXT];
+#pragma unroll
+      for (int m = 0; m < MAXT; ++m) {
+        pa[m] = Jc + kq * nvr + (tbi[m] ^ kqs) * 16 + (lane & 15);
+        pb[m] = Jc + kq * nvr + (tbj[m] ^ kqs) * 16 + (lane & 15);
+      }
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float dk = dc[4 * q + kq];
+#pragma unroll
+        for (int m = 0; m < MAXT; ++m)
+          if (m < mine)
+            acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[m][4 * q * nvr] * dk, pb[m][4 * q * nvr], acc[m], 0, 0, 0);
+      }
     }
     // the other copy was last read one chunk ago, before the barrier that every wavefront has passed since
     stage(32 * c, buf ^ 1, true);
@@ -1434,14 +1489,29 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
 #pragma unroll
   for (int m = 0; m < MAXT; ++m) {
     if (m >= mine) continue;
-    const int j = tbj[m] * 32 + (lane & 31);
+    const int j = tbj[m] * 16 + (lane & 15);
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int i = tbi[m] * 32 + 8 * g + (lane >> 5) * 4 + v;
-        if (i < nv && j < nv && i <= j) out(i, j, acc[m][4 * g + v]);
-      }
+    for (int v = 0; v < 4; ++v) {
+      const int i = tbi[m] * 16 + 4 * kq + v;
+      if (i < nv && j < nv && i <= j) out(i, j, acc[m][v]);
+    }
+  }
+}
+
+template <int NVR, class Out>
+__device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
+                                           const float *__restrict__ D, const int32_t *__restrict__ state,
+                                           const int32_t *__restrict__ nefc_p, int quad, int nv, float *lds,
+                                           const Out &out) {
+  if (NVR == 128 && nv > 112) {  // eight blocks: a code path per wavefront (every path has the same barriers)
+    switch (threadIdx.x >> 6) {
+      case 0: jtdj_tiles_as<NVR, 0>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, out); break;
+      case 1: jtdj_tiles_as<NVR, 1>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, out); break;
+      case 2: jtdj_tiles_as<NVR, 2>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, out); break;
+      default: jtdj_tiles_as<NVR, 3>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, out); break;
+    }
+  } else {
+    jtdj_tiles_as<NVR, -1>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, out);
   }
 }
 

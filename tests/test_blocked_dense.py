@@ -172,19 +172,33 @@ def test_gpu_wavefront_per_world_kernel_for_small_tiles_agrees():
 
 def test_dense_hessian_staging_indices_stay_inside_a_row():
     """The staging step of the dense J'DJ kernel writes row r of a 32-row chunk at
-    Js[r * nvr + c] for the columns c = lane and lane + 64 that lie below nvr = the dofs rounded
-    up to 32 (csrc/blocked_kernels.hip, stage()): replayed here for every supported width, every
-    element of the chunk is written exactly once and nothing outside it."""
+    Js[r * nvr + (c ^ x)] for the columns c = lane and lane + 64 that lie below nvr = the dofs
+    rounded up to 32, with x = 16 * (r & 3) where nvr is a multiple of 64 and 16 * (r & 1)
+    otherwise (csrc/blocked_kernels.hip, stage()): replayed here for every supported width, every
+    element of the chunk is written exactly once and nothing outside it, and the operand reads
+    of the matrix-core loop (row 4 q + l / 16, column block b exchanged the same way) find
+    column 16 b + l % 16 of that row."""
     for nv in (1, 14, 27, 32, 33, 35, 56, 64, 65, 96, 128):
         nvr = (nv + 31) // 32 * 32
+        swz = 3 if nvr % 64 == 0 else 1
         hits = np.zeros(32 * nvr + 32, int)
+        where = {}
         for wave in range(4):
             for lane in range(64):
                 for i in range(8):
                     for c in (lane, lane + 64):
                         if c < nvr:
-                            hits[(wave * 8 + i) * nvr + c] += 1
+                            r = wave * 8 + i
+                            at = r * nvr + (c ^ (16 * (r & swz)))
+                            hits[at] += 1
+                            where[r, c] = at
         assert (hits[: 32 * nvr] == 1).all() and (hits[32 * nvr :] == 0).all(), nv
+        for lane in range(64):
+            kq = lane >> 4
+            for q in range(8):
+                for b in range((nv + 15) // 16):
+                    read = kq * nvr + ((b ^ (kq & swz)) * 16) + (lane & 15) + 4 * q * nvr
+                    assert read == where[4 * q + kq, 16 * b + (lane & 15)], (nv, lane, q, b)
 
 
 def test_multi_solve_oracle_against_the_single_solve_and_fp64():
