@@ -1308,7 +1308,8 @@ constexpr bool jtdj_role_weights(int role, int b) {  // ... and in its weighted 
 // constants that the LDS instructions carry themselves), 0 for any width.
 // ROLE: 0..3 = this wavefront's row of kJtdjTile (eight blocks, NVR 128), -1 = tiles dealt round
 // robin at run time, each with operand reads of its own.
-// `out(i, j, h)` receives every element i <= j < nv of H once, from the lane that holds it.
+// `out(i0, j, h, off)` receives what a lane holds of each tile: rows i0 .. i0 + 3 of column j (the
+// elements with i <= j < nv are H's), and whether the tile lies right of the diagonal blocks.
 template <int NVR, int ROLE, class Out>
 __device__ __forceinline__ void jtdj_tiles_as(const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
                                            const float *__restrict__ D, const int32_t *__restrict__ state,
@@ -1489,12 +1490,25 @@ __device__ __forceinline__ void jtdj_tiles_as(const float *__restrict__ Mdense, 
 #pragma unroll
   for (int m = 0; m < MAXT; ++m) {
     if (m >= mine) continue;
-    const int j = tbj[m] * 16 + (lane & 15);
+    out(tbi[m] * 16 + 4 * kq, tbj[m] * 16 + (lane & 15), acc[m], tbi[m] != tbj[m]);
+  }
+}
+
+// Stores what one lane holds of a tile into H and its mirror image: rows i0 .. i0 + 3 of column j
+// (the elements with i <= j < nv count).  Right of the diagonal blocks (`off`) the mirror image of a
+// lane's four values is four consecutive words of row j: one 16-byte store where H allows it (`vec`).
+__device__ __forceinline__ void store_h_mirrored(float *__restrict__ Hw, int nv, int nv_pad, bool vec, int i0, int j,
+                                                 float4v h, bool off) {
+  if (j >= nv) return;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int i = tbi[m] * 16 + 4 * kq + v;
-      if (i < nv && j < nv && i <= j) out(i, j, acc[m][v]);
-    }
+  for (int v = 0; v < 4; ++v)
+    if (i0 + v < nv && i0 + v <= j) Hw[(int64_t)(i0 + v) * nv_pad + j] = h[v];
+  if (off && vec && i0 + 3 < nv) {
+    *(float4v *)(Hw + (int64_t)j * nv_pad + i0) = h;
+  } else {
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      if (i0 + v < nv && i0 + v < j) Hw[(int64_t)j * nv_pad + i0 + v] = h[v];
   }
 }
 
@@ -1515,17 +1529,19 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
   }
 }
 
+// four workgroups per CU at 128 dofs (measured 0.83 -> 0.77 ms for 16384 worlds in spite of the
+// spilled registers), three otherwise
 template <int NVR>
-__global__ __launch_bounds__(256, 3) void jtdj_mfma_kernel(
+__global__ __launch_bounds__(256, NVR == 128 ? 4 : 3) void jtdj_mfma_kernel(
     const float *__restrict__ Mdense, const float *__restrict__ J, int njmax,
     const float *__restrict__ D, const int32_t *__restrict__ state, const int32_t *__restrict__ nefc_p,
     int quad, float *__restrict__ H, int nv, int nv_pad) {
   extern __shared__ float lds[];
   float *Hw = H + blockIdx.x * (int64_t)nv_pad * nv_pad;
   // upper triangle from the accumulators, lower triangle mirrored: H is symmetric bit for bit
-  jtdj_tiles<NVR>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, [&](int i, int j, float h) {
-    Hw[(int64_t)i * nv_pad + j] = h;
-    if (i != j) Hw[(int64_t)j * nv_pad + i] = h;
+  const bool vec = (nv_pad & 3) == 0 && ((uintptr_t)H & 15) == 0;
+  jtdj_tiles<NVR>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, [&](int i0, int j, float4v h, bool off) {
+    store_h_mirrored(Hw, nv, nv_pad, vec, i0, j, h, off);
   });
 }
 
@@ -1557,12 +1573,12 @@ __global__ __launch_bounds__(256, 4) void jtdj_factor_solve_kernel(
   // go where the rows were staged.  The factor reads the upper triangle below nv only (the rest
   // of a diagonal tile by symmetry, the padding as the identity) and writes every entry of a block
   // row before anything reads it, so the array needs no clearing.
-  jtdj_tiles<NVR>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, [&](int i, int j, float h) {
-    if (Hw) {
-      Hw[(int64_t)i * nv_pad + j] = h;
-      if (i != j) Hw[(int64_t)j * nv_pad + i] = h;
-    }
-    U[S.at(i, j)] = h;
+  const bool vec = (nv_pad & 3) == 0 && ((uintptr_t)H & 15) == 0;
+  jtdj_tiles<NVR>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, [&](int i0, int j, float4v h, bool off) {
+    if (Hw) store_h_mirrored(Hw, nv, nv_pad, vec, i0, j, h, off);
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      if (i0 + v < nv && j < nv && i0 + v <= j) U[S.at(i0 + v, j)] = h[v];
   });
   __syncthreads();
   const LdsSrc<B> src{U, nv, pad};
