@@ -203,7 +203,12 @@ def run(launches: int = 32, only: str | None = None) -> None:
         H = torch.zeros((nworld, pad, pad), device=dev)
         wl = f"stress nv={nv} nefc={nefc} x {nworld} worlds"
         sec = _timeit(torch, lambda i: BD.dense_hessian(Md, J, D, st, ne, H), 1, 8)
-        _line("im_jtdj_mfma", wl, sec, flops=nworld * 2.0 * nv * nv * nefc, nworld=nworld)
+        # the product the matrix cores execute: the 16 x 16 tiles on and right of the diagonal blocks, over the first 32 rows
+        # and the contributing rows behind them in chunks of 32 (the full square over every row would be 2 nv^2 nefc)
+        tail = ((b.state[0][:, 32:] == synth.QUADRATIC) & (np.arange(32, nefc)[None, :] < b.nefc[:, None])).sum(1)
+        chunks = np.where(b.nefc > 0, 1 + (tail + 31) // 32, 0)
+        nb16 = (nv + 15) // 16
+        _line("im_jtdj_mfma (flops executed on the matrix cores)", wl, sec, flops=float(chunks.sum()) * 32 * (nb16 * (nb16 + 1) // 2) * 512, nworld=nworld)
         _line("im_jtdj_mfma (as bytes)", wl, sec, bytes_=nworld * 4 * (nv * nv + nefc * nv + 2 * nefc + pad * pad), nworld=nworld)
         mm = SimpleNamespace(nv=nv, M_tiles=[SimpleNamespace(size=nv, elemid=np.arange(nv * nv))])
         Hc = H[:, :nv, :nv].contiguous().reshape(nworld, -1)
