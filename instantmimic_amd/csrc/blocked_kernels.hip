@@ -928,6 +928,9 @@ __global__ __launch_bounds__(256, 4) void dense_update_factor_kernel(
       constexpr int HELD = 9;  // tiles a wavefront keeps sums for at a time (36 over 4 wavefronts at nv 128: one pass over the rows); more tiles take another pass
       const int lane = tid & 63, p = lane & 15, kq = lane >> 4, wv = tid >> 6, nwv = nt >> 6;
       const int nb = (nv + 15) / 16, ntiles = nb * (nb + 1) / 2;
+      // one pass holds every tile (always, with four wavefronts and up to 128 dofs)
+      const bool one_pass = ntiles <= HELD * nwv;
+      const bool FILLS = false;  // the lanes that add the sums to H also leave the new H in the factor's array
       // thread t asks for the number and the signed weight of changed row t once, at the start: a
       // batch then finds them in registers instead of making two trips to memory of its own
       const bool ids_held = count <= nt;
@@ -1002,32 +1005,61 @@ __global__ __launch_bounds__(256, 4) void dense_update_factor_kernel(
               if (ra[h] >= 0) {  // the same for the whole wavefront
                 const float a = ra[h] < nv ? wgt * row[ra[h]] : 0.0f;  // -(D a) == (-D) a exactly
                 const float b = (t < nrow && ca[h] < nv) ? row[ca[h]] : 0.0f;
-                acc[h] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[h], 0, 0, 0);
+                // operands exchanged: the lane then holds four consecutive columns of one row of H's tile
+                // (16 bytes of H) instead of four rows of one column; a product's bits do not depend on the order
+                acc[h] = __builtin_amdgcn_mfma_f32_16x16x4f32(b, a, acc[h], 0, 0, 0);
               }
             }
           }
         }
         // H's elements of up to five held tiles are requested before the first of their sums is added
-        // (all nine at once would take the registers that let four worlds share a CU)
+        // (all nine at once would take the registers that let four worlds share a CU).  A lane holds
+        // row ra[h] of the tile, columns 4 kq .. 4 kq + 3: right of the diagonal blocks and inside the
+        // dofs that is one 16-byte request; elsewhere element by element.
         constexpr int APPLY = 5;
+        const bool vec = ((uintptr_t)Hw & 15) == 0;  // pad is a multiple of 16
 #pragma unroll
         for (int h0 = 0; h0 < HELD; h0 += APPLY) {
-          float hv[APPLY][4];
+          f32x4 hv[APPLY];
 #pragma unroll
-          for (int h = h0; h < h0 + APPLY && h < HELD; ++h)
+          for (int h = h0; h < h0 + APPLY && h < HELD; ++h) {
+            const int row = ra[h], col0 = ca[h] - p + 4 * kq;
+            const bool wide = vec && ra[h] >= 0 && ra[h] - p != ca[h] - p && row < nv && col0 + 3 < nv;
+            const bool any = acc[h][0] != 0.0f || acc[h][1] != 0.0f || acc[h][2] != 0.0f || acc[h][3] != 0.0f;
+            hv[h - h0] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            if (wide) {
+              if (any || FILLS) hv[h - h0] = *(const f32x4 *)(Hw + (size_t)row * pad + col0);
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int row = ra[h] - p + 4 * kq + i, col = ca[h];
-              const bool mine = ra[h] >= 0 && row <= col && col < nv && acc[h][i] != 0.0f;
-              hv[h - h0][i] = mine ? Hw[(size_t)row * pad + col] : 0.0f;
+              for (int i = 0; i < 4; ++i) {
+                const bool mine = ra[h] >= 0 && row <= col0 + i && col0 + i < nv && (FILLS || acc[h][i] != 0.0f);
+                hv[h - h0][i] = mine ? Hw[(size_t)row * pad + col0 + i] : 0.0f;
+              }
             }
+          }
 #pragma unroll
-          for (int h = h0; h < h0 + APPLY && h < HELD; ++h)
+          for (int h = h0; h < h0 + APPLY && h < HELD; ++h) {
+            const int row = ra[h], col0 = ca[h] - p + 4 * kq;
+            const bool wide = vec && ra[h] >= 0 && ra[h] - p != ca[h] - p && row < nv && col0 + 3 < nv;
+            const bool any = acc[h][0] != 0.0f || acc[h][1] != 0.0f || acc[h][2] != 0.0f || acc[h][3] != 0.0f;
+            f32x4 hn = hv[h - h0];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int row = ra[h] - p + 4 * kq + i, col = ca[h];
-              if (ra[h] >= 0 && row <= col && col < nv && acc[h][i] != 0.0f) Hw[(size_t)row * pad + col] = hv[h - h0][i] + acc[h][i];
+            for (int i = 0; i < 4; ++i)
+              if (acc[h][i] != 0.0f) hn[i] = hn[i] + acc[h][i];
+            if (wide) {
+              if (any) *(f32x4 *)(Hw + (size_t)row * pad + col0) = hn;
+            } else {
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (ra[h] >= 0 && row <= col0 + i && col0 + i < nv && acc[h][i] != 0.0f) Hw[(size_t)row * pad + col0 + i] = hn[i];
             }
+            if (FILLS && ra[h] >= 0) {  // zero below the diagonal and past the dofs
+              f32x4 o;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) o[i] = (row <= col0 + i && col0 + i < nv) ? hn[i] : 0.0f;
+              *(f32x4 *)(U + S.at(row, col0)) = o;
+            }
+          }
         }
       }
       __syncthreads();  // the rows are done with the array; this workgroup's writes to H are read back below
