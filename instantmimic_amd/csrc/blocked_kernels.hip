@@ -930,7 +930,7 @@ __global__ __launch_bounds__(256, 4) void dense_update_factor_kernel(
       const int nb = (nv + 15) / 16, ntiles = nb * (nb + 1) / 2;
       // one pass holds every tile (always, with four wavefronts and up to 128 dofs)
       const bool one_pass = ntiles <= HELD * nwv;
-      const bool FILLS = false;  // the lanes that add the sums to H also leave the new H in the factor's array
+      const bool FILLS = one_pass;  // the lanes that add the sums to H also leave the new H in the factor's array
       // thread t asks for the number and the signed weight of changed row t once, at the start: a
       // batch then finds them in registers instead of making two trips to memory of its own
       const bool ids_held = count <= nt;
@@ -1018,6 +1018,7 @@ __global__ __launch_bounds__(256, 4) void dense_update_factor_kernel(
         // dofs that is one 16-byte request; elsewhere element by element.
         constexpr int APPLY = 5;
         const bool vec = ((uintptr_t)Hw & 15) == 0;  // pad is a multiple of 16
+        if (one_pass) __syncthreads();  // the rows are done with the array: the new H goes there as well
 #pragma unroll
         for (int h0 = 0; h0 < HELD; h0 += APPLY) {
           f32x4 hv[APPLY];
@@ -1064,7 +1065,7 @@ __global__ __launch_bounds__(256, 4) void dense_update_factor_kernel(
       }
       __syncthreads();  // the rows are done with the array; this workgroup's writes to H are read back below
       // 16 bytes per lane and four requests in flight; the tiles below the diagonal are not read
-      const int nvec = pf * pf / 4, last = (pf - 1) * (pad / 4) + pf / 4 - 1;  // pf is a multiple of 16
+      const int nvec = FILLS ? 0 : pf * pf / 4, last = (pf - 1) * (pad / 4) + pf / 4 - 1;  // pf is a multiple of 16
       for (int i0 = tid; i0 < nvec; i0 += 4 * nt) {
         float4 v[4];
 #pragma unroll
