@@ -302,6 +302,42 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
   const int nblk = pad / B;
   constexpr int BB = B * B;
   const Stair<B> S{pad};
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  // v -= the sums over the finished block rows jb0 .. jb1 - 1 for the 16 x 16 tile at columns i0 of
+  // the block row at columns k0, in the block rows' order.  One wavefront, the sums on the matrix
+  // cores: v_mfma_f32_16x16x4_f32 adds its four products to the accumulator one after the other,
+  // each with a fused multiply-add, so four of them chained from zero are the sum over
+  // t = 0..15 ascending of the scalar form.  Two block rows at a time: their sums are
+  // independent chains on the matrix cores (four at a time measured the same).
+  auto schur = [&](f32x4 &v, int k0, int i0, int jb0, int jb1) {
+    const int lane = tid & 63, p = lane & 15, kq = lane >> 4;
+    int jb = jb0;
+    for (; jb + 1 < jb1; jb += 2) {
+      f32x4 sum0 = {0.0f, 0.0f, 0.0f, 0.0f}, sum1 = sum0;
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) {
+        const int at0 = S.in_band(jb, 4 * s4 + kq, p), at1 = S.in_band(jb + 1, 4 * s4 + kq, p);
+        const float a0 = U[at0 + k0], b0 = U[at0 + i0], a1 = U[at1 + k0], b1 = U[at1 + i0];
+        sum0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0, sum0, 0, 0, 0);
+        sum1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1, sum1, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (v[i] - sum0[i]) - sum1[i];
+    }
+    if (jb < jb1) {
+      f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) {
+        const int at = S.in_band(jb, 4 * s4 + kq, p);
+        const float a = U[at + k0], b = U[at + i0];
+        sum = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, sum, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = v[i] - sum[i];
+    }
+  };
+  // look-ahead: while wavefront 0 factors a diagonal tile, the others prepare the next block row
+  const bool ahead = B == 16 && nt > 64;
   for (int kb = 0; kb < nblk; ++kb) {
     const int k = kb * B;
     // the whole block row kb..nblk-1 minus the finished block rows above, in place: a tile's
@@ -309,42 +345,22 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
     // writes them, and the block rows above are final
     const int ntile = nblk - kb;
     if constexpr (B == 16) {
-      // One wavefront per 16 x 16 tile, the sums over a finished block row on the matrix cores:
-      // v_mfma_f32_16x16x4_f32 adds its four products to the accumulator one after the other,
-      // each with a fused multiply-add, so four of them chained from zero are the sum over
-      // t = 0..15 ascending of the scalar form.
-      typedef float f32x4 __attribute__((ext_vector_type(4)));
+      // One wavefront per 16 x 16 tile.
+      // With more than one wavefront, the sums over the block rows above the last finished one were
+      // subtracted while that one's diagonal tile was factored (below), and what is left here is
+      // the last block row's sum.
       const int lane = tid & 63, p = lane & 15, kq = lane >> 4;
       for (int tb = tid >> 6; tb < ntile; tb += nt >> 6) {
         const int ib = kb + tb, i0 = ib * B;
         f32x4 v;
+        if (ahead && kb > 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = src.load(kb, ib, (4 * kq + i) * B + p, 4 * kq + i, p);
-        // two finished block rows at a time: their sums are independent chains on the matrix
-        // cores; they are subtracted in the block rows' order (four at a time measured the same)
-        int jb = 0;
-        for (; jb + 1 < kb; jb += 2) {
-          f32x4 sum0 = {0.0f, 0.0f, 0.0f, 0.0f}, sum1 = sum0;
+          for (int i = 0; i < 4; ++i) v[i] = U[S.in_band(kb, 4 * kq + i, i0 + p)];
+          schur(v, k, i0, kb - 1, kb);
+        } else {
 #pragma unroll
-          for (int s4 = 0; s4 < 4; ++s4) {
-            const int at0 = S.in_band(jb, 4 * s4 + kq, p), at1 = S.in_band(jb + 1, 4 * s4 + kq, p);
-            const float a0 = U[at0 + k], b0 = U[at0 + i0], a1 = U[at1 + k], b1 = U[at1 + i0];
-            sum0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b0, sum0, 0, 0, 0);
-            sum1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1, sum1, 0, 0, 0);
-          }
-#pragma unroll
-          for (int i = 0; i < 4; ++i) v[i] = (v[i] - sum0[i]) - sum1[i];
-        }
-        if (jb < kb) {
-          f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-          for (int s4 = 0; s4 < 4; ++s4) {
-            const int at = S.in_band(jb, 4 * s4 + kq, p);
-            const float a = U[at + k], b = U[at + i0];
-            sum = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, sum, 0, 0, 0);
-          }
-#pragma unroll
-          for (int i = 0; i < 4; ++i) v[i] = v[i] - sum[i];
+          for (int i = 0; i < 4; ++i) v[i] = src.load(kb, ib, (4 * kq + i) * B + p, 4 * kq + i, p);
+          schur(v, k, i0, 0, kb);
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) U[S.in_band(kb, 4 * kq + i, i0 + p)] = v[i];
@@ -399,6 +415,20 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
         for (int j = 0; j < B; ++j) L[j * B + i] = a[j];  // column j of the factor in a row of L; entries above the diagonal are never read
         rhs[k + i] = my_z;
         L[B * B + i] = my_rinv;  // reciprocals of the pivots, behind the tile
+      }
+    } else if (ahead && kb + 1 < nblk) {
+      // Meanwhile the other wavefronts prepare the next block row: its tiles minus the sums over
+      // the block rows above this one, which are final.  This block row's own sum follows when it
+      // is finished, so every element still sees its subtractions in ascending order.
+      const int lane = tid & 63, p = lane & 15, kq = lane >> 4;
+      for (int tb = (tid >> 6) - 1; tb < ntile - 1; tb += (nt >> 6) - 1) {
+        const int ib = kb + 1 + tb, i0 = ib * B;
+        f32x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = src.load(kb + 1, ib, (4 * kq + i) * B + p, 4 * kq + i, p);
+        schur(v, k + B, i0, 0, kb);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) U[S.in_band(kb + 1, 4 * kq + i, i0 + p)] = v[i];
       }
     }
     __syncthreads();
