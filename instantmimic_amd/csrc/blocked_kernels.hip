@@ -451,18 +451,23 @@ __device__ __forceinline__ void factor_forward(const Src &src, float *U, float *
         const float4 t4 = L4[B * B / 4 + q4];
         rinv[4 * q4] = t4.x, rinv[4 * q4 + 1] = t4.y, rinv[4 * q4 + 2] = t4.z, rinv[4 * q4 + 3] = t4.w;
       }
-#pragma unroll
-      for (int j = 0; j < B; ++j) {
-        const float z = col[j] * rinv[j];
-        col[j] = z;
-        float lt[B];
+      // the entries of L for step j + 1 are asked for before step j's chain of multiply-adds
+      float lt[2][B];
+      auto fetch = [&](int j, float *to) {
 #pragma unroll
         for (int q4 = (j + 1) / 4; q4 < B / 4; ++q4) {
           const float4 t4 = L4[j * (B / 4) + q4];
-          lt[4 * q4] = t4.x, lt[4 * q4 + 1] = t4.y, lt[4 * q4 + 2] = t4.z, lt[4 * q4 + 3] = t4.w;
+          to[4 * q4] = t4.x, to[4 * q4 + 1] = t4.y, to[4 * q4 + 2] = t4.z, to[4 * q4 + 3] = t4.w;
         }
+      };
+      fetch(0, lt[0]);
 #pragma unroll
-        for (int i = j + 1; i < B; ++i) col[i] = fma_(-lt[i], z, col[i]);
+      for (int j = 0; j < B; ++j) {
+        if (j + 1 < B) fetch(j + 1, lt[(j + 1) & 1]);
+        const float z = col[j] * rinv[j];
+        col[j] = z;
+#pragma unroll
+        for (int i = j + 1; i < B; ++i) col[i] = fma_(-lt[j & 1][i], z, col[i]);
       }
 #pragma unroll
       for (int r = 0; r < B; ++r) U[S.in_band(kb, r, i0 + c)] = col[r];
