@@ -386,7 +386,11 @@ int im_copy_dense_factor(const float *U, int pad, const int32_t *block_adr, int 
  * J[w]' diag(D [state == quad, row < nefc]) J[w].  Stands in for mujoco_warp's
  * solver._update_gradient JTDAJ kernel, which the reference calls at
  * src/instantmimic/utils/mjw_kernels/newton_fusion.py:470 and sizes at
- * src/instantmimic/utils/mjw_model.py:31-35.  nv <= 128. */
+ * src/instantmimic/utils/mjw_model.py:31-35.  nv <= 128.  Rows of J that do not contribute (past
+ * nefc, or in another state than `quad`) are not read behind the first 32; an element's sum is the
+ * chain fma(J[r][i] * D[r], J[r][j], .) over the rows in order, from Mdense[i][j], for i <= j, and
+ * H[j][i] is a copy of H[i][j].  The list of contributing rows takes 8 bytes of LDS per row of
+ * njmax beside 33 KB of staged rows: IM_ERR_UNSUPPORTED where that exceeds 160 KB. */
 int im_jtdj_mfma(const float *Mdense, const float *J, int njmax, const float *D,
                  const int32_t *state, const int32_t *nefc, int quad, float *H, int nv,
                  int nv_pad, int nworld, void *stream);
