@@ -122,7 +122,8 @@ def test_gpu_dense_hessian_row_counts_and_masks(device):
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
     # widths: one code path per staged width class (32, 64, 96, 128 with seven and with eight blocks of 16 dofs)
     for nv, njmax in ((27, 70), (35, 33), (128, 131), (56, 300), (70, 50), (100, 40), (113, 66),
-                      (1, 34), (16, 40), (17, 36), (48, 65), (64, 33), (65, 47), (96, 35), (97, 64), (112, 97), (127, 34)):
+                      (1, 34), (16, 40), (17, 36), (48, 65), (64, 33), (65, 47), (96, 35), (97, 64), (112, 97), (127, 34),
+                      (35, 9000)):  # the last one: a row list beyond the default 64 KB of LDS
         counts = [0, 1, 31, 32, 33, 63, 64, 65, njmax - 1, njmax]
         nworld = 3 * len(counts)
         nefc = np.array(counts * 3, np.int32)
