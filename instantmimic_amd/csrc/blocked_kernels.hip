@@ -225,8 +225,10 @@ struct LdsSrc {
   const float *U;
   int nv, pad;
   __device__ __forceinline__ float load(int kb, int ib, int, int r, int c) const {
-    const int row = kb * B + r, col = ib * B + c;
     const Stair<B> S{pad};
+    // a tile right of the diagonal and inside the dofs (the same test for a whole tile) is read as it lies
+    if (ib != kb && (ib + 1) * B <= nv) return U[S.in_band(kb, r, ib * B + c)];
+    const int row = kb * B + r, col = ib * B + c;
     if (row < nv && col < nv) return row <= col ? U[S.at(row, col)] : U[S.at(col, row)];
     return row == col ? 1.0f : 0.0f;
   }
