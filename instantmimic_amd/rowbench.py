@@ -23,7 +23,9 @@ MFMA_F32_TFLOPS = 157.3
 GRAPH = True  # False (--no-graph): plain launches, which is what a counter run of rocprofv3 sees per dispatch
 
 
-def _timeit(torch, fn, nsets: int, launches: int) -> float:
+def _timeit(torch, fn, nsets: int, launches: int, prime: bool = True) -> float:
+    """prime=False: no extra fn(0) ahead of the capture, for a fn that changes its own input (the
+    launches of a replay must then leave that input as they found it)."""
     for i in range(min(nsets, 4)):
         fn(i)
     torch.cuda.synchronize()
@@ -39,7 +41,8 @@ def _timeit(torch, fn, nsets: int, launches: int) -> float:
     s = torch.cuda.Stream()
     s.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(s):
-        fn(0)
+        if prime:
+            fn(0)
         with torch.cuda.graph(g, stream=s):
             for i in range(launches):
                 fn(i % nsets)
@@ -151,7 +154,9 @@ def run(launches: int = 32, only: str | None = None) -> None:
                     sec = _timeit(torch, lambda i: launch(None, S[i][4], S[i][1], S[i][2], S[i][3], S[i][0], G[i], hf, search, sd, de), nsets, launches)
                     used = 2 * plan.nfac + nv
                     _line("im_sparse_init_factor", wl, sec, bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv + used + 2), nworld=nworld)
-                    # per-iteration stage: a tenth of the rows change state
+                    # per-iteration stage: a tenth of the rows change state.  The stage updates the packed H
+                    # in hfactor in place, so launches alternate between the mask the factor was made
+                    # with and the one with those rows flipped: H goes there and back and stays a Hessian.
                     rng = np.random.default_rng(1)
                     ids = np.zeros((nworld, nefc), np.int32)
                     k = max(nefc // 10, 1)
@@ -162,7 +167,14 @@ def run(launches: int = 32, only: str | None = None) -> None:
                     stage = NS.factor_factory(nv, plan.nv_pad, plan)
                     s2 = search.reshape(nworld, nv)
                     idt = t(ids)
-                    sec = _timeit(torch, lambda i: stage(S[i][1], S[i][2], S[i][3], idt, chg, chg, None, S[i][5], None, hf, s2, sd, de, uni), nsets, launches)
+                    st0 = b.state[0]
+                    flip = np.zeros((nworld, nefc), bool)
+                    np.put_along_axis(flip, ids[:, :k], True, axis=1)
+                    st1 = t(np.where(flip, np.where(st0 == synth.QUADRATIC, 0, synth.QUADRATIC), st0).astype(np.int32))
+                    launch(None, S[0][4], S[0][1], S[0][2], S[0][3], S[0][0], G[0], hf, search, sd, de)  # the factor of the first mask
+                    sec = _timeit(torch, lambda i: stage(S[i][1], S[i][2], st1 if i % 2 == 0 else S[i][3], idt, chg, chg, None, S[i][5], None, hf, s2, sd, de, uni),
+                                  nsets, launches, prime=False)
+                    assert bool(torch.isfinite(s2).all()), "the stage's matrices left the solver's range"
                     _line("im_sparse_update_factor", wl + f", {k} changed rows", sec, bytes_=nworld * 4 * (k * nv + 2 * used + 2 * nv + nv + 1 + 2), nworld=nworld)
             del S, X
             torch.cuda.empty_cache()
@@ -222,11 +234,13 @@ def run(launches: int = 32, only: str | None = None) -> None:
         sec = _timeit(torch, lambda i: BD.dense_hessian_factor_solve(Md, J, D, st, ne, H, g, xf, factor=Uf), 1, 8)
         _line("im_jtdj_factor_solve (J'DJ + blocked factor + solve in one launch)", wl, sec,
               bytes_=nworld * 4 * (nv * nv + nefc * nv + 2 * nefc + pad * pad + bs.pad * bs.pad + 2 * nv), nworld=nworld)  # fmt: skip
+        # The stage updates H in place, so a launch's input is the launch before's output.  Launches
+        # alternate between two active masks that differ in the changed rows: rows enter and leave,
+        # H goes from the Hessian of one mask to that of the other and back, and stays what a solver
+        # would hand over.  (With one mask applied over and over the rows that left are subtracted
+        # again and again, H stops being positive definite, and every diagonal tile falls back to the
+        # library square root.)
         rng = np.random.default_rng(2)
-        k = nefc // 10
-        ids = np.zeros((nworld, nefc), np.int32)
-        ids[:, :k] = np.sort(rng.permuted(np.tile(np.arange(nefc), (nworld, 1)), axis=1)[:, :k], axis=1)
-        chg = t(np.full(nworld, k, np.int32))
         uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=dev)
         U = torch.zeros((nworld, pad, pad), device=dev)
         g3 = torch.zeros((nworld, pad, 1), device=dev)
@@ -234,14 +248,27 @@ def run(launches: int = 32, only: str | None = None) -> None:
         search = torch.zeros((nworld, pad, 1), device=dev)
         sd, de = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev)
         stage = NS.factor_factory(nv, pad)
-        idt = t(ids)
-        sec = _timeit(torch, lambda i: stage(J, D, st, idt, chg, chg, None, g3, H, U, search, sd, de, uni), 1, 8)
-        _line("im_dense_update_factor", wl + f", {k} changed rows", sec, bytes_=nworld * 4 * (k * nv + 2 * pad * pad + 2 * nv), nworld=nworld)
-        k = nefc // 2
-        ids[:, :k] = np.sort(rng.permuted(np.tile(np.arange(nefc), (nworld, 1)), axis=1)[:, :k], axis=1)
-        idt, chg = t(ids), t(np.full(nworld, k, np.int32))
-        sec = _timeit(torch, lambda i: stage(J, D, st, idt, chg, chg, None, g3, H, U, search, sd, de, uni), 1, 8)
-        _line("im_dense_update_factor", wl + f", {k} changed rows (a fresh active mask)", sec, bytes_=nworld * 4 * (k * nv + 2 * pad * pad + 2 * nv), nworld=nworld)
+        st0 = b.state[0]
+        for label in ("flip", "fresh"):
+            if label == "flip":  # a tenth of the rows change state
+                k = nefc // 10
+                flip = np.zeros((nworld, nefc), bool)
+                np.put_along_axis(flip, rng.permuted(np.tile(np.arange(nefc), (nworld, 1)), axis=1)[:, :k], True, axis=1)
+                st1 = np.where(flip, np.where(st0 == synth.QUADRATIC, 0, synth.QUADRATIC), st0).astype(np.int32)
+            else:  # a fresh active mask
+                st1 = np.where(rng.uniform(size=st0.shape) < b.shape.p_active, synth.QUADRATIC, 0).astype(np.int32)
+            differ = (st1 == synth.QUADRATIC) != (st0 == synth.QUADRATIC)
+            counts = differ.sum(1).astype(np.int32)
+            ids = np.zeros((nworld, nefc), np.int32)
+            order = np.argsort(~differ, axis=1, kind="stable")  # the differing rows first, ascending
+            ids[:] = np.where(np.arange(nefc)[None, :] < counts[:, None], order, 0)
+            idt, chg, masks = t(ids), t(counts), [t(st1), st]
+            BD.dense_hessian(Md, J, D, st, ne, H)  # H of the first mask, whatever ran before
+            sec = _timeit(torch, lambda i: stage(J, D, masks[i % 2], idt, chg, chg, None, g3, H, U, search, sd, de, uni), 2, 8, prime=False)
+            assert bool(torch.isfinite(search[:, :nv]).all()), "the stage's matrices left the solver's range"
+            kmean = float(counts.mean())
+            note = f", {kmean:.0f} changed rows" + (" (a fresh active mask)" if label == "fresh" else "")
+            _line("im_dense_update_factor", wl + note, sec, bytes_=nworld * 4 * (kmean * nv + 2 * pad * pad + 2 * nv), nworld=nworld)
         del J, H, U, Md, Hc
         torch.cuda.empty_cache()
 
