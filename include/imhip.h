@@ -145,8 +145,10 @@ int im_assemble_tree_ldl_solve_iters(const im_tree_plan *plan, const float *M, i
  * im_tree_plan_kernel_key: the 64-bit key of the plan's structure and elimination plan, and whether
  * the plan already has generated kernels.  im_tree_plan_attach_kernels: loads the code object
  * (kept by the plan until it is destroyed) after checking that it was generated for this key;
- * IM_ERR_STRUCTURE otherwise.  The plan's launches then use it.  Once per plan, on the plan's
- * device, not while the plan is in use by another thread. */
+ * IM_ERR_STRUCTURE otherwise; IM_ERR_UNSUPPORTED for a code object whose fused kernels keep a
+ * private segment (register spills to memory): the plan then stays on the table-driven kernel.
+ * The plan's launches then use it.  Once per plan, on the plan's device, not while the plan is in
+ * use by another thread. */
 int im_tree_plan_kernel_key(const im_tree_plan *plan, unsigned long long *key, int *has_kernel);
 int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object);
 

@@ -2,7 +2,8 @@
 
 Besides the hand-written sources, one kernel per known dof tree is generated
 (``codegen/tree_row16.py``) and compiled in: the five benchmark trees' best plans.
-Other trees run on the generic table-driven kernel.
+Kernels for any other tree are generated when its plan is created (``codegen/jit.py``); the
+table-driven kernel serves plans the generator declines.
 """
 
 from __future__ import annotations
@@ -111,6 +112,11 @@ def prebuild_kernels(trees, group_counts=(0,)) -> list[str]:
     otherwise compile on first use."""
     from .codegen import jit, tree_row16
 
+    # code objects of other generator versions or settings are never loaded again: out with them
+    tag = jit._source_tag()
+    for name in os.listdir(jit.cache_dir()):
+        if name.startswith("tree_row16_") and name.endswith(".co") and not name.endswith(f"_{tag}.co"):
+            os.remove(os.path.join(jit.cache_dir(), name))
     keys = set()
     for parents in trees:
         for count in group_counts:
@@ -130,8 +136,35 @@ def _compile(src: str) -> str:
         if os.path.getmtime(obj) > max(os.path.getmtime(d) for d in deps):
             return obj
     cmd = ["hipcc", *FLAGS, "-c", "-x", "hip", src, "-o", obj]
-    subprocess.run(cmd, check=True)
+    if os.path.dirname(src) != GEN:
+        subprocess.run(cmd, check=True)
+        return obj
+    # a generated kernel: the compiler's resource remarks say whether it keeps to registers
+    done = subprocess.run([*cmd, "-Rpass-analysis=kernel-resource-usage"], capture_output=True, text=True)
+    if done.returncode != 0:
+        sys.stderr.write(done.stderr)
+        raise subprocess.CalledProcessError(done.returncode, cmd)
+    spilling = _spilling_fused_kernels(done.stderr)
+    if spilling:
+        os.remove(obj)
+        raise RuntimeError(f"{os.path.basename(src)}: fused kernels spill registers to memory: {spilling}")
     return obj
+
+
+def _spilling_fused_kernels(remarks: str) -> list[str]:
+    """Fused kernels (first template argument true) with a private segment, from the text of
+    ``-Rpass-analysis=kernel-resource-usage``."""
+    import re
+
+    out, name = [], None
+    for line in remarks.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and name and int(m.group(1)) > 0 and "ILb1E" in name:
+            out.append(f"{name}: {m.group(1)} B/lane")
+    return out
 
 
 def build_library(verbose: bool = True) -> str:

@@ -7,7 +7,7 @@ structure key, so a model is compiled once (a few seconds).
 
 ``IMHIP_TREE_JIT=0`` turns this off (plans then run the table-driven kernel);
 ``IMHIP_KERNEL_CACHE`` names the directory (default: ``_obj/kernels`` beside the library, else
-``~/.cache/instantmimic_amd``, else the temporary directory)."""
+``~/.cache/instantmimic_amd``; a directory owned by another user is never used)."""
 
 from __future__ import annotations
 
@@ -37,53 +37,104 @@ def cache_dir() -> str:
     choices = [named] if named else [
         os.path.join(_HERE, "..", "_obj", "kernels"),
         os.path.join(os.path.expanduser("~"), ".cache", "instantmimic_amd"),
-        os.path.join(tempfile.gettempdir(), "instantmimic_amd_kernels"),
     ]
     for path in choices:
         try:
-            os.makedirs(path, exist_ok=True)
-            if os.access(path, os.W_OK):
+            os.makedirs(path, mode=0o700, exist_ok=True)
+            # code objects are loaded into the GPU as they are: only a directory of this user's own
+            if os.access(path, os.W_OK) and os.stat(path).st_uid == os.getuid():
                 return path
         except OSError:
             continue
-    raise OSError("no writable directory for generated kernels")
+    raise OSError("no writable directory of this user's own for generated kernels (set IMHIP_KERNEL_CACHE)")
 
 
 def _source_tag() -> str:
-    """Changes whenever the generator or the header the kernels include changes."""
+    """Changes whenever the generator, the header the kernels include, the compiler flags or one
+    of the environment knobs that alter the generated source changes: a code object built under
+    one setting is never loaded under another."""
     h = hashlib.sha256()
     for path in (os.path.join(_HERE, "tree_row16.py"), os.path.join(_CSRC, "tree_row16.h")):
         with open(path, "rb") as f:
             h.update(f.read())
+    h.update("\0".join(FLAGS).encode())
+    for knob in tree_row16.SOURCE_KNOBS:
+        h.update(f"\0{knob}={os.environ.get(knob, '')}".encode())
     return h.hexdigest()[:12]
+
+
+def kernel_resources(blob: bytes) -> dict[str, tuple[int, int]]:
+    """{kernel name: (LDS bytes, private-segment bytes per lane)} of a gfx9 code object, read from
+    the kernel descriptors (the 64-byte ``<name>.kd`` objects: group segment size at byte 0,
+    private segment size at byte 4).  Takes the ELF itself or clang's offload bundle around it."""
+    import struct
+
+    start = blob.find(b"\x7fELF")
+    if start < 0:
+        raise ValueError("no ELF image in the code object")
+    elf = memoryview(blob)[start:]
+    if elf[4] != 2 or elf[5] != 1:
+        raise ValueError("not a little-endian ELF64 image")
+    shoff, = struct.unpack_from("<Q", elf, 0x28)
+    shentsize, shnum, _ = struct.unpack_from("<HHH", elf, 0x3A)
+    sections = [struct.unpack_from("<IIQQQQIIQQ", elf, shoff + i * shentsize) for i in range(shnum)]
+    out = {}
+    for _, kind, _, _, offset, size, link, _, _, entsize in sections:
+        if kind not in (2, 11) or entsize == 0:  # SHT_SYMTAB, SHT_DYNSYM
+            continue
+        strtab = sections[link]
+        for k in range(size // entsize):
+            name_off, _, _, shndx, value, _ = struct.unpack_from("<IBBHQQ", elf, offset + k * entsize)
+            end = bytes(elf[strtab[4] + name_off : strtab[4] + name_off + 256]).split(b"\0", 1)[0]
+            if not end.endswith(b".kd") or shndx == 0 or shndx >= shnum:
+                continue
+            home = sections[shndx]
+            at = home[4] + (value - home[3])
+            lds, private = struct.unpack_from("<II", elf, at)
+            out[end[:-3].decode()] = (int(lds), int(private))
+    return out
+
+
+def spilling_kernels(blob: bytes) -> list[str]:
+    """The fused kernels of a code object that use a private segment (register spills to memory)."""
+    return sorted(name for name, (_, private) in kernel_resources(blob).items() if private and name != "im_row16_solve")
 
 
 def code_object(structure, groups, trunk) -> bytes | None:
     """The code object of a (structure, plan), from the cache or freshly compiled; ``None`` when no
-    compiler is at hand."""
+    compiler is at hand, when the generator declines the plan, when the compiler fails on the
+    generated source, or when a fused kernel came out with register spills to memory (no such
+    kernel is handed to the library; the plan then keeps the table-driven kernel)."""
     key = tree_row16.structure_key(*structure, groups, trunk)
     path = os.path.join(cache_dir(), f"tree_row16_{key:016x}_{_source_tag()}.co")
     if os.path.exists(path):
         with open(path, "rb") as f:
-            return f.read()
+            blob = f.read()
+        return None if not blob or spilling_kernels(blob) else blob
     hipcc = shutil.which("hipcc") or ("/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else None)
     if hipcc is None:
         return None
-    if any(len(g) == 0 for g in groups):
-        return None  # a plan with an empty group: the table-driven kernel serves it
-    src = tree_row16.generate(f"k{key:016x}", *structure, groups, trunk, module=True)
+    try:
+        src = tree_row16.generate(f"k{key:016x}", *structure, groups, trunk, module=True)
+    except tree_row16.Declined:
+        return None
     with tempfile.TemporaryDirectory(prefix="imhip_jit_") as tmp:
         hip, out = os.path.join(tmp, "kernel.hip"), os.path.join(tmp, "kernel.co")
         with open(hip, "w") as f:
             f.write(src)
-        subprocess.run([hipcc, *FLAGS, "-I", _CSRC, "-x", "hip", hip, "-o", out], check=True, capture_output=True)
+        done = subprocess.run([hipcc, *FLAGS, "-I", _CSRC, "-x", "hip", hip, "-o", out], capture_output=True)
+        if done.returncode != 0 or not os.path.exists(out):
+            import warnings
+
+            warnings.warn(f"hipcc failed on the generated tree kernel {key:016x}: {done.stderr.decode(errors='replace')[-400:]}")
+            return None
         with open(out, "rb") as f:
             blob = f.read()
     tmp_path = f"{path}.{os.getpid()}.tmp"
     with open(tmp_path, "wb") as f:
         f.write(blob)
     os.replace(tmp_path, path)  # whole files only, also with several processes at once
-    return blob
+    return None if spilling_kernels(blob) else blob
 
 
 def attach(plan_ptr, structure, groups, trunk) -> bool:

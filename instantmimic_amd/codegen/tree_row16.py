@@ -47,6 +47,17 @@ import os
 # development aid: IMHIP_EXP=timing makes the fused kernel write clock64() stamps of its phases
 # over the H output buffer instead of H
 EXP = os.environ.get("IMHIP_EXP", "")
+# every environment variable that changes the generated source (the run-time cache keys on them)
+SOURCE_KNOBS = ("IMHIP_EXP", "IMHIP_SP", "IMHIP_OCC")
+
+
+class Declined(ValueError):
+    """The generator does not take this (structure, plan): the caller keeps the table-driven kernel."""
+
+
+def _require(ok, why: str) -> None:
+    if not ok:
+        raise Declined(why)
 
 
 def structure_key(rowadr, rownnz, colind, groups, trunk) -> int:
@@ -147,7 +158,11 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     # several branches reuses the lanes past the fork: `segs[j]` lists, per run of dofs on one
     # chain, the lanes that take new dofs (a copy of the vector keeps the finished branch).
     tpos = {a: t.depth[a] for a in trunk}
-    assert sorted(tpos.values()) == list(range(len(trunk))), "trunk is not a chain from the root"
+    # the trunk's right-hand side is one lane vector with the dof of depth p in lane p: a forest's
+    # trunk (several roots) or a trunk that forks has two dofs for one lane
+    _require(sorted(tpos.values()) == list(range(len(trunk))), "the plan's trunk is not a single chain from one root")
+    _require(all(len(g) > 0 for g in groups), "a plan with an empty group")
+    _require(nv <= 96, "more than 96 dofs")
     # Per group: which owner (trunk accumulator ('t', a) or group dof ('g', b)) sits in which lane
     # while each dof is eliminated.  A new segment starts when the chain of the next dof needs a
     # lane for another owner: the lane then takes a fresh value (the dof's right-hand side, or
@@ -238,14 +253,15 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
                 mask = sum(1 << p for p in range(16) if take["fresh"].get(16 * s_ + p, -1) >= 0)
                 ci = leaf_sets.index((t.leaf_of[k_first], s_)) if (t.leaf_of[k_first], s_) in leaf_sets else None
                 if mask:
-                    assert ci is not None and all(tab[ci][p] == take["fresh"][16 * s_ + p] for p in range(16) if (mask >> p) & 1)
+                    _require(ci is not None and all(tab[ci][p] == take["fresh"][16 * s_ + p] for p in range(16) if (mask >> p) & 1),
+                             "a group's right-hand side does not lie on one chain table")
                 rhs_src[j, i, s_] = (ci, mask)
     if len(trunk):
         below = next(li for li, leaf in enumerate(t.leaves) if trunk[-1] in t.chain[leaf])
         for s_ in range(tsets):
             mask = sum(1 << p for p in range(16) if 16 * s_ + p < len(trunk))
             ci = leaf_sets.index((below, s_))
-            assert all(tab[ci][p] == trunk[16 * s_ + p] for p in range(16) if (mask >> p) & 1)
+            _require(all(tab[ci][p] == trunk[16 * s_ + p] for p in range(16) if (mask >> p) & 1), "the trunk does not lie on one chain table")
             rhs_src["T", 0, s_] = (ci, mask)
     else:
         for s_ in range(tsets):
@@ -315,7 +331,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     lds_floats = xs_off + 4 * nv
     if EXP == "timing":
         emit("  unsigned long long *tdbg = (unsigned long long *)Hout + (size_t)bid * 16; int tn = 0;")
-        emit("  #define STAMP() do { if (threadIdx.x == 0) tdbg[tn] = clock64(); ++tn; } while (0)")
+        emit("  #define STAMP() do { if (Hout && threadIdx.x == 0) tdbg[tn] = clock64(); ++tn; } while (0)")
         emit("  STAMP();")
     else:
         emit("  #define STAMP() do {} while (0)")
@@ -378,7 +394,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     # accumulator index table, M (as a flat copy that is then gathered from LDS, so that the
     # table and M travel together instead of one after the other), the row weights; then J.
     MC = -(-nM // 64)
-    assert MC * 64 <= TW and nM < TW and 4 * nM < 32768
+    _require(MC * 64 <= TW and nM < TW and 4 * nM < 32768, "M does not fit the staging copy")
     for n, (ti, tj) in enumerate(tiles):
         for v in range(4):
             emit(f"    const int ix{n}_{v} = IDX_{name}[{n * 4 + v}][lane];  // byte offset into the copy of M")
@@ -673,7 +689,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
         emitted = {b: -1 for b in dofs}  # -1: the product with d_b is still to come
         complete, seq = set(), []
         while len(complete) < len(dofs):
-            newly = []
+            newly, before = [], len(seq)
             for b in dofs:
                 if b in complete or b in newly:
                     continue
@@ -688,7 +704,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
                     emitted[b] += 1
                 if emitted[b] == t.depth[b]:
                     newly.append(b)
-            assert newly or any(True for _ in seq)
+            _require(bool(newly) or len(seq) > before, "back-substitution order does not close")
             complete.update(newly)
 
         def src_of(b_):
@@ -882,7 +898,13 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     # workgroups per CU that the fused kernel is compiled for: what the 160 KB of LDS admit (with
     # the lists of 128 constraint rows), at most 4 -- fewer workgroups leave each wavefront more
     # registers, which the larger trees need
-    occ = max(1, min(int(os.environ.get("IMHIP_OCC", "4")), 4, (160 * 1024) // (lds_floats * 4 + 32 * 128)))
+    asked = int(os.environ.get("IMHIP_OCC", "4"))
+    if not 1 <= asked <= 4:
+        # a workgroup is four wavefronts, one per SIMD, so this is also the wavefronts per SIMD whose
+        # register budget the compiler keeps to: beyond 4 (fewer than 128 registers) the larger trees
+        # spill to memory, and such a build once ended in a GPU memory fault
+        raise ValueError(f"IMHIP_OCC={asked}: the generated kernels are built for 1 to 4 workgroups per CU")
+    occ = max(1, min(asked, (160 * 1024) // (lds_floats * 4 + 32 * 128)))
     text = "\n".join(out) + "\n"
     header = '#include "tree_row16.h"' if module else '#include "../tree_row16.h"'  # a module is built with -I csrc
     return text.replace('#include "../tree_row16.h"', f'{header}\n#define IM_OCC_{name} {occ}', 1)

@@ -619,6 +619,13 @@ int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object) {
       hipModuleGetFunction(&fused_long, mod, "im_row16_fused_long") != hipSuccess ||
       hipModuleGetFunction(&solve, mod, "im_row16_solve") != hipSuccess)
     return fail(IM_ERR_STRUCTURE);
+  // a fused kernel that spills registers to memory is not taken: the plan keeps the table-driven
+  // kernel (the generator's callers check the code object's descriptors before they get here)
+  auto spills = [](hipFunction_t f) {
+    int bytes = 0;
+    return hipFuncGetAttribute(&bytes, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, f) == hipSuccess && bytes > 0;
+  };
+  if (spills(fused) || spills(fused_long)) return fail(IM_ERR_UNSUPPORTED);
   if (info[2] + 32 * 64 > 48 * 1024) {
     // more than the default dynamic LDS: asked for here; a runtime that refuses the request for a
     // module's function reports it at the launch

@@ -208,8 +208,8 @@ def test_ineligible_models_return_none(device):
 def test_iterations_in_one_call_match_the_oracle_bitwise(device, name, nworld, niter, ragged, per_iter_grad):
     """im_assemble_tree_ldl_solve_iters: the iterations of a step share M, J and D; every iteration
     assembles afresh, so each equals the single call (and the oracle) bit for bit -- on the
-    kernel that keeps J in registers (humanoid, ant: up to 64 rows) and on the launch-per-iteration
-    path behind the same entry point (g1: 96 rows, snu: 128 rows, niter = 1)."""
+    straight-line kernel (humanoid, ant: up to 64 rows) and on the variant that loops over the
+    listed constraint rows (g1: 96 rows, snu: 128 rows); both cover (worlds, iteration) with one grid."""
     import torch
 
     from instantmimic_amd.mjw_kernels import tree_ldl as T

@@ -42,6 +42,64 @@ def test_code_objects_and_keys():
     assert sum(x != y for x, y in zip(la, lb)) <= 12 and abs(len(la) - len(lb)) < 20 and len(la) > 500
 
 
+def _random_forest(rng, nv, nroots):
+    parents = []
+    for k in range(nv):
+        parents.append(-1 if k < nroots and (k == 0 or rng.random() < 0.7) else int(rng.integers(max(0, k - 6), k)))
+    return parents
+
+
+def test_generator_takes_or_declines_random_forests(tmp_path, monkeypatch):
+    """Every eligible plan either gets source or an explicit refusal (a trunk with two roots or a
+    fork does not fit the generator's lane layout): nothing else may escape to the caller that
+    creates a model's scratch, whose table-driven kernel serves the refused ones."""
+    rng = np.random.default_rng(5)
+    taken, declined, reasons = 0, [], set()
+    for case in range(150):
+        nv = int(rng.integers(2, 65))
+        parents = _random_forest(rng, nv, 1 if case % 3 else int(rng.integers(2, 4)))
+        st, groups, trunk, _ = build._plan_of_tree(parents, int(rng.integers(0, 5)))
+        try:
+            src = tree_row16.generate("t", *st, groups, trunk, module=True)
+            assert "im_row16_fused" in src
+            taken += 1
+        except tree_row16.Declined as why:
+            declined.append((st, groups, trunk))
+            reasons.add(str(why))
+    assert taken >= 100 and len(declined) >= 5, (taken, len(declined))
+    assert reasons <= {"the plan's trunk is not a single chain from one root", "a plan with an empty group"}, reasons
+    # the run-time path answers None for a refused plan and does not leave a file behind
+    monkeypatch.setenv("IMHIP_KERNEL_CACHE", str(tmp_path))
+    assert jit.code_object(*declined[0]) is None
+    assert list(tmp_path.iterdir()) == []
+    # an occupancy beyond four workgroups per CU is an error, not a silent clamp
+    monkeypatch.setenv("IMHIP_OCC", "6")
+    st, groups, trunk, _ = build._plan_of_tree(TREES["limbs"])
+    with pytest.raises(ValueError, match="IMHIP_OCC"):
+        tree_row16.generate("t", *st, groups, trunk)
+
+
+def test_cache_is_keyed_by_everything_that_changes_the_source(monkeypatch):
+    base = jit._source_tag()
+    for knob, value in (("IMHIP_EXP", "timing"), ("IMHIP_SP", "3"), ("IMHIP_OCC", "2")):
+        monkeypatch.setenv(knob, value)
+        assert jit._source_tag() != base
+        monkeypatch.delenv(knob)
+    assert jit._source_tag() == base
+    monkeypatch.setattr(jit, "FLAGS", jit.FLAGS + ["-DX"])
+    assert jit._source_tag() != base
+
+
+def test_kernel_descriptors_of_a_code_object():
+    st, groups, trunk, _ = build._plan_of_tree(TREES["limbs"])
+    res = jit.kernel_resources(jit.code_object(st, groups, trunk))
+    assert set(res) == {"im_row16_fused", "im_row16_fused_long", "im_row16_solve"}
+    assert all(private == 0 for _, private in res.values())  # the best plan's kernels keep to registers
+    # one group for the whole tree holds every row in one wavefront's registers and spills
+    st, groups, trunk, _ = build._plan_of_tree(TREES["limbs62"], 1)
+    assert jit.code_object(st, groups, trunk) is None
+
+
 def _has_kernel(scratch) -> bool:
     key, has = C.c_ulonglong(0), C.c_int(0)
     assert _lib.lib().im_tree_plan_kernel_key(scratch.kernel.ptr, C.byref(key), C.byref(has)) == 0
