@@ -313,7 +313,9 @@ int im_sparse_dense_factor(const im_sparse_plan *plan, const uint8_t *done, cons
  * those below it are never written or read); without changed rows the stored U is solved
  * against.  Rows and columns >= nv of H count as the identity.  nv_pad = a multiple of 16
  * above nv (src/instantmimic/utils/mjw_model.py:30).  H and U must be 16-byte aligned
- * (IM_ERR_STRIDE otherwise). */
+ * (IM_ERR_STRIDE otherwise).  changes[w] < 0: no row is applied and H as it lies in memory is
+ * factored -- the first factor of a solve, after the full assembly that upstream's
+ * solver._update_gradient makes there (src/instantmimic/utils/mjw_kernels/newton_fusion.py:470). */
 int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes,
                            const int32_t *changes, const int32_t *ids, int ld_ids,
                            const float *J, int njmax, const float *D, const int32_t *state,
@@ -667,7 +669,10 @@ int im_project_body_wrenches(const im_body_wrenches *wrenches,
  * a shuffle-down tree, the trees in order (the reference leaves that order to Warp's
  * tile_sum) --, newton_decrement = 0, grad_scale = 1, search_unchanged = 0.
  * J (nworld, njmax, nv) contiguous; nefc and done may be null (all rows, no world done);
- * done and search_unchanged are bytes. */
+ * done and search_unchanged are bytes.  A null state_changed_count counts every world as changed:
+ * the first gradient of a solve (upstream's _update_gradient_zero_grad_dot and
+ * _update_gradient_grad as src/instantmimic/utils/mjw_kernels/newton_fusion.py:487-500 launches
+ * them, with qfrc_constraint = J' efc_force formed here as well). */
 int im_newton_gradient(const int32_t *nefc, const float *J, int njmax, const float *efc_force,
                        int64_t ld_force, const float *qfrc_smooth, int64_t ld_smooth,
                        const float *efc_Ma, int64_t ld_Ma, const int32_t *state_changed_count,
@@ -829,6 +834,39 @@ int im_newton_converged(const float *alpha, const float *improvement, const floa
                         const float *stat_meaninertia, int nmeaninertia, int nv, int maxiter,
                         int overflow_bit, int32_t *niter, int32_t *overflow, uint8_t *done,
                         int32_t *nsolving, int nworld, void *stream);
+
+/* Jaref = J qacc - aref for the rows below nefc[w]: what upstream's solver._solve_init_jaref_kernel
+ * leaves in ctx.Jaref when the reference's init_context launches it
+ * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:451-468, with its split of a row into
+ * 50- or 20-dof stretches).  The sum of a row follows im_newton_jv (one chain of fused
+ * multiply-adds up to 50 dofs, 20-dof partial sums added in order beyond; upstream adds the
+ * partial sums with atomics, in no fixed order), then aref is subtracted. */
+int im_newton_init_jaref(const float *J, int njmax, const int32_t *nefc, const float *qacc, int64_t ld_qacc,
+                         const float *aref, int64_t ld_aref, float *Jaref, int64_t ld_Jaref, int nv,
+                         int nworld, void *stream);
+
+/* The dense copy of M that upstream's solver._update_gradient starts the Newton Hessian from
+ * (called at src/instantmimic/utils/mjw_kernels/newton_fusion.py:470): H (nworld, pad, pad)
+ * receives M[w, elemid[i * nv + j]] at (i, j) where elemid (nv x nv, the reference's m.M_elemid
+ * layout, -1 outside M's pattern) names an element, zero elsewhere and in the padding. */
+int im_dense_from_csr(const float *M, int64_t ldM, const int32_t *elemid, int nv, int pad, float *H,
+                      int nworld, void *stream);
+
+/* The factor stage of a Newton iteration on the kinematic tree: for every world whose skip byte
+ * is clear (the reference's stage returns for done[w] or state_changes[w] == 0,
+ * src/instantmimic/utils/mjw_kernels/newton_stages.py:648-649; ctx.search_unchanged is that flag)
+ * H = M + J' diag(D [state == quad]) J is assembled on M's pattern and factored by the tree L'DL
+ * (im_assemble_tree_ldl_solve), search = -H^-1 grad, search_dot = search . search and
+ * decrement = grad . H^-1 grad summed as the stages of the reference sum them (lane l of `block`
+ * lanes adds dofs l, l + block, ..; 32-lane shuffle-down trees; the trees in order:
+ * src/instantmimic/utils/mjw_kernels/sparse_hessian.py:462-479).  The reference has no tree stage
+ * of its own: for a model whose constraint rows stay on single root-to-leaf chains this is its
+ * sparse stage's result computed from the fresh Hessian instead of an incremental update. */
+int im_newton_tree_stage(const im_tree_plan *plan, const uint8_t *skip, const float *M, int64_t ldM,
+                         const float *J, int njmax, const float *D, const int32_t *state,
+                         const int32_t *nefc, int quad, const float *grad, int64_t ldg, float *search,
+                         int64_t ld_search, float *search_dot, float *decrement, int block, int nworld,
+                         void *stream);
 
 /* Replaces _init_efc_settling_empty_worlds
  * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:412-428): solver_niter = 0,

@@ -222,6 +222,12 @@ SIGNATURES = {
          _i, _vp],
     ),  # fmt: skip
     "im_newton_jv": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _vp, _i64, _i, _i, _vp]),
+    "im_newton_init_jaref": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _vp]),
+    "im_dense_from_csr": (_i, [_vp, _i64, _vp, _i, _i, _vp, _i, _vp]),
+    "im_newton_tree_stage": (
+        _i,
+        [_vp, _vp, _vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _vp, _i, _i, _vp],
+    ),
     "im_newton_advance": (
         _i,
         [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _vp],

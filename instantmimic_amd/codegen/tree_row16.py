@@ -224,8 +224,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("    state += it * state_it; y += it * y_it; x += it * x_it;")
     emit("  }")
     emit("  const int w = bid * 4 + (lane >> 4);")
-    emit("  const bool live = w < nworld;")
-    emit("  const int64_t ws = live ? w : nworld - 1;")
+    emit("  const int64_t ws = w < nworld ? w : nworld - 1;")
+    # a world whose `skip` byte is set is read and worked on like its neighbours (a wavefront's
+    # four worlds share every instruction) and nothing of it is stored
+    emit("  const bool live = w < nworld && !(skip && skip[ws]);")
     # ---- right-hand side, uniform per world (wavefront 0 factors and solves)
     emit("  const float *yw = y + ws * ldy;")
     # wavefront j of the fused kernel factors group j of the plan, wavefront 0 also the trunk;
@@ -880,7 +882,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("  #undef STAMP")
     emit("}")
     if module:
-        args = "M, ldM, J, njmax, D, state, nefc_p, quad, y, ldy, x, ldx, Hout, nworld, flags, niter, state_it, y_it, x_it"
+        args = "M, ldM, J, njmax, D, state, nefc_p, quad, y, ldy, x, ldx, Hout, nworld, flags, niter, state_it, y_it, x_it, skip"
         emit("} }  // namespace im::gen")
         for kernel, asm_, long_, bounds in (("fused", "true", "false", f"256, IM_OCC_{name}"), ("fused_long", "true", "true", f"256, IM_OCC_{name}"),
                                             ("solve", "false", "false", "64, 1")):  # fmt: skip

@@ -941,10 +941,12 @@ __global__ __launch_bounds__(256, 4) void dense_update_factor_kernel(
   float *Hw = H_ + w * (int64_t)pad * pad, *Uw = U_ + w * (int64_t)pad * pad;
   const float *Jw = J + w * (int64_t)njmax * nv, *Dw = D + w * njmax, *gw = grad + w * ldg;
   const int32_t *sw = state + w * njmax, *idw = ids + w * ld_ids;
+  // a negative count: H is taken as it lies in memory and factored (the first factor of a solve)
   int count = changes[w];
-  count = count < ld_ids ? count : ld_ids;
+  const bool refactor = count != 0;
+  count = count < 0 ? 0 : (count < ld_ids ? count : ld_ids);
   for (int i = tid; i < pf; i += nt) rhs[i] = i < nv ? gw[i] : 0.0f;
-  if (count > 0) {
+  if (refactor) {
     // The changed rows of J and their signed weights pass through LDS in batches that use the
     // factor's array while it is still free (up to 64 rows each), the pair sums staying in the
     // matrix cores' accumulators from one batch to the next; the sums go to H in memory, and H's

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(kThreads) void newton_gradient_kernel(GradArgs a) {
   int *rowl = (int *)(f + a.njmax);
   float *gl = f + 2 * a.njmax, *part = gl + a.nv;
   const bool done = a.done && a.done[w] != 0;
-  const bool changed = a.changed[w] != 0;
+  const bool changed = !a.changed || a.changed[w] != 0;
   int nefc = a.nefc ? a.nefc[w] : a.njmax;
   nefc = nefc < a.njmax ? nefc : a.njmax;
   nefc = nefc > 0 ? nefc : 0;
@@ -137,7 +137,7 @@ template <int U>
 __global__ __launch_bounds__(64) void newton_jv_kernel(
     const float *__restrict__ J, int njmax, const int32_t *__restrict__ nefc_p,
     const float *__restrict__ search, int64_t lds_, const uint8_t *__restrict__ skip,
-    float *__restrict__ jv, int64_t ldj, int nv, int chunks) {
+    float *__restrict__ jv, int64_t ldj, int nv, int chunks, const float *__restrict__ minus, int64_t ldm) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x;
   const int64_t w = blockIdx.x / chunks;
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(64) void newton_jv_kernel(
     } else {
       acc = chain(0, nv);
     }
-    jv[w * ldj + r0 + lane] = acc;
+    jv[w * ldj + r0 + lane] = minus ? acc - minus[w * ldm + r0 + lane] : acc;
   }
 }
 
@@ -309,6 +309,23 @@ __global__ __launch_bounds__(kThreads) void qfrc_from_grad_kernel(
   out[w * ldo + dof] = v;
 }
 
+// The dense symmetric matrix of a tree CSR M, padded with zeros to (pad, pad): element (i, j)
+// is M[elemid[i * nv + j]] where the table names one, else 0.  One thread per element.
+__global__ __launch_bounds__(kThreads) void dense_from_csr_kernel(
+    const float *__restrict__ M, int64_t ldM, const int32_t *__restrict__ elemid, int nv, int pad,
+    float *__restrict__ H) {
+  const int64_t w = blockIdx.y;
+  const int e = blockIdx.x * kThreads + threadIdx.x;
+  if (e >= pad * pad) return;
+  const int i = e / pad, j = e - i * pad;
+  float v = 0.0f;
+  if (i < nv && j < nv) {
+    const int id = elemid[i * nv + j];
+    if (id >= 0) v = M[w * ldM + id];
+  }
+  H[w * (int64_t)pad * pad + e] = v;
+}
+
 }  // namespace
 }  // namespace im
 
@@ -324,7 +341,7 @@ extern "C" int im_newton_gradient(const int32_t *nefc, const float *J, int njmax
   if (nworld < 0 || nv <= 0 || njmax < 0) return IM_ERR_ARG;
   if (block != 32 && block != 64) return IM_ERR_UNSUPPORTED;
   if (nworld == 0) return IM_OK;
-  if (!J || !efc_force || !qfrc_smooth || !efc_Ma || !state_changed_count || !alpha || !qfrc_constraint || !grad ||
+  if (!J || !efc_force || !qfrc_smooth || !efc_Ma || !alpha || !qfrc_constraint || !grad ||
       !grad_dot || !newton_decrement || !grad_scale || !search_unchanged)
     return IM_ERR_ARG;
   if (ld_force < njmax || ld_smooth < nv || ld_Ma < nv || ld_constraint < nv || ld_grad < nv) return IM_ERR_STRIDE;
@@ -345,12 +362,14 @@ extern "C" int im_newton_gradient(const int32_t *nefc, const float *J, int njmax
   return IM_OK;
 }
 
-extern "C" int im_newton_jv(const float *J, int njmax, const int32_t *nefc, const float *search, int64_t ld_search,
-                            const uint8_t *skip_world, float *jv, int64_t ld_jv, int nv, int nworld, void *stream) {
+namespace {
+int launch_jv(const float *J, int njmax, const int32_t *nefc, const float *search, int64_t ld_search,
+              const uint8_t *skip_world, float *jv, int64_t ld_jv, const float *minus, int64_t ld_minus, int nv,
+              int nworld, void *stream) {
   if (nworld < 0 || nv <= 0 || njmax < 0) return IM_ERR_ARG;
   if (nworld == 0 || njmax == 0) return IM_OK;
   if (!J || !search || !jv) return IM_ERR_ARG;
-  if (ld_search < nv || ld_jv < njmax) return IM_ERR_STRIDE;
+  if (ld_search < nv || ld_jv < njmax || (minus && ld_minus < njmax)) return IM_ERR_STRIDE;
   const size_t lds_bytes = (64 * (size_t)(nv | 1) + nv) * 4;
   if (lds_bytes > kLdsLimit || 64 * (int64_t)nv >= (1 << 20)) return IM_ERR_UNSUPPORTED;
   const int chunks = (njmax + 63) / 64;
@@ -358,13 +377,42 @@ extern "C" int im_newton_jv(const float *J, int njmax, const int32_t *nefc, cons
   const dim3 grid((unsigned)((int64_t)nworld * chunks));
 #define IM_JV(U)                                                                                          \
   hipLaunchKernelGGL(newton_jv_kernel<U>, grid, dim3(64), lds_bytes, (hipStream_t)stream, J, njmax, nefc, \
-                     search, ld_search, skip_world, jv, ld_jv, nv, chunks)
+                     search, ld_search, skip_world, jv, ld_jv, nv, chunks, minus, ld_minus)
   // 64 rows of nv words are nv words per lane
   if (nv <= 16) IM_JV(16);
   else if (nv <= 32) IM_JV(32);
   else if (nv <= 48) IM_JV(48);
   else IM_JV(64);
 #undef IM_JV
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+}  // namespace
+
+extern "C" int im_newton_jv(const float *J, int njmax, const int32_t *nefc, const float *search, int64_t ld_search,
+                            const uint8_t *skip_world, float *jv, int64_t ld_jv, int nv, int nworld, void *stream) {
+  return launch_jv(J, njmax, nefc, search, ld_search, skip_world, jv, ld_jv, nullptr, 0, nv, nworld, stream);
+}
+
+extern "C" int im_newton_init_jaref(const float *J, int njmax, const int32_t *nefc, const float *qacc, int64_t ld_qacc,
+                                    const float *aref, int64_t ld_aref, float *Jaref, int64_t ld_Jaref, int nv,
+                                    int nworld, void *stream) {
+  if (!aref) return IM_ERR_ARG;
+  return launch_jv(J, njmax, nefc, qacc, ld_qacc, nullptr, Jaref, ld_Jaref, aref, ld_aref, nv, nworld, stream);
+}
+
+extern "C" int im_dense_from_csr(const float *M, int64_t ldM, const int32_t *elemid, int nv, int pad, float *H,
+                                 int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || pad < nv) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!M || !elemid || !H) return IM_ERR_ARG;
+  const int per = pad * pad;
+  for (int w0 = 0; w0 < nworld; w0 += 65535) {
+    const int nw = nworld - w0 < 65535 ? nworld - w0 : 65535;
+    hipLaunchKernelGGL(dense_from_csr_kernel, dim3((unsigned)((per + kThreads - 1) / kThreads), (unsigned)nw),
+                       dim3(kThreads), 0, (hipStream_t)stream, M + w0 * ldM, ldM, elemid, nv, pad,
+                       H + (int64_t)w0 * per);
+  }
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }

@@ -82,10 +82,11 @@ __global__ __launch_bounds__(64) void tree_kernel(
     int njmax, const float *__restrict__ D, const int32_t *__restrict__ state,
     const int32_t *__restrict__ nefc_p, int quad, const float *__restrict__ y,
     int64_t ldy, float *__restrict__ x, int64_t ldx, float *__restrict__ Hout,
-    int rc, float inv_nv, int njpad, unsigned flags) {
+    int rc, float inv_nv, int njpad, unsigned flags, const unsigned char *__restrict__ skip) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x;
   const int w = blockIdx.x;
+  if (skip && skip[w]) return;  // the workgroup is this world's one wavefront
   const int nv = P.nv, nM = P.nM;
 
   float *T = lds;                      // [nM]   published rows (unscaled)
@@ -290,7 +291,7 @@ __global__ __launch_bounds__(64) void tree_kernel(
 using KernelFn = void (*)(TreeDev, const float *, int64_t, const float *, int,
                           const float *, const int32_t *, const int32_t *, int,
                           const float *, int64_t, float *, int64_t, float *, int,
-                          float, int, unsigned);
+                          float, int, unsigned, const unsigned char *);
 
 template <int SPL>
 KernelFn pick_nvp(int nvp) {
@@ -390,7 +391,7 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
            const float *J, int njmax, const float *D, const int32_t *state,
            const int32_t *nefc, int quad, const float *y, int64_t ldy, float *x,
            int64_t ldx, float *Hout, int nworld, unsigned flags, void *stream,
-           Iterations its = Iterations()) {
+           Iterations its = Iterations(), const unsigned char *skip = nullptr) {
   if (!plan || nworld < 0) return IM_ERR_ARG;
   if (!plan->device_ready) return IM_ERR_UNSUPPORTED;
   if (nworld == 0) return IM_OK;
@@ -402,7 +403,7 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
     const auto *e = (const gen::Row16Entry *)plan->row16;
     void *args[] = {&M,     &ldM,      &J,         &njmax,        &D,        &state,   &nefc,
                     &quad,  &y,        &ldy,       &x,            &ldx,      &Hout,    &nworld,
-                    &flags, &its.niter, &its.state_it, &its.y_it, &its.x_it};
+                    &flags, &its.niter, &its.state_it, &its.y_it, &its.x_it, &skip};
     // staged rows plus the four worlds' active-row lists (row id and D per constraint row)
     const size_t lds = assemble ? (size_t)e->lds_bytes + 32 * std::max<size_t>(((size_t)njmax + 15) / 16 * 16, 64) : 0;
     if (lds <= 160 * 1024) {
@@ -423,7 +424,8 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
   if (its.niter > 1) {  // the table-driven kernel: one launch per iteration
     for (int it = 0; it < its.niter; ++it) {
       const int st = launch(plan, assemble, M, ldM, J, njmax, D, state + it * its.state_it, nefc, quad,
-                            y + it * its.y_it, ldy, x + it * its.x_it, ldx, nullptr, nworld, flags, stream);
+                            y + it * its.y_it, ldy, x + it * its.x_it, ldx, nullptr, nworld, flags, stream,
+                            Iterations(), skip);
       if (st != IM_OK) return st;
     }
     return IM_OK;
@@ -443,9 +445,39 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
   if (!fn) return IM_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(64), lds_bytes, (hipStream_t)stream, plan->dev, M,
                      ldM, J, njmax, D, state, nefc, quad, y, ldy, x, ldx, Hout, rc,
-                     1.0f / (float)nv, njpad, flags);
+                     1.0f / (float)nv, njpad, flags, skip);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
+}
+
+// search . search and grad . x of the tree stage of a Newton iteration, summed as the reference's
+// factor stages sum them (src/instantmimic/utils/mjw_kernels/sparse_hessian.py:462-479): lane l of
+// a block of `block` lanes adds its dofs l, l + block, .. with fused multiply-adds, every 32 lanes
+// fold in a shuffle-down tree, the folds are added in order.  x = -search.  A wavefront per world.
+__global__ __launch_bounds__(256) void newton_search_sums_kernel(
+    const unsigned char *__restrict__ skip, const float *__restrict__ grad, int64_t ldg,
+    const float *__restrict__ search, int64_t lds_, float *__restrict__ search_dot,
+    float *__restrict__ decrement, int nv, int block, int nworld) {
+  const int lane = threadIdx.x & 63;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (w >= nworld || (skip && skip[w])) return;
+  float s0 = 0.0f, s1 = 0.0f;
+  for (int d = lane; d < nv && lane < block; d += block) {
+    const float v = -search[w * lds_ + d];
+    s0 = fma_(v, v, s0);
+    s1 = fma_(grad[w * ldg + d], v, s1);
+  }
+  for (int o = 16; o > 0; o >>= 1) {
+    s0 = s0 + __shfl_down(s0, o, 32);
+    s1 = s1 + __shfl_down(s1, o, 32);
+  }
+  const float a1 = __shfl(s0, 32, 64), b1 = __shfl(s1, 32, 64);
+  if (lane == 0) {
+    float ra = 0.0f + s0, rb = 0.0f + s1;
+    if (block > 32) ra = ra + a1, rb = rb + b1;
+    search_dot[w] = ra;
+    decrement[w] = rb;
+  }
 }
 
 }  // namespace
@@ -681,6 +713,21 @@ int im_assemble_tree_ldl_solve(const im_tree_plan *plan, const float *M, int64_t
                                float *Hout, int nworld, unsigned flags, void *stream) {
   return im::launch(plan, true, M, ldM, J, njmax, D, state, nefc, quad, grad, ldg, x, ldx,
                     Hout, nworld, flags, stream);
+}
+
+int im_newton_tree_stage(const im_tree_plan *plan, const uint8_t *skip, const float *M, int64_t ldM, const float *J,
+                         int njmax, const float *D, const int32_t *state, const int32_t *nefc, int quad,
+                         const float *grad, int64_t ldg, float *search, int64_t ld_search, float *search_dot,
+                         float *decrement, int block, int nworld, void *stream) {
+  if (!search_dot || !decrement || (block != 32 && block != 64)) return IM_ERR_ARG;
+  const int st = im::launch(plan, true, M, ldM, J, njmax, D, state, nefc, quad, grad, ldg, search, ld_search, nullptr,
+                            nworld, IM_FLAG_NEGATE, stream, im::Iterations(), skip);
+  if (st != IM_OK || nworld == 0) return st;
+  hipLaunchKernelGGL(im::newton_search_sums_kernel, dim3((unsigned)((nworld + 3) / 4)), dim3(256), 0,
+                     (hipStream_t)stream, skip, grad, ldg, search, ld_search, search_dot, decrement, plan->nv, block,
+                     nworld);
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
 }
 
 }  // extern "C"

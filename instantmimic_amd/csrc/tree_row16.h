@@ -19,7 +19,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
       const float *__restrict__ D, const int *__restrict__ state,                         \
       const int *__restrict__ nefc_p, int quad, const float *__restrict__ y, int64_t ldy, \
       float *__restrict__ x, int64_t ldx, float *__restrict__ Hout, int nworld, unsigned flags, \
-      int niter, int64_t state_it, int64_t y_it, int64_t x_it
+      int niter, int64_t state_it, int64_t y_it, int64_t x_it, const unsigned char *__restrict__ skip
 
 // value of lane n of the caller's 16-lane row, in every lane of the row
 #define IM_BC(v, n)                                                                          \

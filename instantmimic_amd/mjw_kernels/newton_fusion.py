@@ -169,7 +169,8 @@ def gradient(nefc, efc_J, efc_force, qfrc_smooth, efc_Ma, state_changed_count, a
     ``newton_decrement`` and ``grad_scale`` for the others; ``search_unchanged`` for all (argument
     names of the reference's gradient_function).  ``efc_J`` (nworld, njmax, nv) contiguous float32;
     ``nefc`` int32 or None; ``done`` and ``search_unchanged`` bool or uint8; ``block`` = the lane
-    count whose summation order ``grad_dot`` follows (32 or 64)."""
+    count whose summation order ``grad_dot`` follows (32 or 64).  ``state_changed_count=None``
+    counts every world as changed: the first gradient of a solve."""
     import torch
 
     if efc_J.dim() != 3 or not efc_J.is_contiguous() or efc_J.dtype != torch.float32 or not efc_J.is_cuda:
@@ -182,7 +183,9 @@ def gradient(nefc, efc_J, efc_force, qfrc_smooth, efc_Ma, state_changed_count, a
     for t in (alpha, grad_dot, newton_decrement, grad_scale):
         if t.dtype != torch.float32 or not t.is_cuda or t.numel() != nworld or not t.is_contiguous():
             raise TypeError("the per-world scalars must be contiguous float32 CUDA tensors")
-    if state_changed_count.dtype != torch.int32 or not state_changed_count.is_contiguous() or state_changed_count.numel() != nworld:
+    if state_changed_count is not None and (
+        state_changed_count.dtype != torch.int32 or not state_changed_count.is_contiguous() or state_changed_count.numel() != nworld
+    ):
         raise TypeError("state_changed_count must be a contiguous int32 tensor with one element per world")
     if nefc is not None and (nefc.dtype != torch.int32 or not nefc.is_contiguous() or nefc.numel() != nworld):
         raise TypeError("nefc must be a contiguous int32 tensor with one element per world")
@@ -195,7 +198,8 @@ def gradient(nefc, efc_J, efc_force, qfrc_smooth, efc_Ma, state_changed_count, a
         status = _lib.lib().im_newton_gradient(
             None if nefc is None else nefc.data_ptr(), efc_J.data_ptr(), int(njmax), efc_force.data_ptr(),
             efc_force.stride(0), qfrc_smooth.data_ptr(), qfrc_smooth.stride(0), efc_Ma.data_ptr(), efc_Ma.stride(0),
-            state_changed_count.data_ptr(), alpha.data_ptr(), None if done is None else done.data_ptr(),
+            None if state_changed_count is None else state_changed_count.data_ptr(), alpha.data_ptr(),
+            None if done is None else done.data_ptr(),
             qfrc_constraint.data_ptr(), qfrc_constraint.stride(0), grad.data_ptr(), grad.stride(0), grad_dot.data_ptr(),
             newton_decrement.data_ptr(), grad_scale.data_ptr(), search_unchanged.data_ptr(), int(nv), int(block),
             int(nworld), int(torch.cuda.current_stream(efc_J.device).cuda_stream),
@@ -439,18 +443,196 @@ def eval_constraints(Jaref, efc_D, efc_frictionloss, ne, nf, nefc, done, ls_exha
 
 OVERFLOW_LS_ITERATIONS = 4  # bits of d.overflow: the caller's OverflowType where it differs
 OVERFLOW_ITERATIONS = 8
+DISABLE_WARMSTART = 1 << 8  # MuJoCo's mjDSBL_WARMSTART, matched by value when the model carries plain integers
+
+
+def init_jaref(nefc, qacc, efc_J, efc_aref, Jaref) -> None:
+    """``Jaref = J qacc - aref`` for the rows below ``nefc`` (upstream's ``_solve_init_jaref_kernel``
+    as newton_fusion.py:451-468 launches it)."""
+    import torch
+
+    if efc_J.dim() != 3 or not efc_J.is_contiguous() or efc_J.dtype != torch.float32 or not efc_J.is_cuda:
+        raise TypeError("efc_J must be a contiguous float32 CUDA tensor (nworld, njmax, nv)")
+    nworld, njmax, nv = efc_J.shape
+    _rows(qacc, nworld, nv, torch.float32, "qacc")
+    _rows(efc_aref, nworld, njmax, torch.float32, "efc_aref")
+    _rows(Jaref, nworld, njmax, torch.float32, "Jaref")
+    if nefc is not None:
+        _per_world(nefc, nworld, (torch.int32,), "nefc")
+    with torch.cuda.device(efc_J.device):
+        status = _lib.lib().im_newton_init_jaref(
+            efc_J.data_ptr(), int(njmax), None if nefc is None else nefc.data_ptr(), qacc.data_ptr(), qacc.stride(0),
+            efc_aref.data_ptr(), efc_aref.stride(0), Jaref.data_ptr(), Jaref.stride(0), int(nv), int(nworld),
+            int(torch.cuda.current_stream(efc_J.device).cuda_stream),
+        )  # fmt: skip
+    _lib.check(status, "im_newton_init_jaref")
+
+
+def dense_from_csr(M, elemid, out) -> None:
+    """``out[w]`` (rows x rows, rows >= nv) = the dense symmetric M of world w, zero outside M's
+    pattern and in the padding; ``elemid`` (nv, nv) int32 names the CSR element of every pair."""
+    import torch
+
+    nv = int(elemid.shape[0])
+    if elemid.dtype != torch.int32 or tuple(elemid.shape) != (nv, nv) or not elemid.is_contiguous() or not elemid.is_cuda:
+        raise TypeError("elemid must be a contiguous (nv, nv) int32 CUDA tensor")
+    nworld = int(M.shape[0])
+    if out.dim() != 3 or out.shape[0] != nworld or out.shape[1] != out.shape[2] or out.shape[1] < nv or not out.is_contiguous():
+        raise ValueError("out must be a contiguous (nworld, rows, rows) tensor with rows >= nv")
+    for t in (M, out):
+        if t.dtype != torch.float32 or not t.is_cuda:
+            raise TypeError("M and out must be float32 CUDA tensors")
+    if M.dim() != 2 or (M.shape[1] > 1 and M.stride(1) != 1):
+        raise ValueError("M needs rows of contiguous floats")
+    with torch.cuda.device(M.device):
+        status = _lib.lib().im_dense_from_csr(M.data_ptr(), M.stride(0), elemid.data_ptr(), nv, int(out.shape[1]),
+                                              out.data_ptr(), nworld, int(torch.cuda.current_stream(M.device).cuda_stream))  # fmt: skip
+    _lib.check(status, "im_dense_from_csr")
+
+
+def elemid_table(rowadr, rownnz, colind) -> np.ndarray:
+    """(nv, nv) int32: the CSR element of M at (i, j) and (j, i), -1 outside the tree pattern (the
+    layout of the reference's ``m.M_elemid``)."""
+    rowadr, rownnz, colind = (np.asarray(a, np.int64) for a in (rowadr, rownnz, colind))
+    nv = rowadr.size
+    out = np.full((nv, nv), -1, np.int32)
+    for i in range(nv):
+        for k in range(rowadr[i], rowadr[i] + rownnz[i]):
+            out[i, colind[k]] = out[colind[k], i] = k
+    return out
+
+
+def default_mul_m_call(m, d, out, vec) -> None:
+    """``out = M vec`` over the model's row tables: the ``mul_m_call`` of the reference's scratch
+    (src/instantmimic/utils/mjw_step_optimized.py:2595, 2709) for callers that have none."""
+    mul_m(d.M, vec, out, m.M_mulm_rowadr, m.M_mulm_col, m.M_mulm_madr)
+
+
+def _fused_plan(ctx):
+    plan = getattr(ctx, "sparse_hessian_plan", None)
+    return plan if plan is not None and plan.path == "fused" else None
+
+
+def _tree_scratch(ctx):
+    """The opt-in tree stage: a scratch of ``tree_ldl.create_tree_factor_solve_scratch`` that the
+    caller has put on ``ctx.newton_tree_scratch`` (for models whose constraint rows stay on single
+    root-to-leaf chains; the reference has no such stage)."""
+    return getattr(ctx, "newton_tree_scratch", None) if ctx is not None else None
+
+
+def attach_scratch(m, d, ctx, device=None) -> None:
+    """Persistent per-world scratch of the fused iteration on ``ctx`` (newton_fusion.py:301-304:
+    the dofs the changed rows touch, ``nv`` slots and their count); the dense path's first factor
+    also keeps a dense copy of M, the M-pattern table and two constant count arrays here."""
+    import torch
+
+    dev = device if device is not None else d.qacc.device
+    nworld, nv = int(d.nworld), int(m.nv)
+    ctx.newton_dof_union = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=dev)
+    if _fused_plan(ctx) is None and _tree_scratch(ctx) is None:
+        ctx.newton_mdense = torch.zeros((nworld, nv, nv), dtype=torch.float32, device=dev)
+        ctx.newton_refactor = torch.full((nworld,), -1, dtype=torch.int32, device=dev)
+        ctx.newton_every = torch.ones((nworld,), dtype=torch.int32, device=dev)
+        elemid = getattr(m, "M_elemid", None)
+        if elemid is None:
+            host = lambda a: a.cpu().numpy() if hasattr(a, "cpu") else np.asarray(a)  # noqa: E731
+            elemid = torch.from_numpy(elemid_table(host(m.M_rowadr), host(m.M_rownnz), host(m.M_colind))).to(dev)
+        ctx.newton_elemid = elemid.to(dtype=torch.int32).reshape(nv, nv).contiguous()
+
+
+def _stage(m, ctx):
+    from . import newton_stages
+
+    return newton_stages.factor_factory(int(m.nv), int(m.nv_pad), _fused_plan(ctx), tree_scratch=_tree_scratch(ctx),
+                                        block=newton_block_dim(m))  # fmt: skip
+
+
+def _launch_stage(stage, m, d, ctx) -> None:
+    if _tree_scratch(ctx) is not None:
+        stage(d.efc.J, d.efc.D, d.efc.state, None, None, None, ctx.done, ctx.grad, None, None, ctx.search, ctx.search_dot,
+              ctx.newton_decrement, None, M=d.M, nefc=d.nefc, skip=ctx.search_unchanged)  # fmt: skip
+        return
+    sparse = _fused_plan(ctx) is not None
+    stage(d.efc.J, d.efc.D, d.efc.state, ctx.quad_changed_ids, ctx.quad_changed_count, ctx.state_changed_count, ctx.done,
+          ctx.grad, None if sparse else ctx.h, ctx.hfactor, ctx.search, ctx.search_dot, ctx.newton_decrement, ctx.newton_dof_union)  # fmt: skip
+
+
+def _update_constraint(m, d, ctx) -> None:
+    """Force and state of every row from ``ctx.Jaref`` (upstream's ``solver._update_constraint`` as
+    newton_fusion.py:469 calls it; ``qfrc_constraint = J' force`` is formed with the gradient)."""
+    eval_constraints(ctx.Jaref, d.efc.D, d.efc.frictionloss, d.ne, d.nf, d.nefc, ctx.done, None, d.efc.force, d.efc.state,
+                     ctx.quad_changed_ids, ctx.quad_changed_count, ctx.state_changed_count)  # fmt: skip
+
+
+def _first_gradient(m, d, ctx) -> None:
+    """``qfrc_constraint``, ``grad`` and ``grad . grad`` of every world that is not done, with
+    ``newton_decrement = 0``, ``grad_scale = 1`` and ``search_unchanged = done`` (upstream's
+    ``_update_gradient_zero_grad_dot`` and ``_update_gradient_grad``, newton_fusion.py:487-500)."""
+    nv = int(m.nv)
+    gradient(d.nefc, d.efc.J, d.efc.force, d.qfrc_smooth, d.efc.Ma, None, ctx.alpha, ctx.done, d.qfrc_constraint,
+             ctx.grad[:, :nv], ctx.grad_dot, ctx.newton_decrement, ctx.grad_scale, ctx.search_unchanged,
+             block=newton_block_dim(m))  # fmt: skip
+
+
+def _update_gradient_sparse(m, d, ctx, plan) -> None:
+    """The first gradient, then H assembled on the sparse pattern, factored and solved
+    (newton_fusion.py:481-519)."""
+    from . import sparse_hessian
+
+    _first_gradient(m, d, ctx)
+    sparse_hessian.init_factor_kernel(plan)(ctx.done, d.nefc, d.efc.J, d.efc.D, d.efc.state, d.M, ctx.grad, ctx.hfactor,
+                                            ctx.search, ctx.search_dot, ctx.newton_decrement)  # fmt: skip
+
+
+def _update_gradient_tree(m, d, ctx) -> None:
+    """The first gradient, then the tree stage for every world that is not done (``search_unchanged``
+    is ``done`` at this point)."""
+    _first_gradient(m, d, ctx)
+    _launch_stage(_stage(m, ctx), m, d, ctx)
+
+
+def _update_gradient(m, d, ctx) -> None:
+    """The dense first factor (upstream's ``solver._update_gradient`` for the dense Newton,
+    newton_fusion.py:470): ``ctx.h = M + J' D_act J`` on the matrix cores, then the augmented
+    blocked Cholesky of the per-iteration stage without an update."""
+    from . import blocked_dense
+
+    if not hasattr(ctx, "newton_mdense"):
+        raise RuntimeError("the dense first factor needs attach_scratch(m, d, ctx)")
+    _first_gradient(m, d, ctx)
+    dense_from_csr(d.M, ctx.newton_elemid, ctx.newton_mdense)
+    blocked_dense.dense_hessian(ctx.newton_mdense, d.efc.J, d.efc.D, d.efc.state, d.nefc, ctx.h)
+    stage = _stage(m, ctx)
+    stage(d.efc.J, d.efc.D, d.efc.state, ctx.quad_changed_ids, ctx.newton_refactor, ctx.newton_every, ctx.done, ctx.grad,
+          ctx.h, ctx.hfactor, ctx.search, ctx.search_dot, ctx.newton_decrement, ctx.newton_dof_union)  # fmt: skip
+
+
+def init_context(m, d, ctx, mul_m_call=None) -> None:
+    """``init_context`` of the fused path (newton_fusion.py:431-478): worlds without constraint rows
+    finish at once with ``qacc = qacc_smooth``; ``Jaref = J qacc - aref``; ``Ma = M qacc`` for every
+    world; forces and states; the first gradient, Hessian, factor and search direction through the
+    sparse plan, the tree stage or the dense path, whichever ``ctx`` carries."""
+    init_empty_worlds(d.nefc, d.qacc_smooth, d.solver_niter, ctx.search_dot, ctx.done, d.qacc)
+    init_jaref(d.nefc, d.qacc, d.efc.J, d.efc.aref, ctx.Jaref)
+    (mul_m_call or default_mul_m_call)(m, d, d.efc.Ma, d.qacc)
+    _update_constraint(m, d, ctx)
+    plan = _fused_plan(ctx)
+    if plan is not None:
+        _update_gradient_sparse(m, d, ctx, plan)
+    elif _tree_scratch(ctx) is not None:
+        _update_gradient_tree(m, d, ctx)
+    else:
+        _update_gradient(m, d, ctx)
 
 
 def iteration(m, d, ctx, nsolving=None, *, stage=None) -> None:
-    """One iteration of the fused Newton loop for every world that is not done, as seven launches in
+    """One iteration of the fused Newton loop for every world that is not done, as eight launches in
     the reference kernel's order (newton_fusion.py:151-296): M search, J search, the scalar search,
     the step, the constraints' new forces and states, the gradient, the factor stage, the
     convergence test."""
-    from . import newton_stages
-
-    nworld, nv = int(d.nworld), int(m.nv)
+    nv = int(m.nv)
     if stage is None:
-        stage = newton_stages.factor_factory(nv, int(m.nv_pad), getattr(ctx, "sparse_hessian_plan", None))
+        stage = _stage(m, ctx)
     mul_m(d.M, ctx.search, ctx.mv, m.M_mulm_rowadr, m.M_mulm_col, m.M_mulm_madr, skip_world=ctx.search_unchanged)
     jv(d.efc.J, ctx.search, ctx.jv, nefc=d.nefc, skip_world=ctx.search_unchanged)
     linesearch(m.opt.tolerance, m.opt.ls_tolerance, m.stat.meaninertia, d.ne, d.nf, d.nefc, d.qfrc_smooth, d.efc.D,
@@ -463,29 +645,31 @@ def iteration(m, d, ctx, nsolving=None, *, stage=None) -> None:
     gradient(d.nefc, d.efc.J, d.efc.force, d.qfrc_smooth, d.efc.Ma, ctx.state_changed_count, ctx.alpha, ctx.done,
              d.qfrc_constraint, ctx.grad[:, :nv], ctx.grad_dot, ctx.newton_decrement, ctx.grad_scale, ctx.search_unchanged,
              block=newton_block_dim(m))  # fmt: skip
-    sparse = getattr(ctx, "sparse_hessian_plan", None) is not None
-    stage(d.efc.J, d.efc.D, d.efc.state, ctx.quad_changed_ids, ctx.quad_changed_count, ctx.state_changed_count, ctx.done,
-          ctx.grad, None if sparse else ctx.h, ctx.hfactor, ctx.search, ctx.search_dot, ctx.newton_decrement, ctx.newton_dof_union)  # fmt: skip
+    _launch_stage(stage, m, d, ctx)
     converged(ctx.alpha, ctx.improvement, ctx.grad_dot, ctx.newton_decrement, m.opt.tolerance, m.stat.meaninertia, nv,
               int(m.opt.iterations), d.solver_niter, ctx.done, overflow=d.overflow, overflow_bit=OVERFLOW_ITERATIONS,
               nsolving=nsolving)  # fmt: skip
 
 
-def run(m, d, ctx, nsolving, *, check_every: int = 4, graph: bool = False) -> int:
+def run(m, d, ctx, nsolving, *, check_every: int | None = None, graph: bool = False) -> int:
     """The fused Newton solve with the reference's signature (newton_fusion.py:330-409): iterates
     until every world is done or ``m.opt.iterations`` is reached.  The reference keeps a world in
-    one resident block for the whole loop; here an iteration is seven launches over all worlds
-    (finished worlds drop out of each through ``ctx.done``), and the host reads ``nsolving`` every
-    ``check_every`` iterations to stop early.  ``graph``: the first iteration runs as plain
-    launches, the second is captured in a graph that the later ones replay (the arrays of ``d`` and
-    ``ctx`` must then stay where they are for the whole solve; they do when the caller does not
-    reallocate them), which takes the seven launches' host cost out of every iteration.  Returns the
-    number of iterations launched."""
+    one resident block for the whole loop; here an iteration is eight launches over all worlds and
+    finished worlds drop out of each through ``ctx.done``, so launching all ``m.opt.iterations``
+    of them is correct whatever the worlds need, touches the host nowhere and can be captured in a
+    caller's graph: that is what happens under stream capture and with ``check_every=0``.
+    Outside a capture the host by default reads ``ctx.done`` every fourth iteration and stops early
+    (``check_every``).  ``graph``: the first iteration runs as plain launches, the second is
+    captured in a graph that the later ones replay (the arrays of ``d`` and ``ctx`` must then stay
+    where they are for the whole solve).  Returns the number of iterations launched."""
     import torch
 
-    from . import newton_stages
-
-    stage = newton_stages.factor_factory(int(m.nv), int(m.nv_pad), getattr(ctx, "sparse_hessian_plan", None))
+    capturing = torch.cuda.is_current_stream_capturing()
+    if check_every is None:
+        check_every = 0 if capturing else 4
+    if capturing and (check_every or graph):
+        raise RuntimeError("under stream capture the solve runs without host checks and without a graph of its own")
+    stage = _stage(m, ctx)
     limit = int(m.opt.iterations)
     captured = None
     launched = 0
@@ -500,6 +684,23 @@ def run(m, d, ctx, nsolving, *, check_every: int = 4, graph: bool = False) -> in
         else:
             captured.replay()
         launched += 1
-        if check_every > 0 and (it + 1) % check_every == 0 and int(nsolving.item()) <= 0:
+        if check_every > 0 and (it + 1) % check_every == 0 and bool(ctx.done.all().item()):
             break
     return launched
+
+
+def solve(m, d, ctx, nsolving, *, mul_m_call=None) -> None:
+    """The constraint solve around the fused loop, in the order of ``_solve_monolithic_with_scratch``
+    for an eligible model (src/instantmimic/utils/mjw_step_optimized.py:2588-2683): the start point
+    (warm start unless disabled), ``init_context``, the loop, the constraint force from the last
+    gradient.  No step reads anything back, so the whole solve can sit in a caller's graph."""
+    flags = getattr(m.opt, "disableflags", 0)
+    warmstart = not (int(flags) & DISABLE_WARMSTART) and getattr(d, "qacc_warmstart", None) is not None
+    d.qacc.copy_(d.qacc_warmstart if warmstart else d.qacc_smooth)
+    d.qfrc_constraint.zero_()
+    init_context(m, d, ctx, mul_m_call)
+    ctx.search_unchanged.zero_()
+    nsolving.fill_(int(d.nworld))
+    run(m, d, ctx, nsolving)
+    nv = int(m.nv)
+    qfrc_constraint_from_grad(d.nefc, d.qfrc_smooth, d.efc.Ma, ctx.grad[:, :nv], ctx.grad_scale, d.qfrc_constraint)

@@ -27,13 +27,51 @@ def _check(tensors, nworld: int) -> None:
             raise ValueError(f"{name} has {t.shape[0]} worlds, expected {nworld}")
 
 
-def factor_factory(nv: int, pad: int, sparse_plan: SparseHessianPlan | None = None):
+def factor_factory(nv: int, pad: int, sparse_plan: SparseHessianPlan | None = None, *, tree_scratch: Any = None,
+                   block: int = 32):
     """Launcher ``kernel(J, D, state, ids, changes, state_changes, done, grad, H, U, search,
     search_dot, decrement, dof_union)`` with the reference kernel's arrays: ids (nworld, njmax)
     changed rows, changes / state_changes (nworld,), grad and search (nworld, nv_pad) or
     (nworld, nv_pad, 1), H and U (nworld, nv_pad, nv_pad), dof_union (nworld, nv + 1).  With a
-    sparse plan ``U`` is the hfactor buffer and ``H`` is not touched."""
+    sparse plan ``U`` is the hfactor buffer and ``H`` is not touched.
+
+    ``tree_scratch`` (a scratch of ``tree_ldl.create_tree_factor_solve_scratch``; the reference
+    has no such stage) selects the stage on the kinematic tree for models whose constraint rows
+    stay on single root-to-leaf chains: the Hessian is assembled afresh on M's pattern and solved
+    by the tree L'DL, nothing is carried from one iteration to the next, and ``H``, ``U``, ``ids``
+    and ``dof_union`` are not touched.  Its launcher also takes ``M=`` (d.M), ``nefc=`` and
+    ``skip=`` (ctx.search_unchanged, the bytes the gradient leaves: done or no state change);
+    ``block`` is the lane count whose summation order the two dot products follow."""
     import torch
+
+    if tree_scratch is not None:
+        if sparse_plan is not None:
+            raise ValueError("a sparse plan and a tree scratch: choose one factor stage")
+        if not getattr(tree_scratch, "cuda", False) or tree_scratch.kernel.info().nv != nv:
+            raise ValueError("the tree scratch belongs to another model or has no device state")
+
+        def tree_kernel(J, D, state, ids, changes, state_changes, done, grad, H, U, search, search_dot, decrement,
+                        dof_union, *, M, nefc=None, skip, quad: int = QUADRATIC) -> None:  # fmt: skip
+            nworld, njmax, nvj = J.shape
+            if nvj != nv:
+                raise ValueError("J does not match the stage's nv")
+            _check(dict(J=J, D=D, state=state, grad=grad, search=search, search_dot=search_dot, decrement=decrement,
+                        M=M, skip=skip, nefc=nefc), nworld)  # fmt: skip
+            if skip.dtype not in (torch.bool, torch.uint8):
+                raise TypeError("skip must be a bool tensor")
+            if M.dim() != 2 or M.shape[1] < tree_scratch.kernel.info().nM:
+                raise ValueError("M must be (nworld, nM)")
+            ldg, lds = grad[0].numel(), search[0].numel()
+            with torch.cuda.device(J.device):
+                status = _lib.lib().im_newton_tree_stage(
+                    tree_scratch.kernel.ptr, skip.data_ptr(), M.data_ptr(), M.stride(0), J.data_ptr(), int(njmax),
+                    D.data_ptr(), state.data_ptr(), None if nefc is None else nefc.data_ptr(), int(quad), grad.data_ptr(),
+                    int(ldg), search.data_ptr(), int(lds), search_dot.data_ptr(), decrement.data_ptr(), int(block),
+                    int(nworld), int(torch.cuda.current_stream(J.device).cuda_stream),
+                )  # fmt: skip
+            _lib.check(status, "im_newton_tree_stage")
+
+        return tree_kernel
 
     if sparse_plan is not None:
         if sparse_plan.handle is None:

@@ -1073,9 +1073,11 @@ int orc_dense_update_factor(int nworld, int nv, int pad, const unsigned char *do
       const int *sw = state + (size_t)w * njmax, *idw = ids + (size_t)w * ld_ids;
       const float *g = grad + (size_t)w * ldg;
       int *uni = uni_out + (size_t)w * (nv + 1);
-      const int count = changes[w] < ld_ids ? changes[w] : ld_ids;
+      /* a negative count: no row is applied, H is factored as it is (the first factor of a solve) */
+      const int refactor = changes[w] != 0;
+      const int count = changes[w] < 0 ? 0 : (changes[w] < ld_ids ? changes[w] : ld_ids);
       for (int i = 0; i < pad; ++i) rhs[i] = i < nv ? g[i] : 0.0f;
-      if (count > 0) {
+      if (refactor) {
         const int nu = dof_union(nv, Jw, idw, count, uni);
         for (int cj = 0; cj < nu; ++cj)
           for (int ri = 0; ri <= cj; ++ri) {
@@ -1606,6 +1608,38 @@ int orc_newton_jv(int nworld, int nv, int njmax, const int *nefc, const float *J
       }
       jv[(size_t)w * njmax + r] = acc;
     }
+  }
+  return 0;
+}
+
+/* search . search and grad . x (x = -search) of the tree factor stage, summed as the reference's
+ * stages sum their two dot products (src/instantmimic/utils/mjw_kernels/sparse_hessian.py:462-479):
+ * lane l of `block` lanes adds its dofs l, l + block, .. with fused multiply-adds, 32 lanes fold in
+ * a shuffle-down tree, the folds are added in order from zero.  Dofs in dof order. */
+int orc_newton_search_sums(int nworld, int nv, int block, const unsigned char *skip, const float *grad,
+                           int ldg, const float *search, int lds, float *sdot, float *decr) {
+  for (int w = 0; w < nworld; ++w) {
+    if (skip && skip[w]) continue;
+    float s0[64] = {0}, s1[64] = {0};
+    for (int lane = 0; lane < block; ++lane)
+      for (int d = lane; d < nv; d += block) {
+        const float v = -search[(size_t)w * lds + d];
+        s0[lane] = fmaf(v, v, s0[lane]);
+        s1[lane] = fmaf(grad[(size_t)w * ldg + d], v, s1[lane]);
+      }
+    float ra = 0.0f, rb = 0.0f;
+    for (int wv = 0; wv < block / 32; ++wv) {
+      float *a = s0 + 32 * wv, *b = s1 + 32 * wv;
+      for (int off = 16; off > 0; off >>= 1)
+        for (int i = 0; i < off; ++i) {  /* lane i takes lane i + off; lanes past the fold are not read again */
+          a[i] = a[i] + a[i + off];
+          b[i] = b[i] + b[i + off];
+        }
+      ra = ra + a[0];
+      rb = rb + b[0];
+    }
+    sdot[w] = ra;
+    decr[w] = rb;
   }
   return 0;
 }

@@ -579,6 +579,41 @@ def newton_jv(J, search, nefc=None, skip=None, out=None):
     return out
 
 
+def newton_init_jaref(J, qacc, aref, nefc=None):
+    """Jaref = J qacc - aref: the row sums of `newton_jv`, then one float32 subtraction (rows at
+    or past nefc stay zero).  Pinned by the fp64 product."""
+    jv = newton_jv(J, qacc, nefc=nefc)
+    njmax = jv.shape[1]
+    ne = np.full(len(jv), njmax) if nefc is None else np.minimum(np.asarray(nefc), njmax)
+    rows = np.arange(njmax)[None, :] < ne[:, None]
+    return np.where(rows, jv - _f(aref), np.float32(0.0)).astype(np.float32)
+
+
+def newton_search_sums(grad, search, block=32, skip=None, sdot=None, decr=None):
+    """(search_dot, decrement) of the tree stage; skipped worlds keep what was passed in.  Pinned
+    by the fp64 dot products and, where every lane holds one dof, by the tree's association."""
+    grad, search = _f(grad), _f(search)
+    nworld, nv = search.shape
+    sdot = np.zeros(nworld, np.float32) if sdot is None else _f(sdot).copy()
+    decr = np.zeros(nworld, np.float32) if decr is None else _f(decr).copy()
+    sk = None if skip is None else np.ascontiguousarray(skip, np.uint8)
+    lib().orc_newton_search_sums(nworld, nv, block, None if sk is None else _p(sk), _p(grad), grad.shape[1], _p(search),
+                                 nv, _p(sdot), _p(decr))  # fmt: skip
+    return sdot, decr
+
+
+def newton_tree_stage(rowadr, rownnz, colind, plan, M, J, D, state, nefc, grad, skip, search, sdot, decr, block=32, quad=1):
+    """The tree factor stage: for the worlds that are not skipped search = -(M + J' D_act J)^-1 grad
+    by the fused assembly + tree L'DL, and the two dot products.  Returns (search, search_dot,
+    decrement) with the skipped worlds' entries as passed in."""
+    nv = len(rowadr)
+    x = assemble_tree_ldl_solve(rowadr, rownnz, colind, plan, M, J, D, state, nefc, _f(grad)[:, :nv], quad=quad)
+    run = np.ones(len(x), bool) if skip is None else np.asarray(skip) == 0
+    new = np.where(run[:, None], -x, _f(search)).astype(np.float32)
+    sd, de = newton_search_sums(_f(grad)[:, :nv], new, block=block, skip=skip, sdot=sdot, decr=decr)
+    return new, sd, de
+
+
 # The step along the search direction and the listing of changed rows
 # (src/instantmimic/utils/mjw_kernels/newton_stages.py:373-381, 403-426), in NumPy.  `advance`
 # is pinned by its closed form in fp64 and, bit for bit, by an exact-product-one-rounding sum;

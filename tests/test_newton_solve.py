@@ -1,0 +1,145 @@
+"""The constraint solve as the reference's step calls it: ``init_context``, the fused Newton loop
+and the force recovery (src/instantmimic/utils/mjw_step_optimized.py:2588-2683,
+src/instantmimic/utils/mjw_kernels/newton_fusion.py:330-539), started from poisoned solver state,
+captured in a graph without any read-back, against the oracle's pieces chained in the same order."""
+
+import numpy as np
+import pytest
+
+import newton_chain as NC
+from instantmimic_amd import synth
+from instantmimic_amd.mjw_kernels import newton_fusion as NF
+from oracle import ref as R
+
+
+# ---------------------------------------------------------------- oracle pinning (CPU)
+
+
+def test_oracle_search_sums_and_init_jaref():
+    rng = np.random.default_rng(2)
+    for nv, block in ((27, 32), (56, 64), (70, 32), (14, 64)):
+        g, s = rng.normal(size=(9, nv)).astype(np.float32), rng.normal(size=(9, nv)).astype(np.float32)
+        skip = np.zeros(9, np.uint8)
+        skip[4] = 1
+        sd, de = R.newton_search_sums(g, s, block=block, skip=skip, sdot=np.full(9, 5.0, np.float32), decr=np.full(9, 6.0, np.float32))
+        assert sd[4] == 5.0 and de[4] == 6.0
+        live = skip == 0
+        np.testing.assert_allclose(sd[live], (s.astype(np.float64) ** 2).sum(1)[live], rtol=1e-6)
+        np.testing.assert_allclose(de[live], -(g.astype(np.float64) * s).sum(1)[live], rtol=1e-5, atol=1e-5)
+    # one dof per lane: the sum is the 32-lane shuffle-down tree over the squares, folds in order
+    v = rng.normal(size=(1, 32)).astype(np.float32)
+    sq = (v[0] * v[0]).astype(np.float32)  # fma(v, v, 0) = the rounded square
+    for off in (16, 8, 4, 2, 1):
+        sq = (sq[:off] + sq[off : 2 * off]).astype(np.float32)
+    assert R.newton_search_sums(np.zeros_like(v), v, block=32)[0][0] == np.float32(0.0) + sq[0]
+    # Jaref = J qacc - aref
+    J, q, a = rng.normal(size=(5, 12, 27)).astype(np.float32), rng.normal(size=(5, 27)).astype(np.float32), rng.normal(size=(5, 12)).astype(np.float32)
+    nefc = np.array([12, 0, 5, 12, 1], np.int32)
+    out = R.newton_init_jaref(J, q, a, nefc=nefc)
+    want = np.einsum("wrj,wj->wr", J.astype(np.float64), q) - a
+    rows = np.arange(12)[None, :] < nefc[:, None]
+    np.testing.assert_allclose(out[rows], want[rows], rtol=1e-5, atol=1e-5)
+    assert not out[~rows].any()
+
+
+def test_oracle_dense_first_factor_is_the_factor_of_h():
+    """A negative count of changed rows: H as it lies there is factored with the gradient as the
+    augmented column, and U'U gives it back."""
+    shape = synth.SHAPES["humanoid"]
+    b = synth.make_batch(shape, 6, ragged_nefc=True)
+    nv, pad = shape.nv, 32
+    Md = synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32)
+    H = R.jtdj_dense(Md.reshape(6, -1), b.J, b.D, b.state[0], b.nefc, pad)
+    every = np.ones(6, np.int32)
+    ids = np.zeros((6, shape.nefc), np.int32)
+    H2, U, uni, search, sdot, decr = R.dense_update_factor(every, -every, ids, b.J, b.D, b.state[0], b.grad, H, np.zeros_like(H))
+    np.testing.assert_array_equal(H2, H)
+    assert not uni[:, nv].any()
+    Hd = H[:, :nv, :nv].astype(np.float64)
+    Hd = np.triu(Hd) + np.triu(Hd, 1).transpose(0, 2, 1)
+    x64 = R.solve64(Hd, b.grad)
+    assert R.rel_l2(-search, x64) < 1e-4
+    Uf = np.triu(U[:, :nv, :nv].astype(np.float64))
+    back = np.einsum("wki,wkj->wij", Uf, Uf)
+    assert np.abs(back - Hd).max() / np.abs(Hd).max() < 2e-6
+    np.testing.assert_allclose(decr, (b.grad * x64).sum(1), rtol=1e-3)
+
+
+def test_elemid_table_matches_the_csr():
+    rowadr, rownnz, colind = synth.csr_from_parents(synth.humanoid_parents())
+    table = NF.elemid_table(rowadr, rownnz, colind)
+    np.testing.assert_array_equal(table, synth.matrix_elemid(rowadr, rownnz, colind))
+    assert (table == table.T).all() and (np.diag(table) == rowadr + rownnz - 1).all()
+
+
+@pytest.mark.parametrize("stage", ["dense", "tree", "sparse"])
+def test_oracle_solve_converges_to_the_fp64_minimum(stage):
+    """The chained oracle from init_context on: every world finishes, no overflow, and at the end
+    the gradient of the fp64 cost vanishes against the problem's scale -- on all three factor
+    stages, with worlds that have no constraint rows and with a warm start."""
+    name = "g1" if stage == "sparse" else "humanoid"
+    p = NC.problem(name, 24, stage, empty_every=7, warmstart=(stage == "tree"))
+    s = NC.oracle_solve(p)
+    assert s.done.all() and not (s.overflow & 8).any() and s.niter.max() < 25
+    assert (s.niter[p.nefc == 0] == 0).all() and (s.niter[p.nefc > 0] > 0).all()
+    np.testing.assert_array_equal(s.qacc[p.nefc == 0], p.qacc_smooth[p.nefc == 0])
+    b = p.b
+    M64 = synth.dense_from_csr(b.M.astype(np.float64), b.rowadr, b.rownnz, b.colind)
+    x = np.einsum("wrj,wj->wr", p.J.astype(np.float64), s.qacc.astype(np.float64)) - p.aref
+    g = np.einsum("wij,wj->wi", M64, s.qacc.astype(np.float64) - p.qacc_smooth)
+    for w in range(p.nworld):
+        ne, nf, nefc = int(p.ne[w]), int(p.nf[w]), int(p.nefc[w])
+        D, fl = p.D[w].astype(np.float64), p.frictionloss[w].astype(np.float64)
+        slope = np.zeros(p.njmax)
+        slope[:ne] = D[:ne] * x[w, :ne]
+        fr = slice(ne, ne + nf)
+        slope[fr] = np.clip(D[fr] * x[w, fr], -fl[fr], fl[fr])
+        rest = slice(ne + nf, nefc)
+        slope[rest] = D[rest] * np.minimum(x[w, rest], 0.0)
+        g[w] += slope[:nefc] @ p.J[w, :nefc].astype(np.float64)
+        # the recovered constraint force is minus that slope pulled back: J' force = -J' slope
+        np.testing.assert_allclose(s.qfrc_constraint[w], -(slope[:nefc] @ p.J[w, :nefc].astype(np.float64)), rtol=2e-3, atol=2e-3 * max(1.0, np.abs(s.qfrc_constraint[w]).max()))
+    g0 = np.linalg.norm(np.einsum("wrj,wr->wj", p.J.astype(np.float64), p.D * np.abs(p.aref)), axis=1)
+    has = p.nefc > 0
+    assert (np.linalg.norm(g, axis=1)[has] / g0[has]).max() < 1e-4
+
+
+# ---------------------------------------------------------------- GPU
+
+
+def _solve_on_gpu(p, device, *, graph: bool):
+    import torch
+
+    m, d, ctx, nsolving = NC.device_objects(p, device)
+    if graph:
+        # the whole solve as one graph of the caller's: nothing in it may touch the host
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            NF.solve(m, d, ctx, nsolving)  # first use outside the capture (lazy initialisations)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        m, d, ctx, nsolving = NC.device_objects(p, device)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            NF.solve(m, d, ctx, nsolving)
+        g.replay()
+    else:
+        NF.solve(m, d, ctx, nsolving)
+    torch.cuda.synchronize()
+    return m, d, ctx, nsolving
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,nworld,stage,graph", [
+    ("humanoid", 300, "dense", False), ("humanoid", 300, "tree", False), ("g1", 200, "sparse", False),
+    ("humanoid", 4096, "tree", True), ("humanoid", 4096, "dense", True), ("g1", 8192, "sparse", True),
+    ("snu", 4096, "sparse", True), ("ant", 64, "tree", True), ("snu", 130, "tree", False),
+])  # fmt: skip
+def test_gpu_solve_from_init_context_matches_the_oracle_chain(device, name, nworld, stage, graph):
+    small = nworld <= 300
+    p = NC.problem(name, nworld, stage, empty_every=11 if small else 97, warmstart=small, maxiter=12)
+    s = NC.oracle_solve(p)
+    m, d, ctx, nsolving = _solve_on_gpu(p, device, graph=graph)
+    NC.compare(p, s, d, ctx)
+    assert int(nsolving.item()) == int((p.nefc == 0).sum())  # every world that had rows has reported done
