@@ -868,6 +868,55 @@ int im_newton_tree_stage(const im_tree_plan *plan, const uint8_t *skip, const fl
                          int64_t ld_search, float *search_dot, float *decrement, int block, int nworld,
                          void *stream);
 
+/* The arrays of the fused Newton loop, named as the reference's run() hands them to its kernel
+ * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:330-393).  Rows are contiguous floats or
+ * int32: nv per world for qacc, efc_Ma, qfrc_smooth, qfrc_constraint, search, mv; njmax per world
+ * for efc_D, efc_frictionloss, efc_force, efc_state, Jaref, jv; one element per world for the
+ * scalars; done, ls_exhausted and search_unchanged are bytes.  ne, nf, nefc, efc_frictionloss (with
+ * nf), overflow and nsolving may be null.  The tolerance arrays are indexed by world modulo their
+ * length. */
+typedef struct im_newton_args {
+  const float *opt_tolerance, *opt_ls_tolerance, *stat_meaninertia;
+  int32_t ntolerance, nls_tolerance, nmeaninertia;
+  int32_t ls_iterations, iterations; /* m.opt.ls_iterations, m.opt.iterations */
+  int32_t block;                     /* lanes whose summation order the dot products follow: 32 or 64 (newton_block_dim) */
+  int32_t quad;                      /* ConstraintState.QUADRATIC */
+  int32_t ls_overflow_bit, iterations_overflow_bit; /* OverflowType bits or-ed into overflow */
+  const int32_t *M_mulm_rowadr, *M_mulm_col, *M_mulm_madr; /* row tables of M v: nv + 1 offsets, nterm terms */
+  int32_t nterm;
+  const int32_t *ne, *nf, *nefc;
+  const float *M; /* (nworld, ldM) tree CSR */
+  int64_t ldM;
+  const float *efc_J; /* (nworld, njmax, nv) */
+  int32_t njmax;
+  const float *efc_D, *efc_frictionloss, *qfrc_smooth;
+  float *qacc, *efc_Ma, *efc_force;
+  int32_t *efc_state;
+  float *Jaref, *search, *search_dot, *mv, *jv, *alpha, *improvement;
+  float *grad; /* (nworld, ld_grad) */
+  int64_t ld_grad;
+  float *grad_dot, *grad_scale, *newton_decrement, *qfrc_constraint;
+  int32_t *quad_changed_ids; /* (nworld, ld_ids) */
+  int32_t ld_ids;
+  int32_t *quad_changed_count, *state_changed_count, *solver_niter, *overflow, *nsolving;
+  uint8_t *done, *ls_exhausted, *search_unchanged;
+  int32_t nworld;
+} im_newton_args;
+
+/* Replaces the launch of solve_incremental_newton_kernel
+ * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:57-298, launched at :396-409) for a model
+ * whose factor stage is the tree stage of im_newton_tree_stage: one resident kernel, a wavefront per
+ * world and four worlds per workgroup, that iterates every world from the state init_context left
+ * until it converges or m.opt.iterations is reached -- M search, J search, line search, step,
+ * constraint states, gradient, factor stage, convergence test, with the operations of
+ * im_mul_m_sparse, im_newton_jv, im_newton_linesearch, im_newton_advance,
+ * im_newton_eval_constraints, im_newton_gradient, im_newton_tree_stage and im_newton_converged in
+ * their order, so the arrays end as after those launches repeated, bit for bit.  No host
+ * synchronisation, nothing allocated; the loop is bounded by `iterations` whatever the data.
+ * Needs generated kernels on the plan (IM_ERR_UNSUPPORTED otherwise: the caller then issues the
+ * stages one by one). */
+int im_newton_solve_tree(const im_tree_plan *plan, const im_newton_args *args, void *stream);
+
 /* Replaces _init_efc_settling_empty_worlds
  * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:412-428): solver_niter = 0,
  * search_dot = 0, done = (nefc == 0), and a world without constraint rows gets

@@ -64,6 +64,29 @@ class MuscleForceVelocityModel(C.Structure):
     _fields_ = [("vmax", C.c_float), ("fvmax", C.c_float), ("clamp_activation", C.c_float), ("include_active", C.c_float)]
 
 
+class NewtonArgs(C.Structure):
+    """im_newton_args"""
+
+    _fields_ = [
+        ("opt_tolerance", C.c_void_p), ("opt_ls_tolerance", C.c_void_p), ("stat_meaninertia", C.c_void_p),
+        ("ntolerance", C.c_int32), ("nls_tolerance", C.c_int32), ("nmeaninertia", C.c_int32),
+        ("ls_iterations", C.c_int32), ("iterations", C.c_int32), ("block", C.c_int32), ("quad", C.c_int32),
+        ("ls_overflow_bit", C.c_int32), ("iterations_overflow_bit", C.c_int32),
+        ("M_mulm_rowadr", C.c_void_p), ("M_mulm_col", C.c_void_p), ("M_mulm_madr", C.c_void_p), ("nterm", C.c_int32),
+        ("ne", C.c_void_p), ("nf", C.c_void_p), ("nefc", C.c_void_p),
+        ("M", C.c_void_p), ("ldM", C.c_int64), ("efc_J", C.c_void_p), ("njmax", C.c_int32),
+        ("efc_D", C.c_void_p), ("efc_frictionloss", C.c_void_p), ("qfrc_smooth", C.c_void_p),
+        ("qacc", C.c_void_p), ("efc_Ma", C.c_void_p), ("efc_force", C.c_void_p), ("efc_state", C.c_void_p),
+        ("Jaref", C.c_void_p), ("search", C.c_void_p), ("search_dot", C.c_void_p), ("mv", C.c_void_p), ("jv", C.c_void_p),
+        ("alpha", C.c_void_p), ("improvement", C.c_void_p), ("grad", C.c_void_p), ("ld_grad", C.c_int64),
+        ("grad_dot", C.c_void_p), ("grad_scale", C.c_void_p), ("newton_decrement", C.c_void_p),
+        ("qfrc_constraint", C.c_void_p), ("quad_changed_ids", C.c_void_p), ("ld_ids", C.c_int32),
+        ("quad_changed_count", C.c_void_p), ("state_changed_count", C.c_void_p), ("solver_niter", C.c_void_p),
+        ("overflow", C.c_void_p), ("nsolving", C.c_void_p),
+        ("done", C.c_void_p), ("ls_exhausted", C.c_void_p), ("search_unchanged", C.c_void_p), ("nworld", C.c_int32),
+    ]  # fmt: skip
+
+
 class RowPairTerm(C.Structure):
     """im_row_pair_term"""
 
@@ -228,6 +251,7 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _vp, _i, _i, _vp],
     ),
+    "im_newton_solve_tree": (_i, [_vp, C.POINTER(NewtonArgs), _vp]),
     "im_newton_advance": (
         _i,
         [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _vp],

@@ -162,7 +162,7 @@ def _spilling_fused_kernels(remarks: str) -> list[str]:
         if m:
             name = m.group(1)
         m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
-        if m and name and int(m.group(1)) > 0 and "ILb1E" in name:
+        if m and name and int(m.group(1)) > 0 and "tree_row16_" in name and "ILb1E" in name:
             out.append(f"{name}: {m.group(1)} B/lane")
     return out
 

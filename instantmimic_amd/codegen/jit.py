@@ -97,7 +97,7 @@ def kernel_resources(blob: bytes) -> dict[str, tuple[int, int]]:
 
 def spilling_kernels(blob: bytes) -> list[str]:
     """The fused kernels of a code object that use a private segment (register spills to memory)."""
-    return sorted(name for name, (_, private) in kernel_resources(blob).items() if private and name != "im_row16_solve")
+    return sorted(name for name, (_, private) in kernel_resources(blob).items() if private and name in ("im_row16_fused", "im_row16_fused_long"))
 
 
 def code_object(structure, groups, trunk) -> bytes | None:

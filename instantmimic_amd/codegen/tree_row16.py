@@ -206,12 +206,16 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
         emit("  {" + ",".join(str(v) for v in row) + "},")
     emit("};")
     # LONG: more constraint rows than the straight-line assembly keeps in flight (a loop instead)
+    # the body as a function: the kernels at the end of the file call it, the resident Newton
+    # kernel once per iteration
     emit("template <bool ASM, bool LONG>")
-    if module:  # the body as a function: the kernels with C names at the end of the file call it
-        emit(f"__device__ __forceinline__ void tree_row16_{name}(IM_ROW16_PARAMS) {{")
-    else:
-        emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? IM_OCC_{name} : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
-    emit("  const int lane = threadIdx.x & 63, p = lane & 15, wv = threadIdx.x >> 6;")
+    emit(f"__device__ __forceinline__ void tree_row16_body_{name}(IM_ROW16_PARAMS) {{")
+    # the lane number as a value the compiler cannot see through: called from a loop (the resident
+    # Newton kernel), nothing derived from it counts as loop-invariant, so no table entry or address
+    # of this body is kept in a register from one call to the next
+    emit("  int lane_ = threadIdx.x & 63;")
+    emit('  asm volatile("" : "+v"(lane_));')
+    emit("  const int lane = lane_, p = lane & 15, wv = threadIdx.x >> 6;")
     # Several iterations in one launch (fused kernels only): the grid covers (four worlds, iteration)
     # pairs.  Workgroups go to the chip's eight XCDs in turn, each with an L2 of its own, so the
     # iterations of one group of worlds take consecutive workgroups of one XCD: they run at about
@@ -881,20 +885,49 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("  STAMP();")
     emit("  #undef STAMP")
     emit("}")
+    args = "M, ldM, J, njmax, D, state, nefc_p, quad, y, ldy, x, ldx, Hout, nworld, flags, niter, state_it, y_it, x_it, skip"
+    ju = 16 if nv <= 16 else 32  # loads in flight per lane while rows of J are staged (a register each)
+    # The resident Newton loop with this tree's fused kernel as its factor stage: search = -H^-1 grad
+    # for the workgroup's four worlds, those whose `unchanged` byte is set left alone.  LONG decides
+    # the rows a lane of the line search keeps in registers: two up to 64 rows, four up to 128.
+    emit("template <bool LONG>")
+    emit(f"__device__ __forceinline__ void newton_row16_body_{name}(const im::resident::NewtonArgs &a) {{")
+    emit("  extern __shared__ float xlds[];")
+    emit("  auto stage = [&]() __attribute__((always_inline)) {")
+    emit(f"    tree_row16_body_{name}<true, LONG>(a.M, a.ldM, a.J, a.njmax, a.D, a.state, a.nefc, a.quad, a.grad, a.ld_grad, a.search,")
+    emit("        (int64_t)a.nv, nullptr, a.nworld, IM_FLAG_NEGATE, 1, 0, 0, 0, a.unchanged);")
+    emit("  };")
+    emit("  if (LONG && a.njmax > 128)")
+    emit(f"    im::resident::newton_loop<0, {ju}>(a, xlds, stage);")
+    emit("  else")
+    emit(f"    im::resident::newton_loop<(LONG ? 4 : 2), {ju}>(a, xlds, stage);")
+    emit("}")
     if module:
-        args = "M, ldM, J, njmax, D, state, nefc_p, quad, y, ldy, x, ldx, Hout, nworld, flags, niter, state_it, y_it, x_it, skip"
         emit("} }  // namespace im::gen")
         for kernel, asm_, long_, bounds in (("fused", "true", "false", f"256, IM_OCC_{name}"), ("fused_long", "true", "true", f"256, IM_OCC_{name}"),
                                             ("solve", "false", "false", "64, 1")):  # fmt: skip
             emit(f'extern "C" __global__ __launch_bounds__({bounds}) void im_row16_{kernel}(IM_ROW16_PARAMS) {{')
-            emit(f"  im::gen::tree_row16_{name}<{asm_}, {long_}>({args});")
+            emit(f"  im::gen::tree_row16_body_{name}<{asm_}, {long_}>({args});")
+            emit("}")
+        for kernel, long_ in (("newton", "false"), ("newton_long", "true")):
+            emit(f'extern "C" __global__ __launch_bounds__(256, IM_OCC_{name}) void im_row16_{kernel}(im::resident::NewtonArgs a) {{')
+            emit(f"  im::gen::newton_row16_body_{name}<{long_}>(a);")
             emit("}")
         emit(f'extern "C" __device__ const unsigned long long im_row16_key = 0x{key:016x}ull;')
         emit(f'extern "C" __device__ const int im_row16_info[4] = {{{nv}, {nM}, {lds_floats * 4}, {4 * PD}}};  // nv, nM, LDS bytes, short rows')
     else:
+        emit("template <bool ASM, bool LONG>")
+        emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? IM_OCC_{name} : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
+        emit(f"  tree_row16_body_{name}<ASM, LONG>({args});")
+        emit("}")
+        emit("template <bool LONG>")
+        emit(f"__global__ __launch_bounds__(256, IM_OCC_{name}) void newton_row16_{name}(im::resident::NewtonArgs a) {{")
+        emit(f"  newton_row16_body_{name}<LONG>(a);")
+        emit("}")
         emit(f"static const Row16Entry entry_{name} = {{0x{key:016x}ull, {nv}, {nM}, {lds_floats * 4}, {4 * PD}, \"{name}\",")
         emit(f"    (const void *)tree_row16_{name}<true, false>, (const void *)tree_row16_{name}<true, true>,")
-        emit(f"    (const void *)tree_row16_{name}<false, false>}};")
+        emit(f"    (const void *)tree_row16_{name}<false, false>, (const void *)newton_row16_{name}<false>,")
+        emit(f"    (const void *)newton_row16_{name}<true>}};")
         emit(f"static const Row16Register reg_{name}(&entry_{name});")
         emit("} }  // namespace im::gen")
     # workgroups per CU that the fused kernel is compiled for: what the 160 KB of LDS admit (with

@@ -1,0 +1,342 @@
+// The resident Newton loop: one wavefront per world from the first line search to convergence,
+// four worlds per workgroup, as the reference keeps a world in one block for the whole loop
+// (src/instantmimic/utils/mjw_kernels/newton_fusion.py:57-298).  Per iteration and world, in the
+// reference kernel's order (:170-296): M search, J search, the scalar line search with the step
+// and the constraints' new forces and states (newton_stages.py:79-444), the gradient (:745-798),
+// the factor stage, the convergence test.  Every stage performs the operations of the per-stage
+// kernels of this library in their order, so a solve gives the same bits whichever way it runs.
+//
+// The factor stage is handed in by the kernel that includes this file (a generated kernel for the
+// model's tree: four wavefronts work on the workgroup's four worlds together), which is why the
+// loop keeps the four wavefronts in step at two workgroup barriers per iteration; a world that is
+// done idles through them until the workgroup's last world finishes.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "newton_search.h"
+
+namespace im {
+namespace resident {
+
+struct NewtonArgs {
+  // options (arrays indexed by world modulo their length)
+  const float *tolerance, *ls_tolerance, *meaninertia;
+  int ntolerance, nls_tolerance, nmeaninertia;
+  int nv, njmax, nworld, ls_iterations, maxiter, block, quad, ls_overflow_bit, iter_overflow_bit;
+  // row tables of M v: nv + 1 offsets, then per term the column and the element of M
+  const int32_t *mulm_rowadr, *mulm_col, *mulm_madr;
+  int nterm, nM;
+  // the step's inputs
+  const int32_t *ne, *nf, *nefc;
+  const float *M;
+  int64_t ldM;
+  const float *J, *D, *frictionloss, *smooth;  // J (nworld, njmax, nv); D, frictionloss (nworld, njmax); smooth (nworld, nv)
+  // solver state, rows of nv or njmax floats per world unless a stride is given
+  float *qacc, *Ma, *force, *Jaref, *search, *search_dot, *mv, *jv, *alpha, *improvement, *grad, *grad_dot,
+      *grad_scale, *decrement, *qfrc_constraint;
+  int64_t ld_grad;
+  int32_t *state, *ids, *quad_count, *state_count, *niter, *overflow, *nsolving;
+  int ld_ids;
+  uint8_t *done, *exhausted, *unchanged;
+  int stage_lds_floats;  // dynamic LDS the factor stage uses from offset 0; the loop's own arrays follow
+};
+
+__device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+
+// orders this wavefront's writes (LDS and memory) before its later reads: the stages hand their
+// results on through memory, written by some lanes and read by others
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__device__ __forceinline__ void block_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// words of LDS of the loop's own arrays behind the factor stage's area: four flags, the row tables of M v
+// (one word per term, nv + 1 offsets), then per wavefront the world's row of M, the search
+// direction, the gradient stage's list of rows with a force (value and row number), its copy of the
+// gradient and 64 words of lane sums.  The factor stage's area must also hold four wavefronts'
+// staged rows of J: 4 x 64 rows, a row nv | 1 words.
+__host__ __device__ inline size_t loop_lds_words(int nv, int njmax, int nM, int nterm) {
+  return 4 + (size_t)nterm + nv + 1 + 4 * ((size_t)nM + nv + 2 * (size_t)njmax + nv + 64);
+}
+__host__ __device__ inline size_t staged_rows_words(int nv) { return 4 * 64 * (size_t)(nv | 1); }
+
+// ---- M search (newton_fusion.py:171-176): lane d owns dofs d, d + 64 --------------------------
+__device__ __forceinline__ void mul_m_world(const NewtonArgs &a, const uint32_t *term, const int *radr, const float *m,
+                                            const float *v, float *out, int lane) {
+  for (int dof = lane; dof < a.nv; dof += 64) {
+    float value = 0.0f;
+    const int end = radr[dof + 1];
+    for (int k = radr[dof]; k < end; k += 4) {  // four terms' operands at a time, a term past the end dropped
+      float x[4], y[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t t = term[k + u < end ? k + u : end - 1];
+        x[u] = m[t >> 16];
+        y[u] = v[t & 0xffffu];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) value = k + u < end ? fma_(x[u], y[u], value) : value;
+    }
+    out[dof] = value;
+  }
+}
+
+// ---- J search (newton_stages.py:157-178): 64 rows at a time through LDS, a lane per row --------
+template <int U>
+__device__ __forceinline__ void jv_world(const NewtonArgs &a, const float *Jw, int nefc, float *rows_lds,
+                                         const float *sv, float *jv, int lane) {
+  const int nv = a.nv, stride = nv | 1;
+  const float inv_nv = 1.0f / (float)nv;
+  for (int r0 = 0; r0 < nefc; r0 += 64) {
+    const int rows = nefc - r0 < 64 ? nefc - r0 : 64;
+    const float *src = Jw + (int64_t)r0 * nv;
+    const int total = rows * nv;
+    for (int i0 = lane; i0 < total; i0 += U * 64) {
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = src[i0 + 64 * u < total ? i0 + 64 * u : total - 1];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = i0 + 64 * u;
+        if (i < total) {
+          const int r = (int)(((float)i + 0.5f) * inv_nv);  // i / nv, exact while i stays below 2^20
+          rows_lds[r * stride + (i - r * nv)] = v[u];
+        }
+      }
+    }
+    wave_sync();
+    if (lane < rows) {
+      const float *row = rows_lds + lane * stride;
+      auto chain = [&](int i0, int i1) {
+        float p = 0.0f;
+        int i = i0;
+        for (; i + 8 <= i1; i += 8) {
+          float x[8], y[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            x[u] = row[i + u];
+            y[u] = sv[i + u];
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) p = fma_(x[u], y[u], p);
+        }
+        for (; i < i1; ++i) p = fma_(row[i], sv[i], p);
+        return p;
+      };
+      float acc = 0.0f;
+      if (nv > 50) {
+        for (int start = 0; start < nv; start += 20) acc = acc + chain(start, start + 20 < nv ? start + 20 : nv);
+      } else {
+        acc = chain(0, nv);
+      }
+      jv[r0 + lane] = acc;
+    }
+    wave_sync();  // the rows are read before the next 64 overwrite them
+  }
+}
+
+// ---- the gradient (newton_stages.py:745-798), a lane per dof ------------------------------------
+// Returns whether the search direction stays as it is (no state changed).
+__device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, const float *Jw, int nefc, float *f,
+                                               int *rowl, float *gl, float *part, int lane) {
+  const bool changed = a.state_count[w] != 0;
+  if (!changed) {
+    if (lane == 0) {
+      const float sigma = a.grad_scale[w], new_sigma = sigma - a.alpha[w];
+      float ratio = 0.0f;
+      if (sigma != 0.0f) ratio = new_sigma / sigma;
+      const float ratio_sq = ratio * ratio;
+      a.grad_dot[w] = a.grad_dot[w] * ratio_sq;
+      a.decrement[w] = a.decrement[w] * ratio_sq;
+      a.grad_scale[w] = new_sigma;
+      a.unchanged[w] = 1;
+    }
+    return true;
+  }
+  const int nv = a.nv;
+  // rows with a force, in order (a satisfied constraint's force is zero and its row adds nothing)
+  int cnt = 0;
+  for (int r0 = 0; r0 < nefc; r0 += 64) {
+    const int r = r0 + lane;
+    const float v = r < nefc ? a.force[w * a.njmax + r] : 0.0f;
+    const unsigned long long mask = __ballot(v != 0.0f);
+    if (v != 0.0f) {
+      const int pos = cnt + __popcll(mask & ((1ull << lane) - 1ull));
+      f[pos] = v;
+      rowl[pos] = r;
+    }
+    cnt += __popcll(mask);
+  }
+  wave_sync();
+  constexpr int ROWS = 8;
+  for (int dof = lane; dof < nv; dof += 64) {
+    const float ma = a.Ma[w * nv + dof], sm = a.smooth[w * nv + dof];
+    float sum = 0.0f;
+    for (int p0 = 0; p0 < cnt; p0 += ROWS) {
+      float jv[ROWS];
+#pragma unroll
+      for (int u = 0; u < ROWS; ++u) jv[u] = Jw[(int64_t)rowl[p0 + u < cnt ? p0 + u : cnt - 1] * nv + dof];
+#pragma unroll
+      for (int u = 0; u < ROWS; ++u) sum = p0 + u < cnt ? fma_(jv[u], f[p0 + u], sum) : sum;
+    }
+    const float g = ma - sm - sum;
+    a.qfrc_constraint[w * nv + dof] = sum;
+    a.grad[w * a.ld_grad + dof] = g;
+    gl[dof] = g;
+  }
+  wave_sync();
+  // grad . grad as a block of `block` lanes sums it: lane `rank` its dofs rank, rank + block, ..,
+  // 32 lanes in a shuffle-down tree, the trees in order
+  float p = 0.0f;
+  if (lane < a.block)
+    for (int dof = lane; dof < nv; dof += a.block) p = fma_(gl[dof], gl[dof], p);
+  for (int off = 16; off > 0; off >>= 1) p = p + __shfl_down(p, off, 32);
+  const float second = __shfl(p, 32, 64);
+  if (lane == 0) {
+    float total = 0.0f + p;
+    if (a.block > 32) total = total + second;
+    a.grad_dot[w] = total;
+    a.decrement[w] = 0.0f;
+    a.grad_scale[w] = 1.0f;
+    a.unchanged[w] = 0;
+  }
+  return false;
+}
+
+// ---- search . search and grad . x of a factor stage that leaves only the search direction -----
+__device__ __forceinline__ void search_sums_world(const NewtonArgs &a, int64_t w, int lane) {
+  float s0 = 0.0f, s1 = 0.0f;
+  for (int d = lane; d < a.nv && lane < a.block; d += a.block) {
+    const float v = -a.search[w * a.nv + d];
+    s0 = fma_(v, v, s0);
+    s1 = fma_(a.grad[w * a.ld_grad + d], v, s1);
+  }
+  for (int o = 16; o > 0; o >>= 1) {
+    s0 = s0 + __shfl_down(s0, o, 32);
+    s1 = s1 + __shfl_down(s1, o, 32);
+  }
+  const float a1 = __shfl(s0, 32, 64), b1 = __shfl(s1, 32, 64);
+  if (lane == 0) {
+    float ra = 0.0f + s0, rb = 0.0f + s1;
+    if (a.block > 32) ra = ra + a1, rb = rb + b1;
+    a.search_dot[w] = ra;
+    a.decrement[w] = rb;
+  }
+}
+
+// ---- the loop ------------------------------------------------------------------------------------
+// HELD: rows of a world a lane keeps in registers during the line search (0: read at every
+// evaluation); JU: loads in flight per lane while rows of J are staged.  `stage()` runs the factor
+// stage for the workgroup's four worlds (every wavefront calls it; it skips the worlds whose
+// `unchanged` byte is set).  `lds`: the workgroup's dynamic LDS.
+template <int HELD, int JU, class Stage>
+__device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Stage &&stage) {
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int64_t w_raw = (int64_t)blockIdx.x * 4 + wv;
+  const bool live = w_raw < a.nworld;
+  const int64_t w = live ? w_raw : (int64_t)a.nworld - 1;
+  const int nv = a.nv, njmax = a.njmax;
+  const int nM = a.nM;
+  // LDS: the factor stage's area (the staged rows of J use it between two stages), then the row
+  // tables of M v for the workgroup, then each wavefront's own arrays
+  int *votes = (int *)(lds + a.stage_lds_floats);  // [4] a wavefront's world is still being solved
+  uint32_t *term = (uint32_t *)(votes + 4);
+  int *radr = (int *)(term + a.nterm);
+  float *mine = (float *)(radr + nv + 1) + wv * (nM + nv + 2 * njmax + nv + 64);
+  float *m_lds = mine;              // [nM]
+  float *sv = m_lds + nM;           // [nv] the search direction
+  float *f = sv + nv;               // [njmax] forces of the listed rows
+  int *rowl = (int *)(f + njmax);   // [njmax] their numbers
+  float *gl = (float *)(rowl + njmax);  // [nv]
+  float *part = gl + nv;            // [64]
+  float *rows_lds = lds + wv * (64 * (nv | 1));  // inside the factor stage's area
+  for (int k = threadIdx.x; k < a.nterm; k += 256) term[k] = (uint32_t)a.mulm_col[k] | (uint32_t)a.mulm_madr[k] << 16;
+  for (int k = threadIdx.x; k <= nv; k += 256) radr[k] = a.mulm_rowadr[k];
+  for (int k = lane; k < nM; k += 64) m_lds[k] = a.M[w * a.ldM + k];
+  bool done = !live || a.done[w] != 0;
+  if (live && done && lane == 0) a.unchanged[w] = 1;  // the factor stage leaves such a world alone
+  bool unchanged = !done && a.unchanged[w] != 0;
+  int nefc = a.nefc ? a.nefc[w] : njmax;
+  nefc = __builtin_amdgcn_readfirstlane(nefc < njmax ? nefc : njmax);
+  const float *Jw = a.J + w * (int64_t)njmax * nv;
+  search::SearchArgs sa{a.tolerance, a.ls_tolerance, a.meaninertia, a.ntolerance, a.nls_tolerance, a.nmeaninertia, a.ne, a.nf,
+                        a.nefc, a.smooth, a.D, a.frictionloss, a.Jaref, a.search, a.search_dot, a.mv, a.jv, a.Ma, nv, njmax,
+                        njmax, njmax, nv, nv, njmax, nv, nullptr, a.alpha, a.improvement, a.exhausted, a.overflow,
+                        a.ls_overflow_bit, nv, njmax, a.ls_iterations, a.nworld};
+  block_sync();
+  // every wavefront leaves the loop after at most maxiter rounds, whatever the data
+  const int lane_fixed = lane;
+  for (int round = 0; round < a.maxiter; ++round) {
+    if (lane_fixed == 0) votes[wv] = done ? 0 : 1;
+    block_sync();
+    if (!(votes[0] | votes[1] | votes[2] | votes[3])) break;  // the workgroup's four worlds are done
+    // the lane number as a value the compiler cannot see through, new in every round: nothing a
+    // stage derives from it is kept in registers across the other stages
+    int lane = lane_fixed;
+    asm volatile("" : "+v"(lane));
+    if (!done) {
+      if (!unchanged) {
+        for (int k = lane; k < nv; k += 64) sv[k] = a.search[w * nv + k];
+        wave_sync();
+        mul_m_world(a, term, radr, m_lds, sv, a.mv + w * nv, lane);
+        jv_world<JU>(a, Jw, nefc, rows_lds, sv, a.jv + w * njmax, lane);
+        wave_sync();
+      }
+      search::linesearch_world<HELD>(sa, w, lane & 31);
+      wave_sync();
+      {  // the step (newton_stages.py:373-381)
+        const float al = a.alpha[w];
+        for (int i = lane; i < nv; i += 64) {
+          a.qacc[w * nv + i] = fma_(al, a.search[w * nv + i], a.qacc[w * nv + i]);
+          a.Ma[w * nv + i] = fma_(al, a.mv[w * nv + i], a.Ma[w * nv + i]);
+        }
+        for (int i = lane; i < nefc; i += 64) a.Jaref[w * njmax + i] = a.Jaref[w * njmax + i] + al * a.jv[w * njmax + i];
+      }
+      wave_sync();
+      search::eval_constraints_world(a.Jaref, njmax, a.D, njmax, a.frictionloss, njmax, a.ne, a.nf, a.nefc, njmax,
+                                     a.exhausted, a.force, njmax, a.state, njmax, a.ids, a.ld_ids, a.quad_count,
+                                     a.state_count, w, lane);
+      wave_sync();
+      unchanged = gradient_world(a, w, Jw, nefc, f, rowl, gl, part, lane);
+    }
+    block_sync();  // gradients, states and the `unchanged` bytes of the four worlds are in place; the rows of J are done with
+    stage();
+    block_sync();  // the four search directions are complete
+    lane = lane_fixed;
+    asm volatile("" : "+v"(lane));  // no address from before the stage is kept through it
+    if (!done) {
+      if (!unchanged) search_sums_world(a, w, lane);
+      wave_sync();
+      int finished = 0;
+      if (lane == 0) {  // newton_fusion.py:265-296
+        const int it = a.niter[w] + 1;
+        a.niter[w] = it;
+        const float tol = a.tolerance[w % a.ntolerance], scale = a.meaninertia[w % a.nmeaninertia] * (float)nv;
+        const float imp = a.improvement[w];
+        const bool converged = a.alpha[w] == 0.0f || (imp > 0.0f && imp / scale < tol) ||
+                               sqrtf(a.grad_dot[w]) / scale < tol || 0.5f * a.decrement[w] / scale < tol;
+        if (converged || it == a.maxiter) {
+          if (!converged && a.overflow) a.overflow[w] = a.overflow[w] | a.iter_overflow_bit;
+          a.done[w] = 1;
+          a.unchanged[w] = 1;
+          if (a.nsolving) atomicAdd(a.nsolving, -1);
+          finished = 1;
+        }
+      }
+      done = __builtin_amdgcn_readfirstlane(finished) != 0;
+    }
+  }
+}
+
+}  // namespace resident
+}  // namespace im

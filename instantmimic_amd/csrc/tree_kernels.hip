@@ -586,6 +586,19 @@ int tree_plan_upload(im_tree_plan *pl) {
       IM_HIP_CHECK(hipFuncSetAttribute(e->fused, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
       IM_HIP_CHECK(hipFuncSetAttribute(e->fused_long, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     }
+    // the resident Newton loop keeps its own arrays behind the stage's
+    // ... and is used only where it keeps to registers and the runtime grants the LDS
+    // (im_newton_solve_tree says unsupported otherwise)
+    auto usable = [](const void *fn) {
+      hipFuncAttributes fa{};
+      const bool ok = hipFuncGetAttributes(&fa, fn) == hipSuccess && fa.localSizeBytes == 0 &&
+                      hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          160 * 1024 - (int)fa.sharedSizeBytes) == hipSuccess;
+      (void)hipGetLastError();
+      return ok;
+    };
+    pl->resident_ok = usable(e->newton);
+    pl->resident_long_ok = usable(e->newton_long);
   }
   return IM_OK;
 }
@@ -646,11 +659,16 @@ int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object) {
   // write out of place
   if (key != im::tree_key(*plan) || info[0] != plan->nv || info[1] != plan->nM) return fail(IM_ERR_STRUCTURE);
   if (info[2] <= 0 || info[2] + 32 * 64 > 160 * 1024 || info[3] <= 0) return fail(IM_ERR_UNSUPPORTED);
-  hipFunction_t fused = nullptr, fused_long = nullptr, solve = nullptr;
+  hipFunction_t fused = nullptr, fused_long = nullptr, solve = nullptr, newton = nullptr, newton_long = nullptr;
   if (hipModuleGetFunction(&fused, mod, "im_row16_fused") != hipSuccess ||
       hipModuleGetFunction(&fused_long, mod, "im_row16_fused_long") != hipSuccess ||
       hipModuleGetFunction(&solve, mod, "im_row16_solve") != hipSuccess)
     return fail(IM_ERR_STRUCTURE);
+  if (hipModuleGetFunction(&newton, mod, "im_row16_newton") != hipSuccess ||
+      hipModuleGetFunction(&newton_long, mod, "im_row16_newton_long") != hipSuccess) {
+    newton = newton_long = nullptr;  // a code object without the resident loop: the stages are launched one by one
+    (void)hipGetLastError();
+  }
   // a fused kernel that spills registers to memory is not taken: the plan keeps the table-driven
   // kernel (the generator's callers check the code object's descriptors before they get here)
   auto spills = [](hipFunction_t f) {
@@ -658,6 +676,7 @@ int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object) {
     return hipFuncGetAttribute(&bytes, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, f) == hipSuccess && bytes > 0;
   };
   if (spills(fused) || spills(fused_long)) return fail(IM_ERR_UNSUPPORTED);
+  const bool newton_ok = newton && !spills(newton), newton_long_ok = newton_long && !spills(newton_long);
   if (info[2] + 32 * 64 > 48 * 1024) {
     // more than the default dynamic LDS: asked for here; a runtime that refuses the request for a
     // module's function reports it at the launch
@@ -665,12 +684,25 @@ int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object) {
     (void)hipFuncSetAttribute((const void *)fused_long, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     (void)hipGetLastError();
   }
+  // the resident loop's own arrays come on top of the stage's
+  auto grant = [](hipFunction_t f) {
+    int fixed = 0;
+    (void)hipFuncGetAttribute(&fixed, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, f);
+    const bool ok = hipFuncSetAttribute((const void *)f, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        160 * 1024 - fixed) == hipSuccess;
+    (void)hipGetLastError();
+    return ok;
+  };
+  const bool newton_lds = newton && grant(newton), newton_long_lds = newton_long && grant(newton_long);
   // plain data, released with free() when the plan goes
   auto *e = (im::gen::Row16Entry *)std::malloc(sizeof(im::gen::Row16Entry));
   if (!e) return fail(IM_ERR_ARG);
   *e = im::gen::Row16Entry{key, info[0], info[1], info[2], info[3], "module", (const void *)fused,
-                           (const void *)fused_long, (const void *)solve};
+                           (const void *)fused_long, (const void *)solve, (const void *)newton,
+                           (const void *)newton_long};
   plan->module = mod;
+  plan->resident_ok = newton_ok && newton_lds;
+  plan->resident_long_ok = newton_long_ok && newton_long_lds;
   plan->row16_own = e;
   plan->row16 = e;
   return IM_OK;
@@ -727,6 +759,62 @@ int im_newton_tree_stage(const im_tree_plan *plan, const uint8_t *skip, const fl
                      (hipStream_t)stream, skip, grad, ldg, search, ld_search, search_dot, decrement, plan->nv, block,
                      nworld);
   IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_newton_solve_tree(const im_tree_plan *plan, const im_newton_args *p, void *stream) {
+  if (!plan || !p || p->nworld < 0) return IM_ERR_ARG;
+  if (!plan->device_ready || !plan->row16) return IM_ERR_UNSUPPORTED;
+  const auto *e = (const im::gen::Row16Entry *)plan->row16;
+  if (!e->newton || !e->newton_long) return IM_ERR_UNSUPPORTED;
+  if (p->nworld == 0) return IM_OK;
+  const int nv = plan->nv, nM = plan->nM, njmax = p->njmax;
+  if (njmax <= 0 || p->iterations < 0 || p->ls_iterations < 0 || (p->block != 32 && p->block != 64) ||
+      p->ntolerance <= 0 || p->nls_tolerance <= 0 || p->nmeaninertia <= 0 || p->nterm <= 0)
+    return IM_ERR_ARG;
+  if (!p->opt_tolerance || !p->opt_ls_tolerance || !p->stat_meaninertia || !p->M_mulm_rowadr || !p->M_mulm_col ||
+      !p->M_mulm_madr || !p->M || !p->efc_J || !p->efc_D || !p->qfrc_smooth || !p->qacc || !p->efc_Ma ||
+      !p->efc_force || !p->efc_state || !p->Jaref || !p->search || !p->search_dot || !p->mv || !p->jv || !p->alpha ||
+      !p->improvement || !p->grad || !p->grad_dot || !p->grad_scale || !p->newton_decrement || !p->qfrc_constraint ||
+      !p->quad_changed_ids || !p->quad_changed_count || !p->state_changed_count || !p->solver_niter || !p->done ||
+      !p->ls_exhausted || !p->search_unchanged || (p->nf && !p->efc_frictionloss))
+    return IM_ERR_ARG;
+  if (p->ldM < nM || p->ld_grad < nv || p->ld_ids < 0) return IM_ERR_STRIDE;
+  if (p->nterm >= 65536 || 64 * (int64_t)nv >= (1 << 20)) return IM_ERR_UNSUPPORTED;
+  im::resident::NewtonArgs a{};
+  a.tolerance = p->opt_tolerance, a.ls_tolerance = p->opt_ls_tolerance, a.meaninertia = p->stat_meaninertia;
+  a.ntolerance = p->ntolerance, a.nls_tolerance = p->nls_tolerance, a.nmeaninertia = p->nmeaninertia;
+  a.nv = nv, a.njmax = njmax, a.nworld = p->nworld, a.ls_iterations = p->ls_iterations, a.maxiter = p->iterations;
+  a.block = p->block, a.quad = p->quad, a.ls_overflow_bit = p->ls_overflow_bit;
+  a.iter_overflow_bit = p->iterations_overflow_bit;
+  a.mulm_rowadr = p->M_mulm_rowadr, a.mulm_col = p->M_mulm_col, a.mulm_madr = p->M_mulm_madr;
+  a.nterm = p->nterm, a.nM = nM;
+  a.ne = p->ne, a.nf = p->nf, a.nefc = p->nefc, a.M = p->M, a.ldM = p->ldM, a.J = p->efc_J, a.D = p->efc_D;
+  a.frictionloss = p->efc_frictionloss, a.smooth = p->qfrc_smooth;
+  a.qacc = p->qacc, a.Ma = p->efc_Ma, a.force = p->efc_force, a.Jaref = p->Jaref, a.search = p->search;
+  a.search_dot = p->search_dot, a.mv = p->mv, a.jv = p->jv, a.alpha = p->alpha, a.improvement = p->improvement;
+  a.grad = p->grad, a.grad_dot = p->grad_dot, a.grad_scale = p->grad_scale, a.decrement = p->newton_decrement;
+  a.qfrc_constraint = p->qfrc_constraint, a.ld_grad = p->ld_grad;
+  a.state = p->efc_state, a.ids = p->quad_changed_ids, a.quad_count = p->quad_changed_count;
+  a.state_count = p->state_changed_count, a.niter = p->solver_niter, a.overflow = p->overflow, a.nsolving = p->nsolving;
+  a.ld_ids = p->ld_ids, a.done = p->done, a.exhausted = p->ls_exhausted, a.unchanged = p->search_unchanged;
+  // the factor stage's LDS (its staged tiles and exchange slots plus the four worlds' row lists), or the
+  // four wavefronts' staged rows of J where those take more; the loop's own arrays behind it
+  const size_t stage_bytes = (size_t)e->lds_bytes + 32 * std::max<size_t>(((size_t)njmax + 15) / 16 * 16, 64);
+  const size_t stage_words = std::max(stage_bytes / 4, im::resident::staged_rows_words(nv));
+  a.stage_lds_floats = (int)stage_words;
+  const size_t lds = 4 * (stage_words + im::resident::loop_lds_words(nv, njmax, nM, p->nterm));
+  if (lds > 160 * 1024) return IM_ERR_UNSUPPORTED;
+  const bool is_long = njmax > e->short_rows;
+  if (!(is_long ? plan->resident_long_ok : plan->resident_ok)) return IM_ERR_UNSUPPORTED;  // the kernel spills registers
+  const void *fn = is_long ? e->newton_long : e->newton;
+  const unsigned grid = (unsigned)((p->nworld + 3) / 4);
+  void *args[] = {&a};
+  if (plan->module)
+    IM_HIP_CHECK(hipModuleLaunchKernel((hipFunction_t)fn, grid, 1, 1, 256, 1, 1, (unsigned)lds, (hipStream_t)stream, args,
+                                       nullptr));
+  else
+    IM_HIP_CHECK(hipLaunchKernel(fn, dim3(grid), dim3(256), args, lds, (hipStream_t)stream));
   return IM_OK;
 }
 

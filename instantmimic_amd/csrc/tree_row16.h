@@ -8,6 +8,7 @@
 #include <cstdint>
 
 #include "../../include/imhip.h"
+#include "newton_wave.h"
 
 namespace im {
 namespace gen {
@@ -89,6 +90,8 @@ struct Row16Entry {
   const void *fused;       // assemble + factor + solve, njmax <= short_rows
   const void *fused_long;  // the same with a loop over the constraint rows
   const void *solve;       // factor + solve
+  const void *newton;      // the resident Newton loop with the fused kernel as its factor stage, njmax <= short_rows
+  const void *newton_long; // the same with the loop over the constraint rows
 };
 
 // Registers a generated kernel at load time.

@@ -22,6 +22,7 @@ module.
 
 from __future__ import annotations
 
+import os
 from typing import Any
 
 import numpy as np
@@ -651,19 +652,126 @@ def iteration(m, d, ctx, nsolving=None, *, stage=None) -> None:
               nsolving=nsolving)  # fmt: skip
 
 
+def _resident_args(m, d, ctx, nsolving):
+    """The arrays of ``run`` as the C ABI's ``im_newton_args``, after the checks that no pointer may
+    leave Python without: one device, float32 / int32 / bytes, rows of the expected length."""
+    import torch
+
+    nworld, nv = int(d.nworld), int(m.nv)
+    J = d.efc.J
+    if J.dim() != 3 or not J.is_contiguous() or J.dtype != torch.float32 or not J.is_cuda or J.shape[0] != nworld or J.shape[2] != nv:
+        raise TypeError("efc_J must be a contiguous float32 CUDA tensor (nworld, njmax, nv)")
+    njmax = int(J.shape[1])
+    dev = J.device
+
+    def rows(t, width, dtype, name):
+        if t.dtype != dtype or t.device != dev or tuple(t.shape) != (nworld, width) or not t.is_contiguous():
+            raise TypeError(f"{name} must be a contiguous ({nworld}, {width}) tensor of {dtype} on {dev}")
+        return t.data_ptr()
+
+    def per_world(t, dtypes, name, optional=False):
+        if t is None and optional:
+            return None
+        if t.dtype not in dtypes or t.device != dev or t.numel() != nworld or not t.is_contiguous():
+            raise TypeError(f"{name} must be a contiguous tensor with one element per world on {dev}")
+        return t.data_ptr()
+
+    def table(t, name):
+        if t.dtype != torch.int32 or t.device != dev or not t.is_contiguous():
+            raise TypeError(f"{name} must be a contiguous int32 tensor on {dev}")
+        return t.data_ptr()
+
+    f32, i32, byte = torch.float32, torch.int32, (torch.bool, torch.uint8)
+    a = _lib.NewtonArgs()
+    for name, t in (("opt_tolerance", m.opt.tolerance), ("opt_ls_tolerance", m.opt.ls_tolerance), ("stat_meaninertia", m.stat.meaninertia)):
+        if t.dtype != f32 or t.device != dev or not t.is_contiguous() or t.numel() < 1:
+            raise TypeError(f"{name} must be a non-empty contiguous float32 tensor on {dev}")
+        setattr(a, name, t.data_ptr())
+    a.ntolerance, a.nls_tolerance, a.nmeaninertia = m.opt.tolerance.numel(), m.opt.ls_tolerance.numel(), m.stat.meaninertia.numel()
+    a.ls_iterations, a.iterations = int(m.opt.ls_iterations), int(m.opt.iterations)
+    a.block, a.quad = newton_block_dim(m), 1
+    a.ls_overflow_bit, a.iterations_overflow_bit = OVERFLOW_LS_ITERATIONS, OVERFLOW_ITERATIONS
+    if m.M_mulm_rowadr.numel() != nv + 1 or m.M_mulm_col.numel() != m.M_mulm_madr.numel():
+        raise ValueError("the row tables of M v do not match the model")
+    a.M_mulm_rowadr, a.M_mulm_col, a.M_mulm_madr = (table(t, "M_mulm_*") for t in (m.M_mulm_rowadr, m.M_mulm_col, m.M_mulm_madr))
+    a.nterm = int(m.M_mulm_col.numel())
+    a.ne, a.nf, a.nefc = (per_world(t, (i32,), n, optional=True) for t, n in ((d.ne, "ne"), (d.nf, "nf"), (d.nefc, "nefc")))
+    M = d.M
+    if M.dtype != f32 or M.device != dev or M.dim() != 2 or M.shape[0] != nworld or (M.shape[1] > 1 and M.stride(1) != 1):
+        raise TypeError("M must be a float32 (nworld, nM) tensor with contiguous rows")
+    a.M, a.ldM = M.data_ptr(), M.stride(0)
+    a.efc_J, a.njmax = J.data_ptr(), njmax
+    a.efc_D = rows(d.efc.D, njmax, f32, "efc_D")
+    a.efc_frictionloss = None if d.efc.frictionloss is None else rows(d.efc.frictionloss, njmax, f32, "efc_frictionloss")
+    a.qfrc_smooth = rows(d.qfrc_smooth, nv, f32, "qfrc_smooth")
+    a.qacc, a.efc_Ma = rows(d.qacc, nv, f32, "qacc"), rows(d.efc.Ma, nv, f32, "efc_Ma")
+    a.efc_force, a.efc_state = rows(d.efc.force, njmax, f32, "efc_force"), rows(d.efc.state, njmax, i32, "efc_state")
+    a.Jaref, a.jv = rows(ctx.Jaref, njmax, f32, "Jaref"), rows(ctx.jv, njmax, f32, "jv")
+    a.search, a.mv = rows(ctx.search.reshape(nworld, -1), nv, f32, "search"), rows(ctx.mv, nv, f32, "mv")
+    a.qfrc_constraint = rows(d.qfrc_constraint, nv, f32, "qfrc_constraint")
+    grad = ctx.grad.reshape(nworld, -1)
+    if grad.dtype != f32 or grad.device != dev or grad.shape[1] < nv or not grad.is_contiguous():
+        raise TypeError("grad must be a contiguous float32 (nworld, >= nv) tensor")
+    a.grad, a.ld_grad = grad.data_ptr(), grad.shape[1]
+    for name, t in (("search_dot", ctx.search_dot), ("alpha", ctx.alpha), ("improvement", ctx.improvement), ("grad_dot", ctx.grad_dot),
+                    ("grad_scale", ctx.grad_scale), ("newton_decrement", ctx.newton_decrement)):  # fmt: skip
+        setattr(a, name, per_world(t, (f32,), name))
+    ids = ctx.quad_changed_ids
+    if ids.dtype != i32 or ids.device != dev or ids.dim() != 2 or ids.shape[0] != nworld or not ids.is_contiguous():
+        raise TypeError("quad_changed_ids must be a contiguous int32 (nworld, width) tensor")
+    a.quad_changed_ids, a.ld_ids = ids.data_ptr(), ids.shape[1]
+    a.quad_changed_count = per_world(ctx.quad_changed_count, (i32,), "quad_changed_count")
+    a.state_changed_count = per_world(ctx.state_changed_count, (i32,), "state_changed_count")
+    a.solver_niter = per_world(d.solver_niter, (i32,), "solver_niter")
+    a.overflow = per_world(getattr(d, "overflow", None), (i32,), "overflow", optional=True)
+    if nsolving is not None and (nsolving.dtype != i32 or nsolving.device != dev or nsolving.numel() != 1):
+        raise TypeError("nsolving must be a one-element int32 tensor")
+    a.nsolving = None if nsolving is None else nsolving.data_ptr()
+    a.done = per_world(ctx.done, byte, "done")
+    a.ls_exhausted = per_world(ctx.ls_exhausted, byte, "ls_exhausted")
+    a.search_unchanged = per_world(ctx.search_unchanged, byte, "search_unchanged")
+    a.nworld = nworld
+    return a
+
+
+def run_resident(m, d, ctx, nsolving) -> bool:
+    """The whole loop as one resident kernel (a wavefront per world until it is done), for a ``ctx``
+    with the tree stage whose plan carries generated kernels; False when there is no such kernel
+    for this model (the caller then launches the stages one by one)."""
+    import ctypes as C
+
+    import torch
+
+    scratch = _tree_scratch(ctx)
+    if scratch is None or os.environ.get("IMHIP_NEWTON") == "stages":
+        return False
+    a = _resident_args(m, d, ctx, nsolving)
+    dev = d.efc.J.device
+    with torch.cuda.device(dev):
+        status = _lib.lib().im_newton_solve_tree(scratch.kernel.ptr, C.byref(a), int(torch.cuda.current_stream(dev).cuda_stream))
+    if status == _lib.IM_ERR_UNSUPPORTED:
+        return False
+    _lib.check(status, "im_newton_solve_tree")
+    return True
+
+
 def run(m, d, ctx, nsolving, *, check_every: int | None = None, graph: bool = False) -> int:
     """The fused Newton solve with the reference's signature (newton_fusion.py:330-409): iterates
     until every world is done or ``m.opt.iterations`` is reached.  The reference keeps a world in
     one resident block for the whole loop; here an iteration is eight launches over all worlds and
     finished worlds drop out of each through ``ctx.done``, so launching all ``m.opt.iterations``
     of them is correct whatever the worlds need, touches the host nowhere and can be captured in a
-    caller's graph: that is what happens under stream capture and with ``check_every=0``.
+    caller's graph: that is what happens under stream capture and with ``check_every=0``.  With
+    the tree stage on ``ctx`` and neither ``check_every`` nor ``graph`` given, the loop is one
+    resident kernel (:func:`run_resident`: the same results, no launch per stage).
     Outside a capture the host by default reads ``ctx.done`` every fourth iteration and stops early
     (``check_every``).  ``graph``: the first iteration runs as plain launches, the second is
     captured in a graph that the later ones replay (the arrays of ``d`` and ``ctx`` must then stay
     where they are for the whole solve).  Returns the number of iterations launched."""
     import torch
 
+    if check_every is None and not graph and run_resident(m, d, ctx, nsolving):
+        return int(m.opt.iterations)
     capturing = torch.cuda.is_current_stream_capturing()
     if check_every is None:
         check_every = 0 if capturing else 4

@@ -131,15 +131,25 @@ def _solve_on_gpu(p, device, *, graph: bool):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,nworld,stage,graph", [
-    ("humanoid", 300, "dense", False), ("humanoid", 300, "tree", False), ("g1", 200, "sparse", False),
-    ("humanoid", 4096, "tree", True), ("humanoid", 4096, "dense", True), ("g1", 8192, "sparse", True),
-    ("snu", 4096, "sparse", True), ("ant", 64, "tree", True), ("snu", 130, "tree", False),
+@pytest.mark.parametrize("name,nworld,stage,graph,loop", [
+    ("humanoid", 300, "dense", False, "stages"), ("humanoid", 300, "tree", False, "stages"), ("g1", 200, "sparse", False, "stages"),
+    ("humanoid", 4096, "tree", True, "stages"), ("humanoid", 4096, "dense", True, "stages"), ("g1", 8192, "sparse", True, "stages"),
+    ("snu", 4096, "sparse", True, "stages"), ("ant", 64, "tree", True, "stages"), ("snu", 130, "tree", False, "stages"),
+    ("humanoid", 301, "tree", False, "resident"), ("humanoid", 4096, "tree", True, "resident"), ("ant", 67, "tree", True, "resident"),
 ])  # fmt: skip
-def test_gpu_solve_from_init_context_matches_the_oracle_chain(device, name, nworld, stage, graph):
-    small = nworld <= 300
+def test_gpu_solve_from_init_context_matches_the_oracle_chain(device, monkeypatch, name, nworld, stage, graph, loop):
+    """``loop``: the iterations as eight launches each (``stages``) or as one resident kernel with a
+    wavefront per world (``resident``, the tree stage with generated kernels): the same arrays at the
+    end either way."""
+    small = nworld <= 301
     p = NC.problem(name, nworld, stage, empty_every=11 if small else 97, warmstart=small, maxiter=12)
     s = NC.oracle_solve(p)
+    taken = []
+    inner = NF.run_resident
+    monkeypatch.setattr(NF, "run_resident", lambda *a: taken.append(inner(*a)) or taken[-1])
+    if loop == "stages":
+        monkeypatch.setenv("IMHIP_NEWTON", "stages")
     m, d, ctx, nsolving = _solve_on_gpu(p, device, graph=graph)
+    assert all(taken) == (loop == "resident") and len(taken) > 0
     NC.compare(p, s, d, ctx)
     assert int(nsolving.item()) == int((p.nefc == 0).sum())  # every world that had rows has reported done

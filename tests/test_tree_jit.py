@@ -39,7 +39,7 @@ def test_code_objects_and_keys():
     st, groups, trunk, _ = build._plan_of_tree(TREES["limbs"])
     a, b = tree_row16.generate("t", *st, groups, trunk), tree_row16.generate("t", *st, groups, trunk, module=True)
     la, lb = a.splitlines(), b.splitlines()
-    assert sum(x != y for x, y in zip(la, lb)) <= 12 and abs(len(la) - len(lb)) < 20 and len(la) > 500
+    assert sum(x != y for x, y in zip(la, lb)) <= 24 and abs(len(la) - len(lb)) < 20 and len(la) > 500
 
 
 def _random_forest(rng, nv, nroots):
@@ -93,7 +93,7 @@ def test_cache_is_keyed_by_everything_that_changes_the_source(monkeypatch):
 def test_kernel_descriptors_of_a_code_object():
     st, groups, trunk, _ = build._plan_of_tree(TREES["limbs"])
     res = jit.kernel_resources(jit.code_object(st, groups, trunk))
-    assert set(res) == {"im_row16_fused", "im_row16_fused_long", "im_row16_solve"}
+    assert set(res) == {"im_row16_fused", "im_row16_fused_long", "im_row16_solve", "im_row16_newton", "im_row16_newton_long"}
     assert all(private == 0 for _, private in res.values())  # the best plan's kernels keep to registers
     # one group for the whole tree holds every row in one wavefront's registers and spills
     st, groups, trunk, _ = build._plan_of_tree(TREES["limbs62"], 1)
