@@ -135,7 +135,7 @@ def _compile(src: str) -> str:
     if os.path.exists(obj) and not os.environ.get("IMHIP_REBUILD"):
         if os.path.getmtime(obj) > max(os.path.getmtime(d) for d in deps):
             return obj
-    cmd = ["hipcc", *FLAGS, "-c", "-x", "hip", src, "-o", obj]
+    cmd = ["hipcc", *FLAGS, *os.environ.get("IMHIP_EXTRA_FLAGS", "").split(), "-c", "-x", "hip", src, "-o", obj]  # extra flags: development aid
     if os.path.dirname(src) != GEN:
         subprocess.run(cmd, check=True)
         return obj

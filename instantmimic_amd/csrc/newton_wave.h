@@ -276,6 +276,12 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Sta
   block_sync();
   // every wavefront leaves the loop after at most maxiter rounds, whatever the data
   const int lane_fixed = lane;
+#ifdef IM_NEWTON_STAMPS  // development aid: time per phase, summed over the rounds, left in the world's row of jv
+  long long t_phase[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t_last = wall_clock64();
+#define IM_STAMP(k) do { const long long t_now = wall_clock64(); t_phase[k] += t_now - t_last; t_last = t_now; } while (0)
+#else
+#define IM_STAMP(k) do {} while (0)
+#endif
   for (int round = 0; round < a.maxiter; ++round) {
     if (lane_fixed == 0) votes[wv] = done ? 0 : 1;
     block_sync();
@@ -284,6 +290,7 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Sta
     // stage derives from it is kept in registers across the other stages
     int lane = lane_fixed;
     asm volatile("" : "+v"(lane));
+    IM_STAMP(0);
     if (!done) {
       if (!unchanged) {
         for (int k = lane; k < nv; k += 64) sv[k] = a.search[w * nv + k];
@@ -292,8 +299,10 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Sta
         jv_world<JU>(a, Jw, nefc, rows_lds, sv, a.jv + w * njmax, lane);
         wave_sync();
       }
+      IM_STAMP(1);
       search::linesearch_world<HELD>(sa, w, lane & 31);
       wave_sync();
+      IM_STAMP(2);
       {  // the step (newton_stages.py:373-381)
         const float al = a.alpha[w];
         for (int i = lane; i < nv; i += 64) {
@@ -307,11 +316,15 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Sta
                                      a.exhausted, a.force, njmax, a.state, njmax, a.ids, a.ld_ids, a.quad_count,
                                      a.state_count, w, lane);
       wave_sync();
+      IM_STAMP(3);
       unchanged = gradient_world(a, w, Jw, nefc, f, rowl, gl, part, lane);
+      IM_STAMP(4);
     }
     block_sync();  // gradients, states and the `unchanged` bytes of the four worlds are in place; the rows of J are done with
+    IM_STAMP(5);
     stage();
     block_sync();  // the four search directions are complete
+    IM_STAMP(6);
     lane = lane_fixed;
     asm volatile("" : "+v"(lane));  // no address from before the stage is kept through it
     if (!done) {
@@ -335,7 +348,12 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Sta
       }
       done = __builtin_amdgcn_readfirstlane(finished) != 0;
     }
+    IM_STAMP(7);
   }
+#ifdef IM_NEWTON_STAMPS
+  if (live && lane_fixed < 8) a.jv[w * njmax + lane_fixed] = (float)t_phase[lane_fixed];
+#endif
+#undef IM_STAMP
 }
 
 }  // namespace resident

@@ -74,7 +74,7 @@ def _line(kernel, workload, seconds, *, bytes_=None, flops=None, nworld=None):
 
 
 def run(launches: int = 32, only: str | None = None) -> None:
-    """``only``: comma-separated section names out of trees, generated, stress, muscles, walks, iteration, implicit, bodies."""
+    """``only``: comma-separated section names out of trees, generated, stress, muscles, walks, iteration, solve, implicit, bodies."""
     import torch
 
     from . import synth
@@ -471,6 +471,94 @@ def run(launches: int = 32, only: str | None = None) -> None:
               f"humanoid nv={nv} nefc={nefc} x {nworld} worlds", sec,
               bytes_=nworld * 4 * (3 * nefc * nv + 2 * nM + 14 * nefc + 20 * nv + 16), nworld=nworld)  # fmt: skip
 
+    # ---- whole constraint solves with dependent iterations: init_context, the Newton loop, the force recovery
+    if section("solve"):
+        import os
+
+        def newton_case(name, stage, seed=21, maxiter=10):
+            """(m, d, ctx, nsolving) of one step on the tree of `name`: 2 equality rows, 3 friction-loss rows, the
+            rest one-sided; everything the solve writes starts as it happens to lie there."""
+            shape = synth.SHAPES[name]
+            b = synth.make_batch(shape, ragged_nefc=True)
+            rng = np.random.default_rng(seed)
+            nworld, nv, njmax = b.nworld, shape.nv, shape.nefc
+            m = synth.model_from_parents(shape.parents)
+            pad = int(m.nv_pad)
+            nefc = np.maximum(b.nefc, 8).astype(np.int32)
+            tables = [t(a) for a in NF.mul_m_tables(b.rowadr, b.rownnz, b.colind)]
+            m.M_mulm_rowadr, m.M_mulm_col, m.M_mulm_madr = tables
+            m.opt = SimpleNamespace(solver=2, cone=0, integrator=3, iterations=maxiter, ls_iterations=50, disableflags=256,
+                                    tolerance=torch.full((1,), 1e-7, device=dev), ls_tolerance=torch.full((1,), 0.01, device=dev))  # fmt: skip
+            m.stat = SimpleNamespace(meaninertia=torch.ones(1, device=dev))
+            f = lambda *shape_: torch.zeros(shape_, device=dev)  # noqa: E731
+            i = lambda *shape_: torch.zeros(shape_, dtype=torch.int32, device=dev)  # noqa: E731
+            u8 = lambda: torch.zeros(nworld, dtype=torch.uint8, device=dev)  # noqa: E731
+            qs = t(rng.normal(size=(nworld, nv)).astype(np.float32))
+            M_ = t(b.M)
+            smooth = f(nworld, nv)
+            NF.mul_m(M_, qs, smooth, *tables)
+            d = SimpleNamespace(nworld=nworld, njmax=njmax, M=M_, ne=t(np.full(nworld, 2, np.int32)), nf=t(np.full(nworld, 3, np.int32)),
+                                nefc=t(nefc), qfrc_smooth=smooth, qacc_smooth=qs, qacc_warmstart=None, qacc=f(nworld, nv),
+                                qfrc_constraint=f(nworld, nv), solver_niter=i(nworld), overflow=i(nworld),
+                                efc=SimpleNamespace(J=t(b.J), D=t((10.0 ** rng.uniform(0, 3, (nworld, njmax))).astype(np.float32)),
+                                                    frictionloss=t(rng.uniform(0.1, 1.0, (nworld, njmax)).astype(np.float32)),
+                                                    aref=t(rng.normal(scale=2.0, size=(nworld, njmax)).astype(np.float32)),
+                                                    Ma=f(nworld, nv), force=f(nworld, njmax), state=i(nworld, njmax)))  # fmt: skip
+            ctx = SimpleNamespace(search=f(nworld, nv), search_dot=f(nworld), mv=f(nworld, nv), jv=f(nworld, njmax), Jaref=f(nworld, njmax),
+                                  done=u8(), alpha=f(nworld), improvement=f(nworld), ls_exhausted=u8(), quad_changed_ids=i(nworld, njmax),
+                                  quad_changed_count=i(nworld), state_changed_count=i(nworld), search_unchanged=u8(), grad=f(nworld, pad),
+                                  grad_dot=f(nworld), grad_scale=f(nworld), newton_decrement=f(nworld), h=f(nworld, pad, pad),
+                                  hfactor=f(nworld, pad, pad))  # fmt: skip
+            if stage == "tree":
+                ctx.newton_tree_scratch = T.create_tree_factor_solve_scratch(m, dev)
+            elif stage == "sparse":
+                ctx.sparse_hessian_plan, why = SH.plan_for_model(m, ctx, [], SH.block_width(pad), device=dev)
+                assert ctx.sparse_hessian_plan is not None, why
+            NF.attach_scratch(m, d, ctx, dev)
+            return m, d, ctx, torch.zeros(1, dtype=torch.int32, device=dev)
+
+        for name, stage, loop in (("humanoid", "tree", "resident"), ("humanoid", "tree", "stages"), ("humanoid", "dense", "stages"),
+                                  ("g1", "tree", "stages"), ("g1", "sparse", "stages"), ("snu", "sparse", "stages")):  # fmt: skip
+            if loop == "stages":
+                os.environ["IMHIP_NEWTON"] = "stages"
+            else:
+                os.environ.pop("IMHIP_NEWTON", None)
+            nsets = 8
+            cases = [newton_case(name, stage, seed=21 + k) for k in range(nsets)]
+            m0, d0, _, _ = cases[0]
+            nworld, nv, njmax, nM = d0.nworld, m0.nv, d0.njmax, int(d0.M.shape[1])
+            NF.solve(*cases[0])
+            torch.cuda.synchronize()
+            its = cases[0][1].solver_niter.cpu().numpy()
+            unfinished = int((cases[0][2].done.cpu().numpy() == 0).sum())
+
+            def start(k):  # what precedes the loop: the start point, init_context, the counters
+                m_, d_, c_, n_ = cases[k]
+                d_.qacc.copy_(d_.qacc_smooth)
+                d_.qfrc_constraint.zero_()
+                NF.init_context(m_, d_, c_)
+                c_.search_unchanged.zero_()
+                n_.fill_(nworld)
+
+            sec_all = _timeit(torch, lambda k: NF.solve(*cases[k]), nsets, max(launches // 4, 4), prime=False)
+            sec_init = _timeit(torch, start, nsets, max(launches // 4, 4), prime=False)
+            rounds = int(its.max())  # dependent iterations the slowest world takes: the length of the loop
+            issued = rounds if loop == "resident" else int(m0.opt.iterations)
+            loop_s = sec_all - sec_init
+            out = {"kernel": f"newton_fusion.solve, {stage} stage, iterations as {'one resident kernel' if loop == 'resident' else 'eight launches each'}",
+                   "workload": f"{name} nv={nv} nefc={njmax} x {nworld} worlds, tolerance 1e-7, at most {m0.opt.iterations} iterations",
+                   "us_per_solve": round(sec_all * 1e6, 1), "us_init_context": round(sec_init * 1e6, 1), "us_loop": round(loop_s * 1e6, 1),
+                   "iterations_mean": round(float(its.mean()), 2), "iterations_max": rounds, "iterations_issued": issued,
+                   "us_per_issued_iteration": round(loop_s * 1e6 / max(issued, 1), 2), "worlds_unfinished": unfinished,
+                   "world_iterations_per_s": round(float(its.sum()) / loop_s)}  # fmt: skip
+            # one pass over M, J, D and the per-row and per-dof vectors per iteration a world takes
+            per_it = 4 * (njmax * nv + nM + 6 * njmax + 10 * nv)
+            out.update(bound="hbm", algorithmic_bytes=int(per_it * its.sum()), achieved_GBs=round(per_it * float(its.sum()) / loop_s / 1e9, 1),
+                       frac=round(per_it * float(its.sum()) / loop_s / 1e9 / HBM_GBS, 4))  # fmt: skip
+            print(json.dumps(out), flush=True)
+            del cases
+        os.environ.pop("IMHIP_NEWTON", None)
+
     # ---- implicit-fast integrator matrix and its solve; the upstream-iteration sparse factor from the dense Hessian
     if section("implicit"):
         from .mjw_kernels import implicit_qh as IQ
@@ -555,7 +643,7 @@ def run(launches: int = 32, only: str | None = None) -> None:
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--launches", type=int, default=32)
-    ap.add_argument("--only", default=None, help="comma-separated sections: trees, generated, stress, muscles, walks, iteration, implicit, bodies")
+    ap.add_argument("--only", default=None, help="comma-separated sections: trees, generated, stress, muscles, walks, iteration, solve, implicit, bodies")
     ap.add_argument("--no-graph", action="store_true", help="plain launches instead of a hipGraph replay")
     args = ap.parse_args()
     GRAPH = not args.no_graph
