@@ -4,12 +4,14 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one pass of the hot path over one synthetic batch of the headline shape: humanoid,
-nv = 27, nefc = 64, 4096 worlds, three Newton iterations with a fresh active mask each -- one
-call of im_assemble_tree_ldl_solve_iters (one launch whose grid covers worlds x iterations).
-Inputs are resident in HBM before the timed region; every step takes the next of 16 distinct
-input sets (> 560 MB in rotation), so no launch finds its M or J in the 256 MB memory-side cache.
-Beside the headline the same batch is timed as three launches of im_assemble_tree_ldl_solve per
-step, each launch on an input set of its own (`single_launch`).  Prints one JSON line.
+nv = 27, nefc = 64, 4096 worlds, three Newton iterations with a fresh active mask each -- three
+calls of im_assemble_tree_ldl_solve, one launch per solve, which is the form a Newton loop can
+issue (an iteration's states come out of the one before).  Inputs are resident in HBM before the
+timed region; every launch takes the next of 16 distinct input sets (> 560 MB in rotation), so no
+launch finds its M or J in the 256 MB memory-side cache.  `value` and `roofline` are this form's.
+Beside it, `iterations_launch`: the three solves of a step as one launch of
+im_assemble_tree_ldl_solve_iters (a grid over worlds x iterations, for callers that know every
+iteration's states in advance; the solves are then independent of one another).  Prints one JSON line.
 """
 
 from __future__ import annotations
@@ -29,8 +31,10 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the iterations kernel (3 solves x 4096 worlds) from two rocprofv3 --pmc
 # runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads
 # for a plain 64 MiB device copy in the same run; recorded in
-# profiles/tree_row16_humanoid_pmc.txt:  (18292.13 * 65536 / 32783.90 + 1344.0) KiB
-TRAFFIC_BYTES_PER_LAUNCH = int((18292.13 * 65536 / 32783.90 + 1344.0) * 1024)
+# profiles/tree_row16_humanoid_pmc.txt:  (18296.13 * 65536 / 32781.77 + 1344.0) KiB
+TRAFFIC_BYTES_PER_LAUNCH = int((18296.13 * 65536 / 32781.77 + 1344.0) * 1024)
+# the same for one launch of the single-solve kernel (4096 worlds):  (15566.19 * 65536 / 32781.77 + 448.0) KiB
+TRAFFIC_BYTES_PER_SINGLE_LAUNCH = int((15566.19 * 65536 / 32781.77 + 448.0) * 1024)
 MIN_TIMED_LAUNCHES = 256  # the kernel duration is averaged over at least this many launches
 
 
@@ -47,8 +51,8 @@ def algorithmic_bytes_fused(nv: int, nM: int, nefc: int, iters: int) -> int:
 def cpu_baseline(batch, plan_struct, gpu_x, seconds: float = 10.0):
     """The CPU oracle (a C restatement of the reference path, OpenMP over worlds) timed on this
     host's cores on the same workload: all threads, then one thread.  As the checker it also
-    compares what the GPU computed for the first worlds of the benchmarked batch (`gpu_x`,
-    (iterations, worlds, nv)) with its own result, bit for bit."""
+    compares what the GPU computed for the first input set of the benchmarked batch (`gpu_x`,
+    (iterations, worlds, nv), every world) with its own result, bit for bit."""
     import numpy as np
 
     from oracle import planner as P
@@ -59,7 +63,7 @@ def cpu_baseline(batch, plan_struct, gpu_x, seconds: float = 10.0):
     threads = R.max_threads()
     iters = batch.state.shape[0]
     n = gpu_x.shape[1]
-    for it in range(iters):
+    for it in range(iters):  # every world of the first input set
         want = R.assemble_tree_ldl_solve(*st, plan, batch.M[:n], batch.J[:n], batch.D[:n], batch.state[it][:n], batch.nefc[:n], batch.grad[:n])
         if not np.array_equal(gpu_x[it], want):
             raise RuntimeError(f"the benchmarked kernel disagrees with the CPU restatement in iteration {it}")
@@ -105,7 +109,7 @@ def main() -> int:
     ap.add_argument("--sets", type=int, default=16, help="distinct input sets rotated over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying hipGraphs")
-    ap.add_argument("--single-only", action="store_true", help="time the three-launch form only (for profiles of the single launch)")
+    ap.add_argument("--single-only", action="store_true", help="time the one-launch-per-solve form only (for profiles of that kernel)")
     ap.add_argument(
         "--copy-calibration",
         type=int,
@@ -172,9 +176,18 @@ def main() -> int:
             M, J, D, st, ne, g, x = sets[(s * iters + it) % nsets]
             T.assemble_tree_factor_solve(scratch, M, J, D, st[it], ne, g, x[it])
 
+    # both forms once on set 0 (the batch as generated), checked against the CPU restatement in the CPU leg:
+    # every world of every iteration
     step(0)
     torch.cuda.synchronize()
-    x_first = sets[0][6][:, :64].cpu().numpy()  # set 0 is the batch as generated: checked in the CPU leg
+    x_first = sets[0][6].cpu().numpy().copy()
+    sets[0][6].zero_()
+    for it in range(iters):
+        M, J, D, st, ne, g, x = sets[0]
+        T.assemble_tree_factor_solve(scratch, M, J, D, st[it], ne, g, x[it])
+    torch.cuda.synchronize()
+    if not np.array_equal(sets[0][6].cpu().numpy(), x_first):
+        raise RuntimeError("one launch per solve and the iterations launch disagree")
 
     use_graph = not args.no_graph
 
@@ -233,37 +246,56 @@ def main() -> int:
         torch.cuda.synchronize()
         return time.perf_counter() - t0, ev0.elapsed_time(ev1) * 1e-3
 
+    def spread(run, launches_per_step: int, regions: int = 32, steps_per_region: int = 8):
+        """Median, 10th and 90th percentile of the per-launch duration over `regions` timed regions of
+        `steps_per_region` steps each (HIP events around every region)."""
+        run.prepare(steps_per_region)
+        per = []
+        for _ in range(regions):
+            _, ev = region(run, steps_per_region)
+            per.append(ev / (steps_per_region * launches_per_step) * 1e6)
+        per.sort()
+        return {"median": per[len(per) // 2], "p10": per[len(per) // 10], "p90": per[(9 * len(per)) // 10], "regions": regions,
+                "launches_per_region": steps_per_region * launches_per_step}
+
     B = algorithmic_bytes(nv, nM, nefc)
     B3 = algorithmic_bytes_fused(nv, nM, nefc, iters)
-    run_single = runner(step_single)
-    n_single = max(args.steps, -(-MIN_TIMED_LAUNCHES // iters))
-    run_single.prepare(n_single)
-    run_single(max(args.warmup, nsets))
-    _, ev_single = region(run_single, n_single)
-    single_us = ev_single / (n_single * iters) * 1e6
-    single = {
-        "kernel_us": single_us,
-        "launches_timed": n_single * iters,
-        "achieved": B * nworld / (single_us * 1e-6) / 1e9,
-        "frac": B * nworld / (single_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
-        "note": "one launch per solve (im_assemble_tree_ldl_solve), every launch on an input set of its own",
-    }
 
+    # ---- the headline: one launch per solve, three launches per step
+    run_single = runner(step_single)
+    n_kernel = max(args.steps, -(-MIN_TIMED_LAUNCHES // iters))
+    for n in (args.warmup, args.steps, n_kernel):
+        run_single.prepare(n)
+    run_single(max(args.warmup, 1))
+    elapsed, _ = region(run_single, args.steps)
+    value = args.steps * iters * nworld / elapsed
+    _, ev_kernel = region(run_single, n_kernel)  # the kernel's duration from a region whose length does not depend on --steps
+    kernel_s = ev_kernel / (n_kernel * iters)  # one launch = one solve of every world
+    achieved = B * nworld / kernel_s / 1e9
     if args.single_only:
-        print(json.dumps({"single_launch": single}))
+        print(json.dumps({"single_launch": {"kernel_us": kernel_s * 1e6, "frac": achieved / HBM_PEAK_GBS}}))
         return 0
 
-    run = runner(step)
-    n_kernel = max(args.steps, MIN_TIMED_LAUNCHES)
-    for n in (args.warmup, args.steps, n_kernel):
-        run.prepare(n)
-    run(args.warmup)
-    elapsed, _ = region(run, args.steps)
-    value = args.steps * iters * nworld / elapsed
-    # the kernel's duration from a region of its own whose length does not depend on --steps
-    _, ev_kernel = region(run, n_kernel)
-    kernel_s = ev_kernel / n_kernel  # one launch = one step = `iters` solves of every world
-    achieved = B * iters * nworld / kernel_s / 1e9
+    # ---- beside it: the step's three solves as one launch over (worlds x iterations)
+    run_iters = runner(step)
+    n_iters = max(args.steps, MIN_TIMED_LAUNCHES)
+    run_iters.prepare(n_iters)
+    run_iters(max(args.warmup, 1))
+    _, ev_iters = region(run_iters, n_iters)
+    iters_s = ev_iters / n_iters
+    iterations_launch = {
+        "entry": "im_assemble_tree_ldl_solve_iters: three independent solves per launch (every iteration's states known before the launch)",
+        "kernel_us": iters_s * 1e6,
+        "us_per_solve": iters_s * 1e6 / iters,
+        "launches_timed": n_iters,
+        "kernel_us_spread": spread(run_iters, 1),
+        "world_solves_per_s": iters * nworld / iters_s,
+        "frac_per_solve_bytes": B * iters * nworld / iters_s / 1e9 / HBM_PEAK_GBS,
+        "frac_per_solve_bytes_definition": f"{B} bytes x {iters} solves x {nworld} worlds per launch: every solve counted as if it read M and J itself, which the launch does not do",
+        "frac_fused_bytes": B3 * nworld / iters_s / 1e9 / HBM_PEAK_GBS,
+        "frac_fused_bytes_definition": f"B3 = {B3} bytes per world and launch: M and J once, state / D / gradient / x per iteration",
+        "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+    }
 
     out = {
         "metric": METRIC,
@@ -279,11 +311,10 @@ def main() -> int:
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": f"humanoid nv={nv} nM={nM} nefc={nefc} x {nworld} worlds, {iters} Newton iterations per step with a fresh active mask each, one launch per step (im_assemble_tree_ldl_solve_iters)",
+            "workload": f"humanoid nv={nv} nM={nM} nefc={nefc} x {nworld} worlds, {iters} Newton iterations per step with a fresh active mask each, one launch per solve (im_assemble_tree_ldl_solve), every launch on an input set of its own",
             "input_sets": nsets,
             "launch": "hipGraph replay" if use_graph else "eager",
             "bytes_per_world_solve": B,
-            "bytes_per_world_step_fused": B3,
         },
         "roofline": {
             "bound": "hbm",
@@ -291,17 +322,15 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic": TRAFFIC_BYTES_PER_SINGLE_LAUNCH,
             "kernel_us": kernel_s * 1e6,
-            "launches_timed": n_kernel,
-            "solves_per_launch": iters,
-            "us_per_solve": kernel_s * 1e6 / iters,
-            "bytes_definition": f"per-solve B = {B} bytes x {iters} solves x {nworld} worlds per launch (every solve counted as if it read M and J itself)",
-            "frac_fused_bytes": B3 * nworld / kernel_s / 1e9 / HBM_PEAK_GBS,
-            "frac_fused_bytes_definition": f"B3 = {B3} bytes per world and launch: M and J once, state / D / gradient / x per iteration",
+            "kernel_us_spread": spread(run_single, iters),
+            "launches_timed": n_kernel * iters,
+            "solves_per_launch": 1,
+            "bytes_definition": f"B = {B} bytes per world*solve (M, J, D, state, gradient in; x out) x {nworld} worlds per launch",
             "throughput_frac": (B * value / 1e9) / HBM_PEAK_GBS,
-            "single_launch": single,
         },
+        "iterations_launch": iterations_launch,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(batch, T.tree_ldl_structure(batch.rowadr, batch.rownnz, batch.colind), x_first)
