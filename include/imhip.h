@@ -917,6 +917,19 @@ typedef struct im_newton_args {
  * stages one by one). */
 int im_newton_solve_tree(const im_tree_plan *plan, const im_newton_args *args, void *stream);
 
+/* The same resident loop with the static-pattern sparse stage of im_sparse_update_factor as its
+ * factor stage, which is the reference's kernel for a model with a fused sparse plan
+ * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:150-169 with sparse_hessian.native_func):
+ * hfactor (nworld, nv_pad, nv_pad) carries packed H, the factor and 1 / D as im_sparse_init_factor
+ * left them and is kept up to date, dof_union (nworld, nv + 1) receives the dofs the changed rows
+ * touch.  A wavefront per world, up to sixteen worlds per workgroup sharing one copy of the plan's
+ * tables in LDS; a wavefront leaves as soon as its world is done.  args->block must be the plan's
+ * block width.  The arrays end as after im_sparse_update_factor and the other stage launches
+ * repeated, bit for bit.  nv <= 64 (IM_ERR_UNSUPPORTED beyond, and where no variant of the kernel
+ * fits the LDS: the caller then issues the stages one by one). */
+int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *args, float *hfactor,
+                           int32_t *dof_union, void *stream);
+
 /* Replaces _init_efc_settling_empty_worlds
  * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:412-428): solver_niter = 0,
  * search_dot = 0, done = (nefc == 0), and a world without constraint rows gets

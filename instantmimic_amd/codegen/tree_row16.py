@@ -897,10 +897,13 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit(f"    tree_row16_body_{name}<true, LONG>(a.M, a.ldM, a.J, a.njmax, a.D, a.state, a.nefc, a.quad, a.grad, a.ld_grad, a.search,")
     emit("        (int64_t)a.nv, nullptr, a.nworld, IM_FLAG_NEGATE, 1, 0, 0, 0, a.unchanged);")
     emit("  };")
+    emit("  const im::resident::LoopLds L = im::resident::coop_layout(a, xlds);")
+    emit("  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);")
+    emit("  im::resident::block_sync();")
     emit("  if (LONG && a.njmax > 128)")
-    emit(f"    im::resident::newton_loop<0, {ju}>(a, xlds, stage);")
+    emit(f"    im::resident::newton_loop<0, {ju}, true>(a, L, w, stage);")
     emit("  else")
-    emit(f"    im::resident::newton_loop<(LONG ? 4 : 2), {ju}>(a, xlds, stage);")
+    emit(f"    im::resident::newton_loop<(LONG ? 4 : 2), {ju}, true>(a, L, w, stage);")
     emit("}")
     if module:
         emit("} }  // namespace im::gen")

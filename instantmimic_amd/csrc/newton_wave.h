@@ -16,6 +16,7 @@
 
 #include <cstdint>
 
+#include "../../include/imhip.h"
 #include "newton_search.h"
 
 namespace im {
@@ -43,6 +44,41 @@ struct NewtonArgs {
   uint8_t *done, *exhausted, *unchanged;
   int stage_lds_floats;  // dynamic LDS the factor stage uses from offset 0; the loop's own arrays follow
 };
+
+// The public argument block checked and turned into the kernels' (host side).
+inline int convert_args(const im_newton_args &p, int nv, int nM, NewtonArgs &a) {
+  const int njmax = p.njmax;
+  if (njmax <= 0 || p.iterations < 0 || p.ls_iterations < 0 || (p.block != 32 && p.block != 64) || p.ntolerance <= 0 ||
+      p.nls_tolerance <= 0 || p.nmeaninertia <= 0 || p.nterm <= 0)
+    return IM_ERR_ARG;
+  if (!p.opt_tolerance || !p.opt_ls_tolerance || !p.stat_meaninertia || !p.M_mulm_rowadr || !p.M_mulm_col ||
+      !p.M_mulm_madr || !p.M || !p.efc_J || !p.efc_D || !p.qfrc_smooth || !p.qacc || !p.efc_Ma || !p.efc_force ||
+      !p.efc_state || !p.Jaref || !p.search || !p.search_dot || !p.mv || !p.jv || !p.alpha || !p.improvement || !p.grad ||
+      !p.grad_dot || !p.grad_scale || !p.newton_decrement || !p.qfrc_constraint || !p.quad_changed_ids ||
+      !p.quad_changed_count || !p.state_changed_count || !p.solver_niter || !p.done || !p.ls_exhausted ||
+      !p.search_unchanged || (p.nf && !p.efc_frictionloss))
+    return IM_ERR_ARG;
+  if (p.ldM < nM || p.ld_grad < nv || p.ld_ids < 0) return IM_ERR_STRIDE;
+  if (p.nterm >= 65536 || nM >= 65536 || 64 * (int64_t)nv >= (1 << 20)) return IM_ERR_UNSUPPORTED;
+  a.tolerance = p.opt_tolerance, a.ls_tolerance = p.opt_ls_tolerance, a.meaninertia = p.stat_meaninertia;
+  a.ntolerance = p.ntolerance, a.nls_tolerance = p.nls_tolerance, a.nmeaninertia = p.nmeaninertia;
+  a.nv = nv, a.njmax = njmax, a.nworld = p.nworld, a.ls_iterations = p.ls_iterations, a.maxiter = p.iterations;
+  a.block = p.block, a.quad = p.quad, a.ls_overflow_bit = p.ls_overflow_bit;
+  a.iter_overflow_bit = p.iterations_overflow_bit;
+  a.mulm_rowadr = p.M_mulm_rowadr, a.mulm_col = p.M_mulm_col, a.mulm_madr = p.M_mulm_madr;
+  a.nterm = p.nterm, a.nM = nM;
+  a.ne = p.ne, a.nf = p.nf, a.nefc = p.nefc, a.M = p.M, a.ldM = p.ldM, a.J = p.efc_J, a.D = p.efc_D;
+  a.frictionloss = p.efc_frictionloss, a.smooth = p.qfrc_smooth;
+  a.qacc = p.qacc, a.Ma = p.efc_Ma, a.force = p.efc_force, a.Jaref = p.Jaref, a.search = p.search;
+  a.search_dot = p.search_dot, a.mv = p.mv, a.jv = p.jv, a.alpha = p.alpha, a.improvement = p.improvement;
+  a.grad = p.grad, a.grad_dot = p.grad_dot, a.grad_scale = p.grad_scale, a.decrement = p.newton_decrement;
+  a.qfrc_constraint = p.qfrc_constraint, a.ld_grad = p.ld_grad;
+  a.state = p.efc_state, a.ids = p.quad_changed_ids, a.quad_count = p.quad_changed_count;
+  a.state_count = p.state_changed_count, a.niter = p.solver_niter, a.overflow = p.overflow, a.nsolving = p.nsolving;
+  a.ld_ids = p.ld_ids, a.done = p.done, a.exhausted = p.ls_exhausted, a.unchanged = p.search_unchanged;
+  a.stage_lds_floats = 0;
+  return IM_OK;
+}
 
 __device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 
@@ -147,7 +183,7 @@ __device__ __forceinline__ void jv_world(const NewtonArgs &a, const float *Jw, i
 // ---- the gradient (newton_stages.py:745-798), a lane per dof ------------------------------------
 // Returns whether the search direction stays as it is (no state changed).
 __device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, const float *Jw, int nefc, float *f,
-                                               int *rowl, float *gl, float *part, int lane) {
+                                               int *rowl, float *gl, int lane) {
   const bool changed = a.state_count[w] != 0;
   if (!changed) {
     if (lane == 0) {
@@ -233,38 +269,78 @@ __device__ __forceinline__ void search_sums_world(const NewtonArgs &a, int64_t w
   }
 }
 
+// ---- J search through a tile of 64 rows x 16 dofs (4.3 KB of LDS whatever the width of J) ------
+// The same chain per row as jv_world: the dofs in order, the 20-dof partial sums of the reference's
+// rule beyond 50 dofs.  A lane loads 16 elements per tile, four rows of 64 bytes per instruction.
+__device__ __forceinline__ void jv_world_tiled(const NewtonArgs &a, const float *Jw, int nefc, float *tile,
+                                               const float *sv, float *jv, int lane) {
+  const int nv = a.nv;
+  const int c = lane & 15, rq = lane >> 4;
+  const bool split = nv > 50;
+  for (int r0 = 0; r0 < nefc; r0 += 64) {
+    const int rows = nefc - r0 < 64 ? nefc - r0 : 64;
+    float acc = 0.0f, p = 0.0f;
+    for (int c0 = 0; c0 < nv; c0 += 16) {
+      const int cw = nv - c0 < 16 ? nv - c0 : 16;
+      float v[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const int r = rq + 4 * k;
+        v[k] = Jw[(int64_t)(r0 + (r < rows ? r : rows - 1)) * nv + c0 + (c < cw ? c : cw - 1)];
+      }
+#pragma unroll
+      for (int k = 0; k < 16; ++k) tile[(rq + 4 * k) * 17 + c] = v[k];
+      wave_sync();
+      if (lane < rows) {
+        const float *row = tile + lane * 17;
+        for (int i = 0; i < cw; ++i) {
+          if (split && (c0 + i) % 20 == 0 && c0 + i > 0) {
+            acc = acc + p;
+            p = 0.0f;
+          }
+          p = fma_(row[i], sv[c0 + i], p);
+        }
+      }
+      wave_sync();  // the tile is read before the next one overwrites it
+    }
+    if (lane < rows) jv[r0 + lane] = split ? acc + p : p;
+  }
+}
+
 // ---- the loop ------------------------------------------------------------------------------------
+// Where the loop's arrays lie in LDS (set up by the kernel around it).
+struct LoopLds {
+  int *votes;            // [4] cooperative stage only
+  const uint32_t *term;  // [nterm] col | madr << 16, shared by the workgroup
+  const int *radr;       // [nv + 1]
+  float *m_lds;          // per wavefront: [nM] the world's row of M
+  float *sv;             // [nv] the search direction
+  float *f;              // [njmax] forces of the listed rows
+  int *rowl;             // [njmax] their numbers
+  float *gl;             // [nv] the gradient
+  float *rows;           // staged rows of J: 64 x (nv | 1), or the 64 x 17 tile
+};
+
 // HELD: rows of a world a lane keeps in registers during the line search (0: read at every
-// evaluation); JU: loads in flight per lane while rows of J are staged.  `stage()` runs the factor
-// stage for the workgroup's four worlds (every wavefront calls it; it skips the worlds whose
-// `unchanged` byte is set).  `lds`: the workgroup's dynamic LDS.
-template <int HELD, int JU, class Stage>
-__device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Stage &&stage) {
-  const int lane = threadIdx.x & 63;
+// evaluation); JU: loads in flight per lane while rows of J are staged, 0 for the tiled staging.
+// COOP: `stage()` works on the workgroup's four worlds together (every wavefront calls it in step,
+// between two workgroup barriers; it skips the worlds whose `unchanged` byte is set), and a world
+// that is done idles through the barriers until the workgroup's last world finishes.  Otherwise
+// `stage()` is the wavefront's own world's stage, called only when that world needs it, and a
+// wavefront leaves as soon as its world is done.  `w_raw`: the wavefront's world.
+template <int HELD, int JU, bool COOP, class Stage>
+__device__ __forceinline__ void newton_loop(const NewtonArgs &a, const LoopLds &L, int64_t w_raw, Stage &&stage) {
+  const int lane_fixed = threadIdx.x & 63;
   const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  const int64_t w_raw = (int64_t)blockIdx.x * 4 + wv;
-  const bool live = w_raw < a.nworld;
-  const int64_t w = live ? w_raw : (int64_t)a.nworld - 1;
+  // the world's number as a scalar: every address below is a scalar base plus a lane offset
+  const int w_lo = __builtin_amdgcn_readfirstlane((int)(w_raw & 0xffffffff)), w_hi = __builtin_amdgcn_readfirstlane((int)(w_raw >> 32));
+  const int64_t w_uniform = ((int64_t)w_hi << 32) | (uint32_t)w_lo;
+  const bool live = w_uniform < a.nworld;
+  const int64_t w = live ? w_uniform : (int64_t)a.nworld - 1;
   const int nv = a.nv, njmax = a.njmax;
-  const int nM = a.nM;
-  // LDS: the factor stage's area (the staged rows of J use it between two stages), then the row
-  // tables of M v for the workgroup, then each wavefront's own arrays
-  int *votes = (int *)(lds + a.stage_lds_floats);  // [4] a wavefront's world is still being solved
-  uint32_t *term = (uint32_t *)(votes + 4);
-  int *radr = (int *)(term + a.nterm);
-  float *mine = (float *)(radr + nv + 1) + wv * (nM + nv + 2 * njmax + nv + 64);
-  float *m_lds = mine;              // [nM]
-  float *sv = m_lds + nM;           // [nv] the search direction
-  float *f = sv + nv;               // [njmax] forces of the listed rows
-  int *rowl = (int *)(f + njmax);   // [njmax] their numbers
-  float *gl = (float *)(rowl + njmax);  // [nv]
-  float *part = gl + nv;            // [64]
-  float *rows_lds = lds + wv * (64 * (nv | 1));  // inside the factor stage's area
-  for (int k = threadIdx.x; k < a.nterm; k += 256) term[k] = (uint32_t)a.mulm_col[k] | (uint32_t)a.mulm_madr[k] << 16;
-  for (int k = threadIdx.x; k <= nv; k += 256) radr[k] = a.mulm_rowadr[k];
-  for (int k = lane; k < nM; k += 64) m_lds[k] = a.M[w * a.ldM + k];
+  for (int k = lane_fixed; k < a.nM; k += 64) L.m_lds[k] = a.M[w * a.ldM + k];
   bool done = !live || a.done[w] != 0;
-  if (live && done && lane == 0) a.unchanged[w] = 1;  // the factor stage leaves such a world alone
+  if (live && done && lane_fixed == 0) a.unchanged[w] = 1;  // the factor stage leaves such a world alone
   bool unchanged = !done && a.unchanged[w] != 0;
   int nefc = a.nefc ? a.nefc[w] : njmax;
   nefc = __builtin_amdgcn_readfirstlane(nefc < njmax ? nefc : njmax);
@@ -273,19 +349,22 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Sta
                         a.nefc, a.smooth, a.D, a.frictionloss, a.Jaref, a.search, a.search_dot, a.mv, a.jv, a.Ma, nv, njmax,
                         njmax, njmax, nv, nv, njmax, nv, nullptr, a.alpha, a.improvement, a.exhausted, a.overflow,
                         a.ls_overflow_bit, nv, njmax, a.ls_iterations, a.nworld};
-  block_sync();
-  // every wavefront leaves the loop after at most maxiter rounds, whatever the data
-  const int lane_fixed = lane;
+  wave_sync();
 #ifdef IM_NEWTON_STAMPS  // development aid: time per phase, summed over the rounds, left in the world's row of jv
   long long t_phase[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t_last = wall_clock64();
 #define IM_STAMP(k) do { const long long t_now = wall_clock64(); t_phase[k] += t_now - t_last; t_last = t_now; } while (0)
 #else
 #define IM_STAMP(k) do {} while (0)
 #endif
+  // every wavefront leaves the loop after at most maxiter rounds, whatever the data
   for (int round = 0; round < a.maxiter; ++round) {
-    if (lane_fixed == 0) votes[wv] = done ? 0 : 1;
-    block_sync();
-    if (!(votes[0] | votes[1] | votes[2] | votes[3])) break;  // the workgroup's four worlds are done
+    if (COOP) {
+      if (lane_fixed == 0) L.votes[wv] = done ? 0 : 1;
+      block_sync();
+      if (!(L.votes[0] | L.votes[1] | L.votes[2] | L.votes[3])) break;  // the workgroup's four worlds are done
+    } else if (done) {
+      break;
+    }
     // the lane number as a value the compiler cannot see through, new in every round: nothing a
     // stage derives from it is kept in registers across the other stages
     int lane = lane_fixed;
@@ -293,10 +372,13 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Sta
     IM_STAMP(0);
     if (!done) {
       if (!unchanged) {
-        for (int k = lane; k < nv; k += 64) sv[k] = a.search[w * nv + k];
+        for (int k = lane; k < nv; k += 64) L.sv[k] = a.search[w * nv + k];
         wave_sync();
-        mul_m_world(a, term, radr, m_lds, sv, a.mv + w * nv, lane);
-        jv_world<JU>(a, Jw, nefc, rows_lds, sv, a.jv + w * njmax, lane);
+        mul_m_world(a, L.term, L.radr, L.m_lds, L.sv, a.mv + w * nv, lane);
+        if constexpr (JU > 0)
+          jv_world<(JU > 0 ? JU : 1)>(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, lane);
+        else
+          jv_world_tiled(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, lane);
         wave_sync();
       }
       IM_STAMP(1);
@@ -317,18 +399,24 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Sta
                                      a.state_count, w, lane);
       wave_sync();
       IM_STAMP(3);
-      unchanged = gradient_world(a, w, Jw, nefc, f, rowl, gl, part, lane);
+      unchanged = gradient_world(a, w, Jw, nefc, L.f, L.rowl, L.gl, lane);
       IM_STAMP(4);
     }
-    block_sync();  // gradients, states and the `unchanged` bytes of the four worlds are in place; the rows of J are done with
-    IM_STAMP(5);
-    stage();
-    block_sync();  // the four search directions are complete
+    if (COOP) {
+      block_sync();  // gradients, states and the `unchanged` bytes of the four worlds are in place; the rows of J are done with
+      IM_STAMP(5);
+      stage();
+      block_sync();  // the four search directions are complete
+    } else {
+      wave_sync();
+      if (!unchanged) stage();
+      wave_sync();
+    }
     IM_STAMP(6);
     lane = lane_fixed;
     asm volatile("" : "+v"(lane));  // no address from before the stage is kept through it
     if (!done) {
-      if (!unchanged) search_sums_world(a, w, lane);
+      if (COOP && !unchanged) search_sums_world(a, w, lane);  // a stage of its own leaves the two sums itself
       wave_sync();
       int finished = 0;
       if (lane == 0) {  // newton_fusion.py:265-296
@@ -354,6 +442,29 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, float *lds, Sta
   if (live && lane_fixed < 8) a.jv[w * njmax + lane_fixed] = (float)t_phase[lane_fixed];
 #endif
 #undef IM_STAMP
+}
+
+// The layout behind a cooperative stage's area of `a.stage_lds_floats` words (the staged rows of J
+// use that area between two stages): four flags, the row tables of M v, then each of the four
+// wavefronts' own arrays.  Fills the tables; the caller synchronises the workgroup before the loop.
+__device__ __forceinline__ LoopLds coop_layout(const NewtonArgs &a, float *lds) {
+  const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int nv = a.nv, njmax = a.njmax, nM = a.nM;
+  LoopLds L;
+  L.votes = (int *)(lds + a.stage_lds_floats);
+  uint32_t *term = (uint32_t *)(L.votes + 4);
+  int *radr = (int *)(term + a.nterm);
+  float *mine = (float *)(radr + nv + 1) + wv * (nM + nv + 2 * njmax + nv + 64);
+  L.term = term, L.radr = radr;
+  L.m_lds = mine;
+  L.sv = L.m_lds + nM;
+  L.f = L.sv + nv;
+  L.rowl = (int *)(L.f + njmax);
+  L.gl = (float *)(L.rowl + njmax);
+  L.rows = lds + wv * (64 * (nv | 1));
+  for (int k = threadIdx.x; k < a.nterm; k += blockDim.x) term[k] = (uint32_t)a.mulm_col[k] | (uint32_t)a.mulm_madr[k] << 16;
+  for (int k = threadIdx.x; k <= nv; k += blockDim.x) radr[k] = a.mulm_rowadr[k];
+  return L;
 }
 
 }  // namespace resident

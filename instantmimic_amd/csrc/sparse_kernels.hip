@@ -17,6 +17,7 @@
 #include <vector>
 
 #include "common.h"
+#include "newton_wave.h"
 #include "sparse_plan.h"
 
 namespace im {
@@ -605,23 +606,15 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
 // and a lane keeps four pairs' table look-ups in flight.
 constexpr int kStagedRows = 16;
 
-template <int WAVES>
-__global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void sparse_update_wave_kernel(
-    SparseWave A, const uint8_t *__restrict__ done, const int32_t *__restrict__ state_changes,
-    const int32_t *__restrict__ changes, const int32_t *__restrict__ ids, int ld_ids,
-    const float *__restrict__ J, int njmax, const float *__restrict__ D,
-    const int32_t *__restrict__ state, int quad, const float *__restrict__ grad, int ldg,
-    float *__restrict__ U_, int32_t *__restrict__ uni_, float *__restrict__ search_,
-    float *__restrict__ search_dot, float *__restrict__ decrement, int nworld) {
-  extern __shared__ float lds[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-  SparseDev Q = A.P;
+// The factor and solve tables of a plan into LDS, for a workgroup of T threads (a flat 16-byte copy,
+// every load issued before the first store); Q's table pointers then address the copy.
+template <int T>
+__device__ __forceinline__ void stage_update_tables(const SparseWave &A, SparseDev &Q, float *lds, int tid) {
   int32_t *tab = (int32_t *)lds;
   {
     const int4 *src = (const int4 *)A.P.t[0];
     const int nvec = A.staged_words >> 2;
-    constexpr int T = 64 * WAVES, NB = 2048 / T;  // the host admits at most 8192 words
+    constexpr int NB = (2048 + T - 1) / T;  // the host admits at most 8192 words
     int4 buf[NB];
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
@@ -640,7 +633,7 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void sparse_update_wave_ker
     // forward-solve tables (at most 16 KB), behind the first stretch
     const int4 *src = (const int4 *)A.P.t[FL];
     const int nvec = A.solve_words >> 2;
-    constexpr int T = 64 * WAVES, NB = 1024 / T;  // at most 4096 words
+    constexpr int NB = (1024 + T - 1) / T;  // at most 4096 words
     int4 buf[NB];
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
@@ -655,13 +648,23 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void sparse_update_wave_ker
 #pragma unroll
     for (int i = 0; i < 5; ++i) Q.t[FL + i] = tab + A.staged_words + A.solve[i];
   }
-  __syncthreads();  // the only workgroup barrier
-  const int w = blockIdx.x * WAVES + wv;
-  if (w >= nworld || (done && done[w]) || state_changes[w] == 0) return;
+}
+__host__ __device__ inline int update_world_words(int nslots, int n, int block) {
+  const int nw = (block + 31) / 32;
+  return (nslots + n + 2 * nw + 2 * n + kStagedRows * (n + 1) + 3) & ~3;
+}
+
+// The stage for one world and one wavefront (`world_lds`: update_world_words of LDS of its own).
+__device__ __forceinline__ void sparse_update_world(
+    const SparseWave &A, const SparseDev &Q, float *world_lds, const int32_t *__restrict__ changes,
+    const int32_t *__restrict__ ids, int ld_ids, const float *__restrict__ J, int njmax,
+    const float *__restrict__ D, const int32_t *__restrict__ state, int quad, const float *__restrict__ grad, int ldg,
+    float *__restrict__ U_, int32_t *__restrict__ uni_, float *__restrict__ search_, float *__restrict__ search_dot,
+    float *__restrict__ decrement, int w, int lane) {
   const int n = Q.nv, nslots = Q.nslots, nfac = nslots - n, rhs = nfac;
   const int nw = (A.block + 31) / 32;
   const int per_world = (nslots + n + 2 * nw + 2 * n + kStagedRows * (n + 1) + 3) & ~3;
-  float *N = lds + A.staged_words + A.solve_words + wv * per_world;  // [nslots]
+  float *N = world_lds;  // [nslots]
   float *iD = N + nslots;                            // [n]
   float *red = iD + n;                               // [2][nw]
   int *ul = (int *)(red + 2 * nw);                   // [n] ascending dofs touched by the changed rows
@@ -806,6 +809,76 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void sparse_update_wave_ker
   }
   backward_sums<true>(Q, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, 64,
                       A.block);
+}
+
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void sparse_update_wave_kernel(
+    SparseWave A, const uint8_t *__restrict__ done, const int32_t *__restrict__ state_changes,
+    const int32_t *__restrict__ changes, const int32_t *__restrict__ ids, int ld_ids,
+    const float *__restrict__ J, int njmax, const float *__restrict__ D,
+    const int32_t *__restrict__ state, int quad, const float *__restrict__ grad, int ldg,
+    float *__restrict__ U_, int32_t *__restrict__ uni_, float *__restrict__ search_,
+    float *__restrict__ search_dot, float *__restrict__ decrement, int nworld) {
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  SparseDev Q = A.P;
+  stage_update_tables<64 * WAVES>(A, Q, lds, tid);
+  __syncthreads();  // the only workgroup barrier
+  const int w = blockIdx.x * WAVES + wv;
+  if (w >= nworld || (done && done[w]) || state_changes[w] == 0) return;
+  float *world_lds = lds + A.staged_words + A.solve_words + wv * update_world_words(Q.nslots, Q.nv, A.block);
+  sparse_update_world(A, Q, world_lds, changes, ids, ld_ids, J, njmax, D, state, quad, grad, ldg, U_, uni_, search_,
+                      search_dot, decrement, w, lane);
+}
+
+// The resident Newton loop with this stage (newton_wave.h): a wavefront per world from the first
+// line search to convergence, WAVES worlds per workgroup sharing one copy of the plan's tables.
+// Per wavefront in LDS: the world's row of M and the search direction, and one area that the staged
+// tile of J, the gradient's row list and the stage's factor use one after the other.
+__host__ __device__ inline int resident_area_words(int nslots, int n, int block, int njmax) {
+  int words = update_world_words(nslots, n, block);
+  const int tile = 64 * 17, grad = 2 * njmax + n;
+  words = words > tile ? words : tile;
+  words = words > grad ? words : grad;
+  return (words + 3) & ~3;
+}
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident_kernel(
+    SparseWave A, resident::NewtonArgs a, float *__restrict__ U_, int32_t *__restrict__ uni_) {
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  SparseDev Q = A.P;
+  stage_update_tables<64 * WAVES>(A, Q, lds, tid);
+  const int nv = a.nv, njmax = a.njmax;
+  uint32_t *term = (uint32_t *)(lds + A.staged_words + A.solve_words);
+  int *radr = (int *)(term + a.nterm);
+  const int area = resident_area_words(Q.nslots, nv, A.block, njmax);
+  float *mine = (float *)(radr + nv + 1) + wv * (area + a.nM + nv);
+  resident::LoopLds L;
+  L.votes = nullptr;
+  L.term = term, L.radr = radr;
+  L.rows = mine;  // the shared area: tile of J, then the gradient's lists, then the stage
+  L.f = mine;
+  L.rowl = (int *)(mine + njmax);
+  L.gl = mine + 2 * njmax;
+  L.m_lds = mine + area;
+  L.sv = L.m_lds + a.nM;
+  for (int k = tid; k < a.nterm; k += 64 * WAVES) term[k] = (uint32_t)a.mulm_col[k] | (uint32_t)a.mulm_madr[k] << 16;
+  for (int k = tid; k <= nv; k += 64 * WAVES) radr[k] = a.mulm_rowadr[k];
+  __syncthreads();  // the only workgroup barrier
+  const int64_t w = (int64_t)blockIdx.x * WAVES + wv;
+  auto stage = [&]() __attribute__((always_inline)) {
+    sparse_update_world(A, Q, mine, a.quad_count, a.ids, a.ld_ids, a.J, njmax, a.D, a.state, a.quad, a.grad,
+                        (int)a.ld_grad, U_, uni_, a.search, a.search_dot, a.decrement, (int)w, threadIdx.x & 63);
+  };
+  if (njmax <= 64)
+    resident::newton_loop<2, 0, false>(a, L, w, stage);
+  else if (njmax <= 128)
+    resident::newton_loop<4, 0, false>(a, L, w, stage);
+  else
+    resident::newton_loop<0, 0, false>(a, L, w, stage);
 }
 
 // Per-iteration factor stage: changed rows' dof union, incremental update of packed H,
@@ -1136,6 +1209,68 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done, con
                      dof_union, search, search_dot, decrement);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
+}
+
+int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *p, float *hfactor, int32_t *dof_union,
+                           void *stream) {
+  if (!plan || !p || !hfactor || !dof_union || p->nworld < 0) return IM_ERR_ARG;
+  if (!plan->device_ready || plan->path != IM_SPARSE_FUSED || plan->nv > 64) return IM_ERR_UNSUPPORTED;
+  if (p->nworld == 0) return IM_OK;
+  const int n = plan->nv, njmax = p->njmax;
+  const int nM = plan->nM;
+  if (nM <= 0) return IM_ERR_UNSUPPORTED;
+  im::resident::NewtonArgs a{};
+  const int bad = im::resident::convert_args(*p, n, nM, a);
+  if (bad != IM_OK) return bad;
+  if (p->block != plan->block) return IM_ERR_ARG;
+  im::SparseWave A;
+  for (int i = 0; i < im::NHOST; ++i) A.P.t[i] = plan->t[i];
+  A.P.nv = plan->nv; A.P.nv_pad = plan->nv_pad; A.P.nslots = plan->nslots; A.P.nlevels = plan->nlevels;
+  for (int i = 0; i < im::kStaged; ++i) A.staged[i] = (int)(plan->t[i] - plan->t[0]);
+  const size_t staged = (size_t)(plan->t[im::kStaged] - plan->t[0]);
+  A.staged_words = (int)staged;
+  A.tile_index = nullptr;
+  A.block = plan->block;
+  A.nM = 0;
+  const int32_t *solve_end = plan->t[im::RK] + ((plan->sizes[im::RK] + 3) & ~3);
+  const size_t solve_words = (size_t)(solve_end - plan->t[im::FL]);
+  for (int i = 0; i < 5; ++i) A.solve[i] = (int)(plan->t[im::FL + i] - plan->t[im::FL]);
+  A.solve_words = (int)solve_words;
+  if (staged > 8192 || solve_words > 4096) return IM_ERR_UNSUPPORTED;
+  const size_t shared = staged + solve_words + (size_t)p->nterm + n + 1;
+  const size_t per_wave = (size_t)im::resident_area_words(plan->nslots, n, plan->block, njmax) + nM + n;
+  // the most worlds per workgroup (one workgroup per CU) that 160 KB of LDS admit and whose kernel
+  // keeps to registers
+  struct Variant {
+    int waves;
+    const void *fn;
+  };
+  static const Variant variants[] = {{16, (const void *)im::newton_sparse_resident_kernel<16>},
+                                     {12, (const void *)im::newton_sparse_resident_kernel<12>},
+                                     {8, (const void *)im::newton_sparse_resident_kernel<8>},
+                                     {4, (const void *)im::newton_sparse_resident_kernel<4>}};
+  static bool usable[4] = {false, false, false, false};
+  static bool probed = false;
+  if (!probed) {  // once per process: register spills and the grant of the large dynamic LDS
+    for (int i = 0; i < 4; ++i) {
+      hipFuncAttributes fa{};
+      usable[i] = hipFuncGetAttributes(&fa, variants[i].fn) == hipSuccess && fa.localSizeBytes == 0 &&
+                  hipFuncSetAttribute(variants[i].fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      160 * 1024 - (int)fa.sharedSizeBytes) == hipSuccess;
+      (void)hipGetLastError();
+    }
+    probed = true;
+  }
+  for (int i = 0; i < 4; ++i) {
+    const size_t lds = 4 * (shared + (size_t)variants[i].waves * per_wave);
+    if (!usable[i] || lds > 158 * 1024) continue;
+    const int waves = variants[i].waves;
+    void *args[] = {&A, &a, &hfactor, &dof_union};
+    IM_HIP_CHECK(hipLaunchKernel(variants[i].fn, dim3((unsigned)((p->nworld + waves - 1) / waves)), dim3(64 * waves), args,
+                                 lds, (hipStream_t)stream));
+    return IM_OK;
+  }
+  return IM_ERR_UNSUPPORTED;
 }
 
 int im_sparse_dense_factor(const im_sparse_plan *plan, const uint8_t *done, const float *grad, int ldg,

@@ -769,35 +769,9 @@ int im_newton_solve_tree(const im_tree_plan *plan, const im_newton_args *p, void
   if (!e->newton || !e->newton_long) return IM_ERR_UNSUPPORTED;
   if (p->nworld == 0) return IM_OK;
   const int nv = plan->nv, nM = plan->nM, njmax = p->njmax;
-  if (njmax <= 0 || p->iterations < 0 || p->ls_iterations < 0 || (p->block != 32 && p->block != 64) ||
-      p->ntolerance <= 0 || p->nls_tolerance <= 0 || p->nmeaninertia <= 0 || p->nterm <= 0)
-    return IM_ERR_ARG;
-  if (!p->opt_tolerance || !p->opt_ls_tolerance || !p->stat_meaninertia || !p->M_mulm_rowadr || !p->M_mulm_col ||
-      !p->M_mulm_madr || !p->M || !p->efc_J || !p->efc_D || !p->qfrc_smooth || !p->qacc || !p->efc_Ma ||
-      !p->efc_force || !p->efc_state || !p->Jaref || !p->search || !p->search_dot || !p->mv || !p->jv || !p->alpha ||
-      !p->improvement || !p->grad || !p->grad_dot || !p->grad_scale || !p->newton_decrement || !p->qfrc_constraint ||
-      !p->quad_changed_ids || !p->quad_changed_count || !p->state_changed_count || !p->solver_niter || !p->done ||
-      !p->ls_exhausted || !p->search_unchanged || (p->nf && !p->efc_frictionloss))
-    return IM_ERR_ARG;
-  if (p->ldM < nM || p->ld_grad < nv || p->ld_ids < 0) return IM_ERR_STRIDE;
-  if (p->nterm >= 65536 || 64 * (int64_t)nv >= (1 << 20)) return IM_ERR_UNSUPPORTED;
   im::resident::NewtonArgs a{};
-  a.tolerance = p->opt_tolerance, a.ls_tolerance = p->opt_ls_tolerance, a.meaninertia = p->stat_meaninertia;
-  a.ntolerance = p->ntolerance, a.nls_tolerance = p->nls_tolerance, a.nmeaninertia = p->nmeaninertia;
-  a.nv = nv, a.njmax = njmax, a.nworld = p->nworld, a.ls_iterations = p->ls_iterations, a.maxiter = p->iterations;
-  a.block = p->block, a.quad = p->quad, a.ls_overflow_bit = p->ls_overflow_bit;
-  a.iter_overflow_bit = p->iterations_overflow_bit;
-  a.mulm_rowadr = p->M_mulm_rowadr, a.mulm_col = p->M_mulm_col, a.mulm_madr = p->M_mulm_madr;
-  a.nterm = p->nterm, a.nM = nM;
-  a.ne = p->ne, a.nf = p->nf, a.nefc = p->nefc, a.M = p->M, a.ldM = p->ldM, a.J = p->efc_J, a.D = p->efc_D;
-  a.frictionloss = p->efc_frictionloss, a.smooth = p->qfrc_smooth;
-  a.qacc = p->qacc, a.Ma = p->efc_Ma, a.force = p->efc_force, a.Jaref = p->Jaref, a.search = p->search;
-  a.search_dot = p->search_dot, a.mv = p->mv, a.jv = p->jv, a.alpha = p->alpha, a.improvement = p->improvement;
-  a.grad = p->grad, a.grad_dot = p->grad_dot, a.grad_scale = p->grad_scale, a.decrement = p->newton_decrement;
-  a.qfrc_constraint = p->qfrc_constraint, a.ld_grad = p->ld_grad;
-  a.state = p->efc_state, a.ids = p->quad_changed_ids, a.quad_count = p->quad_changed_count;
-  a.state_count = p->state_changed_count, a.niter = p->solver_niter, a.overflow = p->overflow, a.nsolving = p->nsolving;
-  a.ld_ids = p->ld_ids, a.done = p->done, a.exhausted = p->ls_exhausted, a.unchanged = p->search_unchanged;
+  const int bad = im::resident::convert_args(*p, nv, nM, a);
+  if (bad != IM_OK) return bad;
   // the factor stage's LDS (its staged tiles and exchange slots plus the four worlds' row lists), or the
   // four wavefronts' staged rows of J where those take more; the loop's own arrays behind it
   const size_t stage_bytes = (size_t)e->lds_bytes + 32 * std::max<size_t>(((size_t)njmax + 15) / 16 * 16, 64);

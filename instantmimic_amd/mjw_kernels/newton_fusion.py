@@ -735,23 +735,37 @@ def _resident_args(m, d, ctx, nsolving):
 
 
 def run_resident(m, d, ctx, nsolving) -> bool:
-    """The whole loop as one resident kernel (a wavefront per world until it is done), for a ``ctx``
-    with the tree stage whose plan carries generated kernels; False when there is no such kernel
-    for this model (the caller then launches the stages one by one)."""
+    """The whole loop as one resident kernel (a wavefront per world until it is done): for a ``ctx``
+    with a fused sparse plan, or with the tree stage whose plan carries generated kernels.  False
+    when there is no such kernel for this model (the caller then launches the stages one by one)."""
     import ctypes as C
 
     import torch
 
-    scratch = _tree_scratch(ctx)
-    if scratch is None or os.environ.get("IMHIP_NEWTON") == "stages":
+    scratch, plan = _tree_scratch(ctx), _fused_plan(ctx)
+    if (scratch is None and plan is None) or os.environ.get("IMHIP_NEWTON") == "stages":
         return False
     a = _resident_args(m, d, ctx, nsolving)
     dev = d.efc.J.device
+    stream = int(torch.cuda.current_stream(dev).cuda_stream)
     with torch.cuda.device(dev):
-        status = _lib.lib().im_newton_solve_tree(scratch.kernel.ptr, C.byref(a), int(torch.cuda.current_stream(dev).cuda_stream))
+        if plan is not None:
+            nworld, nv, pad = int(d.nworld), int(m.nv), int(m.nv_pad)
+            hf, uni = ctx.hfactor, ctx.newton_dof_union
+            if hf.dtype != torch.float32 or hf.device != dev or tuple(hf.shape) != (nworld, pad, pad) or not hf.is_contiguous():
+                raise TypeError("hfactor must be a contiguous float32 (nworld, nv_pad, nv_pad) tensor")
+            if uni.dtype != torch.int32 or uni.device != dev or tuple(uni.shape) != (nworld, nv + 1) or not uni.is_contiguous():
+                raise TypeError("newton_dof_union must be a contiguous int32 (nworld, nv + 1) tensor")
+            if plan.handle is None or plan.nv != nv or plan.nv_pad != pad:
+                raise ValueError("the sparse plan has no device state or belongs to another model")
+            status = _lib.lib().im_newton_solve_sparse(plan.ptr, C.byref(a), hf.data_ptr(), uni.data_ptr(), stream)
+            where = "im_newton_solve_sparse"
+        else:
+            status = _lib.lib().im_newton_solve_tree(scratch.kernel.ptr, C.byref(a), stream)
+            where = "im_newton_solve_tree"
     if status == _lib.IM_ERR_UNSUPPORTED:
         return False
-    _lib.check(status, "im_newton_solve_tree")
+    _lib.check(status, where)
     return True
 
 

@@ -136,11 +136,12 @@ def _solve_on_gpu(p, device, *, graph: bool):
     ("humanoid", 4096, "tree", True, "stages"), ("humanoid", 4096, "dense", True, "stages"), ("g1", 8192, "sparse", True, "stages"),
     ("snu", 4096, "sparse", True, "stages"), ("ant", 64, "tree", True, "stages"), ("snu", 130, "tree", False, "stages"),
     ("humanoid", 301, "tree", False, "resident"), ("humanoid", 4096, "tree", True, "resident"), ("ant", 67, "tree", True, "resident"),
+    ("g1", 203, "sparse", False, "resident"), ("g1", 8192, "sparse", True, "resident"), ("snu", 4096, "sparse", True, "resident"),
 ])  # fmt: skip
 def test_gpu_solve_from_init_context_matches_the_oracle_chain(device, monkeypatch, name, nworld, stage, graph, loop):
     """``loop``: the iterations as eight launches each (``stages``) or as one resident kernel with a
-    wavefront per world (``resident``, the tree stage with generated kernels): the same arrays at the
-    end either way."""
+    wavefront per world (``resident``: the tree stage with generated kernels, the sparse stage): the
+    same arrays at the end either way."""
     small = nworld <= 301
     p = NC.problem(name, nworld, stage, empty_every=11 if small else 97, warmstart=small, maxiter=12)
     s = NC.oracle_solve(p)
