@@ -886,24 +886,22 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("  #undef STAMP")
     emit("}")
     args = "M, ldM, J, njmax, D, state, nefc_p, quad, y, ldy, x, ldx, Hout, nworld, flags, niter, state_it, y_it, x_it, skip"
-    ju = 16 if nv <= 16 else 32  # loads in flight per lane while rows of J are staged (a register each)
     # The resident Newton loop with this tree's fused kernel as its factor stage: search = -H^-1 grad
-    # for the workgroup's four worlds, those whose `unchanged` byte is set left alone.  LONG decides
-    # the rows a lane of the line search keeps in registers: two up to 64 rows, four up to 128.
+    # for the workgroup's four worlds, those whose `unchanged` byte is set left alone.  The line
+    # search keeps a lane's two rows in registers up to 64 rows (the short kernel) and reads the rows
+    # from LDS at every evaluation beyond.
     emit("template <bool LONG>")
     emit(f"__device__ __forceinline__ void newton_row16_body_{name}(const im::resident::NewtonArgs &a) {{")
     emit("  extern __shared__ float xlds[];")
     emit("  auto stage = [&]() __attribute__((always_inline)) {")
+    emit("    const im::resident::NewtonArgs &a = im::resident::kernel_args(0);  // the kernel's only argument")
     emit(f"    tree_row16_body_{name}<true, LONG>(a.M, a.ldM, a.J, a.njmax, a.D, a.state, a.nefc, a.quad, a.grad, a.ld_grad, a.search,")
     emit("        (int64_t)a.nv, nullptr, a.nworld, IM_FLAG_NEGATE, 1, 0, 0, 0, a.unchanged);")
     emit("  };")
     emit("  const im::resident::LoopLds L = im::resident::coop_layout(a, xlds);")
     emit("  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);")
     emit("  im::resident::block_sync();")
-    emit("  if (LONG && a.njmax > 128)")
-    emit(f"    im::resident::newton_loop<0, {ju}, true>(a, L, w, stage);")
-    emit("  else")
-    emit(f"    im::resident::newton_loop<(LONG ? 4 : 2), {ju}, true>(a, L, w, stage);")
+    emit("  im::resident::newton_loop<(LONG ? 0 : 2), 0, true>(0, L, w, stage);")
     emit("}")
     if module:
         emit("} }  // namespace im::gen")

@@ -101,28 +101,35 @@ struct SearchArgs {
   int overflow_bit, nv, njmax, ls_iterations, nworld;
 };
 
-// Two worlds per wavefront, 32 lanes each (the reference's reduction width).  HELD: rows of the
-// world a lane keeps in registers (weight, friction loss, Jaref, jv and the cost at alpha 0) --
-// every candidate step evaluates every row, three candidates per round; 0: more rows than that,
-// read from memory at every evaluation.
+// One world's rows and scalars as the line search reads them (the rows may lie in memory or in LDS).
+struct LsWorld {
+  const float *smooth, *D, *frictionloss, *Jaref, *search, *mv, *jv, *Ma;  // frictionloss may be null
+  float search_dot, tolerance, ls_tolerance, meaninertia;
+  int ne, nf, nefc, nv, ls_iterations;
+};
+struct LsResult {
+  float alpha, improvement;
+  bool exhausted, converged;
+};
+
+// 32 lanes per world (the reference's reduction width), two such groups per wavefront.  HELD: rows
+// of the world a lane keeps in registers (weight, friction loss, Jaref, jv and the cost at alpha 0)
+// -- every candidate step evaluates every row, three candidates per round; 0: more rows than that,
+// read at every evaluation.  Every lane of the group returns the same result.
 template <int HELD>
-__device__ __forceinline__ void linesearch_world(const SearchArgs &a, int64_t w, int lane) {
-  const int nv = a.nv;
-  const int ne = a.ne ? a.ne[w] : 0, nf = a.nf ? a.nf[w] : 0;
-  int nefc = a.nefc ? a.nefc[w] : a.njmax;
-  nefc = nefc < a.njmax ? nefc : a.njmax;
-  const float *D = a.D + w * a.ld_D, *fl = a.frictionloss ? a.frictionloss + w * a.ld_floss : nullptr;
-  const float *Jaref = a.Jaref + w * a.ld_Jaref, *jv = a.jv + w * a.ld_jv;
-  const float tolerance = a.tolerance[w % a.ntolerance], ls_tolerance = a.ls_tolerance[w % a.nls_tolerance];
-  const float snorm = sqrtf(a.search_dot[w]);
-  const float scale = a.meaninertia[w % a.nmeaninertia] * (float)nv;
+__device__ __forceinline__ LsResult linesearch_rows(const LsWorld &wd, int lane) {
+  const int nv = wd.nv, ne = wd.ne, nf = wd.nf, nefc = wd.nefc;
+  const float *D = wd.D, *fl = wd.frictionloss, *Jaref = wd.Jaref, *jv = wd.jv;
+  const float tolerance = wd.tolerance, ls_tolerance = wd.ls_tolerance;
+  const float snorm = sqrtf(wd.search_dot);
+  const float scale = wd.meaninertia * (float)nv;
   const float gtol = fmaxf(tolerance * ls_tolerance * snorm * scale, 1.0e-6f);
   // Gauss term and equality rows: one quadratic (0, g1, g2)
   float g1 = 0.0f, g2 = 0.0f;
   for (int dof = lane; dof < nv; dof += 32) {
-    const float s = a.search[w * a.ld_search + dof];
-    g1 = g1 + s * (a.Ma[w * a.ld_Ma + dof] - a.smooth[w * a.ld_smooth + dof]);
-    g2 = g2 + 0.5f * s * a.mv[w * a.ld_mv + dof];
+    const float s = wd.search[dof];
+    g1 = g1 + s * (wd.Ma[dof] - wd.smooth[dof]);
+    g2 = g2 + 0.5f * s * wd.mv[dof];
   }
   for (int r = lane; r < ne; r += 32) {
     const float jvD = jv[r] * D[r];
@@ -190,7 +197,7 @@ __device__ __forceinline__ void linesearch_world(const SearchArgs &a, int64_t w,
     const bool lo_less = lo_in.g < p0.g;
     Pt lo = lo_less ? lo_in : p0_delta, hi = lo_less ? p0_delta : lo_in;
     float lo_alpha = lo_less ? lo_alpha_in : 0.0f, hi_alpha = lo_less ? 0.0f : lo_alpha_in;
-    for (int it = 0; it < a.ls_iterations; ++it) {
+    for (int it = 0; it < wd.ls_iterations; ++it) {
       const float lo_next_alpha = lo_alpha - safe_div(lo.g, lo.h);
       const float hi_next_alpha = hi_alpha - safe_div(hi.g, hi.h);
       const float mid_alpha = 0.5f * (lo_alpha + hi_alpha);
@@ -246,11 +253,23 @@ __device__ __forceinline__ void linesearch_world(const SearchArgs &a, int64_t w,
       }
     }
   }
+  return {alpha, improvement, fabsf(alpha) < noise_floor, converged};
+}
+
+template <int HELD>
+__device__ __forceinline__ void linesearch_world(const SearchArgs &a, int64_t w, int lane) {
+  int nefc = a.nefc ? a.nefc[w] : a.njmax;
+  nefc = nefc < a.njmax ? nefc : a.njmax;
+  const LsWorld r{a.smooth + w * a.ld_smooth, a.D + w * a.ld_D, a.frictionloss ? a.frictionloss + w * a.ld_floss : nullptr,
+                  a.Jaref + w * a.ld_Jaref, a.search + w * a.ld_search, a.mv + w * a.ld_mv, a.jv + w * a.ld_jv,
+                  a.Ma + w * a.ld_Ma, a.search_dot[w], a.tolerance[w % a.ntolerance], a.ls_tolerance[w % a.nls_tolerance],
+                  a.meaninertia[w % a.nmeaninertia], a.ne ? a.ne[w] : 0, a.nf ? a.nf[w] : 0, nefc, a.nv, a.ls_iterations};
+  const LsResult out = linesearch_rows<HELD>(r, lane);
   if (lane == 0) {
-    a.alpha[w] = alpha;
-    a.improvement[w] = improvement;
-    a.exhausted[w] = fabsf(alpha) < noise_floor ? 1 : 0;
-    if (!converged && a.overflow) a.overflow[w] = a.overflow[w] | a.overflow_bit;
+    a.alpha[w] = out.alpha;
+    a.improvement[w] = out.improvement;
+    a.exhausted[w] = out.exhausted ? 1 : 0;
+    if (!out.converged && a.overflow) a.overflow[w] = a.overflow[w] | a.overflow_bit;
   }
 }
 

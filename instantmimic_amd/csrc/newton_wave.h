@@ -97,17 +97,19 @@ __device__ __forceinline__ void block_sync() {
 
 // words of LDS of the loop's own arrays behind the factor stage's area: four flags, the row tables of M v
 // (one word per term, nv + 1 offsets), then per wavefront the world's row of M, the search
-// direction, the gradient stage's list of rows with a force (value and row number), its copy of the
-// gradient and 64 words of lane sums.  The factor stage's area must also hold four wavefronts'
-// staged rows of J: 4 x 64 rows, a row nv | 1 words.
+// direction, Ma, mv, Jaref, jv, D and the friction losses, the gradient's list of rows with a force
+// (value and row number) and its copy of the gradient.  The factor stage's area must also hold four wavefronts'
+// staged tiles of J: 4 x 64 rows x 16 dofs, a row 17 words.
+// words a wavefront keeps from round to round: M, the search direction, Ma, mv; Jaref, jv, D, friction losses
+__host__ __device__ inline size_t kept_words(int nv, int njmax, int nM) { return (size_t)nM + 3 * (size_t)nv + 4 * (size_t)njmax; }
 __host__ __device__ inline size_t loop_lds_words(int nv, int njmax, int nM, int nterm) {
-  return 4 + (size_t)nterm + nv + 1 + 4 * ((size_t)nM + nv + 2 * (size_t)njmax + nv + 64);
+  return 4 + (size_t)nterm + nv + 1 + 4 * (kept_words(nv, njmax, nM) + 2 * (size_t)njmax + nv);
 }
-__host__ __device__ inline size_t staged_rows_words(int nv) { return 4 * 64 * (size_t)(nv | 1); }
+__host__ __device__ inline size_t staged_rows_words(int) { return 4 * 64 * 17; }  // four wavefronts' tiles of J
 
 // ---- M search (newton_fusion.py:171-176): lane d owns dofs d, d + 64 --------------------------
 __device__ __forceinline__ void mul_m_world(const NewtonArgs &a, const uint32_t *term, const int *radr, const float *m,
-                                            const float *v, float *out, int lane) {
+                                            const float *v, float *out, float *out_lds, int lane) {
   for (int dof = lane; dof < a.nv; dof += 64) {
     float value = 0.0f;
     const int end = radr[dof + 1];
@@ -123,13 +125,14 @@ __device__ __forceinline__ void mul_m_world(const NewtonArgs &a, const uint32_t 
       for (int u = 0; u < 4; ++u) value = k + u < end ? fma_(x[u], y[u], value) : value;
     }
     out[dof] = value;
+    out_lds[dof] = value;
   }
 }
 
 // ---- J search (newton_stages.py:157-178): 64 rows at a time through LDS, a lane per row --------
 template <int U>
 __device__ __forceinline__ void jv_world(const NewtonArgs &a, const float *Jw, int nefc, float *rows_lds,
-                                         const float *sv, float *jv, int lane) {
+                                         const float *sv, float *jv, float *jv_lds, int lane) {
   const int nv = a.nv, stride = nv | 1;
   const float inv_nv = 1.0f / (float)nv;
   for (int r0 = 0; r0 < nefc; r0 += 64) {
@@ -175,47 +178,45 @@ __device__ __forceinline__ void jv_world(const NewtonArgs &a, const float *Jw, i
         acc = chain(0, nv);
       }
       jv[r0 + lane] = acc;
+      jv_lds[r0 + lane] = acc;
     }
     wave_sync();  // the rows are read before the next 64 overwrite them
   }
 }
 
 // ---- the gradient (newton_stages.py:745-798), a lane per dof ------------------------------------
-// Returns whether the search direction stays as it is (no state changed).
-__device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, const float *Jw, int nefc, float *f,
-                                               int *rowl, float *gl, int lane) {
-  const bool changed = a.state_count[w] != 0;
+// The world's scalars that the loop carries in registers (every lane the same values); they are
+// written to memory as they change.
+struct Scalars {
+  float search_dot, grad_dot, decrement, grad_scale, alpha, improvement;
+  int niter;
+};
+// For a world whose states changed: qfrc_constraint = J' force over the listed rows (`cnt` rows with
+// a nonzero force, ascending, in f / rowl), grad = Ma - qfrc_smooth - qfrc_constraint, grad . grad.
+// Otherwise the rescaling of the three scalars.  Returns whether the search direction stays.
+__device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, const float *Jw, bool changed, int cnt,
+                                               const float *f, const int *rowl, const float *Ma_l, float *gl, Scalars &sc,
+                                               int lane) {
   if (!changed) {
+    const float sigma = sc.grad_scale, new_sigma = sigma - sc.alpha;
+    float ratio = 0.0f;
+    if (sigma != 0.0f) ratio = new_sigma / sigma;
+    const float ratio_sq = ratio * ratio;
+    sc.grad_dot = sc.grad_dot * ratio_sq;
+    sc.decrement = sc.decrement * ratio_sq;
+    sc.grad_scale = new_sigma;
     if (lane == 0) {
-      const float sigma = a.grad_scale[w], new_sigma = sigma - a.alpha[w];
-      float ratio = 0.0f;
-      if (sigma != 0.0f) ratio = new_sigma / sigma;
-      const float ratio_sq = ratio * ratio;
-      a.grad_dot[w] = a.grad_dot[w] * ratio_sq;
-      a.decrement[w] = a.decrement[w] * ratio_sq;
-      a.grad_scale[w] = new_sigma;
+      a.grad_dot[w] = sc.grad_dot;
+      a.decrement[w] = sc.decrement;
+      a.grad_scale[w] = sc.grad_scale;
       a.unchanged[w] = 1;
     }
     return true;
   }
   const int nv = a.nv;
-  // rows with a force, in order (a satisfied constraint's force is zero and its row adds nothing)
-  int cnt = 0;
-  for (int r0 = 0; r0 < nefc; r0 += 64) {
-    const int r = r0 + lane;
-    const float v = r < nefc ? a.force[w * a.njmax + r] : 0.0f;
-    const unsigned long long mask = __ballot(v != 0.0f);
-    if (v != 0.0f) {
-      const int pos = cnt + __popcll(mask & ((1ull << lane) - 1ull));
-      f[pos] = v;
-      rowl[pos] = r;
-    }
-    cnt += __popcll(mask);
-  }
-  wave_sync();
-  constexpr int ROWS = 8;
+  constexpr int ROWS = 16;
   for (int dof = lane; dof < nv; dof += 64) {
-    const float ma = a.Ma[w * nv + dof], sm = a.smooth[w * nv + dof];
+    const float ma = Ma_l[dof], sm = a.smooth[w * nv + dof];
     float sum = 0.0f;
     for (int p0 = 0; p0 < cnt; p0 += ROWS) {
       float jv[ROWS];
@@ -236,10 +237,12 @@ __device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, c
   if (lane < a.block)
     for (int dof = lane; dof < nv; dof += a.block) p = fma_(gl[dof], gl[dof], p);
   for (int off = 16; off > 0; off >>= 1) p = p + __shfl_down(p, off, 32);
-  const float second = __shfl(p, 32, 64);
+  float total = 0.0f + __shfl(p, 0, 64);
+  if (a.block > 32) total = total + __shfl(p, 32, 64);
+  sc.grad_dot = total;
+  sc.decrement = 0.0f;
+  sc.grad_scale = 1.0f;
   if (lane == 0) {
-    float total = 0.0f + p;
-    if (a.block > 32) total = total + second;
     a.grad_dot[w] = total;
     a.decrement[w] = 0.0f;
     a.grad_scale[w] = 1.0f;
@@ -249,21 +252,23 @@ __device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, c
 }
 
 // ---- search . search and grad . x of a factor stage that leaves only the search direction -----
-__device__ __forceinline__ void search_sums_world(const NewtonArgs &a, int64_t w, int lane) {
+__device__ __forceinline__ void search_sums_world(const NewtonArgs &a, int64_t w, const float *gl, Scalars &sc, int lane) {
   float s0 = 0.0f, s1 = 0.0f;
   for (int d = lane; d < a.nv && lane < a.block; d += a.block) {
     const float v = -a.search[w * a.nv + d];
     s0 = fma_(v, v, s0);
-    s1 = fma_(a.grad[w * a.ld_grad + d], v, s1);
+    s1 = fma_(gl[d], v, s1);
   }
   for (int o = 16; o > 0; o >>= 1) {
     s0 = s0 + __shfl_down(s0, o, 32);
     s1 = s1 + __shfl_down(s1, o, 32);
   }
   const float a1 = __shfl(s0, 32, 64), b1 = __shfl(s1, 32, 64);
+  float ra = 0.0f + __shfl(s0, 0, 64), rb = 0.0f + __shfl(s1, 0, 64);
+  if (a.block > 32) ra = ra + a1, rb = rb + b1;
+  sc.search_dot = ra;
+  sc.decrement = rb;
   if (lane == 0) {
-    float ra = 0.0f + s0, rb = 0.0f + s1;
-    if (a.block > 32) ra = ra + a1, rb = rb + b1;
     a.search_dot[w] = ra;
     a.decrement[w] = rb;
   }
@@ -273,7 +278,7 @@ __device__ __forceinline__ void search_sums_world(const NewtonArgs &a, int64_t w
 // The same chain per row as jv_world: the dofs in order, the 20-dof partial sums of the reference's
 // rule beyond 50 dofs.  A lane loads 16 elements per tile, four rows of 64 bytes per instruction.
 __device__ __forceinline__ void jv_world_tiled(const NewtonArgs &a, const float *Jw, int nefc, float *tile,
-                                               const float *sv, float *jv, int lane) {
+                                               const float *sv, float *jv, float *jv_lds, int lane) {
   const int nv = a.nv;
   const int c = lane & 15, rq = lane >> 4;
   const bool split = nv > 50;
@@ -303,7 +308,11 @@ __device__ __forceinline__ void jv_world_tiled(const NewtonArgs &a, const float 
       }
       wave_sync();  // the tile is read before the next one overwrites it
     }
-    if (lane < rows) jv[r0 + lane] = split ? acc + p : p;
+    if (lane < rows) {
+      const float out = split ? acc + p : p;
+      jv[r0 + lane] = out;
+      jv_lds[r0 + lane] = out;
+    }
   }
 }
 
@@ -313,23 +322,48 @@ struct LoopLds {
   int *votes;            // [4] cooperative stage only
   const uint32_t *term;  // [nterm] col | madr << 16, shared by the workgroup
   const int *radr;       // [nv + 1]
-  float *m_lds;          // per wavefront: [nM] the world's row of M
+  // per wavefront, kept from round to round:
+  float *m_lds;          // [nM] the world's row of M
   float *sv;             // [nv] the search direction
+  float *Ma, *mv;        // [nv] each
+  float *Jaref, *jv;     // [njmax] each
+  float *D, *fl;         // [njmax] each: the rows' weights and friction losses (read at every step of the line search)
+  // per wavefront, used within a round (may share one area with the factor stage's own arrays):
   float *f;              // [njmax] forces of the listed rows
   int *rowl;             // [njmax] their numbers
-  float *gl;             // [nv] the gradient
+  float *gl;             // [nv] the gradient (a cooperative stage's loop reads it again after the stage)
   float *rows;           // staged rows of J: 64 x (nv | 1), or the 64 x 17 tile
 };
 
-// HELD: rows of a world a lane keeps in registers during the line search (0: read at every
+// A world's vectors stay in LDS and its scalars in registers from round to round; memory receives
+// every value as it is produced (the arrays end as after the stage launches) and is read again only
+// for what another wavefront or the factor stage has written there.
+// HELD: rows of a world a lane keeps in registers during the line search (0: read from LDS at every
 // evaluation); JU: loads in flight per lane while rows of J are staged, 0 for the tiled staging.
 // COOP: `stage()` works on the workgroup's four worlds together (every wavefront calls it in step,
 // between two workgroup barriers; it skips the worlds whose `unchanged` byte is set), and a world
 // that is done idles through the barriers until the workgroup's last world finishes.  Otherwise
-// `stage()` is the wavefront's own world's stage, called only when that world needs it, and a
-// wavefront leaves as soon as its world is done.  `w_raw`: the wavefront's world.
+// `stage()` is the wavefront's own world's stage (it leaves search_dot and newton_decrement in
+// memory itself), called only when that world needs it, and a wavefront leaves as soon as its world
+// is done.  `w_raw`: the wavefront's world.
+//
+// `kernarg_offset`: where the kernel's NewtonArgs parameter lies in its kernel-argument segment.  The
+// loop reads the arguments from there, through a pointer it launders once per round: about sixty
+// pointers cannot stay in scalar registers across the stages (held, they are spilled to vector
+// lanes and read back one by one), and from the segment each is one scalar load next to its use.
+typedef const NewtonArgs __attribute__((address_space(4))) KernelNewtonArgs;
+__device__ __forceinline__ const NewtonArgs &kernel_args(int kernarg_offset) {
+  const char __attribute__((address_space(4))) *seg =
+      (const char __attribute__((address_space(4))) *)__builtin_amdgcn_kernarg_segment_ptr();
+  KernelNewtonArgs *ap = (KernelNewtonArgs *)(seg + kernarg_offset);
+  asm volatile("" : "+s"(ap));
+  return *(const NewtonArgs *)ap;
+}
+
 template <int HELD, int JU, bool COOP, class Stage>
-__device__ __forceinline__ void newton_loop(const NewtonArgs &a, const LoopLds &L, int64_t w_raw, Stage &&stage) {
+__device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L, int64_t w_raw, Stage &&stage) {
+  const NewtonArgs &a0 = kernel_args(kernarg_offset);
+  const NewtonArgs &a = a0;
   const int lane_fixed = threadIdx.x & 63;
   const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   // the world's number as a scalar: every address below is a scalar base plus a lane offset
@@ -338,17 +372,31 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, const LoopLds &
   const bool live = w_uniform < a.nworld;
   const int64_t w = live ? w_uniform : (int64_t)a.nworld - 1;
   const int nv = a.nv, njmax = a.njmax;
-  for (int k = lane_fixed; k < a.nM; k += 64) L.m_lds[k] = a.M[w * a.ldM + k];
   bool done = !live || a.done[w] != 0;
   if (live && done && lane_fixed == 0) a.unchanged[w] = 1;  // the factor stage leaves such a world alone
   bool unchanged = !done && a.unchanged[w] != 0;
   int nefc = a.nefc ? a.nefc[w] : njmax;
   nefc = __builtin_amdgcn_readfirstlane(nefc < njmax ? nefc : njmax);
+  const int ne = __builtin_amdgcn_readfirstlane(a.ne ? a.ne[w] : 0), nf = __builtin_amdgcn_readfirstlane(a.nf ? a.nf[w] : 0);
   const float *Jw = a.J + w * (int64_t)njmax * nv;
-  search::SearchArgs sa{a.tolerance, a.ls_tolerance, a.meaninertia, a.ntolerance, a.nls_tolerance, a.nmeaninertia, a.ne, a.nf,
-                        a.nefc, a.smooth, a.D, a.frictionloss, a.Jaref, a.search, a.search_dot, a.mv, a.jv, a.Ma, nv, njmax,
-                        njmax, njmax, nv, nv, njmax, nv, nullptr, a.alpha, a.improvement, a.exhausted, a.overflow,
-                        a.ls_overflow_bit, nv, njmax, a.ls_iterations, a.nworld};
+  const float tolerance = a.tolerance[w % a.ntolerance], ls_tolerance = a.ls_tolerance[w % a.nls_tolerance];
+  const float meaninertia = a.meaninertia[w % a.nmeaninertia];
+  Scalars sc{a.search_dot[w], a.grad_dot[w], a.decrement[w], a.grad_scale[w], a.alpha[w], a.improvement[w], a.niter[w]};
+  // what the loop keeps: M, Ma, Jaref into LDS (mv and jv are formed before they are read: a world
+  // enters with a new search direction unless it is done), qacc in registers (dofs lane and lane + 64)
+  for (int k = lane_fixed; k < a.nM; k += 64) L.m_lds[k] = a.M[w * a.ldM + k];
+  for (int k = lane_fixed; k < nv; k += 64) {
+    L.Ma[k] = a.Ma[w * nv + k];
+    L.mv[k] = a.mv[w * nv + k];
+  }
+  for (int r = lane_fixed; r < njmax; r += 64) {
+    L.Jaref[r] = a.Jaref[w * njmax + r];
+    L.jv[r] = a.jv[w * njmax + r];
+    L.D[r] = a.D[w * njmax + r];
+    L.fl[r] = a.frictionloss ? a.frictionloss[w * njmax + r] : 0.0f;
+  }
+  float qacc0 = lane_fixed < nv ? a.qacc[w * nv + lane_fixed] : 0.0f;
+  float qacc1 = lane_fixed + 64 < nv ? a.qacc[w * nv + lane_fixed + 64] : 0.0f;
   wave_sync();
 #ifdef IM_NEWTON_STAMPS  // development aid: time per phase, summed over the rounds, left in the world's row of jv
   long long t_phase[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t_last = wall_clock64();
@@ -357,7 +405,9 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, const LoopLds &
 #define IM_STAMP(k) do {} while (0)
 #endif
   // every wavefront leaves the loop after at most maxiter rounds, whatever the data
-  for (int round = 0; round < a.maxiter; ++round) {
+  const int maxiter = a0.maxiter;
+  for (int round = 0; round < maxiter; ++round) {
+    const NewtonArgs &a = kernel_args(kernarg_offset);  // read afresh in every round
     if (COOP) {
       if (lane_fixed == 0) L.votes[wv] = done ? 0 : 1;
       block_sync();
@@ -374,32 +424,86 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, const LoopLds &
       if (!unchanged) {
         for (int k = lane; k < nv; k += 64) L.sv[k] = a.search[w * nv + k];
         wave_sync();
-        mul_m_world(a, L.term, L.radr, L.m_lds, L.sv, a.mv + w * nv, lane);
+        mul_m_world(a, L.term, L.radr, L.m_lds, L.sv, a.mv + w * nv, L.mv, lane);
         if constexpr (JU > 0)
-          jv_world<(JU > 0 ? JU : 1)>(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, lane);
+          jv_world<(JU > 0 ? JU : 1)>(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, L.jv, lane);
         else
-          jv_world_tiled(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, lane);
+          jv_world_tiled(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, L.jv, lane);
         wave_sync();
       }
       IM_STAMP(1);
-      search::linesearch_world<HELD>(sa, w, lane & 31);
-      wave_sync();
+      const search::LsWorld lw{a.smooth + w * nv, L.D, L.fl, L.Jaref, L.sv, L.mv, L.jv, L.Ma, sc.search_dot, tolerance,
+                               ls_tolerance, meaninertia, ne, nf, nefc, nv, a.ls_iterations};
+      const search::LsResult ls = search::linesearch_rows<HELD>(lw, lane & 31);
+      sc.alpha = ls.alpha, sc.improvement = ls.improvement;
+      if (lane == 0) {
+        a.alpha[w] = ls.alpha;
+        a.improvement[w] = ls.improvement;
+        a.exhausted[w] = ls.exhausted ? 1 : 0;
+        if (!ls.converged && a.overflow) a.overflow[w] = a.overflow[w] | a.ls_overflow_bit;
+      }
       IM_STAMP(2);
-      {  // the step (newton_stages.py:373-381)
-        const float al = a.alpha[w];
-        for (int i = lane; i < nv; i += 64) {
-          a.qacc[w * nv + i] = fma_(al, a.search[w * nv + i], a.qacc[w * nv + i]);
-          a.Ma[w * nv + i] = fma_(al, a.mv[w * nv + i], a.Ma[w * nv + i]);
+      // the step (newton_stages.py:373-381), then force and state of every row from the new Jaref, the
+      // rows whose being quadratic flipped (ascending) and the two counts (:385-444); the rows with a
+      // force are listed for the gradient as they are formed
+      const float al = ls.alpha;
+      qacc0 = lane < nv ? fma_(al, L.sv[lane < nv ? lane : 0], qacc0) : qacc0;
+      qacc1 = lane + 64 < nv ? fma_(al, L.sv[lane + 64 < nv ? lane + 64 : 0], qacc1) : qacc1;
+      if (lane < nv) a.qacc[w * nv + lane] = qacc0;
+      if (lane + 64 < nv) a.qacc[w * nv + lane + 64] = qacc1;
+      for (int i = lane; i < nv; i += 64) {
+        const float v = fma_(al, L.mv[i], L.Ma[i]);
+        L.Ma[i] = v;
+        a.Ma[w * nv + i] = v;
+      }
+      int nquad = 0, nstate = 0, cnt = 0;
+      for (int base = 0; base < nefc; base += 64) {
+        const int r = base + lane;
+        bool quad_flip = false, changed = false;
+        float f = 0.0f;
+        if (r < nefc) {
+          const float x = L.Jaref[r] + al * L.jv[r], d = L.D[r];
+          L.Jaref[r] = x;
+          a.Jaref[w * njmax + r] = x;
+          f = -d * x;
+          int st = 1;
+          if (r >= ne && r < ne + nf) {
+            const float fr = L.fl[r], rf = search::safe_div(fr, d);
+            if (x <= -rf) f = fr, st = 2;
+            else if (x >= rf) f = -fr, st = 3;
+          } else if (r >= ne && x >= 0.0f) {
+            f = 0.0f, st = 0;
+          }
+          const int old = a.state[w * njmax + r];
+          a.force[w * njmax + r] = f;
+          a.state[w * njmax + r] = st;
+          quad_flip = (old == 1) != (st == 1);
+          changed = old != st;
         }
-        for (int i = lane; i < nefc; i += 64) a.Jaref[w * njmax + i] = a.Jaref[w * njmax + i] + al * a.jv[w * njmax + i];
+        const unsigned long long below = (1ull << lane) - 1ull;
+        const unsigned long long m = __ballot(quad_flip);
+        if (quad_flip) {
+          const int slot = nquad + __popcll(m & below);
+          if (slot < a.ld_ids) a.ids[w * (int64_t)a.ld_ids + slot] = r;
+        }
+        nquad += __popcll(m);
+        nstate += __popcll(__ballot(changed));
+        const unsigned long long mf = __ballot(f != 0.0f);
+        if (f != 0.0f) {
+          const int pos = cnt + __popcll(mf & below);
+          L.f[pos] = f;
+          L.rowl[pos] = r;
+        }
+        cnt += __popcll(mf);
+      }
+      nstate += ls.exhausted ? 1 : 0;
+      if (lane == 0) {
+        a.quad_count[w] = nquad;
+        a.state_count[w] = nstate;
       }
       wave_sync();
-      search::eval_constraints_world(a.Jaref, njmax, a.D, njmax, a.frictionloss, njmax, a.ne, a.nf, a.nefc, njmax,
-                                     a.exhausted, a.force, njmax, a.state, njmax, a.ids, a.ld_ids, a.quad_count,
-                                     a.state_count, w, lane);
-      wave_sync();
       IM_STAMP(3);
-      unchanged = gradient_world(a, w, Jw, nefc, L.f, L.rowl, L.gl, lane);
+      unchanged = gradient_world(a, w, Jw, nstate != 0, cnt, L.f, L.rowl, L.Ma, L.gl, sc, lane);
       IM_STAMP(4);
     }
     if (COOP) {
@@ -409,37 +513,43 @@ __device__ __forceinline__ void newton_loop(const NewtonArgs &a, const LoopLds &
       block_sync();  // the four search directions are complete
     } else {
       wave_sync();
-      if (!unchanged) stage();
+      if (!done && !unchanged) stage();
       wave_sync();
     }
     IM_STAMP(6);
     lane = lane_fixed;
     asm volatile("" : "+v"(lane));  // no address from before the stage is kept through it
     if (!done) {
-      if (COOP && !unchanged) search_sums_world(a, w, lane);  // a stage of its own leaves the two sums itself
-      wave_sync();
-      int finished = 0;
-      if (lane == 0) {  // newton_fusion.py:265-296
-        const int it = a.niter[w] + 1;
-        a.niter[w] = it;
-        const float tol = a.tolerance[w % a.ntolerance], scale = a.meaninertia[w % a.nmeaninertia] * (float)nv;
-        const float imp = a.improvement[w];
-        const bool converged = a.alpha[w] == 0.0f || (imp > 0.0f && imp / scale < tol) ||
-                               sqrtf(a.grad_dot[w]) / scale < tol || 0.5f * a.decrement[w] / scale < tol;
-        if (converged || it == a.maxiter) {
+      const NewtonArgs &a = kernel_args(kernarg_offset);
+      if (!unchanged) {
+        if (COOP) {
+          search_sums_world(a, w, L.gl, sc, lane);
+        } else {  // the stage has left the two sums in memory
+          sc.search_dot = a.search_dot[w];
+          sc.decrement = a.decrement[w];
+        }
+      }
+      // newton_fusion.py:265-296
+      sc.niter += 1;
+      const float scale = meaninertia * (float)nv;
+      const bool converged = sc.alpha == 0.0f || (sc.improvement > 0.0f && sc.improvement / scale < tolerance) ||
+                             sqrtf(sc.grad_dot) / scale < tolerance || 0.5f * sc.decrement / scale < tolerance;
+      const bool finished = converged || sc.niter == a.maxiter;
+      if (lane == 0) {
+        a.niter[w] = sc.niter;
+        if (finished) {
           if (!converged && a.overflow) a.overflow[w] = a.overflow[w] | a.iter_overflow_bit;
           a.done[w] = 1;
           a.unchanged[w] = 1;
           if (a.nsolving) atomicAdd(a.nsolving, -1);
-          finished = 1;
         }
       }
-      done = __builtin_amdgcn_readfirstlane(finished) != 0;
+      done = finished;
     }
     IM_STAMP(7);
   }
 #ifdef IM_NEWTON_STAMPS
-  if (live && lane_fixed < 8) a.jv[w * njmax + lane_fixed] = (float)t_phase[lane_fixed];
+  if (live && lane_fixed < 8) a0.jv[w * njmax + lane_fixed] = (float)t_phase[lane_fixed];
 #endif
 #undef IM_STAMP
 }
@@ -454,14 +564,20 @@ __device__ __forceinline__ LoopLds coop_layout(const NewtonArgs &a, float *lds) 
   L.votes = (int *)(lds + a.stage_lds_floats);
   uint32_t *term = (uint32_t *)(L.votes + 4);
   int *radr = (int *)(term + a.nterm);
-  float *mine = (float *)(radr + nv + 1) + wv * (nM + nv + 2 * njmax + nv + 64);
+  float *mine = (float *)(radr + nv + 1) + wv * (kept_words(nv, njmax, nM) + 2 * njmax + nv);
   L.term = term, L.radr = radr;
   L.m_lds = mine;
   L.sv = L.m_lds + nM;
-  L.f = L.sv + nv;
+  L.Ma = L.sv + nv;
+  L.mv = L.Ma + nv;
+  L.Jaref = L.mv + nv;
+  L.jv = L.Jaref + njmax;
+  L.D = L.jv + njmax;
+  L.fl = L.D + njmax;
+  L.f = L.fl + njmax;
   L.rowl = (int *)(L.f + njmax);
   L.gl = (float *)(L.rowl + njmax);
-  L.rows = lds + wv * (64 * (nv | 1));
+  L.rows = lds + wv * (64 * 17);
   for (int k = threadIdx.x; k < a.nterm; k += blockDim.x) term[k] = (uint32_t)a.mulm_col[k] | (uint32_t)a.mulm_madr[k] << 16;
   for (int k = threadIdx.x; k <= nv; k += blockDim.x) radr[k] = a.mulm_rowadr[k];
   return L;

@@ -843,7 +843,7 @@ __host__ __device__ inline int resident_area_words(int nslots, int n, int block,
   words = words > grad ? words : grad;
   return (words + 3) & ~3;
 }
-template <int WAVES>
+template <int WAVES, int HELD>
 __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident_kernel(
     SparseWave A, resident::NewtonArgs a, float *__restrict__ U_, int32_t *__restrict__ uni_) {
   extern __shared__ float lds[];
@@ -855,7 +855,7 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
   uint32_t *term = (uint32_t *)(lds + A.staged_words + A.solve_words);
   int *radr = (int *)(term + a.nterm);
   const int area = resident_area_words(Q.nslots, nv, A.block, njmax);
-  float *mine = (float *)(radr + nv + 1) + wv * (area + a.nM + nv);
+  float *mine = (float *)(radr + nv + 1) + wv * (area + resident::kept_words(nv, njmax, a.nM));
   resident::LoopLds L;
   L.votes = nullptr;
   L.term = term, L.radr = radr;
@@ -865,20 +865,25 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
   L.gl = mine + 2 * njmax;
   L.m_lds = mine + area;
   L.sv = L.m_lds + a.nM;
+  L.Ma = L.sv + nv;
+  L.mv = L.Ma + nv;
+  L.Jaref = L.mv + nv;
+  L.jv = L.Jaref + njmax;
+  L.D = L.jv + njmax;
+  L.fl = L.D + njmax;
   for (int k = tid; k < a.nterm; k += 64 * WAVES) term[k] = (uint32_t)a.mulm_col[k] | (uint32_t)a.mulm_madr[k] << 16;
   for (int k = tid; k <= nv; k += 64 * WAVES) radr[k] = a.mulm_rowadr[k];
   __syncthreads();  // the only workgroup barrier
   const int64_t w = (int64_t)blockIdx.x * WAVES + wv;
+  // NewtonArgs is the kernel's second parameter, behind the plan's block
+  constexpr int kArgsOffset = (int)((sizeof(SparseWave) + alignof(resident::NewtonArgs) - 1) / alignof(resident::NewtonArgs) *
+                                    alignof(resident::NewtonArgs));
   auto stage = [&]() __attribute__((always_inline)) {
-    sparse_update_world(A, Q, mine, a.quad_count, a.ids, a.ld_ids, a.J, njmax, a.D, a.state, a.quad, a.grad,
-                        (int)a.ld_grad, U_, uni_, a.search, a.search_dot, a.decrement, (int)w, threadIdx.x & 63);
+    const resident::NewtonArgs &b = resident::kernel_args(kArgsOffset);
+    sparse_update_world(A, Q, mine, b.quad_count, b.ids, b.ld_ids, b.J, b.njmax, b.D, b.state, b.quad, b.grad,
+                        (int)b.ld_grad, U_, uni_, b.search, b.search_dot, b.decrement, (int)w, threadIdx.x & 63);
   };
-  if (njmax <= 64)
-    resident::newton_loop<2, 0, false>(a, L, w, stage);
-  else if (njmax <= 128)
-    resident::newton_loop<4, 0, false>(a, L, w, stage);
-  else
-    resident::newton_loop<0, 0, false>(a, L, w, stage);
+  resident::newton_loop<HELD, 0, false>(kArgsOffset, L, w, stage);  // HELD: 2 up to 64 rows, else 0
 }
 
 // Per-iteration factor stage: changed rows' dof union, incremental update of packed H,
@@ -1238,32 +1243,39 @@ int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *p, 
   A.solve_words = (int)solve_words;
   if (staged > 8192 || solve_words > 4096) return IM_ERR_UNSUPPORTED;
   const size_t shared = staged + solve_words + (size_t)p->nterm + n + 1;
-  const size_t per_wave = (size_t)im::resident_area_words(plan->nslots, n, plan->block, njmax) + nM + n;
+  const size_t per_wave = (size_t)im::resident_area_words(plan->nslots, n, plan->block, njmax) + im::resident::kept_words(n, njmax, nM);
   // the most worlds per workgroup (one workgroup per CU) that 160 KB of LDS admit and whose kernel
   // keeps to registers
   struct Variant {
-    int waves;
+    int waves, held;
     const void *fn;
   };
-  static const Variant variants[] = {{16, (const void *)im::newton_sparse_resident_kernel<16>},
-                                     {12, (const void *)im::newton_sparse_resident_kernel<12>},
-                                     {8, (const void *)im::newton_sparse_resident_kernel<8>},
-                                     {4, (const void *)im::newton_sparse_resident_kernel<4>}};
-  static bool usable[4] = {false, false, false, false};
+  // the line search keeps a lane's two rows in registers up to 64 rows and reads them from LDS beyond
+  static const Variant variants[] = {{16, 2, (const void *)im::newton_sparse_resident_kernel<16, 2>},
+                                     {12, 2, (const void *)im::newton_sparse_resident_kernel<12, 2>},
+                                     {8, 2, (const void *)im::newton_sparse_resident_kernel<8, 2>},
+                                     {4, 2, (const void *)im::newton_sparse_resident_kernel<4, 2>},
+                                     {16, 0, (const void *)im::newton_sparse_resident_kernel<16, 0>},
+                                     {12, 0, (const void *)im::newton_sparse_resident_kernel<12, 0>},
+                                     {8, 0, (const void *)im::newton_sparse_resident_kernel<8, 0>},
+                                     {4, 0, (const void *)im::newton_sparse_resident_kernel<4, 0>}};
+  constexpr int kVariants = 8;
+  static bool usable[kVariants] = {};
   static bool probed = false;
   if (!probed) {  // once per process: register spills and the grant of the large dynamic LDS
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kVariants; ++i) {
       hipFuncAttributes fa{};
-      usable[i] = hipFuncGetAttributes(&fa, variants[i].fn) == hipSuccess && fa.localSizeBytes == 0 &&
+      // (a variant that parks more than a few values of its prologue in memory is left out)
+      usable[i] = hipFuncGetAttributes(&fa, variants[i].fn) == hipSuccess && fa.localSizeBytes <= 16 &&
                   hipFuncSetAttribute(variants[i].fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                       160 * 1024 - (int)fa.sharedSizeBytes) == hipSuccess;
       (void)hipGetLastError();
     }
     probed = true;
   }
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < kVariants; ++i) {
     const size_t lds = 4 * (shared + (size_t)variants[i].waves * per_wave);
-    if (!usable[i] || lds > 158 * 1024) continue;
+    if (!usable[i] || lds > 158 * 1024 || variants[i].held != (njmax <= 64 ? 2 : 0)) continue;
     const int waves = variants[i].waves;
     void *args[] = {&A, &a, &hfactor, &dof_union};
     IM_HIP_CHECK(hipLaunchKernel(variants[i].fn, dim3((unsigned)((p->nworld + waves - 1) / waves)), dim3(64 * waves), args,
