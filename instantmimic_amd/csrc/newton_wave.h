@@ -81,6 +81,10 @@ inline int convert_args(const im_newton_args &p, int nv, int nM, NewtonArgs &a) 
 }
 
 __device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+// a value every lane holds alike, as a scalar (so that it occupies no vector register while it waits)
+__device__ __forceinline__ float uniform(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+}
 
 // orders this wavefront's writes (LDS and memory) before its later reads: the stages hand their
 // results on through memory, written by some lanes and read by others
@@ -100,8 +104,8 @@ __device__ __forceinline__ void block_sync() {
 // direction, Ma, mv, Jaref, jv, D and the friction losses, the gradient's list of rows with a force
 // (value and row number) and its copy of the gradient.  The factor stage's area must also hold four wavefronts'
 // staged tiles of J: 4 x 64 rows x 16 dofs, a row 17 words.
-// words a wavefront keeps from round to round: M, the search direction, Ma, mv; Jaref, jv, D, friction losses
-__host__ __device__ inline size_t kept_words(int nv, int njmax, int nM) { return (size_t)nM + 3 * (size_t)nv + 4 * (size_t)njmax; }
+// words a wavefront keeps from round to round: M, the search direction, Ma, mv, qacc; Jaref, jv, D, friction losses
+__host__ __device__ inline size_t kept_words(int nv, int njmax, int nM) { return (size_t)nM + 4 * (size_t)nv + 4 * (size_t)njmax; }
 __host__ __device__ inline size_t loop_lds_words(int nv, int njmax, int nM, int nterm) {
   return 4 + (size_t)nterm + nv + 1 + 4 * (kept_words(nv, njmax, nM) + 2 * (size_t)njmax + nv);
 }
@@ -202,9 +206,9 @@ __device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, c
     float ratio = 0.0f;
     if (sigma != 0.0f) ratio = new_sigma / sigma;
     const float ratio_sq = ratio * ratio;
-    sc.grad_dot = sc.grad_dot * ratio_sq;
-    sc.decrement = sc.decrement * ratio_sq;
-    sc.grad_scale = new_sigma;
+    sc.grad_dot = uniform(sc.grad_dot * ratio_sq);
+    sc.decrement = uniform(sc.decrement * ratio_sq);
+    sc.grad_scale = uniform(new_sigma);
     if (lane == 0) {
       a.grad_dot[w] = sc.grad_dot;
       a.decrement[w] = sc.decrement;
@@ -214,7 +218,10 @@ __device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, c
     return true;
   }
   const int nv = a.nv;
-  constexpr int ROWS = 16;
+#ifndef IM_GRADIENT_ROWS
+#define IM_GRADIENT_ROWS 16
+#endif
+  constexpr int ROWS = IM_GRADIENT_ROWS;
   for (int dof = lane; dof < nv; dof += 64) {
     const float ma = Ma_l[dof], sm = a.smooth[w * nv + dof];
     float sum = 0.0f;
@@ -239,7 +246,7 @@ __device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, c
   for (int off = 16; off > 0; off >>= 1) p = p + __shfl_down(p, off, 32);
   float total = 0.0f + __shfl(p, 0, 64);
   if (a.block > 32) total = total + __shfl(p, 32, 64);
-  sc.grad_dot = total;
+  sc.grad_dot = uniform(total);
   sc.decrement = 0.0f;
   sc.grad_scale = 1.0f;
   if (lane == 0) {
@@ -266,8 +273,8 @@ __device__ __forceinline__ void search_sums_world(const NewtonArgs &a, int64_t w
   const float a1 = __shfl(s0, 32, 64), b1 = __shfl(s1, 32, 64);
   float ra = 0.0f + __shfl(s0, 0, 64), rb = 0.0f + __shfl(s1, 0, 64);
   if (a.block > 32) ra = ra + a1, rb = rb + b1;
-  sc.search_dot = ra;
-  sc.decrement = rb;
+  sc.search_dot = uniform(ra);
+  sc.decrement = uniform(rb);
   if (lane == 0) {
     a.search_dot[w] = ra;
     a.decrement[w] = rb;
@@ -325,7 +332,7 @@ struct LoopLds {
   // per wavefront, kept from round to round:
   float *m_lds;          // [nM] the world's row of M
   float *sv;             // [nv] the search direction
-  float *Ma, *mv;        // [nv] each
+  float *Ma, *mv, *qacc; // [nv] each
   float *Jaref, *jv;     // [njmax] each
   float *D, *fl;         // [njmax] each: the rows' weights and friction losses (read at every step of the line search)
   // per wavefront, used within a round (may share one area with the factor stage's own arrays):
@@ -381,13 +388,15 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
   const float *Jw = a.J + w * (int64_t)njmax * nv;
   const float tolerance = a.tolerance[w % a.ntolerance], ls_tolerance = a.ls_tolerance[w % a.nls_tolerance];
   const float meaninertia = a.meaninertia[w % a.nmeaninertia];
-  Scalars sc{a.search_dot[w], a.grad_dot[w], a.decrement[w], a.grad_scale[w], a.alpha[w], a.improvement[w], a.niter[w]};
+  Scalars sc{uniform(a.search_dot[w]), uniform(a.grad_dot[w]), uniform(a.decrement[w]), uniform(a.grad_scale[w]),
+             uniform(a.alpha[w]), uniform(a.improvement[w]), __builtin_amdgcn_readfirstlane(a.niter[w])};
   // what the loop keeps: M, Ma, Jaref into LDS (mv and jv are formed before they are read: a world
-  // enters with a new search direction unless it is done), qacc in registers (dofs lane and lane + 64)
+  // enters with a new search direction unless it is done) and qacc
   for (int k = lane_fixed; k < a.nM; k += 64) L.m_lds[k] = a.M[w * a.ldM + k];
   for (int k = lane_fixed; k < nv; k += 64) {
     L.Ma[k] = a.Ma[w * nv + k];
     L.mv[k] = a.mv[w * nv + k];
+    L.qacc[k] = a.qacc[w * nv + k];
   }
   for (int r = lane_fixed; r < njmax; r += 64) {
     L.Jaref[r] = a.Jaref[w * njmax + r];
@@ -395,8 +404,6 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
     L.D[r] = a.D[w * njmax + r];
     L.fl[r] = a.frictionloss ? a.frictionloss[w * njmax + r] : 0.0f;
   }
-  float qacc0 = lane_fixed < nv ? a.qacc[w * nv + lane_fixed] : 0.0f;
-  float qacc1 = lane_fixed + 64 < nv ? a.qacc[w * nv + lane_fixed + 64] : 0.0f;
   wave_sync();
 #ifdef IM_NEWTON_STAMPS  // development aid: time per phase, summed over the rounds, left in the world's row of jv
   long long t_phase[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t_last = wall_clock64();
@@ -435,7 +442,7 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
       const search::LsWorld lw{a.smooth + w * nv, L.D, L.fl, L.Jaref, L.sv, L.mv, L.jv, L.Ma, sc.search_dot, tolerance,
                                ls_tolerance, meaninertia, ne, nf, nefc, nv, a.ls_iterations};
       const search::LsResult ls = search::linesearch_rows<HELD>(lw, lane & 31);
-      sc.alpha = ls.alpha, sc.improvement = ls.improvement;
+      sc.alpha = uniform(ls.alpha), sc.improvement = uniform(ls.improvement);
       if (lane == 0) {
         a.alpha[w] = ls.alpha;
         a.improvement[w] = ls.improvement;
@@ -447,13 +454,11 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
       // rows whose being quadratic flipped (ascending) and the two counts (:385-444); the rows with a
       // force are listed for the gradient as they are formed
       const float al = ls.alpha;
-      qacc0 = lane < nv ? fma_(al, L.sv[lane < nv ? lane : 0], qacc0) : qacc0;
-      qacc1 = lane + 64 < nv ? fma_(al, L.sv[lane + 64 < nv ? lane + 64 : 0], qacc1) : qacc1;
-      if (lane < nv) a.qacc[w * nv + lane] = qacc0;
-      if (lane + 64 < nv) a.qacc[w * nv + lane + 64] = qacc1;
       for (int i = lane; i < nv; i += 64) {
-        const float v = fma_(al, L.mv[i], L.Ma[i]);
+        const float q = fma_(al, L.sv[i], L.qacc[i]), v = fma_(al, L.mv[i], L.Ma[i]);
+        L.qacc[i] = q;
         L.Ma[i] = v;
+        a.qacc[w * nv + i] = q;
         a.Ma[w * nv + i] = v;
       }
       int nquad = 0, nstate = 0, cnt = 0;
@@ -525,8 +530,8 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
         if (COOP) {
           search_sums_world(a, w, L.gl, sc, lane);
         } else {  // the stage has left the two sums in memory
-          sc.search_dot = a.search_dot[w];
-          sc.decrement = a.decrement[w];
+          sc.search_dot = uniform(a.search_dot[w]);
+          sc.decrement = uniform(a.decrement[w]);
         }
       }
       // newton_fusion.py:265-296
@@ -570,7 +575,8 @@ __device__ __forceinline__ LoopLds coop_layout(const NewtonArgs &a, float *lds) 
   L.sv = L.m_lds + nM;
   L.Ma = L.sv + nv;
   L.mv = L.Ma + nv;
-  L.Jaref = L.mv + nv;
+  L.qacc = L.mv + nv;
+  L.Jaref = L.qacc + nv;
   L.jv = L.Jaref + njmax;
   L.D = L.jv + njmax;
   L.fl = L.D + njmax;

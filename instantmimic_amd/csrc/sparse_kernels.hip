@@ -867,7 +867,8 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
   L.sv = L.m_lds + a.nM;
   L.Ma = L.sv + nv;
   L.mv = L.Ma + nv;
-  L.Jaref = L.mv + nv;
+  L.qacc = L.mv + nv;
+  L.Jaref = L.qacc + nv;
   L.jv = L.Jaref + njmax;
   L.D = L.jv + njmax;
   L.fl = L.D + njmax;
