@@ -926,7 +926,9 @@ int im_newton_solve_tree(const im_tree_plan *plan, const im_newton_args *args, v
  * tables in LDS; a wavefront leaves as soon as its world is done.  args->block must be the plan's
  * block width.  The arrays end as after im_sparse_update_factor and the other stage launches
  * repeated, bit for bit.  nv <= 64 (IM_ERR_UNSUPPORTED beyond, and where no variant of the kernel
- * fits the LDS: the caller then issues the stages one by one). */
+ * fits the LDS: the caller then issues the stages one by one).  The launch holds as many
+ * wavefronts as the chip keeps resident and hands a finished wavefront the next world through a
+ * counter that belongs to the plan: two solves with one plan must not overlap on the GPU. */
 int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *args, float *hfactor,
                            int32_t *dof_union, void *stream);
 

@@ -845,13 +845,14 @@ __host__ __device__ inline int resident_area_words(int nslots, int n, int block,
 }
 template <int WAVES, int HELD>
 __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident_kernel(
-    SparseWave A, resident::NewtonArgs a, float *__restrict__ U_, int32_t *__restrict__ uni_) {
+    SparseWave A, resident::NewtonArgs a, float *__restrict__ U_, int32_t *__restrict__ uni_,
+    int *__restrict__ next_world) {
   extern __shared__ float lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   SparseDev Q = A.P;
   stage_update_tables<64 * WAVES>(A, Q, lds, tid);
-  const int nv = a.nv, njmax = a.njmax;
+  const int nv = a.nv, njmax = a.njmax, nworld = a.nworld;
   uint32_t *term = (uint32_t *)(lds + A.staged_words + A.solve_words);
   int *radr = (int *)(term + a.nterm);
   const int area = resident_area_words(Q.nslots, nv, A.block, njmax);
@@ -875,7 +876,11 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
   for (int k = tid; k < a.nterm; k += 64 * WAVES) term[k] = (uint32_t)a.mulm_col[k] | (uint32_t)a.mulm_madr[k] << 16;
   for (int k = tid; k <= nv; k += 64 * WAVES) radr[k] = a.mulm_rowadr[k];
   __syncthreads();  // the only workgroup barrier
-  const int64_t w = (int64_t)blockIdx.x * WAVES + wv;
+  // The grid holds as many wavefronts as the chip keeps resident; a wavefront whose world is done
+  // takes the next world nobody has started (a counter in memory, set to the grid's wavefront count
+  // before the launch), so the worlds that need many iterations do not hold idle neighbours in
+  // place.  The counter only grows: every wavefront reaches the end of the batch.
+  int64_t w = (int64_t)blockIdx.x * WAVES + wv;
   // NewtonArgs is the kernel's second parameter, behind the plan's block
   constexpr int kArgsOffset = (int)((sizeof(SparseWave) + alignof(resident::NewtonArgs) - 1) / alignof(resident::NewtonArgs) *
                                     alignof(resident::NewtonArgs));
@@ -884,8 +889,15 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
     sparse_update_world(A, Q, mine, b.quad_count, b.ids, b.ld_ids, b.J, b.njmax, b.D, b.state, b.quad, b.grad,
                         (int)b.ld_grad, U_, uni_, b.search, b.search_dot, b.decrement, (int)w, threadIdx.x & 63);
   };
-  resident::newton_loop<HELD, 0, false>(kArgsOffset, L, w, stage);  // HELD: 2 up to 64 rows, else 0
+  while (w < nworld) {
+    resident::newton_loop<HELD, 0, false>(kArgsOffset, L, w, stage);  // HELD: 2 up to 64 rows, else 0
+    int next = 0;
+    if ((threadIdx.x & 63) == 0) next = atomicAdd(next_world, 1);
+    w = __builtin_amdgcn_readfirstlane(next);
+  }
 }
+
+__global__ void set_counter_kernel(int *counter, int value) { *counter = value; }
 
 // Per-iteration factor stage: changed rows' dof union, incremental update of packed H,
 // refactor -- or, with no changed row, a forward solve with the stored factor -- then the
@@ -1046,8 +1058,9 @@ int sparse_plan_upload(im_sparse_plan *pl) {
   }
   std::vector<char> host(total, 0);
   for (int i = 0; i < NHOST; ++i) memcpy(host.data() + offs[i], pl->table[i].data(), pl->table[i].size() * 4);
-  IM_HIP_CHECK(hipMalloc(&pl->blob, total));
+  IM_HIP_CHECK(hipMalloc(&pl->blob, total + 16));  // behind the tables: the resident Newton kernel's world counter
   IM_HIP_CHECK(hipMemcpy(pl->blob, host.data(), total, hipMemcpyHostToDevice));
+  pl->next_world = (int *)((char *)pl->blob + total);
   for (int i = 0; i < NHOST; ++i) pl->t[i] = (const int32_t *)((char *)pl->blob + offs[i]);
   if (nv <= 64 && pl->nslots < 65535 && !pl->table[SA].empty()) {
     const int32_t *sa = pl->table[SA].data(), *sb = pl->table[SB].data(), *sm = pl->table[SM].data();
@@ -1278,9 +1291,21 @@ int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *p, 
     const size_t lds = 4 * (shared + (size_t)variants[i].waves * per_wave);
     if (!usable[i] || lds > 158 * 1024 || variants[i].held != (njmax <= 64 ? 2 : 0)) continue;
     const int waves = variants[i].waves;
-    void *args[] = {&A, &a, &hfactor, &dof_union};
-    IM_HIP_CHECK(hipLaunchKernel(variants[i].fn, dim3((unsigned)((p->nworld + waves - 1) / waves)), dim3(64 * waves), args,
-                                 lds, (hipStream_t)stream));
+    // as many workgroups as stay resident at once (LDS, and sixteen wavefronts of up to 128 registers
+    // per CU); the others' worlds are taken up by the wavefronts that finish
+    static int ncu = 0;
+    if (!ncu) {
+      int dev = 0;
+      IM_HIP_CHECK(hipGetDevice(&dev));
+      IM_HIP_CHECK(hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev));
+    }
+    const int per_cu = std::max(1, std::min((int)(160 * 1024 / lds), 16 / waves));
+    const int needed = (p->nworld + waves - 1) / waves;
+    const int grid = std::min(needed, std::max(ncu, 1) * per_cu);
+    int *counter = plan->next_world;
+    hipLaunchKernelGGL(im::set_counter_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, counter, grid * waves);
+    void *args[] = {&A, &a, &hfactor, &dof_union, &counter};
+    IM_HIP_CHECK(hipLaunchKernel(variants[i].fn, dim3((unsigned)grid), dim3(64 * waves), args, lds, (hipStream_t)stream));
     return IM_OK;
   }
   return IM_ERR_UNSUPPORTED;

@@ -36,6 +36,8 @@ struct im_sparse_plan {
   // row of M and which slot it is ((M index + 1) << 16 | (slot + 1)); null when nv > 64
   int32_t *tile_index = nullptr;
   int nM = 0;
+  // one int on the device: the next world of a batch nobody has started (im_newton_solve_sparse)
+  int *next_world = nullptr;
 };
 
 namespace im {
