@@ -1,23 +1,31 @@
-"""The product ``M v`` of the fused Newton kernel on MI355X.
+"""The reference's fused Newton solve on MI355X: ``init_context``, ``run`` and the force recovery.
 
-The reference evaluates it inside its Newton loop, one dof per lane
-(src/instantmimic/utils/mjw_kernels/newton_fusion.py:171-176), from three tables of the
-upstream model (``m.M_mulm_rowadr``, ``m.M_mulm_col``, ``m.M_mulm_madr``, :378-380): for every
-dof the columns of its full symmetric row and where each element sits in M's tree CSR.
-:func:`mul_m` takes those tables as they are; :func:`mul_m_tables` builds them from the CSR
-for a model that does not carry them (ancestors root first, the diagonal, then descendants
-ascending -- the upstream order is not visible from the reference's tree).
+:func:`solve` is the constraint solve as the reference's step issues it
+(src/instantmimic/utils/mjw_step_optimized.py:2588-2683): :func:`init_context`
+(src/instantmimic/utils/mjw_kernels/newton_fusion.py:431-519, with ``_update_gradient_sparse``,
+:480-519), :func:`run` (:330-409) and :func:`qfrc_constraint_from_grad` (:537-555).  Nothing in
+it reads device memory back while the caller's stream is being captured, so a whole solve can be
+one graph of the caller's.
 
-:func:`gradient` is the reference's own ``gradient_function``
-(src/instantmimic/utils/mjw_kernels/newton_stages.py:745-798) and :func:`jv` the ``J v`` step at
-the head of its line search (:157-178); :func:`advance` is the step along the search direction
-at its end (:373-381) and :func:`changed_rows` the listing of the rows whose state changed
-(:403-426), which is what the factor stage of the next iteration takes; :func:`converged` is the
-test that closes an iteration (newton_fusion.py:265-296); :func:`init_empty_worlds` and
-:func:`qfrc_constraint_from_grad` are the two small kernels at the start and the end of the fused
-solve (:412-428, :537-555).  Each runs for all worlds in one launch.  The scalar search itself, the evaluation of the constraints' new states
-and forces and the convergence test are upstream mujoco_warp code and are not part of this
-module.
+:func:`run` takes one of two forms.  Where the context's scratch allows it, the iterations are one
+resident kernel per solve with a wavefront per world, the reference's persistent block
+(:57-298): ``im_newton_solve_tree`` (fused tree stage, plans with generated kernels) or
+``im_newton_solve_sparse`` (static-pattern sparse stage).  Otherwise every iteration is eight
+launches over all worlds (:func:`iteration`), each kernel returning for worlds that are done.
+
+The stages are also callable by themselves.  :func:`mul_m` is the product ``M v`` (:171-176)
+from the three tables of the upstream model (``m.M_mulm_rowadr``, ``m.M_mulm_col``,
+``m.M_mulm_madr``, :378-380); :func:`mul_m_tables` builds them from the CSR for a model that does
+not carry them (ancestors root first, the diagonal, then descendants ascending -- the upstream
+order is not visible from the reference's tree).  :func:`gradient` is ``gradient_function``
+(src/instantmimic/utils/mjw_kernels/newton_stages.py:745-798), :func:`jv` the ``J v`` step at the
+head of the line search (:157-178), :func:`linesearch` its scalar search (:179-372),
+:func:`advance` the step at its end (:373-381), :func:`eval_constraints` the constraints' new
+forces and states (:385-444), :func:`changed_rows` the listing of the rows whose state changed
+(:403-426), :func:`converged` the test that closes an iteration (newton_fusion.py:265-296),
+:func:`init_empty_worlds` the kernel at the start of the solve (:412-428).  The per-row cost of
+the line search and the constraint re-evaluation are upstream mujoco_warp functions that the
+reference's tree does not hold; they are restated from MuJoCo's published primal line search.
 """
 
 from __future__ import annotations
