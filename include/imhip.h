@@ -304,6 +304,36 @@ int im_sparse_dense_factor(const im_sparse_plan *plan, const uint8_t *done, cons
                            float *hfactor, float *search, int ld_search, float *search_dot,
                            float *decrement, int nworld, void *stream);
 
+/* Replaces _tile_cholesky_factorize_solve_no_l_store
+ * (src/instantmimic/utils/mjw_step_optimized.py:672-701, launched from
+ * _factor_solve_i_dense_no_l_store, :839-846): for every world and every tile t, the diagonal
+ * block of tile_size dofs at tile_adr[t] of the dense M (ld_world floats per world, ld_row per
+ * row; its lower triangle is read) is Cholesky-factored and x[w, adr .. adr + size) =
+ * block^-1 y[w, same]; the factor is not kept.  tile_size <= 64 (IM_ERR_UNSUPPORTED beyond);
+ * dofs outside every tile are not written. */
+int im_tile_cholesky_solve(const float *M, int64_t ld_world, int64_t ld_row, const int32_t *tile_adr, int ntile,
+                           int tile_size, const float *y, int64_t ldy, float *x, int64_t ldx, int nworld,
+                           void *stream);
+
+/* Replaces _tile_cholesky_factorize_solve_m_no_l_store (mjw_step_optimized.py:704-750, launched
+ * from :826-836): M holds nM values per world (row stride ldM) and block b's element (r, c) is
+ * M[w, block_elemid[(b tile_size + r) tile_size + c]] (the reference's tile.elemid; an id at or
+ * past nM reads as zero; the upper triangle is read, as fill_mode "upper" does there);
+ * block_dof[b] is the block's first dof in y and x. */
+int im_tile_cholesky_solve_m(const float *M, int64_t ldM, int nM, const int32_t *block_elemid,
+                             const int32_t *block_dof, int nblock, int tile_size, const float *y, int64_t ldy,
+                             float *x, int64_t ldx, int nworld, void *stream);
+
+/* The dense stage below for nv <= 32 (newton_stages.py:723-733): no factor is kept between
+ * iterations; after the update of H the matrix is factored as one tile and solved for the
+ * gradient at every call that state_changes[w] != 0 lets through.  im_dense_update_factor hands
+ * such shapes here itself. */
+int im_dense_update_tile(const uint8_t *done, const int32_t *state_changes, const int32_t *changes,
+                         const int32_t *ids, int ld_ids, const float *J, int njmax, const float *D,
+                         const int32_t *state, int quad, const float *grad, int64_t ldg, float *H, int nv,
+                         int nv_pad, int32_t *dof_union, float *search, int64_t ld_search, float *search_dot,
+                         float *decrement, int nworld, void *stream);
+
 /* The same stage on the dense Hessian (newton_stages.py:614-742 without a sparse plan):
  * H (nworld, nv_pad, nv_pad) receives the deltas on its upper triangle
  * (H[w, row, col] += delta, row <= col, :700-701); with changed rows the augmented blocked
@@ -315,7 +345,8 @@ int im_sparse_dense_factor(const im_sparse_plan *plan, const uint8_t *done, cons
  * above nv (src/instantmimic/utils/mjw_model.py:30).  H and U must be 16-byte aligned
  * (IM_ERR_STRIDE otherwise).  changes[w] < 0: no row is applied and H as it lies in memory is
  * factored -- the first factor of a solve, after the full assembly that upstream's
- * solver._update_gradient makes there (src/instantmimic/utils/mjw_kernels/newton_fusion.py:470). */
+ * solver._update_gradient makes there (src/instantmimic/utils/mjw_kernels/newton_fusion.py:470).
+ * nv <= 32: the single-tile form above (U is neither read nor written). */
 int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes,
                            const int32_t *changes, const int32_t *ids, int ld_ids,
                            const float *J, int njmax, const float *D, const int32_t *state,

@@ -202,6 +202,12 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],
     ),
+    "im_dense_update_tile": (
+        _i,
+        [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],
+    ),
+    "im_tile_cholesky_solve": (_i, [_vp, _i64, _i64, _vp, _i, _i, _vp, _i64, _vp, _i64, _i, _vp]),
+    "im_tile_cholesky_solve_m": (_i, [_vp, _i64, _i, _vp, _vp, _i, _i, _vp, _i64, _vp, _i64, _i, _vp]),
     "im_blocked_factor_solve": (_i, [_vp, _i64, _i, _vp, _i, _i, _i, _vp, _i64, _vp, _vp, _i64, _i, _vp]),
     "im_blocked_index_layout": (_i, [_vp, _i, _i, _i, _vp, _vp]),
     "im_blocked_multi_solve": (_i, [_vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _vp]),

@@ -134,15 +134,115 @@ def _blocked_dense_factor_solve(
             _lib.check(status, "im_copy_dense_factor")
 
 
+def _matrix_tiles(m: Any):
+    return m.M_tiles if hasattr(m, "M_tiles") else m.qM_tiles
+
+
+def _has_m_structure(m: Any, d: Any = None) -> bool:
+    return hasattr(m, "M_tiles") or (d is not None and hasattr(d, "M"))
+
+
+def _has_sparse_m_tail(m: Any, d: Any) -> bool:
+    """Whether an L'DL sparse tail follows the dense blocks of M (:783-787)."""
+    if not hasattr(m, "qLD_block_total"):
+        return bool(getattr(m, "qLD_has_sparse", False))
+    shape = tuple(getattr(d.qLD, "shape", ()))
+    return (int(shape[1]) if len(shape) > 1 else 0) > int(m.qLD_block_total)
+
+
+def _element_count(tile) -> int:
+    elemid = getattr(tile, "elemid", None)
+    if elemid is None:
+        return 0
+    return int(elemid.numel()) if hasattr(elemid, "numel") else int(np.asarray(elemid).size)
+
+
+def _device_ints(a, like):
+    """int32 on ``like``'s device; a host array is uploaded at every call, which a stream capture
+    does not allow: hand over device arrays (the reference's tiles hold them) to be capturable."""
+    import torch
+
+    if isinstance(a, torch.Tensor):
+        return a.to(device=like.device, dtype=torch.int32).contiguous().reshape(-1)
+    return torch.as_tensor(np.ascontiguousarray(np.asarray(a).reshape(-1), np.int32), device=like.device)
+
+
+def _factor_solve_i_dense_no_l_store(m: Any, d: Any, M, x, y, D=None, *, upstream: Callable[..., None] | None = None) -> None:
+    """Dense factor + solve when the factor is not used again (:790-846): one Cholesky tile per
+    dense block of M, gathered through the tile's ``elemid`` where M is stored by its structure
+    (``im_tile_cholesky_solve_m``) or read from the dense (nworld, nv, nv) array
+    (``im_tile_cholesky_solve``).  A sparse tail behind the dense blocks, and M-structure tiles
+    without an ``elemid`` (upstream's small-block kernel, which also writes ``d.qLD``), are
+    upstream mujoco_warp code: ``upstream(False)`` is called for them."""
+    import torch
+
+    nworld = int(d.nworld)
+    structured = _has_m_structure(m, d)
+    tiles = list(_matrix_tiles(m))
+    needs_upstream = structured and (_has_sparse_m_tail(m, d) or any(_element_count(t) == 0 for t in tiles))
+    if needs_upstream:
+        if upstream is None:
+            raise NotImplementedError("a sparse tail or a block without element ids is solved by upstream's factor_solve_i")
+        upstream(False)
+        return
+    for t in (M, x, y):
+        if t.dtype != torch.float32 or not t.is_cuda or t.stride(-1) != 1 or t.device != M.device:
+            raise ValueError("tile solve needs float32 CUDA tensors with contiguous rows on one device")
+    x2, y2 = x.reshape(nworld, -1), y.reshape(nworld, -1)
+    lib = _lib.lib()
+    with torch.cuda.device(M.device):
+        for tile in tiles:
+            adr = _device_ints(tile.adr, M)
+            size = int(tile.size)
+            if structured:
+                if M.dim() != 2 or M.shape[0] != nworld:
+                    raise ValueError("M must be (nworld, nM)")
+                ids = _device_ints(tile.elemid, M)
+                if ids.numel() != adr.numel() * size * size:
+                    raise ValueError("tile.elemid must hold size * size ids per block")
+                status = lib.im_tile_cholesky_solve_m(
+                    M.data_ptr(), M.stride(0), M.shape[1], ids.data_ptr(), adr.data_ptr(), adr.numel(), size,
+                    y2.data_ptr(), y2.stride(0), x2.data_ptr(), x2.stride(0), nworld, _stream(M),
+                )  # fmt: skip
+                _lib.check(status, "im_tile_cholesky_solve_m")
+            else:
+                if M.dim() != 3 or M.shape[0] != nworld or M.stride(2) != 1:
+                    raise ValueError("M must be (nworld, nv, nv) with contiguous rows")
+                status = lib.im_tile_cholesky_solve(
+                    M.data_ptr(), M.stride(0), M.stride(1), adr.data_ptr(), adr.numel(), size, y2.data_ptr(),
+                    y2.stride(0), x2.data_ptr(), x2.stride(0), nworld, _stream(M),
+                )  # fmt: skip
+                _lib.check(status, "im_tile_cholesky_solve")
+
+
+def factor_solve_i_no_l_store(m: Any, d: Any, M, L, D, x, y, tree_factor_solve=None, *,
+                              upstream: Callable[..., None] | None = None) -> None:  # fmt: skip
+    """Factor and solve without the dense factor as an output (:849-873): the tree L'DL when its
+    scratch is given, upstream's factor for a sparse tail (``upstream(True)``: its solve reads
+    ``L`` and ``D``), else the tile solve that keeps the factor on chip."""
+    from . import tree_ldl
+
+    if tree_factor_solve is not None:
+        tree_ldl.tree_factor_solve(tree_factor_solve, M, x, y)
+        return
+    if _has_sparse_m_tail(m, d):
+        if upstream is None:
+            raise NotImplementedError("a sparse tail is factored by upstream's factor_solve_i")
+        upstream(True)
+        return
+    _factor_solve_i_dense_no_l_store(m, d, M, x, y, D, upstream=upstream)
+
+
 def _factor_solve_i_dense(
     m: Any, d: Any, M, x, y, dense_factor_solve: BlockedDenseFactorSolveScratch | None = None, *,
     retain_factor: bool = False, factor_workspace=None, tree_factor_solve=None,
     upstream: Callable[..., None] | None = None,
 ) -> None:  # fmt: skip
     """Dense factor + solve that prefers the tree L'DL when no factor is kept, then the blocked
-    kernel when its scratch exists: the reference's precedence and errors (:1030-1070).  What is
-    left after those two is upstream mujoco_warp code (``smooth.factor_solve_i`` and the
-    single-tile solve), which is not part of this library: pass it as ``upstream(retain_factor)``."""
+    kernel when its scratch exists, then the single-tile solve: the reference's precedence and
+    errors (:1030-1070).  Keeping the factor without a blocked scratch is upstream mujoco_warp's
+    ``smooth.factor_solve_i`` (its ``qLD`` layout is not part of the reference's tree): pass it
+    as ``upstream(retain_factor)``."""
     from . import tree_ldl
 
     if factor_workspace is not None and dense_factor_solve is None:
@@ -156,9 +256,12 @@ def _factor_solve_i_dense(
             factor_out=d.qLD if retain_factor else None, factor_workspace=factor_workspace,
         )  # fmt: skip
         return
-    if upstream is None:
-        raise NotImplementedError("neither a tree nor a blocked scratch: the remaining solves are upstream's")
-    upstream(retain_factor)
+    if retain_factor:
+        if upstream is None:
+            raise NotImplementedError("keeping the factor without a blocked scratch is upstream's factor_solve_i")
+        upstream(True)
+        return
+    _factor_solve_i_dense_no_l_store(m, d, M, x, y, upstream=upstream)
 
 
 def _check_rhs(scratch, nworld: int, y, x, active) -> int:

@@ -131,6 +131,14 @@ def run(launches: int = 32, only: str | None = None) -> None:
                 del St, G3, X3
             sec = _timeit(torch, lambda i: T.tree_factor_solve(sc, S[i][0], X[i], S[i][5]), nsets, launches)
             _line("im_tree_factor_solve", wl, sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
+            if nv <= 32:
+                # the same solve through one Cholesky tile gathered from M's structure (no factor kept)
+                ids = synth.matrix_elemid(b.rowadr, b.rownnz, b.colind)
+                tile = SimpleNamespace(size=nv, adr=torch.zeros(1, dtype=torch.int32, device=dev), elemid=t(np.where(ids < 0, nM, ids).astype(np.int32).reshape(-1)))
+                mt = SimpleNamespace(M_tiles=[tile], nv=nv, qLD_block_total=0)
+                dt = SimpleNamespace(nworld=nworld, qLD=torch.zeros((nworld, 0), device=dev))
+                sec = _timeit(torch, lambda i: BD._factor_solve_i_dense(mt, dt, S[i][0], X[i], S[i][5]), nsets, launches)
+                _line("im_tile_cholesky_solve_m", wl, sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
             if name in ("g1", "snu"):
                 # the same Hessians through the blocked dense factor and the static-pattern sparse L'DL
                 Md = synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32).reshape(nworld, -1)

@@ -1048,13 +1048,84 @@ int orc_blocked_multi_solve(int nworld, int nv, int pad, int B, const float *U, 
   return 0;
 }
 
+/* Cholesky of one tile that fits a block (up to 64 x 64) and the solve of one right-hand side
+ * with it, nothing kept: src/instantmimic/utils/mjw_step_optimized.py:672-750 (the two
+ * "no L store" tile kernels) and the nv <= 32 branch of the Newton factor stage
+ * (src/instantmimic/utils/mjw_kernels/newton_stages.py:723-733).  The reference takes the
+ * arithmetic from Warp's tile library (third party, absent); here the tile is factored as a
+ * diagonal tile of the blocked factor is: row i of L from A's row i, column by column,
+ *   v = A[i][j]; for q < j ascending: v = fmaf(-L[i][q], L[j][q], v); L[i][j] = v * (1 / L[j][j]),
+ * pivots sqrtf of the same chain; then the two substitutions, column oriented.
+ * A: the lower triangle, row major with row length n; s: right-hand side in, solution out. */
+static void tile_factor_solve(int n, const float *A, float *L, float *s) {
+  for (int j = 0; j < n; ++j) {
+    float p = A[j * n + j];
+    for (int q = 0; q < j; ++q) p = fmaf(-L[j * n + q], L[j * n + q], p);
+    const float d = sqrtf(p), inv = 1.0f / d;
+    L[j * n + j] = d;
+    for (int i = j + 1; i < n; ++i) {
+      float v = A[i * n + j];
+      for (int q = 0; q < j; ++q) v = fmaf(-L[i * n + q], L[j * n + q], v);
+      L[i * n + j] = v * inv;
+    }
+  }
+  for (int j = 0; j < n; ++j) {
+    const float z = s[j] * (1.0f / L[j * n + j]);
+    s[j] = z;
+    for (int i = j + 1; i < n; ++i) s[i] = fmaf(-L[i * n + j], z, s[i]);
+  }
+  for (int r = n - 1; r >= 0; --r) {
+    const float xv = s[r] * (1.0f / L[r * n + r]);
+    s[r] = xv;
+    for (int t = 0; t < r; ++t) s[t] = fmaf(-L[r * n + t], xv, s[t]);
+  }
+}
+
+/* x[adr[t] .. + size) = tile_t^-1 y[same] for every world and tile.  elemid == NULL: M is dense,
+ * (ld_world per world, ld_row per row), tile t the diagonal block at adr[t], its lower triangle
+ * read (:672-701).  elemid != NULL: M holds nM values per world and tile t's element (r, c) is
+ * M[elemid[t size size + r size + c]], the upper triangle read (:704-750); an id at or past nM
+ * reads as zero. */
+int orc_tile_cholesky_solve(int nworld, int size, int ntile, const int *adr, const float *M,
+                            long ld_world, long ld_row, const int *elemid, int nM, const float *y,
+                            long ldy, float *x, long ldx) {
+  if (size < 1 || size > 64) return 1;
+#pragma omp parallel
+  {
+    float *A = (float *)malloc(sizeof(float) * (2 * (size_t)size * size + size));
+    float *L = A + (size_t)size * size, *s = L + (size_t)size * size;
+#pragma omp for schedule(static)
+    for (int w = 0; w < nworld; ++w)
+      for (int t = 0; t < ntile; ++t) {
+        const float *Mw = M + (size_t)w * ld_world;
+        const int a0 = adr[t];
+        for (int i = 0; i < size; ++i)
+          for (int c = 0; c <= i; ++c) {
+            if (elemid) {
+              const int id = elemid[((size_t)t * size + c) * size + i];
+              A[i * size + c] = id < nM ? Mw[id] : 0.0f;
+            } else {
+              A[i * size + c] = Mw[(size_t)(a0 + i) * ld_row + a0 + c];
+            }
+          }
+        for (int i = 0; i < size; ++i) s[i] = y[(size_t)w * ldy + a0 + i];
+        tile_factor_solve(size, A, L, s);
+        for (int i = 0; i < size; ++i) x[(size_t)w * ldx + a0 + i] = s[i];
+      }
+    free(A);
+  }
+  return 0;
+}
+
 /* Per-iteration factor stage on the dense Hessian (src/instantmimic/utils/mjw_kernels/
  * newton_stages.py:614-742): incremental update of H's upper triangle over the changed
  * rows' dof union (:451-470, 651-701), then the augmented blocked Cholesky (:473-611; the
  * gradient as column pad - 1, corner 1e30) or, without changed rows, a solve with the stored
  * factor.  The tile arithmetic and the order of the two final sums are this file's
  * conventions (the reference's come from Warp's tile library and mujoco_warp's
- * block_cholesky, both third party): 64 lanes stride the dofs, shuffle-down tree. */
+ * block_cholesky, both third party): 64 lanes stride the dofs, shuffle-down tree.  Up to 32
+ * dofs the stage keeps no factor (:723-733): after the update H is factored as one tile
+ * (tile_factor_solve) at every call, U is not touched. */
 int orc_dense_update_factor(int nworld, int nv, int pad, const unsigned char *done,
                             const int *state_changes, const int *changes, const int *ids,
                             int ld_ids, const float *J, int njmax, const float *D,
@@ -1063,8 +1134,9 @@ int orc_dense_update_factor(int nworld, int nv, int pad, const unsigned char *do
   const int B = 16;
 #pragma omp parallel
   {
-    float *work = (float *)malloc(sizeof(float) * ((size_t)pad * pad + pad + 2 * B * B + 8));
-    float *U = work, *rhs = U + (size_t)pad * pad, *A = rhs + pad, *L = A + B * B;
+    float *work = (float *)malloc(sizeof(float) * ((size_t)pad * pad + pad + 2 * 32 * 32 + 8));
+    float *U = work, *rhs = U + (size_t)pad * pad, *A = rhs + pad, *L = A + 32 * 32;
+    const int single = nv <= 32;
 #pragma omp for schedule(static)
     for (int w = 0; w < nworld; ++w) {
       if ((done && done[w]) || state_changes[w] == 0) continue;
@@ -1077,7 +1149,7 @@ int orc_dense_update_factor(int nworld, int nv, int pad, const unsigned char *do
       const int refactor = changes[w] != 0;
       const int count = changes[w] < 0 ? 0 : (changes[w] < ld_ids ? changes[w] : ld_ids);
       for (int i = 0; i < pad; ++i) rhs[i] = i < nv ? g[i] : 0.0f;
-      if (refactor) {
+      if (refactor || single) {
         const int nu = dof_union(nv, Jw, idw, count, uni);
         for (int cj = 0; cj < nu; ++cj)
           for (int ri = 0; ri <= cj; ++ri) {
@@ -1085,6 +1157,12 @@ int orc_dense_update_factor(int nworld, int nv, int pad, const unsigned char *do
             const float delta = pair_delta(nv, Jw, Dw, sw, quad, idw, count, row, col);
             if (delta != 0.0f) Hw[(size_t)row * pad + col] = Hw[(size_t)row * pad + col] + delta;
           }
+      }
+      if (single) {
+        for (int i = 0; i < nv; ++i)
+          for (int c = 0; c <= i; ++c) A[i * nv + c] = Hw[(size_t)c * pad + i];
+        tile_factor_solve(nv, A, L, rhs);
+      } else if (refactor) {
         blocked_factor_forward(nv, pad, B, 0, Hw, 0, U, rhs, A, L);
         float corner = 1.0e30f;
         for (int i = 0; i < nv; ++i) corner = fmaf(-rhs[i], rhs[i], corner);
@@ -1096,7 +1174,7 @@ int orc_dense_update_factor(int nworld, int nv, int pad, const unsigned char *do
         for (int i = 0; i < pad; ++i) U[(size_t)i * pad + pad - 1] = i == pad - 1 ? 1.0f : 0.0f;
         blocked_forward(pad, B, U, rhs);
       }
-      blocked_backward(pad, B, U, rhs);
+      if (!single) blocked_backward(pad, B, U, rhs);
       float s0[128] = {0}, s1[128] = {0};
       for (int lane = 0; lane < 64; ++lane)
         for (int i = lane; i < nv; i += 64) {

@@ -288,6 +288,28 @@ def blocked_factor_solve(M, block_idx, nv, pad, B, y, want_factor=True):
     return (x, U) if want_factor else x
 
 
+def tile_cholesky_solve(M, adr, size, y, elemid=None):
+    """x = tile^-1 y for every diagonal tile of ``size`` dofs starting at ``adr[t]``: ``M`` dense
+    (nworld, n, n) without ``elemid``, else (nworld, nM) values gathered through ``elemid``
+    (ntile * size * size ids).  Pinned by tests/test_tile_cholesky.py: scipy's ``cho_solve`` in
+    fp64 within conditioning, ``L L' == A`` through the blocked factor of the same matrix (up to
+    16 dofs the two are the same operations: bit-equal), dofs outside every tile untouched."""
+    M, y, adr = _f(M), _f(y), _i(adr)
+    nworld = M.shape[0]
+    x = np.zeros_like(y)
+    L = ctypes.c_long
+    if elemid is None:
+        n = M.shape[1]
+        st = lib().orc_tile_cholesky_solve(nworld, int(size), adr.size, _p(adr), _p(M), L(n * n), L(n), None, 0, _p(y),
+                                           L(y.shape[1]), _p(x), L(x.shape[1]))  # fmt: skip
+    else:
+        ids = _i(elemid)
+        st = lib().orc_tile_cholesky_solve(nworld, int(size), adr.size, _p(adr), _p(M), L(M.shape[1]), L(0), _p(ids),
+                                           M.shape[1], _p(y), L(y.shape[1]), _p(x), L(x.shape[1]))  # fmt: skip
+    assert st == 0
+    return x
+
+
 def blocked_multi_solve(U, nv, B, y, active=None, x=None):
     """Solve with stored factors U (nworld, pad, pad) for y (nworld, nv, nrhs); inactive worlds
     keep ``x`` (zeros when not given)."""

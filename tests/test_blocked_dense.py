@@ -228,8 +228,16 @@ def test_factor_solve_dispatcher_precedence_and_errors():
     # reference: src/instantmimic/utils/mjw_step_optimized.py:1030-1070, 984-986
     with pytest.raises(RuntimeError, match="requires the blocked dense path"):
         BD._factor_solve_i_dense(None, None, None, None, None, None, factor_workspace=object())
+    # keeping the factor without a blocked scratch, and a sparse tail behind the dense blocks, are
+    # upstream's factor_solve_i: without the callback both say so
     with pytest.raises(NotImplementedError):
-        BD._factor_solve_i_dense(None, None, None, None, None, None)
+        BD._factor_solve_i_dense(None, None, None, None, None, None, retain_factor=True)
+    tailed = SimpleNamespace(M_tiles=[], qLD_has_sparse=True)
+    with pytest.raises(NotImplementedError):
+        BD._factor_solve_i_dense(tailed, SimpleNamespace(nworld=1), None, None, None, None)
+    seen = []
+    BD._factor_solve_i_dense(tailed, SimpleNamespace(nworld=1), None, None, None, None, upstream=seen.append)
+    assert seen == [False]
     seen = []
     BD._factor_solve_i_dense(None, None, None, None, None, None, retain_factor=True, upstream=seen.append)
     assert seen == [True]

@@ -44,10 +44,10 @@ def test_oracle_search_sums_and_init_jaref():
 
 def test_oracle_dense_first_factor_is_the_factor_of_h():
     """A negative count of changed rows: H as it lies there is factored with the gradient as the
-    augmented column, and U'U gives it back."""
-    shape = synth.SHAPES["humanoid"]
+    augmented column, and U'U gives it back (beyond 32 dofs: below, no factor is kept)."""
+    shape = synth.SHAPES["g1"]
     b = synth.make_batch(shape, 6, ragged_nefc=True)
-    nv, pad = shape.nv, 32
+    nv, pad = shape.nv, 48
     Md = synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32)
     H = R.jtdj_dense(Md.reshape(6, -1), b.J, b.D, b.state[0], b.nefc, pad)
     every = np.ones(6, np.int32)
@@ -58,11 +58,12 @@ def test_oracle_dense_first_factor_is_the_factor_of_h():
     Hd = H[:, :nv, :nv].astype(np.float64)
     Hd = np.triu(Hd) + np.triu(Hd, 1).transpose(0, 2, 1)
     x64 = R.solve64(Hd, b.grad)
-    assert R.rel_l2(-search, x64) < 1e-4
+    err = np.linalg.norm(-search - x64, axis=1) / np.linalg.norm(x64, axis=1)
+    assert (err / (np.linalg.cond(Hd) * 6e-8)).max() < 4.0
     Uf = np.triu(U[:, :nv, :nv].astype(np.float64))
     back = np.einsum("wki,wkj->wij", Uf, Uf)
     assert np.abs(back - Hd).max() / np.abs(Hd).max() < 2e-6
-    np.testing.assert_allclose(decr, (b.grad * x64).sum(1), rtol=1e-3)
+    np.testing.assert_allclose(decr, (b.grad * x64).sum(1), rtol=5e-3)
 
 
 def test_elemid_table_matches_the_csr():
