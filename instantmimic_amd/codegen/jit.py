@@ -1,11 +1,13 @@
 """Generated tree kernels for models the library was not built with: source from
-:mod:`tree_row16` (module form), compiled to a gfx950 code object with ``hipcc --genco`` and
+:mod:`tree_row16` (module form), compiled to a gfx950 code object inside this process through
+``libhiprtc`` (or, where that library is missing or fails, by a ``hipcc --genco`` subprocess) and
 handed to ``im_tree_plan_attach_kernels``.  The reference does the same when it creates a model's
 scratch (src/instantmimic/utils/mjw_kernels/tree_ldl.py:393-416: straight-line code for the
 model, compiled by Warp at first use).  Code objects are kept on disk under their 64-bit
 structure key, so a model is compiled once (a few seconds).
 
 ``IMHIP_TREE_JIT=0`` turns this off (plans then run the table-driven kernel);
+``IMHIP_JIT_COMPILER=hiprtc`` or ``hipcc`` allows only that one of the two compilers;
 ``IMHIP_KERNEL_CACHE`` names the directory (default: ``_obj/kernels`` beside the library, else
 ``~/.cache/instantmimic_amd``; a directory owned by another user is never used)."""
 
@@ -23,8 +25,9 @@ from . import tree_row16
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.join(_HERE, "..", "csrc")
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fno-fast-math", "-Xclang", "-target-feature",
-         "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "--genco"]  # fmt: skip
+COMMON_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fno-fast-math", "-Xclang",
+                "-target-feature", "-Xclang", "-packed-fp32-ops"]  # fmt: skip
+FLAGS = COMMON_FLAGS + ["-Wno-unused-command-line-argument", "--genco"]  # the subprocess's
 
 
 def enabled() -> bool:
@@ -50,11 +53,12 @@ def cache_dir() -> str:
 
 
 def _source_tag() -> str:
-    """Changes whenever the generator, the header the kernels include, the compiler flags or one
+    """Changes whenever the generator, a header the kernels may include, the compiler flags or one
     of the environment knobs that alter the generated source changes: a code object built under
     one setting is never loaded under another."""
     h = hashlib.sha256()
-    for path in (os.path.join(_HERE, "tree_row16.py"), os.path.join(_CSRC, "tree_row16.h")):
+    headers = sorted(os.path.join(_CSRC, name) for name in os.listdir(_CSRC) if name.endswith(".h"))
+    for path in (os.path.join(_HERE, "tree_row16.py"), *headers):
         with open(path, "rb") as f:
             h.update(f.read())
     h.update("\0".join(FLAGS).encode())
@@ -100,23 +104,70 @@ def spilling_kernels(blob: bytes) -> list[str]:
     return sorted(name for name, (_, private) in kernel_resources(blob).items() if private and name in ("im_row16_fused", "im_row16_fused_long"))
 
 
-def code_object(structure, groups, trunk) -> bytes | None:
-    """The code object of a (structure, plan), from the cache or freshly compiled; ``None`` when no
-    compiler is at hand, when the generator declines the plan, when the compiler fails on the
-    generated source, or when a fused kernel came out with register spills to memory (no such
-    kernel is handed to the library; the plan then keeps the table-driven kernel)."""
-    key = tree_row16.structure_key(*structure, groups, trunk)
-    path = os.path.join(cache_dir(), f"tree_row16_{key:016x}_{_source_tag()}.co")
-    if os.path.exists(path):
-        with open(path, "rb") as f:
-            blob = f.read()
-        return None if not blob or spilling_kernels(blob) else blob
-    hipcc = shutil.which("hipcc") or ("/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else None)
-    if hipcc is None:
+def _rocm_root() -> str:
+    return os.environ.get("ROCM_PATH") or "/opt/rocm"
+
+
+_HIPRTC = None
+
+
+def _hiprtc():
+    """libhiprtc, loaded once; ``None`` where there is none."""
+    global _HIPRTC
+    if _HIPRTC is None:
+        _HIPRTC = False
+        for name in ("libhiprtc.so", os.path.join(_rocm_root(), "lib", "libhiprtc.so")):
+            try:
+                lib = C.CDLL(name)
+            except OSError:
+                continue
+            lib.hiprtcCreateProgram.argtypes = [C.POINTER(C.c_void_p), C.c_char_p, C.c_char_p, C.c_int, C.c_void_p, C.c_void_p]
+            lib.hiprtcCompileProgram.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_char_p)]
+            lib.hiprtcGetProgramLogSize.argtypes = lib.hiprtcGetCodeSize.argtypes = [C.c_void_p, C.POINTER(C.c_size_t)]
+            lib.hiprtcGetProgramLog.argtypes = lib.hiprtcGetCode.argtypes = [C.c_void_p, C.c_char_p]
+            lib.hiprtcDestroyProgram.argtypes = [C.POINTER(C.c_void_p)]
+            _HIPRTC = lib
+            break
+    return _HIPRTC or None
+
+
+def compile_hiprtc(src: str, label: str) -> bytes | None:
+    """The code object of ``src`` from the run-time compiler inside this process; ``None`` (with a
+    warning that carries the compiler's log) when the library is missing or the compile fails."""
+    import warnings
+
+    rtc = _hiprtc()
+    if rtc is None:
+        return None
+    prog = C.c_void_p()
+    if rtc.hiprtcCreateProgram(C.byref(prog), src.encode(), f"tree_row16_{label}.hip".encode(), 0, None, None) != 0:
         return None
     try:
-        src = tree_row16.generate(f"k{key:016x}", *structure, groups, trunk, module=True)
-    except tree_row16.Declined:
+        # the generated source includes this package's headers, which include HIP's by name
+        options = [o.encode() for o in COMMON_FLAGS + ["-I" + os.path.abspath(_CSRC), "-I" + os.path.join(_rocm_root(), "include")]]
+        status = rtc.hiprtcCompileProgram(prog, len(options), (C.c_char_p * len(options))(*options))
+        if status != 0:
+            n = C.c_size_t(0)
+            rtc.hiprtcGetProgramLogSize(prog, C.byref(n))
+            log = C.create_string_buffer(n.value + 1)
+            rtc.hiprtcGetProgramLog(prog, log)
+            warnings.warn(f"hiprtc failed on the generated tree kernel {label}: {log.value.decode(errors='replace')[-400:]}")
+            return None
+        n = C.c_size_t(0)
+        if rtc.hiprtcGetCodeSize(prog, C.byref(n)) != 0 or n.value == 0:
+            return None
+        code = C.create_string_buffer(n.value)
+        if rtc.hiprtcGetCode(prog, code) != 0:
+            return None
+        return code.raw
+    finally:
+        rtc.hiprtcDestroyProgram(C.byref(prog))
+
+
+def compile_hipcc(src: str, label: str) -> bytes | None:
+    """The same from a ``hipcc --genco`` subprocess; ``None`` without a compiler or when it fails."""
+    hipcc = shutil.which("hipcc") or next((p for p in (os.path.join(_rocm_root(), "bin", "hipcc"),) if os.path.exists(p)), None)
+    if hipcc is None:
         return None
     with tempfile.TemporaryDirectory(prefix="imhip_jit_") as tmp:
         hip, out = os.path.join(tmp, "kernel.hip"), os.path.join(tmp, "kernel.co")
@@ -126,10 +177,41 @@ def code_object(structure, groups, trunk) -> bytes | None:
         if done.returncode != 0 or not os.path.exists(out):
             import warnings
 
-            warnings.warn(f"hipcc failed on the generated tree kernel {key:016x}: {done.stderr.decode(errors='replace')[-400:]}")
+            warnings.warn(f"hipcc failed on the generated tree kernel {label}: {done.stderr.decode(errors='replace')[-400:]}")
             return None
         with open(out, "rb") as f:
+            return f.read()
+
+
+def compile_source(src: str, label: str) -> bytes | None:
+    """In this process first, a compiler subprocess second; ``IMHIP_JIT_COMPILER`` names the only one to try."""
+    only = os.environ.get("IMHIP_JIT_COMPILER", "")
+    if only not in ("", "hiprtc", "hipcc"):
+        raise ValueError("IMHIP_JIT_COMPILER is hiprtc or hipcc")
+    blob = compile_hiprtc(src, label) if only in ("", "hiprtc") else None
+    if blob is None and only in ("", "hipcc"):
+        blob = compile_hipcc(src, label)
+    return blob
+
+
+def code_object(structure, groups, trunk) -> bytes | None:
+    """The code object of a (structure, plan), from the cache or freshly compiled; ``None`` when
+    neither compiler is at hand, when the generator declines the plan, when the compiler fails on the
+    generated source, or when a fused kernel came out with register spills to memory (no such
+    kernel is handed to the library; the plan then keeps the table-driven kernel)."""
+    key = tree_row16.structure_key(*structure, groups, trunk)
+    path = os.path.join(cache_dir(), f"tree_row16_{key:016x}_{_source_tag()}.co")
+    if os.path.exists(path):
+        with open(path, "rb") as f:
             blob = f.read()
+        return None if not blob or spilling_kernels(blob) else blob
+    try:
+        src = tree_row16.generate(f"k{key:016x}", *structure, groups, trunk, module=True)
+    except tree_row16.Declined:
+        return None
+    blob = compile_source(src, f"{key:016x}")
+    if blob is None:
+        return None
     tmp_path = f"{path}.{os.getpid()}.tmp"
     with open(tmp_path, "wb") as f:
         f.write(blob)

@@ -100,6 +100,29 @@ def test_kernel_descriptors_of_a_code_object():
     assert jit.code_object(st, groups, trunk) is None
 
 
+def test_both_compilers_give_the_same_kernels(monkeypatch):
+    """The run-time compiler inside the process and the compiler subprocess: the same five kernels
+    with the same LDS and private-segment sizes; ``IMHIP_JIT_COMPILER`` allows one of them only."""
+    st, groups, trunk, _ = build._plan_of_tree(TREES["branched"])
+    src = tree_row16.generate("t", *st, groups, trunk, module=True)
+    inside, outside = jit.compile_hiprtc(src, "t"), jit.compile_hipcc(src, "t")
+    assert inside is not None and outside is not None
+    assert jit.kernel_resources(inside) == jit.kernel_resources(outside)
+    assert b"im_row16_key" in inside and b"im_row16_info" in inside
+    calls = []
+    monkeypatch.setattr(jit, "compile_hiprtc", lambda *a: calls.append("hiprtc"))
+    monkeypatch.setattr(jit, "compile_hipcc", lambda *a: calls.append("hipcc"))
+    jit.compile_source(src, "t")
+    monkeypatch.setenv("IMHIP_JIT_COMPILER", "hipcc")
+    jit.compile_source(src, "t")
+    monkeypatch.setenv("IMHIP_JIT_COMPILER", "hiprtc")
+    jit.compile_source(src, "t")
+    assert calls == ["hiprtc", "hipcc", "hipcc", "hiprtc"]
+    monkeypatch.setenv("IMHIP_JIT_COMPILER", "nvcc")
+    with pytest.raises(ValueError):
+        jit.compile_source(src, "t")
+
+
 def _has_kernel(scratch) -> bool:
     key, has = C.c_ulonglong(0), C.c_int(0)
     assert _lib.lib().im_tree_plan_kernel_key(scratch.kernel.ptr, C.byref(key), C.byref(has)) == 0
@@ -130,6 +153,29 @@ def test_gpu_more_than_64_dofs_run_on_generated_kernels(device, monkeypatch, nam
     m = type("m", (), dict(nv=b.shape.nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind))
     monkeypatch.setenv("IMHIP_TREE_JIT", "0")
     assert T.create_tree_factor_solve_scratch(m, device) is None  # nothing to run it on without generated kernels
+
+
+@pytest.mark.gpu
+def test_gpu_cold_compile_inside_the_process(device, monkeypatch, tmp_path):
+    """An empty cache directory and a tree that nothing was built for beforehand: the kernels are
+    generated and compiled here, in this process (no compiler subprocess), loaded, and right."""
+    rng = np.random.default_rng(20261)
+    parents = [-1, 0, 1, 2, 3, 4]  # a floating base, then five limbs of random lengths off dof 5
+    for _ in range(5):
+        at = 5
+        for _ in range(int(rng.integers(4, 9))):
+            parents.append(at)
+            at = len(parents) - 1
+    assert tuple(parents) not in {tuple(v) for v in TREES.values()}
+    TREES["cold"] = parents
+    monkeypatch.setenv("IMHIP_KERNEL_CACHE", str(tmp_path))
+    monkeypatch.setenv("IMHIP_JIT_COMPILER", "hiprtc")
+    try:
+        _generated_against_oracle(device, monkeypatch, "cold", 150, table_driven_too=True)
+    finally:
+        del TREES["cold"]
+    made = [p.name for p in tmp_path.iterdir()]
+    assert len(made) == 1 and made[0].startswith("tree_row16_") and made[0].endswith(".co")
 
 
 def _generated_against_oracle(device, monkeypatch, name, nworld, table_driven_too):
