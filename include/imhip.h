@@ -778,6 +778,21 @@ int im_implicit_qh(const float *M, int64_t ldM, int nM, const int32_t *elem_dof,
                    float *gain, int64_t ld_gain, int nu, const im_row_pair_term *actuators,
                    const im_row_pair_term *tendons, float *qH, int64_t ld_qH, int nworld, void *stream);
 
+/* Replaces the polynomial part of upstream's _qderiv_actuator_passive (dof_dampingpoly with qvel)
+ * and _qderiv_tendon_damping (tendon_dampingpoly with ten_velocity), as the reference's
+ * deriv_smooth_vel passes them (src/instantmimic/utils/mjw_step_optimized.py:3857-3900): the
+ * damping coefficient that the implicit matrix sees,
+ *   out[w, i] = base[w, i] + sum over k = 1..nterm of (k + 1) poly[w, i, k - 1] |velocity[w, i]|^k,
+ * the slope of a damper whose force is -v (b + p_1 |v| + ... + p_K |v|^K) (Horner's rule, fused
+ * multiply-adds, highest term first).  The result goes where the plain damping went:
+ * dof_damping of im_implicit_qh / im_implicit_qh_base with its world stride, the tendon term's
+ * weight.  ld_base / ld_poly = 0: one set of coefficients for all worlds.  The upstream kernels
+ * are not part of the reference's tree; the form of the polynomial is MuJoCo's as this library
+ * reads it (coefficients of |v|, |v|^2, ... beside the constant damping). */
+int im_polynomial_damping(const float *base, int64_t ld_base, const float *poly, int64_t ld_poly, int nterm,
+                          const float *velocity, int64_t ld_velocity, float *out, int64_t ld_out, int n,
+                          int nworld, void *stream);
+
 /* Velocity gain of actuators with affine gain / bias (what derivative._qderiv_actuator_passive_vel
  * produces for them, mjw_step_optimized.py:3818-3846): gain[w, a] = biasprm[a, 2] (biastype 1)
  * + gainprm[a, 2] * input[w, a] (gaintype 1), zero when forcelimited[a] and force[w, a] is at or

@@ -41,6 +41,25 @@ __global__ __launch_bounds__(256) void implicit_qh_base_kernel(const float *__re
     if (e0 + k < nM) ow[e0 + k] = d[k] >= 0 ? __builtin_fmaf(timestep, dw[d[k]], v[k]) : v[k];
 }
 
+// Damping with polynomial terms, as a damping coefficient for the implicit matrix: a damper whose
+// force is  -v (b + p_1 |v| + ... + p_K |v|^K)  has the slope  -(b + 2 p_1 |v| + ... + (K + 1) p_K |v|^K)
+// in v, evaluated by Horner's rule with fused multiply-adds from the highest term down.
+// One lane per (world, item).
+__global__ __launch_bounds__(256) void polynomial_damping_kernel(const float *__restrict__ base, int64_t ld_base,
+                                                                 const float *__restrict__ poly, int64_t ld_poly,
+                                                                 int nterm, const float *__restrict__ velocity,
+                                                                 int64_t ld_velocity, float *__restrict__ out,
+                                                                 int64_t ld_out, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int64_t w = blockIdx.y;
+  if (i >= n) return;
+  const float a = fabsf(velocity[w * ld_velocity + i]);
+  const float *p = poly + w * ld_poly + (int64_t)i * nterm;
+  float acc = 0.0f;
+  for (int k = nterm; k >= 1; --k) acc = __builtin_fmaf(acc, a, (float)(k + 1) * p[k - 1]);
+  out[w * ld_out + i] = __builtin_fmaf(acc, a, base[w * ld_base + i]);
+}
+
 // d force / d velocity of an actuator with affine gain and bias (MuJoCo mjGAIN_AFFINE = 1,
 // mjBIAS_AFFINE = 1): bias parameter 2 plus gain parameter 2 times the control (or the
 // activation for a stateful actuator: `input` is what the caller's model says drives the gain);
@@ -171,6 +190,24 @@ int im_implicit_qh_base(const float *M, int64_t ldM, int nM, const int32_t *elem
     hipLaunchKernelGGL(im::implicit_qh_base_kernel, dim3((unsigned)((nM + 1023) / 1024), (unsigned)nw), dim3(256), 0,
                        (hipStream_t)stream, M + (int64_t)w0 * ldM, ldM, elem_dof, dof_damping + (int64_t)w0 * ld_damping,
                        ld_damping, timestep, qH + (int64_t)w0 * ld_qH, ld_qH, nM);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+int im_polynomial_damping(const float *base, int64_t ld_base, const float *poly, int64_t ld_poly, int nterm,
+                          const float *velocity, int64_t ld_velocity, float *out, int64_t ld_out, int n, int nworld,
+                          void *stream) {
+  if (nworld < 0 || n < 0 || nterm < 0 || ld_base < 0 || ld_poly < 0) return IM_ERR_ARG;
+  if (nworld == 0 || n == 0) return IM_OK;
+  if (!base || (nterm > 0 && !poly) || !velocity || !out) return IM_ERR_ARG;
+  if (ld_velocity < n || ld_out < n || (ld_base != 0 && ld_base < n) || (ld_poly != 0 && ld_poly < (int64_t)n * nterm))
+    return IM_ERR_STRIDE;
+  for (int w0 = 0; w0 < nworld; w0 += 65535) {
+    const int nw = nworld - w0 < 65535 ? nworld - w0 : 65535;
+    hipLaunchKernelGGL(im::polynomial_damping_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)nw), dim3(256), 0,
+                       (hipStream_t)stream, base + (int64_t)w0 * ld_base, ld_base, poly + (int64_t)w0 * ld_poly, ld_poly, nterm,
+                       velocity + (int64_t)w0 * ld_velocity, ld_velocity, out + (int64_t)w0 * ld_out, ld_out, n);
   }
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;

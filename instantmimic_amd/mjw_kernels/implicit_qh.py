@@ -10,14 +10,16 @@ terms here are the ones MuJoCo's ``mjd_smooth_vel`` documents for this integrato
 * actuators with affine gain / bias: ``- h moment' diag(gain) moment`` with the gain of
   ``im_actuator_velocity_gain``,
 * tendon damping: ``+ h J' diag(tendon_damping) J``,
+* polynomial dampers (``dof_dampingpoly``, ``tendon_dampingpoly``): a damper whose force is
+  ``-v (b + p_1 |v| + ... + p_K |v|^K)`` enters with its slope at the current velocity,
+  ``b + 2 p_1 |v| + ... + (K + 1) p_K |v|^K``, in place of ``b`` (``im_polynomial_damping``),
 * rows of free bodies reset to M (``_implicit_free_body_reset_m``): here those rows never receive
   a term, which leaves them equal to M,
 * the registered contributors (the muscles' ``h A' diag(s) A``) on top.
 
 The three pair sums over sparse rows go through the deterministic gather of
 :mod:`instantmimic_amd.muscle.muscle_qfrc_projector` (``im_muscle_implicit_gather``), element by
-element in a fixed order.  Fluid forces and polynomial damping are not assembled: a model that
-has them is refused.
+element in a fixed order.  Fluid forces are not assembled: a model that has them is refused.
 """
 
 from __future__ import annotations
@@ -152,10 +154,6 @@ def create_implicit_qh_scratch(m: Any, d: Any, device, *, disable_damper=DISABLE
 
     if getattr(m, "has_fluid", False):
         raise NotImplementedError("fluid forces are not part of this qH")
-    for name in ("dof_dampingpoly", "tendon_dampingpoly"):
-        poly = getattr(m, name, None)
-        if poly is not None and np.any(_host(poly, np.float32) != 0):
-            raise NotImplementedError(f"{name} is not part of this qH")
     dev = torch.device(device)
     nworld, nM = int(d.nworld), len(_host(m.M_colind))
     damper = not _flag(m, disable_damper)
@@ -170,16 +168,60 @@ def create_implicit_qh_scratch(m: Any, d: Any, device, *, disable_damper=DISABLE
                                     _host(d.moment_colind).reshape(nworld if _host(d.moment_colind).ndim > 1 else 1, -1)[0], elemid, dev)  # fmt: skip
         gain = torch.zeros((nworld, nu), device=dev)
     nt = int(getattr(m, "ntendon", 0) or 0)
-    if nt > 0 and damper and np.any(_host(m.tendon_damping, np.float32) != 0):
+    tables = {}
+    tendon_poly = _polynomial(getattr(m, "tendon_dampingpoly", None), nt, dev) if nt > 0 and damper else None
+    if nt > 0 and damper and (np.any(_host(m.tendon_damping, np.float32) != 0) or tendon_poly is not None):
         tendons = row_pair_gather(m.ten_J_rownnz, m.ten_J_rowadr, m.ten_J_colind, elemid, dev)
         td = torch.from_numpy(_host(m.tendon_damping, np.float32).reshape(-1, nt)).to(dev)
         tendon_damping = td.expand(nworld, nt).contiguous()
+        if tendon_poly is not None:
+            tables["tendon_poly"], tables["tendon_base"] = tendon_poly, tendon_damping.clone()
+    dof_poly = _polynomial(getattr(m, "dof_dampingpoly", None), int(m.nv), dev) if damper else None
+    if dof_poly is not None:
+        tables["dof_poly"], tables["dof_effective"] = dof_poly, torch.zeros((nworld, int(m.nv)), device=dev)
     return ImplicitQhScratch(
         elem_dof=torch.from_numpy(element_dofs(m, damper)).to(dev), actuators=actuators, tendons=tendons,
         tendon_damping=tendon_damping, implicit_qderiv=torch.zeros((nworld, nM), device=dev),
         implicit_qacc=torch.zeros((nworld, int(m.nv)), device=dev), actuator_gain=gain,
-        timestep=float(np.asarray(_host(m.opt.timestep, np.float32)).reshape(-1)[0]),
+        timestep=float(np.asarray(_host(m.opt.timestep, np.float32)).reshape(-1)[0]), tables=tables,
     )  # fmt: skip
+
+
+def _polynomial(poly, n: int, dev):
+    """The coefficients of |v|, |v|^2, ... of a polynomial damper as a (1 or nworld, n, K) device
+    tensor; ``None`` when the model has none or all are zero."""
+    import torch
+
+    if poly is None:
+        return None
+    p = _host(poly, np.float32)
+    if p.size == 0 or not np.any(p != 0):
+        return None
+    if p.size % n:
+        raise ValueError("polynomial damping coefficients do not match the number of dofs or tendons")
+    if p.ndim == 3:
+        p = p.reshape(p.shape[0], n, -1)
+    else:
+        p = p.reshape(1, n, -1)
+    return torch.from_numpy(np.ascontiguousarray(p)).to(dev)
+
+
+def polynomial_damping(base, poly, velocity, out) -> None:
+    """``out[w, i] = base[w, i] + sum_k (k + 1) poly[w, i, k - 1] |velocity[w, i]|^k``
+    (``im_polynomial_damping``): the damping coefficient the implicit matrix sees."""
+    import torch
+
+    nworld, n = int(velocity.shape[0]), int(out.shape[1])
+    for t in (base, poly, velocity, out):
+        if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous():
+            raise TypeError("polynomial damping takes contiguous float32 CUDA tensors")
+    with torch.cuda.device(out.device):
+        status = _lib.lib().im_polynomial_damping(
+            base.data_ptr(), base.stride(0) if base.shape[0] > 1 else 0, poly.data_ptr(),
+            poly.stride(0) if poly.shape[0] > 1 else 0, int(poly.shape[2]), velocity.data_ptr(), velocity.stride(0),
+            out.data_ptr(), out.stride(0), n, nworld, _stream(out),
+        )  # fmt: skip
+    _lib.check(status, "im_polynomial_damping")
 
 
 def _stream(t) -> int:
@@ -313,6 +355,13 @@ def deriv_smooth_vel(m: Any, d: Any, out, scratch: ImplicitQhScratch, *, fused: 
     if M.dtype != torch.float32 or out.dtype != torch.float32 or M.stride(1) != 1 or out.stride(1) != 1 or M.shape != out.shape:
         raise TypeError("M and out must be float32 (nworld, nM) tensors with contiguous rows")
     nworld, nM = int(M.shape[0]), int(scratch.elem_dof.numel())
+    # polynomial dampers (dof_dampingpoly, tendon_dampingpoly): their slope at the current velocity
+    # takes the place of the constant coefficient
+    if "dof_poly" in scratch.tables:
+        polynomial_damping(damping, scratch.tables["dof_poly"], d.qvel.reshape(nworld, -1), scratch.tables["dof_effective"])
+        damping = scratch.tables["dof_effective"]
+    if "tendon_poly" in scratch.tables:
+        polynomial_damping(scratch.tables["tendon_base"], scratch.tables["tendon_poly"], d.ten_velocity.reshape(nworld, -1), scratch.tendon_damping)
     if fused and _deriv_smooth_vel_fused(m, d, out, scratch, damping, nworld, nM):
         return
     with torch.cuda.device(out.device):

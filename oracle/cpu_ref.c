@@ -832,6 +832,26 @@ int orc_newton_eval_constraints(int nworld, int njmax, const float *Jaref, const
   return 0;
 }
 
+/* The damping coefficient the implicit matrix sees from a damper with polynomial terms: the
+ * slope of  -v (b + p_1 |v| + ... + p_K |v|^K), i.e.  b + sum_k (k + 1) p_k |v|^k, by Horner's rule
+ * from the highest term (upstream's derivative._qderiv_actuator_passive / _qderiv_tendon_damping
+ * take dof_dampingpoly / tendon_dampingpoly beside the plain coefficients:
+ * src/instantmimic/utils/mjw_step_optimized.py:3857-3900; the kernels themselves are third party
+ * and absent).  ld_base / ld_poly = 0: shared by all worlds. */
+int orc_polynomial_damping(int nworld, int n, int nterm, const float *base, long ld_base,
+                           const float *poly, long ld_poly, const float *velocity, long ld_velocity,
+                           float *out, long ld_out) {
+  for (int w = 0; w < nworld; ++w)
+    for (int i = 0; i < n; ++i) {
+      const float a = fabsf(velocity[(size_t)w * ld_velocity + i]);
+      const float *p = poly + (size_t)w * ld_poly + (size_t)i * nterm;
+      float acc = 0.0f;
+      for (int k = nterm; k >= 1; --k) acc = fmaf(acc, a, (float)(k + 1) * p[k - 1]);
+      out[(size_t)w * ld_out + i] = fmaf(acc, a, base[(size_t)w * ld_base + i]);
+    }
+  return 0;
+}
+
 /* ------------------------------------------------------------------ implicit-fast integrator matrix
  * qH = M + h damping on the diagonal elements of damped dofs outside free bodies (elem_dof >= 0),
  * M elsewhere; and the velocity gain of affine actuators.  MuJoCo's published mjd_smooth_vel

@@ -754,6 +754,20 @@ def implicit_qh_base(M, elem_dof, damping, timestep):
     return out
 
 
+def polynomial_damping(base, poly, velocity):
+    """``base + sum_k (k + 1) poly[..., k - 1] |velocity|^k`` per (world, item); ``base`` (n,) or
+    (nworld, n), ``poly`` (n, K) or (nworld, n, K).  Pinned by tests/test_implicit_qh.py: the
+    central difference of the damper's force in fp64, and K = 0 returning ``base``."""
+    base, poly, velocity = _f(base), _f(poly), _f(velocity)
+    nworld, n = velocity.shape
+    nterm = poly.shape[-1]
+    out = np.zeros_like(velocity)
+    L = ctypes.c_long
+    assert lib().orc_polynomial_damping(nworld, n, nterm, _p(base), L(0 if base.ndim == 1 else n), _p(poly),
+                                        L(0 if poly.ndim == 2 else n * nterm), _p(velocity), L(n), _p(out), L(n)) == 0  # fmt: skip
+    return out
+
+
 def actuator_velocity_gain(gaintype, biastype, gainprm, biasprm, inp, forcelimited=None, forcerange=None, force=None):
     gainprm, biasprm, inp = _f(gainprm), _f(biasprm), _f(inp)
     gaintype, biastype = _i(gaintype), _i(biastype)

@@ -85,6 +85,37 @@ def test_oracle_against_fp64():
     assert (qh[:, off] != d.M[:, off]).any()
 
 
+def _with_polynomial_dampers(m, d, rng):
+    m.dof_dampingpoly = (rng.uniform(0.0, 0.5, (m.nv, 2)) * (rng.random((m.nv, 1)) < 0.6)).astype(np.float32)
+    m.tendon_dampingpoly = rng.uniform(0.0, 0.8, (m.ntendon, 3)).astype(np.float32)
+    d.qvel = rng.normal(scale=2.0, size=(d.nworld, m.nv)).astype(np.float32)
+    d.ten_velocity = rng.normal(scale=1.5, size=(d.nworld, m.ntendon)).astype(np.float32)
+
+
+def test_oracle_polynomial_damping_is_the_slope_of_the_force():
+    rng = np.random.default_rng(12)
+    base = rng.uniform(0, 2, 9).astype(np.float32)
+    poly = rng.uniform(0, 1, (9, 3)).astype(np.float32)
+    v = rng.normal(scale=2.0, size=(5, 9)).astype(np.float32)
+    v[0, 0] = 0.0
+    got = R.polynomial_damping(base, poly, v)
+
+    def force(x):
+        a = np.abs(x)
+        return -x * (base.astype(np.float64) + sum(poly[:, k].astype(np.float64) * a ** (k + 1) for k in range(3)))
+
+    eps = 1e-6
+    slope = -(force(v.astype(np.float64) + eps) - force(v.astype(np.float64) - eps)) / (2 * eps)
+    np.testing.assert_allclose(got, slope, rtol=2e-6, atol=1e-6)
+    assert got[0, 0] == base[0]
+    np.testing.assert_array_equal(R.polynomial_damping(base, np.zeros((9, 0), np.float32), v), np.broadcast_to(base, v.shape))
+    # per-world coefficients
+    pw = rng.uniform(0, 1, (5, 9, 2)).astype(np.float32)
+    bw = rng.uniform(0, 1, (5, 9)).astype(np.float32)
+    want = bw + 2 * pw[:, :, 0].astype(np.float64) * np.abs(v) + 3 * pw[:, :, 1].astype(np.float64) * v.astype(np.float64) ** 2
+    np.testing.assert_allclose(R.polynomial_damping(bw, pw, v), want, rtol=2e-6)
+
+
 def test_tables():
     m, d, st, nv0 = _model(1)
     np.testing.assert_array_equal(Q.free_dofs(m), np.arange(nv0, nv0 + 6))
@@ -142,3 +173,43 @@ def test_gpu_qh_and_solve(device):
     torch.cuda.synchronize()
     np.testing.assert_array_equal(scratch.implicit_qderiv.cpu().numpy(), 2.0 * want_qh)
     np.testing.assert_allclose(q2.cpu().numpy(), 0.5 * x_ref, rtol=1e-3, atol=1e-4 * np.abs(x_ref).max())
+
+
+@pytest.mark.gpu
+def test_gpu_qh_with_polynomial_dampers(device):
+    """dof_dampingpoly and tendon_dampingpoly: the slope of each damper at the current velocity takes
+    the place of its constant coefficient; both forms of the assembly, against the oracle chained
+    the same way and against the dense fp64 matrix with those slopes."""
+    import torch
+
+    nworld = 130
+    m, d, st, nv0 = _model(nworld, seed=5)
+    _with_polynomial_dampers(m, d, np.random.default_rng(6))
+    dof_eff = R.polynomial_damping(m.dof_damping, m.dof_dampingpoly, d.qvel)
+    ten_eff = R.polynomial_damping(m.tendon_damping, m.tendon_dampingpoly, d.ten_velocity)
+    assert (dof_eff > m.dof_damping).any() and (ten_eff > m.tendon_damping).all()
+    plain_dof, plain_ten = m.dof_damping, m.tendon_damping
+    want = []
+    for w in range(nworld):  # the oracle's chain takes one set of coefficients: world by world
+        m.dof_damping, m.tendon_damping = dof_eff[w], ten_eff[w]
+        one = SimpleNamespace(**{k: (v[w : w + 1] if isinstance(v, np.ndarray) and v.ndim > 1 and v.shape[0] == nworld else v) for k, v in vars(d).items()})
+        one.nworld = 1
+        want.append(_oracle_qh(m, one, st)[0][0])
+    want = np.stack(want)
+    m.dof_damping, m.tendon_damping = plain_dof, plain_ten
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    dd = SimpleNamespace(nworld=nworld, M=t(d.M), moment_rownnz=d.moment_rownnz, moment_rowadr=d.moment_rowadr, moment_colind=d.moment_colind,
+                         actuator_moment=t(d.actuator_moment), ten_J=t(d.ten_J), ctrl=t(d.ctrl), actuator_force=t(d.actuator_force),
+                         qvel=t(d.qvel), ten_velocity=t(d.ten_velocity), efc=SimpleNamespace(Ma=t(d.efc.Ma)))  # fmt: skip
+    scratch = Q.create_implicit_qh_scratch(m, dd, device)
+    for fused in (True, False):
+        scratch.implicit_qderiv.fill_(float("nan"))
+        Q.deriv_smooth_vel(m, dd, scratch.implicit_qderiv, scratch, fused=fused)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(scratch.tables["dof_effective"].cpu().numpy(), dof_eff)
+        np.testing.assert_array_equal(scratch.tendon_damping.cpu().numpy(), ten_eff)
+        np.testing.assert_array_equal(scratch.implicit_qderiv.cpu().numpy(), want)
+    # a fluid model is still refused
+    m.has_fluid = True
+    with pytest.raises(NotImplementedError):
+        Q.create_implicit_qh_scratch(m, dd, device)

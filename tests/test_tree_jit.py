@@ -178,6 +178,37 @@ def test_gpu_cold_compile_inside_the_process(device, monkeypatch, tmp_path):
     assert len(made) == 1 and made[0].startswith("tree_row16_") and made[0].endswith(".co")
 
 
+@pytest.mark.gpu
+def test_gpu_declined_forest_runs_on_the_table_driven_kernel(device, monkeypatch, tmp_path):
+    """Two roots: the generator declines the plan (its trunk is no single chain); creating the
+    model's scratch must not raise, and the scratch solves on the table-driven kernel."""
+    import torch
+
+    from instantmimic_amd.mjw_kernels import tree_ldl as T
+
+    parents = [-1, 0, 0, 2, -1, 4, 4, 6, 1, 1, 3, 3, 5, 5, 7, 7]
+    st, groups, trunk, _ = build._plan_of_tree(parents)
+    with pytest.raises(tree_row16.Declined):
+        tree_row16.generate("t", *st, groups, trunk, module=True)
+    monkeypatch.setenv("IMHIP_KERNEL_CACHE", str(tmp_path))
+    TREES["forest"] = parents
+    try:
+        b = _batch("forest", 77, nefc=24)
+    finally:
+        del TREES["forest"]
+    m = type("m", (), dict(nv=b.shape.nv, M_rowadr=b.rowadr, M_rownnz=b.rownnz, M_colind=b.colind))
+    scratch = T.create_tree_factor_solve_scratch(m, device)
+    assert scratch is not None and not _has_kernel(scratch) and list(tmp_path.iterdir()) == []
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+    G = t(b.grad)
+    x = torch.full_like(G, float("nan"))
+    T.assemble_tree_factor_solve(scratch, t(b.M), t(b.J), t(b.D), t(b.state[0]), t(b.nefc), G, x)
+    torch.cuda.synchronize()
+    stc = (b.rowadr, b.rownnz, b.colind)
+    want = R.assemble_tree_ldl_solve(*stc, P.best_tree_ldl_plan(*stc), b.M, b.J, b.D, b.state[0], b.nefc, b.grad)
+    np.testing.assert_array_equal(x.cpu().numpy(), want)
+
+
 def _generated_against_oracle(device, monkeypatch, name, nworld, table_driven_too):
     import torch
 
