@@ -1378,7 +1378,7 @@ __device__ __forceinline__ void jtdj_tiles_as(const float *__restrict__ Mdense, 
   const int swz = nvr % 64 == 0 ? 3 : 1;
   const int kq = lane >> 4, kqs = kq & swz;
   // tiles (bi <= bj) distributed over the four waves; each wave keeps its tiles' accumulators
-  constexpr int MAXT = 9;                // up to 36 tiles (nv <= 128) over 4 waves
+  constexpr int MAXT = ROLE >= 0 ? 9 : 7;  // 36 tiles at eight blocks over 4 wavefronts; dealt at run time: up to seven blocks, 28 tiles
   float4v acc[MAXT];
   int tbi[MAXT], tbj[MAXT], mine = 0;
   if (ROLE >= 0) {
@@ -1564,7 +1564,11 @@ __device__ __forceinline__ void jtdj_tiles(const float *__restrict__ Mdense, con
                                            const float *__restrict__ D, const int32_t *__restrict__ state,
                                            const int32_t *__restrict__ nefc_p, int quad, int nv, float *lds,
                                            const Out &out) {
-  if (NVR == 128 && nv > 112) {  // eight blocks: a code path per wavefront (every path has the same barriers)
+  // NVR == 128 is launched for 113 .. 128 dofs only (eight blocks): a code path per wavefront, every
+  // path with the same barriers, and nothing else in the kernel -- the run-time dealing of tiles
+  // needs more registers than four workgroups per CU leave, and a kernel's register and scratch
+  // budget is that of its most expensive path
+  if constexpr (NVR == 128) {
     switch (threadIdx.x >> 6) {
       case 0: jtdj_tiles_as<NVR, 0>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, out); break;
       case 1: jtdj_tiles_as<NVR, 1>(Mdense, J, njmax, D, state, nefc_p, quad, nv, lds, out); break;
@@ -1599,7 +1603,7 @@ __global__ __launch_bounds__(256, NVR == 128 ? 4 : 3) void jtdj_mfma_kernel(
 // of J are staged in the factor's array, which is free until H is complete.  Results are those of
 // im_jtdj_mfma followed by im_blocked_factor_solve (B = 16) bit for bit.
 template <int NVR>
-__global__ __launch_bounds__(256, 4) void jtdj_factor_solve_kernel(
+__global__ __launch_bounds__(256, NVR == 128 ? 4 : 3) void jtdj_factor_solve_kernel(
     const float *__restrict__ Mdense, const float *__restrict__ J, int njmax, const float *__restrict__ D,
     const int32_t *__restrict__ state, const int32_t *__restrict__ nefc_p, int quad, float *__restrict__ H, int nv,
     int nv_pad, const float *__restrict__ y, int64_t ldy, float *__restrict__ Uout, float *__restrict__ x, int64_t ldx,
@@ -1838,7 +1842,7 @@ int im_jtdj_mfma(const float *Mdense, const float *J, int njmax, const float *D,
   // two copies of the staged rows, the list of contributing rows with their weights
   const size_t lds_bytes = sizeof(float) * (2 * (32 * (size_t)nvr + 32) + 2 * (size_t)((njmax + 3) & ~3));
   if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
-  auto fn = nvr == 128 ? im::jtdj_mfma_kernel<128> : im::jtdj_mfma_kernel<0>;
+  auto fn = nv > 112 ? im::jtdj_mfma_kernel<128> : im::jtdj_mfma_kernel<0>;
   if (lds_bytes > 64 * 1024)
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, Mdense, J, njmax, D, state, nefc,
@@ -1861,7 +1865,7 @@ int im_jtdj_factor_solve(const float *Mdense, const float *J, int njmax, const f
   const size_t stage_words = 2 * (32 * (size_t)nvr + 32) + 2 * (size_t)((njmax + 3) & ~3), u_words = im::Stair<16>{pad}.words();
   const size_t lds_bytes = sizeof(float) * ((u_words > stage_words ? u_words : stage_words) + pad + 16 * 16 + 16);
   if (lds_bytes > 160 * 1024) return IM_ERR_UNSUPPORTED;
-  auto fn = nvr == 128 ? im::jtdj_factor_solve_kernel<128> : im::jtdj_factor_solve_kernel<0>;
+  auto fn = nv > 112 ? im::jtdj_factor_solve_kernel<128> : im::jtdj_factor_solve_kernel<0>;
   if (lds_bytes > 64 * 1024)
     IM_HIP_CHECK(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   hipLaunchKernelGGL(fn, dim3(nworld), dim3(256), lds_bytes, (hipStream_t)stream, Mdense, J, njmax, D, state, nefc, quad,

@@ -443,11 +443,12 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
 
   // Every load below is unconditional (clamped address, value selected afterwards) and what
   // is needed first is requested first, so that each wait counts only the loads before it.
-  int tix[NTILE][4];
+  // where in M each accumulator element starts from: two 16-bit indices a word (behind the tile table)
+  int tmi[NTILE][2];
 #pragma unroll
   for (int t = 0; t < NTILE; ++t)
 #pragma unroll
-    for (int v = 0; v < 4; ++v) tix[t][v] = A.tile_index[(t * 4 + v) * 64 + lane];
+    for (int h = 0; h < 2; ++h) tmi[t][h] = A.tile_index[NTILE * 256 + (t * 2 + h) * 64 + lane];
   float mv[16];
 #pragma unroll
   for (int c = 0; c < 16; ++c) {
@@ -511,7 +512,7 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
   for (int t = 0; t < NTILE; ++t)
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      const int mi = (tix[t][v] >> 16) - 1;
+      const int mi = ((tmi[t][v >> 1] >> (16 * (v & 1))) & 0xFFFF) - 1;
       const float m = N[mi < 0 ? 0 : mi];
       acc[t][v] = mi >= 0 ? m : 0.0f;
     }
@@ -575,6 +576,7 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
     }
   }
   // the slots of this lane's accumulator elements (all requested before the first is used)
+  int tix[NTILE][4];
 #pragma unroll
   for (int t = 0; t < NTILE; ++t)
 #pragma unroll
@@ -1076,6 +1078,16 @@ int sparse_plan_upload(im_sparse_plan *pl) {
       const int t = ti * (ti + 1) / 2 + tj, lane = j + 16 * (i / 4), v = i % 4;
       tix[((size_t)t * 4 + v) * 64 + lane] = ((e + 1) << 16) | (sl + 1);
     }
+    // behind it, the M indices alone, two to a word (v = 0, 1 and v = 2, 3 of a lane): what the
+    // kernel holds from its start until the accumulators are set
+    const size_t ntile = (size_t)nt * (nt + 1) / 2;
+    tix.resize(ntile * 256 + ntile * 128, 0);
+    for (size_t t = 0; t < ntile; ++t)
+      for (int h = 0; h < 2; ++h)
+        for (int lane = 0; lane < 64; ++lane) {
+          const uint32_t lo = (uint32_t)tix[(t * 4 + 2 * h) * 64 + lane] >> 16, hi = (uint32_t)tix[(t * 4 + 2 * h + 1) * 64 + lane] >> 16;
+          tix[ntile * 256 + (t * 2 + h) * 64 + lane] = (int32_t)(lo | (hi << 16));
+        }
     if (fits) {
       IM_HIP_CHECK(hipMalloc((void **)&pl->tile_index, tix.size() * 4));
       IM_HIP_CHECK(hipMemcpy(pl->tile_index, tix.data(), tix.size() * 4, hipMemcpyHostToDevice));
