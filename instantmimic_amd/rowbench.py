@@ -621,6 +621,7 @@ def run(launches: int = 32, only: str | None = None) -> None:
     if section("bodies"):
         rig = synth.make_muscle_rig()
         topo = rig.topology
+        nworld = 4096
         nb, nvf = rig.body_count, rig.full_torque_dim
         parent = np.asarray(topo.body_parentid, np.int32)
         order, offsets, _, _ = WP.tree_levels(parent)
