@@ -139,21 +139,29 @@ def _compile(src: str) -> str:
     if os.path.dirname(src) != GEN:
         subprocess.run(cmd, check=True)
         return obj
-    # a generated kernel: the compiler's resource remarks say whether it keeps to registers
-    done = subprocess.run([*cmd, "-Rpass-analysis=kernel-resource-usage"], capture_output=True, text=True)
-    if done.returncode != 0:
-        sys.stderr.write(done.stderr)
-        raise subprocess.CalledProcessError(done.returncode, cmd)
-    spilling = _spilling_fused_kernels(done.stderr)
-    if spilling:
-        os.remove(obj)
-        raise RuntimeError(f"{os.path.basename(src)}: fused kernels spill registers to memory: {spilling}")
+    # a generated kernel: the compiler's resource remarks say whether it keeps to registers.  The
+    # resident Newton kernels get fewer workgroups per CU, one at a time, while they spill.
+    from .codegen import tree_row16
+
+    name, occ = tree_row16.occupancy_of(open(src).read())
+    for newton_occ in range(occ, 0, -1):
+        extra = [] if newton_occ == occ else [f"-DIM_NOCC_{name}={newton_occ}"]
+        done = subprocess.run([*cmd, *extra, "-Rpass-analysis=kernel-resource-usage"], capture_output=True, text=True)
+        if done.returncode != 0:
+            sys.stderr.write(done.stderr)
+            raise subprocess.CalledProcessError(done.returncode, cmd)
+        spilling = _spilling_kernels(done.stderr, fused=True)
+        if spilling:
+            os.remove(obj)
+            raise RuntimeError(f"{os.path.basename(src)}: fused kernels spill registers to memory: {spilling}")
+        if not _spilling_kernels(done.stderr, fused=False):
+            break
     return obj
 
 
-def _spilling_fused_kernels(remarks: str) -> list[str]:
-    """Fused kernels (first template argument true) with a private segment, from the text of
-    ``-Rpass-analysis=kernel-resource-usage``."""
+def _spilling_kernels(remarks: str, *, fused: bool) -> list[str]:
+    """Kernels with a private segment, from the text of ``-Rpass-analysis=kernel-resource-usage``:
+    the fused kernels (first template argument true) or the resident Newton kernels."""
     import re
 
     out, name = [], None
@@ -162,7 +170,9 @@ def _spilling_fused_kernels(remarks: str) -> list[str]:
         if m:
             name = m.group(1)
         m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
-        if m and name and int(m.group(1)) > 0 and "tree_row16_" in name and "ILb1E" in name:
+        if not (m and name and int(m.group(1)) > 0):
+            continue
+        if ("tree_row16_" in name and "ILb1E" in name) if fused else ("newton_row16_" in name):
             out.append(f"{name}: {m.group(1)} B/lane")
     return out
 

@@ -131,7 +131,7 @@ def _hiprtc():
     return _HIPRTC or None
 
 
-def compile_hiprtc(src: str, label: str) -> bytes | None:
+def compile_hiprtc(src: str, label: str, defines: tuple[str, ...] = ()) -> bytes | None:
     """The code object of ``src`` from the run-time compiler inside this process; ``None`` (with a
     warning that carries the compiler's log) when the library is missing or the compile fails."""
     import warnings
@@ -144,7 +144,7 @@ def compile_hiprtc(src: str, label: str) -> bytes | None:
         return None
     try:
         # the generated source includes this package's headers, which include HIP's by name
-        options = [o.encode() for o in COMMON_FLAGS + ["-I" + os.path.abspath(_CSRC), "-I" + os.path.join(_rocm_root(), "include")]]
+        options = [o.encode() for o in COMMON_FLAGS + ["-I" + os.path.abspath(_CSRC), "-I" + os.path.join(_rocm_root(), "include"), *defines]]
         status = rtc.hiprtcCompileProgram(prog, len(options), (C.c_char_p * len(options))(*options))
         if status != 0:
             n = C.c_size_t(0)
@@ -164,7 +164,7 @@ def compile_hiprtc(src: str, label: str) -> bytes | None:
         rtc.hiprtcDestroyProgram(C.byref(prog))
 
 
-def compile_hipcc(src: str, label: str) -> bytes | None:
+def compile_hipcc(src: str, label: str, defines: tuple[str, ...] = ()) -> bytes | None:
     """The same from a ``hipcc --genco`` subprocess; ``None`` without a compiler or when it fails."""
     hipcc = shutil.which("hipcc") or next((p for p in (os.path.join(_rocm_root(), "bin", "hipcc"),) if os.path.exists(p)), None)
     if hipcc is None:
@@ -173,7 +173,7 @@ def compile_hipcc(src: str, label: str) -> bytes | None:
         hip, out = os.path.join(tmp, "kernel.hip"), os.path.join(tmp, "kernel.co")
         with open(hip, "w") as f:
             f.write(src)
-        done = subprocess.run([hipcc, *FLAGS, "-I", _CSRC, "-x", "hip", hip, "-o", out], capture_output=True)
+        done = subprocess.run([hipcc, *FLAGS, *defines, "-I", _CSRC, "-x", "hip", hip, "-o", out], capture_output=True)
         if done.returncode != 0 or not os.path.exists(out):
             import warnings
 
@@ -188,9 +188,25 @@ def compile_source(src: str, label: str) -> bytes | None:
     only = os.environ.get("IMHIP_JIT_COMPILER", "")
     if only not in ("", "hiprtc", "hipcc"):
         raise ValueError("IMHIP_JIT_COMPILER is hiprtc or hipcc")
-    blob = compile_hiprtc(src, label) if only in ("", "hiprtc") else None
-    if blob is None and only in ("", "hipcc"):
-        blob = compile_hipcc(src, label)
+
+    def once(defines):
+        blob = compile_hiprtc(src, label, defines) if only in ("", "hiprtc") else None
+        if blob is None and only in ("", "hipcc"):
+            blob = compile_hipcc(src, label, defines)
+        return blob
+
+    blob = once(())
+    if blob is None:
+        return None
+    # The resident Newton kernels carry the loop's state on top of the stage's rows.  Where they
+    # spill at the fused kernels' occupancy, one more compile gives them a workgroup per CU less;
+    # if they still spill the library leaves them unused (the iterations are then stage launches).
+    name, occ = tree_row16.occupancy_of(src)
+    newton = ("im_row16_newton", "im_row16_newton_long")
+    if occ > 1 and any(kernel_resources(blob).get(k, (0, 0))[1] for k in newton):
+        again = once((f"-DIM_NOCC_{name}={occ - 1}",))
+        if again is not None and sum(kernel_resources(again).get(k, (0, 0))[1] for k in newton) < sum(kernel_resources(blob).get(k, (0, 0))[1] for k in newton):
+            blob = again
     return blob
 
 

@@ -911,7 +911,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
             emit(f"  im::gen::tree_row16_body_{name}<{asm_}, {long_}>({args});")
             emit("}")
         for kernel, long_ in (("newton", "false"), ("newton_long", "true")):
-            emit(f'extern "C" __global__ __launch_bounds__(256, IM_OCC_{name}) void im_row16_{kernel}(im::resident::NewtonArgs a) {{')
+            emit(f'extern "C" __global__ __launch_bounds__(256, IM_NOCC_{name}) void im_row16_{kernel}(im::resident::NewtonArgs a) {{')
             emit(f"  im::gen::newton_row16_body_{name}<{long_}>(a);")
             emit("}")
         emit(f'extern "C" __device__ const unsigned long long im_row16_key = 0x{key:016x}ull;')
@@ -922,7 +922,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
         emit(f"  tree_row16_body_{name}<ASM, LONG>({args});")
         emit("}")
         emit("template <bool LONG>")
-        emit(f"__global__ __launch_bounds__(256, IM_OCC_{name}) void newton_row16_{name}(im::resident::NewtonArgs a) {{")
+        emit(f"__global__ __launch_bounds__(256, IM_NOCC_{name}) void newton_row16_{name}(im::resident::NewtonArgs a) {{")
         emit(f"  newton_row16_body_{name}<LONG>(a);")
         emit("}")
         emit(f"static const Row16Entry entry_{name} = {{0x{key:016x}ull, {nv}, {nM}, {lds_floats * 4}, {4 * PD}, \"{name}\",")
@@ -943,4 +943,18 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     occ = max(1, min(asked, (160 * 1024) // (lds_floats * 4 + 32 * 128)))
     text = "\n".join(out) + "\n"
     header = '#include "tree_row16.h"' if module else '#include "../tree_row16.h"'  # a module is built with -I csrc
-    return text.replace('#include "../tree_row16.h"', f'{header}\n#define IM_OCC_{name} {occ}', 1)
+    # the resident Newton kernels carry the loop's state on top of the stage's rows: whoever compiles
+    # the source may give them fewer workgroups per CU (more registers) with -DIM_NOCC_<name>=n
+    # where they would otherwise spill
+    defines = f"#define IM_OCC_{name} {occ}\n#ifndef IM_NOCC_{name}\n#define IM_NOCC_{name} IM_OCC_{name}\n#endif"
+    return text.replace('#include "../tree_row16.h"', f"{header}\n{defines}", 1)
+
+
+def occupancy_of(source: str) -> tuple[str, int]:
+    """(kernel set name, workgroups per CU) that a generated source was written for."""
+    import re
+
+    m = re.search(r"#define IM_OCC_(\w+) (\d+)", source)
+    if not m:
+        raise ValueError("not a generated tree kernel source")
+    return m.group(1), int(m.group(2))

@@ -138,6 +138,7 @@ def _solve_on_gpu(p, device, *, graph: bool):
     ("snu", 4096, "sparse", True, "stages"), ("ant", 64, "tree", True, "stages"), ("snu", 130, "tree", False, "stages"),
     ("humanoid", 301, "tree", False, "resident"), ("humanoid", 4096, "tree", True, "resident"), ("ant", 67, "tree", True, "resident"),
     ("g1", 203, "sparse", False, "resident"), ("g1", 8192, "sparse", True, "resident"), ("snu", 4096, "sparse", True, "resident"),
+    ("g1", 8192, "tree", True, "resident"), ("snu", 131, "tree", False, "resident"), ("snu", 4096, "tree", True, "resident"),
 ])  # fmt: skip
 def test_gpu_solve_from_init_context_matches_the_oracle_chain(device, monkeypatch, name, nworld, stage, graph, loop):
     """``loop``: the iterations as eight launches each (``stages``) or as one resident kernel with a
