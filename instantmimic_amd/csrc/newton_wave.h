@@ -367,7 +367,9 @@ __device__ __forceinline__ const NewtonArgs &kernel_args(int kernarg_offset) {
   return *(const NewtonArgs *)ap;
 }
 
-template <int HELD, int JU, bool COOP, class Stage>
+// MLDS: the world's row of M is kept in LDS (L.m_lds); otherwise `M search` reads it from memory
+// every round, which leaves the LDS to more worlds per CU.
+template <int HELD, int JU, bool COOP, bool MLDS = true, class Stage>
 __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L, int64_t w_raw, Stage &&stage) {
   const NewtonArgs &a0 = kernel_args(kernarg_offset);
   const NewtonArgs &a = a0;
@@ -392,7 +394,8 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
              uniform(a.alpha[w]), uniform(a.improvement[w]), __builtin_amdgcn_readfirstlane(a.niter[w])};
   // what the loop keeps: M, Ma, Jaref into LDS (mv and jv are formed before they are read: a world
   // enters with a new search direction unless it is done) and qacc
-  for (int k = lane_fixed; k < a.nM; k += 64) L.m_lds[k] = a.M[w * a.ldM + k];
+  if constexpr (MLDS)
+    for (int k = lane_fixed; k < a.nM; k += 64) L.m_lds[k] = a.M[w * a.ldM + k];
   for (int k = lane_fixed; k < nv; k += 64) {
     L.Ma[k] = a.Ma[w * nv + k];
     L.mv[k] = a.mv[w * nv + k];
@@ -431,7 +434,7 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
       if (!unchanged) {
         for (int k = lane; k < nv; k += 64) L.sv[k] = a.search[w * nv + k];
         wave_sync();
-        mul_m_world(a, L.term, L.radr, L.m_lds, L.sv, a.mv + w * nv, L.mv, lane);
+        mul_m_world(a, L.term, L.radr, MLDS ? (const float *)L.m_lds : a.M + w * a.ldM, L.sv, a.mv + w * nv, L.mv, lane);
         if constexpr (JU > 0)
           jv_world<(JU > 0 ? JU : 1)>(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, L.jv, lane);
         else

@@ -858,7 +858,8 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
   uint32_t *term = (uint32_t *)(lds + A.staged_words + A.solve_words);
   int *radr = (int *)(term + a.nterm);
   const int area = resident_area_words(Q.nslots, nv, A.block, njmax);
-  float *mine = (float *)(radr + nv + 1) + wv * (area + resident::kept_words(nv, njmax, a.nM));
+  // (M is read from memory by the round's one product with it: its row would cost a CU a third of its worlds)
+  float *mine = (float *)(radr + nv + 1) + wv * (area + resident::kept_words(nv, njmax, 0));
   resident::LoopLds L;
   L.votes = nullptr;
   L.term = term, L.radr = radr;
@@ -866,8 +867,8 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
   L.f = mine;
   L.rowl = (int *)(mine + njmax);
   L.gl = mine + 2 * njmax;
-  L.m_lds = mine + area;
-  L.sv = L.m_lds + a.nM;
+  L.m_lds = nullptr;
+  L.sv = mine + area;
   L.Ma = L.sv + nv;
   L.mv = L.Ma + nv;
   L.qacc = L.mv + nv;
@@ -892,7 +893,7 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
                         (int)b.ld_grad, U_, uni_, b.search, b.search_dot, b.decrement, (int)w, threadIdx.x & 63);
   };
   while (w < nworld) {
-    resident::newton_loop<HELD, 0, false>(kArgsOffset, L, w, stage);  // HELD: 2 up to 64 rows, else 0
+    resident::newton_loop<HELD, 0, false, false>(kArgsOffset, L, w, stage);  // HELD: 2 up to 64 rows, else 0
     int next = 0;
     if ((threadIdx.x & 63) == 0) next = atomicAdd(next_world, 1);
     w = __builtin_amdgcn_readfirstlane(next);
@@ -1269,7 +1270,7 @@ int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *p, 
   A.solve_words = (int)solve_words;
   if (staged > 8192 || solve_words > 4096) return IM_ERR_UNSUPPORTED;
   const size_t shared = staged + solve_words + (size_t)p->nterm + n + 1;
-  const size_t per_wave = (size_t)im::resident_area_words(plan->nslots, n, plan->block, njmax) + im::resident::kept_words(n, njmax, nM);
+  const size_t per_wave = (size_t)im::resident_area_words(plan->nslots, n, plan->block, njmax) + im::resident::kept_words(n, njmax, 0);
   // the most worlds per workgroup (one workgroup per CU) that 160 KB of LDS admit and whose kernel
   // keeps to registers
   struct Variant {
