@@ -213,3 +213,34 @@ def test_entry_points_that_clamp_rows_refuse_an_empty_row_range():
     assert lib.im_muscle_project(one, 0, one, 4, one, one, one, 0, 4, 3, 0, one, 3, 2, None) == _lib.IM_ERR_ARG
     assert lib.im_muscle_project(one, 0, one, 4, one, one, one, 0, 4, 0, 0, one, 3, 2, None) == _lib.IM_OK
     assert lib.im_dense_update_factor(None, one, one, one, 8, one, 0, one, one, 1, one, 27, 32, 32, 27, 32, one, one, 27, one, one, 4, None) == _lib.IM_ERR_ARG
+
+
+def test_ctypes_structs_match_the_header(tmp_path):
+    """Every structure of include/imhip.h that the Python side fills through ctypes: the same size
+    and the same offset for every field, read from a probe that gcc compiles against the header."""
+    import ctypes as C
+    import os
+    import subprocess
+
+    pairs = {
+        "im_tree_plan_info": _lib.TreePlanInfo, "im_sparse_plan_info": _lib.SparsePlanInfo,
+        "im_muscle_force_model": _lib.MuscleForceModel, "im_muscle_force_velocity_model": _lib.MuscleForceVelocityModel,
+        "im_newton_args": _lib.NewtonArgs, "im_row_pair_term": _lib.RowPairTerm, "im_muscle_geometry": _lib.MuscleGeometry,
+        "im_muscle_segments": _lib.MuscleSegments, "im_muscle_entries": _lib.MuscleEntries,
+        "im_body_wrenches": _lib.BodyWrenches, "im_wrench_topology": _lib.WrenchTopology,
+    }  # fmt: skip
+    lines = ["#include <stddef.h>", "#include <stdio.h>", '#include "imhip.h"', "int main(void) {"]
+    for cname, ctype in pairs.items():
+        lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
+        for field, _ in ctype._fields_:
+            lines.append(f'  printf("{cname}.{field} %zu\\n", offsetof({cname}, {field}));')
+    lines += ["  return 0;", "}"]
+    src, exe = tmp_path / "probe.c", tmp_path / "probe"
+    src.write_text("\n".join(lines))
+    include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    subprocess.run(["gcc", "-std=c11", "-I", include, str(src), "-o", str(exe)], check=True)
+    seen = dict(line.split() for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    for cname, ctype in pairs.items():
+        assert int(seen[cname]) == C.sizeof(ctype), cname
+        for field, _ in ctype._fields_:
+            assert int(seen[f"{cname}.{field}"]) == getattr(ctype, field).offset, f"{cname}.{field}"
