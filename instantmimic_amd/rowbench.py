@@ -210,6 +210,32 @@ def run(launches: int = 32, only: str | None = None) -> None:
                     os.environ.pop("IMHIP_TREE_KERNEL", None)
                 sec = _timeit(torch, lambda i: T.assemble_tree_factor_solve(sc, *S[i], X[i]), 8, launches)
                 _line(f"im_assemble_tree_ldl_solve ({kind} kernel)", wl, sec, bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv), nworld=nworld)
+            if nv > 64:
+                # the same assemble + factor + solve on the static sparse pattern and on the dense matrix:
+                # the sizes at which the reference's sparse path is its fastest (sparse_hessian.py:179-183)
+                model = synth.model_from_parents(list(parents))
+                pad = int(model.nv_pad)
+                plan, why = SH.plan_for_model(model, None, [], SH.block_width(pad), device=dev)
+                if plan is not None:
+                    launch = SH.init_factor_kernel(plan)
+                    hf = torch.zeros((nworld, plan.nv_pad, plan.nv_pad), device=dev)
+                    search = torch.zeros((nworld, nv, 1), device=dev)
+                    sd, de = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev)
+                    G = [s_[5][:, :, None].contiguous() for s_ in S]
+                    sec = _timeit(torch, lambda i: launch(None, S[i][4], S[i][1], S[i][2], S[i][3], S[i][0], G[i], hf, search, sd, de), 8, launches)
+                    _line("im_sparse_init_factor (workgroup per world: beyond 64 dofs)", wl, sec,
+                          bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv + 2 * plan.nfac + nv + 2), nworld=nworld)  # fmt: skip
+                    del hf, G
+                else:
+                    print(json.dumps({"kernel": "im_sparse_init_factor", "workload": wl, "refused": why}), flush=True)
+                Md = [t(synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32).reshape(nworld, -1)) for _ in range(2)]
+                Hd = torch.zeros((nworld, pad, pad), device=dev)
+                padU = -(-nv // 16) * 16
+                Ud = torch.zeros((nworld, padU, padU), device=dev)
+                sec = _timeit(torch, lambda i: BD.dense_hessian_factor_solve(Md[i % 2], S[i][1], S[i][2], S[i][3], S[i][4], Hd, S[i][5], X[i], factor=Ud), 8, launches)
+                _line("im_jtdj_factor_solve (dense J'DJ + blocked factor + solve)", wl, sec,
+                      bytes_=nworld * 4 * (nv * nv + nefc * nv + 2 * nefc + 2 * nv + pad * pad + padU * padU), nworld=nworld)  # fmt: skip
+                del Md, Hd, Ud
             del S, X
             torch.cuda.empty_cache()
 
