@@ -960,7 +960,9 @@ typedef struct im_newton_args {
  * their order, so the arrays end as after those launches repeated, bit for bit.  No host
  * synchronisation, nothing allocated; the loop is bounded by `iterations` whatever the data.
  * Needs generated kernels on the plan (IM_ERR_UNSUPPORTED otherwise: the caller then issues the
- * stages one by one). */
+ * stages one by one).  The launch holds as many workgroups as the chip keeps resident; a wavefront
+ * whose world is done takes the next world through a counter that belongs to the plan, so two solves
+ * with one plan must not overlap on the GPU. */
 int im_newton_solve_tree(const im_tree_plan *plan, const im_newton_args *args, void *stream);
 
 /* The same resident loop with the static-pattern sparse stage of im_sparse_update_factor as its

@@ -209,7 +209,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     # the body as a function: the kernels at the end of the file call it, the resident Newton
     # kernel once per iteration
     emit("template <bool ASM, bool LONG>")
-    emit(f"__device__ __forceinline__ void tree_row16_body_{name}(IM_ROW16_PARAMS) {{")
+    # world_of: null, or four world numbers in LDS, one per wavefront / 16-lane row, in place of the
+    # workgroup's own four (the resident Newton loop hands finished wavefronts new worlds; a number
+    # at or past nworld stands for no world)
+    emit(f"__device__ __forceinline__ void tree_row16_body_{name}(IM_ROW16_PARAMS, const int *world_of) {{")
     # the lane number as a value the compiler cannot see through: called from a loop (the resident
     # Newton kernel), nothing derived from it counts as loop-invariant, so no table entry or address
     # of this body is kept in a register from one call to the next
@@ -227,7 +230,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("    if (bid * 4 >= nworld) return;  // the grid is rounded up to whole rounds of the XCDs")
     emit("    state += it * state_it; y += it * y_it; x += it * x_it;")
     emit("  }")
-    emit("  const int w = bid * 4 + (lane >> 4);")
+    emit("  const int w = world_of ? world_of[lane >> 4] : bid * 4 + (lane >> 4);")
     emit("  const int64_t ws = w < nworld ? w : nworld - 1;")
     # a world whose `skip` byte is set is read and worked on like its neighbours (a wavefront's
     # four worlds share every instruction) and nothing of it is stored
@@ -348,7 +351,8 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("    const int kq = lane >> 4;")
     emit("    const int njp = (njmax + 15) & ~15;")
     emit(f"    float *dcl = lds + {lds_floats} + wv * (LONG ? 2 * njp : 128);  // D per listed row, and the list of rows behind it")
-    emit("    const int64_t wq = bid * 4 + wv < nworld ? bid * 4 + wv : nworld - 1;")
+    emit("    const int wq_ = world_of ? __builtin_amdgcn_readfirstlane(world_of[wv]) : bid * 4 + wv;")
+    emit("    const int64_t wq = wq_ < nworld ? wq_ : nworld - 1;")
     emit("    int ne = nefc_p ? nefc_p[wq] : njmax; ne = ne < njmax ? ne : njmax;")
     emit("    ne = __builtin_amdgcn_readfirstlane(ne);")
     # every load below is unconditional (clamped address, value selected afterwards): a load
@@ -893,10 +897,11 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("template <bool LONG>")
     emit(f"__device__ __forceinline__ void newton_row16_body_{name}(const im::resident::NewtonArgs &a) {{")
     emit("  extern __shared__ float xlds[];")
+    emit("  const int *worlds = (const int *)(xlds + a.stage_lds_floats) + 4;  // behind the four votes (coop_layout)")
     emit("  auto stage = [&]() __attribute__((always_inline)) {")
     emit("    const im::resident::NewtonArgs &a = im::resident::kernel_args(0);  // the kernel's only argument")
     emit(f"    tree_row16_body_{name}<true, LONG>(a.M, a.ldM, a.J, a.njmax, a.D, a.state, a.nefc, a.quad, a.grad, a.ld_grad, a.search,")
-    emit("        (int64_t)a.nv, nullptr, a.nworld, IM_FLAG_NEGATE, 1, 0, 0, 0, a.unchanged);")
+    emit("        (int64_t)a.nv, nullptr, a.nworld, IM_FLAG_NEGATE, 1, 0, 0, 0, a.unchanged, worlds);")
     emit("  };")
     emit("  const im::resident::LoopLds L = im::resident::coop_layout(a, xlds);")
     emit("  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);")
@@ -908,7 +913,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
         for kernel, asm_, long_, bounds in (("fused", "true", "false", f"256, IM_OCC_{name}"), ("fused_long", "true", "true", f"256, IM_OCC_{name}"),
                                             ("solve", "false", "false", "64, 1")):  # fmt: skip
             emit(f'extern "C" __global__ __launch_bounds__({bounds}) void im_row16_{kernel}(IM_ROW16_PARAMS) {{')
-            emit(f"  im::gen::tree_row16_body_{name}<{asm_}, {long_}>({args});")
+            emit(f"  im::gen::tree_row16_body_{name}<{asm_}, {long_}>({args}, nullptr);")
             emit("}")
         for kernel, long_ in (("newton", "false"), ("newton_long", "true")):
             emit(f'extern "C" __global__ __launch_bounds__(256, IM_NOCC_{name}) void im_row16_{kernel}(im::resident::NewtonArgs a) {{')
@@ -919,7 +924,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     else:
         emit("template <bool ASM, bool LONG>")
         emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? IM_OCC_{name} : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
-        emit(f"  tree_row16_body_{name}<ASM, LONG>({args});")
+        emit(f"  tree_row16_body_{name}<ASM, LONG>({args}, nullptr);")
         emit("}")
         emit("template <bool LONG>")
         emit(f"__global__ __launch_bounds__(256, IM_NOCC_{name}) void newton_row16_{name}(im::resident::NewtonArgs a) {{")

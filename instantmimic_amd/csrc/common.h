@@ -60,6 +60,7 @@ struct im_tree_plan {
   void *row16_own = nullptr;
   // whether the resident Newton kernels of row16 keep to registers (short / long variant)
   bool resident_ok = false, resident_long_ok = false;
+  int *next_world = nullptr;  // device int behind dev_blob's tables: the resident Newton kernel's counter of worlds handed out
   // false for 65 to 96 dofs: the table-driven kernel keeps a dof per lane and ancestors in 64-bit
   // masks, so such a plan runs on generated kernels only (device_ready, nothing launched before
   // kernels are attached)

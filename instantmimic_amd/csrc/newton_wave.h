@@ -43,6 +43,10 @@ struct NewtonArgs {
   int ld_ids;
   uint8_t *done, *exhausted, *unchanged;
   int stage_lds_floats;  // dynamic LDS the factor stage uses from offset 0; the loop's own arrays follow
+  // cooperative loop: a counter in memory, set to four times the grid's workgroups before the launch,
+  // from which a wavefront whose world is done takes the next world nobody has started (null: a
+  // workgroup keeps to its own four worlds)
+  int *next_world;
 };
 
 // The public argument block checked and turned into the kernels' (host side).
@@ -77,6 +81,7 @@ inline int convert_args(const im_newton_args &p, int nv, int nM, NewtonArgs &a) 
   a.state_count = p.state_changed_count, a.niter = p.solver_niter, a.overflow = p.overflow, a.nsolving = p.nsolving;
   a.ld_ids = p.ld_ids, a.done = p.done, a.exhausted = p.ls_exhausted, a.unchanged = p.search_unchanged;
   a.stage_lds_floats = 0;
+  a.next_world = nullptr;
   return IM_OK;
 }
 
@@ -107,7 +112,7 @@ __device__ __forceinline__ void block_sync() {
 // words a wavefront keeps from round to round: M, the search direction, Ma, mv, qacc; Jaref, jv, D, friction losses
 __host__ __device__ inline size_t kept_words(int nv, int njmax, int nM) { return (size_t)nM + 4 * (size_t)nv + 4 * (size_t)njmax; }
 __host__ __device__ inline size_t loop_lds_words(int nv, int njmax, int nM, int nterm) {
-  return 4 + (size_t)nterm + nv + 1 + 4 * (kept_words(nv, njmax, nM) + 2 * (size_t)njmax + nv);
+  return 8 + (size_t)nterm + nv + 1 + 4 * (kept_words(nv, njmax, nM) + 2 * (size_t)njmax + nv);
 }
 __host__ __device__ inline size_t staged_rows_words(int) { return 4 * 64 * 17; }  // four wavefronts' tiles of J
 
@@ -327,6 +332,7 @@ __device__ __forceinline__ void jv_world_tiled(const NewtonArgs &a, const float 
 // Where the loop's arrays lie in LDS (set up by the kernel around it).
 struct LoopLds {
   int *votes;            // [4] cooperative stage only
+  int *worlds;           // [4] cooperative stage only: the world of each wavefront (nworld: none), read by the stage
   const uint32_t *term;  // [nterm] col | madr << 16, shared by the workgroup
   const int *radr;       // [nv + 1]
   // per wavefront, kept from round to round:
@@ -348,8 +354,10 @@ struct LoopLds {
 // HELD: rows of a world a lane keeps in registers during the line search (0: read from LDS at every
 // evaluation); JU: loads in flight per lane while rows of J are staged, 0 for the tiled staging.
 // COOP: `stage()` works on the workgroup's four worlds together (every wavefront calls it in step,
-// between two workgroup barriers; it skips the worlds whose `unchanged` byte is set), and a world
-// that is done idles through the barriers until the workgroup's last world finishes.  Otherwise
+// between two workgroup barriers; it takes the worlds' numbers from L.worlds and skips the worlds
+// whose `unchanged` byte is set).  A wavefront whose world is done takes the next world from the
+// counter a.next_world (or, without one, idles through the barriers); the workgroup leaves when all
+// four are idle.  Otherwise
 // `stage()` is the wavefront's own world's stage (it leaves search_dot and newton_decrement in
 // memory itself), called only when that world needs it, and a wavefront leaves as soon as its world
 // is done.  `w_raw`: the wavefront's world.
@@ -375,51 +383,80 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
   const NewtonArgs &a = a0;
   const int lane_fixed = threadIdx.x & 63;
   const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  // the world's number as a scalar: every address below is a scalar base plus a lane offset
-  const int w_lo = __builtin_amdgcn_readfirstlane((int)(w_raw & 0xffffffff)), w_hi = __builtin_amdgcn_readfirstlane((int)(w_raw >> 32));
-  const int64_t w_uniform = ((int64_t)w_hi << 32) | (uint32_t)w_lo;
-  const bool live = w_uniform < a.nworld;
-  const int64_t w = live ? w_uniform : (int64_t)a.nworld - 1;
   const int nv = a.nv, njmax = a.njmax;
-  bool done = !live || a.done[w] != 0;
-  if (live && done && lane_fixed == 0) a.unchanged[w] = 1;  // the factor stage leaves such a world alone
-  bool unchanged = !done && a.unchanged[w] != 0;
-  int nefc = a.nefc ? a.nefc[w] : njmax;
-  nefc = __builtin_amdgcn_readfirstlane(nefc < njmax ? nefc : njmax);
-  const int ne = __builtin_amdgcn_readfirstlane(a.ne ? a.ne[w] : 0), nf = __builtin_amdgcn_readfirstlane(a.nf ? a.nf[w] : 0);
-  const float *Jw = a.J + w * (int64_t)njmax * nv;
-  const float tolerance = a.tolerance[w % a.ntolerance], ls_tolerance = a.ls_tolerance[w % a.nls_tolerance];
-  const float meaninertia = a.meaninertia[w % a.nmeaninertia];
-  Scalars sc{uniform(a.search_dot[w]), uniform(a.grad_dot[w]), uniform(a.decrement[w]), uniform(a.grad_scale[w]),
-             uniform(a.alpha[w]), uniform(a.improvement[w]), __builtin_amdgcn_readfirstlane(a.niter[w])};
-  // what the loop keeps: M, Ma, Jaref into LDS (mv and jv are formed before they are read: a world
-  // enters with a new search direction unless it is done) and qacc
-  if constexpr (MLDS)
-    for (int k = lane_fixed; k < a.nM; k += 64) L.m_lds[k] = a.M[w * a.ldM + k];
-  for (int k = lane_fixed; k < nv; k += 64) {
-    L.Ma[k] = a.Ma[w * nv + k];
-    L.mv[k] = a.mv[w * nv + k];
-    L.qacc[k] = a.qacc[w * nv + k];
-  }
-  for (int r = lane_fixed; r < njmax; r += 64) {
-    L.Jaref[r] = a.Jaref[w * njmax + r];
-    L.jv[r] = a.jv[w * njmax + r];
-    L.D[r] = a.D[w * njmax + r];
-    L.fl[r] = a.frictionloss ? a.frictionloss[w * njmax + r] : 0.0f;
-  }
-  wave_sync();
+  // what belongs to the wavefront's current world
+  int64_t w = 0;
+  bool live = false, done = true, unchanged = false;
+  int nefc = 0, ne = 0, nf = 0, budget = 0;
+  const float *Jw = a.J;
+  float tolerance = 0.0f, ls_tolerance = 0.0f, meaninertia = 1.0f;
+  Scalars sc{};
+  auto enter = [&](int64_t w_raw) __attribute__((always_inline)) {
+    const NewtonArgs &a = kernel_args(kernarg_offset);
+    // the world's number as a scalar: every address below is a scalar base plus a lane offset
+    const int w_lo = __builtin_amdgcn_readfirstlane((int)(w_raw & 0xffffffff)), w_hi = __builtin_amdgcn_readfirstlane((int)(w_raw >> 32));
+    const int64_t w_uniform = ((int64_t)w_hi << 32) | (uint32_t)w_lo;
+    live = w_uniform < a.nworld;
+    w = live ? w_uniform : (int64_t)a.nworld - 1;
+    done = !live || a.done[w] != 0;
+    if (live && done && lane_fixed == 0) a.unchanged[w] = 1;  // the factor stage leaves such a world alone
+    unchanged = !done && a.unchanged[w] != 0;
+    nefc = a.nefc ? a.nefc[w] : njmax;
+    nefc = __builtin_amdgcn_readfirstlane(nefc < njmax ? nefc : njmax);
+    ne = __builtin_amdgcn_readfirstlane(a.ne ? a.ne[w] : 0), nf = __builtin_amdgcn_readfirstlane(a.nf ? a.nf[w] : 0);
+    Jw = a.J + w * (int64_t)njmax * nv;
+    tolerance = a.tolerance[w % a.ntolerance], ls_tolerance = a.ls_tolerance[w % a.nls_tolerance];
+    meaninertia = a.meaninertia[w % a.nmeaninertia];
+    sc = Scalars{uniform(a.search_dot[w]), uniform(a.grad_dot[w]), uniform(a.decrement[w]), uniform(a.grad_scale[w]),
+                 uniform(a.alpha[w]), uniform(a.improvement[w]), __builtin_amdgcn_readfirstlane(a.niter[w])};
+    budget = a.maxiter;  // rounds this wavefront gives the world, whatever the data
+    if (done) return;
+    // what the loop keeps: M, Ma, Jaref into LDS (mv and jv are formed before they are read: a world
+    // enters with a new search direction unless it is done) and qacc
+    if constexpr (MLDS)
+      for (int k = lane_fixed; k < a.nM; k += 64) L.m_lds[k] = a.M[w * a.ldM + k];
+    for (int k = lane_fixed; k < nv; k += 64) {
+      L.Ma[k] = a.Ma[w * nv + k];
+      L.mv[k] = a.mv[w * nv + k];
+      L.qacc[k] = a.qacc[w * nv + k];
+    }
+    for (int r = lane_fixed; r < njmax; r += 64) {
+      L.Jaref[r] = a.Jaref[w * njmax + r];
+      L.jv[r] = a.jv[w * njmax + r];
+      L.D[r] = a.D[w * njmax + r];
+      L.fl[r] = a.frictionloss ? a.frictionloss[w * njmax + r] : 0.0f;
+    }
+    wave_sync();
+  };
+  enter(w_raw);
+  bool queue_empty = !(COOP && a0.next_world);
 #ifdef IM_NEWTON_STAMPS  // development aid: time per phase, summed over the rounds, left in the world's row of jv
   long long t_phase[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t_last = wall_clock64();
 #define IM_STAMP(k) do { const long long t_now = wall_clock64(); t_phase[k] += t_now - t_last; t_last = t_now; } while (0)
 #else
 #define IM_STAMP(k) do {} while (0)
 #endif
-  // every wavefront leaves the loop after at most maxiter rounds, whatever the data
-  const int maxiter = a0.maxiter;
-  for (int round = 0; round < maxiter; ++round) {
+  // Every world gets at most maxiter rounds of its wavefront, whatever the data, and the counter of
+  // worlds only grows: every wavefront leaves the loop.
+  for (;;) {
     const NewtonArgs &a = kernel_args(kernarg_offset);  // read afresh in every round
     if (COOP) {
-      if (lane_fixed == 0) L.votes[wv] = done ? 0 : 1;
+      // a wavefront without a world to work on takes the next one nobody has started; the other
+      // wavefronts' worlds go on with their own rounds beside it (the stage does not care which
+      // iteration a world is in)
+      while (done && !queue_empty) {
+        int next = 0;
+        if (lane_fixed == 0) next = atomicAdd(a.next_world, 1);
+        next = __builtin_amdgcn_readfirstlane(next);
+        if (next < a.nworld)
+          enter(next);
+        else
+          queue_empty = true;
+      }
+      if (lane_fixed == 0) {
+        L.votes[wv] = done ? 0 : 1;
+        L.worlds[wv] = done ? a.nworld : (int)w;
+      }
       block_sync();
       if (!(L.votes[0] | L.votes[1] | L.votes[2] | L.votes[3])) break;  // the workgroup's four worlds are done
     } else if (done) {
@@ -552,7 +589,8 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
           if (a.nsolving) atomicAdd(a.nsolving, -1);
         }
       }
-      done = finished;
+      budget -= 1;
+      done = finished || budget <= 0;
     }
     IM_STAMP(7);
   }
@@ -570,7 +608,8 @@ __device__ __forceinline__ LoopLds coop_layout(const NewtonArgs &a, float *lds) 
   const int nv = a.nv, njmax = a.njmax, nM = a.nM;
   LoopLds L;
   L.votes = (int *)(lds + a.stage_lds_floats);
-  uint32_t *term = (uint32_t *)(L.votes + 4);
+  L.worlds = L.votes + 4;
+  uint32_t *term = (uint32_t *)(L.worlds + 4);
   int *radr = (int *)(term + a.nterm);
   float *mine = (float *)(radr + nv + 1) + wv * (kept_words(nv, njmax, nM) + 2 * njmax + nv);
   L.term = term, L.radr = radr;

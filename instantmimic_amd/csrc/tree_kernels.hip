@@ -559,9 +559,10 @@ int tree_plan_upload(im_tree_plan *pl) {
   std::memcpy(blob.data() + o_col, pl->colind.data(), (size_t)nM * 4);
   std::memcpy(blob.data() + o_rel, related.data(), 64 * sizeof(uint64_t));
   IM_HIP_CHECK(hipGetDevice(&pl->device));
-  IM_HIP_CHECK(hipMalloc(&pl->dev_blob, off));
+  IM_HIP_CHECK(hipMalloc(&pl->dev_blob, off + 16));
   IM_HIP_CHECK(hipMemcpy(pl->dev_blob, blob.data(), off, hipMemcpyHostToDevice));
   char *base = (char *)pl->dev_blob;
+  pl->next_world = (int *)(base + off);
   pl->dev.steps = (const int4 *)(base + o_steps);
   pl->dev.anc = (const uint64_t *)(base + o_anc);
   pl->dev.slot_e = (const int32_t *)(base + o_se);
@@ -603,6 +604,10 @@ int tree_plan_upload(im_tree_plan *pl) {
   return IM_OK;
 }
 
+}  // namespace im
+
+namespace im {
+__global__ void set_world_counter_kernel(int *counter, int value) { *counter = value; }
 }  // namespace im
 
 extern "C" {
@@ -782,7 +787,27 @@ int im_newton_solve_tree(const im_tree_plan *plan, const im_newton_args *p, void
   const bool is_long = njmax > e->short_rows;
   if (!(is_long ? plan->resident_long_ok : plan->resident_ok)) return IM_ERR_UNSUPPORTED;  // the kernel spills registers
   const void *fn = is_long ? e->newton_long : e->newton;
-  const unsigned grid = (unsigned)((p->nworld + 3) / 4);
+  // As many workgroups as the chip keeps resident (registers and LDS); a wavefront whose world is
+  // done takes the next world through the plan's counter, so the worlds that need many iterations
+  // do not hold three idle wavefronts in place.
+  int per_cu = 0;
+  if (plan->module) {
+    IM_HIP_CHECK(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (hipFunction_t)fn, 256, lds));
+  } else {
+    IM_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, lds));
+  }
+  static int ncu = 0;
+  if (!ncu) {
+    int dev = 0;
+    IM_HIP_CHECK(hipGetDevice(&dev));
+    IM_HIP_CHECK(hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev));
+  }
+  const int needed = (p->nworld + 3) / 4;
+  const unsigned grid = (unsigned)std::min(needed, std::max(1, per_cu) * std::max(1, ncu));
+  if ((int)grid < needed) {  // (a batch that is resident all at once has nothing to hand out)
+    a.next_world = plan->next_world;
+    hipLaunchKernelGGL(im::set_world_counter_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, plan->next_world, (int)grid * 4);
+  }
   void *args[] = {&a};
   if (plan->module)
     IM_HIP_CHECK(hipModuleLaunchKernel((hipFunction_t)fn, grid, 1, 1, 256, 1, 1, (unsigned)lds, (hipStream_t)stream, args,
