@@ -87,6 +87,24 @@ __device__ __forceinline__ float lanes_sum(float s) {
   return s + 0.0f;
 }
 __device__ __forceinline__ Pt lanes_sum(Pt p) { return {lanes_sum(p.c), lanes_sum(p.g), lanes_sum(p.h)}; }
+// The same tree with the sums of both halves of the wavefront handed to every lane: `lower` that of
+// lanes 0 - 31, `upper` that of lanes 32 - 63 (for a wavefront whose halves sum different things).
+__device__ __forceinline__ void lanes_sum_halves(float s, float &lower_sum, float &upper_sum) {
+  unsigned upper = __builtin_bit_cast(unsigned, s), lower = upper;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lower), "+v"(upper));
+  s = s + __builtin_bit_cast(float, upper);
+  s = s + row_shl<8>(s);
+  s = s + row_shl<4>(s);
+  s = s + row_shl<2>(s);
+  s = s + row_shl<1>(s);
+  lower_sum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s), 0)) + 0.0f;
+  upper_sum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s), 32)) + 0.0f;
+}
+__device__ __forceinline__ void lanes_sum_halves(Pt p, Pt &lower_sum, Pt &upper_sum) {
+  lanes_sum_halves(p.c, lower_sum.c, upper_sum.c);
+  lanes_sum_halves(p.g, lower_sum.g, upper_sum.g);
+  lanes_sum_halves(p.h, lower_sum.h, upper_sum.h);
+}
 
 struct SearchArgs {
   const float *tolerance, *ls_tolerance, *meaninertia;
@@ -116,7 +134,10 @@ struct LsResult {
 // of the world a lane keeps in registers (weight, friction loss, Jaref, jv and the cost at alpha 0)
 // -- every candidate step evaluates every row, three candidates per round; 0: more rows than that,
 // read at every evaluation.  Every lane of the group returns the same result.
-template <int HELD>
+// SPLIT: both halves of the wavefront work on the same world (each with `lane` = 0 .. 31): of a
+// round's three candidate steps the lower half evaluates the first and the upper half the second
+// (each sum is still one group's 32-lane tree), both evaluate the third.
+template <int HELD, bool SPLIT = false>
 __device__ __forceinline__ LsResult linesearch_rows(const LsWorld &wd, int lane) {
   const int nv = wd.nv, ne = wd.ne, nf = wd.nf, nefc = wd.nefc;
   const float *D = wd.D, *fl = wd.frictionloss, *Jaref = wd.Jaref, *jv = wd.jv;
@@ -202,14 +223,29 @@ __device__ __forceinline__ LsResult linesearch_rows(const LsWorld &wd, int lane)
       const float hi_next_alpha = hi_alpha - safe_div(hi.g, hi.h);
       const float mid_alpha = 0.5f * (lo_alpha + hi_alpha);
       Pt s_lo = {0.0f, 0.0f, 0.0f}, s_hi = s_lo, s_mid = s_lo;
-      rows_sum([&](bool fr, float d, float f, float ja, float v, float c0) {
-        s_lo = s_lo + row_point_from(fr, d, f, ja, v, c0, lo_next_alpha);
-        s_hi = s_hi + row_point_from(fr, d, f, ja, v, c0, hi_next_alpha);
-        s_mid = s_mid + row_point_from(fr, d, f, ja, v, c0, mid_alpha);
-      });
-      const Pt lo_next = eval_pt(gauss, lo_next_alpha) + lanes_sum(s_lo);
-      const Pt hi_next = eval_pt(gauss, hi_next_alpha) + lanes_sum(s_hi);
-      const Pt mid = eval_pt(gauss, mid_alpha) + lanes_sum(s_mid);
+      Pt lo_next, hi_next, mid;
+      if constexpr (SPLIT) {
+        const float mine_alpha = (threadIdx.x & 32) ? hi_next_alpha : lo_next_alpha;
+        rows_sum([&](bool fr, float d, float f, float ja, float v, float c0) {
+          s_lo = s_lo + row_point_from(fr, d, f, ja, v, c0, mine_alpha);
+          s_mid = s_mid + row_point_from(fr, d, f, ja, v, c0, mid_alpha);
+        });
+        Pt rows_lo, rows_hi, rows_mid, same;
+        lanes_sum_halves(s_lo, rows_lo, rows_hi);
+        lanes_sum_halves(s_mid, rows_mid, same);
+        lo_next = eval_pt(gauss, lo_next_alpha) + rows_lo;
+        hi_next = eval_pt(gauss, hi_next_alpha) + rows_hi;
+        mid = eval_pt(gauss, mid_alpha) + rows_mid;
+      } else {
+        rows_sum([&](bool fr, float d, float f, float ja, float v, float c0) {
+          s_lo = s_lo + row_point_from(fr, d, f, ja, v, c0, lo_next_alpha);
+          s_hi = s_hi + row_point_from(fr, d, f, ja, v, c0, hi_next_alpha);
+          s_mid = s_mid + row_point_from(fr, d, f, ja, v, c0, mid_alpha);
+        });
+        lo_next = eval_pt(gauss, lo_next_alpha) + lanes_sum(s_lo);
+        hi_next = eval_pt(gauss, hi_next_alpha) + lanes_sum(s_hi);
+        mid = eval_pt(gauss, mid_alpha) + lanes_sum(s_mid);
+      }
       const bool conv_lo = fabsf(lo_next.g) < gtol_accept && lo_next.c < 0.0f;
       const bool conv_hi = fabsf(hi_next.g) < gtol_accept && hi_next.c < 0.0f;
       const bool conv_mid = fabsf(mid.g) < gtol_accept && mid.c < 0.0f;

@@ -481,7 +481,7 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
       IM_STAMP(1);
       const search::LsWorld lw{a.smooth + w * nv, L.D, L.fl, L.Jaref, L.sv, L.mv, L.jv, L.Ma, sc.search_dot, tolerance,
                                ls_tolerance, meaninertia, ne, nf, nefc, nv, a.ls_iterations};
-      const search::LsResult ls = search::linesearch_rows<HELD>(lw, lane & 31);
+      const search::LsResult ls = search::linesearch_rows<HELD, true>(lw, lane & 31);  // both halves on this world
       sc.alpha = uniform(ls.alpha), sc.improvement = uniform(ls.improvement);
       if (lane == 0) {
         a.alpha[w] = ls.alpha;
