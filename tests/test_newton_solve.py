@@ -156,3 +156,33 @@ def test_gpu_solve_from_init_context_matches_the_oracle_chain(device, monkeypatc
     assert all(taken) == (loop == "resident") and len(taken) > 0
     NC.compare(p, s, d, ctx)
     assert int(nsolving.item()) == int((p.nefc == 0).sum())  # every world that had rows has reported done
+
+
+def _floating_chain(nv: int, limbs: int = 1):
+    """A free body and hinges behind it (the reference's layout-boundary models,
+    tests/test_mjw_newton_fusion.py:100-131): ``nv`` dofs, one chain or ``limbs`` chains off the
+    free body's last dof."""
+    parents = [-1, 0, 1, 2, 3, 4]
+    tips = [5] * limbs
+    for k in range(6, nv):
+        parents.append(tips[k % limbs])
+        tips[k % limbs] = k
+    return tuple(parents[:nv])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("nv,stage", [(13, "dense"), (16, "dense"), (17, "dense"), (31, "dense"), (32, "dense"), (33, "dense"),
+                                      (48, "dense"), (49, "dense"), (63, "dense"), (64, "dense"), (17, "tree"), (33, "tree"), (49, "tree")])  # fmt: skip
+def test_gpu_solve_at_layout_boundaries(device, monkeypatch, nv, stage):
+    """Dof counts on both sides of the padded layouts' boundaries (16, 32, 48, 64: the single tile up
+    to 32 dofs and the blocked factor beyond on the dense stage; kernels generated on the spot on the
+    tree stage), as the reference checks its captured solve there (tests/test_mjw_newton_fusion.py
+    :257-283)."""
+    name = f"chain{nv}"
+    parents = _floating_chain(nv, 3 if stage == "tree" else 1)  # (a single chain's M is dense: the tree factor declines it)
+    monkeypatch.setitem(synth.SHAPES, name, synth.Shape(name, parents, 40, 64, (0.5, 8.0), 0.02, (-4.0, 4.0), 0.6, 1, 1100 + nv))
+    p = NC.problem(name, 37, stage, empty_every=9, maxiter=12)
+    s = NC.oracle_solve(p)
+    assert s.done.all()
+    m, d, ctx, nsolving = _solve_on_gpu(p, device, graph=True)
+    NC.compare(p, s, d, ctx)
