@@ -143,8 +143,21 @@ def _compile(src: str) -> str:
     # resident Newton kernels get fewer workgroups per CU, one at a time, while they spill.
     from .codegen import tree_row16
 
-    name, occ = tree_row16.occupancy_of(open(src).read())
-    for newton_occ in range(occ, 0, -1):
+    import hashlib
+
+    text = open(src).read()
+    name, occ = tree_row16.occupancy_of(text)
+    # the occupancy that an earlier build of the same source and headers settled on is tried first
+    stamp = hashlib.sha256(text.encode())
+    for d in sorted(deps[1:]):
+        stamp.update(open(d, "rb").read())
+    note = obj + ".nocc"
+    first = occ
+    if os.path.exists(note):
+        saved = open(note).read().split()
+        if len(saved) == 2 and saved[0] == stamp.hexdigest() and saved[1].isdigit():
+            first = max(1, min(occ, int(saved[1])))
+    for newton_occ in range(first, 0, -1):
         extra = [] if newton_occ == occ else [f"-DIM_NOCC_{name}={newton_occ}"]
         done = subprocess.run([*cmd, *extra, "-Rpass-analysis=kernel-resource-usage"], capture_output=True, text=True)
         if done.returncode != 0:
@@ -156,6 +169,8 @@ def _compile(src: str) -> str:
             raise RuntimeError(f"{os.path.basename(src)}: fused kernels spill registers to memory: {spilling}")
         if not _spilling_kernels(done.stderr, fused=False):
             break
+    with open(note, "w") as f:
+        f.write(f"{stamp.hexdigest()} {newton_occ}\n")
     return obj
 
 
