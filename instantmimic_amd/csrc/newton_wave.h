@@ -203,6 +203,9 @@ struct Scalars {
 // For a world whose states changed: qfrc_constraint = J' force over the listed rows (`cnt` rows with
 // a nonzero force, ascending, in f / rowl), grad = Ma - qfrc_smooth - qfrc_constraint, grad . grad.
 // Otherwise the rescaling of the three scalars.  Returns whether the search direction stays.
+// AHEAD: the next rows' elements are asked for before the current ones are added (ROWS more
+// registers a lane).
+template <bool AHEAD>
 __device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, const float *Jw, bool changed, int cnt,
                                                const float *f, const int *rowl, const float *Ma_l, float *gl, Scalars &sc,
                                                int lane) {
@@ -230,12 +233,22 @@ __device__ __forceinline__ bool gradient_world(const NewtonArgs &a, int64_t w, c
   for (int dof = lane; dof < nv; dof += 64) {
     const float ma = Ma_l[dof], sm = a.smooth[w * nv + dof];
     float sum = 0.0f;
-    for (int p0 = 0; p0 < cnt; p0 += ROWS) {
-      float jv[ROWS];
+    // the next ROWS rows' elements are asked for before the current ones are added
+    float jv[ROWS], jn[ROWS];
+    auto fetch = [&](int p0, float (&v)[ROWS]) __attribute__((always_inline)) {
 #pragma unroll
-      for (int u = 0; u < ROWS; ++u) jv[u] = Jw[(int64_t)rowl[p0 + u < cnt ? p0 + u : cnt - 1] * nv + dof];
+      for (int u = 0; u < ROWS; ++u) v[u] = Jw[(int64_t)rowl[p0 + u < cnt ? p0 + u : cnt - 1] * nv + dof];
+    };
+    if (AHEAD && cnt > 0) fetch(0, jv);
+    for (int p0 = 0; p0 < cnt; p0 += ROWS) {
+      if (!AHEAD) fetch(p0, jv);
+      if (AHEAD && p0 + ROWS < cnt) fetch(p0 + ROWS, jn);
 #pragma unroll
       for (int u = 0; u < ROWS; ++u) sum = p0 + u < cnt ? fma_(jv[u], f[p0 + u], sum) : sum;
+      if (AHEAD) {
+#pragma unroll
+        for (int u = 0; u < ROWS; ++u) jv[u] = jn[u];
+      }
     }
     const float g = ma - sm - sum;
     a.qfrc_constraint[w * nv + dof] = sum;
@@ -289,33 +302,70 @@ __device__ __forceinline__ void search_sums_world(const NewtonArgs &a, int64_t w
 // ---- J search through a tile of 64 rows x 16 dofs (4.3 KB of LDS whatever the width of J) ------
 // The same chain per row as jv_world: the dofs in order, the 20-dof partial sums of the reference's
 // rule beyond 50 dofs.  A lane loads 16 elements per tile, four rows of 64 bytes per instruction.
+// AHEAD: the next tile's elements are asked for while the current one is worked on (sixteen more
+// registers a lane).  WIDE: a tile row's operands are read eight at a time ahead of their part of
+// the chain (sixteen more again).
+template <bool AHEAD, bool WIDE>
 __device__ __forceinline__ void jv_world_tiled(const NewtonArgs &a, const float *Jw, int nefc, float *tile,
                                                const float *sv, float *jv, float *jv_lds, int lane) {
   const int nv = a.nv;
   const int c = lane & 15, rq = lane >> 4;
   const bool split = nv > 50;
+  // the 16 elements of a lane for the tile at (r0, c0); the next tile's are asked for while the
+  // current one is worked on, so the trips to memory of all but the first tile are hidden
+  auto fetch = [&](int r0, int c0, float (&v)[16]) __attribute__((always_inline)) {
+    const int rows = nefc - r0 < 64 ? nefc - r0 : 64, cw = nv - c0 < 16 ? nv - c0 : 16;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int r = rq + 4 * k;
+      v[k] = Jw[(int64_t)(r0 + (r < rows ? r : rows - 1)) * nv + c0 + (c < cw ? c : cw - 1)];
+    }
+  };
+  float v[16];
+  if (AHEAD && nefc > 0) fetch(0, 0, v);
   for (int r0 = 0; r0 < nefc; r0 += 64) {
     const int rows = nefc - r0 < 64 ? nefc - r0 : 64;
     float acc = 0.0f, p = 0.0f;
     for (int c0 = 0; c0 < nv; c0 += 16) {
       const int cw = nv - c0 < 16 ? nv - c0 : 16;
-      float v[16];
-#pragma unroll
-      for (int k = 0; k < 16; ++k) {
-        const int r = rq + 4 * k;
-        v[k] = Jw[(int64_t)(r0 + (r < rows ? r : rows - 1)) * nv + c0 + (c < cw ? c : cw - 1)];
-      }
+      if (!AHEAD) fetch(r0, c0, v);
 #pragma unroll
       for (int k = 0; k < 16; ++k) tile[(rq + 4 * k) * 17 + c] = v[k];
       wave_sync();
+      const bool more_columns = c0 + 16 < nv;
+      const int next_r0 = more_columns ? r0 : r0 + 64, next_c0 = more_columns ? c0 + 16 : 0;
+      if (AHEAD && next_r0 < nefc) fetch(next_r0, next_c0, v);
       if (lane < rows) {
+        // a tile row's operands are read eight at a time before their part of the chain (two waits
+        // per tile, not sixteen)
         const float *row = tile + lane * 17;
-        for (int i = 0; i < cw; ++i) {
-          if (split && (c0 + i) % 20 == 0 && c0 + i > 0) {
-            acc = acc + p;
-            p = 0.0f;
+        if constexpr (!WIDE) {  // the short form, for a kernel without registers to spare
+          for (int i = 0; i < cw; ++i) {
+            if (split && (c0 + i) % 20 == 0 && c0 + i > 0) {
+              acc = acc + p;
+              p = 0.0f;
+            }
+            p = fma_(row[i], sv[c0 + i], p);
           }
-          p = fma_(row[i], sv[c0 + i], p);
+        } else
+#pragma unroll
+        for (int h = 0; h < 16; h += 8) {
+          float x[8], y[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            x[i] = row[h + i];
+            y[i] = sv[c0 + (h + i < cw ? h + i : 0)];
+          }
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            if (h + i < cw) {  // the same for every lane
+              if (split && (c0 + h + i) % 20 == 0 && c0 + h + i > 0) {
+                acc = acc + p;
+                p = 0.0f;
+              }
+              p = fma_(x[i], y[i], p);
+            }
+          }
         }
       }
       wave_sync();  // the tile is read before the next one overwrites it
@@ -352,7 +402,9 @@ struct LoopLds {
 // every value as it is produced (the arrays end as after the stage launches) and is read again only
 // for what another wavefront or the factor stage has written there.
 // HELD: rows of a world a lane keeps in registers during the line search (0: read from LDS at every
-// evaluation); JU: loads in flight per lane while rows of J are staged, 0 for the tiled staging.
+// evaluation); JU: loads in flight per lane while rows of J are staged, 0 for the tiled staging
+// with the next tile asked for ahead and a tile row's operands read eight at a time, -2 with the
+// first of the two only, -1 with neither (each costs sixteen registers a lane).
 // COOP: `stage()` works on the workgroup's four worlds together (every wavefront calls it in step,
 // between two workgroup barriers; it takes the worlds' numbers from L.worlds and skips the worlds
 // whose `unchanged` byte is set).  A wavefront whose world is done takes the next world from the
@@ -475,7 +527,7 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
         if constexpr (JU > 0)
           jv_world<(JU > 0 ? JU : 1)>(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, L.jv, lane);
         else
-          jv_world_tiled(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, L.jv, lane);
+          jv_world_tiled<(JU == 0 || JU == -2), (JU == 0)>(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, L.jv, lane);
         wave_sync();
       }
       IM_STAMP(1);
@@ -548,7 +600,7 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
       }
       wave_sync();
       IM_STAMP(3);
-      unchanged = gradient_world(a, w, Jw, nstate != 0, cnt, L.f, L.rowl, L.Ma, L.gl, sc, lane);
+      unchanged = gradient_world<(JU == 0 || JU == -2)>(a, w, Jw, nstate != 0, cnt, L.f, L.rowl, L.Ma, L.gl, sc, lane);
       IM_STAMP(4);
     }
     if (COOP) {

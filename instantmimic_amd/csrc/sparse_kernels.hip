@@ -893,7 +893,9 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
                         (int)b.ld_grad, U_, uni_, b.search, b.search_dot, b.decrement, (int)w, threadIdx.x & 63);
   };
   while (w < nworld) {
-    resident::newton_loop<HELD, 0, false, false>(kArgsOffset, L, w, stage);  // HELD: 2 up to 64 rows, else 0
+    // HELD: 2 up to 64 rows, else 0; with eight or twelve wavefronts (up to three per SIMD, 168 registers each) there is
+    // room to ask for the next rows of J ahead
+    resident::newton_loop<HELD, ((WAVES == 8 || WAVES == 12) ? -2 : -1), false, false>(kArgsOffset, L, w, stage);
     int next = 0;
     if ((threadIdx.x & 63) == 0) next = atomicAdd(next_world, 1);
     w = __builtin_amdgcn_readfirstlane(next);
