@@ -31,10 +31,10 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the iterations kernel (3 solves x 4096 worlds) from two rocprofv3 --pmc
 # runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads
 # for a plain 64 MiB device copy in the same run; recorded in
-# profiles/tree_row16_humanoid_pmc.txt:  (18296.13 * 65536 / 32781.77 + 1344.0) KiB
-TRAFFIC_BYTES_PER_LAUNCH = int((18296.13 * 65536 / 32781.77 + 1344.0) * 1024)
-# the same for one launch of the single-solve kernel (4096 worlds):  (15566.19 * 65536 / 32781.77 + 448.0) KiB
-TRAFFIC_BYTES_PER_SINGLE_LAUNCH = int((15566.19 * 65536 / 32781.77 + 448.0) * 1024)
+# profiles/tree_row16_humanoid_pmc.txt:  (18296.13 * 65536 / 32781.84 + 1344.0) KiB
+TRAFFIC_BYTES_PER_LAUNCH = int((18296.13 * 65536 / 32781.84 + 1344.0) * 1024)
+# the same for one launch of the single-solve kernel (4096 worlds):  (15566.21 * 65536 / 32781.84 + 448.0) KiB
+TRAFFIC_BYTES_PER_SINGLE_LAUNCH = int((15566.21 * 65536 / 32781.84 + 448.0) * 1024)
 MIN_TIMED_LAUNCHES = 256  # the kernel duration is averaged over at least this many launches
 
 
