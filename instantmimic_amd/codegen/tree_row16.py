@@ -906,7 +906,14 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("  const im::resident::LoopLds L = im::resident::coop_layout(a, xlds);")
     emit("  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);")
     emit("  im::resident::block_sync();")
-    emit("  im::resident::newton_loop<(LONG ? 0 : 2), 0, true>(0, L, w, stage);")
+    # rows a lane keeps in registers during the line search: two up to 64 rows, four up to 128 (the
+    # same for the whole launch), beyond that the rows are read from LDS at every evaluation
+    emit("  if (!LONG)")
+    emit("    im::resident::newton_loop<2, 0, true>(0, L, w, stage);")
+    emit("  else if (a.njmax <= 128)")
+    emit("    im::resident::newton_loop<4, 0, true>(0, L, w, stage);")
+    emit("  else")
+    emit("    im::resident::newton_loop<0, 0, true>(0, L, w, stage);")
     emit("}")
     if module:
         emit("} }  // namespace im::gen")

@@ -36,10 +36,10 @@ __device__ __forceinline__ bool in_bracket(Pt x, Pt y) { return (x.g < y.g && y.
 
 // The quadratic a row follows at position x: its own where it is in the quadratic zone, the linear
 // pieces of the friction-loss cost outside, nothing for a satisfied inequality.
-__device__ __forceinline__ Pt row_quad(bool friction, float D, float f, float jaref, float jv, float x) {
+// (rf: the friction row's f / D, which does not change during a search: formed once per row)
+__device__ __forceinline__ Pt row_quad(bool friction, float D, float f, float rf, float jaref, float jv, float x) {
   const Pt quad = {0.5f * jaref * jaref * D, jv * jaref * D, 0.5f * jv * jv * D};
   if (friction) {
-    const float rf = safe_div(f, D);
     if (x <= -rf) return {f * (-0.5f * rf - jaref), -f * jv, 0.0f};
     if (x >= rf) return {f * (-0.5f * rf + jaref), f * jv, 0.0f};
     return quad;
@@ -48,14 +48,14 @@ __device__ __forceinline__ Pt row_quad(bool friction, float D, float f, float ja
   return {0.0f, 0.0f, 0.0f};
 }
 // point of a row at alpha, cost relative to alpha 0, with the row's cost at alpha 0 computed beforehand (row_quad(..., jaref).c)
-__device__ __forceinline__ Pt row_point_from(bool friction, float D, float f, float jaref, float jv, float c0, float alpha) {
-  Pt p = eval_pt(row_quad(friction, D, f, jaref, jv, jaref + alpha * jv), alpha);
+__device__ __forceinline__ Pt row_point_from(bool friction, float D, float f, float rf, float jaref, float jv, float c0, float alpha) {
+  Pt p = eval_pt(row_quad(friction, D, f, rf, jaref, jv, jaref + alpha * jv), alpha);
   p.c = p.c - c0;
   return p;
 }
 // point of a row at alpha 0 with its cost itself
-__device__ __forceinline__ Pt row_point_zero(bool friction, float D, float f, float jaref, float jv) {
-  const Pt q = row_quad(friction, D, f, jaref, jv, jaref);
+__device__ __forceinline__ Pt row_point_zero(bool friction, float D, float f, float rf, float jaref, float jv) {
+  const Pt q = row_quad(friction, D, f, rf, jaref, jv, jaref);
   return {q.c, q.g, 2.0f * q.h};
 }
 
@@ -124,6 +124,9 @@ struct LsWorld {
   const float *smooth, *D, *frictionloss, *Jaref, *search, *mv, *jv, *Ma;  // frictionloss may be null
   float search_dot, tolerance, ls_tolerance, meaninertia;
   int ne, nf, nefc, nv, ls_iterations;
+  // optional, two arrays of nefc floats each that the search may use for what it forms once per row
+  // (a friction row's f / D, the row's cost at step 0) when it does not hold the rows in registers
+  float *row_scratch0 = nullptr, *row_scratch1 = nullptr;
 };
 struct LsResult {
   float alpha, improvement;
@@ -160,17 +163,18 @@ __device__ __forceinline__ LsResult linesearch_rows(const LsWorld &wd, int lane)
   const Pt gauss = {0.0f, lanes_sum(g1), lanes_sum(g2)};
   // this lane's rows ne + lane, ne + lane + 32, ...
   constexpr int NH = HELD > 0 ? HELD : 1;
-  float hd[NH], hf[NH], hja[NH], hv[NH], hc0[NH];
+  float hd[NH], hf[NH], hrf[NH], hja[NH], hv[NH], hc0[NH];
   if constexpr (HELD > 0) {
 #pragma unroll
     for (int k = 0; k < HELD; ++k) {
       const int r = ne + lane + 32 * k, rc = r < nefc ? r : (nefc > 0 ? nefc - 1 : 0);
-      const bool in = r < nefc;
+      const bool in = r < nefc, fr = r < ne + nf;
       hd[k] = in ? D[rc] : 0.0f;
       hf[k] = (in && fl) ? fl[rc] : 0.0f;
       hja[k] = in ? Jaref[rc] : 0.0f;
       hv[k] = in ? jv[rc] : 0.0f;
-      hc0[k] = row_quad(r < ne + nf, hd[k], hf[k], hja[k], hv[k], hja[k]).c;
+      hrf[k] = (in && fr) ? safe_div(hf[k], hd[k]) : 0.0f;
+      hc0[k] = row_quad(fr, hd[k], hf[k], hrf[k], hja[k], hv[k], hja[k]).c;
     }
   }
   // sum over this lane's rows of the rows' points at one or three step lengths
@@ -179,23 +183,37 @@ __device__ __forceinline__ LsResult linesearch_rows(const LsWorld &wd, int lane)
 #pragma unroll
       for (int k = 0; k < HELD; ++k) {
         const int r = ne + lane + 32 * k;
-        if (r < nefc) point(r < ne + nf, hd[k], hf[k], hja[k], hv[k], hc0[k]);
+        if (r < nefc) point(r < ne + nf, hd[k], hf[k], hrf[k], hja[k], hv[k], hc0[k]);
       }
+    } else if (wd.row_scratch0) {
+      for (int r = ne + lane; r < nefc; r += 32)
+        point(r < ne + nf, D[r], fl ? fl[r] : 0.0f, wd.row_scratch0[r], Jaref[r], jv[r], wd.row_scratch1[r]);
     } else {
       for (int r = ne + lane; r < nefc; r += 32) {
         const bool fr = r < ne + nf;
         const float d = D[r], f = fl ? fl[r] : 0.0f, ja = Jaref[r], v = jv[r];
-        point(fr, d, f, ja, v, row_quad(fr, d, f, ja, v, ja).c);
+        const float rf = fr ? safe_div(f, d) : 0.0f;
+        point(fr, d, f, rf, ja, v, row_quad(fr, d, f, rf, ja, v, ja).c);
       }
     }
   };
+  if (HELD == 0 && wd.row_scratch0) {
+    // a lane writes and later reads its own rows only (a wavefront's two halves write the same values)
+    for (int r = ne + lane; r < nefc; r += 32) {
+      const bool fr = r < ne + nf;
+      const float d = D[r], f = fl ? fl[r] : 0.0f, ja = Jaref[r], v = jv[r];
+      const float rf = fr ? safe_div(f, d) : 0.0f;
+      wd.row_scratch0[r] = rf;
+      wd.row_scratch1[r] = row_quad(fr, d, f, rf, ja, v, ja).c;
+    }
+  }
   auto rows_at = [&](float alpha) {
     Pt s = {0.0f, 0.0f, 0.0f};
-    rows_sum([&](bool fr, float d, float f, float ja, float v, float c0) { s = s + row_point_from(fr, d, f, ja, v, c0, alpha); });
+    rows_sum([&](bool fr, float d, float f, float rf, float ja, float v, float c0) { s = s + row_point_from(fr, d, f, rf, ja, v, c0, alpha); });
     return lanes_sum(s);
   };
   Pt z = {0.0f, 0.0f, 0.0f};
-  rows_sum([&](bool fr, float d, float f, float ja, float v, float) { z = z + row_point_zero(fr, d, f, ja, v); });
+  rows_sum([&](bool fr, float d, float f, float rf, float ja, float v, float) { z = z + row_point_zero(fr, d, f, rf, ja, v); });
   const Pt rows0 = lanes_sum(z);
   const Pt p0 = {gauss.c + rows0.c, gauss.g + rows0.g, 2.0f * gauss.h + rows0.h};
   const Pt p0_delta = {0.0f, p0.g, p0.h};
@@ -226,9 +244,9 @@ __device__ __forceinline__ LsResult linesearch_rows(const LsWorld &wd, int lane)
       Pt lo_next, hi_next, mid;
       if constexpr (SPLIT) {
         const float mine_alpha = (threadIdx.x & 32) ? hi_next_alpha : lo_next_alpha;
-        rows_sum([&](bool fr, float d, float f, float ja, float v, float c0) {
-          s_lo = s_lo + row_point_from(fr, d, f, ja, v, c0, mine_alpha);
-          s_mid = s_mid + row_point_from(fr, d, f, ja, v, c0, mid_alpha);
+        rows_sum([&](bool fr, float d, float f, float rf, float ja, float v, float c0) {
+          s_lo = s_lo + row_point_from(fr, d, f, rf, ja, v, c0, mine_alpha);
+          s_mid = s_mid + row_point_from(fr, d, f, rf, ja, v, c0, mid_alpha);
         });
         Pt rows_lo, rows_hi, rows_mid, same;
         lanes_sum_halves(s_lo, rows_lo, rows_hi);
@@ -237,10 +255,10 @@ __device__ __forceinline__ LsResult linesearch_rows(const LsWorld &wd, int lane)
         hi_next = eval_pt(gauss, hi_next_alpha) + rows_hi;
         mid = eval_pt(gauss, mid_alpha) + rows_mid;
       } else {
-        rows_sum([&](bool fr, float d, float f, float ja, float v, float c0) {
-          s_lo = s_lo + row_point_from(fr, d, f, ja, v, c0, lo_next_alpha);
-          s_hi = s_hi + row_point_from(fr, d, f, ja, v, c0, hi_next_alpha);
-          s_mid = s_mid + row_point_from(fr, d, f, ja, v, c0, mid_alpha);
+        rows_sum([&](bool fr, float d, float f, float rf, float ja, float v, float c0) {
+          s_lo = s_lo + row_point_from(fr, d, f, rf, ja, v, c0, lo_next_alpha);
+          s_hi = s_hi + row_point_from(fr, d, f, rf, ja, v, c0, hi_next_alpha);
+          s_mid = s_mid + row_point_from(fr, d, f, rf, ja, v, c0, mid_alpha);
         });
         lo_next = eval_pt(gauss, lo_next_alpha) + lanes_sum(s_lo);
         hi_next = eval_pt(gauss, hi_next_alpha) + lanes_sum(s_hi);

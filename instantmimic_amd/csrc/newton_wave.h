@@ -531,8 +531,9 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
         wave_sync();
       }
       IM_STAMP(1);
+      // (the force list and the row list of the gradient are free until the step is taken)
       const search::LsWorld lw{a.smooth + w * nv, L.D, L.fl, L.Jaref, L.sv, L.mv, L.jv, L.Ma, sc.search_dot, tolerance,
-                               ls_tolerance, meaninertia, ne, nf, nefc, nv, a.ls_iterations};
+                               ls_tolerance, meaninertia, ne, nf, nefc, nv, a.ls_iterations, L.f, (float *)L.rowl};
       const search::LsResult ls = search::linesearch_rows<HELD, true>(lw, lane & 31);  // both halves on this world
       sc.alpha = uniform(ls.alpha), sc.improvement = uniform(ls.improvement);
       if (lane == 0) {
