@@ -949,6 +949,20 @@ typedef struct im_newton_args {
   int32_t nworld;
 } im_newton_args;
 
+/* Replaces the part of init_context before the first Hessian
+ * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:431-500: _init_efc_settling_empty_worlds,
+ * Jaref = J qacc - aref, Ma = M qacc, upstream's _update_constraint and the first gradient) in
+ * one launch, a wavefront per world: solver_niter = 0, search_dot = 0, done = (nefc == 0), a world
+ * without constraint rows gets qacc = qacc_smooth; then for every world efc_Ma, and for the others
+ * Jaref, efc_force, efc_state with the list and the counts of changed rows, qfrc_constraint, grad,
+ * grad_dot, newton_decrement = 0, grad_scale = 1, search_unchanged = done.  The same operations in
+ * the same order as im_newton_init_empty_worlds, im_newton_init_jaref, im_mul_m_sparse,
+ * im_newton_eval_constraints and im_newton_gradient called one after the other (the same bits);
+ * the caller's first factor stage follows.  args as for im_newton_solve_tree; nv, nM: dofs and
+ * length of a row of M. */
+int im_newton_init_context(const im_newton_args *args, const float *qacc_smooth, int64_t ld_qacc_smooth,
+                           const float *efc_aref, int64_t ld_aref, int nv, int nM, void *stream);
+
 /* Replaces the launch of solve_incremental_newton_kernel
  * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:57-298, launched at :396-409) for a model
  * whose factor stage is the tree stage of im_newton_tree_stage: one resident kernel, a wavefront per

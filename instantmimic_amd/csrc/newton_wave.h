@@ -372,7 +372,7 @@ __device__ __forceinline__ void jv_world_tiled(const NewtonArgs &a, const float 
     }
     if (lane < rows) {
       const float out = split ? acc + p : p;
-      jv[r0 + lane] = out;
+      if (jv) jv[r0 + lane] = out;
       jv_lds[r0 + lane] = out;
     }
   }

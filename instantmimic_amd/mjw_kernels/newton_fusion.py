@@ -583,24 +583,26 @@ def _first_gradient(m, d, ctx) -> None:
              block=newton_block_dim(m))  # fmt: skip
 
 
-def _update_gradient_sparse(m, d, ctx, plan) -> None:
+def _update_gradient_sparse(m, d, ctx, plan, *, gradient_done: bool = False) -> None:
     """The first gradient, then H assembled on the sparse pattern, factored and solved
     (newton_fusion.py:481-519)."""
     from . import sparse_hessian
 
-    _first_gradient(m, d, ctx)
+    if not gradient_done:
+        _first_gradient(m, d, ctx)
     sparse_hessian.init_factor_kernel(plan)(ctx.done, d.nefc, d.efc.J, d.efc.D, d.efc.state, d.M, ctx.grad, ctx.hfactor,
                                             ctx.search, ctx.search_dot, ctx.newton_decrement)  # fmt: skip
 
 
-def _update_gradient_tree(m, d, ctx) -> None:
+def _update_gradient_tree(m, d, ctx, *, gradient_done: bool = False) -> None:
     """The first gradient, then the tree stage for every world that is not done (``search_unchanged``
     is ``done`` at this point)."""
-    _first_gradient(m, d, ctx)
+    if not gradient_done:
+        _first_gradient(m, d, ctx)
     _launch_stage(_stage(m, ctx), m, d, ctx)
 
 
-def _update_gradient(m, d, ctx) -> None:
+def _update_gradient(m, d, ctx, *, gradient_done: bool = False) -> None:
     """The dense first factor (upstream's ``solver._update_gradient`` for the dense Newton,
     newton_fusion.py:470): ``ctx.h = M + J' D_act J`` on the matrix cores, then the augmented
     blocked Cholesky of the per-iteration stage without an update."""
@@ -608,7 +610,8 @@ def _update_gradient(m, d, ctx) -> None:
 
     if not hasattr(ctx, "newton_mdense"):
         raise RuntimeError("the dense first factor needs attach_scratch(m, d, ctx)")
-    _first_gradient(m, d, ctx)
+    if not gradient_done:
+        _first_gradient(m, d, ctx)
     dense_from_csr(d.M, ctx.newton_elemid, ctx.newton_mdense)
     blocked_dense.dense_hessian(ctx.newton_mdense, d.efc.J, d.efc.D, d.efc.state, d.nefc, ctx.h)
     stage = _stage(m, ctx)
@@ -621,17 +624,49 @@ def init_context(m, d, ctx, mul_m_call=None) -> None:
     finish at once with ``qacc = qacc_smooth``; ``Jaref = J qacc - aref``; ``Ma = M qacc`` for every
     world; forces and states; the first gradient, Hessian, factor and search direction through the
     sparse plan, the tree stage or the dense path, whichever ``ctx`` carries."""
-    init_empty_worlds(d.nefc, d.qacc_smooth, d.solver_niter, ctx.search_dot, ctx.done, d.qacc)
-    init_jaref(d.nefc, d.qacc, d.efc.J, d.efc.aref, ctx.Jaref)
-    (mul_m_call or default_mul_m_call)(m, d, d.efc.Ma, d.qacc)
-    _update_constraint(m, d, ctx)
+    first = _init_before_factor(m, d, ctx) if mul_m_call is None else False
+    if not first:
+        init_empty_worlds(d.nefc, d.qacc_smooth, d.solver_niter, ctx.search_dot, ctx.done, d.qacc)
+        init_jaref(d.nefc, d.qacc, d.efc.J, d.efc.aref, ctx.Jaref)
+        (mul_m_call or default_mul_m_call)(m, d, d.efc.Ma, d.qacc)
+        _update_constraint(m, d, ctx)
     plan = _fused_plan(ctx)
     if plan is not None:
-        _update_gradient_sparse(m, d, ctx, plan)
+        _update_gradient_sparse(m, d, ctx, plan, gradient_done=first)
     elif _tree_scratch(ctx) is not None:
-        _update_gradient_tree(m, d, ctx)
+        _update_gradient_tree(m, d, ctx, gradient_done=first)
     else:
-        _update_gradient(m, d, ctx)
+        _update_gradient(m, d, ctx, gradient_done=first)
+
+
+def _init_before_factor(m, d, ctx) -> bool:
+    """Everything of ``init_context`` before the first Hessian in one launch, a wavefront per world
+    (``im_newton_init_context``: the same values as the five launches it stands for).  False, with
+    nothing done, under ``IMHIP_NEWTON=stages``, for arrays the one launch does not take (rows of
+    ``qacc_smooth`` or ``efc.aref`` that are not contiguous) and for sizes beyond a workgroup's LDS."""
+    import ctypes as C
+
+    import torch
+
+    if os.environ.get("IMHIP_NEWTON") == "stages":
+        return False
+    smooth, aref = d.qacc_smooth, d.efc.aref
+    nworld, nv = int(d.nworld), int(m.nv)
+    dev = d.efc.J.device
+    for t, width in ((smooth, nv), (aref, int(d.efc.J.shape[1]))):
+        if t.dtype != torch.float32 or t.device != dev or t.dim() != 2 or t.shape[0] != nworld or t.shape[1] < width or (
+            t.shape[1] > 1 and t.stride(1) != 1
+        ):
+            return False
+    a = _resident_args(m, d, ctx, None)
+    with torch.cuda.device(dev):
+        status = _lib.lib().im_newton_init_context(
+            C.byref(a), smooth.data_ptr(), smooth.stride(0), aref.data_ptr(), aref.stride(0), nv, int(d.M.shape[1]),
+            int(torch.cuda.current_stream(dev).cuda_stream))  # fmt: skip
+    if status == _lib.IM_ERR_UNSUPPORTED:
+        return False
+    _lib.check(status, "im_newton_init_context")
+    return True
 
 
 def iteration(m, d, ctx, nsolving=None, *, stage=None) -> None:

@@ -158,6 +158,37 @@ def test_gpu_solve_from_init_context_matches_the_oracle_chain(device, monkeypatc
     assert int(nsolving.item()) == int((p.nefc == 0).sum())  # every world that had rows has reported done
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,nworld,stage", [("humanoid", 301, "tree"), ("g1", 203, "sparse"), ("snu", 131, "tree"), ("ant", 67, "dense")])
+def test_gpu_init_context_in_one_launch_leaves_what_the_five_launches_leave(device, monkeypatch, name, nworld, stage):
+    """Everything before the first Hessian as one launch (a wavefront per world) against the same
+    steps as launches of their own: every array of ``d``, ``d.efc`` and ``ctx`` bit for bit, poison
+    included where neither writes."""
+    import torch
+
+    p = NC.problem(name, nworld, stage, empty_every=7, warmstart=True, maxiter=12)
+    taken = []
+    inner = NF._init_before_factor
+    monkeypatch.setattr(NF, "_init_before_factor", lambda *a: taken.append(inner(*a)) or taken[-1])
+    got = []
+    for env in ("stages", None):
+        if env:
+            monkeypatch.setenv("IMHIP_NEWTON", env)
+        else:
+            monkeypatch.delenv("IMHIP_NEWTON")
+        m, d, ctx, _ = NC.device_objects(p, device)
+        d.qacc.copy_(d.qacc_warmstart)
+        NF.init_context(m, d, ctx)
+        torch.cuda.synchronize()
+        got.append({f"{where}.{k}": v.cpu().numpy() for where, ns in (("d", d), ("efc", d.efc), ("ctx", ctx))
+                    for k, v in vars(ns).items() if isinstance(v, torch.Tensor)})  # fmt: skip
+    assert taken == [False, True]
+    assert got[0].keys() == got[1].keys() and "ctx.grad" in got[0] and "efc.Ma" in got[0]
+    for key in got[0]:
+        a, b = got[0][key], got[1][key]
+        assert a.tobytes() == b.tobytes(), key
+
+
 def _floating_chain(nv: int, limbs: int = 1):
     """A free body and hinges behind it (the reference's layout-boundary models,
     tests/test_mjw_newton_fusion.py:100-131): ``nv`` dofs, one chain or ``limbs`` chains off the
