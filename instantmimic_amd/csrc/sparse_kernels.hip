@@ -607,6 +607,9 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
 // of them, else they are read from memory), packed H is updated in LDS and written back whole,
 // and a lane keeps four pairs' table look-ups in flight.
 constexpr int kStagedRows = 16;
+// a dof's elements of the staged rows lie side by side, 17 words per dof: the row number is then a
+// constant offset in every access, and lanes that read different dofs meet in no LDS bank
+constexpr int kStagedStride = kStagedRows + 1;
 
 // The factor and solve tables of a plan into LDS, for a workgroup of T threads (a flat 16-byte copy,
 // every load issued before the first store); Q's table pointers then address the copy.
@@ -653,7 +656,7 @@ __device__ __forceinline__ void stage_update_tables(const SparseWave &A, SparseD
 }
 __host__ __device__ inline int update_world_words(int nslots, int n, int block) {
   const int nw = (block + 31) / 32;
-  return (nslots + n + 2 * nw + 2 * n + kStagedRows * (n + 1) + 3) & ~3;
+  return (nslots + n + 2 * nw + 2 * n + kStagedStride * n + kStagedRows + 3) & ~3;
 }
 
 // The stage for one world and one wavefront (`world_lds`: update_world_words of LDS of its own).
@@ -662,17 +665,20 @@ __device__ __forceinline__ void sparse_update_world(
     const int32_t *__restrict__ ids, int ld_ids, const float *__restrict__ J, int njmax,
     const float *__restrict__ D, const int32_t *__restrict__ state, int quad, const float *__restrict__ grad, int ldg,
     float *__restrict__ U_, int32_t *__restrict__ uni_, float *__restrict__ search_, float *__restrict__ search_dot,
-    float *__restrict__ decrement, int w, int lane) {
+    float *__restrict__ decrement, int w, int lane_in) {
+  // The lane number through an opaque step: inside a resident loop the addresses formed from it
+  // are then worked out where a round uses them instead of each holding a register from round to round.
+  int lane = lane_in;
+  asm volatile("" : "+v"(lane));
   const int n = Q.nv, nslots = Q.nslots, nfac = nslots - n, rhs = nfac;
   const int nw = (A.block + 31) / 32;
-  const int per_world = (nslots + n + 2 * nw + 2 * n + kStagedRows * (n + 1) + 3) & ~3;
   float *N = world_lds;  // [nslots]
   float *iD = N + nslots;                            // [n]
   float *red = iD + n;                               // [2][nw]
   int *ul = (int *)(red + 2 * nw);                   // [n] ascending dofs touched by the changed rows
   unsigned *mkl = (unsigned *)(ul + n);              // [n] per dof: bit t set where staged row t is nonzero there
-  float *jr = (float *)(mkl + n);                    // [kStagedRows][n] changed rows of J
-  float *sd = jr + kStagedRows * n;                  // [kStagedRows] D of the row, negated for a row that left the quadratic state
+  float *jr = (float *)(mkl + n);                    // [n][kStagedStride] changed rows of J, a dof's elements together
+  float *sd = jr + kStagedStride * n;                // [kStagedRows] D of the row, negated for a row that left the quadratic state
   float *U = U_ + (size_t)w * Q.nv_pad * Q.nv_pad;
   const float *gw = grad + (size_t)w * ldg;
   const float *Jw = J + (size_t)w * njmax * n;
@@ -682,9 +688,16 @@ __device__ __forceinline__ void sparse_update_world(
   int count = changes[w];
   count = count < ld_ids ? count : ld_ids;
   count = __builtin_amdgcn_readfirstlane(count);
+#ifdef IM_NEWTON_STAMPS  // development aid: time per part of the stage, summed over the rounds, left in the world's dof-union row
+  long long t_last = wall_clock64();
+#define IM_SSTAMP(k) do { const long long t_now = wall_clock64(); if (lane == 0) uni_[(size_t)w * (n + 1) + (k)] += (int)(t_now - t_last); t_last = wall_clock64(); } while (0)
+#else
+#define IM_SSTAMP(k) do {} while (0)
+#endif
   if (count > 0) {
     const bool staged = count <= kStagedRows;
     // requests first: the changed rows, their weights, packed H
+    bool hit = false;  // whether a changed row touches this lane's dof
     if (staged) {
       const int tq = lane < count ? lane : count - 1;
       const int rq = idw[tq];
@@ -698,41 +711,47 @@ __device__ __forceinline__ void sparse_update_world(
       }
       for (int s = lane; s < nfac; s += 64) N[s] = U[s];
       if (lane < kStagedRows) sd[lane] = sq == quad ? dq : -dq;
-#pragma unroll
-      for (int t = 0; t < kStagedRows; ++t)
-        if (t < count && lane < n) jr[t * n + lane] = rowv[t];
-    } else {
-      for (int s = lane; s < nfac; s += 64) N[s] = U[s];
-    }
-    sync_world<true>();
-    // dofs touched by the changed rows, ascending (n <= 64: one ballot)
-    bool hit = false;
-    if (lane < n) {
-      if (staged) {
+      if (lane < n) {
         unsigned mk = 0u;
-        for (int t = 0; t < count; ++t) mk |= (unsigned)(jr[t * n + lane] != 0.0f) << t;
+        float *mine = jr + lane * kStagedStride;
+#pragma unroll
+        for (int t = 0; t < kStagedRows; ++t) {
+          if (t < count) {
+            mine[t] = rowv[t];
+            mk |= (unsigned)(rowv[t] != 0.0f) << t;
+          }
+        }
         mkl[lane] = mk;
         hit = mk != 0u;
-      } else {
-        for (int t = 0; t < count && !hit; ++t) hit = Jw[idw[t] * n + lane] != 0.0f;
       }
+    } else {
+      for (int s = lane; s < nfac; s += 64) N[s] = U[s];
+      if (lane < n)
+        for (int t = 0; t < count && !hit; ++t) hit = Jw[idw[t] * n + lane] != 0.0f;
     }
+    // dofs touched by the changed rows, ascending (n <= 64: one ballot)
     const unsigned long long mask = __ballot(hit);
     const int nu = __popcll(mask);
     if (hit) ul[__popcll(mask & ((1ull << lane) - 1ull))] = lane;
-    sync_world<true>();
     int32_t *uni = uni_ + (size_t)w * (n + 1);
-    for (int i = lane; i < nu; i += 64) uni[i] = ul[i];
+#ifndef IM_NEWTON_STAMPS
+    if (hit) uni[__popcll(mask & ((1ull << lane) - 1ull))] = lane;
     if (lane == 0) uni[n] = nu;
+#endif
     const int32_t *PAIRt = Q.t[PAIR];
-    const int npair = nu * (nu + 1) / 2;
     int nbad = 0;
+    sync_world<true>();  // `ul`, `mkl` and the staged rows are read from here on
+    IM_SSTAMP(0);
+    const int npair = nu * (nu + 1) / 2;
     for (int e0 = lane; e0 < npair; e0 += 4 * 64) {
       int row[4], col[4], sl[4];
+      bool live[4];
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        const int e = e0 + 64 * k < npair ? e0 + 64 * k : npair - 1;
-        // e = cj (cj + 1) / 2 + ri with ri <= cj, found exactly
+        live[k] = e0 + 64 * k < npair;
+        const int e = live[k] ? e0 + 64 * k : npair - 1;
+        // e = cj (cj + 1) / 2 + ri with ri <= cj, found exactly (walking the pairs in 8 x 8 blocks
+        // of (ri, cj) instead, without this arithmetic, was measured a quarter slower)
         int cj = (int)((sqrtf((float)(8 * e + 1)) - 1.0f) * 0.5f);
         while ((cj + 1) * (cj + 2) / 2 <= e) ++cj;
         while (cj * (cj + 1) / 2 > e) --cj;
@@ -746,9 +765,10 @@ __device__ __forceinline__ void sparse_update_world(
         if (staged) {
           // only the rows in which both dofs are nonzero add to the pair, ascending: most pairs
           // of the union share no row at all
+          const float *jrow = jr + row[k] * kStagedStride, *jcol = jr + col[k] * kStagedStride;
           for (unsigned mm = mkl[row[k]] & mkl[col[k]]; mm; mm &= mm - 1u) {
             const int t = __builtin_ctz(mm);
-            delta = fma_(sd[t] * jr[t * n + row[k]], jr[t * n + col[k]], delta);
+            delta = fma_(sd[t] * jrow[t], jcol[t], delta);
           }
         } else {
           for (int t = 0; t < count; ++t) {
@@ -759,7 +779,7 @@ __device__ __forceinline__ void sparse_update_world(
             if (a != 0.0f && b != 0.0f) delta = fma_(da, b, delta);
           }
         }
-        if (e0 + 64 * k < npair && delta != 0.0f) {
+        if (live[k] && delta != 0.0f) {
           if (sl[k] >= 0) N[sl[k]] = N[sl[k]] + delta;  // one pair per slot: no two lanes meet
           else ++nbad;
         }
@@ -768,12 +788,16 @@ __device__ __forceinline__ void sparse_update_world(
     for (int o = 32; o > 0; o >>= 1) nbad += __shfl_down(nbad, o, 64);
     if (lane == 0 && nbad) atomicAdd(U + Q.nv_pad * Q.nv_pad - 1, (float)nbad);
     sync_world<true>();
+    IM_SSTAMP(1);
     for (int s = lane; s < nfac; s += 64) U[s] = N[s];
     for (int j = lane; j < n; j += 64) N[rhs + j] = gw[ORIGt[j]];
     sync_world<true>();
+    IM_SSTAMP(2);
     factor_levels<true>(Q, N, iD, lane, 64);
+    IM_SSTAMP(3);
     for (int s = lane; s < nfac; s += 64) U[nfac + s] = N[s];
     for (int j = lane; j < n; j += 64) U[2 * nfac + j] = iD[j];
+    IM_SSTAMP(4);
   } else {
     float *gl = (float *)ul;  // [n] right-hand side in elimination order
     for (int s = lane; s < nfac; s += 64) N[s] = U[nfac + s];
@@ -808,9 +832,12 @@ __device__ __forceinline__ void sparse_update_world(
       }
       sync_world<true>();
     }
+    IM_SSTAMP(5);
   }
   backward_sums<true>(Q, N, iD, gw, search_ + (size_t)w * n, red, search_dot + w, decrement + w, lane, 64,
                       A.block);
+  IM_SSTAMP(6);
+#undef IM_SSTAMP
 }
 
 template <int WAVES>
@@ -893,9 +920,8 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
                         (int)b.ld_grad, U_, uni_, b.search, b.search_dot, b.decrement, (int)w, threadIdx.x & 63);
   };
   while (w < nworld) {
-    // HELD: 2 up to 64 rows, else 0; with eight or twelve wavefronts (up to three per SIMD, 168 registers each) there is
-    // room to ask for the next rows of J ahead
-    resident::newton_loop<HELD, ((WAVES == 8 || WAVES == 12) ? -2 : -1), false, false>(kArgsOffset, L, w, stage);
+    // HELD: the rows a lane keeps in registers during the line search; the next tile of J is asked for ahead
+    resident::newton_loop<HELD, -2, false, false>(kArgsOffset, L, w, stage);
     int next = 0;
     if ((threadIdx.x & 63) == 0) next = atomicAdd(next_world, 1);
     w = __builtin_amdgcn_readfirstlane(next);
@@ -1197,7 +1223,7 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done, con
     A.block = plan->block;
     A.nM = 0;
     const size_t per_world =
-        ((size_t)plan->nslots + n + 2 * nw + 2 * n + (size_t)im::kStagedRows * (n + 1) + 3) & ~(size_t)3;
+        ((size_t)plan->nslots + n + 2 * nw + 2 * n + (size_t)im::kStagedStride * n + im::kStagedRows + 3) & ~(size_t)3;
     const int32_t *solve_end = plan->t[im::RK] + ((plan->sizes[im::RK] + 3) & ~3);
     const size_t solve_words = (size_t)(solve_end - plan->t[im::FL]);
     for (int i = 0; i < 5; ++i) A.solve[i] = (int)(plan->t[im::FL + i] - plan->t[im::FL]);
@@ -1280,6 +1306,7 @@ int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *p, 
     const void *fn;
   };
   // the line search keeps a lane's two rows in registers up to 64 rows and reads them from LDS beyond
+  // (four rows a lane up to 128 rows was measured slower here: 997 against 930 us per loop at g1)
   static const Variant variants[] = {{16, 2, (const void *)im::newton_sparse_resident_kernel<16, 2>},
                                      {12, 2, (const void *)im::newton_sparse_resident_kernel<12, 2>},
                                      {8, 2, (const void *)im::newton_sparse_resident_kernel<8, 2>},
