@@ -176,7 +176,8 @@ def _compile(src: str) -> str:
 
 def _spilling_kernels(remarks: str, *, fused: bool) -> list[str]:
     """Kernels with a private segment, from the text of ``-Rpass-analysis=kernel-resource-usage``:
-    the fused kernels (first template argument true) or the resident Newton kernels."""
+    the fused kernels (first template argument true), or the kernels built for the Newton
+    occupancy (the resident Newton kernels and the solve-only kernel)."""
     import re
 
     out, name = [], None
@@ -187,7 +188,7 @@ def _spilling_kernels(remarks: str, *, fused: bool) -> list[str]:
         m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
         if not (m and name and int(m.group(1)) > 0):
             continue
-        if ("tree_row16_" in name and "ILb1E" in name) if fused else ("newton_row16_" in name):
+        if ("tree_row16_" in name and "ILb1E" in name) if fused else ("newton_row16_" in name or ("tree_row16_" in name and "ILb0E" in name)):
             out.append(f"{name}: {m.group(1)} B/lane")
     return out
 

@@ -202,7 +202,7 @@ def compile_source(src: str, label: str) -> bytes | None:
     # spill at the fused kernels' occupancy, one more compile gives them a workgroup per CU less;
     # if they still spill the library leaves them unused (the iterations are then stage launches).
     name, occ = tree_row16.occupancy_of(src)
-    newton = ("im_row16_newton", "im_row16_newton_long")
+    newton = ("im_row16_newton", "im_row16_newton_long", "im_row16_solve")  # the kernels built for IM_NOCC
     if occ > 1 and any(kernel_resources(blob).get(k, (0, 0))[1] for k in newton):
         again = once((f"-DIM_NOCC_{name}={occ - 1}",))
         if again is not None and sum(kernel_resources(again).get(k, (0, 0))[1] for k in newton) < sum(kernel_resources(blob).get(k, (0, 0))[1] for k in newton):

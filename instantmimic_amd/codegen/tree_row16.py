@@ -31,8 +31,9 @@ Fused kernel: one workgroup of four wavefronts per four worlds.
   updates are single ``v_fmac_f32_dpp`` with the scaled pivot row
   ``T[k] = h[k] * -1/h[k][k]`` as the broadcast operand.
 
-The solve-only kernel is one wavefront per four worlds that reads M in the row16 layout
-and takes every role in turn.
+The solve-only kernel has the same four wavefronts per four worlds and the same roles; it
+reads H in the row16 layout from memory (a role fetches the rows it works on) and hands the
+groups' sums to the trunk through LDS as the fused kernel does.
 
 DPP reads of a register written by one of the two preceding VALU instructions are a
 hardware hazard that the compiler does not see inside inline assembly: every block that
@@ -208,7 +209,11 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     # LONG: more constraint rows than the straight-line assembly keeps in flight (a loop instead)
     # the body as a function: the kernels at the end of the file call it, the resident Newton
     # kernel once per iteration
-    emit("template <bool ASM, bool LONG>")
+    # SPLIT: the workgroup's four wavefronts share the work on its four worlds by role (group j
+    # on wavefront j, the trunk on wavefront 0) and hand their results on through LDS; without it
+    # one wavefront takes every role in turn.  The fused kernels always split; the solve-only
+    # kernel does too (taking every role, a wavefront would have to hold every row of H at once).
+    emit("template <bool ASM, bool LONG, bool SPLIT = ASM>")
     # world_of: null, or four world numbers in LDS, one per wavefront / 16-lane row, in place of the
     # workgroup's own four (the resident Newton loop hands finished wavefronts new worlds; a number
     # at or past nworld stands for no world)
@@ -237,9 +242,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("  const bool live = w < nworld && !(skip && skip[ws]);")
     # ---- right-hand side, uniform per world (wavefront 0 factors and solves)
     emit("  const float *yw = y + ws * ldy;")
-    # wavefront j of the fused kernel factors group j of the plan, wavefront 0 also the trunk;
-    # the solve-only kernel is one wavefront that takes every role in turn
-    emit("  #define ROLE(j) (!ASM || wv == (j))")
+    # wavefront j factors group j of the plan, wavefront 0 also the trunk
     emit("  float " + ", ".join(f"S{b} = 0.0f" for b in range(nv)) + ";")
 
     def sv(j, i, s_):
@@ -287,16 +290,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
         names += [f"SY{j}_{i}_{s_}" for i in range(1, len(segs[j])) for s_ in range(vsets[j])]
         names += [f"SP{j}_{s_}" for s_ in range(vsets[j])]
         emit("  float " + ", ".join(f"{n_} = 0.0f" for n_ in names) + ";")
-        emit(f"  if (!ASM) {{")
-        for i in range(len(segs[j])):
-            for s_ in range(vsets[j]):
-                load_sv(j, i, s_, sv(j, 0, s_) if i == 0 else f"SY{j}_{i}_{s_}")
-        emit("  }")
     emit("  float " + ", ".join(f"SVT_{s_} = 0.0f" for s_ in range(tsets)) + ";")
-    emit("  if (!ASM) {")
-    for s_ in range(tsets):
-        load_sv("T", 0, s_, f"SVT_{s_}")
-    emit("  }")
     emit("  float " + ", ".join(f"h{b}_{s}" for b in range(nv) for s in range(t.sets(b))) + ";")
     # ---- assembly on the matrix cores: wavefront v of the workgroup assembles world v of the four
     NT = -(-nv // 16)  # 16-wide blocks of dofs
@@ -338,6 +332,11 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
         xslots.append(sl)
     xs_off = xoff
     lds_floats = xs_off + 4 * nv
+
+    def xo(off):
+        """LDS word of an exchange slot: behind the four staging copies in the fused kernels, from
+        word 0 in the solve-only kernel (which has no staging copy)"""
+        return f"(ASM ? {off} : {off - 4 * TW})"
     if EXP == "timing":
         emit("  unsigned long long *tdbg = (unsigned long long *)Hout + (size_t)bid * 16; int tn = 0;")
         emit("  #define STAMP() do { if (Hout && threadIdx.x == 0) tdbg[tn] = clock64(); ++tn; } while (0)")
@@ -505,12 +504,6 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("    STAMP();  // hand-over barrier passed")
     for i, (li, s) in enumerate(leaf_sets):
         emit(f"    lh{i} = lds + kq * {TW} + chc{i};")
-    emit("  } else {")
-    emit("    const float *Mw = M + ws * ldM;")
-    for b in range(nv):
-        for s in range(t.sets(b)):
-            hi = t.depth[b] - 16 * s
-            emit(f"    h{b}_{s} = Mw[{t.rowadr[b] + 16 * s} + (p < {hi} ? p : {hi})];")
     emit("  }")
 
     def bc(expr, pos):
@@ -529,6 +522,12 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
                 hi = t.depth[b] - 16 * s
                 emit(f"        if (p <= {hi}) Hout[(int64_t)w * {nM} + {t.rowadr[b] + 16 * s} + p] = h{b}_{s};")
         emit("      }")
+        emit("    } else {")
+        emit("      const float *Mw = M + ws * ldM;")
+        for b in dofs:
+            for s in range(t.sets(b)):
+                hi = t.depth[b] - 16 * s
+                emit(f"      h{b}_{s} = Mw[{t.rowadr[b] + 16 * s} + (p < {hi} ? p : {hi})];")
         emit("    }")
 
     # group accumulators start from zero (tree_ldl.py:252-255)
@@ -795,6 +794,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
         for i in range(len(segs[j])):
             for s_ in range(vsets[j]):
                 take_rhs(j, i, s_, sv(j, 0, s_) if i == 0 else f"SY{j}_{i}_{s_}")
+        emit("    } else {")
+        for i in range(len(segs[j])):
+            for s_ in range(vsets[j]):
+                load_sv(j, i, s_, sv(j, 0, s_) if i == 0 else f"SY{j}_{i}_{s_}")
         emit("    }")
         fetch_rows(sorted(g))
         if j == 0:
@@ -813,10 +816,10 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
             for src, mask in sorted(by_src.items()):
                 expr = f"im_lane_select2({sv(j, src, s_)}, {expr}, IM_ROW_MASK(0x{mask:x}))"
             emit(f"    SP{j}_{s_} = {expr};")
-        emit("    if (ASM) {")
+        emit("    if (SPLIT) {")
         for (a, s_), off in xslots[j].items():
             src = f"SP{j}_{s_}" if a == "S" else f"ga{j}_{a}_{s_}"
-            emit(f"      xlds[{off} + lane] = {src};")
+            emit(f"      xlds[{xo(off)} + lane] = {src};")
         emit("    }")
         emit("  };")
     # ---- phase 2: trunk rows = own value plus the groups' contributions in group order
@@ -825,28 +828,31 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     emit("    if (ASM) {")
     for s_ in range(tsets):
         take_rhs("T", 0, s_, f"SVT_{s_}")
+    emit("    } else {")
+    for s_ in range(tsets):
+        load_sv("T", 0, s_, f"SVT_{s_}")
     emit("    }")
     fetch_rows(list(trunk))
     for a in trunk:
         for j in range(ngroups):
             if a in touched[j]:
                 for s in range(t.sets(a)):
-                    emit(f"    h{a}_{s} = h{a}_{s} + (ASM ? xlds[{xslots[j][a, s]} + lane] : ga{j}_{a}_{s});")
+                    emit(f"    h{a}_{s} = h{a}_{s} + (SPLIT ? xlds[{xo(xslots[j][a, s])} + lane] : ga{j}_{a}_{s});")
     # right-hand side: the lanes a group touched take its sums, in group order
     for j in range(ngroups):
         for s_ in range(min(tsets, vsets[j])):
             mask = sum(1 << p for p in range(16) if any(t.depth[a] == 16 * s_ + p for a in touched[j]))
             if mask:
-                emit(f"    SVT_{s_} = im_lane_select2(SVT_{s_} + (ASM ? xlds[{xslots[j]['S', s_]} + lane] : SP{j}_{s_}), SVT_{s_}, IM_ROW_MASK(0x{mask:x}));")
+                emit(f"    SVT_{s_} = im_lane_select2(SVT_{s_} + (SPLIT ? xlds[{xo(xslots[j]['S', s_])} + lane] : SP{j}_{s_}), SVT_{s_}, IM_ROW_MASK(0x{mask:x}));")
     emit("    STAMP();  // trunk: rows fetched and merged")
     for k in reversed(trunk):
         eliminate(k, None)
     emit("    STAMP();  // trunk: eliminated")
     backsub_many(trunk)
     emit("    STAMP();  // trunk: solved")
-    emit("    if (ASM && p == 0) {")
+    emit("    if (SPLIT && p == 0) {")
     for b in trunk:
-        emit(f"      xlds[{xs_off} + (lane >> 4) * {nv} + {b}] = S{b};")
+        emit(f"      xlds[{xo(xs_off)} + (lane >> 4) * {nv} + {b}] = S{b};")
     emit("    }")
     store_x(list(trunk))
     emit("  };")
@@ -854,14 +860,14 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     for j, g in enumerate(groups):
         emit(f"  auto phase3_{j} = {LAMBDA} {{")
         if j != 0:
-            emit("    if (ASM) {")
+            emit("    if (SPLIT) {")
             for a in sorted(touched[j]):
-                emit(f"      S{a} = xlds[{xs_off} + (lane >> 4) * {nv} + {a}];")
+                emit(f"      S{a} = xlds[{xo(xs_off)} + (lane >> 4) * {nv} + {a}];")
             emit("    }")
         backsub_many(list(reversed(g)))
         store_x(sorted(g))
         emit("  };")
-    emit("  if (ASM) {")
+    emit("  if (SPLIT) {")
     for j in range(max(ngroups, 1)):
         emit(("    if" if j == 0 else "    } else if") + f" (wv == {j}) {{")
         if j < ngroups:
@@ -918,20 +924,22 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
     if module:
         emit("} }  // namespace im::gen")
         for kernel, asm_, long_, bounds in (("fused", "true", "false", f"256, IM_OCC_{name}"), ("fused_long", "true", "true", f"256, IM_OCC_{name}"),
-                                            ("solve", "false", "false", "64, 1")):  # fmt: skip
+                                            ("solve", "false", "false", f"256, IM_NOCC_{name}")):  # fmt: skip
             emit(f'extern "C" __global__ __launch_bounds__({bounds}) void im_row16_{kernel}(IM_ROW16_PARAMS) {{')
-            emit(f"  im::gen::tree_row16_body_{name}<{asm_}, {long_}>({args}, nullptr);")
+            emit(f"  im::gen::tree_row16_body_{name}<{asm_}, {long_}, true>({args}, nullptr);")
             emit("}")
         for kernel, long_ in (("newton", "false"), ("newton_long", "true")):
             emit(f'extern "C" __global__ __launch_bounds__(256, IM_NOCC_{name}) void im_row16_{kernel}(im::resident::NewtonArgs a) {{')
             emit(f"  im::gen::newton_row16_body_{name}<{long_}>(a);")
             emit("}")
         emit(f'extern "C" __device__ const unsigned long long im_row16_key = 0x{key:016x}ull;')
-        emit(f'extern "C" __device__ const int im_row16_info[4] = {{{nv}, {nM}, {lds_floats * 4}, {4 * PD}}};  // nv, nM, LDS bytes, short rows')
+        emit(f'extern "C" __device__ const int im_row16_info[5] = {{{nv}, {nM}, {lds_floats * 4}, {4 * PD}, {(lds_floats - 4 * TW) * 4}}};  // nv, nM, LDS bytes, short rows, LDS bytes of the solve-only kernel')
     else:
         emit("template <bool ASM, bool LONG>")
-        emit(f"__global__ __launch_bounds__(ASM ? 256 : 64, ASM ? IM_OCC_{name} : 1) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
-        emit(f"  tree_row16_body_{name}<ASM, LONG>({args}, nullptr);")
+        # (the solve-only kernel fetches a group's rows of H from memory at once and holds a few values
+        # more than the fused one: it shares the Newton kernels' occupancy)
+        emit(f"__global__ __launch_bounds__(256, ASM ? IM_OCC_{name} : IM_NOCC_{name}) void tree_row16_{name}(IM_ROW16_PARAMS) {{")
+        emit(f"  tree_row16_body_{name}<ASM, LONG, true>({args}, nullptr);")
         emit("}")
         emit("template <bool LONG>")
         emit(f"__global__ __launch_bounds__(256, IM_NOCC_{name}) void newton_row16_{name}(im::resident::NewtonArgs a) {{")
@@ -940,7 +948,7 @@ def generate(name, rowadr, rownnz, colind, groups, trunk, *, module: bool = Fals
         emit(f"static const Row16Entry entry_{name} = {{0x{key:016x}ull, {nv}, {nM}, {lds_floats * 4}, {4 * PD}, \"{name}\",")
         emit(f"    (const void *)tree_row16_{name}<true, false>, (const void *)tree_row16_{name}<true, true>,")
         emit(f"    (const void *)tree_row16_{name}<false, false>, (const void *)newton_row16_{name}<false>,")
-        emit(f"    (const void *)newton_row16_{name}<true>}};")
+        emit(f"    (const void *)newton_row16_{name}<true>, {(lds_floats - 4 * TW) * 4}}};")
         emit(f"static const Row16Register reg_{name}(&entry_{name});")
         emit("} }  // namespace im::gen")
     # workgroups per CU that the fused kernel is compiled for: what the 160 KB of LDS admit (with

@@ -405,18 +405,20 @@ int launch(const im_tree_plan *plan, bool assemble, const float *M, int64_t ldM,
                     &quad,  &y,        &ldy,       &x,            &ldx,      &Hout,    &nworld,
                     &flags, &its.niter, &its.state_it, &its.y_it, &its.x_it, &skip};
     // staged rows plus the four worlds' active-row lists (row id and D per constraint row)
-    const size_t lds = assemble ? (size_t)e->lds_bytes + 32 * std::max<size_t>(((size_t)njmax + 15) / 16 * 16, 64) : 0;
-    if (lds <= 160 * 1024) {
-      // fused: one wavefront per world assembles, the first one factors and solves all four
-      const void *fn = !assemble ? e->solve : (njmax <= e->short_rows ? e->fused : e->fused_long);
+    const size_t lds = assemble ? (size_t)e->lds_bytes + 32 * std::max<size_t>(((size_t)njmax + 15) / 16 * 16, 64)
+                                : (size_t)e->solve_lds_bytes;
+    const void *fn = !assemble ? e->solve : (njmax <= e->short_rows ? e->fused : e->fused_long);
+    if (fn && lds <= 160 * 1024) {
+      // four wavefronts per four worlds: in the fused kernel each assembles one world, then (in
+      // both) wavefront j factors group j of all four and the first one the trunk
       // several iterations: whole rounds of the eight XCDs per iteration (spare workgroups exit)
       const unsigned quads = (unsigned)((nworld + 3) / 4);
       const unsigned grid = its.niter > 1 ? (quads + 7) / 8 * 8 * (unsigned)its.niter : quads;
       if (plan->module)
-        IM_HIP_CHECK(hipModuleLaunchKernel((hipFunction_t)fn, grid, 1, 1, assemble ? 256 : 64, 1, 1, (unsigned)lds,
+        IM_HIP_CHECK(hipModuleLaunchKernel((hipFunction_t)fn, grid, 1, 1, 256, 1, 1, (unsigned)lds,
                                            (hipStream_t)stream, args, nullptr));
       else
-        IM_HIP_CHECK(hipLaunchKernel(fn, dim3(grid), dim3(assemble ? 256 : 64), args, lds, (hipStream_t)stream));
+        IM_HIP_CHECK(hipLaunchKernel(fn, dim3(grid), dim3(256), args, lds, (hipStream_t)stream));
       return IM_OK;
     }
   }
@@ -587,6 +589,8 @@ int tree_plan_upload(im_tree_plan *pl) {
       IM_HIP_CHECK(hipFuncSetAttribute(e->fused, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
       IM_HIP_CHECK(hipFuncSetAttribute(e->fused_long, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     }
+    if (e->solve_lds_bytes > 48 * 1024)
+      IM_HIP_CHECK(hipFuncSetAttribute(e->solve, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     // the resident Newton loop keeps its own arrays behind the stage's
     // ... and is used only where it keeps to registers and the runtime grants the LDS
     // (im_newton_solve_tree says unsupported otherwise)
@@ -651,7 +655,7 @@ int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object) {
     return code;
   };
   unsigned long long key = 0;
-  int info[4] = {0, 0, 0, 0};
+  int info[5] = {0, 0, 0, 0, 0};
   hipDeviceptr_t sym = nullptr;
   size_t bytes = 0;
   if (hipModuleGetGlobal(&sym, &bytes, mod, "im_row16_key") != hipSuccess || bytes != sizeof(key) ||
@@ -663,7 +667,8 @@ int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object) {
   // the kernels are straight-line code for one structure and plan: anything else would read and
   // write out of place
   if (key != im::tree_key(*plan) || info[0] != plan->nv || info[1] != plan->nM) return fail(IM_ERR_STRUCTURE);
-  if (info[2] <= 0 || info[2] + 32 * 64 > 160 * 1024 || info[3] <= 0) return fail(IM_ERR_UNSUPPORTED);
+  if (info[2] <= 0 || info[2] + 32 * 64 > 160 * 1024 || info[3] <= 0 || info[4] < 0 || info[4] > info[2])
+    return fail(IM_ERR_UNSUPPORTED);
   hipFunction_t fused = nullptr, fused_long = nullptr, solve = nullptr, newton = nullptr, newton_long = nullptr;
   if (hipModuleGetFunction(&fused, mod, "im_row16_fused") != hipSuccess ||
       hipModuleGetFunction(&fused_long, mod, "im_row16_fused_long") != hipSuccess ||
@@ -681,6 +686,7 @@ int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object) {
     return hipFuncGetAttribute(&bytes, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, f) == hipSuccess && bytes > 0;
   };
   if (spills(fused) || spills(fused_long)) return fail(IM_ERR_UNSUPPORTED);
+  if (spills(solve)) solve = nullptr;  // im_tree_factor_solve then takes the table-driven kernel
   const bool newton_ok = newton && !spills(newton), newton_long_ok = newton_long && !spills(newton_long);
   if (info[2] + 32 * 64 > 48 * 1024) {
     // more than the default dynamic LDS: asked for here; a runtime that refuses the request for a
@@ -704,7 +710,11 @@ int im_tree_plan_attach_kernels(im_tree_plan *plan, const void *code_object) {
   if (!e) return fail(IM_ERR_ARG);
   *e = im::gen::Row16Entry{key, info[0], info[1], info[2], info[3], "module", (const void *)fused,
                            (const void *)fused_long, (const void *)solve, (const void *)newton,
-                           (const void *)newton_long};
+                           (const void *)newton_long, info[4]};
+  if (solve && info[4] > 48 * 1024) {
+    (void)hipFuncSetAttribute((const void *)solve, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipGetLastError();
+  }
   plan->module = mod;
   plan->resident_ok = newton_ok && newton_lds;
   plan->resident_long_ok = newton_long_ok && newton_long_lds;

@@ -89,9 +89,10 @@ struct Row16Entry {
   const char *name;
   const void *fused;       // assemble + factor + solve, njmax <= short_rows
   const void *fused_long;  // the same with a loop over the constraint rows
-  const void *solve;       // factor + solve
+  const void *solve;       // factor + solve of a given H, the same four wavefronts per four worlds
   const void *newton;      // the resident Newton loop with the fused kernel as its factor stage, njmax <= short_rows
   const void *newton_long; // the same with the loop over the constraint rows
+  int solve_lds_bytes;     // dynamic LDS of the solve-only kernel (the roles' hand-over area)
 };
 
 // Registers a generated kernel at load time.
