@@ -47,6 +47,9 @@ struct NewtonArgs {
   // from which a wavefront whose world is done takes the next world nobody has started (null: a
   // workgroup keeps to its own four worlds)
   int *next_world;
+  // cooperative loop: whether a wavefront keeps its world's row of M in LDS (1) or reads it from
+  // memory in the round's one product with it (0: the LDS saved admits another workgroup per CU)
+  int m_lds;
 };
 
 // The public argument block checked and turned into the kernels' (host side).
@@ -82,6 +85,7 @@ inline int convert_args(const im_newton_args &p, int nv, int nM, NewtonArgs &a) 
   a.ld_ids = p.ld_ids, a.done = p.done, a.exhausted = p.ls_exhausted, a.unchanged = p.search_unchanged;
   a.stage_lds_floats = 0;
   a.next_world = nullptr;
+  a.m_lds = 1;
   return IM_OK;
 }
 
@@ -427,7 +431,7 @@ __device__ __forceinline__ const NewtonArgs &kernel_args(int kernarg_offset) {
   return *(const NewtonArgs *)ap;
 }
 
-// MLDS: the world's row of M is kept in LDS (L.m_lds); otherwise `M search` reads it from memory
+// MLDS: the world's row of M is kept in LDS (where L.m_lds is not null); otherwise `M search` reads it from memory
 // every round, which leaves the LDS to more worlds per CU.
 template <int HELD, int JU, bool COOP, bool MLDS = true, class Stage>
 __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L, int64_t w_raw, Stage &&stage) {
@@ -466,7 +470,8 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
     // what the loop keeps: M, Ma, Jaref into LDS (mv and jv are formed before they are read: a world
     // enters with a new search direction unless it is done) and qacc
     if constexpr (MLDS)
-      for (int k = lane_fixed; k < a.nM; k += 64) L.m_lds[k] = a.M[w * a.ldM + k];
+      if (L.m_lds)
+        for (int k = lane_fixed; k < a.nM; k += 64) L.m_lds[k] = a.M[w * a.ldM + k];
     for (int k = lane_fixed; k < nv; k += 64) {
       L.Ma[k] = a.Ma[w * nv + k];
       L.mv[k] = a.mv[w * nv + k];
@@ -523,7 +528,7 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
       if (!unchanged) {
         for (int k = lane; k < nv; k += 64) L.sv[k] = a.search[w * nv + k];
         wave_sync();
-        mul_m_world(a, L.term, L.radr, MLDS ? (const float *)L.m_lds : a.M + w * a.ldM, L.sv, a.mv + w * nv, L.mv, lane);
+        mul_m_world(a, L.term, L.radr, (MLDS && L.m_lds) ? (const float *)L.m_lds : a.M + w * a.ldM, L.sv, a.mv + w * nv, L.mv, lane);
         if constexpr (JU > 0)
           jv_world<(JU > 0 ? JU : 1)>(a, Jw, nefc, L.rows, L.sv, a.jv + w * njmax, L.jv, lane);
         else
@@ -658,7 +663,7 @@ __device__ __forceinline__ void newton_loop(int kernarg_offset, const LoopLds &L
 // wavefronts' own arrays.  Fills the tables; the caller synchronises the workgroup before the loop.
 __device__ __forceinline__ LoopLds coop_layout(const NewtonArgs &a, float *lds) {
   const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  const int nv = a.nv, njmax = a.njmax, nM = a.nM;
+  const int nv = a.nv, njmax = a.njmax, nM = a.m_lds ? a.nM : 0;
   LoopLds L;
   L.votes = (int *)(lds + a.stage_lds_floats);
   L.worlds = L.votes + 4;
@@ -666,8 +671,8 @@ __device__ __forceinline__ LoopLds coop_layout(const NewtonArgs &a, float *lds) 
   int *radr = (int *)(term + a.nterm);
   float *mine = (float *)(radr + nv + 1) + wv * (kept_words(nv, njmax, nM) + 2 * njmax + nv);
   L.term = term, L.radr = radr;
-  L.m_lds = mine;
-  L.sv = L.m_lds + nM;
+  L.m_lds = a.m_lds ? mine : nullptr;
+  L.sv = mine + nM;
   L.Ma = L.sv + nv;
   L.mv = L.Ma + nv;
   L.qacc = L.mv + nv;

@@ -792,19 +792,28 @@ int im_newton_solve_tree(const im_tree_plan *plan, const im_newton_args *p, void
   const size_t stage_bytes = (size_t)e->lds_bytes + 32 * std::max<size_t>(((size_t)njmax + 15) / 16 * 16, 64);
   const size_t stage_words = std::max(stage_bytes / 4, im::resident::staged_rows_words(nv));
   a.stage_lds_floats = (int)stage_words;
-  const size_t lds = 4 * (stage_words + im::resident::loop_lds_words(nv, njmax, nM, p->nterm));
-  if (lds > 160 * 1024) return IM_ERR_UNSUPPORTED;
+  size_t lds = 4 * (stage_words + im::resident::loop_lds_words(nv, njmax, nM, p->nterm));
+  const size_t lds_lean = 4 * (stage_words + im::resident::loop_lds_words(nv, njmax, 0, p->nterm));
+  if (lds_lean > 160 * 1024) return IM_ERR_UNSUPPORTED;
   const bool is_long = njmax > e->short_rows;
   if (!(is_long ? plan->resident_long_ok : plan->resident_ok)) return IM_ERR_UNSUPPORTED;  // the kernel spills registers
   const void *fn = is_long ? e->newton_long : e->newton;
   // As many workgroups as the chip keeps resident (registers and LDS); a wavefront whose world is
   // done takes the next world through the plan's counter, so the worlds that need many iterations
   // do not hold three idle wavefronts in place.
-  int per_cu = 0;
-  if (plan->module) {
-    IM_HIP_CHECK(hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (hipFunction_t)fn, 256, lds));
-  } else {
-    IM_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, lds));
+  auto resident_per_cu = [&](size_t bytes, int *per_cu) {
+    if (plan->module) return hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, (hipFunction_t)fn, 256, bytes);
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(per_cu, fn, 256, bytes);
+  };
+  int per_cu = 0, per_cu_lean = 0;
+  if (lds <= 160 * 1024) IM_HIP_CHECK(resident_per_cu(lds, &per_cu));
+  IM_HIP_CHECK(resident_per_cu(lds_lean, &per_cu_lean));
+  // the worlds' rows of M stay in LDS unless leaving them in memory admits another workgroup per CU
+  // (snu: 81 KB a workgroup with them, one per CU; 70 KB without, two)
+  if (per_cu_lean > per_cu) {
+    a.m_lds = 0;
+    lds = lds_lean;
+    per_cu = per_cu_lean;
   }
   static int ncu = 0;
   if (!ncu) {
