@@ -178,6 +178,41 @@ def test_newton_entry_points_check_their_arguments_before_any_launch():
     assert lib.im_qfrc_constraint_from_grad(one, one, 27, one, 27, one, 27, None, one, 27, 27, 4, None) == _lib.IM_ERR_ARG
 
 
+def _newton_args(**over):
+    """An ``im_newton_args`` block with every pointer non-null (nothing is dereferenced before the checks)."""
+    import ctypes as C
+
+    a = _lib.NewtonArgs()
+    for name, kind in a._fields_:
+        setattr(a, name, 16 if kind is C.c_void_p else 0)
+    a.ntolerance = a.nls_tolerance = a.nmeaninertia = 1
+    a.ls_iterations, a.iterations, a.block, a.quad = 50, 10, 32, 1
+    a.nterm, a.ldM, a.njmax, a.ld_grad, a.ld_ids, a.nworld = 243, 243, 64, 32, 64, 4
+    for k, v in over.items():
+        setattr(a, k, v)
+    return a
+
+
+def test_init_context_entry_point_checks_its_arguments_before_any_launch():
+    import ctypes as C
+
+    lib = _lib.lib()
+    one = 16
+    call = lambda a, smooth=one, lds=27, aref=one, lda=64, nv=27, nM=243: lib.im_newton_init_context(  # noqa: E731
+        C.byref(a), smooth, lds, aref, lda, nv, nM, None)
+    assert call(_newton_args(nworld=0)) == _lib.IM_OK
+    assert call(_newton_args(nworld=-1)) == _lib.IM_ERR_ARG
+    assert call(_newton_args(), smooth=None) == _lib.IM_ERR_ARG and call(_newton_args(), aref=None) == _lib.IM_ERR_ARG
+    assert call(_newton_args(efc_J=None)) == _lib.IM_ERR_ARG and call(_newton_args(block=48)) == _lib.IM_ERR_ARG
+    assert call(_newton_args(), lds=26) == _lib.IM_ERR_STRIDE and call(_newton_args(), lda=63) == _lib.IM_ERR_STRIDE
+    assert call(_newton_args(ldM=242)) == _lib.IM_ERR_STRIDE and call(_newton_args(ld_grad=26)) == _lib.IM_ERR_STRIDE
+    # four worlds' vectors and a tile of J per workgroup: 4 (3 nv + 3 njmax + 1088) words must fit a CU's LDS
+    assert call(_newton_args(njmax=4000, ld_ids=4000), lda=4000) == _lib.IM_ERR_UNSUPPORTED
+    # the resident solves: no plan, no argument block
+    assert lib.im_newton_solve_tree(None, C.byref(_newton_args()), None) == _lib.IM_ERR_ARG
+    assert lib.im_newton_solve_sparse(None, C.byref(_newton_args()), one, one, None) == _lib.IM_ERR_ARG
+
+
 def test_implicit_matrix_entry_points_check_their_arguments_before_any_launch():
     lib = _lib.lib()
     one = 16
