@@ -310,7 +310,7 @@ __device__ __forceinline__ LsResult linesearch_rows(const LsWorld &wd, int lane)
   return {alpha, improvement, fabsf(alpha) < noise_floor, converged};
 }
 
-template <int HELD>
+template <int HELD, bool SPLIT = false>
 __device__ __forceinline__ void linesearch_world(const SearchArgs &a, int64_t w, int lane) {
   int nefc = a.nefc ? a.nefc[w] : a.njmax;
   nefc = nefc < a.njmax ? nefc : a.njmax;
@@ -318,8 +318,8 @@ __device__ __forceinline__ void linesearch_world(const SearchArgs &a, int64_t w,
                   a.Jaref + w * a.ld_Jaref, a.search + w * a.ld_search, a.mv + w * a.ld_mv, a.jv + w * a.ld_jv,
                   a.Ma + w * a.ld_Ma, a.search_dot[w], a.tolerance[w % a.ntolerance], a.ls_tolerance[w % a.nls_tolerance],
                   a.meaninertia[w % a.nmeaninertia], a.ne ? a.ne[w] : 0, a.nf ? a.nf[w] : 0, nefc, a.nv, a.ls_iterations};
-  const LsResult out = linesearch_rows<HELD>(r, lane);
-  if (lane == 0) {
+  const LsResult out = linesearch_rows<HELD, SPLIT>(r, lane);
+  if (SPLIT ? (threadIdx.x & 63) == 0 : lane == 0) {
     a.alpha[w] = out.alpha;
     a.improvement[w] = out.improvement;
     a.exhausted[w] = out.exhausted ? 1 : 0;

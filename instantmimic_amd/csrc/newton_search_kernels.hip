@@ -12,14 +12,15 @@ namespace {
 
 using namespace search;
 
-// Two worlds per wavefront, 32 lanes each (the reference's reduction width).
+// A wavefront per world: the sums run over 32 lanes (the reference's reduction width) and the two
+// halves of the wavefront evaluate different candidate steps of a round side by side.
 template <int HELD>
 __global__ __launch_bounds__(64) void newton_linesearch_kernel(SearchArgs a) {
   const int lane = threadIdx.x & 31;
-  const int64_t w = (int64_t)blockIdx.x * 2 + (threadIdx.x >> 5);
+  const int64_t w = blockIdx.x;
   if (w >= a.nworld) return;
   if (a.done && a.done[w]) return;
-  linesearch_world<HELD>(a, w, lane);
+  linesearch_world<HELD, true>(a, w, lane);
 }
 
 // A wavefront per world.
@@ -75,7 +76,7 @@ extern "C" int im_newton_linesearch(const float *opt_tolerance, int ntolerance, 
   // rows per lane: two up to 64 rows, four up to 128, eight up to 256
   auto fn = njmax <= 64 ? newton_linesearch_kernel<2> : njmax <= 128 ? newton_linesearch_kernel<4>
             : njmax <= 256 ? newton_linesearch_kernel<8> : newton_linesearch_kernel<0>;
-  hipLaunchKernelGGL(fn, dim3((unsigned)((nworld + 1) / 2)), dim3(64), 0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(fn, dim3((unsigned)nworld), dim3(64), 0, (hipStream_t)stream, a);
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;
 }
