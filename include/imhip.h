@@ -994,6 +994,18 @@ int im_newton_solve_tree(const im_tree_plan *plan, const im_newton_args *args, v
 int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *args, float *hfactor,
                            int32_t *dof_union, void *stream);
 
+/* The same launch for a dense model of up to 32 dofs, whose factor stage is the single-tile branch
+ * of the reference's stage (src/instantmimic/utils/mjw_kernels/newton_stages.py:723-733, inside
+ * the loop of newton_fusion.py:57-298): one resident kernel, a wavefront per world, the stage of
+ * im_dense_update_tile once per round for the worlds whose states changed.  H: ctx.h,
+ * (nworld, nv_pad, nv_pad), updated in place; dof_union (nworld, nv + 1) as in
+ * im_dense_update_tile.  next_world: one int32 of the caller's on the device, the batch's world
+ * counter (two solves that share it must not overlap on the GPU).  Leaves the arrays as nv <= 32
+ * launches of the stages would.  IM_ERR_UNSUPPORTED beyond 32 dofs and where a CU's LDS does not
+ * hold four worlds. */
+int im_newton_solve_dense_tile(const im_newton_args *args, float *H, int32_t *dof_union, int nv, int nv_pad, int nM,
+                               int32_t *next_world, void *stream);
+
 /* Replaces _init_efc_settling_empty_worlds
  * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:412-428): solver_niter = 0,
  * search_dot = 0, done = (nefc == 0), and a world without constraint rows gets

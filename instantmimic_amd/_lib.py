@@ -260,6 +260,7 @@ SIGNATURES = {
         [_vp, _vp, _vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _i64, _vp, _i64, _vp, _vp, _i, _i, _vp],
     ),
     "im_newton_solve_tree": (_i, [_vp, C.POINTER(NewtonArgs), _vp]),
+    "im_newton_solve_dense_tile": (_i, [C.POINTER(NewtonArgs), _vp, _vp, _i, _i, _i, _vp, _vp]),
     "im_newton_solve_sparse": (_i, [_vp, C.POINTER(NewtonArgs), _vp, _vp, _vp]),
     "im_newton_advance": (
         _i,

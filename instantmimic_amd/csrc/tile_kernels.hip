@@ -16,17 +16,16 @@
 
 #include <cstdint>
 
+#include <algorithm>
+
 #include "common.h"
+#include "newton_wave.h"
 #include "pivot.h"
 
 namespace im {
 namespace {
 
-__device__ __forceinline__ void wave_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
+using resident::wave_sync;
 
 // LDS words of one group: the column being handed round, the right-hand side entries, the pivots'
 // reciprocals, and the tile itself (staged in, later the factor), rows NP + 1 words apart
@@ -152,27 +151,14 @@ __global__ __launch_bounds__(256) void tile_cholesky_solve_kernel(
 // H's upper triangle (in memory and in the staged copy), then H factored as one tile and solved
 // for the gradient, at every call; U is not used.  search = -x, search_dot = x.x,
 // decrement = grad.x.  Two worlds per wavefront, 32 lanes each.
+// One world's stage on a group of 32 lanes (lane i of the group); both groups of a wavefront may
+// work on the same world, they then write the same values to the same places.
 template <int NP>
-__global__ __launch_bounds__(256) void dense_update_tile_kernel(
-    const uint8_t *__restrict__ done, const int32_t *__restrict__ state_changes,
-    const int32_t *__restrict__ changes, const int32_t *__restrict__ ids, int ld_ids,
-    const float *__restrict__ J, int njmax, const float *__restrict__ D, const int32_t *__restrict__ state,
-    int quad, const float *__restrict__ grad, int64_t ldg, float *H_, int32_t *__restrict__ uni_,
-    float *__restrict__ search, int64_t ld_search, float *__restrict__ search_dot,
-    float *__restrict__ decrement, int nv, int pad, int nworld) {
-  extern __shared__ float lds[];
+__device__ __forceinline__ void dense_tile_world(const TileArea<NP> &T, int *ul, float *Hw, const float *Jw, const float *Dw,
+                                                 const float *gw, const int32_t *sw, const int32_t *idw, int count, int quad,
+                                                 int32_t *uni, float *search_w, float *search_dot_w, float *decrement_w,
+                                                 int nv, int pad, int i) {
   constexpr int LG = 32, kRow = TileArea<NP>::kRow;
-  const int group = threadIdx.x / LG, i = threadIdx.x % LG;
-  const int64_t w = (int64_t)blockIdx.x * (256 / LG) + group;
-  if (w >= nworld) return;
-  if ((done && done[w]) || state_changes[w] == 0) return;
-  const TileArea<NP> T(lds + group * (TileArea<NP>::kWords + 36));
-  int *ul = (int *)(lds + group * (TileArea<NP>::kWords + 36) + TileArea<NP>::kWords);  // [nv + 1]
-  float *Hw = H_ + w * (int64_t)pad * pad;
-  const float *Jw = J + w * (int64_t)njmax * nv, *Dw = D + w * njmax, *gw = grad + w * ldg;
-  const int32_t *sw = state + w * njmax, *idw = ids + w * ld_ids;
-  int count = changes[w];
-  count = count < 0 ? 0 : (count < ld_ids ? count : ld_ids);
   // H's rows into LDS (both triangles as they lie there; only the upper one is read)
   for (int e = i; e < nv * nv; e += LG) {
     const int r = e / nv, c = e - r * nv;
@@ -188,9 +174,9 @@ __global__ __launch_bounds__(256) void dense_update_tile_kernel(
   if (hit) {
     const int at = __popc(mask & ((1u << i) - 1u));
     ul[at] = i;
-    uni_[w * (nv + 1) + at] = i;
+    uni[at] = i;
   }
-  if (i == 0) uni_[w * (nv + 1) + nv] = nu;
+  if (i == 0) uni[nv] = nu;
   wave_sync();
   for (int e = i; e < nu * (nu + 1) / 2; e += LG) {
     int cj = (int)((sqrtf((float)(8 * e + 1)) - 1.0f) * 0.5f);
@@ -219,7 +205,7 @@ __global__ __launch_bounds__(256) void dense_update_tile_kernel(
   for (int c = 0; c < NP; ++c) a[c] = (i < nv && c <= i) ? T.tile[c * kRow + i] : 0.0f;  // upper triangle: element (c, i)
   wave_sync();
   s = tile_factor_solve<NP, LG>(a, s, i, nv, T);
-  if (i < nv) search[w * ld_search + i] = -s;
+  if (i < nv) search_w[i] = -s;
   // as 64 lanes striding the dofs would sum them: one term per lane, the upper 32 lanes' zeros change nothing
   float s0 = fma_(s, s, 0.0f), s1 = fma_(g, s, 0.0f);
 #pragma unroll
@@ -228,10 +214,104 @@ __global__ __launch_bounds__(256) void dense_update_tile_kernel(
     s1 = s1 + __shfl_down(s1, off, LG);
   }
   if (i == 0) {
-    search_dot[w] = s0;
-    decrement[w] = s1;
+    *search_dot_w = s0;
+    *decrement_w = s1;
   }
 }
+
+template <int NP>
+__global__ __launch_bounds__(256) void dense_update_tile_kernel(
+    const uint8_t *__restrict__ done, const int32_t *__restrict__ state_changes,
+    const int32_t *__restrict__ changes, const int32_t *__restrict__ ids, int ld_ids,
+    const float *__restrict__ J, int njmax, const float *__restrict__ D, const int32_t *__restrict__ state,
+    int quad, const float *__restrict__ grad, int64_t ldg, float *H_, int32_t *__restrict__ uni_,
+    float *__restrict__ search, int64_t ld_search, float *__restrict__ search_dot,
+    float *__restrict__ decrement, int nv, int pad, int nworld) {
+  extern __shared__ float lds[];
+  constexpr int LG = 32;
+  const int group = threadIdx.x / LG, i = threadIdx.x % LG;
+  const int64_t w = (int64_t)blockIdx.x * (256 / LG) + group;
+  if (w >= nworld) return;
+  if ((done && done[w]) || state_changes[w] == 0) return;
+  const TileArea<NP> T(lds + group * (TileArea<NP>::kWords + 36));
+  int *ul = (int *)(lds + group * (TileArea<NP>::kWords + 36) + TileArea<NP>::kWords);  // [nv + 1]
+  int count = changes[w];
+  count = count < 0 ? 0 : (count < ld_ids ? count : ld_ids);
+  dense_tile_world<NP>(T, ul, H_ + w * (int64_t)pad * pad, J + w * (int64_t)njmax * nv, D + w * njmax, grad + w * ldg,
+                       state + w * njmax, ids + w * ld_ids, count, quad, uni_ + w * (nv + 1), search + w * ld_search,
+                       search_dot + w, decrement + w, nv, pad, i);
+}
+
+// The resident Newton loop (newton_wave.h) with this stage: a wavefront per world from the first
+// line search to convergence, WAVES worlds per workgroup.  Both halves of the wavefront run the
+// stage on the wavefront's world.  Per wavefront in LDS: what the loop keeps from round to round
+// and one area that the staged tile of J, the gradient's row list and the stage's tile use one
+// after the other.
+template <int NP>
+__host__ __device__ inline int dense_resident_area_words(int nv, int njmax) {
+  int words = TileArea<NP>::kWords + 36;
+  const int tile = 64 * 17, grad = 2 * njmax + nv;
+  words = words > tile ? words : tile;
+  words = words > grad ? words : grad;
+  return (words + 3) & ~3;
+}
+__host__ __device__ inline int dense_resident_shared_words(int nterm, int nv) { return (nterm + nv + 1 + 3) & ~3; }
+
+template <int NP, int WAVES, int HELD>
+__global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_dense_tile_resident_kernel(
+    resident::NewtonArgs a, float *__restrict__ H_, int32_t *__restrict__ uni_, int pad, int *__restrict__ next_world) {
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nv = a.nv, njmax = a.njmax, nworld = a.nworld;
+  uint32_t *term = (uint32_t *)lds;
+  int *radr = (int *)(term + a.nterm);
+  const int area = dense_resident_area_words<NP>(nv, njmax);
+  float *mine = lds + dense_resident_shared_words(a.nterm, nv) + wv * (area + resident::kept_words(nv, njmax, 0));
+  resident::LoopLds L;
+  L.votes = nullptr;
+  L.worlds = nullptr;
+  L.term = term, L.radr = radr;
+  L.rows = mine;  // the shared area: tile of J, then the gradient's lists, then the stage's tile
+  L.f = mine;
+  L.rowl = (int *)(mine + njmax);
+  L.gl = mine + 2 * njmax;
+  L.m_lds = nullptr;  // M is read from memory by the round's one product with it
+  L.sv = mine + area;
+  L.Ma = L.sv + nv;
+  L.mv = L.Ma + nv;
+  L.qacc = L.mv + nv;
+  L.Jaref = L.qacc + nv;
+  L.jv = L.Jaref + njmax;
+  L.D = L.jv + njmax;
+  L.fl = L.D + njmax;
+  for (int k = tid; k < a.nterm; k += 64 * WAVES) term[k] = (uint32_t)a.mulm_col[k] | (uint32_t)a.mulm_madr[k] << 16;
+  for (int k = tid; k <= nv; k += 64 * WAVES) radr[k] = a.mulm_rowadr[k];
+  __syncthreads();  // the only workgroup barrier
+  int64_t w = (int64_t)blockIdx.x * WAVES + wv;
+  auto stage = [&]() __attribute__((always_inline)) {
+    const resident::NewtonArgs &b = resident::kernel_args(0);  // the kernel's first parameter
+    int lane = threadIdx.x & 31;
+    asm volatile("" : "+v"(lane));  // (nothing formed from it is kept in registers from round to round)
+    const TileArea<NP> T(mine);
+    int count = b.quad_count[w];
+    count = count < 0 ? 0 : (count < b.ld_ids ? count : b.ld_ids);
+    dense_tile_world<NP>(T, (int *)(mine + TileArea<NP>::kWords), H_ + w * (int64_t)pad * pad,
+                         b.J + w * (int64_t)b.njmax * b.nv, b.D + w * b.njmax, b.grad + w * b.ld_grad,
+                         b.state + w * b.njmax, b.ids + w * (int64_t)b.ld_ids, count, b.quad, uni_ + w * (b.nv + 1),
+                         b.search + w * b.nv, b.search_dot + w, b.decrement + w, b.nv, pad, lane);
+  };
+  // as many wavefronts as the chip keeps resident; one whose world is done takes the next world
+  // nobody has started (a counter in memory that only grows: every wavefront reaches the end)
+  while (w < nworld) {
+    resident::newton_loop<HELD, -2, false, false>(0, L, w, stage);
+    int next = 0;
+    if ((threadIdx.x & 63) == 0) next = atomicAdd(next_world, 1);
+    w = __builtin_amdgcn_readfirstlane(next);
+  }
+}
+
+__global__ void set_dense_counter_kernel(int *counter, int value) { *counter = value; }
 
 template <int NP, int LG>
 int launch_tiles(const float *M, int64_t ld_world, int64_t ld_row, const int32_t *adr, int ntile, int size,
@@ -310,6 +390,65 @@ int im_dense_update_tile(const uint8_t *done, const int32_t *state_changes, cons
   }
   IM_STAGE_CASE(8) IM_STAGE_CASE(16) IM_STAGE_CASE(24) IM_STAGE_CASE(32)
 #undef IM_STAGE_CASE
+  return IM_ERR_UNSUPPORTED;
+}
+
+int im_newton_solve_dense_tile(const im_newton_args *p, float *H, int32_t *dof_union, int nv, int nv_pad, int nM,
+                               int32_t *next_world, void *stream) {
+  if (!p || !H || !dof_union || !next_world || p->nworld < 0 || nv <= 0 || nv_pad < nv || nM <= 0) return IM_ERR_ARG;
+  if (nv > 32) return IM_ERR_UNSUPPORTED;
+  if (p->nworld == 0) return IM_OK;
+  im::resident::NewtonArgs a{};
+  const int bad = im::resident::convert_args(*p, nv, nM, a);
+  if (bad != IM_OK) return bad;
+  const int njmax = p->njmax;
+  struct Variant {
+    int np, waves, held;
+    const void *fn;
+  };
+#define IM_DENSE_VARIANT(NP, WAVES, HELD) {NP, WAVES, HELD, (const void *)im::newton_dense_tile_resident_kernel<NP, WAVES, HELD>}
+  // tile of 16 or 32 dofs; sixteen or eight worlds per workgroup; the line search keeps a lane's two
+  // rows in registers up to 64 rows and reads them from LDS beyond
+  static const Variant variants[] = {IM_DENSE_VARIANT(16, 16, 2), IM_DENSE_VARIANT(16, 8, 2), IM_DENSE_VARIANT(16, 16, 0),
+                                     IM_DENSE_VARIANT(16, 8, 0),  IM_DENSE_VARIANT(32, 16, 2), IM_DENSE_VARIANT(32, 8, 2),
+                                     IM_DENSE_VARIANT(32, 16, 0), IM_DENSE_VARIANT(32, 8, 0)};
+#undef IM_DENSE_VARIANT
+  constexpr int kVariants = 8;
+  static bool usable[kVariants] = {};
+  static bool probed = false;
+  if (!probed) {  // once per process: a variant that spills registers is left out; the large dynamic LDS is asked for
+    for (int i = 0; i < kVariants; ++i) {
+      hipFuncAttributes fa{};
+      usable[i] = hipFuncGetAttributes(&fa, variants[i].fn) == hipSuccess && fa.localSizeBytes == 0 &&
+                  hipFuncSetAttribute(variants[i].fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      160 * 1024 - (int)fa.sharedSizeBytes) == hipSuccess;
+      (void)hipGetLastError();
+    }
+    probed = true;
+  }
+  const int np = nv <= 16 ? 16 : 32;
+  for (int i = 0; i < kVariants; ++i) {
+    const Variant &v = variants[i];
+    if (!usable[i] || v.np != np || v.held != (njmax <= 64 ? 2 : 0)) continue;
+    const int area = np == 16 ? im::dense_resident_area_words<16>(nv, njmax) : im::dense_resident_area_words<32>(nv, njmax);
+    const size_t per_wave = (size_t)area + im::resident::kept_words(nv, njmax, 0);
+    const size_t lds = 4 * ((size_t)im::dense_resident_shared_words(p->nterm, nv) + v.waves * per_wave);
+    if (lds > 158 * 1024) continue;
+    static int ncu = 0;
+    if (!ncu) {
+      int dev = 0;
+      IM_HIP_CHECK(hipGetDevice(&dev));
+      IM_HIP_CHECK(hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev));
+    }
+    // as many workgroups as stay resident at once (LDS, and sixteen wavefronts of up to 128 registers per CU)
+    const int per_cu = std::max(1, std::min((int)(160 * 1024 / lds), 16 / v.waves));
+    const int needed = (p->nworld + v.waves - 1) / v.waves;
+    const int grid = std::min(needed, std::max(ncu, 1) * per_cu);
+    hipLaunchKernelGGL(im::set_dense_counter_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, next_world, grid * v.waves);
+    void *args[] = {&a, &H, &dof_union, &nv_pad, &next_world};
+    IM_HIP_CHECK(hipLaunchKernel(v.fn, dim3((unsigned)grid), dim3(64 * v.waves), args, lds, (hipStream_t)stream));
+    return IM_OK;
+  }
   return IM_ERR_UNSUPPORTED;
 }
 

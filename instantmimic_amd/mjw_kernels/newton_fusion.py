@@ -547,6 +547,7 @@ def attach_scratch(m, d, ctx, device=None) -> None:
             host = lambda a: a.cpu().numpy() if hasattr(a, "cpu") else np.asarray(a)  # noqa: E731
             elemid = torch.from_numpy(elemid_table(host(m.M_rowadr), host(m.M_rownnz), host(m.M_colind))).to(dev)
         ctx.newton_elemid = elemid.to(dtype=torch.int32).reshape(nv, nv).contiguous()
+        ctx.newton_next_world = torch.zeros(1, dtype=torch.int32, device=dev)  # the resident kernel's world counter
 
 
 def _stage(m, ctx):
@@ -779,20 +780,34 @@ def _resident_args(m, d, ctx, nsolving):
 
 def run_resident(m, d, ctx, nsolving) -> bool:
     """The whole loop as one resident kernel (a wavefront per world until it is done): for a ``ctx``
-    with a fused sparse plan, or with the tree stage whose plan carries generated kernels.  False
-    when there is no such kernel for this model (the caller then launches the stages one by one)."""
+    with a fused sparse plan, with the tree stage whose plan carries generated kernels, or for a
+    dense model of up to 32 dofs (the single-tile stage).  False when there is no such kernel for
+    this model (the caller then launches the stages one by one)."""
     import ctypes as C
 
     import torch
 
     scratch, plan = _tree_scratch(ctx), _fused_plan(ctx)
-    if (scratch is None and plan is None) or os.environ.get("IMHIP_NEWTON") == "stages":
+    dense_tile = scratch is None and plan is None and int(m.nv) <= 32 and getattr(ctx, "newton_next_world", None) is not None
+    if (scratch is None and plan is None and not dense_tile) or os.environ.get("IMHIP_NEWTON") == "stages":
         return False
     a = _resident_args(m, d, ctx, nsolving)
     dev = d.efc.J.device
     stream = int(torch.cuda.current_stream(dev).cuda_stream)
     with torch.cuda.device(dev):
-        if plan is not None:
+        if dense_tile:
+            nworld, nv, pad = int(d.nworld), int(m.nv), int(m.nv_pad)
+            h, uni, counter = ctx.h, ctx.newton_dof_union, ctx.newton_next_world
+            if h.dtype != torch.float32 or h.device != dev or tuple(h.shape) != (nworld, pad, pad) or not h.is_contiguous():
+                raise TypeError("h must be a contiguous float32 (nworld, nv_pad, nv_pad) tensor")
+            if uni.dtype != torch.int32 or uni.device != dev or tuple(uni.shape) != (nworld, nv + 1) or not uni.is_contiguous():
+                raise TypeError("newton_dof_union must be a contiguous int32 (nworld, nv + 1) tensor")
+            if counter.dtype != torch.int32 or counter.device != dev or counter.numel() != 1:
+                raise TypeError("newton_next_world must be a one-element int32 tensor")
+            status = _lib.lib().im_newton_solve_dense_tile(C.byref(a), h.data_ptr(), uni.data_ptr(), nv, pad, int(d.M.shape[1]),
+                                                           counter.data_ptr(), stream)  # fmt: skip
+            where = "im_newton_solve_dense_tile"
+        elif plan is not None:
             nworld, nv, pad = int(d.nworld), int(m.nv), int(m.nv_pad)
             hf, uni = ctx.hfactor, ctx.newton_dof_union
             if hf.dtype != torch.float32 or hf.device != dev or tuple(hf.shape) != (nworld, pad, pad) or not hf.is_contiguous():
