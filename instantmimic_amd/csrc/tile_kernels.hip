@@ -151,6 +151,13 @@ __global__ __launch_bounds__(256) void tile_cholesky_solve_kernel(
 // H's upper triangle (in memory and in the staged copy), then H factored as one tile and solved
 // for the gradient, at every call; U is not used.  search = -x, search_dot = x.x,
 // decrement = grad.x.  Two worlds per wavefront, 32 lanes each.
+constexpr int kTileStagedRows = 16;
+// LDS words of one group's stage: the tile's area, the dof union (36), the staged rows, their weights and the dofs' masks
+template <int NP>
+__host__ __device__ constexpr int dense_tile_stage_words() {
+  return TileArea<NP>::kWords + 36 + (kTileStagedRows + 1) * NP + kTileStagedRows + NP;
+}
+
 // One world's stage on a group of 32 lanes (lane i of the group); both groups of a wavefront may
 // work on the same world, they then write the same values to the same places.
 template <int NP>
@@ -160,14 +167,57 @@ __device__ __forceinline__ void dense_tile_world(const TileArea<NP> &T, int *ul,
                                                  int nv, int pad, int i) {
   constexpr int LG = 32, kRow = TileArea<NP>::kRow;
   // H's rows into LDS (both triangles as they lie there; only the upper one is read)
-  for (int e = i; e < nv * nv; e += LG) {
-    const int r = e / nv, c = e - r * nv;
-    T.tile[r * kRow + c] = Hw[(size_t)r * pad + c];
+  const float inv_nv = 1.0f / (float)nv;
+  for (int e0 = i; e0 < nv * nv; e0 += 4 * LG) {  // four loads in flight per lane
+    float v[4];
+    int at[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int e = e0 + k * LG < nv * nv ? e0 + k * LG : nv * nv - 1;
+      const int r = (int)(((float)e + 0.5f) * inv_nv), c = e - r * nv;  // e / nv, exact for these sizes
+      v[k] = Hw[(size_t)r * pad + c];
+      at[k] = r * kRow + c;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (e0 + k * LG < nv * nv) T.tile[at[k]] = v[k];
+  }
+  // The changed rows of J come into LDS dof-major (a dof's elements of up to kTileStagedRows rows
+  // side by side, 17 words a dof) with a mask per dof of the rows that are nonzero there; more
+  // changed rows than that are read from memory pair by pair.
+  const bool staged = count <= kTileStagedRows;
+  float *jr = (float *)(ul + 36);             // [nv][kTileStagedRows + 1]
+  float *sd = jr + (kTileStagedRows + 1) * NP;  // [kTileStagedRows] D of the row, negated for a row that left the quadratic state
+  unsigned *mkl = (unsigned *)(sd + kTileStagedRows);  // [nv]
+  int hit = 0;
+  if (staged && count > 0) {
+    const int tq = i < count ? i : count - 1;
+    const int rq = idw[tq];
+    const float dq = Dw[rq];
+    const int sq = sw[rq];
+    float rowv[kTileStagedRows];
+#pragma unroll
+    for (int t = 0; t < kTileStagedRows; ++t) {
+      const int r = __shfl(rq, t < count ? t : 0, LG);
+      rowv[t] = Jw[(size_t)r * nv + (i < nv ? i : nv - 1)];
+    }
+    if (i < kTileStagedRows) sd[i] = sq == quad ? dq : -dq;
+    if (i < nv) {
+      unsigned mk = 0u;
+#pragma unroll
+      for (int t = 0; t < kTileStagedRows; ++t) {
+        if (t < count) {
+          jr[i * (kTileStagedRows + 1) + t] = rowv[t];
+          mk |= (unsigned)(rowv[t] != 0.0f) << t;
+        }
+      }
+      mkl[i] = mk;
+      hit = mk != 0u;
+    }
+  } else if (i < nv) {
+    for (int t = 0; t < count && !hit; ++t) hit = Jw[(size_t)idw[t] * nv + i] != 0.0f;
   }
   // dof union, ascending: lane d looks at dof d
-  int hit = 0;
-  if (i < nv)
-    for (int t = 0; t < count && !hit; ++t) hit = Jw[(size_t)idw[t] * nv + i] != 0.0f;
   const unsigned long long both = __ballot(hit);
   const unsigned mask = (unsigned)(both >> (threadIdx.x & 32));
   const int nu = __popc(mask);
@@ -184,12 +234,20 @@ __device__ __forceinline__ void dense_tile_world(const TileArea<NP> &T, int *ul,
     while (cj * (cj + 1) / 2 > e) --cj;
     const int row = ul[e - cj * (cj + 1) / 2], col = ul[cj];
     float delta = 0.0f;
-    for (int t = 0; t < count; ++t) {
-      const int r = idw[t];
-      const float av = Jw[(size_t)r * nv + row], bv = Jw[(size_t)r * nv + col];
-      float da = Dw[r] * av;
-      if (sw[r] != quad) da = -da;
-      if (av != 0.0f && bv != 0.0f) delta = fma_(da, bv, delta);
+    if (staged) {  // the rows in which both dofs are nonzero, ascending
+      const float *jrow = jr + row * (kTileStagedRows + 1), *jcol = jr + col * (kTileStagedRows + 1);
+      for (unsigned mm = mkl[row] & mkl[col]; mm; mm &= mm - 1u) {
+        const int t = __builtin_ctz(mm);
+        delta = fma_(sd[t] * jrow[t], jcol[t], delta);
+      }
+    } else {
+      for (int t = 0; t < count; ++t) {
+        const int r = idw[t];
+        const float av = Jw[(size_t)r * nv + row], bv = Jw[(size_t)r * nv + col];
+        float da = Dw[r] * av;
+        if (sw[r] != quad) da = -da;
+        if (av != 0.0f && bv != 0.0f) delta = fma_(da, bv, delta);
+      }
     }
     if (delta != 0.0f) {
       const float h = T.tile[row * kRow + col] + delta;
@@ -233,8 +291,8 @@ __global__ __launch_bounds__(256) void dense_update_tile_kernel(
   const int64_t w = (int64_t)blockIdx.x * (256 / LG) + group;
   if (w >= nworld) return;
   if ((done && done[w]) || state_changes[w] == 0) return;
-  const TileArea<NP> T(lds + group * (TileArea<NP>::kWords + 36));
-  int *ul = (int *)(lds + group * (TileArea<NP>::kWords + 36) + TileArea<NP>::kWords);  // [nv + 1]
+  const TileArea<NP> T(lds + group * dense_tile_stage_words<NP>());
+  int *ul = (int *)(lds + group * dense_tile_stage_words<NP>() + TileArea<NP>::kWords);  // [nv + 1], the staged rows behind it
   int count = changes[w];
   count = count < 0 ? 0 : (count < ld_ids ? count : ld_ids);
   dense_tile_world<NP>(T, ul, H_ + w * (int64_t)pad * pad, J + w * (int64_t)njmax * nv, D + w * njmax, grad + w * ldg,
@@ -249,7 +307,7 @@ __global__ __launch_bounds__(256) void dense_update_tile_kernel(
 // after the other.
 template <int NP>
 __host__ __device__ inline int dense_resident_area_words(int nv, int njmax) {
-  int words = TileArea<NP>::kWords + 36;
+  int words = dense_tile_stage_words<NP>();
   const int tile = 64 * 17, grad = 2 * njmax + nv;
   words = words > tile ? words : tile;
   words = words > grad ? words : grad;
@@ -381,7 +439,7 @@ int im_dense_update_tile(const uint8_t *done, const int32_t *state_changes, cons
   const unsigned grid = (unsigned)((nworld + 7) / 8);
 #define IM_STAGE_CASE(NP)                                                                                            \
   if (nv <= NP) {                                                                                                    \
-    const size_t lds = sizeof(float) * 8 * (im::TileArea<NP>::kWords + 36);                                          \
+    const size_t lds = sizeof(float) * 8 * im::dense_tile_stage_words<NP>();                                         \
     hipLaunchKernelGGL(im::dense_update_tile_kernel<NP>, dim3(grid), dim3(256), lds, st, done, state_changes, changes, \
                        ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, dof_union, search, ld_search, search_dot, \
                        decrement, nv, nv_pad, nworld);                                                               \
