@@ -354,6 +354,15 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes,
                            int nv_pad, int32_t *dof_union, float *search, int64_t ld_search,
                            float *search_dot, float *decrement, int nworld, void *stream);
 
+/* The same stage for nv_pad = 48 or 64 (33 to 63 dofs) on one wavefront per world, a lane per
+ * column of the padded matrix: same arguments, same results bit for bit; im_dense_update_factor
+ * hands such shapes here.  IM_ERR_UNSUPPORTED for other paddings. */
+int im_dense_update_column(const uint8_t *done, const int32_t *state_changes, const int32_t *changes,
+                           const int32_t *ids, int ld_ids, const float *J, int njmax, const float *D,
+                           const int32_t *state, int quad, const float *grad, int64_t ldg, float *H, float *U, int nv,
+                           int nv_pad, int32_t *dof_union, float *search, int64_t ld_search, float *search_dot,
+                           float *decrement, int nworld, void *stream);
+
 /* Blocked dense factor + solve, dense J'DJ ----------------------------------- */
 
 /* Replaces _blocked_dense_factor_solve (src/instantmimic/utils/mjw_step_optimized.py:
@@ -1005,6 +1014,13 @@ int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *arg
  * hold four worlds. */
 int im_newton_solve_dense_tile(const im_newton_args *args, float *H, int32_t *dof_union, int nv, int nv_pad, int nM,
                                int32_t *next_world, void *stream);
+
+/* The same for a dense model of 33 to 63 dofs with nv_pad = 48 or 64, whose factor stage is the
+ * augmented blocked Cholesky (newton_stages.py:473-611, 614-742) run as im_dense_update_column
+ * runs it, a wavefront per world with a lane per column.  U: ctx.hfactor, (nworld, nv_pad, nv_pad).
+ * IM_ERR_UNSUPPORTED for other shapes. */
+int im_newton_solve_dense_column(const im_newton_args *args, float *H, float *U, int32_t *dof_union, int nv, int nv_pad,
+                                 int nM, int32_t *next_world, void *stream);
 
 /* Replaces _init_efc_settling_empty_worlds
  * (src/instantmimic/utils/mjw_kernels/newton_fusion.py:412-428): solver_niter = 0,

@@ -202,6 +202,10 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],
     ),
+    "im_dense_update_column": (
+        _i,
+        [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],
+    ),
     "im_newton_init_context": (_i, [C.POINTER(NewtonArgs), _vp, _i64, _vp, _i64, _i, _i, _vp]),
     "im_polynomial_damping": (_i, [_vp, _i64, _vp, _i64, _i, _vp, _i64, _vp, _i64, _i, _i, _vp]),
     "im_dense_update_tile": (
@@ -261,6 +265,7 @@ SIGNATURES = {
     ),
     "im_newton_solve_tree": (_i, [_vp, C.POINTER(NewtonArgs), _vp]),
     "im_newton_solve_dense_tile": (_i, [C.POINTER(NewtonArgs), _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "im_newton_solve_dense_column": (_i, [C.POINTER(NewtonArgs), _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "im_newton_solve_sparse": (_i, [_vp, C.POINTER(NewtonArgs), _vp, _vp, _vp]),
     "im_newton_advance": (
         _i,

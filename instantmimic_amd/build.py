@@ -19,7 +19,7 @@ GEN = os.path.join(CSRC, "gen")
 OBJ = os.path.join(HERE, "_obj")
 LIB = os.path.join(HERE, "libimhip.so")
 
-SOURCES = ["tree_plan.cpp", "sparse_plan.cpp", "tree_kernels.hip", "muscle_kernels.hip", "muscle_geometry.hip", "sparse_kernels.hip", "blocked_kernels.hip", "tile_kernels.hip", "tree_reduce_kernels.hip", "newton_kernels.hip", "newton_search_kernels.hip", "newton_init_kernels.hip", "implicit_kernels.hip"]
+SOURCES = ["tree_plan.cpp", "sparse_plan.cpp", "tree_kernels.hip", "muscle_kernels.hip", "muscle_geometry.hip", "sparse_kernels.hip", "blocked_kernels.hip", "tile_kernels.hip", "dense_column_kernels.hip", "tree_reduce_kernels.hip", "newton_kernels.hip", "newton_search_kernels.hip", "newton_init_kernels.hip", "implicit_kernels.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950",

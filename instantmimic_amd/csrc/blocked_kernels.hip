@@ -1889,6 +1889,15 @@ int im_dense_update_factor(const uint8_t *done, const int32_t *state_changes, co
   if (nv <= 32)  // no factor is kept for such a matrix: one tile, factored at every call
     return im_dense_update_tile(done, state_changes, changes, ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, nv,
                                 nv_pad, dof_union, search, ld_search, search_dot, decrement, nworld, stream);
+  // up to 64 columns: a wavefront per world with a lane per column (IMHIP_DENSE_STAGE=blocked keeps
+  // the workgroup-per-world kernel below, which serves the larger matrices)
+  static const bool column_off = [] {
+    const char *e = std::getenv("IMHIP_DENSE_STAGE");
+    return e && std::strcmp(e, "blocked") == 0;
+  }();
+  if (!column_off && (nv_pad == 48 || nv_pad == 64))
+    return im_dense_update_column(done, state_changes, changes, ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, U,
+                                  nv, nv_pad, dof_union, search, ld_search, search_dot, decrement, nworld, stream);
   if (((uintptr_t)H | (uintptr_t)U) & 15) return IM_ERR_STRIDE;  // read and written 16 bytes at a time
   constexpr int B = 16;
   const int pf = (nv + B - 1) / B * B;  // the factor in LDS covers the dofs; the kernel writes the identity beyond them itself

@@ -781,21 +781,24 @@ def _resident_args(m, d, ctx, nsolving):
 def run_resident(m, d, ctx, nsolving) -> bool:
     """The whole loop as one resident kernel (a wavefront per world until it is done): for a ``ctx``
     with a fused sparse plan, with the tree stage whose plan carries generated kernels, or for a
-    dense model of up to 32 dofs (the single-tile stage).  False when there is no such kernel for
+    dense model of up to 63 dofs (the single-tile stage up to 32, the blocked stage on a wavefront
+    per world for a padded size of 48 or 64).  False when there is no such kernel for
     this model (the caller then launches the stages one by one)."""
     import ctypes as C
 
     import torch
 
     scratch, plan = _tree_scratch(ctx), _fused_plan(ctx)
-    dense_tile = scratch is None and plan is None and int(m.nv) <= 32 and getattr(ctx, "newton_next_world", None) is not None
-    if (scratch is None and plan is None and not dense_tile) or os.environ.get("IMHIP_NEWTON") == "stages":
+    dense = scratch is None and plan is None and getattr(ctx, "newton_next_world", None) is not None
+    dense_tile = dense and int(m.nv) <= 32
+    dense_column = dense and int(m.nv) > 32 and int(m.nv_pad) in (48, 64)
+    if (scratch is None and plan is None and not (dense_tile or dense_column)) or os.environ.get("IMHIP_NEWTON") == "stages":
         return False
     a = _resident_args(m, d, ctx, nsolving)
     dev = d.efc.J.device
     stream = int(torch.cuda.current_stream(dev).cuda_stream)
     with torch.cuda.device(dev):
-        if dense_tile:
+        if dense_tile or dense_column:
             nworld, nv, pad = int(d.nworld), int(m.nv), int(m.nv_pad)
             h, uni, counter = ctx.h, ctx.newton_dof_union, ctx.newton_next_world
             if h.dtype != torch.float32 or h.device != dev or tuple(h.shape) != (nworld, pad, pad) or not h.is_contiguous():
@@ -804,9 +807,17 @@ def run_resident(m, d, ctx, nsolving) -> bool:
                 raise TypeError("newton_dof_union must be a contiguous int32 (nworld, nv + 1) tensor")
             if counter.dtype != torch.int32 or counter.device != dev or counter.numel() != 1:
                 raise TypeError("newton_next_world must be a one-element int32 tensor")
-            status = _lib.lib().im_newton_solve_dense_tile(C.byref(a), h.data_ptr(), uni.data_ptr(), nv, pad, int(d.M.shape[1]),
-                                                           counter.data_ptr(), stream)  # fmt: skip
-            where = "im_newton_solve_dense_tile"
+            if dense_tile:
+                status = _lib.lib().im_newton_solve_dense_tile(C.byref(a), h.data_ptr(), uni.data_ptr(), nv, pad, int(d.M.shape[1]),
+                                                               counter.data_ptr(), stream)  # fmt: skip
+                where = "im_newton_solve_dense_tile"
+            else:
+                hf = ctx.hfactor
+                if hf.dtype != torch.float32 or hf.device != dev or tuple(hf.shape) != (nworld, pad, pad) or not hf.is_contiguous():
+                    raise TypeError("hfactor must be a contiguous float32 (nworld, nv_pad, nv_pad) tensor")
+                status = _lib.lib().im_newton_solve_dense_column(C.byref(a), h.data_ptr(), hf.data_ptr(), uni.data_ptr(), nv, pad,
+                                                                 int(d.M.shape[1]), counter.data_ptr(), stream)  # fmt: skip
+                where = "im_newton_solve_dense_column"
         elif plan is not None:
             nworld, nv, pad = int(d.nworld), int(m.nv), int(m.nv_pad)
             hf, uni = ctx.hfactor, ctx.newton_dof_union

@@ -552,7 +552,7 @@ def run(launches: int = 32, only: str | None = None) -> None:
             return m, d, ctx, torch.zeros(1, dtype=torch.int32, device=dev)
 
         for name, stage, loop in (("humanoid", "tree", "resident"), ("humanoid", "tree", "stages"), ("humanoid", "dense", "resident"), ("humanoid", "dense", "stages"),
-                                  ("g1", "dense", "stages"), ("g1", "tree", "resident"), ("g1", "tree", "stages"), ("g1", "sparse", "resident"), ("g1", "sparse", "stages"),
+                                  ("g1", "dense", "resident"), ("g1", "dense", "stages"), ("g1", "tree", "resident"), ("g1", "tree", "stages"), ("g1", "sparse", "resident"), ("g1", "sparse", "stages"),
                                   ("snu", "tree", "resident"), ("snu", "sparse", "resident"), ("snu", "sparse", "stages")):  # fmt: skip
             if loop == "stages":
                 os.environ["IMHIP_NEWTON"] = "stages"
