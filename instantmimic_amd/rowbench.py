@@ -553,7 +553,7 @@ def run(launches: int = 32, only: str | None = None) -> None:
 
         for name, stage, loop in (("humanoid", "tree", "resident"), ("humanoid", "tree", "stages"), ("humanoid", "dense", "resident"), ("humanoid", "dense", "stages"),
                                   ("g1", "dense", "resident"), ("g1", "dense", "stages"), ("g1", "tree", "resident"), ("g1", "tree", "stages"), ("g1", "sparse", "resident"), ("g1", "sparse", "stages"),
-                                  ("snu", "tree", "resident"), ("snu", "sparse", "resident"), ("snu", "sparse", "stages")):  # fmt: skip
+                                  ("snu", "dense", "resident"), ("snu", "dense", "stages"), ("snu", "tree", "resident"), ("snu", "sparse", "resident"), ("snu", "sparse", "stages")):  # fmt: skip
             if loop == "stages":
                 os.environ["IMHIP_NEWTON"] = "stages"
             else:

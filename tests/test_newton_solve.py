@@ -141,11 +141,12 @@ def _solve_on_gpu(p, device, *, graph: bool):
     ("g1", 8192, "tree", True, "resident"), ("snu", 131, "tree", False, "resident"), ("snu", 4096, "tree", True, "resident"),
     ("humanoid", 303, "dense", False, "resident"), ("humanoid", 4096, "dense", True, "resident"), ("ant", 69, "dense", True, "resident"),
     ("g1", 205, "dense", False, "resident"), ("g1", 8192, "dense", True, "resident"), ("g1", 207, "dense", False, "stages"),
+    ("snu", 133, "dense", False, "resident"), ("snu", 4096, "dense", True, "resident"), ("snu", 135, "dense", False, "stages"),
 ])  # fmt: skip
 def test_gpu_solve_from_init_context_matches_the_oracle_chain(device, monkeypatch, name, nworld, stage, graph, loop):
     """``loop``: the iterations as eight launches each (``stages``) or as one resident kernel with a
     wavefront per world (``resident``: the tree stage with generated kernels, the sparse stage, the
-    dense single-tile stage up to 32 dofs, the dense blocked stage for a padded size of 48): the same
+    dense single-tile stage up to 32 dofs, the dense blocked stage for a padded size of 48 or 64): the same
     arrays at the end either way."""
     small = nworld <= 301
     p = NC.problem(name, nworld, stage, empty_every=11 if small else 97, warmstart=small, maxiter=12)
