@@ -11,7 +11,9 @@ timed region; every launch takes the next of 16 distinct input sets (> 560 MB in
 launch finds its M or J in the 256 MB memory-side cache.  `value` and `roofline` are this form's.
 Beside it, `iterations_launch`: the three solves of a step as one launch of
 im_assemble_tree_ldl_solve_iters (a grid over worlds x iterations, for callers that know every
-iteration's states in advance; the solves are then independent of one another).  Prints one JSON line.
+iteration's states in advance; the solves are then independent of one another), and `newton_solve`:
+whole constraint solves of the same batch shape with dependent iterations (init_context, the resident
+Newton kernel, force recovery), informative.  Prints one JSON line.
 """
 
 from __future__ import annotations
@@ -101,6 +103,57 @@ def cpu_baseline(batch, plan_struct, gpu_x, seconds: float = 10.0):
     }
 
 
+def newton_solve_leg(torch, use_graph: bool, nsets: int = 8, replays: int = 5, solves_per_replay: int = 8):
+    """Beside the headline: whole constraint solves of the same batch shape with dependent iterations
+    (newton_fusion.solve: init_context, the resident Newton kernel with the fused tree stage, force
+    recovery; tolerance 1e-7, at most 10 iterations), on rotating input sets.  Informative: the
+    headline's metric is the factor-and-solve launch."""
+    from instantmimic_amd.mjw_kernels import newton_fusion as NF
+    from instantmimic_amd.rowbench import newton_case
+
+    cases = [newton_case("humanoid", "tree", seed=21 + k) for k in range(nsets)]
+    for c in cases[:2]:
+        NF.solve(*c)
+    torch.cuda.synchronize()
+    its = cases[0][1].solver_niter.cpu().numpy()
+    unfinished = int((cases[0][2].done.cpu().numpy() == 0).sum())
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    times = []
+    if use_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                for k in range(solves_per_replay):
+                    NF.solve(*cases[k % nsets])
+        torch.cuda.current_stream().wait_stream(side)
+        g.replay()
+        torch.cuda.synchronize()
+    for _ in range(replays):
+        a.record()
+        if use_graph:
+            g.replay()
+        else:
+            for k in range(solves_per_replay):
+                NF.solve(*cases[k % nsets])
+        b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b) * 1e-3 / solves_per_replay)
+    sec = min(times)
+    m, d = cases[0][0], cases[0][1]
+    return {
+        "entry": "newton_fusion.solve: im_newton_init_context, im_newton_tree_stage, im_newton_solve_tree (one resident kernel for the dependent iterations), im_qfrc_constraint_from_grad",
+        "workload": f"humanoid nv={int(m.nv)} nefc={int(d.njmax)} x {int(d.nworld)} worlds, tolerance 1e-7, at most {int(m.opt.iterations)} iterations",
+        "us_per_solve": sec * 1e6,
+        "iterations_mean": float(its.mean()),
+        "iterations_max": int(its.max()),
+        "worlds_unfinished": unfinished,
+        "world_iterations_per_s": float(its.sum()) / sec,
+        "input_sets": nsets,
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -108,6 +161,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--sets", type=int, default=16, help="distinct input sets rotated over")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-solve", action="store_true", help="skip the whole-solve figure (newton_solve)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying hipGraphs")
     ap.add_argument("--single-only", action="store_true", help="time the one-launch-per-solve form only (for profiles of that kernel)")
     ap.add_argument(
@@ -297,6 +351,8 @@ def main() -> int:
         "traffic": TRAFFIC_BYTES_PER_LAUNCH,
     }
 
+    newton = None if args.no_solve else newton_solve_leg(torch, use_graph)
+
     out = {
         "metric": METRIC,
         "value": value,
@@ -332,6 +388,8 @@ def main() -> int:
         },
         "iterations_launch": iterations_launch,
     }
+    if newton is not None:
+        out["newton_solve"] = newton
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(batch, T.tree_ldl_structure(batch.rowadr, batch.rownnz, batch.colind), x_first)
     print(json.dumps(out))

@@ -73,6 +73,61 @@ def _line(kernel, workload, seconds, *, bytes_=None, flops=None, nworld=None):
     print(json.dumps(out), flush=True)
 
 
+def newton_case(name, stage, seed=21, maxiter=10, device="cuda:0"):
+    """(m, d, ctx, nsolving) of one step on the tree of `name`: 2 equality rows, 3 friction-loss rows, the
+    rest one-sided; everything the solve writes starts as it happens to lie there."""
+    import torch
+
+    from . import synth
+    from .mjw_kernels import newton_fusion as NF
+    from .mjw_kernels import sparse_hessian as SH
+    from .mjw_kernels import tree_ldl as T
+
+    dev = torch.device(device)
+
+    def t(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    shape = synth.SHAPES[name]
+    b = synth.make_batch(shape, ragged_nefc=True)
+    rng = np.random.default_rng(seed)
+    nworld, nv, njmax = b.nworld, shape.nv, shape.nefc
+    m = synth.model_from_parents(shape.parents)
+    pad = int(m.nv_pad)
+    nefc = np.maximum(b.nefc, 8).astype(np.int32)
+    tables = [t(a) for a in NF.mul_m_tables(b.rowadr, b.rownnz, b.colind)]
+    m.M_mulm_rowadr, m.M_mulm_col, m.M_mulm_madr = tables
+    m.opt = SimpleNamespace(solver=2, cone=0, integrator=3, iterations=maxiter, ls_iterations=50, disableflags=256,
+                            tolerance=torch.full((1,), 1e-7, device=dev), ls_tolerance=torch.full((1,), 0.01, device=dev))  # fmt: skip
+    m.stat = SimpleNamespace(meaninertia=torch.ones(1, device=dev))
+    f = lambda *shape_: torch.zeros(shape_, device=dev)  # noqa: E731
+    i = lambda *shape_: torch.zeros(shape_, dtype=torch.int32, device=dev)  # noqa: E731
+    u8 = lambda: torch.zeros(nworld, dtype=torch.uint8, device=dev)  # noqa: E731
+    qs = t(rng.normal(size=(nworld, nv)).astype(np.float32))
+    M_ = t(b.M)
+    smooth = f(nworld, nv)
+    NF.mul_m(M_, qs, smooth, *tables)
+    d = SimpleNamespace(nworld=nworld, njmax=njmax, M=M_, ne=t(np.full(nworld, 2, np.int32)), nf=t(np.full(nworld, 3, np.int32)),
+                        nefc=t(nefc), qfrc_smooth=smooth, qacc_smooth=qs, qacc_warmstart=None, qacc=f(nworld, nv),
+                        qfrc_constraint=f(nworld, nv), solver_niter=i(nworld), overflow=i(nworld),
+                        efc=SimpleNamespace(J=t(b.J), D=t((10.0 ** rng.uniform(0, 3, (nworld, njmax))).astype(np.float32)),
+                                            frictionloss=t(rng.uniform(0.1, 1.0, (nworld, njmax)).astype(np.float32)),
+                                            aref=t(rng.normal(scale=2.0, size=(nworld, njmax)).astype(np.float32)),
+                                            Ma=f(nworld, nv), force=f(nworld, njmax), state=i(nworld, njmax)))  # fmt: skip
+    ctx = SimpleNamespace(search=f(nworld, nv), search_dot=f(nworld), mv=f(nworld, nv), jv=f(nworld, njmax), Jaref=f(nworld, njmax),
+                          done=u8(), alpha=f(nworld), improvement=f(nworld), ls_exhausted=u8(), quad_changed_ids=i(nworld, njmax),
+                          quad_changed_count=i(nworld), state_changed_count=i(nworld), search_unchanged=u8(), grad=f(nworld, pad),
+                          grad_dot=f(nworld), grad_scale=f(nworld), newton_decrement=f(nworld), h=f(nworld, pad, pad),
+                          hfactor=f(nworld, pad, pad))  # fmt: skip
+    if stage == "tree":
+        ctx.newton_tree_scratch = T.create_tree_factor_solve_scratch(m, dev)
+    elif stage == "sparse":
+        ctx.sparse_hessian_plan, why = SH.plan_for_model(m, ctx, [], SH.block_width(pad), device=dev)
+        assert ctx.sparse_hessian_plan is not None, why
+    NF.attach_scratch(m, d, ctx, dev)
+    return m, d, ctx, torch.zeros(1, dtype=torch.int32, device=dev)
+
+
 def run(launches: int = 32, only: str | None = None) -> None:
     """``only``: comma-separated section names out of trees, generated, stress, muscles, walks, iteration, solve, implicit, bodies."""
     import torch
@@ -509,47 +564,6 @@ def run(launches: int = 32, only: str | None = None) -> None:
     if section("solve"):
         import os
 
-        def newton_case(name, stage, seed=21, maxiter=10):
-            """(m, d, ctx, nsolving) of one step on the tree of `name`: 2 equality rows, 3 friction-loss rows, the
-            rest one-sided; everything the solve writes starts as it happens to lie there."""
-            shape = synth.SHAPES[name]
-            b = synth.make_batch(shape, ragged_nefc=True)
-            rng = np.random.default_rng(seed)
-            nworld, nv, njmax = b.nworld, shape.nv, shape.nefc
-            m = synth.model_from_parents(shape.parents)
-            pad = int(m.nv_pad)
-            nefc = np.maximum(b.nefc, 8).astype(np.int32)
-            tables = [t(a) for a in NF.mul_m_tables(b.rowadr, b.rownnz, b.colind)]
-            m.M_mulm_rowadr, m.M_mulm_col, m.M_mulm_madr = tables
-            m.opt = SimpleNamespace(solver=2, cone=0, integrator=3, iterations=maxiter, ls_iterations=50, disableflags=256,
-                                    tolerance=torch.full((1,), 1e-7, device=dev), ls_tolerance=torch.full((1,), 0.01, device=dev))  # fmt: skip
-            m.stat = SimpleNamespace(meaninertia=torch.ones(1, device=dev))
-            f = lambda *shape_: torch.zeros(shape_, device=dev)  # noqa: E731
-            i = lambda *shape_: torch.zeros(shape_, dtype=torch.int32, device=dev)  # noqa: E731
-            u8 = lambda: torch.zeros(nworld, dtype=torch.uint8, device=dev)  # noqa: E731
-            qs = t(rng.normal(size=(nworld, nv)).astype(np.float32))
-            M_ = t(b.M)
-            smooth = f(nworld, nv)
-            NF.mul_m(M_, qs, smooth, *tables)
-            d = SimpleNamespace(nworld=nworld, njmax=njmax, M=M_, ne=t(np.full(nworld, 2, np.int32)), nf=t(np.full(nworld, 3, np.int32)),
-                                nefc=t(nefc), qfrc_smooth=smooth, qacc_smooth=qs, qacc_warmstart=None, qacc=f(nworld, nv),
-                                qfrc_constraint=f(nworld, nv), solver_niter=i(nworld), overflow=i(nworld),
-                                efc=SimpleNamespace(J=t(b.J), D=t((10.0 ** rng.uniform(0, 3, (nworld, njmax))).astype(np.float32)),
-                                                    frictionloss=t(rng.uniform(0.1, 1.0, (nworld, njmax)).astype(np.float32)),
-                                                    aref=t(rng.normal(scale=2.0, size=(nworld, njmax)).astype(np.float32)),
-                                                    Ma=f(nworld, nv), force=f(nworld, njmax), state=i(nworld, njmax)))  # fmt: skip
-            ctx = SimpleNamespace(search=f(nworld, nv), search_dot=f(nworld), mv=f(nworld, nv), jv=f(nworld, njmax), Jaref=f(nworld, njmax),
-                                  done=u8(), alpha=f(nworld), improvement=f(nworld), ls_exhausted=u8(), quad_changed_ids=i(nworld, njmax),
-                                  quad_changed_count=i(nworld), state_changed_count=i(nworld), search_unchanged=u8(), grad=f(nworld, pad),
-                                  grad_dot=f(nworld), grad_scale=f(nworld), newton_decrement=f(nworld), h=f(nworld, pad, pad),
-                                  hfactor=f(nworld, pad, pad))  # fmt: skip
-            if stage == "tree":
-                ctx.newton_tree_scratch = T.create_tree_factor_solve_scratch(m, dev)
-            elif stage == "sparse":
-                ctx.sparse_hessian_plan, why = SH.plan_for_model(m, ctx, [], SH.block_width(pad), device=dev)
-                assert ctx.sparse_hessian_plan is not None, why
-            NF.attach_scratch(m, d, ctx, dev)
-            return m, d, ctx, torch.zeros(1, dtype=torch.int32, device=dev)
 
         for name, stage, loop in (("humanoid", "tree", "resident"), ("humanoid", "tree", "stages"), ("humanoid", "dense", "resident"), ("humanoid", "dense", "stages"),
                                   ("g1", "dense", "resident"), ("g1", "dense", "stages"), ("g1", "tree", "resident"), ("g1", "tree", "stages"), ("g1", "sparse", "resident"), ("g1", "sparse", "stages"),
