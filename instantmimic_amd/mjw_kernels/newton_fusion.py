@@ -651,6 +651,10 @@ def _init_before_factor(m, d, ctx) -> bool:
 
     if os.environ.get("IMHIP_NEWTON") == "stages":
         return False
+    # the one launch takes the argument block of the resident loop: a context without the loop's own
+    # arrays (a caller that only wants the start of a solve) keeps the five launches
+    if any(getattr(ctx, name, None) is None for name in ("mv", "jv", "alpha", "improvement", "ls_exhausted", "search")):
+        return False
     smooth, aref = d.qacc_smooth, d.efc.aref
     nworld, nv = int(d.nworld), int(m.nv)
     dev = d.efc.J.device
