@@ -9,10 +9,11 @@
 // Lane c keeps column c of the upper triangle in registers, u[r] = U[r][c].  A block row's
 // elements first lose the earlier block rows' sums (for every element a sum of 16 fused
 // multiply-adds started from zero per earlier block row, then one subtraction: the blocked order),
-// the factor of the other column arriving by lane reads; inside the block row every lane --
+// the factor of the other column arriving inside the multiply-add (the block row's columns copied
+// into every row of sixteen lanes, then a DPP row broadcast); inside the block row every lane --
 // diagonal block, blocks to its right, gradient column alike -- runs
 //   u[k + r] = (u[k + r] - sum_{q < r} U[k + q][k + r] * u[k + q]) / U[k + r][k + r]
-// with column k + r's elements read from its lane, which is the diagonal tile's Cholesky and the
+// with column k + r's elements broadcast the same way, which is the diagonal tile's Cholesky and the
 // triangular solves of the tiles to its right in one.  The backward solve needs rows of U across
 // lanes: a 16 x 16 tile at a time is turned round through LDS.  The gradient column rides in lane
 // 63 (a padding column that no other lane reads).
@@ -38,6 +39,30 @@ constexpr int kColStagedRows = 32;  // the changed rows a stage keeps in LDS (a 
 template <int NBLK>
 __host__ __device__ constexpr int column_stage_words() {
   return 16 * 17 + (kColStagedRows + 1) * 16 * NBLK + kColStagedRows + 16 * NBLK;
+}
+
+// acc[r] = fma(value of lane r of the caller's row of sixteen lanes of `other`, own, acc[r]), r = 0 .. 15:
+// the broadcast rides in the multiply-add (DPP).  The leading wait covers a register written just
+// before: a DPP read needs two idle cycles after a vector write of its source, which the compiler
+// does not see inside the block.
+__device__ __forceinline__ void row_fmac16(float (&acc)[16], float other, float own) {
+#define IM_ROW_FMAC(n) "v_fmac_f32_dpp %" #n ", %16, %17 row_newbcast:" #n " row_mask:0xf bank_mask:0xf\n\t"
+  asm("s_nop 1\n\t" IM_ROW_FMAC(0) IM_ROW_FMAC(1) IM_ROW_FMAC(2) IM_ROW_FMAC(3) IM_ROW_FMAC(4) IM_ROW_FMAC(5) IM_ROW_FMAC(6)
+          IM_ROW_FMAC(7) IM_ROW_FMAC(8) IM_ROW_FMAC(9) IM_ROW_FMAC(10) IM_ROW_FMAC(11) IM_ROW_FMAC(12) IM_ROW_FMAC(13)
+              IM_ROW_FMAC(14) IM_ROW_FMAC(15)
+      : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7]),
+        "+v"(acc[8]), "+v"(acc[9]), "+v"(acc[10]), "+v"(acc[11]), "+v"(acc[12]), "+v"(acc[13]), "+v"(acc[14]), "+v"(acc[15])
+      : "v"(other), "v"(own));
+#undef IM_ROW_FMAC
+}
+// v = fma(value of lane r of the row of minus_row[q], own[q], v) for q = 0 .. r - 1 in order (r a
+// constant after unrolling): the statements keep their order among themselves, the first one waits
+__device__ __forceinline__ void row_chain(float &v, const float (&minus_row)[16], const float *own, int r) {
+  asm volatile("s_nop 1");
+#pragma unroll
+  for (int q = 0; q < 15; ++q)
+    if (q < r)
+      asm volatile("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "+v"(v) : "v"(minus_row[q]), "v"(own[q]), "n"(r));
 }
 
 __device__ __forceinline__ float lane_value(float v, int lane) {  // `lane` the same for the whole wavefront
@@ -143,28 +168,41 @@ __device__ __forceinline__ void dense_column_world(float *scr, float *Hw, float 
 #pragma unroll
     for (int kb = 0; kb < NBLK; ++kb) {
       const int k = 16 * kb;
+      // lane L's copy of a register of lane k + (L & 15): the block row's sixteen columns side by side in
+      // every row of sixteen lanes, from where one lane's value reaches its row inside the multiply-add
+      // (a DPP row broadcast; the copy comes through the LDS crossbar)
+      const int from_block = 4 * (k + (lane & 15));
 #pragma unroll
       for (int jb = 0; jb < kb; ++jb) {
         const int j = 16 * jb;
+        float sum[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float sum = 0.0f;
+        for (int r = 0; r < 16; ++r) sum[r] = 0.0f;
 #pragma unroll
-          for (int t = 0; t < 16; ++t) sum = fma_(lane_value(u[j + t], k + r), u[j + t], sum);
-          u[k + r] = u[k + r] - sum;
+        for (int t = 0; t < 16; ++t) {
+          const float other = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from_block, __builtin_bit_cast(int, u[j + t])));
+          row_fmac16(sum, other, u[j + t]);  // sum[r] = fma(U[j + t][k + r], u[j + t], sum[r])
         }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) u[k + r] = u[k + r] - sum[r];
       }
+      float minus_row[16];  // minus_row[q]: minus the block copy of row k + q, once that row is final
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         if (k + r == RHS) continue;  // (a matrix of 64 columns: its last one is padding, and lane 63 holds the gradient)
         float v = u[k + r];
-#pragma unroll
-        for (int q = 0; q < r; ++q) v = fma_(-lane_value(u[k + q], k + r), u[k + q], v);
+        row_chain(v, minus_row, &u[k], r);  // v = fma(-U[k + q][k + r], u[k + q], v) for q < r, in order
         // the pivot is lane k + r's value
         float d, inv;
         pivot_sqrt_rcp(lane_value(v, k + r), true, d, inv);
         u[k + r] = lane == k + r ? d : v * inv;
         if (lane == k + r) rdiag = inv;
+        if (r < 15) {
+          minus_row[r] = -__builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from_block, __builtin_bit_cast(int, u[k + r])));
+          // in its register here, ahead of the next step's wait: the negation is a vector write that
+          // the DPP reads of the steps to come must not follow too closely
+          asm volatile("" : "+v"(minus_row[r]));
+        }
       }
     }
     // ---- the corner of the augmented column, the factor out
@@ -306,7 +344,7 @@ __host__ __device__ inline int column_resident_area_words(int nv, int njmax) {
 __host__ __device__ inline int column_resident_shared_words(int nterm, int nv) { return (nterm + nv + 1 + 3) & ~3; }
 
 template <int NBLK, int WAVES, int HELD>
-__global__ __launch_bounds__(64 * WAVES, 2) void newton_dense_column_resident_kernel(
+__global__ __launch_bounds__(64 * WAVES, NBLK == 3 ? 3 : 2) void newton_dense_column_resident_kernel(
     resident::NewtonArgs a, float *__restrict__ H_, float *__restrict__ U_, int32_t *__restrict__ uni_,
     int *__restrict__ next_world) {
   extern __shared__ float lds[];
@@ -393,8 +431,7 @@ extern "C" int im_newton_solve_dense_column(const im_newton_args *p, float *H, f
   if (!probed) {  // once per process: a variant that spills registers is left out; the large dynamic LDS is asked for
     for (int i = 0; i < kVariants; ++i) {
       hipFuncAttributes fa{};
-      // (the 64-column kernels park one register that holds scalar values in memory: 28 bytes a lane)
-      usable[i] = hipFuncGetAttributes(&fa, variants[i].fn) == hipSuccess && fa.localSizeBytes <= 32 &&
+      usable[i] = hipFuncGetAttributes(&fa, variants[i].fn) == hipSuccess && fa.localSizeBytes == 0 &&
                   hipFuncSetAttribute(variants[i].fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                       160 * 1024 - (int)fa.sharedSizeBytes) == hipSuccess;
       regs[i] = fa.numRegs;
