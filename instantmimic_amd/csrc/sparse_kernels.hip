@@ -385,6 +385,7 @@ struct SparseWave {
   int solve_words;            // length of that stretch, a multiple of 4 (0: not staged)
   const int32_t *tile_index;  // [tile][4][64]: (index into M + 1) << 16 | (slot + 1), 0 = none
   int block, nM;              // the plan's block width; length of a row of M
+  int staged_rows;            // update stage: changed rows of J a world keeps in LDS, 16 or 32 (more are read from memory)
 };
 
 template <int NT>
@@ -603,13 +604,12 @@ __global__ __launch_bounds__(256, 4) void sparse_init_mfma_kernel(
 
 // Per-iteration factor stage, one wavefront per world (WAVES worlds per workgroup share the LDS
 // copy of the factor and solve tables: four, eight or sixteen, chosen by the launcher).  Same arithmetic as
-// sparse_update_kernel below; the changed constraint rows are staged in LDS (up to kStagedRows
+// sparse_update_kernel below; the changed constraint rows are staged in LDS (up to A.staged_rows
 // of them, else they are read from memory), packed H is updated in LDS and written back whole,
 // and a lane keeps four pairs' table look-ups in flight.
-constexpr int kStagedRows = 16;
-// a dof's elements of the staged rows lie side by side, 17 words per dof: the row number is then a
-// constant offset in every access, and lanes that read different dofs meet in no LDS bank
-constexpr int kStagedStride = kStagedRows + 1;
+// a dof's elements of the staged rows lie side by side, one word more than rows per dof (17 or 33): lanes that
+// read different dofs meet in no LDS bank.  32 rows where that costs a CU no world, 16 otherwise.
+constexpr int kStagedRowsMax = 32;
 
 // The factor and solve tables of a plan into LDS, for a workgroup of T threads (a flat 16-byte copy,
 // every load issued before the first store); Q's table pointers then address the copy.
@@ -654,9 +654,9 @@ __device__ __forceinline__ void stage_update_tables(const SparseWave &A, SparseD
     for (int i = 0; i < 5; ++i) Q.t[FL + i] = tab + A.staged_words + A.solve[i];
   }
 }
-__host__ __device__ inline int update_world_words(int nslots, int n, int block) {
+__host__ __device__ inline int update_world_words(int nslots, int n, int block, int staged_rows) {
   const int nw = (block + 31) / 32;
-  return (nslots + n + 2 * nw + 2 * n + kStagedStride * n + kStagedRows + 3) & ~3;
+  return (nslots + n + 2 * nw + 2 * n + (staged_rows + 1) * n + staged_rows + 3) & ~3;
 }
 
 // The stage for one world and one wavefront (`world_lds`: update_world_words of LDS of its own).
@@ -677,8 +677,9 @@ __device__ __forceinline__ void sparse_update_world(
   float *red = iD + n;                               // [2][nw]
   int *ul = (int *)(red + 2 * nw);                   // [n] ascending dofs touched by the changed rows
   unsigned *mkl = (unsigned *)(ul + n);              // [n] per dof: bit t set where staged row t is nonzero there
-  float *jr = (float *)(mkl + n);                    // [n][kStagedStride] changed rows of J, a dof's elements together
-  float *sd = jr + kStagedStride * n;                // [kStagedRows] D of the row, negated for a row that left the quadratic state
+  const int cap = A.staged_rows, stride = cap + 1;
+  float *jr = (float *)(mkl + n);                    // [n][stride] changed rows of J, a dof's elements together
+  float *sd = jr + stride * n;                       // [cap] D of the row, negated for a row that left the quadratic state
   float *U = U_ + (size_t)w * Q.nv_pad * Q.nv_pad;
   const float *gw = grad + (size_t)w * ldg;
   const float *Jw = J + (size_t)w * njmax * n;
@@ -695,7 +696,7 @@ __device__ __forceinline__ void sparse_update_world(
 #define IM_SSTAMP(k) do {} while (0)
 #endif
   if (count > 0) {
-    const bool staged = count <= kStagedRows;
+    const bool staged = count <= cap;
     // requests first: the changed rows, their weights, packed H
     bool hit = false;  // whether a changed row touches this lane's dof
     if (staged) {
@@ -703,24 +704,31 @@ __device__ __forceinline__ void sparse_update_world(
       const int rq = idw[tq];
       const float dq = Dw[rq];
       const int sq = sw[rq];
-      float rowv[kStagedRows];
-#pragma unroll
-      for (int t = 0; t < kStagedRows; ++t) {
-        const int r = __builtin_amdgcn_readlane(rq, t < count ? t : 0);
-        rowv[t] = Jw[r * n + (lane < n ? lane : n - 1)];
-      }
       for (int s = lane; s < nfac; s += 64) N[s] = U[s];
-      if (lane < kStagedRows) sd[lane] = sq == quad ? dq : -dq;
-      if (lane < n) {
-        unsigned mk = 0u;
-        float *mine = jr + lane * kStagedStride;
+      if (lane < cap) sd[lane] = sq == quad ? dq : -dq;
+      unsigned mk = 0u;
+      float *mine = jr + (lane < n ? lane : 0) * stride;
+      // sixteen rows at a time: their elements of this lane's dof asked for together
 #pragma unroll
-        for (int t = 0; t < kStagedRows; ++t) {
-          if (t < count) {
-            mine[t] = rowv[t];
-            mk |= (unsigned)(rowv[t] != 0.0f) << t;
+      for (int half = 0; half < kStagedRowsMax / 16; ++half) {
+        if (16 * half >= count) break;  // the same for every lane
+        float rowv[16];
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+          const int r = __builtin_amdgcn_readlane(rq, 16 * half + t);  // (lanes at or past count hold row count - 1)
+          rowv[t] = Jw[r * n + (lane < n ? lane : n - 1)];
+        }
+        if (lane < n) {
+#pragma unroll
+          for (int t = 0; t < 16; ++t) {
+            if (16 * half + t < count) {
+              mine[16 * half + t] = rowv[t];
+              mk |= (unsigned)(rowv[t] != 0.0f) << (16 * half + t);
+            }
           }
         }
+      }
+      if (lane < n) {
         mkl[lane] = mk;
         hit = mk != 0u;
       }
@@ -765,7 +773,7 @@ __device__ __forceinline__ void sparse_update_world(
         if (staged) {
           // only the rows in which both dofs are nonzero add to the pair, ascending: most pairs
           // of the union share no row at all
-          const float *jrow = jr + row[k] * kStagedStride, *jcol = jr + col[k] * kStagedStride;
+          const float *jrow = jr + row[k] * stride, *jcol = jr + col[k] * stride;
           for (unsigned mm = mkl[row[k]] & mkl[col[k]]; mm; mm &= mm - 1u) {
             const int t = __builtin_ctz(mm);
             delta = fma_(sd[t] * jrow[t], jcol[t], delta);
@@ -856,7 +864,7 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void sparse_update_wave_ker
   __syncthreads();  // the only workgroup barrier
   const int w = blockIdx.x * WAVES + wv;
   if (w >= nworld || (done && done[w]) || state_changes[w] == 0) return;
-  float *world_lds = lds + A.staged_words + A.solve_words + wv * update_world_words(Q.nslots, Q.nv, A.block);
+  float *world_lds = lds + A.staged_words + A.solve_words + wv * update_world_words(Q.nslots, Q.nv, A.block, A.staged_rows);
   sparse_update_world(A, Q, world_lds, changes, ids, ld_ids, J, njmax, D, state, quad, grad, ldg, U_, uni_, search_,
                       search_dot, decrement, w, lane);
 }
@@ -865,8 +873,8 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void sparse_update_wave_ker
 // line search to convergence, WAVES worlds per workgroup sharing one copy of the plan's tables.
 // Per wavefront in LDS: the world's row of M and the search direction, and one area that the staged
 // tile of J, the gradient's row list and the stage's factor use one after the other.
-__host__ __device__ inline int resident_area_words(int nslots, int n, int block, int njmax) {
-  int words = update_world_words(nslots, n, block);
+__host__ __device__ inline int resident_area_words(int nslots, int n, int block, int njmax, int staged_rows) {
+  int words = update_world_words(nslots, n, block, staged_rows);
   const int tile = 64 * 17, grad = 2 * njmax + n;
   words = words > tile ? words : tile;
   words = words > grad ? words : grad;
@@ -884,7 +892,7 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_sparse_resident
   const int nv = a.nv, njmax = a.njmax, nworld = a.nworld;
   uint32_t *term = (uint32_t *)(lds + A.staged_words + A.solve_words);
   int *radr = (int *)(term + a.nterm);
-  const int area = resident_area_words(Q.nslots, nv, A.block, njmax);
+  const int area = resident_area_words(Q.nslots, nv, A.block, njmax, A.staged_rows);
   // (M is read from memory by the round's one product with it: its row would cost a CU a third of its worlds)
   float *mine = (float *)(radr + nv + 1) + wv * (area + resident::kept_words(nv, njmax, 0));
   resident::LoopLds L;
@@ -1162,6 +1170,7 @@ int im_sparse_init_factor(const im_sparse_plan *plan, const uint8_t *done, const
     const size_t staged = (size_t)(plan->t[im::kStaged] - plan->t[0]);  // tables are padded to 16 bytes
     A.staged_words = (int)staged;
     A.tile_index = plan->tile_index;
+    A.staged_rows = 0;  // (the update stage's)
     A.solve_words = 0;
     A.block = plan->block;
     A.nM = plan->nM;
@@ -1222,10 +1231,12 @@ int im_sparse_update_factor(const im_sparse_plan *plan, const uint8_t *done, con
     A.tile_index = nullptr;
     A.block = plan->block;
     A.nM = 0;
-    const size_t per_world =
-        ((size_t)plan->nslots + n + 2 * nw + 2 * n + (size_t)im::kStagedStride * n + im::kStagedRows + 3) & ~(size_t)3;
     const int32_t *solve_end = plan->t[im::RK] + ((plan->sizes[im::RK] + 3) & ~3);
     const size_t solve_words = (size_t)(solve_end - plan->t[im::FL]);
+    // 32 staged rows where a CU still holds sixteen worlds with them, else 16
+    A.staged_rows =
+        4 * (staged + solve_words + 16 * (size_t)im::update_world_words(plan->nslots, n, plan->block, 32)) <= 160 * 1024 ? 32 : 16;
+    const size_t per_world = (size_t)im::update_world_words(plan->nslots, n, plan->block, A.staged_rows);
     for (int i = 0; i < 5; ++i) A.solve[i] = (int)(plan->t[im::FL + i] - plan->t[im::FL]);
     A.solve_words = (int)solve_words;
     const size_t wave_lds = 4 * (staged + solve_words + 4 * per_world);
@@ -1298,7 +1309,9 @@ int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *p, 
   A.solve_words = (int)solve_words;
   if (staged > 8192 || solve_words > 4096) return IM_ERR_UNSUPPORTED;
   const size_t shared = staged + solve_words + (size_t)p->nterm + n + 1;
-  const size_t per_wave = (size_t)im::resident_area_words(plan->nslots, n, plan->block, njmax) + im::resident::kept_words(n, njmax, 0);
+  auto wave_words = [&](int staged_rows) {
+    return (size_t)im::resident_area_words(plan->nslots, n, plan->block, njmax, staged_rows) + im::resident::kept_words(n, njmax, 0);
+  };
   // the most worlds per workgroup (one workgroup per CU) that 160 KB of LDS admit and whose kernel
   // keeps to registers
   struct Variant {
@@ -1330,8 +1343,12 @@ int im_newton_solve_sparse(const im_sparse_plan *plan, const im_newton_args *p, 
     probed = true;
   }
   for (int i = 0; i < kVariants; ++i) {
-    const size_t lds = 4 * (shared + (size_t)variants[i].waves * per_wave);
-    if (!usable[i] || lds > 158 * 1024 || variants[i].held != (njmax <= 64 ? 2 : 0)) continue;
+    if (!usable[i] || variants[i].held != (njmax <= 64 ? 2 : 0)) continue;
+    // 32 staged rows where the workgroup still fits with them (they cost a CU no world then), else 16
+    // (snu: 32 rows with eight worlds per CU instead of twelve was measured slower, 1344 against 1283 us per loop)
+    A.staged_rows = 4 * (shared + (size_t)variants[i].waves * wave_words(32)) <= 158 * 1024 ? 32 : 16;
+    const size_t lds = 4 * (shared + (size_t)variants[i].waves * wave_words(A.staged_rows));
+    if (lds > 158 * 1024) continue;
     const int waves = variants[i].waves;
     // as many workgroups as stay resident at once (LDS, and sixteen wavefronts of up to 128 registers
     // per CU); the others' worlds are taken up by the wavefronts that finish
