@@ -697,6 +697,7 @@ __device__ __forceinline__ void sparse_update_world(
 #endif
   if (count > 0) {
     const bool staged = count <= cap;
+    const bool masked = !staged && count <= 128 && 2 * count + 4 * n <= stride * n + cap;
     // requests first: the changed rows, their weights, packed H
     bool hit = false;  // whether a changed row touches this lane's dof
     if (staged) {
@@ -732,6 +733,38 @@ __device__ __forceinline__ void sparse_update_world(
         mkl[lane] = mk;
         hit = mk != 0u;
       }
+    } else if (masked) {
+      // more rows than the staged capacity: their numbers, their weights and a mask of up to 128
+      // rows per dof go where the staged rows would lie; J's elements then come from memory, but
+      // only those of the rows that a pair's two dofs share
+      int *rid = (int *)jr;                         // [count]
+      float *sdv = jr + count;                      // [count]
+      unsigned *mk4 = (unsigned *)(jr + 2 * count);  // [n][4]
+      for (int s = lane; s < nfac; s += 64) N[s] = U[s];
+      for (int t = lane; t < count; t += 64) {
+        const int r = idw[t];
+        rid[t] = r;
+        sdv[t] = sw[r] == quad ? Dw[r] : -Dw[r];
+      }
+      unsigned any = 0u;
+#pragma unroll
+      for (int word = 0; word < 4; ++word) {
+        unsigned mk = 0u;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int t0 = 32 * word + 16 * half;
+          if (t0 >= count) break;  // the same for every lane
+          float rowv[16];
+#pragma unroll
+          for (int t = 0; t < 16; ++t) rowv[t] = Jw[idw[t0 + t < count ? t0 + t : count - 1] * n + (lane < n ? lane : n - 1)];
+#pragma unroll
+          for (int t = 0; t < 16; ++t)
+            if (t0 + t < count) mk |= (unsigned)(rowv[t] != 0.0f) << (16 * half + t);
+        }
+        if (lane < n) mk4[4 * lane + word] = mk;
+        any |= mk;
+      }
+      hit = lane < n && any != 0u;
     } else {
       for (int s = lane; s < nfac; s += 64) N[s] = U[s];
       if (lane < n)
@@ -777,6 +810,19 @@ __device__ __forceinline__ void sparse_update_world(
           for (unsigned mm = mkl[row[k]] & mkl[col[k]]; mm; mm &= mm - 1u) {
             const int t = __builtin_ctz(mm);
             delta = fma_(sd[t] * jrow[t], jcol[t], delta);
+          }
+        } else if (masked) {
+          const int *rid = (const int *)jr;
+          const float *sdv = jr + count;
+          const unsigned *mk4 = (const unsigned *)(jr + 2 * count);
+#pragma unroll
+          for (int word = 0; word < 4; ++word) {
+            if (32 * word >= count) break;  // the same for every lane
+            for (unsigned mm = mk4[4 * row[k] + word] & mk4[4 * col[k] + word]; mm; mm &= mm - 1u) {
+              const int t = 32 * word + __builtin_ctz(mm);
+              const int r = rid[t];
+              delta = fma_(sdv[t] * Jw[r * n + row[k]], Jw[r * n + col[k]], delta);
+            }
           }
         } else {
           for (int t = 0; t < count; ++t) {
