@@ -186,6 +186,7 @@ __device__ __forceinline__ void dense_tile_world(const TileArea<NP> &T, int *ul,
   // side by side, 17 words a dof) with a mask per dof of the rows that are nonzero there; more
   // changed rows than that are read from memory pair by pair.
   const bool staged = count <= kTileStagedRows;
+  const bool masked = !staged && count <= 128 && 2 * count + 4 * nv <= (kTileStagedRows + 1) * NP;
   float *jr = (float *)(ul + 36);             // [nv][kTileStagedRows + 1]
   float *sd = jr + (kTileStagedRows + 1) * NP;  // [kTileStagedRows] D of the row, negated for a row that left the quadratic state
   unsigned *mkl = (unsigned *)(sd + kTileStagedRows);  // [nv]
@@ -214,6 +215,39 @@ __device__ __forceinline__ void dense_tile_world(const TileArea<NP> &T, int *ul,
       mkl[i] = mk;
       hit = mk != 0u;
     }
+  } else if (masked) {
+    // more rows than the staged capacity: their numbers, their weights and a mask of up to 128 rows per
+    // dof go where the staged rows would lie; J's elements then come from memory, but only those of
+    // the rows that a pair's two dofs share
+    int *rid = (int *)jr;                          // [count]
+    float *sdv = jr + count;                       // [count]
+    unsigned *mk4 = (unsigned *)(jr + 2 * count);  // [nv][4]
+    for (int t = i; t < count; t += LG) {
+      const int r = idw[t];
+      rid[t] = r;
+      sdv[t] = sw[r] == quad ? Dw[r] : -Dw[r];
+    }
+    unsigned any = 0u;
+#pragma unroll
+    for (int word = 0; word < 4; ++word) {
+      unsigned mw = 0u;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int t0 = 32 * word + 16 * half;
+        if (t0 < count) {  // (a group's count: the two groups of a wavefront may differ)
+          float rowv[16];
+#pragma unroll
+          for (int t = 0; t < 16; ++t)
+            rowv[t] = Jw[(size_t)idw[t0 + t < count ? t0 + t : count - 1] * nv + (i < nv ? i : nv - 1)];
+#pragma unroll
+          for (int t = 0; t < 16; ++t)
+            if (t0 + t < count) mw |= (unsigned)(rowv[t] != 0.0f) << (16 * half + t);
+        }
+      }
+      if (i < nv) mk4[4 * i + word] = mw;
+      any |= mw;
+    }
+    hit = i < nv && any != 0u;
   } else if (i < nv) {
     for (int t = 0; t < count && !hit; ++t) hit = Jw[(size_t)idw[t] * nv + i] != 0.0f;
   }
@@ -239,6 +273,20 @@ __device__ __forceinline__ void dense_tile_world(const TileArea<NP> &T, int *ul,
       for (unsigned mm = mkl[row] & mkl[col]; mm; mm &= mm - 1u) {
         const int t = __builtin_ctz(mm);
         delta = fma_(sd[t] * jrow[t], jcol[t], delta);
+      }
+    } else if (masked) {
+      const int *rid = (const int *)jr;
+      const float *sdv = jr + count;
+      const unsigned *mk4 = (const unsigned *)(jr + 2 * count);
+#pragma unroll
+      for (int word = 0; word < 4; ++word) {
+        if (32 * word < count) {
+          for (unsigned mm = mk4[4 * row + word] & mk4[4 * col + word]; mm; mm &= mm - 1u) {
+            const int t = 32 * word + __builtin_ctz(mm);
+            const int r = rid[t];
+            delta = fma_(sdv[t] * Jw[(size_t)r * nv + row], Jw[(size_t)r * nv + col], delta);
+          }
+        }
       }
     } else {
       for (int t = 0; t < count; ++t) {
