@@ -90,6 +90,7 @@ __device__ __forceinline__ void dense_column_world(float *scr, float *Hw, float 
   if (refactor) {
     // ---- the changed rows, the dof union
     const bool staged = count <= kColStagedRows;
+    const bool masked = !staged && count <= 128 && 2 * count + 4 * nv <= (kColStagedRows + 1) * PAD;
     unsigned mk = 0u;
     bool hit = false;
     if (staged && count > 0) {
@@ -122,12 +123,75 @@ __device__ __forceinline__ void dense_column_world(float *scr, float *Hw, float 
         mkl[lane] = mk;
         hit = mk != 0u;
       }
+    } else if (masked) {
+      // more rows than the staged capacity: their numbers, their weights and a mask of up to 128 rows per
+      // dof go where the staged rows would lie; J's elements then come from memory, but only those of
+      // the rows that a pair's two dofs share
+      int *rid = (int *)jr;                          // [count]
+      float *sdv = jr + count;                       // [count]
+      unsigned *mk4 = (unsigned *)(jr + 2 * count);  // [nv][4]
+      for (int t = lane; t < count; t += 64) {
+        const int r = idw[t];
+        rid[t] = r;
+        sdv[t] = sw[r] == quad ? Dw[r] : -Dw[r];
+      }
+      unsigned any = 0u;
+#pragma unroll
+      for (int word = 0; word < 4; ++word) {
+        unsigned mw = 0u;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int t0 = 32 * word + 16 * half;
+          if (t0 >= count) break;  // the same for every lane
+          float rowv[16];
+#pragma unroll
+          for (int t = 0; t < 16; ++t)
+            rowv[t] = Jw[(size_t)idw[t0 + t < count ? t0 + t : count - 1] * nv + (lane < nv ? lane : nv - 1)];
+#pragma unroll
+          for (int t = 0; t < 16; ++t)
+            if (t0 + t < count) mw |= (unsigned)(rowv[t] != 0.0f) << (16 * half + t);
+        }
+        if (lane < nv) mk4[4 * lane + word] = mw;
+        any |= mw;
+      }
+      hit = lane < nv && any != 0u;
     } else if (lane < nv) {
       for (int t = 0; t < count && !hit; ++t) hit = Jw[(size_t)idw[t] * nv + lane] != 0.0f;
     }
     const unsigned long long umask = __ballot(hit);
     if (hit) uni[__popcll(umask & ((1ull << lane) - 1ull))] = lane;
     if (lane == 0) uni[nv] = __popcll(umask);
+    if (!staged) {
+      // the update in memory, a union row at a time, ahead of the column's load: lane c adds to the
+      // elements of column c that it reads back itself
+      wave_sync();
+      for (unsigned long long rest = umask; rest; rest &= rest - 1ull) {
+        const int r = __builtin_ctzll(rest);  // the same for every lane
+        if (!(hit && lane >= r)) continue;
+        float delta = 0.0f;
+        if (masked) {
+          const int *rid = (const int *)jr;
+          const float *sdv = jr + count;
+          const unsigned *mk4 = (const unsigned *)(jr + 2 * count);
+          for (int word = 0; 32 * word < count; ++word) {
+            for (unsigned mm = mk4[4 * r + word] & mk4[4 * lane + word]; mm; mm &= mm - 1u) {
+              const int t = 32 * word + __builtin_ctz(mm);
+              const int rr = rid[t];
+              delta = fma_(sdv[t] * Jw[(size_t)rr * nv + r], Jw[(size_t)rr * nv + lane], delta);
+            }
+          }
+        } else {
+          for (int t = 0; t < count; ++t) {
+            const int rr = idw[t];
+            const float av = Jw[(size_t)rr * nv + r], bv = Jw[(size_t)rr * nv + lane];
+            float da = Dw[rr] * av;
+            if (sw[rr] != quad) da = -da;
+            if (av != 0.0f && bv != 0.0f) delta = fma_(da, bv, delta);
+          }
+        }
+        if (delta != 0.0f) Hw[(size_t)r * PAD + lane] = Hw[(size_t)r * PAD + lane] + delta;
+      }
+    }
     // ---- H's column: the upper triangle up to nv, the identity beyond; lane RHS takes the gradient
 #pragma unroll
     for (int r = 0; r < PAD; ++r) {
@@ -138,25 +202,17 @@ __device__ __forceinline__ void dense_column_world(float *scr, float *Hw, float 
       u[r] = mine ? v : ((r == lane && !rhs_lane) ? 1.0f : 0.0f);
     }
     wave_sync();
-    // ---- update over the pairs (row <= column) of the union, a union row at a time: lane c owns pair (r, c)
+    // ---- update over the pairs (row <= column) of the union from the staged rows, a union row at a time: lane c owns pair (r, c)
 #pragma unroll
     for (int r = 0; r < PAD; ++r) {
-      if (!((umask >> r) & 1ull)) continue;  // the same for every lane
+      if (!staged || !((umask >> r) & 1ull)) continue;  // the same for every lane
       float delta = 0.0f;
-      if (staged) {
+      {
         const unsigned mk_r = (unsigned)__builtin_amdgcn_readlane((int)mk, r);
         const float *jrow = jr + r * (kColStagedRows + 1), *jcol = jr + (lane < PAD ? lane : 0) * (kColStagedRows + 1);
         for (unsigned mm = (hit && lane >= r) ? (mk_r & mk) : 0u; mm; mm &= mm - 1u) {
           const int t = __builtin_ctz(mm);
           delta = fma_(sd[t] * jrow[t], jcol[t], delta);
-        }
-      } else if (hit && lane >= r) {
-        for (int t = 0; t < count; ++t) {
-          const int rr = idw[t];
-          const float av = Jw[(size_t)rr * nv + r], bv = Jw[(size_t)rr * nv + lane];
-          float da = Dw[rr] * av;
-          if (sw[rr] != quad) da = -da;
-          if (av != 0.0f && bv != 0.0f) delta = fma_(da, bv, delta);
         }
       }
       if (delta != 0.0f) {
@@ -431,7 +487,8 @@ extern "C" int im_newton_solve_dense_column(const im_newton_args *p, float *H, f
   if (!probed) {  // once per process: a variant that spills registers is left out; the large dynamic LDS is asked for
     for (int i = 0; i < kVariants; ++i) {
       hipFuncAttributes fa{};
-      usable[i] = hipFuncGetAttributes(&fa, variants[i].fn) == hipSuccess && fa.localSizeBytes == 0 &&
+      // (a variant that parks more than a register or two of its prologue in memory is left out)
+      usable[i] = hipFuncGetAttributes(&fa, variants[i].fn) == hipSuccess && fa.localSizeBytes <= 16 &&
                   hipFuncSetAttribute(variants[i].fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                       160 * 1024 - (int)fa.sharedSizeBytes) == hipSuccess;
       regs[i] = fa.numRegs;
