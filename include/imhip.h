@@ -363,6 +363,30 @@ int im_dense_update_column(const uint8_t *done, const int32_t *state_changes, co
                            int nv_pad, int32_t *dof_union, float *search, int64_t ld_search, float *search_dot,
                            float *decrement, int nworld, void *stream);
 
+/* The first Hessian of a dense Newton solve and its factor in one launch, a wavefront per world:
+ * H = M + J' diag(D [state == quad]) J (upstream's solver._update_gradient as
+ * src/instantmimic/utils/mjw_kernels/newton_fusion.py:470 calls it for the dense Newton) for every
+ * world, written to H (nworld, nv_pad, nv_pad) in both triangles, then, for the worlds that are not
+ * done, what im_dense_update_factor does with changes[w] < 0: the factor of H as it lies there
+ * (into U above 32 dofs), the solve for the gradient, search, search_dot, decrement and an empty
+ * dof_union.  M (nworld rows of ldM floats) is the tree-sparse inertia, elemid (nv, nv) the element
+ * of a row of M at every pair of dofs, negative outside its pattern (the layout of the reference's
+ * m.M_elemid).  nefc may be null (every world has njmax rows).  Same results, bit for bit, as
+ * im_dense_from_csr, im_jtdj_mfma and im_dense_update_factor one after the other.  nv <= 32 (any
+ * nv_pad that is a multiple of four; U may be null) or nv_pad = 48 or 64; IM_ERR_UNSUPPORTED
+ * otherwise: the caller then issues the three launches.  H must be 16-byte aligned. */
+int im_dense_init_factor(const uint8_t *done, const int32_t *nefc, const float *J, int njmax, const float *D,
+                         const int32_t *state, int quad, const float *M, int64_t ldM, const int32_t *elemid,
+                         const float *grad, int64_t ldg, float *H, float *U, int nv, int nv_pad, int32_t *dof_union,
+                         float *search, int64_t ld_search, float *search_dot, float *decrement, int nworld,
+                         void *stream);
+
+/* The same for nv <= 32 alone; im_dense_init_factor hands such shapes here. */
+int im_dense_init_tile(const uint8_t *done, const int32_t *nefc, const float *J, int njmax, const float *D,
+                       const int32_t *state, int quad, const float *M, int64_t ldM, const int32_t *elemid,
+                       const float *grad, int64_t ldg, float *H, int nv, int nv_pad, int32_t *dof_union, float *search,
+                       int64_t ld_search, float *search_dot, float *decrement, int nworld, void *stream);
+
 /* Blocked dense factor + solve, dense J'DJ ----------------------------------- */
 
 /* Replaces _blocked_dense_factor_solve (src/instantmimic/utils/mjw_step_optimized.py:

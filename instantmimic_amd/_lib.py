@@ -206,6 +206,14 @@ SIGNATURES = {
         _i,
         [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],
     ),
+    "im_dense_init_factor": (
+        _i,
+        [_vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],
+    ),
+    "im_dense_init_tile": (
+        _i,
+        [_vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _i64, _vp, _vp, _i64, _vp, _i, _i, _vp, _vp, _i64, _vp, _vp, _i, _vp],
+    ),
     "im_newton_init_context": (_i, [C.POINTER(NewtonArgs), _vp, _i64, _vp, _i64, _i, _i, _vp]),
     "im_polynomial_damping": (_i, [_vp, _i64, _vp, _i64, _i, _vp, _i64, _vp, _i64, _i, _i, _vp]),
     "im_dense_update_tile": (

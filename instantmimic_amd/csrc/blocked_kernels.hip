@@ -18,6 +18,7 @@
 #include <cstring>
 
 #include "common.h"
+#include "jtdj_wave.h"
 #include "pivot.h"
 
 namespace im {
@@ -1327,7 +1328,6 @@ __global__ __launch_bounds__(256) void copy_dense_factor_kernel(const float *__r
 // copies used in turn; the next 32 rows are already on their way into registers while the matrix
 // cores work on the current ones, and the weighted operand (J Dc) is formed when it is fed.
 // An element's sum is the chain fma(J[r][i] * Dc[r], J[r][j], .) over the rows in order, from M.
-typedef float float4v __attribute__((ext_vector_type(4)));
 
 // The 36 tiles of a matrix of eight 16-column blocks, nine per wavefront, chosen so that a
 // wavefront's tiles share operands: wavefronts 0 and 1 take the triangles of blocks 0-3 and 4-7
@@ -1538,24 +1538,6 @@ __device__ __forceinline__ void jtdj_tiles_as(const float *__restrict__ Mdense, 
   for (int m = 0; m < MAXT; ++m) {
     if (m >= mine) continue;
     out(tbi[m] * 16 + 4 * kq, tbj[m] * 16 + (lane & 15), acc[m], tbi[m] != tbj[m]);
-  }
-}
-
-// Stores what one lane holds of a tile into H and its mirror image: rows i0 .. i0 + 3 of column j
-// (the elements with i <= j < nv count).  Right of the diagonal blocks (`off`) the mirror image of a
-// lane's four values is four consecutive words of row j: one 16-byte store where H allows it (`vec`).
-__device__ __forceinline__ void store_h_mirrored(float *__restrict__ Hw, int nv, int nv_pad, bool vec, int i0, int j,
-                                                 float4v h, bool off) {
-  if (j >= nv) return;
-#pragma unroll
-  for (int v = 0; v < 4; ++v)
-    if (i0 + v < nv && i0 + v <= j) Hw[(int64_t)(i0 + v) * nv_pad + j] = h[v];
-  if (off && vec && i0 + 3 < nv) {
-    *(float4v *)(Hw + (int64_t)j * nv_pad + i0) = h;
-  } else {
-#pragma unroll
-    for (int v = 0; v < 4; ++v)
-      if (i0 + v < nv && i0 + v < j) Hw[(int64_t)j * nv_pad + i0 + v] = h[v];
   }
 }
 

@@ -25,6 +25,7 @@
 #include <cstdint>
 
 #include "common.h"
+#include "jtdj_wave.h"
 #include "newton_wave.h"
 #include "pivot.h"
 
@@ -385,6 +386,35 @@ __global__ __launch_bounds__(256) void dense_update_column_kernel(
                            decrement + w, nv, lane);
 }
 
+// The first Hessian and its factor in one launch: H = M + J' D_act J of every world on the matrix
+// cores of its wavefront (jtdj_wave.h), stored, then the stage above on H as it lies there for the
+// worlds that are not done.
+template <int NBLK>
+__global__ __launch_bounds__(256, NBLK == 3 ? 3 : 2) void dense_init_column_kernel(
+    const uint8_t *__restrict__ done, const int32_t *__restrict__ nefc_p, const float *__restrict__ J, int njmax,
+    const float *__restrict__ D, const int32_t *__restrict__ state, int quad, const float *__restrict__ M, int64_t ldM,
+    const int32_t *__restrict__ elemid, const float *__restrict__ grad, int64_t ldg, float *H_, float *U_,
+    int32_t *__restrict__ uni_, float *__restrict__ search, int64_t ld_search, float *__restrict__ search_dot,
+    float *__restrict__ decrement, int nv, int nworld) {
+  extern __shared__ float lds[];
+  constexpr int PAD = 16 * NBLK;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t w = (int64_t)blockIdx.x * 4 + wv;
+  if (w >= nworld) return;
+  int nefc = nefc_p ? nefc_p[w] : njmax;
+  nefc = nefc < njmax ? nefc : njmax;
+  float *Hw = H_ + w * (int64_t)PAD * PAD;
+  const float *Jw = J + w * (int64_t)njmax * nv;
+  jtdj_wave<NBLK>(M + w * ldM, elemid, Jw, D + w * njmax, state + w * njmax, nefc, quad, nv, Hw, PAD, true, lane);
+  if (done && done[w]) return;
+  // the lanes read back one another's stores (one CU: its vector cache sees them once they are issued and waited for)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  dense_column_world<NBLK>(lds + wv * column_stage_words<NBLK>(), Hw, U_ + w * (int64_t)PAD * PAD, Jw, D + w * njmax,
+                           grad + w * ldg, state + w * njmax, nullptr, -1, 0, quad, uni_ + w * (nv + 1),
+                           search + w * ld_search, search_dot + w, decrement + w, nv, lane);
+}
+
 // The resident Newton loop (newton_wave.h) with this stage: a wavefront per world from the first
 // line search to convergence, WAVES worlds per workgroup.  Per wavefront in LDS: what the loop
 // keeps from round to round and one area that the staged tile of J, the gradient's row list and
@@ -545,6 +575,41 @@ extern "C" int im_dense_update_column(const uint8_t *done, const int32_t *state_
     hipLaunchKernelGGL(im::dense_update_column_kernel<4>, dim3(grid), dim3(256), 16 * im::column_stage_words<4>(),
                        (hipStream_t)stream, done, state_changes, changes, ids, ld_ids, J, njmax, D, state, quad, grad, ldg,
                        H, U, dof_union, search, ld_search, search_dot, decrement, nv, nworld);
+  }
+  IM_HIP_CHECK(hipGetLastError());
+  return IM_OK;
+}
+
+extern "C" int im_dense_init_tile(const uint8_t *done, const int32_t *nefc, const float *J, int njmax, const float *D,
+                                  const int32_t *state, int quad, const float *M, int64_t ldM, const int32_t *elemid,
+                                  const float *grad, int64_t ldg, float *H, int nv, int nv_pad, int32_t *dof_union,
+                                  float *search, int64_t ld_search, float *search_dot, float *decrement, int nworld,
+                                  void *stream);
+
+extern "C" int im_dense_init_factor(const uint8_t *done, const int32_t *nefc, const float *J, int njmax, const float *D,
+                                    const int32_t *state, int quad, const float *M, int64_t ldM, const int32_t *elemid,
+                                    const float *grad, int64_t ldg, float *H, float *U, int nv, int nv_pad,
+                                    int32_t *dof_union, float *search, int64_t ld_search, float *search_dot,
+                                    float *decrement, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || nv_pad < nv || njmax <= 0) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!J || !D || !state || !M || !elemid || !grad || !H || !dof_union || !search || !search_dot || !decrement)
+    return IM_ERR_ARG;
+  if (ldg < nv || ld_search < nv || ((uintptr_t)H & 15) != 0 || (nv_pad & 3) != 0) return IM_ERR_STRIDE;
+  if (nv <= 32)
+    return im_dense_init_tile(done, nefc, J, njmax, D, state, quad, M, ldM, elemid, grad, ldg, H, nv, nv_pad, dof_union,
+                              search, ld_search, search_dot, decrement, nworld, stream);
+  if (!U) return IM_ERR_ARG;
+  if (nv_pad <= nv || (nv_pad != 48 && nv_pad != 64)) return IM_ERR_UNSUPPORTED;
+  const unsigned grid = (unsigned)((nworld + 3) / 4);
+  if (nv_pad == 48) {
+    hipLaunchKernelGGL(im::dense_init_column_kernel<3>, dim3(grid), dim3(256), 16 * im::column_stage_words<3>(),
+                       (hipStream_t)stream, done, nefc, J, njmax, D, state, quad, M, ldM, elemid, grad, ldg, H, U, dof_union,
+                       search, ld_search, search_dot, decrement, nv, nworld);
+  } else {
+    hipLaunchKernelGGL(im::dense_init_column_kernel<4>, dim3(grid), dim3(256), 16 * im::column_stage_words<4>(),
+                       (hipStream_t)stream, done, nefc, J, njmax, D, state, quad, M, ldM, elemid, grad, ldg, H, U, dof_union,
+                       search, ld_search, search_dot, decrement, nv, nworld);
   }
   IM_HIP_CHECK(hipGetLastError());
   return IM_OK;

@@ -19,6 +19,7 @@
 #include <algorithm>
 
 #include "common.h"
+#include "jtdj_wave.h"
 #include "newton_wave.h"
 #include "pivot.h"
 
@@ -348,6 +349,37 @@ __global__ __launch_bounds__(256) void dense_update_tile_kernel(
                        search_dot + w, decrement + w, nv, pad, i);
 }
 
+// The first Hessian and its factor in one launch, a wavefront per world: H = M + J' D_act J on the
+// wavefront's matrix cores (jtdj_wave.h), stored, then the stage above without changed rows for the
+// worlds that are not done (both halves of the wavefront run it on the same world).
+template <int NP>
+__global__ __launch_bounds__(256) void dense_init_tile_kernel(
+    const uint8_t *__restrict__ done, const int32_t *__restrict__ nefc_p, const float *__restrict__ J, int njmax,
+    const float *__restrict__ D, const int32_t *__restrict__ state, int quad, const float *__restrict__ M, int64_t ldM,
+    const int32_t *__restrict__ elemid, const float *__restrict__ grad, int64_t ldg, float *H_,
+    int32_t *__restrict__ uni_, float *__restrict__ search, int64_t ld_search, float *__restrict__ search_dot,
+    float *__restrict__ decrement, int nv, int pad, int nworld) {
+  extern __shared__ float lds[];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t w = (int64_t)blockIdx.x * 4 + wv;
+  if (w >= nworld) return;
+  int nefc = nefc_p ? nefc_p[w] : njmax;
+  nefc = nefc < njmax ? nefc : njmax;
+  float *Hw = H_ + w * (int64_t)pad * pad;
+  const float *Jw = J + w * (int64_t)njmax * nv;
+  jtdj_wave<(NP + 15) / 16>(M + w * ldM, elemid, Jw, D + w * njmax, state + w * njmax, nefc, quad, nv, Hw, pad,
+                            (pad & 3) == 0, lane);
+  if (done && done[w]) return;
+  // the lanes read back one another's stores (one CU: its vector cache sees them once they are issued and waited for)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  float *mine = lds + wv * dense_tile_stage_words<NP>();
+  const TileArea<NP> T(mine);
+  dense_tile_world<NP>(T, (int *)(mine + TileArea<NP>::kWords), Hw, Jw, D + w * njmax, grad + w * ldg, state + w * njmax,
+                       nullptr, 0, quad, uni_ + w * (nv + 1), search + w * ld_search, search_dot + w, decrement + w, nv, pad,
+                       lane & 31);
+}
+
 // The resident Newton loop (newton_wave.h) with this stage: a wavefront per world from the first
 // line search to convergence, WAVES worlds per workgroup.  Both halves of the wavefront run the
 // stage on the wavefront's world.  Per wavefront in LDS: what the loop keeps from round to round
@@ -496,6 +528,32 @@ int im_dense_update_tile(const uint8_t *done, const int32_t *state_changes, cons
   }
   IM_STAGE_CASE(8) IM_STAGE_CASE(16) IM_STAGE_CASE(24) IM_STAGE_CASE(32)
 #undef IM_STAGE_CASE
+  return IM_ERR_UNSUPPORTED;
+}
+
+// the first Hessian and factor of a dense solve up to 32 dofs; im_dense_init_factor hands such shapes here
+int im_dense_init_tile(const uint8_t *done, const int32_t *nefc, const float *J, int njmax, const float *D,
+                       const int32_t *state, int quad, const float *M, int64_t ldM, const int32_t *elemid, const float *grad,
+                       int64_t ldg, float *H, int nv, int nv_pad, int32_t *dof_union, float *search, int64_t ld_search,
+                       float *search_dot, float *decrement, int nworld, void *stream) {
+  if (nworld < 0 || nv <= 0 || nv > 32 || nv_pad < nv || njmax <= 0) return IM_ERR_ARG;
+  if (nworld == 0) return IM_OK;
+  if (!J || !D || !state || !M || !elemid || !grad || !H || !dof_union || !search || !search_dot || !decrement)
+    return IM_ERR_ARG;
+  if (ldg < nv || ld_search < nv || ((uintptr_t)H & 15) != 0) return IM_ERR_STRIDE;
+  hipStream_t st = (hipStream_t)stream;
+  const unsigned grid = (unsigned)((nworld + 3) / 4);
+#define IM_INIT_CASE(NP)                                                                                              \
+  if (nv <= NP) {                                                                                                     \
+    const size_t lds = sizeof(float) * 4 * im::dense_tile_stage_words<NP>();                                          \
+    hipLaunchKernelGGL(im::dense_init_tile_kernel<NP>, dim3(grid), dim3(256), lds, st, done, nefc, J, njmax, D, state, \
+                       quad, M, ldM, elemid, grad, ldg, H, dof_union, search, ld_search, search_dot, decrement, nv,   \
+                       nv_pad, nworld);                                                                               \
+    IM_HIP_CHECK(hipGetLastError());                                                                                  \
+    return IM_OK;                                                                                                     \
+  }
+  IM_INIT_CASE(8) IM_INIT_CASE(16) IM_INIT_CASE(24) IM_INIT_CASE(32)
+#undef IM_INIT_CASE
   return IM_ERR_UNSUPPORTED;
 }
 

@@ -334,6 +334,55 @@ def dense_hessian(M_dense, J, D, state, nefc, H, *, quad: int = QUADRATIC) -> No
     _lib.check(status, "im_jtdj_mfma")
 
 
+def dense_init_factor(M, elemid, J, D, state, nefc, done, grad, H, U, search, search_dot, decrement, dof_union,
+                      *, quad: int = QUADRATIC) -> bool:  # fmt: skip
+    """The first Hessian of a dense Newton solve and its factor in one launch
+    (``im_dense_init_factor``): ``H = M + J' D_act J`` from the tree-sparse ``M`` (nworld, nM) and
+    ``elemid`` (nv, nv), then for the worlds that are not ``done`` the dense stage without changed
+    rows (factor into ``U`` above 32 dofs, solve for ``grad``, ``search``, ``search_dot``,
+    ``decrement``, an empty ``dof_union``).  Returns False, with nothing launched, for a shape
+    the launch does not take (64 dofs and more) or arrays it cannot address; the caller then issues
+    ``dense_from_csr``, :func:`dense_hessian` and the stage."""
+    import torch
+
+    nworld, njmax, nv = J.shape
+    pad = int(H.shape[1])
+    if nv > 32 and pad not in (48, 64):
+        return False
+    tensors = dict(M=M, J=J, D=D, state=state, grad=grad, H=H, U=U, search=search, search_dot=search_dot, decrement=decrement)
+    for name, t in tensors.items():
+        if not t.is_cuda or t.device != J.device or t.dtype != (torch.int32 if name == "state" else torch.float32):
+            return False
+    for t in (J, D, state, H, U, search_dot, decrement, elemid, dof_union):
+        if not t.is_contiguous():
+            return False
+    if M.dim() != 2 or M.shape[0] != nworld or (M.shape[1] > 1 and M.stride(1) != 1) or grad.stride(-1) != 1 or search.stride(-1) != 1:
+        return False
+    if tuple(H.shape) != (nworld, pad, pad) or tuple(U.shape) != (nworld, pad, pad) or pad % 4 or H.data_ptr() % 16:
+        return False
+    if elemid.dtype != torch.int32 or tuple(elemid.shape) != (nv, nv) or dof_union.dtype != torch.int32 or tuple(dof_union.shape) != (nworld, nv + 1):
+        return False
+    if njmax < 1 or tuple(D.shape) != (nworld, njmax) or tuple(state.shape) != (nworld, njmax):
+        return False
+    if nefc is not None and (nefc.dtype != torch.int32 or nefc.numel() != nworld or not nefc.is_contiguous()):
+        return False
+    if done is not None and (done.dtype not in (torch.bool, torch.uint8) or done.numel() != nworld or not done.is_contiguous()):
+        return False
+    if grad.shape[0] != nworld or search.shape[0] != nworld or grad[0].numel() < nv or search[0].numel() < nv:
+        return False
+    with torch.cuda.device(J.device):
+        status = _lib.lib().im_dense_init_factor(
+            None if done is None else done.data_ptr(), None if nefc is None else nefc.data_ptr(), J.data_ptr(), int(njmax),
+            D.data_ptr(), state.data_ptr(), int(quad), M.data_ptr(), int(M.stride(0)), elemid.data_ptr(), grad.data_ptr(),
+            int(grad.stride(0)), H.data_ptr(), U.data_ptr(), int(nv), pad, dof_union.data_ptr(), search.data_ptr(),
+            int(search.stride(0)), search_dot.data_ptr(), decrement.data_ptr(), int(nworld), _stream(J),
+        )  # fmt: skip
+    if status == _lib.IM_ERR_UNSUPPORTED:
+        return False
+    _lib.check(status, "im_dense_init_factor")
+    return True
+
+
 def dense_hessian_factor_solve(M_dense, J, D, state, nefc, H, y, x, *, factor=None, quad: int = QUADRATIC) -> None:
     """:func:`dense_hessian` and the blocked Cholesky (16 x 16 tiles) with its solve in one launch:
     ``H`` (nworld, nv_pad, nv_pad) or None, ``x = H^-1 y`` (nworld, nv), ``factor`` (nworld, pad,

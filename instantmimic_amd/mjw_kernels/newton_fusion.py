@@ -613,6 +613,11 @@ def _update_gradient(m, d, ctx, *, gradient_done: bool = False) -> None:
         raise RuntimeError("the dense first factor needs attach_scratch(m, d, ctx)")
     if not gradient_done:
         _first_gradient(m, d, ctx)
+    # one launch where the shape has one (up to 63 dofs); IMHIP_NEWTON=stages keeps the three
+    if os.environ.get("IMHIP_NEWTON") != "stages" and blocked_dense.dense_init_factor(
+            d.M, ctx.newton_elemid, d.efc.J, d.efc.D, d.efc.state, d.nefc, ctx.done, ctx.grad, ctx.h, ctx.hfactor, ctx.search,
+            ctx.search_dot, ctx.newton_decrement, ctx.newton_dof_union):  # fmt: skip
+        return
     dense_from_csr(d.M, ctx.newton_elemid, ctx.newton_mdense)
     blocked_dense.dense_hessian(ctx.newton_mdense, d.efc.J, d.efc.D, d.efc.state, d.nefc, ctx.h)
     stage = _stage(m, ctx)

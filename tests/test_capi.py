@@ -213,6 +213,25 @@ def test_init_context_entry_point_checks_its_arguments_before_any_launch():
     assert lib.im_newton_solve_sparse(None, C.byref(_newton_args()), one, one, None) == _lib.IM_ERR_ARG
 
 
+def test_dense_init_entry_point_checks_its_arguments_before_any_launch():
+    lib = _lib.lib()
+    one = 16
+    call = lambda **k: lib.im_dense_init_factor(  # noqa: E731
+        None, None, k.get("J", one), k.get("njmax", 96), one, one, 1, k.get("M", one), 341, k.get("elemid", one), one,
+        k.get("ldg", 48), k.get("H", one), k.get("U", one), k.get("nv", 35), k.get("pad", 48), one, one, k.get("lds", 35), one,
+        one, k.get("nworld", 4), None)  # fmt: skip
+    assert call(nworld=0) == _lib.IM_OK and call(nworld=-1) == _lib.IM_ERR_ARG and call(njmax=0) == _lib.IM_ERR_ARG
+    assert call(J=None) == _lib.IM_ERR_ARG and call(M=None) == _lib.IM_ERR_ARG and call(elemid=None) == _lib.IM_ERR_ARG
+    assert call(U=None) == _lib.IM_ERR_ARG and call(H=None) == _lib.IM_ERR_ARG and call(pad=32) == _lib.IM_ERR_ARG
+    assert call(ldg=34) == _lib.IM_ERR_STRIDE and call(lds=34) == _lib.IM_ERR_STRIDE and call(H=20) == _lib.IM_ERR_STRIDE
+    # 64 dofs and more (a padded size of 80 and up) have no launch of this kind
+    assert call(nv=64, pad=80, ldg=80, lds=64) == _lib.IM_ERR_UNSUPPORTED and call(nv=35, pad=52) == _lib.IM_ERR_UNSUPPORTED
+    # the single tile: at most 32 dofs
+    tile = lambda nv, pad: lib.im_dense_init_tile(None, None, one, 64, one, one, 1, one, 243, one, one, 32, one, nv, pad, one,  # noqa: E731
+                                                  one, 32, one, one, 4, None)  # fmt: skip
+    assert tile(33, 48) == _lib.IM_ERR_ARG and tile(27, 16) == _lib.IM_ERR_ARG
+
+
 def test_implicit_matrix_entry_points_check_their_arguments_before_any_launch():
     lib = _lib.lib()
     one = 16

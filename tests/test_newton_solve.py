@@ -163,11 +163,14 @@ def test_gpu_solve_from_init_context_matches_the_oracle_chain(device, monkeypatc
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,nworld,stage", [("humanoid", 301, "tree"), ("g1", 203, "sparse"), ("snu", 131, "tree"), ("ant", 67, "dense")])
+@pytest.mark.parametrize("name,nworld,stage", [("humanoid", 301, "tree"), ("g1", 203, "sparse"), ("snu", 131, "tree"), ("ant", 67, "dense"),
+                                               ("humanoid", 299, "dense"), ("g1", 201, "dense"), ("snu", 129, "dense")])  # fmt: skip
 def test_gpu_init_context_in_one_launch_leaves_what_the_five_launches_leave(device, monkeypatch, name, nworld, stage):
     """Everything before the first Hessian as one launch (a wavefront per world) against the same
     steps as launches of their own: every array of ``d``, ``d.efc`` and ``ctx`` bit for bit, poison
-    included where neither writes."""
+    included where neither writes.  On the dense stage the first Hessian and its factor are one
+    launch as well (``im_dense_init_factor``: a single tile up to 32 dofs, 48 or 64 columns beyond)
+    against dense M, ``J' D J`` and the stage as three; the dense copy of M is scratch of the three."""
     import torch
 
     p = NC.problem(name, nworld, stage, empty_every=7, warmstart=True, maxiter=12)
@@ -189,8 +192,12 @@ def test_gpu_init_context_in_one_launch_leaves_what_the_five_launches_leave(devi
     assert taken == [False, True]
     assert got[0].keys() == got[1].keys() and "ctx.grad" in got[0] and "efc.Ma" in got[0]
     for key in got[0]:
+        if key == "ctx.newton_mdense":
+            continue
         a, b = got[0][key], got[1][key]
         assert a.tobytes() == b.tobytes(), key
+    if stage == "dense":
+        assert "ctx.h" in got[0] and "ctx.hfactor" in got[0] and np.nanmax(np.abs(got[1]["ctx.h"])) > 0
 
 
 def _floating_chain(nv: int, limbs: int = 1):

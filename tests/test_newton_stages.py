@@ -257,6 +257,104 @@ def test_gpu_dense_stage_bitwise(device, name, nworld):
     np.testing.assert_array_equal(decr.cpu().numpy()[live], want2[5][live])
 
 
+def _toggled(b, rng, counts):
+    """World w has counts[w % len(counts)] rows whose quadratic-ness flips (rows below nefc, ascending);
+    every world is live."""
+    nworld, njmax = b.D.shape
+    new = b.state[0].copy()
+    ids = np.zeros((nworld, njmax), np.int32)
+    changes = np.zeros(nworld, np.int32)
+    for w in range(nworld):
+        k = min(int(counts[w % len(counts)]), int(b.nefc[w]))
+        rows = np.sort(rng.choice(int(b.nefc[w]), size=k, replace=False))
+        new[w, rows] = np.where(b.state[0][w, rows] == Q, 0, Q)
+        ids[w, :k] = rows
+        changes[w] = k
+    grad = rng.standard_normal(b.grad.shape).astype(np.float32)
+    return new, ids, changes, np.ones(nworld, np.int32), np.zeros(nworld, np.uint8), grad
+
+
+# changed rows per world: inside the staged capacities (16 and 32 rows), inside what the masks hold
+# (128), and beyond, where the pairs read J row by row
+_MANY = (0, 3, 16, 17, 32, 33, 64, 127, 128, 129, 150, 160)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["humanoid", "g1", "snu"])
+def test_gpu_dense_stage_with_up_to_160_changed_rows(device, name):
+    """The single tile (humanoid) and the 48- and 64-column stages with 160 rows per world, of which
+    0 to 160 change: every form of the update (staged rows, masks, row by row) against the CPU
+    restatement, bit for bit."""
+    import dataclasses
+
+    import torch
+
+    shape = dataclasses.replace(synth.SHAPES[name], nefc=160, iterations=1)
+    nworld = 2 * len(_MANY) + 1
+    b = synth.make_batch(shape, nworld, ragged_nefc=False)
+    nv = shape.nv
+    pad = ((nv + 1 + 15) // 16) * 16
+    rng = np.random.default_rng(31)
+    _, H0 = _dense_start(b, pad)
+    new, ids, changes, sc, done, grad = _toggled(b, rng, _MANY)
+    assert changes.max() == 160 and set(_MANY) <= set(changes.tolist())
+    U0 = np.broadcast_to(np.eye(pad, dtype=np.float32), H0.shape).copy()
+    want = R.dense_update_factor(sc, changes, ids, b.J, b.D, new, grad, H0, U0, done=done)
+    H, U = _t(H0, device), _t(U0, device)
+    uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=device)
+    search = torch.zeros((nworld, pad, 1), device=device)
+    sdot, decr = torch.zeros(nworld, device=device), torch.zeros(nworld, device=device)
+    g3 = torch.zeros((nworld, pad, 1), device=device)
+    g3[:, :nv, 0] = _t(grad, device)
+    NS.factor_factory(nv, pad)(_t(b.J, device), _t(b.D, device), _t(new, device), _t(ids, device), _t(changes, device),
+                               _t(sc, device), _t(done, device), g3, H, U, search, sdot, decr, uni)  # fmt: skip
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(H.cpu().numpy(), want[0])
+    np.testing.assert_array_equal(U.cpu().numpy(), want[1])
+    refactored = changes > 0
+    np.testing.assert_array_equal(uni.cpu().numpy()[refactored], want[2][refactored])
+    np.testing.assert_array_equal(search.cpu().numpy()[:, :nv, 0], want[3])
+    np.testing.assert_array_equal(sdot.cpu().numpy(), want[4])
+    np.testing.assert_array_equal(decr.cpu().numpy(), want[5])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["g1", "snu"])
+def test_gpu_sparse_stage_with_up_to_160_changed_rows(device, name):
+    """The same for the sparse stage on the benchmark trees' plans."""
+    import dataclasses
+
+    import torch
+
+    shape = dataclasses.replace(synth.SHAPES[name], nefc=160, iterations=1)
+    m = synth.model_from_parents(shape.parents)
+    block = S.block_width(m.nv_pad)
+    plan, reason = S.plan_for_model(m, None, [], block, device=device)
+    assert plan is not None, reason
+    oplan = R.sparse_plan(m, [], block)
+    nworld = 2 * len(_MANY) + 1
+    b = synth.make_batch(shape, nworld, ragged_nefc=False)
+    rng = np.random.default_rng(37)
+    hf0, *_ = R.sparse_init_factor(oplan, b.nefc, b.J, b.D, b.state[0], b.M, b.grad)
+    new, ids, changes, sc, done, grad = _toggled(b, rng, _MANY)
+    want = R.sparse_update_factor(oplan, sc, changes, ids, b.J, b.D, new, grad, hf0, done=done)
+    nv = m.nv
+    hf = _t(hf0, device)
+    uni = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=device)
+    search = torch.zeros((nworld, nv), device=device)
+    sdot, decr = torch.zeros(nworld, device=device), torch.zeros(nworld, device=device)
+    NS.factor_factory(nv, m.nv_pad, plan)(_t(b.J, device), _t(b.D, device), _t(new, device), _t(ids, device), _t(changes, device),
+                                          _t(sc, device), _t(done, device), _t(grad, device), None, hf, search, sdot, decr, uni)  # fmt: skip
+    torch.cuda.synchronize()
+    n_used = 2 * plan.nfac + nv
+    np.testing.assert_array_equal(hf.cpu().numpy().reshape(nworld, -1)[:, :n_used], want[0].reshape(nworld, -1)[:, :n_used])
+    refactored = changes > 0
+    np.testing.assert_array_equal(uni.cpu().numpy()[refactored], want[1][refactored])
+    np.testing.assert_array_equal(search.cpu().numpy(), want[2])
+    np.testing.assert_array_equal(sdot.cpu().numpy(), want[3])
+    np.testing.assert_array_equal(decr.cpu().numpy(), want[4])
+
+
 @pytest.mark.gpu
 def test_gpu_block_per_world_sparse_kernels_agree():
     """The sparse factor has two kernels per entry point (a wavefront per world with the tables in
