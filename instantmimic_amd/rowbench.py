@@ -194,6 +194,20 @@ def run(launches: int = 32, only: str | None = None) -> None:
                 dt = SimpleNamespace(nworld=nworld, qLD=torch.zeros((nworld, 0), device=dev))
                 sec = _timeit(torch, lambda i: BD._factor_solve_i_dense(mt, dt, S[i][0], X[i], S[i][5]), nsets, launches)
                 _line("im_tile_cholesky_solve_m", wl, sec, bytes_=nworld * 4 * (nM + 2 * nv), nworld=nworld)
+            if name != "ant":
+                # the dense Newton's first Hessian and factor as one launch (M through the element table, J'DJ, the stage)
+                pad = (nv // 16 + 1) * 16
+                eid = t(NF.elemid_table(b.rowadr, b.rownnz, b.colind))
+                Hd, Ud = torch.zeros((nworld, pad, pad), device=dev), torch.zeros((nworld, pad, pad), device=dev)
+                un = torch.zeros((nworld, nv + 1), dtype=torch.int32, device=dev)
+                se = torch.zeros((nworld, nv), device=dev)
+                sd_, de_ = torch.zeros(nworld, device=dev), torch.zeros(nworld, device=dev)
+                ok = BD.dense_init_factor(S[0][0], eid, S[0][1], S[0][2], S[0][3], S[0][4], None, S[0][5], Hd, Ud, se, sd_, de_, un)
+                assert ok, "no one-launch dense first factor for this shape"
+                sec = _timeit(torch, lambda i: BD.dense_init_factor(S[i][0], eid, S[i][1], S[i][2], S[i][3], S[i][4], None, S[i][5], Hd, Ud, se, sd_, de_, un), nsets, launches)
+                _line("im_dense_init_factor (M + J'DJ, factor, solve)", wl, sec,
+                      bytes_=nworld * 4 * (nM + nefc * nv + 2 * nefc + 2 * nv + pad * pad + (pad * pad if nv > 32 else 0) + 2), nworld=nworld)  # fmt: skip
+                del Hd, Ud
             if name in ("g1", "snu"):
                 # the same Hessians through the blocked dense factor and the static-pattern sparse L'DL
                 Md = synth.dense_from_csr(b.M, b.rowadr, b.rownnz, b.colind).astype(np.float32).reshape(nworld, -1)
