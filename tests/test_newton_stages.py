@@ -280,9 +280,9 @@ _MANY = (0, 3, 16, 17, 32, 33, 64, 127, 128, 129, 150, 160)
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name", ["humanoid", "g1", "snu"])
+@pytest.mark.parametrize("name", ["ant", "humanoid", "g1", "snu"])
 def test_gpu_dense_stage_with_up_to_160_changed_rows(device, name):
-    """The single tile (humanoid) and the 48- and 64-column stages with 160 rows per world, of which
+    """The single tile (ant: 16 columns, humanoid: 32) and the 48- and 64-column stages with 160 rows per world, of which
     0 to 160 change: every form of the update (staged rows, masks, row by row) against the CPU
     restatement, bit for bit."""
     import dataclasses
