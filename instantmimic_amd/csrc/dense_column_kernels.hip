@@ -17,6 +17,8 @@
 // triangular solves of the tiles to its right in one.  The backward solve needs rows of U across
 // lanes: a 16 x 16 tile at a time is turned round through LDS.  The gradient column rides in lane
 // 63 (a padding column that no other lane reads).
+// The first factor of a solve has a launch of its own in which the wavefront assembles H first
+// (dense_init_column_kernel; newton_fusion.py:470 of the reference calls upstream's assembly there).
 // Same operations in the same order as the workgroup-per-world kernel of blocked_kernels.hip and
 // the CPU restatement both are tested against.
 #include <hip/hip_runtime.h>
@@ -34,7 +36,7 @@ namespace {
 
 using resident::wave_sync;
 
-constexpr int kColStagedRows = 32;  // the changed rows a stage keeps in LDS (a 32-bit mask per dof); more are read from memory
+constexpr int kColStagedRows = 32;  // the changed rows a stage keeps in LDS (a 32-bit mask per dof); beyond, up to 128 rows, their masks only
 // LDS words of one world's stage: a 16 x 16 tile turned round (rows 17 words apart), the staged
 // changed rows dof-major (33 words a dof), their weights, the dofs' masks
 template <int NBLK>

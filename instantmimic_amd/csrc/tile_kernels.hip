@@ -1,7 +1,8 @@
 // Cholesky of a matrix that fits one tile (up to 64 x 64) with the solve of one right-hand side,
 // nothing kept: the reference's two "no L store" tile kernels
 // (src/instantmimic/utils/mjw_step_optimized.py:672-750) and the nv <= 32 branch of the Newton
-// factor stage (src/instantmimic/utils/mjw_kernels/newton_stages.py:723-733).
+// factor stage (src/instantmimic/utils/mjw_kernels/newton_stages.py:723-733), with a launch for the first
+// factor of a solve in which the world's wavefront assembles H ahead of it (dense_init_tile_kernel).
 //
 // A group of 32 or 64 lanes owns a tile; lane i holds row i of the lower triangle in registers and
 // its right-hand side entry.  Column j, once final, goes through LDS to every lane of the group
