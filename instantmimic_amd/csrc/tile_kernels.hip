@@ -92,6 +92,59 @@ __device__ __forceinline__ float tile_factor_solve(float (&a)[NP], float s, int 
   return s;
 }
 
+// The same factor and solve by a whole wavefront on one tile of up to 32 rows: lane i of either half
+// holds row i, the lower half its even columns and the upper half the odd ones (a2[k] = element
+// (i, 2 k + half)), so a column's update of the columns to its right is shared between the two.
+// Every element sees the same operations in the same order as above; s and the backward
+// substitution run in both halves alike.
+template <int NP>
+__device__ __forceinline__ float tile_factor_solve_halves(float (&a2)[NP / 2], float s, int i, int half, int n,
+                                                          const TileArea<NP> &T) {
+  static_assert(NP % 2 == 0 && NP <= 32, "two columns a step, a row a lane of a half");
+  const int ic = i < NP ? i : 0;
+  const float *colh = T.col + half;
+#pragma unroll
+  for (int j = 0; j < NP; ++j) {
+    if (j < n) {  // the same for every lane of the launch
+      const int kj = j >> 1, hj = j & 1;
+      if (half == hj && i < NP) {
+        T.col[i] = a2[kj];
+        T.rhs[i] = s;
+      }
+      wave_sync();
+      const float aj = i < NP ? T.col[ic] : 0.0f, pv = T.col[j];  // (a half has more lanes than a small tile has rows)
+      float cv[NP / 2];
+#pragma unroll
+      for (int k = (j + 1) >> 1; k < NP / 2; ++k) cv[k] = colh[2 * k];  // column 2 k + half
+      float d, rinv;
+      pivot_sqrt_rcp(pv, true, d, rinv);
+      const float lj = aj * rinv;  // rows below the diagonal; what the others compute is not read
+      const float z = T.rhs[j] * rinv;
+#pragma unroll
+      for (int k = (j + 1) >> 1; k < NP / 2; ++k) {
+        const float v = fma_(-lj, cv[k] * rinv, a2[k]);
+        a2[k] = (2 * k > j || half == 1) ? v : a2[k];  // column 2 k + half lies right of column j
+      }
+      s = i > j ? fma_(-lj, z, s) : (i == j ? z : s);
+      a2[kj] = half == hj ? (i == j ? d : lj) : a2[kj];
+      if (i == j && half == hj) T.rinv[j] = rinv;
+      wave_sync();  // the column's words are read before the next column is written over them
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NP / 2; ++k)
+    if (2 * k + half <= i && i < NP) T.tile[i * TileArea<NP>::kRow + 2 * k + half] = a2[k];
+  wave_sync();
+  float l_next = n > 0 ? T.tile[(n - 1) * TileArea<NP>::kRow + ic] : 0.0f;
+  for (int r = n - 1; r >= 0; --r) {
+    const float l_r = l_next;
+    if (r > 0) l_next = T.tile[(r - 1) * TileArea<NP>::kRow + ic];
+    const float xr = group_bcast<32>(s, r) * T.rinv[r];
+    s = i < r ? fma_(-l_r, xr, s) : (i == r ? xr : s);
+  }
+  return s;
+}
+
 // One tile per group of LG lanes, 256 / LG tiles per workgroup.  elemid == nullptr: M is dense
 // with ld_world floats per world and ld_row per row, tile t the diagonal block at adr[t] (lower
 // triangle read); else M holds nM values per world and tile t's element (r, c) is
@@ -152,7 +205,7 @@ __global__ __launch_bounds__(256) void tile_cholesky_solve_kernel(
 // The Newton factor stage up to 32 dofs: dofs touched by the changed rows, incremental update of
 // H's upper triangle (in memory and in the staged copy), then H factored as one tile and solved
 // for the gradient, at every call; U is not used.  search = -x, search_dot = x.x,
-// decrement = grad.x.  Two worlds per wavefront, 32 lanes each.
+// decrement = grad.x.  A wavefront per world: the rows on 32 lanes, the two halves sharing the work.
 constexpr int kTileStagedRows = 16;
 // LDS words of one group's stage: the tile's area, the dof union (36), the staged rows, their weights and the dofs' masks
 template <int NP>
@@ -160,9 +213,10 @@ __host__ __device__ constexpr int dense_tile_stage_words() {
   return TileArea<NP>::kWords + 36 + (kTileStagedRows + 1) * NP + kTileStagedRows + NP;
 }
 
-// One world's stage on a group of 32 lanes (lane i of the group); both groups of a wavefront may
-// work on the same world, they then write the same values to the same places.
-template <int NP>
+// One world's stage on a group of 32 lanes (lane i of the group).  WHOLE: both groups of the
+// wavefront work on this world: they share H's load, the pairs of the update and the columns of
+// the factor between them and write the same values to the same places otherwise.
+template <int NP, bool WHOLE = false>
 __device__ __forceinline__ void dense_tile_world(const TileArea<NP> &T, int *ul, float *Hw, const float *Jw, const float *Dw,
                                                  const float *gw, const int32_t *sw, const int32_t *idw, int count, int quad,
                                                  int32_t *uni, float *search_w, float *search_dot_w, float *decrement_w,
@@ -170,19 +224,22 @@ __device__ __forceinline__ void dense_tile_world(const TileArea<NP> &T, int *ul,
   constexpr int LG = 32, kRow = TileArea<NP>::kRow;
   // H's rows into LDS (both triangles as they lie there; only the upper one is read)
   const float inv_nv = 1.0f / (float)nv;
-  for (int e0 = i; e0 < nv * nv; e0 += 4 * LG) {  // four loads in flight per lane
+  constexpr int LW = WHOLE ? 64 : LG;                       // lanes that share a loop over the world's elements
+  const int iw = WHOLE ? (int)(threadIdx.x & 63) : i;       // this lane among them
+  const int half = WHOLE ? (int)((threadIdx.x >> 5) & 1) : 0;
+  for (int e0 = iw; e0 < nv * nv; e0 += 4 * LW) {  // four loads in flight per lane
     float v[4];
     int at[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      const int e = e0 + k * LG < nv * nv ? e0 + k * LG : nv * nv - 1;
+      const int e = e0 + k * LW < nv * nv ? e0 + k * LW : nv * nv - 1;
       const int r = (int)(((float)e + 0.5f) * inv_nv), c = e - r * nv;  // e / nv, exact for these sizes
       v[k] = Hw[(size_t)r * pad + c];
       at[k] = r * kRow + c;
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k)
-      if (e0 + k * LG < nv * nv) T.tile[at[k]] = v[k];
+      if (e0 + k * LW < nv * nv) T.tile[at[k]] = v[k];
   }
   // The changed rows of J come into LDS dof-major (a dof's elements of up to kTileStagedRows rows
   // side by side, 17 words a dof) with a mask per dof of the rows that are nonzero there; more
@@ -264,7 +321,7 @@ __device__ __forceinline__ void dense_tile_world(const TileArea<NP> &T, int *ul,
   }
   if (i == 0) uni[nv] = nu;
   wave_sync();
-  for (int e = i; e < nu * (nu + 1) / 2; e += LG) {
+  for (int e = iw; e < nu * (nu + 1) / 2; e += LW) {
     int cj = (int)((sqrtf((float)(8 * e + 1)) - 1.0f) * 0.5f);
     while ((cj + 1) * (cj + 2) / 2 <= e) ++cj;
     while (cj * (cj + 1) / 2 > e) --cj;
@@ -308,11 +365,19 @@ __device__ __forceinline__ void dense_tile_world(const TileArea<NP> &T, int *ul,
   float s = i < nv ? gw[i] : 0.0f;
   const float g = s;
   wave_sync();
-  float a[NP];
+  if constexpr (WHOLE) {
+    float a2[NP / 2];
 #pragma unroll
-  for (int c = 0; c < NP; ++c) a[c] = (i < nv && c <= i) ? T.tile[c * kRow + i] : 0.0f;  // upper triangle: element (c, i)
-  wave_sync();
-  s = tile_factor_solve<NP, LG>(a, s, i, nv, T);
+    for (int k = 0; k < NP / 2; ++k) a2[k] = (i < nv && 2 * k + half <= i) ? T.tile[(2 * k + half) * kRow + i] : 0.0f;
+    wave_sync();
+    s = tile_factor_solve_halves<NP>(a2, s, i, half, nv, T);
+  } else {
+    float a[NP];
+#pragma unroll
+    for (int c = 0; c < NP; ++c) a[c] = (i < nv && c <= i) ? T.tile[c * kRow + i] : 0.0f;  // upper triangle: element (c, i)
+    wave_sync();
+    s = tile_factor_solve<NP, LG>(a, s, i, nv, T);
+  }
   if (i < nv) search_w[i] = -s;
   // as 64 lanes striding the dofs would sum them: one term per lane, the upper 32 lanes' zeros change nothing
   float s0 = fma_(s, s, 0.0f), s1 = fma_(g, s, 0.0f);
@@ -336,16 +401,16 @@ __global__ __launch_bounds__(256) void dense_update_tile_kernel(
     float *__restrict__ search, int64_t ld_search, float *__restrict__ search_dot,
     float *__restrict__ decrement, int nv, int pad, int nworld) {
   extern __shared__ float lds[];
-  constexpr int LG = 32;
-  const int group = threadIdx.x / LG, i = threadIdx.x % LG;
-  const int64_t w = (int64_t)blockIdx.x * (256 / LG) + group;
+  // a wavefront per world, its two halves sharing the work
+  const int group = threadIdx.x >> 6, i = threadIdx.x & 31;
+  const int64_t w = (int64_t)blockIdx.x * 4 + group;
   if (w >= nworld) return;
   if ((done && done[w]) || state_changes[w] == 0) return;
   const TileArea<NP> T(lds + group * dense_tile_stage_words<NP>());
   int *ul = (int *)(lds + group * dense_tile_stage_words<NP>() + TileArea<NP>::kWords);  // [nv + 1], the staged rows behind it
   int count = changes[w];
   count = count < 0 ? 0 : (count < ld_ids ? count : ld_ids);
-  dense_tile_world<NP>(T, ul, H_ + w * (int64_t)pad * pad, J + w * (int64_t)njmax * nv, D + w * njmax, grad + w * ldg,
+  dense_tile_world<NP, true>(T, ul, H_ + w * (int64_t)pad * pad, J + w * (int64_t)njmax * nv, D + w * njmax, grad + w * ldg,
                        state + w * njmax, ids + w * ld_ids, count, quad, uni_ + w * (nv + 1), search + w * ld_search,
                        search_dot + w, decrement + w, nv, pad, i);
 }
@@ -376,7 +441,7 @@ __global__ __launch_bounds__(256) void dense_init_tile_kernel(
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   float *mine = lds + wv * dense_tile_stage_words<NP>();
   const TileArea<NP> T(mine);
-  dense_tile_world<NP>(T, (int *)(mine + TileArea<NP>::kWords), Hw, Jw, D + w * njmax, grad + w * ldg, state + w * njmax,
+  dense_tile_world<NP, true>(T, (int *)(mine + TileArea<NP>::kWords), Hw, Jw, D + w * njmax, grad + w * ldg, state + w * njmax,
                        nullptr, 0, quad, uni_ + w * (nv + 1), search + w * ld_search, search_dot + w, decrement + w, nv, pad,
                        lane & 31);
 }
@@ -435,7 +500,7 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void newton_dense_tile_resi
     const TileArea<NP> T(mine);
     int count = b.quad_count[w];
     count = count < 0 ? 0 : (count < b.ld_ids ? count : b.ld_ids);
-    dense_tile_world<NP>(T, (int *)(mine + TileArea<NP>::kWords), H_ + w * (int64_t)pad * pad,
+    dense_tile_world<NP, true>(T, (int *)(mine + TileArea<NP>::kWords), H_ + w * (int64_t)pad * pad,
                          b.J + w * (int64_t)b.njmax * b.nv, b.D + w * b.njmax, b.grad + w * b.ld_grad,
                          b.state + w * b.njmax, b.ids + w * (int64_t)b.ld_ids, count, b.quad, uni_ + w * (b.nv + 1),
                          b.search + w * b.nv, b.search_dot + w, b.decrement + w, b.nv, pad, lane);
@@ -517,10 +582,10 @@ int im_dense_update_tile(const uint8_t *done, const int32_t *state_changes, cons
     return IM_ERR_ARG;
   if (ldg < nv || ld_search < nv) return IM_ERR_STRIDE;
   hipStream_t st = (hipStream_t)stream;
-  const unsigned grid = (unsigned)((nworld + 7) / 8);
+  const unsigned grid = (unsigned)((nworld + 3) / 4);
 #define IM_STAGE_CASE(NP)                                                                                            \
   if (nv <= NP) {                                                                                                    \
-    const size_t lds = sizeof(float) * 8 * im::dense_tile_stage_words<NP>();                                         \
+    const size_t lds = sizeof(float) * 4 * im::dense_tile_stage_words<NP>();                                         \
     hipLaunchKernelGGL(im::dense_update_tile_kernel<NP>, dim3(grid), dim3(256), lds, st, done, state_changes, changes, \
                        ids, ld_ids, J, njmax, D, state, quad, grad, ldg, H, dof_union, search, ld_search, search_dot, \
                        decrement, nv, nv_pad, nworld);                                                               \
@@ -584,7 +649,8 @@ int im_newton_solve_dense_tile(const im_newton_args *p, float *H, int32_t *dof_u
   if (!probed) {  // once per process: a variant that spills registers is left out; the large dynamic LDS is asked for
     for (int i = 0; i < kVariants; ++i) {
       hipFuncAttributes fa{};
-      usable[i] = hipFuncGetAttributes(&fa, variants[i].fn) == hipSuccess && fa.localSizeBytes == 0 &&
+      // (a variant that parks more than a register or two in memory is left out)
+      usable[i] = hipFuncGetAttributes(&fa, variants[i].fn) == hipSuccess && fa.localSizeBytes <= 16 &&
                   hipFuncSetAttribute(variants[i].fn, hipFuncAttributeMaxDynamicSharedMemorySize,
                                       160 * 1024 - (int)fa.sharedSizeBytes) == hipSuccess;
       (void)hipGetLastError();
