@@ -13,7 +13,8 @@ Beside it, `iterations_launch`: the three solves of a step as one launch of
 im_assemble_tree_ldl_solve_iters (a grid over worlds x iterations, for callers that know every
 iteration's states in advance; the solves are then independent of one another), and `newton_solve`:
 whole constraint solves of the same batch shape with dependent iterations (init_context, the resident
-Newton kernel, force recovery), informative.  Prints one JSON line.
+Newton kernel, force recovery) with the fused tree stage, and `newton_solve_dense_stage`: the same with
+the single-tile dense stage of the reference's own loop; both informative.  Prints one JSON line.
 """
 
 from __future__ import annotations
@@ -103,15 +104,16 @@ def cpu_baseline(batch, plan_struct, gpu_x, seconds: float = 10.0):
     }
 
 
-def newton_solve_leg(torch, use_graph: bool, nsets: int = 8, replays: int = 5, solves_per_replay: int = 8):
+def newton_solve_leg(torch, use_graph: bool, stage: str = "tree", nsets: int = 8, replays: int = 5, solves_per_replay: int = 8):
     """Beside the headline: whole constraint solves of the same batch shape with dependent iterations
-    (newton_fusion.solve: init_context, the resident Newton kernel with the fused tree stage, force
-    recovery; tolerance 1e-7, at most 10 iterations), on rotating input sets.  Informative: the
-    headline's metric is the factor-and-solve launch."""
+    (newton_fusion.solve: init_context, the resident Newton kernel with the fused tree stage -- or,
+    ``stage="dense"``, with the single-tile dense stage that the reference's own loop runs at this
+    size -- and the force recovery; tolerance 1e-7, at most 10 iterations), on rotating input sets.
+    Informative: the headline's metric is the factor-and-solve launch."""
     from instantmimic_amd.mjw_kernels import newton_fusion as NF
     from instantmimic_amd.rowbench import newton_case
 
-    cases = [newton_case("humanoid", "tree", seed=21 + k) for k in range(nsets)]
+    cases = [newton_case("humanoid", stage, seed=21 + k) for k in range(nsets)]
     for c in cases[:2]:
         NF.solve(*c)
     torch.cuda.synchronize()
@@ -143,7 +145,9 @@ def newton_solve_leg(torch, use_graph: bool, nsets: int = 8, replays: int = 5, s
     sec = min(times)
     m, d = cases[0][0], cases[0][1]
     return {
-        "entry": "newton_fusion.solve: im_newton_init_context, im_newton_tree_stage, im_newton_solve_tree (one resident kernel for the dependent iterations), im_qfrc_constraint_from_grad",
+        "entry": ("newton_fusion.solve: im_newton_init_context, im_newton_tree_stage, im_newton_solve_tree (one resident kernel for the dependent iterations), im_qfrc_constraint_from_grad"
+                  if stage == "tree" else
+                  "newton_fusion.solve: im_newton_init_context, im_dense_init_factor, im_newton_solve_dense_tile (one resident kernel for the dependent iterations), im_qfrc_constraint_from_grad"),
         "workload": f"humanoid nv={int(m.nv)} nefc={int(d.njmax)} x {int(d.nworld)} worlds, tolerance 1e-7, at most {int(m.opt.iterations)} iterations",
         "us_per_solve": sec * 1e6,
         "iterations_mean": float(its.mean()),
@@ -352,6 +356,7 @@ def main() -> int:
     }
 
     newton = None if args.no_solve else newton_solve_leg(torch, use_graph)
+    newton_dense = None if args.no_solve else newton_solve_leg(torch, use_graph, stage="dense")
 
     out = {
         "metric": METRIC,
@@ -390,6 +395,7 @@ def main() -> int:
     }
     if newton is not None:
         out["newton_solve"] = newton
+        out["newton_solve_dense_stage"] = newton_dense
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(batch, T.tree_ldl_structure(batch.rowadr, batch.rownnz, batch.colind), x_first)
     print(json.dumps(out))
